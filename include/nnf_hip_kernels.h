@@ -1,0 +1,140 @@
+/*
+ * nnf_hip_kernels.h -- C ABI of the gfx950 (MI355X) low-bit GEMM/GEMV launcher library
+ * (libnnf_hip_kernels.so).
+ *
+ * These entry points are what an nnfusion kernel emitter for the quantized Dot/MatMul node
+ * puts in its emitted function body, in the place where the reference's cuda::Dot emitter
+ * puts a cuBLAS call (src/nnfusion/core/kernels/cuda_gpu/kernels/dot.cpp:128-205 for fp32,
+ * :271-363 for fp16) and where FunctionFile emits the `extern void <kernel>_Call(grids, blocks,
+ * mem, stream, args...)` host wrappers (src/nnfusion/engine/pass/codegen/codegenerator_helper.cpp:
+ * 143-177).  Every function
+ *   - takes plain device pointers and sizes (no C++ types, no torch types),
+ *   - is stream ordered: it enqueues on `stream` and returns without synchronising,
+ *   - never allocates: scratch memory is passed in (`workspace`), sized by the matching
+ *     `*_workspace_bytes` query so that an emitter can reserve it at compile time with
+ *     KernelEmitter::allocate_tensor (src/nnfusion/core/kernels/kernel_emitter.cpp:282-319),
+ *   - never throws: it returns NNF_OK (0), a negative NNF_ERR_* code for a rejected call, or a
+ *     positive hipError_t value reported by the HIP runtime.
+ *
+ * Tensor layouts (all dense, row-major, base pointers 16-byte aligned; the reference's memory
+ * planner aligns every tensor to 64 bytes, src/nnfusion/engine/device/rocm.cpp:86):
+ *   A       fp16  [M, K]            activations
+ *   Wq      u8    [N, K/2]          unsigned 4-bit weights, two per byte along K:
+ *                                   low nibble of byte b of a row = k 2b, high nibble = k 2b+1
+ *   scales  fp16  [N, K/group]      one scale per output channel and K-group (group = 128)
+ *   zp      int   scalar            zero point (8): W[n,k] = (q[n,k] - zp) * scales[n, k/group]
+ *   Y       fp16  [M, N]            Y = A . W^T, accumulated in fp32, rounded to nearest even
+ *   W8A8:   A i8 [M,K], s_tok f32 [M], W i8 [N,K], s_ch f32 [N], acc i32 [M,N] (exact),
+ *           Y = fp16( (float)acc * s_tok[m] * s_ch[n] ) evaluated left to right in fp32
+ */
+#ifndef NNF_HIP_KERNELS_H
+#define NNF_HIP_KERNELS_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* A hipStream_t, passed as an opaque pointer so that this header needs no HIP include. */
+typedef void* nnf_stream_t;
+
+enum nnf_status
+{
+    NNF_OK = 0,
+    NNF_ERR_INVALID_ARGUMENT = -1, /* null pointer, non-positive size, misaligned pointer */
+    NNF_ERR_UNSUPPORTED_SHAPE = -2, /* K % group != 0, group != 128, K % 32 != 0, zp outside 0..15 ... */
+    NNF_ERR_WORKSPACE_TOO_SMALL = -3,
+    NNF_ERR_NO_DEVICE = -4 /* no gfx950 device is current */
+};
+
+/* ABI version of this header (bumped on any signature change). */
+int nnf_abi_version(void);
+
+/* Human-readable text for a status returned by any function below (static storage). */
+const char* nnf_status_string(int status);
+
+/* ---------------------------------------------------------------------------------------------
+ * fp16 x int4 (group-scaled) GEMM / GEMV:  Y[M,N] = A[M,K] . ((Wq - zp) * scales)^T
+ * Replaces the cublasHgemm / cublasSgemm call of cuda::Dot (cuda_gpu/kernels/dot.cpp:128-205,
+ * :271-363) for a weight-quantized Dot node with transpose_B = true.  M <= 16 takes the
+ * bandwidth-bound split-K GEMV path, larger M the MFMA path.
+ * ------------------------------------------------------------------------------------------- */
+size_t nnf_w4a16_gemm_workspace_bytes(int M, int N, int K, int group);
+
+int nnf_w4a16_gemm(nnf_stream_t stream,
+                   const void* A, const void* Wq, const void* scales, void* Y,
+                   int M, int N, int K, int group, int zp,
+                   void* workspace, size_t workspace_bytes);
+
+/* Epilogue / prologue selectors for nnf_w4a16_gemm_fused. */
+enum nnf_activation
+{
+    NNF_ACT_NONE = 0,
+    /* Wq/scales hold 2N rows: rows [0,N) are the gate projection, rows [N,2N) the up projection;
+       Y[M,N] = SiLU(gate) * up with SiLU(g) = g * 1/(1+exp(-g))
+       (sigmoid as in cuda_gpu/cuda_kernelops.hpp:447-451, multiply :416). */
+    NNF_ACT_SILU_GATE = 1
+};
+
+/* Same GEMM with the Welder-style fused prologue/epilogue kept on chip:
+ *   rms_gamma != NULL : A is replaced by RMSNorm(A) = A * rsqrt(mean_k(A^2) + rms_eps) * gamma[k]
+ *                       (rsqrt(x + eps) as in LayerNorm, cuda_gpu/cuda_langunit.cpp:618)
+ *   bias      != NULL : fp16 [N], added to every row (MatMulAdd precedent,
+ *                       cuda_gpu/kernels/matmuladd.cpp:29-93)
+ *   residual  != NULL : fp16 [M,N], added element-wise (Add, cuda_kernelops.hpp:408);
+ *                       may alias Y
+ *   act               : nnf_activation
+ */
+size_t nnf_w4a16_gemm_fused_workspace_bytes(int M, int N, int K, int group, int act);
+
+int nnf_w4a16_gemm_fused(nnf_stream_t stream,
+                         const void* A, const void* Wq, const void* scales, void* Y,
+                         int M, int N, int K, int group, int zp,
+                         const void* rms_gamma, float rms_eps,
+                         const void* bias, const void* residual, int act,
+                         void* workspace, size_t workspace_bytes);
+
+/* ---------------------------------------------------------------------------------------------
+ * W8A8: int8 x int8 -> int32 on the int8 MFMA, then the per-token / per-channel dequantisation.
+ * The reference has no emitter for this; the nearest routine in its tree is MLAS's u8 x s8
+ * MlasGemm (thirdparty/mlas/inc/mlas.h:147-163).
+ * ------------------------------------------------------------------------------------------- */
+size_t nnf_w8a8_gemm_workspace_bytes(int M, int N, int K);
+
+/* Y fp16 [M,N] = fp16((float)acc * s_tok[m] * s_ch[n]) */
+int nnf_w8a8_gemm(nnf_stream_t stream,
+                  const void* A, const void* s_tok, const void* W, const void* s_ch, void* Y,
+                  int M, int N, int K,
+                  void* workspace, size_t workspace_bytes);
+
+/* Raw accumulators: acc i32 [M,N] = A . W^T (exact). */
+int nnf_w8a8_gemm_acc(nnf_stream_t stream,
+                      const void* A, const void* W, void* acc,
+                      int M, int N, int K,
+                      void* workspace, size_t workspace_bytes);
+
+/* ---------------------------------------------------------------------------------------------
+ * Fused Llama-style MLP block (one emitted function for the sub-graph
+ *   RMSNorm -> QuantDot(gate|up) -> SiLU*mul -> QuantDot(down) -> Add(residual) ):
+ *   out[M,H] = x + W_down . ( SiLU(W_gate . n) * (W_up . n) ),  n = RMSNorm(x, gamma, eps)
+ * Wgu u8 [2I, H/2] (gate rows then up rows), Sgu fp16 [2I, H/group], Wd u8 [H, I/2],
+ * Sd fp16 [H, I/group].  The only intermediate that touches HBM is h fp16 [M, I] in workspace.
+ * The element-wise semantics follow the reference's ops (Sigmoid, Multiply, Add, Rsqrt:
+ * cuda_gpu/cuda_kernelops.hpp:206-210,408,416,447-451); the reference has no RMSNorm op.
+ * ------------------------------------------------------------------------------------------- */
+size_t nnf_fused_mlp_w4a16_workspace_bytes(int M, int H, int I, int group);
+
+int nnf_fused_mlp_w4a16(nnf_stream_t stream,
+                        const void* x, const void* gamma, float eps,
+                        const void* Wgu, const void* Sgu, const void* Wd, const void* Sd,
+                        void* out,
+                        int M, int H, int I, int group, int zp,
+                        void* workspace, size_t workspace_bytes);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* NNF_HIP_KERNELS_H */

@@ -1,0 +1,93 @@
+// Device-side helpers shared by the gfx950 kernels: vector types, int4 -> fp16 unpacking,
+// wave64 reductions.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace nnf
+{
+    typedef _Float16 half_t;
+    typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+    typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+    typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+    typedef float floatx4 __attribute__((ext_vector_type(4)));
+    typedef float floatx16 __attribute__((ext_vector_type(16)));
+    typedef int intx4 __attribute__((ext_vector_type(4)));
+    typedef int intx16 __attribute__((ext_vector_type(16)));
+    typedef uint32_t uintx4 __attribute__((ext_vector_type(4)));
+    typedef uint32_t uintx2 __attribute__((ext_vector_type(2)));
+
+    constexpr int WAVE = 64;
+
+    __device__ __forceinline__ half2_t as_half2(uint32_t u)
+    {
+        return __builtin_bit_cast(half2_t, u);
+    }
+    __device__ __forceinline__ uint32_t as_u32(half2_t h)
+    {
+        return __builtin_bit_cast(uint32_t, h);
+    }
+
+    // One 32-bit word holds eight 4-bit weights q0..q7 (q_i at bits 4i..4i+3, i.e. k = i within
+    // the word).  fp16 0x6400 is 1024.0 with an ulp of 1, so (nibble | 0x6400) is 1024 + q and a
+    // nibble four bits higher gives 1024 + 16 q; both are turned into the exact integer (q - zp)
+    // with one packed op.  Output pairs are (q0,q4) (q1,q5) (q2,q6) (q3,q7): the activation
+    // operand is stored in the same order (see permute_a8).
+    //   c_lo = -(1024 + zp)  (packed),  c_hi = -(64 + zp)  (packed),  sixteenth = 1/16 (packed)
+    struct DequantConst
+    {
+        half2_t c_lo, c_hi, sixteenth;
+    };
+
+    __device__ __forceinline__ DequantConst make_dequant_const(int zp)
+    {
+        DequantConst c;
+        half_t lo = (half_t)(-(1024.0f + (float)zp));
+        half_t hi = (half_t)(-(64.0f + (float)zp));
+        c.c_lo = half2_t{lo, lo};
+        c.c_hi = half2_t{hi, hi};
+        c.sixteenth = half2_t{(half_t)0.0625f, (half_t)0.0625f};
+        return c;
+    }
+
+    __device__ __forceinline__ void dequant8(uint32_t w, const DequantConst& c, half2_t out[4])
+    {
+        const uint32_t MAGIC = 0x64006400u;
+        uint32_t w8 = w >> 8;
+        half2_t lo0 = as_half2((w & 0x000F000Fu) | MAGIC);
+        half2_t hi0 = as_half2((w & 0x00F000F0u) | MAGIC);
+        half2_t lo1 = as_half2((w8 & 0x000F000Fu) | MAGIC);
+        half2_t hi1 = as_half2((w8 & 0x00F000F0u) | MAGIC);
+        out[0] = lo0 + c.c_lo;                                        // (q0, q4) - zp
+        out[1] = __builtin_elementwise_fma(hi0, c.sixteenth, c.c_hi); // (q1, q5) - zp
+        out[2] = lo1 + c.c_lo;                                        // (q2, q6) - zp
+        out[3] = __builtin_elementwise_fma(hi1, c.sixteenth, c.c_hi); // (q3, q7) - zp
+    }
+
+    // Reorder eight consecutive fp16 activations a0..a7 (as four 32-bit words) into the pair
+    // order produced by dequant8: (a0,a4) (a1,a5) (a2,a6) (a3,a7).
+    __device__ __forceinline__ uintx4 permute_a8(uintx4 a)
+    {
+        uintx4 r;
+        // v_perm_b32(S0, S1, sel): byte selectors 0-3 pick from S1, 4-7 from S0
+        r.x = __builtin_amdgcn_perm(a.z, a.x, 0x05040100u); // lo(a.x)=a0, lo(a.z)=a4
+        r.y = __builtin_amdgcn_perm(a.z, a.x, 0x07060302u); // hi(a.x)=a1, hi(a.z)=a5
+        r.z = __builtin_amdgcn_perm(a.w, a.y, 0x05040100u); // a2, a6
+        r.w = __builtin_amdgcn_perm(a.w, a.y, 0x07060302u); // a3, a7
+        return r;
+    }
+
+    __device__ __forceinline__ float dot2(half2_t a, half2_t b, float c)
+    {
+        return __builtin_amdgcn_fdot2(a, b, c, false);
+    }
+
+    __device__ __forceinline__ float wave_sum(float v)
+    {
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1)
+            v += __shfl_xor(v, off, WAVE);
+        return v;
+    }
+} // namespace nnf

@@ -1,0 +1,18 @@
+// Internal launch functions behind the C ABI (one per kernel family).  Each validates nothing:
+// nnf_api.hip checks shapes, alignment and workspace before calling in.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+namespace nnf
+{
+    // largest dynamic LDS a workgroup may ask for on gfx950 (160 KiB per CU)
+    constexpr size_t MAX_LDS_BYTES = 160 * 1024;
+
+    hipError_t launch_w4a16_gemv(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y,
+                                 int M, int N, int K, int zp, int num_cu);
+    // true when launch_w4a16_gemv can stage the activations of one pass in LDS
+    bool w4a16_gemv_supported(int M, int K);
+} // namespace nnf

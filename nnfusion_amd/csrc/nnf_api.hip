@@ -1,0 +1,130 @@
+// C ABI of libnnf_hip_kernels.so: argument checks, dispatch by shape, error mapping.
+// Declarations and the contract of each entry point are in include/nnf_hip_kernels.h.
+#include "nnf_hip_kernels.h"
+#include "kernels/nnf_launch.h"
+
+#include <hip/hip_runtime.h>
+
+namespace
+{
+    struct DeviceInfo
+    {
+        int valid = 0;
+        int num_cu = 0;
+    };
+
+    // Lazily cached properties of each device (the only global state of the library).
+    DeviceInfo g_dev[64];
+
+    int current_device_info(DeviceInfo& out)
+    {
+        int dev = -1;
+        hipError_t e = hipGetDevice(&dev);
+        if (e != hipSuccess || dev < 0 || dev >= 64)
+            return NNF_ERR_NO_DEVICE;
+        if (!g_dev[dev].valid)
+        {
+            hipDeviceProp_t prop;
+            e = hipGetDeviceProperties(&prop, dev);
+            if (e != hipSuccess)
+                return (int)e;
+            g_dev[dev].num_cu = prop.multiProcessorCount;
+            g_dev[dev].valid = 1;
+        }
+        out = g_dev[dev];
+        return NNF_OK;
+    }
+
+    inline bool aligned16(const void* p)
+    {
+        return (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
+    }
+
+    int check_w4a16(const void* A, const void* Wq, const void* S, const void* Y, int M, int N, int K, int group,
+                    int zp)
+    {
+        if (!A || !Wq || !S || !Y || M <= 0 || N <= 0 || K <= 0)
+            return NNF_ERR_INVALID_ARGUMENT;
+        if (!aligned16(A) || !aligned16(Wq) || !aligned16(S) || !aligned16(Y))
+            return NNF_ERR_INVALID_ARGUMENT;
+        if (group != 128 || K % group != 0 || zp < 0 || zp > 15)
+            return NNF_ERR_UNSUPPORTED_SHAPE;
+        return NNF_OK;
+    }
+} // namespace
+
+extern "C" {
+
+int nnf_abi_version(void)
+{
+    return 1;
+}
+
+const char* nnf_status_string(int status)
+{
+    switch (status)
+    {
+    case NNF_OK: return "ok";
+    case NNF_ERR_INVALID_ARGUMENT: return "invalid argument (null/misaligned pointer or non-positive size)";
+    case NNF_ERR_UNSUPPORTED_SHAPE: return "unsupported shape or quantisation parameters";
+    case NNF_ERR_WORKSPACE_TOO_SMALL: return "workspace too small";
+    case NNF_ERR_NO_DEVICE: return "no current HIP device";
+    default: break;
+    }
+    if (status > 0)
+        return hipGetErrorString((hipError_t)status);
+    return "unknown nnf status";
+}
+
+size_t nnf_w4a16_gemm_workspace_bytes(int M, int N, int K, int group)
+{
+    (void)M;
+    (void)N;
+    (void)K;
+    (void)group;
+    return 0;
+}
+
+int nnf_w4a16_gemm(nnf_stream_t stream, const void* A, const void* Wq, const void* scales, void* Y, int M, int N,
+                   int K, int group, int zp, void* workspace, size_t workspace_bytes)
+{
+    (void)workspace;
+    int st = check_w4a16(A, Wq, scales, Y, M, N, K, group, zp);
+    if (st != NNF_OK)
+        return st;
+    if (workspace_bytes < nnf_w4a16_gemm_workspace_bytes(M, N, K, group))
+        return NNF_ERR_WORKSPACE_TOO_SMALL;
+    DeviceInfo dev;
+    st = current_device_info(dev);
+    if (st != NNF_OK)
+        return st;
+    if (!nnf::w4a16_gemv_supported(M, K))
+        return NNF_ERR_UNSUPPORTED_SHAPE;
+    return (int)nnf::launch_w4a16_gemv((hipStream_t)stream, A, Wq, scales, Y, M, N, K, zp, dev.num_cu);
+}
+
+// ---- entry points whose kernels are not wired yet: reject every call -------------------------
+size_t nnf_w4a16_gemm_fused_workspace_bytes(int, int, int, int, int) { return 0; }
+int nnf_w4a16_gemm_fused(nnf_stream_t, const void*, const void*, const void*, void*, int, int, int, int, int,
+                         const void*, float, const void*, const void*, int, void*, size_t)
+{
+    return NNF_ERR_UNSUPPORTED_SHAPE;
+}
+size_t nnf_w8a8_gemm_workspace_bytes(int, int, int) { return 0; }
+int nnf_w8a8_gemm(nnf_stream_t, const void*, const void*, const void*, const void*, void*, int, int, int, void*,
+                  size_t)
+{
+    return NNF_ERR_UNSUPPORTED_SHAPE;
+}
+int nnf_w8a8_gemm_acc(nnf_stream_t, const void*, const void*, void*, int, int, int, void*, size_t)
+{
+    return NNF_ERR_UNSUPPORTED_SHAPE;
+}
+size_t nnf_fused_mlp_w4a16_workspace_bytes(int, int, int, int) { return 0; }
+int nnf_fused_mlp_w4a16(nnf_stream_t, const void*, const void*, float, const void*, const void*, const void*,
+                        const void*, void*, int, int, int, int, int, void*, size_t)
+{
+    return NNF_ERR_UNSUPPORTED_SHAPE;
+}
+
+} // extern "C"

@@ -1,0 +1,118 @@
+"""Thin torch-tensor front over the C ABI (device pointers + the current HIP stream).
+
+torch is used for device memory and streams only; every computation happens in
+libnnf_hip_kernels.so.  A non-zero status from the library raises NnfError (the emitted host
+wrappers of the codegen path throw std::runtime_error in the same situation).
+"""
+import torch
+
+from . import _lib
+
+
+class NnfError(RuntimeError):
+    def __init__(self, status, where):
+        self.status = status
+        msg = _lib.kernels().nnf_status_string(status).decode()
+        super().__init__(f"{where}: status {status} ({msg})")
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _check(status, where):
+    if status != 0:
+        raise NnfError(status, where)
+
+
+def _ws(nbytes, device):
+    # the library never allocates; the caller (here: the test/bench harness) owns the workspace
+    return torch.empty(max(int(nbytes), 16), dtype=torch.uint8, device=device)
+
+
+def _p(t):
+    return 0 if t is None else t.data_ptr()
+
+
+def w4a16_gemm(a, wq, scales, group=128, zp=8, out=None, workspace=None):
+    """Y[M,N] = A[M,K] . ((Wq - zp) * scales)^T ; a fp16 [M,K], wq u8 [N,K/2], scales fp16 [N,K/group]."""
+    lib = _lib.kernels()
+    m, k = a.shape
+    n = wq.shape[0]
+    assert a.dtype == torch.float16 and wq.dtype == torch.uint8 and scales.dtype == torch.float16
+    assert a.is_contiguous() and wq.is_contiguous() and scales.is_contiguous()
+    assert wq.shape[1] * 2 == k and tuple(scales.shape) == (n, k // group)
+    if out is None:
+        out = torch.empty((m, n), dtype=torch.float16, device=a.device)
+    need = lib.nnf_w4a16_gemm_workspace_bytes(m, n, k, group)
+    if workspace is None:
+        workspace = _ws(need, a.device)
+    _check(lib.nnf_w4a16_gemm(_stream(), a.data_ptr(), wq.data_ptr(), scales.data_ptr(), out.data_ptr(),
+                              m, n, k, group, zp, workspace.data_ptr(), workspace.numel()), "nnf_w4a16_gemm")
+    return out
+
+
+def w4a16_gemm_fused(a, wq, scales, group=128, zp=8, rms_gamma=None, rms_eps=1e-6, bias=None, residual=None,
+                     act=0, out=None, workspace=None):
+    """GEMM with the fused RMSNorm prologue / bias, residual, SiLU-gate epilogues (see the C header)."""
+    lib = _lib.kernels()
+    m, k = a.shape
+    n = wq.shape[0] // (2 if act == 1 else 1)
+    if out is None:
+        out = torch.empty((m, n), dtype=torch.float16, device=a.device)
+    need = lib.nnf_w4a16_gemm_fused_workspace_bytes(m, n, k, group, act)
+    if workspace is None:
+        workspace = _ws(need, a.device)
+    _check(lib.nnf_w4a16_gemm_fused(_stream(), a.data_ptr(), wq.data_ptr(), scales.data_ptr(), out.data_ptr(),
+                                    m, n, k, group, zp, _p(rms_gamma), float(rms_eps), _p(bias), _p(residual),
+                                    int(act), workspace.data_ptr(), workspace.numel()), "nnf_w4a16_gemm_fused")
+    return out
+
+
+def w8a8_gemm(a, s_tok, w, s_ch, out=None, workspace=None):
+    """Y fp16 [M,N] = fp16((float)(A . W^T) * s_tok[m] * s_ch[n]) ; a i8 [M,K], w i8 [N,K]."""
+    lib = _lib.kernels()
+    m, k = a.shape
+    n = w.shape[0]
+    assert a.dtype == torch.int8 and w.dtype == torch.int8
+    assert s_tok.dtype == torch.float32 and s_ch.dtype == torch.float32
+    if out is None:
+        out = torch.empty((m, n), dtype=torch.float16, device=a.device)
+    need = lib.nnf_w8a8_gemm_workspace_bytes(m, n, k)
+    if workspace is None:
+        workspace = _ws(need, a.device)
+    _check(lib.nnf_w8a8_gemm(_stream(), a.data_ptr(), s_tok.data_ptr(), w.data_ptr(), s_ch.data_ptr(),
+                             out.data_ptr(), m, n, k, workspace.data_ptr(), workspace.numel()), "nnf_w8a8_gemm")
+    return out
+
+
+def w8a8_gemm_acc(a, w, out=None, workspace=None):
+    """acc i32 [M,N] = A . W^T, exact."""
+    lib = _lib.kernels()
+    m, k = a.shape
+    n = w.shape[0]
+    assert a.dtype == torch.int8 and w.dtype == torch.int8
+    if out is None:
+        out = torch.empty((m, n), dtype=torch.int32, device=a.device)
+    need = lib.nnf_w8a8_gemm_workspace_bytes(m, n, k)
+    if workspace is None:
+        workspace = _ws(need, a.device)
+    _check(lib.nnf_w8a8_gemm_acc(_stream(), a.data_ptr(), w.data_ptr(), out.data_ptr(), m, n, k,
+                                 workspace.data_ptr(), workspace.numel()), "nnf_w8a8_gemm_acc")
+    return out
+
+
+def fused_mlp_w4a16(x, gamma, wgu, sgu, wd, sd, eps=1e-6, group=128, zp=8, out=None, workspace=None):
+    """out = x + Wd . (SiLU(Wg . n) * (Wu . n)), n = RMSNorm(x, gamma, eps)."""
+    lib = _lib.kernels()
+    m, h = x.shape
+    i = wgu.shape[0] // 2
+    if out is None:
+        out = torch.empty((m, h), dtype=torch.float16, device=x.device)
+    need = lib.nnf_fused_mlp_w4a16_workspace_bytes(m, h, i, group)
+    if workspace is None:
+        workspace = _ws(need, x.device)
+    _check(lib.nnf_fused_mlp_w4a16(_stream(), x.data_ptr(), gamma.data_ptr(), float(eps), wgu.data_ptr(),
+                                   sgu.data_ptr(), wd.data_ptr(), sd.data_ptr(), out.data_ptr(), m, h, i, group, zp,
+                                   workspace.data_ptr(), workspace.numel()), "nnf_fused_mlp_w4a16")
+    return out

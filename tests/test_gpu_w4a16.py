@@ -1,0 +1,73 @@
+"""Parity of the fp16 x int4 GEMV/GEMM (HIP, through the C ABI) against the CPU oracle.
+
+Tolerance (stated by the task): max|y - y_ref| <= 1e-2 * RMS(y_ref), y_ref = the fp32-accumulated
+dequant-GEMM of the oracle (un-rounded fp32 output).
+"""
+import numpy as np
+import pytest
+
+import oracle
+from nnfusion_amd import datagen
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-2
+
+
+def _run(gpu, a, wq, s, zp=8):
+    import torch
+
+    from nnfusion_amd import ops
+
+    y = ops.w4a16_gemm(torch.from_numpy(a).to(gpu), torch.from_numpy(wq).to(gpu), torch.from_numpy(s).to(gpu), zp=zp)
+    torch.cuda.synchronize()
+    return y.cpu().numpy()
+
+
+def _check(y, ref):
+    rms = float(np.sqrt(np.mean(ref.astype(np.float64) ** 2)))
+    err = float(np.abs(y.astype(np.float32) - ref).max())
+    assert err <= TOL * max(rms, 1e-6), (err, rms)
+    return err, rms
+
+
+@pytest.mark.parametrize("m,n,k", [
+    (1, 4096, 4096),      # configs[0]
+    (1, 12288, 4096), (1, 22016, 4096), (1, 4096, 11008),  # configs[1]
+    (1, 7, 128), (1, 1, 256), (2, 33, 384), (3, 100, 2048), (4, 257, 2176),
+    (5, 64, 4096), (7, 130, 1024), (8, 512, 8192), (16, 1024, 8192),
+])
+def test_gemv_matches_oracle(gpu, m, n, k):
+    print(f"case M={m} N={n} K={k}", flush=True)
+    a, wq, s = datagen.w4a16_case(0, m, n, k)
+    y = _run(gpu, a, wq, s)
+    ref = oracle.w4a16_gemm(a, wq, s, f32_out=True)
+    _check(y, ref)
+
+
+def test_gemv_all_zero_point_is_zero(gpu):
+    # every q == zp  =>  Y == 0 exactly
+    a, wq, s = datagen.w4a16_case(1, 2, 96, 512)
+    wq[:] = 0x88
+    y = _run(gpu, a, wq, s)
+    assert np.all(y == 0)
+
+
+def test_gemv_one_hot_reads_single_weight(gpu):
+    # A = e_k  =>  Y[n] = fp16((q[n,k]-8) * s[n,k/128]) : pins nibble order and scale indexing
+    n, k = 64, 512
+    _, wq, s = datagen.w4a16_case(2, 1, n, k)
+    wd = oracle.dequantize_w4(wq, s)
+    for kk in (0, 1, 2, 7, 8, 31, 32, 127, 128, 129, 255, 511):
+        a = np.zeros((1, k), np.float16)
+        a[0, kk] = 1.0
+        y = _run(gpu, a, wq, s)
+        np.testing.assert_array_equal(y[0], wd[:, kk].astype(np.float16))
+
+
+@pytest.mark.parametrize("zp", [0, 7, 15])
+def test_gemv_other_zero_points(gpu, zp):
+    a, wq, s = datagen.w4a16_case(3, 2, 128, 1024)
+    y = _run(gpu, a, wq, s, zp=zp)
+    ref = oracle.w4a16_gemm(a, wq, s, zp=zp, f32_out=True)
+    _check(y, ref)
