@@ -83,6 +83,13 @@ namespace nnf
         return __builtin_amdgcn_fdot2(a, b, c, false);
     }
 
+    // Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every
+    // outstanding global load (vmcnt(0)), which would drain software-pipelined prefetches.
+    __device__ __forceinline__ void lds_barrier()
+    {
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    }
+
     __device__ __forceinline__ float wave_sum(float v)
     {
 #pragma unroll

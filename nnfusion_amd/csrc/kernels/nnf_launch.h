@@ -15,4 +15,18 @@ namespace nnf
                                  int M, int N, int K, int zp, int num_cu);
     // true when launch_w4a16_gemv can stage the activations of one pass in LDS
     bool w4a16_gemv_supported(int M, int K);
+
+    hipError_t launch_w4a16_skinny(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M,
+                                   int N, int K, int zp, int num_cu);
+    // true when one workgroup can hold the activations (M <= 16 rows of K) in LDS
+    bool w4a16_skinny_supported(int M, int K);
+
+    // Tuning knobs for experiments (not part of the public ABI): 0 = automatic.
+    struct Tuning
+    {
+        int force_path = 0;  // 1 = VALU GEMV, 2 = MFMA skinny
+        int skinny_cps = 0;  // chunks (groups of 128) per wavefront
+        int skinny_wg_per_cu = 0;
+    };
+    extern Tuning g_tuning;
 } // namespace nnf

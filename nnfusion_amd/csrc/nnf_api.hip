@@ -53,7 +53,24 @@ namespace
     }
 } // namespace
 
+namespace nnf
+{
+    Tuning g_tuning;
+}
+
 extern "C" {
+
+// experiment hook, deliberately absent from the public header
+int nnf_internal_tune(int key, int value)
+{
+    switch (key)
+    {
+    case 0: nnf::g_tuning.force_path = value; return 0;
+    case 1: nnf::g_tuning.skinny_cps = value; return 0;
+    case 2: nnf::g_tuning.skinny_wg_per_cu = value; return 0;
+    default: return -1;
+    }
+}
 
 int nnf_abi_version(void)
 {
@@ -98,6 +115,9 @@ int nnf_w4a16_gemm(nnf_stream_t stream, const void* A, const void* Wq, const voi
     st = current_device_info(dev);
     if (st != NNF_OK)
         return st;
+    const int force = nnf::g_tuning.force_path;
+    if (force != 1 && M <= 16 && nnf::w4a16_skinny_supported(M, K))
+        return (int)nnf::launch_w4a16_skinny((hipStream_t)stream, A, Wq, scales, Y, M, N, K, zp, dev.num_cu);
     if (!nnf::w4a16_gemv_supported(M, K))
         return NNF_ERR_UNSUPPORTED_SHAPE;
     return (int)nnf::launch_w4a16_gemv((hipStream_t)stream, A, Wq, scales, Y, M, N, K, zp, dev.num_cu);

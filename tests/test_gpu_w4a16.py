@@ -14,6 +14,17 @@ pytestmark = pytest.mark.gpu
 TOL = 1e-2
 
 
+@pytest.fixture(params=["auto", "valu_gemv", "mfma_skinny"])
+def path(request):
+    """Runs a test once per kernel family that can serve M <= 16 (auto = the library's own choice)."""
+    from nnfusion_amd import _lib
+
+    tune = _lib.kernels().nnf_internal_tune
+    tune(0, {"auto": 0, "valu_gemv": 1, "mfma_skinny": 2}[request.param])
+    yield request.param
+    tune(0, 0)
+
+
 def _run(gpu, a, wq, s, zp=8):
     import torch
 
@@ -37,7 +48,7 @@ def _check(y, ref):
     (1, 7, 128), (1, 1, 256), (2, 33, 384), (3, 100, 2048), (4, 257, 2176),
     (5, 64, 4096), (7, 130, 1024), (8, 512, 8192), (16, 1024, 8192),
 ])
-def test_gemv_matches_oracle(gpu, m, n, k):
+def test_gemv_matches_oracle(gpu, path, m, n, k):
     print(f"case M={m} N={n} K={k}", flush=True)
     a, wq, s = datagen.w4a16_case(0, m, n, k)
     y = _run(gpu, a, wq, s)
@@ -45,15 +56,23 @@ def test_gemv_matches_oracle(gpu, m, n, k):
     _check(y, ref)
 
 
-def test_gemv_all_zero_point_is_zero(gpu):
-    # every q == zp  =>  Y == 0 exactly
-    a, wq, s = datagen.w4a16_case(1, 2, 96, 512)
+def test_gemv_all_zero_point_is_zero(gpu, path):
+    # every q == zp  =>  Y == 0: exactly on the VALU path (it dequantises to the exact integer
+    # q - zp); the MFMA path removes the 1024 + zp offset of its operand encoding from the fp32
+    # group sum, which leaves fp32 rounding residue: bounded here at 2e-4 of the RMS a random
+    # weight matrix of this K would give (50x below the parity tolerance).
+    k = 512
+    a, wq, s = datagen.w4a16_case(1, 2, 96, k)
     wq[:] = 0x88
     y = _run(gpu, a, wq, s)
-    assert np.all(y == 0)
+    if path == "valu_gemv":
+        assert np.all(y == 0)
+    else:
+        rms_typical = np.sqrt(k * 21.25 * 1.75e-4)
+        assert np.abs(y.astype(np.float32)).max() <= 2e-4 * rms_typical
 
 
-def test_gemv_one_hot_reads_single_weight(gpu):
+def test_gemv_one_hot_reads_single_weight(gpu, path):
     # A = e_k  =>  Y[n] = fp16((q[n,k]-8) * s[n,k/128]) : pins nibble order and scale indexing
     n, k = 64, 512
     _, wq, s = datagen.w4a16_case(2, 1, n, k)
@@ -66,7 +85,7 @@ def test_gemv_one_hot_reads_single_weight(gpu):
 
 
 @pytest.mark.parametrize("zp", [0, 7, 15])
-def test_gemv_other_zero_points(gpu, zp):
+def test_gemv_other_zero_points(gpu, path, zp):
     a, wq, s = datagen.w4a16_case(3, 2, 128, 1024)
     y = _run(gpu, a, wq, s, zp=zp)
     ref = oracle.w4a16_gemm(a, wq, s, zp=zp, f32_out=True)
