@@ -21,10 +21,17 @@ namespace nnf
     // true when one workgroup can hold the activations (M <= 16 rows of K) in LDS
     bool w4a16_skinny_supported(int M, int K);
 
+    // MFMA GEMM (any M) with the fused RMSNorm prologue and bias / residual / SiLU-gate epilogues.
+    // workspace: w4a16_gemm_fused_workspace(M, rms) bytes (the per-row rstd of the RMSNorm).
+    hipError_t launch_w4a16_gemm(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M,
+                                 int N, int K, int zp, const void* rms_gamma, float rms_eps, const void* bias,
+                                 const void* residual, int act, void* workspace);
+    size_t w4a16_gemm_fused_workspace(int M, bool rms);
+
     // Tuning knobs for experiments (not part of the public ABI): 0 = automatic.
     struct Tuning
     {
-        int force_path = 0;  // 1 = VALU GEMV, 2 = MFMA skinny
+        int force_path = 0;  // 1 = VALU GEMV, 2 = MFMA skinny, 3 = MFMA GEMM
         int skinny_cps = 0;  // chunks (groups of 128) per wavefront
         int skinny_wg_per_cu = 0;
     };

@@ -1,0 +1,449 @@
+// fp16 x int4 (g128) GEMM for M > 16 on the gfx950 matrix cores (v_mfma_f32_32x32x16_f16).
+//
+//   Y[M,N] = epilogue( prologue(A)[M,K] . ((Wq - zp) * S)^T )
+//
+// Workgroup tile 256 (M) x 256 (N) x 64 (K), four wavefronts in a 2 x 2 arrangement, each owning a
+// 128 x 128 sub-tile = 4 x 4 MFMA tiles of 32 x 32 (256 fp32 accumulators per lane).
+//   * A (fp16) and Wq (raw int4) tiles of the next K step are fetched global -> registers while
+//     the current step is computed from LDS; LDS is double buffered, one barrier per K step.
+//   * LDS layouts are XOR-swizzled at 16-byte granularity so that both the 128-bit stores and the
+//     128-bit MFMA operand reads are bank-conflict free.
+//   * int4 -> fp16 happens in registers right before the MFMA: (q | 0x6400) = 1024 + q, then one
+//     packed add (or fma for the nibble four bits up) gives the exact integer q - zp, one packed
+//     multiply applies the group scale.  A dequantised fragment feeds four MFMAs (the four M
+//     tiles of the wavefront).  The pair order of the unpacking, (q0,q4)(q1,q5)(q2,q6)(q3,q7), is
+//     matched by permuting the activations once while they are staged into LDS.
+//   * The K index inside a 64-wide tile is assigned to MFMA slots as k = 32*h + 8*s + e
+//     (h = lane / 32, s = MFMA step 0..3, e = element), so that a lane's 16 weight bytes of a tile
+//     row are one 128-bit LDS read and the matching activations are 16 contiguous bytes.
+//   * Fused prologue / epilogues (template flags): RMSNorm (per-row rstd from a small pre-pass,
+//     applied with gamma while staging A), bias, residual add, SiLU(gate) * up with the gate and
+//     up projections as two halves of the N tile.
+#include "nnf_device.h"
+#include "nnf_launch.h"
+
+#include <algorithm>
+
+namespace nnf
+{
+    namespace gemm
+    {
+        constexpr int BM = 256, BN = 256, BK = 64;
+        constexpr int A_TILE_BYTES = BM * BK * 2;     // 32 KiB
+        constexpr int W_TILE_BYTES = BN * BK / 2;     // 8 KiB
+        constexpr int STAGE_BYTES = A_TILE_BYTES + W_TILE_BYTES;
+        constexpr int LDS_BYTES = 2 * STAGE_BYTES;    // 80 KiB
+
+        // byte offset of 16-byte piece p (0..7) of row r in the swizzled A tile
+        __device__ __forceinline__ int a_off(int r, int p)
+        {
+            return r * 128 + ((p ^ ((r >> 1) & 7)) << 4);
+        }
+        // byte offset of 16-byte piece h (0..1) of row r in the swizzled W tile
+        __device__ __forceinline__ int w_off(int r, int h)
+        {
+            return r * 32 + ((h ^ ((r >> 3) & 1)) << 4);
+        }
+    } // namespace gemm
+
+    struct GemmParams
+    {
+        const half_t* A;
+        const uint8_t* Wq;
+        const half_t* S;
+        half_t* Y;
+        int M, N, K, zp;
+        int ldy;              // row stride of Y (= N of the output)
+        int up_row_offset;    // GATE: weight row of the up projection that pairs with gate row 0
+        const float* rstd;    // RMS: per-row 1/sqrt(mean(x^2)+eps)
+        const half_t* gamma;  // RMS: [K]
+        const half_t* bias;   // BIAS: [N]
+        const half_t* residual; // RESID: [M, ldy]
+    };
+
+    // one row of rstd per wavefront: rstd[m] = rsqrt(mean_k(x[m,k]^2) + eps)
+    __global__ __launch_bounds__(256) void rms_rstd_kernel(const half_t* __restrict__ X, float* __restrict__ rstd,
+                                                           int M, int K, float eps)
+    {
+        const int lane = threadIdx.x & 63;
+        const int m = blockIdx.x * 4 + (threadIdx.x >> 6);
+        if (m >= M)
+            return;
+        const uintx4* row = reinterpret_cast<const uintx4*>(X + (size_t)m * K);
+        float ss = 0.f;
+        for (int i = lane; i < (K >> 3); i += 64)
+        {
+            uintx4 v = row[i];
+            const uint32_t vv[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+            {
+                half2_t h = as_half2(vv[j]);
+                float a = (float)h.x, b = (float)h.y;
+                ss = __builtin_fmaf(a, a, ss);
+                ss = __builtin_fmaf(b, b, ss);
+            }
+        }
+        ss = wave_sum(ss);
+        if (lane == 0)
+            rstd[m] = 1.0f / __builtin_sqrtf(ss / (float)K + eps);
+    }
+
+    template <bool GATE, bool RMS, bool BIAS, bool RESID>
+    __global__ __launch_bounds__(256) void w4a16_gemm_kernel(GemmParams p)
+    {
+        using namespace gemm;
+        extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+        const int tid = threadIdx.x;
+        const int lane = tid & 63;
+        const int wave = tid >> 6;
+        const int wm = wave >> 1, wn = wave & 1;
+        const int l32 = lane & 31, h = lane >> 5;
+        const int K = p.K;
+        const int G = K >> 7;
+        constexpr int BN_OUT = GATE ? BN / 2 : BN; // output columns of a workgroup tile
+
+        // XCD-aware tile order: workgroup ids are dealt round-robin to the 8 XCDs (each with its own
+        // L2); give each XCD a contiguous run of tiles, and walk tiles M-fastest so that tiles that
+        // are resident together share the weight panel.
+        const int tiles_m = (p.M + BM - 1) / BM;
+        const int tiles_n = (p.N + BN_OUT - 1) / BN_OUT;
+        const int n_wg = tiles_m * tiles_n;
+        int pid = blockIdx.x;
+        {
+            const int per_xcd = (n_wg + 7) >> 3;
+            const int full = n_wg - (per_xcd - 1) * 8; // XCDs that own per_xcd tiles (1..8)
+            const int xcd = pid & 7, idx = pid >> 3;
+            pid = (xcd < full) ? xcd * per_xcd + idx : full * per_xcd + (xcd - full) * (per_xcd - 1) + idx;
+        }
+        const int tm = pid % tiles_m, tn = pid / tiles_m;
+        const int m0 = tm * BM, n0 = tn * BN_OUT;
+
+        // ---- global -> register staging maps -------------------------------------------------------
+        // A: 2048 pieces of 16 B, 8 per thread: row = i*32 + tid/8, piece = tid%8
+        const int a_p = tid & 7;
+        const int a_r0 = tid >> 3;
+        const half_t* a_src[8];
+        int a_dst[8];
+        float a_rstd[RMS ? 8 : 1];
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+        {
+            int r = i * 32 + a_r0;
+            int gm = min(m0 + r, p.M - 1);
+            a_src[i] = p.A + (size_t)gm * K + a_p * 8;
+            a_dst[i] = a_off(r, a_p);
+            if (RMS)
+                a_rstd[i] = p.rstd[gm];
+        }
+        // W: 512 pieces of 16 B, 2 per thread: row = i*128 + tid/2, piece = tid%2
+        const int w_h = tid & 1;
+        const uint8_t* w_src[2];
+        int w_dst[2];
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+        {
+            int r = i * 128 + (tid >> 1);
+            int gn;
+            if (GATE)
+                gn = (r < BN / 2) ? (n0 + r) : (p.up_row_offset + n0 + (r - BN / 2));
+            else
+                gn = n0 + r;
+            // rows past the end of N are clamped (their results are never stored)
+            gn = GATE ? min(gn, p.up_row_offset + p.N - 1) : min(gn, p.N - 1);
+            w_src[i] = p.Wq + (size_t)gn * (K >> 1) + w_h * 16;
+            w_dst[i] = A_TILE_BYTES + w_off(r, w_h);
+        }
+
+        // ---- per-lane fragment addresses in LDS ------------------------------------------------------
+        int a_frag[4]; // row part of the A fragment address for M tile i (piece added per step)
+        int a_swz[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+        {
+            int r = wm * 128 + i * 32 + l32;
+            a_frag[i] = r * 128;
+            a_swz[i] = (r >> 1) & 7;
+        }
+        int w_frag[4];
+        size_t s_idx[4];        // element index of this lane's column scale, group 0, in N tile j
+        int col_out[4];         // output column of N tile j
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+        {
+            int r; // row of the W tile
+            int gn;
+            if (GATE)
+            {
+                int half_sel = j >> 1; // 0 = gate, 1 = up
+                int c = wn * 64 + (j & 1) * 32 + l32;
+                r = half_sel * (BN / 2) + c;
+                gn = half_sel ? (p.up_row_offset + n0 + c) : (n0 + c);
+                gn = min(gn, p.up_row_offset + p.N - 1);
+                col_out[j] = n0 + c;
+            }
+            else
+            {
+                r = wn * 128 + j * 32 + l32;
+                gn = min(n0 + r, p.N - 1);
+                col_out[j] = n0 + r;
+            }
+            w_frag[j] = A_TILE_BYTES + w_off(r, h);
+            s_idx[j] = (size_t)gn * G;
+        }
+
+        floatx16 acc[4][4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int e = 0; e < 16; ++e)
+                    acc[i][j][e] = 0.f;
+
+        const DequantConst dq = make_dequant_const(p.zp);
+        uint32_t MAGIC;
+        asm("s_mov_b32 %0, 0x64006400" : "=s"(MAGIC));
+
+        // Group scales are fetched one group (two K steps) ahead as the aligned 32-bit word that
+        // holds the fp16 (a 16-bit load would be widened at its point of use and force a wait for
+        // every younger load, i.e. the tile prefetch).
+        const uint32_t* s32 = reinterpret_cast<const uint32_t*>(p.S);
+        uint32_t s_nxt[4];
+        auto load_scales = [&](int g) {
+            g = min(g, G - 1);
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                s_nxt[j] = s32[(s_idx[j] + g) >> 1];
+        };
+
+        uintx4 a_reg[8], w_reg[2], g_reg;
+        auto load_global = [&](int kt) {
+            const int k0 = kt * BK;
+            if (RMS)
+                g_reg = *reinterpret_cast<const uintx4*>(p.gamma + k0 + a_p * 8);
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                a_reg[i] = *reinterpret_cast<const uintx4*>(a_src[i] + k0);
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+                w_reg[i] = *reinterpret_cast<const uintx4*>(w_src[i] + (k0 >> 1));
+        };
+        auto store_lds = [&](int kt, int stage) {
+            uint8_t* base = smem + stage * STAGE_BYTES;
+            (void)kt;
+            const uintx4 g4 = g_reg;
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+            {
+                uintx4 a = a_reg[i];
+                if (RMS)
+                {
+                    // x * rstd * gamma in fp32, rounded to fp16 (the normalised activation tensor
+                    // of the unfused graph is fp16)
+                    const uint32_t av[4] = {a.x, a.y, a.z, a.w};
+                    const uint32_t gv[4] = {g4.x, g4.y, g4.z, g4.w};
+                    uint32_t ov[4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                    {
+                        half2_t x = as_half2(av[e]), g = as_half2(gv[e]);
+                        half2_t o;
+                        o.x = (half_t)((float)x.x * a_rstd[i] * (float)g.x);
+                        o.y = (half_t)((float)x.y * a_rstd[i] * (float)g.y);
+                        ov[e] = as_u32(o);
+                    }
+                    a = uintx4{ov[0], ov[1], ov[2], ov[3]};
+                }
+                *reinterpret_cast<uintx4*>(base + a_dst[i]) = permute_a8(a);
+            }
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+                *reinterpret_cast<uintx4*>(base + w_dst[i]) = w_reg[i];
+        };
+
+        const int KT = K / BK;
+        load_scales(0);
+        load_global(0);
+        store_lds(0, 0);
+        __syncthreads();
+
+        half2_t sc[4]; // group scale of this lane's column in each N tile, both halves equal
+        for (int kt = 0; kt < KT; ++kt)
+        {
+            const int stage = kt & 1;
+            if ((kt & 1) == 0)
+            {
+                const int g = kt >> 1;
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                {
+                    uint32_t bits = s_nxt[j] >> ((((uint32_t)s_idx[j] + (uint32_t)g) & 1u) << 4);
+                    half_t s = as_half2(bits).x;
+                    sc[j] = half2_t{s, s};
+                }
+                load_scales(g + 1);
+            }
+            if (kt + 1 < KT)
+                load_global(kt + 1);
+            const uint8_t* base = smem + stage * STAGE_BYTES;
+            uintx4 wq[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                wq[j] = *reinterpret_cast<const uintx4*>(base + w_frag[j]);
+#pragma unroll
+            for (int s = 0; s < 4; ++s)
+            {
+                half8_t af[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                {
+                    int pc = (h * 4 + s) ^ a_swz[i];
+                    af[i] = *reinterpret_cast<const half8_t*>(base + a_frag[i] + (pc << 4));
+                }
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                {
+                    uint32_t w = (s == 0) ? wq[j].x : (s == 1) ? wq[j].y : (s == 2) ? wq[j].z : wq[j].w;
+                    uint32_t w8 = w >> 8;
+                    half2_t q0 = as_half2((w & 0x000F000Fu) | MAGIC) + dq.c_lo;
+                    half2_t q1 = __builtin_elementwise_fma(as_half2((w & 0x00F000F0u) | MAGIC), dq.sixteenth, dq.c_hi);
+                    half2_t q2 = as_half2((w8 & 0x000F000Fu) | MAGIC) + dq.c_lo;
+                    half2_t q3 = __builtin_elementwise_fma(as_half2((w8 & 0x00F000F0u) | MAGIC), dq.sixteenth, dq.c_hi);
+                    uintx4 bw;
+                    bw.x = as_u32(q0 * sc[j]);
+                    bw.y = as_u32(q1 * sc[j]);
+                    bw.z = as_u32(q2 * sc[j]);
+                    bw.w = as_u32(q3 * sc[j]);
+                    half8_t bf = __builtin_bit_cast(half8_t, bw);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf, acc[i][j], 0, 0, 0);
+                }
+            }
+            if (kt + 1 < KT)
+                store_lds(kt + 1, stage ^ 1);
+            __syncthreads();
+        }
+
+        // ---- epilogue ---------------------------------------------------------------------------------
+        // D layout of a 32x32 tile: lane (col = l32, h), element e: row = 8*(e/4) + 4*h + (e%4)
+        constexpr int NJ = GATE ? 2 : 4;
+#pragma unroll
+        for (int j = 0; j < NJ; ++j)
+        {
+            const int n = col_out[j];
+            if (n >= p.N)
+                continue;
+            float bias = 0.f;
+            if (BIAS)
+                bias = (float)p.bias[n];
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+            {
+#pragma unroll
+                for (int e = 0; e < 16; ++e)
+                {
+                    const int m = m0 + wm * 128 + i * 32 + 8 * (e >> 2) + 4 * h + (e & 3);
+                    if (m >= p.M)
+                        continue;
+                    float v;
+                    if (GATE)
+                    {
+                        // SiLU(gate) * up on the values the unfused graph would see: both
+                        // projections rounded to fp16 first
+                        float g = (float)(half_t)acc[i][j][e];
+                        float u = (float)(half_t)acc[i][j + 2][e];
+                        v = g * (1.0f / (1.0f + __expf(-g))) * u;
+                    }
+                    else
+                    {
+                        v = acc[i][j][e];
+                    }
+                    if (BIAS)
+                        v = (float)(half_t)v + bias;
+                    if (RESID)
+                        v = (float)(half_t)v + (float)p.residual[(size_t)m * p.ldy + n];
+                    p.Y[(size_t)m * p.ldy + n] = (half_t)v;
+                }
+            }
+        }
+    }
+
+    namespace
+    {
+        template <bool GATE, bool RMS, bool BIAS, bool RESID>
+        hipError_t launch_gemm_variant(hipStream_t stream, const GemmParams& p)
+        {
+            using namespace gemm;
+            constexpr int BN_OUT = GATE ? BN / 2 : BN;
+            const int tiles_m = (p.M + BM - 1) / BM;
+            const int tiles_n = (p.N + BN_OUT - 1) / BN_OUT;
+            static bool attr_set = false;
+            if (!attr_set)
+            {
+                hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&w4a16_gemm_kernel<GATE, RMS, BIAS, RESID>),
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
+                if (e != hipSuccess)
+                    return e;
+                attr_set = true;
+            }
+            hipLaunchKernelGGL((w4a16_gemm_kernel<GATE, RMS, BIAS, RESID>), dim3(tiles_m * tiles_n), dim3(256), LDS_BYTES,
+                               stream, p);
+            return hipGetLastError();
+        }
+    } // namespace
+
+    size_t w4a16_gemm_fused_workspace(int M, bool rms)
+    {
+        return rms ? (((size_t)M * sizeof(float) + 255) & ~(size_t)255) : 0;
+    }
+
+    hipError_t launch_w4a16_gemm(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M,
+                                 int N, int K, int zp, const void* rms_gamma, float rms_eps, const void* bias,
+                                 const void* residual, int act, void* workspace)
+    {
+        GemmParams p;
+        p.A = (const half_t*)A;
+        p.Wq = (const uint8_t*)Wq;
+        p.S = (const half_t*)S;
+        p.Y = (half_t*)Y;
+        p.M = M;
+        p.N = N;
+        p.K = K;
+        p.zp = zp;
+        p.ldy = N;
+        p.up_row_offset = N; // gate rows [0,N), up rows [N,2N)
+        p.rstd = (const float*)workspace;
+        p.gamma = (const half_t*)rms_gamma;
+        p.bias = (const half_t*)bias;
+        p.residual = (const half_t*)residual;
+        const bool rms = rms_gamma != nullptr, hb = bias != nullptr, hr = residual != nullptr, gate = act == 1;
+        if (rms)
+        {
+            hipLaunchKernelGGL(rms_rstd_kernel, dim3((M + 3) / 4), dim3(256), 0, stream, (const half_t*)A,
+                               (float*)workspace, M, K, rms_eps);
+            hipError_t e = hipGetLastError();
+            if (e != hipSuccess)
+                return e;
+        }
+        // the combinations the fused entry points use; anything else is composed by the caller
+        if (gate && rms && !hb && !hr)
+            return launch_gemm_variant<true, true, false, false>(stream, p);
+        if (gate && !rms && !hb && !hr)
+            return launch_gemm_variant<true, false, false, false>(stream, p);
+        if (!gate && !rms && !hb && !hr)
+            return launch_gemm_variant<false, false, false, false>(stream, p);
+        if (!gate && !rms && !hb && hr)
+            return launch_gemm_variant<false, false, false, true>(stream, p);
+        if (!gate && !rms && hb && !hr)
+            return launch_gemm_variant<false, false, true, false>(stream, p);
+        if (!gate && !rms && hb && hr)
+            return launch_gemm_variant<false, false, true, true>(stream, p);
+        if (!gate && rms && !hb && !hr)
+            return launch_gemm_variant<false, true, false, false>(stream, p);
+        if (!gate && rms && hb && !hr)
+            return launch_gemm_variant<false, true, true, false>(stream, p);
+        return hipErrorInvalidValue;
+    }
+} // namespace nnf

@@ -116,20 +116,51 @@ int nnf_w4a16_gemm(nnf_stream_t stream, const void* A, const void* Wq, const voi
     if (st != NNF_OK)
         return st;
     const int force = nnf::g_tuning.force_path;
-    if (force != 1 && M <= 16 && nnf::w4a16_skinny_supported(M, K))
+    if ((force == 0 || force == 2) && M <= 16 && nnf::w4a16_skinny_supported(M, K))
         return (int)nnf::launch_w4a16_skinny((hipStream_t)stream, A, Wq, scales, Y, M, N, K, zp, dev.num_cu);
-    if (!nnf::w4a16_gemv_supported(M, K))
+    if (force == 1 && M <= 16 && nnf::w4a16_gemv_supported(M, K))
+        return (int)nnf::launch_w4a16_gemv((hipStream_t)stream, A, Wq, scales, Y, M, N, K, zp, dev.num_cu);
+    return (int)nnf::launch_w4a16_gemm((hipStream_t)stream, A, Wq, scales, Y, M, N, K, zp, nullptr, 0.f, nullptr,
+                                       nullptr, NNF_ACT_NONE, nullptr);
+}
+
+size_t nnf_w4a16_gemm_fused_workspace_bytes(int M, int N, int K, int group, int act)
+{
+    (void)N;
+    (void)K;
+    (void)group;
+    (void)act;
+    // room for the RMSNorm row statistics whether or not the call uses them
+    return nnf::w4a16_gemm_fused_workspace(M, true);
+}
+
+int nnf_w4a16_gemm_fused(nnf_stream_t stream, const void* A, const void* Wq, const void* scales, void* Y, int M, int N,
+                         int K, int group, int zp, const void* rms_gamma, float rms_eps, const void* bias,
+                         const void* residual, int act, void* workspace, size_t workspace_bytes)
+{
+    int st = check_w4a16(A, Wq, scales, Y, M, N, K, group, zp);
+    if (st != NNF_OK)
+        return st;
+    if (act != NNF_ACT_NONE && act != NNF_ACT_SILU_GATE)
+        return NNF_ERR_INVALID_ARGUMENT;
+    if ((rms_gamma && !aligned16(rms_gamma)) || (bias && !aligned16(bias)) || (residual && !aligned16(residual)))
+        return NNF_ERR_INVALID_ARGUMENT;
+    // combinations without a fused kernel (see launch_w4a16_gemm)
+    if (act == NNF_ACT_SILU_GATE && (bias || residual))
         return NNF_ERR_UNSUPPORTED_SHAPE;
-    return (int)nnf::launch_w4a16_gemv((hipStream_t)stream, A, Wq, scales, Y, M, N, K, zp, dev.num_cu);
+    if (rms_gamma && residual)
+        return NNF_ERR_UNSUPPORTED_SHAPE;
+    if (rms_gamma && (!workspace || workspace_bytes < nnf::w4a16_gemm_fused_workspace(M, true)))
+        return NNF_ERR_WORKSPACE_TOO_SMALL;
+    DeviceInfo dev;
+    st = current_device_info(dev);
+    if (st != NNF_OK)
+        return st;
+    return (int)nnf::launch_w4a16_gemm((hipStream_t)stream, A, Wq, scales, Y, M, N, K, zp, rms_gamma, rms_eps, bias,
+                                       residual, act, workspace);
 }
 
 // ---- entry points whose kernels are not wired yet: reject every call -------------------------
-size_t nnf_w4a16_gemm_fused_workspace_bytes(int, int, int, int, int) { return 0; }
-int nnf_w4a16_gemm_fused(nnf_stream_t, const void*, const void*, const void*, void*, int, int, int, int, int,
-                         const void*, float, const void*, const void*, int, void*, size_t)
-{
-    return NNF_ERR_UNSUPPORTED_SHAPE;
-}
 size_t nnf_w8a8_gemm_workspace_bytes(int, int, int) { return 0; }
 int nnf_w8a8_gemm(nnf_stream_t, const void*, const void*, const void*, const void*, void*, int, int, int, void*,
                   size_t)

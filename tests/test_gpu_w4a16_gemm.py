@@ -1,0 +1,202 @@
+"""Parity of the fp16 x int4 MFMA GEMM (M > 16) and its fused prologue/epilogues against the CPU oracle.
+
+Tolerance: max|y - y_ref| <= 1e-2 * RMS(y_ref) (stated by the task for the fp16 x int4 path).
+Full-size shapes are checked on a sample of output columns (the oracle GEMM of the whole matrix would
+take minutes on the host), plus size-independent properties.
+"""
+import numpy as np
+import pytest
+
+import oracle
+from nnfusion_amd import datagen
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-2
+
+
+def _t(gpu, *arrays):
+    import torch
+
+    return [None if a is None else torch.from_numpy(np.ascontiguousarray(a)).to(gpu) for a in arrays]
+
+
+def _rms(x):
+    return float(np.sqrt(np.mean(np.asarray(x, np.float64) ** 2)))
+
+
+def _check(y, ref, tol=TOL):
+    err = float(np.abs(y.astype(np.float32) - ref.astype(np.float32)).max())
+    rms = _rms(ref)
+    assert err <= tol * max(rms, 1e-6), (err, rms)
+
+
+@pytest.fixture
+def force_gemm():
+    """Route every M through the MFMA GEMM kernel (the library would pick the skinny kernel for M <= 16)."""
+    from nnfusion_amd import _lib
+
+    tune = _lib.kernels().nnf_internal_tune
+    tune(0, 3)
+    yield
+    tune(0, 0)
+
+
+@pytest.mark.parametrize("m,n,k", [
+    (128, 256, 128), (256, 256, 256), (17, 32, 128), (100, 96, 384), (300, 520, 1024),
+    (512, 1024, 2048), (257, 33, 512), (1024, 512, 4096),
+])
+def test_gemm_matches_oracle(gpu, m, n, k):
+    import torch
+
+    from nnfusion_amd import ops
+
+    print(f"case M={m} N={n} K={k}", flush=True)
+    a, wq, s = datagen.w4a16_case(0, m, n, k)
+    ta, tw, ts = _t(gpu, a, wq, s)
+    y = ops.w4a16_gemm(ta, tw, ts)
+    torch.cuda.synchronize()
+    ref = oracle.w4a16_gemm(a, wq, s, f32_out=True)
+    _check(y.cpu().numpy(), ref)
+
+
+@pytest.mark.parametrize("m", [1, 5, 16])
+def test_gemm_kernel_serves_small_m(gpu, force_gemm, m):
+    import torch
+
+    from nnfusion_amd import ops
+
+    a, wq, s = datagen.w4a16_case(4, m, 320, 512)
+    ta, tw, ts = _t(gpu, a, wq, s)
+    y = ops.w4a16_gemm(ta, tw, ts)
+    torch.cuda.synchronize()
+    _check(y.cpu().numpy(), oracle.w4a16_gemm(a, wq, s, f32_out=True))
+
+
+def test_gemm_one_hot_rows_select_weights(gpu):
+    """A = rows of the identity  =>  Y[m, n] = fp16((q[n, m] - 8) * s[n, m/128]) exactly:
+    pins nibble order, the K-slot permutation shared by the A and W fragments, and scale indexing."""
+    import torch
+
+    from nnfusion_amd import ops
+
+    n, k = 160, 256
+    _, wq, s = datagen.w4a16_case(5, 1, n, k)
+    a = np.eye(k, dtype=np.float16)
+    ta, tw, ts = _t(gpu, a, wq, s)
+    y = ops.w4a16_gemm(ta, tw, ts).cpu().numpy()
+    torch.cuda.synchronize()
+    wd = oracle.dequantize_w4(wq, s)  # [n, k]
+    np.testing.assert_array_equal(y, wd.T.astype(np.float16))
+
+
+@pytest.mark.parametrize("m,n,k", [(128, 8192, 8192), (1024, 8192, 8192), (4096, 8192, 8192)])
+def test_gemm_full_size_sampled_columns(gpu, m, n, k):
+    """configs[2] shapes: all M rows, 192 sampled output columns against the oracle; and linearity in A
+    on the whole output (Y(2A) == 2 Y(A) bit for bit, as scaling by 2 is exact outside the subnormal range)."""
+    import torch
+
+    from nnfusion_amd import ops
+
+    print(f"case M={m} N={n} K={k}", flush=True)
+    a, wq, s = datagen.w4a16_case(0, m, n, k)
+    ta, tw, ts = _t(gpu, a, wq, s)
+    y = ops.w4a16_gemm(ta, tw, ts)
+    y2 = ops.w4a16_gemm(ta * 2, tw, ts)
+    torch.cuda.synchronize()
+    rng = np.random.default_rng(0)
+    cols = np.sort(rng.choice(n, 192, replace=False))
+    ref = oracle.w4a16_gemm(a, wq[cols], s[cols], f32_out=True)
+    _check(y.cpu().numpy()[:, cols], ref)
+    # scaling by two is exact everywhere except where the fp16 result is subnormal
+    normal = y.abs() >= 2.0 ** -13
+    assert torch.equal(y2[normal], (y * 2)[normal])
+
+
+def test_fused_bias_residual(gpu):
+    import torch
+
+    from nnfusion_amd import ops
+
+    m, n, k = 200, 288, 512
+    a, wq, s = datagen.w4a16_case(6, m, n, k)
+    bias = datagen.normal_f16(6, datagen.S_BIAS, (n,))
+    res = datagen.normal_f16(6, datagen.S_RES, (m, n))
+    ta, tw, ts, tb, tr = _t(gpu, a, wq, s, bias, res)
+    y_b = ops.w4a16_gemm_fused(ta, tw, ts, bias=tb).cpu().numpy()
+    y_r = ops.w4a16_gemm_fused(ta, tw, ts, residual=tr).cpu().numpy()
+    y_br = ops.w4a16_gemm_fused(ta, tw, ts, bias=tb, residual=tr).cpu().numpy()
+    torch.cuda.synchronize()
+    d = oracle.w4a16_gemm(a, wq, s)  # fp16 tensor of the unfused Dot
+    ref_b = oracle.add_f16(d, np.broadcast_to(bias, (m, n)).copy())
+    ref_r = oracle.add_f16(d, res)
+    ref_br = oracle.add_f16(ref_b, res)
+    _check(y_b, ref_b)
+    _check(y_r, ref_r)
+    _check(y_br, ref_br)
+
+
+def test_fused_rmsnorm_prologue(gpu):
+    import torch
+
+    from nnfusion_amd import ops
+
+    m, n, k = 130, 256, 1024
+    a, wq, s = datagen.w4a16_case(7, m, n, k)
+    gamma = datagen.normal_f16(7, datagen.S_GAMMA, (k,), 1.0, 0.1)
+    ta, tw, ts, tg = _t(gpu, a, wq, s, gamma)
+    y = ops.w4a16_gemm_fused(ta, tw, ts, rms_gamma=tg, rms_eps=1e-6).cpu().numpy()
+    torch.cuda.synchronize()
+    xn = oracle.rmsnorm_f16(a, gamma, 1e-6)
+    _check(y, oracle.w4a16_gemm(xn, wq, s, f32_out=True))
+
+
+def test_fused_silu_gate(gpu):
+    import torch
+
+    from nnfusion_amd import ops
+
+    m, n, k = 150, 192, 512  # n = intermediate size; weights hold 2n rows (gate then up)
+    a, wq, s = datagen.w4a16_case(8, m, 2 * n, k)
+    ta, tw, ts = _t(gpu, a, wq, s)
+    y = ops.w4a16_gemm_fused(ta, tw, ts, act=1).cpu().numpy()
+    torch.cuda.synchronize()
+    gu = oracle.w4a16_gemm(a, wq, s)
+    g = np.ascontiguousarray(gu[:, :n])
+    u = np.ascontiguousarray(gu[:, n:])
+    ref = oracle.silu_mul_f16(g, u)
+    assert y.shape == (m, n)
+    # The stated tolerance applies to the GEMM outputs g and u: delta = 1e-2 * RMS(gu).  It is
+    # carried through h = silu(g) * u element-wise: |dh| <= |dh/dg| delta + |dh/du| delta with
+    # |dh/dg| <= 1.1 |u| and |dh/du| = |silu(g)|, plus one fp16 rounding of h.
+    delta = TOL * _rms(gu)
+    g32, u32 = g.astype(np.float32), u.astype(np.float32)
+    silu = g32 / (1.0 + np.exp(-g32))
+    bound = delta * (1.1 * np.abs(u32) + np.abs(silu)) + np.abs(ref.astype(np.float32)) * 2.0 ** -10 + 1e-6
+    err = np.abs(y.astype(np.float32) - ref.astype(np.float32))
+    assert np.all(err <= bound), float((err - bound).max())
+    # and the typical error is far smaller: RMS of the error within 1e-3 of RMS(h)
+    assert _rms(err) <= 1e-3 * _rms(ref)
+
+
+def test_rejects_bad_arguments(gpu):
+    import torch
+
+    from nnfusion_amd import ops
+
+    a, wq, s = datagen.w4a16_case(9, 4, 64, 256)
+    ta, tw, ts = _t(gpu, a, wq, s)
+    with pytest.raises(ops.NnfError) as e:
+        ops.w4a16_gemm(ta, tw, ts, zp=16)
+    assert e.value.status == -2
+    from nnfusion_amd import _lib
+
+    lib = _lib.kernels()
+    y = torch.empty((4, 64), dtype=torch.float16, device=gpu)
+    args = (ta.data_ptr(), tw.data_ptr(), ts.data_ptr(), y.data_ptr())
+    assert lib.nnf_w4a16_gemm(None, *args, 4, 64, 256, 64, 8, None, 0) == -2      # group != 128
+    assert lib.nnf_w4a16_gemm(None, *args, 4, 64, 192, 128, 8, None, 0) == -2     # K % group != 0
+    assert lib.nnf_w4a16_gemm(None, *args, 0, 64, 256, 128, 8, None, 0) == -1     # empty M
+    assert lib.nnf_w4a16_gemm(None, None, *args[1:], 4, 64, 256, 128, 8, None, 0) == -1  # null pointer
+    assert lib.nnf_w4a16_gemm(None, args[0] + 2, *args[1:], 4, 64, 256, 128, 8, None, 0) == -1  # misaligned
+    assert b"unsupported" in lib.nnf_status_string(-2)
