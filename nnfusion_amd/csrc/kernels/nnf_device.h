@@ -90,6 +90,15 @@ namespace nnf
         asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
     }
 
+    // fp32 value -> fp16, as two roundings (the value is first a rounded fp32).  Without the opaque
+    // asm the compiler folds a preceding fp32 multiply into v_fma_mixlo_f16, which rounds the exact
+    // product once, straight to fp16, and differs from the two-step result on ties.
+    __device__ __forceinline__ half_t f32_to_f16_two_step(float v)
+    {
+        asm volatile("" : "+v"(v));
+        return (half_t)v;
+    }
+
     __device__ __forceinline__ float wave_sum(float v)
     {
 #pragma unroll

@@ -28,6 +28,11 @@ namespace nnf
                                  const void* residual, int act, void* workspace);
     size_t w4a16_gemm_fused_workspace(int M, bool rms);
 
+    // W8A8: acc != nullptr writes the raw int32 accumulators, otherwise Y = fp16(acc * s_tok * s_ch).
+    hipError_t launch_w8a8(hipStream_t stream, const void* A, const void* s_tok, const void* W, const void* s_ch,
+                           void* Y, void* acc, int M, int N, int K, int num_cu);
+    bool w8a8_skinny_supported(int M, int K);
+
     // Tuning knobs for experiments (not part of the public ABI): 0 = automatic.
     struct Tuning
     {

@@ -160,22 +160,98 @@ int nnf_w4a16_gemm_fused(nnf_stream_t stream, const void* A, const void* Wq, con
                                        residual, act, workspace);
 }
 
-// ---- entry points whose kernels are not wired yet: reject every call -------------------------
-size_t nnf_w8a8_gemm_workspace_bytes(int, int, int) { return 0; }
-int nnf_w8a8_gemm(nnf_stream_t, const void*, const void*, const void*, const void*, void*, int, int, int, void*,
-                  size_t)
+// ---- W8A8 ---------------------------------------------------------------------------------------
+size_t nnf_w8a8_gemm_workspace_bytes(int M, int N, int K)
 {
-    return NNF_ERR_UNSUPPORTED_SHAPE;
+    (void)M;
+    (void)N;
+    (void)K;
+    return 0;
 }
-int nnf_w8a8_gemm_acc(nnf_stream_t, const void*, const void*, void*, int, int, int, void*, size_t)
+
+static int check_w8a8(const void* A, const void* W, const void* out, int M, int N, int K)
 {
-    return NNF_ERR_UNSUPPORTED_SHAPE;
+    if (!A || !W || !out || M <= 0 || N <= 0 || K <= 0)
+        return NNF_ERR_INVALID_ARGUMENT;
+    if (!aligned16(A) || !aligned16(W) || !aligned16(out))
+        return NNF_ERR_INVALID_ARGUMENT;
+    // rows must be whole 128-byte K tiles; the exact int32 sum needs K * 127 * 127 < 2^31
+    if (K % 128 != 0 || K > 133000)
+        return NNF_ERR_UNSUPPORTED_SHAPE;
+    return NNF_OK;
 }
-size_t nnf_fused_mlp_w4a16_workspace_bytes(int, int, int, int) { return 0; }
-int nnf_fused_mlp_w4a16(nnf_stream_t, const void*, const void*, float, const void*, const void*, const void*,
-                        const void*, void*, int, int, int, int, int, void*, size_t)
+
+int nnf_w8a8_gemm(nnf_stream_t stream, const void* A, const void* s_tok, const void* W, const void* s_ch, void* Y,
+                  int M, int N, int K, void* workspace, size_t workspace_bytes)
 {
-    return NNF_ERR_UNSUPPORTED_SHAPE;
+    (void)workspace;
+    (void)workspace_bytes;
+    int st = check_w8a8(A, W, Y, M, N, K);
+    if (st != NNF_OK)
+        return st;
+    if (!s_tok || !s_ch)
+        return NNF_ERR_INVALID_ARGUMENT;
+    DeviceInfo dev;
+    st = current_device_info(dev);
+    if (st != NNF_OK)
+        return st;
+    return (int)nnf::launch_w8a8((hipStream_t)stream, A, s_tok, W, s_ch, Y, nullptr, M, N, K, dev.num_cu);
+}
+
+int nnf_w8a8_gemm_acc(nnf_stream_t stream, const void* A, const void* W, void* acc, int M, int N, int K,
+                      void* workspace, size_t workspace_bytes)
+{
+    (void)workspace;
+    (void)workspace_bytes;
+    int st = check_w8a8(A, W, acc, M, N, K);
+    if (st != NNF_OK)
+        return st;
+    DeviceInfo dev;
+    st = current_device_info(dev);
+    if (st != NNF_OK)
+        return st;
+    return (int)nnf::launch_w8a8((hipStream_t)stream, A, nullptr, W, nullptr, nullptr, acc, M, N, K, dev.num_cu);
+}
+
+// ---- fused MLP block ------------------------------------------------------------------------------
+// workspace = [ rstd: M floats, padded to 256 B ][ h: M x I fp16 ]
+size_t nnf_fused_mlp_w4a16_workspace_bytes(int M, int H, int I, int group)
+{
+    (void)H;
+    (void)group;
+    if (M <= 0 || I <= 0)
+        return 0;
+    return nnf::w4a16_gemm_fused_workspace(M, true) + (((size_t)M * I * 2 + 255) & ~(size_t)255);
+}
+
+int nnf_fused_mlp_w4a16(nnf_stream_t stream, const void* x, const void* gamma, float eps, const void* Wgu,
+                        const void* Sgu, const void* Wd, const void* Sd, void* out, int M, int H, int I, int group,
+                        int zp, void* workspace, size_t workspace_bytes)
+{
+    if (!x || !gamma || !Wgu || !Sgu || !Wd || !Sd || !out || M <= 0 || H <= 0 || I <= 0)
+        return NNF_ERR_INVALID_ARGUMENT;
+    if (!aligned16(x) || !aligned16(gamma) || !aligned16(Wgu) || !aligned16(Sgu) || !aligned16(Wd) ||
+        !aligned16(Sd) || !aligned16(out) || !aligned16(workspace))
+        return NNF_ERR_INVALID_ARGUMENT;
+    if (group != 128 || H % group != 0 || I % group != 0 || zp < 0 || zp > 15)
+        return NNF_ERR_UNSUPPORTED_SHAPE;
+    if (!workspace || workspace_bytes < nnf_fused_mlp_w4a16_workspace_bytes(M, H, I, group))
+        return NNF_ERR_WORKSPACE_TOO_SMALL;
+    DeviceInfo dev;
+    int st = current_device_info(dev);
+    if (st != NNF_OK)
+        return st;
+    uint8_t* ws = (uint8_t*)workspace;
+    void* h = ws + nnf::w4a16_gemm_fused_workspace(M, true);
+    // h = SiLU(gate) * up, gate|up = RMSNorm(x) . Wgu^T : one kernel (after the row-statistics pre-pass)
+    hipError_t e = nnf::launch_w4a16_gemm((hipStream_t)stream, x, Wgu, Sgu, h, M, I, H, zp, gamma, eps, nullptr,
+                                          nullptr, NNF_ACT_SILU_GATE, ws);
+    if (e != hipSuccess)
+        return (int)e;
+    // out = h . Wd^T + x
+    e = nnf::launch_w4a16_gemm((hipStream_t)stream, h, Wd, Sd, out, M, H, I, zp, nullptr, 0.f, nullptr, x, NNF_ACT_NONE,
+                               nullptr);
+    return (int)e;
 }
 
 } // extern "C"

@@ -1,0 +1,84 @@
+"""W8A8 on the int8 MFMA: the int32 accumulators must be bit-identical to the CPU oracle (pure integer
+arithmetic), and the fp16 output identical to fp16((float)acc * s_tok * s_ch) evaluated left to right."""
+import numpy as np
+import pytest
+
+import oracle
+from nnfusion_amd import datagen
+
+pytestmark = pytest.mark.gpu
+
+
+def _t(gpu, *arrays):
+    import torch
+
+    return [torch.from_numpy(np.ascontiguousarray(a)).to(gpu) for a in arrays]
+
+
+@pytest.fixture(params=["auto", "mfma_gemm"])
+def path(request):
+    from nnfusion_amd import _lib
+
+    tune = _lib.kernels().nnf_internal_tune
+    tune(0, {"auto": 0, "mfma_gemm": 3}[request.param])
+    yield request.param
+    tune(0, 0)
+
+
+@pytest.mark.parametrize("m,n,k", [
+    (1, 64, 128), (1, 1000, 1024), (3, 17, 256), (16, 512, 8192), (32, 300, 512), (100, 257, 384),
+    (256, 256, 128), (512, 1024, 2048), (1, 8192, 8192), (32, 8192, 8192),
+])
+def test_accumulators_bit_exact(gpu, path, m, n, k):
+    import torch
+
+    from nnfusion_amd import ops
+
+    print(f"case M={m} N={n} K={k} path={path}", flush=True)
+    a, s_tok, w, s_ch = datagen.w8a8_case(0, m, n, k)
+    ta, tw, tst, tsc = _t(gpu, a, w, s_tok, s_ch)
+    acc = ops.w8a8_gemm_acc(ta, tw).cpu().numpy()
+    y = ops.w8a8_gemm(ta, tst, tw, tsc).cpu().numpy()
+    torch.cuda.synchronize()
+    ref = oracle.w8a8_acc(a, w)
+    assert np.array_equal(acc, ref)
+    # the epilogue is a closed form of exact inputs: bit-identical fp16
+    assert np.array_equal(y.view(np.uint16), oracle.w8a8_epilogue(ref, s_tok, s_ch).view(np.uint16))
+
+
+def test_extreme_values_do_not_overflow(gpu, path):
+    """All operands at -127 / +127 with K = 8192: |acc| = 8192 * 127^2 = 132 128 768 < 2^31."""
+    import torch
+
+    from nnfusion_amd import ops
+
+    m, n, k = 4, 48, 8192
+    a = np.full((m, k), 127, np.int8)
+    a[1] = -127
+    w = np.full((n, k), 127, np.int8)
+    w[::2] = -127
+    ta, tw = _t(gpu, a, w)
+    acc = ops.w8a8_gemm_acc(ta, tw).cpu().numpy()
+    torch.cuda.synchronize()
+    assert np.array_equal(acc, oracle.w8a8_acc(a, w))
+    assert abs(int(acc[0, 1])) == 8192 * 127 * 127
+
+
+@pytest.mark.parametrize("m", [512, 4096])
+def test_full_size_sampled(gpu, m):
+    """configs[3] at N = K = 8192: sampled output columns against the oracle bit for bit, and the
+    checksum identity  sum_n acc[m, n] == A[m, :] . (sum_n W[n, :])  over the whole output in int64."""
+    import torch
+
+    from nnfusion_amd import ops
+
+    n = k = 8192
+    print(f"case M={m}", flush=True)
+    a, s_tok, w, s_ch = datagen.w8a8_case(0, m, n, k)
+    ta, tw = _t(gpu, a, w)
+    acc = ops.w8a8_gemm_acc(ta, tw).cpu().numpy()
+    torch.cuda.synchronize()
+    cols = np.sort(np.random.default_rng(1).choice(n, 128, replace=False))
+    assert np.array_equal(acc[:, cols], oracle.w8a8_acc(a, w[cols]))
+    wsum = w.astype(np.int64).sum(axis=0)
+    assert np.array_equal(acc.astype(np.int64).sum(axis=1), a.astype(np.int64) @ wsum)
