@@ -1,0 +1,301 @@
+#!/usr/bin/env python3
+"""Benchmark of the low-bit GEMM/GEMV hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--no-extra]
+
+A "step" is one pass of the decode-shape sweep of the benchmark configuration: the four fp16 x int4
+(g128) M = 1 linear layers of a Llama-7B-like block -- (N,K) = (12288,4096) fused QKV, (4096,4096)
+O-proj, (22016,4096) gate+up, (4096,11008) down -- one launch each, through the C ABI.  To keep the
+figure an HBM figure, the weights of `layers` independent layers (same distributions, > 600 MB in
+total, more than the 256 MB last-level cache) are resident and step i uses layer i mod layers, as a
+decoder walks its layers.  Inputs are resident in HBM before the timed region; the timed region is K
+steps captured in one HIP graph (launch-bound otherwise: each kernel runs for a few microseconds),
+bracketed by synchronisation.
+
+Prints ONE JSON line.  `value` = algorithmic bytes of a step (every operand read once, output written
+once) / time per step.  `roofline` covers the kernel that dominates the step; `cpu_baseline` times the
+same sweep on the host cores with the reference's CPU GEMM (MLAS built from the reference tree, or the
+oracle's own port when that library is absent) on fp32 weights dequantised beforehand.  `extra` holds
+the other configurations (prefill GEMM, W8A8, fused MLP), each measured for a few iterations.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
+MFMA_F16_PEAK_TFLOPS = 2500.0  # dense fp16 MFMA
+MFMA_I8_PEAK_TOPS = 5000.0     # dense int8 MFMA
+
+DECODE_SHAPES = [(12288, 4096), (4096, 4096), (22016, 4096), (4096, 11008)]  # (N, K), M = 1
+GROUP = 128
+
+
+def w4a16_bytes(m, n, k):
+    """Algorithmic bytes: int4 weights + fp16 group scales + fp16 activations + fp16 output."""
+    return n * k // 2 + n * (k // GROUP) * 2 + m * k * 2 + m * n * 2
+
+
+def w8a8_bytes(m, n, k):
+    return n * k + n * 4 + m * k + m * 4 + m * n * 2
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=120)
+    ap.add_argument("--warmup", type=int, default=12)
+    ap.add_argument("--layers", type=int, default=6, help="independent weight sets walked by the steps")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extra", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU (no sharding, no collectives); use --gpus 1")
+
+    import numpy as np
+    import torch
+
+    from nnfusion_amd import _lib, datagen, ops
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    dev = torch.device("cuda:0")
+    lib = _lib.kernels()
+
+    def dev_t(a):
+        return torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+
+    # ---- resident inputs ------------------------------------------------------------------------
+    layers = []
+    host_layer0 = []
+    for layer in range(args.layers):
+        shapes = []
+        for (n, k) in DECODE_SHAPES:
+            a, wq, s = datagen.w4a16_case(layer, 1, n, k)  # seed = layer index; layer 0 is "seed 0"
+            if layer == 0:
+                host_layer0.append((a, wq, s))
+            shapes.append((dev_t(a), dev_t(wq), dev_t(s), torch.empty((1, n), dtype=torch.float16, device=dev)))
+        layers.append(shapes)
+    ws = torch.empty(1 << 20, dtype=torch.uint8, device=dev)
+
+    def launch(shape_tensors):
+        a, wq, s, y = shape_tensors
+        n, k = wq.shape[0], a.shape[1]
+        # the current stream: torch's capture stream while a graph is being recorded
+        st = lib.nnf_w4a16_gemm(torch.cuda.current_stream().cuda_stream, a.data_ptr(), wq.data_ptr(), s.data_ptr(), y.data_ptr(),
+                                1, n, k, GROUP, 8, ws.data_ptr(), ws.numel())
+        if st != 0:
+            raise RuntimeError(f"nnf_w4a16_gemm failed: {st} {lib.nnf_status_string(st).decode()}")
+
+    def step(i):
+        for sh in layers[i % args.layers]:
+            launch(sh)
+
+    def timed_graph(fn_list, reps):
+        """Capture fn_list (callables that enqueue launches) into one graph; return mean microseconds of
+        one replay over `reps` replays, measured with events on the launch stream."""
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for fn in fn_list:
+                fn()
+        g.replay()
+        torch.cuda.synchronize()
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            g.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1000.0 / reps
+
+    # ---- warm-up (untimed), then exactly K steps in the timed region ------------------------------
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        for i in range(args.steps):
+            step(i)
+    g.replay()  # graph upload, untimed
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    g.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1000.0
+    ms_per_step = e0.elapsed_time(e1) / args.steps
+    step_bytes = sum(w4a16_bytes(1, n, k) for (n, k) in DECODE_SHAPES)
+    value = step_bytes / (ms_per_step * 1e-3) / 1e9
+
+    # ---- per-shape launch durations (events around graphs of one shape walking the layers) --------
+    per_shape = []
+    for si, (n, k) in enumerate(DECODE_SHAPES):
+        def make(layer, si=si):
+            return lambda: launch(layers[layer][si])
+        fns = [make(layer % args.layers) for layer in range(4 * args.layers)]
+        us = timed_graph(fns, 10) / len(fns)
+        per_shape.append({"N": n, "K": k, "us": round(us, 3), "GB/s": round(w4a16_bytes(1, n, k) / us / 1e3, 1),
+                          "frac_hbm": round(w4a16_bytes(1, n, k) / us / 1e3 / HBM_PEAK_GBS, 4)})
+    # dominant kernel: the K = 4096 instantiation of the skinny kernel serves three of the four launches
+    k4096 = [p for p in per_shape if p["K"] == 4096]
+    dom_us = sum(p["us"] for p in k4096) / len(k4096)
+    dom_bytes = sum(w4a16_bytes(1, p["N"], p["K"]) for p in k4096) / len(k4096)
+    roofline = {
+        "bound": "hbm",
+        "kernel": "nnf::w4a16_skinny_kernel (K=4096 instantiation; mean over its three launches per step)",
+        "achieved": round(dom_bytes / dom_us / 1e3, 1),
+        "peak": HBM_PEAK_GBS,
+        "unit": "GB/s",
+        "frac": round(dom_bytes / dom_us / 1e3 / HBM_PEAK_GBS, 4),
+        "traffic": None,
+        "bytes_per_launch": int(dom_bytes),
+        "us_per_launch": round(dom_us, 3),
+    }
+
+    extra = {}
+    if not args.no_extra:
+        extra = run_extra(torch, np, dev, lib, datagen, ops)
+
+    cpu_baseline = None
+    if not args.no_cpu_baseline:
+        cpu_baseline = run_cpu_baseline(np, host_layer0, step_bytes)
+
+    out = {
+        "metric": "fp16xint4 g128 decode GEMV sweep, HBM GB/s (algorithmic bytes / time), M=1, 1 MI355X",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 6),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "config": {
+            "workload": "configs[1]: decode-shape sweep M=1, (N,K) in (12288,4096),(4096,4096),(22016,4096),"
+                        "(4096,11008), fp16 x int4 g128 zp8",
+            "layers_resident": args.layers,
+            "bytes_per_step": step_bytes,
+            "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
+            "timed_region_wall_ms": round(wall_ms, 3),
+        },
+        "per_shape": per_shape,
+        "roofline": roofline,
+        "cpu_baseline": cpu_baseline,
+        "extra": extra,
+    }
+    print(json.dumps(out))
+
+
+def run_extra(torch, np, dev, lib, datagen, ops):
+    """The other benchmark configurations, a few iterations each (not part of `value`)."""
+
+    def dev_t(a):
+        return torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+
+    def time_us(fn, iters):
+        for _ in range(2):
+            fn()
+        torch.cuda.synchronize()
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(iters):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1000.0 / iters
+
+    res = {}
+    # configs[2]: fp16 x int4 GEMM, N = K = 8192
+    n = k = 8192
+    _, wq, s = datagen.w4a16_case(0, 1, n, k)
+    twq, ts = dev_t(wq), dev_t(s)
+    ws = torch.empty(1 << 24, dtype=torch.uint8, device=dev)
+    rows = []
+    for m in (16, 128, 1024, 4096):
+        a = dev_t(datagen.normal_f16(0, datagen.S_ACT, (m, k)))
+        y = torch.empty((m, n), dtype=torch.float16, device=dev)
+        us = time_us(lambda: ops.w4a16_gemm(a, twq, ts, out=y, workspace=ws), 20 if m <= 1024 else 8)
+        fl = 2.0 * m * n * k
+        rows.append({"M": m, "us": round(us, 2), "TFLOP/s": round(fl / us / 1e6, 1),
+                     "frac_mfma_f16": round(fl / us / 1e6 / MFMA_F16_PEAK_TFLOPS, 4),
+                     "GB/s": round(w4a16_bytes(m, n, k) / us / 1e3, 1)})
+    res["w4a16_gemm_N8192_K8192"] = rows
+    del twq, ts
+    # configs[3]: W8A8, N = K = 8192
+    _, _, w8, s_ch = datagen.w8a8_case(0, 1, n, k)
+    tw8, tsch = dev_t(w8), dev_t(s_ch)
+    rows = []
+    for m in (1, 32, 512, 4096):
+        a8 = dev_t(datagen.uniform_i8(0, datagen.S_A8, (m, k)))
+        st = dev_t(datagen.uniform_f32(0, datagen.S_STOK, (m,), 0.001, 0.01))
+        y = torch.empty((m, n), dtype=torch.float16, device=dev)
+        us = time_us(lambda: ops.w8a8_gemm(a8, st, tw8, tsch, out=y, workspace=ws), 20 if m <= 512 else 8)
+        op = 2.0 * m * n * k
+        rows.append({"M": m, "us": round(us, 2), "TOP/s": round(op / us / 1e6, 1),
+                     "frac_mfma_i8": round(op / us / 1e6 / MFMA_I8_PEAK_TOPS, 4),
+                     "GB/s": round(w8a8_bytes(m, n, k) / us / 1e3, 1)})
+    res["w8a8_gemm_N8192_K8192"] = rows
+    del tw8, tsch
+    # configs[4]: fused MLP block, M = 256
+    m, h, i = 256, 4096, 11008
+    tens = [dev_t(t) for t in datagen.mlp_case(0, m, h, i)]
+    out = torch.empty((m, h), dtype=torch.float16, device=dev)
+    wsz = lib.nnf_fused_mlp_w4a16_workspace_bytes(m, h, i, GROUP)
+    wsm = torch.empty(wsz, dtype=torch.uint8, device=dev)
+    us = time_us(lambda: ops.fused_mlp_w4a16(*tens, out=out, workspace=wsm), 20)
+    fl = 2.0 * m * (2 * i) * h + 2.0 * m * h * i
+    res["fused_mlp_M256_4096_11008"] = {"us": round(us, 2), "TFLOP/s": round(fl / us / 1e6, 1),
+                                        "frac_mfma_f16": round(fl / us / 1e6 / MFMA_F16_PEAK_TFLOPS, 4)}
+    return res
+
+
+def run_cpu_baseline(np, host_layer0, step_bytes):
+    """The reference's CPU path for the same sweep, on this host's cores: fp32 GEMM on weights
+    dequantised once beforehand (constants are folded at init in the reference), 5 warm-ups + 100
+    timed calls per shape (the loop of the generated CPU main_test)."""
+    import oracle
+
+    use_ref = oracle.mlas_ref() is not None
+    total_ms = 0.0
+    detail = []
+    for (a, wq, s) in host_layer0:
+        wd = oracle.dequantize_w4(wq, s)
+        a32 = oracle.f16_to_f32(a)
+        if use_ref:
+            mean_ms, min_ms = oracle.mlas_time_sgemm_nt(a32, wd, warmup=5, iters=100)
+        else:
+            mean_ms, min_ms = oracle.time_dot_f32(a32, wd, warmup=5, iters=100, threads=16)
+        total_ms += mean_ms
+        detail.append({"N": int(wq.shape[0]), "K": int(a.shape[1]), "mean_ms": round(mean_ms, 4),
+                       "min_ms": round(min_ms, 4)})
+        del wd
+    cores = os.cpu_count() or 1
+    threads = min(16, cores)  # MLAS caps its own partitioning at 16 threads
+    return {
+        "value": round(step_bytes / (total_ms * 1e-3) / 1e9, 3),
+        "unit": "GB/s",
+        "cores": threads,
+        "kind": "reference" if use_ref else "port",
+        "sample": "the whole sweep (4 shapes, layer 0): 5 warm-up + 100 timed fp32 GEMM calls per shape on "
+                  "weights dequantised once (untimed); value = int4-path algorithmic bytes / summed mean time",
+        "ms_per_step": round(total_ms, 4),
+        "host_cpus": cores,
+        "per_shape": detail,
+    }
+
+
+if __name__ == "__main__":
+    main()

@@ -214,6 +214,7 @@ void oracle_f32_to_f16(const float* in, uint16_t* out, size_t n)
 void oracle_dequantize_w4(const uint8_t* wq, const uint16_t* scales, int N, int K, int group, int zp, float* out)
 {
     const int G = K / group;
+#pragma omp parallel for schedule(static)
     for (int n = 0; n < N; ++n)
         for (int k = 0; k < K; ++k)
         {

@@ -1,0 +1,59 @@
+"""The C-ABI library loads (no GPU needed for that) and exports every function include/*.h declares."""
+import ctypes
+import glob
+import os
+import re
+
+from nnfusion_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_functions():
+    names = []
+    for path in glob.glob(os.path.join(ROOT, "include", "*.h")):
+        text = open(path).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        text = re.sub(r"//[^\n]*", "", text)
+        # a declaration: <type> nnf_name( ... );
+        names += re.findall(r"\b(nnf_[a-z0-9_]+)\s*\(", text)
+    return sorted(set(names))
+
+
+def test_header_declares_the_expected_entry_points():
+    names = _declared_functions()
+    for must in ("nnf_w4a16_gemm", "nnf_w4a16_gemm_workspace_bytes", "nnf_w4a16_gemm_fused", "nnf_w8a8_gemm",
+                 "nnf_w8a8_gemm_acc", "nnf_fused_mlp_w4a16", "nnf_status_string", "nnf_abi_version"):
+        assert must in names
+
+
+def test_library_exports_every_declared_symbol():
+    lib = ctypes.CDLL(_lib.KERNELS_SO)
+    missing = [n for n in _declared_functions() if not hasattr(lib, n)]
+    assert not missing, missing
+
+
+def test_ctypes_table_covers_the_header():
+    assert sorted(_lib.KERNEL_ABI) == _declared_functions()
+
+
+def test_pure_host_queries_work_without_a_gpu():
+    lib = _lib.kernels()
+    assert lib.nnf_abi_version() == 1
+    assert lib.nnf_status_string(0) == b"ok"
+    assert b"workspace" in lib.nnf_status_string(-3)
+    assert lib.nnf_w4a16_gemm_workspace_bytes(1, 4096, 4096, 128) == 0
+    m, h, i = 256, 4096, 11008
+    assert lib.nnf_fused_mlp_w4a16_workspace_bytes(m, h, i, 128) >= m * i * 2 + m * 4
+    # argument checks come before any device access
+    assert lib.nnf_w4a16_gemm(None, None, None, None, None, 1, 1, 128, 128, 8, None, 0) == -1
+    assert lib.nnf_w8a8_gemm_acc(None, None, None, None, 1, 1, 128, None, 0) == -1
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    import pytest
+
+    monkeypatch.setattr(_lib, "KERNELS_SO", str(tmp_path / "nope.so"))
+    monkeypatch.setattr(_lib, "_kernels", None)
+    with pytest.raises(_lib.NativeLibraryMissing):
+        _lib.kernels()
