@@ -1,0 +1,177 @@
+// Kernel emitters of the quantized operators for ROCM_GPU.  Each emits a host function whose body is
+// one call into the gfx950 launcher library (include/nnf_hip_kernels.h) -- the slot where the
+// reference's cuda::Dot emits a cuBLAS call (src/nnfusion/core/kernels/cuda_gpu/kernels/dot.cpp:128-205).
+// Shapes are written into the body as literals: the code generator de-duplicates kernel definitions by
+// signature + body text, so two layers with different N or K must not share a body.
+// Registered with TypeConstraint(element::f32) because kernel selection always looks up that key
+// (src/nnfusion/engine/pass/graph/kernel_selection.cpp:185-187) and with a priority above every Dot
+// emitter of the reference (2); an unsupported node is declined by returning nullptr.
+#include "../../nnf_workspace.h"
+#include "nnfusion/core/kernels/hip_gpu/hip_emitter.hpp"
+#include "nnfusion/core/kernels/kernel_registration.hpp"
+#include "nnfusion/core/operators/generic_op/generic_op.hpp"
+
+#include <iomanip>
+
+namespace nnfusion
+{
+    namespace kernels
+    {
+        namespace hip
+        {
+            namespace
+            {
+                std::string float_literal(double v)
+                {
+                    std::ostringstream ss;
+                    ss << std::scientific << std::setprecision(9) << v << "f";
+                    return ss.str();
+                }
+            } // namespace
+
+            class QuantDot : public HipLibEmitter
+            {
+            public:
+                explicit QuantDot(std::shared_ptr<KernelContext> ctx)
+                    : HipLibEmitter(ctx)
+                {
+                }
+
+                LanguageUnit_p emit_function_body() override
+                {
+                    auto gop = std::dynamic_pointer_cast<op::GenericOp>(m_context->op);
+                    if (!gop)
+                        return nullptr;
+                    auto& cfg = gop->localOpConfig.getRoot();
+                    const int group = cfg["group_size"].get<int>();
+                    const int zp = cfg["zero_point"].get<int>();
+                    const bool rms = cfg["rms_norm"].get<bool>();
+                    const bool has_bias = cfg["has_bias"].get<bool>();
+                    const bool has_res = cfg["has_residual"].get<bool>();
+                    const bool gate = cfg["act"].get<std::string>() == "silu_gate";
+                    // what the launcher supports; anything else is left to other emitters
+                    if (cfg["bits"].get<int>() != 4 || group != 128 || !cfg["transpose_B"].get<bool>())
+                        return nullptr;
+                    if (m_context->inputs[0]->get_element_type() != element::f16 ||
+                        m_context->inputs[2]->get_element_type() != element::f16)
+                        return nullptr;
+                    if (gate && (has_bias || has_res))
+                        return nullptr;
+                    if (rms && has_res)
+                        return nullptr;
+                    const Shape& a = m_context->inputs[0]->get_shape();
+                    const Shape& w = m_context->inputs[1]->get_shape();
+                    const size_t K = a.back();
+                    const size_t M = shape_size(a) / K;
+                    const size_t N = gate ? w[0] / 2 : w[0];
+                    if (K % 128 != 0 || M == 0 || N == 0)
+                        return nullptr;
+
+                    size_t idx = 3;
+                    std::string gamma = "nullptr", bias = "nullptr", residual = "nullptr";
+                    if (rms)
+                        gamma = "input" + std::to_string(idx++);
+                    if (has_bias)
+                        bias = "input" + std::to_string(idx++);
+                    if (has_res)
+                        residual = "input" + std::to_string(idx++);
+
+                    const bool fused = rms || has_bias || has_res || gate;
+                    const size_t ws_bytes = fused ? nnf::workspace::w4a16_gemm_fused((int)M, (int)N, (int)K, group, gate)
+                                                  : nnf::workspace::w4a16_gemm((int)M, (int)N, (int)K, group);
+                    std::string ws = "nullptr";
+                    if (ws_bytes > 0)
+                        ws = allocate_tensor(Shape{ws_bytes}, element::character)->get_name();
+
+                    LanguageUnit_p lu(new LanguageUnit(get_function_name()));
+                    if (!fused)
+                    {
+                        *lu << "NNF_HIP_CHECK(nnf_w4a16_gemm(stream, input0, input1, input2, output0, " << M << ", " << N
+                            << ", " << K << ", " << group << ", " << zp << ", " << ws << ", " << ws_bytes << "));\n";
+                    }
+                    else
+                    {
+                        *lu << "NNF_HIP_CHECK(nnf_w4a16_gemm_fused(stream, input0, input1, input2, output0, " << M << ", "
+                            << N << ", " << K << ", " << group << ", " << zp << ", " << gamma << ", "
+                            << float_literal(cfg["rms_eps"].get<double>()) << ", " << bias << ", " << residual << ", "
+                            << (gate ? "NNF_ACT_SILU_GATE" : "NNF_ACT_NONE") << ", " << ws << ", " << ws_bytes
+                            << "));\n";
+                    }
+                    return lu;
+                }
+            };
+
+            class QuantDotW8A8 : public HipLibEmitter
+            {
+            public:
+                explicit QuantDotW8A8(std::shared_ptr<KernelContext> ctx)
+                    : HipLibEmitter(ctx)
+                {
+                }
+
+                LanguageUnit_p emit_function_body() override
+                {
+                    auto gop = std::dynamic_pointer_cast<op::GenericOp>(m_context->op);
+                    if (!gop)
+                        return nullptr;
+                    const Shape& a = m_context->inputs[0]->get_shape();
+                    const Shape& w = m_context->inputs[2]->get_shape();
+                    const size_t M = a[0], K = a[1], N = w[0];
+                    if (K % 128 != 0 || K > 133000 || M == 0 || N == 0)
+                        return nullptr;
+                    const bool raw = gop->localOpConfig.getRoot()["out_type"].get<std::string>() == "i32";
+                    LanguageUnit_p lu(new LanguageUnit(get_function_name()));
+                    if (raw)
+                        *lu << "NNF_HIP_CHECK(nnf_w8a8_gemm_acc(stream, input0, input2, output0, " << M << ", " << N << ", "
+                            << K << ", nullptr, 0));\n";
+                    else
+                        *lu << "NNF_HIP_CHECK(nnf_w8a8_gemm(stream, input0, input1, input2, input3, output0, " << M << ", "
+                            << N << ", " << K << ", nullptr, 0));\n";
+                    return lu;
+                }
+            };
+
+            class FusedQuantMLP : public HipLibEmitter
+            {
+            public:
+                explicit FusedQuantMLP(std::shared_ptr<KernelContext> ctx)
+                    : HipLibEmitter(ctx)
+                {
+                }
+
+                LanguageUnit_p emit_function_body() override
+                {
+                    auto gop = std::dynamic_pointer_cast<op::GenericOp>(m_context->op);
+                    if (!gop)
+                        return nullptr;
+                    auto& cfg = gop->localOpConfig.getRoot();
+                    const int group = cfg["group_size"].get<int>();
+                    const int zp = cfg["zero_point"].get<int>();
+                    const Shape& x = m_context->inputs[0]->get_shape();
+                    const size_t M = x[0], H = x[1], I = m_context->inputs[2]->get_shape()[0] / 2;
+                    if (group != 128 || H % 128 != 0 || I % 128 != 0 || M == 0)
+                        return nullptr;
+                    const size_t ws_bytes = nnf::workspace::fused_mlp_w4a16((int)M, (int)H, (int)I, group);
+                    // the only intermediate that reaches HBM: h [M, I] fp16 (plus M row statistics)
+                    auto ws = allocate_tensor(Shape{ws_bytes}, element::character);
+                    LanguageUnit_p lu(new LanguageUnit(get_function_name()));
+                    *lu << "NNF_HIP_CHECK(nnf_fused_mlp_w4a16(stream, input0, input1, "
+                        << float_literal(cfg["rms_eps"].get<double>()) << ", input2, input3, input4, input5, output0, " << M
+                        << ", " << H << ", " << I << ", " << group << ", " << zp << ", " << ws->get_name() << ", "
+                        << ws_bytes << "));\n";
+                    return lu;
+                }
+            };
+        } // namespace hip
+
+        REGISTER_KERNEL_EMITTER("QuantDot",
+                                Device(ROCM_GPU).TypeConstraint(element::f32).Tag("nnf_hip_gfx950").Priority(5),
+                                hip::QuantDot)
+        REGISTER_KERNEL_EMITTER("QuantDotW8A8",
+                                Device(ROCM_GPU).TypeConstraint(element::f32).Tag("nnf_hip_gfx950").Priority(5),
+                                hip::QuantDotW8A8)
+        REGISTER_KERNEL_EMITTER("FusedQuantMLP",
+                                Device(ROCM_GPU).TypeConstraint(element::f32).Tag("nnf_hip_gfx950").Priority(5),
+                                hip::FusedQuantMLP)
+    } // namespace kernels
+} // namespace nnfusion

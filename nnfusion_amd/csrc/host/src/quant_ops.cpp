@@ -1,0 +1,114 @@
+// The quantized operators, declared through the operator-plugin interface (REGISTER_OP / GenericOp,
+// precedent: src/nnfusion/core/operators/generic_op/generic_op_define/MatMulAdd.cpp:6-35).
+// They are GenericOps, not op::Dot: Dot's validation merges the element types of its two inputs and
+// rejects fp16 x u8 (src/nnfusion/core/operators/op_define/dot.cpp:47-53).
+//
+//   QuantDot       inputs: A f16 [M,K], Wq u8 [N,K/2] (int4 x2) , S f16 [N,K/group]
+//                          [, gamma f16 [K]] [, bias f16 [N]] [, residual f16 [M,N]]   (in this order, by attribute)
+//                  attrs : bits 4, group_size 128, zero_point 8, transpose_B true,
+//                          rms_norm false, rms_eps 1e-6, has_bias false, has_residual false, act "none"|"silu_gate"
+//                  output: Y f16 [M, N]   (N = rows of Wq; half of them when act == "silu_gate")
+//   QuantDotW8A8   inputs: A i8 [M,K], s_tok f32 [M], W i8 [N,K], s_ch f32 [N];  attr out_type "f16"|"i32"
+//                  output: Y f16 [M,N] = fp16((float)acc * s_tok * s_ch), or the raw i32 accumulators
+//   FusedQuantMLP  inputs: x f16 [M,H], gamma f16 [H], Wgu u8 [2I,H/2], Sgu f16 [2I,H/g], Wd u8 [H,I/2], Sd f16 [H,I/g]
+//                  attrs : group_size 128, zero_point 8, rms_eps 1e-6
+//                  output: out f16 [M,H] = x + Wd . (SiLU(Wg . n) * (Wu . n)), n = RMSNorm(x)
+#include "nnfusion/core/operators/generic_op/generic_op.hpp"
+
+using namespace nnfusion;
+
+namespace
+{
+    int int_attr(std::shared_ptr<op::GenericOp> gop, const std::string& key)
+    {
+        return gop->localOpConfig.getRoot()[key].get<int>();
+    }
+    bool bool_attr(std::shared_ptr<op::GenericOp> gop, const std::string& key)
+    {
+        return gop->localOpConfig.getRoot()[key].get<bool>();
+    }
+} // namespace
+
+REGISTER_OP(QuantDot)
+    .attr<int>("bits", 4)
+    .attr<int>("group_size", 128)
+    .attr<int>("zero_point", 8)
+    .attr<bool>("transpose_B", true)
+    .attr<bool>("rms_norm", false)
+    .attr<double>("rms_eps", 1e-6)
+    .attr<bool>("has_bias", false)
+    .attr<bool>("has_residual", false)
+    .attr<std::string>("act", "none")
+    .constrait([](const op::OpConfig::any& config) -> bool {
+        if (config.at("bits").get<int>() != 4)
+            return false;
+        int zp = config.at("zero_point").get<int>();
+        if (zp < 0 || zp > 15 || config.at("group_size").get<int>() <= 0)
+            return false;
+        auto act = config.at("act").get<std::string>();
+        return act == "none" || act == "silu_gate";
+    })
+    .infershape([](std::shared_ptr<graph::GNode> gnode) -> void {
+        auto gop = std::dynamic_pointer_cast<op::GenericOp>(gnode->get_op_ptr());
+        NNFUSION_CHECK_NOT_NULLPTR(gop);
+        size_t expect = 3 + (bool_attr(gop, "rms_norm") ? 1 : 0) + (bool_attr(gop, "has_bias") ? 1 : 0) +
+                        (bool_attr(gop, "has_residual") ? 1 : 0);
+        OP_VALIDATION(gop, gnode->get_input_size() == expect) << "expected " << expect << " inputs";
+        const Shape& a = gnode->get_input_shape(0);
+        const Shape& w = gnode->get_input_shape(1);
+        const Shape& s = gnode->get_input_shape(2);
+        OP_VALIDATION(gop, a.size() >= 1 && w.size() == 2 && s.size() == 2) << "bad ranks";
+        OP_VALIDATION(gop, gnode->get_input_element_type(1) == element::u8) << "packed int4 weights travel as u8";
+        const size_t K = a.back();
+        const size_t group = (size_t)int_attr(gop, "group_size");
+        OP_VALIDATION(gop, w[1] * 2 == K) << "Wq must be [N, K/2]";
+        OP_VALIDATION(gop, K % group == 0 && s[0] == w[0] && s[1] == K / group) << "scales must be [N, K/group]";
+        size_t N = w[0];
+        if (gop->localOpConfig.getRoot()["act"].get<std::string>() == "silu_gate")
+        {
+            OP_VALIDATION(gop, N % 2 == 0) << "gate|up weights need an even row count";
+            N /= 2;
+        }
+        Shape out(a.begin(), a.end() - 1);
+        out.push_back(N);
+        gnode->set_output_type_and_shape(0, gnode->get_input_element_type(0), out);
+    });
+
+REGISTER_OP(QuantDotW8A8)
+    .attr<std::string>("out_type", "f16")
+    .constrait([](const op::OpConfig::any& config) -> bool {
+        auto t = config.at("out_type").get<std::string>();
+        return t == "f16" || t == "i32";
+    })
+    .infershape([](std::shared_ptr<graph::GNode> gnode) -> void {
+        auto gop = std::dynamic_pointer_cast<op::GenericOp>(gnode->get_op_ptr());
+        NNFUSION_CHECK_NOT_NULLPTR(gop);
+        OP_VALIDATION(gop, gnode->get_input_size() == 4) << "inputs: A, s_tok, W, s_ch";
+        const Shape& a = gnode->get_input_shape(0);
+        const Shape& w = gnode->get_input_shape(2);
+        OP_VALIDATION(gop, a.size() == 2 && w.size() == 2 && a[1] == w[1]) << "A [M,K], W [N,K]";
+        OP_VALIDATION(gop, gnode->get_input_element_type(0) == element::i8 &&
+                               gnode->get_input_element_type(2) == element::i8)
+            << "int8 operands";
+        OP_VALIDATION(gop, shape_size(gnode->get_input_shape(1)) == a[0] && shape_size(gnode->get_input_shape(3)) == w[0])
+            << "one scale per token and per output channel";
+        bool raw = gop->localOpConfig.getRoot()["out_type"].get<std::string>() == "i32";
+        gnode->set_output_type_and_shape(0, raw ? element::i32 : element::f16, Shape{a[0], w[0]});
+    });
+
+REGISTER_OP(FusedQuantMLP)
+    .attr<int>("group_size", 128)
+    .attr<int>("zero_point", 8)
+    .attr<double>("rms_eps", 1e-6)
+    .infershape([](std::shared_ptr<graph::GNode> gnode) -> void {
+        auto gop = std::dynamic_pointer_cast<op::GenericOp>(gnode->get_op_ptr());
+        NNFUSION_CHECK_NOT_NULLPTR(gop);
+        OP_VALIDATION(gop, gnode->get_input_size() == 6) << "inputs: x, gamma, Wgu, Sgu, Wd, Sd";
+        const Shape& x = gnode->get_input_shape(0);
+        const Shape& wgu = gnode->get_input_shape(2);
+        const Shape& wd = gnode->get_input_shape(4);
+        OP_VALIDATION(gop, x.size() == 2 && wgu.size() == 2 && wd.size() == 2) << "bad ranks";
+        const size_t H = x[1], I = wgu[0] / 2;
+        OP_VALIDATION(gop, wgu[1] * 2 == H && wd[0] == H && wd[1] * 2 == I && wgu[0] % 2 == 0) << "shape mismatch";
+        gnode->set_output_type_and_shape(0, gnode->get_input_element_type(0), x);
+    });

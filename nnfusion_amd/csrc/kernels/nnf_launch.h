@@ -22,11 +22,10 @@ namespace nnf
     bool w4a16_skinny_supported(int M, int K);
 
     // MFMA GEMM (any M) with the fused RMSNorm prologue and bias / residual / SiLU-gate epilogues.
-    // workspace: w4a16_gemm_fused_workspace(M, rms) bytes (the per-row rstd of the RMSNorm).
+    // workspace: M floats (the per-row rstd), needed when rms_gamma != nullptr.
     hipError_t launch_w4a16_gemm(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M,
                                  int N, int K, int zp, const void* rms_gamma, float rms_eps, const void* bias,
                                  const void* residual, int act, void* workspace);
-    size_t w4a16_gemm_fused_workspace(int M, bool rms);
 
     // W8A8: acc != nullptr writes the raw int32 accumulators, otherwise Y = fp16(acc * s_tok * s_ch).
     hipError_t launch_w8a8(hipStream_t stream, const void* A, const void* s_tok, const void* W, const void* s_ch,

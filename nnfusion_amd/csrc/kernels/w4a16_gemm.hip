@@ -394,11 +394,6 @@ namespace nnf
         }
     } // namespace
 
-    size_t w4a16_gemm_fused_workspace(int M, bool rms)
-    {
-        return rms ? (((size_t)M * sizeof(float) + 255) & ~(size_t)255) : 0;
-    }
-
     hipError_t launch_w4a16_gemm(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M,
                                  int N, int K, int zp, const void* rms_gamma, float rms_eps, const void* bias,
                                  const void* residual, int act, void* workspace)

@@ -2,6 +2,7 @@
 // Declarations and the contract of each entry point are in include/nnf_hip_kernels.h.
 #include "nnf_hip_kernels.h"
 #include "kernels/nnf_launch.h"
+#include "nnf_workspace.h"
 
 #include <hip/hip_runtime.h>
 
@@ -95,11 +96,7 @@ const char* nnf_status_string(int status)
 
 size_t nnf_w4a16_gemm_workspace_bytes(int M, int N, int K, int group)
 {
-    (void)M;
-    (void)N;
-    (void)K;
-    (void)group;
-    return 0;
+    return nnf::workspace::w4a16_gemm(M, N, K, group);
 }
 
 int nnf_w4a16_gemm(nnf_stream_t stream, const void* A, const void* Wq, const void* scales, void* Y, int M, int N,
@@ -126,12 +123,8 @@ int nnf_w4a16_gemm(nnf_stream_t stream, const void* A, const void* Wq, const voi
 
 size_t nnf_w4a16_gemm_fused_workspace_bytes(int M, int N, int K, int group, int act)
 {
-    (void)N;
-    (void)K;
-    (void)group;
-    (void)act;
     // room for the RMSNorm row statistics whether or not the call uses them
-    return nnf::w4a16_gemm_fused_workspace(M, true);
+    return nnf::workspace::w4a16_gemm_fused(M, N, K, group, act);
 }
 
 int nnf_w4a16_gemm_fused(nnf_stream_t stream, const void* A, const void* Wq, const void* scales, void* Y, int M, int N,
@@ -150,7 +143,7 @@ int nnf_w4a16_gemm_fused(nnf_stream_t stream, const void* A, const void* Wq, con
         return NNF_ERR_UNSUPPORTED_SHAPE;
     if (rms_gamma && residual)
         return NNF_ERR_UNSUPPORTED_SHAPE;
-    if (rms_gamma && (!workspace || workspace_bytes < nnf::w4a16_gemm_fused_workspace(M, true)))
+    if (rms_gamma && (!workspace || workspace_bytes < nnf::workspace::rms_rows(M)))
         return NNF_ERR_WORKSPACE_TOO_SMALL;
     DeviceInfo dev;
     st = current_device_info(dev);
@@ -163,10 +156,7 @@ int nnf_w4a16_gemm_fused(nnf_stream_t stream, const void* A, const void* Wq, con
 // ---- W8A8 ---------------------------------------------------------------------------------------
 size_t nnf_w8a8_gemm_workspace_bytes(int M, int N, int K)
 {
-    (void)M;
-    (void)N;
-    (void)K;
-    return 0;
+    return nnf::workspace::w8a8_gemm(M, N, K);
 }
 
 static int check_w8a8(const void* A, const void* W, const void* out, int M, int N, int K)
@@ -217,11 +207,7 @@ int nnf_w8a8_gemm_acc(nnf_stream_t stream, const void* A, const void* W, void* a
 // workspace = [ rstd: M floats, padded to 256 B ][ h: M x I fp16 ]
 size_t nnf_fused_mlp_w4a16_workspace_bytes(int M, int H, int I, int group)
 {
-    (void)H;
-    (void)group;
-    if (M <= 0 || I <= 0)
-        return 0;
-    return nnf::w4a16_gemm_fused_workspace(M, true) + (((size_t)M * I * 2 + 255) & ~(size_t)255);
+    return nnf::workspace::fused_mlp_w4a16(M, H, I, group);
 }
 
 int nnf_fused_mlp_w4a16(nnf_stream_t stream, const void* x, const void* gamma, float eps, const void* Wgu,
@@ -242,7 +228,7 @@ int nnf_fused_mlp_w4a16(nnf_stream_t stream, const void* x, const void* gamma, f
     if (st != NNF_OK)
         return st;
     uint8_t* ws = (uint8_t*)workspace;
-    void* h = ws + nnf::w4a16_gemm_fused_workspace(M, true);
+    void* h = ws + nnf::workspace::rms_rows(M);
     // h = SiLU(gate) * up, gate|up = RMSNorm(x) . Wgu^T : one kernel (after the row-statistics pre-pass)
     hipError_t e = nnf::launch_w4a16_gemm((hipStream_t)stream, x, Wgu, Sgu, h, M, I, H, zp, gamma, eps, nullptr,
                                           nullptr, NNF_ACT_SILU_GATE, ws);

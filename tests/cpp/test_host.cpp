@@ -1,0 +1,523 @@
+// Host-side unit tests (no GPU): the kernel plugin API restated from the reference -- registry,
+// selection order, decline-by-nullptr, naming, the f32 lookup key -- exercised with fake emitters, the
+// quantized operators' shape inference, the text the quantized emitters produce, the code generator's
+// hook order and output, and the single-kernel harness source.  Run by tests/test_host_cpp.py; prints one
+// line per case and exits non-zero on the first failure of any case.
+#include "nnfusion/core/kernels/hip_gpu/hip_emitter.hpp"
+#include "nnfusion/core/kernels/kernel_registration.hpp"
+#include "nnfusion/core/operators/generic_op/generic_op.hpp"
+#include "nnfusion/engine/pass/codegen/base_codegen_pass.hpp"
+#include "nnfusion/engine/pass/graph/kernel_selection.hpp"
+#include "nnfusion/engine/profiler/hip_runtime.hpp"
+
+#include <cstdio>
+#include <cstdlib>
+#include <fstream>
+
+using namespace nnfusion;
+using namespace nnfusion::kernels;
+
+static int g_failures = 0;
+static std::string g_case;
+
+#define EXPECT(cond)                                                                                           \
+    do                                                                                                         \
+    {                                                                                                          \
+        if (!(cond))                                                                                           \
+        {                                                                                                      \
+            printf("FAIL %s: %s (line %d)\n", g_case.c_str(), #cond, __LINE__);                                \
+            ++g_failures;                                                                                      \
+        }                                                                                                      \
+    } while (0)
+
+#define CONTAINS(text, needle) EXPECT((text).find(needle) != std::string::npos)
+
+template <typename F>
+void run_case(const std::string& name, F f)
+{
+    g_case = name;
+    int before = g_failures;
+    try
+    {
+        f();
+    }
+    catch (const std::exception& e)
+    {
+        printf("FAIL %s: exception %s\n", name.c_str(), e.what());
+        ++g_failures;
+    }
+    if (g_failures == before)
+        printf("PASS %s\n", name.c_str());
+}
+
+// ---- fake operator and emitters ----------------------------------------------------------------
+REGISTER_OP(FakeOp).attr<int>("answer", 42).infershape([](std::shared_ptr<graph::GNode> gnode) -> void {
+    gnode->set_output_type_and_shape(0, gnode->get_input_element_type(0), gnode->get_input_shape(0));
+});
+
+namespace
+{
+    std::vector<std::string> g_emit_log;
+
+    class FakeEmitter : public KernelEmitter
+    {
+    public:
+        FakeEmitter(std::shared_ptr<KernelContext> ctx, const std::string& type, const std::string& label, bool declines)
+            : KernelEmitter(ctx, type)
+            , m_label(label)
+            , m_declines(declines)
+        {
+        }
+        LanguageUnit_p emit_function_body() override
+        {
+            g_emit_log.push_back(m_label);
+            if (m_declines)
+                return nullptr;
+            LanguageUnit_p lu(new LanguageUnit(get_function_name()));
+            *lu << "// body of " << m_label << "\n";
+            return lu;
+        }
+        LanguageUnit_p emit_dependency() override
+        {
+            LanguageUnit_p lu(new LanguageUnit(get_function_name() + "_dep"));
+            lu->require(header::stdio);
+            return lu;
+        }
+        std::string m_label;
+        bool m_declines;
+    };
+
+    struct RocmLow : FakeEmitter { RocmLow(std::shared_ptr<KernelContext> c) : FakeEmitter(c, "rocm", "rocm_p2", false) {} };
+    struct RocmHighDeclines : FakeEmitter { RocmHighDeclines(std::shared_ptr<KernelContext> c) : FakeEmitter(c, "rocm", "rocm_p7_declines", true) {} };
+    struct CudaMid : FakeEmitter { CudaMid(std::shared_ptr<KernelContext> c) : FakeEmitter(c, "cuda", "cuda_p3", false) {} };
+    struct CudaSame : FakeEmitter { CudaSame(std::shared_ptr<KernelContext> c) : FakeEmitter(c, "cuda", "cuda_p2", false) {} };
+    struct F16Only : FakeEmitter { F16Only(std::shared_ptr<KernelContext> c) : FakeEmitter(c, "rocm", "rocm_f16_p9", false) {} };
+    struct CpuOnly : FakeEmitter { CpuOnly(std::shared_ptr<KernelContext> c) : FakeEmitter(c, "cpu", "cpu_p9", false) {} };
+} // namespace
+
+REGISTER_KERNEL_EMITTER("FakeOp", Device(ROCM_GPU).TypeConstraint(element::f32).Tag("low").Priority(2), RocmLow)
+REGISTER_KERNEL_EMITTER("FakeOp", Device(ROCM_GPU).TypeConstraint(element::f32).Tag("high").Priority(7), RocmHighDeclines)
+REGISTER_KERNEL_EMITTER("FakeOp", Device(CUDA_GPU).TypeConstraint(element::f32).Tag("mid").Priority(3), CudaMid)
+REGISTER_KERNEL_EMITTER("FakeOp", Device(CUDA_GPU).TypeConstraint(element::f32).Tag("same").Priority(2), CudaSame)
+REGISTER_KERNEL_EMITTER("FakeOp", Device(ROCM_GPU).TypeConstraint(element::f16).Tag("f16").Priority(9), F16Only)
+REGISTER_KERNEL_EMITTER("FakeOp", Device(GENERIC_CPU).TypeConstraint(element::f32).Tag("cpu").Priority(9), CpuOnly)
+
+namespace
+{
+    std::shared_ptr<graph::GNode> param(graph::Graph& g, const element::Type& t, const Shape& s)
+    {
+        return g.add_node_and_edge(std::make_shared<op::Parameter>(t, s), graph::GNodeVector{});
+    }
+
+    std::shared_ptr<graph::GNode> quant_dot_graph(graph::Graph& g, size_t M, size_t N, size_t K, const std::string& cfg = "",
+                                                  bool with_gamma = false, bool with_bias = false, bool with_res = false,
+                                                  size_t rows_mul = 1)
+    {
+        auto a = param(g, element::f16, Shape{M, K});
+        auto w = param(g, element::u8, Shape{N * rows_mul, K / 2});
+        auto s = param(g, element::f16, Shape{N * rows_mul, K / 128});
+        graph::GNodeVector in{a, w, s};
+        if (with_gamma)
+            in.push_back(param(g, element::f16, Shape{K}));
+        if (with_bias)
+            in.push_back(param(g, element::f16, Shape{N}));
+        if (with_res)
+            in.push_back(param(g, element::f16, Shape{M, N}));
+        auto config = cfg.empty() ? op::OpConfig::any() : op::OpConfig::any::parse(cfg);
+        return g.add_node_and_edge(std::make_shared<op::GenericOp>("qd", "QuantDot", config), in);
+    }
+
+    std::string read_file(const std::string& path)
+    {
+        std::ifstream f(path);
+        std::stringstream ss;
+        ss << f.rdbuf();
+        return ss.str();
+    }
+} // namespace
+
+int main(int argc, char** argv)
+{
+    const std::string tmp = argc > 1 ? argv[1] : "/tmp/nnf_host_test";
+
+    run_case("element_types", [] {
+        EXPECT(element::f16.c_type_string() == "half" && element::f16.size() == 2);
+        EXPECT(element::u8.c_type_string() == "uint8_t" && element::u8.is_quantized() && !element::u8.is_signed());
+        EXPECT(element::i8.c_type_string() == "int8_t" && element::i8.is_quantized());
+        EXPECT(element::f32.c_type_string() == "float" && element::f32.is_real());
+        element::Type merged;
+        EXPECT(!element::Type::merge(merged, element::f16, element::u8)); // why a quantized Dot cannot be op::Dot
+        EXPECT(element::Type::merge(merged, element::f16, element::f16) && merged == element::f16);
+        EXPECT(get_device_str(ROCM_GPU) == "ROCM_GPU" && (int)ROCM_GPU == 1 && get_device_type("ROCm") == ROCM_GPU);
+    });
+
+    run_case("language_units", [] {
+        LanguageUnit_p h(new LanguageUnit("header::a", "#include <a>\n"));
+        LanguageUnit_p m(new LanguageUnit("macro::b", "#define B\n"));
+        LanguageUnit_p d(new LanguageUnit("declaration::c", "typedef int c;\n"));
+        LanguageUnit_p body(new LanguageUnit("body", "body();\n"));
+        body->require(d);
+        body->require(m);
+        body->require(h);
+        EXPECT(body->collect_code() == "#include <a>\n#define B\ntypedef int c;\nbody();\n");
+        EXPECT(body->required.count("macro::b") == 1);
+        body->clean_require();
+        EXPECT(body->collect_code() == "body();\n");
+        LanguageUnit w("w");
+        w << "if (x)\n";
+        w.block_begin();
+        w << "y();\n";
+        w.block_end();
+        EXPECT(w.get_code() == "if (x)\n{\n    y();\n}\n");
+        FunctionUnit fu;
+        fu.name_unit = LanguageUnit_p(new LanguageUnit("n", "my_kernel"));
+        fu.signature_unit = LanguageUnit_p(new LanguageUnit("s", "void (float* input0, float* output0)"));
+        fu.call_unit = LanguageUnit_p(new LanguageUnit("c", "(a, b);\n"));
+        EXPECT(fu.get_specialized_signature() == "void my_kernel(float* input0, float* output0)");
+        EXPECT(fu.get_specialized_function_call() == "my_kernel(a, b);\n");
+        EXPECT(fu.get_specialized_function_call("other") == "other(a, b);\n");
+    });
+
+    run_case("json_lite", [] {
+        auto j = json_lite::parse("{\"group\": 128, \"eps\": 1e-6, \"act\": \"silu_gate\", \"flag\": true, \"v\": [1, 2, 3]}");
+        EXPECT(j["group"].get<int>() == 128 && j["flag"].get<bool>() && j["act"].get<std::string>() == "silu_gate");
+        EXPECT(j["eps"].get<double>() == 1e-6 && j["v"].size() == 3 && j["v"][2].get<int>() == 3);
+        EXPECT(json_lite::parse(j.dump()).dump() == j.dump());
+        bool threw = false;
+        try
+        {
+            json_lite::parse("{\"a\": }");
+        }
+        catch (const CheckError&)
+        {
+            threw = true;
+        }
+        EXPECT(threw);
+    });
+
+    run_case("registry_lookup", [] {
+        auto* reg = KernelRegistry::Global();
+        EXPECT(reg->FindKernelRegistrations("FakeOp", ROCM_GPU, element::f32).size() == 2);
+        EXPECT(reg->FindKernelRegistrations("FakeOp", CUDA_GPU, element::f32).size() == 2);
+        EXPECT(reg->FindKernelRegistrations("FakeOp", ROCM_GPU, element::f16).size() == 1);
+        EXPECT(reg->FindKernelRegistrations("NoSuchOp", ROCM_GPU, element::f32).empty());
+        auto best = reg->FindKernelRegistration("FakeOp", ROCM_GPU, element::f32);
+        EXPECT(best && best->m_tag == "high" && best->m_priority == 7);
+        EXPECT(reg->FindKernelRegistrations("QuantDot", ROCM_GPU, element::f32).size() == 1);
+        EXPECT(reg->FindKernelRegistrations("QuantDotW8A8", ROCM_GPU, element::f32).size() == 1);
+        EXPECT(reg->FindKernelRegistrations("FusedQuantMLP", ROCM_GPU, element::f32).size() == 1);
+        bool threw = false;
+        try
+        {
+            Name("Broken").Device(ROCM_GPU).Build(); // no factory
+        }
+        catch (const CheckError&)
+        {
+            threw = true;
+        }
+        EXPECT(threw);
+    });
+
+    run_case("selection_order_and_decline", [] {
+        graph::Graph g;
+        auto x = param(g, element::f16, Shape{2, 3}); // fp16 node: the lookup key is still element::f32
+        auto node = g.add_node_and_edge(std::make_shared<op::GenericOp>("fake", "FakeOp", op::OpConfig::any()), {x});
+        pass::graph::DefaultKernelSelector sel;
+        g_emit_log.clear();
+        auto ans = sel.pick_first(node, ROCM_GPU);
+        EXPECT(ans.second != nullptr);
+        // candidates: rocm_p7 (7+1, declines), cuda_p3 (3), rocm_p2 (2+1), cuda_p2 (2): tie 3 vs 3 broken by
+        // kernel type string "cuda" < "rocm"
+        EXPECT(g_emit_log.size() == 2 && g_emit_log[0] == "rocm_p7_declines" && g_emit_log[1] == "cuda_p3");
+        auto* won = dynamic_cast<FakeEmitter*>(ans.second.get());
+        EXPECT(won && won->m_label == "cuda_p3");
+        EXPECT(ans.second->get_device_type() == CUDA_GPU && ans.first == ROCM_GPU);
+        // the f16 registration (priority 9) and the CPU one are never candidates for a ROCm node
+        for (auto& l : g_emit_log)
+            EXPECT(l != "rocm_f16_p9" && l != "cpu_p9");
+        // on a CUDA node only CUDA registrations are looked at
+        g_emit_log.clear();
+        auto ans2 = sel.pick_first(node, CUDA_GPU);
+        EXPECT(dynamic_cast<FakeEmitter*>(ans2.second.get())->m_label == "cuda_p3" && g_emit_log.size() == 1);
+        // no registration at all
+        auto ans3 = sel.pick_first(node, HLSL);
+        EXPECT(ans3.second == nullptr);
+    });
+
+    run_case("emitter_name_signature_call", [] {
+        graph::Graph g;
+        auto x = param(g, element::f16, Shape{2, 3});
+        auto node = g.add_node_and_edge(std::make_shared<op::GenericOp>("fake", "FakeOp", op::OpConfig::any()), {x});
+        auto ctx = std::make_shared<KernelContext>(node);
+        EXPECT(ctx->dtypes.size() == 2 && ctx->dtypes[0] == "half" && ctx->gpu_num_sm == 20);
+        EXPECT(ctx->generate_identifier() == "FakeOp_i2x3_o2x3_half_half");
+        RocmLow k(ctx);
+        auto fu = k.get_or_emit_source();
+        EXPECT(fu != nullptr && k.is_emitted());
+        const std::string uname = node->get_op_ptr()->get_unique_name();
+        EXPECT(fu->name_unit->get_code() == "FakeOp_half_half_rocm_" + uname);
+        EXPECT(fu->signature_unit->get_code() == "void (half* input0, half* output0)");
+        EXPECT(fu->call_unit->get_code() == "(" + x->get_output_tensor_ptr(0)->get_name() + ", " +
+                                                node->get_output_tensor_ptr(0)->get_name() + ");\n");
+        // body requires dep, call requires body (orders headers before kernels)
+        EXPECT(fu->body_unit->required.count(fu->dep_unit->symbol) == 1);
+        EXPECT(fu->call_unit->required.count(fu->body_unit->symbol) == 1);
+        CONTAINS(fu->comment_unit->get_code(), "// Description:\tFakeOp");
+        // second call returns the same unit; with emit_func_call the call unit is rebuilt
+        auto before = fu->call_unit;
+        EXPECT(k.get_or_emit_source() == fu && fu->call_unit == before);
+        EXPECT(k.get_or_emit_source(true) == fu && fu->call_unit != before);
+        RocmHighDeclines d(ctx);
+        EXPECT(d.get_or_emit_source() == nullptr);
+    });
+
+    run_case("quant_dot_infershape", [] {
+        graph::Graph g;
+        auto n = quant_dot_graph(g, 1, 4096, 4096);
+        EXPECT(n->get_output_shape(0) == (Shape{1, 4096}) && n->get_output_element_type(0) == element::f16);
+        graph::Graph g2;
+        auto n2 = quant_dot_graph(g2, 256, 11008, 4096, "{\"act\": \"silu_gate\", \"rms_norm\": true}", true, false, false, 2);
+        EXPECT(n2->get_output_shape(0) == (Shape{256, 11008}));
+        // wrong scale shape, wrong packing, wrong input count, bad attribute
+        auto expect_throw = [](std::function<void()> f) {
+            bool threw = false;
+            try
+            {
+                f();
+            }
+            catch (const CheckError&)
+            {
+                threw = true;
+            }
+            return threw;
+        };
+        EXPECT(expect_throw([] {
+            graph::Graph g3;
+            auto a = param(g3, element::f16, Shape{1, 256});
+            auto w = param(g3, element::u8, Shape{8, 128});
+            auto s = param(g3, element::f16, Shape{8, 1}); // K/group = 2 expected
+            g3.add_node_and_edge(std::make_shared<op::GenericOp>("x", "QuantDot", op::OpConfig::any()), {a, w, s});
+        }));
+        EXPECT(expect_throw([] {
+            graph::Graph g3;
+            auto a = param(g3, element::f16, Shape{1, 256});
+            auto w = param(g3, element::u8, Shape{8, 256}); // not K/2
+            auto s = param(g3, element::f16, Shape{8, 2});
+            g3.add_node_and_edge(std::make_shared<op::GenericOp>("x", "QuantDot", op::OpConfig::any()), {a, w, s});
+        }));
+        EXPECT(expect_throw([] {
+            graph::Graph g3;
+            quant_dot_graph(g3, 1, 8, 256, "{\"has_bias\": true}"); // bias input missing
+        }));
+        EXPECT(expect_throw([] {
+            graph::Graph g3;
+            quant_dot_graph(g3, 1, 8, 256, "{\"zero_point\": 16}");
+        }));
+        EXPECT(expect_throw([] {
+            graph::Graph g3;
+            quant_dot_graph(g3, 1, 8, 256, "{\"act\": \"gelu\"}");
+        }));
+    });
+
+    run_case("quant_dot_emitter_text", [] {
+        graph::Graph g;
+        auto n = quant_dot_graph(g, 1, 12288, 4096);
+        pass::graph::DefaultKernelSelector sel;
+        auto ans = sel.pick_first(n, ROCM_GPU);
+        EXPECT(ans.second != nullptr && ans.second->get_kernel_type() == "rocm");
+        auto fu = ans.second->get_or_emit_source();
+        EXPECT(fu->name_unit->get_code() == "QuantDot_half_uint8_t_half_half_rocm_" + n->get_op_ptr()->get_unique_name());
+        EXPECT(fu->signature_unit->get_code() == "void (hipStream_t stream, half* input0, uint8_t* input1, half* input2, half* output0)");
+        EXPECT(fu->body_unit->get_code() ==
+               "NNF_HIP_CHECK(nnf_w4a16_gemm(stream, input0, input1, input2, output0, 1, 12288, 4096, 128, 8, nullptr, 0));\n");
+        // the signature asks for a stream, so the call starts with one
+        CONTAINS(fu->call_unit->get_code(), "(0, ");
+        std::string deps = fu->dep_unit->collect_required_code();
+        CONTAINS(deps, "#include <hip/hip_runtime.h>");
+        CONTAINS(deps, "#include \"nnf_hip_kernels.h\"");
+        CONTAINS(deps, "#define NNF_HIP_CHECK(x)");
+        CONTAINS(deps, "typedef _Float16 half;");
+        EXPECT(deps.find("cuda") == std::string::npos && deps.find("cublas") == std::string::npos);
+
+        // fused variant: gamma, bias; scratch tensor for the row statistics appears in signature and call
+        graph::Graph g2;
+        auto n2 = quant_dot_graph(g2, 256, 4096, 4096, "{\"rms_norm\": true, \"has_bias\": true, \"rms_eps\": 1e-5}", true, true);
+        auto k2 = sel.pick_first(n2, ROCM_GPU).second;
+        auto fu2 = k2->get_or_emit_source();
+        CONTAINS(fu2->body_unit->get_code(), "nnf_w4a16_gemm_fused(stream, input0, input1, input2, output0, 256, 4096, 4096, 128, 8, input3, 1.000000000e-05f, input4, nullptr, NNF_ACT_NONE, ");
+        EXPECT(k2->m_context->tensors.size() == 1 && k2->m_context->tensors[0]->size() == 1024);
+        CONTAINS(fu2->signature_unit->get_code(), "char* " + k2->m_context->tensors[0]->get_name());
+        CONTAINS(fu2->call_unit->get_code(), k2->m_context->tensors[0]->get_name() + ");");
+        // SiLU gate: N is half the weight rows
+        graph::Graph g3;
+        auto n3 = quant_dot_graph(g3, 256, 11008, 4096, "{\"act\": \"silu_gate\"}", false, false, false, 2);
+        CONTAINS(sel.pick_first(n3, ROCM_GPU).second->get_or_emit_source()->body_unit->get_code(),
+                 "256, 11008, 4096, 128, 8, nullptr, 1.000000000e-06f, nullptr, nullptr, NNF_ACT_SILU_GATE");
+    });
+
+    run_case("quant_dot_emitter_declines", [] {
+        pass::graph::DefaultKernelSelector sel;
+        {
+            graph::Graph g; // group 64 is a legal op, but this emitter does not serve it
+            auto a = param(g, element::f16, Shape{1, 256});
+            auto w = param(g, element::u8, Shape{8, 128});
+            auto s = param(g, element::f16, Shape{8, 4});
+            auto n = g.add_node_and_edge(std::make_shared<op::GenericOp>("x", "QuantDot", op::OpConfig::any::parse("{\"group_size\": 64}")),
+                                         {a, w, s});
+            EXPECT(sel.pick_first(n, ROCM_GPU).second == nullptr);
+        }
+        {
+            graph::Graph g; // fp32 activations
+            auto a = param(g, element::f32, Shape{1, 256});
+            auto w = param(g, element::u8, Shape{8, 128});
+            auto s = param(g, element::f16, Shape{8, 2});
+            auto n = g.add_node_and_edge(std::make_shared<op::GenericOp>("x", "QuantDot", op::OpConfig::any()), {a, w, s});
+            EXPECT(sel.pick_first(n, ROCM_GPU).second == nullptr);
+        }
+        {
+            graph::Graph g; // gate + bias has no fused kernel
+            auto n = quant_dot_graph(g, 4, 8, 256, "{\"act\": \"silu_gate\", \"has_bias\": true}", false, true, false, 2);
+            EXPECT(sel.pick_first(n, ROCM_GPU).second == nullptr);
+        }
+        {
+            graph::Graph g; // a CUDA node finds no emitter for this op
+            auto n = quant_dot_graph(g, 1, 8, 256);
+            EXPECT(sel.pick_first(n, CUDA_GPU).second == nullptr);
+        }
+    });
+
+    run_case("w8a8_and_mlp_emitters", [] {
+        pass::graph::DefaultKernelSelector sel;
+        graph::Graph g;
+        auto a = param(g, element::i8, Shape{32, 8192});
+        auto st = param(g, element::f32, Shape{32});
+        auto w = param(g, element::i8, Shape{8192, 8192});
+        auto sc = param(g, element::f32, Shape{8192});
+        auto n = g.add_node_and_edge(std::make_shared<op::GenericOp>("q", "QuantDotW8A8", op::OpConfig::any()), {a, st, w, sc});
+        EXPECT(n->get_output_element_type(0) == element::f16 && n->get_output_shape(0) == (Shape{32, 8192}));
+        auto fu = sel.pick_first(n, ROCM_GPU).second->get_or_emit_source();
+        EXPECT(fu->body_unit->get_code() ==
+               "NNF_HIP_CHECK(nnf_w8a8_gemm(stream, input0, input1, input2, input3, output0, 32, 8192, 8192, nullptr, 0));\n");
+        auto n2 = g.add_node_and_edge(std::make_shared<op::GenericOp>("q", "QuantDotW8A8", op::OpConfig::any::parse("{\"out_type\": \"i32\"}")),
+                                      {a, st, w, sc});
+        EXPECT(n2->get_output_element_type(0) == element::i32);
+        CONTAINS(sel.pick_first(n2, ROCM_GPU).second->get_or_emit_source()->body_unit->get_code(),
+                 "nnf_w8a8_gemm_acc(stream, input0, input2, output0, 32, 8192, 8192");
+
+        graph::Graph g2;
+        auto x = param(g2, element::f16, Shape{256, 4096});
+        auto gamma = param(g2, element::f16, Shape{4096});
+        auto wgu = param(g2, element::u8, Shape{22016, 2048});
+        auto sgu = param(g2, element::f16, Shape{22016, 32});
+        auto wd = param(g2, element::u8, Shape{4096, 5504});
+        auto sd = param(g2, element::f16, Shape{4096, 86});
+        auto mlp = g2.add_node_and_edge(std::make_shared<op::GenericOp>("mlp", "FusedQuantMLP", op::OpConfig::any()),
+                                        {x, gamma, wgu, sgu, wd, sd});
+        EXPECT(mlp->get_output_shape(0) == (Shape{256, 4096}));
+        auto k = sel.pick_first(mlp, ROCM_GPU).second;
+        auto fm = k->get_or_emit_source();
+        CONTAINS(fm->body_unit->get_code(), "nnf_fused_mlp_w4a16(stream, input0, input1, 1.000000000e-06f, input2, input3, input4, input5, output0, 256, 4096, 11008, 128, 8, ");
+        // h [256, 11008] fp16 + 256 floats, each padded to 256 bytes
+        EXPECT(k->m_context->tensors.size() == 1 && k->m_context->tensors[0]->size() == 1024 + 256 * 11008 * 2);
+    });
+
+    run_case("codegen_project", [&] {
+        auto g = std::make_shared<graph::Graph>();
+        auto a = param(*g, element::f16, Shape{4, 256});
+        std::vector<uint8_t> wbytes(16 * 128, 0x98);
+        std::vector<uint16_t> sbytes(16 * 2, 0x2000);
+        auto w = g->add_node_and_edge(std::make_shared<op::Constant>(element::u8, Shape{16, 128}, wbytes.data()), graph::GNodeVector{});
+        auto s = g->add_node_and_edge(std::make_shared<op::Constant>(element::f16, Shape{16, 2}, sbytes.data()), graph::GNodeVector{});
+        // two layers with identical shapes share one definition; a third with another N gets its own
+        auto l1 = g->add_node_and_edge(std::make_shared<op::GenericOp>("l1", "QuantDot", op::OpConfig::any()), {a, w, s});
+        auto l2 = g->add_node_and_edge(std::make_shared<op::GenericOp>("l2", "QuantDot", op::OpConfig::any()), {a, w, s});
+        std::vector<uint8_t> w2bytes(32 * 128, 0x77);
+        std::vector<uint16_t> s2bytes(32 * 2, 0x2000);
+        auto w2 = g->add_node_and_edge(std::make_shared<op::Constant>(element::u8, Shape{32, 128}, w2bytes.data()), graph::GNodeVector{});
+        auto s2 = g->add_node_and_edge(std::make_shared<op::Constant>(element::f16, Shape{32, 2}, s2bytes.data()), graph::GNodeVector{});
+        auto l3 = g->add_node_and_edge(std::make_shared<op::GenericOp>("l3", "QuantDot", op::OpConfig::any()), {a, w2, s2});
+        auto r1 = g->add_node_and_edge(std::make_shared<op::Result>(), {l1});
+        auto r2 = g->add_node_and_edge(std::make_shared<op::Result>(), {l2});
+        auto r3 = g->add_node_and_edge(std::make_shared<op::Result>(), {l3});
+        (void)r1; (void)r2; (void)r3;
+
+        ROCmEngine engine(tmp + "/codegen_project/");
+        engine.pass.exit_after_codegen = false;
+        engine.pass.kernels_include_dir = "/inc";
+        engine.pass.kernels_lib_dir = "/lib";
+        EXPECT(engine.run_on_graph(g));
+        auto& trace = engine.pass.hook_trace;
+        std::vector<std::string> expected{"initialize", "collect_mem", "collect_stream", "collect_funcs", "modify_codegen", "codegen", "after_projgen"};
+        EXPECT(trace == expected);
+        EXPECT((*l1)["Kernel_Selection_Result"].is_valid() && (*l1)["DeviceType"].as<NNFusion_DeviceType>() == ROCM_GPU);
+
+        std::string rt = read_file(tmp + "/codegen_project/nnfusion_rt.cpp");
+        std::string hdr = read_file(tmp + "/codegen_project/nnfusion_rt.h");
+        std::string mk = read_file(tmp + "/codegen_project/Makefile");
+        std::string pj = read_file(tmp + "/codegen_project/para_info.json");
+        std::string mt = read_file(tmp + "/codegen_project/main_test.cpp");
+        EXPECT(!rt.empty() && !hdr.empty() && !mk.empty() && !pj.empty() && !mt.empty());
+        // headers before macros before declarations before code
+        size_t p_h = rt.find("#include <hip/hip_runtime.h>"), p_m = rt.find("#define NNF_HIP_CHECK"), p_d = rt.find("typedef _Float16 half;"),
+               p_k = rt.find("void QuantDot_half_uint8_t_half_half_rocm_");
+        EXPECT(p_h != std::string::npos && p_h < p_m && p_m < p_d && p_d < p_k);
+        // l1 and l2: one definition, two calls; l3: its own definition
+        size_t defs = 0, pos = 0;
+        while ((pos = rt.find("\nvoid QuantDot_half_uint8_t_half_half_rocm_", pos)) != std::string::npos)
+        {
+            ++defs;
+            ++pos;
+        }
+        EXPECT(defs == 2);
+        const std::string f1 = "QuantDot_half_uint8_t_half_half_rocm_" + l1->get_op_ptr()->get_unique_name();
+        size_t calls = 0;
+        pos = 0;
+        while ((pos = rt.find(f1 + "(nnf_stream_0, ", pos)) != std::string::npos)
+        {
+            ++calls;
+            ++pos;
+        }
+        EXPECT(calls == 2);
+        CONTAINS(rt, "extern \"C\" int kernel_entry(half* " + a->get_output_tensor_ptr(0)->get_name());
+        CONTAINS(rt, "extern \"C\" void rocm_init()");
+        CONTAINS(rt, "extern \"C\" void cuda_init()");
+        CONTAINS(rt, "extern \"C\" int get_device_type()\n{\n    return 1;");
+        CONTAINS(rt, "nnf_load_constant((void**)&" + w->get_output_tensor_ptr(0)->get_name() + ", \"./Constant/" +
+                         w->get_output_tensor_ptr(0)->get_name() + ".bin\", 2048);");
+        CONTAINS(rt, "nnf_w4a16_gemm(stream, input0, input1, input2, output0, 4, 16, 256, 128, 8, nullptr, 0)");
+        CONTAINS(rt, "nnf_w4a16_gemm(stream, input0, input1, input2, output0, 4, 32, 256, 128, 8, nullptr, 0)");
+        // results are written in place: the producing tensor aliases the caller's buffer
+        CONTAINS(rt, "half* " + l1->get_output_tensor_ptr(0)->get_name() + " = " + r1->get_output_tensor_ptr(0)->get_name() + ";");
+        // HIP text only
+        for (const char* banned : {"cuda_runtime", "cublas", "cudnn", "hipify", "rocm_adapter", "__global__"})
+            EXPECT(rt.find(banned) == std::string::npos);
+        CONTAINS(hdr, "extern \"C\" int64_t get_workspace_size();");
+        CONTAINS(mk, "--offload-arch=gfx950");
+        CONTAINS(mk, "NNF_INC ?= /inc");
+        CONTAINS(pj, "\"shape\": [4, 256]");
+        CONTAINS(mt, "Summary: [min, max, mean]");
+        std::string cbin = read_file(tmp + "/codegen_project/Constant/" + w->get_output_tensor_ptr(0)->get_name() + ".bin");
+        EXPECT(cbin.size() == 2048 && (uint8_t)cbin[0] == 0x98);
+    });
+
+    run_case("profiler_harness_source", [&] {
+        graph::Graph g;
+        auto n = quant_dot_graph(g, 2, 64, 256);
+        pass::graph::DefaultKernelSelector sel;
+        auto k = sel.pick_first(n, ROCM_GPU).second;
+        auto pc = std::make_shared<profiler::ProfilingContext>(k);
+        pc->warmup_times = 2;
+        pc->runtime_times = 7;
+        profiler::HipDefaultRuntime rt("/inc", "/lib");
+        EXPECT(rt.codegen(pc));
+        EXPECT(pc->entry_name == k->get_function_name() + "_entry");
+        CONTAINS(pc->source_code, "extern \"C\" double " + pc->entry_name + "(void** args, void** outputs)");
+        CONTAINS(pc->source_code, "(half*)args[0], (uint8_t*)args[1], (half*)args[2], (half*)outputs[0]");
+        CONTAINS(pc->source_code, "for (size_t i = 0; i < 7; ++i)");
+        CONTAINS(pc->source_code, "return (double)ms / 7;");
+        CONTAINS(pc->source_code, "hipMemcpyHostToDevice");
+    });
+
+    printf("%s (%d failure%s)\n", g_failures ? "FAILED" : "OK", g_failures, g_failures == 1 ? "" : "s");
+    return g_failures ? 1 : 0;
+}
