@@ -19,7 +19,7 @@ namespace nnf
     hipError_t launch_w4a16_skinny(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M,
                                    int N, int K, int zp, int num_cu);
     // true when one workgroup can hold the activations (M <= 16 rows of K) in LDS
-    bool w4a16_skinny_supported(int M, int K);
+    bool w4a16_skinny_supported(int M, int N, int K);
 
     // MFMA GEMM (any M) with the fused RMSNorm prologue and bias / residual / SiLU-gate epilogues.
     // workspace: M floats (the per-row rstd), needed when rms_gamma != nullptr.
