@@ -13,8 +13,8 @@
 //     -- per-lane scale loads would double the number of memory requests of the kernel;
 //   * the dot products run on v_mfma_f32_16x16x32_f16 with the weight tile as the B operand
 //     (columns = n) and the M <= 16 activation rows as the A operand (rows = m), so the cost per
-//     weight byte does not depend on M.  The A operand lives in registers (K <= 4096: 16 VGPRs per
-//     group) or in LDS (larger K);
+//     weight byte does not depend on M.  The A operand is staged once per workgroup in LDS (already
+//     permuted and pre-scaled); with up to two groups per wavefront it is then kept in registers;
 //   * nibbles are turned into fp16 with one v_and_or_b32 per pair: (q | 0x6400) = 1024 + q, and a
 //     nibble four bits up gives 1024 + 16 q.  Instead of subtracting the 1024 / zero point from
 //     every weight, the activations of the "16 q" slots are pre-divided by 16 and the constant part
@@ -34,7 +34,7 @@
 namespace nnf
 {
     // LDS, in this order:
-    //   [A_REGS == false] activations as 16-byte units  unit(c, j, kq, m) = ((c*4 + j)*4 + kq)*M + m  holding
+    //   activations as 16-byte units  unit(c, j, kq, m) = ((c*4 + j)*4 + kq)*M + m  holding
     //       the eight fp16  a[m][c*128 + kq*32 + j*8 + {0,4,1,5,2,6,3,7}]  with slots 2,3,6,7 (odd k) times 1/16
     //   scales   sc[2][16 rows][G] fp16 (as in memory), each copy padded to 16 bytes
     //   red      [2][KS][16 m][16 n] fp32 partial tiles
@@ -57,7 +57,7 @@ namespace nnf
         const int col = lane & 15; // n within the tile (B operand / D column), m for the A operand
         const int kq = lane >> 4;  // K quarter of the MFMA (A/B operands), row quad of D
         const int G = K >> 7;
-        const int a_units = A_REGS ? 0 : G * 16 * M;
+        const int a_units = G * 16 * M;
         const int sc_units = (16 * G * 2 + 15) >> 4; // 16-byte units of one scale copy
         uintx4* sc_lds = lds + a_units;
         float* red = reinterpret_cast<float*>(sc_lds + 2 * sc_units); // [2][KS][16][16]
@@ -116,34 +116,24 @@ namespace nnf
             a.w = as_u32(as_half2(a.w) * sixteenth);
             return a;
         };
-        uintx4 areg[A_REGS ? CPS : 1][4];
-        int a_unit[H][CPS];
-        if (A_REGS)
+        // Staged once per workgroup (one coalesced 16-byte load per thread and unit); every wavefront
+        // loading its own operand straight from global memory would cost 8 load instructions per
+        // wavefront, almost all of whose lanes are redundant.
+        for (int u = tid; u < a_units; u += blockDim.x)
         {
+            int m = u % M;
+            int rest = u / M;
+            int q = rest & 3;
+            int j = (rest >> 2) & 3;
+            int c = rest >> 4;
+            lds[u] = prep_a(*reinterpret_cast<const uintx4*>(A + (size_t)m * K + (c << 7) + (q << 5) + (j << 3)));
+        }
+        int a_unit[H][CPS];
+#pragma unroll
+        for (int h = 0; h < H; ++h)
 #pragma unroll
             for (int c = 0; c < CPS; ++c)
-#pragma unroll
-                for (int j = 0; j < 4; ++j)
-                    areg[A_REGS ? c : 0][j] = prep_a(*reinterpret_cast<const uintx4*>(
-                        A + (size_t)m_rd * K + (chunk_of[0][c] << 7) + (kq << 5) + (j << 3)));
-        }
-        else
-        {
-            for (int u = tid; u < a_units; u += blockDim.x)
-            {
-                int m = u % M;
-                int rest = u / M;
-                int q = rest & 3;
-                int j = (rest >> 2) & 3;
-                int c = rest >> 4;
-                lds[u] = prep_a(*reinterpret_cast<const uintx4*>(A + (size_t)m * K + (c << 7) + (q << 5) + (j << 3)));
-            }
-#pragma unroll
-            for (int h = 0; h < H; ++h)
-#pragma unroll
-                for (int c = 0; c < CPS; ++c)
-                    a_unit[h][c] = (chunk_of[h][c] * 16 + kq) * M + m_rd;
-        }
+                a_unit[h][c] = (chunk_of[h][c] * 16 + kq) * M + m_rd;
         // scales of the first tile -> LDS copy 0, then fetch the second tile's
         if (s_loader)
         {
@@ -152,6 +142,17 @@ namespace nnf
                 sreg = load_s(tile_at(1));
         }
         lds_barrier();
+
+        // A_REGS: this wavefront's operand is read from LDS once and kept (16 VGPRs per group)
+        uintx4 areg[A_REGS ? CPS : 1][4];
+        if (A_REGS)
+        {
+#pragma unroll
+            for (int c = 0; c < CPS; ++c)
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    areg[A_REGS ? c : 0][j] = lds[a_unit[0][c] + j * 4 * M];
+        }
 
         auto a_op = [&](int h, int c, int j) -> uintx4 {
             if (A_REGS)
@@ -392,7 +393,7 @@ namespace nnf
                 return p;
             // the A operand fits in registers up to two groups per wavefront (32 VGPRs)
             p.a_regs = p.cps <= 2 && p.h == 1;
-            const size_t a_bytes = p.a_regs ? 0 : (size_t)G * 16 * M * 16;
+            const size_t a_bytes = (size_t)G * 16 * M * 16;
             const size_t sc_bytes = 2 * (((size_t)16 * G * 2 + 15) & ~(size_t)15);
             p.lds = a_bytes + sc_bytes + (size_t)2 * p.ks * 256 * 4;
             return p;
