@@ -38,6 +38,7 @@ namespace nnf
         int force_path = 0;  // 1 = VALU GEMV, 2 = MFMA skinny, 3 = MFMA GEMM
         int skinny_cps = 0;  // chunks (groups of 128) per wavefront
         int skinny_wg_per_cu = 0;
+        int gemm_no_direct_loads = 0; // 1 = the register-staged GEMM kernel for every variant
     };
     extern Tuning g_tuning;
 } // namespace nnf

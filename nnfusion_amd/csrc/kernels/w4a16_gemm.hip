@@ -2,8 +2,11 @@
 //
 //   Y[M,N] = epilogue( prologue(A)[M,K] . ((Wq - zp) * S)^T )
 //
-// Workgroup tile 256 (M) x 256 (N) x 64 (K), four wavefronts in a 2 x 2 arrangement, each owning a
-// 128 x 128 sub-tile = 4 x 4 MFMA tiles of 32 x 32 (256 fp32 accumulators per lane).
+// Workgroup tile 256 (M) x 256 (N) x 64 (K), eight wavefronts in a 2 (M) x 4 (N) arrangement, each
+// owning a 128 x 64 sub-tile = 4 x 2 MFMA tiles of 32 x 32 (128 fp32 accumulators per lane).  Two
+// wavefronts share a SIMD: while one waits for LDS operands or runs the int4 -> fp16 VALU work, the
+// other keeps the matrix core busy (one wavefront of 128 x 128 per SIMD left the MFMA pipe idle
+// for about half of the time).
 //   * A (fp16) and Wq (raw int4) tiles of the next K step are fetched global -> registers while
 //     the current step is computed from LDS; LDS is double buffered, one barrier per K step.
 //   * LDS layouts are XOR-swizzled at 16-byte granularity so that both the 128-bit stores and the
@@ -29,6 +32,9 @@ namespace nnf
     namespace gemm
     {
         constexpr int BM = 256, BN = 256, BK = 64;
+        constexpr int THREADS = 512;            // 8 wavefronts: 2 along M x 4 along N
+        constexpr int TM = 4, TN = 2;           // 32 x 32 MFMA tiles per wavefront along M, N
+        constexpr int NA = BM * BK * 2 / 16 / THREADS; // 16-byte pieces of the A tile per thread (4)
         constexpr int A_TILE_BYTES = BM * BK * 2;     // 32 KiB
         constexpr int W_TILE_BYTES = BN * BK / 2;     // 8 KiB
         constexpr int STAGE_BYTES = A_TILE_BYTES + W_TILE_BYTES;
@@ -90,14 +96,14 @@ namespace nnf
     }
 
     template <bool GATE, bool RMS, bool BIAS, bool RESID>
-    __global__ __launch_bounds__(256) void w4a16_gemm_kernel(GemmParams p)
+    __global__ __launch_bounds__(512) void w4a16_gemm_kernel(GemmParams p)
     {
         using namespace gemm;
         extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
         const int tid = threadIdx.x;
         const int lane = tid & 63;
         const int wave = tid >> 6;
-        const int wm = wave >> 1, wn = wave & 1;
+        const int wm = wave >> 2, wn = wave & 3;
         const int l32 = lane & 31, h = lane >> 5;
         const int K = p.K;
         const int G = K >> 7;
@@ -120,30 +126,30 @@ namespace nnf
         const int m0 = tm * BM, n0 = tn * BN_OUT;
 
         // ---- global -> register staging maps -------------------------------------------------------
-        // A: 2048 pieces of 16 B, 8 per thread: row = i*32 + tid/8, piece = tid%8
+        // A: 2048 pieces of 16 B, NA per thread: row = i*64 + tid/8, piece = tid%8
         const int a_p = tid & 7;
         const int a_r0 = tid >> 3;
-        const half_t* a_src[8];
-        int a_dst[8];
-        float a_rstd[RMS ? 8 : 1];
+        const half_t* a_src[NA];
+        int a_dst[NA];
+        float a_rstd[RMS ? NA : 1];
 #pragma unroll
-        for (int i = 0; i < 8; ++i)
+        for (int i = 0; i < NA; ++i)
         {
-            int r = i * 32 + a_r0;
+            int r = i * (THREADS / 8) + a_r0;
             int gm = min(m0 + r, p.M - 1);
             a_src[i] = p.A + (size_t)gm * K + a_p * 8;
             a_dst[i] = a_off(r, a_p);
             if (RMS)
                 a_rstd[i] = p.rstd[gm];
         }
-        // W: 512 pieces of 16 B, 2 per thread: row = i*128 + tid/2, piece = tid%2
+        // W: 512 pieces of 16 B, one per thread: row = tid/2, piece = tid%2
         const int w_h = tid & 1;
-        const uint8_t* w_src[2];
-        int w_dst[2];
+        const uint8_t* w_src[1];
+        int w_dst[1];
 #pragma unroll
-        for (int i = 0; i < 2; ++i)
+        for (int i = 0; i < 1; ++i)
         {
-            int r = i * 128 + (tid >> 1);
+            int r = tid >> 1;
             int gn;
             if (GATE)
                 gn = (r < BN / 2) ? (n0 + r) : (p.up_row_offset + n0 + (r - BN / 2));
@@ -165,18 +171,18 @@ namespace nnf
             a_frag[i] = r * 128;
             a_swz[i] = (r >> 1) & 7;
         }
-        int w_frag[4];
-        size_t s_idx[4];        // element index of this lane's column scale, group 0, in N tile j
-        int col_out[4];         // output column of N tile j
+        int w_frag[TN];
+        size_t s_idx[TN];        // element index of this lane's column scale, group 0, in N tile j
+        int col_out[TN];         // output column of N tile j
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int j = 0; j < TN; ++j)
         {
             int r; // row of the W tile
             int gn;
             if (GATE)
             {
-                int half_sel = j >> 1; // 0 = gate, 1 = up
-                int c = wn * 64 + (j & 1) * 32 + l32;
+                int half_sel = j; // 0 = gate, 1 = up
+                int c = wn * 32 + l32;
                 r = half_sel * (BN / 2) + c;
                 gn = half_sel ? (p.up_row_offset + n0 + c) : (n0 + c);
                 gn = min(gn, p.up_row_offset + p.N - 1);
@@ -184,7 +190,7 @@ namespace nnf
             }
             else
             {
-                r = wn * 128 + j * 32 + l32;
+                r = wn * 64 + j * 32 + l32;
                 gn = min(n0 + r, p.N - 1);
                 col_out[j] = n0 + r;
             }
@@ -192,11 +198,11 @@ namespace nnf
             s_idx[j] = (size_t)gn * G;
         }
 
-        floatx16 acc[4][4];
+        floatx16 acc[TM][TN];
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+        for (int i = 0; i < TM; ++i)
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
+            for (int j = 0; j < TN; ++j)
 #pragma unroll
                 for (int e = 0; e < 16; ++e)
                     acc[i][j][e] = 0.f;
@@ -209,32 +215,30 @@ namespace nnf
         // holds the fp16 (a 16-bit load would be widened at its point of use and force a wait for
         // every younger load, i.e. the tile prefetch).
         const uint32_t* s32 = reinterpret_cast<const uint32_t*>(p.S);
-        uint32_t s_nxt[4];
+        uint32_t s_nxt[TN];
         auto load_scales = [&](int g) {
             g = min(g, G - 1);
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
+            for (int j = 0; j < TN; ++j)
                 s_nxt[j] = s32[(s_idx[j] + g) >> 1];
         };
 
-        uintx4 a_reg[8], w_reg[2], g_reg;
+        uintx4 a_reg[NA], w_reg[1], g_reg;
         auto load_global = [&](int kt) {
             const int k0 = kt * BK;
             if (RMS)
                 g_reg = *reinterpret_cast<const uintx4*>(p.gamma + k0 + a_p * 8);
 #pragma unroll
-            for (int i = 0; i < 8; ++i)
+            for (int i = 0; i < NA; ++i)
                 a_reg[i] = *reinterpret_cast<const uintx4*>(a_src[i] + k0);
-#pragma unroll
-            for (int i = 0; i < 2; ++i)
-                w_reg[i] = *reinterpret_cast<const uintx4*>(w_src[i] + (k0 >> 1));
+            w_reg[0] = *reinterpret_cast<const uintx4*>(w_src[0] + (k0 >> 1));
         };
         auto store_lds = [&](int kt, int stage) {
             uint8_t* base = smem + stage * STAGE_BYTES;
             (void)kt;
             const uintx4 g4 = g_reg;
 #pragma unroll
-            for (int i = 0; i < 8; ++i)
+            for (int i = 0; i < NA; ++i)
             {
                 uintx4 a = a_reg[i];
                 if (RMS)
@@ -257,9 +261,7 @@ namespace nnf
                 }
                 *reinterpret_cast<uintx4*>(base + a_dst[i]) = permute_a8(a);
             }
-#pragma unroll
-            for (int i = 0; i < 2; ++i)
-                *reinterpret_cast<uintx4*>(base + w_dst[i]) = w_reg[i];
+            *reinterpret_cast<uintx4*>(base + w_dst[0]) = w_reg[0];
         };
 
         const int KT = K / BK;
@@ -268,7 +270,7 @@ namespace nnf
         store_lds(0, 0);
         __syncthreads();
 
-        half2_t sc[4]; // group scale of this lane's column in each N tile, both halves equal
+        half2_t sc[TN]; // group scale of this lane's column in each N tile, both halves equal
         for (int kt = 0; kt < KT; ++kt)
         {
             const int stage = kt & 1;
@@ -276,7 +278,7 @@ namespace nnf
             {
                 const int g = kt >> 1;
 #pragma unroll
-                for (int j = 0; j < 4; ++j)
+                for (int j = 0; j < TN; ++j)
                 {
                     uint32_t bits = s_nxt[j] >> ((((uint32_t)s_idx[j] + (uint32_t)g) & 1u) << 4);
                     half_t s = as_half2(bits).x;
@@ -287,9 +289,9 @@ namespace nnf
             if (kt + 1 < KT)
                 load_global(kt + 1);
             const uint8_t* base = smem + stage * STAGE_BYTES;
-            uintx4 wq[4];
+            uintx4 wq[TN];
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
+            for (int j = 0; j < TN; ++j)
                 wq[j] = *reinterpret_cast<const uintx4*>(base + w_frag[j]);
 #pragma unroll
             for (int s = 0; s < 4; ++s)
@@ -302,7 +304,7 @@ namespace nnf
                     af[i] = *reinterpret_cast<const half8_t*>(base + a_frag[i] + (pc << 4));
                 }
 #pragma unroll
-                for (int j = 0; j < 4; ++j)
+                for (int j = 0; j < TN; ++j)
                 {
                     uint32_t w = (s == 0) ? wq[j].x : (s == 1) ? wq[j].y : (s == 2) ? wq[j].z : wq[j].w;
                     uint32_t w8 = w >> 8;
@@ -328,7 +330,7 @@ namespace nnf
 
         // ---- epilogue ---------------------------------------------------------------------------------
         // D layout of a 32x32 tile: lane (col = l32, h), element e: row = 8*(e/4) + 4*h + (e%4)
-        constexpr int NJ = GATE ? 2 : 4;
+        constexpr int NJ = GATE ? 1 : TN;
 #pragma unroll
         for (int j = 0; j < NJ; ++j)
         {
@@ -353,7 +355,293 @@ namespace nnf
                         // SiLU(gate) * up on the values the unfused graph would see: both
                         // projections rounded to fp16 first
                         float g = (float)(half_t)acc[i][j][e];
-                        float u = (float)(half_t)acc[i][j + 2][e];
+                        float u = (float)(half_t)acc[i][j + 1][e];
+                        v = g * (1.0f / (1.0f + __expf(-g))) * u;
+                    }
+                    else
+                    {
+                        v = acc[i][j][e];
+                    }
+                    if (BIAS)
+                        v = (float)(half_t)v + bias;
+                    if (RESID)
+                        v = (float)(half_t)v + (float)p.residual[(size_t)m * p.ldy + n];
+                    p.Y[(size_t)m * p.ldy + n] = (half_t)v;
+                }
+            }
+        }
+    }
+
+    // -------------------------------------------------------------------------------------------------
+    // The same GEMM with asynchronous global -> LDS loads (global_load_lds_dwordx4: no register staging,
+    // no LDS store instructions) and a three-stage LDS ring, so that the operands of two K steps are in
+    // flight while a K step is computed.  Used whenever the activations need no rewriting on the way in
+    // (every variant except the RMSNorm prologue).
+    //   * A wavefront-wide direct load fills 1 KiB of consecutive LDS; the XOR swizzle is obtained by
+    //     choosing which 16-byte piece of global memory each lane fetches.
+    //   * Nothing can be permuted on the way, so the activations stay in natural K order and the
+    //     weights are unpacked in natural order too: v_perm_b32 copies byte i of a word (nibbles 2i,
+    //     2i+1) into bytes 0 and 2, one v_and_or_b32 makes (1024 + q_2i, 1024 + 16 q_2i+1), one packed fma
+    //     with the constants (1, 1/16) and (-(1024+zp), -(64+zp)) gives the exact (q - zp) pair, one packed
+    //     multiply applies the group scale: 16 VALU operations per 8 weights, feeding four MFMAs.
+    //   * One barrier per K step: after it, every wavefront's loads for this step have landed and every
+    //     wavefront has finished reading the stage that is about to be refilled.
+    namespace gemm_dl
+    {
+        constexpr int BM = 256, BN = 256, BK = 64;
+        constexpr int THREADS = 512;  // 8 wavefronts: 2 along M x 4 along N
+        constexpr int TM = 4, TN = 2; // 32 x 32 MFMA tiles per wavefront along M, N
+        constexpr int STAGES = 3;
+        constexpr int A_TILE_BYTES = BM * BK * 2; // 32 KiB
+        constexpr int W_TILE_BYTES = BN * BK / 2; // 8 KiB
+        constexpr int STAGE_BYTES = A_TILE_BYTES + W_TILE_BYTES;
+        constexpr int LDS_BYTES = STAGES * STAGE_BYTES; // 120 KiB
+        constexpr int A_LOADS = A_TILE_BYTES / 1024 / 8;  // wavefront-wide loads of the A tile per wavefront (4)
+        constexpr int TILE_LOADS = A_LOADS + 1;           // plus one for the W tile
+
+        // s_waitcnt with only the vector-memory counter set (gfx9 encoding: vmcnt = bits 3:0 and 15:14)
+        constexpr int vmcnt_imm(int n) { return (n & 0xF) | ((n >> 4) << 14) | (0x7 << 4) | (0xF << 8); }
+    } // namespace gemm_dl
+
+    template <bool GATE, bool BIAS, bool RESID>
+    __global__ __launch_bounds__(512) void w4a16_gemm_dl_kernel(GemmParams p)
+    {
+        using namespace gemm_dl;
+        extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+        const int tid = threadIdx.x;
+        const int lane = tid & 63;
+        const int wave = tid >> 6;
+        const int wm = wave >> 2, wn = wave & 3;
+        const int l32 = lane & 31, h = lane >> 5;
+        const int K = p.K;
+        const int G = K >> 7;
+        constexpr int BN_OUT = GATE ? BN / 2 : BN;
+
+        const int tiles_m = (p.M + BM - 1) / BM;
+        const int tiles_n = (p.N + BN_OUT - 1) / BN_OUT;
+        const int n_wg = tiles_m * tiles_n;
+        int pid = blockIdx.x;
+        {
+            // contiguous run of tiles per XCD (workgroup ids are dealt round-robin to the 8 XCDs)
+            const int per_xcd = (n_wg + 7) >> 3;
+            const int full = n_wg - (per_xcd - 1) * 8;
+            const int xcd = pid & 7, idx = pid >> 3;
+            pid = (xcd < full) ? xcd * per_xcd + idx : full * per_xcd + (xcd - full) * (per_xcd - 1) + idx;
+        }
+        const int tm = pid % tiles_m, tn = pid / tiles_m;
+        const int m0 = tm * BM, n0 = tn * BN_OUT;
+
+        // ---- direct-load maps -------------------------------------------------------------------------
+        // A: wavefront w, load i fills LDS rows (w*4 + i)*8 .. +7; lane l lands at (row = .. + l/8, slot = l%8)
+        // and therefore fetches piece  slot ^ ((row >> 1) & 7)  of that row.
+        const half_t* a_src[A_LOADS];
+#pragma unroll
+        for (int i = 0; i < A_LOADS; ++i)
+        {
+            int row = (wave * A_LOADS + i) * 8 + (lane >> 3);
+            int piece = (lane & 7) ^ ((row >> 1) & 7);
+            a_src[i] = p.A + (size_t)min(m0 + row, p.M - 1) * K + piece * 8;
+        }
+        // W: wavefront w fills LDS rows w*32 .. +31 (32 B each); lane l lands at (row = w*32 + l/2, slot = l%2)
+        const uint8_t* w_src;
+        {
+            int row = wave * 32 + (lane >> 1);
+            int piece = (lane & 1) ^ ((row >> 3) & 1);
+            int gn;
+            if (GATE)
+                gn = (row < BN / 2) ? (n0 + row) : (p.up_row_offset + n0 + (row - BN / 2));
+            else
+                gn = n0 + row;
+            gn = GATE ? min(gn, p.up_row_offset + p.N - 1) : min(gn, p.N - 1);
+            w_src = p.Wq + (size_t)gn * (K >> 1) + piece * 16;
+        }
+        auto issue_tile_loads = [&](int kt, int stage) {
+            uint8_t* base = smem + stage * STAGE_BYTES;
+            const int k0 = kt * BK;
+#pragma unroll
+            for (int i = 0; i < A_LOADS; ++i)
+                __builtin_amdgcn_global_load_lds(
+                    (const void __attribute__((address_space(1)))*)(a_src[i] + k0),
+                    (void __attribute__((address_space(3)))*)(base + (wave * A_LOADS + i) * 1024), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1)))*)(w_src + (k0 >> 1)),
+                                             (void __attribute__((address_space(3)))*)(base + A_TILE_BYTES + wave * 1024),
+                                             16, 0, 0);
+        };
+
+        // ---- per-lane fragment addresses in LDS ------------------------------------------------------
+        int a_frag[TM], a_swz[TM];
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+        {
+            int r = wm * 128 + i * 32 + l32;
+            a_frag[i] = r * 128;
+            a_swz[i] = (r >> 1) & 7;
+        }
+        int w_frag[TN];
+        size_t s_idx[TN];
+        int col_out[TN];
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+        {
+            int r, gn;
+            if (GATE)
+            {
+                int c = wn * 32 + l32;
+                r = j * (BN / 2) + c; // j = 0: gate, 1: up
+                gn = j ? (p.up_row_offset + n0 + c) : (n0 + c);
+                gn = min(gn, p.up_row_offset + p.N - 1);
+                col_out[j] = n0 + c;
+            }
+            else
+            {
+                r = wn * 64 + j * 32 + l32;
+                gn = min(n0 + r, p.N - 1);
+                col_out[j] = n0 + r;
+            }
+            w_frag[j] = A_TILE_BYTES + r * 32 + ((h ^ ((r >> 3) & 1)) << 4);
+            s_idx[j] = (size_t)gn * G;
+        }
+
+        floatx16 acc[TM][TN];
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int e = 0; e < 16; ++e)
+                    acc[i][j][e] = 0.f;
+
+        // constants of the unpacking; kept opaque so that each lands in the register class the VOP3
+        // encodings need (one scalar operand per instruction, no 32-bit literals)
+        uint32_t MASK, MAGIC, SEL[4];
+        asm("s_mov_b32 %0, 0x00F0000F" : "=s"(MASK));
+        asm("v_mov_b32 %0, 0x64006400" : "=v"(MAGIC));
+        asm("s_mov_b32 %0, 0x0c000c00" : "=s"(SEL[0]));
+        asm("s_mov_b32 %0, 0x0c010c01" : "=s"(SEL[1]));
+        asm("s_mov_b32 %0, 0x0c020c02" : "=s"(SEL[2]));
+        asm("s_mov_b32 %0, 0x0c030c03" : "=s"(SEL[3]));
+        const half2_t dq_mul = half2_t{(half_t)1.0f, (half_t)0.0625f};
+        const half2_t dq_add = half2_t{(half_t)(-(1024.0f + (float)p.zp)), (half_t)(-(64.0f + (float)p.zp))};
+
+        // group scales, fetched one group (two K steps) ahead as the aligned 32-bit word holding the fp16
+        const uint32_t* s32 = reinterpret_cast<const uint32_t*>(p.S);
+        uint32_t s_nxt[TN];
+        auto load_scales = [&](int g) {
+            g = min(g, G - 1);
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+                s_nxt[j] = s32[(s_idx[j] + g) >> 1];
+        };
+        half2_t sc[TN];
+        auto take_scales = [&](int g) {
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+            {
+                uint32_t bits = s_nxt[j] >> ((((uint32_t)s_idx[j] + (uint32_t)g) & 1u) << 4);
+                half_t s = as_half2(bits).x;
+                sc[j] = half2_t{s, s};
+            }
+        };
+
+        auto compute = [&](int stage) {
+            const uint8_t* base = smem + stage * STAGE_BYTES;
+            uintx4 wq[TN];
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+                wq[j] = *reinterpret_cast<const uintx4*>(base + w_frag[j]);
+#pragma unroll
+            for (int s = 0; s < 4; ++s)
+            {
+                half8_t af[TM];
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+                    af[i] = *reinterpret_cast<const half8_t*>(base + a_frag[i] + ((((h << 2) + s) ^ a_swz[i]) << 4));
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                {
+                    const uint32_t w = (s == 0) ? wq[j].x : (s == 1) ? wq[j].y : (s == 2) ? wq[j].z : wq[j].w;
+                    uint32_t bw[4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                    {
+                        uint32_t x = __builtin_amdgcn_perm(w, w, SEL[e]);        // bytes (b_e, 0, b_e, 0)
+                        half2_t y = as_half2((x & MASK) | MAGIC);                // (1024 + q_2e, 1024 + 16 q_2e+1)
+                        half2_t z = __builtin_elementwise_fma(y, dq_mul, dq_add); // (q_2e - zp, q_2e+1 - zp)
+                        bw[e] = as_u32(z * sc[j]);
+                    }
+                    half8_t bf = __builtin_bit_cast(half8_t, uintx4{bw[0], bw[1], bw[2], bw[3]});
+#pragma unroll
+                    for (int i = 0; i < TM; ++i)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf, acc[i][j], 0, 0, 0);
+                }
+            }
+        };
+
+        // ---- K loop: stages kt % 3; loads run two K steps ahead -------------------------------------------
+        const int KT = K / BK; // even (K % 128 == 0)
+        load_scales(0);
+        issue_tile_loads(0, 0);
+        issue_tile_loads(1, 1);
+        // Vector-memory operations complete in order.  Before the barrier of step kt a wavefront waits
+        // until at most the operations it issued during step kt-1 are outstanding: then its own loads
+        // for step kt (issued during step kt-2) have landed.  Even steps issue the scale loads (TN) and a
+        // tile (TILE_LOADS), odd steps a tile only.
+        int stage = 0;
+        for (int kt = 0; kt < KT; kt += 2)
+        {
+            // even step
+            __builtin_amdgcn_s_waitcnt(vmcnt_imm(TILE_LOADS));
+            __builtin_amdgcn_s_barrier();
+            take_scales(kt >> 1);
+            load_scales((kt >> 1) + 1);
+            {
+                const int nk = min(kt + 2, KT - 1); // past the end: reload a valid tile into the free stage
+                int st = stage + 2;
+                st = st >= STAGES ? st - STAGES : st;
+                issue_tile_loads(nk, st);
+            }
+            compute(stage);
+            stage = stage + 1 == STAGES ? 0 : stage + 1;
+            // odd step
+            __builtin_amdgcn_s_waitcnt(vmcnt_imm(TILE_LOADS + TN));
+            __builtin_amdgcn_s_barrier();
+            {
+                const int nk = min(kt + 3, KT - 1);
+                int st = stage + 2;
+                st = st >= STAGES ? st - STAGES : st;
+                issue_tile_loads(nk, st);
+            }
+            compute(stage);
+            stage = stage + 1 == STAGES ? 0 : stage + 1;
+        }
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm(0)); // drain the tail loads before the LDS goes away
+
+        // ---- epilogue ---------------------------------------------------------------------------------
+        // D layout of a 32x32 tile: lane (col = l32, h), element e: row = 8*(e/4) + 4*h + (e%4)
+        constexpr int NJ = GATE ? 1 : TN;
+#pragma unroll
+        for (int j = 0; j < NJ; ++j)
+        {
+            const int n = col_out[j];
+            if (n >= p.N)
+                continue;
+            float bias = 0.f;
+            if (BIAS)
+                bias = (float)p.bias[n];
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+            {
+#pragma unroll
+                for (int e = 0; e < 16; ++e)
+                {
+                    const int m = m0 + wm * 128 + i * 32 + 8 * (e >> 2) + 4 * h + (e & 3);
+                    if (m >= p.M)
+                        continue;
+                    float v;
+                    if (GATE)
+                    {
+                        float g = (float)(half_t)acc[i][0][e];
+                        float u = (float)(half_t)acc[i][1][e];
                         v = g * (1.0f / (1.0f + __expf(-g))) * u;
                     }
                     else
@@ -388,8 +676,28 @@ namespace nnf
                     return e;
                 attr_set = true;
             }
-            hipLaunchKernelGGL((w4a16_gemm_kernel<GATE, RMS, BIAS, RESID>), dim3(tiles_m * tiles_n), dim3(256), LDS_BYTES,
+            hipLaunchKernelGGL((w4a16_gemm_kernel<GATE, RMS, BIAS, RESID>), dim3(tiles_m * tiles_n), dim3(THREADS), LDS_BYTES,
                                stream, p);
+            return hipGetLastError();
+        }
+        template <bool GATE, bool BIAS, bool RESID>
+        hipError_t launch_gemm_dl_variant(hipStream_t stream, const GemmParams& p)
+        {
+            using namespace gemm_dl;
+            constexpr int BN_OUT = GATE ? BN / 2 : BN;
+            const int tiles_m = (p.M + BM - 1) / BM;
+            const int tiles_n = (p.N + BN_OUT - 1) / BN_OUT;
+            static bool attr_set = false;
+            if (!attr_set)
+            {
+                hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&w4a16_gemm_dl_kernel<GATE, BIAS, RESID>),
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
+                if (e != hipSuccess)
+                    return e;
+                attr_set = true;
+            }
+            hipLaunchKernelGGL((w4a16_gemm_dl_kernel<GATE, BIAS, RESID>), dim3(tiles_m * tiles_n), dim3(THREADS),
+                               LDS_BYTES, stream, p);
             return hipGetLastError();
         }
     } // namespace
@@ -425,16 +733,22 @@ namespace nnf
         // the combinations the fused entry points use; anything else is composed by the caller
         if (gate && rms && !hb && !hr)
             return launch_gemm_variant<true, true, false, false>(stream, p);
+        const bool dl = g_tuning.gemm_no_direct_loads == 0;
         if (gate && !rms && !hb && !hr)
-            return launch_gemm_variant<true, false, false, false>(stream, p);
+            return dl ? launch_gemm_dl_variant<true, false, false>(stream, p)
+                      : launch_gemm_variant<true, false, false, false>(stream, p);
         if (!gate && !rms && !hb && !hr)
-            return launch_gemm_variant<false, false, false, false>(stream, p);
+            return dl ? launch_gemm_dl_variant<false, false, false>(stream, p)
+                      : launch_gemm_variant<false, false, false, false>(stream, p);
         if (!gate && !rms && !hb && hr)
-            return launch_gemm_variant<false, false, false, true>(stream, p);
+            return dl ? launch_gemm_dl_variant<false, false, true>(stream, p)
+                      : launch_gemm_variant<false, false, false, true>(stream, p);
         if (!gate && !rms && hb && !hr)
-            return launch_gemm_variant<false, false, true, false>(stream, p);
+            return dl ? launch_gemm_dl_variant<false, true, false>(stream, p)
+                      : launch_gemm_variant<false, false, true, false>(stream, p);
         if (!gate && !rms && hb && hr)
-            return launch_gemm_variant<false, false, true, true>(stream, p);
+            return dl ? launch_gemm_dl_variant<false, true, true>(stream, p)
+                      : launch_gemm_variant<false, false, true, true>(stream, p);
         if (!gate && rms && !hb && !hr)
             return launch_gemm_variant<false, true, false, false>(stream, p);
         if (!gate && rms && hb && !hr)

@@ -69,6 +69,7 @@ int nnf_internal_tune(int key, int value)
     case 0: nnf::g_tuning.force_path = value; return 0;
     case 1: nnf::g_tuning.skinny_cps = value; return 0;
     case 2: nnf::g_tuning.skinny_wg_per_cu = value; return 0;
+    case 3: nnf::g_tuning.gemm_no_direct_loads = value; return 0;
     default: return -1;
     }
 }
