@@ -34,6 +34,7 @@ MFMA_I8_PEAK_TOPS = 5000.0     # dense int8 MFMA
 
 DECODE_SHAPES = [(12288, 4096), (4096, 4096), (22016, 4096), (4096, 11008)]  # (N, K), M = 1
 GROUP = 128
+PROBE_BYTES = 1 << 30  # size of the calibration copy of --pmc-probe
 
 
 def w4a16_bytes(m, n, k):
@@ -53,6 +54,9 @@ def main():
     ap.add_argument("--layers", type=int, default=6, help="independent weight sets walked by the steps")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true")
+    ap.add_argument("--pmc-probe", action="store_true",
+                    help="for hardware-counter runs: a plain copy of known size, then the sweep launched eagerly; "
+                         "no timing, no JSON")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU (no sharding, no collectives); use --gpus 1")
@@ -113,6 +117,21 @@ def main():
         e1.record()
         torch.cuda.synchronize()
         return e0.elapsed_time(e1) * 1000.0 / reps
+
+    if args.pmc_probe:
+        # Calibration for FETCH_SIZE / WRITE_SIZE: a device-to-device copy that reads and writes exactly
+        # PROBE_BYTES, larger than the last-level cache, followed by the sweep over every resident layer.
+        src = torch.empty(PROBE_BYTES // 4, dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        for _ in range(4):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        for i in range(2 * args.layers):
+            step(i)
+        torch.cuda.synchronize()
+        print(f"pmc probe: copy of {PROBE_BYTES} bytes x4, then {2 * args.layers} sweeps", flush=True)
+        return
 
     # ---- warm-up (untimed), then exactly K steps in the timed region ------------------------------
     for i in range(args.warmup):
