@@ -99,6 +99,24 @@ namespace nnf
         return (half_t)v;
     }
 
+    // sum over the four lanes of a quad (lanes 4i .. 4i+3), in every lane; two DPP moves
+    __device__ __forceinline__ float quad_sum(float v)
+    {
+        v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, false)); // 1,0,3,2
+        v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, false)); // 2,3,0,1
+        return v;
+    }
+
+    // sum over a row of 16 lanes (lanes 16i .. 16i+15), in every lane; four DPP row rotations
+    __device__ __forceinline__ float row16_sum(float v)
+    {
+        v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x128, 0xF, 0xF, false)); // row_ror:8
+        v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x124, 0xF, 0xF, false)); // row_ror:4
+        v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x122, 0xF, 0xF, false)); // row_ror:2
+        v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x121, 0xF, 0xF, false)); // row_ror:1
+        return v;
+    }
+
     __device__ __forceinline__ float wave_sum(float v)
     {
 #pragma unroll

@@ -515,7 +515,7 @@ namespace nnf
         // encodings need (one scalar operand per instruction, no 32-bit literals)
         uint32_t MASK, MAGIC, SEL[4];
         asm("s_mov_b32 %0, 0x00F0000F" : "=s"(MASK));
-        asm("v_mov_b32 %0, 0x64006400" : "=v"(MAGIC));
+        asm volatile("v_mov_b32 %0, 0x64006400" : "=v"(MAGIC));
         asm("s_mov_b32 %0, 0x0c000c00" : "=s"(SEL[0]));
         asm("s_mov_b32 %0, 0x0c010c01" : "=s"(SEL[1]));
         asm("s_mov_b32 %0, 0x0c020c02" : "=s"(SEL[2]));

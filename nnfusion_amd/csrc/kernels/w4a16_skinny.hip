@@ -24,7 +24,8 @@
 //     is of order 1e4 at fp32 precision, i.e. an absolute error of ~1e-3 on a group sum of order 50;
 //   * the group scale multiplies the fp32 group sum (4 FMAs per group and lane);
 //   * the partial tiles of the KS wavefronts meet in LDS (one LDS-only barrier per tile, so the
-//     prefetched global loads stay in flight); results are parked in LDS and written once at the end.
+//     prefetched global loads stay in flight); results are parked in LDS and written after the last
+//     tile's barrier, when no load is left to protect.
 #include "nnf_device.h"
 #include "nnf_launch.h"
 
@@ -34,10 +35,13 @@
 namespace nnf
 {
     // LDS, in this order:
-    //   activations as 16-byte units  unit(c, j, kq, m) = ((c*4 + j)*4 + kq)*M + m  holding
+    //   activations as 16-byte units  unit(m, c, kq, j) = m*(16 G + 1) + (c*4 + kq)*4 + j  holding
     //       the eight fp16  a[m][c*128 + kq*32 + j*8 + {0,4,1,5,2,6,3,7}]  with slots 2,3,6,7 (odd k) times 1/16
+    //       (a row of A is staged in memory order; the odd row stride keeps rows on different banks)
+    //   ncorr    [G][16 m] fp32: constant part of every group sum, negated
     //   scales   sc[2][16 rows][G] fp16 (as in memory), each copy padded to 16 bytes
-    //   red      [2][KS][16 m][16 n] fp32 partial tiles
+    //   red      [2][M][16 n][KSP] fp32 partial sums, the KS wavefronts of one output side by side
+    //            (KSP = KS rounded up to a multiple of 4; the padding stays zero)
     //   outb     [tiles of this workgroup][M][16] fp32
     // Group (chunk) index of wavefront w, pass h, slot c:  (h*KS + w)*CPS + c.
     template <int CPS, bool A_REGS, int H>
@@ -50,18 +54,27 @@ namespace nnf
         static_assert(H == 1 || H == 2, "one or two passes over K");
         static_assert(!A_REGS || H == 1, "register-resident activations only with one pass");
         extern __shared__ uintx4 lds[];
+        // volatile: the vector move must stay here, where every lane is active
+        uint32_t MAGIC, MASK_LO, MASK_HI;
+        asm volatile("v_mov_b32 %0, 0x64006400" : "=v"(MAGIC));
+        asm volatile("s_mov_b32 %0, 0x000F000F" : "=s"(MASK_LO));
+        asm volatile("s_mov_b32 %0, 0x00F000F0" : "=s"(MASK_HI));
         const int tid = threadIdx.x;
         const int lane = tid & 63;
-        const int wave = tid >> 6;
+        const int wave = __builtin_amdgcn_readfirstlane(tid >> 6); // in a scalar register, and what follows from it
         const int KS = blockDim.x >> 6;
         const int col = lane & 15; // n within the tile (B operand / D column), m for the A operand
         const int kq = lane >> 4;  // K quarter of the MFMA (A/B operands), row quad of D
         const int G = K >> 7;
-        const int a_units = G * 16 * M;
+        const int row_units = G * 16 + 1; // 16-byte units per staged row of A (one unit of padding)
+        const int a_units = row_units * M;
         const int sc_units = (16 * G * 2 + 15) >> 4; // 16-byte units of one scale copy
-        uintx4* sc_lds = lds + a_units;
-        float* red = reinterpret_cast<float*>(sc_lds + 2 * sc_units); // [2][KS][16][16]
-        float* outb = red + 2 * KS * 256;
+        floatx4* nc_lds = reinterpret_cast<floatx4*>(lds + a_units); // [G][4 kq] x (4 m)
+        uintx4* sc_lds = lds + a_units + G * 4;
+        const int KSP = (KS + 3) & ~3;
+        const int red_copy = M * 16 * KSP;
+        float* red = reinterpret_cast<float*>(sc_lds + 2 * sc_units); // [2][M][16][KSP]
+        float* outb = red + 2 * red_copy;
         const size_t row_bytes = (size_t)(K >> 1);
         const int m_rd = min(col, M - 1); // rows >= M read a valid row; their D rows are never stored
         int chunk_of[H][CPS];             // clamped to valid memory; chunks past the end of K are masked at use
@@ -77,20 +90,24 @@ namespace nnf
             }
 
         // ---- loads: unconditional, so that no branch separates a load from its use ---------------------
+        // A tile is 16 whole rows: the last tile of an N that is not a multiple of 16 is moved back to
+        // rows N-16 .. N-1 (some rows are then computed twice, with identical results), so that no
+        // address needs a per-lane clamp: every load is  uniform 64-bit base + 32-bit lane offset.
+        auto row0_of = [&](int tile) { return __builtin_amdgcn_readfirstlane(min(tile * 16, N - 16)); };
+        const uint32_t w_lane_off = (uint32_t)col * (uint32_t)row_bytes + (uint32_t)kq * 16u;
         auto load_w = [&](int tile, int h, uintx4* w) {
-            int n = min(tile * 16 + col, N - 1);
-            const uint8_t* wrow = Wq + (size_t)n * row_bytes + kq * 16;
+            const uint8_t* tile_base = Wq + (size_t)row0_of(tile) * row_bytes;
 #pragma unroll
             for (int c = 0; c < CPS; ++c)
-                w[c] = *reinterpret_cast<const uintx4*>(wrow + (size_t)chunk_of[h][c] * 64);
+                w[c] = *reinterpret_cast<const uintx4*>(tile_base + (size_t)chunk_of[h][c] * 64 + w_lane_off);
         };
-        // scale block of a tile: bytes [tile*16*G*2, +16*G*2) of S; thread t carries bytes [16t, 16t+16)
-        const size_t s_total = (size_t)N * G * 2;
+        // scale block of a tile: 16 rows x G fp16, contiguous; thread t carries bytes [16t, 16t+16) of it
+        // (the threads of the last loading wavefront beyond the block re-read its last 16 bytes)
         const bool s_loader = tid < sc_units;
+        const uint32_t s_lane_off = (uint32_t)min(tid, sc_units - 1) * 16u;
         auto load_s = [&](int tile) -> uintx4 {
-            size_t off = (size_t)tile * 16 * G * 2 + (size_t)tid * 16;
-            off = min(off, s_total - 16); // rows past N (last tile) are never stored
-            return *reinterpret_cast<const uintx4*>(reinterpret_cast<const uint8_t*>(S) + off);
+            const uint8_t* tile_base = reinterpret_cast<const uint8_t*>(S) + (size_t)row0_of(tile) * G * 2;
+            return *reinterpret_cast<const uintx4*>(tile_base + s_lane_off);
         };
 
         const int stride = gridDim.x;
@@ -98,92 +115,115 @@ namespace nnf
         const int T = (n_tiles - tile0 + stride - 1) / stride;
         auto tile_at = [&](int k) { return tile0 + k * stride; };
 
-        // register set 0 / 1: H == 1: even / odd tiles;  H == 2: first / second pass of the current tile
-        uintx4 w0[CPS], w1[CPS], sreg = {0, 0, 0, 0};
-        load_w(tile_at(0), 0, w0);
+        // ---- prologue loads ----------------------------------------------------------------------------
+        // Row 0 of the activations (all of them for M = 1) and the scales of the first two tiles are
+        // requested before the weights: they are small and shared by every workgroup (cache hits), loads
+        // complete in order, and the barrier that publishes them in LDS should not have to wait for the
+        // first weights, which come from HBM.  The address arithmetic before the weight loads is kept
+        // minimal: with four wavefronts per SIMD every instruction here delays the weight stream.
+        constexpr int A_EARLY = 2;
+        const int row0_units = G * 16;
+        uintx4 a_early[A_EARLY];
+#pragma unroll
+        for (int e = 0; e < A_EARLY; ++e)
+        {
+            int u = min(tid + e * (int)blockDim.x, row0_units - 1);
+            a_early[e] = *reinterpret_cast<const uintx4*>(A + u * 8);
+        }
+        // A load issued at the end of the prologue would be the newest one when the tile loop is entered,
+        // and the loop's wait for the scale registers would then wait for every weight load in flight:
+        // hence the second tile's scales here, and the second register set loaded without a branch
+        // (a workgroup with a single tile fetches it twice).
+        // Register set 0 / 1: H == 1: even / odd tiles;  H == 2: first / second pass of the current tile.
+        uintx4 w0[CPS], w1[CPS], sreg = {0, 0, 0, 0}, sfirst = {0, 0, 0, 0};
         if (s_loader)
-            sreg = load_s(tile_at(0));
+        {
+            sfirst = load_s(tile_at(0));
+            sreg = load_s(tile_at(min(1, T - 1)));
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        load_w(tile_at(0), 0, w0);
         if (H == 2)
             load_w(tile_at(0), H - 1, w1);
-        else if (T > 1)
-            load_w(tile_at(1), 0, w1);
+        else
+            load_w(tile_at(min(1, T - 1)), 0, w1);
+        __builtin_amdgcn_sched_barrier(0);
 
-        // ---- activations ---------------------------------------------------------------------------
-        const half2_t sixteenth = half2_t{(half_t)0.0625f, (half_t)0.0625f};
-        auto prep_a = [&](uintx4 a) {
-            a = permute_a8(a);
-            a.y = as_u32(as_half2(a.y) * sixteenth);
-            a.w = as_u32(as_half2(a.w) * sixteenth);
-            return a;
-        };
+        // ---- activations -> LDS ---------------------------------------------------------------------
         // Staged once per workgroup (one coalesced 16-byte load per thread and unit); every wavefront
         // loading its own operand straight from global memory would cost 8 load instructions per
         // wavefront, almost all of whose lanes are redundant.
-        for (int u = tid; u < a_units; u += blockDim.x)
+        // The constant part of a group sum,
+        //     corr[m, group] = (1024 + zp) * sum_even a + 16 (64 + zp) * sum_odd (a / 16),
+        // is accumulated on the way: the 16 units of a group sit in 16 consecutive lanes.
+        const half2_t sixteenth = half2_t{(half_t)0.0625f, (half_t)0.0625f};
+        const float ce = -(1024.0f + (float)zp);
+        const float co = -16.0f * (64.0f + (float)zp);
+        auto stage_unit = [&](uintx4 a, int m, int u) {
+            a = permute_a8(a);
+            a.y = as_u32(as_half2(a.y) * sixteenth);
+            a.w = as_u32(as_half2(a.w) * sixteenth);
+            lds[m * row_units + u] = a;
+            const half2_t x = as_half2(a.x), y = as_half2(a.y), z = as_half2(a.z), w = as_half2(a.w);
+            float se = ((float)x.x + (float)x.y) + ((float)z.x + (float)z.y);
+            float so = ((float)y.x + (float)y.y) + ((float)w.x + (float)w.y);
+            float pc = row16_sum(ce * se + co * so);
+            if ((u & 15) == 0)
+                reinterpret_cast<float*>(nc_lds)[(u >> 4) * 16 + m] = pc;
+        };
+#pragma unroll
+        for (int e = 0; e < A_EARLY; ++e)
         {
-            int m = u % M;
-            int rest = u / M;
-            int q = rest & 3;
-            int j = (rest >> 2) & 3;
-            int c = rest >> 4;
-            lds[u] = prep_a(*reinterpret_cast<const uintx4*>(A + (size_t)m * K + (c << 7) + (q << 5) + (j << 3)));
+            int u = tid + e * (int)blockDim.x;
+            if (u < row0_units)
+                stage_unit(a_early[e], 0, u);
         }
+        for (int m = 0; m < M; ++m)
+            for (int u = tid + (m == 0 ? A_EARLY * (int)blockDim.x : 0); u < row0_units; u += blockDim.x)
+                stage_unit(*reinterpret_cast<const uintx4*>(A + (size_t)m * K + u * 8), m, u);
+        if (KSP != KS)
+            for (int i = tid; i < 2 * red_copy; i += blockDim.x)
+                red[i] = 0.f;
         int a_unit[H][CPS];
 #pragma unroll
         for (int h = 0; h < H; ++h)
 #pragma unroll
             for (int c = 0; c < CPS; ++c)
-                a_unit[h][c] = (chunk_of[h][c] * 16 + kq) * M + m_rd;
-        // scales of the first tile -> LDS copy 0, then fetch the second tile's
+                a_unit[h][c] = m_rd * row_units + chunk_of[h][c] * 16 + kq * 4;
+        // scales of the first tile -> LDS copy 0
         if (s_loader)
-        {
-            sc_lds[tid] = sreg;
-            if (T > 1)
-                sreg = load_s(tile_at(1));
-        }
+            sc_lds[tid] = sfirst;
         lds_barrier();
 
-        // A_REGS: this wavefront's operand is read from LDS once and kept (16 VGPRs per group)
+        // A_REGS: this wavefront's operand and its constants are read from LDS once and kept
+        // (16 + 4 VGPRs per group); otherwise both are re-read for every tile
         uintx4 areg[A_REGS ? CPS : 1][4];
+        floatx4 ncreg[A_REGS ? CPS : 1];
         if (A_REGS)
         {
 #pragma unroll
             for (int c = 0; c < CPS; ++c)
+            {
 #pragma unroll
                 for (int j = 0; j < 4; ++j)
-                    areg[A_REGS ? c : 0][j] = lds[a_unit[0][c] + j * 4 * M];
+                    areg[A_REGS ? c : 0][j] = lds[a_unit[0][c] + j];
+                ncreg[A_REGS ? c : 0] = nc_lds[chunk_of[0][c] * 4 + kq];
+            }
         }
-
         auto a_op = [&](int h, int c, int j) -> uintx4 {
             if (A_REGS)
                 return areg[A_REGS ? c : 0][j];
-            return lds[a_unit[h][c] + j * 4 * M];
+            return lds[a_unit[h][c] + j];
+        };
+        auto ncorr = [&](int h, int c) -> floatx4 {
+            if (A_REGS)
+                return ncreg[A_REGS ? c : 0];
+            return nc_lds[chunk_of[h][c] * 4 + kq];
         };
 
-        // ---- constant part of every group sum, negated: ncorr[h][c][r] for m = 4*kq + r ---------------
-        floatx4 ncorr[H][CPS];
-        {
-            const half_t ce = (half_t)(-(1024.0f + (float)zp));
-            const half_t co = (half_t)(-16.0f * (64.0f + (float)zp));
-            const half8_t bconst = {ce, ce, co, co, ce, ce, co, co};
-#pragma unroll
-            for (int h = 0; h < H; ++h)
-#pragma unroll
-                for (int c = 0; c < CPS; ++c)
-                {
-                    floatx4 t = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                    for (int j = 0; j < 4; ++j)
-                        t = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, a_op(h, c, j)), bconst, t,
-                                                                   0, 0, 0);
-                    ncorr[h][c] = t;
-                }
-        }
-
-        // 0x64006400 in a scalar register, so that (w & mask) | magic is a single v_and_or_b32
-        // (an instruction can carry only one 32-bit literal)
-        uint32_t MAGIC;
-        asm("s_mov_b32 %0, 0x64006400" : "=s"(MAGIC));
+        // (w & mask) | magic as a single v_and_or_b32: the instruction takes no 32-bit literal and only one
+        // scalar operand, so the masks live in scalar registers and the magic number in a vector register
+        // (MAGIC is set at the top of the kernel, with every lane active)
 
         int local_tile = 0;
         // MFMAs of one pass h of a tile from register set wt, scales from LDS copy `par`, added to acc
@@ -197,7 +237,7 @@ namespace nnf
 #pragma unroll
             for (int c = 0; c < CPS; ++c)
             {
-                floatx4 t = ncorr[h][c];
+                floatx4 t = ncorr(h, c);
                 const uint32_t ww[4] = {wt[c].x, wt[c].y, wt[c].z, wt[c].w};
 #pragma unroll
                 for (int j = 0; j < 4; ++j)
@@ -205,10 +245,10 @@ namespace nnf
                     uint32_t w = ww[j];
                     uint32_t w8 = w >> 8;
                     uintx4 b;
-                    b.x = (w & 0x000F000Fu) | MAGIC;  // 1024 + (q0, q4)
-                    b.y = (w & 0x00F000F0u) | MAGIC;  // 1024 + 16 (q1, q5)
-                    b.z = (w8 & 0x000F000Fu) | MAGIC; // 1024 + (q2, q6)
-                    b.w = (w8 & 0x00F000F0u) | MAGIC; // 1024 + 16 (q3, q7)
+                    b.x = (w & MASK_LO) | MAGIC;  // 1024 + (q0, q4)
+                    b.y = (w & MASK_HI) | MAGIC;  // 1024 + 16 (q1, q5)
+                    b.z = (w8 & MASK_LO) | MAGIC; // 1024 + (q2, q6)
+                    b.w = (w8 & MASK_HI) | MAGIC; // 1024 + 16 (q3, q7)
                     t = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, a_op(h, c, j)),
                                                                __builtin_bit_cast(half8_t, b), t, 0, 0, 0);
                 }
@@ -229,12 +269,15 @@ namespace nnf
         // loop has no branch around a load (a load on one side of a branch makes the compiler wait for
         // all loads at the join).
         auto finish = [&](floatx4 acc, int par, auto put_s, auto get_s, int tile_s, auto get_w, int tile_w, int h_w,
-                          uintx4* w_free) {
-            float* rp = red + ((par * KS + wave) * 16 + kq * 4) * 16 + col;
-            rp[0] = acc.x;
-            rp[16] = acc.y;
-            rp[32] = acc.z;
-            rp[48] = acc.w;
+                          uintx4* w_free, auto last, int tile_cur) {
+            {
+                float* rp = red + par * red_copy + col * KSP + wave;
+                const float av[4] = {acc.x, acc.y, acc.z, acc.w};
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    if (kq * 4 + r < M)
+                        rp[(kq * 4 + r) * 16 * KSP] = av[r];
+            }
             // Order matters for the in-order load counter: the scale registers (loaded one tile ago) are
             // consumed first, then reloaded, and only then is the freed weight register set reloaded --
             // so waiting for the scales next time does not also wait for these weight loads.
@@ -251,26 +294,39 @@ namespace nnf
                 __builtin_amdgcn_sched_barrier(0);
             }
             lds_barrier(); // LDS only: the prefetched global loads stay in flight
-            // The sums are parked in LDS and written to Y after the last tile: a global store inside
-            // the loop would make later address arithmetic wait for it, and with it for every
-            // prefetched load issued before it (one in-order counter covers both).
-            if (tid < M * 16)
+            // Four lanes per output: each adds four of the KSP partial sums, then the quad is summed.
+            // Except after the last tile the sums are parked in LDS: a global store inside the loop
+            // would make later address arithmetic wait for it, and with it for every prefetched load
+            // issued before it (one in-order counter covers both).
+            if (tid < M * 64)
             {
-                const float* rr = red + par * KS * 256 + tid; // tid = m*16 + n
-                float v = 0.f;
-                for (int w = 0; w < KS; w += 4)
+                const int o = tid >> 2, q = tid & 3; // o = m*16 + n
+                floatx4 p4 = {0.f, 0.f, 0.f, 0.f};
+                if (q * 4 < KSP)
+                    p4 = *reinterpret_cast<const floatx4*>(red + par * red_copy + o * KSP + q * 4);
+                float v = quad_sum((p4.x + p4.y) + (p4.z + p4.w));
+                if (decltype(last)::value)
                 {
-                    // four independent reads per step (clamped: a repeated slot is not added)
-                    float p0 = rr[w * 256];
-                    float p1 = rr[min(w + 1, KS - 1) * 256];
-                    float p2 = rr[min(w + 2, KS - 1) * 256];
-                    float p3 = rr[min(w + 3, KS - 1) * 256];
-                    v += p0;
-                    v += (w + 1 < KS) ? p1 : 0.f;
-                    v += (w + 2 < KS) ? p2 : 0.f;
-                    v += (w + 3 < KS) ? p3 : 0.f;
+                    const int n = row0_of(tile_cur) + (o & 15);
+                    if (q == 0)
+                        Y[(size_t)(o >> 4) * N + n] = (half_t)v;
                 }
-                outb[local_tile * M * 16 + tid] = v;
+                else if (q == 0)
+                {
+                    outb[local_tile * M * 16 + o] = v;
+                }
+            }
+            if (decltype(last)::value)
+            {
+                // the sums parked by earlier tiles (written before the barrier above)
+                const int per_tile = M * 16;
+                for (int i = tid; i < local_tile * per_tile; i += blockDim.x)
+                {
+                    int lt = i / per_tile;
+                    int r = i - lt * per_tile;
+                    int n = min((tile0 + lt * stride) * 16, N - 16) + (r & 15); // per lane: no scalar row0_of here
+                    Y[(size_t)(r >> 4) * N + n] = (half_t)outb[i];
+                }
             }
             ++local_tile;
         };
@@ -288,31 +344,31 @@ namespace nnf
             for (; k + 3 < T; k += 2)
             {
                 floatx4 acc = compute(zero, w0, h0, 0);
-                finish(acc, 0, yes, yes, tile_at(k + 2), yes, tile_at(k + 2), 0, w0);
+                finish(acc, 0, yes, yes, tile_at(k + 2), yes, tile_at(k + 2), 0, w0, no, 0);
                 acc = compute(zero, w1, h0, 1);
-                finish(acc, 1, yes, yes, tile_at(k + 3), yes, tile_at(k + 3), 0, w1);
+                finish(acc, 1, yes, yes, tile_at(k + 3), yes, tile_at(k + 3), 0, w1, no, 0);
             }
             const int rest = T - k; // 1, 2 or 3
             if (rest == 3)
             {
                 floatx4 acc = compute(zero, w0, h0, 0);
-                finish(acc, 0, yes, yes, tile_at(k + 2), yes, tile_at(k + 2), 0, w0);
+                finish(acc, 0, yes, yes, tile_at(k + 2), yes, tile_at(k + 2), 0, w0, no, 0);
                 acc = compute(zero, w1, h0, 1);
-                finish(acc, 1, yes, no, 0, no, 0, 0, w1);
+                finish(acc, 1, yes, no, 0, no, 0, 0, w1, no, 0);
                 acc = compute(zero, w0, h0, 0);
-                finish(acc, 0, no, no, 0, no, 0, 0, w0);
+                finish(acc, 0, no, no, 0, no, 0, 0, w0, yes, tile_at(k + 2));
             }
             else if (rest == 2)
             {
                 floatx4 acc = compute(zero, w0, h0, 0);
-                finish(acc, 0, yes, no, 0, no, 0, 0, w0);
+                finish(acc, 0, yes, no, 0, no, 0, 0, w0, no, 0);
                 acc = compute(zero, w1, h0, 1);
-                finish(acc, 1, no, no, 0, no, 0, 0, w1);
+                finish(acc, 1, no, no, 0, no, 0, 0, w1, yes, tile_at(k + 1));
             }
             else
             {
                 floatx4 acc = compute(zero, w0, h0, 0);
-                finish(acc, 0, no, no, 0, no, 0, 0, w0);
+                finish(acc, 0, no, no, 0, no, 0, 0, w0, yes, tile_at(k));
             }
         }
         else
@@ -326,7 +382,7 @@ namespace nnf
                 load_w(tile_at(k + 1), 0, w0);
                 __builtin_amdgcn_sched_barrier(0);
                 acc = compute(acc, w1, h1, k & 1);
-                finish(acc, k & 1, yes, yes, tile_at(k + 2), yes, tile_at(k + 1), H - 1, w1);
+                finish(acc, k & 1, yes, yes, tile_at(k + 2), yes, tile_at(k + 1), H - 1, w1, no, 0);
             }
             if (T - k == 2)
             {
@@ -334,25 +390,12 @@ namespace nnf
                 load_w(tile_at(k + 1), 0, w0);
                 __builtin_amdgcn_sched_barrier(0);
                 acc = compute(acc, w1, h1, k & 1);
-                finish(acc, k & 1, yes, no, 0, yes, tile_at(k + 1), H - 1, w1);
+                finish(acc, k & 1, yes, no, 0, yes, tile_at(k + 1), H - 1, w1, no, 0);
                 ++k;
             }
             floatx4 acc = compute(zero, w0, h0, k & 1);
             acc = compute(acc, w1, h1, k & 1);
-            finish(acc, k & 1, no, no, 0, no, 0, 0, w1);
-        }
-
-        // ---- write Y ----------------------------------------------------------------------------
-        __syncthreads();
-        const int per_tile = M * 16;
-        for (int i = tid; i < local_tile * per_tile; i += blockDim.x)
-        {
-            int lt = i / per_tile;
-            int r = i - lt * per_tile;
-            int m = r >> 4;
-            int n = ((int)blockIdx.x + lt * stride) * 16 + (r & 15);
-            if (n < N)
-                Y[(size_t)m * N + n] = (half_t)outb[i];
+            finish(acc, k & 1, no, no, 0, no, 0, 0, w1, yes, tile_at(k));
         }
     }
 
@@ -393,9 +436,9 @@ namespace nnf
                 return p;
             // the A operand fits in registers up to two groups per wavefront (32 VGPRs)
             p.a_regs = p.cps <= 2 && p.h == 1;
-            const size_t a_bytes = (size_t)G * 16 * M * 16;
+            const size_t a_bytes = ((size_t)G * 16 + 1) * M * 16 + (size_t)G * 64;
             const size_t sc_bytes = 2 * (((size_t)16 * G * 2 + 15) & ~(size_t)15);
-            p.lds = a_bytes + sc_bytes + (size_t)2 * p.ks * 256 * 4;
+            p.lds = a_bytes + sc_bytes + (size_t)2 * M * 16 * ((p.ks + 3) & ~3) * 4;
             return p;
         }
 
@@ -435,7 +478,7 @@ namespace nnf
 
     bool w4a16_skinny_supported(int M, int N, int K)
     {
-        if (M < 1 || M > 16 || (K & 127))
+        if (M < 1 || M > 16 || (K & 127) || N < 16)
             return false;
         // the scale block of a tile is fetched in whole 16-byte pieces
         if (((size_t)N * (K >> 7) * 2) % 16 != 0 || (size_t)N * (K >> 7) * 2 < 16)
