@@ -241,11 +241,11 @@ def run_extra(torch, np, dev, lib, datagen, ops):
     n = k = 8192
     _, wq, s = datagen.w4a16_case(0, 1, n, k)
     twq, ts = dev_t(wq), dev_t(s)
-    ws = torch.empty(1 << 24, dtype=torch.uint8, device=dev)
     rows = []
     for m in (16, 128, 1024, 4096):
         a = dev_t(datagen.normal_f16(0, datagen.S_ACT, (m, k)))
         y = torch.empty((m, n), dtype=torch.float16, device=dev)
+        ws = torch.empty(max(lib.nnf_w4a16_gemm_workspace_bytes(m, n, k, GROUP), 256), dtype=torch.uint8, device=dev)
         us = time_us(lambda: ops.w4a16_gemm(a, twq, ts, out=y, workspace=ws), 20 if m <= 1024 else 8)
         fl = 2.0 * m * n * k
         rows.append({"M": m, "us": round(us, 2), "TFLOP/s": round(fl / us / 1e6, 1),
@@ -256,6 +256,7 @@ def run_extra(torch, np, dev, lib, datagen, ops):
     # configs[3]: W8A8, N = K = 8192
     _, _, w8, s_ch = datagen.w8a8_case(0, 1, n, k)
     tw8, tsch = dev_t(w8), dev_t(s_ch)
+    ws = torch.empty(max(lib.nnf_w8a8_gemm_workspace_bytes(4096, n, k), 256), dtype=torch.uint8, device=dev)
     rows = []
     for m in (1, 32, 512, 4096):
         a8 = dev_t(datagen.uniform_i8(0, datagen.S_A8, (m, k)))

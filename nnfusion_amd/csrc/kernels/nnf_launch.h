@@ -21,11 +21,12 @@ namespace nnf
     // true when one workgroup can hold the activations (M <= 16 rows of K) in LDS
     bool w4a16_skinny_supported(int M, int N, int K);
 
-    // MFMA GEMM (any M) with the fused RMSNorm prologue and bias / residual / SiLU-gate epilogues.
-    // workspace: M floats (the per-row rstd), needed when rms_gamma != nullptr.
+    // MFMA GEMM (any M) with the RMSNorm prologue and bias / residual / SiLU-gate epilogues.
+    // rms_ws: nnf::workspace::rms_rows(M, K) bytes, needed when rms_gamma != nullptr;
+    // partial_ws: nnf::workspace::gemm_partial_bytes(...) for the plan of the shape (may be 0 bytes).
     hipError_t launch_w4a16_gemm(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M,
                                  int N, int K, int zp, const void* rms_gamma, float rms_eps, const void* bias,
-                                 const void* residual, int act, void* workspace);
+                                 const void* residual, int act, void* rms_ws, void* partial_ws);
 
     // W8A8: acc != nullptr writes the raw int32 accumulators, otherwise Y = fp16(acc * s_tok * s_ch).
     hipError_t launch_w8a8(hipStream_t stream, const void* A, const void* s_tok, const void* W, const void* s_ch,
@@ -38,7 +39,8 @@ namespace nnf
         int force_path = 0;  // 1 = VALU GEMV, 2 = MFMA skinny, 3 = MFMA GEMM
         int skinny_cps = 0;  // chunks (groups of 128) per wavefront
         int skinny_wg_per_cu = 0;
-        int gemm_no_direct_loads = 0; // 1 = the register-staged GEMM kernel for every variant
+        int gemm_tile = 0;   // 1 + nnf::workspace::GemmTile
+        int gemm_splits = 0; // K ranges of the mid / small tile kernels
     };
     extern Tuning g_tuning;
 } // namespace nnf

@@ -1,75 +1,27 @@
-// fp16 x int4 (g128) GEMM for M > 16 on the gfx950 matrix cores (v_mfma_f32_32x32x16_f16).
+// fp16 x int4 (g128) GEMM for M > 16 on the gfx950 matrix cores: dispatcher, the big-tile
+// instantiations of the kernel template in w4a16_gemm_dl.h, the RMSNorm pre-pass and the split-K
+// reduction pass.
 //
 //   Y[M,N] = epilogue( prologue(A)[M,K] . ((Wq - zp) * S)^T )
 //
-// Workgroup tile 256 (M) x 256 (N) x 64 (K), eight wavefronts in a 2 (M) x 4 (N) arrangement, each
-// owning a 128 x 64 sub-tile = 4 x 2 MFMA tiles of 32 x 32 (128 fp32 accumulators per lane).  Two
-// wavefronts share a SIMD: while one waits for LDS operands or runs the int4 -> fp16 VALU work, the
-// other keeps the matrix core busy (one wavefront of 128 x 128 per SIMD left the MFMA pipe idle
-// for about half of the time).
-//   * A (fp16) and Wq (raw int4) tiles of the next K step are fetched global -> registers while
-//     the current step is computed from LDS; LDS is double buffered, one barrier per K step.
-//   * LDS layouts are XOR-swizzled at 16-byte granularity so that both the 128-bit stores and the
-//     128-bit MFMA operand reads are bank-conflict free.
-//   * int4 -> fp16 happens in registers right before the MFMA: (q | 0x6400) = 1024 + q, then one
-//     packed add (or fma for the nibble four bits up) gives the exact integer q - zp, one packed
-//     multiply applies the group scale.  A dequantised fragment feeds four MFMAs (the four M
-//     tiles of the wavefront).  The pair order of the unpacking, (q0,q4)(q1,q5)(q2,q6)(q3,q7), is
-//     matched by permuting the activations once while they are staged into LDS.
-//   * The K index inside a 64-wide tile is assigned to MFMA slots as k = 32*h + 8*s + e
-//     (h = lane / 32, s = MFMA step 0..3, e = element), so that a lane's 16 weight bytes of a tile
-//     row are one 128-bit LDS read and the matching activations are 16 contiguous bytes.
-//   * Fused prologue / epilogues (template flags): RMSNorm (per-row rstd from a small pre-pass,
-//     applied with gamma while staging A), bias, residual add, SiLU(gate) * up with the gate and
-//     up projections as two halves of the N tile.
-#include "nnf_device.h"
-#include "nnf_launch.h"
+//   * prologue: RMSNorm.  x * rsqrt(mean(x^2) + eps) * gamma is computed in fp32 and rounded to fp16 into
+//     scratch memory (the normalised activation tensor of the unfused graph); the GEMM then reads that.
+//   * epilogues: bias, residual add, SiLU(gate) * up with the gate and up projections as two halves of
+//     the N tile -- in the GEMM kernel, or in the reduction pass when K is split.
+//   * the tile shape and the number of K ranges follow nnf::workspace::plan_w4a16_gemm: 256 x 256 tiles
+//     when they fill the GPU, otherwise 128 x 128 or 64 x 256 tiles with K split across workgroups so
+//     that about two workgroups per CU are in flight.
+#include "w4a16_gemm_dl.h"
+
+#include "../nnf_workspace.h"
 
 #include <algorithm>
 
 namespace nnf
 {
-    namespace gemm
-    {
-        constexpr int BM = 256, BN = 256, BK = 64;
-        constexpr int THREADS = 512;            // 8 wavefronts: 2 along M x 4 along N
-        constexpr int TM = 4, TN = 2;           // 32 x 32 MFMA tiles per wavefront along M, N
-        constexpr int NA = BM * BK * 2 / 16 / THREADS; // 16-byte pieces of the A tile per thread (4)
-        constexpr int A_TILE_BYTES = BM * BK * 2;     // 32 KiB
-        constexpr int W_TILE_BYTES = BN * BK / 2;     // 8 KiB
-        constexpr int STAGE_BYTES = A_TILE_BYTES + W_TILE_BYTES;
-        constexpr int LDS_BYTES = 2 * STAGE_BYTES;    // 80 KiB
-
-        // byte offset of 16-byte piece p (0..7) of row r in the swizzled A tile
-        __device__ __forceinline__ int a_off(int r, int p)
-        {
-            return r * 128 + ((p ^ ((r >> 1) & 7)) << 4);
-        }
-        // byte offset of 16-byte piece h (0..1) of row r in the swizzled W tile
-        __device__ __forceinline__ int w_off(int r, int h)
-        {
-            return r * 32 + ((h ^ ((r >> 3) & 1)) << 4);
-        }
-    } // namespace gemm
-
-    struct GemmParams
-    {
-        const half_t* A;
-        const uint8_t* Wq;
-        const half_t* S;
-        half_t* Y;
-        int M, N, K, zp;
-        int ldy;              // row stride of Y (= N of the output)
-        int up_row_offset;    // GATE: weight row of the up projection that pairs with gate row 0
-        const float* rstd;    // RMS: per-row 1/sqrt(mean(x^2)+eps)
-        const half_t* gamma;  // RMS: [K]
-        const half_t* bias;   // BIAS: [N]
-        const half_t* residual; // RESID: [M, ldy]
-    };
-
-    // one row of rstd per wavefront: rstd[m] = rsqrt(mean_k(x[m,k]^2) + eps)
-    __global__ __launch_bounds__(256) void rms_rstd_kernel(const half_t* __restrict__ X, float* __restrict__ rstd,
-                                                           int M, int K, float eps)
+    // one row per wavefront: Xn[m, :] = fp16( x * rsqrt(mean_k(x^2) + eps) * gamma )
+    __global__ __launch_bounds__(256) void rms_norm_kernel(const half_t* __restrict__ X, const half_t* __restrict__ gamma,
+                                                           half_t* __restrict__ Xn, int M, int K, float eps)
     {
         const int lane = threadIdx.x & 63;
         const int m = blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -85,627 +37,158 @@ namespace nnf
             for (int j = 0; j < 4; ++j)
             {
                 half2_t h = as_half2(vv[j]);
-                float a = (float)h.x, b = (float)h.y;
-                ss = __builtin_fmaf(a, a, ss);
-                ss = __builtin_fmaf(b, b, ss);
+                ss += (float)h.x * (float)h.x + (float)h.y * (float)h.y;
             }
         }
         ss = wave_sum(ss);
-        if (lane == 0)
-            rstd[m] = 1.0f / __builtin_sqrtf(ss / (float)K + eps);
-    }
-
-    template <bool GATE, bool RMS, bool BIAS, bool RESID>
-    __global__ __launch_bounds__(512) void w4a16_gemm_kernel(GemmParams p)
-    {
-        using namespace gemm;
-        extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-        const int tid = threadIdx.x;
-        const int lane = tid & 63;
-        const int wave = tid >> 6;
-        const int wm = wave >> 2, wn = wave & 3;
-        const int l32 = lane & 31, h = lane >> 5;
-        const int K = p.K;
-        const int G = K >> 7;
-        constexpr int BN_OUT = GATE ? BN / 2 : BN; // output columns of a workgroup tile
-
-        // XCD-aware tile order: workgroup ids are dealt round-robin to the 8 XCDs (each with its own
-        // L2); give each XCD a contiguous run of tiles, and walk tiles M-fastest so that tiles that
-        // are resident together share the weight panel.
-        const int tiles_m = (p.M + BM - 1) / BM;
-        const int tiles_n = (p.N + BN_OUT - 1) / BN_OUT;
-        const int n_wg = tiles_m * tiles_n;
-        int pid = blockIdx.x;
+        const float rstd = 1.0f / __builtin_sqrtf(ss / (float)K + eps);
+        const uintx4* grow = reinterpret_cast<const uintx4*>(gamma);
+        uintx4* out = reinterpret_cast<uintx4*>(Xn + (size_t)m * K);
+        for (int i = lane; i < (K >> 3); i += 64)
         {
-            const int per_xcd = (n_wg + 7) >> 3;
-            const int full = n_wg - (per_xcd - 1) * 8; // XCDs that own per_xcd tiles (1..8)
-            const int xcd = pid & 7, idx = pid >> 3;
-            pid = (xcd < full) ? xcd * per_xcd + idx : full * per_xcd + (xcd - full) * (per_xcd - 1) + idx;
-        }
-        const int tm = pid % tiles_m, tn = pid / tiles_m;
-        const int m0 = tm * BM, n0 = tn * BN_OUT;
-
-        // ---- global -> register staging maps -------------------------------------------------------
-        // A: 2048 pieces of 16 B, NA per thread: row = i*64 + tid/8, piece = tid%8
-        const int a_p = tid & 7;
-        const int a_r0 = tid >> 3;
-        const half_t* a_src[NA];
-        int a_dst[NA];
-        float a_rstd[RMS ? NA : 1];
+            uintx4 v = row[i], g = grow[i], o;
+            const uint32_t vv[4] = {v.x, v.y, v.z, v.w};
+            const uint32_t gg[4] = {g.x, g.y, g.z, g.w};
+            uint32_t oo[4];
 #pragma unroll
-        for (int i = 0; i < NA; ++i)
-        {
-            int r = i * (THREADS / 8) + a_r0;
-            int gm = min(m0 + r, p.M - 1);
-            a_src[i] = p.A + (size_t)gm * K + a_p * 8;
-            a_dst[i] = a_off(r, a_p);
-            if (RMS)
-                a_rstd[i] = p.rstd[gm];
-        }
-        // W: 512 pieces of 16 B, one per thread: row = tid/2, piece = tid%2
-        const int w_h = tid & 1;
-        const uint8_t* w_src[1];
-        int w_dst[1];
-#pragma unroll
-        for (int i = 0; i < 1; ++i)
-        {
-            int r = tid >> 1;
-            int gn;
-            if (GATE)
-                gn = (r < BN / 2) ? (n0 + r) : (p.up_row_offset + n0 + (r - BN / 2));
-            else
-                gn = n0 + r;
-            // rows past the end of N are clamped (their results are never stored)
-            gn = GATE ? min(gn, p.up_row_offset + p.N - 1) : min(gn, p.N - 1);
-            w_src[i] = p.Wq + (size_t)gn * (K >> 1) + w_h * 16;
-            w_dst[i] = A_TILE_BYTES + w_off(r, w_h);
-        }
-
-        // ---- per-lane fragment addresses in LDS ------------------------------------------------------
-        int a_frag[4]; // row part of the A fragment address for M tile i (piece added per step)
-        int a_swz[4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-        {
-            int r = wm * 128 + i * 32 + l32;
-            a_frag[i] = r * 128;
-            a_swz[i] = (r >> 1) & 7;
-        }
-        int w_frag[TN];
-        size_t s_idx[TN];        // element index of this lane's column scale, group 0, in N tile j
-        int col_out[TN];         // output column of N tile j
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-        {
-            int r; // row of the W tile
-            int gn;
-            if (GATE)
+            for (int j = 0; j < 4; ++j)
             {
-                int half_sel = j; // 0 = gate, 1 = up
-                int c = wn * 32 + l32;
-                r = half_sel * (BN / 2) + c;
-                gn = half_sel ? (p.up_row_offset + n0 + c) : (n0 + c);
-                gn = min(gn, p.up_row_offset + p.N - 1);
-                col_out[j] = n0 + c;
+                half2_t x = as_half2(vv[j]), w = as_half2(gg[j]), r;
+                r.x = (half_t)((float)x.x * rstd * (float)w.x);
+                r.y = (half_t)((float)x.y * rstd * (float)w.y);
+                oo[j] = as_u32(r);
             }
-            else
-            {
-                r = wn * 64 + j * 32 + l32;
-                gn = min(n0 + r, p.N - 1);
-                col_out[j] = n0 + r;
-            }
-            w_frag[j] = A_TILE_BYTES + w_off(r, h);
-            s_idx[j] = (size_t)gn * G;
-        }
-
-        floatx16 acc[TM][TN];
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-            for (int j = 0; j < TN; ++j)
-#pragma unroll
-                for (int e = 0; e < 16; ++e)
-                    acc[i][j][e] = 0.f;
-
-        const DequantConst dq = make_dequant_const(p.zp);
-        uint32_t MAGIC;
-        asm("s_mov_b32 %0, 0x64006400" : "=s"(MAGIC));
-
-        // Group scales are fetched one group (two K steps) ahead as the aligned 32-bit word that
-        // holds the fp16 (a 16-bit load would be widened at its point of use and force a wait for
-        // every younger load, i.e. the tile prefetch).
-        const uint32_t* s32 = reinterpret_cast<const uint32_t*>(p.S);
-        uint32_t s_nxt[TN];
-        auto load_scales = [&](int g) {
-            g = min(g, G - 1);
-#pragma unroll
-            for (int j = 0; j < TN; ++j)
-                s_nxt[j] = s32[(s_idx[j] + g) >> 1];
-        };
-
-        uintx4 a_reg[NA], w_reg[1], g_reg;
-        auto load_global = [&](int kt) {
-            const int k0 = kt * BK;
-            if (RMS)
-                g_reg = *reinterpret_cast<const uintx4*>(p.gamma + k0 + a_p * 8);
-#pragma unroll
-            for (int i = 0; i < NA; ++i)
-                a_reg[i] = *reinterpret_cast<const uintx4*>(a_src[i] + k0);
-            w_reg[0] = *reinterpret_cast<const uintx4*>(w_src[0] + (k0 >> 1));
-        };
-        auto store_lds = [&](int kt, int stage) {
-            uint8_t* base = smem + stage * STAGE_BYTES;
-            (void)kt;
-            const uintx4 g4 = g_reg;
-#pragma unroll
-            for (int i = 0; i < NA; ++i)
-            {
-                uintx4 a = a_reg[i];
-                if (RMS)
-                {
-                    // x * rstd * gamma in fp32, rounded to fp16 (the normalised activation tensor
-                    // of the unfused graph is fp16)
-                    const uint32_t av[4] = {a.x, a.y, a.z, a.w};
-                    const uint32_t gv[4] = {g4.x, g4.y, g4.z, g4.w};
-                    uint32_t ov[4];
-#pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                    {
-                        half2_t x = as_half2(av[e]), g = as_half2(gv[e]);
-                        half2_t o;
-                        o.x = (half_t)((float)x.x * a_rstd[i] * (float)g.x);
-                        o.y = (half_t)((float)x.y * a_rstd[i] * (float)g.y);
-                        ov[e] = as_u32(o);
-                    }
-                    a = uintx4{ov[0], ov[1], ov[2], ov[3]};
-                }
-                *reinterpret_cast<uintx4*>(base + a_dst[i]) = permute_a8(a);
-            }
-            *reinterpret_cast<uintx4*>(base + w_dst[0]) = w_reg[0];
-        };
-
-        const int KT = K / BK;
-        load_scales(0);
-        load_global(0);
-        store_lds(0, 0);
-        __syncthreads();
-
-        half2_t sc[TN]; // group scale of this lane's column in each N tile, both halves equal
-        for (int kt = 0; kt < KT; ++kt)
-        {
-            const int stage = kt & 1;
-            if ((kt & 1) == 0)
-            {
-                const int g = kt >> 1;
-#pragma unroll
-                for (int j = 0; j < TN; ++j)
-                {
-                    uint32_t bits = s_nxt[j] >> ((((uint32_t)s_idx[j] + (uint32_t)g) & 1u) << 4);
-                    half_t s = as_half2(bits).x;
-                    sc[j] = half2_t{s, s};
-                }
-                load_scales(g + 1);
-            }
-            if (kt + 1 < KT)
-                load_global(kt + 1);
-            const uint8_t* base = smem + stage * STAGE_BYTES;
-            uintx4 wq[TN];
-#pragma unroll
-            for (int j = 0; j < TN; ++j)
-                wq[j] = *reinterpret_cast<const uintx4*>(base + w_frag[j]);
-#pragma unroll
-            for (int s = 0; s < 4; ++s)
-            {
-                half8_t af[4];
-#pragma unroll
-                for (int i = 0; i < 4; ++i)
-                {
-                    int pc = (h * 4 + s) ^ a_swz[i];
-                    af[i] = *reinterpret_cast<const half8_t*>(base + a_frag[i] + (pc << 4));
-                }
-#pragma unroll
-                for (int j = 0; j < TN; ++j)
-                {
-                    uint32_t w = (s == 0) ? wq[j].x : (s == 1) ? wq[j].y : (s == 2) ? wq[j].z : wq[j].w;
-                    uint32_t w8 = w >> 8;
-                    half2_t q0 = as_half2((w & 0x000F000Fu) | MAGIC) + dq.c_lo;
-                    half2_t q1 = __builtin_elementwise_fma(as_half2((w & 0x00F000F0u) | MAGIC), dq.sixteenth, dq.c_hi);
-                    half2_t q2 = as_half2((w8 & 0x000F000Fu) | MAGIC) + dq.c_lo;
-                    half2_t q3 = __builtin_elementwise_fma(as_half2((w8 & 0x00F000F0u) | MAGIC), dq.sixteenth, dq.c_hi);
-                    uintx4 bw;
-                    bw.x = as_u32(q0 * sc[j]);
-                    bw.y = as_u32(q1 * sc[j]);
-                    bw.z = as_u32(q2 * sc[j]);
-                    bw.w = as_u32(q3 * sc[j]);
-                    half8_t bf = __builtin_bit_cast(half8_t, bw);
-#pragma unroll
-                    for (int i = 0; i < 4; ++i)
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf, acc[i][j], 0, 0, 0);
-                }
-            }
-            if (kt + 1 < KT)
-                store_lds(kt + 1, stage ^ 1);
-            __syncthreads();
-        }
-
-        // ---- epilogue ---------------------------------------------------------------------------------
-        // D layout of a 32x32 tile: lane (col = l32, h), element e: row = 8*(e/4) + 4*h + (e%4)
-        constexpr int NJ = GATE ? 1 : TN;
-#pragma unroll
-        for (int j = 0; j < NJ; ++j)
-        {
-            const int n = col_out[j];
-            if (n >= p.N)
-                continue;
-            float bias = 0.f;
-            if (BIAS)
-                bias = (float)p.bias[n];
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-            {
-#pragma unroll
-                for (int e = 0; e < 16; ++e)
-                {
-                    const int m = m0 + wm * 128 + i * 32 + 8 * (e >> 2) + 4 * h + (e & 3);
-                    if (m >= p.M)
-                        continue;
-                    float v;
-                    if (GATE)
-                    {
-                        // SiLU(gate) * up on the values the unfused graph would see: both
-                        // projections rounded to fp16 first
-                        float g = (float)(half_t)acc[i][j][e];
-                        float u = (float)(half_t)acc[i][j + 1][e];
-                        v = g * (1.0f / (1.0f + __expf(-g))) * u;
-                    }
-                    else
-                    {
-                        v = acc[i][j][e];
-                    }
-                    if (BIAS)
-                        v = (float)(half_t)v + bias;
-                    if (RESID)
-                        v = (float)(half_t)v + (float)p.residual[(size_t)m * p.ldy + n];
-                    p.Y[(size_t)m * p.ldy + n] = (half_t)v;
-                }
-            }
+            o.x = oo[0];
+            o.y = oo[1];
+            o.z = oo[2];
+            o.w = oo[3];
+            out[i] = o;
         }
     }
 
-    // -------------------------------------------------------------------------------------------------
-    // The same GEMM with asynchronous global -> LDS loads (global_load_lds_dwordx4: no register staging,
-    // no LDS store instructions) and a three-stage LDS ring, so that the operands of two K steps are in
-    // flight while a K step is computed.  Used whenever the activations need no rewriting on the way in
-    // (every variant except the RMSNorm prologue).
-    //   * A wavefront-wide direct load fills 1 KiB of consecutive LDS; the XOR swizzle is obtained by
-    //     choosing which 16-byte piece of global memory each lane fetches.
-    //   * Nothing can be permuted on the way, so the activations stay in natural K order and the
-    //     weights are unpacked in natural order too: v_perm_b32 copies byte i of a word (nibbles 2i,
-    //     2i+1) into bytes 0 and 2, one v_and_or_b32 makes (1024 + q_2i, 1024 + 16 q_2i+1), one packed fma
-    //     with the constants (1, 1/16) and (-(1024+zp), -(64+zp)) gives the exact (q - zp) pair, one packed
-    //     multiply applies the group scale: 16 VALU operations per 8 weights, feeding four MFMAs.
-    //   * One barrier per K step: after it, every wavefront's loads for this step have landed and every
-    //     wavefront has finished reading the stage that is about to be refilled.
-    namespace gemm_dl
-    {
-        constexpr int BM = 256, BN = 256, BK = 64;
-        constexpr int THREADS = 512;  // 8 wavefronts: 2 along M x 4 along N
-        constexpr int TM = 4, TN = 2; // 32 x 32 MFMA tiles per wavefront along M, N
-        constexpr int STAGES = 3;
-        constexpr int A_TILE_BYTES = BM * BK * 2; // 32 KiB
-        constexpr int W_TILE_BYTES = BN * BK / 2; // 8 KiB
-        constexpr int STAGE_BYTES = A_TILE_BYTES + W_TILE_BYTES;
-        constexpr int LDS_BYTES = STAGES * STAGE_BYTES; // 120 KiB
-        constexpr int A_LOADS = A_TILE_BYTES / 1024 / 8;  // wavefront-wide loads of the A tile per wavefront (4)
-        constexpr int TILE_LOADS = A_LOADS + 1;           // plus one for the W tile
-
-        // s_waitcnt with only the vector-memory counter set (gfx9 encoding: vmcnt = bits 3:0 and 15:14)
-        constexpr int vmcnt_imm(int n) { return (n & 0xF) | ((n >> 4) << 14) | (0x7 << 4) | (0xF << 8); }
-    } // namespace gemm_dl
-
+    // Y[m, n] = epilogue( sum_s partial[s][m][n] ); four consecutive columns per thread.
+    // GATE: partial columns [0, N) are the gate, [N, 2N) the up projection.
     template <bool GATE, bool BIAS, bool RESID>
-    __global__ __launch_bounds__(512) void w4a16_gemm_dl_kernel(GemmParams p)
+    __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ partial, int splits, int M,
+                                                                int N, int ld_partial, const half_t* __restrict__ bias,
+                                                                const half_t* __restrict__ residual, half_t* __restrict__ Y,
+                                                                int ldy)
     {
-        using namespace gemm_dl;
-        extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-        const int tid = threadIdx.x;
-        const int lane = tid & 63;
-        const int wave = tid >> 6;
-        const int wm = wave >> 2, wn = wave & 3;
-        const int l32 = lane & 31, h = lane >> 5;
-        const int K = p.K;
-        const int G = K >> 7;
-        constexpr int BN_OUT = GATE ? BN / 2 : BN;
-
-        const int tiles_m = (p.M + BM - 1) / BM;
-        const int tiles_n = (p.N + BN_OUT - 1) / BN_OUT;
-        const int n_wg = tiles_m * tiles_n;
-        int pid = blockIdx.x;
+        const int quads = (N + 3) >> 2;
+        const long long t = (long long)blockIdx.x * 256 + threadIdx.x;
+        if (t >= (long long)M * quads)
+            return;
+        const int m = (int)(t / quads);
+        const int n = (int)(t - (long long)m * quads) * 4;
+        const size_t plane = (size_t)M * ld_partial;
+        const float* src = partial + (size_t)m * ld_partial + n;
+        // ld_partial and n are multiples of 4 when N is; otherwise fall back to scalar accesses
+        const bool vec = ((ld_partial | N) & 3) == 0;
+        float a[4] = {0.f, 0.f, 0.f, 0.f}, u[4] = {0.f, 0.f, 0.f, 0.f};
+        for (int s = 0; s < splits; ++s)
         {
-            // contiguous run of tiles per XCD (workgroup ids are dealt round-robin to the 8 XCDs)
-            const int per_xcd = (n_wg + 7) >> 3;
-            const int full = n_wg - (per_xcd - 1) * 8;
-            const int xcd = pid & 7, idx = pid >> 3;
-            pid = (xcd < full) ? xcd * per_xcd + idx : full * per_xcd + (xcd - full) * (per_xcd - 1) + idx;
-        }
-        const int tm = pid % tiles_m, tn = pid / tiles_m;
-        const int m0 = tm * BM, n0 = tn * BN_OUT;
-
-        // ---- direct-load maps -------------------------------------------------------------------------
-        // A: wavefront w, load i fills LDS rows (w*4 + i)*8 .. +7; lane l lands at (row = .. + l/8, slot = l%8)
-        // and therefore fetches piece  slot ^ ((row >> 1) & 7)  of that row.
-        const half_t* a_src[A_LOADS];
-#pragma unroll
-        for (int i = 0; i < A_LOADS; ++i)
-        {
-            int row = (wave * A_LOADS + i) * 8 + (lane >> 3);
-            int piece = (lane & 7) ^ ((row >> 1) & 7);
-            a_src[i] = p.A + (size_t)min(m0 + row, p.M - 1) * K + piece * 8;
-        }
-        // W: wavefront w fills LDS rows w*32 .. +31 (32 B each); lane l lands at (row = w*32 + l/2, slot = l%2)
-        const uint8_t* w_src;
-        {
-            int row = wave * 32 + (lane >> 1);
-            int piece = (lane & 1) ^ ((row >> 3) & 1);
-            int gn;
-            if (GATE)
-                gn = (row < BN / 2) ? (n0 + row) : (p.up_row_offset + n0 + (row - BN / 2));
-            else
-                gn = n0 + row;
-            gn = GATE ? min(gn, p.up_row_offset + p.N - 1) : min(gn, p.N - 1);
-            w_src = p.Wq + (size_t)gn * (K >> 1) + piece * 16;
-        }
-        auto issue_tile_loads = [&](int kt, int stage) {
-            uint8_t* base = smem + stage * STAGE_BYTES;
-            const int k0 = kt * BK;
-#pragma unroll
-            for (int i = 0; i < A_LOADS; ++i)
-                __builtin_amdgcn_global_load_lds(
-                    (const void __attribute__((address_space(1)))*)(a_src[i] + k0),
-                    (void __attribute__((address_space(3)))*)(base + (wave * A_LOADS + i) * 1024), 16, 0, 0);
-            __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1)))*)(w_src + (k0 >> 1)),
-                                             (void __attribute__((address_space(3)))*)(base + A_TILE_BYTES + wave * 1024),
-                                             16, 0, 0);
-        };
-
-        // ---- per-lane fragment addresses in LDS ------------------------------------------------------
-        int a_frag[TM], a_swz[TM];
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-        {
-            int r = wm * 128 + i * 32 + l32;
-            a_frag[i] = r * 128;
-            a_swz[i] = (r >> 1) & 7;
-        }
-        int w_frag[TN];
-        size_t s_idx[TN];
-        int col_out[TN];
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-        {
-            int r, gn;
-            if (GATE)
+            const float* ps = src + (size_t)s * plane;
+            if (vec)
             {
-                int c = wn * 32 + l32;
-                r = j * (BN / 2) + c; // j = 0: gate, 1: up
-                gn = j ? (p.up_row_offset + n0 + c) : (n0 + c);
-                gn = min(gn, p.up_row_offset + p.N - 1);
-                col_out[j] = n0 + c;
-            }
-            else
-            {
-                r = wn * 64 + j * 32 + l32;
-                gn = min(n0 + r, p.N - 1);
-                col_out[j] = n0 + r;
-            }
-            w_frag[j] = A_TILE_BYTES + r * 32 + ((h ^ ((r >> 3) & 1)) << 4);
-            s_idx[j] = (size_t)gn * G;
-        }
-
-        floatx16 acc[TM][TN];
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-            for (int j = 0; j < TN; ++j)
-#pragma unroll
-                for (int e = 0; e < 16; ++e)
-                    acc[i][j][e] = 0.f;
-
-        // constants of the unpacking; kept opaque so that each lands in the register class the VOP3
-        // encodings need (one scalar operand per instruction, no 32-bit literals)
-        uint32_t MASK, MAGIC, SEL[4];
-        asm("s_mov_b32 %0, 0x00F0000F" : "=s"(MASK));
-        asm volatile("v_mov_b32 %0, 0x64006400" : "=v"(MAGIC));
-        asm("s_mov_b32 %0, 0x0c000c00" : "=s"(SEL[0]));
-        asm("s_mov_b32 %0, 0x0c010c01" : "=s"(SEL[1]));
-        asm("s_mov_b32 %0, 0x0c020c02" : "=s"(SEL[2]));
-        asm("s_mov_b32 %0, 0x0c030c03" : "=s"(SEL[3]));
-        const half2_t dq_mul = half2_t{(half_t)1.0f, (half_t)0.0625f};
-        const half2_t dq_add = half2_t{(half_t)(-(1024.0f + (float)p.zp)), (half_t)(-(64.0f + (float)p.zp))};
-
-        // group scales, fetched one group (two K steps) ahead as the aligned 32-bit word holding the fp16
-        const uint32_t* s32 = reinterpret_cast<const uint32_t*>(p.S);
-        uint32_t s_nxt[TN];
-        auto load_scales = [&](int g) {
-            g = min(g, G - 1);
-#pragma unroll
-            for (int j = 0; j < TN; ++j)
-                s_nxt[j] = s32[(s_idx[j] + g) >> 1];
-        };
-        half2_t sc[TN];
-        auto take_scales = [&](int g) {
-#pragma unroll
-            for (int j = 0; j < TN; ++j)
-            {
-                uint32_t bits = s_nxt[j] >> ((((uint32_t)s_idx[j] + (uint32_t)g) & 1u) << 4);
-                half_t s = as_half2(bits).x;
-                sc[j] = half2_t{s, s};
-            }
-        };
-
-        auto compute = [&](int stage) {
-            const uint8_t* base = smem + stage * STAGE_BYTES;
-            uintx4 wq[TN];
-#pragma unroll
-            for (int j = 0; j < TN; ++j)
-                wq[j] = *reinterpret_cast<const uintx4*>(base + w_frag[j]);
-#pragma unroll
-            for (int s = 0; s < 4; ++s)
-            {
-                half8_t af[TM];
-#pragma unroll
-                for (int i = 0; i < TM; ++i)
-                    af[i] = *reinterpret_cast<const half8_t*>(base + a_frag[i] + ((((h << 2) + s) ^ a_swz[i]) << 4));
-#pragma unroll
-                for (int j = 0; j < TN; ++j)
+                floatx4 v = *reinterpret_cast<const floatx4*>(ps);
+                a[0] += v.x, a[1] += v.y, a[2] += v.z, a[3] += v.w;
+                if (GATE)
                 {
-                    const uint32_t w = (s == 0) ? wq[j].x : (s == 1) ? wq[j].y : (s == 2) ? wq[j].z : wq[j].w;
-                    uint32_t bw[4];
-#pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                    {
-                        uint32_t x = __builtin_amdgcn_perm(w, w, SEL[e]);        // bytes (b_e, 0, b_e, 0)
-                        half2_t y = as_half2((x & MASK) | MAGIC);                // (1024 + q_2e, 1024 + 16 q_2e+1)
-                        half2_t z = __builtin_elementwise_fma(y, dq_mul, dq_add); // (q_2e - zp, q_2e+1 - zp)
-                        bw[e] = as_u32(z * sc[j]);
-                    }
-                    half8_t bf = __builtin_bit_cast(half8_t, uintx4{bw[0], bw[1], bw[2], bw[3]});
-#pragma unroll
-                    for (int i = 0; i < TM; ++i)
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf, acc[i][j], 0, 0, 0);
+                    floatx4 w = *reinterpret_cast<const floatx4*>(ps + N);
+                    u[0] += w.x, u[1] += w.y, u[2] += w.z, u[3] += w.w;
                 }
             }
-        };
-
-        // ---- K loop: stages kt % 3; loads run two K steps ahead -------------------------------------------
-        const int KT = K / BK; // even (K % 128 == 0)
-        load_scales(0);
-        issue_tile_loads(0, 0);
-        issue_tile_loads(1, 1);
-        // Vector-memory operations complete in order.  Before the barrier of step kt a wavefront waits
-        // until at most the operations it issued during step kt-1 are outstanding: then its own loads
-        // for step kt (issued during step kt-2) have landed.  Even steps issue the scale loads (TN) and a
-        // tile (TILE_LOADS), odd steps a tile only.
-        int stage = 0;
-        for (int kt = 0; kt < KT; kt += 2)
-        {
-            // even step
-            __builtin_amdgcn_s_waitcnt(vmcnt_imm(TILE_LOADS));
-            __builtin_amdgcn_s_barrier();
-            take_scales(kt >> 1);
-            load_scales((kt >> 1) + 1);
+            else
             {
-                const int nk = min(kt + 2, KT - 1); // past the end: reload a valid tile into the free stage
-                int st = stage + 2;
-                st = st >= STAGES ? st - STAGES : st;
-                issue_tile_loads(nk, st);
+                for (int j = 0; j < 4; ++j)
+                    if (n + j < N)
+                    {
+                        a[j] += ps[j];
+                        if (GATE)
+                            u[j] += ps[N + j];
+                    }
             }
-            compute(stage);
-            stage = stage + 1 == STAGES ? 0 : stage + 1;
-            // odd step
-            __builtin_amdgcn_s_waitcnt(vmcnt_imm(TILE_LOADS + TN));
-            __builtin_amdgcn_s_barrier();
-            {
-                const int nk = min(kt + 3, KT - 1);
-                int st = stage + 2;
-                st = st >= STAGES ? st - STAGES : st;
-                issue_tile_loads(nk, st);
-            }
-            compute(stage);
-            stage = stage + 1 == STAGES ? 0 : stage + 1;
         }
-        __builtin_amdgcn_s_waitcnt(vmcnt_imm(0)); // drain the tail loads before the LDS goes away
-
-        // ---- epilogue ---------------------------------------------------------------------------------
-        // D layout of a 32x32 tile: lane (col = l32, h), element e: row = 8*(e/4) + 4*h + (e%4)
-        constexpr int NJ = GATE ? 1 : TN;
-#pragma unroll
-        for (int j = 0; j < NJ; ++j)
+        for (int j = 0; j < 4; ++j)
         {
-            const int n = col_out[j];
-            if (n >= p.N)
-                continue;
-            float bias = 0.f;
+            if (n + j >= N)
+                break;
+            float v = a[j];
+            if (GATE)
+            {
+                float g = (float)(half_t)a[j];
+                float up = (float)(half_t)u[j];
+                v = g * (1.0f / (1.0f + __expf(-g))) * up;
+            }
             if (BIAS)
-                bias = (float)p.bias[n];
-#pragma unroll
-            for (int i = 0; i < TM; ++i)
-            {
-#pragma unroll
-                for (int e = 0; e < 16; ++e)
-                {
-                    const int m = m0 + wm * 128 + i * 32 + 8 * (e >> 2) + 4 * h + (e & 3);
-                    if (m >= p.M)
-                        continue;
-                    float v;
-                    if (GATE)
-                    {
-                        float g = (float)(half_t)acc[i][0][e];
-                        float u = (float)(half_t)acc[i][1][e];
-                        v = g * (1.0f / (1.0f + __expf(-g))) * u;
-                    }
-                    else
-                    {
-                        v = acc[i][j][e];
-                    }
-                    if (BIAS)
-                        v = (float)(half_t)v + bias;
-                    if (RESID)
-                        v = (float)(half_t)v + (float)p.residual[(size_t)m * p.ldy + n];
-                    p.Y[(size_t)m * p.ldy + n] = (half_t)v;
-                }
-            }
+                v = (float)(half_t)v + (float)bias[n + j];
+            if (RESID)
+                v = (float)(half_t)v + (float)residual[(size_t)m * ldy + n + j];
+            Y[(size_t)m * ldy + n + j] = (half_t)v;
         }
     }
 
     namespace
     {
-        template <bool GATE, bool RMS, bool BIAS, bool RESID>
-        hipError_t launch_gemm_variant(hipStream_t stream, const GemmParams& p)
+        template <bool GATE, bool BIAS, bool RESID>
+        hipError_t launch_reduce(hipStream_t stream, const GemmParams& p)
         {
-            using namespace gemm;
-            constexpr int BN_OUT = GATE ? BN / 2 : BN;
-            const int tiles_m = (p.M + BM - 1) / BM;
-            const int tiles_n = (p.N + BN_OUT - 1) / BN_OUT;
-            static bool attr_set = false;
-            if (!attr_set)
-            {
-                hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&w4a16_gemm_kernel<GATE, RMS, BIAS, RESID>),
-                                                   hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
-                if (e != hipSuccess)
-                    return e;
-                attr_set = true;
-            }
-            hipLaunchKernelGGL((w4a16_gemm_kernel<GATE, RMS, BIAS, RESID>), dim3(tiles_m * tiles_n), dim3(THREADS), LDS_BYTES,
-                               stream, p);
+            const long long threads = (long long)p.M * ((p.N + 3) >> 2);
+            hipLaunchKernelGGL((splitk_reduce_kernel<GATE, BIAS, RESID>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0,
+                               stream, (const float*)p.partial, p.splits, p.M, p.N, p.ld_partial, p.bias, p.residual, p.Y,
+                               p.ldy);
             return hipGetLastError();
         }
-        template <bool GATE, bool BIAS, bool RESID>
-        hipError_t launch_gemm_dl_variant(hipStream_t stream, const GemmParams& p)
+
+        hipError_t launch_reduce_any(hipStream_t stream, const GemmParams& p, bool gate, bool hb, bool hr)
         {
-            using namespace gemm_dl;
-            constexpr int BN_OUT = GATE ? BN / 2 : BN;
-            const int tiles_m = (p.M + BM - 1) / BM;
-            const int tiles_n = (p.N + BN_OUT - 1) / BN_OUT;
-            static bool attr_set = false;
-            if (!attr_set)
-            {
-                hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&w4a16_gemm_dl_kernel<GATE, BIAS, RESID>),
-                                                   hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
-                if (e != hipSuccess)
-                    return e;
-                attr_set = true;
-            }
-            hipLaunchKernelGGL((w4a16_gemm_dl_kernel<GATE, BIAS, RESID>), dim3(tiles_m * tiles_n), dim3(THREADS),
-                               LDS_BYTES, stream, p);
-            return hipGetLastError();
+            if (gate)
+                return launch_reduce<true, false, false>(stream, p);
+            if (hb && hr)
+                return launch_reduce<false, true, true>(stream, p);
+            if (hb)
+                return launch_reduce<false, true, false>(stream, p);
+            if (hr)
+                return launch_reduce<false, false, true>(stream, p);
+            return launch_reduce<false, false, false>(stream, p);
+        }
+
+        // 256 x 256 tiles: wavefronts 2 (M) x 4 (N), each 4 x 2 MFMA tiles; one workgroup per CU
+        hipError_t launch_gemm_big(hipStream_t stream, const GemmParams& p, bool gate, bool hb, bool hr)
+        {
+            if (gate)
+                return launch_gemm_dl<2, 4, 4, 2, true, false, false, false, 2>(stream, p);
+            if (hb && hr)
+                return launch_gemm_dl<2, 4, 4, 2, false, true, true, false, 2>(stream, p);
+            if (hb)
+                return launch_gemm_dl<2, 4, 4, 2, false, true, false, false, 2>(stream, p);
+            if (hr)
+                return launch_gemm_dl<2, 4, 4, 2, false, false, true, false, 2>(stream, p);
+            return launch_gemm_dl<2, 4, 4, 2, false, false, false, false, 2>(stream, p);
         }
     } // namespace
 
     hipError_t launch_w4a16_gemm(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M,
                                  int N, int K, int zp, const void* rms_gamma, float rms_eps, const void* bias,
-                                 const void* residual, int act, void* workspace)
+                                 const void* residual, int act, void* rms_ws, void* partial_ws)
     {
+        const bool rms = rms_gamma != nullptr, hb = bias != nullptr, hr = residual != nullptr, gate = act == 1;
+        // the combinations the fused entry points use; anything else is composed by the caller
+        if (gate && (hb || hr))
+            return hipErrorInvalidValue;
+        if (rms)
+        {
+            if (!rms_ws)
+                return hipErrorInvalidValue;
+            hipLaunchKernelGGL(rms_norm_kernel, dim3((M + 3) / 4), dim3(256), 0, stream, (const half_t*)A,
+                               (const half_t*)rms_gamma, (half_t*)rms_ws, M, K, rms_eps);
+            hipError_t e = hipGetLastError();
+            if (e != hipSuccess)
+                return e;
+            A = rms_ws;
+        }
+        const workspace::GemmPlan plan =
+            workspace::plan_w4a16_gemm(M, N, K, gate, g_tuning.gemm_tile - 1, g_tuning.gemm_splits);
         GemmParams p;
         p.A = (const half_t*)A;
         p.Wq = (const uint8_t*)Wq;
@@ -717,42 +200,22 @@ namespace nnf
         p.zp = zp;
         p.ldy = N;
         p.up_row_offset = N; // gate rows [0,N), up rows [N,2N)
-        p.rstd = (const float*)workspace;
-        p.gamma = (const half_t*)rms_gamma;
         p.bias = (const half_t*)bias;
         p.residual = (const half_t*)residual;
-        const bool rms = rms_gamma != nullptr, hb = bias != nullptr, hr = residual != nullptr, gate = act == 1;
-        if (rms)
+        if (plan.reduce_pass && !partial_ws)
+            return hipErrorInvalidValue;
+        p.partial = plan.reduce_pass ? (float*)partial_ws : nullptr;
+        p.splits = plan.splits;
+        p.ld_partial = gate ? 2 * N : N;
+        hipError_t e;
+        switch (plan.tile)
         {
-            hipLaunchKernelGGL(rms_rstd_kernel, dim3((M + 3) / 4), dim3(256), 0, stream, (const half_t*)A,
-                               (float*)workspace, M, K, rms_eps);
-            hipError_t e = hipGetLastError();
-            if (e != hipSuccess)
-                return e;
+        case workspace::GEMM_TILE_BIG: return launch_gemm_big(stream, p, gate, hb, hr);
+        case workspace::GEMM_TILE_MID: e = launch_gemm_mid(stream, p, gate, hb, hr); break;
+        default: e = launch_gemm_small(stream, p, gate, hb, hr); break;
         }
-        // the combinations the fused entry points use; anything else is composed by the caller
-        if (gate && rms && !hb && !hr)
-            return launch_gemm_variant<true, true, false, false>(stream, p);
-        const bool dl = g_tuning.gemm_no_direct_loads == 0;
-        if (gate && !rms && !hb && !hr)
-            return dl ? launch_gemm_dl_variant<true, false, false>(stream, p)
-                      : launch_gemm_variant<true, false, false, false>(stream, p);
-        if (!gate && !rms && !hb && !hr)
-            return dl ? launch_gemm_dl_variant<false, false, false>(stream, p)
-                      : launch_gemm_variant<false, false, false, false>(stream, p);
-        if (!gate && !rms && !hb && hr)
-            return dl ? launch_gemm_dl_variant<false, false, true>(stream, p)
-                      : launch_gemm_variant<false, false, false, true>(stream, p);
-        if (!gate && !rms && hb && !hr)
-            return dl ? launch_gemm_dl_variant<false, true, false>(stream, p)
-                      : launch_gemm_variant<false, false, true, false>(stream, p);
-        if (!gate && !rms && hb && hr)
-            return dl ? launch_gemm_dl_variant<false, true, true>(stream, p)
-                      : launch_gemm_variant<false, false, true, true>(stream, p);
-        if (!gate && rms && !hb && !hr)
-            return launch_gemm_variant<false, true, false, false>(stream, p);
-        if (!gate && rms && hb && !hr)
-            return launch_gemm_variant<false, true, true, false>(stream, p);
-        return hipErrorInvalidValue;
+        if (e != hipSuccess || !plan.reduce_pass)
+            return e;
+        return launch_reduce_any(stream, p, gate, hb, hr);
     }
 } // namespace nnf

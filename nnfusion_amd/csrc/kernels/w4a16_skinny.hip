@@ -29,6 +29,8 @@
 #include "nnf_device.h"
 #include "nnf_launch.h"
 
+#include "../nnf_workspace.h"
+
 #include <algorithm>
 #include <type_traits>
 
@@ -401,46 +403,8 @@ namespace nnf
 
     namespace
     {
-        struct SkinnyPlan
-        {
-            int cps = 0, ks = 0, h = 0;
-            bool a_regs = false;
-            size_t lds = 0; // without the output parking area
-        };
-
-        // groups per wavefront and pass, wavefronts per workgroup, passes: one workgroup spans all of K
-        SkinnyPlan plan_skinny(int M, int K)
-        {
-            SkinnyPlan p;
-            const int G = K >> 7;
-            struct Option
-            {
-                int cps, h;
-            };
-            // fewest groups per wavefront first (more wavefronts in flight); two passes beyond 16 * 4 groups
-            static const Option options[] = {{1, 1}, {2, 1}, {3, 1}, {4, 1}, {3, 2}, {4, 2}};
-            for (const Option& o : options)
-            {
-                int ks = (G + o.cps * o.h - 1) / (o.cps * o.h);
-                if (g_tuning.skinny_cps != 0 && o.cps != g_tuning.skinny_cps)
-                    continue;
-                if (ks <= 16)
-                {
-                    p.cps = o.cps;
-                    p.h = o.h;
-                    p.ks = ks;
-                    break;
-                }
-            }
-            if (p.cps == 0)
-                return p;
-            // the A operand fits in registers up to two groups per wavefront (32 VGPRs)
-            p.a_regs = p.cps <= 2 && p.h == 1;
-            const size_t a_bytes = ((size_t)G * 16 + 1) * M * 16 + (size_t)G * 64;
-            const size_t sc_bytes = 2 * (((size_t)16 * G * 2 + 15) & ~(size_t)15);
-            p.lds = a_bytes + sc_bytes + (size_t)2 * M * 16 * ((p.ks + 3) & ~3) * 4;
-            return p;
-        }
+        using workspace::SkinnyPlan;
+        SkinnyPlan plan_skinny(int M, int K) { return workspace::plan_w4a16_skinny(M, K, g_tuning.skinny_cps); }
 
         template <int CPS, bool A_REGS, int H>
         hipError_t launch_cps(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M, int N,
@@ -478,14 +442,7 @@ namespace nnf
 
     bool w4a16_skinny_supported(int M, int N, int K)
     {
-        if (M < 1 || M > 16 || (K & 127) || N < 16)
-            return false;
-        // the scale block of a tile is fetched in whole 16-byte pieces
-        if (((size_t)N * (K >> 7) * 2) % 16 != 0 || (size_t)N * (K >> 7) * 2 < 16)
-            return false;
-        SkinnyPlan p = plan_skinny(M, K);
-        // leave room for the output parking area (a few tiles of M x 16 floats)
-        return p.cps != 0 && p.lds + 16 * 1024 <= MAX_LDS_BYTES;
+        return workspace::w4a16_skinny_fits(M, N, K, g_tuning.skinny_cps);
     }
 
     hipError_t launch_w4a16_skinny(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M,

@@ -69,7 +69,8 @@ int nnf_internal_tune(int key, int value)
     case 0: nnf::g_tuning.force_path = value; return 0;
     case 1: nnf::g_tuning.skinny_cps = value; return 0;
     case 2: nnf::g_tuning.skinny_wg_per_cu = value; return 0;
-    case 3: nnf::g_tuning.gemm_no_direct_loads = value; return 0;
+    case 3: nnf::g_tuning.gemm_tile = value; return 0;
+    case 4: nnf::g_tuning.gemm_splits = value; return 0;
     default: return -1;
     }
 }
@@ -95,6 +96,21 @@ const char* nnf_status_string(int status)
     return "unknown nnf status";
 }
 
+} // extern "C"
+
+namespace
+{
+    // partial-sum bytes of the GEMM plan in force (the automatic one unless an experiment overrides it)
+    size_t tuned_partial_bytes(int M, int N, int K, bool gate)
+    {
+        return nnf::workspace::gemm_partial_bytes(
+            M, N, gate,
+            nnf::workspace::plan_w4a16_gemm(M, N, K, gate, nnf::g_tuning.gemm_tile - 1, nnf::g_tuning.gemm_splits));
+    }
+} // namespace
+
+extern "C" {
+
 size_t nnf_w4a16_gemm_workspace_bytes(int M, int N, int K, int group)
 {
     return nnf::workspace::w4a16_gemm(M, N, K, group);
@@ -103,12 +119,9 @@ size_t nnf_w4a16_gemm_workspace_bytes(int M, int N, int K, int group)
 int nnf_w4a16_gemm(nnf_stream_t stream, const void* A, const void* Wq, const void* scales, void* Y, int M, int N,
                    int K, int group, int zp, void* workspace, size_t workspace_bytes)
 {
-    (void)workspace;
     int st = check_w4a16(A, Wq, scales, Y, M, N, K, group, zp);
     if (st != NNF_OK)
         return st;
-    if (workspace_bytes < nnf_w4a16_gemm_workspace_bytes(M, N, K, group))
-        return NNF_ERR_WORKSPACE_TOO_SMALL;
     DeviceInfo dev;
     st = current_device_info(dev);
     if (st != NNF_OK)
@@ -118,13 +131,17 @@ int nnf_w4a16_gemm(nnf_stream_t stream, const void* A, const void* Wq, const voi
         return (int)nnf::launch_w4a16_skinny((hipStream_t)stream, A, Wq, scales, Y, M, N, K, zp, dev.num_cu);
     if (force == 1 && M <= 16 && nnf::w4a16_gemv_supported(M, K))
         return (int)nnf::launch_w4a16_gemv((hipStream_t)stream, A, Wq, scales, Y, M, N, K, zp, dev.num_cu);
+    // the MFMA GEMM may split K and then needs room for its partial sums (the GEMV kernels need none)
+    const size_t need = tuned_partial_bytes(M, N, K, false);
+    if (need > 0 && (!workspace || !aligned16(workspace) || workspace_bytes < need))
+        return NNF_ERR_WORKSPACE_TOO_SMALL;
     return (int)nnf::launch_w4a16_gemm((hipStream_t)stream, A, Wq, scales, Y, M, N, K, zp, nullptr, 0.f, nullptr,
-                                       nullptr, NNF_ACT_NONE, nullptr);
+                                       nullptr, NNF_ACT_NONE, nullptr, workspace);
 }
 
 size_t nnf_w4a16_gemm_fused_workspace_bytes(int M, int N, int K, int group, int act)
 {
-    // room for the RMSNorm row statistics whether or not the call uses them
+    // room for the normalised activations of the RMSNorm prologue whether or not the call uses it
     return nnf::workspace::w4a16_gemm_fused(M, N, K, group, act);
 }
 
@@ -142,16 +159,16 @@ int nnf_w4a16_gemm_fused(nnf_stream_t stream, const void* A, const void* Wq, con
     // combinations without a fused kernel (see launch_w4a16_gemm)
     if (act == NNF_ACT_SILU_GATE && (bias || residual))
         return NNF_ERR_UNSUPPORTED_SHAPE;
-    if (rms_gamma && residual)
-        return NNF_ERR_UNSUPPORTED_SHAPE;
-    if (rms_gamma && (!workspace || workspace_bytes < nnf::workspace::rms_rows(M)))
+    const size_t need = (rms_gamma ? nnf::workspace::rms_rows(M, K) : 0) + tuned_partial_bytes(M, N, K, act == NNF_ACT_SILU_GATE);
+    if (need > 0 && (!workspace || !aligned16(workspace) || workspace_bytes < need))
         return NNF_ERR_WORKSPACE_TOO_SMALL;
     DeviceInfo dev;
     st = current_device_info(dev);
     if (st != NNF_OK)
         return st;
+    uint8_t* ws = (uint8_t*)workspace;
     return (int)nnf::launch_w4a16_gemm((hipStream_t)stream, A, Wq, scales, Y, M, N, K, zp, rms_gamma, rms_eps, bias,
-                                       residual, act, workspace);
+                                       residual, act, ws, ws ? ws + (rms_gamma ? nnf::workspace::rms_rows(M, K) : 0) : nullptr);
 }
 
 // ---- W8A8 ---------------------------------------------------------------------------------------
@@ -205,7 +222,7 @@ int nnf_w8a8_gemm_acc(nnf_stream_t stream, const void* A, const void* W, void* a
 }
 
 // ---- fused MLP block ------------------------------------------------------------------------------
-// workspace = [ rstd: M floats, padded to 256 B ][ h: M x I fp16 ]
+// workspace = [ RMSNorm(x): M x H fp16 ][ h: M x I fp16 ][ split-K partial sums of either GEMM ]
 size_t nnf_fused_mlp_w4a16_workspace_bytes(int M, int H, int I, int group)
 {
     return nnf::workspace::fused_mlp_w4a16(M, H, I, group);
@@ -222,22 +239,27 @@ int nnf_fused_mlp_w4a16(nnf_stream_t stream, const void* x, const void* gamma, f
         return NNF_ERR_INVALID_ARGUMENT;
     if (group != 128 || H % group != 0 || I % group != 0 || zp < 0 || zp > 15)
         return NNF_ERR_UNSUPPORTED_SHAPE;
-    if (!workspace || workspace_bytes < nnf_fused_mlp_w4a16_workspace_bytes(M, H, I, group))
-        return NNF_ERR_WORKSPACE_TOO_SMALL;
+    {
+        const size_t a = tuned_partial_bytes(M, I, H, true), b = tuned_partial_bytes(M, H, I, false);
+        if (!workspace || workspace_bytes < nnf::workspace::fused_mlp_partial_offset(M, H, I) + (a > b ? a : b))
+            return NNF_ERR_WORKSPACE_TOO_SMALL;
+    }
     DeviceInfo dev;
     int st = current_device_info(dev);
     if (st != NNF_OK)
         return st;
     uint8_t* ws = (uint8_t*)workspace;
-    void* h = ws + nnf::workspace::rms_rows(M);
-    // h = SiLU(gate) * up, gate|up = RMSNorm(x) . Wgu^T : one kernel (after the row-statistics pre-pass)
+    void* h = ws + nnf::workspace::fused_mlp_h_offset(M, H);
+    void* partial = ws + nnf::workspace::fused_mlp_partial_offset(M, H, I);
+    // h = SiLU(gate) * up, gate|up = RMSNorm(x) . Wgu^T : the normalisation pre-pass, then one GEMM with the
+    // gate and up projections as the two halves of every N tile
     hipError_t e = nnf::launch_w4a16_gemm((hipStream_t)stream, x, Wgu, Sgu, h, M, I, H, zp, gamma, eps, nullptr,
-                                          nullptr, NNF_ACT_SILU_GATE, ws);
+                                          nullptr, NNF_ACT_SILU_GATE, ws, partial);
     if (e != hipSuccess)
         return (int)e;
     // out = h . Wd^T + x
     e = nnf::launch_w4a16_gemm((hipStream_t)stream, h, Wd, Sd, out, M, H, I, zp, nullptr, 0.f, nullptr, x, NNF_ACT_NONE,
-                               nullptr);
+                               nullptr, partial);
     return (int)e;
 }
 

@@ -1,5 +1,6 @@
-// Scratch-memory sizes of the launcher entry points: pure host arithmetic, shared by the library
-// (nnf_*_workspace_bytes) and by the emitters, which reserve the scratch tensor at compile time.
+// Scratch-memory sizes of the launcher entry points and the tile plan they follow: pure host
+// arithmetic, shared by the library (nnf_*_workspace_bytes, the GEMM dispatcher) and by the emitters,
+// which reserve the scratch tensor at compile time.  Nothing here may depend on the device at hand.
 #pragma once
 
 #include <stddef.h>
@@ -9,15 +10,143 @@ namespace nnf
     namespace workspace
     {
         inline size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
-        // per-row statistics of the RMSNorm prologue
-        inline size_t rms_rows(int M) { return M > 0 ? align256((size_t)M * sizeof(float)) : 0; }
-        inline size_t w4a16_gemm(int, int, int, int) { return 0; }
-        inline size_t w4a16_gemm_fused(int M, int, int, int, int) { return rms_rows(M); }
-        inline size_t w8a8_gemm(int, int, int) { return 0; }
-        // [ rstd: M floats ][ h: M x I fp16 ]
-        inline size_t fused_mlp_w4a16(int M, int, int I, int)
+
+        // ---- tile plan of the fp16 x int4 MFMA GEMM -------------------------------------------------
+        enum GemmTile
         {
-            return (M > 0 && I > 0) ? rms_rows(M) + align256((size_t)M * I * 2) : 0;
+            GEMM_TILE_BIG = 0,   // 256 x 256 outputs (SiLU-gate: 256 x 128)
+            GEMM_TILE_MID = 1,   // 128 x 128
+            GEMM_TILE_SMALL = 2, //  64 x 256
+        };
+        struct GemmPlan
+        {
+            int tile = GEMM_TILE_BIG;
+            int splits = 1; // K ranges; > 1 (and always for the small tile): fp32 partial sums + a reduction pass
+            bool reduce_pass = false;
+        };
+        constexpr int PLAN_CUS = 256; // the plan is made for the CU count of an MI355X
+
+        inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
+
+        // N: output columns.  forced_splits > 0 overrides the split count (experiments).
+        inline GemmPlan plan_w4a16_gemm(int M, int N, int K, bool gate, int forced_tile = -1, int forced_splits = 0)
+        {
+            GemmPlan p;
+            const int G = K / 128;
+            const int big_tiles = ceil_div(M, 256) * ceil_div(N, gate ? 128 : 256);
+            if (M <= 64)
+                p.tile = GEMM_TILE_SMALL;
+            else if (M <= 128 || big_tiles < (PLAN_CUS * 3) / 4)
+                p.tile = GEMM_TILE_MID;
+            else
+                p.tile = GEMM_TILE_BIG;
+            if (forced_tile >= 0)
+                p.tile = forced_tile;
+            if (p.tile == GEMM_TILE_BIG)
+                return p;
+            const int tiles = p.tile == GEMM_TILE_MID ? ceil_div(M, 128) * ceil_div(N, 128)
+                                                      : ceil_div(M, 64) * ceil_div(N, 256);
+            // two workgroups fit a CU; every split keeps at least four groups (eight K steps)
+            int s = (2 * PLAN_CUS) / (tiles > 0 ? tiles : 1);
+            if (s > G / 4)
+                s = G / 4;
+            if (s < 1)
+                s = 1;
+            if (forced_splits > 0)
+                s = forced_splits < G ? forced_splits : G;
+            p.splits = s;
+            p.reduce_pass = s > 1 || p.tile == GEMM_TILE_SMALL;
+            return p;
+        }
+        inline size_t gemm_partial_bytes(int M, int N, bool gate, const GemmPlan& p)
+        {
+            return p.reduce_pass ? align256((size_t)p.splits * M * (gate ? 2 : 1) * N * sizeof(float)) : 0;
+        }
+
+        // ---- plan of the skinny (M <= 16) MFMA GEMV kernel ---------------------------------------------
+        constexpr size_t LDS_BYTES_PER_CU = 160 * 1024; // gfx950
+        struct SkinnyPlan
+        {
+            int cps = 0, ks = 0, h = 0; // groups per wavefront and pass, wavefronts per workgroup, passes over K
+            bool a_regs = false;        // activations kept in registers
+            size_t lds = 0;             // LDS bytes without the output parking area
+        };
+        // one workgroup spans all of K: fewest groups per wavefront first (more wavefronts in flight), two
+        // passes beyond 16 * 4 groups
+        inline SkinnyPlan plan_w4a16_skinny(int M, int K, int forced_cps = 0)
+        {
+            SkinnyPlan p;
+            const int G = K >> 7;
+            static const int options[6][2] = {{1, 1}, {2, 1}, {3, 1}, {4, 1}, {3, 2}, {4, 2}};
+            for (const auto& o : options)
+            {
+                const int ks = (G + o[0] * o[1] - 1) / (o[0] * o[1]);
+                if (forced_cps != 0 && o[0] != forced_cps)
+                    continue;
+                if (ks <= 16)
+                {
+                    p.cps = o[0];
+                    p.h = o[1];
+                    p.ks = ks;
+                    break;
+                }
+            }
+            if (p.cps == 0)
+                return p;
+            // the A operand fits in registers up to two groups per wavefront (32 VGPRs)
+            p.a_regs = p.cps <= 2 && p.h == 1;
+            const size_t a_bytes = ((size_t)G * 16 + 1) * M * 16 + (size_t)G * 64;
+            const size_t sc_bytes = 2 * (((size_t)16 * G * 2 + 15) & ~(size_t)15);
+            p.lds = a_bytes + sc_bytes + (size_t)2 * M * 16 * ((p.ks + 3) & ~3) * 4;
+            return p;
+        }
+        // true when one workgroup can hold the activations (M <= 16 rows of K) in LDS
+        inline bool w4a16_skinny_fits(int M, int N, int K, int forced_cps = 0)
+        {
+            if (M < 1 || M > 16 || K < 128 || (K & 127) || N < 16)
+                return false;
+            // the scale block of a tile (16 rows x K/128 fp16) is fetched in whole, aligned 16-byte pieces
+            if (((size_t)N * (K >> 7) * 2) % 16 != 0)
+                return false;
+            const SkinnyPlan p = plan_w4a16_skinny(M, K, forced_cps);
+            // leave room for the output parking area (a few tiles of M x 16 floats)
+            return p.cps != 0 && p.lds + 16 * 1024 <= LDS_BYTES_PER_CU;
+        }
+
+        // normalised activations of the RMSNorm prologue (fp16 [M, K])
+        inline size_t rms_rows(int M, int K) { return (M > 0 && K > 0) ? align256((size_t)M * K * 2) : 0; }
+
+        // nnf_w4a16_gemm: [ partial sums ]
+        inline size_t w4a16_gemm(int M, int N, int K, int)
+        {
+            if (M <= 0 || N <= 0 || K < 128)
+                return 0;
+            if (w4a16_skinny_fits(M, N, K))
+                return 0; // served by the skinny kernel
+            return gemm_partial_bytes(M, N, false, plan_w4a16_gemm(M, N, K, false));
+        }
+        // nnf_w4a16_gemm_fused: [ normalised activations ][ partial sums ]
+        inline size_t w4a16_gemm_fused(int M, int N, int K, int, int act)
+        {
+            if (M <= 0 || N <= 0 || K < 128)
+                return 0;
+            const bool gate = act == 1;
+            return rms_rows(M, K) + gemm_partial_bytes(M, N, gate, plan_w4a16_gemm(M, N, K, gate));
+        }
+        inline size_t w8a8_gemm(int, int, int) { return 0; }
+        // nnf_fused_mlp_w4a16: [ normalised x: M x H fp16 ][ h: M x I fp16 ][ partial sums of either GEMM ]
+        inline size_t fused_mlp_h_offset(int M, int H) { return rms_rows(M, H); }
+        inline size_t fused_mlp_partial_offset(int M, int H, int I)
+        {
+            return rms_rows(M, H) + align256((size_t)M * I * 2);
+        }
+        inline size_t fused_mlp_w4a16(int M, int H, int I, int)
+        {
+            if (M <= 0 || I <= 0 || H < 128 || I < 128)
+                return 0;
+            size_t a = gemm_partial_bytes(M, I, true, plan_w4a16_gemm(M, I, H, true));
+            size_t b = gemm_partial_bytes(M, H, false, plan_w4a16_gemm(M, H, I, false));
+            return fused_mlp_partial_offset(M, H, I) + (a > b ? a : b);
         }
     } // namespace workspace
 } // namespace nnf

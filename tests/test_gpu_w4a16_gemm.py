@@ -42,9 +42,47 @@ def force_gemm():
     tune(0, 0)
 
 
+# (tile, splits) of the MFMA GEMM: None = the library's own plan; tiles 1 big 256x256, 2 mid 128x128,
+# 3 small 64x256; splits = K ranges (> 1, and always for the small tile: fp32 partial sums + reduction pass)
+PLANS = [None, (1, 0), (2, 1), (2, 3), (3, 1), (3, 2)]
+
+
+@pytest.fixture(params=PLANS, ids=lambda p: "auto" if p is None else f"tile{p[0]}-splits{p[1]}")
+def plan(request):
+    from nnfusion_amd import _lib
+
+    tune = _lib.kernels().nnf_internal_tune
+    if request.param is not None:
+        tune(3, request.param[0])
+        tune(4, request.param[1])
+    yield request.param
+    tune(3, 0)
+    tune(4, 0)
+
+
+def _big_ws(gpu):
+    import torch
+
+    return torch.empty(64 << 20, dtype=torch.uint8, device=gpu)
+
+
+@pytest.mark.parametrize("m,n,k", [(200, 300, 1024), (64, 520, 2048), (130, 128, 512), (17, 40, 1280)])
+def test_gemm_every_tile_plan_matches_oracle(gpu, plan, m, n, k):
+    import torch
+
+    from nnfusion_amd import ops
+
+    print(f"case plan={plan} M={m} N={n} K={k}", flush=True)
+    a, wq, s = datagen.w4a16_case(2, m, n, k)
+    ta, tw, ts = _t(gpu, a, wq, s)
+    y = ops.w4a16_gemm(ta, tw, ts, workspace=_big_ws(gpu))
+    torch.cuda.synchronize()
+    _check(y.cpu().numpy(), oracle.w4a16_gemm(a, wq, s, f32_out=True))
+
+
 @pytest.mark.parametrize("m,n,k", [
     (128, 256, 128), (256, 256, 256), (17, 32, 128), (100, 96, 384), (300, 520, 1024),
-    (512, 1024, 2048), (257, 33, 512), (1024, 512, 4096),
+    (512, 1024, 2048), (257, 33, 512), (1024, 512, 4096), (2048, 2048, 512),
 ])
 def test_gemm_matches_oracle(gpu, m, n, k):
     import torch
@@ -68,7 +106,7 @@ def test_gemm_kernel_serves_small_m(gpu, force_gemm, m):
 
     a, wq, s = datagen.w4a16_case(4, m, 320, 512)
     ta, tw, ts = _t(gpu, a, wq, s)
-    y = ops.w4a16_gemm(ta, tw, ts)
+    y = ops.w4a16_gemm(ta, tw, ts, workspace=_big_ws(gpu))
     torch.cuda.synchronize()
     _check(y.cpu().numpy(), oracle.w4a16_gemm(a, wq, s, f32_out=True))
 
@@ -113,7 +151,7 @@ def test_gemm_full_size_sampled_columns(gpu, m, n, k):
     assert torch.equal(y2[normal], (y * 2)[normal])
 
 
-def test_fused_bias_residual(gpu):
+def test_fused_bias_residual(gpu, plan):
     import torch
 
     from nnfusion_amd import ops
@@ -123,9 +161,10 @@ def test_fused_bias_residual(gpu):
     bias = datagen.normal_f16(6, datagen.S_BIAS, (n,))
     res = datagen.normal_f16(6, datagen.S_RES, (m, n))
     ta, tw, ts, tb, tr = _t(gpu, a, wq, s, bias, res)
-    y_b = ops.w4a16_gemm_fused(ta, tw, ts, bias=tb).cpu().numpy()
-    y_r = ops.w4a16_gemm_fused(ta, tw, ts, residual=tr).cpu().numpy()
-    y_br = ops.w4a16_gemm_fused(ta, tw, ts, bias=tb, residual=tr).cpu().numpy()
+    ws = _big_ws(gpu)
+    y_b = ops.w4a16_gemm_fused(ta, tw, ts, bias=tb, workspace=ws).cpu().numpy()
+    y_r = ops.w4a16_gemm_fused(ta, tw, ts, residual=tr, workspace=ws).cpu().numpy()
+    y_br = ops.w4a16_gemm_fused(ta, tw, ts, bias=tb, residual=tr, workspace=ws).cpu().numpy()
     torch.cuda.synchronize()
     d = oracle.w4a16_gemm(a, wq, s)  # fp16 tensor of the unfused Dot
     ref_b = oracle.add_f16(d, np.broadcast_to(bias, (m, n)).copy())
@@ -136,7 +175,7 @@ def test_fused_bias_residual(gpu):
     _check(y_br, ref_br)
 
 
-def test_fused_rmsnorm_prologue(gpu):
+def test_fused_rmsnorm_prologue(gpu, plan):
     import torch
 
     from nnfusion_amd import ops
@@ -145,13 +184,13 @@ def test_fused_rmsnorm_prologue(gpu):
     a, wq, s = datagen.w4a16_case(7, m, n, k)
     gamma = datagen.normal_f16(7, datagen.S_GAMMA, (k,), 1.0, 0.1)
     ta, tw, ts, tg = _t(gpu, a, wq, s, gamma)
-    y = ops.w4a16_gemm_fused(ta, tw, ts, rms_gamma=tg, rms_eps=1e-6).cpu().numpy()
+    y = ops.w4a16_gemm_fused(ta, tw, ts, rms_gamma=tg, rms_eps=1e-6, workspace=_big_ws(gpu)).cpu().numpy()
     torch.cuda.synchronize()
     xn = oracle.rmsnorm_f16(a, gamma, 1e-6)
     _check(y, oracle.w4a16_gemm(xn, wq, s, f32_out=True))
 
 
-def test_fused_silu_gate(gpu):
+def test_fused_silu_gate(gpu, plan):
     import torch
 
     from nnfusion_amd import ops
@@ -159,7 +198,7 @@ def test_fused_silu_gate(gpu):
     m, n, k = 150, 192, 512  # n = intermediate size; weights hold 2n rows (gate then up)
     a, wq, s = datagen.w4a16_case(8, m, 2 * n, k)
     ta, tw, ts = _t(gpu, a, wq, s)
-    y = ops.w4a16_gemm_fused(ta, tw, ts, act=1).cpu().numpy()
+    y = ops.w4a16_gemm_fused(ta, tw, ts, act=1, workspace=_big_ws(gpu)).cpu().numpy()
     torch.cuda.synchronize()
     gu = oracle.w4a16_gemm(a, wq, s)
     g = np.ascontiguousarray(gu[:, :n])
