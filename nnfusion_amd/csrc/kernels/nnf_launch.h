@@ -29,8 +29,12 @@ namespace nnf
                                  const void* residual, int act, void* rms_ws, void* partial_ws);
 
     // W8A8: acc != nullptr writes the raw int32 accumulators, otherwise Y = fp16(acc * s_tok * s_ch).
+    // partial_ws: nnf::workspace::w8a8_gemm(M, N, K) bytes (0 for the M <= 16 kernel)
     hipError_t launch_w8a8(hipStream_t stream, const void* A, const void* s_tok, const void* W, const void* s_ch,
-                           void* Y, void* acc, int M, int N, int K, int num_cu);
+                           void* Y, void* acc, int M, int N, int K, int num_cu, void* partial_ws);
+    // the MFMA GEMM behind launch_w8a8 (any M)
+    hipError_t launch_w8a8_gemm(hipStream_t stream, const void* A, const void* s_tok, const void* W, const void* s_ch,
+                                void* Y, void* acc, int M, int N, int K, void* partial_ws);
     bool w8a8_skinny_supported(int M, int K);
 
     // Tuning knobs for experiments (not part of the public ABI): 0 = automatic.

@@ -1,0 +1,362 @@
+// W8A8 for M > 16: int8 x int8 -> int32 GEMM on v_mfma_i32_32x32x32_i8, exact accumulators.
+//
+//   acc[M,N] = A[M,K] . W[N,K]^T  (int32, bit exact);  Y = fp16((float)acc * s_tok[m] * s_ch[n])
+//
+// Nothing in the reference computes this on a GPU; the nearest is MLAS's u8 x s8 MlasGemm
+// (thirdparty/mlas/inc/mlas.h:147-163).
+//
+// Same skeleton as the fp16 x int4 GEMM: eight wavefronts (WM x WN) over a BM x BN tile, operands
+// global -> LDS by asynchronous 1 KiB wavefront loads into a ring of stages (loads run STAGES-1 K steps
+// ahead, one barrier per K step), tiles numbered so that an XCD works on a compact block of the output,
+// optional split of K with int32 partial sums (added exactly by a reduction pass).  Both operands are
+// K-contiguous int8 and need no unpacking: a K step is 64 bytes of every row, a lane's MFMA operand is
+// 16 consecutive bytes (K index in the step = 32*s + 16*h + e), and the 16-byte pieces of a 64-byte row
+// are XOR-swizzled with bits 2..3 of the row so that the 128-bit fragment reads are conflict free.
+#include "nnf_device.h"
+#include "nnf_launch.h"
+
+#include "../nnf_workspace.h"
+
+namespace nnf
+{
+    struct Q8GemmParams
+    {
+        const int8_t* A;
+        const int8_t* W;
+        const float* s_tok;
+        const float* s_ch;
+        half_t* Y;       // fp16 output, or
+        int32_t* acc;    // raw accumulators (RAW)
+        int32_t* partial; // SPLITK: [splits][M][N]
+        int M, N, K, splits;
+    };
+
+    namespace q8dl
+    {
+        constexpr int BK = 64; // bytes (= int8 elements) of K per step
+        constexpr int THREADS = 512;
+
+        template <int WM, int WN, int TM, int TN, int STAGES_>
+        struct Tile
+        {
+            static_assert(WM * WN == 8, "eight wavefronts per workgroup");
+            static constexpr int STAGES = STAGES_;
+            static constexpr int BM = WM * TM * 32;
+            static constexpr int BN = WN * TN * 32;
+            static constexpr int A_TILE_BYTES = BM * BK;
+            static constexpr int W_TILE_BYTES = BN * BK;
+            static constexpr int STAGE_BYTES = A_TILE_BYTES + W_TILE_BYTES;
+            static constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
+            // a wavefront-wide load covers 16 rows of 64 bytes; every wavefront issues the same number of loads
+            // (with fewer than 8 chunks two wavefronts fetch the same chunk into the same place)
+            static constexpr int A_CHUNKS = BM / 16;
+            static constexpr int W_CHUNKS = BN / 16;
+            static constexpr int A_LOADS = A_CHUNKS >= 8 ? A_CHUNKS / 8 : 1;
+            static constexpr int W_LOADS = W_CHUNKS >= 8 ? W_CHUNKS / 8 : 1;
+            static constexpr int TILE_LOADS = A_LOADS + W_LOADS;
+        };
+
+        constexpr int vmcnt_imm(int n) { return (n & 0xF) | ((n >> 4) << 14) | (0x7 << 4) | (0xF << 8); }
+    } // namespace q8dl
+
+    template <int WM, int WN, int TM, int TN, int STAGES, bool RAW, bool SPLITK, int MINW>
+    __global__ __launch_bounds__(512, MINW) void w8a8_gemm_dl_kernel(Q8GemmParams p)
+    {
+        using namespace q8dl;
+        using T = Tile<WM, WN, TM, TN, STAGES>;
+        constexpr int BM = T::BM, BN = T::BN;
+        constexpr int A_LOADS = T::A_LOADS, W_LOADS = T::W_LOADS, TILE_LOADS = T::TILE_LOADS;
+        constexpr int A_TILE_BYTES = T::A_TILE_BYTES, STAGE_BYTES = T::STAGE_BYTES;
+        extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+        const int tid = threadIdx.x;
+        const int lane = tid & 63;
+        const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+        const int wm = wave / WN, wn = wave % WN;
+        const int l32 = lane & 31, h = lane >> 5;
+        const int K = p.K;
+        const int G = K >> 7;
+
+        const int tiles_m = (p.M + BM - 1) / BM;
+        const int tiles_n = (p.N + BN - 1) / BN;
+        const int n_wg = tiles_m * tiles_n;
+        const int split = SPLITK ? (int)blockIdx.x / n_wg : 0;
+        int pid = SPLITK ? (int)blockIdx.x - split * n_wg : (int)blockIdx.x;
+        {
+            // contiguous run of tiles per XCD (workgroup ids are dealt round-robin to the 8 XCDs)
+            const int per_xcd = (n_wg + 7) >> 3;
+            const int full = n_wg - (per_xcd - 1) * 8;
+            const int xcd = pid & 7, idx = pid >> 3;
+            pid = (xcd < full) ? xcd * per_xcd + idx : full * per_xcd + (xcd - full) * (per_xcd - 1) + idx;
+        }
+        int tm, tn;
+        {
+            // four tile rows advance together along N
+            constexpr int GM = 4;
+            const int per_group = GM * tiles_n;
+            const int g = pid / per_group;
+            const int first_m = g * GM;
+            const int gm = min(GM, tiles_m - first_m);
+            const int r = pid - g * per_group;
+            tm = first_m + r % gm;
+            tn = r / gm;
+        }
+        const int m0 = tm * BM, n0 = tn * BN;
+
+        // this workgroup's K range, in units of 128 (all of K without SPLITK)
+        const int g_begin = SPLITK ? (int)(((long long)split * G) / p.splits) : 0;
+        const int g_end = SPLITK ? (int)(((long long)(split + 1) * G) / p.splits) : G;
+        const int KT = 2 * (g_end - g_begin);
+        const int k_begin = g_begin * 128;
+
+        // ---- direct-load maps: chunk c fills LDS rows c*16 .. +15 (64 B each); lane l lands at
+        // (row = c*16 + l/4, slot = l%4) and therefore fetches piece  slot ^ ((row >> 2) & 3)  of that row
+        const int8_t* a_src[A_LOADS];
+        int a_chunk[A_LOADS];
+#pragma unroll
+        for (int i = 0; i < A_LOADS; ++i)
+        {
+            a_chunk[i] = (wave * A_LOADS + i) % T::A_CHUNKS;
+            int row = a_chunk[i] * 16 + (lane >> 2);
+            int piece = (lane & 3) ^ ((row >> 2) & 3);
+            a_src[i] = p.A + (size_t)min(m0 + row, p.M - 1) * K + k_begin + piece * 16;
+        }
+        const int8_t* w_src[W_LOADS];
+        int w_chunk[W_LOADS];
+#pragma unroll
+        for (int i = 0; i < W_LOADS; ++i)
+        {
+            w_chunk[i] = (wave * W_LOADS + i) % T::W_CHUNKS;
+            int row = w_chunk[i] * 16 + (lane >> 2);
+            int piece = (lane & 3) ^ ((row >> 2) & 3);
+            w_src[i] = p.W + (size_t)min(n0 + row, p.N - 1) * K + k_begin + piece * 16;
+        }
+        auto issue_tile_loads = [&](int kt, int stage) {
+            uint8_t* base = smem + stage * STAGE_BYTES;
+            const int k0 = kt * BK;
+#pragma unroll
+            for (int i = 0; i < A_LOADS; ++i)
+                __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1)))*)(a_src[i] + k0),
+                                                 (void __attribute__((address_space(3)))*)(base + a_chunk[i] * 1024), 16, 0,
+                                                 0);
+#pragma unroll
+            for (int i = 0; i < W_LOADS; ++i)
+                __builtin_amdgcn_global_load_lds(
+                    (const void __attribute__((address_space(1)))*)(w_src[i] + k0),
+                    (void __attribute__((address_space(3)))*)(base + A_TILE_BYTES + w_chunk[i] * 1024), 16, 0, 0);
+        };
+
+        // ---- per-lane fragment addresses in LDS ------------------------------------------------------
+        int a_frag[TM], a_swz[TM], w_frag[TN], w_swz[TN];
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+        {
+            int r = wm * (TM * 32) + i * 32 + l32;
+            a_frag[i] = r * 64;
+            a_swz[i] = (r >> 2) & 3;
+        }
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+        {
+            int r = wn * (TN * 32) + j * 32 + l32;
+            w_frag[j] = A_TILE_BYTES + r * 64;
+            w_swz[j] = (r >> 2) & 3;
+        }
+
+        intx16 acc[TM][TN];
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int e = 0; e < 16; ++e)
+                    acc[i][j][e] = 0;
+
+        auto compute = [&](int stage) {
+            const uint8_t* base = smem + stage * STAGE_BYTES;
+#pragma unroll
+            for (int s = 0; s < 2; ++s)
+            {
+                intx4 af[TM], bf[TN];
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+                    af[i] = *reinterpret_cast<const intx4*>(base + a_frag[i] + (((2 * s + h) ^ a_swz[i]) << 4));
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    bf[j] = *reinterpret_cast<const intx4*>(base + w_frag[j] + (((2 * s + h) ^ w_swz[j]) << 4));
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int i = 0; i < TM; ++i)
+                        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i], bf[j], acc[i][j], 0, 0, 0);
+            }
+        };
+
+        // ---- K loop: stage kt % STAGES; loads run STAGES-1 K steps ahead ------------------------------------
+        // Vector-memory operations complete in order and every step issues TILE_LOADS of them: before the
+        // barrier of step kt at most the loads of the STAGES-2 steps after kt may still be outstanding.
+#pragma unroll
+        for (int s = 0; s < STAGES - 1; ++s)
+            issue_tile_loads(min(s, KT - 1), s);
+        int stage = 0;
+        for (int kt = 0; kt < KT; ++kt)
+        {
+            __builtin_amdgcn_s_waitcnt(vmcnt_imm((STAGES - 2) * TILE_LOADS));
+            __builtin_amdgcn_s_barrier();
+            {
+                // past the end: reload a valid tile into the free stage
+                int st = stage + STAGES - 1;
+                st = st >= STAGES ? st - STAGES : st;
+                issue_tile_loads(min(kt + STAGES - 1, KT - 1), st);
+            }
+            compute(stage);
+            stage = stage + 1 == STAGES ? 0 : stage + 1;
+        }
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm(0)); // drain the tail loads before the LDS goes away
+
+        // ---- epilogue: D layout of a 32x32 tile: lane (col = l32, h), element e: row = 8*(e/4) + 4*h + (e%4)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+        {
+            const int n = n0 + wn * (TN * 32) + j * 32 + l32;
+            if (n >= p.N)
+                continue;
+            float sch = 0.f;
+            if (!RAW && !SPLITK)
+                sch = p.s_ch[n];
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int e = 0; e < 16; ++e)
+                {
+                    const int m = m0 + wm * (TM * 32) + i * 32 + 8 * (e >> 2) + 4 * h + (e & 3);
+                    if (m >= p.M)
+                        continue;
+                    if (SPLITK)
+                        p.partial[((size_t)split * p.M + m) * p.N + n] = acc[i][j][e];
+                    else if (RAW)
+                        p.acc[(size_t)m * p.N + n] = acc[i][j][e];
+                    else
+                    {
+                        float t = (float)acc[i][j][e] * p.s_tok[m];
+                        p.Y[(size_t)m * p.N + n] = f32_to_f16_two_step(t * sch);
+                    }
+                }
+        }
+    }
+
+    // acc[m, n] = sum_s partial[s][m][n] (exact), then the same epilogue; four columns per thread
+    template <bool RAW>
+    __global__ __launch_bounds__(256) void w8a8_splitk_reduce_kernel(Q8GemmParams p)
+    {
+        const int quads = (p.N + 3) >> 2;
+        const long long t = (long long)blockIdx.x * 256 + threadIdx.x;
+        if (t >= (long long)p.M * quads)
+            return;
+        const int m = (int)(t / quads);
+        const int n = (int)(t - (long long)m * quads) * 4;
+        const size_t plane = (size_t)p.M * p.N;
+        const int32_t* src = p.partial + (size_t)m * p.N + n;
+        const bool vec = (p.N & 3) == 0;
+        int a[4] = {0, 0, 0, 0};
+        for (int s = 0; s < p.splits; ++s)
+        {
+            const int32_t* ps = src + (size_t)s * plane;
+            if (vec)
+            {
+                intx4 v = *reinterpret_cast<const intx4*>(ps);
+                a[0] += v.x, a[1] += v.y, a[2] += v.z, a[3] += v.w;
+            }
+            else
+            {
+                for (int j = 0; j < 4; ++j)
+                    if (n + j < p.N)
+                        a[j] += ps[j];
+            }
+        }
+        const float st = RAW ? 0.f : p.s_tok[m];
+        for (int j = 0; j < 4 && n + j < p.N; ++j)
+        {
+            if (RAW)
+                p.acc[(size_t)m * p.N + n + j] = a[j];
+            else
+            {
+                float v = (float)a[j] * st;
+                p.Y[(size_t)m * p.N + n + j] = f32_to_f16_two_step(v * p.s_ch[n + j]);
+            }
+        }
+    }
+
+    namespace
+    {
+        template <int WM, int WN, int TM, int TN, int STAGES, bool RAW, bool SPLITK, int MINW>
+        hipError_t launch_tile(hipStream_t stream, const Q8GemmParams& p)
+        {
+            using T = q8dl::Tile<WM, WN, TM, TN, STAGES>;
+            const int tiles_m = (p.M + T::BM - 1) / T::BM;
+            const int tiles_n = (p.N + T::BN - 1) / T::BN;
+            auto kernel = &w8a8_gemm_dl_kernel<WM, WN, TM, TN, STAGES, RAW, SPLITK, MINW>;
+            if (T::LDS_BYTES > 64 * 1024)
+            {
+                static bool attr_set = false;
+                if (!attr_set)
+                {
+                    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize, T::LDS_BYTES);
+                    if (e != hipSuccess)
+                        return e;
+                    attr_set = true;
+                }
+            }
+            const int splits = SPLITK ? p.splits : 1;
+            hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n * splits), dim3(q8dl::THREADS), T::LDS_BYTES, stream, p);
+            return hipGetLastError();
+        }
+
+        template <bool RAW>
+        hipError_t launch_plan(hipStream_t stream, const Q8GemmParams& p, const workspace::GemmPlan& plan)
+        {
+            hipError_t e;
+            switch (plan.tile)
+            {
+            case workspace::GEMM_TILE_BIG: // 256 x 256, four stages, one workgroup per CU
+                return launch_tile<2, 4, 4, 2, 4, RAW, false, 2>(stream, p);
+            case workspace::GEMM_TILE_MID: // 128 x 128
+                if (!plan.reduce_pass)
+                    return launch_tile<2, 4, 2, 1, 3, RAW, false, 4>(stream, p);
+                e = launch_tile<2, 4, 2, 1, 3, RAW, true, 4>(stream, p);
+                break;
+            default: // 64 x 256, always through the partial sums
+                e = launch_tile<1, 8, 2, 1, 3, RAW, true, 4>(stream, p);
+                break;
+            }
+            if (e != hipSuccess)
+                return e;
+            const long long threads = (long long)p.M * ((p.N + 3) >> 2);
+            hipLaunchKernelGGL((w8a8_splitk_reduce_kernel<RAW>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, stream,
+                               p);
+            return hipGetLastError();
+        }
+    } // namespace
+
+    hipError_t launch_w8a8_gemm(hipStream_t stream, const void* A, const void* s_tok, const void* W, const void* s_ch,
+                                void* Y, void* acc, int M, int N, int K, void* partial_ws)
+    {
+        const workspace::GemmPlan plan =
+            workspace::plan_w4a16_gemm(M, N, K, false, g_tuning.gemm_tile - 1, g_tuning.gemm_splits);
+        if (plan.reduce_pass && !partial_ws)
+            return hipErrorInvalidValue;
+        Q8GemmParams p;
+        p.A = (const int8_t*)A;
+        p.W = (const int8_t*)W;
+        p.s_tok = (const float*)s_tok;
+        p.s_ch = (const float*)s_ch;
+        p.Y = (half_t*)Y;
+        p.acc = (int32_t*)acc;
+        p.partial = (int32_t*)partial_ws;
+        p.M = M;
+        p.N = N;
+        p.K = K;
+        p.splits = plan.splits;
+        return acc ? launch_plan<true>(stream, p, plan) : launch_plan<false>(stream, p, plan);
+    }
+} // namespace nnf

@@ -177,6 +177,17 @@ size_t nnf_w8a8_gemm_workspace_bytes(int M, int N, int K)
     return nnf::workspace::w8a8_gemm(M, N, K);
 }
 
+// room for the int32 partial sums when the MFMA GEMM serves the shape (the M <= 16 kernel needs none)
+static int check_w8a8_workspace(int M, int N, int K, const void* workspace, size_t workspace_bytes)
+{
+    if (nnf::g_tuning.force_path != 3 && nnf::w8a8_skinny_supported(M, K))
+        return NNF_OK;
+    const size_t need = tuned_partial_bytes(M, N, K, false);
+    if (need > 0 && (!workspace || !aligned16(workspace) || workspace_bytes < need))
+        return NNF_ERR_WORKSPACE_TOO_SMALL;
+    return NNF_OK;
+}
+
 static int check_w8a8(const void* A, const void* W, const void* out, int M, int N, int K)
 {
     if (!A || !W || !out || M <= 0 || N <= 0 || K <= 0)
@@ -192,33 +203,36 @@ static int check_w8a8(const void* A, const void* W, const void* out, int M, int 
 int nnf_w8a8_gemm(nnf_stream_t stream, const void* A, const void* s_tok, const void* W, const void* s_ch, void* Y,
                   int M, int N, int K, void* workspace, size_t workspace_bytes)
 {
-    (void)workspace;
-    (void)workspace_bytes;
     int st = check_w8a8(A, W, Y, M, N, K);
     if (st != NNF_OK)
         return st;
     if (!s_tok || !s_ch)
         return NNF_ERR_INVALID_ARGUMENT;
+    st = check_w8a8_workspace(M, N, K, workspace, workspace_bytes);
+    if (st != NNF_OK)
+        return st;
     DeviceInfo dev;
     st = current_device_info(dev);
     if (st != NNF_OK)
         return st;
-    return (int)nnf::launch_w8a8((hipStream_t)stream, A, s_tok, W, s_ch, Y, nullptr, M, N, K, dev.num_cu);
+    return (int)nnf::launch_w8a8((hipStream_t)stream, A, s_tok, W, s_ch, Y, nullptr, M, N, K, dev.num_cu, workspace);
 }
 
 int nnf_w8a8_gemm_acc(nnf_stream_t stream, const void* A, const void* W, void* acc, int M, int N, int K,
                       void* workspace, size_t workspace_bytes)
 {
-    (void)workspace;
-    (void)workspace_bytes;
     int st = check_w8a8(A, W, acc, M, N, K);
+    if (st != NNF_OK)
+        return st;
+    st = check_w8a8_workspace(M, N, K, workspace, workspace_bytes);
     if (st != NNF_OK)
         return st;
     DeviceInfo dev;
     st = current_device_info(dev);
     if (st != NNF_OK)
         return st;
-    return (int)nnf::launch_w8a8((hipStream_t)stream, A, nullptr, W, nullptr, nullptr, acc, M, N, K, dev.num_cu);
+    return (int)nnf::launch_w8a8((hipStream_t)stream, A, nullptr, W, nullptr, nullptr, acc, M, N, K, dev.num_cu,
+                                 workspace);
 }
 
 // ---- fused MLP block ------------------------------------------------------------------------------

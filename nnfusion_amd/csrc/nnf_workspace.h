@@ -133,7 +133,47 @@ namespace nnf
             const bool gate = act == 1;
             return rms_rows(M, K) + gemm_partial_bytes(M, N, gate, plan_w4a16_gemm(M, N, K, gate));
         }
-        inline size_t w8a8_gemm(int, int, int) { return 0; }
+        // ---- W8A8 ---------------------------------------------------------------------------------------
+        struct Q8SkinnyPlan
+        {
+            int cps = 0, ks = 0; // 64-byte chunks of K per wavefront, wavefronts per workgroup
+            size_t lds = 0;      // LDS bytes without the output parking area
+        };
+        inline Q8SkinnyPlan plan_w8a8_skinny(int M, int K)
+        {
+            Q8SkinnyPlan pl;
+            const int C = K >> 6;
+            static const int options[] = {1, 2, 4, 8, 16};
+            for (int cps : options)
+            {
+                const int ks = (C + cps - 1) / cps;
+                if (ks <= 16)
+                {
+                    pl.cps = cps;
+                    pl.ks = ks;
+                    break;
+                }
+            }
+            if (pl.cps)
+                pl.lds = (size_t)C * 4 * M * 16 + (size_t)2 * pl.ks * 256 * 4;
+            return pl;
+        }
+        inline bool w8a8_skinny_fits(int M, int K)
+        {
+            if (M < 1 || M > 16 || (K & 63))
+                return false;
+            const Q8SkinnyPlan pl = plan_w8a8_skinny(M, K);
+            return pl.cps != 0 && pl.lds + 16 * 1024 <= LDS_BYTES_PER_CU;
+        }
+        // nnf_w8a8_gemm / nnf_w8a8_gemm_acc: [ int32 partial sums ] (same tile plan as the fp16 x int4 GEMM)
+        inline size_t w8a8_gemm(int M, int N, int K)
+        {
+            if (M <= 0 || N <= 0 || K < 128)
+                return 0;
+            if (w8a8_skinny_fits(M, K))
+                return 0;
+            return gemm_partial_bytes(M, N, false, plan_w4a16_gemm(M, N, K, false));
+        }
         // nnf_fused_mlp_w4a16: [ normalised x: M x H fp16 ][ h: M x I fp16 ][ partial sums of either GEMM ]
         inline size_t fused_mlp_h_offset(int M, int H) { return rms_rows(M, H); }
         inline size_t fused_mlp_partial_offset(int M, int H, int I)

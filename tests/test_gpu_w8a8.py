@@ -15,19 +15,34 @@ def _t(gpu, *arrays):
     return [torch.from_numpy(np.ascontiguousarray(a)).to(gpu) for a in arrays]
 
 
-@pytest.fixture(params=["auto", "mfma_gemm"])
+# "auto": the library's own choice (the M <= 16 kernel where it applies); otherwise the MFMA GEMM with a
+# forced tile (1 big 256x256, 2 mid 128x128, 3 small 64x256) and number of K ranges (int32 partial sums,
+# added exactly by the reduction pass)
+@pytest.fixture(params=["auto", (0, 0), (1, 0), (2, 1), (2, 3), (3, 1), (3, 2)],
+                ids=lambda p: p if isinstance(p, str) else f"gemm-tile{p[0]}-splits{p[1]}")
 def path(request):
     from nnfusion_amd import _lib
 
     tune = _lib.kernels().nnf_internal_tune
-    tune(0, {"auto": 0, "mfma_gemm": 3}[request.param])
+    if request.param != "auto":
+        tune(0, 3)
+        tune(3, request.param[0])
+        tune(4, request.param[1])
     yield request.param
     tune(0, 0)
+    tune(3, 0)
+    tune(4, 0)
+
+
+def _big_ws(gpu):
+    import torch
+
+    return torch.empty(64 << 20, dtype=torch.uint8, device=gpu)
 
 
 @pytest.mark.parametrize("m,n,k", [
     (1, 64, 128), (1, 1000, 1024), (3, 17, 256), (16, 512, 8192), (32, 300, 512), (100, 257, 384),
-    (256, 256, 128), (512, 1024, 2048), (1, 8192, 8192), (32, 8192, 8192),
+    (256, 256, 128), (512, 1024, 2048), (1, 8192, 8192), (32, 4096, 4096),
 ])
 def test_accumulators_bit_exact(gpu, path, m, n, k):
     import torch
@@ -37,8 +52,9 @@ def test_accumulators_bit_exact(gpu, path, m, n, k):
     print(f"case M={m} N={n} K={k} path={path}", flush=True)
     a, s_tok, w, s_ch = datagen.w8a8_case(0, m, n, k)
     ta, tw, tst, tsc = _t(gpu, a, w, s_tok, s_ch)
-    acc = ops.w8a8_gemm_acc(ta, tw).cpu().numpy()
-    y = ops.w8a8_gemm(ta, tst, tw, tsc).cpu().numpy()
+    ws = _big_ws(gpu)
+    acc = ops.w8a8_gemm_acc(ta, tw, workspace=ws).cpu().numpy()
+    y = ops.w8a8_gemm(ta, tst, tw, tsc, workspace=ws).cpu().numpy()
     torch.cuda.synchronize()
     ref = oracle.w8a8_acc(a, w)
     assert np.array_equal(acc, ref)
@@ -58,7 +74,7 @@ def test_extreme_values_do_not_overflow(gpu, path):
     w = np.full((n, k), 127, np.int8)
     w[::2] = -127
     ta, tw = _t(gpu, a, w)
-    acc = ops.w8a8_gemm_acc(ta, tw).cpu().numpy()
+    acc = ops.w8a8_gemm_acc(ta, tw, workspace=_big_ws(gpu)).cpu().numpy()
     torch.cuda.synchronize()
     assert np.array_equal(acc, oracle.w8a8_acc(a, w))
     assert abs(int(acc[0, 1])) == 8192 * 127 * 127
