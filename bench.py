@@ -57,6 +57,8 @@ def main():
     ap.add_argument("--pmc-probe", action="store_true",
                     help="for hardware-counter runs: a plain copy of known size, then the sweep launched eagerly; "
                          "no timing, no JSON")
+    ap.add_argument("--mfma-probe", action="store_true",
+                    help="print the MFMA-only rates (no memory traffic) for different operand values and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU (no sharding, no collectives); use --gpus 1")
@@ -117,6 +119,10 @@ def main():
         e1.record()
         torch.cuda.synchronize()
         return e0.elapsed_time(e1) * 1000.0 / reps
+
+    if args.mfma_probe:
+        print(json.dumps(run_mfma_probe(torch, lib)))
+        return
 
     if args.pmc_probe:
         # Calibration for FETCH_SIZE / WRITE_SIZE: a device-to-device copy that reads and writes exactly
@@ -215,6 +221,27 @@ def main():
         "extra": extra,
     }
     print(json.dumps(out))
+
+
+def run_mfma_probe(torch, lib):
+    """MFMA-only loops (operands in registers, two wavefronts per SIMD, eight accumulators each): the rate the
+    matrix cores sustain depends on the operand values, because the chip is power managed."""
+    import ctypes
+
+    fn = lib.nnf_internal_mfma_probe
+    fn.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_double),
+                   ctypes.POINTER(ctypes.c_double)]
+    fn.restype = ctypes.c_int
+    num_cu = torch.cuda.get_device_properties(0).multi_processor_count
+    out = {"num_cu": num_cu, "unit": "Tera-op/s", "note": "published dense peaks: fp16 2500, int8 5000"}
+    for kind, kname in ((0, "f16_32x32x16"), (1, "i8_32x32x32")):
+        for mode, mname in ((0, "all_ones"), (1, "normal_or_uniform_random"), (2, "small_integers")):
+            tops, mhz = ctypes.c_double(0.0), ctypes.c_double(0.0)
+            st = fn(kind, mode, 60000, num_cu, ctypes.byref(tops), ctypes.byref(mhz))
+            if st != 0:
+                raise RuntimeError(f"nnf_internal_mfma_probe failed: {st}")
+            out[f"{kname}.{mname}"] = {"tops": round(tops.value, 1), "shader_mhz": round(mhz.value)}
+    return out
 
 
 def run_extra(torch, np, dev, lib, datagen, ops):
