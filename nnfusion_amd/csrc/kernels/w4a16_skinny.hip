@@ -42,8 +42,8 @@ namespace nnf
     //       (a row of A is staged in memory order; the odd row stride keeps rows on different banks)
     //   ncorr    [G][16 m] fp32: constant part of every group sum, negated
     //   scales   sc[2][16 rows][G] fp16 (as in memory), each copy padded to 16 bytes
-    //   red      [2][M][16 n][KSP] fp32 partial sums, the KS wavefronts of one output side by side
-    //            (KSP = KS rounded up to a multiple of 4; the padding stays zero)
+    //   red      [2][M][16 n][16] fp32 partial sums, the KS <= 16 wavefronts of one output side by side
+    //            (slots of absent wavefronts stay zero)
     //   outb     [tiles of this workgroup][M][16] fp32
     // Group (chunk) index of wavefront w, pass h, slot c:  (h*KS + w)*CPS + c.
     template <int CPS, bool A_REGS, int H>
@@ -73,7 +73,7 @@ namespace nnf
         const int sc_units = (16 * G * 2 + 15) >> 4; // 16-byte units of one scale copy
         floatx4* nc_lds = reinterpret_cast<floatx4*>(lds + a_units); // [G][4 kq] x (4 m)
         uintx4* sc_lds = lds + a_units + G * 4;
-        const int KSP = (KS + 3) & ~3;
+        constexpr int KSP = 16; // partial-sum slots per output: a constant, so that the row stride below is an immediate
         const int red_copy = M * 16 * KSP;
         float* red = reinterpret_cast<float*>(sc_lds + 2 * sc_units); // [2][M][16][KSP]
         float* outb = red + 2 * red_copy;
@@ -273,12 +273,16 @@ namespace nnf
         auto finish = [&](floatx4 acc, int par, auto put_s, auto get_s, int tile_s, auto get_w, int tile_w, int h_w,
                           uintx4* w_free, auto last, int tile_cur) {
             {
-                float* rp = red + par * red_copy + col * KSP + wave;
+                // The address is recomputed at every call (two instructions): kept across the unrolled
+                // tail of the tile loop it would be spilled.
+                int slot = (kq * 64 + col) * KSP + wave;
+                asm volatile("" : "+v"(slot));
+                float* rp = red + par * red_copy + slot;
                 const float av[4] = {acc.x, acc.y, acc.z, acc.w};
 #pragma unroll
                 for (int r = 0; r < 4; ++r)
                     if (kq * 4 + r < M)
-                        rp[(kq * 4 + r) * 16 * KSP] = av[r];
+                        rp[r * 16 * KSP] = av[r];
             }
             // Order matters for the in-order load counter: the scale registers (loaded one tile ago) are
             // consumed first, then reloaded, and only then is the freed weight register set reloaded --
@@ -304,8 +308,7 @@ namespace nnf
             {
                 const int o = tid >> 2, q = tid & 3; // o = m*16 + n
                 floatx4 p4 = {0.f, 0.f, 0.f, 0.f};
-                if (q * 4 < KSP)
-                    p4 = *reinterpret_cast<const floatx4*>(red + par * red_copy + o * KSP + q * 4);
+                p4 = *reinterpret_cast<const floatx4*>(red + par * red_copy + o * KSP + q * 4);
                 float v = quad_sum((p4.x + p4.y) + (p4.z + p4.w));
                 if (decltype(last)::value)
                 {

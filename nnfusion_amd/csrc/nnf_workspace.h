@@ -97,7 +97,7 @@ namespace nnf
             p.a_regs = p.cps <= 2 && p.h == 1;
             const size_t a_bytes = ((size_t)G * 16 + 1) * M * 16 + (size_t)G * 64;
             const size_t sc_bytes = 2 * (((size_t)16 * G * 2 + 15) & ~(size_t)15);
-            p.lds = a_bytes + sc_bytes + (size_t)2 * M * 16 * ((p.ks + 3) & ~3) * 4;
+            p.lds = a_bytes + sc_bytes + (size_t)2 * M * 16 * 16 * 4;
             return p;
         }
         // true when one workgroup can hold the activations (M <= 16 rows of K) in LDS
