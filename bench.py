@@ -35,6 +35,10 @@ MFMA_I8_PEAK_TOPS = 5000.0     # dense int8 MFMA
 DECODE_SHAPES = [(12288, 4096), (4096, 4096), (22016, 4096), (4096, 11008)]  # (N, K), M = 1
 GROUP = 128
 PROBE_BYTES = 1 << 30  # size of the calibration copy of --pmc-probe
+# HBM bytes per launch of the K = 4096 skinny kernel (mean over its three launches of a step), from two
+# rocprofv3 --pmc runs of `bench.py --pmc-probe`: FETCH_SIZE 13302.8 KiB x 2.000 (the factor by which the
+# counter under-reports the 1 GiB calibration copy) + WRITE_SIZE 25.0 KiB x 1.000.  Algorithmic: 27 067 392.
+SKINNY_K4096_TRAFFIC_BYTES = int((13302.8 * 2.0 + 25.0) * 1024)
 
 
 def w4a16_bytes(m, n, k):
@@ -181,7 +185,7 @@ def main():
         "peak": HBM_PEAK_GBS,
         "unit": "GB/s",
         "frac": round(dom_bytes / dom_us / 1e3 / HBM_PEAK_GBS, 4),
-        "traffic": None,
+        "traffic": SKINNY_K4096_TRAFFIC_BYTES,
         "bytes_per_launch": int(dom_bytes),
         "us_per_launch": round(dom_us, 3),
     }
@@ -251,7 +255,7 @@ def run_extra(torch, np, dev, lib, datagen, ops):
         return torch.from_numpy(np.ascontiguousarray(a)).to(dev)
 
     def time_us(fn, iters):
-        for _ in range(2):
+        for _ in range(3):
             fn()
         torch.cuda.synchronize()
         e0 = torch.cuda.Event(enable_timing=True)
@@ -273,7 +277,7 @@ def run_extra(torch, np, dev, lib, datagen, ops):
         a = dev_t(datagen.normal_f16(0, datagen.S_ACT, (m, k)))
         y = torch.empty((m, n), dtype=torch.float16, device=dev)
         ws = torch.empty(max(lib.nnf_w4a16_gemm_workspace_bytes(m, n, k, GROUP), 256), dtype=torch.uint8, device=dev)
-        us = time_us(lambda: ops.w4a16_gemm(a, twq, ts, out=y, workspace=ws), 20 if m <= 1024 else 8)
+        us = time_us(lambda: ops.w4a16_gemm(a, twq, ts, out=y, workspace=ws), 20)
         fl = 2.0 * m * n * k
         rows.append({"M": m, "us": round(us, 2), "TFLOP/s": round(fl / us / 1e6, 1),
                      "frac_mfma_f16": round(fl / us / 1e6 / MFMA_F16_PEAK_TFLOPS, 4),
@@ -283,13 +287,13 @@ def run_extra(torch, np, dev, lib, datagen, ops):
     # configs[3]: W8A8, N = K = 8192
     _, _, w8, s_ch = datagen.w8a8_case(0, 1, n, k)
     tw8, tsch = dev_t(w8), dev_t(s_ch)
-    ws = torch.empty(max(lib.nnf_w8a8_gemm_workspace_bytes(4096, n, k), 256), dtype=torch.uint8, device=dev)
     rows = []
     for m in (1, 32, 512, 4096):
         a8 = dev_t(datagen.uniform_i8(0, datagen.S_A8, (m, k)))
         st = dev_t(datagen.uniform_f32(0, datagen.S_STOK, (m,), 0.001, 0.01))
         y = torch.empty((m, n), dtype=torch.float16, device=dev)
-        us = time_us(lambda: ops.w8a8_gemm(a8, st, tw8, tsch, out=y, workspace=ws), 20 if m <= 512 else 8)
+        ws = torch.empty(max(lib.nnf_w8a8_gemm_workspace_bytes(m, n, k), 256), dtype=torch.uint8, device=dev)
+        us = time_us(lambda: ops.w8a8_gemm(a8, st, tw8, tsch, out=y, workspace=ws), 20)
         op = 2.0 * m * n * k
         rows.append({"M": m, "us": round(us, 2), "TOP/s": round(op / us / 1e6, 1),
                      "frac_mfma_i8": round(op / us / 1e6 / MFMA_I8_PEAK_TOPS, 4),
