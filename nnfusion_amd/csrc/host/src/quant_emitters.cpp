@@ -57,8 +57,6 @@ namespace nnfusion
                         return nullptr;
                     if (gate && (has_bias || has_res))
                         return nullptr;
-                    if (rms && has_res)
-                        return nullptr;
                     const Shape& a = m_context->inputs[0]->get_shape();
                     const Shape& w = m_context->inputs[1]->get_shape();
                     const size_t K = a.back();
@@ -120,13 +118,18 @@ namespace nnfusion
                     if (K % 128 != 0 || K > 133000 || M == 0 || N == 0)
                         return nullptr;
                     const bool raw = gop->localOpConfig.getRoot()["out_type"].get<std::string>() == "i32";
+                    // int32 partial sums when the tile plan of the shape splits K
+                    const size_t ws_bytes = nnf::workspace::w8a8_gemm((int)M, (int)N, (int)K);
+                    std::string ws = "nullptr";
+                    if (ws_bytes > 0)
+                        ws = allocate_tensor(Shape{ws_bytes}, element::character)->get_name();
                     LanguageUnit_p lu(new LanguageUnit(get_function_name()));
                     if (raw)
                         *lu << "NNF_HIP_CHECK(nnf_w8a8_gemm_acc(stream, input0, input2, output0, " << M << ", " << N << ", "
-                            << K << ", nullptr, 0));\n";
+                            << K << ", " << ws << ", " << ws_bytes << "));\n";
                     else
                         *lu << "NNF_HIP_CHECK(nnf_w8a8_gemm(stream, input0, input1, input2, input3, output0, " << M << ", "
-                            << N << ", " << K << ", nullptr, 0));\n";
+                            << N << ", " << K << ", " << ws << ", " << ws_bytes << "));\n";
                     return lu;
                 }
             };

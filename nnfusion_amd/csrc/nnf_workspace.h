@@ -46,8 +46,9 @@ namespace nnf
                 return p;
             const int tiles = p.tile == GEMM_TILE_MID ? ceil_div(M, 128) * ceil_div(N, 128)
                                                       : ceil_div(M, 64) * ceil_div(N, 256);
-            // two workgroups fit a CU; every split keeps at least four groups (eight K steps)
-            int s = (2 * PLAN_CUS) / (tiles > 0 ? tiles : 1);
+            // about one workgroup per CU (measured: more splits cost more in partial-sum traffic than they gain in
+            // balance); every split keeps at least four groups (eight K steps)
+            int s = PLAN_CUS / (tiles > 0 ? tiles : 1);
             if (s > G / 4)
                 s = G / 4;
             if (s < 1)

@@ -341,14 +341,14 @@ int main(int argc, char** argv)
 
         // fused variant: gamma, bias; the scratch tensor appears in signature and call.  Its size: the normalised
         // activations (256 x 4096 fp16) + the partial sums of the plan for this shape (128 x 128 tiles: 2 x 32 of
-        // them, K split 8 ways: 8 x 256 x 4096 fp32)
+        // them, K split 4 ways: 4 x 256 x 4096 fp32)
         graph::Graph g2;
         auto n2 = quant_dot_graph(g2, 256, 4096, 4096, "{\"rms_norm\": true, \"has_bias\": true, \"rms_eps\": 1e-5}", true, true);
         auto k2 = sel.pick_first(n2, ROCM_GPU).second;
         auto fu2 = k2->get_or_emit_source();
         CONTAINS(fu2->body_unit->get_code(), "nnf_w4a16_gemm_fused(stream, input0, input1, input2, output0, 256, 4096, 4096, 128, 8, input3, 1.000000000e-05f, input4, nullptr, NNF_ACT_NONE, ");
         EXPECT(k2->m_context->tensors.size() == 1 &&
-               k2->m_context->tensors[0]->size() == (size_t)256 * 4096 * 2 + (size_t)8 * 256 * 4096 * 4);
+               k2->m_context->tensors[0]->size() == (size_t)256 * 4096 * 2 + (size_t)4 * 256 * 4096 * 4);
         CONTAINS(fu2->signature_unit->get_code(), "char* " + k2->m_context->tensors[0]->get_name());
         CONTAINS(fu2->call_unit->get_code(), k2->m_context->tensors[0]->get_name() + ");");
         // SiLU gate: N is half the weight rows
@@ -398,9 +398,13 @@ int main(int argc, char** argv)
         auto sc = param(g, element::f32, Shape{8192});
         auto n = g.add_node_and_edge(std::make_shared<op::GenericOp>("q", "QuantDotW8A8", op::OpConfig::any()), {a, st, w, sc});
         EXPECT(n->get_output_element_type(0) == element::f16 && n->get_output_shape(0) == (Shape{32, 8192}));
-        auto fu = sel.pick_first(n, ROCM_GPU).second->get_or_emit_source();
+        auto kq = sel.pick_first(n, ROCM_GPU).second;
+        auto fu = kq->get_or_emit_source();
+        // M = 32: 64 x 256 tiles (32 of them), K split 8 ways: 8 x 32 x 8192 int32 partial sums in a scratch tensor
+        EXPECT(kq->m_context->tensors.size() == 1 && kq->m_context->tensors[0]->size() == (size_t)8 * 32 * 8192 * 4);
         EXPECT(fu->body_unit->get_code() ==
-               "NNF_HIP_CHECK(nnf_w8a8_gemm(stream, input0, input1, input2, input3, output0, 32, 8192, 8192, nullptr, 0));\n");
+               "NNF_HIP_CHECK(nnf_w8a8_gemm(stream, input0, input1, input2, input3, output0, 32, 8192, 8192, " +
+                   kq->m_context->tensors[0]->get_name() + ", 8388608));\n");
         auto n2 = g.add_node_and_edge(std::make_shared<op::GenericOp>("q", "QuantDotW8A8", op::OpConfig::any::parse("{\"out_type\": \"i32\"}")),
                                       {a, st, w, sc});
         EXPECT(n2->get_output_element_type(0) == element::i32);
@@ -421,10 +425,10 @@ int main(int argc, char** argv)
         auto fm = k->get_or_emit_source();
         CONTAINS(fm->body_unit->get_code(), "nnf_fused_mlp_w4a16(stream, input0, input1, 1.000000000e-06f, input2, input3, input4, input5, output0, 256, 4096, 11008, 128, 8, ");
         // RMSNorm(x) [256, 4096] fp16 + h [256, 11008] fp16 + the larger of the two partial-sum areas: gate/up
-        // (2 x 86 tiles of 128 x (128 + 128), K split in 2: 2 x 256 x 22016 fp32) vs down (64 tiles, split 8)
+        // (2 x 86 tiles of 128 x (128 + 128), K not split: none) vs down (2 x 32 tiles, K split 4 ways)
         EXPECT(k->m_context->tensors.size() == 1 &&
                k->m_context->tensors[0]->size() ==
-                   (size_t)256 * 4096 * 2 + (size_t)256 * 11008 * 2 + (size_t)2 * 256 * 22016 * 4);
+                   (size_t)256 * 4096 * 2 + (size_t)256 * 11008 * 2 + (size_t)4 * 256 * 4096 * 4);
     });
 
     run_case("codegen_project", [&] {
