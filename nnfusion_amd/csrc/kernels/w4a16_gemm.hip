@@ -156,6 +156,12 @@ namespace nnf
         // 256 x 256 tiles: wavefronts 2 (M) x 4 (N), each 4 x 2 MFMA tiles; one workgroup per CU
         hipError_t launch_gemm_big(hipStream_t stream, const GemmParams& p, bool gate, bool hb, bool hr)
         {
+            if (p.partial)
+            {
+                if (gate)
+                    return launch_gemm_dl<2, 4, 4, 2, true, false, false, true, 2>(stream, p);
+                return launch_gemm_dl<2, 4, 4, 2, false, false, false, true, 2>(stream, p);
+            }
             if (gate)
                 return launch_gemm_dl<2, 4, 4, 2, true, false, false, false, 2>(stream, p);
             if (hb && hr)
@@ -210,7 +216,7 @@ namespace nnf
         hipError_t e;
         switch (plan.tile)
         {
-        case workspace::GEMM_TILE_BIG: return launch_gemm_big(stream, p, gate, hb, hr);
+        case workspace::GEMM_TILE_BIG: e = launch_gemm_big(stream, p, gate, hb, hr); break;
         case workspace::GEMM_TILE_MID: e = launch_gemm_mid(stream, p, gate, hb, hr); break;
         default: e = launch_gemm_small(stream, p, gate, hb, hr); break;
         }

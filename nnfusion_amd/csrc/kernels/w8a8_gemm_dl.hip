@@ -319,7 +319,10 @@ namespace nnf
             switch (plan.tile)
             {
             case workspace::GEMM_TILE_BIG: // 256 x 256, four stages, one workgroup per CU
-                return launch_tile<2, 4, 4, 2, 4, RAW, false, 2>(stream, p);
+                if (!plan.reduce_pass)
+                    return launch_tile<2, 4, 4, 2, 4, RAW, false, 2>(stream, p);
+                e = launch_tile<2, 4, 4, 2, 4, RAW, true, 2>(stream, p);
+                break;
             case workspace::GEMM_TILE_MID: // 128 x 128
                 if (!plan.reduce_pass)
                     return launch_tile<2, 4, 2, 1, 3, RAW, false, 4>(stream, p);
@@ -342,7 +345,7 @@ namespace nnf
                                 void* Y, void* acc, int M, int N, int K, void* partial_ws)
     {
         const workspace::GemmPlan plan =
-            workspace::plan_w4a16_gemm(M, N, K, false, g_tuning.gemm_tile - 1, g_tuning.gemm_splits);
+            workspace::plan_w8a8_gemm(M, N, K, g_tuning.gemm_tile - 1, g_tuning.gemm_splits);
         if (plan.reduce_pass && !partial_ws)
             return hipErrorInvalidValue;
         Q8GemmParams p;

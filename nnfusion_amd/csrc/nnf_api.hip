@@ -182,7 +182,8 @@ static int check_w8a8_workspace(int M, int N, int K, const void* workspace, size
 {
     if (nnf::g_tuning.force_path != 3 && nnf::w8a8_skinny_supported(M, K))
         return NNF_OK;
-    const size_t need = tuned_partial_bytes(M, N, K, false);
+    const size_t need = nnf::workspace::gemm_partial_bytes(
+        M, N, false, nnf::workspace::plan_w8a8_gemm(M, N, K, nnf::g_tuning.gemm_tile - 1, nnf::g_tuning.gemm_splits));
     if (need > 0 && (!workspace || !aligned16(workspace) || workspace_bytes < need))
         return NNF_ERR_WORKSPACE_TOO_SMALL;
     return NNF_OK;

@@ -3,6 +3,7 @@
 // which reserve the scratch tensor at compile time.  Nothing here may depend on the device at hand.
 #pragma once
 
+#include <math.h>
 #include <stddef.h>
 
 namespace nnf
@@ -28,36 +29,75 @@ namespace nnf
 
         inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
-        // N: output columns.  forced_splits > 0 overrides the split count (experiments).
+        // Estimated run time (seconds) of one tile shape and split count, from rates measured on an MI355X with
+        // N(0,1) activations (the GEMMs are power bound: ~950 / 700 / 450 TFLOP/s for the three tile shapes when
+        // every CU has a workgroup, and a CU runs faster when fewer are busy: hence the square root), ~6 TB/s for
+        // the partial sums (written, then read by the reduction pass) and ~3 us for the second launch.
+        // rate_scale: 1 for the fp16 x int4 GEMM, 1.7 for W8A8 (same tiles on the int8 matrix cores; its weight
+        // bytes differ too, but a memory-bound W8A8 shape is decided by the partial-sum term either way)
+        inline double estimate_gemm(int M, int N, int K, bool gate, int tile, int splits, double rate_scale)
+        {
+            const int bm = tile == GEMM_TILE_BIG ? 256 : tile == GEMM_TILE_MID ? 128 : 64;
+            const int bn = tile == GEMM_TILE_BIG ? (gate ? 128 : 256) : tile == GEMM_TILE_MID ? 128 : 256;
+            const double rate = rate_scale * (tile == GEMM_TILE_BIG ? 950e12 : tile == GEMM_TILE_MID ? 700e12 : 450e12);
+            const int tiles_m = ceil_div(M, bm), tiles_n = ceil_div(N, bn);
+            const double blocks = (double)tiles_m * tiles_n * splits;
+            const double rounds = (double)(((long long)blocks + PLAN_CUS - 1) / PLAN_CUS);
+            const double util = blocks / (rounds * PLAN_CUS);
+            const double n_total = (gate ? 2.0 : 1.0) * N;
+            const double flops = 2.0 * tiles_m * bm * n_total * K; // whole tile rows are computed
+            double t = flops / (rate * sqrt(util));
+            const double weight_time = n_total * K / 2.0 / 4e12;
+            if (t < weight_time)
+                t = weight_time;
+            if (splits > 1 || tile == GEMM_TILE_SMALL)
+                t += 2.0 * splits * M * n_total * 4.0 / 6e12 + 3e-6;
+            return t;
+        }
+
+        inline double estimate_w4a16_gemm(int M, int N, int K, bool gate, int tile, int splits)
+        {
+            return estimate_gemm(M, N, K, gate, tile, splits, 1.0);
+        }
+
+        // N: output columns.  forced_tile >= 0 / forced_splits > 0 override the choice (experiments).
+        inline GemmPlan plan_gemm(int M, int N, int K, bool gate, double rate_scale, int forced_tile, int forced_splits)
+        {
+            static const int split_options[] = {1, 2, 3, 4, 6, 8, 12, 16};
+            const int G = K / 128;
+            GemmPlan best;
+            double best_t = -1.0;
+            for (int tile = GEMM_TILE_BIG; tile <= GEMM_TILE_SMALL; ++tile)
+            {
+                if (forced_tile >= 0 ? tile != forced_tile
+                                     : ((tile == GEMM_TILE_BIG && M <= 128) || (tile == GEMM_TILE_SMALL && M > 64) ||
+                                        (tile == GEMM_TILE_MID && M <= 64)))
+                    continue;
+                for (int s : split_options)
+                {
+                    // every split keeps at least four groups (eight K steps)
+                    if (forced_splits > 0 ? s != 1 : (s > 1 && G / s < 4))
+                        continue;
+                    const int splits = forced_splits > 0 ? (forced_splits < G ? forced_splits : G) : s;
+                    const double t = estimate_gemm(M, N, K, gate, tile, splits, rate_scale);
+                    if (best_t < 0.0 || t < best_t)
+                    {
+                        best_t = t;
+                        best.tile = tile;
+                        best.splits = splits;
+                    }
+                }
+            }
+            best.reduce_pass = best.splits > 1 || best.tile == GEMM_TILE_SMALL;
+            return best;
+        }
         inline GemmPlan plan_w4a16_gemm(int M, int N, int K, bool gate, int forced_tile = -1, int forced_splits = 0)
         {
-            GemmPlan p;
-            const int G = K / 128;
-            const int big_tiles = ceil_div(M, 256) * ceil_div(N, gate ? 128 : 256);
-            if (M <= 64)
-                p.tile = GEMM_TILE_SMALL;
-            else if (M <= 128 || big_tiles < (PLAN_CUS * 3) / 4)
-                p.tile = GEMM_TILE_MID;
-            else
-                p.tile = GEMM_TILE_BIG;
-            if (forced_tile >= 0)
-                p.tile = forced_tile;
-            if (p.tile == GEMM_TILE_BIG)
-                return p;
-            const int tiles = p.tile == GEMM_TILE_MID ? ceil_div(M, 128) * ceil_div(N, 128)
-                                                      : ceil_div(M, 64) * ceil_div(N, 256);
-            // about one workgroup per CU (measured: more splits cost more in partial-sum traffic than they gain in
-            // balance); every split keeps at least four groups (eight K steps)
-            int s = PLAN_CUS / (tiles > 0 ? tiles : 1);
-            if (s > G / 4)
-                s = G / 4;
-            if (s < 1)
-                s = 1;
-            if (forced_splits > 0)
-                s = forced_splits < G ? forced_splits : G;
-            p.splits = s;
-            p.reduce_pass = s > 1 || p.tile == GEMM_TILE_SMALL;
-            return p;
+            return plan_gemm(M, N, K, gate, 1.0, forced_tile, forced_splits);
+        }
+        inline GemmPlan plan_w8a8_gemm(int M, int N, int K, int forced_tile = -1, int forced_splits = 0)
+        {
+            return plan_gemm(M, N, K, false, 1.7, forced_tile, forced_splits);
         }
         inline size_t gemm_partial_bytes(int M, int N, bool gate, const GemmPlan& p)
         {
@@ -173,7 +213,7 @@ namespace nnf
                 return 0;
             if (w8a8_skinny_fits(M, K))
                 return 0;
-            return gemm_partial_bytes(M, N, false, plan_w4a16_gemm(M, N, K, false));
+            return gemm_partial_bytes(M, N, false, plan_w8a8_gemm(M, N, K));
         }
         // nnf_fused_mlp_w4a16: [ normalised x: M x H fp16 ][ h: M x I fp16 ][ partial sums of either GEMM ]
         inline size_t fused_mlp_h_offset(int M, int H) { return rms_rows(M, H); }

@@ -425,10 +425,11 @@ int main(int argc, char** argv)
         auto fm = k->get_or_emit_source();
         CONTAINS(fm->body_unit->get_code(), "nnf_fused_mlp_w4a16(stream, input0, input1, 1.000000000e-06f, input2, input3, input4, input5, output0, 256, 4096, 11008, 128, 8, ");
         // RMSNorm(x) [256, 4096] fp16 + h [256, 11008] fp16 + the larger of the two partial-sum areas: gate/up
-        // (2 x 86 tiles of 128 x (128 + 128), K not split: none) vs down (2 x 32 tiles, K split 4 ways)
+        // (86 tiles of 256 x (128 + 128), K split in 2: 2 x 256 x 22016 fp32) vs down (2 x 32 tiles of 128 x 128,
+        // K split 4 ways: 4 x 256 x 4096 fp32)
         EXPECT(k->m_context->tensors.size() == 1 &&
                k->m_context->tensors[0]->size() ==
-                   (size_t)256 * 4096 * 2 + (size_t)256 * 11008 * 2 + (size_t)4 * 256 * 4096 * 4);
+                   (size_t)256 * 4096 * 2 + (size_t)256 * 11008 * 2 + (size_t)2 * 256 * 22016 * 4);
     });
 
     run_case("codegen_project", [&] {

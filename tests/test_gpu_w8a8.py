@@ -18,7 +18,7 @@ def _t(gpu, *arrays):
 # "auto": the library's own choice (the M <= 16 kernel where it applies); otherwise the MFMA GEMM with a
 # forced tile (1 big 256x256, 2 mid 128x128, 3 small 64x256) and number of K ranges (int32 partial sums,
 # added exactly by the reduction pass)
-@pytest.fixture(params=["auto", (0, 0), (1, 0), (2, 1), (2, 3), (3, 1), (3, 2)],
+@pytest.fixture(params=["auto", (0, 0), (1, 1), (1, 2), (2, 1), (2, 3), (3, 1), (3, 2)],
                 ids=lambda p: p if isinstance(p, str) else f"gemm-tile{p[0]}-splits{p[1]}")
 def path(request):
     from nnfusion_amd import _lib
