@@ -126,7 +126,7 @@ namespace nnfusion
     } // namespace codegen
 
     // The ROCm engine reduced to the passes this path needs (src/nnfusion/engine/device/rocm.cpp:41-90):
-    // device dispatch -> kernel selection -> visitor -> HipCodegenPass.
+    // quantized-op fusion passes -> device dispatch -> kernel selection -> visitor -> HipCodegenPass.
     class ROCmEngine
     {
     public:
@@ -136,5 +136,7 @@ namespace nnfusion
         }
         bool run_on_graph(std::shared_ptr<graph::Graph> graph);
         codegen::HipCodegenPass pass;
+        bool quant_epilogue_fusion = true; // QuantEpilogueFusionPass
+        bool quant_gemm_fusion = false;    // QuantGemmFusionPass (off by default, like -fgemm_fusion)
     };
 } // namespace nnfusion

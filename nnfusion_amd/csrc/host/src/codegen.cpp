@@ -13,6 +13,7 @@
 #include "nnfusion/engine/pass/codegen/base_codegen_pass.hpp"
 #include "nnfusion/core/kernels/common_langunit.hpp"
 #include "nnfusion/engine/pass/graph/kernel_selection.hpp"
+#include "nnfusion/engine/pass/graph/quant_fusion_pass.hpp"
 
 #include <cerrno>
 #include <cstdlib>
@@ -555,6 +556,16 @@ namespace nnfusion
 
     bool ROCmEngine::run_on_graph(std::shared_ptr<graph::Graph> graph)
     {
+        if (quant_epilogue_fusion)
+        {
+            pass::graph::QuantEpilogueFusionPass fusion;
+            NNFUSION_CHECK(fusion.run_on_graph(graph));
+        }
+        if (quant_gemm_fusion)
+        {
+            pass::graph::QuantGemmFusionPass merge;
+            NNFUSION_CHECK(merge.run_on_graph(graph));
+        }
         pass::graph::DefaultGNodeDeviceDispatcher dispatcher(ROCM_GPU);
         NNFUSION_CHECK(dispatcher.run_on_graph(graph));
         pass::graph::DefaultKernelSelector selector;

@@ -165,8 +165,47 @@ namespace nnfusion
                     return lu;
                 }
             };
+
+            // Slice of the last axis (what QuantGemmFusionPass puts behind a merged QuantDot): a strided
+            // device-to-device copy, no kernel of its own.
+            class Slice : public HipLibEmitter
+            {
+            public:
+                explicit Slice(std::shared_ptr<KernelContext> ctx)
+                    : HipLibEmitter(ctx)
+                {
+                }
+
+                LanguageUnit_p emit_function_body() override
+                {
+                    auto gop = std::dynamic_pointer_cast<op::GenericOp>(m_context->op);
+                    if (!gop)
+                        return nullptr;
+                    const Shape& in = m_context->inputs[0]->get_shape();
+                    const Shape& out = m_context->outputs[0]->get_shape();
+                    if (in.empty() || in.size() != out.size())
+                        return nullptr;
+                    const size_t elt = m_context->inputs[0]->get_element_type().size();
+                    const size_t rows = shape_size(in) / in.back();
+                    const size_t begin = (size_t)gop->localOpConfig.getRoot()["begin"].get<int>();
+                    LanguageUnit_p lu(new LanguageUnit(get_function_name()));
+                    *lu << "HIP_SAFE_CALL(hipMemcpy2DAsync(output0, " << out.back() * elt << ", (const char*)input0 + "
+                        << begin * elt << ", " << in.back() * elt << ", " << out.back() * elt << ", " << rows
+                        << ", hipMemcpyDeviceToDevice, stream));\n";
+                    return lu;
+                }
+
+                LanguageUnit_p emit_dependency() override
+                {
+                    LanguageUnit_p lu = HipLibEmitter::emit_dependency();
+                    lu->require(macro::HIP_SAFE_CALL);
+                    return lu;
+                }
+            };
         } // namespace hip
 
+        REGISTER_KERNEL_EMITTER("Slice", Device(ROCM_GPU).TypeConstraint(element::f32).Tag("nnf_hip_gfx950").Priority(5),
+                                hip::Slice)
         REGISTER_KERNEL_EMITTER("QuantDot",
                                 Device(ROCM_GPU).TypeConstraint(element::f32).Tag("nnf_hip_gfx950").Priority(5),
                                 hip::QuantDot)

@@ -9,6 +9,10 @@
 //   nnf_compile_example w8a8      <out_dir> M N K
 //   nnf_compile_example mlp       <out_dir> M H I       (one FusedQuantMLP node)
 //   nnf_compile_example mlp_nodes <out_dir> M H I       (two QuantDot nodes: rms+gate|up, down+residual)
+//   nnf_compile_example mlp_graph <out_dir> M H I       (the unfused block: RMSNorm, gate / up / down QuantDots,
+//                                                         Swish, Multiply, Add; the fusion pass folds it into one node)
+//   nnf_compile_example qkv_graph <out_dir> M N K       (RMSNorm feeding three QuantDots of N rows each; merged
+//                                                         into one 3N-row QuantDot + three Slices; three results)
 #include "../nnf_datagen.h"
 #include "nnfusion/core/operators/generic_op/generic_op.hpp"
 #include "nnfusion/engine/pass/codegen/base_codegen_pass.hpp"
@@ -44,7 +48,7 @@ int main(int argc, char** argv)
 {
     if (argc < 6)
     {
-        fprintf(stderr, "usage: %s <quant_dot|w8a8|mlp|mlp_nodes> <out_dir> <d0> <d1> <d2> [include_dir lib_dir]\n", argv[0]);
+        fprintf(stderr, "usage: %s <quant_dot|w8a8|mlp|mlp_nodes|mlp_graph|qkv_graph> <out_dir> <d0> <d1> <d2> [include_dir lib_dir]\n", argv[0]);
         return 2;
     }
     const std::string kind = argv[1], out_dir = argv[2];
@@ -105,12 +109,70 @@ int main(int argc, char** argv)
             }
             g->add_node_and_edge(std::make_shared<op::Result>(), {out});
         }
+        else if (kind == "mlp_graph")
+        {
+            const size_t M = d0, H = d1, I = d2;
+            auto x = g->add_node_and_edge(std::make_shared<op::Parameter>(element::f16, Shape{M, H}), graph::GNodeVector{});
+            std::vector<uint16_t> gam(H);
+            nnf_gen_normal_f16(0, S_GAMMA, 1.0, 0.1, gam.data(), H);
+            auto gamma = g->add_node_and_edge(std::make_shared<op::Constant>(element::f16, Shape{H}, gam.data()), graph::GNodeVector{});
+            // the same [gate; up] bytes as the other MLP kinds, cut into the two projections
+            std::vector<uint8_t> wgu(2 * I * H / 2);
+            nnf_gen_uniform_u4_packed(0, S_WQ, wgu.data(), 2 * I * H);
+            std::vector<uint16_t> sgu(2 * I * (H / 128));
+            nnf_gen_uniform_f16(0, S_SCALE, 0.005, 0.02, sgu.data(), sgu.size());
+            auto cst = [&](const element::Type& t, const Shape& s, const void* p) {
+                return g->add_node_and_edge(std::make_shared<op::Constant>(t, s, p), graph::GNodeVector{});
+            };
+            auto wg = cst(element::u8, Shape{I, H / 2}, wgu.data());
+            auto wu = cst(element::u8, Shape{I, H / 2}, wgu.data() + I * H / 2);
+            auto sg = cst(element::f16, Shape{I, H / 128}, sgu.data());
+            auto su = cst(element::f16, Shape{I, H / 128}, sgu.data() + I * (H / 128));
+            auto wd = constant_u4(*g, S_WQ2, H, I);
+            auto sd = constant_scales(*g, S_SCALE2, H, I / 128);
+            auto any = op::OpConfig::any();
+            auto n = g->add_node_and_edge(std::make_shared<op::GenericOp>("norm", "RMSNorm", any), {x, gamma});
+            auto gate = g->add_node_and_edge(std::make_shared<op::GenericOp>("gate", "QuantDot", any), {n, wg, sg});
+            auto up = g->add_node_and_edge(std::make_shared<op::GenericOp>("up", "QuantDot", any), {n, wu, su});
+            auto act = g->add_node_and_edge(std::make_shared<op::GenericOp>("act", "Swish", any), {gate});
+            auto h = g->add_node_and_edge(std::make_shared<op::GenericOp>("h", "Multiply", any), {act, up});
+            auto down = g->add_node_and_edge(std::make_shared<op::GenericOp>("down", "QuantDot", any), {h, wd, sd});
+            auto out = g->add_node_and_edge(std::make_shared<op::GenericOp>("out", "Add", any), {x, down});
+            g->add_node_and_edge(std::make_shared<op::Result>(), {out});
+        }
+        else if (kind == "qkv_graph")
+        {
+            const size_t M = d0, N = d1, K = d2;
+            auto x = g->add_node_and_edge(std::make_shared<op::Parameter>(element::f16, Shape{M, K}), graph::GNodeVector{});
+            std::vector<uint16_t> gam(K);
+            nnf_gen_normal_f16(0, S_GAMMA, 1.0, 0.1, gam.data(), K);
+            auto gamma = g->add_node_and_edge(std::make_shared<op::Constant>(element::f16, Shape{K}, gam.data()), graph::GNodeVector{});
+            // one [3N, K] weight block (the bytes of quant_dot with N' = 3N), cut into q, k and v
+            std::vector<uint8_t> w(3 * N * K / 2);
+            nnf_gen_uniform_u4_packed(0, S_WQ, w.data(), 3 * N * K);
+            std::vector<uint16_t> sc(3 * N * (K / 128));
+            nnf_gen_uniform_f16(0, S_SCALE, 0.005, 0.02, sc.data(), sc.size());
+            auto any = op::OpConfig::any();
+            auto n = g->add_node_and_edge(std::make_shared<op::GenericOp>("norm", "RMSNorm", any), {x, gamma});
+            const char* names[3] = {"q_proj", "k_proj", "v_proj"};
+            for (int i = 0; i < 3; ++i)
+            {
+                auto wq = g->add_node_and_edge(std::make_shared<op::Constant>(element::u8, Shape{N, K / 2}, w.data() + i * N * K / 2),
+                                               graph::GNodeVector{});
+                auto s = g->add_node_and_edge(
+                    std::make_shared<op::Constant>(element::f16, Shape{N, K / 128}, sc.data() + i * N * (K / 128)),
+                    graph::GNodeVector{});
+                auto dot = g->add_node_and_edge(std::make_shared<op::GenericOp>(names[i], "QuantDot", any), {n, wq, s});
+                g->add_node_and_edge(std::make_shared<op::Result>(), {dot});
+            }
+        }
         else
         {
             fprintf(stderr, "unknown kind %s\n", kind.c_str());
             return 2;
         }
         ROCmEngine engine(out_dir);
+        engine.quant_gemm_fusion = kind == "qkv_graph";
         if (argc >= 8)
         {
             engine.pass.kernels_include_dir = argv[6];

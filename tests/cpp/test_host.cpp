@@ -8,6 +8,7 @@
 #include "nnfusion/core/operators/generic_op/generic_op.hpp"
 #include "nnfusion/engine/pass/codegen/base_codegen_pass.hpp"
 #include "nnfusion/engine/pass/graph/kernel_selection.hpp"
+#include "nnfusion/engine/pass/graph/quant_fusion_pass.hpp"
 #include "nnfusion/engine/profiler/hip_runtime.hpp"
 
 #include <cstdio>
@@ -527,6 +528,159 @@ int main(int argc, char** argv)
         CONTAINS(pc->source_code, "for (size_t i = 0; i < 7; ++i)");
         CONTAINS(pc->source_code, "return (double)ms / 7;");
         CONTAINS(pc->source_code, "hipMemcpyHostToDevice");
+    });
+
+    run_case("quant_fusion_passes", [] {
+        auto cst = [](graph::Graph& g, const element::Type& t, const Shape& s, uint8_t fill) {
+            std::vector<uint8_t> d(shape_size(s) * t.size(), fill);
+            return g.add_node_and_edge(std::make_shared<op::Constant>(t, s, d.data()), graph::GNodeVector{});
+        };
+        auto gen = [](graph::Graph& g, const std::string& name, const std::string& type, const graph::GNodeVector& in,
+                      const std::string& cfg = "") {
+            return g.add_node_and_edge(
+                std::make_shared<op::GenericOp>(name, type, cfg.empty() ? op::OpConfig::any() : op::OpConfig::any::parse(cfg)), in);
+        };
+        auto count = [](const std::shared_ptr<graph::Graph>& g, const std::string& type) {
+            size_t n = 0;
+            for (auto& node : g->get_ordered_ops())
+                n += node->get_op_type() == type;
+            return n;
+        };
+        auto find = [](const std::shared_ptr<graph::Graph>& g, const std::string& type) {
+            for (auto& node : g->get_ordered_ops())
+                if (node->get_op_type() == type)
+                    return node;
+            return std::shared_ptr<graph::GNode>();
+        };
+        const size_t M = 8, H = 256, I = 384;
+        // the unfused MLP block; `extra_gate_user` adds a second Result on the gate projection
+        auto build_mlp = [&](bool swish_as_one_node, bool extra_gate_user) {
+            auto g = std::make_shared<graph::Graph>();
+            auto x = param(*g, element::f16, Shape{M, H});
+            auto gamma = cst(*g, element::f16, Shape{H}, 0x3c);
+            auto wg = cst(*g, element::u8, Shape{I, H / 2}, 0x11), sg = cst(*g, element::f16, Shape{I, H / 128}, 0x21);
+            auto wu = cst(*g, element::u8, Shape{I, H / 2}, 0x12), su = cst(*g, element::f16, Shape{I, H / 128}, 0x22);
+            auto wd = cst(*g, element::u8, Shape{H, I / 2}, 0x13), sd = cst(*g, element::f16, Shape{H, I / 128}, 0x23);
+            auto n = gen(*g, "norm", "RMSNorm", {x, gamma}, "{\"eps\": 1e-5}");
+            auto gate = gen(*g, "gate", "QuantDot", {n, wg, sg});
+            auto up = gen(*g, "up", "QuantDot", {n, wu, su});
+            std::shared_ptr<graph::GNode> act;
+            if (swish_as_one_node)
+                act = gen(*g, "act", "Swish", {gate});
+            else
+                act = gen(*g, "act", "Multiply", {gen(*g, "sig", "Sigmoid", {gate}), gate});
+            auto h = gen(*g, "h", "Multiply", {up, act});
+            auto down = gen(*g, "down", "QuantDot", {h, wd, sd});
+            auto out = gen(*g, "out", "Add", {down, x});
+            g->add_node_and_edge(std::make_shared<op::Result>(), {out});
+            if (extra_gate_user)
+                g->add_node_and_edge(std::make_shared<op::Result>(), {gate});
+            return g;
+        };
+        for (int variant = 0; variant < 2; ++variant)
+        {
+            auto g = build_mlp(variant == 0, false);
+            pass::graph::QuantEpilogueFusionPass fusion;
+            EXPECT(fusion.run_on_graph(g));
+            // everything folds into one node: parameter, gamma, 4 stacked/kept constants, the MLP, the result
+            EXPECT(count(g, "FusedQuantMLP") == 1 && count(g, "QuantDot") == 0 && count(g, "RMSNorm") == 0 &&
+                   count(g, "Multiply") == 0 && count(g, "Add") == 0 && count(g, "Swish") == 0 && count(g, "Sigmoid") == 0);
+            EXPECT(g->get_ordered_ops().size() == 8);
+            auto mlp = find(g, "FusedQuantMLP");
+            EXPECT(mlp && mlp->get_input_size() == 6 && mlp->get_output_shape(0) == (Shape{M, H}));
+            EXPECT(mlp->get_input_shape(2) == (Shape{2 * I, H / 2}) && mlp->get_input_shape(3) == (Shape{2 * I, H / 128}));
+            auto wgu = std::dynamic_pointer_cast<op::Constant>(mlp->get_in_edge(2).src->get_op_ptr());
+            // gate rows first, then up rows
+            EXPECT(wgu && wgu->get_data().front() == 0x11 && wgu->get_data().back() == 0x12 &&
+                   wgu->get_data()[I * H / 2 - 1] == 0x11 && wgu->get_data()[I * H / 2] == 0x12);
+            auto gop = std::dynamic_pointer_cast<op::GenericOp>(mlp->get_op_ptr());
+            EXPECT(std::abs(gop->localOpConfig.getRoot()["rms_eps"].get<double>() - 1e-5) < 1e-12);
+            EXPECT(mlp->get_in_edge(0).src->is_parameter() && mlp->get_in_edge(4).src->get_output_shape(0) == (Shape{H, I / 2}));
+        }
+        {
+            // the gate projection is also a graph output: gate and up stay separate; RMSNorm and the residual still fold
+            auto g = build_mlp(true, true);
+            pass::graph::QuantEpilogueFusionPass fusion;
+            EXPECT(fusion.run_on_graph(g));
+            EXPECT(count(g, "FusedQuantMLP") == 0 && count(g, "QuantDot") == 3 && count(g, "RMSNorm") == 0 &&
+                   count(g, "Add") == 0 && count(g, "Swish") == 1 && count(g, "Multiply") == 1);
+            size_t with_rms = 0, with_res = 0;
+            for (auto& node : g->get_ordered_ops())
+                if (node->get_op_type() == "QuantDot")
+                {
+                    auto& cfg = std::dynamic_pointer_cast<op::GenericOp>(node->get_op_ptr())->localOpConfig.getRoot();
+                    with_rms += cfg["rms_norm"].get<bool>();
+                    with_res += cfg["has_residual"].get<bool>();
+                }
+            EXPECT(with_rms == 2 && with_res == 1);
+        }
+        {
+            // bias (constant row) then residual (same shape) fold in that order; a second Add of a constant does not
+            auto g = std::make_shared<graph::Graph>();
+            auto x = param(*g, element::f16, Shape{M, H});
+            auto r = param(*g, element::f16, Shape{M, I});
+            auto w = cst(*g, element::u8, Shape{I, H / 2}, 1), s = cst(*g, element::f16, Shape{I, H / 128}, 2);
+            auto b = cst(*g, element::f16, Shape{I}, 3), b2 = cst(*g, element::f16, Shape{I}, 4);
+            auto d = gen(*g, "d", "QuantDot", {x, w, s});
+            auto y = gen(*g, "y", "Add", {gen(*g, "yb", "Add", {d, b}), r});
+            auto z = gen(*g, "z", "Add", {y, b2});
+            g->add_node_and_edge(std::make_shared<op::Result>(), {z});
+            pass::graph::QuantEpilogueFusionPass fusion;
+            EXPECT(fusion.run_on_graph(g) && fusion.fused == 2);
+            EXPECT(count(g, "QuantDot") == 1 && count(g, "Add") == 1);
+            auto q = find(g, "QuantDot");
+            auto& cfg = std::dynamic_pointer_cast<op::GenericOp>(q->get_op_ptr())->localOpConfig.getRoot();
+            EXPECT(cfg["has_bias"].get<bool>() && cfg["has_residual"].get<bool>() && q->get_input_size() == 5);
+            EXPECT(q->get_input_shape(3) == (Shape{I}) && q->get_input_shape(4) == (Shape{M, I}));
+            // and the fused node still finds its emitter
+            pass::graph::DefaultKernelSelector sel;
+            auto fu = sel.pick_first(q, ROCM_GPU).second->get_or_emit_source();
+            CONTAINS(fu->body_unit->get_code(), "nullptr, 1.000000000e-06f, input3, input4, NNF_ACT_NONE");
+        }
+        {
+            // q / k / v read the same normalised activations: one 3N-row QuantDot and three Slices
+            auto g = std::make_shared<graph::Graph>();
+            auto x = param(*g, element::f16, Shape{M, H});
+            auto gamma = cst(*g, element::f16, Shape{H}, 0x3c);
+            auto n = gen(*g, "norm", "RMSNorm", {x, gamma});
+            auto other = param(*g, element::f16, Shape{M, H});
+            const size_t rows[3] = {128, 64, 64};
+            for (int i = 0; i < 3; ++i)
+            {
+                auto w = cst(*g, element::u8, Shape{rows[i], H / 2}, (uint8_t)(0x40 + i));
+                auto s = cst(*g, element::f16, Shape{rows[i], H / 128}, (uint8_t)(0x50 + i));
+                g->add_node_and_edge(std::make_shared<op::Result>(), {gen(*g, "p" + std::to_string(i), "QuantDot", {n, w, s})});
+            }
+            // a QuantDot on other activations is left alone
+            auto w = cst(*g, element::u8, Shape{32, H / 2}, 9), s = cst(*g, element::f16, Shape{32, H / 128}, 9);
+            g->add_node_and_edge(std::make_shared<op::Result>(), {gen(*g, "lone", "QuantDot", {other, w, s})});
+            pass::graph::QuantEpilogueFusionPass fusion;
+            pass::graph::QuantGemmFusionPass merge;
+            EXPECT(fusion.run_on_graph(g) && merge.run_on_graph(g) && merge.merged_groups == 1);
+            EXPECT(count(g, "QuantDot") == 2 && count(g, "Slice") == 3 && count(g, "RMSNorm") == 0 && count(g, "Result") == 4);
+            std::shared_ptr<graph::GNode> wide;
+            std::vector<std::pair<int, int>> ranges;
+            for (auto& node : g->get_ordered_ops())
+            {
+                if (node->get_op_type() == "QuantDot" && node->get_output_shape(0).back() == 256)
+                    wide = node;
+                if (node->get_op_type() == "Slice")
+                {
+                    auto& cfg = std::dynamic_pointer_cast<op::GenericOp>(node->get_op_ptr())->localOpConfig.getRoot();
+                    ranges.push_back({cfg["begin"].get<int>(), cfg["end"].get<int>()});
+                }
+            }
+            EXPECT(wide && wide->get_input_size() == 4 && wide->get_input_shape(1) == (Shape{256, H / 2}));
+            EXPECT(ranges.size() == 3 && ranges[0] == std::make_pair(0, 128) && ranges[1] == std::make_pair(128, 192) &&
+                   ranges[2] == std::make_pair(192, 256));
+            auto wc = std::dynamic_pointer_cast<op::Constant>(wide->get_in_edge(1).src->get_op_ptr());
+            EXPECT(wc && wc->get_data()[0] == 0x40 && wc->get_data()[128 * H / 2] == 0x41 && wc->get_data().back() == 0x42);
+            // the Slice has an emitter: a strided device-to-device copy
+            pass::graph::DefaultKernelSelector sel;
+            auto sl = find(g, "Slice");
+            CONTAINS(sel.pick_first(sl, ROCM_GPU).second->get_or_emit_source()->body_unit->get_code(),
+                     "hipMemcpy2DAsync(output0, 256, (const char*)input0 + 0, 512, 256, 8, hipMemcpyDeviceToDevice, stream)");
+        }
     });
 
     printf("%s (%d failure%s)\n", g_failures ? "FAILED" : "OK", g_failures, g_failures == 1 ? "" : "s");

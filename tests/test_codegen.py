@@ -44,8 +44,8 @@ def test_generated_project_compiles_and_exports_the_runtime_abi(tmp_path):
     assert len(consts) == 2 and sum(os.path.getsize(out + "Constant/" + c) for c in consts) == 64 * 128 + 64 * 2 * 2
 
 
-def _run_generated(name, inputs, out_shape, out_dtype, gpu):
-    """dlopen nnfusion_amd/generated/<name>, init, kernel_entry(inputs..., output), free."""
+def _run_generated(name, inputs, out_shape, out_dtype, gpu, n_outputs=1):
+    """dlopen nnfusion_amd/generated/<name>, init, kernel_entry(inputs..., outputs...), free."""
     import torch
 
     d = os.path.join(GEN, name)
@@ -58,12 +58,12 @@ def _run_generated(name, inputs, out_shape, out_dtype, gpu):
         assert rt.get_device_type() == 1
         rt.rocm_init()
         dev_in = [torch.from_numpy(np.ascontiguousarray(a)).to(gpu) for a in inputs]
-        out = torch.empty(out_shape, dtype=out_dtype, device=gpu)
-        rt.kernel_entry.argtypes = [ctypes.c_void_p] * (len(dev_in) + 1)
+        outs = [torch.empty(out_shape, dtype=out_dtype, device=gpu) for _ in range(n_outputs)]
+        rt.kernel_entry.argtypes = [ctypes.c_void_p] * (len(dev_in) + n_outputs)
         rt.kernel_entry.restype = ctypes.c_int
-        assert rt.kernel_entry(*[t.data_ptr() for t in dev_in], out.data_ptr()) == 0
+        assert rt.kernel_entry(*[t.data_ptr() for t in dev_in], *[o.data_ptr() for o in outs]) == 0
         torch.cuda.synchronize()
-        res = out.cpu().numpy()
+        res = outs[0].cpu().numpy() if n_outputs == 1 else [o.cpu().numpy() for o in outs]
         rt.rocm_free()
     finally:
         os.chdir(cwd)
@@ -96,7 +96,7 @@ def test_generated_w8a8_runtime(gpu):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("name,m,h,i", [("mlp", 16, 256, 384), ("mlp_nodes", 48, 512, 1408)])
+@pytest.mark.parametrize("name,m,h,i", [("mlp", 16, 256, 384), ("mlp_nodes", 48, 512, 1408), ("mlp_graph", 40, 512, 1024)])
 def test_generated_mlp_runtime(gpu, name, m, h, i):
     import torch
 
@@ -104,3 +104,20 @@ def test_generated_mlp_runtime(gpu, name, m, h, i):
     y = _run_generated(name, [x], (m, h), torch.float16, gpu)
     ref = oracle.fused_mlp_w4a16(x, gamma, wgu, sgu, wd, sd)
     assert np.abs(y.astype(np.float32) - ref.astype(np.float32)).max() <= 1e-2 * _rms(ref)
+
+
+@pytest.mark.gpu
+def test_generated_qkv_graph_runtime(gpu):
+    """RMSNorm feeding three QuantDots: the passes fold the norm in and merge the three into one 3N-row QuantDot
+    followed by three Slices; the three results are the column blocks of the wide product."""
+    import torch
+
+    m, n, k = 4, 256, 512
+    a, wq, s = datagen.w4a16_case(0, m, 3 * n, k)
+    gamma = datagen.normal_f16(0, datagen.S_GAMMA, (k,), 1.0, 0.1)
+    ys = _run_generated("qkv_graph", [a], (m, n), torch.float16, gpu, n_outputs=3)
+    ref = oracle.w4a16_gemm(oracle.rmsnorm_f16(a, gamma, 1e-6), wq, s, f32_out=True)
+    src = open(os.path.join(GEN, "qkv_graph", "nnfusion_rt.cpp")).read()
+    assert src.count("NNF_HIP_CHECK(nnf_w4a16_gemm") == 1 and src.count("hipMemcpy2DAsync(") == 3
+    for i, y in enumerate(ys):
+        assert np.abs(y.astype(np.float32) - ref[:, i * n:(i + 1) * n]).max() <= 1e-2 * _rms(ref)
