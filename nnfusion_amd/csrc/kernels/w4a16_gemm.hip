@@ -128,6 +128,34 @@ namespace nnf
         }
     }
 
+    // Epilogues for the M <= 16 path, whose GEMV kernel writes plain fp16 products.
+    // T [M, 2N] = (gate | up) products  ->  Y [M, N] = SiLU(gate) * up
+    __global__ __launch_bounds__(256) void skinny_silu_gate_kernel(const half_t* __restrict__ T, half_t* __restrict__ Y,
+                                                                   int M, int N)
+    {
+        const int i = blockIdx.x * 256 + threadIdx.x;
+        if (i >= M * N)
+            return;
+        const int m = i / N, n = i - m * N;
+        const float g = (float)T[(size_t)m * 2 * N + n];
+        const float u = (float)T[(size_t)m * 2 * N + N + n];
+        Y[i] = (half_t)(g * (1.0f / (1.0f + __expf(-g))) * u);
+    }
+    // Y [M, N] += bias [N] (rounded to fp16), then += residual [M, N]
+    __global__ __launch_bounds__(256) void skinny_bias_residual_kernel(half_t* __restrict__ Y, const half_t* __restrict__ bias,
+                                                                       const half_t* __restrict__ residual, int M, int N)
+    {
+        const int i = blockIdx.x * 256 + threadIdx.x;
+        if (i >= M * N)
+            return;
+        float v = (float)Y[i];
+        if (bias)
+            v = (float)(half_t)(v + (float)bias[i % N]);
+        if (residual)
+            v = v + (float)residual[i];
+        Y[i] = (half_t)v;
+    }
+
     namespace
     {
         template <bool GATE, bool BIAS, bool RESID>
@@ -176,7 +204,7 @@ namespace nnf
 
     hipError_t launch_w4a16_gemm(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M,
                                  int N, int K, int zp, const void* rms_gamma, float rms_eps, const void* bias,
-                                 const void* residual, int act, void* rms_ws, void* partial_ws)
+                                 const void* residual, int act, void* rms_ws, void* partial_ws, int num_cu)
     {
         const bool rms = rms_gamma != nullptr, hb = bias != nullptr, hr = residual != nullptr, gate = act == 1;
         // the combinations the fused entry points use; anything else is composed by the caller
@@ -192,6 +220,24 @@ namespace nnf
             if (e != hipSuccess)
                 return e;
             A = rms_ws;
+        }
+        // M <= 16: the bandwidth-bound GEMV kernel on the (normalised) activations, then a small element-wise
+        // kernel for whatever epilogue is asked for
+        const int n_rows = gate ? 2 * N : N;
+        if (g_tuning.force_path != 3 && M <= 16 && w4a16_skinny_supported(M, n_rows, K) && (!gate || partial_ws))
+        {
+            void* y_gemv = gate ? partial_ws : Y; // gate: the [M, 2N] products go to scratch first
+            hipError_t e = launch_w4a16_skinny(stream, A, Wq, S, y_gemv, M, n_rows, K, zp, num_cu);
+            if (e != hipSuccess || (!gate && !hb && !hr))
+                return e;
+            const int blocks = (M * N + 255) / 256;
+            if (gate)
+                hipLaunchKernelGGL(skinny_silu_gate_kernel, dim3(blocks), dim3(256), 0, stream, (const half_t*)y_gemv,
+                                   (half_t*)Y, M, N);
+            else
+                hipLaunchKernelGGL(skinny_bias_residual_kernel, dim3(blocks), dim3(256), 0, stream, (half_t*)Y,
+                                   (const half_t*)bias, (const half_t*)residual, M, N);
+            return hipGetLastError();
         }
         const workspace::GemmPlan plan =
             workspace::plan_w4a16_gemm(M, N, K, gate, g_tuning.gemm_tile - 1, g_tuning.gemm_splits);

@@ -304,9 +304,10 @@ namespace nnf
             // Except after the last tile the sums are parked in LDS: a global store inside the loop
             // would make later address arithmetic wait for it, and with it for every prefetched load
             // issued before it (one in-order counter covers both).
-            if (tid < M * 64)
+            // (a workgroup with fewer than M wavefronts takes several rounds; whole wavefronts stay together)
+            for (int t = tid; t < M * 64; t += (int)blockDim.x)
             {
-                const int o = tid >> 2, q = tid & 3; // o = m*16 + n
+                const int o = t >> 2, q = t & 3; // o = m*16 + n
                 floatx4 p4 = {0.f, 0.f, 0.f, 0.f};
                 p4 = *reinterpret_cast<const floatx4*>(red + par * red_copy + o * KSP + q * 4);
                 float v = quad_sum((p4.x + p4.y) + (p4.z + p4.w));

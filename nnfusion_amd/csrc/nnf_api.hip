@@ -136,7 +136,7 @@ int nnf_w4a16_gemm(nnf_stream_t stream, const void* A, const void* Wq, const voi
     if (need > 0 && (!workspace || !aligned16(workspace) || workspace_bytes < need))
         return NNF_ERR_WORKSPACE_TOO_SMALL;
     return (int)nnf::launch_w4a16_gemm((hipStream_t)stream, A, Wq, scales, Y, M, N, K, zp, nullptr, 0.f, nullptr,
-                                       nullptr, NNF_ACT_NONE, nullptr, workspace);
+                                       nullptr, NNF_ACT_NONE, nullptr, workspace, dev.num_cu);
 }
 
 size_t nnf_w4a16_gemm_fused_workspace_bytes(int M, int N, int K, int group, int act)
@@ -168,7 +168,8 @@ int nnf_w4a16_gemm_fused(nnf_stream_t stream, const void* A, const void* Wq, con
         return st;
     uint8_t* ws = (uint8_t*)workspace;
     return (int)nnf::launch_w4a16_gemm((hipStream_t)stream, A, Wq, scales, Y, M, N, K, zp, rms_gamma, rms_eps, bias,
-                                       residual, act, ws, ws ? ws + (rms_gamma ? nnf::workspace::rms_rows(M, K) : 0) : nullptr);
+                                       residual, act, ws, ws ? ws + (rms_gamma ? nnf::workspace::rms_rows(M, K) : 0) : nullptr,
+                                       dev.num_cu);
 }
 
 // ---- W8A8 ---------------------------------------------------------------------------------------
@@ -269,12 +270,12 @@ int nnf_fused_mlp_w4a16(nnf_stream_t stream, const void* x, const void* gamma, f
     // h = SiLU(gate) * up, gate|up = RMSNorm(x) . Wgu^T : the normalisation pre-pass, then one GEMM with the
     // gate and up projections as the two halves of every N tile
     hipError_t e = nnf::launch_w4a16_gemm((hipStream_t)stream, x, Wgu, Sgu, h, M, I, H, zp, gamma, eps, nullptr,
-                                          nullptr, NNF_ACT_SILU_GATE, ws, partial);
+                                          nullptr, NNF_ACT_SILU_GATE, ws, partial, dev.num_cu);
     if (e != hipSuccess)
         return (int)e;
     // out = h . Wd^T + x
     e = nnf::launch_w4a16_gemm((hipStream_t)stream, h, Wd, Sd, out, M, H, I, zp, nullptr, 0.f, nullptr, x, NNF_ACT_NONE,
-                               nullptr, partial);
+                               nullptr, partial, dev.num_cu);
     return (int)e;
 }
 

@@ -47,6 +47,7 @@ def _check(y, ref):
     (1, 12288, 4096), (1, 22016, 4096), (1, 4096, 11008),  # configs[1]
     (1, 7, 128), (1, 1, 256), (2, 33, 384), (3, 100, 2048), (4, 257, 2176),
     (5, 64, 4096), (7, 130, 1024), (8, 512, 8192), (16, 1024, 8192),
+    (16, 256, 1024), (12, 96, 2048), (16, 48, 3072), (9, 400, 512),  # more rows than wavefronts in the workgroup
 ])
 def test_gemv_matches_oracle(gpu, path, m, n, k):
     print(f"case M={m} N={n} K={k}", flush=True)

@@ -218,6 +218,35 @@ def test_fused_silu_gate(gpu, plan):
     assert _rms(err) <= 1e-3 * _rms(ref)
 
 
+@pytest.mark.parametrize("m", [1, 5, 16])
+def test_fused_small_m_goes_through_the_gemv_kernel(gpu, m):
+    """Decode shapes with a prologue / epilogue: RMSNorm pre-pass, the M <= 16 GEMV kernel, an element-wise epilogue."""
+    import torch
+
+    from nnfusion_amd import ops
+
+    n, k = 320, 1024
+    a, wq, s = datagen.w4a16_case(11, m, 2 * n, k)
+    gamma = datagen.normal_f16(11, datagen.S_GAMMA, (k,), 1.0, 0.1)
+    bias = datagen.normal_f16(11, datagen.S_BIAS, (n,))
+    res = datagen.normal_f16(11, datagen.S_RES, (m, n))
+    ta, tw, ts, tg, tb, tr = _t(gpu, a, wq, s, gamma, bias, res)
+    xn = oracle.rmsnorm_f16(a, gamma, 1e-6)
+    # RMSNorm + bias + residual on the first n weight rows
+    y = ops.w4a16_gemm_fused(ta, tw[:n].contiguous(), ts[:n].contiguous(), rms_gamma=tg, rms_eps=1e-6, bias=tb,
+                             residual=tr).cpu().numpy()
+    d = oracle.w4a16_gemm(xn, wq[:n], s[:n])
+    ref = oracle.add_f16(oracle.add_f16(d, np.broadcast_to(bias, (m, n)).copy()), res)
+    _check(y, ref)
+    # RMSNorm + SiLU gate over all 2n rows (gate rows, then up rows)
+    yg = ops.w4a16_gemm_fused(ta, tw, ts, rms_gamma=tg, rms_eps=1e-6, act=1).cpu().numpy()
+    torch.cuda.synchronize()
+    gu = oracle.w4a16_gemm(xn, wq, s)
+    refg = oracle.silu_mul_f16(np.ascontiguousarray(gu[:, :n]), np.ascontiguousarray(gu[:, n:]))
+    err = np.abs(yg.astype(np.float32) - refg.astype(np.float32))
+    assert _rms(err) <= 1e-3 * _rms(refg) and err.max() <= 5e-2 * _rms(refg)
+
+
 def test_rejects_bad_arguments(gpu):
     import torch
 
