@@ -10,9 +10,12 @@
  * 143-177).  Every function
  *   - takes plain device pointers and sizes (no C++ types, no torch types),
  *   - is stream ordered: it enqueues on `stream` and returns without synchronising,
- *   - never allocates: scratch memory is passed in (`workspace`), sized by the matching
- *     `*_workspace_bytes` query so that an emitter can reserve it at compile time with
- *     KernelEmitter::allocate_tensor (src/nnfusion/core/kernels/kernel_emitter.cpp:282-319),
+ *   - never allocates: scratch memory is passed in (`workspace`, 16-byte aligned), sized by the
+ *     matching `*_workspace_bytes` query -- pure host arithmetic on the shape, an upper bound, 0 for
+ *     shapes that need none -- so that an emitter can reserve it at compile time with
+ *     KernelEmitter::allocate_tensor (src/nnfusion/core/kernels/kernel_emitter.cpp:282-319).
+ *     It holds, as the shape requires: the normalised activations of the RMSNorm prologue, the
+ *     fp32 / int32 partial sums of a GEMM whose K range is split across workgroups, the MLP's h,
  *   - never throws: it returns NNF_OK (0), a negative NNF_ERR_* code for a rejected call, or a
  *     positive hipError_t value reported by the HIP runtime.
  *
@@ -78,7 +81,9 @@ enum nnf_activation
     NNF_ACT_SILU_GATE = 1
 };
 
-/* Same GEMM with the Welder-style fused prologue/epilogue kept on chip:
+/* Same GEMM with prologue / epilogue in one call (the epilogues run inside the GEMM kernel or its
+ * reduction pass; RMSNorm writes the normalised activations to `workspace` first, rounded to fp16 as
+ * the unfused graph would hold them; M <= 16 runs the GEMV kernel plus one element-wise kernel):
  *   rms_gamma != NULL : A is replaced by RMSNorm(A) = A * rsqrt(mean_k(A^2) + rms_eps) * gamma[k]
  *                       (rsqrt(x + eps) as in LayerNorm, cuda_gpu/cuda_langunit.cpp:618)
  *   bias      != NULL : fp16 [N], added to every row (MatMulAdd precedent,
@@ -120,7 +125,9 @@ int nnf_w8a8_gemm_acc(nnf_stream_t stream,
  *   RMSNorm -> QuantDot(gate|up) -> SiLU*mul -> QuantDot(down) -> Add(residual) ):
  *   out[M,H] = x + W_down . ( SiLU(W_gate . n) * (W_up . n) ),  n = RMSNorm(x, gamma, eps)
  * Wgu u8 [2I, H/2] (gate rows then up rows), Sgu fp16 [2I, H/group], Wd u8 [H, I/2],
- * Sd fp16 [H, I/group].  The only intermediate that touches HBM is h fp16 [M, I] in workspace.
+ * Sd fp16 [H, I/group].  Intermediates in `workspace`: RMSNorm(x) fp16 [M, H], h fp16 [M, I], and
+ * the partial sums of a split GEMM; SiLU, the gate product and the residual add touch no memory of
+ * their own.
  * The element-wise semantics follow the reference's ops (Sigmoid, Multiply, Add, Rsqrt:
  * cuda_gpu/cuda_kernelops.hpp:206-210,408,416,447-451); the reference has no RMSNorm op.
  * ------------------------------------------------------------------------------------------- */

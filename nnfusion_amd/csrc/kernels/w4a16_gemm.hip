@@ -141,14 +141,14 @@ namespace nnf
         const float u = (float)T[(size_t)m * 2 * N + N + n];
         Y[i] = (half_t)(g * (1.0f / (1.0f + __expf(-g))) * u);
     }
-    // Y [M, N] += bias [N] (rounded to fp16), then += residual [M, N]
-    __global__ __launch_bounds__(256) void skinny_bias_residual_kernel(half_t* __restrict__ Y, const half_t* __restrict__ bias,
-                                                                       const half_t* __restrict__ residual, int M, int N)
+    // Y [M, N] = T [M, N] + bias [N] (rounded to fp16), then + residual [M, N]; T may be Y, residual may be Y
+    __global__ __launch_bounds__(256) void skinny_bias_residual_kernel(const half_t* T, half_t* Y, const half_t* bias,
+                                                                       const half_t* residual, int M, int N)
     {
         const int i = blockIdx.x * 256 + threadIdx.x;
         if (i >= M * N)
             return;
-        float v = (float)Y[i];
+        float v = (float)T[i];
         if (bias)
             v = (float)(half_t)(v + (float)bias[i % N]);
         if (residual)
@@ -224,9 +224,12 @@ namespace nnf
         // M <= 16: the bandwidth-bound GEMV kernel on the (normalised) activations, then a small element-wise
         // kernel for whatever epilogue is asked for
         const int n_rows = gate ? 2 * N : N;
-        if (g_tuning.force_path != 3 && M <= 16 && w4a16_skinny_supported(M, n_rows, K) && (!gate || partial_ws))
+        // the products go to scratch first when the epilogue cannot work in place: the [M, 2N] gate | up pair, or a
+        // residual that is the output buffer itself
+        const bool via_scratch = gate || (hr && residual == Y);
+        if (g_tuning.force_path != 3 && M <= 16 && w4a16_skinny_supported(M, n_rows, K) && (!via_scratch || partial_ws))
         {
-            void* y_gemv = gate ? partial_ws : Y; // gate: the [M, 2N] products go to scratch first
+            void* y_gemv = via_scratch ? partial_ws : Y;
             hipError_t e = launch_w4a16_skinny(stream, A, Wq, S, y_gemv, M, n_rows, K, zp, num_cu);
             if (e != hipSuccess || (!gate && !hb && !hr))
                 return e;
@@ -235,8 +238,8 @@ namespace nnf
                 hipLaunchKernelGGL(skinny_silu_gate_kernel, dim3(blocks), dim3(256), 0, stream, (const half_t*)y_gemv,
                                    (half_t*)Y, M, N);
             else
-                hipLaunchKernelGGL(skinny_bias_residual_kernel, dim3(blocks), dim3(256), 0, stream, (half_t*)Y,
-                                   (const half_t*)bias, (const half_t*)residual, M, N);
+                hipLaunchKernelGGL(skinny_bias_residual_kernel, dim3(blocks), dim3(256), 0, stream, (const half_t*)y_gemv,
+                                   (half_t*)Y, (const half_t*)bias, (const half_t*)residual, M, N);
             return hipGetLastError();
         }
         const workspace::GemmPlan plan =

@@ -247,6 +247,21 @@ def test_fused_small_m_goes_through_the_gemv_kernel(gpu, m):
     assert _rms(err) <= 1e-3 * _rms(refg) and err.max() <= 5e-2 * _rms(refg)
 
 
+@pytest.mark.parametrize("m", [3, 200])
+def test_residual_may_alias_the_output(gpu, m):
+    import torch
+
+    from nnfusion_amd import ops
+
+    n, k = 288, 512
+    a, wq, s = datagen.w4a16_case(12, m, n, k)
+    res = datagen.normal_f16(12, datagen.S_RES, (m, n))
+    ta, tw, ts, tr = _t(gpu, a, wq, s, res)
+    y = ops.w4a16_gemm_fused(ta, tw, ts, residual=tr, out=tr, workspace=_big_ws(gpu)).cpu().numpy()
+    torch.cuda.synchronize()
+    _check(y, oracle.add_f16(oracle.w4a16_gemm(a, wq, s), res))
+
+
 def test_rejects_bad_arguments(gpu):
     import torch
 
