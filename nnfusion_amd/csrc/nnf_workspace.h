@@ -33,13 +33,14 @@ namespace nnf
         // N(0,1) activations (the GEMMs are power bound: ~950 / 700 / 450 TFLOP/s for the three tile shapes when
         // every CU has a workgroup, and a CU runs faster when fewer are busy: hence the square root), ~6 TB/s for
         // the partial sums (written, then read by the reduction pass) and ~3 us for the second launch.
-        // rate_scale: 1 for the fp16 x int4 GEMM, 1.7 for W8A8 (same tiles on the int8 matrix cores; its weight
-        // bytes differ too, but a memory-bound W8A8 shape is decided by the partial-sum term either way)
-        inline double estimate_gemm(int M, int N, int K, bool gate, int tile, int splits, double rate_scale)
+        // w8a8: the same tiles on the int8 matrix cores (~1640 / 1450 / 900 TOP/s; its weight bytes differ too, but
+        // a memory-bound W8A8 shape is decided by the partial-sum term either way)
+        inline double estimate_gemm(int M, int N, int K, bool gate, int tile, int splits, bool w8a8)
         {
             const int bm = tile == GEMM_TILE_BIG ? 256 : tile == GEMM_TILE_MID ? 128 : 64;
             const int bn = tile == GEMM_TILE_BIG ? (gate ? 128 : 256) : tile == GEMM_TILE_MID ? 128 : 256;
-            const double rate = rate_scale * (tile == GEMM_TILE_BIG ? 950e12 : tile == GEMM_TILE_MID ? 700e12 : 450e12);
+            const double rate = w8a8 ? (tile == GEMM_TILE_BIG ? 1640e12 : tile == GEMM_TILE_MID ? 1450e12 : 900e12)
+                                     : (tile == GEMM_TILE_BIG ? 950e12 : tile == GEMM_TILE_MID ? 700e12 : 450e12);
             const int tiles_m = ceil_div(M, bm), tiles_n = ceil_div(N, bn);
             const double blocks = (double)tiles_m * tiles_n * splits;
             const double rounds = (double)(((long long)blocks + PLAN_CUS - 1) / PLAN_CUS);
@@ -57,11 +58,11 @@ namespace nnf
 
         inline double estimate_w4a16_gemm(int M, int N, int K, bool gate, int tile, int splits)
         {
-            return estimate_gemm(M, N, K, gate, tile, splits, 1.0);
+            return estimate_gemm(M, N, K, gate, tile, splits, false);
         }
 
         // N: output columns.  forced_tile >= 0 / forced_splits > 0 override the choice (experiments).
-        inline GemmPlan plan_gemm(int M, int N, int K, bool gate, double rate_scale, int forced_tile, int forced_splits)
+        inline GemmPlan plan_gemm(int M, int N, int K, bool gate, bool w8a8, int forced_tile, int forced_splits)
         {
             static const int split_options[] = {1, 2, 3, 4, 6, 8, 12, 16};
             const int G = K / 128;
@@ -79,7 +80,7 @@ namespace nnf
                     if (forced_splits > 0 ? s != 1 : (s > 1 && G / s < 4))
                         continue;
                     const int splits = forced_splits > 0 ? (forced_splits < G ? forced_splits : G) : s;
-                    const double t = estimate_gemm(M, N, K, gate, tile, splits, rate_scale);
+                    const double t = estimate_gemm(M, N, K, gate, tile, splits, w8a8);
                     if (best_t < 0.0 || t < best_t)
                     {
                         best_t = t;
@@ -93,11 +94,11 @@ namespace nnf
         }
         inline GemmPlan plan_w4a16_gemm(int M, int N, int K, bool gate, int forced_tile = -1, int forced_splits = 0)
         {
-            return plan_gemm(M, N, K, gate, 1.0, forced_tile, forced_splits);
+            return plan_gemm(M, N, K, gate, false, forced_tile, forced_splits);
         }
         inline GemmPlan plan_w8a8_gemm(int M, int N, int K, int forced_tile = -1, int forced_splits = 0)
         {
-            return plan_gemm(M, N, K, false, 1.7, forced_tile, forced_splits);
+            return plan_gemm(M, N, K, false, true, forced_tile, forced_splits);
         }
         inline size_t gemm_partial_bytes(int M, int N, bool gate, const GemmPlan& p)
         {
