@@ -51,7 +51,8 @@ namespace nnf
                                                                 const uint8_t* __restrict__ Wq,
                                                                 const half_t* __restrict__ S,
                                                                 half_t* __restrict__ Y,
-                                                                int M, int N, int K, int zp, int n_tiles)
+                                                                int M, int N, int K, int zp, int n_tiles,
+                                                                int tiles_q, int tiles_r)
     {
         static_assert(H == 1 || H == 2, "one or two passes over K");
         static_assert(!A_REGS || H == 1, "register-resident activations only with one pass");
@@ -114,7 +115,9 @@ namespace nnf
 
         const int stride = gridDim.x;
         const int tile0 = blockIdx.x; // the grid never exceeds n_tiles
-        const int T = (n_tiles - tile0 + stride - 1) / stride;
+        // tiles of this workgroup: n_tiles = tiles_q * gridDim + tiles_r, computed on the host (a division here
+        // would delay the first loads of all sixteen wavefronts)
+        const int T = tiles_q + ((int)blockIdx.x < tiles_r ? 1 : 0);
         auto tile_at = [&](int k) { return tile0 + k * stride; };
 
         // ---- prologue loads ----------------------------------------------------------------------------
@@ -439,7 +442,8 @@ namespace nnf
                     return e;
             }
             hipLaunchKernelGGL((w4a16_skinny_kernel<CPS, A_REGS, H>), dim3(grid), dim3(p.ks * 64), lds_total, stream,
-                               (const half_t*)A, (const uint8_t*)Wq, (const half_t*)S, (half_t*)Y, M, N, K, zp, n_tiles);
+                               (const half_t*)A, (const uint8_t*)Wq, (const half_t*)S, (half_t*)Y, M, N, K, zp, n_tiles,
+                               n_tiles / grid, n_tiles % grid);
             return hipGetLastError();
         }
     } // namespace
