@@ -267,7 +267,8 @@ namespace nnf
         {
         case workspace::GEMM_TILE_BIG: e = launch_gemm_big(stream, p, gate, hb, hr); break;
         case workspace::GEMM_TILE_MID: e = launch_gemm_mid(stream, p, gate, hb, hr); break;
-        default: e = launch_gemm_small(stream, p, gate, hb, hr); break;
+        case workspace::GEMM_TILE_SMALL: e = launch_gemm_small(stream, p, gate, hb, hr); break;
+        default: e = launch_gemm_tiny(stream, p, gate, hb, hr); break;
         }
         if (e != hipSuccess || !plan.reduce_pass)
             return e;

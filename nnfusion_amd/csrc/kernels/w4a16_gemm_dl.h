@@ -62,12 +62,13 @@ namespace nnf
             static_assert(WM * WN == 8, "eight wavefronts per workgroup");
             static constexpr int BM = WM * TM * 32;
             static constexpr int BN = WN * TN * 32;
-            static_assert(BM >= 64 && BN >= 128, "a wavefront-wide load covers 8 A rows / 32 W rows");
+            static_assert(BM >= 32 && BN >= 128, "a wavefront-wide load covers 8 A rows / 32 W rows");
             static constexpr int A_TILE_BYTES = BM * BK * 2;
             static constexpr int W_TILE_BYTES = BN * BK / 2;
             static constexpr int STAGE_BYTES = A_TILE_BYTES + W_TILE_BYTES;
             static constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
-            static constexpr int A_LOADS = BM / 64;    // wavefront-wide loads of the A tile, per wavefront
+            static constexpr int A_CHUNKS = BM / 8;    // wavefront-wide loads in one A tile
+            static constexpr int A_LOADS = A_CHUNKS >= 8 ? A_CHUNKS / 8 : 1; // per wavefront
             static constexpr int W_CHUNKS = BN / 32;   // wavefront-wide loads in one W tile
             // every wavefront issues the same number of loads (the wait counts below rely on it): with
             // fewer than 8 chunks two wavefronts fetch the same chunk into the same place
@@ -140,13 +141,15 @@ namespace nnf
         const int k_begin = g_begin * 128;
 
         // ---- direct-load maps -------------------------------------------------------------------------
-        // A: wavefront w, load i fills LDS rows (w*A_LOADS + i)*8 .. +7; lane l lands at (row = .. + l/8,
-        // slot = l%8) and therefore fetches piece  slot ^ ((row >> 1) & 7)  of that row.
+        // A: chunk c fills LDS rows c*8 .. +7; lane l lands at (row = c*8 + l/8, slot = l%8) and therefore
+        // fetches piece  slot ^ ((row >> 1) & 7)  of that row.
         const half_t* a_src[A_LOADS];
+        int a_chunk[A_LOADS];
 #pragma unroll
         for (int i = 0; i < A_LOADS; ++i)
         {
-            int row = (wave * A_LOADS + i) * 8 + (lane >> 3);
+            a_chunk[i] = (wave * A_LOADS + i) % T::A_CHUNKS;
+            int row = a_chunk[i] * 8 + (lane >> 3);
             int piece = (lane & 7) ^ ((row >> 1) & 7);
             a_src[i] = p.A + (size_t)min(m0 + row, p.M - 1) * K + k_begin + piece * 8;
         }
@@ -178,7 +181,7 @@ namespace nnf
             for (int i = 0; i < A_LOADS; ++i)
                 __builtin_amdgcn_global_load_lds(
                     (const void __attribute__((address_space(1)))*)(a_src[i] + k0),
-                    (void __attribute__((address_space(3)))*)(base + (wave * A_LOADS + i) * 1024), 16, 0, 0);
+                    (void __attribute__((address_space(3)))*)(base + a_chunk[i] * 1024), 16, 0, 0);
 #pragma unroll
             for (int i = 0; i < W_LOADS; ++i)
                 __builtin_amdgcn_global_load_lds(
@@ -417,6 +420,8 @@ namespace nnf
     //   big   256 x 256 (GATE: 256 x (128 + 128))    one workgroup per CU
     //   mid   128 x 128 (GATE: 128 x (128 + 128))    two per CU
     //   small  64 x 256 (GATE:  64 x (256 + 256))    two per CU
+    //   tiny   32 x 256 (GATE:  32 x (256 + 256))    two per CU
     hipError_t launch_gemm_mid(hipStream_t stream, const GemmParams& p, bool gate, bool has_bias, bool has_resid);
     hipError_t launch_gemm_small(hipStream_t stream, const GemmParams& p, bool gate, bool has_bias, bool has_resid);
+    hipError_t launch_gemm_tiny(hipStream_t stream, const GemmParams& p, bool gate, bool has_bias, bool has_resid);
 } // namespace nnf

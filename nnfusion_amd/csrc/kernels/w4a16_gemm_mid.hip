@@ -35,4 +35,15 @@ namespace nnf
             return launch_gemm_dl<1, 8, 2, 2, true, false, false, true, 4>(stream, p);
         return launch_gemm_dl<1, 8, 2, 1, false, false, false, true, 4>(stream, p);
     }
+
+    // 32 x 256 (GATE: 32 x (256 + 256)): wavefronts 1 (M) x 8 (N), each 1 x 1 (GATE: 1 x 2) MFMA tiles; for
+    // M <= 32, where a 64-row tile would fetch as many (repeated) activation rows as weights
+    hipError_t launch_gemm_tiny(hipStream_t stream, const GemmParams& p, bool gate, bool, bool)
+    {
+        if (!p.partial)
+            return hipErrorInvalidValue;
+        if (gate)
+            return launch_gemm_dl<1, 8, 1, 2, true, false, false, true, 4>(stream, p);
+        return launch_gemm_dl<1, 8, 1, 1, false, false, false, true, 4>(stream, p);
+    }
 } // namespace nnf

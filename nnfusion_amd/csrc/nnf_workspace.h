@@ -18,11 +18,12 @@ namespace nnf
             GEMM_TILE_BIG = 0,   // 256 x 256 outputs (SiLU-gate: 256 x 128)
             GEMM_TILE_MID = 1,   // 128 x 128
             GEMM_TILE_SMALL = 2, //  64 x 256
+            GEMM_TILE_TINY = 3,  //  32 x 256
         };
         struct GemmPlan
         {
             int tile = GEMM_TILE_BIG;
-            int splits = 1; // K ranges; > 1 (and always for the small tile): fp32 partial sums + a reduction pass
+            int splits = 1; // K ranges; > 1 (and always for the small and tiny tiles): partial sums + a reduction pass
             bool reduce_pass = false;
         };
         constexpr int PLAN_CUS = 256; // the plan is made for the CU count of an MI355X
@@ -37,10 +38,10 @@ namespace nnf
         // a memory-bound W8A8 shape is decided by the partial-sum term either way)
         inline double estimate_gemm(int M, int N, int K, bool gate, int tile, int splits, bool w8a8)
         {
-            const int bm = tile == GEMM_TILE_BIG ? 256 : tile == GEMM_TILE_MID ? 128 : 64;
+            const int bm = tile == GEMM_TILE_BIG ? 256 : tile == GEMM_TILE_MID ? 128 : tile == GEMM_TILE_SMALL ? 64 : 32;
             const int bn = tile == GEMM_TILE_BIG ? (gate ? 128 : 256) : tile == GEMM_TILE_MID ? 128 : 256;
-            const double rate = w8a8 ? (tile == GEMM_TILE_BIG ? 1640e12 : tile == GEMM_TILE_MID ? 1450e12 : 900e12)
-                                     : (tile == GEMM_TILE_BIG ? 950e12 : tile == GEMM_TILE_MID ? 700e12 : 450e12);
+            static const double rates[2][4] = {{950e12, 700e12, 450e12, 300e12}, {1640e12, 1450e12, 900e12, 600e12}};
+            const double rate = rates[w8a8 ? 1 : 0][tile];
             const int tiles_m = ceil_div(M, bm), tiles_n = ceil_div(N, bn);
             const double blocks = (double)tiles_m * tiles_n * splits;
             const double rounds = (double)(((long long)blocks + PLAN_CUS - 1) / PLAN_CUS);
@@ -51,7 +52,7 @@ namespace nnf
             const double weight_time = n_total * K / 2.0 / 4e12;
             if (t < weight_time)
                 t = weight_time;
-            if (splits > 1 || tile == GEMM_TILE_SMALL)
+            if (splits > 1 || tile >= GEMM_TILE_SMALL)
                 t += 2.0 * splits * M * n_total * 4.0 / 6e12 + 3e-6;
             return t;
         }
@@ -68,11 +69,11 @@ namespace nnf
             const int G = K / 128;
             GemmPlan best;
             double best_t = -1.0;
-            for (int tile = GEMM_TILE_BIG; tile <= GEMM_TILE_SMALL; ++tile)
+            for (int tile = GEMM_TILE_BIG; tile <= GEMM_TILE_TINY; ++tile)
             {
                 if (forced_tile >= 0 ? tile != forced_tile
                                      : ((tile == GEMM_TILE_BIG && M <= 128) || (tile == GEMM_TILE_SMALL && M > 64) ||
-                                        (tile == GEMM_TILE_MID && M <= 64)))
+                                        (tile == GEMM_TILE_MID && M <= 64) || (tile == GEMM_TILE_TINY && (M > 32 || w8a8))))
                     continue;
                 for (int s : split_options)
                 {
@@ -89,7 +90,7 @@ namespace nnf
                     }
                 }
             }
-            best.reduce_pass = best.splits > 1 || best.tile == GEMM_TILE_SMALL;
+            best.reduce_pass = best.splits > 1 || best.tile >= GEMM_TILE_SMALL;
             return best;
         }
         inline GemmPlan plan_w4a16_gemm(int M, int N, int K, bool gate, int forced_tile = -1, int forced_splits = 0)

@@ -43,8 +43,8 @@ def force_gemm():
 
 
 # (tile, splits) of the MFMA GEMM: None = the library's own plan; tiles 1 big 256x256, 2 mid 128x128,
-# 3 small 64x256; splits = K ranges (> 1, and always for the small tile: fp32 partial sums + reduction pass)
-PLANS = [None, (1, 1), (1, 2), (2, 1), (2, 3), (3, 1), (3, 2)]
+# 3 small 64x256, 4 tiny 32x256; splits = K ranges (> 1, and always for the small tile: fp32 partial sums + reduction pass)
+PLANS = [None, (1, 1), (1, 2), (2, 1), (2, 3), (3, 1), (3, 2), (4, 1), (4, 3)]
 
 
 @pytest.fixture(params=PLANS, ids=lambda p: "auto" if p is None else f"tile{p[0]}-splits{p[1]}")
