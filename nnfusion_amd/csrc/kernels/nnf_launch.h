@@ -21,6 +21,12 @@ namespace nnf
     // true when one workgroup can hold the activations (M <= 16 rows of K) in LDS
     bool w4a16_skinny_supported(int M, int N, int K);
 
+    // M <= 16 with activations too large for LDS: the same kernel over `ksplits` ranges of K, fp32 partial sums
+    // [ksplits][M][N] (to be added by the GEMM's reduction pass); w4a16_skinny_ksplits returns 0 when not applicable
+    int w4a16_skinny_ksplits(int M, int N, int K);
+    hipError_t launch_w4a16_skinny_split(hipStream_t stream, const void* A, const void* Wq, const void* S, float* partial,
+                                         int M, int N, int K, int zp, int ksplits, int num_cu);
+
     // MFMA GEMM (any M) with the RMSNorm prologue and bias / residual / SiLU-gate epilogues.
     // rms_ws: nnf::workspace::rms_rows(M, K) bytes, needed when rms_gamma != nullptr;
     // partial_ws: nnf::workspace::gemm_partial_bytes(...) for the plan of the shape (may be 0 bytes).

@@ -242,6 +242,32 @@ namespace nnf
                                    (half_t*)Y, (const half_t*)bias, (const half_t*)residual, M, N);
             return hipGetLastError();
         }
+        // M <= 16 with too many activations for one workgroup's LDS: the GEMV kernel over ranges of K, then the
+        // reduction pass (which applies the epilogue)
+        const int ksplits = (g_tuning.force_path != 3 && partial_ws) ? w4a16_skinny_ksplits(M, n_rows, K) : 0;
+        if (ksplits > 0)
+        {
+            hipError_t e = launch_w4a16_skinny_split(stream, A, Wq, S, (float*)partial_ws, M, n_rows, K, zp, ksplits, num_cu);
+            if (e != hipSuccess)
+                return e;
+            GemmParams p;
+            p.A = nullptr;
+            p.Wq = nullptr;
+            p.S = nullptr;
+            p.Y = (half_t*)Y;
+            p.M = M;
+            p.N = N;
+            p.K = K;
+            p.zp = zp;
+            p.ldy = N;
+            p.up_row_offset = N;
+            p.bias = (const half_t*)bias;
+            p.residual = (const half_t*)residual;
+            p.partial = (float*)partial_ws;
+            p.splits = ksplits;
+            p.ld_partial = n_rows;
+            return launch_reduce_any(stream, p, gate, hb, hr);
+        }
         const workspace::GemmPlan plan =
             workspace::plan_w4a16_gemm(M, N, K, gate, g_tuning.gemm_tile - 1, g_tuning.gemm_splits);
         GemmParams p;

@@ -36,7 +36,8 @@
 
 namespace nnf
 {
-    // LDS, in this order:
+    // LDS, in this order (A_REGS: the partial sums and the parked outputs reuse the space of the staged
+    // activations, which are only needed until every wavefront has copied its share into registers):
     //   activations as 16-byte units  unit(m, c, kq, j) = m*(16 G + 1) + (c*4 + kq)*4 + j  holding
     //       the eight fp16  a[m][c*128 + kq*32 + j*8 + {0,4,1,5,2,6,3,7}]  with slots 2,3,6,7 (odd k) times 1/16
     //       (a row of A is staged in memory order; the odd row stride keeps rows on different banks)
@@ -46,13 +47,26 @@ namespace nnf
     //            (slots of absent wavefronts stay zero)
     //   outb     [tiles of this workgroup][M][16] fp32
     // Group (chunk) index of wavefront w, pass h, slot c:  (h*KS + w)*CPS + c.
-    template <int CPS, bool A_REGS, int H>
+    //
+    // KSPLIT: K is cut into ranges of K columns each (the kernel's K is the range length) handled by different
+    // workgroups, for shapes whose M x K activations do not fit in LDS at once; workgroup b works on range
+    // b % ksplits and writes fp32 partial sums [range][M][N], which the GEMM's reduction pass adds up.
+    struct SkinnySplit
+    {
+        int ksplits;       // number of K ranges
+        int lda;           // row stride of A (elements) = the full K
+        int w_row_bytes;   // row stride of Wq (bytes)
+        int s_row_groups;  // row stride of S (elements) = full K / 128
+        float* partial;    // [ksplits][M][N]
+    };
+
+    template <int CPS, bool A_REGS, int H, bool KSPLIT>
     __global__ __launch_bounds__(1024) void w4a16_skinny_kernel(const half_t* __restrict__ A,
                                                                 const uint8_t* __restrict__ Wq,
                                                                 const half_t* __restrict__ S,
                                                                 half_t* __restrict__ Y,
                                                                 int M, int N, int K, int zp, int n_tiles,
-                                                                int tiles_q, int tiles_r)
+                                                                int tiles_q, int tiles_r, SkinnySplit sp)
     {
         static_assert(H == 1 || H == 2, "one or two passes over K");
         static_assert(!A_REGS || H == 1, "register-resident activations only with one pass");
@@ -69,16 +83,31 @@ namespace nnf
         const int col = lane & 15; // n within the tile (B operand / D column), m for the A operand
         const int kq = lane >> 4;  // K quarter of the MFMA (A/B operands), row quad of D
         const int G = K >> 7;
+        // this workgroup among those of its K range
+        const int k_range = KSPLIT ? (int)blockIdx.x % sp.ksplits : 0;
+        const int wg = KSPLIT ? (int)blockIdx.x / sp.ksplits : (int)blockIdx.x;
+        const int n_wg = KSPLIT ? (int)gridDim.x / sp.ksplits : (int)gridDim.x;
+        const int lda = KSPLIT ? sp.lda : K;
+        if (KSPLIT)
+        {
+            A += (size_t)k_range * K;
+            Wq += (size_t)k_range * (K >> 1);
+            S += (size_t)k_range * G;
+        }
         const int row_units = G * 16 + 1; // 16-byte units per staged row of A (one unit of padding)
         const int a_units = row_units * M;
         const int sc_units = (16 * G * 2 + 15) >> 4; // 16-byte units of one scale copy
-        floatx4* nc_lds = reinterpret_cast<floatx4*>(lds + a_units); // [G][4 kq] x (4 m)
-        uintx4* sc_lds = lds + a_units + G * 4;
         constexpr int KSP = 16; // partial-sum slots per output: a constant, so that the row stride below is an immediate
         const int red_copy = M * 16 * KSP;
-        float* red = reinterpret_cast<float*>(sc_lds + 2 * sc_units); // [2][M][16][KSP]
+        // 16-byte units of the first region: the staged activations, or (A_REGS) whichever is larger of them and
+        // the partial sums + parked outputs of the tiles_q (+1) tiles of a workgroup
+        const int tail_units = (2 * red_copy + (tiles_q + (tiles_r ? 1 : 0)) * M * 16 + 3) >> 2;
+        const int first_units = A_REGS ? max(a_units, tail_units) : a_units;
+        floatx4* nc_lds = reinterpret_cast<floatx4*>(lds + first_units); // [G][4 kq] x (4 m)
+        uintx4* sc_lds = lds + first_units + G * 4;
+        float* red = A_REGS ? reinterpret_cast<float*>(lds) : reinterpret_cast<float*>(sc_lds + 2 * sc_units); // [2][M][16][KSP]
         float* outb = red + 2 * red_copy;
-        const size_t row_bytes = (size_t)(K >> 1);
+        const size_t row_bytes = KSPLIT ? (size_t)sp.w_row_bytes : (size_t)(K >> 1);
         const int m_rd = min(col, M - 1); // rows >= M read a valid row; their D rows are never stored
         int chunk_of[H][CPS];             // clamped to valid memory; chunks past the end of K are masked at use
         float s_mask[H][CPS];
@@ -106,18 +135,25 @@ namespace nnf
         };
         // scale block of a tile: 16 rows x G fp16, contiguous; thread t carries bytes [16t, 16t+16) of it
         // (the threads of the last loading wavefront beyond the block re-read its last 16 bytes)
+        // (KSPLIT: the rows of the block are s_row_groups apart; a row's share is G / 8 whole 16-byte pieces)
         const bool s_loader = tid < sc_units;
-        const uint32_t s_lane_off = (uint32_t)min(tid, sc_units - 1) * 16u;
+        const int s_row_groups = KSPLIT ? sp.s_row_groups : G;
+        uint32_t s_lane_off = (uint32_t)min(tid, sc_units - 1) * 16u;
+        if (KSPLIT)
+        {
+            const int t = min(tid, sc_units - 1), pieces = G >> 3;
+            s_lane_off = (uint32_t)(t / pieces) * (uint32_t)s_row_groups * 2u + (uint32_t)(t % pieces) * 16u;
+        }
         auto load_s = [&](int tile) -> uintx4 {
-            const uint8_t* tile_base = reinterpret_cast<const uint8_t*>(S) + (size_t)row0_of(tile) * G * 2;
+            const uint8_t* tile_base = reinterpret_cast<const uint8_t*>(S) + (size_t)row0_of(tile) * s_row_groups * 2;
             return *reinterpret_cast<const uintx4*>(tile_base + s_lane_off);
         };
 
-        const int stride = gridDim.x;
-        const int tile0 = blockIdx.x; // the grid never exceeds n_tiles
+        const int stride = n_wg;
+        const int tile0 = wg; // the grid never exceeds n_tiles (per K range)
         // tiles of this workgroup: n_tiles = tiles_q * gridDim + tiles_r, computed on the host (a division here
         // would delay the first loads of all sixteen wavefronts)
-        const int T = tiles_q + ((int)blockIdx.x < tiles_r ? 1 : 0);
+        const int T = tiles_q + (wg < tiles_r ? 1 : 0);
         auto tile_at = [&](int k) { return tile0 + k * stride; };
 
         // ---- prologue loads ----------------------------------------------------------------------------
@@ -183,10 +219,32 @@ namespace nnf
             if (u < row0_units)
                 stage_unit(a_early[e], 0, u);
         }
-        for (int m = 0; m < M; ++m)
-            for (int u = tid + (m == 0 ? A_EARLY * (int)blockDim.x : 0); u < row0_units; u += blockDim.x)
-                stage_unit(*reinterpret_cast<const uintx4*>(A + (size_t)m * K + u * 8), m, u);
-        if (KSP != KS)
+        // what the early loads did not cover of row 0 (very long rows only) ...
+        for (int u = tid + A_EARLY * (int)blockDim.x; u < row0_units; u += blockDim.x)
+            stage_unit(*reinterpret_cast<const uintx4*>(A + u * 8), 0, u);
+        // ... and rows 1 .. M-1, as one index space over all threads with four loads in flight per thread: row by
+        // row, each row would cost a full memory round trip of its own
+        {
+            const int rest = (M - 1) * row0_units;
+            for (int v0 = tid; v0 < rest; v0 += 4 * (int)blockDim.x)
+            {
+                uintx4 av[4];
+                int am[4], au[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                {
+                    const int v = min(v0 + e * (int)blockDim.x, rest - 1);
+                    am[e] = 1 + v / row0_units;
+                    au[e] = v - (am[e] - 1) * row0_units;
+                    av[e] = *reinterpret_cast<const uintx4*>(A + (size_t)am[e] * lda + au[e] * 8);
+                }
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (v0 + e * (int)blockDim.x < rest)
+                        stage_unit(av[e], am[e], au[e]);
+            }
+        }
+        if (!A_REGS && KSP != KS)
             for (int i = tid; i < 2 * red_copy; i += blockDim.x)
                 red[i] = 0.f;
         int a_unit[H][CPS];
@@ -214,6 +272,14 @@ namespace nnf
                     areg[A_REGS ? c : 0][j] = lds[a_unit[0][c] + j];
                 ncreg[A_REGS ? c : 0] = nc_lds[chunk_of[0][c] * 4 + kq];
             }
+        }
+        if (A_REGS)
+        {
+            // from here on the staging area holds the partial sums: wait until every wavefront has its copy
+            lds_barrier();
+            if (KSP != KS)
+                for (int i = tid; i < 2 * red_copy; i += blockDim.x)
+                    red[i] = 0.f;
         }
         auto a_op = [&](int h, int c, int j) -> uintx4 {
             if (A_REGS)
@@ -318,7 +384,12 @@ namespace nnf
                 {
                     const int n = row0_of(tile_cur) + (o & 15);
                     if (q == 0)
-                        Y[(size_t)(o >> 4) * N + n] = (half_t)v;
+                    {
+                        if (KSPLIT)
+                            sp.partial[((size_t)k_range * M + (o >> 4)) * N + n] = v;
+                        else
+                            Y[(size_t)(o >> 4) * N + n] = (half_t)v;
+                    }
                 }
                 else if (q == 0)
                 {
@@ -334,7 +405,10 @@ namespace nnf
                     int lt = i / per_tile;
                     int r = i - lt * per_tile;
                     int n = min((tile0 + lt * stride) * 16, N - 16) + (r & 15); // per lane: no scalar row0_of here
-                    Y[(size_t)(r >> 4) * N + n] = (half_t)outb[i];
+                    if (KSPLIT)
+                        sp.partial[((size_t)k_range * M + (r >> 4)) * N + n] = outb[i];
+                    else
+                        Y[(size_t)(r >> 4) * N + n] = (half_t)outb[i];
                 }
             }
             ++local_tile;
@@ -413,37 +487,40 @@ namespace nnf
         using workspace::SkinnyPlan;
         SkinnyPlan plan_skinny(int M, int K) { return workspace::plan_w4a16_skinny(M, K, g_tuning.skinny_cps); }
 
-        template <int CPS, bool A_REGS, int H>
+        // K: the length of a K range (all of K without KSPLIT)
+        template <int CPS, bool A_REGS, int H, bool KSPLIT = false>
         hipError_t launch_cps(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M, int N,
-                              int K, int zp, const SkinnyPlan& p, int num_cu)
+                              int K, int zp, const SkinnyPlan& p, int num_cu, SkinnySplit sp = SkinnySplit())
         {
             const int n_tiles = (N + 15) / 16;
+            const int ksplits = KSPLIT ? sp.ksplits : 1;
             // persistent workgroups: one per CU when it has >= 8 wavefronts, else two
             int per_cu = p.ks >= 8 ? 1 : 2;
             if (g_tuning.skinny_wg_per_cu > 0)
                 per_cu = g_tuning.skinny_wg_per_cu;
-            int grid = std::min(n_tiles, num_cu * per_cu);
+            // workgroups per K range
+            int grid = std::min(n_tiles, std::max(1, num_cu * per_cu / ksplits));
             int tiles_per_wg = (n_tiles + grid - 1) / grid;
-            size_t lds_total = p.lds + (size_t)tiles_per_wg * M * 16 * 4;
+            size_t lds_total = p.lds((size_t)tiles_per_wg * M * 16 * 4);
             while (lds_total > MAX_LDS_BYTES && grid < n_tiles)
             {
                 // a very large N: more, shorter workgroups so that the parked outputs fit
                 grid = std::min(n_tiles, grid * 2);
                 tiles_per_wg = (n_tiles + grid - 1) / grid;
-                lds_total = p.lds + (size_t)tiles_per_wg * M * 16 * 4;
+                lds_total = p.lds((size_t)tiles_per_wg * M * 16 * 4);
             }
             if (lds_total > MAX_LDS_BYTES)
                 return hipErrorInvalidValue;
             if (lds_total > 64 * 1024)
             {
-                hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&w4a16_skinny_kernel<CPS, A_REGS, H>),
+                hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&w4a16_skinny_kernel<CPS, A_REGS, H, KSPLIT>),
                                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_total);
                 if (e != hipSuccess)
                     return e;
             }
-            hipLaunchKernelGGL((w4a16_skinny_kernel<CPS, A_REGS, H>), dim3(grid), dim3(p.ks * 64), lds_total, stream,
-                               (const half_t*)A, (const uint8_t*)Wq, (const half_t*)S, (half_t*)Y, M, N, K, zp, n_tiles,
-                               n_tiles / grid, n_tiles % grid);
+            hipLaunchKernelGGL((w4a16_skinny_kernel<CPS, A_REGS, H, KSPLIT>), dim3(grid * ksplits), dim3(p.ks * 64), lds_total,
+                               stream, (const half_t*)A, (const uint8_t*)Wq, (const half_t*)S, (half_t*)Y, M, N, K, zp, n_tiles,
+                               n_tiles / grid, n_tiles % grid, sp);
             return hipGetLastError();
         }
     } // namespace
@@ -465,6 +542,30 @@ namespace nnf
         case 41: return launch_cps<4, false, 1>(stream, A, Wq, S, Y, M, N, K, zp, p, num_cu);
         case 32: return launch_cps<3, false, 2>(stream, A, Wq, S, Y, M, N, K, zp, p, num_cu);
         case 42: return launch_cps<4, false, 2>(stream, A, Wq, S, Y, M, N, K, zp, p, num_cu);
+        default: return hipErrorInvalidValue;
+        }
+    }
+
+    int w4a16_skinny_ksplits(int M, int N, int K)
+    {
+        return g_tuning.skinny_cps == 0 ? workspace::w4a16_skinny_ksplits(M, N, K) : 0;
+    }
+
+    hipError_t launch_w4a16_skinny_split(hipStream_t stream, const void* A, const void* Wq, const void* S, float* partial,
+                                         int M, int N, int K, int zp, int ksplits, int num_cu)
+    {
+        const int k_range = K / ksplits;
+        SkinnyPlan p = workspace::plan_w4a16_skinny(M, k_range);
+        SkinnySplit sp;
+        sp.ksplits = ksplits;
+        sp.lda = K;
+        sp.w_row_bytes = K >> 1;
+        sp.s_row_groups = K >> 7;
+        sp.partial = partial;
+        switch (p.cps * 10 + p.h)
+        {
+        case 11: return launch_cps<1, true, 1, true>(stream, A, Wq, S, nullptr, M, N, k_range, zp, p, num_cu, sp);
+        case 21: return launch_cps<2, true, 1, true>(stream, A, Wq, S, nullptr, M, N, k_range, zp, p, num_cu, sp);
         default: return hipErrorInvalidValue;
         }
     }

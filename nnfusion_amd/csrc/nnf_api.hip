@@ -103,9 +103,12 @@ namespace
     // partial-sum bytes of the GEMM plan in force (the automatic one unless an experiment overrides it)
     size_t tuned_partial_bytes(int M, int N, int K, bool gate)
     {
-        return nnf::workspace::gemm_partial_bytes(
+        const size_t a = nnf::workspace::gemm_partial_bytes(
             M, N, gate,
             nnf::workspace::plan_w4a16_gemm(M, N, K, gate, nnf::g_tuning.gemm_tile - 1, nnf::g_tuning.gemm_splits));
+        // the M <= 16 kernel over ranges of K writes partial sums too
+        const size_t b = nnf::workspace::skinny_split_bytes(M, gate ? 2 * N : N, K);
+        return a > b ? a : b;
     }
 } // namespace
 

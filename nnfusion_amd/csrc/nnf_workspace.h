@@ -112,7 +112,15 @@ namespace nnf
         {
             int cps = 0, ks = 0, h = 0; // groups per wavefront and pass, wavefronts per workgroup, passes over K
             bool a_regs = false;        // activations kept in registers
-            size_t lds = 0;             // LDS bytes without the output parking area
+            // LDS bytes: staged activations; correction constants + scales; partial sums.  With a_regs the
+            // activations are only staged until every wavefront has copied its share, and the partial sums and the
+            // output parking area then reuse that space.
+            size_t a_bytes = 0, fixed_bytes = 0, red_bytes = 0;
+            size_t lds(size_t parking_bytes) const
+            {
+                const size_t tail = red_bytes + parking_bytes;
+                return fixed_bytes + (a_regs ? (a_bytes > tail ? a_bytes : tail) : a_bytes + tail);
+            }
         };
         // one workgroup spans all of K: fewest groups per wavefront first (more wavefronts in flight), two
         // passes beyond 16 * 4 groups
@@ -138,9 +146,9 @@ namespace nnf
                 return p;
             // the A operand fits in registers up to two groups per wavefront (32 VGPRs)
             p.a_regs = p.cps <= 2 && p.h == 1;
-            const size_t a_bytes = ((size_t)G * 16 + 1) * M * 16 + (size_t)G * 64;
-            const size_t sc_bytes = 2 * (((size_t)16 * G * 2 + 15) & ~(size_t)15);
-            p.lds = a_bytes + sc_bytes + (size_t)2 * M * 16 * 16 * 4;
+            p.a_bytes = ((size_t)G * 16 + 1) * M * 16;
+            p.fixed_bytes = (size_t)G * 64 + 2 * (((size_t)16 * G * 2 + 15) & ~(size_t)15);
+            p.red_bytes = (size_t)2 * M * 16 * 16 * 4;
             return p;
         }
         // true when one workgroup can hold the activations (M <= 16 rows of K) in LDS
@@ -153,7 +161,30 @@ namespace nnf
                 return false;
             const SkinnyPlan p = plan_w4a16_skinny(M, K, forced_cps);
             // leave room for the output parking area (a few tiles of M x 16 floats)
-            return p.cps != 0 && p.lds + 16 * 1024 <= LDS_BYTES_PER_CU;
+            return p.cps != 0 && p.lds(16 * 1024) <= LDS_BYTES_PER_CU;
+        }
+
+        // M <= 16 shapes whose activations do not fit at once: number of K ranges (each a multiple of 1024 columns,
+        // at most 4096, whose activations fit) the skinny kernel is run over, or 0 when that does not apply
+        inline int w4a16_skinny_ksplits(int M, int N, int K)
+        {
+            if (M < 1 || M > 16 || N < 16 || K < 2048 || (K & 1023) || w4a16_skinny_fits(M, N, K))
+                return 0;
+            static const int options[] = {2, 4, 8, 16};
+            for (int s : options)
+            {
+                const int k_range = K / s;
+                if (K % s != 0 || (k_range & 1023) || k_range > 4096)
+                    continue;
+                if (w4a16_skinny_fits(M, N, k_range))
+                    return s;
+            }
+            return 0;
+        }
+        inline size_t skinny_split_bytes(int M, int N_total, int K)
+        {
+            const int s = w4a16_skinny_ksplits(M, N_total, K);
+            return s ? align256((size_t)s * M * N_total * sizeof(float)) : 0;
         }
 
         // normalised activations of the RMSNorm prologue (fp16 [M, K])
@@ -166,7 +197,9 @@ namespace nnf
                 return 0;
             if (w4a16_skinny_fits(M, N, K))
                 return 0; // served by the skinny kernel
-            return gemm_partial_bytes(M, N, false, plan_w4a16_gemm(M, N, K, false));
+            const size_t a = gemm_partial_bytes(M, N, false, plan_w4a16_gemm(M, N, K, false));
+            const size_t b = skinny_split_bytes(M, N, K);
+            return a > b ? a : b;
         }
         // nnf_w4a16_gemm_fused: [ normalised activations ][ partial sums ]
         inline size_t w4a16_gemm_fused(int M, int N, int K, int, int act)
@@ -174,7 +207,9 @@ namespace nnf
             if (M <= 0 || N <= 0 || K < 128)
                 return 0;
             const bool gate = act == 1;
-            return rms_rows(M, K) + gemm_partial_bytes(M, N, gate, plan_w4a16_gemm(M, N, K, gate));
+            const size_t a = gemm_partial_bytes(M, N, gate, plan_w4a16_gemm(M, N, K, gate));
+            const size_t b = skinny_split_bytes(M, gate ? 2 * N : N, K);
+            return rms_rows(M, K) + (a > b ? a : b);
         }
         // ---- W8A8 ---------------------------------------------------------------------------------------
         struct Q8SkinnyPlan
@@ -229,6 +264,9 @@ namespace nnf
                 return 0;
             size_t a = gemm_partial_bytes(M, I, true, plan_w4a16_gemm(M, I, H, true));
             size_t b = gemm_partial_bytes(M, H, false, plan_w4a16_gemm(M, H, I, false));
+            const size_t c = skinny_split_bytes(M, 2 * I, H), d = skinny_split_bytes(M, H, I);
+            a = a > b ? a : b;
+            b = c > d ? c : d;
             return fused_mlp_partial_offset(M, H, I) + (a > b ? a : b);
         }
     } // namespace workspace

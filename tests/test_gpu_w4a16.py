@@ -48,6 +48,7 @@ def _check(y, ref):
     (1, 7, 128), (1, 1, 256), (2, 33, 384), (3, 100, 2048), (4, 257, 2176),
     (5, 64, 4096), (7, 130, 1024), (8, 512, 8192), (16, 1024, 8192),
     (16, 256, 1024), (12, 96, 2048), (16, 48, 3072), (9, 400, 512),  # more rows than wavefronts in the workgroup
+    (16, 1040, 8192), (8, 520, 8192), (13, 77, 4096), (16, 64, 16384),  # activations too large for LDS: K in ranges
 ])
 def test_gemv_matches_oracle(gpu, path, m, n, k):
     print(f"case M={m} N={n} K={k}", flush=True)
