@@ -58,6 +58,24 @@ def test_gemv_matches_oracle(gpu, path, m, n, k):
     _check(y, ref)
 
 
+def test_gemv_very_large_n_parks_outputs_in_more_workgroups(gpu):
+    """N so large that one workgroup per CU could not park its tiles' outputs in LDS: the launcher uses more,
+    shorter workgroups.  Checked on sampled columns."""
+    import torch
+
+    from nnfusion_amd import ops
+
+    m, n, k = 16, 500000, 128
+    a, wq, s = datagen.w4a16_case(3, m, n, k)
+    y = ops.w4a16_gemm(torch.from_numpy(a).to(gpu), torch.from_numpy(wq).to(gpu), torch.from_numpy(s).to(gpu))
+    torch.cuda.synchronize()
+    cols = np.sort(np.random.default_rng(5).choice(n, 4096, replace=False))
+    cols[:32] = np.arange(32)
+    cols[-32:] = np.arange(n - 32, n)
+    ref = oracle.w4a16_gemm(a, wq[cols], s[cols], f32_out=True)
+    _check(y.cpu().numpy()[:, cols], ref)
+
+
 def test_gemv_all_zero_point_is_zero(gpu, path):
     # every q == zp  =>  Y == 0: exactly on the VALU path (it dequantises to the exact integer
     # q - zp); the MFMA path removes the 1024 + zp offset of its operand encoding from the fp32
