@@ -150,19 +150,20 @@ extern "C" int nnf_internal_mfma_probe(int kind, int mode, int iters, int num_cu
         return (int)e;
     for (int rep = 0; rep < 2; ++rep) // the first run warms up clocks and code
     {
-        hipEventRecord(e0, 0);
+        if ((e = hipEventRecord(e0, 0)) != hipSuccess)
+            return (int)e;
         if (kind == 0)
             hipLaunchKernelGGL(probe_f16_kernel, dim3(num_cu), dim3(512), 0, 0, tab, out, iters);
         else
             hipLaunchKernelGGL(probe_i8_kernel, dim3(num_cu), dim3(512), 0, 0, tab, out, iters);
-        hipEventRecord(e1, 0);
-        if ((e = hipEventSynchronize(e1)) != hipSuccess)
+        if ((e = hipEventRecord(e1, 0)) != hipSuccess || (e = hipEventSynchronize(e1)) != hipSuccess)
             return (int)e;
     }
     float ms = 0.f;
-    hipEventElapsedTime(&ms, e0, e1);
-    hipEventDestroy(e0);
-    hipEventDestroy(e1);
+    if ((e = hipEventElapsedTime(&ms, e0, e1)) != hipSuccess)
+        return (int)e;
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
     const double ops_per_mfma = kind == 0 ? 32768.0 : 65536.0;
     *tops = (double)num_cu * 8 * (double)iters * 8 * ops_per_mfma / ((double)ms * 1e9);
     unsigned long long clocks[2] = {0, 0};

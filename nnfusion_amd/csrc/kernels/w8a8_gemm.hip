@@ -27,7 +27,9 @@ namespace nnf
         int M, N, K;
     };
 
-    template <int CPS, bool RAW_ACC>
+    // CPS: 64-byte chunks of K per wavefront and pass; KH: passes over K per tile (the weights of a
+    // pass sit in one of two register buffers that take turns; 1 or even).
+    template <int CPS, int KH, bool RAW_ACC>
     __global__ __launch_bounds__(1024) void w8a8_skinny_kernel(W8A8Params p, int n_tiles)
     {
         extern __shared__ uintx4 lds[];
@@ -38,58 +40,84 @@ namespace nnf
         const int col = lane & 15;
         const int kq = lane >> 4;
         const int M = p.M, N = p.N, K = p.K;
-        const int C = K >> 6; // 64-byte chunks per row
-        const int n_units = C * 4 * M;
-        int32_t* red = reinterpret_cast<int32_t*>(lds + n_units);
+        const int C = K >> 6;            // 64-byte chunks per row
+        const int c_pad = KS * CPS * KH; // chunks the workgroup walks; activations past C are zero
+        const int rows_c4 = C * 4, rows_pad = c_pad * 4;
+        int32_t* red = reinterpret_cast<int32_t*>(lds + rows_pad * M);
         int32_t* outb = red + 2 * KS * 256;
-        const int chunk0 = wave * CPS;
 
-        auto load_tile = [&](int tile, uintx4* w) {
-            int n = min(tile * 16 + col, N - 1);
-            const int8_t* wrow = p.W + (size_t)n * K + kq * 16;
+        // A tile index past the end of the matrix loads one cache line over and over (the loads stay
+        // unconditional so that the loop's wait counts do not depend on a branch; the values are unused).
+        // Chunks past the end of K read the last chunk again and meet zero activations.
+        auto load_seq = [&](int seq, uintx4* w) {
+            const int tile = (int)blockIdx.x + (seq / KH) * (int)gridDim.x;
+            const int h = seq % KH;
+            const bool real = tile < n_tiles;
+            const int n = min(tile * 16 + col, N - 1);
+            const int8_t* wrow = real ? p.W + (size_t)n * K + kq * 16 : p.W;
+            const size_t step = real ? 64 : 0;
+            const int chunk0 = (h * KS + wave) * CPS;
 #pragma unroll
             for (int c = 0; c < CPS; ++c)
-                w[c] = *reinterpret_cast<const uintx4*>(wrow + (size_t)min(chunk0 + c, C - 1) * 64);
+                w[c] = *reinterpret_cast<const uintx4*>(wrow + (size_t)min(chunk0 + c, C - 1) * step);
         };
 
-        uintx4 w0[CPS], w1[CPS];
-        int tile = blockIdx.x;
-        load_tile(tile, w0);
-
-        for (int u = tid; u < n_units; u += blockDim.x)
+        // Activations first (a few loads, needed by the first product), then two buffers of weights:
+        // everything a workgroup with two passes needs is requested before the first wait.
+        const uintx4 zero = {0u, 0u, 0u, 0u};
+        uintx4 a_first[4];
         {
-            int m = u % M;
-            int rest = u / M; // c*4 + kq
-            lds[u] = *reinterpret_cast<const uintx4*>(p.A + (size_t)m * K + (size_t)rest * 16);
+            const int r = min(tid, rows_c4 - 1);
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                a_first[j] = *reinterpret_cast<const uintx4*>(p.A + (size_t)min(j, M - 1) * K + (size_t)r * 16);
+        }
+
+        uintx4 w0[CPS], w1[CPS];
+        load_seq(0, w0);
+        load_seq(1, w1);
+
+        if (tid < rows_pad)
+        {
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                if (j < M)
+                    lds[tid * M + j] = tid < rows_c4 ? a_first[j] : zero;
+        }
+        // rows 4.. of the activations and the part of a row past the workgroup's width
+        for (int m0 = 0; m0 < M; m0 += 4)
+        {
+            for (int r = tid + (m0 == 0 ? (int)blockDim.x : 0); r < rows_pad; r += blockDim.x)
+            {
+                const int rl = min(r, rows_c4 - 1);
+                uintx4 t[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    t[j] = *reinterpret_cast<const uintx4*>(p.A + (size_t)min(m0 + j, M - 1) * K + (size_t)rl * 16);
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    if (m0 + j < M)
+                        lds[r * M + m0 + j] = r < rows_c4 ? t[j] : zero;
+            }
         }
         __syncthreads();
 
-        const int m_rd = min(col, M - 1);
-        int a_unit[CPS];
-        int valid[CPS];
-#pragma unroll
-        for (int c = 0; c < CPS; ++c)
-        {
-            a_unit[c] = (min(chunk0 + c, C - 1) * 4 + kq) * M + m_rd;
-            valid[c] = (chunk0 + c < C) ? -1 : 0;
-        }
+        const int a_base = (wave * CPS * 4 + kq) * M + min(col, M - 1);
+        const int a_chunk = 4 * M;          // units between the chunks of a wavefront
+        const int a_pass = KS * CPS * 4 * M; // units between the passes
 
         int buf = 0, local_tile = 0;
-        auto compute_store = [&](const uintx4* wt) {
-            intx4 acc = {0, 0, 0, 0};
+        auto accumulate = [&](const uintx4* wt, int h, intx4 acc) {
 #pragma unroll
             for (int c = 0; c < CPS; ++c)
             {
-                uintx4 a = lds[a_unit[c]];
-                uintx4 w = wt[c];
-                // chunks past the end of K contribute nothing
-                w.x &= valid[c];
-                w.y &= valid[c];
-                w.z &= valid[c];
-                w.w &= valid[c];
-                acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(intx4, a), __builtin_bit_cast(intx4, w),
-                                                            acc, 0, 0, 0);
+                uintx4 a = lds[a_base + h * a_pass + c * a_chunk];
+                acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(intx4, a),
+                                                            __builtin_bit_cast(intx4, wt[c]), acc, 0, 0, 0);
             }
+            return acc;
+        };
+        auto reduce_store = [&](intx4 acc) {
             int32_t* rp = red + ((buf * KS + wave) * 16 + kq * 4) * 16 + col;
             rp[0] = acc.x;
             rp[16] = acc.y;
@@ -108,21 +136,44 @@ namespace nnf
             ++local_tile;
         };
 
+        const intx4 acc0 = {0, 0, 0, 0};
         const int stride = gridDim.x;
-        const int my_tiles = (n_tiles - tile + stride - 1) / stride;
-        const int last_tile = tile + (my_tiles - 1) * stride;
-        for (int it = 0; it < (my_tiles >> 1); ++it)
+        const int my_tiles = (n_tiles - (int)blockIdx.x + stride - 1) / stride;
+        int seq = 0;
+        if (KH >= 2)
         {
-            load_tile(tile + stride, w1);
-            __builtin_amdgcn_sched_barrier(0);
-            compute_store(w0);
-            load_tile(min(tile + 2 * stride, last_tile), w0);
-            __builtin_amdgcn_sched_barrier(0);
-            compute_store(w1);
-            tile += 2 * stride;
+            for (int it = 0; it < my_tiles; ++it)
+            {
+                intx4 acc = acc0;
+#pragma unroll
+                for (int h = 0; h < KH; h += 2)
+                {
+                    acc = accumulate(w0, h, acc);
+                    load_seq(seq + 2, w0);
+                    __builtin_amdgcn_sched_barrier(0);
+                    acc = accumulate(w1, h + 1, acc);
+                    load_seq(seq + 3, w1);
+                    __builtin_amdgcn_sched_barrier(0);
+                    seq += 2;
+                }
+                reduce_store(acc);
+            }
         }
-        if (my_tiles & 1)
-            compute_store(w0);
+        else
+        {
+            for (int it = 0; it < (my_tiles >> 1); ++it)
+            {
+                reduce_store(accumulate(w0, 0, acc0));
+                load_seq(seq + 2, w0);
+                __builtin_amdgcn_sched_barrier(0);
+                reduce_store(accumulate(w1, 0, acc0));
+                load_seq(seq + 3, w1);
+                __builtin_amdgcn_sched_barrier(0);
+                seq += 2;
+            }
+            if (my_tiles & 1)
+                reduce_store(accumulate(w0, 0, acc0));
+        }
 
         __syncthreads();
         const int per_tile = M * 16;
@@ -150,9 +201,9 @@ namespace nnf
     namespace
     {
         using Q8SkinnyPlan = workspace::Q8SkinnyPlan;
-        Q8SkinnyPlan plan_q8_skinny(int M, int K) { return workspace::plan_w8a8_skinny(M, K); }
+        Q8SkinnyPlan plan_q8_skinny(int M, int K) { return workspace::plan_w8a8_skinny(M, K, g_tuning.skinny_cps); }
 
-        template <int CPS, bool RAW_ACC>
+        template <int CPS, int KH, bool RAW_ACC>
         hipError_t launch_q8_skinny_cps(hipStream_t stream, const W8A8Params& p, const Q8SkinnyPlan& pl, int num_cu)
         {
             const int n_tiles = (p.N + 15) / 16;
@@ -169,12 +220,12 @@ namespace nnf
                 return hipErrorInvalidValue;
             if (lds_total > 64 * 1024)
             {
-                hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&w8a8_skinny_kernel<CPS, RAW_ACC>),
+                hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&w8a8_skinny_kernel<CPS, KH, RAW_ACC>),
                                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_total);
                 if (e != hipSuccess)
                     return e;
             }
-            hipLaunchKernelGGL((w8a8_skinny_kernel<CPS, RAW_ACC>), dim3(grid), dim3(pl.ks * 64), lds_total, stream, p,
+            hipLaunchKernelGGL((w8a8_skinny_kernel<CPS, KH, RAW_ACC>), dim3(grid), dim3(pl.ks * 64), lds_total, stream, p,
                                n_tiles);
             return hipGetLastError();
         }
@@ -183,13 +234,24 @@ namespace nnf
         hipError_t launch_q8_skinny(hipStream_t stream, const W8A8Params& p, int num_cu)
         {
             Q8SkinnyPlan pl = plan_q8_skinny(p.M, p.K);
-            switch (pl.cps)
+            switch (pl.cps * 16 + pl.kh)
             {
-            case 1: return launch_q8_skinny_cps<1, RAW_ACC>(stream, p, pl, num_cu);
-            case 2: return launch_q8_skinny_cps<2, RAW_ACC>(stream, p, pl, num_cu);
-            case 4: return launch_q8_skinny_cps<4, RAW_ACC>(stream, p, pl, num_cu);
-            case 8: return launch_q8_skinny_cps<8, RAW_ACC>(stream, p, pl, num_cu);
-            case 16: return launch_q8_skinny_cps<16, RAW_ACC>(stream, p, pl, num_cu);
+#define NNF_Q8_CASE(CPS, KH)                                                                                           \
+    case CPS * 16 + KH: return launch_q8_skinny_cps<CPS, KH, RAW_ACC>(stream, p, pl, num_cu);
+                NNF_Q8_CASE(1, 1)
+                NNF_Q8_CASE(2, 1)
+                NNF_Q8_CASE(4, 1)
+                NNF_Q8_CASE(8, 1)
+                NNF_Q8_CASE(1, 2)
+                NNF_Q8_CASE(2, 2)
+                NNF_Q8_CASE(4, 2)
+                NNF_Q8_CASE(8, 2)
+                NNF_Q8_CASE(1, 4)
+                NNF_Q8_CASE(2, 4)
+                NNF_Q8_CASE(4, 4)
+                NNF_Q8_CASE(1, 8)
+                NNF_Q8_CASE(2, 8)
+#undef NNF_Q8_CASE
             default: return hipErrorInvalidValue;
             }
         }

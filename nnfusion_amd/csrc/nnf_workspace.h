@@ -212,28 +212,31 @@ namespace nnf
             return rms_rows(M, K) + (a > b ? a : b);
         }
         // ---- W8A8 ---------------------------------------------------------------------------------------
+        constexpr int Q8_SKINNY_CPS = 2; // preferred chunks per wavefront and pass (more in flight measured slower)
         struct Q8SkinnyPlan
         {
-            int cps = 0, ks = 0; // 64-byte chunks of K per wavefront, wavefronts per workgroup
-            size_t lds = 0;      // LDS bytes without the output parking area
+            int cps = 0, kh = 0, ks = 0; // 64-byte chunks of K per wavefront and pass, passes, wavefronts
+            size_t lds = 0;              // LDS bytes without the output parking area
         };
-        inline Q8SkinnyPlan plan_w8a8_skinny(int M, int K)
+        inline Q8SkinnyPlan plan_w8a8_skinny(int M, int K, int forced_cps = 0)
         {
             Q8SkinnyPlan pl;
             const int C = K >> 6;
-            static const int options[] = {1, 2, 4, 8, 16};
-            for (int cps : options)
-            {
-                const int ks = (C + cps - 1) / cps;
-                if (ks <= 16)
-                {
-                    pl.cps = cps;
-                    pl.ks = ks;
-                    break;
-                }
-            }
-            if (pl.cps)
-                pl.lds = (size_t)C * 4 * M * 16 + (size_t)2 * pl.ks * 256 * 4;
+            // chunks per wavefront and tile: the smallest power of two that needs at most 16 wavefronts
+            int per_wave = 1;
+            while (per_wave <= 16 && (C + per_wave - 1) / per_wave > 16)
+                per_wave *= 2;
+            if (per_wave > 16)
+                return pl;
+            int cps = forced_cps > 0 ? forced_cps : Q8_SKINNY_CPS;
+            if (cps > per_wave)
+                cps = per_wave;
+            while (per_wave / cps > 8)
+                cps *= 2;
+            pl.cps = cps;
+            pl.kh = per_wave / cps;
+            pl.ks = (C + per_wave - 1) / per_wave;
+            pl.lds = (size_t)pl.ks * per_wave * 4 * M * 16 + (size_t)2 * pl.ks * 256 * 4;
             return pl;
         }
         inline bool w8a8_skinny_fits(int M, int K)

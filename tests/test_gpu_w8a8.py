@@ -43,6 +43,8 @@ def _big_ws(gpu):
 @pytest.mark.parametrize("m,n,k", [
     (1, 64, 128), (1, 1000, 1024), (3, 17, 256), (16, 512, 8192), (32, 300, 512), (100, 257, 384),
     (256, 256, 128), (512, 1024, 2048), (1, 8192, 8192), (32, 4096, 4096),
+    # M <= 16 with chunk counts that leave wavefronts partly idle, two passes over K per tile, many tiles
+    (5, 200, 2176), (2, 100, 11008), (7, 48, 16384), (9, 1000, 8320), (1, 33000, 1024), (13, 8200, 4096),
 ])
 def test_accumulators_bit_exact(gpu, path, m, n, k):
     import torch
