@@ -174,6 +174,8 @@ def main():
         us = timed_graph(fns, 10) / len(fns)
         per_shape.append({"N": n, "K": k, "us": round(us, 3), "GB/s": round(w4a16_bytes(1, n, k) / us / 1e3, 1),
                           "frac_hbm": round(w4a16_bytes(1, n, k) / us / 1e3 / HBM_PEAK_GBS, 4)})
+    if not args.no_extra:
+        run_read_probe(torch, dev, lib, args.layers, per_shape, timed_graph)
     # dominant kernel: the K = 4096 instantiation of the skinny kernel serves three of the four launches
     k4096 = [p for p in per_shape if p["K"] == 4096]
     dom_us = sum(p["us"] for p in k4096) / len(k4096)
@@ -225,6 +227,43 @@ def main():
         "extra": extra,
     }
     print(json.dumps(out))
+
+
+def run_read_probe(torch, dev, lib, n_layers, per_shape, timed_graph):
+    """What a launch costs that does nothing but read the same number of bytes once (plain 128-bit loads,
+    one workgroup per CU, three depths of loads in flight, the best is kept): timed exactly like the GEMV
+    launches, walking as many distinct buffers, and written next to them as plain_read_us."""
+    import ctypes
+
+    fn = lib.nnf_internal_read_probe
+    fn.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_longlong, ctypes.c_int, ctypes.c_int]
+    fn.restype = ctypes.c_int
+    num_cu = torch.cuda.get_device_properties(0).multi_processor_count
+    for entry in per_shape:
+        nbytes = (w4a16_bytes(1, entry["N"], entry["K"]) + 15) // 16 * 16
+        bufs = [torch.randint(0, 255, (nbytes,), dtype=torch.uint8, device=dev) for _ in range(n_layers)]
+        best = None
+        by_depth = []
+        for variant in range(5):
+            def make(buf, variant=variant):
+                def call():
+                    st = fn(torch.cuda.current_stream().cuda_stream, buf.data_ptr(), nbytes, variant, num_cu)
+                    if st != 0:
+                        raise RuntimeError(f"nnf_internal_read_probe failed: {st}")
+                return call
+            fns = [make(bufs[i % n_layers]) for i in range(4 * n_layers)]
+            fns[0]()
+            torch.cuda.synchronize()
+            us = timed_graph(fns, 10) / len(fns)
+            if variant < 3:
+                best = us if best is None else min(best, us)
+            by_depth.append(round(us, 3))
+        entry["plain_read_us"] = round(best, 3)
+        entry["plain_read_us_32_64_128KiB_in_flight_per_cu"] = by_depth[:3]
+        entry["read_us_in_gemv_order"] = by_depth[3]
+        entry["read_us_through_lds"] = by_depth[4]
+        entry["gemv_time_over_plain_read"] = round(entry["us"] / best, 3)
+        del bufs
 
 
 def run_mfma_probe(torch, lib):

@@ -16,6 +16,11 @@ namespace nnf
     // true when launch_w4a16_gemv can stage the activations of one pass in LDS
     bool w4a16_gemv_supported(int M, int K);
 
+    // one activation row (M = 1): the row-streaming kernel
+    hipError_t launch_w4a16_gemv_rows(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int N,
+                                      int K, int zp, int num_cu);
+    bool w4a16_gemv_rows_supported(int M, int N, int K, int num_cu);
+
     hipError_t launch_w4a16_skinny(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M,
                                    int N, int K, int zp, int num_cu);
     // true when one workgroup can hold the activations (M <= 16 rows of K) in LDS
@@ -47,7 +52,7 @@ namespace nnf
     // Tuning knobs for experiments (not part of the public ABI): 0 = automatic.
     struct Tuning
     {
-        int force_path = 0;  // 1 = VALU GEMV, 2 = MFMA skinny, 3 = MFMA GEMM
+        int force_path = 0;  // 1 = VALU GEMV, 2 = MFMA skinny, 3 = MFMA GEMM, 4 = row-streaming GEMV (M = 1)
         int skinny_cps = 0;  // chunks (groups of 128) per wavefront
         int skinny_wg_per_cu = 0;
         int gemm_tile = 0;   // 1 + nnf::workspace::GemmTile

@@ -60,13 +60,16 @@ namespace nnf
         float* partial;    // [ksplits][M][N]
     };
 
+    // pack = M | zp << 8 | wavefronts per workgroup << 16;  n_wg: workgroups per K range;  a workgroup's tiles:
+    // tiles_q, one more for the first tiles_r workgroups (n_tiles = tiles_q * n_wg + tiles_r, divided on the host).
+    // The first arguments are the ones the first loads need: they arrive preloaded in scalar registers.
     template <int CPS, bool A_REGS, int H, bool KSPLIT>
     __global__ __launch_bounds__(1024) void w4a16_skinny_kernel(const half_t* __restrict__ A,
                                                                 const uint8_t* __restrict__ Wq,
                                                                 const half_t* __restrict__ S,
                                                                 half_t* __restrict__ Y,
-                                                                int M, int N, int K, int zp, int n_tiles,
-                                                                int tiles_q, int tiles_r, SkinnySplit sp)
+                                                                int N, int K, int tiles_q, int tiles_r, int n_wg,
+                                                                int pack, SkinnySplit sp)
     {
         static_assert(H == 1 || H == 2, "one or two passes over K");
         static_assert(!A_REGS || H == 1, "register-resident activations only with one pass");
@@ -76,17 +79,22 @@ namespace nnf
         asm volatile("v_mov_b32 %0, 0x64006400" : "=v"(MAGIC));
         asm volatile("s_mov_b32 %0, 0x000F000F" : "=s"(MASK_LO));
         asm volatile("s_mov_b32 %0, 0x00F000F0" : "=s"(MASK_HI));
+        // ---- up to the first loads: as few instructions as possible ----------------------------------------
+        // Sixteen wavefronts share one scalar unit and four share a vector unit: every instruction ahead of the
+        // weight loads is paid sixteen (four) times over before the workgroup's memory stream starts.  So: all
+        // loads are  kernel-argument base + 32-bit offset  (the host checks that the offsets fit), a wavefront's
+        // groups are consecutive (immediate offsets), and everything the loads do not need comes after them.
         const int tid = threadIdx.x;
         const int lane = tid & 63;
         const int wave = __builtin_amdgcn_readfirstlane(tid >> 6); // in a scalar register, and what follows from it
-        const int KS = blockDim.x >> 6;
+        const int M = pack & 0xff, zp = (pack >> 8) & 0xff, KS = pack >> 16;
+        const int n_threads = KS << 6;
         const int col = lane & 15; // n within the tile (B operand / D column), m for the A operand
         const int kq = lane >> 4;  // K quarter of the MFMA (A/B operands), row quad of D
         const int G = K >> 7;
         // this workgroup among those of its K range
         const int k_range = KSPLIT ? (int)blockIdx.x % sp.ksplits : 0;
         const int wg = KSPLIT ? (int)blockIdx.x / sp.ksplits : (int)blockIdx.x;
-        const int n_wg = KSPLIT ? (int)gridDim.x / sp.ksplits : (int)gridDim.x;
         const int lda = KSPLIT ? sp.lda : K;
         if (KSPLIT)
         {
@@ -94,9 +102,103 @@ namespace nnf
             Wq += (size_t)k_range * (K >> 1);
             S += (size_t)k_range * G;
         }
+        const uint32_t row_bytes = KSPLIT ? (uint32_t)sp.w_row_bytes : (uint32_t)(K >> 1);
+        const int s_row_groups = KSPLIT ? sp.s_row_groups : G;
+        const int stride = n_wg;
+        const int tile0 = wg; // the grid never exceeds the number of tiles (per K range)
+        const int T = tiles_q + (wg < tiles_r ? 1 : 0);
+        auto tile_at = [&](int k) { return tile0 + k * stride; };
+        // A tile is 16 whole rows: the last tile of an N that is not a multiple of 16 is moved back to
+        // rows N-16 .. N-1 (some rows are then computed twice, with identical results), so that no
+        // address needs a per-lane clamp.
+        auto row0_of = [&](int tile) { return __builtin_amdgcn_readfirstlane(min(tile * 16, N - 16)); };
+
+        // Groups (chunks) of wavefront w in pass h: CPS consecutive ones from (h*KS + w)*CPS; where that runs past
+        // the end of K the window is moved back to end at the last group, and the groups that then belong to
+        // another wavefront are masked out at use (chunk_ok).
+        int chunk_start[H], chunk_base[H];
+        uint32_t w_voff[H];
+#pragma unroll
+        for (int h = 0; h < H; ++h)
+        {
+            chunk_start[h] = (h * KS + wave) * CPS;
+            chunk_base[h] = min(chunk_start[h], G - CPS);
+            w_voff[h] = (uint32_t)col * row_bytes + (uint32_t)kq * 16u + (uint32_t)chunk_base[h] * 64u;
+        }
+        // (real = false: every lane reads the first bytes of the matrix instead -- a load that costs next to
+        // nothing, for a register set that will not be used, where a branch around the loads would cost more)
+        auto load_w = [&](int tile, int h, uintx4* w, bool real = true) {
+            const uint32_t off = real ? w_voff[h] + (uint32_t)row0_of(tile) * row_bytes : 0u;
+#pragma unroll
+            for (int c = 0; c < CPS; ++c)
+                w[c] = *reinterpret_cast<const uintx4*>(Wq + (size_t)off + c * 64);
+        };
+        // scale block of a tile: 16 rows x G fp16, contiguous; thread t carries bytes [16t, 16t+16) of it
+        // (threads beyond the block re-read its last 16 bytes)
+        // (KSPLIT: the rows of the block are s_row_groups apart; a row's share is G / 8 whole 16-byte pieces)
+        const int sc_units = 2 * G; // 16-byte units of one scale copy
+        uint32_t s_lane_off = (uint32_t)min(tid, sc_units - 1) * 16u;
+        if (KSPLIT)
+        {
+            const int t = min(tid, sc_units - 1), pieces = G >> 3;
+            s_lane_off = (uint32_t)(t / pieces) * (uint32_t)s_row_groups * 2u + (uint32_t)(t % pieces) * 16u;
+        }
+        auto load_s = [&](int tile) -> uintx4 {
+            const uint32_t off = s_lane_off + (uint32_t)row0_of(tile) * (uint32_t)s_row_groups * 2u;
+            return *reinterpret_cast<const uintx4*>(reinterpret_cast<const uint8_t*>(S) + (size_t)off);
+        };
+
+        // ---- prologue loads ----------------------------------------------------------------------------
+        // Row 0 of the activations (all of them for M = 1) and the scales of the first two tiles are
+        // requested before the weights: they are small and shared by every workgroup (cache hits), loads
+        // complete in order, and the barrier that publishes them in LDS should not have to wait for the
+        // first weights, which come from HBM.
+        constexpr int A_EARLY = H; // one pass: K <= 8192, a row of A is at most one 16-byte unit per thread
+        const int row0_units = G * 16;
+        // Every wavefront-wide load instruction occupies the CU's one address unit for the same time whether its
+        // lanes fetch distinct data or not, so wavefronts without a share of the activations or of the scales
+        // skip those loads (branches on wavefront-uniform conditions, ahead of the unconditional weight loads).
+        uintx4 a_early[A_EARLY];
+#pragma unroll
+        for (int e = 0; e < A_EARLY; ++e)
+            a_early[e] = uintx4{0u, 0u, 0u, 0u};
+        if (wave * 64 < row0_units)
+        {
+            // Through a pointer the compiler knows nothing about, and with a compiler-level memory barrier behind:
+            // otherwise these loads are moved down into the block that uses them, behind the weights.
+            typedef const uint8_t __attribute__((address_space(1))) * global_bytes_t;
+            typedef const uintx4 __attribute__((address_space(1))) * global_units_t;
+            global_bytes_t a_bytes = (global_bytes_t) reinterpret_cast<const uint8_t*>(A);
+            asm volatile("" : "+s"(a_bytes));
+#pragma unroll
+            for (int e = 0; e < A_EARLY; ++e)
+            {
+                const uint32_t u = (uint32_t)min(tid + e * n_threads, row0_units - 1);
+                a_early[e] = *(global_units_t)(a_bytes + (size_t)(u * 16u));
+            }
+            asm volatile("" ::: "memory");
+        }
+        // A load issued at the end of the prologue would be the newest one when the tile loop is entered,
+        // and the loop's wait for the scale registers would then wait for every weight load in flight:
+        // hence the second tile's scales here, and the second register set loaded without a branch.
+        // Register set 0 / 1: H == 1: even / odd tiles;  H == 2: first / second pass of the current tile.
+        uintx4 w0[CPS], w1[CPS], sreg = {0u, 0u, 0u, 0u}, sfirst = {0u, 0u, 0u, 0u};
+        const int tile_second = tile_at(min(1, T - 1));
+        if (wave * 64 < sc_units)
+        {
+            sfirst = load_s(tile0);
+            sreg = load_s(tile_second);
+        }
+        load_w(tile0, 0, w0);
+        if (H == 2)
+            load_w(tile0, H - 1, w1);
+        else
+            load_w(tile_second, 0, w1, T > 1);
+        __builtin_amdgcn_sched_barrier(0);
+
+        // ---- everything else ---------------------------------------------------------------------------
         const int row_units = G * 16 + 1; // 16-byte units per staged row of A (one unit of padding)
         const int a_units = row_units * M;
-        const int sc_units = (16 * G * 2 + 15) >> 4; // 16-byte units of one scale copy
         constexpr int KSP = 16; // partial-sum slots per output: a constant, so that the row stride below is an immediate
         const int red_copy = M * 16 * KSP;
         // 16-byte units of the first region: the staged activations, or (A_REGS) whichever is larger of them and
@@ -107,88 +209,18 @@ namespace nnf
         uintx4* sc_lds = lds + first_units + G * 4;
         float* red = A_REGS ? reinterpret_cast<float*>(lds) : reinterpret_cast<float*>(sc_lds + 2 * sc_units); // [2][M][16][KSP]
         float* outb = red + 2 * red_copy;
-        const size_t row_bytes = KSPLIT ? (size_t)sp.w_row_bytes : (size_t)(K >> 1);
         const int m_rd = min(col, M - 1); // rows >= M read a valid row; their D rows are never stored
-        int chunk_of[H][CPS];             // clamped to valid memory; chunks past the end of K are masked at use
+        const bool s_loader = tid < sc_units;
+        int chunk_of[H][CPS];
         float s_mask[H][CPS];
 #pragma unroll
         for (int h = 0; h < H; ++h)
 #pragma unroll
             for (int c = 0; c < CPS; ++c)
             {
-                int ch = (h * KS + wave) * CPS + c;
-                chunk_of[h][c] = min(ch, G - 1);
-                s_mask[h][c] = ch < G ? 1.0f : 0.0f;
+                chunk_of[h][c] = chunk_base[h] + c;
+                s_mask[h][c] = chunk_of[h][c] >= chunk_start[h] ? 1.0f : 0.0f;
             }
-
-        // ---- loads: unconditional, so that no branch separates a load from its use ---------------------
-        // A tile is 16 whole rows: the last tile of an N that is not a multiple of 16 is moved back to
-        // rows N-16 .. N-1 (some rows are then computed twice, with identical results), so that no
-        // address needs a per-lane clamp: every load is  uniform 64-bit base + 32-bit lane offset.
-        auto row0_of = [&](int tile) { return __builtin_amdgcn_readfirstlane(min(tile * 16, N - 16)); };
-        const uint32_t w_lane_off = (uint32_t)col * (uint32_t)row_bytes + (uint32_t)kq * 16u;
-        auto load_w = [&](int tile, int h, uintx4* w) {
-            const uint8_t* tile_base = Wq + (size_t)row0_of(tile) * row_bytes;
-#pragma unroll
-            for (int c = 0; c < CPS; ++c)
-                w[c] = *reinterpret_cast<const uintx4*>(tile_base + (size_t)chunk_of[h][c] * 64 + w_lane_off);
-        };
-        // scale block of a tile: 16 rows x G fp16, contiguous; thread t carries bytes [16t, 16t+16) of it
-        // (the threads of the last loading wavefront beyond the block re-read its last 16 bytes)
-        // (KSPLIT: the rows of the block are s_row_groups apart; a row's share is G / 8 whole 16-byte pieces)
-        const bool s_loader = tid < sc_units;
-        const int s_row_groups = KSPLIT ? sp.s_row_groups : G;
-        uint32_t s_lane_off = (uint32_t)min(tid, sc_units - 1) * 16u;
-        if (KSPLIT)
-        {
-            const int t = min(tid, sc_units - 1), pieces = G >> 3;
-            s_lane_off = (uint32_t)(t / pieces) * (uint32_t)s_row_groups * 2u + (uint32_t)(t % pieces) * 16u;
-        }
-        auto load_s = [&](int tile) -> uintx4 {
-            const uint8_t* tile_base = reinterpret_cast<const uint8_t*>(S) + (size_t)row0_of(tile) * s_row_groups * 2;
-            return *reinterpret_cast<const uintx4*>(tile_base + s_lane_off);
-        };
-
-        const int stride = n_wg;
-        const int tile0 = wg; // the grid never exceeds n_tiles (per K range)
-        // tiles of this workgroup: n_tiles = tiles_q * gridDim + tiles_r, computed on the host (a division here
-        // would delay the first loads of all sixteen wavefronts)
-        const int T = tiles_q + (wg < tiles_r ? 1 : 0);
-        auto tile_at = [&](int k) { return tile0 + k * stride; };
-
-        // ---- prologue loads ----------------------------------------------------------------------------
-        // Row 0 of the activations (all of them for M = 1) and the scales of the first two tiles are
-        // requested before the weights: they are small and shared by every workgroup (cache hits), loads
-        // complete in order, and the barrier that publishes them in LDS should not have to wait for the
-        // first weights, which come from HBM.  The address arithmetic before the weight loads is kept
-        // minimal: with four wavefronts per SIMD every instruction here delays the weight stream.
-        constexpr int A_EARLY = 2;
-        const int row0_units = G * 16;
-        uintx4 a_early[A_EARLY];
-#pragma unroll
-        for (int e = 0; e < A_EARLY; ++e)
-        {
-            int u = min(tid + e * (int)blockDim.x, row0_units - 1);
-            a_early[e] = *reinterpret_cast<const uintx4*>(A + u * 8);
-        }
-        // A load issued at the end of the prologue would be the newest one when the tile loop is entered,
-        // and the loop's wait for the scale registers would then wait for every weight load in flight:
-        // hence the second tile's scales here, and the second register set loaded without a branch
-        // (a workgroup with a single tile fetches it twice).
-        // Register set 0 / 1: H == 1: even / odd tiles;  H == 2: first / second pass of the current tile.
-        uintx4 w0[CPS], w1[CPS], sreg = {0, 0, 0, 0}, sfirst = {0, 0, 0, 0};
-        if (s_loader)
-        {
-            sfirst = load_s(tile_at(0));
-            sreg = load_s(tile_at(min(1, T - 1)));
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        load_w(tile_at(0), 0, w0);
-        if (H == 2)
-            load_w(tile_at(0), H - 1, w1);
-        else
-            load_w(tile_at(min(1, T - 1)), 0, w1);
-        __builtin_amdgcn_sched_barrier(0);
 
         // ---- activations -> LDS ---------------------------------------------------------------------
         // Staged once per workgroup (one coalesced 16-byte load per thread and unit); every wavefront
@@ -215,37 +247,37 @@ namespace nnf
 #pragma unroll
         for (int e = 0; e < A_EARLY; ++e)
         {
-            int u = tid + e * (int)blockDim.x;
+            int u = tid + e * n_threads;
             if (u < row0_units)
                 stage_unit(a_early[e], 0, u);
         }
         // what the early loads did not cover of row 0 (very long rows only) ...
-        for (int u = tid + A_EARLY * (int)blockDim.x; u < row0_units; u += blockDim.x)
+        for (int u = tid + A_EARLY * n_threads; u < row0_units; u += n_threads)
             stage_unit(*reinterpret_cast<const uintx4*>(A + u * 8), 0, u);
         // ... and rows 1 .. M-1, as one index space over all threads with four loads in flight per thread: row by
         // row, each row would cost a full memory round trip of its own
         {
             const int rest = (M - 1) * row0_units;
-            for (int v0 = tid; v0 < rest; v0 += 4 * (int)blockDim.x)
+            for (int v0 = tid; v0 < rest; v0 += 4 * n_threads)
             {
                 uintx4 av[4];
                 int am[4], au[4];
 #pragma unroll
                 for (int e = 0; e < 4; ++e)
                 {
-                    const int v = min(v0 + e * (int)blockDim.x, rest - 1);
+                    const int v = min(v0 + e * n_threads, rest - 1);
                     am[e] = 1 + v / row0_units;
                     au[e] = v - (am[e] - 1) * row0_units;
                     av[e] = *reinterpret_cast<const uintx4*>(A + (size_t)am[e] * lda + au[e] * 8);
                 }
 #pragma unroll
                 for (int e = 0; e < 4; ++e)
-                    if (v0 + e * (int)blockDim.x < rest)
+                    if (v0 + e * n_threads < rest)
                         stage_unit(av[e], am[e], au[e]);
             }
         }
         if (!A_REGS && KSP != KS)
-            for (int i = tid; i < 2 * red_copy; i += blockDim.x)
+            for (int i = tid; i < 2 * red_copy; i += n_threads)
                 red[i] = 0.f;
         int a_unit[H][CPS];
 #pragma unroll
@@ -278,7 +310,7 @@ namespace nnf
             // from here on the staging area holds the partial sums: wait until every wavefront has its copy
             lds_barrier();
             if (KSP != KS)
-                for (int i = tid; i < 2 * red_copy; i += blockDim.x)
+                for (int i = tid; i < 2 * red_copy; i += n_threads)
                     red[i] = 0.f;
         }
         auto a_op = [&](int h, int c, int j) -> uintx4 {
@@ -374,7 +406,7 @@ namespace nnf
             // would make later address arithmetic wait for it, and with it for every prefetched load
             // issued before it (one in-order counter covers both).
             // (a workgroup with fewer than M wavefronts takes several rounds; whole wavefronts stay together)
-            for (int t = tid; t < M * 64; t += (int)blockDim.x)
+            for (int t = tid; t < M * 64; t += n_threads)
             {
                 const int o = t >> 2, q = t & 3; // o = m*16 + n
                 floatx4 p4 = {0.f, 0.f, 0.f, 0.f};
@@ -400,7 +432,7 @@ namespace nnf
             {
                 // the sums parked by earlier tiles (written before the barrier above)
                 const int per_tile = M * 16;
-                for (int i = tid; i < local_tile * per_tile; i += blockDim.x)
+                for (int i = tid; i < local_tile * per_tile; i += n_threads)
                 {
                     int lt = i / per_tile;
                     int r = i - lt * per_tile;
@@ -519,8 +551,8 @@ namespace nnf
                     return e;
             }
             hipLaunchKernelGGL((w4a16_skinny_kernel<CPS, A_REGS, H, KSPLIT>), dim3(grid * ksplits), dim3(p.ks * 64), lds_total,
-                               stream, (const half_t*)A, (const uint8_t*)Wq, (const half_t*)S, (half_t*)Y, M, N, K, zp, n_tiles,
-                               n_tiles / grid, n_tiles % grid, sp);
+                               stream, (const half_t*)A, (const uint8_t*)Wq, (const half_t*)S, (half_t*)Y, N, K,
+                               n_tiles / grid, n_tiles % grid, grid, M | (zp << 8) | (p.ks << 16), sp);
             return hipGetLastError();
         }
     } // namespace

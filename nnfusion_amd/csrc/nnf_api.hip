@@ -130,7 +130,9 @@ int nnf_w4a16_gemm(nnf_stream_t stream, const void* A, const void* Wq, const voi
     if (st != NNF_OK)
         return st;
     const int force = nnf::g_tuning.force_path;
-    if ((force == 0 || force == 2) && M <= 16 && nnf::w4a16_skinny_supported(M, N, K))
+    if ((force == 0 || force == 4) && nnf::w4a16_gemv_rows_supported(M, N, K, dev.num_cu))
+        return (int)nnf::launch_w4a16_gemv_rows((hipStream_t)stream, A, Wq, scales, Y, N, K, zp, dev.num_cu);
+    if ((force == 0 || force == 2 || force == 4) && M <= 16 && nnf::w4a16_skinny_supported(M, N, K))
         return (int)nnf::launch_w4a16_skinny((hipStream_t)stream, A, Wq, scales, Y, M, N, K, zp, dev.num_cu);
     if (force == 1 && M <= 16 && nnf::w4a16_gemv_supported(M, K))
         return (int)nnf::launch_w4a16_gemv((hipStream_t)stream, A, Wq, scales, Y, M, N, K, zp, dev.num_cu);

@@ -159,9 +159,12 @@ namespace nnf
             // the scale block of a tile (16 rows x K/128 fp16) is fetched in whole, aligned 16-byte pieces
             if (((size_t)N * (K >> 7) * 2) % 16 != 0)
                 return false;
+            // the kernel addresses weights and scales with 32-bit offsets from their base
+            if ((size_t)N * (size_t)(K >> 1) >= ((size_t)1 << 32))
+                return false;
             const SkinnyPlan p = plan_w4a16_skinny(M, K, forced_cps);
             // leave room for the output parking area (a few tiles of M x 16 floats)
-            return p.cps != 0 && p.lds(16 * 1024) <= LDS_BYTES_PER_CU;
+            return p.cps != 0 && p.cps <= (K >> 7) && p.lds(16 * 1024) <= LDS_BYTES_PER_CU;
         }
 
         // M <= 16 shapes whose activations do not fit at once: number of K ranges (each a multiple of 1024 columns,
@@ -169,6 +172,8 @@ namespace nnf
         inline int w4a16_skinny_ksplits(int M, int N, int K)
         {
             if (M < 1 || M > 16 || N < 16 || K < 2048 || (K & 1023) || w4a16_skinny_fits(M, N, K))
+                return 0;
+            if ((size_t)N * (size_t)(K >> 1) >= ((size_t)1 << 32)) // 32-bit offsets over whole rows
                 return 0;
             static const int options[] = {2, 4, 8, 16};
             for (int s : options)
@@ -185,6 +190,48 @@ namespace nnf
         {
             const int s = w4a16_skinny_ksplits(M, N_total, K);
             return s ? align256((size_t)s * M * N_total * sizeof(float)) : 0;
+        }
+
+        // ---- one activation row: the row-streaming GEMV (w4a16_gemv_rows.hip) ----
+        struct RowsPlan
+        {
+            int seg = 0;    // wavefront-wide loads (1 KiB of a weight row) per row and wavefront; 0: not applicable
+            int kshift = 0; // log2 of the wavefronts that share a row
+            int depth = 0;  // rows in flight per wavefront
+            // ring + scale chunks + activations + parked outputs of one workgroup (16 wavefronts)
+            size_t lds_bytes(int N, int K, int grid) const
+            {
+                const int n_groups = grid * (16 >> kshift);
+                const size_t a_pad = ((size_t)(K >> 3) + 63) & ~(size_t)63; // 16-byte units of activations
+                return (size_t)16 * depth * seg * 1024 + 16 * 2048 + a_pad * 16 + a_pad * 4 +
+                       (size_t)16 * (N / n_groups + 1) * sizeof(float);
+            }
+        };
+        inline RowsPlan plan_w4a16_rows(int M, int N, int K, int num_cu)
+        {
+            RowsPlan p;
+            // whole 16-byte pieces of scales per segment, 4-byte aligned: K a multiple of 256
+            // (the activations are fetched in at most two rounds of 1024 16-byte units: K <= 16384)
+            if (M != 1 || N < 1 || K < 1024 || K > 16384 || (K & 255) || num_cu < 1)
+                return p;
+            const int loads_per_row = ((K >> 1) + 1023) >> 10;
+            int kshift = 0;
+            while (kshift <= 4 && (loads_per_row + (1 << kshift) - 1) >> kshift > 3)
+                ++kshift;
+            if (kshift > 4)
+                return p;
+            p.kshift = kshift;
+            p.seg = (loads_per_row + (1 << kshift) - 1) >> kshift;
+            const int n_groups = num_cu * (16 >> kshift);
+            const int rows_q = N / n_groups;
+            // A CU takes about 64 wavefront-wide loads in flight: beyond that the wavefronts stall at issue
+            const int depth_max = p.seg == 1 ? 4 : (p.seg == 2 ? 2 : 1);
+            p.depth = rows_q < 1 ? 1 : (rows_q > depth_max ? depth_max : rows_q);
+            while (p.depth > 1 && p.lds_bytes(N, K, num_cu) > LDS_BYTES_PER_CU)
+                --p.depth;
+            if (p.lds_bytes(N, K, num_cu) > LDS_BYTES_PER_CU)
+                p.seg = 0;
+            return p;
         }
 
         // normalised activations of the RMSNorm prologue (fp16 [M, K])

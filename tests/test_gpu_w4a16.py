@@ -14,13 +14,14 @@ pytestmark = pytest.mark.gpu
 TOL = 1e-2
 
 
-@pytest.fixture(params=["auto", "valu_gemv", "mfma_skinny"])
+@pytest.fixture(params=["auto", "valu_gemv", "mfma_skinny", "rows_gemv"])
 def path(request):
-    """Runs a test once per kernel family that can serve M <= 16 (auto = the library's own choice)."""
+    """Runs a test once per kernel family that can serve M <= 16 (auto = the library's own choice;
+    rows_gemv = the M = 1 row-streaming kernel where it applies, otherwise the library's choice)."""
     from nnfusion_amd import _lib
 
     tune = _lib.kernels().nnf_internal_tune
-    tune(0, {"auto": 0, "valu_gemv": 1, "mfma_skinny": 2}[request.param])
+    tune(0, {"auto": 0, "valu_gemv": 1, "mfma_skinny": 2, "rows_gemv": 4}[request.param])
     yield request.param
     tune(0, 0)
 
@@ -49,6 +50,10 @@ def _check(y, ref):
     (5, 64, 4096), (7, 130, 1024), (8, 512, 8192), (16, 1024, 8192),
     (16, 256, 1024), (12, 96, 2048), (16, 48, 3072), (9, 400, 512),  # more rows than wavefronts in the workgroup
     (16, 1040, 8192), (8, 520, 8192), (13, 77, 4096), (16, 64, 16384),  # activations too large for LDS: K in ranges
+    # one activation row: rows shared by 1, 2, 4 wavefronts, ragged last K segment, fewer rows than wavefronts,
+    # more rows per wavefront than one chunk of scales holds
+    (1, 300, 1024), (1, 4096, 8192), (1, 1000, 2048), (1, 5000, 1280), (1, 513, 5120), (1, 2000, 14336),
+    (1, 4100, 16384), (1, 151936, 1024), (1, 80000, 3072), (1, 40, 4096),
 ])
 def test_gemv_matches_oracle(gpu, path, m, n, k):
     print(f"case M={m} N={n} K={k}", flush=True)
