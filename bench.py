@@ -28,6 +28,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
+COLD_FOOTPRINT_BYTES = 600 * 1000 * 1000  # buffers walked by a timing loop: more than the last-level cache holds
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
 MFMA_F16_PEAK_TFLOPS = 2500.0  # dense fp16 MFMA
 MFMA_I8_PEAK_TOPS = 5000.0     # dense int8 MFMA
@@ -165,24 +166,30 @@ def main():
     step_bytes = sum(w4a16_bytes(1, n, k) for (n, k) in DECODE_SHAPES)
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
 
-    # ---- per-shape launch durations (events around graphs of one shape walking the layers) --------
+    # ---- per-shape launch durations -------------------------------------------------------------
+    # Events around a graph of one shape walking enough copies of its weights (device-side clones of the
+    # layers) that no launch finds them in the last-level cache, as in the timed region above.
     per_shape = []
     for si, (n, k) in enumerate(DECODE_SHAPES):
-        def make(layer, si=si):
-            return lambda: launch(layers[layer][si])
-        fns = [make(layer % args.layers) for layer in range(4 * args.layers)]
-        us = timed_graph(fns, 10) / len(fns)
+        n_copies = max(args.layers, -(-COLD_FOOTPRINT_BYTES // w4a16_bytes(1, n, k)))
+        copies = []
+        for c in range(n_copies):
+            a, wq, s, y = layers[c % args.layers][si]
+            copies.append((a, wq, s, y) if c < args.layers else (a, wq.clone(), s.clone(), y))
+        fns = [(lambda t=t: launch(t)) for t in copies]
+        us = timed_graph(fns, 4) / len(fns)
+        del copies
         per_shape.append({"N": n, "K": k, "us": round(us, 3), "GB/s": round(w4a16_bytes(1, n, k) / us / 1e3, 1),
                           "frac_hbm": round(w4a16_bytes(1, n, k) / us / 1e3 / HBM_PEAK_GBS, 4)})
     if not args.no_extra:
         run_read_probe(torch, dev, lib, args.layers, per_shape, timed_graph)
-    # dominant kernel: the K = 4096 instantiation of the skinny kernel serves three of the four launches
+    # dominant kernel: the K = 4096 instantiations of the row-streaming kernel serve three of the four launches
     k4096 = [p for p in per_shape if p["K"] == 4096]
     dom_us = sum(p["us"] for p in k4096) / len(k4096)
     dom_bytes = sum(w4a16_bytes(1, p["N"], p["K"]) for p in k4096) / len(k4096)
     roofline = {
         "bound": "hbm",
-        "kernel": "nnf::w4a16_skinny_kernel (K=4096 instantiation; mean over its three launches per step)",
+        "kernel": "nnf::w4a16_gemv_rows_kernel<2, D, 8> (K=4096: two KiB per row; mean over its three launches per step)",
         "achieved": round(dom_bytes / dom_us / 1e3, 1),
         "peak": HBM_PEAK_GBS,
         "unit": "GB/s",
@@ -230,9 +237,10 @@ def main():
 
 
 def run_read_probe(torch, dev, lib, n_layers, per_shape, timed_graph):
-    """What a launch costs that does nothing but read the same number of bytes once (plain 128-bit loads,
-    one workgroup per CU, three depths of loads in flight, the best is kept): timed exactly like the GEMV
-    launches, walking as many distinct buffers, and written next to them as plain_read_us."""
+    """What a launch costs that does nothing but read the same number of bytes once: plain 128-bit loads, one
+    workgroup per CU, three depths of loads in flight (the best is kept as plain_read_us); the same bytes in the
+    M <= 16 kernel's tile order; and in plain order but through LDS.  Timed exactly like the GEMV launches, over
+    as many distinct buffers (nothing is found in the last-level cache)."""
     import ctypes
 
     fn = lib.nnf_internal_read_probe
@@ -241,9 +249,10 @@ def run_read_probe(torch, dev, lib, n_layers, per_shape, timed_graph):
     num_cu = torch.cuda.get_device_properties(0).multi_processor_count
     for entry in per_shape:
         nbytes = (w4a16_bytes(1, entry["N"], entry["K"]) + 15) // 16 * 16
-        bufs = [torch.randint(0, 255, (nbytes,), dtype=torch.uint8, device=dev) for _ in range(n_layers)]
+        n_bufs = max(n_layers, -(-COLD_FOOTPRINT_BYTES // nbytes))
+        bufs = [torch.randint(0, 255, (nbytes,), dtype=torch.uint8, device=dev) for _ in range(n_bufs)]
         best = None
-        by_depth = []
+        by_variant = []
         for variant in range(5):
             def make(buf, variant=variant):
                 def call():
@@ -251,17 +260,17 @@ def run_read_probe(torch, dev, lib, n_layers, per_shape, timed_graph):
                     if st != 0:
                         raise RuntimeError(f"nnf_internal_read_probe failed: {st}")
                 return call
-            fns = [make(bufs[i % n_layers]) for i in range(4 * n_layers)]
+            fns = [make(b) for b in bufs]
             fns[0]()
             torch.cuda.synchronize()
-            us = timed_graph(fns, 10) / len(fns)
+            us = timed_graph(fns, 4) / len(fns)
             if variant < 3:
                 best = us if best is None else min(best, us)
-            by_depth.append(round(us, 3))
+            by_variant.append(round(us, 3))
         entry["plain_read_us"] = round(best, 3)
-        entry["plain_read_us_32_64_128KiB_in_flight_per_cu"] = by_depth[:3]
-        entry["read_us_in_gemv_order"] = by_depth[3]
-        entry["read_us_through_lds"] = by_depth[4]
+        entry["plain_read_us_32_64_128KiB_in_flight_per_cu"] = by_variant[:3]
+        entry["read_us_in_tile_order"] = by_variant[3]
+        entry["read_us_through_lds"] = by_variant[4]
         entry["gemv_time_over_plain_read"] = round(entry["us"] / best, 3)
         del bufs
 

@@ -193,43 +193,54 @@ namespace nnf
         }
 
         // ---- one activation row: the row-streaming GEMV (w4a16_gemv_rows.hip) ----
+        // Eight wavefronts per workgroup (one workgroup per CU) measured fastest: sixteen pay the per-wavefront
+        // parts of the kernel twice as often, four leave the vector units idle between dependent instructions.
+        constexpr int ROWS_WAVES = 8;
+        inline int rows_grid(int N, int num_cu) { return N < num_cu ? N : num_cu; } // one workgroup per CU
         struct RowsPlan
         {
             int seg = 0;    // wavefront-wide loads (1 KiB of a weight row) per row and wavefront; 0: not applicable
             int kshift = 0; // log2 of the wavefronts that share a row
             int depth = 0;  // rows in flight per wavefront
-            // ring + scale chunks + activations + parked outputs of one workgroup (16 wavefronts)
+            // ring + activations (+ zeros) + their constants + the workgroup's scales + parked outputs + row counters
             size_t lds_bytes(int N, int K, int grid) const
             {
-                const int n_groups = grid * (16 >> kshift);
-                const size_t a_pad = ((size_t)(K >> 3) + 63) & ~(size_t)63; // 16-byte units of activations
-                return (size_t)16 * depth * seg * 1024 + 16 * 2048 + a_pad * 16 + a_pad * 4 +
-                       (size_t)16 * (N / n_groups + 1) * sizeof(float);
+                const size_t rows = (size_t)(N / grid + 1);                       // of a workgroup, at most
+                const size_t a_pad = (((size_t)(K >> 3) + 63) & ~(size_t)63) + 4; // 16-byte units of activations
+                return (size_t)ROWS_WAVES * depth * seg * 1024 + a_pad * 16 + a_pad * 4 +
+                       ((rows * (size_t)(K >> 7) * 2 + 1023) & ~(size_t)1023) + (rows << kshift) * sizeof(float) + 64;
             }
         };
-        inline RowsPlan plan_w4a16_rows(int M, int N, int K, int num_cu)
+        // forced_depth: for experiments (0: the plan's own choice)
+        inline RowsPlan plan_w4a16_rows(int M, int N, int K, int num_cu, int forced_depth = 0)
         {
             RowsPlan p;
             // whole 16-byte pieces of scales per segment, 4-byte aligned: K a multiple of 256
-            // (the activations are fetched in at most two rounds of 1024 16-byte units: K <= 16384)
+            // (the activations are fetched as at most 2048 16-byte units: K <= 16384)
             if (M != 1 || N < 1 || K < 1024 || K > 16384 || (K & 255) || num_cu < 1)
                 return p;
             const int loads_per_row = ((K >> 1) + 1023) >> 10;
             int kshift = 0;
-            while (kshift <= 4 && (loads_per_row + (1 << kshift) - 1) >> kshift > 3)
+            while ((1 << kshift) <= ROWS_WAVES && (loads_per_row + (1 << kshift) - 1) >> kshift > 3)
                 ++kshift;
-            if (kshift > 4)
+            if ((1 << kshift) > ROWS_WAVES)
                 return p;
             p.kshift = kshift;
             p.seg = (loads_per_row + (1 << kshift) - 1) >> kshift;
-            const int n_groups = num_cu * (16 >> kshift);
-            const int rows_q = N / n_groups;
-            // A CU takes about 64 wavefront-wide loads in flight: beyond that the wavefronts stall at issue
-            const int depth_max = p.seg == 1 ? 4 : (p.seg == 2 ? 2 : 1);
-            p.depth = rows_q < 1 ? 1 : (rows_q > depth_max ? depth_max : rows_q);
-            while (p.depth > 1 && p.lds_bytes(N, K, num_cu) > LDS_BYTES_PER_CU)
+            const int grid = rows_grid(N, num_cu);
+            // rows per wavefront of a K segment: the first `depth` of them are fixed
+            const int rows_q = (N / grid) / (ROWS_WAVES >> kshift);
+            // Two rows in flight per wavefront (a CU takes about 64 wavefront-wide loads in flight; more and the
+            // wavefronts stall at issue), a little deeper when a wavefront has many rows to walk (measured).
+            const int depth_max = p.seg == 3 ? 2 : 4;
+            p.depth = forced_depth > 0 ? forced_depth : (rows_q >= 8 ? (p.seg == 1 ? 4 : 3) : 2);
+            if (p.depth > depth_max)
+                p.depth = depth_max;
+            if (p.depth > rows_q)
+                p.depth = rows_q < 1 ? 1 : rows_q;
+            while (p.depth > 1 && p.lds_bytes(N, K, grid) > LDS_BYTES_PER_CU)
                 --p.depth;
-            if (p.lds_bytes(N, K, num_cu) > LDS_BYTES_PER_CU)
+            if (p.lds_bytes(N, K, grid) > LDS_BYTES_PER_CU)
                 p.seg = 0;
             return p;
         }
