@@ -230,7 +230,11 @@ namespace nnf
         if (g_tuning.force_path != 3 && M <= 16 && w4a16_skinny_supported(M, n_rows, K) && (!via_scratch || partial_ws))
         {
             void* y_gemv = via_scratch ? partial_ws : Y;
-            hipError_t e = launch_w4a16_skinny(stream, A, Wq, S, y_gemv, M, n_rows, K, zp, num_cu);
+            // one activation row: the row-streaming kernel where it applies
+            const bool rows = (g_tuning.force_path == 0 || g_tuning.force_path == 4) &&
+                              w4a16_gemv_rows_supported(M, n_rows, K, num_cu);
+            hipError_t e = rows ? launch_w4a16_gemv_rows(stream, A, Wq, S, y_gemv, n_rows, K, zp, num_cu)
+                                : launch_w4a16_skinny(stream, A, Wq, S, y_gemv, M, n_rows, K, zp, num_cu);
             if (e != hipSuccess || (!gate && !hb && !hr))
                 return e;
             const int blocks = (M * N + 255) / 256;
