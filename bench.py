@@ -36,10 +36,10 @@ MFMA_I8_PEAK_TOPS = 5000.0     # dense int8 MFMA
 DECODE_SHAPES = [(12288, 4096), (4096, 4096), (22016, 4096), (4096, 11008)]  # (N, K), M = 1
 GROUP = 128
 PROBE_BYTES = 1 << 30  # size of the calibration copy of --pmc-probe
-# HBM bytes per launch of the K = 4096 skinny kernel (mean over its three launches of a step), from two
-# rocprofv3 --pmc runs of `bench.py --pmc-probe`: FETCH_SIZE 13302.8 KiB x 2.000 (the factor by which the
-# counter under-reports the 1 GiB calibration copy) + WRITE_SIZE 25.0 KiB x 1.000.  Algorithmic: 27 067 392.
-SKINNY_K4096_TRAFFIC_BYTES = int((13302.8 * 2.0 + 25.0) * 1024)
+# HBM bytes per launch of the K = 4096 row-streaming kernel (mean over its three launches of a step), from two
+# rocprofv3 --pmc runs of `bench.py --pmc-probe`: FETCH_SIZE 13269.1 KiB x 2.000 (the factor by which the
+# counter under-reports the 1 GiB calibration copy) + WRITE_SIZE 27.3 KiB x 1.000.  Algorithmic: 27 067 392.
+ROWS_K4096_TRAFFIC_BYTES = int((13269.1 * 2.0 + 27.3) * 1024)
 
 
 def w4a16_bytes(m, n, k):
@@ -194,7 +194,7 @@ def main():
         "peak": HBM_PEAK_GBS,
         "unit": "GB/s",
         "frac": round(dom_bytes / dom_us / 1e3 / HBM_PEAK_GBS, 4),
-        "traffic": SKINNY_K4096_TRAFFIC_BYTES,
+        "traffic": ROWS_K4096_TRAFFIC_BYTES,
         "bytes_per_launch": int(dom_bytes),
         "us_per_launch": round(dom_us, 3),
     }

@@ -233,7 +233,7 @@ namespace nnf
             // Two rows in flight per wavefront (a CU takes about 64 wavefront-wide loads in flight; more and the
             // wavefronts stall at issue), a little deeper when a wavefront has many rows to walk (measured).
             const int depth_max = p.seg == 3 ? 2 : 4;
-            p.depth = forced_depth > 0 ? forced_depth : (rows_q >= 8 ? (p.seg == 1 ? 4 : 3) : 2);
+            p.depth = forced_depth > 0 ? forced_depth : (rows_q >= 16 ? (p.seg == 1 ? 4 : 3) : 2);
             if (p.depth > depth_max)
                 p.depth = depth_max;
             if (p.depth > rows_q)
