@@ -106,19 +106,12 @@ namespace nnf
         // ---- activations and scales: requested first (few loads, cache hits), once per workgroup ------------
         // (global -> LDS like the weights: a load into registers followed by an LDS write would be made to wait
         // for every LDS-bound load in flight, i.e. for the first weights)
-        constexpr int A_ROUNDS = 2048 / (WAVES * 64); // K <= 16384: at most 2048 units
-        bool a_loader = false;                        // this wavefront fetches a share of the activations
-#pragma unroll
-        for (int e = 0; e < A_ROUNDS; ++e)
+        const bool a_loader = wave * 64 < a_units; // this wavefront fetches a share of the activations
+        for (int u0 = wave * 64; u0 < a_units; u0 += WAVES * 64)
         {
-            const int u0 = e * (WAVES * 64) + wave * 64;
-            if (u0 < a_units)
-            {
-                const uint32_t u = (uint32_t)min(u0 + lane, a_units - 1);
-                __builtin_amdgcn_global_load_lds((global_ptr_t)(reinterpret_cast<const uint8_t*>(A) + (size_t)(u * 16u)),
-                                                 (lds_ptr_t)(reinterpret_cast<uint8_t*>(act) + u0 * 16), 16, 0, 0);
-                a_loader = true;
-            }
+            const uint32_t u = (uint32_t)min(u0 + lane, a_units - 1);
+            __builtin_amdgcn_global_load_lds((global_ptr_t)(reinterpret_cast<const uint8_t*>(A) + (size_t)(u * 16u)),
+                                             (lds_ptr_t)(reinterpret_cast<uint8_t*>(act) + u0 * 16), 16, 0, 0);
         }
         {
             // whole KiB of the block with 16 bytes per lane, the rest (a multiple of 4 bytes) with 4 bytes per
@@ -184,21 +177,17 @@ namespace nnf
             const half2_t sixteenth = half2_t{(half_t)0.0625f, (half_t)0.0625f};
             const float ce = -(1024.0f + (float)zp);
             const float co = -16.0f * (64.0f + (float)zp);
-#pragma unroll
-            for (int e = 0; e < A_ROUNDS; ++e)
+            for (int u0 = wave * 64; u0 < a_units; u0 += WAVES * 64)
             {
-                const int u = e * (WAVES * 64) + wave * 64 + lane;
-                if (e * (WAVES * 64) + wave * 64 < a_units)
-                {
-                    uintx4 a = permute_a8(act[u]);
-                    a.y = as_u32(as_half2(a.y) * sixteenth);
-                    a.w = as_u32(as_half2(a.w) * sixteenth);
-                    const half2_t x = as_half2(a.x), y = as_half2(a.y), z = as_half2(a.z), w = as_half2(a.w);
-                    const float se = ((float)x.x + (float)x.y) + ((float)z.x + (float)z.y);
-                    const float so = ((float)y.x + (float)y.y) + ((float)w.x + (float)w.y);
-                    act[u] = a;
-                    corr[u] = ce * se + co * so;
-                }
+                const int u = u0 + lane;
+                uintx4 a = permute_a8(act[u]);
+                a.y = as_u32(as_half2(a.y) * sixteenth);
+                a.w = as_u32(as_half2(a.w) * sixteenth);
+                const half2_t x = as_half2(a.x), y = as_half2(a.y), z = as_half2(a.z), w = as_half2(a.w);
+                const float se = ((float)x.x + (float)x.y) + ((float)z.x + (float)z.y);
+                const float so = ((float)y.x + (float)y.y) + ((float)w.x + (float)w.y);
+                act[u] = a;
+                corr[u] = ce * se + co * so;
             }
         }
         lds_barrier();
@@ -249,54 +238,64 @@ namespace nnf
                 }
                 v = __builtin_fmaf(t, sv[j], v);
             }
+            // the 16 lanes of a row, then the four rows: row_bcast:15 adds lane 15 of rows 0 and 2 into rows 1 and 3,
+            // row_bcast:31 adds lane 31 into rows 2 and 3 -- lane 63 ends up with everything
             v = row16_sum(v);
-            // the four rows of 16 lanes
-            const int vb = __builtin_bit_cast(int, v);
-            const float total = (__builtin_bit_cast(float, __builtin_amdgcn_readlane(vb, 0)) +
-                                 __builtin_bit_cast(float, __builtin_amdgcn_readlane(vb, 16))) +
-                                (__builtin_bit_cast(float, __builtin_amdgcn_readlane(vb, 32)) +
-                                 __builtin_bit_cast(float, __builtin_amdgcn_readlane(vb, 48)));
-            if (lane == 0)
-                outb[(r << kshift) + kpart] = total;
+            v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x142, 0xA, 0xF, false));
+            v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x143, 0xC, 0xF, false));
+            if (lane == 63)
+                outb[(r << kshift) + kpart] = v;
         };
 
         // D rows are in flight at the top of every iteration; a wavefront leaves the loop when the counter has run
         // past the workgroup's rows, with D - 1 rows (all of them real) still to come.  (D > 1 is only chosen when
         // every wavefront has at least D rows.)
-        int rows_v = 0; // lane s: the row in ring slot s
+        // The loop body is written out once per ring slot, so that slots and the rows in them are compile-time
+        // registers and addresses.
+        int in_slot[D]; // the row in each ring slot
 #pragma unroll
         for (int d = 0; d < D; ++d)
-            rows_v = lane == d ? widx + d * gpw : rows_v;
+            in_slot[d] = widx + d * gpw;
         const uint32_t next_addr = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) int*)(next_row + kpart);
-        int slot = 0;
-        int row = widx;
-        if (row < n_rows)
+        if (in_slot[0] < n_rows)
         {
-            while (true)
+            int exit_slot = -1;
+            while (exit_slot < 0)
             {
-                // The counter is bumped by hand: ahead of an LDS atomic that it can see, the compiler waits for
-                // every LDS-bound load in flight.  The result is there after the wait below.
-                int nx = 0;
-                if (lane == 0)
-                    asm volatile("ds_add_rtn_u32 %0, %1, %2" : "=v"(nx) : "v"(next_addr), "v"(1) : "memory");
-                __builtin_amdgcn_s_waitcnt(rows_vmcnt((D - 1) * SEG));
-                read_slot(row, slot);
-                asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(nx)::"memory"); // the slot has been read before it is refilled
-                nx = __builtin_amdgcn_readfirstlane(nx);
-                const bool more = nx < n_rows;
-                if (more)
-                    issue(nx, slot);
-                compute(row);
-                if (!more)
-                    break;
-                rows_v = lane == slot ? nx : rows_v;
-                slot = slot + 1 == D ? 0 : slot + 1;
-                row = __builtin_amdgcn_readlane(rows_v, slot);
+                static_for<0, D>([&](auto sc) {
+                    constexpr int slot = decltype(sc)::value;
+                    if (slot == 0 || exit_slot < 0)
+                    {
+                        // The counter is bumped by hand: ahead of an LDS atomic that it can see, the compiler waits
+                        // for every LDS-bound load in flight.  The result is there after the wait below.
+                        int nx = 0;
+                        if (lane == 0)
+                            asm volatile("ds_add_rtn_u32 %0, %1, %2" : "=v"(nx) : "v"(next_addr), "v"(1) : "memory");
+                        __builtin_amdgcn_s_waitcnt(rows_vmcnt((D - 1) * SEG));
+                        read_slot(in_slot[slot], slot);
+                        // the slot has been read before it is refilled
+                        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(nx)::"memory");
+                        nx = __builtin_amdgcn_readfirstlane(nx);
+                        const bool more = nx < n_rows;
+                        if (more)
+                            issue(nx, slot);
+                        compute(in_slot[slot]);
+                        if (more)
+                            in_slot[slot] = nx;
+                        else
+                            exit_slot = slot;
+                    }
+                });
             }
+            // the D - 1 rows still in flight, oldest first: the slots after the one the loop was left in
             static_for<0, D - 1>([&](auto tc) {
                 constexpr int t = decltype(tc)::value;
-                slot = slot + 1 == D ? 0 : slot + 1;
-                row = __builtin_amdgcn_readlane(rows_v, slot);
+                int slot = exit_slot + 1 + t;
+                slot = slot >= D ? slot - D : slot;
+                int row = in_slot[0];
+#pragma unroll
+                for (int d = 1; d < D; ++d)
+                    row = slot == d ? in_slot[d] : row;
                 __builtin_amdgcn_s_waitcnt(rows_vmcnt((D - 2 - t) * SEG));
                 read_slot(row, slot);
                 compute(row);
