@@ -11,6 +11,8 @@
 #include "nnfusion/engine/pass/graph/quant_fusion_pass.hpp"
 #include "nnfusion/engine/profiler/hip_runtime.hpp"
 
+#include "../../nnfusion_amd/csrc/nnf_workspace.h"
+
 #include <cstdio>
 #include <cstdlib>
 #include <fstream>
@@ -680,6 +682,89 @@ int main(int argc, char** argv)
             auto sl = find(g, "Slice");
             CONTAINS(sel.pick_first(sl, ROCM_GPU).second->get_or_emit_source()->body_unit->get_code(),
                      "hipMemcpy2DAsync(output0, 256, (const char*)input0 + 0, 512, 256, 8, hipMemcpyDeviceToDevice, stream)");
+        }
+    });
+
+    // the host arithmetic that picks a kernel variant for a shape and sizes its LDS / workspace
+    run_case("kernel_plans", [] {
+        namespace ws = nnf::workspace;
+        // one activation row: the row-streaming kernel
+        {
+            auto p = ws::plan_w4a16_rows(1, 4096, 4096, 256);
+            EXPECT(p.seg == 2 && p.kshift == 0 && p.depth == 2);
+            p = ws::plan_w4a16_rows(1, 22016, 4096, 256);
+            EXPECT(p.seg == 2 && p.kshift == 0 && p.depth == 2);
+            p = ws::plan_w4a16_rows(1, 4096, 11008, 256);
+            EXPECT(p.seg == 3 && p.kshift == 1 && p.depth == 2);
+            p = ws::plan_w4a16_rows(1, 8192, 8192, 256);
+            EXPECT(p.seg == 2 && p.kshift == 1);
+            p = ws::plan_w4a16_rows(1, 152064, 2048, 256);
+            EXPECT(p.seg == 1 && p.kshift == 0 && p.depth == 4);
+            // fewer rows than wavefronts: no prefetch beyond the first row
+            EXPECT(ws::plan_w4a16_rows(1, 300, 1024, 256).depth == 1);
+            EXPECT(ws::rows_grid(40, 256) == 40 && ws::rows_grid(4096, 256) == 256);
+            // not this kernel's shapes
+            EXPECT(ws::plan_w4a16_rows(2, 4096, 4096, 256).seg == 0);
+            EXPECT(ws::plan_w4a16_rows(1, 4096, 128, 256).seg == 0);
+            EXPECT(ws::plan_w4a16_rows(1, 4096, 4096 + 128, 256).seg == 0);
+            EXPECT(ws::plan_w4a16_rows(1, 4096, 32768, 256).seg == 0);
+            EXPECT(ws::plan_w4a16_rows(1, 0, 4096, 256).seg == 0);
+            const int ns[] = {1, 7, 40, 256, 300, 513, 4096, 5000, 12288, 22016, 32000, 80000, 152064, 1000000};
+            for (int n : ns)
+                for (int k = 1024; k <= 16384; k += 256)
+                {
+                    p = ws::plan_w4a16_rows(1, n, k, 256);
+                    if (p.seg == 0)
+                        continue; // (a very tall matrix with long rows: the workgroup's scales do not fit)
+                    const int grid = ws::rows_grid(n, 256);
+                    EXPECT(p.seg >= 1 && p.seg <= 3 && p.kshift >= 0 && p.kshift <= 3 && p.depth >= 1 && p.depth <= 4);
+                    EXPECT(((size_t)p.seg << p.kshift) * 1024 >= (size_t)k / 2);        // the segments cover a row
+                    EXPECT(((size_t)p.seg << p.kshift) * 1024 < (size_t)k / 2 + 1024 * (size_t)(1 << p.kshift)); // tightly
+                    EXPECT(p.lds_bytes(n, k, grid) <= ws::LDS_BYTES_PER_CU);
+                    // the first `depth` rows of every wavefront are fixed: they must exist
+                    EXPECT(p.depth == 1 || p.depth * (ws::ROWS_WAVES >> p.kshift) <= n / grid);
+                }
+            EXPECT(ws::plan_w4a16_rows(1, 1000000, 16384, 256).seg == 0);
+        }
+        // M <= 16: one workgroup holds the activations, or K is cut into ranges
+        {
+            for (int m = 1; m <= 16; ++m)
+                EXPECT(ws::w4a16_skinny_fits(m, 22016, 4096));
+            EXPECT(ws::w4a16_skinny_fits(7, 8192, 8192) && !ws::w4a16_skinny_fits(8, 8192, 8192));
+            EXPECT(ws::w4a16_skinny_ksplits(16, 8192, 8192) == 2 && ws::w4a16_skinny_ksplits(7, 8192, 8192) == 0);
+            EXPECT(ws::w4a16_skinny_ksplits(16, 8192, 8192 + 128) == 0);
+            EXPECT(!ws::w4a16_skinny_fits(17, 4096, 4096) && !ws::w4a16_skinny_fits(4, 4096, 4096 + 64) &&
+                   !ws::w4a16_skinny_fits(4, 8, 4096));
+            // weights addressed with 32-bit offsets
+            EXPECT(!ws::w4a16_skinny_fits(1, 1 << 20, 8192) && ws::w4a16_skinny_fits(1, 1 << 19, 8192));
+            EXPECT(ws::w4a16_gemm(1, 4096, 4096, 128) == 0 && ws::w4a16_gemm(16, 8192, 8192, 128) > 0);
+            for (int k = 128; k <= 16384; k += 128)
+            {
+                const auto p = ws::plan_w4a16_skinny(4, k);
+                EXPECT(p.cps >= 1 && p.ks >= 1 && p.ks <= 16 && p.cps * p.h * p.ks >= k / 128);
+            }
+        }
+        // W8A8, M <= 16
+        for (int k = 128; k <= 16384; k += 128)
+        {
+            const auto p = ws::plan_w8a8_skinny(1, k);
+            EXPECT(p.cps >= 1 && p.ks >= 1 && p.ks <= 16 && (p.kh == 1 || p.kh == 2 || p.kh == 4 || p.kh == 8));
+            EXPECT(p.cps * p.kh * p.ks >= k / 64 && p.cps * p.kh * (p.ks - 1) < k / 64);
+            EXPECT(ws::w8a8_skinny_fits(1, k) && ws::w8a8_gemm(1, 4096, k) == 0);
+        }
+        EXPECT(!ws::w8a8_skinny_fits(16, 8192) && ws::w8a8_gemm(16, 8192, 8192) > 0);
+        // GEMM tile plans: a split count the K loop can be cut into, partial sums sized for it
+        {
+            const int ms[] = {17, 64, 128, 256, 1024, 4096};
+            for (int m : ms)
+                for (int gate = 0; gate < 2; ++gate)
+                {
+                    const auto p = ws::plan_w4a16_gemm(m, 8192, 8192, gate != 0);
+                    EXPECT(p.splits >= 1 && p.splits <= 16 && (8192 / 128) / p.splits >= 4);
+                    EXPECT((p.splits > 1 || p.reduce_pass) == (ws::gemm_partial_bytes(m, 8192, gate != 0, p) > 0));
+                }
+            EXPECT(ws::plan_w4a16_gemm(4096, 8192, 8192, false).tile == ws::GEMM_TILE_BIG);
+            EXPECT(ws::plan_w4a16_gemm(32, 8192, 8192, false).reduce_pass);
         }
     });
 
