@@ -57,6 +57,7 @@ namespace nnf
         int lda;           // row stride of A (elements) = the full K
         int w_row_bytes;   // row stride of Wq (bytes)
         int s_row_groups;  // row stride of S (elements) = full K / 128
+        int k_last;        // length of the last range (the kernel's K is the length of the others)
         float* partial;    // [ksplits][M][N]
     };
 
@@ -91,7 +92,6 @@ namespace nnf
         const int n_threads = KS << 6;
         const int col = lane & 15; // n within the tile (B operand / D column), m for the A operand
         const int kq = lane >> 4;  // K quarter of the MFMA (A/B operands), row quad of D
-        const int G = K >> 7;
         // this workgroup among those of its K range
         const int k_range = KSPLIT ? (int)blockIdx.x % sp.ksplits : 0;
         const int wg = KSPLIT ? (int)blockIdx.x / sp.ksplits : (int)blockIdx.x;
@@ -100,8 +100,11 @@ namespace nnf
         {
             A += (size_t)k_range * K;
             Wq += (size_t)k_range * (K >> 1);
-            S += (size_t)k_range * G;
+            S += (size_t)k_range * (K >> 7);
+            if (k_range == sp.ksplits - 1)
+                K = sp.k_last; // the last range may be shorter
         }
+        const int G = K >> 7;
         const uint32_t row_bytes = KSPLIT ? (uint32_t)sp.w_row_bytes : (uint32_t)(K >> 1);
         const int s_row_groups = KSPLIT ? sp.s_row_groups : G;
         const int stride = n_wg;
@@ -135,13 +138,16 @@ namespace nnf
         };
         // scale block of a tile: 16 rows x G fp16, contiguous; thread t carries bytes [16t, 16t+16) of it
         // (threads beyond the block re-read its last 16 bytes)
-        // (KSPLIT: the rows of the block are s_row_groups apart; a row's share is G / 8 whole 16-byte pieces)
-        const int sc_units = 2 * G; // 16-byte units of one scale copy
+        // (KSPLIT: the rows of the block are s_row_groups apart; a row's share is ceil(G / 8) 16-byte pieces, the
+        // last of them moved back to end with the range, so that nothing is read past it)
+        const int pieces = (G + 7) >> 3;
+        const int sc_units = KSPLIT ? 16 * pieces : 2 * G; // 16-byte units of one scale copy
+        const int sc_stride = KSPLIT ? pieces * 8 : G;     // fp16 per row of it
         uint32_t s_lane_off = (uint32_t)min(tid, sc_units - 1) * 16u;
         if (KSPLIT)
         {
-            const int t = min(tid, sc_units - 1), pieces = G >> 3;
-            s_lane_off = (uint32_t)(t / pieces) * (uint32_t)s_row_groups * 2u + (uint32_t)(t % pieces) * 16u;
+            const int t = min(tid, sc_units - 1);
+            s_lane_off = (uint32_t)(t / pieces) * (uint32_t)s_row_groups * 2u + (uint32_t)min((t % pieces) * 16, G * 2 - 16);
         }
         auto load_s = [&](int tile) -> uintx4 {
             const uint32_t off = s_lane_off + (uint32_t)row0_of(tile) * (uint32_t)s_row_groups * 2u;
@@ -212,6 +218,7 @@ namespace nnf
         const int m_rd = min(col, M - 1); // rows >= M read a valid row; their D rows are never stored
         const bool s_loader = tid < sc_units;
         int chunk_of[H][CPS];
+        int sc_of[H][CPS]; // where the scale of the group sits in a row of the LDS copy
         float s_mask[H][CPS];
 #pragma unroll
         for (int h = 0; h < H; ++h)
@@ -220,6 +227,9 @@ namespace nnf
             {
                 chunk_of[h][c] = chunk_base[h] + c;
                 s_mask[h][c] = chunk_of[h][c] >= chunk_start[h] ? 1.0f : 0.0f;
+                sc_of[h][c] = chunk_of[h][c];
+                if (KSPLIT && chunk_of[h][c] >= (pieces - 1) * 8) // in the piece that was moved back
+                    sc_of[h][c] = (pieces - 1) * 8 + chunk_of[h][c] - (G - 8);
             }
 
         // ---- activations -> LDS ---------------------------------------------------------------------
@@ -355,7 +365,7 @@ namespace nnf
                     t = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, a_op(h, c, j)),
                                                                __builtin_bit_cast(half8_t, b), t, 0, 0, 0);
                 }
-                float s = (float)sc[col * G + chunk_of[h][c]] * s_mask[h][c];
+                float s = (float)sc[col * sc_stride + sc_of[h][c]] * s_mask[h][c];
                 acc.x = __builtin_fmaf(t.x, s, acc.x);
                 acc.y = __builtin_fmaf(t.y, s, acc.y);
                 acc.z = __builtin_fmaf(t.z, s, acc.z);
@@ -586,13 +596,16 @@ namespace nnf
     hipError_t launch_w4a16_skinny_split(hipStream_t stream, const void* A, const void* Wq, const void* S, float* partial,
                                          int M, int N, int K, int zp, int ksplits, int num_cu)
     {
-        const int k_range = K / ksplits;
+        const int k_range = workspace::w4a16_skinny_split_range(M, N, K);
+        if (k_range <= 0 || (K + k_range - 1) / k_range != ksplits)
+            return hipErrorInvalidValue;
         SkinnyPlan p = workspace::plan_w4a16_skinny(M, k_range);
         SkinnySplit sp;
         sp.ksplits = ksplits;
         sp.lda = K;
         sp.w_row_bytes = K >> 1;
         sp.s_row_groups = K >> 7;
+        sp.k_last = K - (ksplits - 1) * k_range;
         sp.partial = partial;
         switch (p.cps * 10 + p.h)
         {

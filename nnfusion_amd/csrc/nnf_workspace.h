@@ -168,24 +168,37 @@ namespace nnf
             return p.cps != 0 && p.cps <= (K >> 7) && p.lds(16 * 1024) <= LDS_BYTES_PER_CU;
         }
 
-        // M <= 16 shapes whose activations do not fit at once: number of K ranges (each a multiple of 1024 columns,
-        // at most 4096, whose activations fit) the skinny kernel is run over, or 0 when that does not apply
-        inline int w4a16_skinny_ksplits(int M, int N, int K)
+        // M <= 16 shapes whose activations do not fit at once are run over ranges of K whose activations do fit:
+        // equal ranges (multiples of 1024 columns, at most 4096) when K divides that way, otherwise ranges of a
+        // multiple of 1024 and a shorter last one of at least 1024.  Returns the length of the ranges (of all but
+        // the last), or 0 when this does not apply.
+        inline int w4a16_skinny_split_range(int M, int N, int K)
         {
-            if (M < 1 || M > 16 || N < 16 || K < 2048 || (K & 1023) || w4a16_skinny_fits(M, N, K))
+            if (M < 1 || M > 16 || N < 16 || K < 2048 || (K & 127) || w4a16_skinny_fits(M, N, K))
                 return 0;
             if ((size_t)N * (size_t)(K >> 1) >= ((size_t)1 << 32)) // 32-bit offsets over whole rows
                 return 0;
-            static const int options[] = {2, 4, 8, 16};
-            for (int s : options)
+            static const int equal[] = {2, 4, 8, 16};
+            for (int s : equal)
             {
-                const int k_range = K / s;
-                if (K % s != 0 || (k_range & 1023) || k_range > 4096)
-                    continue;
-                if (w4a16_skinny_fits(M, N, k_range))
-                    return s;
+                const int r = K / s;
+                if (K % s == 0 && (r & 1023) == 0 && r <= 4096 && w4a16_skinny_fits(M, N, r))
+                    return r;
+            }
+            static const int lengths[] = {4096, 3072, 2048, 1024};
+            for (int r : lengths)
+            {
+                const int s = (K + r - 1) / r;
+                if (w4a16_skinny_fits(M, N, r) && s <= 16 && K - (s - 1) * r >= 1024)
+                    return r;
             }
             return 0;
+        }
+        // the number of those ranges (0: does not apply)
+        inline int w4a16_skinny_ksplits(int M, int N, int K)
+        {
+            const int r = w4a16_skinny_split_range(M, N, K);
+            return r ? (K + r - 1) / r : 0;
         }
         inline size_t skinny_split_bytes(int M, int N_total, int K)
         {

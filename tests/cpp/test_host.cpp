@@ -732,7 +732,11 @@ int main(int argc, char** argv)
                 EXPECT(ws::w4a16_skinny_fits(m, 22016, 4096));
             EXPECT(ws::w4a16_skinny_fits(7, 8192, 8192) && !ws::w4a16_skinny_fits(8, 8192, 8192));
             EXPECT(ws::w4a16_skinny_ksplits(16, 8192, 8192) == 2 && ws::w4a16_skinny_ksplits(7, 8192, 8192) == 0);
-            EXPECT(ws::w4a16_skinny_ksplits(16, 8192, 8192 + 128) == 0);
+            // K that does not divide into equal ranges of a multiple of 1024: a shorter last range
+            EXPECT(ws::w4a16_skinny_split_range(16, 8192, 8192 + 128) == 3072 && ws::w4a16_skinny_ksplits(16, 8192, 8192 + 128) == 3);
+            EXPECT(ws::w4a16_skinny_split_range(8, 4096, 11008) == 4096 && ws::w4a16_skinny_ksplits(8, 4096, 11008) == 3);
+            EXPECT(ws::w4a16_skinny_ksplits(16, 4096, 13824) == 4 && ws::w4a16_skinny_ksplits(4, 4096, 11008) == 0);
+            EXPECT(ws::skinny_split_bytes(8, 4096, 11008) == (size_t)3 * 8 * 4096 * 4);
             EXPECT(!ws::w4a16_skinny_fits(17, 4096, 4096) && !ws::w4a16_skinny_fits(4, 4096, 4096 + 64) &&
                    !ws::w4a16_skinny_fits(4, 8, 4096));
             // weights addressed with 32-bit offsets

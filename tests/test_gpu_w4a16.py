@@ -50,6 +50,7 @@ def _check(y, ref):
     (5, 64, 4096), (7, 130, 1024), (8, 512, 8192), (16, 1024, 8192),
     (16, 256, 1024), (12, 96, 2048), (16, 48, 3072), (9, 400, 512),  # more rows than wavefronts in the workgroup
     (16, 1040, 8192), (8, 520, 8192), (13, 77, 4096), (16, 64, 16384),  # activations too large for LDS: K in ranges
+    (8, 100, 11008), (16, 260, 11008), (12, 64, 13824), (16, 48, 8320), (9, 33, 5248),  # ... with a shorter last range
     (4, 300, 8192), (3, 200, 12288), (2, 96, 6144),  # two passes over K per tile
     # one activation row: rows shared by 1, 2, 4 wavefronts, ragged last K segment, fewer rows than wavefronts,
     # more rows per wavefront than one chunk of scales holds
