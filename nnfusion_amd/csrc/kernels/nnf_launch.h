@@ -48,6 +48,10 @@ namespace nnf
     hipError_t launch_w8a8_gemm(hipStream_t stream, const void* A, const void* s_tok, const void* W, const void* s_ch,
                                 void* Y, void* acc, int M, int N, int K, void* partial_ws);
     bool w8a8_skinny_supported(int M, int K);
+    // one activation row (M = 1): the row-streaming kernel; acc != nullptr writes the raw int32 sums
+    hipError_t launch_w8a8_gemv_rows(hipStream_t stream, const void* A, const void* s_tok, const void* W, const void* s_ch,
+                                     void* Y, void* acc, int N, int K, int num_cu);
+    bool w8a8_gemv_rows_supported(int M, int N, int K, int num_cu);
 
     // Tuning knobs for experiments (not part of the public ABI): 0 = automatic.
     struct Tuning

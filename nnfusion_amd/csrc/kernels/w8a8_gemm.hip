@@ -273,6 +273,8 @@ namespace nnf
         p.N = N;
         p.K = K;
         const bool raw = acc != nullptr;
+        if ((g_tuning.force_path == 0 || g_tuning.force_path == 4) && w8a8_gemv_rows_supported(M, N, K, num_cu))
+            return launch_w8a8_gemv_rows(stream, A, s_tok, W, s_ch, Y, acc, N, K, num_cu);
         const bool skinny = g_tuning.force_path != 3 && w8a8_skinny_supported(M, K);
         if (skinny)
             return raw ? launch_q8_skinny<true>(stream, p, num_cu) : launch_q8_skinny<false>(stream, p, num_cu);

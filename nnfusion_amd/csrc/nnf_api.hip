@@ -184,8 +184,10 @@ size_t nnf_w8a8_gemm_workspace_bytes(int M, int N, int K)
 }
 
 // room for the int32 partial sums when the MFMA GEMM serves the shape (the M <= 16 kernel needs none)
-static int check_w8a8_workspace(int M, int N, int K, const void* workspace, size_t workspace_bytes)
+static int check_w8a8_workspace(int M, int N, int K, int num_cu, const void* workspace, size_t workspace_bytes)
 {
+    if ((nnf::g_tuning.force_path == 0 || nnf::g_tuning.force_path == 4) && nnf::w8a8_gemv_rows_supported(M, N, K, num_cu))
+        return NNF_OK;
     if (nnf::g_tuning.force_path != 3 && nnf::w8a8_skinny_supported(M, K))
         return NNF_OK;
     const size_t need = nnf::workspace::gemm_partial_bytes(
@@ -215,11 +217,11 @@ int nnf_w8a8_gemm(nnf_stream_t stream, const void* A, const void* s_tok, const v
         return st;
     if (!s_tok || !s_ch)
         return NNF_ERR_INVALID_ARGUMENT;
-    st = check_w8a8_workspace(M, N, K, workspace, workspace_bytes);
-    if (st != NNF_OK)
-        return st;
     DeviceInfo dev;
     st = current_device_info(dev);
+    if (st != NNF_OK)
+        return st;
+    st = check_w8a8_workspace(M, N, K, dev.num_cu, workspace, workspace_bytes);
     if (st != NNF_OK)
         return st;
     return (int)nnf::launch_w8a8((hipStream_t)stream, A, s_tok, W, s_ch, Y, nullptr, M, N, K, dev.num_cu, workspace);
@@ -231,11 +233,11 @@ int nnf_w8a8_gemm_acc(nnf_stream_t stream, const void* A, const void* W, void* a
     int st = check_w8a8(A, W, acc, M, N, K);
     if (st != NNF_OK)
         return st;
-    st = check_w8a8_workspace(M, N, K, workspace, workspace_bytes);
-    if (st != NNF_OK)
-        return st;
     DeviceInfo dev;
     st = current_device_info(dev);
+    if (st != NNF_OK)
+        return st;
+    st = check_w8a8_workspace(M, N, K, dev.num_cu, workspace, workspace_bytes);
     if (st != NNF_OK)
         return st;
     return (int)nnf::launch_w8a8((hipStream_t)stream, A, nullptr, W, nullptr, nullptr, acc, M, N, K, dev.num_cu,

@@ -318,6 +318,48 @@ namespace nnf
             const Q8SkinnyPlan pl = plan_w8a8_skinny(M, K);
             return pl.cps != 0 && pl.lds + 16 * 1024 <= LDS_BYTES_PER_CU;
         }
+        // ---- W8A8, one activation row: the row-streaming GEMV (w8a8_gemv_rows.hip) ----
+        struct Q8RowsPlan
+        {
+            int seg = 0;    // wavefront-wide loads (1 KiB of a weight row) per row and wavefront; 0: not applicable
+            int kshift = 0; // log2 of the wavefronts that share a row
+            int depth = 0;  // rows in flight per wavefront
+            // ring + activations (+ zeros) + parked sums + row counters
+            size_t lds_bytes(int N, int K, int grid) const
+            {
+                const size_t rows = (size_t)(N / grid + 1); // of a workgroup, at most
+                return (size_t)ROWS_WAVES * depth * seg * 1024 + (((size_t)K + 1023) & ~(size_t)1023) + 16 +
+                       (rows << kshift) * sizeof(int) + 64;
+            }
+        };
+        // forced_depth: for experiments (0: the plan's own choice)
+        inline Q8RowsPlan plan_w8a8_rows(int M, int N, int K, int num_cu, int forced_depth = 0)
+        {
+            Q8RowsPlan p;
+            if (M != 1 || N < 1 || K < 1024 || (K & 127) || num_cu < 1)
+                return p;
+            const int loads_per_row = (K + 1023) >> 10;
+            int kshift = 0;
+            while ((1 << kshift) <= ROWS_WAVES && (loads_per_row + (1 << kshift) - 1) >> kshift > 3)
+                ++kshift;
+            if ((1 << kshift) > ROWS_WAVES)
+                return p; // K > 24576
+            p.kshift = kshift;
+            p.seg = (loads_per_row + (1 << kshift) - 1) >> kshift;
+            const int grid = rows_grid(N, num_cu);
+            const int rows_q = (N / grid) / (ROWS_WAVES >> kshift); // rows per wavefront of a K segment
+            const int depth_max = p.seg == 3 ? 2 : 4;
+            p.depth = forced_depth > 0 ? forced_depth : (rows_q >= 16 ? (p.seg == 1 ? 4 : 3) : 2);
+            if (p.depth > depth_max)
+                p.depth = depth_max;
+            if (p.depth > rows_q)
+                p.depth = rows_q < 1 ? 1 : rows_q;
+            while (p.depth > 1 && p.lds_bytes(N, K, grid) > LDS_BYTES_PER_CU)
+                --p.depth;
+            if (p.lds_bytes(N, K, grid) > LDS_BYTES_PER_CU)
+                p.seg = 0;
+            return p;
+        }
         // nnf_w8a8_gemm / nnf_w8a8_gemm_acc: [ int32 partial sums ] (same tile plan as the fp16 x int4 GEMM)
         inline size_t w8a8_gemm(int M, int N, int K)
         {
