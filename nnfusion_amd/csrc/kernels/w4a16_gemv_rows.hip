@@ -149,8 +149,11 @@ namespace nnf
                 __builtin_amdgcn_global_load_lds((global_ptr_t)(src + w_off[j]),
                                                  (lds_ptr_t)(ring + (slot * SEG + j) * 1024), 16, 0, 0);
         };
+        // (two rows now; the rest of the ring after the activations are in registers: with everything asked for at
+        // once the last wavefronts stall at issue -- a CU takes about 64 wavefront-wide loads -- and hold up the barrier)
+        constexpr int D0 = D < 2 ? D : 2;
 #pragma unroll
-        for (int d = 0; d < D; ++d)
+        for (int d = 0; d < D0; ++d)
             issue(widx + d * gpw, d);
         __builtin_amdgcn_sched_barrier(0);
         if (tid < ksw)
@@ -171,7 +174,7 @@ namespace nnf
         // it stores the unit as (a0,a4) (a1,a5)/16 (a2,a6) (a3,a7)/16 and, next to it, the unit's part of the
         // constant  (1024 + zp) sum a_even + (64 + zp) sum a_odd  that the nibble trick adds to every row.
         // Only the weights asked for above may still be in flight afterwards: the scales have landed too.
-        __builtin_amdgcn_s_waitcnt(rows_vmcnt(D * SEG));
+        __builtin_amdgcn_s_waitcnt(rows_vmcnt(D0 * SEG));
         if (a_loader)
         {
             const half2_t sixteenth = half2_t{(half_t)0.0625f, (half_t)0.0625f};
@@ -256,6 +259,9 @@ namespace nnf
 #pragma unroll
         for (int d = 0; d < D; ++d)
             in_slot[d] = widx + d * gpw;
+#pragma unroll
+        for (int d = D0; d < D; ++d)
+            issue(in_slot[d], d);
         const uint32_t next_addr = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) int*)(next_row + kpart);
         if (in_slot[0] < n_rows)
         {
