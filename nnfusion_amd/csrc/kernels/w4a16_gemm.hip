@@ -19,19 +19,21 @@
 
 namespace nnf
 {
-    // one row per wavefront: Xn[m, :] = fp16( x * rsqrt(mean_k(x^2) + eps) * gamma )
+    // one row per workgroup of four wavefronts: Xn[m, :] = fp16( x * rsqrt(mean_k(x^2) + eps) * gamma ).
+    // The row is read once: a thread keeps its 16-byte units in registers between the two passes (up to K = 16384;
+    // the units beyond that are read again).
     __global__ __launch_bounds__(256) void rms_norm_kernel(const half_t* __restrict__ X, const half_t* __restrict__ gamma,
                                                            half_t* __restrict__ Xn, int M, int K, float eps)
     {
-        const int lane = threadIdx.x & 63;
-        const int m = blockIdx.x * 4 + (threadIdx.x >> 6);
-        if (m >= M)
-            return;
+        constexpr int KEEP = 8; // units per thread kept in registers
+        __shared__ float part[4];
+        const int tid = threadIdx.x;
+        const int m = blockIdx.x;
+        const int units = K >> 3;
         const uintx4* row = reinterpret_cast<const uintx4*>(X + (size_t)m * K);
+        uintx4 kept[KEEP];
         float ss = 0.f;
-        for (int i = lane; i < (K >> 3); i += 64)
-        {
-            uintx4 v = row[i];
+        auto sq = [&](const uintx4& v) {
             const uint32_t vv[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
             for (int j = 0; j < 4; ++j)
@@ -39,14 +41,27 @@ namespace nnf
                 half2_t h = as_half2(vv[j]);
                 ss += (float)h.x * (float)h.x + (float)h.y * (float)h.y;
             }
+        };
+#pragma unroll
+        for (int e = 0; e < KEEP; ++e)
+        {
+            const int i = tid + e * 256;
+            kept[e] = i < units ? row[i] : uintx4{0u, 0u, 0u, 0u};
         }
+#pragma unroll
+        for (int e = 0; e < KEEP; ++e)
+            sq(kept[e]);
+        for (int i = tid + KEEP * 256; i < units; i += 256)
+            sq(row[i]);
         ss = wave_sum(ss);
+        if ((tid & 63) == 0)
+            part[tid >> 6] = ss;
+        __syncthreads();
+        ss = (part[0] + part[1]) + (part[2] + part[3]);
         const float rstd = 1.0f / __builtin_sqrtf(ss / (float)K + eps);
         const uintx4* grow = reinterpret_cast<const uintx4*>(gamma);
         uintx4* out = reinterpret_cast<uintx4*>(Xn + (size_t)m * K);
-        for (int i = lane; i < (K >> 3); i += 64)
-        {
-            uintx4 v = row[i], g = grow[i], o;
+        auto norm = [&](const uintx4& v, const uintx4& g) {
             const uint32_t vv[4] = {v.x, v.y, v.z, v.w};
             const uint32_t gg[4] = {g.x, g.y, g.z, g.w};
             uint32_t oo[4];
@@ -58,12 +73,17 @@ namespace nnf
                 r.y = (half_t)((float)x.y * rstd * (float)w.y);
                 oo[j] = as_u32(r);
             }
-            o.x = oo[0];
-            o.y = oo[1];
-            o.z = oo[2];
-            o.w = oo[3];
-            out[i] = o;
+            return uintx4{oo[0], oo[1], oo[2], oo[3]};
+        };
+#pragma unroll
+        for (int e = 0; e < KEEP; ++e)
+        {
+            const int i = tid + e * 256;
+            if (i < units)
+                out[i] = norm(kept[e], grow[i]);
         }
+        for (int i = tid + KEEP * 256; i < units; i += 256)
+            out[i] = norm(row[i], grow[i]);
     }
 
     // Y[m, n] = epilogue( sum_s partial[s][m][n] ); four consecutive columns per thread.
@@ -214,7 +234,7 @@ namespace nnf
         {
             if (!rms_ws)
                 return hipErrorInvalidValue;
-            hipLaunchKernelGGL(rms_norm_kernel, dim3((M + 3) / 4), dim3(256), 0, stream, (const half_t*)A,
+            hipLaunchKernelGGL(rms_norm_kernel, dim3(M), dim3(256), 0, stream, (const half_t*)A,
                                (const half_t*)rms_gamma, (half_t*)rms_ws, M, K, rms_eps);
             hipError_t e = hipGetLastError();
             if (e != hipSuccess)
