@@ -94,17 +94,20 @@ namespace nnf
                                                                 const half_t* __restrict__ residual, half_t* __restrict__ Y,
                                                                 int ldy)
     {
+        // grid: x over groups of four columns, y = row
         const int quads = (N + 3) >> 2;
-        const long long t = (long long)blockIdx.x * 256 + threadIdx.x;
-        if (t >= (long long)M * quads)
+        const int q = (int)blockIdx.x * 256 + (int)threadIdx.x;
+        if (q >= quads)
             return;
-        const int m = (int)(t / quads);
-        const int n = (int)(t - (long long)m * quads) * 4;
+        const int m = blockIdx.y;
+        const int n = q * 4;
         const size_t plane = (size_t)M * ld_partial;
         const float* src = partial + (size_t)m * ld_partial + n;
         // ld_partial and n are multiples of 4 when N is; otherwise fall back to scalar accesses
         const bool vec = ((ld_partial | N) & 3) == 0;
         float a[4] = {0.f, 0.f, 0.f, 0.f}, u[4] = {0.f, 0.f, 0.f, 0.f};
+        // (the ranges are added in order, whatever the unrolling: the sums do not depend on it)
+#pragma unroll 4
         for (int s = 0; s < splits; ++s)
         {
             const float* ps = src + (size_t)s * plane;
@@ -129,6 +132,7 @@ namespace nnf
                     }
             }
         }
+        half_t out[4];
         for (int j = 0; j < 4; ++j)
         {
             if (n + j >= N)
@@ -144,7 +148,17 @@ namespace nnf
                 v = (float)(half_t)v + (float)bias[n + j];
             if (RESID)
                 v = (float)(half_t)v + (float)residual[(size_t)m * ldy + n + j];
-            Y[(size_t)m * ldy + n + j] = (half_t)v;
+            out[j] = (half_t)v;
+        }
+        half_t* dst = Y + (size_t)m * ldy + n;
+        if (vec && (ldy & 3) == 0)
+        {
+            *reinterpret_cast<uintx2*>(dst) = uintx2{as_u32(half2_t{out[0], out[1]}), as_u32(half2_t{out[2], out[3]})};
+        }
+        else
+        {
+            for (int j = 0; j < 4 && n + j < N; ++j)
+                dst[j] = out[j];
         }
     }
 
@@ -181,8 +195,8 @@ namespace nnf
         template <bool GATE, bool BIAS, bool RESID>
         hipError_t launch_reduce(hipStream_t stream, const GemmParams& p)
         {
-            const long long threads = (long long)p.M * ((p.N + 3) >> 2);
-            hipLaunchKernelGGL((splitk_reduce_kernel<GATE, BIAS, RESID>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0,
+            const int quads = (p.N + 3) >> 2;
+            hipLaunchKernelGGL((splitk_reduce_kernel<GATE, BIAS, RESID>), dim3((unsigned)((quads + 255) / 256), (unsigned)p.M), dim3(256), 0,
                                stream, (const float*)p.partial, p.splits, p.M, p.N, p.ld_partial, p.bias, p.residual, p.Y,
                                p.ldy);
             return hipGetLastError();

@@ -248,16 +248,18 @@ namespace nnf
     template <bool RAW>
     __global__ __launch_bounds__(256) void w8a8_splitk_reduce_kernel(Q8GemmParams p)
     {
+        // grid: x over groups of four columns, y = row
         const int quads = (p.N + 3) >> 2;
-        const long long t = (long long)blockIdx.x * 256 + threadIdx.x;
-        if (t >= (long long)p.M * quads)
+        const int q = (int)blockIdx.x * 256 + (int)threadIdx.x;
+        if (q >= quads)
             return;
-        const int m = (int)(t / quads);
-        const int n = (int)(t - (long long)m * quads) * 4;
+        const int m = blockIdx.y;
+        const int n = q * 4;
         const size_t plane = (size_t)p.M * p.N;
         const int32_t* src = p.partial + (size_t)m * p.N + n;
         const bool vec = (p.N & 3) == 0;
         int a[4] = {0, 0, 0, 0};
+#pragma unroll 4
         for (int s = 0; s < p.splits; ++s)
         {
             const int32_t* ps = src + (size_t)s * plane;
@@ -334,9 +336,9 @@ namespace nnf
             }
             if (e != hipSuccess)
                 return e;
-            const long long threads = (long long)p.M * ((p.N + 3) >> 2);
-            hipLaunchKernelGGL((w8a8_splitk_reduce_kernel<RAW>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, stream,
-                               p);
+            const int quads = (p.N + 3) >> 2;
+            hipLaunchKernelGGL((w8a8_splitk_reduce_kernel<RAW>), dim3((unsigned)((quads + 255) / 256), (unsigned)p.M), dim3(256), 0,
+                               stream, p);
             return hipGetLastError();
         }
     } // namespace
