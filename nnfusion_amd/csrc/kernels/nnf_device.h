@@ -4,6 +4,7 @@
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <type_traits>
 
 namespace nnf
 {
@@ -88,6 +89,47 @@ namespace nnf
     __device__ __forceinline__ void lds_barrier()
     {
         asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    }
+
+    // f(integral_constant<int, I>) for I = BEGIN .. END-1: for bodies that need I as a compile-time constant
+    // (instruction offsets, wait counts)
+    template <int BEGIN, int END, class F>
+    __device__ __forceinline__ void unroll_for(F&& f)
+    {
+        if constexpr (BEGIN < END)
+        {
+            f(std::integral_constant<int, BEGIN>{});
+            unroll_for<BEGIN + 1, END>(f);
+        }
+    }
+
+    // 128-bit LDS read that the compiler's wait-count insertion does not see.  The compiler waits for ALL
+    // LDS reads in flight (lgkmcnt(0)) ahead of the first use of any of them once reads issued in different
+    // loop iterations are pending; with these, fragments for the next MFMA group stay in flight while the
+    // current group is issued.  The value is valid only after lds_wait<N>() on it, N = number of LDS
+    // operations issued after the read (LDS operations complete in order).
+    template <int OFFSET, class V>
+    __device__ __forceinline__ void lds_read_b128_nowait(V& dst, uint32_t lds_addr)
+    {
+        static_assert(sizeof(V) == 16 && OFFSET >= 0 && OFFSET < 65536, "ds_read_b128 with a 16-bit offset");
+        asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(lds_addr), "n"(OFFSET) : "memory");
+    }
+    // s_waitcnt lgkmcnt(N); `first` is tied to the wait, `also` (values read before it) to `first`'s
+    // position through the order of volatile statements: none of them can be used ahead of the wait.
+    template <int N, class V>
+    __device__ __forceinline__ void lds_wait(V& first)
+    {
+        static_assert(N >= 0 && N <= 15, "lgkmcnt is four bits wide");
+        asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(first) : "n"(N) : "memory");
+    }
+    template <class V>
+    __device__ __forceinline__ void lds_wait_also(V& v)
+    {
+        asm volatile("" : "+v"(v));
+    }
+    __device__ __forceinline__ uint32_t lds_address(const void* p)
+    {
+        return (uint32_t)(uintptr_t)(const void __attribute__((address_space(3)))*)p;
     }
 
     // fp32 value -> fp16, as two roundings (the value is first a rounded fp32).  Without the opaque

@@ -171,36 +171,69 @@ namespace nnf
                 for (int e = 0; e < 16; ++e)
                     acc[i][j][e] = 0;
 
-        auto compute = [&](int stage) {
-            const uint8_t* base = smem + stage * STAGE_BYTES;
+        // A K step is two sub-steps of 32 bytes; the fragments of a sub-step (TM + TN 128-bit reads) are
+        // fetched from LDS while the MFMAs of the sub-step before it run, into the other of two register sets.
+        // Row r of a fragment and row r + 32 share their swizzle: the reads of a set are one address per
+        // operand plus constant offsets.
+        intx4 af[2][TM], bf[2][TN];
+        uint32_t a_addr[2], w_addr[2];
 #pragma unroll
-            for (int s = 0; s < 2; ++s)
-            {
-                intx4 af[TM], bf[TN];
+        for (int s = 0; s < 2; ++s)
+        {
+            const uint32_t piece = (uint32_t)(((2 * s + h) ^ ((l32 >> 2) & 3)) << 4);
+            a_addr[s] = lds_address(smem) + (uint32_t)((wm * (TM * 32) + l32) * 64) + piece;
+            w_addr[s] = lds_address(smem) + (uint32_t)((wn * (TN * 32) + l32) * 64) + piece;
+        }
+        constexpr int FRAG_READS = TM + TN;
+        auto read_frags = [&](int stage, auto s_c, auto set_c) {
+            constexpr int s = decltype(s_c)::value, set = decltype(set_c)::value;
+            const uint32_t off = (uint32_t)(stage * STAGE_BYTES);
+            const uint32_t aa = a_addr[s] + off, ww = w_addr[s] + off;
+            unroll_for<0, TM>([&](auto i) { lds_read_b128_nowait<decltype(i)::value * 2048>(af[set][i], aa); });
+            unroll_for<0, TN>(
+                [&](auto j) { lds_read_b128_nowait<A_TILE_BYTES + decltype(j)::value * 2048>(bf[set][j], ww); });
+        };
+        // the set is usable once at most `later` LDS reads issued after it are in flight
+        auto wait_frags = [&](auto set_c, auto later_c) {
+            constexpr int set = decltype(set_c)::value;
+            lds_wait<decltype(later_c)::value>(af[set][0]);
+            unroll_for<1, TM>([&](auto i) { lds_wait_also(af[set][i]); });
+            unroll_for<0, TN>([&](auto j) { lds_wait_also(bf[set][j]); });
+        };
+        auto mfmas = [&](auto set_c) {
+            constexpr int set = decltype(set_c)::value;
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
 #pragma unroll
                 for (int i = 0; i < TM; ++i)
-                    af[i] = *reinterpret_cast<const intx4*>(base + a_frag[i] + (((2 * s + h) ^ a_swz[i]) << 4));
-#pragma unroll
-                for (int j = 0; j < TN; ++j)
-                    bf[j] = *reinterpret_cast<const intx4*>(base + w_frag[j] + (((2 * s + h) ^ w_swz[j]) << 4));
-#pragma unroll
-                for (int j = 0; j < TN; ++j)
-#pragma unroll
-                    for (int i = 0; i < TM; ++i)
-                        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i], bf[j], acc[i][j], 0, 0, 0);
-            }
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[set][j], af[set][i], acc[i][j], 0, 0, 0);
         };
+        using I0 = std::integral_constant<int, 0>;
+        using I1 = std::integral_constant<int, 1>;
+        using NONE = std::integral_constant<int, 0>;
+        using ONE_SET = std::integral_constant<int, FRAG_READS>;
 
         // ---- K loop: stage kt % STAGES; loads run STAGES-1 K steps ahead ------------------------------------
-        // Vector-memory operations complete in order and every step issues TILE_LOADS of them: before the
-        // barrier of step kt at most the loads of the STAGES-2 steps after kt may still be outstanding.
+        // Vector-memory operations complete in order and every step issues TILE_LOADS of them.
+        // AHEAD (four stages or more): the barrier of step kt also certifies stage kt+1 (at most the loads
+        // issued during step kt-1 are outstanding), so the first fragments of step kt+1 are read during
+        // step kt and no MFMA waits for LDS behind a barrier.  The stage refilled during step kt is the one
+        // of step kt-1, whose last fragment reads every wavefront has waited for before its MFMAs of kt-1.
+        constexpr bool AHEAD = STAGES >= 4;
+        constexpr int WAIT_LOADS = AHEAD ? (STAGES - 3) * TILE_LOADS : (STAGES - 2) * TILE_LOADS;
 #pragma unroll
         for (int s = 0; s < STAGES - 1; ++s)
             issue_tile_loads(min(s, KT - 1), s);
         int stage = 0;
-        for (int kt = 0; kt < KT; ++kt)
+        if (AHEAD)
         {
             __builtin_amdgcn_s_waitcnt(vmcnt_imm((STAGES - 2) * TILE_LOADS));
+            __builtin_amdgcn_s_barrier();
+            read_frags(0, I0{}, I0{});
+        }
+        for (int kt = 0; kt < KT; ++kt)
+        {
+            __builtin_amdgcn_s_waitcnt(vmcnt_imm(WAIT_LOADS));
             __builtin_amdgcn_s_barrier();
             {
                 // past the end: reload a valid tile into the free stage
@@ -208,39 +241,134 @@ namespace nnf
                 st = st >= STAGES ? st - STAGES : st;
                 issue_tile_loads(min(kt + STAGES - 1, KT - 1), st);
             }
-            compute(stage);
-            stage = stage + 1 == STAGES ? 0 : stage + 1;
+            const int next_stage = stage + 1 == STAGES ? 0 : stage + 1;
+            if (!AHEAD)
+                read_frags(stage, I0{}, I0{});
+            read_frags(stage, I1{}, I1{});
+            wait_frags(I0{}, ONE_SET{});
+            __builtin_amdgcn_sched_barrier(0);
+            mfmas(I0{});
+            __builtin_amdgcn_sched_barrier(0);
+            if (AHEAD)
+            {
+                read_frags(next_stage, I0{}, I0{}); // after the last step: a stage nobody uses any more
+                wait_frags(I1{}, ONE_SET{});
+            }
+            else
+            {
+                wait_frags(I1{}, NONE{});
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            mfmas(I1{});
+            __builtin_amdgcn_sched_barrier(0);
+            stage = next_stage;
         }
+        if (AHEAD)
+            wait_frags(I0{}, NONE{}); // the registers of the last, unused set are free only now
         __builtin_amdgcn_s_waitcnt(vmcnt_imm(0)); // drain the tail loads before the LDS goes away
 
-        // ---- epilogue: D layout of a 32x32 tile: lane (col = l32, h), element e: row = 8*(e/4) + 4*h + (e%4)
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
+        // ---- epilogue -------------------------------------------------------------------------------------
+        // The weight fragment is the MFMA's first operand, so a 32x32 result is D[n][m]: lane (m = l32, h)
+        // holds, in element e, column n = 8*(e/4) + 4*h + (e%4): four consecutive output columns per group
+        // of four elements.
+        const int m_wave = m0 + wm * (TM * 32), n_wave = n0 + wn * (TN * 32);
+        if (RAW || SPLITK)
         {
-            const int n = n0 + wn * (TN * 32) + j * 32 + l32;
-            if (n >= p.N)
-                continue;
-            float sch = 0.f;
-            if (!RAW && !SPLITK)
-                sch = p.s_ch[n];
+            // int32 results: 16 bytes per lane straight from the registers
+            int32_t* out = SPLITK ? p.partial + (size_t)split * p.M * p.N : p.acc;
+            const bool vec = ((p.N & 3) == 0) && ((reinterpret_cast<uintptr_t>(out) & 15) == 0);
 #pragma unroll
             for (int i = 0; i < TM; ++i)
+            {
+                const int m = m_wave + i * 32 + l32;
+                if (m >= p.M)
+                    continue;
+                int32_t* row = out + (size_t)m * p.N;
 #pragma unroll
-                for (int e = 0; e < 16; ++e)
-                {
-                    const int m = m0 + wm * (TM * 32) + i * 32 + 8 * (e >> 2) + 4 * h + (e & 3);
-                    if (m >= p.M)
-                        continue;
-                    if (SPLITK)
-                        p.partial[((size_t)split * p.M + m) * p.N + n] = acc[i][j][e];
-                    else if (RAW)
-                        p.acc[(size_t)m * p.N + n] = acc[i][j][e];
-                    else
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int g = 0; g < 4; ++g)
                     {
-                        float t = (float)acc[i][j][e] * p.s_tok[m];
-                        p.Y[(size_t)m * p.N + n] = f32_to_f16_two_step(t * sch);
+                        const int n = n_wave + j * 32 + 8 * g + 4 * h;
+                        if (vec && n + 3 < p.N)
+                            *reinterpret_cast<intx4*>(row + n) = intx4{acc[i][j][4 * g], acc[i][j][4 * g + 1],
+                                                                       acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+                        else
+                            for (int k = 0; k < 4; ++k)
+                                if (n + k < p.N)
+                                    row[n + k] = acc[i][j][4 * g + k];
                     }
+            }
+            return;
+        }
+        // fp16 results: scaled in registers, turned through a private piece of LDS (the ring is free after
+        // the barrier) and written as whole rows of the wavefront's sub-tile, 16 bytes per lane.
+        constexpr int ROUND_TM = TM >= 2 ? 2 : 1;  // 32-row blocks per pass through LDS
+        constexpr int PITCH = TN * 64 + 16;        // bytes per staged row (padding spreads the banks)
+        constexpr int REGION = ROUND_TM * 32 * PITCH;
+        static_assert(8 * REGION <= T::LDS_BYTES, "the staging regions reuse the ring");
+        constexpr int LANES_PER_ROW = TN * 4, ROWS_PER_READ = 64 / LANES_PER_ROW;
+        __builtin_amdgcn_s_barrier(); // every wavefront has read its last fragments
+        uint8_t* region = smem + wave * REGION;
+        const bool sch_vec = (reinterpret_cast<uintptr_t>(p.s_ch) & 15) == 0;
+        const bool y_vec = ((p.N & 7) == 0) && ((reinterpret_cast<uintptr_t>(p.Y) & 15) == 0);
+#pragma unroll
+        for (int r = 0; r < TM / ROUND_TM; ++r)
+        {
+#pragma unroll
+            for (int ii = 0; ii < ROUND_TM; ++ii)
+            {
+                const int i = r * ROUND_TM + ii;
+                const float st = p.s_tok[min(m_wave + i * 32 + l32, p.M - 1)];
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int g = 0; g < 4; ++g)
+                    {
+                        const int n = n_wave + j * 32 + 8 * g + 4 * h;
+                        float sch[4];
+                        if (sch_vec && n + 3 < p.N)
+                        {
+                            const floatx4 v = *reinterpret_cast<const floatx4*>(p.s_ch + n);
+                            sch[0] = v.x, sch[1] = v.y, sch[2] = v.z, sch[3] = v.w;
+                        }
+                        else
+                        {
+                            for (int k = 0; k < 4; ++k)
+                                sch[k] = p.s_ch[min(n + k, p.N - 1)];
+                        }
+                        half4_t y;
+#pragma unroll
+                        for (int k = 0; k < 4; ++k)
+                        {
+                            const float t = (float)acc[i][j][4 * g + k] * st;
+                            y[k] = f32_to_f16_two_step(t * sch[k]);
+                        }
+                        *reinterpret_cast<half4_t*>(region + (ii * 32 + l32) * PITCH + (j * 32 + 8 * g + 4 * h) * 2) = y;
+                    }
+            }
+            // LDS operations of one wavefront execute in order: no barrier around the private region
+#pragma unroll
+            for (int it = 0; it < ROUND_TM * 32 / ROWS_PER_READ; ++it)
+            {
+                const int row = it * ROWS_PER_READ + lane / LANES_PER_ROW;
+                const int piece = lane % LANES_PER_ROW;
+                const uintx4 v = *reinterpret_cast<const uintx4*>(region + row * PITCH + piece * 16);
+                const int m = m_wave + r * (ROUND_TM * 32) + row;
+                const int n = n_wave + piece * 8;
+                if (m >= p.M || n >= p.N)
+                    continue;
+                half_t* dst = p.Y + (size_t)m * p.N + n;
+                if (y_vec)
+                    *reinterpret_cast<uintx4*>(dst) = v;
+                else
+                {
+                    const half8_t hv = __builtin_bit_cast(half8_t, v);
+                    for (int k = 0; k < 8; ++k)
+                        if (n + k < p.N)
+                            dst[k] = hv[k];
                 }
+            }
         }
     }
 
