@@ -200,7 +200,6 @@ namespace nnf
         }
         int w_frag[TN];
         size_t s_idx[TN];
-        int col_out[TN]; // output column (GATE: of the gate / up pair)
 #pragma unroll
         for (int j = 0; j < TN; ++j)
         {
@@ -211,13 +210,11 @@ namespace nnf
                 r = j * (BN / 2) + c; // j = 0: gate, 1: up
                 gn = j ? (p.up_row_offset + n0 + c) : (n0 + c);
                 gn = min(gn, p.up_row_offset + p.N - 1);
-                col_out[j] = n0 + c;
             }
             else
             {
                 r = wn * (TN * 32) + j * 32 + l32;
                 gn = min(n0 + r, p.N - 1);
-                col_out[j] = n0 + r;
             }
             w_frag[j] = A_TILE_BYTES + r * 32 + ((h ^ ((r >> 3) & 1)) << 4);
             s_idx[j] = (size_t)gn * G + g_begin;
@@ -285,7 +282,7 @@ namespace nnf
                     half8_t bf = __builtin_bit_cast(half8_t, uintx4{bw[0], bw[1], bw[2], bw[3]});
 #pragma unroll
                     for (int i = 0; i < TM; ++i)
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf, acc[i][j], 0, 0, 0);
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf, af[i], acc[i][j], 0, 0, 0);
                 }
             }
         };
@@ -329,64 +326,129 @@ namespace nnf
         __builtin_amdgcn_s_waitcnt(vmcnt_imm(0)); // drain the tail loads before the LDS goes away
 
         // ---- epilogue ---------------------------------------------------------------------------------
-        // D layout of a 32x32 tile: lane (col = l32, h), element e: row = 8*(e/4) + 4*h + (e%4)
+        // The weight fragment is the MFMA's first operand, so a 32x32 result is D[n][m]: lane (m = l32, h)
+        // holds, in element e, column n = 8*(e/4) + 4*h + (e%4) of its weight tile: four consecutive
+        // columns per group of four elements.
+        const int m_wave = m0 + wm * (TM * 32);
         if (SPLITK)
         {
+            // fp32 partial sums: 16 bytes per lane straight from the registers
             float* part = p.partial + (size_t)split * p.M * p.ld_partial;
+            const bool vec = ((p.N & 3) == 0) && ((p.ld_partial & 3) == 0) && ((reinterpret_cast<uintptr_t>(part) & 15) == 0);
 #pragma unroll
-            for (int j = 0; j < TN; ++j)
+            for (int i = 0; i < TM; ++i)
             {
-                if (col_out[j] >= p.N)
+                const int m = m_wave + i * 32 + l32;
+                if (m >= p.M)
                     continue;
-                const int pc = (GATE && j == 1) ? p.N + col_out[j] : col_out[j];
+                float* row = part + (size_t)m * p.ld_partial;
 #pragma unroll
-                for (int i = 0; i < TM; ++i)
+                for (int j = 0; j < TN; ++j)
 #pragma unroll
-                    for (int e = 0; e < 16; ++e)
+                    for (int g = 0; g < 4; ++g)
                     {
-                        const int m = m0 + wm * (TM * 32) + i * 32 + 8 * (e >> 2) + 4 * h + (e & 3);
-                        if (m < p.M)
-                            part[(size_t)m * p.ld_partial + pc] = acc[i][j][e];
+                        // column of the output (GATE: of the gate / up pair); up columns follow the N gate columns
+                        const int n = GATE ? n0 + wn * 32 + 8 * g + 4 * h : n0 + wn * (TN * 32) + j * 32 + 8 * g + 4 * h;
+                        float* dst = row + ((GATE && j == 1) ? p.N + n : n);
+                        if (vec && n + 3 < p.N)
+                            *reinterpret_cast<floatx4*>(dst) = floatx4{acc[i][j][4 * g], acc[i][j][4 * g + 1],
+                                                                       acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+                        else
+                            for (int k = 0; k < 4; ++k)
+                                if (n + k < p.N)
+                                    dst[k] = acc[i][j][4 * g + k];
                     }
             }
             return;
         }
-        constexpr int NJ = GATE ? 1 : TN;
-#pragma unroll
-        for (int j = 0; j < NJ; ++j)
+        // fp16 results: rounded (GATE: combined) in registers, turned through a private piece of LDS (the
+        // ring is free after the barrier) and finished as whole rows of the wavefront's sub-tile, 16 bytes
+        // (8 columns) per lane: bias, residual and the store.
+        constexpr int OUT_TN = GATE ? 1 : TN;
+        constexpr int ROUND_TM = TM >= 2 ? 2 : 1;      // 32-row blocks per pass through LDS
+        constexpr int PITCH = OUT_TN * 64 + 16;        // bytes per staged row (padding spreads the banks)
+        constexpr int REGION = ROUND_TM * 32 * PITCH;
+        static_assert(8 * REGION <= T::LDS_BYTES, "the staging regions reuse the ring");
+        constexpr int LANES_PER_ROW = OUT_TN * 4, ROWS_PER_READ = 64 / LANES_PER_ROW;
+        __builtin_amdgcn_s_barrier(); // every wavefront has read its last fragments
+        uint8_t* region = smem + wave * REGION;
+        const int n_wave = GATE ? n0 + wn * 32 : n0 + wn * (TN * 32);
+        const int piece = lane % LANES_PER_ROW;
+        const int n_lane = n_wave + piece * 8; // first of this lane's 8 columns in the row phase
+        bool vec = ((p.N & 7) == 0) && ((p.ldy & 7) == 0) && ((reinterpret_cast<uintptr_t>(p.Y) & 15) == 0);
+        if (RESID)
+            vec = vec && ((reinterpret_cast<uintptr_t>(p.residual) & 15) == 0);
+        float bias[8];
+        if (BIAS)
         {
-            const int n = col_out[j];
-            if (n >= p.N)
-                continue;
-            float bias = 0.f;
-            if (BIAS)
-                bias = (float)p.bias[n];
 #pragma unroll
-            for (int i = 0; i < TM; ++i)
+            for (int k = 0; k < 8; ++k)
+                bias[k] = (float)p.bias[min(n_lane + k, p.N - 1)];
+        }
+#pragma unroll
+        for (int r = 0; r < TM / ROUND_TM; ++r)
+        {
+#pragma unroll
+            for (int ii = 0; ii < ROUND_TM; ++ii)
             {
+                const int i = r * ROUND_TM + ii;
 #pragma unroll
-                for (int e = 0; e < 16; ++e)
+                for (int j = 0; j < OUT_TN; ++j)
+#pragma unroll
+                    for (int g = 0; g < 4; ++g)
+                    {
+                        half4_t y;
+#pragma unroll
+                        for (int k = 0; k < 4; ++k)
+                        {
+                            if (GATE)
+                            {
+                                const float gt = (float)(half_t)acc[i][0][4 * g + k];
+                                const float up = (float)(half_t)acc[i][1][4 * g + k];
+                                y[k] = (half_t)(gt * (1.0f / (1.0f + __expf(-gt))) * up);
+                            }
+                            else
+                            {
+                                y[k] = (half_t)acc[i][j][4 * g + k];
+                            }
+                        }
+                        *reinterpret_cast<half4_t*>(region + (ii * 32 + l32) * PITCH + (j * 32 + 8 * g + 4 * h) * 2) = y;
+                    }
+            }
+            // LDS operations of one wavefront execute in order: no barrier around the private region
+#pragma unroll
+            for (int it = 0; it < ROUND_TM * 32 / ROWS_PER_READ; ++it)
+            {
+                const int row = it * ROWS_PER_READ + lane / LANES_PER_ROW;
+                half8_t v = *reinterpret_cast<const half8_t*>(region + row * PITCH + piece * 16);
+                const int m = m_wave + r * (ROUND_TM * 32) + row;
+                if (m >= p.M || n_lane >= p.N)
+                    continue;
+                const size_t at = (size_t)m * p.ldy + n_lane;
+                if (BIAS)
                 {
-                    const int m = m0 + wm * (TM * 32) + i * 32 + 8 * (e >> 2) + 4 * h + (e & 3);
-                    if (m >= p.M)
-                        continue;
-                    float v;
-                    if (GATE)
-                    {
-                        float g = (float)(half_t)acc[i][0][e];
-                        float u = (float)(half_t)acc[i][1][e];
-                        v = g * (1.0f / (1.0f + __expf(-g))) * u;
-                    }
-                    else
-                    {
-                        v = acc[i][j][e];
-                    }
-                    if (BIAS)
-                        v = (float)(half_t)v + bias;
-                    if (RESID)
-                        v = (float)(half_t)v + (float)p.residual[(size_t)m * p.ldy + n];
-                    p.Y[(size_t)m * p.ldy + n] = (half_t)v;
+#pragma unroll
+                    for (int k = 0; k < 8; ++k)
+                        v[k] = (half_t)((float)v[k] + bias[k]);
                 }
+                if (RESID)
+                {
+                    half8_t res;
+                    if (vec)
+                        res = *reinterpret_cast<const half8_t*>(p.residual + at);
+                    else
+                        for (int k = 0; k < 8; ++k)
+                            res[k] = p.residual[n_lane + k < p.N ? at + k : at];
+#pragma unroll
+                    for (int k = 0; k < 8; ++k)
+                        v[k] = (half_t)((float)v[k] + (float)res[k]);
+                }
+                if (vec)
+                    *reinterpret_cast<half8_t*>(p.Y + at) = v;
+                else
+                    for (int k = 0; k < 8; ++k)
+                        if (n_lane + k < p.N)
+                            p.Y[at + k] = v[k];
             }
         }
     }
