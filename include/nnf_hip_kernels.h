@@ -71,6 +71,27 @@ int nnf_w4a16_gemm(nnf_stream_t stream,
                    int M, int N, int K, int group, int zp,
                    void* workspace, size_t workspace_bytes);
 
+/* The kernels behind nnf_w4a16_gemm as separate, selectable variants: what several registered emitters
+ * for one operator are to ProfilingBasedKernelSelector::profiling_best
+ * (engine/pass/graph/kernel_selection.cpp:21-73), which times every emitter that accepts the node and keeps
+ * the fastest.  NNF_W4A16_AUTO is nnf_w4a16_gemm itself (a built-in choice by shape). */
+enum nnf_w4a16_variant
+{
+    NNF_W4A16_AUTO = 0,
+    NNF_W4A16_GEMV_VALU = 1, /* M <= 16: v_dot2 GEMV, exact (q - zp) unpacking; cross-check implementation */
+    NNF_W4A16_GEMV_MFMA = 2, /* M <= 16: MFMA 16x16x32 weight-streaming kernel (activations held per workgroup) */
+    NNF_W4A16_GEMM_MFMA = 3, /* any M: MFMA 32x32x16 tile GEMM (may split K: workspace) */
+    NNF_W4A16_GEMV_ROWS = 4  /* M = 1: row-streaming GEMV */
+};
+/* 1 when the variant can serve the shape (decided on the host, for a 256-CU device), else 0. */
+int nnf_w4a16_variant_supported(int M, int N, int K, int group, int variant);
+size_t nnf_w4a16_gemm_variant_workspace_bytes(int M, int N, int K, int group, int variant);
+/* As nnf_w4a16_gemm through the given variant; NNF_ERR_UNSUPPORTED_SHAPE when it cannot serve the shape. */
+int nnf_w4a16_gemm_variant(nnf_stream_t stream,
+                           const void* A, const void* Wq, const void* scales, void* Y,
+                           int M, int N, int K, int group, int zp, int variant,
+                           void* workspace, size_t workspace_bytes);
+
 /* Epilogue / prologue selectors for nnf_w4a16_gemm_fused. */
 enum nnf_activation
 {

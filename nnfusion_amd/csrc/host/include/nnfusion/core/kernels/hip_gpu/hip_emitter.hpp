@@ -19,6 +19,11 @@ namespace nnfusion
                     : KernelEmitter(ctx, "rocm")
                 {
                 }
+                // kernel_type tells apart several emitters of one operator (it is part of the function name)
+                HipLibEmitter(std::shared_ptr<KernelContext> ctx, const std::string& kernel_type)
+                    : KernelEmitter(ctx, kernel_type)
+                {
+                }
                 bool is_static_function() override { return false; }
 
             protected:

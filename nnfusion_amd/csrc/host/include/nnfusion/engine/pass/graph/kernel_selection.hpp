@@ -4,6 +4,9 @@
 #pragma once
 
 #include "nnfusion/core/kernels/kernel_registration.hpp"
+#include "nnfusion/engine/profiler/hip_runtime.hpp"
+
+#include <map>
 
 namespace nnfusion
 {
@@ -38,6 +41,44 @@ namespace nnfusion
                 bool register_custom_kernel(const std::string& op_name, NNFusion_DeviceType devtype);
                 // stores the winner under the tag "Kernel_Selection_Result"; nodes already tagged are kept
                 bool run_on_graph(std::shared_ptr<nnfusion::graph::Graph>& graph);
+            };
+
+            // ProfilingBasedKernelSelector (src/nnfusion/engine/pass/graph/kernel_selection.cpp:21-137): for the
+            // operators of a white list, every registered emitter that accepts the node is run through the
+            // single-kernel harness and the fastest is stored as "Kernel_Selection_Result", which
+            // DefaultKernelSelector then keeps.  The reference's white list is {"Broadcast"}; here it is
+            // {"QuantDot"}, whose emitters are the automatic one and the four kernel variants.
+            class ProfilingBasedKernelSelector
+            {
+            public:
+                using Result = DefaultKernelSelector::Result;
+                struct Timing
+                {
+                    std::string kernel_type;
+                    double ms; // mean of runtime_times runs; < 0: failed to compile or run
+                };
+                bool enable = true; // the reference's -fkernel_selection
+                size_t warmup_times = 5, runtime_times = 100;
+                std::string working_dir = "./kernel_profiling/";
+
+                // every registered emitter of the node's operator (ROCM_GPU: CUDA_GPU registrations too) that emits for it
+                std::vector<kernels::KernelEmitter::Pointer> candidates(std::shared_ptr<nnfusion::graph::GNode> gnode,
+                                                                        NNFusion_DeviceType devtype);
+                // harness contexts of the candidates, sources generated (no compiler, no device)
+                std::vector<profiler::ProfilingContext::Pointer> contexts(std::shared_ptr<nnfusion::graph::GNode> gnode,
+                                                                          NNFusion_DeviceType devtype,
+                                                                          profiler::HipDefaultRuntime& runtime);
+                // Compiles and runs every candidate on deterministic pseudo-random inputs; second == nullptr if
+                // fewer than two candidates exist (nothing to choose) or none ran.  timings (optional): one entry
+                // per candidate; outputs (optional): the first output blob of every candidate that ran.
+                Result profiling_best(std::shared_ptr<nnfusion::graph::GNode> gnode, NNFusion_DeviceType devtype,
+                                      profiler::HipDefaultRuntime& runtime, std::vector<Timing>* timings = nullptr,
+                                      std::vector<std::vector<uint8_t>>* outputs = nullptr);
+                // nodes of equal identifier (operator, shapes, types) are profiled once
+                bool run_on_graph(std::shared_ptr<nnfusion::graph::Graph>& graph, profiler::HipDefaultRuntime& runtime);
+
+            private:
+                std::map<std::string, std::string> m_best_type; // identifier -> kernel type of the winner
             };
         } // namespace graph
     } // namespace pass

@@ -9,6 +9,7 @@
 #include <cstdlib>
 #include <dlfcn.h>
 #include <fstream>
+#include <iterator>
 #include <sys/stat.h>
 #include <unistd.h>
 
@@ -126,6 +127,17 @@ namespace nnfusion
             mkdir(dir.c_str(), 0755);
             ke->source_path = dir + ke->entry_name + ".cpp";
             ke->object_path = dir + "lib" + ke->entry_name + ".so";
+            {
+                // an object built earlier from the same source (e.g. ahead of time, on a host without the
+                // device) is kept
+                std::ifstream old_src(ke->source_path);
+                if (old_src.is_open())
+                {
+                    std::string old_text((std::istreambuf_iterator<char>(old_src)), std::istreambuf_iterator<char>());
+                    if (old_text == ke->source_code && access(ke->object_path.c_str(), R_OK) == 0)
+                        return true;
+                }
+            }
             {
                 std::ofstream f(ke->source_path, std::ios::trunc);
                 if (!f.good())

@@ -99,6 +99,66 @@ namespace nnfusion
                 }
             };
 
+            // One kernel variant of the plain fp16 x int4 product (no fused prologue / epilogue): the emitters
+            // that ProfilingBasedKernelSelector times against the automatic one.  A variant that cannot serve
+            // the node's shape declines it.
+            template <int VARIANT>
+            class QuantDotVariant : public HipLibEmitter
+            {
+            public:
+                explicit QuantDotVariant(std::shared_ptr<KernelContext> ctx)
+                    : HipLibEmitter(ctx, std::string("rocm_") + variant_name())
+                {
+                }
+                static const char* variant_name()
+                {
+                    return VARIANT == 1 ? "gemv_valu" : VARIANT == 2 ? "gemv_mfma" : VARIANT == 3 ? "gemm_mfma" : "gemv_rows";
+                }
+                static const char* variant_enum()
+                {
+                    return VARIANT == 1 ? "NNF_W4A16_GEMV_VALU"
+                                        : VARIANT == 2 ? "NNF_W4A16_GEMV_MFMA"
+                                                       : VARIANT == 3 ? "NNF_W4A16_GEMM_MFMA" : "NNF_W4A16_GEMV_ROWS";
+                }
+
+                LanguageUnit_p emit_function_body() override
+                {
+                    auto gop = std::dynamic_pointer_cast<op::GenericOp>(m_context->op);
+                    if (!gop)
+                        return nullptr;
+                    auto& cfg = gop->localOpConfig.getRoot();
+                    const int group = cfg["group_size"].get<int>();
+                    const int zp = cfg["zero_point"].get<int>();
+                    if (cfg["rms_norm"].get<bool>() || cfg["has_bias"].get<bool>() || cfg["has_residual"].get<bool>() ||
+                        cfg["act"].get<std::string>() == "silu_gate")
+                        return nullptr;
+                    if (cfg["bits"].get<int>() != 4 || group != 128 || !cfg["transpose_B"].get<bool>())
+                        return nullptr;
+                    if (m_context->inputs[0]->get_element_type() != element::f16 ||
+                        m_context->inputs[2]->get_element_type() != element::f16)
+                        return nullptr;
+                    const Shape& a = m_context->inputs[0]->get_shape();
+                    const Shape& w = m_context->inputs[1]->get_shape();
+                    const size_t K = a.back();
+                    const size_t M = shape_size(a) / K;
+                    const size_t N = w[0];
+                    if (!nnf::workspace::w4a16_variant_fits((int)M, (int)N, (int)K, VARIANT))
+                        return nullptr;
+                    size_t ws_bytes = 0;
+                    if (VARIANT == 3)
+                        ws_bytes = nnf::workspace::gemm_partial_bytes(
+                            (int)M, (int)N, false, nnf::workspace::plan_w4a16_gemm((int)M, (int)N, (int)K, false));
+                    std::string ws = "nullptr";
+                    if (ws_bytes > 0)
+                        ws = allocate_tensor(Shape{ws_bytes}, element::character)->get_name();
+                    LanguageUnit_p lu(new LanguageUnit(get_function_name()));
+                    *lu << "NNF_HIP_CHECK(nnf_w4a16_gemm_variant(stream, input0, input1, input2, output0, " << M << ", " << N
+                        << ", " << K << ", " << group << ", " << zp << ", " << variant_enum() << ", " << ws << ", "
+                        << ws_bytes << "));\n";
+                    return lu;
+                }
+            };
+
             class QuantDotW8A8 : public HipLibEmitter
             {
             public:
@@ -209,6 +269,20 @@ namespace nnfusion
         REGISTER_KERNEL_EMITTER("QuantDot",
                                 Device(ROCM_GPU).TypeConstraint(element::f32).Tag("nnf_hip_gfx950").Priority(5),
                                 hip::QuantDot)
+        // the variants rank below the automatic emitter (DefaultKernelSelector keeps picking that one) and above
+        // the reference's Dot emitters
+        REGISTER_KERNEL_EMITTER("QuantDot",
+                                Device(ROCM_GPU).TypeConstraint(element::f32).Tag("nnf_hip_gfx950_gemv_rows").Priority(3),
+                                hip::QuantDotVariant<4>)
+        REGISTER_KERNEL_EMITTER("QuantDot",
+                                Device(ROCM_GPU).TypeConstraint(element::f32).Tag("nnf_hip_gfx950_gemv_mfma").Priority(3),
+                                hip::QuantDotVariant<2>)
+        REGISTER_KERNEL_EMITTER("QuantDot",
+                                Device(ROCM_GPU).TypeConstraint(element::f32).Tag("nnf_hip_gfx950_gemm_mfma").Priority(3),
+                                hip::QuantDotVariant<3>)
+        REGISTER_KERNEL_EMITTER("QuantDot",
+                                Device(ROCM_GPU).TypeConstraint(element::f32).Tag("nnf_hip_gfx950_gemv_valu").Priority(3),
+                                hip::QuantDotVariant<1>)
         REGISTER_KERNEL_EMITTER("QuantDotW8A8",
                                 Device(ROCM_GPU).TypeConstraint(element::f32).Tag("nnf_hip_gfx950").Priority(5),
                                 hip::QuantDotW8A8)

@@ -3,6 +3,8 @@
 #include "nnfusion/core/operators/generic_op/generic_op.hpp"
 #include "nnfusion/engine/pass/graph/kernel_selection.hpp"
 
+#include <algorithm>
+
 namespace nnfusion
 {
     namespace pass
@@ -142,6 +144,148 @@ namespace nnfusion
                     auto ans = pick_first(node, dev);
                     if (ans.second != nullptr)
                         (*node)["Kernel_Selection_Result"] = ans;
+                }
+                return true;
+            }
+
+            // ---- ProfilingBasedKernelSelector -----------------------------------------------------------------
+            std::vector<KernelEmitter::Pointer>
+                ProfilingBasedKernelSelector::candidates(std::shared_ptr<nnfusion::graph::GNode> gnode,
+                                                         NNFusion_DeviceType devtype)
+            {
+                std::vector<KernelEmitter::Pointer> out;
+                if (gnode->is_constant() || gnode->is_parameter() || gnode->is_output())
+                    return out;
+                auto regs = KernelRegistry::Global()->FindKernelRegistrations(gnode->get_op_type(), devtype, element::f32);
+                if (devtype == ROCM_GPU)
+                    for (auto& r : KernelRegistry::Global()->FindKernelRegistrations(gnode->get_op_type(), CUDA_GPU, element::f32))
+                        regs.push_back(r);
+                std::stable_sort(regs.begin(), regs.end(),
+                                 [](const std::shared_ptr<const KernelRegistration>& x,
+                                    const std::shared_ptr<const KernelRegistration>& y) { return x->m_priority > y->m_priority; });
+                for (auto& r : regs)
+                {
+                    std::shared_ptr<KernelContext> ctx(new KernelContext(gnode)); // emitters may add scratch tensors
+                    auto kernel = r->m_factory(ctx);
+                    if (kernel->get_or_emit_source())
+                        out.push_back(kernel);
+                }
+                return out;
+            }
+
+            std::vector<profiler::ProfilingContext::Pointer>
+                ProfilingBasedKernelSelector::contexts(std::shared_ptr<nnfusion::graph::GNode> gnode,
+                                                       NNFusion_DeviceType devtype, profiler::HipDefaultRuntime& runtime)
+            {
+                std::vector<profiler::ProfilingContext::Pointer> out;
+                for (auto& k : candidates(gnode, devtype))
+                {
+                    auto pc = std::make_shared<profiler::ProfilingContext>(k);
+                    pc->warmup_times = warmup_times;
+                    pc->runtime_times = runtime_times;
+                    pc->working_dir = working_dir;
+                    if (runtime.codegen(pc))
+                        out.push_back(pc);
+                }
+                return out;
+            }
+
+            namespace
+            {
+                // deterministic bytes; fp16 tensors get finite values of magnitude below two
+                void fill_blob(std::vector<uint8_t>& blob, const element::Type& type, uint64_t seed)
+                {
+                    uint64_t x = seed * 0x9E3779B97F4A7C15ull + 0x2545F4914F6CDD1Dull;
+                    for (size_t i = 0; i + 1 < blob.size() + 1; i += 2)
+                    {
+                        x ^= x << 13, x ^= x >> 7, x ^= x << 17;
+                        uint16_t v = (uint16_t)(x >> 24);
+                        if (type == element::f16)
+                            v &= 0xBBFF;
+                        else if (type == element::f32)
+                            v = (i & 2) ? (uint16_t)(0x3A00 | (v & 0x80FF)) : v; // high half: sign, exponent ~2^-11
+                        blob[i] = (uint8_t)v;
+                        if (i + 1 < blob.size())
+                            blob[i + 1] = (uint8_t)(v >> 8);
+                    }
+                }
+            } // namespace
+
+            ProfilingBasedKernelSelector::Result
+                ProfilingBasedKernelSelector::profiling_best(std::shared_ptr<nnfusion::graph::GNode> gnode,
+                                                             NNFusion_DeviceType devtype, profiler::HipDefaultRuntime& runtime,
+                                                             std::vector<Timing>* timings,
+                                                             std::vector<std::vector<uint8_t>>* outputs)
+            {
+                auto pcs = contexts(gnode, devtype, runtime);
+                // nothing to choose between (the reference skips nodes with a single registration)
+                if (pcs.size() < 2)
+                    return std::make_pair(devtype, KernelEmitter::Pointer());
+                KernelEmitter::Pointer best;
+                double best_ms = -1.0;
+                for (auto& pc : pcs)
+                {
+                    auto& ctx = pc->kernel->m_context;
+                    std::vector<std::vector<uint8_t>> in(ctx->inputs.size()), out(ctx->outputs.size());
+                    std::vector<void*> in_p, out_p;
+                    for (size_t i = 0; i < in.size(); ++i)
+                    {
+                        in[i].resize(std::max<size_t>(ctx->inputs[i]->size(), 2));
+                        fill_blob(in[i], ctx->inputs[i]->get_element_type(), i + 1);
+                        in_p.push_back(in[i].data());
+                    }
+                    for (size_t i = 0; i < out.size(); ++i)
+                    {
+                        out[i].assign(std::max<size_t>(ctx->outputs[i]->size(), 2), 0);
+                        out_p.push_back(out[i].data());
+                    }
+                    const double ms = runtime.execute(pc, in_p.data(), out_p.data());
+                    NNFUSION_LOG(INFO) << "Kernel Emitter " << pc->kernel->get_kernel_type() << " time cost(ms): " << ms;
+                    if (timings)
+                        timings->push_back(Timing{pc->kernel->get_kernel_type(), ms});
+                    if (ms < 0)
+                        continue;
+                    if (outputs && !out.empty())
+                        outputs->push_back(out[0]);
+                    if (best_ms < 0 || ms < best_ms)
+                    {
+                        best_ms = ms;
+                        best = pc->kernel;
+                    }
+                }
+                return std::make_pair(devtype, best);
+            }
+
+            bool ProfilingBasedKernelSelector::run_on_graph(std::shared_ptr<nnfusion::graph::Graph>& graph,
+                                                            profiler::HipDefaultRuntime& runtime)
+            {
+                if (!enable)
+                    return true;
+                static const std::vector<std::string> white_list{"QuantDot"};
+                for (auto& node : graph->get_nodes())
+                {
+                    if (std::find(white_list.begin(), white_list.end(), node->get_op_type()) == white_list.end())
+                        continue;
+                    NNFUSION_CHECK((*node)["DeviceType"].is_valid())
+                        << "GNode DeviceType should be assigned before this pass: " << node->get_name();
+                    auto dev = (*node)["DeviceType"].as<NNFusion_DeviceType>();
+                    if (dev != ROCM_GPU)
+                        continue;
+                    const std::string id = KernelContext(node).generate_identifier();
+                    auto known = m_best_type.find(id);
+                    if (known != m_best_type.end())
+                    {
+                        for (auto& k : candidates(node, dev))
+                            if (k->get_kernel_type() == known->second)
+                                (*node)["Kernel_Selection_Result"] = std::make_pair(dev, k);
+                        continue;
+                    }
+                    auto ans = profiling_best(node, dev, runtime);
+                    if (ans.second != nullptr)
+                    {
+                        m_best_type[id] = ans.second->get_kernel_type();
+                        (*node)["Kernel_Selection_Result"] = ans;
+                    }
                 }
                 return true;
             }

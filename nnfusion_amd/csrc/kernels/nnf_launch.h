@@ -35,10 +35,12 @@ namespace nnf
     // MFMA GEMM (any M) with the RMSNorm prologue and bias / residual / SiLU-gate epilogues.
     // rms_ws: nnf::workspace::rms_rows(M, K) bytes, needed when rms_gamma != nullptr;
     // partial_ws: nnf::workspace::gemm_partial_bytes(...) for the plan of the shape (may be 0 bytes).
-    // M <= 16 shapes that the GEMV kernel can serve go through it (plus an element-wise epilogue kernel).
+    // M <= 16 shapes that the GEMV kernel can serve go through it (plus an element-wise epilogue kernel),
+    // unless gemm_only asks for the MFMA GEMM tiles whatever M is.
     hipError_t launch_w4a16_gemm(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M,
                                  int N, int K, int zp, const void* rms_gamma, float rms_eps, const void* bias,
-                                 const void* residual, int act, void* rms_ws, void* partial_ws, int num_cu);
+                                 const void* residual, int act, void* rms_ws, void* partial_ws, int num_cu,
+                                 bool gemm_only = false);
 
     // W8A8: acc != nullptr writes the raw int32 accumulators, otherwise Y = fp16(acc * s_tok * s_ch).
     // partial_ws: nnf::workspace::w8a8_gemm(M, N, K) bytes (0 for the M <= 16 kernel)

@@ -238,8 +238,10 @@ namespace nnf
 
     hipError_t launch_w4a16_gemm(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M,
                                  int N, int K, int zp, const void* rms_gamma, float rms_eps, const void* bias,
-                                 const void* residual, int act, void* rms_ws, void* partial_ws, int num_cu)
+                                 const void* residual, int act, void* rms_ws, void* partial_ws, int num_cu,
+                                 bool gemm_only)
     {
+        gemm_only = gemm_only || g_tuning.force_path == 3;
         const bool rms = rms_gamma != nullptr, hb = bias != nullptr, hr = residual != nullptr, gate = act == 1;
         // the combinations the fused entry points use; anything else is composed by the caller
         if (gate && (hb || hr))
@@ -261,7 +263,7 @@ namespace nnf
         // the products go to scratch first when the epilogue cannot work in place: the [M, 2N] gate | up pair, or a
         // residual that is the output buffer itself
         const bool via_scratch = gate || (hr && residual == Y);
-        if (g_tuning.force_path != 3 && M <= 16 && w4a16_skinny_supported(M, n_rows, K) && (!via_scratch || partial_ws))
+        if (!gemm_only && M <= 16 && w4a16_skinny_supported(M, n_rows, K) && (!via_scratch || partial_ws))
         {
             void* y_gemv = via_scratch ? partial_ws : Y;
             // one activation row: the row-streaming kernel where it applies
@@ -282,7 +284,7 @@ namespace nnf
         }
         // M <= 16 with too many activations for one workgroup's LDS: the GEMV kernel over ranges of K, then the
         // reduction pass (which applies the epilogue)
-        const int ksplits = (g_tuning.force_path != 3 && partial_ws) ? w4a16_skinny_ksplits(M, n_rows, K) : 0;
+        const int ksplits = (!gemm_only && partial_ws) ? w4a16_skinny_ksplits(M, n_rows, K) : 0;
         if (ksplits > 0)
         {
             hipError_t e = launch_w4a16_skinny_split(stream, A, Wq, S, (float*)partial_ws, M, n_rows, K, zp, ksplits, num_cu);

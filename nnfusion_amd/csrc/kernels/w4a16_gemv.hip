@@ -9,6 +9,8 @@
 #include "nnf_device.h"
 #include "nnf_launch.h"
 
+#include "../nnf_workspace.h"
+
 namespace nnf
 {
     // LDS layout of the staged activations: 16-byte slots; slot(m, c, j, l) = ((m*C + c)*4 + j)*64 + l
@@ -122,9 +124,7 @@ namespace nnf
 
     bool w4a16_gemv_supported(int M, int K)
     {
-        int mb = M >= 4 ? 4 : M;
-        size_t lds = (size_t)mb * ((K + 2047) >> 11) * 4 * 64 * 16;
-        return (K % 32) == 0 && lds <= MAX_LDS_BYTES;
+        return workspace::w4a16_gemv_valu_fits(M, K);
     }
 
     // M rows are processed in passes of 4/2/1 rows (each pass re-reads the weights; the MFMA

@@ -144,6 +144,59 @@ int nnf_w4a16_gemm(nnf_stream_t stream, const void* A, const void* Wq, const voi
                                        nullptr, NNF_ACT_NONE, nullptr, workspace, dev.num_cu);
 }
 
+int nnf_w4a16_variant_supported(int M, int N, int K, int group, int variant)
+{
+    return (group == 128 && nnf::workspace::w4a16_variant_fits(M, N, K, variant)) ? 1 : 0;
+}
+
+size_t nnf_w4a16_gemm_variant_workspace_bytes(int M, int N, int K, int group, int variant)
+{
+    if (M <= 0 || N <= 0 || K < 128)
+        return 0;
+    if (variant == NNF_W4A16_GEMM_MFMA)
+        return nnf::workspace::gemm_partial_bytes(M, N, false, nnf::workspace::plan_w4a16_gemm(M, N, K, false));
+    if (variant == NNF_W4A16_AUTO)
+        return nnf::workspace::w4a16_gemm(M, N, K, group);
+    return 0;
+}
+
+int nnf_w4a16_gemm_variant(nnf_stream_t stream, const void* A, const void* Wq, const void* scales, void* Y, int M,
+                           int N, int K, int group, int zp, int variant, void* workspace, size_t workspace_bytes)
+{
+    if (variant == NNF_W4A16_AUTO)
+        return nnf_w4a16_gemm(stream, A, Wq, scales, Y, M, N, K, group, zp, workspace, workspace_bytes);
+    int st = check_w4a16(A, Wq, scales, Y, M, N, K, group, zp);
+    if (st != NNF_OK)
+        return st;
+    if (variant < NNF_W4A16_AUTO || variant > NNF_W4A16_GEMV_ROWS)
+        return NNF_ERR_INVALID_ARGUMENT;
+    DeviceInfo dev;
+    st = current_device_info(dev);
+    if (st != NNF_OK)
+        return st;
+    switch (variant)
+    {
+    case NNF_W4A16_GEMV_ROWS:
+        if (!nnf::w4a16_gemv_rows_supported(M, N, K, dev.num_cu))
+            return NNF_ERR_UNSUPPORTED_SHAPE;
+        return (int)nnf::launch_w4a16_gemv_rows((hipStream_t)stream, A, Wq, scales, Y, N, K, zp, dev.num_cu);
+    case NNF_W4A16_GEMV_MFMA:
+        if (!nnf::workspace::w4a16_skinny_fits(M, N, K))
+            return NNF_ERR_UNSUPPORTED_SHAPE;
+        return (int)nnf::launch_w4a16_skinny((hipStream_t)stream, A, Wq, scales, Y, M, N, K, zp, dev.num_cu);
+    case NNF_W4A16_GEMV_VALU:
+        if (M > 16 || !nnf::w4a16_gemv_supported(M, K))
+            return NNF_ERR_UNSUPPORTED_SHAPE;
+        return (int)nnf::launch_w4a16_gemv((hipStream_t)stream, A, Wq, scales, Y, M, N, K, zp, dev.num_cu);
+    default: break;
+    }
+    const size_t need = nnf_w4a16_gemm_variant_workspace_bytes(M, N, K, group, NNF_W4A16_GEMM_MFMA);
+    if (need > 0 && (!workspace || !aligned16(workspace) || workspace_bytes < need))
+        return NNF_ERR_WORKSPACE_TOO_SMALL;
+    return (int)nnf::launch_w4a16_gemm((hipStream_t)stream, A, Wq, scales, Y, M, N, K, zp, nullptr, 0.f, nullptr,
+                                       nullptr, NNF_ACT_NONE, nullptr, workspace, dev.num_cu, true);
+}
+
 size_t nnf_w4a16_gemm_fused_workspace_bytes(int M, int N, int K, int group, int act)
 {
     // room for the normalised activations of the RMSNorm prologue whether or not the call uses it

@@ -206,6 +206,17 @@ namespace nnf
             return s ? align256((size_t)s * M * N_total * sizeof(float)) : 0;
         }
 
+        // ---- the VALU GEMV (w4a16_gemv.hip): up to four activation rows of K staged in LDS ----
+        inline bool w4a16_gemv_valu_fits(int M, int K)
+        {
+            if (M < 1 || M > 16 || K < 32 || (K % 32) != 0)
+                return false;
+            const int mb = M >= 4 ? 4 : M;
+            return (size_t)mb * ((K + 2047) >> 11) * 4 * 64 * 16 <= LDS_BYTES_PER_CU;
+        }
+        // ---- which kernel variants of the fp16 x int4 product can serve a shape (values of nnf_w4a16_variant) ----
+        inline bool w4a16_variant_fits(int M, int N, int K, int variant, int num_cu = PLAN_CUS);
+
         // ---- one activation row: the row-streaming GEMV (w4a16_gemv_rows.hip) ----
         // Eight wavefronts per workgroup (one workgroup per CU) measured fastest: sixteen pay the per-wavefront
         // parts of the kernel twice as often, four leave the vector units idle between dependent instructions.
@@ -317,6 +328,21 @@ namespace nnf
                 return false;
             const Q8SkinnyPlan pl = plan_w8a8_skinny(M, K);
             return pl.cps != 0 && pl.lds + 16 * 1024 <= LDS_BYTES_PER_CU;
+        }
+        inline bool w4a16_variant_fits(int M, int N, int K, int variant, int num_cu)
+        {
+            if (M <= 0 || N <= 0 || K < 128 || (K & 127))
+                return false;
+            switch (variant)
+            {
+            case 0: // automatic
+            case 3: // MFMA tile GEMM
+                return true;
+            case 1: return w4a16_gemv_valu_fits(M, K);
+            case 2: return w4a16_skinny_fits(M, N, K);
+            case 4: return plan_w4a16_rows(M, N, K, num_cu, 0).seg != 0;
+            default: return false;
+            }
         }
         // ---- W8A8, one activation row: the row-streaming GEMV (w8a8_gemv_rows.hip) ----
         struct Q8RowsPlan

@@ -11,6 +11,8 @@
 #include "nnfusion/engine/pass/graph/quant_fusion_pass.hpp"
 #include "nnfusion/engine/profiler/hip_runtime.hpp"
 
+#include <algorithm>
+
 #include "../../nnfusion_amd/csrc/nnf_workspace.h"
 
 #include <cstdio>
@@ -206,7 +208,10 @@ int main(int argc, char** argv)
         EXPECT(reg->FindKernelRegistrations("NoSuchOp", ROCM_GPU, element::f32).empty());
         auto best = reg->FindKernelRegistration("FakeOp", ROCM_GPU, element::f32);
         EXPECT(best && best->m_tag == "high" && best->m_priority == 7);
-        EXPECT(reg->FindKernelRegistrations("QuantDot", ROCM_GPU, element::f32).size() == 1);
+        // the automatic emitter (priority 5) and four kernel variants (priority 3)
+        EXPECT(reg->FindKernelRegistrations("QuantDot", ROCM_GPU, element::f32).size() == 5);
+        auto qd = reg->FindKernelRegistration("QuantDot", ROCM_GPU, element::f32);
+        EXPECT(qd && qd->m_tag == "nnf_hip_gfx950" && qd->m_priority == 5);
         EXPECT(reg->FindKernelRegistrations("QuantDotW8A8", ROCM_GPU, element::f32).size() == 1);
         EXPECT(reg->FindKernelRegistrations("FusedQuantMLP", ROCM_GPU, element::f32).size() == 1);
         bool threw = false;
@@ -530,6 +535,62 @@ int main(int argc, char** argv)
         CONTAINS(pc->source_code, "for (size_t i = 0; i < 7; ++i)");
         CONTAINS(pc->source_code, "return (double)ms / 7;");
         CONTAINS(pc->source_code, "hipMemcpyHostToDevice");
+    });
+
+    run_case("profiling_selector_candidates", [&] {
+        // the automatic emitter and the kernel variants that can serve the shape, in priority order; the
+        // default selector keeps picking the automatic one
+        auto kinds = [](size_t M, size_t N, size_t K, const std::string& cfg = "", bool gamma = false) {
+            graph::Graph g;
+            auto n = quant_dot_graph(g, M, N, K, cfg, gamma);
+            pass::graph::ProfilingBasedKernelSelector sel;
+            std::vector<std::string> out;
+            for (auto& k : sel.candidates(n, ROCM_GPU))
+                out.push_back(k->get_kernel_type());
+            pass::graph::DefaultKernelSelector def;
+            EXPECT(def.pick_first(n, ROCM_GPU).second->get_kernel_type() == "rocm");
+            return out;
+        };
+        auto has = [](const std::vector<std::string>& v, const std::string& x) {
+            return std::find(v.begin(), v.end(), x) != v.end();
+        };
+        auto k1 = kinds(1, 4096, 4096);
+        EXPECT(k1.size() == 5 && k1[0] == "rocm");
+        EXPECT(has(k1, "rocm_gemv_rows") && has(k1, "rocm_gemv_mfma") && has(k1, "rocm_gemm_mfma") && has(k1, "rocm_gemv_valu"));
+        auto k8 = kinds(8, 4096, 4096);
+        EXPECT(k8.size() == 4 && !has(k8, "rocm_gemv_rows"));
+        auto k16 = kinds(16, 8192, 8192); // too many activations for one workgroup's LDS: no single-pass MFMA GEMV
+        EXPECT(!has(k16, "rocm_gemv_mfma") && has(k16, "rocm_gemm_mfma"));
+        auto kbig = kinds(4096, 8192, 8192);
+        EXPECT(kbig.size() == 2 && kbig[1] == "rocm_gemm_mfma");
+        auto kfused = kinds(4, 256, 256, "{\"rms_norm\": true}", true);
+        EXPECT(kfused.size() == 1 && kfused[0] == "rocm");
+        // the emitted call names the variant; the harness source of a variant differs from the automatic one's
+        graph::Graph g;
+        auto n = quant_dot_graph(g, 1, 4096, 4096);
+        pass::graph::ProfilingBasedKernelSelector sel;
+        sel.runtime_times = 9;
+        profiler::HipDefaultRuntime rt("/inc", "/lib");
+        auto pcs = sel.contexts(n, ROCM_GPU, rt);
+        EXPECT(pcs.size() == 5);
+        size_t rows = 0;
+        for (auto& pc : pcs)
+        {
+            CONTAINS(pc->source_code, "for (size_t i = 0; i < 9; ++i)");
+            if (pc->kernel->get_kernel_type() == "rocm_gemv_rows")
+            {
+                ++rows;
+                CONTAINS(pc->source_code, "nnf_w4a16_gemm_variant(stream, input0, input1, input2, output0, 1, 4096, 4096, 128, 8, NNF_W4A16_GEMV_ROWS, nullptr, 0)");
+                CONTAINS(pc->entry_name, "_rocm_gemv_rows_");
+            }
+        }
+        EXPECT(rows == 1);
+        // a disabled selector leaves the graph alone
+        auto gp = std::make_shared<graph::Graph>();
+        auto n2 = quant_dot_graph(*gp, 1, 4096, 4096);
+        pass::graph::DefaultGNodeDeviceDispatcher().run_on_graph(gp);
+        sel.enable = false;
+        EXPECT(sel.run_on_graph(gp, rt) && !(*n2)["Kernel_Selection_Result"].is_valid());
     });
 
     run_case("quant_fusion_passes", [] {

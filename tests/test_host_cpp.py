@@ -13,4 +13,4 @@ def test_host_cpp_suite(tmp_path):
     lines = [l for l in proc.stdout.splitlines() if l.startswith(("PASS", "FAIL"))]
     failed = [l for l in lines if l.startswith("FAIL")]
     assert proc.returncode == 0 and not failed, proc.stdout
-    assert len(lines) >= 13
+    assert len(lines) >= 14
