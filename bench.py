@@ -64,6 +64,9 @@ def main():
                          "no timing, no JSON")
     ap.add_argument("--mfma-probe", action="store_true",
                     help="print the MFMA-only rates (no memory traffic) for different operand values and exit")
+    ap.add_argument("--gemm-probe", action="store_true",
+                    help="for hardware-counter runs: the fp16 x int4 and the W8A8 GEMM at M=4096, N=K=8192, twelve "
+                         "launches each; prints their event-timed means, no JSON line of the benchmark")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU (no sharding, no collectives); use --gpus 1")
@@ -80,6 +83,10 @@ def main():
 
     def dev_t(a):
         return torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+
+    if args.gemm_probe:
+        print(json.dumps(run_gemm_probe(torch, dev, datagen, ops)))
+        return
 
     # ---- resident inputs ------------------------------------------------------------------------
     layers = []
@@ -273,6 +280,37 @@ def run_read_probe(torch, dev, lib, n_layers, per_shape, timed_graph):
         entry["read_us_through_lds"] = by_variant[4]
         entry["gemv_time_over_plain_read"] = round(entry["us"] / best, 3)
         del bufs
+
+
+def run_gemm_probe(torch, dev, datagen, ops, m=4096, n=8192, k=8192, launches=12):
+    """The two compute-bound GEMMs of the extra configurations on their own (what a counter run looks at)."""
+    ws = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
+
+    def timed(fn):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(launches):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1000.0 / launches
+
+    a, wq, s = datagen.w4a16_case(0, m, n, k)
+    ta, tw, ts = (torch.from_numpy(x).to(dev) for x in (a, wq, s))
+    y = torch.empty((m, n), dtype=torch.float16, device=dev)
+    us16 = timed(lambda: ops.w4a16_gemm(ta, tw, ts, out=y, workspace=ws))
+    _, _, w8, s_ch = datagen.w8a8_case(0, 1, n, k)
+    tw8, tsch = torch.from_numpy(w8).to(dev), torch.from_numpy(s_ch).to(dev)
+    a8 = torch.from_numpy(datagen.uniform_i8(0, datagen.S_A8, (m, k))).to(dev)
+    st = torch.from_numpy(datagen.uniform_f32(0, datagen.S_STOK, (m,), 0.001, 0.01)).to(dev)
+    us8 = timed(lambda: ops.w8a8_gemm(a8, st, tw8, tsch, out=y, workspace=ws))
+    ops_total = 2.0 * m * n * k
+    return {"shape": [m, n, k], "launches": launches,
+            "w4a16_us": round(us16, 1), "w4a16_tflops": round(ops_total / us16 / 1e6, 1),
+            "w8a8_us": round(us8, 1), "w8a8_tops": round(ops_total / us8 / 1e6, 1)}
 
 
 def run_mfma_probe(torch, lib):

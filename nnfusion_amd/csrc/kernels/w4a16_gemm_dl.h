@@ -282,7 +282,14 @@ namespace nnf
                     half8_t bf = __builtin_bit_cast(half8_t, uintx4{bw[0], bw[1], bw[2], bw[3]});
 #pragma unroll
                     for (int i = 0; i < TM; ++i)
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf, af[i], acc[i][j], 0, 0, 0);
+                        {
+                            // fp16 results are written by rows (D[n][m]: four consecutive columns per lane);
+                            // partial sums by columns (D[m][n]: 32 consecutive columns per store)
+                            if (SPLITK)
+                                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf, acc[i][j], 0, 0, 0);
+                            else
+                                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf, af[i], acc[i][j], 0, 0, 0);
+                        }
                 }
             }
         };
@@ -326,42 +333,36 @@ namespace nnf
         __builtin_amdgcn_s_waitcnt(vmcnt_imm(0)); // drain the tail loads before the LDS goes away
 
         // ---- epilogue ---------------------------------------------------------------------------------
-        // The weight fragment is the MFMA's first operand, so a 32x32 result is D[n][m]: lane (m = l32, h)
-        // holds, in element e, column n = 8*(e/4) + 4*h + (e%4) of its weight tile: four consecutive
-        // columns per group of four elements.
         const int m_wave = m0 + wm * (TM * 32);
         if (SPLITK)
         {
-            // fp32 partial sums: 16 bytes per lane straight from the registers
+            // fp32 partial sums straight from the registers.  Here the activation fragment is the MFMA's first
+            // operand: D[m][n], lane (n = l32, h), element e: row m = 8*(e/4) + 4*h + (e%4), so a store covers
+            // 32 consecutive columns (128 bytes) of two rows.
             float* part = p.partial + (size_t)split * p.M * p.ld_partial;
-            const bool vec = ((p.N & 3) == 0) && ((p.ld_partial & 3) == 0) && ((reinterpret_cast<uintptr_t>(part) & 15) == 0);
 #pragma unroll
-            for (int i = 0; i < TM; ++i)
+            for (int j = 0; j < TN; ++j)
             {
-                const int m = m_wave + i * 32 + l32;
-                if (m >= p.M)
+                const int n = GATE ? n0 + wn * 32 + l32 : n0 + wn * (TN * 32) + j * 32 + l32;
+                if (n >= p.N)
                     continue;
-                float* row = part + (size_t)m * p.ld_partial;
+                const int pc = (GATE && j == 1) ? p.N + n : n; // up columns follow the N gate columns
 #pragma unroll
-                for (int j = 0; j < TN; ++j)
+                for (int i = 0; i < TM; ++i)
 #pragma unroll
-                    for (int g = 0; g < 4; ++g)
+                    for (int e = 0; e < 16; ++e)
                     {
-                        // column of the output (GATE: of the gate / up pair); up columns follow the N gate columns
-                        const int n = GATE ? n0 + wn * 32 + 8 * g + 4 * h : n0 + wn * (TN * 32) + j * 32 + 8 * g + 4 * h;
-                        float* dst = row + ((GATE && j == 1) ? p.N + n : n);
-                        if (vec && n + 3 < p.N)
-                            *reinterpret_cast<floatx4*>(dst) = floatx4{acc[i][j][4 * g], acc[i][j][4 * g + 1],
-                                                                       acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
-                        else
-                            for (int k = 0; k < 4; ++k)
-                                if (n + k < p.N)
-                                    dst[k] = acc[i][j][4 * g + k];
+                        const int m = m_wave + i * 32 + 8 * (e >> 2) + 4 * h + (e & 3);
+                        if (m < p.M)
+                            part[(size_t)m * p.ld_partial + pc] = acc[i][j][e];
                     }
             }
             return;
         }
-        // fp16 results: rounded (GATE: combined) in registers, turned through a private piece of LDS (the
+        // fp16 results.  The weight fragment is the MFMA's first operand, so a 32x32 result is D[n][m]: lane
+        // (m = l32, h) holds, in element e, column n = 8*(e/4) + 4*h + (e%4) of its weight tile: four
+        // consecutive columns per group of four elements.  They are rounded (GATE: combined) in registers,
+        // turned through a private piece of LDS (the
         // ring is free after the barrier) and finished as whole rows of the wavefront's sub-tile, 16 bytes
         // (8 columns) per lane: bias, residual and the store.
         constexpr int OUT_TN = GATE ? 1 : TN;

@@ -206,7 +206,14 @@ namespace nnf
             for (int j = 0; j < TN; ++j)
 #pragma unroll
                 for (int i = 0; i < TM; ++i)
-                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[set][j], af[set][i], acc[i][j], 0, 0, 0);
+                    {
+                        // fp16 results are written by rows (D[n][m]: four consecutive columns per lane); int32
+                        // results by columns (D[m][n]: 32 consecutive columns per store)
+                        if (RAW || SPLITK)
+                            acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[set][i], bf[set][j], acc[i][j], 0, 0, 0);
+                        else
+                            acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[set][j], af[set][i], acc[i][j], 0, 0, 0);
+                    }
         };
         using I0 = std::integral_constant<int, 0>;
         using I1 = std::integral_constant<int, 1>;
@@ -268,41 +275,36 @@ namespace nnf
         __builtin_amdgcn_s_waitcnt(vmcnt_imm(0)); // drain the tail loads before the LDS goes away
 
         // ---- epilogue -------------------------------------------------------------------------------------
-        // The weight fragment is the MFMA's first operand, so a 32x32 result is D[n][m]: lane (m = l32, h)
-        // holds, in element e, column n = 8*(e/4) + 4*h + (e%4): four consecutive output columns per group
-        // of four elements.
         const int m_wave = m0 + wm * (TM * 32), n_wave = n0 + wn * (TN * 32);
         if (RAW || SPLITK)
         {
-            // int32 results: 16 bytes per lane straight from the registers
+            // int32 results straight from the registers.  Here the activation fragment is the MFMA's first
+            // operand: D[m][n], lane (n = l32, h), element e: row m = 8*(e/4) + 4*h + (e%4), so a store covers
+            // 32 consecutive columns (128 bytes) of two rows.
             int32_t* out = SPLITK ? p.partial + (size_t)split * p.M * p.N : p.acc;
-            const bool vec = ((p.N & 3) == 0) && ((reinterpret_cast<uintptr_t>(out) & 15) == 0);
 #pragma unroll
-            for (int i = 0; i < TM; ++i)
+            for (int j = 0; j < TN; ++j)
             {
-                const int m = m_wave + i * 32 + l32;
-                if (m >= p.M)
+                const int n = n_wave + j * 32 + l32;
+                if (n >= p.N)
                     continue;
-                int32_t* row = out + (size_t)m * p.N;
 #pragma unroll
-                for (int j = 0; j < TN; ++j)
+                for (int i = 0; i < TM; ++i)
 #pragma unroll
-                    for (int g = 0; g < 4; ++g)
+                    for (int e = 0; e < 16; ++e)
                     {
-                        const int n = n_wave + j * 32 + 8 * g + 4 * h;
-                        if (vec && n + 3 < p.N)
-                            *reinterpret_cast<intx4*>(row + n) = intx4{acc[i][j][4 * g], acc[i][j][4 * g + 1],
-                                                                       acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
-                        else
-                            for (int k = 0; k < 4; ++k)
-                                if (n + k < p.N)
-                                    row[n + k] = acc[i][j][4 * g + k];
+                        const int m = m_wave + i * 32 + 8 * (e >> 2) + 4 * h + (e & 3);
+                        if (m < p.M)
+                            out[(size_t)m * p.N + n] = acc[i][j][e];
                     }
             }
             return;
         }
-        // fp16 results: scaled in registers, turned through a private piece of LDS (the ring is free after
-        // the barrier) and written as whole rows of the wavefront's sub-tile, 16 bytes per lane.
+        // fp16 results.  The weight fragment is the MFMA's first operand, so a 32x32 result is D[n][m]: lane
+        // (m = l32, h) holds, in element e, column n = 8*(e/4) + 4*h + (e%4): four consecutive output columns
+        // per group of four elements.  They are scaled in registers, turned through a private piece of LDS
+        // (the ring is free after the barrier) and written as whole rows of the wavefront's sub-tile, 16
+        // bytes per lane.
         constexpr int ROUND_TM = TM >= 2 ? 2 : 1;  // 32-row blocks per pass through LDS
         constexpr int PITCH = TN * 64 + 16;        // bytes per staged row (padding spreads the banks)
         constexpr int REGION = ROUND_TM * 32 * PITCH;

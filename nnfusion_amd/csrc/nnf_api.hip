@@ -71,6 +71,7 @@ int nnf_internal_tune(int key, int value)
     case 2: nnf::g_tuning.skinny_wg_per_cu = value; return 0;
     case 3: nnf::g_tuning.gemm_tile = value; return 0;
     case 4: nnf::g_tuning.gemm_splits = value; return 0;
+    case 5: nnf::workspace::skinny_min_splits() = value; return 0;
     default: return -1;
     }
 }

@@ -172,6 +172,12 @@ namespace nnf
         // equal ranges (multiples of 1024 columns, at most 4096) when K divides that way, otherwise ranges of a
         // multiple of 1024 and a shorter last one of at least 1024.  Returns the length of the ranges (of all but
         // the last), or 0 when this does not apply.
+        // experiments only: the smallest number of equal ranges to consider (0: no preference)
+        inline int& skinny_min_splits()
+        {
+            static int v = 0;
+            return v;
+        }
         inline int w4a16_skinny_split_range(int M, int N, int K)
         {
             if (M < 1 || M > 16 || N < 16 || K < 2048 || (K & 127) || w4a16_skinny_fits(M, N, K))
@@ -182,6 +188,8 @@ namespace nnf
             for (int s : equal)
             {
                 const int r = K / s;
+                if (s < skinny_min_splits())
+                    continue;
                 if (K % s == 0 && (r & 1023) == 0 && r <= 4096 && w4a16_skinny_fits(M, N, r))
                     return r;
             }

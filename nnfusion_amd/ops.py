@@ -52,6 +52,28 @@ def w4a16_gemm(a, wq, scales, group=128, zp=8, out=None, workspace=None):
     return out
 
 
+VARIANTS = {"auto": 0, "gemv_valu": 1, "gemv_mfma": 2, "gemm_mfma": 3, "gemv_rows": 4}
+
+
+def w4a16_gemm_variant(a, wq, scales, variant, group=128, zp=8, out=None, workspace=None):
+    """As w4a16_gemm through one kernel variant (a key of VARIANTS); raises NnfError with status -2 when the
+    variant cannot serve the shape."""
+    lib = _lib.kernels()
+    m, k = a.shape
+    n = wq.shape[0]
+    v = VARIANTS[variant]
+    assert a.dtype == torch.float16 and wq.dtype == torch.uint8 and scales.dtype == torch.float16
+    assert a.is_contiguous() and wq.is_contiguous() and scales.is_contiguous()
+    if out is None:
+        out = torch.empty((m, n), dtype=torch.float16, device=a.device)
+    if workspace is None:
+        workspace = _ws(lib.nnf_w4a16_gemm_variant_workspace_bytes(m, n, k, group, v), a.device)
+    _check(lib.nnf_w4a16_gemm_variant(_stream(), a.data_ptr(), wq.data_ptr(), scales.data_ptr(), out.data_ptr(),
+                                      m, n, k, group, zp, v, workspace.data_ptr(), workspace.numel()),
+           "nnf_w4a16_gemm_variant")
+    return out
+
+
 def w4a16_gemm_fused(a, wq, scales, group=128, zp=8, rms_gamma=None, rms_eps=1e-6, bias=None, residual=None,
                      act=0, out=None, workspace=None):
     """GEMM with the fused RMSNorm prologue / bias, residual, SiLU-gate epilogues (see the C header)."""

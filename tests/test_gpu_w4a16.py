@@ -117,3 +117,31 @@ def test_gemv_other_zero_points(gpu, path, zp):
     y = _run(gpu, a, wq, s, zp=zp)
     ref = oracle.w4a16_gemm(a, wq, s, zp=zp, f32_out=True)
     _check(y, ref)
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 512, 4096), (8, 300, 2048), (16, 128, 8192), (40, 256, 1024)])
+def test_every_kernel_variant_that_accepts_a_shape_matches_the_oracle(gpu, m, n, k):
+    """nnf_w4a16_gemm_variant: the entry point behind the per-variant emitters of profiling-based kernel selection.
+    nnf_w4a16_variant_supported (host only) and the call itself agree on which variants serve a shape."""
+    import torch
+
+    from nnfusion_amd import _lib, ops
+
+    a, wq, s = datagen.w4a16_case(0, m, n, k)
+    ref = oracle.w4a16_gemm(a, wq, s, f32_out=True)
+    ta, tw, ts = (torch.from_numpy(x).to(gpu) for x in (a, wq, s))
+    served = []
+    for name, v in ops.VARIANTS.items():
+        ok = _lib.kernels().nnf_w4a16_variant_supported(m, n, k, 128, v)
+        if ok:
+            y = ops.w4a16_gemm_variant(ta, tw, ts, name)
+            torch.cuda.synchronize()
+            _check(y.cpu().numpy(), ref)
+            served.append(name)
+        else:
+            with pytest.raises(ops.NnfError) as e:
+                ops.w4a16_gemm_variant(ta, tw, ts, name)
+            assert e.value.status == -2
+    assert "auto" in served and "gemm_mfma" in served
+    assert ("gemv_rows" in served) == (m == 1)
+    assert ("gemv_valu" in served) == (m <= 16)
