@@ -37,9 +37,9 @@ DECODE_SHAPES = [(12288, 4096), (4096, 4096), (22016, 4096), (4096, 11008)]  # (
 GROUP = 128
 PROBE_BYTES = 1 << 30  # size of the calibration copy of --pmc-probe
 # HBM bytes per launch of the K = 4096 row-streaming kernel (mean over its three launches of a step), from two
-# rocprofv3 --pmc runs of `bench.py --pmc-probe`: FETCH_SIZE 13269.1 KiB x 2.000 (the factor by which the
+# rocprofv3 --pmc runs of `bench.py --pmc-probe`: FETCH_SIZE 13268.7 KiB x 2.000 (the factor by which the
 # counter under-reports the 1 GiB calibration copy) + WRITE_SIZE 27.3 KiB x 1.000.  Algorithmic: 27 067 392.
-ROWS_K4096_TRAFFIC_BYTES = int((13269.1 * 2.0 + 27.3) * 1024)
+ROWS_K4096_TRAFFIC_BYTES = int((13268.7 * 2.0 + 27.3) * 1024)
 
 
 def w4a16_bytes(m, n, k):
