@@ -175,6 +175,44 @@ def test_fused_bias_residual(gpu, plan):
     _check(y_br, ref_br)
 
 
+@pytest.mark.parametrize("m,n,k", [(257, 300, 512), (90, 36, 384), (33, 1001, 256)])
+def test_fused_bias_residual_ragged_columns(gpu, plan, m, n, k):
+    """N not a multiple of 8 (no 16-byte row pieces), M not a multiple of the tile: the element-wise tail of the
+    row-major epilogue, with bias and residual."""
+    import torch
+
+    from nnfusion_amd import ops
+
+    a, wq, s = datagen.w4a16_case(13, m, n, k)
+    bias = datagen.normal_f16(13, datagen.S_BIAS, (n,))
+    res = datagen.normal_f16(13, datagen.S_RES, (m, n))
+    ta, tw, ts, tb, tr = _t(gpu, a, wq, s, bias, res)
+    ws = _big_ws(gpu)
+    y = ops.w4a16_gemm(ta, tw, ts, workspace=ws).cpu().numpy()
+    y_br = ops.w4a16_gemm_fused(ta, tw, ts, bias=tb, residual=tr, workspace=ws).cpu().numpy()
+    torch.cuda.synchronize()
+    d = oracle.w4a16_gemm(a, wq, s)
+    _check(y, oracle.w4a16_gemm(a, wq, s, f32_out=True))
+    _check(y_br, oracle.add_f16(oracle.add_f16(d, np.broadcast_to(bias, (m, n)).copy()), res))
+
+
+def test_fused_silu_gate_ragged_columns(gpu, plan):
+    import torch
+
+    from nnfusion_amd import ops
+
+    m, n, k = 70, 100, 256
+    a, wq, s = datagen.w4a16_case(14, m, 2 * n, k)
+    ta, tw, ts = _t(gpu, a, wq, s)
+    y = ops.w4a16_gemm_fused(ta, tw, ts, act=1, workspace=_big_ws(gpu)).cpu().numpy()
+    torch.cuda.synchronize()
+    gu = oracle.w4a16_gemm(a, wq, s)
+    ref = oracle.silu_mul_f16(np.ascontiguousarray(gu[:, :n]), np.ascontiguousarray(gu[:, n:]))
+    err = np.abs(y.astype(np.float32) - ref.astype(np.float32))
+    assert y.shape == (m, n)
+    assert _rms(err) <= 1e-3 * _rms(ref) and err.max() <= 5e-2 * max(_rms(ref), 1e-3)
+
+
 def test_fused_rmsnorm_prologue(gpu, plan):
     import torch
 
