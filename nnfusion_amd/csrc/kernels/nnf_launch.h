@@ -25,6 +25,7 @@ namespace nnf
                                    int N, int K, int zp, int num_cu);
     // true when one workgroup can hold the activations (M <= 16 rows of K) in LDS
     bool w4a16_skinny_supported(int M, int N, int K);
+    int& skinny_direct_min_rows(); // experiments: see w4a16_skinny.hip
 
     // M <= 16 with activations too large for LDS: the same kernel over `ksplits` ranges of K, fp32 partial sums
     // [ksplits][M][N] (to be added by the GEMM's reduction pass); w4a16_skinny_ksplits returns 0 when not applicable

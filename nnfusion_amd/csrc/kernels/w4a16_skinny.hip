@@ -14,7 +14,9 @@
 //   * the dot products run on v_mfma_f32_16x16x32_f16 with the weight tile as the B operand
 //     (columns = n) and the M <= 16 activation rows as the A operand (rows = m), so the cost per
 //     weight byte does not depend on M.  The A operand is staged once per workgroup in LDS (already
-//     permuted and pre-scaled); with up to two groups per wavefront it is then kept in registers;
+//     permuted and pre-scaled); with up to two groups per wavefront it is then kept in registers --
+//     and from six rows on each wavefront loads its share straight from global memory into those
+//     registers, in the MFMA operand layout (16 rows x 64 bytes per load), instead of the staging;
 //   * nibbles are turned into fp16 with one v_and_or_b32 per pair: (q | 0x6400) = 1024 + q, and a
 //     nibble four bits up gives 1024 + 16 q.  Instead of subtracting the 1024 / zero point from
 //     every weight, the activations of the "16 q" slots are pre-divided by 16 and the constant part
@@ -61,7 +63,16 @@ namespace nnf
         float* partial;    // [ksplits][M][N]
     };
 
-    // pack = M | zp << 8 | wavefronts per workgroup << 16;  n_wg: workgroups per K range;  a workgroup's tiles:
+    // rows of activations from which a wavefront loads its own operand instead of staging all rows in LDS
+    // (below it the sixteen-fold repetition of the few rows costs more than the staging)
+    int& skinny_direct_min_rows()
+    {
+        static int v = 6; // measured: equal at 4 rows, 3-10 % faster from 6 rows on
+        return v;
+    }
+
+    // pack = M | zp << 8 | wavefronts per workgroup << 16 | direct << 24 (A_REGS: every wavefront loads its own
+    // share of the activations straight into registers, no staging in LDS);  n_wg: workgroups per K range;  a workgroup's tiles:
     // tiles_q, one more for the first tiles_r workgroups (n_tiles = tiles_q * n_wg + tiles_r, divided on the host).
     // The first arguments are the ones the first loads need: they arrive preloaded in scalar registers.
     template <int CPS, bool A_REGS, int H, bool KSPLIT>
@@ -88,7 +99,8 @@ namespace nnf
         const int tid = threadIdx.x;
         const int lane = tid & 63;
         const int wave = __builtin_amdgcn_readfirstlane(tid >> 6); // in a scalar register, and what follows from it
-        const int M = pack & 0xff, zp = (pack >> 8) & 0xff, KS = pack >> 16;
+        const int M = pack & 0xff, zp = (pack >> 8) & 0xff, KS = (pack >> 16) & 0xff;
+        const bool direct = A_REGS && ((pack >> 24) & 1); // uniform over the grid
         const int n_threads = KS << 6;
         const int col = lane & 15; // n within the tile (B operand / D column), m for the A operand
         const int kq = lane >> 4;  // K quarter of the MFMA (A/B operands), row quad of D
@@ -168,14 +180,30 @@ namespace nnf
 #pragma unroll
         for (int e = 0; e < A_EARLY; ++e)
             a_early[e] = uintx4{0u, 0u, 0u, 0u};
-        if (wave * 64 < row0_units)
+        // Through a pointer the compiler knows nothing about, and with a compiler-level memory barrier behind:
+        // otherwise these loads are moved down into the block that uses them, behind the weights.
+        typedef const uint8_t __attribute__((address_space(1))) * global_bytes_t;
+        typedef const uintx4 __attribute__((address_space(1))) * global_units_t;
+        global_bytes_t a_bytes = (global_bytes_t) reinterpret_cast<const uint8_t*>(A);
+        asm volatile("" : "+s"(a_bytes));
+        // direct: lane (m = col, kq) of a wavefront fetches the 64 bytes of row m that its MFMA operand holds of
+        // each of the wavefront's groups (k = 32 kq .. 32 kq + 31 of the group); rows past M repeat row M-1
+        // A_REGS: a wavefront's operand and its constants are kept in registers (16 + 4 VGPRs per group);
+        // otherwise both are re-read from LDS for every tile
+        uintx4 areg[A_REGS ? CPS : 1][4];
+        floatx4 ncreg[A_REGS ? CPS : 1];
+        if (A_REGS && direct)
         {
-            // Through a pointer the compiler knows nothing about, and with a compiler-level memory barrier behind:
-            // otherwise these loads are moved down into the block that uses them, behind the weights.
-            typedef const uint8_t __attribute__((address_space(1))) * global_bytes_t;
-            typedef const uintx4 __attribute__((address_space(1))) * global_units_t;
-            global_bytes_t a_bytes = (global_bytes_t) reinterpret_cast<const uint8_t*>(A);
-            asm volatile("" : "+s"(a_bytes));
+            const uint32_t a_off = (uint32_t)min(col, M - 1) * (uint32_t)lda * 2u + (uint32_t)chunk_base[0] * 256u + (uint32_t)kq * 64u;
+#pragma unroll
+            for (int c = 0; c < CPS; ++c)
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    areg[A_REGS ? c : 0][j] = *(global_units_t)(a_bytes + (size_t)(a_off + c * 256 + j * 16));
+            asm volatile("" ::: "memory");
+        }
+        if (!direct && wave * 64 < row0_units)
+        {
 #pragma unroll
             for (int e = 0; e < A_EARLY; ++e)
             {
@@ -254,18 +282,22 @@ namespace nnf
             if ((u & 15) == 0)
                 reinterpret_cast<float*>(nc_lds)[(u >> 4) * 16 + m] = pc;
         };
-#pragma unroll
-        for (int e = 0; e < A_EARLY; ++e)
+        if (!direct)
         {
-            int u = tid + e * n_threads;
-            if (u < row0_units)
-                stage_unit(a_early[e], 0, u);
+#pragma unroll
+            for (int e = 0; e < A_EARLY; ++e)
+            {
+                int u = tid + e * n_threads;
+                if (u < row0_units)
+                    stage_unit(a_early[e], 0, u);
+            }
+            // what the early loads did not cover of row 0 (very long rows only) ...
+            for (int u = tid + A_EARLY * n_threads; u < row0_units; u += n_threads)
+                stage_unit(*reinterpret_cast<const uintx4*>(A + u * 8), 0, u);
         }
-        // what the early loads did not cover of row 0 (very long rows only) ...
-        for (int u = tid + A_EARLY * n_threads; u < row0_units; u += n_threads)
-            stage_unit(*reinterpret_cast<const uintx4*>(A + u * 8), 0, u);
         // ... and rows 1 .. M-1, as one index space over all threads with four loads in flight per thread: row by
         // row, each row would cost a full memory round trip of its own
+        if (!direct)
         {
             const int rest = (M - 1) * row0_units;
             for (int v0 = tid; v0 < rest; v0 += 4 * n_threads)
@@ -300,11 +332,32 @@ namespace nnf
             sc_lds[tid] = sfirst;
         lds_barrier();
 
-        // A_REGS: this wavefront's operand and its constants are read from LDS once and kept
-        // (16 + 4 VGPRs per group); otherwise both are re-read for every tile
-        uintx4 areg[A_REGS ? CPS : 1][4];
-        floatx4 ncreg[A_REGS ? CPS : 1];
-        if (A_REGS)
+        // A_REGS without direct loads: the operand and its constants are read from LDS once
+        if (A_REGS && direct)
+        {
+            // the pair order and the 1/16 of the nibble trick in registers; the constant part of a group sum is
+            // a product with a constant vector: four MFMAs whose B operand is (ce, co, ce, co) for every column
+            const half_t ceh = (half_t)ce, coh = (half_t)co; // -(1024 + zp) and -16 (64 + zp): exact in fp16
+            const uint32_t ce2 = as_u32(half2_t{ceh, ceh}), co2 = as_u32(half2_t{coh, coh});
+            const uintx4 cvec = {ce2, co2, ce2, co2};
+#pragma unroll
+            for (int c = 0; c < CPS; ++c)
+            {
+                floatx4 t = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                {
+                    uintx4 a = permute_a8(areg[A_REGS ? c : 0][j]);
+                    a.y = as_u32(as_half2(a.y) * sixteenth);
+                    a.w = as_u32(as_half2(a.w) * sixteenth);
+                    areg[A_REGS ? c : 0][j] = a;
+                    t = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, a),
+                                                               __builtin_bit_cast(half8_t, cvec), t, 0, 0, 0);
+                }
+                ncreg[A_REGS ? c : 0] = t;
+            }
+        }
+        else if (A_REGS)
         {
 #pragma unroll
             for (int c = 0; c < CPS; ++c)
@@ -562,7 +615,8 @@ namespace nnf
             }
             hipLaunchKernelGGL((w4a16_skinny_kernel<CPS, A_REGS, H, KSPLIT>), dim3(grid * ksplits), dim3(p.ks * 64), lds_total,
                                stream, (const half_t*)A, (const uint8_t*)Wq, (const half_t*)S, (half_t*)Y, N, K,
-                               n_tiles / grid, n_tiles % grid, grid, M | (zp << 8) | (p.ks << 16), sp);
+                               n_tiles / grid, n_tiles % grid, grid,
+                               M | (zp << 8) | (p.ks << 16) | ((A_REGS && M >= skinny_direct_min_rows()) ? (1 << 24) : 0), sp);
             return hipGetLastError();
         }
     } // namespace

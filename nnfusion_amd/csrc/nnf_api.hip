@@ -72,6 +72,7 @@ int nnf_internal_tune(int key, int value)
     case 3: nnf::g_tuning.gemm_tile = value; return 0;
     case 4: nnf::g_tuning.gemm_splits = value; return 0;
     case 5: nnf::workspace::skinny_min_splits() = value; return 0;
+    case 6: nnf::skinny_direct_min_rows() = value > 0 ? value : 6; return 0;
     default: return -1;
     }
 }
