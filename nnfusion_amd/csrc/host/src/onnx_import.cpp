@@ -1,0 +1,573 @@
+// ONNX front door: a reader of the protobuf wire format for the ONNX messages the importer needs, and the
+// conversion of a model into the graph IR (the part of src/nnfusion/frontend/onnx_import/{onnx.cpp,
+// util/graph_convert.cpp} that the quantized path needs).
+#include "nnfusion/frontend/onnx_import/onnx.hpp"
+
+#include "../nnf_datagen.h"
+#include "nnfusion/core/operators/generic_op/generic_op.hpp"
+
+#include <cmath>
+#include <cstring>
+#include <fstream>
+#include <iterator>
+
+namespace nnfusion
+{
+    namespace frontend
+    {
+        namespace onnx_lite
+        {
+            namespace
+            {
+                // one message: a bounded byte range walked field by field
+                class Reader
+                {
+                public:
+                    Reader(const uint8_t* p, size_t n)
+                        : m_p(p)
+                        , m_end(p + n)
+                    {
+                    }
+                    bool done() const { return m_p >= m_end; }
+                    uint64_t varint()
+                    {
+                        uint64_t v = 0;
+                        for (int shift = 0; shift < 64; shift += 7)
+                        {
+                            NNFUSION_CHECK(m_p < m_end) << "onnx: truncated varint";
+                            const uint8_t c = *m_p++;
+                            v |= (uint64_t)(c & 0x7F) << shift;
+                            if (!(c & 0x80))
+                                return v;
+                        }
+                        NNFUSION_CHECK(false) << "onnx: varint longer than 10 bytes";
+                        return 0;
+                    }
+                    // next field: number and wire type
+                    void key(uint32_t& field, uint32_t& wire)
+                    {
+                        const uint64_t k = varint();
+                        field = (uint32_t)(k >> 3);
+                        wire = (uint32_t)(k & 7);
+                    }
+                    Reader bytes()
+                    {
+                        const uint64_t n = varint();
+                        NNFUSION_CHECK(n <= (uint64_t)(m_end - m_p)) << "onnx: length-delimited field runs past its message";
+                        Reader r(m_p, (size_t)n);
+                        m_p += n;
+                        return r;
+                    }
+                    std::string str()
+                    {
+                        Reader r = bytes();
+                        return std::string(reinterpret_cast<const char*>(r.m_p), r.size());
+                    }
+                    uint32_t fixed32()
+                    {
+                        NNFUSION_CHECK(m_end - m_p >= 4) << "onnx: truncated 32-bit field";
+                        uint32_t v;
+                        memcpy(&v, m_p, 4);
+                        m_p += 4;
+                        return v;
+                    }
+                    uint64_t fixed64()
+                    {
+                        NNFUSION_CHECK(m_end - m_p >= 8) << "onnx: truncated 64-bit field";
+                        uint64_t v;
+                        memcpy(&v, m_p, 8);
+                        m_p += 8;
+                        return v;
+                    }
+                    void skip(uint32_t wire)
+                    {
+                        switch (wire)
+                        {
+                        case 0: varint(); break;
+                        case 1: fixed64(); break;
+                        case 2: bytes(); break;
+                        case 5: fixed32(); break;
+                        default: NNFUSION_CHECK(false) << "onnx: unsupported wire type " << wire;
+                        }
+                    }
+                    const uint8_t* data() const { return m_p; }
+                    size_t size() const { return (size_t)(m_end - m_p); }
+
+                private:
+                    const uint8_t* m_p;
+                    const uint8_t* m_end;
+                };
+
+                // repeated scalar field: packed (wire type 2) or one element per key
+                template <class T, class F>
+                void repeated(Reader& r, uint32_t wire, uint32_t scalar_wire, std::vector<T>& out, F read_one)
+                {
+                    if (wire == 2)
+                    {
+                        Reader p = r.bytes();
+                        while (!p.done())
+                            out.push_back(read_one(p));
+                    }
+                    else
+                    {
+                        NNFUSION_CHECK(wire == scalar_wire) << "onnx: unexpected wire type in a repeated field";
+                        out.push_back(read_one(r));
+                    }
+                }
+                float as_float(uint32_t bits)
+                {
+                    float f;
+                    memcpy(&f, &bits, 4);
+                    return f;
+                }
+                size_t type_size(int dt)
+                {
+                    switch (dt)
+                    {
+                    case UINT8: case INT8: case BOOL: return 1;
+                    case UINT16: case INT16: case FLOAT16: return 2;
+                    case FLOAT: case INT32: case UINT32: return 4;
+                    case INT64: case UINT64: case DOUBLE: return 8;
+                    default: return 0;
+                    }
+                }
+
+                Tensor parse_tensor(Reader r)
+                {
+                    Tensor t;
+                    std::vector<float> float_data;
+                    std::vector<int64_t> int32_data, int64_data;
+                    std::vector<uint64_t> uint64_data, double_bits;
+                    bool raw = false;
+                    while (!r.done())
+                    {
+                        uint32_t f, w;
+                        r.key(f, w);
+                        switch (f)
+                        {
+                        case 1: repeated(r, w, 0, t.dims, [](Reader& x) { return (int64_t)x.varint(); }); break;
+                        case 2: t.data_type = (int)r.varint(); break;
+                        case 4: repeated(r, w, 5, float_data, [](Reader& x) { return as_float(x.fixed32()); }); break;
+                        case 5: repeated(r, w, 0, int32_data, [](Reader& x) { return (int64_t)x.varint(); }); break;
+                        case 7: repeated(r, w, 0, int64_data, [](Reader& x) { return (int64_t)x.varint(); }); break;
+                        case 8: t.name = r.str(); break;
+                        case 9:
+                        {
+                            Reader b = r.bytes();
+                            t.bytes.assign(b.data(), b.data() + b.size());
+                            raw = true;
+                            break;
+                        }
+                        case 10: repeated(r, w, 1, double_bits, [](Reader& x) { return x.fixed64(); }); break;
+                        case 11: repeated(r, w, 0, uint64_data, [](Reader& x) { return x.varint(); }); break;
+                        default: r.skip(w);
+                        }
+                    }
+                    if (!raw)
+                    {
+                        // typed fields: widen / narrow to the tensor's own element type
+                        const size_t es = type_size(t.data_type);
+                        auto put = [&](const void* p) { t.bytes.insert(t.bytes.end(), (const uint8_t*)p, (const uint8_t*)p + es); };
+                        if (t.data_type == FLOAT)
+                            for (float v : float_data)
+                                put(&v);
+                        else if (t.data_type == DOUBLE)
+                            for (uint64_t v : double_bits)
+                                put(&v);
+                        else if (t.data_type == INT64)
+                            for (int64_t v : int64_data)
+                                put(&v);
+                        else if (t.data_type == UINT64 || t.data_type == UINT32)
+                            for (uint64_t v : uint64_data)
+                                put(&v); // little endian: the low bytes
+                        else
+                            for (int64_t v : int32_data)
+                                put(&v); // int32_data carries INT32, INT16, INT8, UINT16, UINT8, BOOL and FLOAT16 bit patterns
+                    }
+                    return t;
+                }
+
+                Attribute parse_attribute(Reader r)
+                {
+                    Attribute a;
+                    while (!r.done())
+                    {
+                        uint32_t f, w;
+                        r.key(f, w);
+                        switch (f)
+                        {
+                        case 1: a.name = r.str(); break;
+                        case 2: a.f = as_float(r.fixed32()); break;
+                        case 3: a.i = (int64_t)r.varint(); break;
+                        case 4: a.s = r.str(); break;
+                        case 5: a.t = parse_tensor(r.bytes()); break;
+                        case 7: repeated(r, w, 5, a.floats, [](Reader& x) { return as_float(x.fixed32()); }); break;
+                        case 8: repeated(r, w, 0, a.ints, [](Reader& x) { return (int64_t)x.varint(); }); break;
+                        case 20: a.type = (int)r.varint(); break;
+                        default: r.skip(w);
+                        }
+                    }
+                    return a;
+                }
+
+                Node parse_node(Reader r)
+                {
+                    Node n;
+                    while (!r.done())
+                    {
+                        uint32_t f, w;
+                        r.key(f, w);
+                        switch (f)
+                        {
+                        case 1: n.inputs.push_back(r.str()); break;
+                        case 2: n.outputs.push_back(r.str()); break;
+                        case 3: n.name = r.str(); break;
+                        case 4: n.op_type = r.str(); break;
+                        case 5:
+                        {
+                            Attribute a = parse_attribute(r.bytes());
+                            n.attributes[a.name] = a;
+                            break;
+                        }
+                        case 7: n.domain = r.str(); break;
+                        default: r.skip(w);
+                        }
+                    }
+                    return n;
+                }
+
+                ValueInfo parse_value_info(Reader r)
+                {
+                    ValueInfo v;
+                    while (!r.done())
+                    {
+                        uint32_t f, w;
+                        r.key(f, w);
+                        if (f == 1)
+                            v.name = r.str();
+                        else if (f == 2)
+                        {
+                            Reader type = r.bytes(); // TypeProto
+                            while (!type.done())
+                            {
+                                uint32_t tf, tw;
+                                type.key(tf, tw);
+                                if (tf != 1)
+                                {
+                                    type.skip(tw);
+                                    continue;
+                                }
+                                Reader tt = type.bytes(); // TypeProto.Tensor
+                                while (!tt.done())
+                                {
+                                    uint32_t f2, w2;
+                                    tt.key(f2, w2);
+                                    if (f2 == 1)
+                                        v.elem_type = (int)tt.varint();
+                                    else if (f2 == 2)
+                                    {
+                                        Reader shape = tt.bytes(); // TensorShapeProto
+                                        while (!shape.done())
+                                        {
+                                            uint32_t f3, w3;
+                                            shape.key(f3, w3);
+                                            if (f3 != 1)
+                                            {
+                                                shape.skip(w3);
+                                                continue;
+                                            }
+                                            Reader dim = shape.bytes();
+                                            int64_t value = -1;
+                                            std::string param;
+                                            while (!dim.done())
+                                            {
+                                                uint32_t f4, w4;
+                                                dim.key(f4, w4);
+                                                if (f4 == 1)
+                                                    value = (int64_t)dim.varint();
+                                                else if (f4 == 2)
+                                                    param = dim.str();
+                                                else
+                                                    dim.skip(w4);
+                                            }
+                                            v.dims.push_back(value);
+                                            v.dim_params.push_back(param);
+                                        }
+                                    }
+                                    else
+                                        tt.skip(w2);
+                                }
+                            }
+                        }
+                        else
+                            r.skip(w);
+                    }
+                    return v;
+                }
+
+                void parse_graph(Reader r, Model& m)
+                {
+                    while (!r.done())
+                    {
+                        uint32_t f, w;
+                        r.key(f, w);
+                        switch (f)
+                        {
+                        case 1: m.nodes.push_back(parse_node(r.bytes())); break;
+                        case 2: m.graph_name = r.str(); break;
+                        case 5: m.initializers.push_back(parse_tensor(r.bytes())); break;
+                        case 11: m.inputs.push_back(parse_value_info(r.bytes())); break;
+                        case 12: m.outputs.push_back(parse_value_info(r.bytes())); break;
+                        default: r.skip(w);
+                        }
+                    }
+                }
+            } // namespace
+
+            size_t Tensor::element_count() const
+            {
+                size_t n = 1;
+                for (int64_t d : dims)
+                    n *= (size_t)d;
+                return n;
+            }
+            int64_t Node::get_int(const std::string& key, int64_t dflt) const
+            {
+                auto it = attributes.find(key);
+                return it == attributes.end() ? dflt : it->second.i;
+            }
+            float Node::get_float(const std::string& key, float dflt) const
+            {
+                auto it = attributes.find(key);
+                return it == attributes.end() ? dflt : it->second.f;
+            }
+
+            Model parse_model(const std::vector<uint8_t>& file)
+            {
+                Model m;
+                Reader r(file.data(), file.size());
+                while (!r.done())
+                {
+                    uint32_t f, w;
+                    r.key(f, w);
+                    switch (f)
+                    {
+                    case 1: m.ir_version = (int64_t)r.varint(); break;
+                    case 2: m.producer_name = r.str(); break;
+                    case 7: parse_graph(r.bytes(), m); break;
+                    case 8:
+                    {
+                        Reader o = r.bytes(); // OperatorSetIdProto
+                        std::string domain;
+                        int64_t version = 0;
+                        while (!o.done())
+                        {
+                            uint32_t f2, w2;
+                            o.key(f2, w2);
+                            if (f2 == 1)
+                                domain = o.str();
+                            else if (f2 == 2)
+                                version = (int64_t)o.varint();
+                            else
+                                o.skip(w2);
+                        }
+                        m.opset[domain] = version;
+                        break;
+                    }
+                    default: r.skip(w);
+                    }
+                }
+                return m;
+            }
+
+            Model parse_model_file(const std::string& path)
+            {
+                std::ifstream f(path, std::ios::binary);
+                NNFUSION_CHECK(f.is_open()) << "onnx: cannot open " << path;
+                std::vector<uint8_t> bytes((std::istreambuf_iterator<char>(f)), std::istreambuf_iterator<char>());
+                return parse_model(bytes);
+            }
+        } // namespace onnx_lite
+
+        namespace
+        {
+            using namespace onnx_lite;
+
+            const element::Type& element_type_of(int dt)
+            {
+                switch (dt)
+                {
+                case FLOAT: return element::f32;
+                case FLOAT16: return element::f16;
+                case DOUBLE: return element::f64;
+                case UINT8: return element::u8;
+                case INT8: return element::i8;
+                case INT32: return element::i32;
+                case INT64: return element::i64;
+                case BOOL: return element::boolean;
+                default: NNFUSION_CHECK(false) << "onnx: unsupported tensor element type " << dt; return element::dynamic;
+                }
+            }
+
+            // fp32 -> fp16 bits, round to nearest even (scales stored as fp32 in a model)
+            uint16_t float_to_half_bits(float f)
+            {
+                return nnf_f32_to_f16_bits(f);
+            }
+        } // namespace
+
+        std::shared_ptr<graph::Graph> load_onnx_model(const std::string& path,
+                                                      const std::unordered_map<std::string, size_t>& dim_params)
+        {
+            const Model model = parse_model_file(path);
+            auto g = std::make_shared<graph::Graph>();
+            std::map<std::string, std::shared_ptr<graph::GNode>> value; // ONNX value name -> producing node
+            std::map<std::string, const Tensor*> init;
+            for (auto& t : model.initializers)
+                init[t.name] = &t;
+
+            auto add_constant = [&](const Tensor& t, const std::string& name) {
+                const element::Type& et = element_type_of(t.data_type);
+                Shape shape;
+                for (int64_t d : t.dims)
+                    shape.push_back((size_t)d);
+                NNFUSION_CHECK(t.bytes.size() == shape_size(shape) * et.size())
+                    << "onnx: tensor " << name << " carries " << t.bytes.size() << " bytes for " << shape_size(shape) << " elements";
+                value[name] = g->add_node_and_edge(std::make_shared<op::Constant>(et, shape, t.bytes.data()), graph::GNodeVector{});
+            };
+            // graph inputs that are not initializers are the parameters, in file order
+            for (auto& in : model.inputs)
+            {
+                if (init.count(in.name))
+                    continue;
+                Shape shape;
+                for (size_t i = 0; i < in.dims.size(); ++i)
+                {
+                    int64_t d = in.dims[i];
+                    if (d < 0)
+                    {
+                        auto it = dim_params.find(in.dim_params[i]);
+                        NNFUSION_CHECK(it != dim_params.end()) << "onnx: no value for the symbolic dimension '" << in.dim_params[i]
+                                                               << "' of input " << in.name;
+                        d = (int64_t)it->second;
+                    }
+                    shape.push_back((size_t)d);
+                }
+                value[in.name] = g->add_node_and_edge(std::make_shared<op::Parameter>(element_type_of(in.elem_type), shape),
+                                                      graph::GNodeVector{});
+            }
+            auto input_of = [&](const Node& n, size_t i) -> std::shared_ptr<graph::GNode> {
+                NNFUSION_CHECK(i < n.inputs.size()) << "onnx: " << n.op_type << " " << n.name << " has no input " << i;
+                const std::string& name = n.inputs[i];
+                auto it = value.find(name);
+                if (it != value.end())
+                    return it->second;
+                auto ti = init.find(name);
+                NNFUSION_CHECK(ti != init.end()) << "onnx: " << n.op_type << " " << n.name << " reads undefined value " << name;
+                add_constant(*ti->second, name); // initializers become constants where they are first used
+                return value[name];
+            };
+            auto has_input = [](const Node& n, size_t i) { return i < n.inputs.size() && !n.inputs[i].empty(); };
+            auto generic = [&](const Node& n, const std::string& type, const graph::GNodeVector& in, const std::string& cfg = "") {
+                auto config = cfg.empty() ? op::OpConfig::any() : op::OpConfig::any::parse(cfg);
+                const std::string name = n.name.empty() ? n.outputs.at(0) : n.name;
+                return g->add_node_and_edge(std::make_shared<op::GenericOp>(name, type, config), in);
+            };
+
+            for (auto& n : model.nodes) // ONNX keeps nodes in topological order
+            {
+                NNFUSION_CHECK(!n.outputs.empty()) << "onnx: node without outputs";
+                std::shared_ptr<graph::GNode> out;
+                if (n.op_type == "Constant")
+                {
+                    auto it = n.attributes.find("value");
+                    NNFUSION_CHECK(it != n.attributes.end()) << "onnx: Constant without a value tensor";
+                    add_constant(it->second.t, n.outputs[0]);
+                    continue;
+                }
+                else if (n.op_type == "MatMulNBits")
+                {
+                    // A [.., K]; B u8 [N, K/block, block/2] (two 4-bit values per byte, low nibble first);
+                    // scales [N * K/block]; optional zero_points (packed 4-bit, one per block)
+                    const int64_t K = n.get_int("K", 0), N = n.get_int("N", 0);
+                    const int64_t bits = n.get_int("bits", 4), block = n.get_int("block_size", 0);
+                    NNFUSION_CHECK(bits == 4 && block == 128 && K > 0 && N > 0 && K % block == 0)
+                        << "onnx: MatMulNBits " << n.name << ": only bits = 4, block_size = 128 (K a multiple of it) is supported";
+                    NNFUSION_CHECK(!has_input(n, 4) && !has_input(n, 5)) << "onnx: MatMulNBits with g_idx or bias is not supported";
+                    auto wi = init.find(n.inputs.at(1));
+                    auto si = init.find(n.inputs.at(2));
+                    NNFUSION_CHECK(wi != init.end() && si != init.end()) << "onnx: MatMulNBits weights and scales must be initializers";
+                    const Tensor& wt = *wi->second;
+                    NNFUSION_CHECK(wt.data_type == UINT8 && wt.bytes.size() == (size_t)(N * K / 2))
+                        << "onnx: MatMulNBits B must be uint8 with N*K/2 bytes";
+                    int zp = 8;
+                    if (has_input(n, 3))
+                    {
+                        auto zi = init.find(n.inputs[3]);
+                        NNFUSION_CHECK(zi != init.end() && zi->second->data_type == UINT8 && !zi->second->bytes.empty())
+                            << "onnx: MatMulNBits zero points must be a packed uint8 initializer";
+                        const std::vector<uint8_t>& z = zi->second->bytes;
+                        zp = z[0] & 0xF;
+                        const int64_t blocks = K / block;
+                        for (int64_t r = 0; r < N; ++r)
+                            for (int64_t b = 0; b < blocks; ++b)
+                            {
+                                const uint8_t byte = z[(size_t)(r * ((blocks + 1) / 2) + b / 2)];
+                                NNFUSION_CHECK(((b & 1) ? (byte >> 4) : (byte & 0xF)) == zp)
+                                    << "onnx: MatMulNBits with per-block zero points is not supported (a uniform one is)";
+                            }
+                    }
+                    auto wq = g->add_node_and_edge(
+                        std::make_shared<op::Constant>(element::u8, Shape{(size_t)N, (size_t)(K / 2)}, wt.bytes.data()), graph::GNodeVector{});
+                    const Tensor& st = *si->second;
+                    const size_t n_scales = (size_t)(N * (K / block));
+                    std::vector<uint16_t> sc(n_scales);
+                    if (st.data_type == FLOAT16)
+                    {
+                        NNFUSION_CHECK(st.bytes.size() == n_scales * 2) << "onnx: MatMulNBits scales: wrong size";
+                        memcpy(sc.data(), st.bytes.data(), n_scales * 2);
+                    }
+                    else
+                    {
+                        NNFUSION_CHECK(st.data_type == FLOAT && st.bytes.size() == n_scales * 4) << "onnx: MatMulNBits scales must be fp16 or fp32";
+                        for (size_t i = 0; i < n_scales; ++i)
+                        {
+                            float f;
+                            memcpy(&f, st.bytes.data() + 4 * i, 4);
+                            sc[i] = float_to_half_bits(f);
+                        }
+                    }
+                    auto s = g->add_node_and_edge(
+                        std::make_shared<op::Constant>(element::f16, Shape{(size_t)N, (size_t)(K / block)}, sc.data()), graph::GNodeVector{});
+                    out = generic(n, "QuantDot", {input_of(n, 0), wq, s}, "{\"zero_point\": " + std::to_string(zp) + "}");
+                }
+                else if (n.op_type == "SimplifiedLayerNormalization" || n.op_type == "RMSNormalization")
+                {
+                    const int64_t axis = n.get_int("axis", -1);
+                    auto x = input_of(n, 0);
+                    NNFUSION_CHECK(axis == -1 || axis == (int64_t)x->get_output_shape(0).size() - 1)
+                        << "onnx: " << n.op_type << " over an axis other than the last is not supported";
+                    char eps[64];
+                    snprintf(eps, sizeof(eps), "{\"eps\": %.9g}", (double)n.get_float("epsilon", 1e-5f));
+                    out = generic(n, "RMSNorm", {x, input_of(n, 1)}, eps);
+                }
+                else if (n.op_type == "Sigmoid")
+                    out = generic(n, "Sigmoid", {input_of(n, 0)});
+                else if (n.op_type == "Mul")
+                    out = generic(n, "Multiply", {input_of(n, 0), input_of(n, 1)});
+                else if (n.op_type == "Add")
+                    out = generic(n, "Add", {input_of(n, 0), input_of(n, 1)});
+                else
+                    NNFUSION_CHECK(false) << "onnx: unsupported operator " << (n.domain.empty() ? "" : n.domain + "::") << n.op_type;
+                value[n.outputs[0]] = out;
+            }
+            for (auto& o : model.outputs)
+            {
+                auto it = value.find(o.name);
+                NNFUSION_CHECK(it != value.end()) << "onnx: graph output " << o.name << " is not produced";
+                g->add_node_and_edge(std::make_shared<op::Result>(), {it->second});
+            }
+            return g;
+        }
+    } // namespace frontend
+} // namespace nnfusion

@@ -13,9 +13,13 @@
 //                                                         Swish, Multiply, Add; the fusion pass folds it into one node)
 //   nnf_compile_example qkv_graph <out_dir> M N K       (RMSNorm feeding three QuantDots of N rows each; merged
 //                                                         into one 3N-row QuantDot + three Slices; three results)
+//   nnf_compile_example onnx      <out_dir> <model.onnx> [include_dir lib_dir]
+//                                                        (an ONNX model of the quantized path: MatMulNBits,
+//                                                         SimplifiedLayerNormalization, Sigmoid, Mul, Add)
 #include "../nnf_datagen.h"
 #include "nnfusion/core/operators/generic_op/generic_op.hpp"
 #include "nnfusion/engine/pass/codegen/base_codegen_pass.hpp"
+#include "nnfusion/frontend/onnx_import/onnx.hpp"
 
 #include <cstdlib>
 #include <cstring>
@@ -46,16 +50,23 @@ namespace
 
 int main(int argc, char** argv)
 {
-    if (argc < 6)
+    const bool from_onnx = argc >= 4 && std::string(argv[1]) == "onnx";
+    if (argc < 6 && !(from_onnx && argc >= 4))
     {
-        fprintf(stderr, "usage: %s <quant_dot|w8a8|mlp|mlp_nodes|mlp_graph|qkv_graph> <out_dir> <d0> <d1> <d2> [include_dir lib_dir]\n", argv[0]);
+        fprintf(stderr, "usage: %s <quant_dot|w8a8|mlp|mlp_nodes|mlp_graph|qkv_graph> <out_dir> <d0> <d1> <d2> [include_dir lib_dir]\n"
+                        "       %s onnx <out_dir> <model.onnx> [include_dir lib_dir]\n", argv[0], argv[0]);
         return 2;
     }
     const std::string kind = argv[1], out_dir = argv[2];
-    const size_t d0 = strtoul(argv[3], nullptr, 10), d1 = strtoul(argv[4], nullptr, 10), d2 = strtoul(argv[5], nullptr, 10);
+    const size_t d0 = from_onnx ? 0 : strtoul(argv[3], nullptr, 10), d1 = from_onnx ? 0 : strtoul(argv[4], nullptr, 10),
+                 d2 = from_onnx ? 0 : strtoul(argv[5], nullptr, 10);
+    const int dirs_at = from_onnx ? 4 : 6; // where the optional include / library directories start
     auto g = std::make_shared<graph::Graph>();
     try
     {
+        if (from_onnx)
+            g = frontend::load_onnx_model(argv[3]);
+        else
         if (kind == "quant_dot")
         {
             const size_t M = d0, N = d1, K = d2;
@@ -173,10 +184,10 @@ int main(int argc, char** argv)
         }
         ROCmEngine engine(out_dir);
         engine.quant_gemm_fusion = kind == "qkv_graph";
-        if (argc >= 8)
+        if (argc >= dirs_at + 2)
         {
-            engine.pass.kernels_include_dir = argv[6];
-            engine.pass.kernels_lib_dir = argv[7];
+            engine.pass.kernels_include_dir = argv[dirs_at];
+            engine.pass.kernels_lib_dir = argv[dirs_at + 1];
         }
         engine.pass.exit_after_codegen = false;
         engine.run_on_graph(g);

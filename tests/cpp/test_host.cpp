@@ -10,6 +10,7 @@
 #include "nnfusion/engine/pass/graph/kernel_selection.hpp"
 #include "nnfusion/engine/pass/graph/quant_fusion_pass.hpp"
 #include "nnfusion/engine/profiler/hip_runtime.hpp"
+#include "nnfusion/frontend/onnx_import/onnx.hpp"
 
 #include <algorithm>
 
@@ -17,7 +18,9 @@
 
 #include <cstdio>
 #include <cstdlib>
+#include <cstring>
 #include <fstream>
+#include <iterator>
 
 using namespace nnfusion;
 using namespace nnfusion::kernels;
@@ -144,6 +147,8 @@ namespace
 int main(int argc, char** argv)
 {
     const std::string tmp = argc > 1 ? argv[1] : "/tmp/nnf_host_test";
+    // where tests/golden lives (second argument; default: relative to the repository root as working directory)
+    const std::string golden = argc > 2 ? argv[2] : "tests/golden";
 
     run_case("element_types", [] {
         EXPECT(element::f16.c_type_string() == "half" && element::f16.size() == 2);
@@ -591,6 +596,87 @@ int main(int argc, char** argv)
         pass::graph::DefaultGNodeDeviceDispatcher().run_on_graph(gp);
         sel.enable = false;
         EXPECT(sel.run_on_graph(gp, rt) && !(*n2)["Kernel_Selection_Result"].is_valid());
+    });
+
+    run_case("onnx_reader_on_reference_models", [&] {
+        using namespace frontend::onnx_lite;
+        const std::string dir = golden + "/onnx/";
+        // add_abc_initializers: packed int64_data initializer, tensor attribute with packed float_data
+        Model m = parse_model_file(dir + "add_abc_initializers.onnx");
+        EXPECT(m.ir_version == 3 && m.producer_name == "ngraph ONNXImporter" && m.graph_name == "test_graph");
+        EXPECT(m.opset.at("") == 4);
+        EXPECT(m.nodes.size() == 3 && m.nodes[0].op_type == "Constant" && m.nodes[1].op_type == "Add" && m.nodes[2].op_type == "Add");
+        EXPECT(m.nodes[1].inputs == (std::vector<std::string>{"A", "B"}) && m.nodes[1].outputs == (std::vector<std::string>{"X"}));
+        EXPECT(m.nodes[2].inputs == (std::vector<std::string>{"X", "C"}) && m.nodes[2].name == "add_node2");
+        const Attribute& val = m.nodes[0].attributes.at("value");
+        EXPECT(val.type == 4 && val.t.data_type == FLOAT && val.t.dims == (std::vector<int64_t>{2, 2}) && val.t.name == "const_tensor");
+        EXPECT(val.t.bytes.size() == 16);
+        float fb[4];
+        memcpy(fb, val.t.bytes.data(), 16);
+        EXPECT(fb[0] == 1.f && fb[1] == 2.f && fb[2] == 3.f && fb[3] == 4.f);
+        EXPECT(m.initializers.size() == 1 && m.initializers[0].name == "A" && m.initializers[0].data_type == INT64);
+        int64_t ia[4];
+        EXPECT(m.initializers[0].bytes.size() == 32);
+        memcpy(ia, m.initializers[0].bytes.data(), 32);
+        // the reference's expectation: C = {1,2,3,4} gives Y = A + B + C = {3,6,9,12}
+        const float c_in[4] = {1, 2, 3, 4}, want[4] = {3, 6, 9, 12};
+        for (int i = 0; i < 4; ++i)
+            EXPECT((float)ia[i] + fb[i] + c_in[i] == want[i]);
+        EXPECT(m.inputs.size() == 2 && m.inputs[0].name == "A" && m.inputs[1].name == "C" && m.inputs[1].elem_type == FLOAT);
+        EXPECT(m.inputs[1].dims == (std::vector<int64_t>{2, 2}) && m.outputs.size() == 1 && m.outputs[0].name == "Y");
+
+        // gemm_op: float and integer attributes, value infos
+        Model gm = parse_model_file(dir + "gemm_op.onnx");
+        EXPECT(gm.ir_version == 6 && gm.opset.at("") == 11 && gm.graph_name == "gemm" && gm.nodes.size() == 1);
+        const Node& ge = gm.nodes[0];
+        EXPECT(ge.op_type == "Gemm" && ge.inputs == (std::vector<std::string>{"a", "b", "c"}) && ge.outputs[0] == "y");
+        EXPECT(ge.get_float("alpha", 1.f) == 0.25f && ge.get_float("beta", 1.f) == 0.35f);
+        EXPECT(ge.get_int("transA", 0) == 1 && ge.get_int("transB", 0) == 1 && ge.get_int("absent", 7) == 7);
+        EXPECT(ge.attributes.at("alpha").type == 1 && ge.attributes.at("transA").type == 2);
+        EXPECT(gm.inputs.size() == 3 && gm.inputs[0].dims == (std::vector<int64_t>{4, 3}) && gm.inputs[1].dims == (std::vector<int64_t>{5, 4}));
+        EXPECT(gm.inputs[2].dims == (std::vector<int64_t>{1, 5}) && gm.outputs[0].dims == (std::vector<int64_t>{3, 5}));
+
+        Model mm = parse_model_file(dir + "matmul_op_3.onnx");
+        EXPECT(mm.nodes.size() == 1 && mm.nodes[0].op_type == "MatMul");
+        EXPECT(mm.inputs[0].dims == (std::vector<int64_t>{2}) && mm.inputs[1].dims == (std::vector<int64_t>{3, 2, 1}));
+        EXPECT(mm.outputs[0].dims == (std::vector<int64_t>{3, 1}));
+
+        // truncated files raise instead of reading past the end
+        std::ifstream f(dir + "gemm_op.onnx", std::ios::binary);
+        std::vector<uint8_t> bytes((std::istreambuf_iterator<char>(f)), std::istreambuf_iterator<char>());
+        bytes.resize(bytes.size() - 7);
+        bool threw = false;
+        try
+        {
+            parse_model(bytes);
+        }
+        catch (const CheckError&)
+        {
+            threw = true;
+        }
+        EXPECT(threw);
+        // operators outside the quantized path are refused by the importer, as unsupported operators are in the reference
+        threw = false;
+        try
+        {
+            frontend::load_onnx_model(dir + "gemm_op.onnx");
+        }
+        catch (const CheckError& e)
+        {
+            threw = std::string(e.what()).find("unsupported operator Gemm") != std::string::npos;
+        }
+        EXPECT(threw);
+        // Add is on the path: the reference's model imports (int64 initializer + float constant: types are the graph's business)
+        auto g = frontend::load_onnx_model(dir + "add_abc_initializers.onnx");
+        size_t adds = 0, consts = 0, params = 0, results = 0;
+        for (auto& n : g->get_nodes())
+        {
+            adds += n->get_op_type() == "Add";
+            consts += n->is_constant();
+            params += n->is_parameter();
+            results += n->is_output();
+        }
+        EXPECT(adds == 2 && consts == 2 && params == 1 && results == 1);
     });
 
     run_case("quant_fusion_passes", [] {

@@ -44,6 +44,36 @@ def test_generated_project_compiles_and_exports_the_runtime_abi(tmp_path):
     assert len(consts) == 2 and sum(os.path.getsize(out + "Constant/" + c) for c in consts) == 64 * 128 + 64 * 2 * 2
 
 
+def test_onnx_front_door_imports_fuses_and_generates(tmp_path):
+    """An ONNX model of the Llama MLP block (SimplifiedLayerNormalization, three MatMulNBits, Sigmoid, Mul, Add) is
+    imported, folded into one FusedQuantMLP by the fusion pass and generated as one launcher call; its constants are
+    the model's bytes ([gate; up] concatenated by the pass)."""
+    from nnfusion_amd import onnx_writer
+
+    m, h, i = 8, 256, 384
+    _, gamma, wgu, sgu, wd, sd = datagen.mlp_case(0, m, h, i)
+    model = str(tmp_path / "mlp.onnx")
+    onnx_writer.write_quant_mlp(model, m, gamma, wgu[:i], sgu[:i], wgu[i:], sgu[i:], wd, sd, 1e-6)
+    out = str(tmp_path / "rt") + "/"
+    subprocess.run([TOOL, "onnx", out, model], check=True, timeout=60)
+    text = open(out + "nnfusion_rt.cpp").read()
+    assert text.count("NNF_HIP_CHECK(nnf_") == 1
+    assert "nnf_fused_mlp_w4a16(stream, input0, input1," in text and ", 8, 256, 384, 128, 8, " in text
+    blobs = {os.path.getsize(out + "Constant/" + c): open(out + "Constant/" + c, "rb").read() for c in os.listdir(out + "Constant")}
+    assert blobs[wgu.nbytes] == wgu.tobytes() and blobs[wd.nbytes] == wd.tobytes() and blobs[gamma.nbytes] == gamma.tobytes()
+    assert blobs[sgu.nbytes] == sgu.tobytes()
+    # a single linear layer becomes one nnf_w4a16_gemm call; unsupported models are refused with the operator's name
+    _, wq, s = datagen.w4a16_case(0, 2, 64, 256)
+    lin = str(tmp_path / "linear.onnx")
+    onnx_writer.write_quant_linear(lin, 2, wq, s)
+    out2 = str(tmp_path / "rt2") + "/"
+    subprocess.run([TOOL, "onnx", out2, lin], check=True, timeout=60)
+    assert "nnf_w4a16_gemm(stream, input0, input1, input2, output0, 2, 64, 256, 128, 8, nullptr, 0)" in open(out2 + "nnfusion_rt.cpp").read()
+    bad = subprocess.run([TOOL, "onnx", str(tmp_path / "rt3") + "/", os.path.join(ROOT, "tests", "golden", "onnx", "gemm_op.onnx")],
+                         stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=60)
+    assert bad.returncode == 1 and "unsupported operator Gemm" in bad.stderr
+
+
 def _run_generated(name, inputs, out_shape, out_dtype, gpu, n_outputs=1):
     """dlopen nnfusion_amd/generated/<name>, init, kernel_entry(inputs..., outputs...), free."""
     import torch
@@ -104,6 +134,25 @@ def test_generated_mlp_runtime(gpu, name, m, h, i):
     y = _run_generated(name, [x], (m, h), torch.float16, gpu)
     ref = oracle.fused_mlp_w4a16(x, gamma, wgu, sgu, wd, sd)
     assert np.abs(y.astype(np.float32) - ref.astype(np.float32)).max() <= 1e-2 * _rms(ref)
+
+
+@pytest.mark.gpu
+def test_generated_runtime_of_an_onnx_model(gpu):
+    """The runtimes generated at build time from ONNX files (MatMulNBits models written by nnfusion_amd.onnx_writer)."""
+    import torch
+
+    import __graft_entry__ as entry
+
+    _, m, h, i = entry.ONNX_EXAMPLES["onnx_mlp"]
+    x, gamma, wgu, sgu, wd, sd = datagen.mlp_case(0, m, h, i)
+    y = _run_generated("onnx_mlp", [x], (m, h), torch.float16, gpu)
+    ref = oracle.fused_mlp_w4a16(x, gamma, wgu, sgu, wd, sd)
+    assert np.abs(y.astype(np.float32) - ref.astype(np.float32)).max() <= 1e-2 * _rms(ref)
+    _, m, n, k = entry.ONNX_EXAMPLES["onnx_linear"]
+    a, wq, s = datagen.w4a16_case(0, m, n, k)
+    y = _run_generated("onnx_linear", [a], (m, n), torch.float16, gpu)
+    ref = oracle.w4a16_gemm(a, wq, s, f32_out=True)
+    assert np.abs(y.astype(np.float32) - ref).max() <= 1e-2 * _rms(ref)
 
 
 @pytest.mark.gpu
