@@ -432,6 +432,22 @@ def run_extra(torch, np, dev, lib, datagen, ops):
     fl = 2.0 * m * (2 * i) * h + 2.0 * m * h * i
     res["fused_mlp_M256_4096_11008"] = {"us": round(us, 2), "TFLOP/s": round(fl / us / 1e6, 1),
                                         "frac_mfma_f16": round(fl / us / 1e6 / MFMA_F16_PEAK_TFLOPS, 4)}
+    del tens, out, wsm
+    # For scale only: the vendor library's unquantized GEMMs on the same box and value distributions (fp16 weights,
+    # four times the bytes, no unpacking; int8 x int8 -> int32 without the scaling epilogue), M = 4096, N = K = 8192.
+    try:
+        m, n, k = 4096, 8192, 8192
+        a = torch.randn(m, k, device=dev, dtype=torch.float16)
+        w = torch.randn(n, k, device=dev, dtype=torch.float16)
+        y = torch.empty(m, n, device=dev, dtype=torch.float16)
+        us16 = time_us(lambda: torch.matmul(a, w.t(), out=y), 20)
+        a8 = torch.randint(-127, 128, (m, k), device=dev, dtype=torch.int8)
+        w8 = torch.randint(-127, 128, (n, k), device=dev, dtype=torch.int8)
+        us8 = time_us(lambda: torch._int_mm(a8, w8.t()), 20)
+        res["vendor_library_for_scale_M4096"] = {"fp16_matmul_us": round(us16, 1), "fp16_TFLOP/s": round(2.0 * m * n * k / us16 / 1e6, 1),
+                                                 "int8_mm_us": round(us8, 1), "int8_TOP/s": round(2.0 * m * n * k / us8 / 1e6, 1)}
+    except Exception as e:  # a yardstick, not part of the benchmark
+        res["vendor_library_for_scale_M4096"] = {"error": str(e)[:200]}
     return res
 
 
