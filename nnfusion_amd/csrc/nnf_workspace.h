@@ -34,13 +34,13 @@ namespace nnf
         // N(0,1) activations (the GEMMs are power bound: ~950 / 700 / 450 TFLOP/s for the three tile shapes when
         // every CU has a workgroup, and a CU runs faster when fewer are busy: hence the square root), ~6 TB/s for
         // the partial sums (written, then read by the reduction pass) and ~3 us for the second launch.
-        // w8a8: the same tiles on the int8 matrix cores (~1640 / 1450 / 900 TOP/s; its weight bytes differ too, but
+        // w8a8: the same tiles on the int8 matrix cores (~1870 / 1450 / 900 TOP/s; its weight bytes differ too, but
         // a memory-bound W8A8 shape is decided by the partial-sum term either way)
         inline double estimate_gemm(int M, int N, int K, bool gate, int tile, int splits, bool w8a8)
         {
             const int bm = tile == GEMM_TILE_BIG ? 256 : tile == GEMM_TILE_MID ? 128 : tile == GEMM_TILE_SMALL ? 64 : 32;
             const int bn = tile == GEMM_TILE_BIG ? (gate ? 128 : 256) : tile == GEMM_TILE_MID ? 128 : 256;
-            static const double rates[2][4] = {{950e12, 700e12, 450e12, 300e12}, {1640e12, 1450e12, 900e12, 600e12}};
+            static const double rates[2][4] = {{950e12, 700e12, 450e12, 300e12}, {1870e12, 1450e12, 900e12, 600e12}};
             const double rate = rates[w8a8 ? 1 : 0][tile];
             const int tiles_m = ceil_div(M, bm), tiles_n = ceil_div(N, bn);
             const double blocks = (double)tiles_m * tiles_n * splits;
