@@ -138,5 +138,11 @@ namespace nnfusion
         codegen::HipCodegenPass pass;
         bool quant_epilogue_fusion = true; // QuantEpilogueFusionPass
         bool quant_gemm_fusion = false;    // QuantGemmFusionPass (off by default, like -fgemm_fusion)
+        // ProfilingBasedKernelSelector ahead of the default selector (off by default, like -fkernel_selection):
+        // needs hipcc and a GPU at compile time; harness objects already in kernel_profiling_dir are reused
+        bool kernel_selection = false;
+        std::string kernel_profiling_dir = "./kernel_profiling/";
+        size_t kernel_profiling_runs = 100;
+        bool kernel_selection_prepare_only = false; // build the harnesses and stop before code generation
     };
 } // namespace nnfusion

@@ -58,6 +58,9 @@ namespace nnfusion
                     double ms; // mean of runtime_times runs; < 0: failed to compile or run
                 };
                 bool enable = true; // the reference's -fkernel_selection
+                // only generate and compile the harnesses (a host without the device): nothing runs, nothing is chosen;
+                // a later run with the same working_dir finds the objects and compiles nothing
+                bool prepare_only = false;
                 size_t warmup_times = 5, runtime_times = 100;
                 std::string working_dir = "./kernel_profiling/";
 

@@ -568,6 +568,17 @@ namespace nnfusion
         }
         pass::graph::DefaultGNodeDeviceDispatcher dispatcher(ROCM_GPU);
         NNFUSION_CHECK(dispatcher.run_on_graph(graph));
+        if (kernel_selection)
+        {
+            profiler::HipDefaultRuntime runtime(pass.kernels_include_dir, pass.kernels_lib_dir);
+            pass::graph::ProfilingBasedKernelSelector profiling;
+            profiling.working_dir = kernel_profiling_dir;
+            profiling.runtime_times = kernel_profiling_runs;
+            profiling.prepare_only = kernel_selection_prepare_only;
+            NNFUSION_CHECK(profiling.run_on_graph(graph, runtime));
+            if (kernel_selection_prepare_only)
+                return true;
+        }
         pass::graph::DefaultKernelSelector selector;
         NNFUSION_CHECK(selector.run_on_graph(graph));
         auto tu = visit_graph(graph);

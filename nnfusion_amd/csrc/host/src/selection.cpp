@@ -221,6 +221,13 @@ namespace nnfusion
                 // nothing to choose between (the reference skips nodes with a single registration)
                 if (pcs.size() < 2)
                     return std::make_pair(devtype, KernelEmitter::Pointer());
+                if (prepare_only)
+                {
+                    for (auto& pc : pcs)
+                        NNFUSION_CHECK(runtime.compile(pc)) << "kernel selection: cannot build the harness of "
+                                                            << pc->kernel->get_function_name();
+                    return std::make_pair(devtype, KernelEmitter::Pointer());
+                }
                 KernelEmitter::Pointer best;
                 double best_ms = -1.0;
                 for (auto& pc : pcs)

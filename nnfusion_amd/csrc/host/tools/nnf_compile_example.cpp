@@ -13,6 +13,8 @@
 //                                                         Swish, Multiply, Add; the fusion pass folds it into one node)
 //   nnf_compile_example qkv_graph <out_dir> M N K       (RMSNorm feeding three QuantDots of N rows each; merged
 //                                                         into one 3N-row QuantDot + three Slices; three results)
+// every form: [include_dir lib_dir [kernel_profiling_dir [prepare]]] at the end; a kernel_profiling_dir switches
+// profiling-based kernel selection on (every candidate kernel of a QuantDot node is timed on the GPU)
 //   nnf_compile_example onnx      <out_dir> <model.onnx> [include_dir lib_dir]
 //                                                        (an ONNX model of the quantized path: MatMulNBits,
 //                                                         SimplifiedLayerNormalization, Sigmoid, Mul, Add)
@@ -189,6 +191,16 @@ int main(int argc, char** argv)
             engine.pass.kernels_include_dir = argv[dirs_at];
             engine.pass.kernels_lib_dir = argv[dirs_at + 1];
         }
+        // [kernel_profiling_dir [prepare]]: profiling-based kernel selection (-fkernel_selection of the reference);
+        // "prepare" only builds the single-kernel harnesses, for a later run on a host with the GPU
+        if (argc >= dirs_at + 3)
+        {
+            engine.kernel_selection = true;
+            nnfusion::min_log_level() = 1; // the time of every candidate is logged at INFO
+            engine.kernel_profiling_dir = argv[dirs_at + 2];
+            engine.kernel_profiling_runs = 50;
+            engine.kernel_selection_prepare_only = argc >= dirs_at + 4 && std::string(argv[dirs_at + 3]) == "prepare";
+        }
         engine.pass.exit_after_codegen = false;
         engine.run_on_graph(g);
     }
@@ -197,6 +209,9 @@ int main(int argc, char** argv)
         fprintf(stderr, "nnf_compile_example: %s\n", e.what());
         return 1;
     }
-    printf("generated %s in %s\n", kind.c_str(), out_dir.c_str());
+    if (argc >= dirs_at + 4 && std::string(argv[dirs_at + 3]) == "prepare")
+        printf("kernel-selection harnesses of %s built in %s\n", kind.c_str(), argv[dirs_at + 2]);
+    else
+        printf("generated %s in %s\n", kind.c_str(), out_dir.c_str());
     return 0;
 }

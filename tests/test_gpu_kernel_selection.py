@@ -44,3 +44,21 @@ def test_profiling_selector_times_every_candidate_and_keeps_the_fastest(gpu, nam
         # a single row: the streaming GEMV kernels, never the MFMA tile GEMM
         assert res["best"] in ("rocm", "rocm_gemv_rows", "rocm_gemv_mfma"), res
         assert times["rocm_gemm_mfma"] > times[res["best"]]
+
+
+@pytest.mark.gpu
+def test_code_generation_with_kernel_selection_emits_the_fastest_candidate(gpu, tmp_path):
+    """The compile flow with -fkernel_selection semantics: device dispatch, profiling of every QuantDot candidate (the
+    harness objects were built by build()), then the default selector keeps the profiled winner and the code
+    generator emits that kernel's call."""
+    out = str(tmp_path / "rt") + "/"
+    cmd = entry.compile_with_kernel_selection_command(out, False)
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=110)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    text = open(out + "nnfusion_rt.cpp").read()
+    calls = [l.strip() for l in text.splitlines() if "NNF_HIP_CHECK(nnf_" in l]
+    assert len(calls) == 1, calls
+    # one activation row: a streaming GEMV kernel wins (the automatic emitter resolves to the same kernel as gemv_rows)
+    assert ("nnf_w4a16_gemm(stream" in calls[0] or "NNF_W4A16_GEMV_ROWS" in calls[0] or "NNF_W4A16_GEMV_MFMA" in calls[0]), calls
+    timed = [l for l in proc.stderr.splitlines() + proc.stdout.splitlines() if "time cost(ms)" in l]
+    assert len(timed) == 5, proc.stderr[-2000:]
