@@ -21,6 +21,12 @@ namespace nnf
                                       int K, int zp, int num_cu);
     bool w4a16_gemv_rows_supported(int M, int N, int K, int num_cu);
 
+    // 2 <= M <= 16, K = 1024 / 2048 / 4096 / 8192: weights streamed through LDS rings, activations in registers
+    hipError_t launch_w4a16_mrows(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M, int N,
+                                  int K, int zp, int num_cu);
+    bool w4a16_mrows_supported(int M, int N, int K, int num_cu);
+    bool w4a16_mrows_preferred(int M, int N, int K, int num_cu); // where the library picks it without being told
+
     hipError_t launch_w4a16_skinny(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M,
                                    int N, int K, int zp, int num_cu);
     // true when one workgroup can hold the activations (M <= 16 rows of K) in LDS
@@ -59,7 +65,8 @@ namespace nnf
     // Tuning knobs for experiments (not part of the public ABI): 0 = automatic.
     struct Tuning
     {
-        int force_path = 0;  // 1 = VALU GEMV, 2 = MFMA skinny, 3 = MFMA GEMM, 4 = row-streaming GEMV (M = 1)
+        int force_path = 0;  // 1 = VALU GEMV, 2 = MFMA skinny, 3 = MFMA GEMM, 4 = row-streaming GEMV (M = 1),
+                             // 5 = row-streaming MFMA kernel (2 <= M <= 16) where it applies
         int skinny_cps = 0;  // chunks (groups of 128) per wavefront
         int skinny_wg_per_cu = 0;
         int gemm_tile = 0;   // 1 + nnf::workspace::GemmTile

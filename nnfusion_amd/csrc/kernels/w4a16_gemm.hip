@@ -263,14 +263,17 @@ namespace nnf
         // the products go to scratch first when the epilogue cannot work in place: the [M, 2N] gate | up pair, or a
         // residual that is the output buffer itself
         const bool via_scratch = gate || (hr && residual == Y);
-        if (!gemm_only && M <= 16 && w4a16_skinny_supported(M, n_rows, K) && (!via_scratch || partial_ws))
+        // one activation row: the row-streaming kernel where it applies; a handful of rows: the row-streaming MFMA kernel
+        const bool rows = !gemm_only && (g_tuning.force_path == 0 || g_tuning.force_path == 4) &&
+                          w4a16_gemv_rows_supported(M, n_rows, K, num_cu);
+        const bool mrows = !gemm_only && ((g_tuning.force_path == 5 && w4a16_mrows_supported(M, n_rows, K, num_cu)) ||
+                                          (g_tuning.force_path == 0 && w4a16_mrows_preferred(M, n_rows, K, num_cu)));
+        if (!gemm_only && M <= 16 && (rows || mrows || w4a16_skinny_supported(M, n_rows, K)) && (!via_scratch || partial_ws))
         {
             void* y_gemv = via_scratch ? partial_ws : Y;
-            // one activation row: the row-streaming kernel where it applies
-            const bool rows = (g_tuning.force_path == 0 || g_tuning.force_path == 4) &&
-                              w4a16_gemv_rows_supported(M, n_rows, K, num_cu);
             hipError_t e = rows ? launch_w4a16_gemv_rows(stream, A, Wq, S, y_gemv, n_rows, K, zp, num_cu)
-                                : launch_w4a16_skinny(stream, A, Wq, S, y_gemv, M, n_rows, K, zp, num_cu);
+                                : mrows ? launch_w4a16_mrows(stream, A, Wq, S, y_gemv, M, n_rows, K, zp, num_cu)
+                                        : launch_w4a16_skinny(stream, A, Wq, S, y_gemv, M, n_rows, K, zp, num_cu);
             if (e != hipSuccess || (!gate && !hb && !hr))
                 return e;
             const int blocks = (M * N + 255) / 256;

@@ -1,0 +1,282 @@
+// fp16 x int4 (g128) for 2 <= M <= 16 activation rows and K = 1024, 2048, 4096 or 8192: the memory pipeline of the
+// row-streaming GEMV (w4a16_gemv_rows.hip) under the arithmetic of the M <= 16 MFMA kernel (w4a16_skinny.hip).
+//
+//   Y[M,N] = A[M,K] . ((Wq - zp) * S)^T
+//
+// Replaces the cublasHgemm call of cuda::Dot (src/nnfusion/core/kernels/cuda_gpu/kernels/dot.cpp:271-363) for a
+// weight-quantized Dot node with a handful of activation rows.
+//
+//   * One workgroup of eight wavefronts per CU owns a contiguous run of 16-row weight tiles.  All eight work on
+//     the same tile; wavefront w owns the K slice [w K/8, (w+1) K/8) = GW groups of 128.
+//   * A wavefront's slice of a tile (16 rows x GW*64 bytes = GW KiB) goes global -> LDS without registers
+//     (global_load_lds_dwordx4, 1 KiB per wavefront-wide load) into a private two-slot ring, together with its
+//     16 x GW group scales (one 4-byte load per lane); the slot of the tile after next is requested as soon as
+//     the current one has been copied into registers.  Nothing but the wavefront's own loads feeds its MFMAs:
+//     no barrier on the load path.  The 16-byte pieces of a row are XOR-swizzled with the row number on the
+//     way (each lane chooses which piece it fetches), so the 128-bit operand reads are conflict free.
+//   * The activations never touch LDS: lane (m, kq) loads the 64 bytes of row m that its MFMA operand holds of
+//     each of the wavefront's groups, once, and keeps them (16 VGPRs per group; hence K <= 8192), in the pair
+//     order and with the 1/16 of the nibble trick; the constant part of a group sum is an MFMA against a
+//     constant operand and becomes the (negative) initial accumulator of the group (see w4a16_skinny.hip).
+//   * Per tile: GW x 4 MFMAs (v_mfma_f32_16x16x32_f16, weights as the B operand) per wavefront, the group sum
+//     times the group scale in fp32, the eight partial 16 x 16 tiles meet in LDS (one LDS-only barrier per
+//     tile, two alternating buffers), 256 threads add them and park the sums in LDS; Y is written after the
+//     last tile.  Every workgroup reads all of A (M x K x 2 bytes, from the L2): with 16 rows of K = 8192 that
+//     is twice the bytes of its weights, which bounds the kernel at ~1.4x the time of the weight stream.
+//   * LDS writes inside the tile loop are inline ds_write instructions: ahead of an LDS write that it can see,
+//     the compiler waits for every LDS-bound load in flight.
+#include "nnf_device.h"
+#include "nnf_launch.h"
+
+#include "../nnf_workspace.h"
+
+namespace nnf
+{
+    namespace
+    {
+        constexpr int MR_WAVES = 8;
+        typedef const void __attribute__((address_space(1))) * mr_global_ptr_t;
+        typedef void __attribute__((address_space(3))) * mr_lds_ptr_t;
+        // s_waitcnt with only the vector-memory counter set (gfx9 encoding: vmcnt = bits 3:0 and 15:14)
+        constexpr int mr_vmcnt(int n) { return (n & 0xF) | ((n >> 4) << 14) | (0x7 << 4) | (0xF << 8); }
+    } // namespace
+
+    // LDS (bytes): weights [8 wavefronts][2 slots][GW KiB] | scales [8][2][256] | partial tiles [2][8][1 KiB] |
+    //              parked sums [tiles of the workgroup][M][16] fp32
+    // pack = M | zp << 8;  a workgroup's tiles: tiles_q, one more for the first tiles_r workgroups.
+    template <int GW>
+    __global__ __launch_bounds__(512) void w4a16_mrows_kernel(const half_t* __restrict__ A, const uint8_t* __restrict__ Wq,
+                                                              const half_t* __restrict__ S, half_t* __restrict__ Y, int N,
+                                                              int tiles_q, int tiles_r, int pack)
+    {
+        static_assert(GW == 1 || GW == 2 || GW == 4 || GW == 8, "K = GW * 1024");
+        constexpr int K = GW * 1024, G = GW * 8;
+        constexpr int ROW_BYTES = K / 2;       // a weight row
+        constexpr int SLICE = GW * 64;         // a wavefront's bytes of a weight row
+        constexpr int TILE_BYTES = 16 * SLICE; // = GW KiB: GW wavefront-wide loads
+        constexpr int LT = GW + 1;             // loads per tile and wavefront (weights + scales)
+        constexpr int SC_LANES = GW >= 2 ? GW / 2 : 1; // 4-byte scale loads per row
+        extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+        uint32_t MAGIC, MASK_LO, MASK_HI;
+        asm volatile("v_mov_b32 %0, 0x64006400" : "=v"(MAGIC));
+        asm volatile("s_mov_b32 %0, 0x000F000F" : "=s"(MASK_LO));
+        asm volatile("s_mov_b32 %0, 0x00F000F0" : "=s"(MASK_HI));
+
+        const int tid = threadIdx.x;
+        const int lane = tid & 63;
+        const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+        const int col = lane & 15; // n within the tile (B operand / D column), m for the A operand
+        const int kq = lane >> 4;  // K quarter of the MFMA operands, row quad of D
+        const int M = pack & 0xff, zp = (pack >> 8) & 0xff;
+        const int b = blockIdx.x;
+        const int t0 = b * tiles_q + min(b, tiles_r);
+        const int T = tiles_q + (b < tiles_r ? 1 : 0);
+        // the last tile of an N that is not a multiple of 16 is moved back to rows N-16 .. N-1
+        auto row0_of = [&](int tile) { return __builtin_amdgcn_readfirstlane(min(tile * 16, N - 16)); };
+
+        uint8_t* ring = smem + wave * (2 * TILE_BYTES);
+        uint8_t* sc_ring = smem + MR_WAVES * 2 * TILE_BYTES + wave * 512;
+        uint8_t* red = smem + MR_WAVES * 2 * TILE_BYTES + MR_WAVES * 512; // [2][8][1024]
+        float* parked = reinterpret_cast<float*>(red + 2 * MR_WAVES * 1024);
+
+        // ---- what each lane fetches -------------------------------------------------------------------------
+        // Load c of a tile fills bytes [c KiB, (c+1) KiB) of the slot; lane i lands at byte c*1024 + 16 i =
+        // (row r, position q) of the [16][SLICE] image and fetches piece q ^ swz(r) of that row's slice.
+        // swz: the rows that share a 256-byte bank period get different values (rows 0..15 all different for
+        // SLICE >= 256; pairs / quads of rows for the shorter slices).
+        auto swz = [](int r) { return GW >= 4 ? (r & 15) & (GW * 4 - 1) : GW == 2 ? (r >> 1) & 7 : (r >> 2) & 3; };
+        uint32_t w_off[GW];
+#pragma unroll
+        for (int c = 0; c < GW; ++c)
+        {
+            const int pos = c * 1024 + 16 * lane;
+            const int r = pos / SLICE, q = (pos % SLICE) >> 4;
+            w_off[c] = (uint32_t)r * ROW_BYTES + (uint32_t)wave * SLICE + (uint32_t)((q ^ swz(r)) << 4);
+        }
+        // scales: lane l fetches 4 bytes (two groups) of row l / SC_LANES; GW = 1: the 4 bytes that hold this
+        // wavefront's group and its neighbour's
+        const int s_row = min(lane / SC_LANES, 15);
+        const uint32_t s_off = (uint32_t)s_row * (G * 2) +
+                               (GW >= 2 ? (uint32_t)wave * (GW * 2) + (uint32_t)(lane % SC_LANES) * 4u : (uint32_t)(wave & ~1) * 2u);
+
+        auto issue = [&](int tile, int slot) {
+            const uint32_t row0 = (uint32_t)row0_of(tile);
+            const uint8_t* wsrc = Wq + (size_t)row0 * ROW_BYTES;
+#pragma unroll
+            for (int c = 0; c < GW; ++c)
+                __builtin_amdgcn_global_load_lds((mr_global_ptr_t)(wsrc + w_off[c]),
+                                                 (mr_lds_ptr_t)(ring + slot * TILE_BYTES + c * 1024), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((mr_global_ptr_t)(reinterpret_cast<const uint8_t*>(S) + (size_t)row0 * (G * 2) + s_off),
+                                             (mr_lds_ptr_t)(sc_ring + slot * 256), 4, 0, 0);
+        };
+
+        // ---- the first two tiles, then the activations: straight into the MFMA operand registers -----------------
+        // (the activations are requested last: vector-memory operations complete in order and the compiler waits
+        // for them where they are used, which then also covers the two tiles -- requested first, those tiles'
+        // loads are not held back by anything)
+        issue(t0, 0);
+        issue(t0 + min(1, T - 1), 1);
+        uintx4 areg[GW][4];
+        {
+            const uint8_t* a_bytes = reinterpret_cast<const uint8_t*>(A);
+            const uint32_t a_off = (uint32_t)min(col, M - 1) * (uint32_t)(K * 2) + (uint32_t)wave * (GW * 256) + (uint32_t)kq * 64u;
+#pragma unroll
+            for (int g = 0; g < GW; ++g)
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    areg[g][j] = *reinterpret_cast<const uintx4*>(a_bytes + (size_t)(a_off + g * 256 + j * 16));
+        }
+        floatx4 ncorr[GW];
+        {
+            const half2_t sixteenth = half2_t{(half_t)0.0625f, (half_t)0.0625f};
+            const half_t ceh = (half_t)(-(1024.0f + (float)zp)), coh = (half_t)(-16.0f * (64.0f + (float)zp)); // exact
+            const uint32_t ce2 = as_u32(half2_t{ceh, ceh}), co2 = as_u32(half2_t{coh, coh});
+            const uintx4 cvec = {ce2, co2, ce2, co2};
+#pragma unroll
+            for (int g = 0; g < GW; ++g)
+            {
+                floatx4 t = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                {
+                    uintx4 a = permute_a8(areg[g][j]);
+                    a.y = as_u32(as_half2(a.y) * sixteenth);
+                    a.w = as_u32(as_half2(a.w) * sixteenth);
+                    areg[g][j] = a;
+                    t = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, a), __builtin_bit_cast(half8_t, cvec), t,
+                                                               0, 0, 0);
+                }
+                ncorr[g] = t;
+            }
+        }
+
+        // ---- tile loop ---------------------------------------------------------------------------------------
+        // operand reads of a slot: lane (n = col, kq), group g: piece g*4 + kq of row n
+        const uint32_t rd_base = (uint32_t)col * SLICE;
+        const int rd_swz = swz(col);
+        const uint32_t red_addr = lds_address(red) + (uint32_t)(wave * 1024 + lane * 16);
+        const uint32_t parked_addr = lds_address(parked);
+        for (int it = 0; it < T; ++it)
+        {
+            const int slot = it & 1;
+            // this tile has landed when at most the next tile's loads are outstanding
+            __builtin_amdgcn_s_waitcnt(mr_vmcnt(LT));
+            uintx4 wv[GW];
+            float sv[GW];
+            {
+                const uint8_t* sl = ring + slot * TILE_BYTES + rd_base;
+                const half_t* sc = reinterpret_cast<const half_t*>(sc_ring + slot * 256);
+#pragma unroll
+                for (int g = 0; g < GW; ++g)
+                {
+                    wv[g] = *reinterpret_cast<const uintx4*>(sl + (((g * 4 + kq) ^ rd_swz) << 4));
+                    sv[g] = GW >= 2 ? (float)sc[col * GW + g] : (float)sc[col * 2 + (wave & 1)];
+                }
+            }
+            // the slot has been read before it is refilled (past the end: a valid tile again, so that the wait
+            // count above holds for every iteration)
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            issue(t0 + min(it + 2, T - 1), slot);
+
+            floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int g = 0; g < GW; ++g)
+            {
+                floatx4 t = ncorr[g];
+                const uint32_t ww[4] = {wv[g].x, wv[g].y, wv[g].z, wv[g].w};
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                {
+                    const uint32_t w = ww[j];
+                    const uint32_t w8 = w >> 8;
+                    uintx4 bq;
+                    bq.x = (w & MASK_LO) | MAGIC;  // 1024 + (q0, q4)
+                    bq.y = (w & MASK_HI) | MAGIC;  // 1024 + 16 (q1, q5)
+                    bq.z = (w8 & MASK_LO) | MAGIC; // 1024 + (q2, q6)
+                    bq.w = (w8 & MASK_HI) | MAGIC; // 1024 + 16 (q3, q7)
+                    t = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, areg[g][j]),
+                                                               __builtin_bit_cast(half8_t, bq), t, 0, 0, 0);
+                }
+                acc.x = __builtin_fmaf(t.x, sv[g], acc.x);
+                acc.y = __builtin_fmaf(t.y, sv[g], acc.y);
+                acc.z = __builtin_fmaf(t.z, sv[g], acc.z);
+                acc.w = __builtin_fmaf(t.w, sv[g], acc.w);
+            }
+            // partial tile -> LDS (D layout: lane (n = col, kq), element e: row m = 4 kq + e)
+            {
+                const uint32_t at = red_addr + (uint32_t)(slot * MR_WAVES * 1024);
+                asm volatile("ds_write_b128 %0, %1" ::"v"(at), "v"(acc) : "memory");
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+            // 256 threads: thread (e, lane') adds the eight partial sums of output (m = 4 (lane' >> 4) + e, n = lane' & 15)
+            if (tid < 256)
+            {
+                const int e = tid >> 6;
+                const float* rp = reinterpret_cast<const float*>(red + slot * MR_WAVES * 1024) + lane * 4 + e;
+                float sum = 0.f;
+#pragma unroll
+                for (int w = 0; w < MR_WAVES; ++w)
+                    sum += rp[w * 256];
+                const int m = 4 * kq + e;
+                if (m < M)
+                {
+                    const uint32_t at = parked_addr + (uint32_t)(((it * M + m) * 16 + col) * 4);
+                    asm volatile("ds_write_b32 %0, %1" ::"v"(at), "v"(sum) : "memory");
+                }
+            }
+        }
+        __builtin_amdgcn_s_waitcnt(mr_vmcnt(0)); // the reloads past the end, before the LDS goes away
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        // ---- flush: parked sums -> Y -----------------------------------------------------------------------------
+        for (int idx = tid; idx < T * M * 16; idx += 512)
+        {
+            const int n = idx & 15;
+            const int im = idx >> 4;
+            const int it = im / M, m = im - it * M;
+            Y[(size_t)m * N + min((t0 + it) * 16, N - 16) + n] = (half_t)parked[idx];
+        }
+    }
+
+    namespace
+    {
+        template <int GW>
+        hipError_t launch_mrows(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M, int N, int zp,
+                                int num_cu)
+        {
+            const int n_tiles = (N + 15) / 16;
+            const int grid = n_tiles < num_cu ? n_tiles : num_cu;
+            const int tiles_q = n_tiles / grid, tiles_r = n_tiles % grid;
+            const size_t lds = workspace::w4a16_mrows_lds_bytes(GW << 10, M, tiles_q + (tiles_r ? 1 : 0));
+            if (lds > MAX_LDS_BYTES)
+                return hipErrorInvalidValue;
+            auto kernel = &w4a16_mrows_kernel<GW>;
+            if (lds > 64 * 1024)
+            {
+                hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                   (int)lds);
+                if (e != hipSuccess)
+                    return e;
+            }
+            hipLaunchKernelGGL(kernel, dim3(grid), dim3(MR_WAVES * 64), lds, stream, (const half_t*)A, (const uint8_t*)Wq,
+                               (const half_t*)S, (half_t*)Y, N, tiles_q, tiles_r, M | (zp << 8));
+            return hipGetLastError();
+        }
+    } // namespace
+
+    bool w4a16_mrows_supported(int M, int N, int K, int num_cu) { return workspace::w4a16_mrows_fits(M, N, K, num_cu); }
+    bool w4a16_mrows_preferred(int M, int N, int K, int num_cu) { return workspace::w4a16_mrows_preferred(M, N, K, num_cu); }
+
+    hipError_t launch_w4a16_mrows(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M, int N,
+                                  int K, int zp, int num_cu)
+    {
+        if (!w4a16_mrows_supported(M, N, K, num_cu))
+            return hipErrorInvalidValue;
+        switch (K >> 10)
+        {
+        case 1: return launch_mrows<1>(stream, A, Wq, S, Y, M, N, zp, num_cu);
+        case 2: return launch_mrows<2>(stream, A, Wq, S, Y, M, N, zp, num_cu);
+        case 4: return launch_mrows<4>(stream, A, Wq, S, Y, M, N, zp, num_cu);
+        default: return launch_mrows<8>(stream, A, Wq, S, Y, M, N, zp, num_cu);
+        }
+    }
+} // namespace nnf

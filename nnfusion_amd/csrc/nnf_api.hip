@@ -134,7 +134,10 @@ int nnf_w4a16_gemm(nnf_stream_t stream, const void* A, const void* Wq, const voi
     const int force = nnf::g_tuning.force_path;
     if ((force == 0 || force == 4) && nnf::w4a16_gemv_rows_supported(M, N, K, dev.num_cu))
         return (int)nnf::launch_w4a16_gemv_rows((hipStream_t)stream, A, Wq, scales, Y, N, K, zp, dev.num_cu);
-    if ((force == 0 || force == 2 || force == 4) && M <= 16 && nnf::w4a16_skinny_supported(M, N, K))
+    if ((force == 5 && nnf::w4a16_mrows_supported(M, N, K, dev.num_cu)) ||
+        (force == 0 && nnf::w4a16_mrows_preferred(M, N, K, dev.num_cu)))
+        return (int)nnf::launch_w4a16_mrows((hipStream_t)stream, A, Wq, scales, Y, M, N, K, zp, dev.num_cu);
+    if ((force == 0 || force == 2 || force == 4 || force == 5) && M <= 16 && nnf::w4a16_skinny_supported(M, N, K))
         return (int)nnf::launch_w4a16_skinny((hipStream_t)stream, A, Wq, scales, Y, M, N, K, zp, dev.num_cu);
     if (force == 1 && M <= 16 && nnf::w4a16_gemv_supported(M, K))
         return (int)nnf::launch_w4a16_gemv((hipStream_t)stream, A, Wq, scales, Y, M, N, K, zp, dev.num_cu);
@@ -179,6 +182,8 @@ int nnf_w4a16_gemm_variant(nnf_stream_t stream, const void* A, const void* Wq, c
     switch (variant)
     {
     case NNF_W4A16_GEMV_ROWS:
+        if (M > 1 && nnf::w4a16_mrows_supported(M, N, K, dev.num_cu))
+            return (int)nnf::launch_w4a16_mrows((hipStream_t)stream, A, Wq, scales, Y, M, N, K, zp, dev.num_cu);
         if (!nnf::w4a16_gemv_rows_supported(M, N, K, dev.num_cu))
             return NNF_ERR_UNSUPPORTED_SHAPE;
         return (int)nnf::launch_w4a16_gemv_rows((hipStream_t)stream, A, Wq, scales, Y, N, K, zp, dev.num_cu);

@@ -337,6 +337,34 @@ namespace nnf
             const Q8SkinnyPlan pl = plan_w8a8_skinny(M, K);
             return pl.cps != 0 && pl.lds + 16 * 1024 <= LDS_BYTES_PER_CU;
         }
+        // ---- 2 .. 16 activation rows: the row-streaming MFMA kernel (w4a16_mrows.hip) ----
+        // One workgroup per CU, eight wavefronts that each own an eighth of K and keep their share of the activations
+        // in registers; K is a compile-time constant of the kernel (1, 2, 4 or 8 KiB of activations per row and
+        // wavefront-eighth).  LDS: per wavefront two slots of a 16-row weight tile and of its scales, two sets of
+        // eight partial tiles, and the workgroup's finished tiles parked until the end.
+        inline size_t w4a16_mrows_lds_bytes(int K, int M, int tiles)
+        {
+            return (size_t)8 * 2 * (K >> 10) * 1024 + 8 * 512 + 2 * 8 * 1024 + (size_t)tiles * M * 64;
+        }
+        inline bool w4a16_mrows_fits(int M, int N, int K, int num_cu)
+        {
+            if (M < 2 || M > 16 || N < 16 || num_cu < 1)
+                return false;
+            if (K != 1024 && K != 2048 && K != 4096 && K != 8192)
+                return false;
+            if ((size_t)N * (size_t)(K >> 1) >= ((size_t)1 << 32)) // 32-bit offsets over the weight rows
+                return false;
+            const int n_tiles = (N + 15) / 16;
+            const int grid = n_tiles < num_cu ? n_tiles : num_cu;
+            return w4a16_mrows_lds_bytes(K, M, (n_tiles + grid - 1) / grid) <= LDS_BYTES_PER_CU;
+        }
+        // Where the library picks it by itself: measured against the split-K MFMA GEMV on cold weights it is level at
+        // N = K = 4096 and 5-35 % faster elsewhere for K <= 4096 (most at small K and large N); at K = 8192 its
+        // 240-register wavefronts and two tiles per workgroup (N = 8192) lose 5-25 %.
+        inline bool w4a16_mrows_preferred(int M, int N, int K, int num_cu)
+        {
+            return K <= 4096 && w4a16_mrows_fits(M, N, K, num_cu);
+        }
         inline bool w4a16_variant_fits(int M, int N, int K, int variant, int num_cu)
         {
             if (M <= 0 || N <= 0 || K < 128 || (K & 127))
@@ -348,7 +376,7 @@ namespace nnf
                 return true;
             case 1: return w4a16_gemv_valu_fits(M, K);
             case 2: return w4a16_skinny_fits(M, N, K);
-            case 4: return plan_w4a16_rows(M, N, K, num_cu, 0).seg != 0;
+            case 4: return plan_w4a16_rows(M, N, K, num_cu, 0).seg != 0 || w4a16_mrows_fits(M, N, K, num_cu);
             default: return false;
             }
         }
