@@ -401,6 +401,27 @@ def run_extra(torch, np, dev, lib, datagen, ops):
                      "GB/s": round(w4a16_bytes(m, n, k) / us / 1e3, 1)})
     res["w4a16_gemm_N8192_K8192"] = rows
     del twq, ts
+    # the decode sweep's shapes with a handful of rows (batched decode; not one of the benchmark's configurations):
+    # cold weights, the time of the whole sweep per batch size
+    rows = []
+    shapes = [(12288, 4096), (4096, 4096), (22016, 4096), (4096, 11008)]
+    weights = []
+    for (sn, sk) in shapes:
+        _, wq, s = datagen.w4a16_case(0, 1, sn, sk)
+        weights.append((dev_t(wq), dev_t(s)))
+    for m in (2, 4, 8, 16):
+        total_us, total_bytes = 0.0, 0
+        for (sn, sk), (twq, ts) in zip(shapes, weights):
+            a = dev_t(datagen.normal_f16(0, datagen.S_ACT, (m, sk)))
+            y = torch.empty((m, sn), dtype=torch.float16, device=dev)
+            ws = torch.empty(max(lib.nnf_w4a16_gemm_workspace_bytes(m, sn, sk, GROUP), 256), dtype=torch.uint8, device=dev)
+            sets = copies_of(twq, ts)
+            total_us += time_cold_us(lambda w, sc: (lambda: ops.w4a16_gemm(a, w, sc, out=y, workspace=ws)), sets)
+            total_bytes += w4a16_bytes(m, sn, sk)
+            del sets
+        rows.append({"M": m, "us_per_sweep": round(total_us, 2), "GB/s": round(total_bytes / total_us / 1e3, 1)})
+    res["w4a16_decode_sweep_small_batches"] = rows
+    del weights
     # configs[3]: W8A8, N = K = 8192
     _, _, w8, s_ch = datagen.w8a8_case(0, 1, n, k)
     tw8, tsch = dev_t(w8), dev_t(s_ch)
