@@ -1,4 +1,4 @@
-// fp16 x int4 (g128) for 2 <= M <= 16 activation rows and K = 1024, 2048, 4096 or 8192: the memory pipeline of the
+// fp16 x int4 (g128) for 2 <= M <= 16 activation rows and K = 1024, 2048, ... 8192: the memory pipeline of the
 // row-streaming GEMV (w4a16_gemv_rows.hip) under the arithmetic of the M <= 16 MFMA kernel (w4a16_skinny.hip).
 //
 //   Y[M,N] = A[M,K] . ((Wq - zp) * S)^T
@@ -49,13 +49,13 @@ namespace nnf
                                                               const half_t* __restrict__ S, half_t* __restrict__ Y, int N,
                                                               int tiles_q, int tiles_r, int pack)
     {
-        static_assert(GW == 1 || GW == 2 || GW == 4 || GW == 8, "K = GW * 1024");
+        static_assert(GW >= 1 && GW <= 8, "K = GW * 1024");
         constexpr int K = GW * 1024, G = GW * 8;
         constexpr int ROW_BYTES = K / 2;       // a weight row
         constexpr int SLICE = GW * 64;         // a wavefront's bytes of a weight row
         constexpr int TILE_BYTES = 16 * SLICE; // = GW KiB: GW wavefront-wide loads
         constexpr int LT = GW + 1;             // loads per tile and wavefront (weights + scales)
-        constexpr int SC_LANES = GW >= 2 ? GW / 2 : 1; // 4-byte scale loads per row
+        constexpr int SC_LANES = (GW + 1) / 2; // 4-byte scale loads per row (odd GW: one half-word of a neighbour comes along)
         extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
         uint32_t MAGIC, MASK_LO, MASK_HI;
         asm volatile("v_mov_b32 %0, 0x64006400" : "=v"(MAGIC));
@@ -82,9 +82,10 @@ namespace nnf
         // ---- what each lane fetches -------------------------------------------------------------------------
         // Load c of a tile fills bytes [c KiB, (c+1) KiB) of the slot; lane i lands at byte c*1024 + 16 i =
         // (row r, position q) of the [16][SLICE] image and fetches piece q ^ swz(r) of that row's slice.
-        // swz: the rows that share a 256-byte bank period get different values (rows 0..15 all different for
-        // SLICE >= 256; pairs / quads of rows for the shorter slices).
-        auto swz = [](int r) { return GW >= 4 ? (r & 15) & (GW * 4 - 1) : GW == 2 ? (r >> 1) & 7 : (r >> 2) & 3; };
+        // swz: the rows whose slices start in the same 64-byte quarter of the 256-byte bank period get different
+        // values: all 16 rows when SLICE is a multiple of 256, 8 when of 128, else 4.  The XOR stays inside an
+        // aligned block of 16 / 8 / 4 pieces, which the slice is a multiple of.
+        auto swz = [](int r) { return GW % 4 == 0 ? (r & 15) : GW % 2 == 0 ? (r >> 1) & 7 : (r >> 2) & 3; };
         uint32_t w_off[GW];
 #pragma unroll
         for (int c = 0; c < GW; ++c)
@@ -93,11 +94,12 @@ namespace nnf
             const int r = pos / SLICE, q = (pos % SLICE) >> 4;
             w_off[c] = (uint32_t)r * ROW_BYTES + (uint32_t)wave * SLICE + (uint32_t)((q ^ swz(r)) << 4);
         }
-        // scales: lane l fetches 4 bytes (two groups) of row l / SC_LANES; GW = 1: the 4 bytes that hold this
-        // wavefront's group and its neighbour's
+        // scales: lane l fetches 4 bytes (two groups) of row l / SC_LANES, from the 4-byte boundary at or below the
+        // wavefront's first group (odd GW, odd wavefront: one group below it; sc_skip)
         const int s_row = min(lane / SC_LANES, 15);
         const uint32_t s_off = (uint32_t)s_row * (G * 2) +
-                               (GW >= 2 ? (uint32_t)wave * (GW * 2) + (uint32_t)(lane % SC_LANES) * 4u : (uint32_t)(wave & ~1) * 2u);
+                               (((uint32_t)wave * (GW * 2)) & ~3u) + (uint32_t)(lane % SC_LANES) * 4u;
+        const int sc_skip = (wave * GW) & 1;
 
         auto issue = [&](int tile, int slot) {
             const uint32_t row0 = (uint32_t)row0_of(tile);
@@ -170,7 +172,7 @@ namespace nnf
                 for (int g = 0; g < GW; ++g)
                 {
                     wv[g] = *reinterpret_cast<const uintx4*>(sl + (((g * 4 + kq) ^ rd_swz) << 4));
-                    sv[g] = GW >= 2 ? (float)sc[col * GW + g] : (float)sc[col * 2 + (wave & 1)];
+                    sv[g] = (float)sc[col * (SC_LANES * 2) + sc_skip + g];
                 }
             }
             // the slot has been read before it is refilled (past the end: a valid tile again, so that the wait
@@ -275,7 +277,11 @@ namespace nnf
         {
         case 1: return launch_mrows<1>(stream, A, Wq, S, Y, M, N, zp, num_cu);
         case 2: return launch_mrows<2>(stream, A, Wq, S, Y, M, N, zp, num_cu);
+        case 3: return launch_mrows<3>(stream, A, Wq, S, Y, M, N, zp, num_cu);
         case 4: return launch_mrows<4>(stream, A, Wq, S, Y, M, N, zp, num_cu);
+        case 5: return launch_mrows<5>(stream, A, Wq, S, Y, M, N, zp, num_cu);
+        case 6: return launch_mrows<6>(stream, A, Wq, S, Y, M, N, zp, num_cu);
+        case 7: return launch_mrows<7>(stream, A, Wq, S, Y, M, N, zp, num_cu);
         default: return launch_mrows<8>(stream, A, Wq, S, Y, M, N, zp, num_cu);
         }
     }

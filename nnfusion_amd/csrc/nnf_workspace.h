@@ -339,9 +339,9 @@ namespace nnf
         }
         // ---- 2 .. 16 activation rows: the row-streaming MFMA kernel (w4a16_mrows.hip) ----
         // One workgroup per CU, eight wavefronts that each own an eighth of K and keep their share of the activations
-        // in registers; K is a compile-time constant of the kernel (1, 2, 4 or 8 KiB of activations per row and
-        // wavefront-eighth).  LDS: per wavefront two slots of a 16-row weight tile and of its scales, two sets of
-        // eight partial tiles, and the workgroup's finished tiles parked until the end.
+        // in registers; K is a compile-time constant of the kernel (a multiple of 1024 up to 8192).  LDS: per
+        // wavefront two slots of a 16-row weight tile and of its scales, two sets of eight partial tiles, and the
+        // workgroup's finished tiles parked until the end.
         inline size_t w4a16_mrows_lds_bytes(int K, int M, int tiles)
         {
             return (size_t)8 * 2 * (K >> 10) * 1024 + 8 * 512 + 2 * 8 * 1024 + (size_t)tiles * M * 64;
@@ -350,7 +350,7 @@ namespace nnf
         {
             if (M < 2 || M > 16 || N < 16 || num_cu < 1)
                 return false;
-            if (K != 1024 && K != 2048 && K != 4096 && K != 8192)
+            if (K < 1024 || K > 8192 || (K & 1023)) // K / 1024 is a template parameter of the kernel
                 return false;
             if ((size_t)N * (size_t)(K >> 1) >= ((size_t)1 << 32)) // 32-bit offsets over the weight rows
                 return false;
@@ -358,12 +358,13 @@ namespace nnf
             const int grid = n_tiles < num_cu ? n_tiles : num_cu;
             return w4a16_mrows_lds_bytes(K, M, (n_tiles + grid - 1) / grid) <= LDS_BYTES_PER_CU;
         }
-        // Where the library picks it by itself: measured against the split-K MFMA GEMV on cold weights it is level at
-        // N = K = 4096 and 5-35 % faster elsewhere for K <= 4096 (most at small K and large N); at K = 8192 its
-        // 240-register wavefronts and two tiles per workgroup (N = 8192) lose 5-25 %.
+        // Where the library picks it by itself, from measurements against the split-K MFMA GEMV on cold weights:
+        // K <= 4096: level at N = K = 4096, 5-35 % faster elsewhere (most at small K and large N, and at M = 16);
+        // K = 5120 .. 7168: 5-30 % faster from eight rows on, level to 15 % slower below;
+        // K = 8192 (240 registers per lane): 5-25 % slower except at M = 16 with N >> 8192.
         inline bool w4a16_mrows_preferred(int M, int N, int K, int num_cu)
         {
-            return K <= 4096 && w4a16_mrows_fits(M, N, K, num_cu);
+            return (K <= 4096 || (K <= 7168 && M >= 8)) && w4a16_mrows_fits(M, N, K, num_cu);
         }
         inline bool w4a16_variant_fits(int M, int N, int K, int variant, int num_cu)
         {

@@ -18,7 +18,7 @@ TOL = 1e-2
 def path(request):
     """Runs a test once per kernel family that can serve M <= 16 (auto = the library's own choice;
     rows_gemv = the M = 1 row-streaming kernel where it applies, otherwise the library's choice;
-    mfma_rows = the row-streaming MFMA kernel for 2 <= M <= 16 and K = 1024 .. 8192 where it applies)."""
+    mfma_rows = the row-streaming MFMA kernel for 2 <= M <= 16 and K = 1024, 2048 .. 8192 where it applies)."""
     from nnfusion_amd import _lib
 
     tune = _lib.kernels().nnf_internal_tune
@@ -60,7 +60,7 @@ def _check(y, ref):
     # a handful of rows through the row-streaming MFMA kernel: every K it takes, ragged N, more tiles than CUs,
     # fewer tiles than CUs, a single tile
     (2, 4096, 1024), (3, 8200, 2048), (16, 4111, 4096), (9, 22016, 4096), (16, 12288, 8192), (6, 16, 8192), (11, 48, 2048),
-    (16, 40000, 1024),
+    (16, 40000, 1024), (5, 4096, 3072), (16, 13824, 5120), (7, 1000, 6144), (16, 2050, 7168), (2, 640, 5120),
 ])
 def test_gemv_matches_oracle(gpu, path, m, n, k):
     print(f"case M={m} N={n} K={k}", flush=True)
@@ -124,7 +124,7 @@ def test_gemv_other_zero_points(gpu, path, zp):
     _check(y, ref)
 
 
-@pytest.mark.parametrize("m,n,k", [(1, 512, 4096), (8, 300, 2048), (16, 128, 8192), (40, 256, 1024), (8, 300, 3072)])
+@pytest.mark.parametrize("m,n,k", [(1, 512, 4096), (8, 300, 2048), (16, 128, 8192), (40, 256, 1024), (8, 300, 3072), (8, 300, 2176)])
 def test_every_kernel_variant_that_accepts_a_shape_matches_the_oracle(gpu, m, n, k):
     """nnf_w4a16_gemm_variant: the entry point behind the per-variant emitters of profiling-based kernel selection.
     nnf_w4a16_variant_supported (host only) and the call itself agree on which variants serve a shape."""
@@ -148,5 +148,5 @@ def test_every_kernel_variant_that_accepts_a_shape_matches_the_oracle(gpu, m, n,
                 ops.w4a16_gemm_variant(ta, tw, ts, name)
             assert e.value.status == -2
     assert "auto" in served and "gemm_mfma" in served
-    assert ("gemv_rows" in served) == (m == 1 or (m <= 16 and k in (1024, 2048, 4096, 8192)))
+    assert ("gemv_rows" in served) == (m == 1 or (m <= 16 and k % 1024 == 0 and k <= 8192))
     assert ("gemv_valu" in served) == (m <= 16)
