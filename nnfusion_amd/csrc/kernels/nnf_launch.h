@@ -61,6 +61,11 @@ namespace nnf
     hipError_t launch_w8a8_gemv_rows(hipStream_t stream, const void* A, const void* s_tok, const void* W, const void* s_ch,
                                      void* Y, void* acc, int N, int K, int num_cu);
     bool w8a8_gemv_rows_supported(int M, int N, int K, int num_cu);
+    // 2 <= M <= 32, K = 2048, 4096, 6144 or 8192: the row-streaming MFMA kernel (w8a8_mrows.hip)
+    hipError_t launch_w8a8_mrows(hipStream_t stream, const void* A, const void* s_tok, const void* W, const void* s_ch,
+                                 void* Y, void* acc, int M, int N, int K, int num_cu);
+    bool w8a8_mrows_supported(int M, int N, int K, int num_cu);
+    bool w8a8_mrows_preferred(int M, int N, int K, int num_cu); // where the library picks it without being told
 
     // Tuning knobs for experiments (not part of the public ABI): 0 = automatic.
     struct Tuning

@@ -275,6 +275,9 @@ namespace nnf
         const bool raw = acc != nullptr;
         if ((g_tuning.force_path == 0 || g_tuning.force_path == 4) && w8a8_gemv_rows_supported(M, N, K, num_cu))
             return launch_w8a8_gemv_rows(stream, A, s_tok, W, s_ch, Y, acc, N, K, num_cu);
+        if ((g_tuning.force_path == 5 && w8a8_mrows_supported(M, N, K, num_cu)) ||
+            (g_tuning.force_path == 0 && w8a8_mrows_preferred(M, N, K, num_cu)))
+            return launch_w8a8_mrows(stream, A, s_tok, W, s_ch, Y, acc, M, N, K, num_cu);
         const bool skinny = g_tuning.force_path != 3 && w8a8_skinny_supported(M, K);
         if (skinny)
             return raw ? launch_q8_skinny<true>(stream, p, num_cu) : launch_q8_skinny<false>(stream, p, num_cu);

@@ -1,0 +1,263 @@
+// W8A8 (int8 x int8 -> int32, exact) for 2 <= M <= 32 activation rows and K = 2048, 4096, 6144 or 8192: the
+// row-streaming kernel of w4a16_mrows.hip on the int8 matrix cores.
+//
+//   acc[M,N] = A[M,K] . W[N,K]^T  (int32, bit exact);  Y = fp16((float)acc * s_tok[m] * s_ch[n])
+//
+// Replaces the cublas GEMM behind cuda::Dot (src/nnfusion/core/kernels/cuda_gpu/kernels/dot.cpp:271-363) for an
+// int8-quantized Dot node with a few activation rows.
+//
+//   * One workgroup of eight wavefronts per CU owns a contiguous run of 16-row weight tiles.  All eight work on
+//     the same tile, in steps of 2 KiB of K: wavefront w owns bytes [256 w, 256 (w+1)) of every step, so that the
+//     workgroup's loads of a step cover 2 KiB of each of the 16 rows without gaps.
+//   * A step of a wavefront (16 rows x 256 bytes = 4 KiB) goes global -> LDS without registers
+//     (global_load_lds_dwordx4, four wavefront-wide loads) into a private ring of NS slots; a slot is requested
+//     again as soon as it has been copied into registers (16 VGPRs).  Nothing but the wavefront's own loads
+//     feeds its MFMAs: no barrier on the load path.  The 16-byte pieces of a row are XOR-swizzled with the row
+//     number on the way (each lane chooses which piece it fetches): conflict-free 128-bit operand reads.
+//   * The activations never touch LDS: lane (m, kq) loads the 16 bytes of row m that its MFMA operand holds of
+//     every 64-byte chunk of the wavefront's slice, once, and keeps them (K/512 x 4 VGPRs per block of 16 rows).
+//   * Per step 4 (M <= 16) or 8 v_mfma_i32_16x16x64_i8, weights as the B operand.  Per tile the eight partial
+//     16 x 16 (x 2) tiles meet in LDS (one LDS-only barrier, two alternating buffers), integer adds (the result
+//     does not depend on the order); the sums are parked in LDS and scaled / written after the last tile.
+//   * LDS writes inside the loop are inline ds_write instructions: ahead of an LDS write that it can see, the
+//     compiler waits for every LDS-bound load in flight.
+#include "nnf_device.h"
+#include "nnf_launch.h"
+
+#include "../nnf_workspace.h"
+
+namespace nnf
+{
+    namespace
+    {
+        constexpr int Q8MR_WAVES = 8;
+        constexpr int Q8MR_STEP_BYTES = 256;                   // of a weight row, per wavefront and step
+        constexpr int Q8MR_SLOT_BYTES = 16 * Q8MR_STEP_BYTES;  // 4 KiB: four wavefront-wide loads
+        typedef const void __attribute__((address_space(1))) * q8mr_global_ptr_t;
+        typedef void __attribute__((address_space(3))) * q8mr_lds_ptr_t;
+        // s_waitcnt with only the vector-memory counter set (gfx9 encoding: vmcnt = bits 3:0 and 15:14)
+        constexpr int q8mr_vmcnt(int n) { return (n & 0xF) | ((n >> 4) << 14) | (0x7 << 4) | (0xF << 8); }
+    } // namespace
+
+    // LDS (bytes): weights [8 wavefronts][NS slots][4 KiB] | partial tiles [2][8][MB KiB] |
+    //              parked sums [tiles of the workgroup][M][16] int32
+    // STEPS = K / 2048 (steps per tile and wavefront), MB = blocks of 16 activation rows (1 or 2), NS = ring slots.
+    // A workgroup's tiles: tiles_q, one more for the first tiles_r workgroups.
+    template <int STEPS, int MB, int NS, bool RAW_ACC>
+    __global__ __launch_bounds__(512) void w8a8_mrows_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ W,
+                                                             const float* __restrict__ s_tok, const float* __restrict__ s_ch,
+                                                             half_t* __restrict__ Y, int32_t* __restrict__ ACC, int M, int N,
+                                                             int tiles_q, int tiles_r)
+    {
+        static_assert(STEPS >= 1 && STEPS <= 4 && (MB == 1 || MB == 2) && NS >= 2 && NS <= 4, "shape of the kernel");
+        constexpr int K = STEPS * 2048;
+        constexpr int CH = K / 8 / 64;   // a wavefront's 64-byte chunks of a row (one MFMA each)
+        constexpr int LPS = 4;           // loads per step and wavefront
+        extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+
+        const int tid = threadIdx.x;
+        const int lane = tid & 63;
+        const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+        const int col = lane & 15; // n within the tile (B operand / D column), m for the A operand
+        const int kq = lane >> 4;  // K quarter of the MFMA operands, row quad of D
+        const int b = blockIdx.x;
+        const int t0 = b * tiles_q + min(b, tiles_r);
+        const int T = tiles_q + (b < tiles_r ? 1 : 0);
+        // the last tile of an N that is not a multiple of 16 is moved back to rows N-16 .. N-1
+        auto row0_of = [&](int tile) { return __builtin_amdgcn_readfirstlane(min(tile * 16, N - 16)); };
+
+        uint8_t* ring = smem + wave * (NS * Q8MR_SLOT_BYTES);
+        uint8_t* red = smem + Q8MR_WAVES * NS * Q8MR_SLOT_BYTES; // [2][8][MB][1024]
+        int32_t* parked = reinterpret_cast<int32_t*>(red + 2 * Q8MR_WAVES * MB * 1024);
+
+        // ---- what each lane fetches -------------------------------------------------------------------------
+        // Load c of a step fills bytes [c KiB, (c+1) KiB) of the slot; lane i lands at byte c*1024 + 16 i =
+        // (row r = 4c + i/16, position q = i%16) of the [16][256] image and fetches piece q ^ r of that row's step.
+        uint32_t w_off[LPS];
+#pragma unroll
+        for (int c = 0; c < LPS; ++c)
+        {
+            const int r = c * 4 + kq, q = col;
+            w_off[c] = (uint32_t)r * K + (uint32_t)wave * Q8MR_STEP_BYTES + (uint32_t)((q ^ r) << 4);
+        }
+        // step st (0 .. STEPS-1) of tile `tile` into slot `slot`
+        auto issue = [&](int tile, int st, int slot) {
+            const int8_t* wsrc = W + (size_t)row0_of(tile) * K + st * (Q8MR_WAVES * Q8MR_STEP_BYTES);
+#pragma unroll
+            for (int c = 0; c < LPS; ++c)
+                __builtin_amdgcn_global_load_lds((q8mr_global_ptr_t)(wsrc + w_off[c]),
+                                                 (q8mr_lds_ptr_t)(ring + slot * Q8MR_SLOT_BYTES + c * 1024), 16, 0, 0);
+        };
+
+        // ---- the first NS steps, then the activations: straight into the MFMA operand registers -----------------
+        // (the activations are requested last: vector-memory operations complete in order and the compiler waits
+        // for them where they are used, which then also covers the first steps -- requested first, those are not
+        // held back by anything)
+#pragma unroll
+        for (int s = 0; s < NS; ++s)
+            issue(t0 + min(s / STEPS, T - 1), s % STEPS, s);
+        uintx4 areg[MB][CH];
+        {
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb)
+            {
+                const uint32_t a_off = (uint32_t)min(mb * 16 + col, M - 1) * (uint32_t)K + (uint32_t)wave * Q8MR_STEP_BYTES + (uint32_t)kq * 16u;
+#pragma unroll
+                for (int c = 0; c < CH; ++c)
+                    areg[mb][c] = *reinterpret_cast<const uintx4*>(reinterpret_cast<const uint8_t*>(A) +
+                                                                    (size_t)(a_off + (c >> 2) * (Q8MR_WAVES * Q8MR_STEP_BYTES) + (c & 3) * 64));
+            }
+        }
+
+        // ---- tile loop ---------------------------------------------------------------------------------------
+        // operand reads of a slot: lane (n = col, kq), chunk c of the step: piece c*4 + kq of row n
+        const uint32_t rd_base = (uint32_t)col * Q8MR_STEP_BYTES;
+        const uint32_t red_addr = lds_address(red) + (uint32_t)(wave * (MB * 1024) + lane * 16);
+        const uint32_t parked_addr = lds_address(parked);
+        // step s of the workgroup sits in slot s % NS; NS and STEPS are small: walk the slot number by hand
+        int slot = 0;
+        for (int it = 0; it < T; ++it)
+        {
+            intx4 acc[MB];
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb)
+                acc[mb] = intx4{0, 0, 0, 0};
+#pragma unroll
+            for (int st = 0; st < STEPS; ++st)
+            {
+                // this step has landed when at most the NS-1 steps requested after it are outstanding
+                __builtin_amdgcn_s_waitcnt(q8mr_vmcnt((NS - 1) * LPS));
+                uintx4 wv[4];
+                {
+                    const uint8_t* sl = ring + slot * Q8MR_SLOT_BYTES + rd_base;
+#pragma unroll
+                    for (int c = 0; c < 4; ++c)
+                        wv[c] = *reinterpret_cast<const uintx4*>(sl + (((c * 4 + kq) ^ col) << 4));
+                }
+                // the slot has been read before it is refilled: step s + NS (past the end: a valid tile again, so
+                // that the wait count above holds for every step)
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                issue(t0 + min(it + (st + NS) / STEPS, T - 1), (st + NS) % STEPS, slot);
+                slot = slot + 1 == NS ? 0 : slot + 1;
+#pragma unroll
+                for (int c = 0; c < 4; ++c)
+#pragma unroll
+                    for (int mb = 0; mb < MB; ++mb)
+                        acc[mb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(intx4, areg[mb][st * 4 + c]),
+                                                                        __builtin_bit_cast(intx4, wv[c]), acc[mb], 0, 0, 0);
+            }
+            // partial tiles -> LDS (D layout: lane (n = col, kq), element e: row m = 16 mb + 4 kq + e)
+            const int rbuf = it & 1;
+            // The accumulators come straight from the matrix cores, and the writes below are inline instructions:
+            // the compiler does not count the wait states between an MFMA and an LDS instruction that reads its
+            // result for them (up to 18 for this MFMA).  These no-ops, tied to the registers, stand in.
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb)
+                asm volatile("s_nop 15\n\ts_nop 7" : "+v"(acc[mb]));
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb)
+            {
+                const uint32_t at = red_addr + (uint32_t)(rbuf * Q8MR_WAVES * MB * 1024 + mb * 1024);
+                asm volatile("ds_write_b128 %0, %1" ::"v"(at), "v"(acc[mb]) : "memory");
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+            // MB x 256 threads: thread (mb, e, lane') adds the eight partial sums of output
+            // (m = 16 mb + 4 (lane' >> 4) + e, n = lane' & 15)
+            if (tid < MB * 256)
+            {
+                const int mb = tid >> 8, e = (tid >> 6) & 3;
+                const int32_t* rp = reinterpret_cast<const int32_t*>(red + rbuf * Q8MR_WAVES * MB * 1024 + mb * 1024) + lane * 4 + e;
+                int32_t sum = 0;
+#pragma unroll
+                for (int w = 0; w < Q8MR_WAVES; ++w)
+                    sum += rp[w * (MB * 256)];
+                const int m = 16 * mb + 4 * kq + e;
+                if (m < M)
+                {
+                    const uint32_t at = parked_addr + (uint32_t)(((it * M + m) * 16 + col) * 4);
+                    asm volatile("ds_write_b32 %0, %1" ::"v"(at), "v"(sum) : "memory");
+                }
+            }
+        }
+        __builtin_amdgcn_s_waitcnt(q8mr_vmcnt(0)); // the reloads past the end, before the LDS goes away
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        // ---- flush: parked sums -> Y (scaled) or ACC ---------------------------------------------------------------
+        for (int idx = tid; idx < T * M * 16; idx += 512)
+        {
+            const int n = idx & 15;
+            const int im = idx >> 4;
+            const int it = im / M, m = im - it * M;
+            const int gn = min((t0 + it) * 16, N - 16) + n;
+            if (RAW_ACC)
+            {
+                ACC[(size_t)m * N + gn] = parked[idx];
+            }
+            else
+            {
+                const float t = (float)parked[idx] * s_tok[m];
+                Y[(size_t)m * N + gn] = f32_to_f16_two_step(t * s_ch[gn]);
+            }
+        }
+    }
+
+    namespace
+    {
+        template <int STEPS, int MB, int NS, bool RAW>
+        hipError_t launch_q8_mrows(hipStream_t stream, const void* A, const void* s_tok, const void* W, const void* s_ch, void* Y,
+                                   void* acc, int M, int N, int num_cu)
+        {
+            const int n_tiles = (N + 15) / 16;
+            const int grid = n_tiles < num_cu ? n_tiles : num_cu;
+            const int tiles_q = n_tiles / grid, tiles_r = n_tiles % grid;
+            const size_t lds = workspace::w8a8_mrows_lds_bytes(M, NS, tiles_q + (tiles_r ? 1 : 0));
+            if (lds > MAX_LDS_BYTES)
+                return hipErrorInvalidValue;
+            auto kernel = &w8a8_mrows_kernel<STEPS, MB, NS, RAW>;
+            if (lds > 64 * 1024)
+            {
+                hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                   (int)lds);
+                if (e != hipSuccess)
+                    return e;
+            }
+            hipLaunchKernelGGL(kernel, dim3(grid), dim3(Q8MR_WAVES * 64), lds, stream, (const int8_t*)A, (const int8_t*)W,
+                               (const float*)s_tok, (const float*)s_ch, (half_t*)Y, (int32_t*)acc, M, N, tiles_q, tiles_r);
+            return hipGetLastError();
+        }
+
+        template <int STEPS, bool RAW>
+        hipError_t launch_q8_mrows_m(hipStream_t stream, const void* A, const void* s_tok, const void* W, const void* s_ch,
+                                     void* Y, void* acc, int M, int N, int num_cu)
+        {
+            constexpr int NS = workspace::W8A8_MROWS_SLOTS;
+            return M <= 16 ? launch_q8_mrows<STEPS, 1, NS, RAW>(stream, A, s_tok, W, s_ch, Y, acc, M, N, num_cu)
+                           : launch_q8_mrows<STEPS, 2, NS, RAW>(stream, A, s_tok, W, s_ch, Y, acc, M, N, num_cu);
+        }
+
+        template <bool RAW>
+        hipError_t launch_q8_mrows_any(hipStream_t stream, const void* A, const void* s_tok, const void* W, const void* s_ch,
+                                       void* Y, void* acc, int M, int N, int K, int num_cu)
+        {
+            switch (K >> 11)
+            {
+            case 1: return launch_q8_mrows_m<1, RAW>(stream, A, s_tok, W, s_ch, Y, acc, M, N, num_cu);
+            case 2: return launch_q8_mrows_m<2, RAW>(stream, A, s_tok, W, s_ch, Y, acc, M, N, num_cu);
+            case 3: return launch_q8_mrows_m<3, RAW>(stream, A, s_tok, W, s_ch, Y, acc, M, N, num_cu);
+            default: return launch_q8_mrows_m<4, RAW>(stream, A, s_tok, W, s_ch, Y, acc, M, N, num_cu);
+            }
+        }
+    } // namespace
+
+    bool w8a8_mrows_supported(int M, int N, int K, int num_cu) { return workspace::w8a8_mrows_fits(M, N, K, num_cu); }
+    bool w8a8_mrows_preferred(int M, int N, int K, int num_cu) { return workspace::w8a8_mrows_preferred(M, N, K, num_cu); }
+
+    // acc != nullptr: the raw int32 sums, otherwise Y = fp16(acc * s_tok[m] * s_ch[n])
+    hipError_t launch_w8a8_mrows(hipStream_t stream, const void* A, const void* s_tok, const void* W, const void* s_ch, void* Y,
+                                 void* acc, int M, int N, int K, int num_cu)
+    {
+        if (!w8a8_mrows_supported(M, N, K, num_cu))
+            return hipErrorInvalidValue;
+        return acc ? launch_q8_mrows_any<true>(stream, A, s_tok, W, s_ch, Y, acc, M, N, K, num_cu)
+                   : launch_q8_mrows_any<false>(stream, A, s_tok, W, s_ch, Y, acc, M, N, K, num_cu);
+    }
+} // namespace nnf

@@ -248,6 +248,9 @@ static int check_w8a8_workspace(int M, int N, int K, int num_cu, const void* wor
 {
     if ((nnf::g_tuning.force_path == 0 || nnf::g_tuning.force_path == 4) && nnf::w8a8_gemv_rows_supported(M, N, K, num_cu))
         return NNF_OK;
+    if ((nnf::g_tuning.force_path == 5 && nnf::w8a8_mrows_supported(M, N, K, num_cu)) ||
+        (nnf::g_tuning.force_path == 0 && nnf::w8a8_mrows_preferred(M, N, K, num_cu)))
+        return NNF_OK;
     if (nnf::g_tuning.force_path != 3 && nnf::w8a8_skinny_supported(M, K))
         return NNF_OK;
     const size_t need = nnf::workspace::gemm_partial_bytes(

@@ -337,6 +337,30 @@ namespace nnf
             const Q8SkinnyPlan pl = plan_w8a8_skinny(M, K);
             return pl.cps != 0 && pl.lds + 16 * 1024 <= LDS_BYTES_PER_CU;
         }
+        // ---- W8A8, 2 .. 32 activation rows: the row-streaming MFMA kernel (w8a8_mrows.hip) ----
+        // One workgroup per CU, eight wavefronts that each own an eighth of K (256 bytes of every 2 KiB) and keep
+        // their share of the activations in registers.  LDS: per wavefront a ring of 4-KiB slots, two sets of eight
+        // partial tiles (one or two blocks of 16 rows), the workgroup's finished tiles parked until the end.
+        // Two slots (64 KiB in flight per CU) measured 2-9 % faster than three.
+        constexpr int W8A8_MROWS_SLOTS = 2;
+        inline size_t w8a8_mrows_lds_bytes(int M, int slots, int tiles)
+        {
+            return (size_t)8 * slots * 4096 + (size_t)2 * 8 * (M <= 16 ? 1 : 2) * 1024 + (size_t)tiles * M * 64;
+        }
+        inline bool w8a8_mrows_fits(int M, int N, int K, int num_cu)
+        {
+            if (M < 2 || M > 32 || N < 16 || num_cu < 1)
+                return false;
+            if (K < 2048 || K > 8192 || (K & 2047)) // K / 2048 is a template parameter of the kernel
+                return false;
+            const int n_tiles = (N + 15) / 16;
+            const int grid = n_tiles < num_cu ? n_tiles : num_cu;
+            return w8a8_mrows_lds_bytes(M, W8A8_MROWS_SLOTS, (n_tiles + grid - 1) / grid) <= LDS_BYTES_PER_CU;
+        }
+        // Where the library picks it by itself: everywhere it applies.  Measured on cold weights against the split-K
+        // M <= 16 kernel it is level to 10 % faster up to M = 14 (2 % slower at M = 2, N = K = 8192), 5-30 % faster at
+        // M = 16, and 12-33 % faster than the MFMA tile GEMM at M = 17 .. 32.
+        inline bool w8a8_mrows_preferred(int M, int N, int K, int num_cu) { return w8a8_mrows_fits(M, N, K, num_cu); }
         // ---- 2 .. 16 activation rows: the row-streaming MFMA kernel (w4a16_mrows.hip) ----
         // One workgroup per CU, eight wavefronts that each own an eighth of K and keep their share of the activations
         // in registers; K is a compile-time constant of the kernel (a multiple of 1024 up to 8192).  LDS: per

@@ -15,10 +15,11 @@ def _t(gpu, *arrays):
     return [torch.from_numpy(np.ascontiguousarray(a)).to(gpu) for a in arrays]
 
 
-# "auto": the library's own choice (the M = 1 / M <= 16 kernels where they apply); otherwise the MFMA GEMM with a
+# "auto": the library's own choice (the M = 1 / M <= 16 / M <= 32 kernels where they apply); "skinny": the split-K
+# M <= 16 kernel; "mfma_rows": the row-streaming MFMA kernel (2 <= M <= 32, K = 2048 .. 8192); otherwise the MFMA GEMM with a
 # forced tile (1 big 256x256, 2 mid 128x128, 3 small 64x256) and number of K ranges (int32 partial sums,
 # added exactly by the reduction pass)
-@pytest.fixture(params=["auto", "skinny", (0, 0), (1, 1), (1, 2), (2, 1), (2, 3), (3, 1), (3, 2)],
+@pytest.fixture(params=["auto", "skinny", "mfma_rows", (0, 0), (1, 1), (1, 2), (2, 1), (2, 3), (3, 1), (3, 2)],
                 ids=lambda p: p if isinstance(p, str) else f"gemm-tile{p[0]}-splits{p[1]}")
 def path(request):
     from nnfusion_amd import _lib
@@ -26,6 +27,8 @@ def path(request):
     tune = _lib.kernels().nnf_internal_tune
     if request.param == "skinny":
         tune(0, 2)  # the M <= 16 kernel where it applies (never the M = 1 row-streaming one)
+    elif request.param == "mfma_rows":
+        tune(0, 5)
     elif request.param != "auto":
         tune(0, 3)
         tune(3, request.param[0])
@@ -49,6 +52,10 @@ def _big_ws(gpu):
     (5, 200, 2176), (2, 100, 11008), (7, 48, 16384), (9, 1000, 8320), (1, 33000, 1024), (13, 8200, 4096),
     # one activation row: rows shared by 1..8 wavefronts, ragged last K segment, fewer rows than wavefronts
     (1, 300, 4096), (1, 4096, 11008), (1, 100, 16384), (1, 50, 2048), (1, 513, 5248), (1, 2000, 24576), (1, 40, 1152),
+    # 2 .. 32 rows through the row-streaming MFMA kernel: every K it takes, one and two blocks of 16 rows, ragged N,
+    # a single tile, more tiles than CUs
+    (2, 512, 2048), (16, 4111, 4096), (17, 1000, 6144), (32, 8192, 8192), (31, 16, 8192), (24, 12288, 4096),
+    (8, 40000, 2048), (20, 77, 4096),
 ])
 def test_accumulators_bit_exact(gpu, path, m, n, k):
     import torch
