@@ -44,17 +44,19 @@ namespace nnf
     // LDS (bytes): weights [8 wavefronts][2 slots][GW KiB] | scales [8][2][256] | partial tiles [2][8][1 KiB] |
     //              parked sums [tiles of the workgroup][M][16] fp32
     // pack = M | zp << 8;  a workgroup's tiles: tiles_q, one more for the first tiles_r workgroups.
-    template <int GW>
+    template <int GW, int STEPS>
     __global__ __launch_bounds__(512) void w4a16_mrows_kernel(const half_t* __restrict__ A, const uint8_t* __restrict__ Wq,
                                                               const half_t* __restrict__ S, half_t* __restrict__ Y, int N,
                                                               int tiles_q, int tiles_r, int pack)
     {
-        static_assert(GW >= 1 && GW <= 8, "K = GW * 1024");
-        constexpr int K = GW * 1024, G = GW * 8;
+        static_assert(GW >= 1 && GW <= 8 && STEPS >= 1 && GW * STEPS <= 8, "K = GW * STEPS * 1024");
+        constexpr int K = GW * STEPS * 1024, G = K / 128;
+        constexpr int GA = GW * STEPS;         // groups of a wavefront
         constexpr int ROW_BYTES = K / 2;       // a weight row
-        constexpr int SLICE = GW * 64;         // a wavefront's bytes of a weight row
+        constexpr int SLICE = GW * 64;         // a wavefront's bytes of a weight row per step
+        constexpr int SPAN = 8 * SLICE;        // bytes of a weight row that the workgroup covers per step
         constexpr int TILE_BYTES = 16 * SLICE; // = GW KiB: GW wavefront-wide loads
-        constexpr int LT = GW + 1;             // loads per tile and wavefront (weights + scales)
+        constexpr int LT = GW + 1;             // loads per step and wavefront (weights + scales)
         constexpr int SC_LANES = (GW + 1) / 2; // 4-byte scale loads per row (odd GW: one half-word of a neighbour comes along)
         extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
         uint32_t MAGIC, MASK_LO, MASK_HI;
@@ -101,14 +103,15 @@ namespace nnf
                                (((uint32_t)wave * (GW * 2)) & ~3u) + (uint32_t)(lane % SC_LANES) * 4u;
         const int sc_skip = (wave * GW) & 1;
 
-        auto issue = [&](int tile, int slot) {
+        // step st (0 .. STEPS-1) of tile `tile` into slot `slot`
+        auto issue = [&](int tile, int st, int slot) {
             const uint32_t row0 = (uint32_t)row0_of(tile);
-            const uint8_t* wsrc = Wq + (size_t)row0 * ROW_BYTES;
+            const uint8_t* wsrc = Wq + (size_t)row0 * ROW_BYTES + st * SPAN;
 #pragma unroll
             for (int c = 0; c < GW; ++c)
                 __builtin_amdgcn_global_load_lds((mr_global_ptr_t)(wsrc + w_off[c]),
                                                  (mr_lds_ptr_t)(ring + slot * TILE_BYTES + c * 1024), 16, 0, 0);
-            __builtin_amdgcn_global_load_lds((mr_global_ptr_t)(reinterpret_cast<const uint8_t*>(S) + (size_t)row0 * (G * 2) + s_off),
+            __builtin_amdgcn_global_load_lds((mr_global_ptr_t)(reinterpret_cast<const uint8_t*>(S) + (size_t)row0 * (G * 2) + st * (8 * GW * 2) + s_off),
                                              (mr_lds_ptr_t)(sc_ring + slot * 256), 4, 0, 0);
         };
 
@@ -116,26 +119,27 @@ namespace nnf
         // (the activations are requested last: vector-memory operations complete in order and the compiler waits
         // for them where they are used, which then also covers the two tiles -- requested first, those tiles'
         // loads are not held back by anything)
-        issue(t0, 0);
-        issue(t0 + min(1, T - 1), 1);
-        uintx4 areg[GW][4];
+        issue(t0, 0, 0);
+        issue(t0 + min(1 / STEPS, T - 1), 1 % STEPS, 1);
+        uintx4 areg[GA][4];
         {
             const uint8_t* a_bytes = reinterpret_cast<const uint8_t*>(A);
             const uint32_t a_off = (uint32_t)min(col, M - 1) * (uint32_t)(K * 2) + (uint32_t)wave * (GW * 256) + (uint32_t)kq * 64u;
 #pragma unroll
-            for (int g = 0; g < GW; ++g)
+            for (int g = 0; g < GA; ++g)
 #pragma unroll
                 for (int j = 0; j < 4; ++j)
-                    areg[g][j] = *reinterpret_cast<const uintx4*>(a_bytes + (size_t)(a_off + g * 256 + j * 16));
+                    areg[g][j] = *reinterpret_cast<const uintx4*>(a_bytes +
+                                                                  (size_t)(a_off + (g / GW) * (SPAN * 4) + (g % GW) * 256 + j * 16));
         }
-        floatx4 ncorr[GW];
+        floatx4 ncorr[GA];
         {
             const half2_t sixteenth = half2_t{(half_t)0.0625f, (half_t)0.0625f};
             const half_t ceh = (half_t)(-(1024.0f + (float)zp)), coh = (half_t)(-16.0f * (64.0f + (float)zp)); // exact
             const uint32_t ce2 = as_u32(half2_t{ceh, ceh}), co2 = as_u32(half2_t{coh, coh});
             const uintx4 cvec = {ce2, co2, ce2, co2};
 #pragma unroll
-            for (int g = 0; g < GW; ++g)
+            for (int g = 0; g < GA; ++g)
             {
                 floatx4 t = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -158,55 +162,60 @@ namespace nnf
         const int rd_swz = swz(col);
         const uint32_t red_addr = lds_address(red) + (uint32_t)(wave * 1024 + lane * 16);
         const uint32_t parked_addr = lds_address(parked);
+        int slot = 0; // step s of the workgroup sits in slot s & 1
         for (int it = 0; it < T; ++it)
         {
-            const int slot = it & 1;
-            // this tile has landed when at most the next tile's loads are outstanding
-            __builtin_amdgcn_s_waitcnt(mr_vmcnt(LT));
-            uintx4 wv[GW];
-            float sv[GW];
+            floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int st = 0; st < STEPS; ++st)
             {
-                const uint8_t* sl = ring + slot * TILE_BYTES + rd_base;
-                const half_t* sc = reinterpret_cast<const half_t*>(sc_ring + slot * 256);
+                // this step has landed when at most the next step's loads are outstanding
+                __builtin_amdgcn_s_waitcnt(mr_vmcnt(LT));
+                uintx4 wv[GW];
+                float sv[GW];
+                {
+                    const uint8_t* sl = ring + slot * TILE_BYTES + rd_base;
+                    const half_t* sc = reinterpret_cast<const half_t*>(sc_ring + slot * 256);
+#pragma unroll
+                    for (int g = 0; g < GW; ++g)
+                    {
+                        wv[g] = *reinterpret_cast<const uintx4*>(sl + (((g * 4 + kq) ^ rd_swz) << 4));
+                        sv[g] = (float)sc[col * (SC_LANES * 2) + sc_skip + g];
+                    }
+                }
+                // the slot has been read before it is refilled with the step after next (past the end: a valid
+                // tile again, so that the wait count above holds for every step)
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                issue(t0 + min(it + (st + 2) / STEPS, T - 1), (st + 2) % STEPS, slot);
+                slot ^= 1;
 #pragma unroll
                 for (int g = 0; g < GW; ++g)
                 {
-                    wv[g] = *reinterpret_cast<const uintx4*>(sl + (((g * 4 + kq) ^ rd_swz) << 4));
-                    sv[g] = (float)sc[col * (SC_LANES * 2) + sc_skip + g];
+                    floatx4 t = ncorr[st * GW + g];
+                    const uint32_t ww[4] = {wv[g].x, wv[g].y, wv[g].z, wv[g].w};
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                    {
+                        const uint32_t w = ww[j];
+                        const uint32_t w8 = w >> 8;
+                        uintx4 bq;
+                        bq.x = (w & MASK_LO) | MAGIC;  // 1024 + (q0, q4)
+                        bq.y = (w & MASK_HI) | MAGIC;  // 1024 + 16 (q1, q5)
+                        bq.z = (w8 & MASK_LO) | MAGIC; // 1024 + (q2, q6)
+                        bq.w = (w8 & MASK_HI) | MAGIC; // 1024 + 16 (q3, q7)
+                        t = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, areg[st * GW + g][j]),
+                                                                   __builtin_bit_cast(half8_t, bq), t, 0, 0, 0);
+                    }
+                    acc.x = __builtin_fmaf(t.x, sv[g], acc.x);
+                    acc.y = __builtin_fmaf(t.y, sv[g], acc.y);
+                    acc.z = __builtin_fmaf(t.z, sv[g], acc.z);
+                    acc.w = __builtin_fmaf(t.w, sv[g], acc.w);
                 }
             }
-            // the slot has been read before it is refilled (past the end: a valid tile again, so that the wait
-            // count above holds for every iteration)
-            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-            issue(t0 + min(it + 2, T - 1), slot);
-
-            floatx4 acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int g = 0; g < GW; ++g)
-            {
-                floatx4 t = ncorr[g];
-                const uint32_t ww[4] = {wv[g].x, wv[g].y, wv[g].z, wv[g].w};
-#pragma unroll
-                for (int j = 0; j < 4; ++j)
-                {
-                    const uint32_t w = ww[j];
-                    const uint32_t w8 = w >> 8;
-                    uintx4 bq;
-                    bq.x = (w & MASK_LO) | MAGIC;  // 1024 + (q0, q4)
-                    bq.y = (w & MASK_HI) | MAGIC;  // 1024 + 16 (q1, q5)
-                    bq.z = (w8 & MASK_LO) | MAGIC; // 1024 + (q2, q6)
-                    bq.w = (w8 & MASK_HI) | MAGIC; // 1024 + 16 (q3, q7)
-                    t = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, areg[g][j]),
-                                                               __builtin_bit_cast(half8_t, bq), t, 0, 0, 0);
-                }
-                acc.x = __builtin_fmaf(t.x, sv[g], acc.x);
-                acc.y = __builtin_fmaf(t.y, sv[g], acc.y);
-                acc.z = __builtin_fmaf(t.z, sv[g], acc.z);
-                acc.w = __builtin_fmaf(t.w, sv[g], acc.w);
-            }
+            const int rbuf = it & 1;
             // partial tile -> LDS (D layout: lane (n = col, kq), element e: row m = 4 kq + e)
             {
-                const uint32_t at = red_addr + (uint32_t)(slot * MR_WAVES * 1024);
+                const uint32_t at = red_addr + (uint32_t)(rbuf * MR_WAVES * 1024);
                 asm volatile("ds_write_b128 %0, %1" ::"v"(at), "v"(acc) : "memory");
             }
             asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
@@ -214,7 +223,7 @@ namespace nnf
             if (tid < 256)
             {
                 const int e = tid >> 6;
-                const float* rp = reinterpret_cast<const float*>(red + slot * MR_WAVES * 1024) + lane * 4 + e;
+                const float* rp = reinterpret_cast<const float*>(red + rbuf * MR_WAVES * 1024) + lane * 4 + e;
                 float sum = 0.f;
 #pragma unroll
                 for (int w = 0; w < MR_WAVES; ++w)
@@ -241,17 +250,17 @@ namespace nnf
 
     namespace
     {
-        template <int GW>
+        template <int GW, int STEPS>
         hipError_t launch_mrows(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M, int N, int zp,
                                 int num_cu)
         {
             const int n_tiles = (N + 15) / 16;
             const int grid = n_tiles < num_cu ? n_tiles : num_cu;
             const int tiles_q = n_tiles / grid, tiles_r = n_tiles % grid;
-            const size_t lds = workspace::w4a16_mrows_lds_bytes(GW << 10, M, tiles_q + (tiles_r ? 1 : 0));
+            const size_t lds = workspace::w4a16_mrows_lds_bytes(GW * STEPS * 1024, M, tiles_q + (tiles_r ? 1 : 0));
             if (lds > MAX_LDS_BYTES)
                 return hipErrorInvalidValue;
-            auto kernel = &w4a16_mrows_kernel<GW>;
+            auto kernel = &w4a16_mrows_kernel<GW, STEPS>;
             if (lds > 64 * 1024)
             {
                 hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -273,16 +282,20 @@ namespace nnf
     {
         if (!w4a16_mrows_supported(M, N, K, num_cu))
             return hipErrorInvalidValue;
+        // K / 1024 = groups per wavefront and tile, walked in STEPS steps of GW groups.  Two steps per tile where
+        // K / 1024 is even: with the two ring slots that is one tile in flight per wavefront (32 KiB per CU at
+        // K = 4096, 64 KiB at 8192).  Measured against one step (two tiles in flight) and four steps (half a tile):
+        // 5-25 % faster than either at K = 4096, 6144 and 8192.
         switch (K >> 10)
         {
-        case 1: return launch_mrows<1>(stream, A, Wq, S, Y, M, N, zp, num_cu);
-        case 2: return launch_mrows<2>(stream, A, Wq, S, Y, M, N, zp, num_cu);
-        case 3: return launch_mrows<3>(stream, A, Wq, S, Y, M, N, zp, num_cu);
-        case 4: return launch_mrows<4>(stream, A, Wq, S, Y, M, N, zp, num_cu);
-        case 5: return launch_mrows<5>(stream, A, Wq, S, Y, M, N, zp, num_cu);
-        case 6: return launch_mrows<6>(stream, A, Wq, S, Y, M, N, zp, num_cu);
-        case 7: return launch_mrows<7>(stream, A, Wq, S, Y, M, N, zp, num_cu);
-        default: return launch_mrows<8>(stream, A, Wq, S, Y, M, N, zp, num_cu);
+        case 1: return launch_mrows<1, 1>(stream, A, Wq, S, Y, M, N, zp, num_cu);
+        case 2: return launch_mrows<1, 2>(stream, A, Wq, S, Y, M, N, zp, num_cu);
+        case 3: return launch_mrows<3, 1>(stream, A, Wq, S, Y, M, N, zp, num_cu);
+        case 4: return launch_mrows<2, 2>(stream, A, Wq, S, Y, M, N, zp, num_cu);
+        case 5: return launch_mrows<5, 1>(stream, A, Wq, S, Y, M, N, zp, num_cu);
+        case 6: return launch_mrows<3, 2>(stream, A, Wq, S, Y, M, N, zp, num_cu);
+        case 7: return launch_mrows<7, 1>(stream, A, Wq, S, Y, M, N, zp, num_cu);
+        default: return launch_mrows<4, 2>(stream, A, Wq, S, Y, M, N, zp, num_cu);
         }
     }
 } // namespace nnf

@@ -368,7 +368,8 @@ namespace nnf
         // workgroup's finished tiles parked until the end.
         inline size_t w4a16_mrows_lds_bytes(int K, int M, int tiles)
         {
-            return (size_t)8 * 2 * (K >> 10) * 1024 + 8 * 512 + 2 * 8 * 1024 + (size_t)tiles * M * 64;
+            const int kw = K >> 10, gw = (kw & 1) ? kw : kw / 2; // groups per wavefront and step (even K / 1024: two steps)
+            return (size_t)8 * 2 * gw * 1024 + 8 * 512 + 2 * 8 * 1024 + (size_t)tiles * M * 64;
         }
         inline bool w4a16_mrows_fits(int M, int N, int K, int num_cu)
         {
@@ -383,12 +384,12 @@ namespace nnf
             return w4a16_mrows_lds_bytes(K, M, (n_tiles + grid - 1) / grid) <= LDS_BYTES_PER_CU;
         }
         // Where the library picks it by itself, from measurements against the split-K MFMA GEMV on cold weights:
-        // K <= 4096: level at N = K = 4096, 5-35 % faster elsewhere (most at small K and large N, and at M = 16);
-        // K = 5120 .. 7168: 5-30 % faster from eight rows on, level to 15 % slower below;
-        // K = 8192 (240 registers per lane): 5-25 % slower except at M = 16 with N >> 8192.
+        // K = 2048, 4096, 6144, 8192 (two steps per tile): 0-15 % faster at M = 2, 15-30 % at M = 16;
+        // K = 1024, 3072: 5-35 % faster;  K = 5120, 7168 (one step per tile: two whole tiles in flight): 5-30 %
+        // faster from eight rows on, level to 15 % slower below.
         inline bool w4a16_mrows_preferred(int M, int N, int K, int num_cu)
         {
-            return (K <= 4096 || (K <= 7168 && M >= 8)) && w4a16_mrows_fits(M, N, K, num_cu);
+            return (!(K & 2047) || K <= 4096 || M >= 8) && w4a16_mrows_fits(M, N, K, num_cu);
         }
         inline bool w4a16_variant_fits(int M, int N, int K, int variant, int num_cu)
         {
