@@ -7,22 +7,24 @@
 // weight-quantized Dot node with a handful of activation rows.
 //
 //   * One workgroup of eight wavefronts per CU owns a contiguous run of 16-row weight tiles.  All eight work on
-//     the same tile; wavefront w owns the K slice [w K/8, (w+1) K/8) = GW groups of 128.
-//   * A wavefront's slice of a tile (16 rows x GW*64 bytes = GW KiB) goes global -> LDS without registers
+//     the same tile, in STEPS steps of 8 x GW groups of 128 along K; wavefront w owns GW groups of every step
+//     (GW*64 bytes of a weight row), so that the workgroup's loads of a step cover the 16 rows without gaps.
+//   * A wavefront's part of a step (16 rows x GW*64 bytes = GW KiB) goes global -> LDS without registers
 //     (global_load_lds_dwordx4, 1 KiB per wavefront-wide load) into a private two-slot ring, together with its
-//     16 x GW group scales (one 4-byte load per lane); the slot of the tile after next is requested as soon as
+//     16 x GW group scales (one 4-byte load per lane); the slot of the step after next is requested as soon as
 //     the current one has been copied into registers.  Nothing but the wavefront's own loads feeds its MFMAs:
-//     no barrier on the load path.  The 16-byte pieces of a row are XOR-swizzled with the row number on the
-//     way (each lane chooses which piece it fetches), so the 128-bit operand reads are conflict free.
+//     no barrier on the load path.  Two steps per tile (one tile in flight per wavefront) measured fastest.
+//     The 16-byte pieces of a row are XOR-swizzled with the row number on the way (each lane chooses which
+//     piece it fetches), so the 128-bit operand reads are conflict free.
 //   * The activations never touch LDS: lane (m, kq) loads the 64 bytes of row m that its MFMA operand holds of
 //     each of the wavefront's groups, once, and keeps them (16 VGPRs per group; hence K <= 8192), in the pair
 //     order and with the 1/16 of the nibble trick; the constant part of a group sum is an MFMA against a
 //     constant operand and becomes the (negative) initial accumulator of the group (see w4a16_skinny.hip).
-//   * Per tile: GW x 4 MFMAs (v_mfma_f32_16x16x32_f16, weights as the B operand) per wavefront, the group sum
-//     times the group scale in fp32, the eight partial 16 x 16 tiles meet in LDS (one LDS-only barrier per
-//     tile, two alternating buffers), 256 threads add them and park the sums in LDS; Y is written after the
+//   * Per step: GW x 4 MFMAs (v_mfma_f32_16x16x32_f16, weights as the B operand) per wavefront, the group sum
+//     times the group scale in fp32; per tile the eight partial 16 x 16 tiles meet in LDS (one LDS-only barrier,
+//     two alternating buffers), 256 threads add them and park the sums in LDS; Y is written after the
 //     last tile.  Every workgroup reads all of A (M x K x 2 bytes, from the L2): with 16 rows of K = 8192 that
-//     is twice the bytes of its weights, which bounds the kernel at ~1.4x the time of the weight stream.
+//     is twice the bytes of its weights.
 //   * LDS writes inside the tile loop are inline ds_write instructions: ahead of an LDS write that it can see,
 //     the compiler waits for every LDS-bound load in flight.
 #include "nnf_device.h"
@@ -41,6 +43,7 @@ namespace nnf
         constexpr int mr_vmcnt(int n) { return (n & 0xF) | ((n >> 4) << 14) | (0x7 << 4) | (0xF << 8); }
     } // namespace
 
+    // K = GW * STEPS * 1024.
     // LDS (bytes): weights [8 wavefronts][2 slots][GW KiB] | scales [8][2][256] | partial tiles [2][8][1 KiB] |
     //              parked sums [tiles of the workgroup][M][16] fp32
     // pack = M | zp << 8;  a workgroup's tiles: tiles_q, one more for the first tiles_r workgroups.
