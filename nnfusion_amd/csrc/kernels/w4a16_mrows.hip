@@ -1,5 +1,7 @@
-// fp16 x int4 (g128) for 2 <= M <= 16 activation rows and K = 1024, 2048, ... 8192: the memory pipeline of the
-// row-streaming GEMV (w4a16_gemv_rows.hip) under the arithmetic of the M <= 16 MFMA kernel (w4a16_skinny.hip).
+// fp16 x int4 (g128) for 2 <= M <= 16 activation rows and K = 1024, 2048, ... 8192 (M <= 32 up to K = 4096): the
+// memory pipeline of the
+// row-streaming GEMV (w4a16_gemv_rows.hip) under the arithmetic of the M <= 16 MFMA kernel
+// (w4a16_skinny.hip).
 //
 //   Y[M,N] = A[M,K] . ((Wq - zp) * S)^T
 //
@@ -43,16 +45,17 @@ namespace nnf
         constexpr int mr_vmcnt(int n) { return (n & 0xF) | ((n >> 4) << 14) | (0x7 << 4) | (0xF << 8); }
     } // namespace
 
-    // K = GW * STEPS * 1024.
-    // LDS (bytes): weights [8 wavefronts][2 slots][GW KiB] | scales [8][2][256] | partial tiles [2][8][1 KiB] |
+    // K = GW * STEPS * 1024; MB = blocks of 16 activation rows (1 or 2).
+    // LDS (bytes): weights [8 wavefronts][2 slots][GW KiB] | scales [8][2][256] | partial tiles [2][8][MB KiB] |
     //              parked sums [tiles of the workgroup][M][16] fp32
     // pack = M | zp << 8;  a workgroup's tiles: tiles_q, one more for the first tiles_r workgroups.
-    template <int GW, int STEPS>
+    template <int GW, int STEPS, int MB>
     __global__ __launch_bounds__(512) void w4a16_mrows_kernel(const half_t* __restrict__ A, const uint8_t* __restrict__ Wq,
                                                               const half_t* __restrict__ S, half_t* __restrict__ Y, int N,
                                                               int tiles_q, int tiles_r, int pack)
     {
         static_assert(GW >= 1 && GW <= 8 && STEPS >= 1 && GW * STEPS <= 8, "K = GW * STEPS * 1024");
+        static_assert(MB == 1 || (MB == 2 && GW * STEPS <= 4), "two blocks of rows: 32 VGPRs per group");
         constexpr int K = GW * STEPS * 1024, G = K / 128;
         constexpr int GA = GW * STEPS;         // groups of a wavefront
         constexpr int ROW_BYTES = K / 2;       // a weight row
@@ -82,7 +85,7 @@ namespace nnf
         uint8_t* ring = smem + wave * (2 * TILE_BYTES);
         uint8_t* sc_ring = smem + MR_WAVES * 2 * TILE_BYTES + wave * 512;
         uint8_t* red = smem + MR_WAVES * 2 * TILE_BYTES + MR_WAVES * 512; // [2][8][1024]
-        float* parked = reinterpret_cast<float*>(red + 2 * MR_WAVES * 1024);
+        float* parked = reinterpret_cast<float*>(red + 2 * MR_WAVES * MB * 1024);
 
         // ---- what each lane fetches -------------------------------------------------------------------------
         // Load c of a tile fills bytes [c KiB, (c+1) KiB) of the slot; lane i lands at byte c*1024 + 16 i =
@@ -124,51 +127,59 @@ namespace nnf
         // loads are not held back by anything)
         issue(t0, 0, 0);
         issue(t0 + min(1 / STEPS, T - 1), 1 % STEPS, 1);
-        uintx4 areg[GA][4];
+        uintx4 areg[MB][GA][4];
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
         {
             const uint8_t* a_bytes = reinterpret_cast<const uint8_t*>(A);
-            const uint32_t a_off = (uint32_t)min(col, M - 1) * (uint32_t)(K * 2) + (uint32_t)wave * (GW * 256) + (uint32_t)kq * 64u;
+            const uint32_t a_off =
+                (uint32_t)min(mb * 16 + col, M - 1) * (uint32_t)(K * 2) + (uint32_t)wave * (GW * 256) + (uint32_t)kq * 64u;
 #pragma unroll
             for (int g = 0; g < GA; ++g)
 #pragma unroll
                 for (int j = 0; j < 4; ++j)
-                    areg[g][j] = *reinterpret_cast<const uintx4*>(a_bytes +
-                                                                  (size_t)(a_off + (g / GW) * (SPAN * 4) + (g % GW) * 256 + j * 16));
+                    areg[mb][g][j] = *reinterpret_cast<const uintx4*>(
+                        a_bytes + (size_t)(a_off + (g / GW) * (SPAN * 4) + (g % GW) * 256 + j * 16));
         }
-        floatx4 ncorr[GA];
+        floatx4 ncorr[MB][GA];
         {
             const half2_t sixteenth = half2_t{(half_t)0.0625f, (half_t)0.0625f};
             const half_t ceh = (half_t)(-(1024.0f + (float)zp)), coh = (half_t)(-16.0f * (64.0f + (float)zp)); // exact
             const uint32_t ce2 = as_u32(half2_t{ceh, ceh}), co2 = as_u32(half2_t{coh, coh});
             const uintx4 cvec = {ce2, co2, ce2, co2};
 #pragma unroll
-            for (int g = 0; g < GA; ++g)
-            {
-                floatx4 t = {0.f, 0.f, 0.f, 0.f};
+            for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-                for (int j = 0; j < 4; ++j)
+                for (int g = 0; g < GA; ++g)
                 {
-                    uintx4 a = permute_a8(areg[g][j]);
-                    a.y = as_u32(as_half2(a.y) * sixteenth);
-                    a.w = as_u32(as_half2(a.w) * sixteenth);
-                    areg[g][j] = a;
-                    t = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, a), __builtin_bit_cast(half8_t, cvec), t,
-                                                               0, 0, 0);
+                    floatx4 t = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                    {
+                        uintx4 a = permute_a8(areg[mb][g][j]);
+                        a.y = as_u32(as_half2(a.y) * sixteenth);
+                        a.w = as_u32(as_half2(a.w) * sixteenth);
+                        areg[mb][g][j] = a;
+                        t = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, a),
+                                                                   __builtin_bit_cast(half8_t, cvec), t, 0, 0, 0);
+                    }
+                    ncorr[mb][g] = t;
                 }
-                ncorr[g] = t;
-            }
         }
 
         // ---- tile loop ---------------------------------------------------------------------------------------
         // operand reads of a slot: lane (n = col, kq), group g: piece g*4 + kq of row n
         const uint32_t rd_base = (uint32_t)col * SLICE;
         const int rd_swz = swz(col);
-        const uint32_t red_addr = lds_address(red) + (uint32_t)(wave * 1024 + lane * 16);
+        const uint32_t red_addr = lds_address(red) + (uint32_t)(wave * (MB * 1024) + lane * 16);
         const uint32_t parked_addr = lds_address(parked);
         int slot = 0; // step s of the workgroup sits in slot s & 1
         for (int it = 0; it < T; ++it)
         {
-            floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+            floatx4 acc[MB];
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb)
+                acc[mb] = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int st = 0; st < STEPS; ++st)
             {
@@ -194,7 +205,10 @@ namespace nnf
 #pragma unroll
                 for (int g = 0; g < GW; ++g)
                 {
-                    floatx4 t = ncorr[st * GW + g];
+                    floatx4 t[MB];
+#pragma unroll
+                    for (int mb = 0; mb < MB; ++mb)
+                        t[mb] = ncorr[mb][st * GW + g];
                     const uint32_t ww[4] = {wv[g].x, wv[g].y, wv[g].z, wv[g].w};
 #pragma unroll
                     for (int j = 0; j < 4; ++j)
@@ -206,32 +220,41 @@ namespace nnf
                         bq.y = (w & MASK_HI) | MAGIC;  // 1024 + 16 (q1, q5)
                         bq.z = (w8 & MASK_LO) | MAGIC; // 1024 + (q2, q6)
                         bq.w = (w8 & MASK_HI) | MAGIC; // 1024 + 16 (q3, q7)
-                        t = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, areg[st * GW + g][j]),
-                                                                   __builtin_bit_cast(half8_t, bq), t, 0, 0, 0);
+#pragma unroll
+                        for (int mb = 0; mb < MB; ++mb)
+                            t[mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, areg[mb][st * GW + g][j]),
+                                                                           __builtin_bit_cast(half8_t, bq), t[mb], 0, 0, 0);
                     }
-                    acc.x = __builtin_fmaf(t.x, sv[g], acc.x);
-                    acc.y = __builtin_fmaf(t.y, sv[g], acc.y);
-                    acc.z = __builtin_fmaf(t.z, sv[g], acc.z);
-                    acc.w = __builtin_fmaf(t.w, sv[g], acc.w);
+#pragma unroll
+                    for (int mb = 0; mb < MB; ++mb)
+                    {
+                        acc[mb].x = __builtin_fmaf(t[mb].x, sv[g], acc[mb].x);
+                        acc[mb].y = __builtin_fmaf(t[mb].y, sv[g], acc[mb].y);
+                        acc[mb].z = __builtin_fmaf(t[mb].z, sv[g], acc[mb].z);
+                        acc[mb].w = __builtin_fmaf(t[mb].w, sv[g], acc[mb].w);
+                    }
                 }
             }
             const int rbuf = it & 1;
-            // partial tile -> LDS (D layout: lane (n = col, kq), element e: row m = 4 kq + e)
+            // partial tiles -> LDS (D layout: lane (n = col, kq), element e: row m = 16 mb + 4 kq + e)
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb)
             {
-                const uint32_t at = red_addr + (uint32_t)(rbuf * MR_WAVES * 1024);
-                asm volatile("ds_write_b128 %0, %1" ::"v"(at), "v"(acc) : "memory");
+                const uint32_t at = red_addr + (uint32_t)(rbuf * MR_WAVES * MB * 1024 + mb * 1024);
+                asm volatile("ds_write_b128 %0, %1" ::"v"(at), "v"(acc[mb]) : "memory");
             }
             asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-            // 256 threads: thread (e, lane') adds the eight partial sums of output (m = 4 (lane' >> 4) + e, n = lane' & 15)
-            if (tid < 256)
+            // MB x 256 threads: thread (mb, e, lane') adds the eight partial sums of output
+            // (m = 16 mb + 4 (lane' >> 4) + e, n = lane' & 15)
+            if (tid < MB * 256)
             {
-                const int e = tid >> 6;
-                const float* rp = reinterpret_cast<const float*>(red + rbuf * MR_WAVES * 1024) + lane * 4 + e;
+                const int mb = tid >> 8, e = (tid >> 6) & 3;
+                const float* rp = reinterpret_cast<const float*>(red + rbuf * MR_WAVES * MB * 1024 + mb * 1024) + lane * 4 + e;
                 float sum = 0.f;
 #pragma unroll
                 for (int w = 0; w < MR_WAVES; ++w)
-                    sum += rp[w * 256];
-                const int m = 4 * kq + e;
+                    sum += rp[w * (MB * 256)];
+                const int m = 16 * mb + 4 * kq + e;
                 if (m < M)
                 {
                     const uint32_t at = parked_addr + (uint32_t)(((it * M + m) * 16 + col) * 4);
@@ -253,8 +276,8 @@ namespace nnf
 
     namespace
     {
-        template <int GW, int STEPS>
-        hipError_t launch_mrows(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M, int N, int zp,
+        template <int GW, int STEPS, int MB>
+        hipError_t launch_mrows_mb(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M, int N, int zp,
                                 int num_cu)
         {
             const int n_tiles = (N + 15) / 16;
@@ -263,7 +286,7 @@ namespace nnf
             const size_t lds = workspace::w4a16_mrows_lds_bytes(GW * STEPS * 1024, M, tiles_q + (tiles_r ? 1 : 0));
             if (lds > MAX_LDS_BYTES)
                 return hipErrorInvalidValue;
-            auto kernel = &w4a16_mrows_kernel<GW, STEPS>;
+            auto kernel = &w4a16_mrows_kernel<GW, STEPS, MB>;
             if (lds > 64 * 1024)
             {
                 hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -274,6 +297,17 @@ namespace nnf
             hipLaunchKernelGGL(kernel, dim3(grid), dim3(MR_WAVES * 64), lds, stream, (const half_t*)A, (const uint8_t*)Wq,
                                (const half_t*)S, (half_t*)Y, N, tiles_q, tiles_r, M | (zp << 8));
             return hipGetLastError();
+        }
+
+        template <int GW, int STEPS>
+        hipError_t launch_mrows(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M, int N, int zp,
+                                int num_cu)
+        {
+            if (M <= 16)
+                return launch_mrows_mb<GW, STEPS, 1>(stream, A, Wq, S, Y, M, N, zp, num_cu);
+            if constexpr (GW * STEPS <= 4)
+                return launch_mrows_mb<GW, STEPS, 2>(stream, A, Wq, S, Y, M, N, zp, num_cu);
+            return hipErrorInvalidValue;
         }
     } // namespace
 

@@ -361,7 +361,7 @@ namespace nnf
         // M <= 16 kernel it is level to 10 % faster up to M = 14 (2 % slower at M = 2, N = K = 8192), 5-30 % faster at
         // M = 16, and 12-33 % faster than the MFMA tile GEMM at M = 17 .. 32.
         inline bool w8a8_mrows_preferred(int M, int N, int K, int num_cu) { return w8a8_mrows_fits(M, N, K, num_cu); }
-        // ---- 2 .. 16 activation rows: the row-streaming MFMA kernel (w4a16_mrows.hip) ----
+        // ---- 2 .. 16 activation rows (.. 32 up to K = 4096): the row-streaming MFMA kernel (w4a16_mrows.hip) ----
         // One workgroup per CU, eight wavefronts that each own an eighth of K and keep their share of the activations
         // in registers; K is a compile-time constant of the kernel (a multiple of 1024 up to 8192).  LDS: per
         // wavefront two slots of a 16-row weight tile and of its scales, two sets of eight partial tiles, and the
@@ -369,13 +369,15 @@ namespace nnf
         inline size_t w4a16_mrows_lds_bytes(int K, int M, int tiles)
         {
             const int kw = K >> 10, gw = (kw & 1) ? kw : kw / 2; // groups per wavefront and step (even K / 1024: two steps)
-            return (size_t)8 * 2 * gw * 1024 + 8 * 512 + 2 * 8 * 1024 + (size_t)tiles * M * 64;
+            return (size_t)8 * 2 * gw * 1024 + 8 * 512 + (size_t)2 * 8 * (M <= 16 ? 1 : 2) * 1024 + (size_t)tiles * M * 64;
         }
         inline bool w4a16_mrows_fits(int M, int N, int K, int num_cu)
         {
-            if (M < 2 || M > 16 || N < 16 || num_cu < 1)
+            if (M < 2 || M > 32 || N < 16 || num_cu < 1)
                 return false;
             if (K < 1024 || K > 8192 || (K & 1023)) // K / 1024 is a template parameter of the kernel
+                return false;
+            if (M > 16 && K > 4096) // two blocks of 16 rows: 32 VGPRs of activations per group of K
                 return false;
             if ((size_t)N * (size_t)(K >> 1) >= ((size_t)1 << 32)) // 32-bit offsets over the weight rows
                 return false;

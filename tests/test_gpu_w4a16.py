@@ -61,6 +61,8 @@ def _check(y, ref):
     # fewer tiles than CUs, a single tile
     (2, 4096, 1024), (3, 8200, 2048), (16, 4111, 4096), (9, 22016, 4096), (16, 12288, 8192), (6, 16, 8192), (11, 48, 2048),
     (16, 40000, 1024), (5, 4096, 3072), (16, 13824, 5120), (7, 1000, 6144), (16, 2050, 7168), (2, 640, 5120),
+    # 17 .. 32 rows (two blocks of 16), K <= 4096
+    (17, 4096, 4096), (32, 22016, 4096), (24, 1000, 2048), (31, 77, 3072), (32, 300, 1024),
 ])
 def test_gemv_matches_oracle(gpu, path, m, n, k):
     print(f"case M={m} N={n} K={k}", flush=True)
@@ -124,7 +126,7 @@ def test_gemv_other_zero_points(gpu, path, zp):
     _check(y, ref)
 
 
-@pytest.mark.parametrize("m,n,k", [(1, 512, 4096), (8, 300, 2048), (16, 128, 8192), (40, 256, 1024), (8, 300, 3072), (8, 300, 2176)])
+@pytest.mark.parametrize("m,n,k", [(1, 512, 4096), (8, 300, 2048), (16, 128, 8192), (40, 256, 1024), (8, 300, 3072), (8, 300, 2176), (24, 300, 4096), (24, 300, 8192)])
 def test_every_kernel_variant_that_accepts_a_shape_matches_the_oracle(gpu, m, n, k):
     """nnf_w4a16_gemm_variant: the entry point behind the per-variant emitters of profiling-based kernel selection.
     nnf_w4a16_variant_supported (host only) and the call itself agree on which variants serve a shape."""
@@ -148,5 +150,5 @@ def test_every_kernel_variant_that_accepts_a_shape_matches_the_oracle(gpu, m, n,
                 ops.w4a16_gemm_variant(ta, tw, ts, name)
             assert e.value.status == -2
     assert "auto" in served and "gemm_mfma" in served
-    assert ("gemv_rows" in served) == (m == 1 or (m <= 16 and k % 1024 == 0 and k <= 8192))
+    assert ("gemv_rows" in served) == (m == 1 or (m <= 32 and k % 1024 == 0 and k <= (8192 if m <= 16 else 4096)))
     assert ("gemv_valu" in served) == (m <= 16)
