@@ -274,6 +274,207 @@ namespace nnf
         }
     }
 
+    // The same kernel with K as a run-time value: any multiple of 256 up to 8 * GW * STEPS groups (2 <= M <= 16).
+    // A wavefront whose GW groups of a step would reach past the end of K fetches the last GW groups of the row
+    // instead (the loads of every wavefront and step stay the same in number, which the hand-written wait counts
+    // need) and multiplies what another wavefront already covers by a scale of zero.
+    // (Longer K in several passes over the tiles, each with its own part of the activations in registers, was
+    // measured: every pass pays the start of the kernel again, and the split-K kernel is faster.)
+    // LDS as above (MB = 1).  pack = M | zp << 8.
+    template <int GW, int STEPS>
+    __global__ __launch_bounds__(512) void w4a16_mrows_any_kernel(const half_t* __restrict__ A, const uint8_t* __restrict__ Wq,
+                                                                  const half_t* __restrict__ S, half_t* __restrict__ Y, int N, int K,
+                                                                  int tiles_q, int tiles_r, int pack)
+    {
+        static_assert(GW >= 1 && GW <= 7 && STEPS >= 1 && GW * STEPS <= 8, "groups per wavefront and pass");
+        constexpr int GA = GW * STEPS;         // groups of a wavefront
+        constexpr int SLICE = GW * 64;         // a wavefront's bytes of a weight row per step
+        constexpr int TILE_BYTES = 16 * SLICE; // = GW KiB: GW wavefront-wide loads
+        constexpr int LT = GW + 1;             // loads per step and wavefront (weights + scales)
+        constexpr int SC_LANES = GW / 2 + 1;   // 4-byte scale loads per row: GW groups from any 2-byte offset
+        extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+        uint32_t MAGIC, MASK_LO, MASK_HI;
+        asm volatile("v_mov_b32 %0, 0x64006400" : "=v"(MAGIC));
+        asm volatile("s_mov_b32 %0, 0x000F000F" : "=s"(MASK_LO));
+        asm volatile("s_mov_b32 %0, 0x00F000F0" : "=s"(MASK_HI));
+
+        const int tid = threadIdx.x;
+        const int lane = tid & 63;
+        const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+        const int col = lane & 15;
+        const int kq = lane >> 4;
+        const int M = pack & 0xff, zp = (pack >> 8) & 0xff;
+        const int G = K >> 7, ROW_BYTES = K >> 1;
+        const int b = blockIdx.x;
+        const int t0 = b * tiles_q + min(b, tiles_r);
+        const int T = tiles_q + (b < tiles_r ? 1 : 0);
+        auto row0_of = [&](int tile) { return __builtin_amdgcn_readfirstlane(min(tile * 16, N - 16)); };
+        // first group that wavefront `wave` owns in step st, and the first group it fetches
+        auto own_group = [&](int st) { return st * (8 * GW) + wave * GW; };
+        auto fetch_group = [&](int st) { return min(own_group(st), G - GW); };
+
+        uint8_t* ring = smem + wave * (2 * TILE_BYTES);
+        uint8_t* sc_ring = smem + MR_WAVES * 2 * TILE_BYTES + wave * 512;
+        uint8_t* red = smem + MR_WAVES * 2 * TILE_BYTES + MR_WAVES * 512; // [2][8][1024]
+        float* parked = reinterpret_cast<float*>(red + 2 * MR_WAVES * 1024);
+
+        auto swz = [](int r) { return GW % 4 == 0 ? (r & 15) : GW % 2 == 0 ? (r >> 1) & 7 : (r >> 2) & 3; };
+        uint32_t w_off[GW];
+#pragma unroll
+        for (int c = 0; c < GW; ++c)
+        {
+            const int pos = c * 1024 + 16 * lane;
+            const int r = pos / SLICE, q = (pos % SLICE) >> 4;
+            w_off[c] = (uint32_t)r * (uint32_t)ROW_BYTES + (uint32_t)((q ^ swz(r)) << 4);
+        }
+        // scales: lane l fetches 4 bytes of row l / SC_LANES, counted from the 4-byte boundary at or below the first
+        // fetched group (never past the end of the row: the last word is fetched twice instead)
+        const uint32_t s_lane_row = (uint32_t)min(lane / SC_LANES, 15) * (uint32_t)(G * 2);
+        const int s_lane_word = lane % SC_LANES;
+
+        auto issue = [&](int tile, int st, int slot) {
+            const uint32_t row0 = (uint32_t)row0_of(tile);
+            const int gs = fetch_group(st);
+            const uint8_t* wsrc = Wq + (size_t)row0 * ROW_BYTES + gs * 64;
+#pragma unroll
+            for (int c = 0; c < GW; ++c)
+                __builtin_amdgcn_global_load_lds((mr_global_ptr_t)(wsrc + w_off[c]),
+                                                 (mr_lds_ptr_t)(ring + slot * TILE_BYTES + c * 1024), 16, 0, 0);
+            const int first = (gs * 2) & ~3;                  // byte offset of the first word within the row's scales
+            const int last_word = ((G * 2 - first) >> 2) - 1; // of this window that is still inside the row
+            const uint32_t s_off = s_lane_row + (uint32_t)(first + 4 * min(s_lane_word, last_word));
+            __builtin_amdgcn_global_load_lds((mr_global_ptr_t)(reinterpret_cast<const uint8_t*>(S) + (size_t)row0 * (G * 2) + s_off),
+                                             (mr_lds_ptr_t)(sc_ring + slot * 256), 4, 0, 0);
+        };
+        issue(t0, 0, 0);
+        issue(t0 + min(1 / STEPS, T - 1), 1 % STEPS, 1);
+
+        const half2_t sixteenth = half2_t{(half_t)0.0625f, (half_t)0.0625f};
+        const half_t ceh = (half_t)(-(1024.0f + (float)zp)), coh = (half_t)(-16.0f * (64.0f + (float)zp)); // exact
+        const uint32_t ce2 = as_u32(half2_t{ceh, ceh}), co2 = as_u32(half2_t{coh, coh});
+        const uintx4 cvec = {ce2, co2, ce2, co2};
+        const uint32_t rd_base = (uint32_t)col * SLICE;
+        const int rd_swz = swz(col);
+        const uint32_t red_addr = lds_address(red) + (uint32_t)(wave * 1024 + lane * 16);
+        const uint32_t parked_addr = lds_address(parked);
+        const uint8_t* a_row = reinterpret_cast<const uint8_t*>(A) + (size_t)min(col, M - 1) * (size_t)(K * 2) + kq * 64;
+        int slot = 0;
+        {
+            // ---- the activations: straight into the MFMA operand registers ------------------------------------------
+            uintx4 areg[GA][4];
+            floatx4 ncorr[GA];
+#pragma unroll
+            for (int st = 0; st < STEPS; ++st)
+            {
+                const uint8_t* a_src = a_row + (size_t)fetch_group(st) * 256;
+#pragma unroll
+                for (int g = 0; g < GW; ++g)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        areg[st * GW + g][j] = *reinterpret_cast<const uintx4*>(a_src + g * 256 + j * 16);
+            }
+#pragma unroll
+            for (int g = 0; g < GA; ++g)
+            {
+                floatx4 t = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                {
+                    uintx4 a = permute_a8(areg[g][j]);
+                    a.y = as_u32(as_half2(a.y) * sixteenth);
+                    a.w = as_u32(as_half2(a.w) * sixteenth);
+                    areg[g][j] = a;
+                    t = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, a), __builtin_bit_cast(half8_t, cvec), t,
+                                                               0, 0, 0);
+                }
+                ncorr[g] = t;
+            }
+            for (int it = 0; it < T; ++it)
+            {
+                floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int st = 0; st < STEPS; ++st)
+                {
+                    // the groups of this step that no other wavefront covers: from `fresh` on
+                    const int gs = fetch_group(st);
+                    const int fresh = own_group(st) - gs;
+                    const int sc_skip = gs & 1;
+                    // this step has landed when at most the next step's loads are outstanding
+                    __builtin_amdgcn_s_waitcnt(mr_vmcnt(LT));
+                    uintx4 wv[GW];
+                    float sv[GW];
+                    {
+                        const uint8_t* sl = ring + slot * TILE_BYTES + rd_base;
+                        const half_t* sc = reinterpret_cast<const half_t*>(sc_ring + slot * 256);
+#pragma unroll
+                        for (int g = 0; g < GW; ++g)
+                        {
+                            wv[g] = *reinterpret_cast<const uintx4*>(sl + (((g * 4 + kq) ^ rd_swz) << 4));
+                            const float sg = (float)sc[col * (SC_LANES * 2) + sc_skip + g];
+                            sv[g] = g >= fresh ? sg : 0.f;
+                        }
+                    }
+                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                    issue(t0 + min(it + (st + 2) / STEPS, T - 1), (st + 2) % STEPS, slot);
+                    slot ^= 1;
+#pragma unroll
+                    for (int g = 0; g < GW; ++g)
+                    {
+                        floatx4 t = ncorr[st * GW + g];
+                        const uint32_t ww[4] = {wv[g].x, wv[g].y, wv[g].z, wv[g].w};
+#pragma unroll
+                        for (int j = 0; j < 4; ++j)
+                        {
+                            const uint32_t w = ww[j];
+                            const uint32_t w8 = w >> 8;
+                            uintx4 bq;
+                            bq.x = (w & MASK_LO) | MAGIC;
+                            bq.y = (w & MASK_HI) | MAGIC;
+                            bq.z = (w8 & MASK_LO) | MAGIC;
+                            bq.w = (w8 & MASK_HI) | MAGIC;
+                            t = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, areg[st * GW + g][j]),
+                                                                       __builtin_bit_cast(half8_t, bq), t, 0, 0, 0);
+                        }
+                        acc.x = __builtin_fmaf(t.x, sv[g], acc.x);
+                        acc.y = __builtin_fmaf(t.y, sv[g], acc.y);
+                        acc.z = __builtin_fmaf(t.z, sv[g], acc.z);
+                        acc.w = __builtin_fmaf(t.w, sv[g], acc.w);
+                    }
+                }
+                const int rbuf = it & 1;
+                {
+                    const uint32_t at = red_addr + (uint32_t)(rbuf * MR_WAVES * 1024);
+                    asm volatile("ds_write_b128 %0, %1" ::"v"(at), "v"(acc) : "memory");
+                }
+                asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+                if (tid < 256)
+                {
+                    const int e = tid >> 6;
+                    const float* rp = reinterpret_cast<const float*>(red + rbuf * MR_WAVES * 1024) + lane * 4 + e;
+                    float sum = 0.f;
+#pragma unroll
+                    for (int w = 0; w < MR_WAVES; ++w)
+                        sum += rp[w * 256];
+                    const int m = 4 * kq + e;
+                    if (m < M)
+                    {
+                        const uint32_t at = parked_addr + (uint32_t)(((it * M + m) * 16 + col) * 4);
+                        asm volatile("ds_write_b32 %0, %1" ::"v"(at), "v"(sum) : "memory");
+                    }
+                }
+            }
+        }
+        __builtin_amdgcn_s_waitcnt(mr_vmcnt(0)); // the reloads past the end, before the LDS goes away
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        for (int idx = tid; idx < T * M * 16; idx += 512)
+        {
+            const int n = idx & 15;
+            const int im = idx >> 4;
+            const int it = im / M, m = im - it * M;
+            Y[(size_t)m * N + min((t0 + it) * 16, N - 16) + n] = (half_t)parked[idx];
+        }
+    }
+
     namespace
     {
         template <int GW, int STEPS, int MB>
@@ -311,6 +512,32 @@ namespace nnf
         }
     } // namespace
 
+    namespace
+    {
+        template <int GW, int STEPS>
+        hipError_t launch_mrows_any(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M, int N, int K,
+                                    int zp, int num_cu)
+        {
+            const int n_tiles = (N + 15) / 16;
+            const int grid = n_tiles < num_cu ? n_tiles : num_cu;
+            const int tiles_q = n_tiles / grid, tiles_r = n_tiles % grid;
+            const size_t lds = workspace::w4a16_mrows_lds_bytes(K, M, tiles_q + (tiles_r ? 1 : 0));
+            if (lds > MAX_LDS_BYTES)
+                return hipErrorInvalidValue;
+            auto kernel = &w4a16_mrows_any_kernel<GW, STEPS>;
+            if (lds > 64 * 1024)
+            {
+                hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                   (int)lds);
+                if (e != hipSuccess)
+                    return e;
+            }
+            hipLaunchKernelGGL(kernel, dim3(grid), dim3(MR_WAVES * 64), lds, stream, (const half_t*)A, (const uint8_t*)Wq,
+                               (const half_t*)S, (half_t*)Y, N, K, tiles_q, tiles_r, M | (zp << 8));
+            return hipGetLastError();
+        }
+    } // namespace
+
     bool w4a16_mrows_supported(int M, int N, int K, int num_cu) { return workspace::w4a16_mrows_fits(M, N, K, num_cu); }
     bool w4a16_mrows_preferred(int M, int N, int K, int num_cu) { return workspace::w4a16_mrows_preferred(M, N, K, num_cu); }
 
@@ -319,6 +546,15 @@ namespace nnf
     {
         if (!w4a16_mrows_supported(M, N, K, num_cu))
             return hipErrorInvalidValue;
+        if (!workspace::w4a16_mrows_fixed_k(M, K))
+        {
+            switch (workspace::w4a16_mrows_step_groups(M, K))
+            {
+            case 2: return launch_mrows_any<2, 2>(stream, A, Wq, S, Y, M, N, K, zp, num_cu);
+            case 3: return launch_mrows_any<3, 2>(stream, A, Wq, S, Y, M, N, K, zp, num_cu);
+            default: return launch_mrows_any<4, 2>(stream, A, Wq, S, Y, M, N, K, zp, num_cu);
+            }
+        }
         // K / 1024 = groups per wavefront and tile, walked in STEPS steps of GW groups.  Two steps per tile where
         // K / 1024 is even: with the two ring slots that is one tile in flight per wavefront (32 KiB per CU at
         // K = 4096, 64 KiB at 8192).  Measured against one step (two tiles in flight) and four steps (half a tile):
@@ -329,9 +565,7 @@ namespace nnf
         case 2: return launch_mrows<1, 2>(stream, A, Wq, S, Y, M, N, zp, num_cu);
         case 3: return launch_mrows<3, 1>(stream, A, Wq, S, Y, M, N, zp, num_cu);
         case 4: return launch_mrows<2, 2>(stream, A, Wq, S, Y, M, N, zp, num_cu);
-        case 5: return launch_mrows<5, 1>(stream, A, Wq, S, Y, M, N, zp, num_cu);
         case 6: return launch_mrows<3, 2>(stream, A, Wq, S, Y, M, N, zp, num_cu);
-        case 7: return launch_mrows<7, 1>(stream, A, Wq, S, Y, M, N, zp, num_cu);
         default: return launch_mrows<4, 2>(stream, A, Wq, S, Y, M, N, zp, num_cu);
         }
     }

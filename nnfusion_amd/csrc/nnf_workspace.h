@@ -362,36 +362,50 @@ namespace nnf
         // M = 16, and 12-33 % faster than the MFMA tile GEMM at M = 17 .. 32.
         inline bool w8a8_mrows_preferred(int M, int N, int K, int num_cu) { return w8a8_mrows_fits(M, N, K, num_cu); }
         // ---- 2 .. 16 activation rows (.. 32 up to K = 4096): the row-streaming MFMA kernel (w4a16_mrows.hip) ----
-        // One workgroup per CU, eight wavefronts that each own an eighth of K and keep their share of the activations
-        // in registers; K is a compile-time constant of the kernel (a multiple of 1024 up to 8192).  LDS: per
-        // wavefront two slots of a 16-row weight tile and of its scales, two sets of eight partial tiles, and the
-        // workgroup's finished tiles parked until the end.
+        // One workgroup per CU, eight wavefronts that each own an eighth of K (GW groups of every step of a tile) and
+        // keep their share of the activations in registers.  LDS: per wavefront two slots of GW KiB of weights and of
+        // their scales, two sets of eight partial tiles (one or two blocks of 16 rows), and the workgroup's finished
+        // tiles parked until the end.
+        // Two forms.  K / 1024 = 1, 2, 3, 4, 6, 8: K is a compile-time constant of the kernel.  Any other multiple of
+        // 256 up to 8192 (M <= 16): K is a run-time value, two steps of 8 * GW groups with the smallest GW (2, 3, 4)
+        // that covers K; wavefronts past the end of K fetch groups that another one already covers and discard them.
+        inline bool w4a16_mrows_fixed_k(int M, int K)
+        {
+            const int kw = K >> 10;
+            return !(K & 1023) && kw >= 1 && kw <= 8 && kw != 5 && kw != 7 && (M <= 16 || kw <= 4);
+        }
+        inline int w4a16_mrows_step_groups(int M, int K) // GW
+        {
+            const int kw = K >> 10, G = K >> 7;
+            if (w4a16_mrows_fixed_k(M, K))
+                return (kw & 1) ? kw : kw / 2; // even K / 1024: two steps per tile
+            return G <= 32 ? 2 : G <= 48 ? 3 : 4;
+        }
         inline size_t w4a16_mrows_lds_bytes(int K, int M, int tiles)
         {
-            const int kw = K >> 10, gw = (kw & 1) ? kw : kw / 2; // groups per wavefront and step (even K / 1024: two steps)
-            return (size_t)8 * 2 * gw * 1024 + 8 * 512 + (size_t)2 * 8 * (M <= 16 ? 1 : 2) * 1024 + (size_t)tiles * M * 64;
+            return (size_t)8 * 2 * w4a16_mrows_step_groups(M, K) * 1024 + 8 * 512 + (size_t)2 * 8 * (M <= 16 ? 1 : 2) * 1024 +
+                   (size_t)tiles * M * 64;
         }
         inline bool w4a16_mrows_fits(int M, int N, int K, int num_cu)
         {
-            if (M < 2 || M > 32 || N < 16 || num_cu < 1)
+            if (M < 2 || M > 32 || N < 16 || num_cu < 1 || K < 1024 || K > 8192 || (K & 255))
                 return false;
-            if (K < 1024 || K > 8192 || (K & 1023)) // K / 1024 is a template parameter of the kernel
-                return false;
-            if (M > 16 && K > 4096) // two blocks of 16 rows: 32 VGPRs of activations per group of K
-                return false;
-            if ((size_t)N * (size_t)(K >> 1) >= ((size_t)1 << 32)) // 32-bit offsets over the weight rows
+            if (!w4a16_mrows_fixed_k(M, K) && M > 16)
                 return false;
             const int n_tiles = (N + 15) / 16;
             const int grid = n_tiles < num_cu ? n_tiles : num_cu;
             return w4a16_mrows_lds_bytes(K, M, (n_tiles + grid - 1) / grid) <= LDS_BYTES_PER_CU;
         }
-        // Where the library picks it by itself, from measurements against the split-K MFMA GEMV on cold weights:
-        // K = 2048, 4096, 6144, 8192 (two steps per tile): 0-15 % faster at M = 2, 15-30 % at M = 16;
-        // K = 1024, 3072: 5-35 % faster;  K = 5120, 7168 (one step per tile: two whole tiles in flight): 5-30 %
-        // faster from eight rows on, level to 15 % slower below.
+        // Where the library picks it by itself, from measurements against the split-K MFMA GEMV on cold weights
+        // (M = 2 / 16): K = 2048, 4096, 6144, 8192: 0-15 % / 15-30 % faster;  K = 1024, 3072: 5-35 % faster;
+        // run-time K: 3-10 % / 15-35 % faster at K = 3584, 5120, 7168 (one case 10 % slower: N = K = 7168, M = 2), level
+        // at K = 2560, slower at K = 1536 and 2304, where most of what the wavefronts fetch is discarded: taken when at
+        // least three quarters of the fetched groups count.
         inline bool w4a16_mrows_preferred(int M, int N, int K, int num_cu)
         {
-            return (!(K & 2047) || K <= 4096 || M >= 8) && w4a16_mrows_fits(M, N, K, num_cu);
+            if (!w4a16_mrows_fits(M, N, K, num_cu))
+                return false;
+            return w4a16_mrows_fixed_k(M, K) || 4 * (K >> 7) >= 3 * 16 * w4a16_mrows_step_groups(M, K);
         }
         inline bool w4a16_variant_fits(int M, int N, int K, int variant, int num_cu)
         {

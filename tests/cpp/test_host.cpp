@@ -564,7 +564,7 @@ int main(int argc, char** argv)
         EXPECT(has(k1, "rocm_gemv_rows") && has(k1, "rocm_gemv_mfma") && has(k1, "rocm_gemm_mfma") && has(k1, "rocm_gemv_valu"));
         auto k8 = kinds(8, 4096, 4096);
         EXPECT(k8.size() == 5 && has(k8, "rocm_gemv_rows")); // 2 .. 16 rows: the row-streaming MFMA kernel
-        auto k8odd = kinds(8, 4096, 4224);                   // ... which takes multiples of 1024 up to 8192 only
+        auto k8odd = kinds(8, 4096, 4224);                   // ... which takes multiples of 256 (1024 .. 8192) only
         EXPECT(k8odd.size() == 4 && !has(k8odd, "rocm_gemv_rows"));
         auto k16 = kinds(16, 8192, 8192); // too many activations for one workgroup's LDS: no single-pass MFMA GEMV
         EXPECT(!has(k16, "rocm_gemv_mfma") && has(k16, "rocm_gemm_mfma"));

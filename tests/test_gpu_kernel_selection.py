@@ -31,7 +31,7 @@ def test_profiling_selector_times_every_candidate_and_keeps_the_fastest(gpu, nam
     expected = {"rocm", "rocm_gemm_mfma"}
     if m <= 16:
         expected |= {"rocm_gemv_mfma", "rocm_gemv_valu"}
-    if m <= 16:  # the row-streaming kernels: one row, or 2 .. 16 rows at K = 1024, 2048 .. 8192
+    if m <= 16:  # the row-streaming kernels: one row, or 2 .. 16 rows at K = 1024, 1280 .. 8192
         expected.add("rocm_gemv_rows")
     assert kinds == expected
     assert all(c["ms"] > 0 for c in res["candidates"]), res

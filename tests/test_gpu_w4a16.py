@@ -18,7 +18,7 @@ TOL = 1e-2
 def path(request):
     """Runs a test once per kernel family that can serve M <= 16 (auto = the library's own choice;
     rows_gemv = the M = 1 row-streaming kernel where it applies, otherwise the library's choice;
-    mfma_rows = the row-streaming MFMA kernel for 2 <= M <= 16 and K = 1024, 2048 .. 8192 where it applies)."""
+    mfma_rows = the row-streaming MFMA kernel for 2 <= M <= 16 and K = 1024, 1280 .. 8192 where it applies)."""
     from nnfusion_amd import _lib
 
     tune = _lib.kernels().nnf_internal_tune
@@ -61,6 +61,8 @@ def _check(y, ref):
     # fewer tiles than CUs, a single tile
     (2, 4096, 1024), (3, 8200, 2048), (16, 4111, 4096), (9, 22016, 4096), (16, 12288, 8192), (6, 16, 8192), (11, 48, 2048),
     (16, 40000, 1024), (5, 4096, 3072), (16, 13824, 5120), (7, 1000, 6144), (16, 2050, 7168), (2, 640, 5120),
+    # K a multiple of 256 but not of 1024 (and 5120 / 7168 above): the run-time-K form, wavefronts past the end of K
+    (3, 77, 3584), (16, 520, 2560), (9, 16, 1280), (11, 333, 4352), (5, 1000, 7936), (16, 18944, 3584),
     # 17 .. 32 rows (two blocks of 16), K <= 4096
     (17, 4096, 4096), (32, 22016, 4096), (24, 1000, 2048), (31, 77, 3072), (32, 300, 1024),
 ])
@@ -150,5 +152,5 @@ def test_every_kernel_variant_that_accepts_a_shape_matches_the_oracle(gpu, m, n,
                 ops.w4a16_gemm_variant(ta, tw, ts, name)
             assert e.value.status == -2
     assert "auto" in served and "gemm_mfma" in served
-    assert ("gemv_rows" in served) == (m == 1 or (m <= 32 and k % 1024 == 0 and k <= (8192 if m <= 16 else 4096)))
+    assert ("gemv_rows" in served) == (m == 1 or ((m <= 16 and k % 256 == 0 and 1024 <= k <= 8192) or (m <= 32 and k in (1024, 2048, 3072, 4096))))
     assert ("gemv_valu" in served) == (m <= 16)
