@@ -26,6 +26,10 @@ namespace nnf
                                   int K, int zp, int num_cu);
     bool w4a16_mrows_supported(int M, int N, int K, int num_cu);
     bool w4a16_mrows_preferred(int M, int N, int K, int num_cu); // where the library picks it without being told
+    // K above 8192: the same kernel over ranges of K, fp32 sums to partial[ranges][M][N] for the reduction pass
+    int w4a16_mrows_ksplits(int M, int N, int K, int num_cu); // 0: does not apply
+    hipError_t launch_w4a16_mrows_split(hipStream_t stream, const void* A, const void* Wq, const void* S, float* partial,
+                                        int M, int N, int K, int zp, int num_cu);
 
     hipError_t launch_w4a16_skinny(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M,
                                    int N, int K, int zp, int num_cu);

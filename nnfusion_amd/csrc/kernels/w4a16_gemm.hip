@@ -287,10 +287,16 @@ namespace nnf
         }
         // M <= 16 with too many activations for one workgroup's LDS: the GEMV kernel over ranges of K, then the
         // reduction pass (which applies the epilogue)
-        const int ksplits = (!gemm_only && partial_ws) ? w4a16_skinny_ksplits(M, n_rows, K) : 0;
+        // (K above 8192 in multiples of 256: the row-streaming MFMA kernel, otherwise the split-K one)
+        const int mr_splits = (!gemm_only && partial_ws && (g_tuning.force_path == 0 || g_tuning.force_path == 5))
+                                  ? w4a16_mrows_ksplits(M, n_rows, K, num_cu)
+                                  : 0;
+        const int ksplits = mr_splits ? mr_splits : (!gemm_only && partial_ws) ? w4a16_skinny_ksplits(M, n_rows, K) : 0;
         if (ksplits > 0)
         {
-            hipError_t e = launch_w4a16_skinny_split(stream, A, Wq, S, (float*)partial_ws, M, n_rows, K, zp, ksplits, num_cu);
+            hipError_t e = mr_splits
+                               ? launch_w4a16_mrows_split(stream, A, Wq, S, (float*)partial_ws, M, n_rows, K, zp, num_cu)
+                               : launch_w4a16_skinny_split(stream, A, Wq, S, (float*)partial_ws, M, n_rows, K, zp, ksplits, num_cu);
             if (e != hipSuccess)
                 return e;
             GemmParams p;

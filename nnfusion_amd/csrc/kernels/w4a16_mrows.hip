@@ -280,10 +280,13 @@ namespace nnf
     // need) and multiplies what another wavefront already covers by a scale of zero.
     // (Longer K in several passes over the tiles, each with its own part of the activations in registers, was
     // measured: every pass pays the start of the kernel again, and the split-K kernel is faster.)
+    // K above 8192: blockIdx.y numbers ranges of range_groups groups of K (the last one may be shorter, at least GW
+    // groups); the workgroups of a range write its fp32 sums to partial[range][M][N] for the reduction pass.
     // LDS as above (MB = 1).  pack = M | zp << 8.
     template <int GW, int STEPS>
     __global__ __launch_bounds__(512) void w4a16_mrows_any_kernel(const half_t* __restrict__ A, const uint8_t* __restrict__ Wq,
-                                                                  const half_t* __restrict__ S, half_t* __restrict__ Y, int N, int K,
+                                                                  const half_t* __restrict__ S, half_t* __restrict__ Y,
+                                                                  float* __restrict__ partial, int N, int K, int range_groups,
                                                                   int tiles_q, int tiles_r, int pack)
     {
         static_assert(GW >= 1 && GW <= 7 && STEPS >= 1 && GW * STEPS <= 8, "groups per wavefront and pass");
@@ -309,9 +312,10 @@ namespace nnf
         const int t0 = b * tiles_q + min(b, tiles_r);
         const int T = tiles_q + (b < tiles_r ? 1 : 0);
         auto row0_of = [&](int tile) { return __builtin_amdgcn_readfirstlane(min(tile * 16, N - 16)); };
+        const int g_lo = (int)blockIdx.y * range_groups, g_hi = min(G, g_lo + range_groups); // this workgroup's part of K
         // first group that wavefront `wave` owns in step st, and the first group it fetches
-        auto own_group = [&](int st) { return st * (8 * GW) + wave * GW; };
-        auto fetch_group = [&](int st) { return min(own_group(st), G - GW); };
+        auto own_group = [&](int st) { return g_lo + st * (8 * GW) + wave * GW; };
+        auto fetch_group = [&](int st) { return min(own_group(st), g_hi - GW); };
 
         uint8_t* ring = smem + wave * (2 * TILE_BYTES);
         uint8_t* sc_ring = smem + MR_WAVES * 2 * TILE_BYTES + wave * 512;
@@ -471,7 +475,11 @@ namespace nnf
             const int n = idx & 15;
             const int im = idx >> 4;
             const int it = im / M, m = im - it * M;
-            Y[(size_t)m * N + min((t0 + it) * 16, N - 16) + n] = (half_t)parked[idx];
+            const size_t at = (size_t)m * N + min((t0 + it) * 16, N - 16) + n;
+            if (partial)
+                partial[(size_t)blockIdx.y * M * N + at] = parked[idx];
+            else
+                Y[at] = (half_t)parked[idx];
         }
     }
 
@@ -514,14 +522,16 @@ namespace nnf
 
     namespace
     {
+        // ranges == 1: the whole of K, fp16 results to Y; otherwise ranges of range_groups groups, fp32 sums to partial
         template <int GW, int STEPS>
         hipError_t launch_mrows_any(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M, int N, int K,
-                                    int zp, int num_cu)
+                                    int zp, int num_cu, float* partial = nullptr, int ranges = 1, int range_groups = 64)
         {
             const int n_tiles = (N + 15) / 16;
-            const int grid = n_tiles < num_cu ? n_tiles : num_cu;
+            const int per_range = num_cu / ranges > 0 ? num_cu / ranges : 1;
+            const int grid = n_tiles < per_range ? n_tiles : per_range;
             const int tiles_q = n_tiles / grid, tiles_r = n_tiles % grid;
-            const size_t lds = workspace::w4a16_mrows_lds_bytes(K, M, tiles_q + (tiles_r ? 1 : 0));
+            const size_t lds = workspace::w4a16_mrows_lds_bytes_gw(GW, M, tiles_q + (tiles_r ? 1 : 0));
             if (lds > MAX_LDS_BYTES)
                 return hipErrorInvalidValue;
             auto kernel = &w4a16_mrows_any_kernel<GW, STEPS>;
@@ -532,8 +542,9 @@ namespace nnf
                 if (e != hipSuccess)
                     return e;
             }
-            hipLaunchKernelGGL(kernel, dim3(grid), dim3(MR_WAVES * 64), lds, stream, (const half_t*)A, (const uint8_t*)Wq,
-                               (const half_t*)S, (half_t*)Y, N, K, tiles_q, tiles_r, M | (zp << 8));
+            hipLaunchKernelGGL(kernel, dim3(grid, ranges), dim3(MR_WAVES * 64), lds, stream, (const half_t*)A, (const uint8_t*)Wq,
+                               (const half_t*)S, (half_t*)Y, ranges > 1 ? partial : nullptr, N, K, range_groups, tiles_q, tiles_r,
+                               M | (zp << 8));
             return hipGetLastError();
         }
     } // namespace
@@ -567,6 +578,24 @@ namespace nnf
         case 4: return launch_mrows<2, 2>(stream, A, Wq, S, Y, M, N, zp, num_cu);
         case 6: return launch_mrows<3, 2>(stream, A, Wq, S, Y, M, N, zp, num_cu);
         default: return launch_mrows<4, 2>(stream, A, Wq, S, Y, M, N, zp, num_cu);
+        }
+    }
+
+    // K above 8192 (a multiple of 256, 2 <= M <= 16): the run-time-K kernel over ranges of K, fp32 sums to
+    // partial[ranges][M][N] (the caller runs the reduction pass).  Returns the number of ranges; 0: does not apply.
+    int w4a16_mrows_ksplits(int M, int N, int K, int num_cu) { return workspace::w4a16_mrows_split(M, N, K, num_cu).ranges; }
+
+    hipError_t launch_w4a16_mrows_split(hipStream_t stream, const void* A, const void* Wq, const void* S, float* partial, int M,
+                                        int N, int K, int zp, int num_cu)
+    {
+        const workspace::MrowsSplit sp = workspace::w4a16_mrows_split(M, N, K, num_cu);
+        if (sp.ranges < 2 || !partial)
+            return hipErrorInvalidValue;
+        switch (sp.gw)
+        {
+        case 2: return launch_mrows_any<2, 2>(stream, A, Wq, S, nullptr, M, N, K, zp, num_cu, partial, sp.ranges, sp.range_groups);
+        case 3: return launch_mrows_any<3, 2>(stream, A, Wq, S, nullptr, M, N, K, zp, num_cu, partial, sp.ranges, sp.range_groups);
+        default: return launch_mrows_any<4, 2>(stream, A, Wq, S, nullptr, M, N, K, zp, num_cu, partial, sp.ranges, sp.range_groups);
         }
     }
 } // namespace nnf

@@ -73,6 +73,7 @@ int nnf_internal_tune(int key, int value)
     case 4: nnf::g_tuning.gemm_splits = value; return 0;
     case 5: nnf::workspace::skinny_min_splits() = value; return 0;
     case 6: nnf::skinny_direct_min_rows() = value > 0 ? value : 6; return 0;
+    case 7: nnf::workspace::mrows_forced_ranges() = value; return 0;
     default: return -1;
     }
 }
@@ -108,9 +109,10 @@ namespace
         const size_t a = nnf::workspace::gemm_partial_bytes(
             M, N, gate,
             nnf::workspace::plan_w4a16_gemm(M, N, K, gate, nnf::g_tuning.gemm_tile - 1, nnf::g_tuning.gemm_splits));
-        // the M <= 16 kernel over ranges of K writes partial sums too
+        // the M <= 16 kernels over ranges of K write partial sums too
         const size_t b = nnf::workspace::skinny_split_bytes(M, gate ? 2 * N : N, K);
-        return a > b ? a : b;
+        const size_t c = nnf::workspace::mrows_split_bytes(M, gate ? 2 * N : N, K);
+        return a > b ? (a > c ? a : c) : (b > c ? b : c);
     }
 } // namespace
 

@@ -281,6 +281,8 @@ namespace nnf
         // normalised activations of the RMSNorm prologue (fp16 [M, K])
         inline size_t rms_rows(int M, int K) { return (M > 0 && K > 0) ? align256((size_t)M * K * 2) : 0; }
 
+        inline size_t mrows_split_bytes(int M, int N_total, int K); // the row-streaming MFMA kernel over ranges of K
+
         // nnf_w4a16_gemm: [ partial sums ]
         inline size_t w4a16_gemm(int M, int N, int K, int)
         {
@@ -289,8 +291,8 @@ namespace nnf
             if (w4a16_skinny_fits(M, N, K))
                 return 0; // served by the skinny kernel
             const size_t a = gemm_partial_bytes(M, N, false, plan_w4a16_gemm(M, N, K, false));
-            const size_t b = skinny_split_bytes(M, N, K);
-            return a > b ? a : b;
+            const size_t b = skinny_split_bytes(M, N, K), c = mrows_split_bytes(M, N, K);
+            return a > b ? (a > c ? a : c) : (b > c ? b : c);
         }
         // nnf_w4a16_gemm_fused: [ normalised activations ][ partial sums ]
         inline size_t w4a16_gemm_fused(int M, int N, int K, int, int act)
@@ -299,8 +301,8 @@ namespace nnf
                 return 0;
             const bool gate = act == 1;
             const size_t a = gemm_partial_bytes(M, N, gate, plan_w4a16_gemm(M, N, K, gate));
-            const size_t b = skinny_split_bytes(M, gate ? 2 * N : N, K);
-            return rms_rows(M, K) + (a > b ? a : b);
+            const size_t b = skinny_split_bytes(M, gate ? 2 * N : N, K), c = mrows_split_bytes(M, gate ? 2 * N : N, K);
+            return rms_rows(M, K) + (a > b ? (a > c ? a : c) : (b > c ? b : c));
         }
         // ---- W8A8 ---------------------------------------------------------------------------------------
         constexpr int Q8_SKINNY_CPS = 2; // preferred chunks per wavefront and pass (more in flight measured slower)
@@ -381,10 +383,13 @@ namespace nnf
                 return (kw & 1) ? kw : kw / 2; // even K / 1024: two steps per tile
             return G <= 32 ? 2 : G <= 48 ? 3 : 4;
         }
+        inline size_t w4a16_mrows_lds_bytes_gw(int gw, int M, int tiles)
+        {
+            return (size_t)8 * 2 * gw * 1024 + 8 * 512 + (size_t)2 * 8 * (M <= 16 ? 1 : 2) * 1024 + (size_t)tiles * M * 64;
+        }
         inline size_t w4a16_mrows_lds_bytes(int K, int M, int tiles)
         {
-            return (size_t)8 * 2 * w4a16_mrows_step_groups(M, K) * 1024 + 8 * 512 + (size_t)2 * 8 * (M <= 16 ? 1 : 2) * 1024 +
-                   (size_t)tiles * M * 64;
+            return w4a16_mrows_lds_bytes_gw(w4a16_mrows_step_groups(M, K), M, tiles);
         }
         inline bool w4a16_mrows_fits(int M, int N, int K, int num_cu)
         {
@@ -395,6 +400,48 @@ namespace nnf
             const int n_tiles = (N + 15) / 16;
             const int grid = n_tiles < num_cu ? n_tiles : num_cu;
             return w4a16_mrows_lds_bytes(K, M, (n_tiles + grid - 1) / grid) <= LDS_BYTES_PER_CU;
+        }
+        // K above 8192 (a multiple of 256, 2 <= M <= 16): the run-time-K form over equal ranges of K (in whole pairs of
+        // groups; the last range may be shorter), each on its share of the CUs; fp32 sums per range, added by the
+        // reduction pass.  Every workgroup fetches the activations of its range, so shorter ranges mean less of that
+        // traffic (CUs x M x K / ranges x 2 bytes): ranges of at most 32 groups (GW = 2) measured fastest (K = 11008:
+        // 3 ranges, 14336: 4, 28672: 7-8; 10-25 % faster than the fewest ranges that fit the registers).
+        // experiments only: a number of ranges to use instead of the plan's (0: no preference)
+        inline int& mrows_forced_ranges()
+        {
+            static int v = 0;
+            return v;
+        }
+        struct MrowsSplit
+        {
+            int ranges = 0, range_groups = 0, gw = 0;
+        };
+        inline MrowsSplit w4a16_mrows_split(int M, int N, int K, int num_cu)
+        {
+            MrowsSplit sp;
+            if (M < 2 || M > 16 || N < 16 || K <= 8192 || K > 65536 || (K & 255) || num_cu < 16)
+                return sp;
+            const int G = K >> 7;
+            int ranges = (G + 31) / 32;
+            if (mrows_forced_ranges() >= 2)
+                ranges = mrows_forced_ranges();
+            const int rg = (((G + ranges - 1) / ranges) + 1) & ~1;
+            const int gw = rg <= 32 ? 2 : rg <= 48 ? 3 : 4;
+            if (G - (ranges - 1) * rg < gw) // the last range holds at least one wavefront's groups
+                return sp;
+            const int n_tiles = (N + 15) / 16, per_range = num_cu / ranges;
+            const int grid = n_tiles < per_range ? n_tiles : per_range;
+            if (w4a16_mrows_lds_bytes_gw(gw, M, (n_tiles + grid - 1) / grid) > LDS_BYTES_PER_CU)
+                return sp;
+            sp.ranges = ranges;
+            sp.range_groups = rg;
+            sp.gw = gw;
+            return sp;
+        }
+        inline size_t mrows_split_bytes(int M, int N_total, int K)
+        {
+            const int r = w4a16_mrows_split(M, N_total, K, PLAN_CUS).ranges;
+            return r ? align256((size_t)r * M * N_total * sizeof(float)) : 0;
         }
         // Where the library picks it by itself, from measurements against the split-K MFMA GEMV on cold weights
         // (M = 2 / 16): K = 2048, 4096, 6144, 8192: 0-15 % / 15-30 % faster;  K = 1024, 3072: 5-35 % faster;
@@ -485,7 +532,10 @@ namespace nnf
                 return 0;
             size_t a = gemm_partial_bytes(M, I, true, plan_w4a16_gemm(M, I, H, true));
             size_t b = gemm_partial_bytes(M, H, false, plan_w4a16_gemm(M, H, I, false));
-            const size_t c = skinny_split_bytes(M, 2 * I, H), d = skinny_split_bytes(M, H, I);
+            size_t c = skinny_split_bytes(M, 2 * I, H), d = skinny_split_bytes(M, H, I);
+            const size_t e = mrows_split_bytes(M, 2 * I, H), f = mrows_split_bytes(M, H, I);
+            c = c > e ? c : e;
+            d = d > f ? d : f;
             a = a > b ? a : b;
             b = c > d ? c : d;
             return fused_mlp_partial_offset(M, H, I) + (a > b ? a : b);

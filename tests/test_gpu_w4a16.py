@@ -63,6 +63,8 @@ def _check(y, ref):
     (16, 40000, 1024), (5, 4096, 3072), (16, 13824, 5120), (7, 1000, 6144), (16, 2050, 7168), (2, 640, 5120),
     # K a multiple of 256 but not of 1024 (and 5120 / 7168 above): the run-time-K form, wavefronts past the end of K
     (3, 77, 3584), (16, 520, 2560), (9, 16, 1280), (11, 333, 4352), (5, 1000, 7936), (16, 18944, 3584),
+    # K above 8192: ranges of K on the run-time-K form, fp32 partial sums, reduction pass
+    (16, 4111, 11008), (8, 1000, 14336), (16, 300, 28672), (7, 4096, 11008), (12, 333, 8448), (6, 16, 16384),
     # 17 .. 32 rows (two blocks of 16), K <= 4096
     (17, 4096, 4096), (32, 22016, 4096), (24, 1000, 2048), (31, 77, 3072), (32, 300, 1024),
 ])
