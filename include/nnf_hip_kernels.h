@@ -82,7 +82,7 @@ enum nnf_w4a16_variant
     NNF_W4A16_GEMV_MFMA = 2, /* M <= 16: MFMA 16x16x32 weight-streaming kernel (activations held per workgroup) */
     NNF_W4A16_GEMM_MFMA = 3, /* any M: MFMA 32x32x16 tile GEMM (may split K: workspace) */
     NNF_W4A16_GEMV_ROWS = 4  /* row-streaming kernels, one workgroup per CU: M = 1 (K a multiple of 256, 1024 .. 16384),
-                                M = 2 .. 16 on MFMA (K a multiple of 256, 1024 .. 8192, N >= 16), M = 17 .. 32 for K = 1024, 2048, 3072, 4096 */
+                                M = 2 .. 16 on MFMA (K a multiple of 256, 1024 .. 8192, N >= 16), M = 17 .. 32 up to K = 4096 */
 };
 /* 1 when the variant can serve the shape (decided on the host, for a 256-CU device), else 0. */
 int nnf_w4a16_variant_supported(int M, int N, int K, int group, int variant);

@@ -282,14 +282,15 @@ namespace nnf
     // measured: every pass pays the start of the kernel again, and the split-K kernel is faster.)
     // K above 8192: blockIdx.y numbers ranges of range_groups groups of K (the last one may be shorter, at least GW
     // groups); the workgroups of a range write its fp32 sums to partial[range][M][N] for the reduction pass.
-    // LDS as above (MB = 1).  pack = M | zp << 8.
-    template <int GW, int STEPS>
+    // MB = 2 (17 .. 32 rows): at most four groups per wavefront.  LDS as above.  pack = M | zp << 8.
+    template <int GW, int STEPS, int MB>
     __global__ __launch_bounds__(512) void w4a16_mrows_any_kernel(const half_t* __restrict__ A, const uint8_t* __restrict__ Wq,
                                                                   const half_t* __restrict__ S, half_t* __restrict__ Y,
                                                                   float* __restrict__ partial, int N, int K, int range_groups,
                                                                   int tiles_q, int tiles_r, int pack)
     {
-        static_assert(GW >= 1 && GW <= 7 && STEPS >= 1 && GW * STEPS <= 8, "groups per wavefront and pass");
+        static_assert(GW >= 1 && GW <= 7 && STEPS >= 1 && GW * STEPS <= 8, "groups per wavefront");
+        static_assert(MB == 1 || (MB == 2 && GW * STEPS <= 4), "two blocks of rows: 32 VGPRs per group");
         constexpr int GA = GW * STEPS;         // groups of a wavefront
         constexpr int SLICE = GW * 64;         // a wavefront's bytes of a weight row per step
         constexpr int TILE_BYTES = 16 * SLICE; // = GW KiB: GW wavefront-wide loads
@@ -320,7 +321,7 @@ namespace nnf
         uint8_t* ring = smem + wave * (2 * TILE_BYTES);
         uint8_t* sc_ring = smem + MR_WAVES * 2 * TILE_BYTES + wave * 512;
         uint8_t* red = smem + MR_WAVES * 2 * TILE_BYTES + MR_WAVES * 512; // [2][8][1024]
-        float* parked = reinterpret_cast<float*>(red + 2 * MR_WAVES * 1024);
+        float* parked = reinterpret_cast<float*>(red + 2 * MR_WAVES * MB * 1024);
 
         auto swz = [](int r) { return GW % 4 == 0 ? (r & 15) : GW % 2 == 0 ? (r >> 1) & 7 : (r >> 2) & 3; };
         uint32_t w_off[GW];
@@ -359,43 +360,53 @@ namespace nnf
         const uintx4 cvec = {ce2, co2, ce2, co2};
         const uint32_t rd_base = (uint32_t)col * SLICE;
         const int rd_swz = swz(col);
-        const uint32_t red_addr = lds_address(red) + (uint32_t)(wave * 1024 + lane * 16);
+        const uint32_t red_addr = lds_address(red) + (uint32_t)(wave * (MB * 1024) + lane * 16);
         const uint32_t parked_addr = lds_address(parked);
-        const uint8_t* a_row = reinterpret_cast<const uint8_t*>(A) + (size_t)min(col, M - 1) * (size_t)(K * 2) + kq * 64;
+        const uint8_t* a_row[MB];
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+            a_row[mb] = reinterpret_cast<const uint8_t*>(A) + (size_t)min(mb * 16 + col, M - 1) * (size_t)(K * 2) + kq * 64;
         int slot = 0;
         {
             // ---- the activations: straight into the MFMA operand registers ------------------------------------------
-            uintx4 areg[GA][4];
-            floatx4 ncorr[GA];
+            uintx4 areg[MB][GA][4];
+            floatx4 ncorr[MB][GA];
 #pragma unroll
-            for (int st = 0; st < STEPS; ++st)
-            {
-                const uint8_t* a_src = a_row + (size_t)fetch_group(st) * 256;
+            for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-                for (int g = 0; g < GW; ++g)
+                for (int st = 0; st < STEPS; ++st)
+                {
+                    const uint8_t* a_src = a_row[mb] + (size_t)fetch_group(st) * 256;
+#pragma unroll
+                    for (int g = 0; g < GW; ++g)
+#pragma unroll
+                        for (int j = 0; j < 4; ++j)
+                            areg[mb][st * GW + g][j] = *reinterpret_cast<const uintx4*>(a_src + g * 256 + j * 16);
+                }
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+                for (int g = 0; g < GA; ++g)
+                {
+                    floatx4 t = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                     for (int j = 0; j < 4; ++j)
-                        areg[st * GW + g][j] = *reinterpret_cast<const uintx4*>(a_src + g * 256 + j * 16);
-            }
-#pragma unroll
-            for (int g = 0; g < GA; ++g)
-            {
-                floatx4 t = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                for (int j = 0; j < 4; ++j)
-                {
-                    uintx4 a = permute_a8(areg[g][j]);
-                    a.y = as_u32(as_half2(a.y) * sixteenth);
-                    a.w = as_u32(as_half2(a.w) * sixteenth);
-                    areg[g][j] = a;
-                    t = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, a), __builtin_bit_cast(half8_t, cvec), t,
-                                                               0, 0, 0);
+                    {
+                        uintx4 a = permute_a8(areg[mb][g][j]);
+                        a.y = as_u32(as_half2(a.y) * sixteenth);
+                        a.w = as_u32(as_half2(a.w) * sixteenth);
+                        areg[mb][g][j] = a;
+                        t = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, a),
+                                                                   __builtin_bit_cast(half8_t, cvec), t, 0, 0, 0);
+                    }
+                    ncorr[mb][g] = t;
                 }
-                ncorr[g] = t;
-            }
             for (int it = 0; it < T; ++it)
             {
-                floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+                floatx4 acc[MB];
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb)
+                    acc[mb] = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int st = 0; st < STEPS; ++st)
                 {
@@ -424,7 +435,10 @@ namespace nnf
 #pragma unroll
                     for (int g = 0; g < GW; ++g)
                     {
-                        floatx4 t = ncorr[st * GW + g];
+                        floatx4 t[MB];
+#pragma unroll
+                        for (int mb = 0; mb < MB; ++mb)
+                            t[mb] = ncorr[mb][st * GW + g];
                         const uint32_t ww[4] = {wv[g].x, wv[g].y, wv[g].z, wv[g].w};
 #pragma unroll
                         for (int j = 0; j < 4; ++j)
@@ -436,30 +450,38 @@ namespace nnf
                             bq.y = (w & MASK_HI) | MAGIC;
                             bq.z = (w8 & MASK_LO) | MAGIC;
                             bq.w = (w8 & MASK_HI) | MAGIC;
-                            t = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, areg[st * GW + g][j]),
-                                                                       __builtin_bit_cast(half8_t, bq), t, 0, 0, 0);
+#pragma unroll
+                            for (int mb = 0; mb < MB; ++mb)
+                                t[mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, areg[mb][st * GW + g][j]),
+                                                                               __builtin_bit_cast(half8_t, bq), t[mb], 0, 0, 0);
                         }
-                        acc.x = __builtin_fmaf(t.x, sv[g], acc.x);
-                        acc.y = __builtin_fmaf(t.y, sv[g], acc.y);
-                        acc.z = __builtin_fmaf(t.z, sv[g], acc.z);
-                        acc.w = __builtin_fmaf(t.w, sv[g], acc.w);
+#pragma unroll
+                        for (int mb = 0; mb < MB; ++mb)
+                        {
+                            acc[mb].x = __builtin_fmaf(t[mb].x, sv[g], acc[mb].x);
+                            acc[mb].y = __builtin_fmaf(t[mb].y, sv[g], acc[mb].y);
+                            acc[mb].z = __builtin_fmaf(t[mb].z, sv[g], acc[mb].z);
+                            acc[mb].w = __builtin_fmaf(t[mb].w, sv[g], acc[mb].w);
+                        }
                     }
                 }
                 const int rbuf = it & 1;
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb)
                 {
-                    const uint32_t at = red_addr + (uint32_t)(rbuf * MR_WAVES * 1024);
-                    asm volatile("ds_write_b128 %0, %1" ::"v"(at), "v"(acc) : "memory");
+                    const uint32_t at = red_addr + (uint32_t)(rbuf * MR_WAVES * MB * 1024 + mb * 1024);
+                    asm volatile("ds_write_b128 %0, %1" ::"v"(at), "v"(acc[mb]) : "memory");
                 }
                 asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-                if (tid < 256)
+                if (tid < MB * 256)
                 {
-                    const int e = tid >> 6;
-                    const float* rp = reinterpret_cast<const float*>(red + rbuf * MR_WAVES * 1024) + lane * 4 + e;
+                    const int mb = tid >> 8, e = (tid >> 6) & 3;
+                    const float* rp = reinterpret_cast<const float*>(red + rbuf * MR_WAVES * MB * 1024 + mb * 1024) + lane * 4 + e;
                     float sum = 0.f;
 #pragma unroll
                     for (int w = 0; w < MR_WAVES; ++w)
-                        sum += rp[w * 256];
-                    const int m = 4 * kq + e;
+                        sum += rp[w * (MB * 256)];
+                    const int m = 16 * mb + 4 * kq + e;
                     if (m < M)
                     {
                         const uint32_t at = parked_addr + (uint32_t)(((it * M + m) * 16 + col) * 4);
@@ -523,9 +545,9 @@ namespace nnf
     namespace
     {
         // ranges == 1: the whole of K, fp16 results to Y; otherwise ranges of range_groups groups, fp32 sums to partial
-        template <int GW, int STEPS>
-        hipError_t launch_mrows_any(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M, int N, int K,
-                                    int zp, int num_cu, float* partial = nullptr, int ranges = 1, int range_groups = 64)
+        template <int GW, int STEPS, int MB>
+        hipError_t launch_mrows_any_mb(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M, int N, int K,
+                                    int zp, int num_cu, float* partial, int ranges, int range_groups)
         {
             const int n_tiles = (N + 15) / 16;
             const int per_range = num_cu / ranges > 0 ? num_cu / ranges : 1;
@@ -534,7 +556,7 @@ namespace nnf
             const size_t lds = workspace::w4a16_mrows_lds_bytes_gw(GW, M, tiles_q + (tiles_r ? 1 : 0));
             if (lds > MAX_LDS_BYTES)
                 return hipErrorInvalidValue;
-            auto kernel = &w4a16_mrows_any_kernel<GW, STEPS>;
+            auto kernel = &w4a16_mrows_any_kernel<GW, STEPS, MB>;
             if (lds > 64 * 1024)
             {
                 hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -546,6 +568,17 @@ namespace nnf
                                (const half_t*)S, (half_t*)Y, ranges > 1 ? partial : nullptr, N, K, range_groups, tiles_q, tiles_r,
                                M | (zp << 8));
             return hipGetLastError();
+        }
+
+        template <int GW, int STEPS>
+        hipError_t launch_mrows_any(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M, int N, int K,
+                                    int zp, int num_cu, float* partial = nullptr, int ranges = 1, int range_groups = 64)
+        {
+            if (M <= 16)
+                return launch_mrows_any_mb<GW, STEPS, 1>(stream, A, Wq, S, Y, M, N, K, zp, num_cu, partial, ranges, range_groups);
+            if constexpr (GW * STEPS <= 4)
+                return launch_mrows_any_mb<GW, STEPS, 2>(stream, A, Wq, S, Y, M, N, K, zp, num_cu, partial, ranges, range_groups);
+            return hipErrorInvalidValue;
         }
     } // namespace
 

@@ -395,13 +395,13 @@ namespace nnf
         {
             if (M < 2 || M > 32 || N < 16 || num_cu < 1 || K < 1024 || K > 8192 || (K & 255))
                 return false;
-            if (!w4a16_mrows_fixed_k(M, K) && M > 16)
+            if (!w4a16_mrows_fixed_k(M, K) && M > 16 && K > 4096) // two blocks of rows: at most four groups per wavefront
                 return false;
             const int n_tiles = (N + 15) / 16;
             const int grid = n_tiles < num_cu ? n_tiles : num_cu;
             return w4a16_mrows_lds_bytes(K, M, (n_tiles + grid - 1) / grid) <= LDS_BYTES_PER_CU;
         }
-        // K above 8192 (a multiple of 256, 2 <= M <= 16): the run-time-K form over equal ranges of K (in whole pairs of
+        // K above 8192 (above 4096 for 17 .. 32 rows; a multiple of 256): the run-time-K form over equal ranges of K (in whole pairs of
         // groups; the last range may be shorter), each on its share of the CUs; fp32 sums per range, added by the
         // reduction pass.  Every workgroup fetches the activations of its range, so shorter ranges mean less of that
         // traffic (CUs x M x K / ranges x 2 bytes): ranges of at most 32 groups (GW = 2) measured fastest (K = 11008:
@@ -419,7 +419,7 @@ namespace nnf
         inline MrowsSplit w4a16_mrows_split(int M, int N, int K, int num_cu)
         {
             MrowsSplit sp;
-            if (M < 2 || M > 16 || N < 16 || K <= 8192 || K > 65536 || (K & 255) || num_cu < 16)
+            if (M < 2 || M > 32 || N < 16 || K <= (M <= 16 ? 8192 : 4096) || K > 65536 || (K & 255) || num_cu < 16)
                 return sp;
             const int G = K >> 7;
             int ranges = (G + 31) / 32;

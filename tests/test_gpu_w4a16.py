@@ -65,6 +65,8 @@ def _check(y, ref):
     (3, 77, 3584), (16, 520, 2560), (9, 16, 1280), (11, 333, 4352), (5, 1000, 7936), (16, 18944, 3584),
     # K above 8192: ranges of K on the run-time-K form, fp32 partial sums, reduction pass
     (16, 4111, 11008), (8, 1000, 14336), (16, 300, 28672), (7, 4096, 11008), (12, 333, 8448), (6, 16, 16384),
+    # 17 .. 32 rows over ranges of K (K above 4096), and in one launch with a run-time K
+    (32, 4111, 8192), (17, 1000, 11008), (24, 300, 14336), (32, 520, 5120), (20, 77, 3584), (31, 2000, 2560),
     # 17 .. 32 rows (two blocks of 16), K <= 4096
     (17, 4096, 4096), (32, 22016, 4096), (24, 1000, 2048), (31, 77, 3072), (32, 300, 1024),
 ])
@@ -154,5 +156,5 @@ def test_every_kernel_variant_that_accepts_a_shape_matches_the_oracle(gpu, m, n,
                 ops.w4a16_gemm_variant(ta, tw, ts, name)
             assert e.value.status == -2
     assert "auto" in served and "gemm_mfma" in served
-    assert ("gemv_rows" in served) == (m == 1 or ((m <= 16 and k % 256 == 0 and 1024 <= k <= 8192) or (m <= 32 and k in (1024, 2048, 3072, 4096))))
+    assert ("gemv_rows" in served) == (m == 1 or (m <= 32 and k % 256 == 0 and 1024 <= k <= (8192 if m <= 16 else 4096)))
     assert ("gemv_valu" in served) == (m <= 16)
