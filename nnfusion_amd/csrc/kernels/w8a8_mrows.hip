@@ -1,4 +1,5 @@
-// W8A8 (int8 x int8 -> int32, exact) for 2 <= M <= 32 activation rows and K = 2048, 4096, 6144 or 8192: the
+// W8A8 (int8 x int8 -> int32, exact) for 2 <= M <= 32 activation rows and K a multiple of 256 from 2048 to 16384
+// (M <= 16; to 8192 for 17 .. 32 rows): the
 // row-streaming kernel of w4a16_mrows.hip on the int8 matrix cores.
 //
 //   acc[M,N] = A[M,K] . W[N,K]^T  (int32, bit exact);  Y = fp16((float)acc * s_tok[m] * s_ch[n])
@@ -19,6 +20,9 @@
 //   * Per step 4 (M <= 16) or 8 v_mfma_i32_16x16x64_i8, weights as the B operand.  Per tile the eight partial
 //     16 x 16 (x 2) tiles meet in LDS (one LDS-only barrier, two alternating buffers), integer adds (the result
 //     does not depend on the order); the sums are parked in LDS and scaled / written after the last tile.
+//   * K need not fill the last step: a wavefront whose 256 bytes would lie past the end of K fetches the last
+//     256 bytes of the row instead (every wavefront issues the same number of loads, which the hand-written wait
+//     counts need) and multiplies them with activations of zero.
 //   * LDS writes inside the loop are inline ds_write instructions: ahead of an LDS write that it can see, the
 //     compiler waits for every LDS-bound load in flight.
 #include "nnf_device.h"
@@ -41,17 +45,16 @@ namespace nnf
 
     // LDS (bytes): weights [8 wavefronts][NS slots][4 KiB] | partial tiles [2][8][MB KiB] |
     //              parked sums [tiles of the workgroup][M][16] int32
-    // STEPS = K / 2048 (steps per tile and wavefront), MB = blocks of 16 activation rows (1 or 2), NS = ring slots.
+    // STEPS = ceil(K / 2048) (steps per tile and wavefront), MB = blocks of 16 activation rows (1 or 2), NS = ring slots.
     // A workgroup's tiles: tiles_q, one more for the first tiles_r workgroups.
     template <int STEPS, int MB, int NS, bool RAW_ACC>
     __global__ __launch_bounds__(512) void w8a8_mrows_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ W,
                                                              const float* __restrict__ s_tok, const float* __restrict__ s_ch,
                                                              half_t* __restrict__ Y, int32_t* __restrict__ ACC, int M, int N,
-                                                             int tiles_q, int tiles_r)
+                                                             int K, int tiles_q, int tiles_r)
     {
-        static_assert(STEPS >= 1 && STEPS <= 4 && (MB == 1 || MB == 2) && NS >= 2 && NS <= 4, "shape of the kernel");
-        constexpr int K = STEPS * 2048;
-        constexpr int CH = K / 8 / 64;   // a wavefront's 64-byte chunks of a row (one MFMA each)
+        static_assert(STEPS >= 1 && STEPS * MB <= 8 && (MB == 1 || MB == 2) && NS >= 2 && NS <= 4, "shape of the kernel");
+        constexpr int CH = STEPS * 4;    // a wavefront's 64-byte chunks of a row (one MFMA each)
         constexpr int LPS = 4;           // loads per step and wavefront
         extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
 
@@ -78,11 +81,14 @@ namespace nnf
         for (int c = 0; c < LPS; ++c)
         {
             const int r = c * 4 + kq, q = col;
-            w_off[c] = (uint32_t)r * K + (uint32_t)wave * Q8MR_STEP_BYTES + (uint32_t)((q ^ r) << 4);
+            w_off[c] = (uint32_t)r * (uint32_t)K + (uint32_t)((q ^ r) << 4);
         }
+        // where this wavefront's 256 bytes of step st start within a row; past the end of K: the row's last 256 bytes
+        auto own_byte = [&](int st) { return st * (Q8MR_WAVES * Q8MR_STEP_BYTES) + wave * Q8MR_STEP_BYTES; };
+        auto fetch_byte = [&](int st) { return min(own_byte(st), K - Q8MR_STEP_BYTES); };
         // step st (0 .. STEPS-1) of tile `tile` into slot `slot`
         auto issue = [&](int tile, int st, int slot) {
-            const int8_t* wsrc = W + (size_t)row0_of(tile) * K + st * (Q8MR_WAVES * Q8MR_STEP_BYTES);
+            const int8_t* wsrc = W + (size_t)row0_of(tile) * K + fetch_byte(st);
 #pragma unroll
             for (int c = 0; c < LPS; ++c)
                 __builtin_amdgcn_global_load_lds((q8mr_global_ptr_t)(wsrc + w_off[c]),
@@ -101,11 +107,14 @@ namespace nnf
 #pragma unroll
             for (int mb = 0; mb < MB; ++mb)
             {
-                const uint32_t a_off = (uint32_t)min(mb * 16 + col, M - 1) * (uint32_t)K + (uint32_t)wave * Q8MR_STEP_BYTES + (uint32_t)kq * 16u;
+                const uint8_t* a_row = reinterpret_cast<const uint8_t*>(A) + (size_t)min(mb * 16 + col, M - 1) * (size_t)K + kq * 16;
 #pragma unroll
                 for (int c = 0; c < CH; ++c)
-                    areg[mb][c] = *reinterpret_cast<const uintx4*>(reinterpret_cast<const uint8_t*>(A) +
-                                                                    (size_t)(a_off + (c >> 2) * (Q8MR_WAVES * Q8MR_STEP_BYTES) + (c & 3) * 64));
+                {
+                    const uintx4 v = *reinterpret_cast<const uintx4*>(a_row + fetch_byte(c >> 2) + (c & 3) * 64);
+                    const bool inside = own_byte(c >> 2) < K; // otherwise another wavefront covers these bytes
+                    areg[mb][c] = inside ? v : uintx4{0u, 0u, 0u, 0u};
+                }
             }
         }
 
@@ -204,7 +213,7 @@ namespace nnf
     {
         template <int STEPS, int MB, int NS, bool RAW>
         hipError_t launch_q8_mrows(hipStream_t stream, const void* A, const void* s_tok, const void* W, const void* s_ch, void* Y,
-                                   void* acc, int M, int N, int num_cu)
+                                   void* acc, int M, int N, int K, int num_cu)
         {
             const int n_tiles = (N + 15) / 16;
             const int grid = n_tiles < num_cu ? n_tiles : num_cu;
@@ -221,29 +230,36 @@ namespace nnf
                     return e;
             }
             hipLaunchKernelGGL(kernel, dim3(grid), dim3(Q8MR_WAVES * 64), lds, stream, (const int8_t*)A, (const int8_t*)W,
-                               (const float*)s_tok, (const float*)s_ch, (half_t*)Y, (int32_t*)acc, M, N, tiles_q, tiles_r);
+                               (const float*)s_tok, (const float*)s_ch, (half_t*)Y, (int32_t*)acc, M, N, K, tiles_q, tiles_r);
             return hipGetLastError();
         }
 
         template <int STEPS, bool RAW>
         hipError_t launch_q8_mrows_m(hipStream_t stream, const void* A, const void* s_tok, const void* W, const void* s_ch,
-                                     void* Y, void* acc, int M, int N, int num_cu)
+                                     void* Y, void* acc, int M, int N, int K, int num_cu)
         {
             constexpr int NS = workspace::W8A8_MROWS_SLOTS;
-            return M <= 16 ? launch_q8_mrows<STEPS, 1, NS, RAW>(stream, A, s_tok, W, s_ch, Y, acc, M, N, num_cu)
-                           : launch_q8_mrows<STEPS, 2, NS, RAW>(stream, A, s_tok, W, s_ch, Y, acc, M, N, num_cu);
+            if (M <= 16)
+                return launch_q8_mrows<STEPS, 1, NS, RAW>(stream, A, s_tok, W, s_ch, Y, acc, M, N, K, num_cu);
+            if constexpr (STEPS <= 4)
+                return launch_q8_mrows<STEPS, 2, NS, RAW>(stream, A, s_tok, W, s_ch, Y, acc, M, N, K, num_cu);
+            return hipErrorInvalidValue;
         }
 
         template <bool RAW>
         hipError_t launch_q8_mrows_any(hipStream_t stream, const void* A, const void* s_tok, const void* W, const void* s_ch,
                                        void* Y, void* acc, int M, int N, int K, int num_cu)
         {
-            switch (K >> 11)
+            switch ((K + 2047) >> 11) // steps of 2 KiB of K
             {
-            case 1: return launch_q8_mrows_m<1, RAW>(stream, A, s_tok, W, s_ch, Y, acc, M, N, num_cu);
-            case 2: return launch_q8_mrows_m<2, RAW>(stream, A, s_tok, W, s_ch, Y, acc, M, N, num_cu);
-            case 3: return launch_q8_mrows_m<3, RAW>(stream, A, s_tok, W, s_ch, Y, acc, M, N, num_cu);
-            default: return launch_q8_mrows_m<4, RAW>(stream, A, s_tok, W, s_ch, Y, acc, M, N, num_cu);
+            case 1: return launch_q8_mrows_m<1, RAW>(stream, A, s_tok, W, s_ch, Y, acc, M, N, K, num_cu);
+            case 2: return launch_q8_mrows_m<2, RAW>(stream, A, s_tok, W, s_ch, Y, acc, M, N, K, num_cu);
+            case 3: return launch_q8_mrows_m<3, RAW>(stream, A, s_tok, W, s_ch, Y, acc, M, N, K, num_cu);
+            case 4: return launch_q8_mrows_m<4, RAW>(stream, A, s_tok, W, s_ch, Y, acc, M, N, K, num_cu);
+            case 5: return launch_q8_mrows_m<5, RAW>(stream, A, s_tok, W, s_ch, Y, acc, M, N, K, num_cu);
+            case 6: return launch_q8_mrows_m<6, RAW>(stream, A, s_tok, W, s_ch, Y, acc, M, N, K, num_cu);
+            case 7: return launch_q8_mrows_m<7, RAW>(stream, A, s_tok, W, s_ch, Y, acc, M, N, K, num_cu);
+            default: return launch_q8_mrows_m<8, RAW>(stream, A, s_tok, W, s_ch, Y, acc, M, N, K, num_cu);
             }
         }
     } // namespace

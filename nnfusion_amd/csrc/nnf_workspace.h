@@ -340,6 +340,7 @@ namespace nnf
             return pl.cps != 0 && pl.lds + 16 * 1024 <= LDS_BYTES_PER_CU;
         }
         // ---- W8A8, 2 .. 32 activation rows: the row-streaming MFMA kernel (w8a8_mrows.hip) ----
+        // K a multiple of 256 up to 16384 (8192 for 17 .. 32 rows).
         // One workgroup per CU, eight wavefronts that each own an eighth of K (256 bytes of every 2 KiB) and keep
         // their share of the activations in registers.  LDS: per wavefront a ring of 4-KiB slots, two sets of eight
         // partial tiles (one or two blocks of 16 rows), the workgroup's finished tiles parked until the end.
@@ -353,7 +354,8 @@ namespace nnf
         {
             if (M < 2 || M > 32 || N < 16 || num_cu < 1)
                 return false;
-            if (K < 2048 || K > 8192 || (K & 2047)) // K / 2048 is a template parameter of the kernel
+            // ceil(K / 2048) steps per tile (a template parameter): 16 VGPRs of activations per step and block of rows
+            if (K < 1024 || K > (M <= 16 ? 16384 : 8192) || (K & 255))
                 return false;
             const int n_tiles = (N + 15) / 16;
             const int grid = n_tiles < num_cu ? n_tiles : num_cu;
@@ -362,7 +364,12 @@ namespace nnf
         // Where the library picks it by itself: everywhere it applies.  Measured on cold weights against the split-K
         // M <= 16 kernel it is level to 10 % faster up to M = 14 (2 % slower at M = 2, N = K = 8192), 5-30 % faster at
         // M = 16, and 12-33 % faster than the MFMA tile GEMM at M = 17 .. 32.
-        inline bool w8a8_mrows_preferred(int M, int N, int K, int num_cu) { return w8a8_mrows_fits(M, N, K, num_cu); }
+        // (Where K does not fill the last step, wavefronts fetch bytes that do not count: at least three quarters of what
+        // is fetched must count.)
+        inline bool w8a8_mrows_preferred(int M, int N, int K, int num_cu)
+        {
+            return w8a8_mrows_fits(M, N, K, num_cu) && 4 * K >= 3 * 2048 * ((K + 2047) >> 11);
+        }
         // ---- 2 .. 16 activation rows (.. 32 up to K = 4096): the row-streaming MFMA kernel (w4a16_mrows.hip) ----
         // One workgroup per CU, eight wavefronts that each own an eighth of K (GW groups of every step of a tile) and
         // keep their share of the activations in registers.  LDS: per wavefront two slots of GW KiB of weights and of

@@ -16,7 +16,7 @@ def _t(gpu, *arrays):
 
 
 # "auto": the library's own choice (the M = 1 / M <= 16 / M <= 32 kernels where they apply); "skinny": the split-K
-# M <= 16 kernel; "mfma_rows": the row-streaming MFMA kernel (2 <= M <= 32, K = 2048 .. 8192); otherwise the MFMA GEMM with a
+# M <= 16 kernel; "mfma_rows": the row-streaming MFMA kernel (2 <= M <= 32, K = 1024 .. 16384 in multiples of 256); otherwise the MFMA GEMM with a
 # forced tile (1 big 256x256, 2 mid 128x128, 3 small 64x256) and number of K ranges (int32 partial sums,
 # added exactly by the reduction pass)
 @pytest.fixture(params=["auto", "skinny", "mfma_rows", (0, 0), (1, 1), (1, 2), (2, 1), (2, 3), (3, 1), (3, 2)],
@@ -56,6 +56,9 @@ def _big_ws(gpu):
     # a single tile, more tiles than CUs
     (2, 512, 2048), (16, 4111, 4096), (17, 1000, 6144), (32, 8192, 8192), (31, 16, 8192), (24, 12288, 4096),
     (8, 40000, 2048), (20, 77, 4096),
+    # K that does not fill the last 2-KiB step, K above 8192
+    (16, 4111, 11008), (5, 100, 1024), (9, 520, 2560), (32, 300, 7168), (24, 1000, 3584), (12, 2000, 14336), (16, 64, 16384),
+    (17, 250, 5376),
 ])
 def test_accumulators_bit_exact(gpu, path, m, n, k):
     import torch
