@@ -45,6 +45,106 @@ namespace nnf
         constexpr int mr_vmcnt(int n) { return (n & 0xF) | ((n >> 4) << 14) | (0x7 << 4) | (0xF << 8); }
     } // namespace
 
+    // ---- pieces shared by the two forms of the kernel ----------------------------------------------------------------
+    // The activations of a wavefront as loaded -> the MFMA operand order of the nibble trick (pairs (a0,a4) (a1,a5)
+    // (a2,a6) (a3,a7), the odd words times 1/16), and per group the constant part of its sum (an MFMA against a
+    // constant operand), negative, as the initial accumulator of the group.
+    template <int MB, int GA>
+    __device__ __forceinline__ void mrows_prepare_a(uintx4 (&areg)[MB][GA][4], floatx4 (&ncorr)[MB][GA], int zp)
+    {
+        const half2_t sixteenth = half2_t{(half_t)0.0625f, (half_t)0.0625f};
+        const half_t ceh = (half_t)(-(1024.0f + (float)zp)), coh = (half_t)(-16.0f * (64.0f + (float)zp)); // exact
+        const uint32_t ce2 = as_u32(half2_t{ceh, ceh}), co2 = as_u32(half2_t{coh, coh});
+        const uintx4 cvec = {ce2, co2, ce2, co2};
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+            for (int g = 0; g < GA; ++g)
+            {
+                floatx4 t = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                {
+                    uintx4 a = permute_a8(areg[mb][g][j]);
+                    a.y = as_u32(as_half2(a.y) * sixteenth);
+                    a.w = as_u32(as_half2(a.w) * sixteenth);
+                    areg[mb][g][j] = a;
+                    t = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, a), __builtin_bit_cast(half8_t, cvec), t,
+                                                               0, 0, 0);
+                }
+                ncorr[mb][g] = t;
+            }
+    }
+
+    // One group of 128 along K: the lane's 16 bytes of weights (32 nibbles) against group ga of the activations,
+    // the fp32 group sum times the group's scale onto acc.  consts = {0x64006400, 0x000F000F, 0x00F000F0}.
+    template <int MB, int GA>
+    __device__ __forceinline__ void mrows_group(floatx4 (&acc)[MB], const uintx4 (&areg)[MB][GA][4],
+                                                const floatx4 (&ncorr)[MB][GA], int ga, uintx4 wv, float scale, uint32_t MAGIC,
+                                                uint32_t MASK_LO, uint32_t MASK_HI)
+    {
+        floatx4 t[MB];
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+            t[mb] = ncorr[mb][ga];
+        const uint32_t ww[4] = {wv.x, wv.y, wv.z, wv.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+        {
+            const uint32_t w = ww[j];
+            const uint32_t w8 = w >> 8;
+            uintx4 bq;
+            bq.x = (w & MASK_LO) | MAGIC;  // 1024 + (q0, q4)
+            bq.y = (w & MASK_HI) | MAGIC;  // 1024 + 16 (q1, q5)
+            bq.z = (w8 & MASK_LO) | MAGIC; // 1024 + (q2, q6)
+            bq.w = (w8 & MASK_HI) | MAGIC; // 1024 + 16 (q3, q7)
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb)
+                t[mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, areg[mb][ga][j]),
+                                                               __builtin_bit_cast(half8_t, bq), t[mb], 0, 0, 0);
+        }
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+        {
+            acc[mb].x = __builtin_fmaf(t[mb].x, scale, acc[mb].x);
+            acc[mb].y = __builtin_fmaf(t[mb].y, scale, acc[mb].y);
+            acc[mb].z = __builtin_fmaf(t[mb].z, scale, acc[mb].z);
+            acc[mb].w = __builtin_fmaf(t[mb].w, scale, acc[mb].w);
+        }
+    }
+
+    // End of a tile: the partial 16 x 16 tiles of the eight wavefronts meet in LDS (red: [2][8][MB KiB], buffer
+    // rbuf), MB x 256 threads add them and park the sums of tile `it` ([tile][M][16] fp32 at parked_addr).
+    // D layout: lane (n = col, kq), element e: row m = 16 mb + 4 kq + e.
+    template <int MB>
+    __device__ __forceinline__ void mrows_reduce_park(const floatx4 (&acc)[MB], const uint8_t* red, uint32_t red_addr,
+                                                      uint32_t parked_addr, int rbuf, int it, int M, int tid)
+    {
+        const int lane = tid & 63, col = lane & 15, kq = lane >> 4;
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+        {
+            const uint32_t at = red_addr + (uint32_t)(rbuf * MR_WAVES * MB * 1024 + mb * 1024);
+            asm volatile("ds_write_b128 %0, %1" ::"v"(at), "v"(acc[mb]) : "memory");
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        if (tid < MB * 256)
+        {
+            const int mb = tid >> 8, e = (tid >> 6) & 3;
+            const float* rp = reinterpret_cast<const float*>(red + rbuf * MR_WAVES * MB * 1024 + mb * 1024) + lane * 4 + e;
+            float sum = 0.f;
+#pragma unroll
+            for (int w = 0; w < MR_WAVES; ++w)
+                sum += rp[w * (MB * 256)];
+            const int m = 16 * mb + 4 * kq + e;
+            if (m < M)
+            {
+                const uint32_t at = parked_addr + (uint32_t)(((it * M + m) * 16 + col) * 4);
+                asm volatile("ds_write_b32 %0, %1" ::"v"(at), "v"(sum) : "memory");
+            }
+        }
+    }
+
     // K = GW * STEPS * 1024; MB = blocks of 16 activation rows (1 or 2).
     // LDS (bytes): weights [8 wavefronts][2 slots][GW KiB] | scales [8][2][256] | partial tiles [2][8][MB KiB] |
     //              parked sums [tiles of the workgroup][M][16] fp32
@@ -142,30 +242,7 @@ namespace nnf
                         a_bytes + (size_t)(a_off + (g / GW) * (SPAN * 4) + (g % GW) * 256 + j * 16));
         }
         floatx4 ncorr[MB][GA];
-        {
-            const half2_t sixteenth = half2_t{(half_t)0.0625f, (half_t)0.0625f};
-            const half_t ceh = (half_t)(-(1024.0f + (float)zp)), coh = (half_t)(-16.0f * (64.0f + (float)zp)); // exact
-            const uint32_t ce2 = as_u32(half2_t{ceh, ceh}), co2 = as_u32(half2_t{coh, coh});
-            const uintx4 cvec = {ce2, co2, ce2, co2};
-#pragma unroll
-            for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-                for (int g = 0; g < GA; ++g)
-                {
-                    floatx4 t = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                    for (int j = 0; j < 4; ++j)
-                    {
-                        uintx4 a = permute_a8(areg[mb][g][j]);
-                        a.y = as_u32(as_half2(a.y) * sixteenth);
-                        a.w = as_u32(as_half2(a.w) * sixteenth);
-                        areg[mb][g][j] = a;
-                        t = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, a),
-                                                                   __builtin_bit_cast(half8_t, cvec), t, 0, 0, 0);
-                    }
-                    ncorr[mb][g] = t;
-                }
-        }
+        mrows_prepare_a<MB, GA>(areg, ncorr, zp);
 
         // ---- tile loop ---------------------------------------------------------------------------------------
         // operand reads of a slot: lane (n = col, kq), group g: piece g*4 + kq of row n
@@ -204,63 +281,9 @@ namespace nnf
                 slot ^= 1;
 #pragma unroll
                 for (int g = 0; g < GW; ++g)
-                {
-                    floatx4 t[MB];
-#pragma unroll
-                    for (int mb = 0; mb < MB; ++mb)
-                        t[mb] = ncorr[mb][st * GW + g];
-                    const uint32_t ww[4] = {wv[g].x, wv[g].y, wv[g].z, wv[g].w};
-#pragma unroll
-                    for (int j = 0; j < 4; ++j)
-                    {
-                        const uint32_t w = ww[j];
-                        const uint32_t w8 = w >> 8;
-                        uintx4 bq;
-                        bq.x = (w & MASK_LO) | MAGIC;  // 1024 + (q0, q4)
-                        bq.y = (w & MASK_HI) | MAGIC;  // 1024 + 16 (q1, q5)
-                        bq.z = (w8 & MASK_LO) | MAGIC; // 1024 + (q2, q6)
-                        bq.w = (w8 & MASK_HI) | MAGIC; // 1024 + 16 (q3, q7)
-#pragma unroll
-                        for (int mb = 0; mb < MB; ++mb)
-                            t[mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, areg[mb][st * GW + g][j]),
-                                                                           __builtin_bit_cast(half8_t, bq), t[mb], 0, 0, 0);
-                    }
-#pragma unroll
-                    for (int mb = 0; mb < MB; ++mb)
-                    {
-                        acc[mb].x = __builtin_fmaf(t[mb].x, sv[g], acc[mb].x);
-                        acc[mb].y = __builtin_fmaf(t[mb].y, sv[g], acc[mb].y);
-                        acc[mb].z = __builtin_fmaf(t[mb].z, sv[g], acc[mb].z);
-                        acc[mb].w = __builtin_fmaf(t[mb].w, sv[g], acc[mb].w);
-                    }
-                }
+                    mrows_group<MB, GA>(acc, areg, ncorr, st * GW + g, wv[g], sv[g], MAGIC, MASK_LO, MASK_HI);
             }
-            const int rbuf = it & 1;
-            // partial tiles -> LDS (D layout: lane (n = col, kq), element e: row m = 16 mb + 4 kq + e)
-#pragma unroll
-            for (int mb = 0; mb < MB; ++mb)
-            {
-                const uint32_t at = red_addr + (uint32_t)(rbuf * MR_WAVES * MB * 1024 + mb * 1024);
-                asm volatile("ds_write_b128 %0, %1" ::"v"(at), "v"(acc[mb]) : "memory");
-            }
-            asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-            // MB x 256 threads: thread (mb, e, lane') adds the eight partial sums of output
-            // (m = 16 mb + 4 (lane' >> 4) + e, n = lane' & 15)
-            if (tid < MB * 256)
-            {
-                const int mb = tid >> 8, e = (tid >> 6) & 3;
-                const float* rp = reinterpret_cast<const float*>(red + rbuf * MR_WAVES * MB * 1024 + mb * 1024) + lane * 4 + e;
-                float sum = 0.f;
-#pragma unroll
-                for (int w = 0; w < MR_WAVES; ++w)
-                    sum += rp[w * (MB * 256)];
-                const int m = 16 * mb + 4 * kq + e;
-                if (m < M)
-                {
-                    const uint32_t at = parked_addr + (uint32_t)(((it * M + m) * 16 + col) * 4);
-                    asm volatile("ds_write_b32 %0, %1" ::"v"(at), "v"(sum) : "memory");
-                }
-            }
+            mrows_reduce_park<MB>(acc, red, red_addr, parked_addr, it & 1, it, M, tid);
         }
         __builtin_amdgcn_s_waitcnt(mr_vmcnt(0)); // the reloads past the end, before the LDS goes away
         asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
@@ -354,10 +377,6 @@ namespace nnf
         issue(t0, 0, 0);
         issue(t0 + min(1 / STEPS, T - 1), 1 % STEPS, 1);
 
-        const half2_t sixteenth = half2_t{(half_t)0.0625f, (half_t)0.0625f};
-        const half_t ceh = (half_t)(-(1024.0f + (float)zp)), coh = (half_t)(-16.0f * (64.0f + (float)zp)); // exact
-        const uint32_t ce2 = as_u32(half2_t{ceh, ceh}), co2 = as_u32(half2_t{coh, coh});
-        const uintx4 cvec = {ce2, co2, ce2, co2};
         const uint32_t rd_base = (uint32_t)col * SLICE;
         const int rd_swz = swz(col);
         const uint32_t red_addr = lds_address(red) + (uint32_t)(wave * (MB * 1024) + lane * 16);
@@ -383,24 +402,7 @@ namespace nnf
                         for (int j = 0; j < 4; ++j)
                             areg[mb][st * GW + g][j] = *reinterpret_cast<const uintx4*>(a_src + g * 256 + j * 16);
                 }
-#pragma unroll
-            for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-                for (int g = 0; g < GA; ++g)
-                {
-                    floatx4 t = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                    for (int j = 0; j < 4; ++j)
-                    {
-                        uintx4 a = permute_a8(areg[mb][g][j]);
-                        a.y = as_u32(as_half2(a.y) * sixteenth);
-                        a.w = as_u32(as_half2(a.w) * sixteenth);
-                        areg[mb][g][j] = a;
-                        t = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, a),
-                                                                   __builtin_bit_cast(half8_t, cvec), t, 0, 0, 0);
-                    }
-                    ncorr[mb][g] = t;
-                }
+            mrows_prepare_a<MB, GA>(areg, ncorr, zp);
             for (int it = 0; it < T; ++it)
             {
                 floatx4 acc[MB];
@@ -434,60 +436,9 @@ namespace nnf
                     slot ^= 1;
 #pragma unroll
                     for (int g = 0; g < GW; ++g)
-                    {
-                        floatx4 t[MB];
-#pragma unroll
-                        for (int mb = 0; mb < MB; ++mb)
-                            t[mb] = ncorr[mb][st * GW + g];
-                        const uint32_t ww[4] = {wv[g].x, wv[g].y, wv[g].z, wv[g].w};
-#pragma unroll
-                        for (int j = 0; j < 4; ++j)
-                        {
-                            const uint32_t w = ww[j];
-                            const uint32_t w8 = w >> 8;
-                            uintx4 bq;
-                            bq.x = (w & MASK_LO) | MAGIC;
-                            bq.y = (w & MASK_HI) | MAGIC;
-                            bq.z = (w8 & MASK_LO) | MAGIC;
-                            bq.w = (w8 & MASK_HI) | MAGIC;
-#pragma unroll
-                            for (int mb = 0; mb < MB; ++mb)
-                                t[mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, areg[mb][st * GW + g][j]),
-                                                                               __builtin_bit_cast(half8_t, bq), t[mb], 0, 0, 0);
-                        }
-#pragma unroll
-                        for (int mb = 0; mb < MB; ++mb)
-                        {
-                            acc[mb].x = __builtin_fmaf(t[mb].x, sv[g], acc[mb].x);
-                            acc[mb].y = __builtin_fmaf(t[mb].y, sv[g], acc[mb].y);
-                            acc[mb].z = __builtin_fmaf(t[mb].z, sv[g], acc[mb].z);
-                            acc[mb].w = __builtin_fmaf(t[mb].w, sv[g], acc[mb].w);
-                        }
-                    }
+                        mrows_group<MB, GA>(acc, areg, ncorr, st * GW + g, wv[g], sv[g], MAGIC, MASK_LO, MASK_HI);
                 }
-                const int rbuf = it & 1;
-#pragma unroll
-                for (int mb = 0; mb < MB; ++mb)
-                {
-                    const uint32_t at = red_addr + (uint32_t)(rbuf * MR_WAVES * MB * 1024 + mb * 1024);
-                    asm volatile("ds_write_b128 %0, %1" ::"v"(at), "v"(acc[mb]) : "memory");
-                }
-                asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-                if (tid < MB * 256)
-                {
-                    const int mb = tid >> 8, e = (tid >> 6) & 3;
-                    const float* rp = reinterpret_cast<const float*>(red + rbuf * MR_WAVES * MB * 1024 + mb * 1024) + lane * 4 + e;
-                    float sum = 0.f;
-#pragma unroll
-                    for (int w = 0; w < MR_WAVES; ++w)
-                        sum += rp[w * (MB * 256)];
-                    const int m = 16 * mb + 4 * kq + e;
-                    if (m < M)
-                    {
-                        const uint32_t at = parked_addr + (uint32_t)(((it * M + m) * 16 + col) * 4);
-                        asm volatile("ds_write_b32 %0, %1" ::"v"(at), "v"(sum) : "memory");
-                    }
-                }
+                mrows_reduce_park<MB>(acc, red, red_addr, parked_addr, it & 1, it, M, tid);
             }
         }
         __builtin_amdgcn_s_waitcnt(mr_vmcnt(0)); // the reloads past the end, before the LDS goes away
