@@ -257,7 +257,8 @@ namespace nnf
                 return e;
             A = rms_ws;
         }
-        // M <= 16: the bandwidth-bound GEMV kernel on the (normalised) activations, then a small element-wise
+        // M <= 16 (<= 32 where the row-streaming MFMA kernel applies): the bandwidth-bound GEMV kernel on the
+        // (normalised) activations, then a small element-wise
         // kernel for whatever epilogue is asked for
         const int n_rows = gate ? 2 * N : N;
         // the products go to scratch first when the epilogue cannot work in place: the [M, 2N] gate | up pair, or a
@@ -268,7 +269,7 @@ namespace nnf
                           w4a16_gemv_rows_supported(M, n_rows, K, num_cu);
         const bool mrows = !gemm_only && ((g_tuning.force_path == 5 && w4a16_mrows_supported(M, n_rows, K, num_cu)) ||
                                           (g_tuning.force_path == 0 && w4a16_mrows_preferred(M, n_rows, K, num_cu)));
-        if (!gemm_only && M <= 16 && (rows || mrows || w4a16_skinny_supported(M, n_rows, K)) && (!via_scratch || partial_ws))
+        if (!gemm_only && (rows || mrows || (M <= 16 && w4a16_skinny_supported(M, n_rows, K))) && (!via_scratch || partial_ws))
         {
             void* y_gemv = via_scratch ? partial_ws : Y;
             hipError_t e = rows ? launch_w4a16_gemv_rows(stream, A, Wq, S, y_gemv, n_rows, K, zp, num_cu)

@@ -104,7 +104,8 @@ const char* nnf_status_string(int status)
 namespace
 {
     // partial-sum bytes of the GEMM plan in force (the automatic one unless an experiment overrides it)
-    size_t tuned_partial_bytes(int M, int N, int K, bool gate)
+    // fused: a call that may run the GEMV kernel into scratch (fp16 [M, N or 2N]) ahead of an element-wise epilogue
+    size_t tuned_partial_bytes(int M, int N, int K, bool gate, bool fused = false)
     {
         const size_t a = nnf::workspace::gemm_partial_bytes(
             M, N, gate,
@@ -112,7 +113,9 @@ namespace
         // the M <= 16 kernels over ranges of K write partial sums too
         const size_t b = nnf::workspace::skinny_split_bytes(M, gate ? 2 * N : N, K);
         const size_t c = nnf::workspace::mrows_split_bytes(M, gate ? 2 * N : N, K);
-        return a > b ? (a > c ? a : c) : (b > c ? b : c);
+        const size_t d = fused ? nnf::workspace::gemv_scratch_bytes(M, gate ? 2 * N : N) : 0;
+        const size_t bc = b > c ? b : c, ad = a > d ? a : d;
+        return ad > bc ? ad : bc;
     }
 } // namespace
 
@@ -226,7 +229,7 @@ int nnf_w4a16_gemm_fused(nnf_stream_t stream, const void* A, const void* Wq, con
     // combinations without a fused kernel (see launch_w4a16_gemm)
     if (act == NNF_ACT_SILU_GATE && (bias || residual))
         return NNF_ERR_UNSUPPORTED_SHAPE;
-    const size_t need = (rms_gamma ? nnf::workspace::rms_rows(M, K) : 0) + tuned_partial_bytes(M, N, K, act == NNF_ACT_SILU_GATE);
+    const size_t need = (rms_gamma ? nnf::workspace::rms_rows(M, K) : 0) + tuned_partial_bytes(M, N, K, act == NNF_ACT_SILU_GATE, true);
     if (need > 0 && (!workspace || !aligned16(workspace) || workspace_bytes < need))
         return NNF_ERR_WORKSPACE_TOO_SMALL;
     DeviceInfo dev;
@@ -328,7 +331,7 @@ int nnf_fused_mlp_w4a16(nnf_stream_t stream, const void* x, const void* gamma, f
     if (group != 128 || H % group != 0 || I % group != 0 || zp < 0 || zp > 15)
         return NNF_ERR_UNSUPPORTED_SHAPE;
     {
-        const size_t a = tuned_partial_bytes(M, I, H, true), b = tuned_partial_bytes(M, H, I, false);
+        const size_t a = tuned_partial_bytes(M, I, H, true, true), b = tuned_partial_bytes(M, H, I, false);
         if (!workspace || workspace_bytes < nnf::workspace::fused_mlp_partial_offset(M, H, I) + (a > b ? a : b))
             return NNF_ERR_WORKSPACE_TOO_SMALL;
     }

@@ -282,6 +282,9 @@ namespace nnf
         inline size_t rms_rows(int M, int K) { return (M > 0 && K > 0) ? align256((size_t)M * K * 2) : 0; }
 
         inline size_t mrows_split_bytes(int M, int N_total, int K); // the row-streaming MFMA kernel over ranges of K
+        // Fused calls with at most 32 rows may run the GEMV kernel into scratch and an element-wise epilogue from
+        // there (the [M, 2N] gate | up pair; a residual that is the output buffer): fp16 [M, N_total].
+        inline size_t gemv_scratch_bytes(int M, int N_total) { return (M > 0 && M <= 32) ? align256((size_t)M * N_total * 2) : 0; }
 
         // nnf_w4a16_gemm: [ partial sums ]
         inline size_t w4a16_gemm(int M, int N, int K, int)
@@ -302,7 +305,9 @@ namespace nnf
             const bool gate = act == 1;
             const size_t a = gemm_partial_bytes(M, N, gate, plan_w4a16_gemm(M, N, K, gate));
             const size_t b = skinny_split_bytes(M, gate ? 2 * N : N, K), c = mrows_split_bytes(M, gate ? 2 * N : N, K);
-            return rms_rows(M, K) + (a > b ? (a > c ? a : c) : (b > c ? b : c));
+            const size_t d = gemv_scratch_bytes(M, gate ? 2 * N : N);
+            const size_t bc = b > c ? b : c, ad = a > d ? a : d;
+            return rms_rows(M, K) + (ad > bc ? ad : bc);
         }
         // ---- W8A8 ---------------------------------------------------------------------------------------
         constexpr int Q8_SKINNY_CPS = 2; // preferred chunks per wavefront and pass (more in flight measured slower)
@@ -541,7 +546,9 @@ namespace nnf
             size_t b = gemm_partial_bytes(M, H, false, plan_w4a16_gemm(M, H, I, false));
             size_t c = skinny_split_bytes(M, 2 * I, H), d = skinny_split_bytes(M, H, I);
             const size_t e = mrows_split_bytes(M, 2 * I, H), f = mrows_split_bytes(M, H, I);
+            const size_t g = gemv_scratch_bytes(M, 2 * I); // gate | up of the first GEMM at M <= 32
             c = c > e ? c : e;
+            c = c > g ? c : g;
             d = d > f ? d : f;
             a = a > b ? a : b;
             b = c > d ? c : d;

@@ -19,7 +19,10 @@ def _rms(x):
     return float(np.sqrt(np.mean(np.asarray(x, np.float64) ** 2)))
 
 
-@pytest.mark.parametrize("m,h,i", [(64, 256, 384), (256, 512, 1408), (37, 1024, 2816)])
+# the last four: the decode route (GEMV kernels with element-wise epilogues; M = 1, a few rows, two blocks of 16 rows,
+# a down projection over ranges of K)
+@pytest.mark.parametrize("m,h,i", [(64, 256, 384), (256, 512, 1408), (37, 1024, 2816), (1, 1024, 2816), (8, 2048, 5632),
+                                   (24, 1024, 2816), (16, 1024, 8704)])
 def test_mlp_matches_unfused_oracle(gpu, m, h, i):
     import torch
 

@@ -256,14 +256,15 @@ def test_fused_silu_gate(gpu, plan):
     assert _rms(err) <= 1e-3 * _rms(ref)
 
 
-@pytest.mark.parametrize("m", [1, 5, 16])
-def test_fused_small_m_goes_through_the_gemv_kernel(gpu, m):
-    """Decode shapes with a prologue / epilogue: RMSNorm pre-pass, the M <= 16 GEMV kernel, an element-wise epilogue."""
+@pytest.mark.parametrize("m,n,k", [(1, 320, 1024), (5, 320, 1024), (16, 320, 1024), (2, 520, 4096), (24, 320, 2048), (32, 1000, 4096),
+                                   (16, 136, 11008), (24, 264, 8192), (7, 320, 3584)])
+def test_fused_small_m_goes_through_the_gemv_kernel(gpu, m, n, k):
+    """Decode shapes with a prologue / epilogue: RMSNorm pre-pass, a GEMV kernel (M = 1; 2 .. 32 rows in one launch or
+    over ranges of K), an element-wise epilogue or the reduction pass's."""
     import torch
 
     from nnfusion_amd import ops
 
-    n, k = 320, 1024
     a, wq, s = datagen.w4a16_case(11, m, 2 * n, k)
     gamma = datagen.normal_f16(11, datagen.S_GAMMA, (k,), 1.0, 0.1)
     bias = datagen.normal_f16(11, datagen.S_BIAS, (n,))
@@ -285,7 +286,7 @@ def test_fused_small_m_goes_through_the_gemv_kernel(gpu, m):
     assert _rms(err) <= 1e-3 * _rms(refg) and err.max() <= 5e-2 * _rms(refg)
 
 
-@pytest.mark.parametrize("m", [3, 200])
+@pytest.mark.parametrize("m", [3, 24, 200])
 def test_residual_may_alias_the_output(gpu, m):
     import torch
 
