@@ -148,7 +148,15 @@ def main():
         for i in range(2 * args.layers):
             step(i)
         torch.cuda.synchronize()
-        print(f"pmc probe: copy of {PROBE_BYTES} bytes x4, then {2 * args.layers} sweeps", flush=True)
+        # the same weights with 16 activation rows (the row-streaming MFMA kernel; K = 11008: three ranges of K
+        # and the reduction pass), over every resident layer
+        ws16 = torch.empty(16 << 20, dtype=torch.uint8, device=dev)
+        for shapes in layers:
+            for (_, wq, s, _) in shapes:
+                a16 = torch.empty((16, wq.shape[1] * 2), dtype=torch.float16, device=dev).normal_()
+                ops.w4a16_gemm(a16, wq, s, workspace=ws16)
+        torch.cuda.synchronize()
+        print(f"pmc probe: copy of {PROBE_BYTES} bytes x4, then {2 * args.layers} sweeps, then {args.layers} sweeps with 16 rows", flush=True)
         return
 
     # ---- warm-up (untimed), then exactly K steps in the timed region ------------------------------
