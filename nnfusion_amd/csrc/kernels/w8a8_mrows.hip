@@ -1,5 +1,5 @@
 // W8A8 (int8 x int8 -> int32, exact) for 2 <= M <= 32 activation rows and K a multiple of 256 from 2048 to 16384
-// (M <= 16; to 8192 for 17 .. 32 rows): the
+// (M <= 16; to 12288 for 17 .. 32 rows): the
 // row-streaming kernel of w4a16_mrows.hip on the int8 matrix cores.
 //
 //   acc[M,N] = A[M,K] . W[N,K]^T  (int32, bit exact);  Y = fp16((float)acc * s_tok[m] * s_ch[n])
@@ -53,7 +53,7 @@ namespace nnf
                                                              half_t* __restrict__ Y, int32_t* __restrict__ ACC, int M, int N,
                                                              int K, int tiles_q, int tiles_r)
     {
-        static_assert(STEPS >= 1 && STEPS * MB <= 8 && (MB == 1 || MB == 2) && NS >= 2 && NS <= 4, "shape of the kernel");
+        static_assert(STEPS >= 1 && STEPS * MB <= 12 && STEPS <= 8 && (MB == 1 || MB == 2) && NS >= 2 && NS <= 4, "shape of the kernel");
         constexpr int CH = STEPS * 4;    // a wavefront's 64-byte chunks of a row (one MFMA each)
         constexpr int LPS = 4;           // loads per step and wavefront
         extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -241,7 +241,7 @@ namespace nnf
             constexpr int NS = workspace::W8A8_MROWS_SLOTS;
             if (M <= 16)
                 return launch_q8_mrows<STEPS, 1, NS, RAW>(stream, A, s_tok, W, s_ch, Y, acc, M, N, K, num_cu);
-            if constexpr (STEPS <= 4)
+            if constexpr (STEPS <= 6) // 16 VGPRs of activations per step and block of rows
                 return launch_q8_mrows<STEPS, 2, NS, RAW>(stream, A, s_tok, W, s_ch, Y, acc, M, N, K, num_cu);
             return hipErrorInvalidValue;
         }

@@ -345,7 +345,7 @@ namespace nnf
             return pl.cps != 0 && pl.lds + 16 * 1024 <= LDS_BYTES_PER_CU;
         }
         // ---- W8A8, 2 .. 32 activation rows: the row-streaming MFMA kernel (w8a8_mrows.hip) ----
-        // K a multiple of 256 up to 16384 (8192 for 17 .. 32 rows).
+        // K a multiple of 256 up to 16384 (12288 for 17 .. 32 rows).
         // One workgroup per CU, eight wavefronts that each own an eighth of K (256 bytes of every 2 KiB) and keep
         // their share of the activations in registers.  LDS: per wavefront a ring of 4-KiB slots, two sets of eight
         // partial tiles (one or two blocks of 16 rows), the workgroup's finished tiles parked until the end.
@@ -360,7 +360,7 @@ namespace nnf
             if (M < 2 || M > 32 || N < 16 || num_cu < 1)
                 return false;
             // ceil(K / 2048) steps per tile (a template parameter): 16 VGPRs of activations per step and block of rows
-            if (K < 1024 || K > (M <= 16 ? 16384 : 8192) || (K & 255))
+            if (K < 1024 || K > (M <= 16 ? 16384 : 12288) || (K & 255))
                 return false;
             const int n_tiles = (N + 15) / 16;
             const int grid = n_tiles < num_cu ? n_tiles : num_cu;

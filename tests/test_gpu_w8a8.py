@@ -58,7 +58,7 @@ def _big_ws(gpu):
     (8, 40000, 2048), (20, 77, 4096),
     # K that does not fill the last 2-KiB step, K above 8192
     (16, 4111, 11008), (5, 100, 1024), (9, 520, 2560), (32, 300, 7168), (24, 1000, 3584), (12, 2000, 14336), (16, 64, 16384),
-    (17, 250, 5376),
+    (17, 250, 5376), (32, 4111, 11008), (20, 300, 12288), (24, 100, 9216),
 ])
 def test_accumulators_bit_exact(gpu, path, m, n, k):
     import torch
