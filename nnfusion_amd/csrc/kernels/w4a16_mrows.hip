@@ -114,7 +114,7 @@ namespace nnf
     }
 
     // End of a tile: the partial 16 x 16 tiles of the eight wavefronts meet in LDS (red: [2][8][MB KiB], buffer
-    // rbuf), MB x 256 threads add them and park the sums of tile `it` ([tile][M][16] fp32 at parked_addr).
+    // rbuf), MB x 256 outputs per tile are added by the 512 threads and parked: they add them and park the sums of tile `it` ([tile][M][16] fp32 at parked_addr).
     // D layout: lane (n = col, kq), element e: row m = 16 mb + 4 kq + e.
     template <int MB>
     __device__ __forceinline__ void mrows_reduce_park(const floatx4 (&acc)[MB], const uint8_t* red, uint32_t red_addr,
@@ -128,9 +128,9 @@ namespace nnf
             asm volatile("ds_write_b128 %0, %1" ::"v"(at), "v"(acc[mb]) : "memory");
         }
         asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-        if (tid < MB * 256)
+        for (int o = tid; o < MB * 256; o += MR_WAVES * 64) // (o & 63 == lane)
         {
-            const int mb = tid >> 8, e = (tid >> 6) & 3;
+            const int mb = o >> 8, e = (o >> 6) & 3;
             const float* rp = reinterpret_cast<const float*>(red + rbuf * MR_WAVES * MB * 1024 + mb * 1024) + lane * 4 + e;
             float sum = 0.f;
 #pragma unroll
@@ -305,7 +305,8 @@ namespace nnf
     // measured: every pass pays the start of the kernel again, and the split-K kernel is faster.)
     // K above 8192: blockIdx.y numbers ranges of range_groups groups of K (the last one may be shorter, at least GW
     // groups); the workgroups of a range write its fp32 sums to partial[range][M][N] for the reduction pass.
-    // MB = 2 (17 .. 32 rows): at most four groups per wavefront.  LDS as above.  pack = M | zp << 8.
+    // MB = 2 (17 .. 32 rows): at most four groups per wavefront; MB = 4 (33 .. 64 rows): at most two.  LDS as above.
+    // pack = M | zp << 8.
     template <int GW, int STEPS, int MB>
     __global__ __launch_bounds__(512) void w4a16_mrows_any_kernel(const half_t* __restrict__ A, const uint8_t* __restrict__ Wq,
                                                                   const half_t* __restrict__ S, half_t* __restrict__ Y,
@@ -313,7 +314,7 @@ namespace nnf
                                                                   int tiles_q, int tiles_r, int pack)
     {
         static_assert(GW >= 1 && GW <= 7 && STEPS >= 1 && GW * STEPS <= 8, "groups per wavefront");
-        static_assert(MB == 1 || (MB == 2 && GW * STEPS <= 4), "two blocks of rows: 32 VGPRs per group");
+        static_assert(MB == 1 || (MB == 2 && GW * STEPS <= 4) || (MB == 4 && GW * STEPS <= 2), "16 VGPRs per group and block of rows");
         constexpr int GA = GW * STEPS;         // groups of a wavefront
         constexpr int SLICE = GW * 64;         // a wavefront's bytes of a weight row per step
         constexpr int TILE_BYTES = 16 * SLICE; // = GW KiB: GW wavefront-wide loads
@@ -528,7 +529,11 @@ namespace nnf
             if (M <= 16)
                 return launch_mrows_any_mb<GW, STEPS, 1>(stream, A, Wq, S, Y, M, N, K, zp, num_cu, partial, ranges, range_groups);
             if constexpr (GW * STEPS <= 4)
-                return launch_mrows_any_mb<GW, STEPS, 2>(stream, A, Wq, S, Y, M, N, K, zp, num_cu, partial, ranges, range_groups);
+                if (M <= 32)
+                    return launch_mrows_any_mb<GW, STEPS, 2>(stream, A, Wq, S, Y, M, N, K, zp, num_cu, partial, ranges, range_groups);
+            if constexpr (GW * STEPS <= 2)
+                if (M <= 64)
+                    return launch_mrows_any_mb<GW, STEPS, 4>(stream, A, Wq, S, Y, M, N, K, zp, num_cu, partial, ranges, range_groups);
             return hipErrorInvalidValue;
         }
     } // namespace
@@ -577,6 +582,7 @@ namespace nnf
             return hipErrorInvalidValue;
         switch (sp.gw)
         {
+        case 1: return launch_mrows_any<1, 2>(stream, A, Wq, S, nullptr, M, N, K, zp, num_cu, partial, sp.ranges, sp.range_groups);
         case 2: return launch_mrows_any<2, 2>(stream, A, Wq, S, nullptr, M, N, K, zp, num_cu, partial, sp.ranges, sp.range_groups);
         case 3: return launch_mrows_any<3, 2>(stream, A, Wq, S, nullptr, M, N, K, zp, num_cu, partial, sp.ranges, sp.range_groups);
         default: return launch_mrows_any<4, 2>(stream, A, Wq, S, nullptr, M, N, K, zp, num_cu, partial, sp.ranges, sp.range_groups);

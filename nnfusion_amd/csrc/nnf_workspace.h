@@ -397,7 +397,7 @@ namespace nnf
         }
         inline size_t w4a16_mrows_lds_bytes_gw(int gw, int M, int tiles)
         {
-            return (size_t)8 * 2 * gw * 1024 + 8 * 512 + (size_t)2 * 8 * (M <= 16 ? 1 : 2) * 1024 + (size_t)tiles * M * 64;
+            return (size_t)8 * 2 * gw * 1024 + 8 * 512 + (size_t)2 * 8 * (M <= 16 ? 1 : M <= 32 ? 2 : 4) * 1024 + (size_t)tiles * M * 64;
         }
         inline size_t w4a16_mrows_lds_bytes(int K, int M, int tiles)
         {
@@ -413,7 +413,7 @@ namespace nnf
             const int grid = n_tiles < num_cu ? n_tiles : num_cu;
             return w4a16_mrows_lds_bytes(K, M, (n_tiles + grid - 1) / grid) <= LDS_BYTES_PER_CU;
         }
-        // K above 8192 (above 4096 for 17 .. 32 rows; a multiple of 256): the run-time-K form over equal ranges of K (in whole pairs of
+        // K above 8192 (above 4096 for 17 .. 32 rows, above 2048 for 33 .. 64; a multiple of 256): the run-time-K form over equal ranges of K (in whole pairs of
         // groups; the last range may be shorter), each on its share of the CUs; fp32 sums per range, added by the
         // reduction pass.  Every workgroup fetches the activations of its range, so shorter ranges mean less of that
         // traffic (CUs x M x K / ranges x 2 bytes): ranges of at most 32 groups (GW = 2) measured fastest (K = 11008:
@@ -431,14 +431,20 @@ namespace nnf
         inline MrowsSplit w4a16_mrows_split(int M, int N, int K, int num_cu)
         {
             MrowsSplit sp;
-            if (M < 2 || M > 32 || N < 16 || K <= (M <= 16 ? 8192 : 4096) || K > 65536 || (K & 255) || num_cu < 16)
+            // (the kernel takes up to 64 rows; from about 48 on the tile GEMM is as fast or faster: 33 / 48 / 64 rows take
+            // 26.8 / 30.1 / 33.4 us against 32.3 / 32.8 / 33.8 at N = 22016, K = 4096, and 21.0 / 23.3 / 25.8 against 22.1 / 22.5 / 23.7 at
+            // N = 4096, K = 11008)
+            if (M < 2 || M > 40 || N < 16 || K <= (M <= 16 ? 8192 : M <= 32 ? 4096 : 2048) || K > 65536 || (K & 255) || num_cu < 16)
                 return sp;
             const int G = K >> 7;
-            int ranges = (G + 31) / 32;
+            // 33 .. 64 rows: four blocks of rows leave registers for two groups per wavefront: ranges of 16 groups
+            int ranges = M <= 32 ? (G + 31) / 32 : (G + 15) / 16;
             if (mrows_forced_ranges() >= 2)
                 ranges = mrows_forced_ranges();
             const int rg = (((G + ranges - 1) / ranges) + 1) & ~1;
-            const int gw = rg <= 32 ? 2 : rg <= 48 ? 3 : 4;
+            const int gw = rg <= 16 ? (M <= 32 ? 2 : 1) : rg <= 32 ? 2 : rg <= 48 ? 3 : 4;
+            if ((M > 32 && gw > 1) || (M > 16 && gw > 2)) // (only with a forced number of ranges)
+                return sp;
             if (G - (ranges - 1) * rg < gw) // the last range holds at least one wavefront's groups
                 return sp;
             const int n_tiles = (N + 15) / 16, per_range = num_cu / ranges;
