@@ -431,10 +431,11 @@ namespace nnf
         inline MrowsSplit w4a16_mrows_split(int M, int N, int K, int num_cu)
         {
             MrowsSplit sp;
-            // (the kernel takes up to 64 rows; from about 48 on the tile GEMM is as fast or faster: 33 / 48 / 64 rows take
-            // 26.8 / 30.1 / 33.4 us against 32.3 / 32.8 / 33.8 at N = 22016, K = 4096, and 21.0 / 23.3 / 25.8 against 22.1 / 22.5 / 23.7 at
-            // N = 4096, K = 11008)
-            if (M < 2 || M > 40 || N < 16 || K <= (M <= 16 ? 8192 : M <= 32 ? 4096 : 2048) || K > 65536 || (K & 255) || num_cu < 16)
+            // (33 .. 64 rows run on the kernel, but against the tile GEMM, measured alternately: 33 / 40 rows take 25.9 / 27.4 us
+            // against 29.1 / 29.3 at N = 22016, K = 4096 and 12.2 / 12.9 against 14.8 / 15.3 at N = K = 4096, are level at K = 8192 and
+            // 11008, 8-10 % slower at K = 5120, and slower everywhere from about 48 rows on: taken up to 40 rows and K = 4096)
+            if (M < 2 || M > 40 || N < 16 || K <= (M <= 16 ? 8192 : M <= 32 ? 4096 : 2048) || K > (M <= 32 ? 65536 : 4096) || (K & 255) ||
+                num_cu < 16)
                 return sp;
             const int G = K >> 7;
             // 33 .. 64 rows: four blocks of rows leave registers for two groups per wavefront: ranges of 16 groups

@@ -67,8 +67,8 @@ def _check(y, ref):
     (16, 4111, 11008), (8, 1000, 14336), (16, 300, 28672), (7, 4096, 11008), (12, 333, 8448), (6, 16, 16384),
     # 17 .. 32 rows over ranges of K (K above 4096), and in one launch with a run-time K
     (32, 4111, 8192), (17, 1000, 11008), (24, 300, 14336), (32, 520, 5120), (20, 77, 3584), (31, 2000, 2560),
-    # 33 .. 40 rows over ranges of K (four blocks of 16)
-    (33, 4111, 4096), (40, 1000, 8192), (36, 300, 11008), (40, 77, 2560), (38, 22016, 4096),
+    # 33 .. 40 rows over ranges of K (four blocks of 16; 2048 < K <= 4096)
+    (33, 4111, 4096), (40, 1000, 3072), (36, 300, 3584), (40, 77, 2560), (38, 22016, 4096),
     # 17 .. 32 rows (two blocks of 16), K <= 4096
     (17, 4096, 4096), (32, 22016, 4096), (24, 1000, 2048), (31, 77, 3072), (32, 300, 1024),
 ])
