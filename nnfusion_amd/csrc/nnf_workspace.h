@@ -464,14 +464,19 @@ namespace nnf
         }
         // Where the library picks it by itself, from measurements against the split-K MFMA GEMV on cold weights
         // (M = 2 / 16): K = 2048, 4096, 6144, 8192: 0-15 % / 15-30 % faster;  K = 1024, 3072: 5-35 % faster;
-        // run-time K: 3-10 % / 15-35 % faster at K = 3584, 5120, 7168 (one case 10 % slower: N = K = 7168, M = 2), level
+        // run-time K: 0-5 % / 15-35 % faster at K = 3584, 5120, 7168 (but up to 19 % slower below eight rows at K = 7168), level
         // at K = 2560, slower at K = 1536 and 2304, where most of what the wavefronts fetch is discarded: taken when at
         // least three quarters of the fetched groups count.
         inline bool w4a16_mrows_preferred(int M, int N, int K, int num_cu)
         {
             if (!w4a16_mrows_fits(M, N, K, num_cu))
                 return false;
-            return w4a16_mrows_fixed_k(M, K) || 4 * (K >> 7) >= 3 * 16 * w4a16_mrows_step_groups(M, K);
+            if (w4a16_mrows_fixed_k(M, K))
+                return true;
+            const int gw = w4a16_mrows_step_groups(M, K);
+            if (gw == 4 && M < 8) // K = 6400 .. 7936: N = K = 7168 takes 10.7 us at M = 2 against 9.0 (level from M = 6 on)
+                return false;
+            return 4 * (K >> 7) >= 3 * 16 * gw;
         }
         inline bool w4a16_variant_fits(int M, int N, int K, int variant, int num_cu)
         {
