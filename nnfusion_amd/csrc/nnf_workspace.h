@@ -366,13 +366,15 @@ namespace nnf
             const int grid = n_tiles < num_cu ? n_tiles : num_cu;
             return w8a8_mrows_lds_bytes(M, W8A8_MROWS_SLOTS, (n_tiles + grid - 1) / grid) <= LDS_BYTES_PER_CU;
         }
-        // Where the library picks it by itself: everywhere it applies.  Measured on cold weights against the split-K
-        // M <= 16 kernel it is level to 10 % faster up to M = 14 (2 % slower at M = 2, N = K = 8192), 5-30 % faster at
-        // M = 16, and 12-33 % faster than the MFMA tile GEMM at M = 17 .. 32.
+        // Where the library picks it by itself.  Measured alternately on cold weights against the split-K M <= 16 kernel
+        // it is level to 10 % faster up to M = 14 (6 % slower at M = 2, N = K = 8192: not taken below eight rows there),
+        // 5-30 % faster at M = 16, and 4-38 % faster than the MFMA tile GEMM at M = 17 .. 32.
         // (Where K does not fill the last step, wavefronts fetch bytes that do not count: at least three quarters of what
         // is fetched must count.)
         inline bool w8a8_mrows_preferred(int M, int N, int K, int num_cu)
         {
+            if (((K + 2047) >> 11) == 4 && M < 8) // N = K = 8192: 16.2 us at M = 2 against 15.3 (level from M = 8 on)
+                return false;
             return w8a8_mrows_fits(M, N, K, num_cu) && 4 * K >= 3 * 2048 * ((K + 2047) >> 11);
         }
         // ---- 2 .. 16 activation rows (.. 32 up to K = 4096): the row-streaming MFMA kernel (w4a16_mrows.hip) ----
