@@ -350,7 +350,7 @@ def run_extra(torch, np, dev, lib, datagen, ops):
         return torch.from_numpy(np.ascontiguousarray(a)).to(dev)
 
     def time_us(fn, iters):
-        for _ in range(3):
+        for _ in range(10):
             fn()
         torch.cuda.synchronize()
         e0 = torch.cuda.Event(enable_timing=True)
@@ -372,16 +372,18 @@ def run_extra(torch, np, dev, lib, datagen, ops):
         with torch.cuda.graph(g):
             for f in fns:
                 f()
-        g.replay()
+        # untimed replays first: after the host-side preparation of a row the first replays run 5-13 % slow
+        for _ in range(6):
+            g.replay()
         torch.cuda.synchronize()
         e0 = torch.cuda.Event(enable_timing=True)
         e1 = torch.cuda.Event(enable_timing=True)
         e0.record()
-        for _ in range(4):
+        for _ in range(6):
             g.replay()
         e1.record()
         torch.cuda.synchronize()
-        return e0.elapsed_time(e1) * 1000.0 / (4 * len(fns))
+        return e0.elapsed_time(e1) * 1000.0 / (6 * len(fns))
 
     def copies_of(*tensors):
         nbytes = sum(t.numel() * t.element_size() for t in tensors)
