@@ -128,9 +128,10 @@ def test_gemm_one_hot_rows_select_weights(gpu):
     np.testing.assert_array_equal(y, wd.T.astype(np.float16))
 
 
-@pytest.mark.parametrize("m,n,k", [(128, 8192, 8192), (1024, 8192, 8192), (4096, 8192, 8192)])
+@pytest.mark.parametrize("m,n,k", [(16, 8192, 8192), (128, 8192, 8192), (1024, 8192, 8192), (4096, 8192, 8192),
+                                   (32, 8192, 8192), (16, 22016, 4096), (16, 4096, 11008)])
 def test_gemm_full_size_sampled_columns(gpu, m, n, k):
-    """configs[2] shapes: all M rows, 192 sampled output columns against the oracle; and linearity in A
+    """configs[2] shapes (and batched-decode shapes on the row-streaming kernels: one launch, over ranges of K): all M rows, 192 sampled output columns against the oracle; and linearity in A
     on the whole output (Y(2A) == 2 Y(A) bit for bit, as scaling by 2 is exact outside the subnormal range)."""
     import torch
 
@@ -140,15 +141,20 @@ def test_gemm_full_size_sampled_columns(gpu, m, n, k):
     a, wq, s = datagen.w4a16_case(0, m, n, k)
     ta, tw, ts = _t(gpu, a, wq, s)
     y = ops.w4a16_gemm(ta, tw, ts)
-    y2 = ops.w4a16_gemm(ta * 2, tw, ts)
     torch.cuda.synchronize()
     rng = np.random.default_rng(0)
     cols = np.sort(rng.choice(n, 192, replace=False))
     ref = oracle.w4a16_gemm(a, wq[cols], s[cols], f32_out=True)
     _check(y.cpu().numpy()[:, cols], ref)
-    # scaling by two is exact everywhere except where the fp16 result is subnormal
-    normal = y.abs() >= 2.0 ** -13
-    assert torch.equal(y2[normal], (y * 2)[normal])
+    # Scaling by two is exact everywhere except where an fp16 value is subnormal: the result itself, and, in the
+    # kernels for a few rows (which carry the 1/16 of the high nibbles on the activations), an activation below
+    # 2^-10; those activations are set to zero for this check.
+    ta_lin = torch.where(ta.abs() < 2.0 ** -9, torch.zeros_like(ta), ta) if m <= 40 else ta
+    y1 = ops.w4a16_gemm(ta_lin, tw, ts)
+    y2 = ops.w4a16_gemm(ta_lin * 2, tw, ts)
+    torch.cuda.synchronize()
+    normal = y1.abs() >= 2.0 ** -13
+    assert torch.equal(y2[normal], (y1 * 2)[normal])
 
 
 def test_fused_bias_residual(gpu, plan):
