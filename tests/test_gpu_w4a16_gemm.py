@@ -147,7 +147,7 @@ def test_gemm_full_size_sampled_columns(gpu, m, n, k):
     ref = oracle.w4a16_gemm(a, wq[cols], s[cols], f32_out=True)
     _check(y.cpu().numpy()[:, cols], ref)
     # Scaling by two is exact everywhere except where an fp16 value is subnormal: the result itself, and, in the
-    # kernels for a few rows (which carry the 1/16 of the high nibbles on the activations), an activation below
+    # GEMV kernels for a few rows (which carry the 1/16 of the high nibbles on the activations), an activation below
     # 2^-10; those activations are set to zero for this check.
     ta_lin = torch.where(ta.abs() < 2.0 ** -9, torch.zeros_like(ta), ta) if m <= 40 else ta
     y1 = ops.w4a16_gemm(ta_lin, tw, ts)
