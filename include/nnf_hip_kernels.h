@@ -49,7 +49,8 @@ enum nnf_status
     NNF_ERR_INVALID_ARGUMENT = -1, /* null pointer, non-positive size, misaligned pointer */
     NNF_ERR_UNSUPPORTED_SHAPE = -2, /* K % group != 0, group != 128, K % 32 != 0, zp outside 0..15 ... */
     NNF_ERR_WORKSPACE_TOO_SMALL = -3,
-    NNF_ERR_NO_DEVICE = -4 /* no gfx950 device is current */
+    NNF_ERR_NO_DEVICE = -4, /* no gfx950 device is current */
+    NNF_ERR_STATIC_SCRATCH_LIMIT = -5 /* nnf_w4a16_gemm_static_scratch: the shape needs more than NNF_STATIC_SCRATCH_BYTES */
 };
 
 /* ABI version of this header (bumped on any signature change). */
@@ -70,6 +71,20 @@ int nnf_w4a16_gemm(nnf_stream_t stream,
                    const void* A, const void* Wq, const void* scales, void* Y,
                    int M, int N, int K, int group, int zp,
                    void* workspace, size_t workspace_bytes);
+
+/* nnf_w4a16_gemm for callers that can neither allocate nor pass a workspace (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same kernels and
+ * results as nnf_w4a16_gemm; the partial sums of a GEMM whose K range is split go to a buffer of
+ * NNF_STATIC_SCRATCH_BYTES that the library holds in device memory (a static __device__ array: each GPU the
+ * library is used on keeps its own copy until the process ends).  Calls no hipMalloc / hipFree.  A shape whose
+ * nnf_w4a16_gemm_workspace_bytes exceeds the buffer is rejected with NNF_ERR_STATIC_SCRATCH_LIMIT.  All calls
+ * on one GPU share the buffer: calls that overlap on one GPU (different streams) race; calls on one stream
+ * are ordered and safe.  The first call of any entry point on a device looks the buffer's address up
+ * (hipGetSymbolAddress): make that call outside stream capture. */
+#define NNF_STATIC_SCRATCH_BYTES ((size_t)32 << 20)
+int nnf_w4a16_gemm_static_scratch(nnf_stream_t stream,
+                                  const void* A, const void* Wq, const void* scales, void* Y,
+                                  int M, int N, int K, int group, int zp);
 
 /* The kernels behind nnf_w4a16_gemm as separate, selectable variants: what several registered emitters
  * for one operator are to ProfilingBasedKernelSelector::profiling_best

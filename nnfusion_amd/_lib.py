@@ -34,6 +34,7 @@ KERNEL_ABI = {
     "nnf_status_string": (ctypes.c_char_p, [_c_int]),
     "nnf_w4a16_gemm_workspace_bytes": (_c_sz, [_c_int] * 4),
     "nnf_w4a16_gemm": (_c_int, [_c_vp] * 5 + [_c_int] * 5 + [_c_vp, _c_sz]),
+    "nnf_w4a16_gemm_static_scratch": (_c_int, [_c_vp] * 5 + [_c_int] * 5),
     "nnf_w4a16_variant_supported": (_c_int, [_c_int] * 5),
     "nnf_w4a16_gemm_variant_workspace_bytes": (_c_sz, [_c_int] * 5),
     "nnf_w4a16_gemm_variant": (_c_int, [_c_vp] * 5 + [_c_int] * 6 + [_c_vp, _c_sz]),

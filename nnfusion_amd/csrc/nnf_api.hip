@@ -12,9 +12,16 @@ namespace
     {
         int valid = 0;
         int num_cu = 0;
+        void* static_scratch = nullptr; // this device's copy of `scratch` below
     };
 
-    // Lazily cached properties of each device (the only global state of the library).
+    // Scratch memory owned by the library, for nnf_w4a16_gemm_static_scratch (callers that cannot allocate).
+    // Every device the library runs on holds its own copy, at its own address, until the process ends.  In host
+    // code the array's name is only a handle: the device address comes from hipGetSymbolAddress, once per device.
+    constexpr size_t STATIC_SCRATCH_BYTES = NNF_STATIC_SCRATCH_BYTES;
+    static __device__ __align__(256) unsigned char scratch[STATIC_SCRATCH_BYTES];
+
+    // Lazily cached properties of each device (with `scratch`, the only global state of the library).
     DeviceInfo g_dev[64];
 
     int current_device_info(DeviceInfo& out)
@@ -30,6 +37,12 @@ namespace
             if (e != hipSuccess)
                 return (int)e;
             g_dev[dev].num_cu = prop.multiProcessorCount;
+            // device `dev` is current here: the address is that of its own copy
+            void* ptr = nullptr;
+            e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+            if (e != hipSuccess)
+                return (int)e;
+            g_dev[dev].static_scratch = ptr;
             g_dev[dev].valid = 1;
         }
         out = g_dev[dev];
@@ -92,6 +105,8 @@ const char* nnf_status_string(int status)
     case NNF_ERR_UNSUPPORTED_SHAPE: return "unsupported shape or quantisation parameters";
     case NNF_ERR_WORKSPACE_TOO_SMALL: return "workspace too small";
     case NNF_ERR_NO_DEVICE: return "no current HIP device";
+    case NNF_ERR_STATIC_SCRATCH_LIMIT:
+        return "shape needs more scratch memory than the library's static buffer holds (NNF_STATIC_SCRATCH_BYTES)";
     default: break;
     }
     if (status > 0)
@@ -152,6 +167,24 @@ int nnf_w4a16_gemm(nnf_stream_t stream, const void* A, const void* Wq, const voi
         return NNF_ERR_WORKSPACE_TOO_SMALL;
     return (int)nnf::launch_w4a16_gemm((hipStream_t)stream, A, Wq, scales, Y, M, N, K, zp, nullptr, 0.f, nullptr,
                                        nullptr, NNF_ACT_NONE, nullptr, workspace, dev.num_cu);
+}
+
+int nnf_w4a16_gemm_static_scratch(nnf_stream_t stream, const void* A, const void* Wq, const void* scales, void* Y,
+                                  int M, int N, int K, int group, int zp)
+{
+    int st = check_w4a16(A, Wq, scales, Y, M, N, K, group, zp);
+    if (st != NNF_OK)
+        return st;
+    // the partial sums of every path nnf_w4a16_gemm may take for this shape
+    if (nnf::workspace::w4a16_gemm(M, N, K, group) > STATIC_SCRATCH_BYTES)
+        return NNF_ERR_STATIC_SCRATCH_LIMIT;
+    DeviceInfo dev;
+    st = current_device_info(dev);
+    if (st != NNF_OK)
+        return st;
+    // Same kernels, with the device's static buffer in the place of the caller's workspace.  Nothing in it has to
+    // start at zero: every partial sum is written by the GEMM kernel before the reduction pass reads it.
+    return nnf_w4a16_gemm(stream, A, Wq, scales, Y, M, N, K, group, zp, dev.static_scratch, STATIC_SCRATCH_BYTES);
 }
 
 int nnf_w4a16_variant_supported(int M, int N, int K, int group, int variant)
