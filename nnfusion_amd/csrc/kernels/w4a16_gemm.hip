@@ -11,7 +11,7 @@
 //   * the tile shape and the number of K ranges follow nnf::workspace::plan_w4a16_gemm: 256 x 256 tiles
 //     when they fill the GPU, otherwise 128 x 128 or 64 x 256 tiles with K split across workgroups so
 //     that about two workgroups per CU are in flight.
-#include "w4a16_gemm_dl.h"
+#include "w4a16_gemm_sk_launch.h"
 
 #include "../nnf_workspace.h"
 
@@ -19,6 +19,19 @@
 
 namespace nnf
 {
+    // what the reduction pass behind the GEMV kernels that run over ranges of K needs to know
+    struct GemmParams
+    {
+        half_t* Y;
+        int M, N;               // N = output columns
+        int ldy;                // row stride of Y
+        const half_t* bias;     // BIAS: [N]
+        const half_t* residual; // RESID: [M, ldy]
+        float* partial;         // [splits][M][ld_partial] fp32
+        int splits;             // number of K ranges
+        int ld_partial;         // N, or 2 N with GATE (gate columns, then up columns)
+    };
+
     // one row per workgroup of four wavefronts: Xn[m, :] = fp16( x * rsqrt(mean_k(x^2) + eps) * gamma ).
     // The row is read once: a thread keeps its 16-byte units in registers between the two passes (up to K = 16384;
     // the units beyond that are read again).
@@ -84,6 +97,37 @@ namespace nnf
         }
         for (int i = tid + KEEP * 256; i < units; i += 256)
             out[i] = norm(row[i], grow[i]);
+    }
+
+    // RMSNorm for the tile GEMM, which never materialises the normalised activations: only
+    // rstd[m] = rsqrt(mean_k(x[m,k]^2) + eps) is computed here (one workgroup of four wavefronts per row; same
+    // summation order as rms_norm_kernel); gamma joins the weights inside the GEMM.
+    __global__ __launch_bounds__(256) void rms_rstd_kernel(const half_t* __restrict__ X, float* __restrict__ rstd, int M, int K,
+                                                           float eps)
+    {
+        __shared__ float part[4];
+        const int tid = threadIdx.x;
+        const int m = blockIdx.x;
+        const int units = K >> 3;
+        const uintx4* row = reinterpret_cast<const uintx4*>(X + (size_t)m * K);
+        float ss = 0.f;
+        for (int i = tid; i < units; i += 256)
+        {
+            const uintx4 v = row[i];
+            const uint32_t vv[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+            {
+                const half2_t hh = as_half2(vv[j]);
+                ss += (float)hh.x * (float)hh.x + (float)hh.y * (float)hh.y;
+            }
+        }
+        ss = wave_sum(ss);
+        if ((tid & 63) == 0)
+            part[tid >> 6] = ss;
+        __syncthreads();
+        if (tid == 0)
+            rstd[m] = 1.0f / __builtin_sqrtf(((part[0] + part[1]) + (part[2] + part[3])) / (float)K + eps);
     }
 
     // Y[m, n] = epilogue( sum_s partial[s][m][n] ); four consecutive columns per thread.
@@ -214,26 +258,6 @@ namespace nnf
                 return launch_reduce<false, false, true>(stream, p);
             return launch_reduce<false, false, false>(stream, p);
         }
-
-        // 256 x 256 tiles: wavefronts 2 (M) x 4 (N), each 4 x 2 MFMA tiles; one workgroup per CU
-        hipError_t launch_gemm_big(hipStream_t stream, const GemmParams& p, bool gate, bool hb, bool hr)
-        {
-            if (p.partial)
-            {
-                if (gate)
-                    return launch_gemm_dl<2, 4, 4, 2, true, false, false, true, 2>(stream, p);
-                return launch_gemm_dl<2, 4, 4, 2, false, false, false, true, 2>(stream, p);
-            }
-            if (gate)
-                return launch_gemm_dl<2, 4, 4, 2, true, false, false, false, 2>(stream, p);
-            if (hb && hr)
-                return launch_gemm_dl<2, 4, 4, 2, false, true, true, false, 2>(stream, p);
-            if (hb)
-                return launch_gemm_dl<2, 4, 4, 2, false, true, false, false, 2>(stream, p);
-            if (hr)
-                return launch_gemm_dl<2, 4, 4, 2, false, false, true, false, 2>(stream, p);
-            return launch_gemm_dl<2, 4, 4, 2, false, false, false, false, 2>(stream, p);
-        }
     } // namespace
 
     hipError_t launch_w4a16_gemm(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M,
@@ -246,8 +270,24 @@ namespace nnf
         // the combinations the fused entry points use; anything else is composed by the caller
         if (gate && (hb || hr))
             return hipErrorInvalidValue;
-        if (rms)
+        // which kernel serves the (gate: 2N) weight rows
+        const int n_rows = gate ? 2 * N : N;
+        const bool rows = !gemm_only && (g_tuning.force_path == 0 || g_tuning.force_path == 4) &&
+                          w4a16_gemv_rows_supported(M, n_rows, K, num_cu);
+        const bool mrows = !gemm_only && ((g_tuning.force_path == 5 && w4a16_mrows_supported(M, n_rows, K, num_cu)) ||
+                                          (g_tuning.force_path == 0 && w4a16_mrows_preferred(M, n_rows, K, num_cu)));
+        const bool one_launch_gemv = !gemm_only && (rows || mrows || (M <= 16 && w4a16_skinny_supported(M, n_rows, K)));
+        const int mr_splits = (!gemm_only && partial_ws && (g_tuning.force_path == 0 || g_tuning.force_path == 5))
+                                  ? w4a16_mrows_ksplits(M, n_rows, K, num_cu)
+                                  : 0;
+        const int ksplits = mr_splits ? mr_splits : (!gemm_only && partial_ws) ? w4a16_skinny_ksplits(M, n_rows, K) : 0;
+        // the products go to scratch first when the epilogue cannot work in place: the [M, 2N] gate | up pair, or a
+        // residual that is the output buffer itself
+        const bool via_scratch = gate || (hr && residual == Y);
+        const bool gemv_path = (one_launch_gemv && (!via_scratch || partial_ws)) || ksplits > 0;
+        if (rms && gemv_path)
         {
+            // the GEMV kernels read normalised activations (the tile GEMM folds the normalisation in: below)
             if (!rms_ws)
                 return hipErrorInvalidValue;
             hipLaunchKernelGGL(rms_norm_kernel, dim3(M), dim3(256), 0, stream, (const half_t*)A,
@@ -260,16 +300,7 @@ namespace nnf
         // M <= 16 (<= 32 where the row-streaming MFMA kernel applies): the bandwidth-bound GEMV kernel on the
         // (normalised) activations, then a small element-wise
         // kernel for whatever epilogue is asked for
-        const int n_rows = gate ? 2 * N : N;
-        // the products go to scratch first when the epilogue cannot work in place: the [M, 2N] gate | up pair, or a
-        // residual that is the output buffer itself
-        const bool via_scratch = gate || (hr && residual == Y);
-        // one activation row: the row-streaming kernel where it applies; a handful of rows: the row-streaming MFMA kernel
-        const bool rows = !gemm_only && (g_tuning.force_path == 0 || g_tuning.force_path == 4) &&
-                          w4a16_gemv_rows_supported(M, n_rows, K, num_cu);
-        const bool mrows = !gemm_only && ((g_tuning.force_path == 5 && w4a16_mrows_supported(M, n_rows, K, num_cu)) ||
-                                          (g_tuning.force_path == 0 && w4a16_mrows_preferred(M, n_rows, K, num_cu)));
-        if (!gemm_only && (rows || mrows || (M <= 16 && w4a16_skinny_supported(M, n_rows, K))) && (!via_scratch || partial_ws))
+        if (one_launch_gemv && (!via_scratch || partial_ws))
         {
             void* y_gemv = via_scratch ? partial_ws : Y;
             hipError_t e = rows ? launch_w4a16_gemv_rows(stream, A, Wq, S, y_gemv, n_rows, K, zp, num_cu)
@@ -289,10 +320,6 @@ namespace nnf
         // M <= 16 with too many activations for one workgroup's LDS: the GEMV kernel over ranges of K, then the
         // reduction pass (which applies the epilogue)
         // (K above 8192 in multiples of 256: the row-streaming MFMA kernel, otherwise the split-K one)
-        const int mr_splits = (!gemm_only && partial_ws && (g_tuning.force_path == 0 || g_tuning.force_path == 5))
-                                  ? w4a16_mrows_ksplits(M, n_rows, K, num_cu)
-                                  : 0;
-        const int ksplits = mr_splits ? mr_splits : (!gemm_only && partial_ws) ? w4a16_skinny_ksplits(M, n_rows, K) : 0;
         if (ksplits > 0)
         {
             hipError_t e = mr_splits
@@ -301,16 +328,10 @@ namespace nnf
             if (e != hipSuccess)
                 return e;
             GemmParams p;
-            p.A = nullptr;
-            p.Wq = nullptr;
-            p.S = nullptr;
             p.Y = (half_t*)Y;
             p.M = M;
             p.N = N;
-            p.K = K;
-            p.zp = zp;
             p.ldy = N;
-            p.up_row_offset = N;
             p.bias = (const half_t*)bias;
             p.residual = (const half_t*)residual;
             p.partial = (float*)partial_ws;
@@ -318,9 +339,16 @@ namespace nnf
             p.ld_partial = n_rows;
             return launch_reduce_any(stream, p, gate, hb, hr);
         }
-        const workspace::GemmPlan plan =
-            workspace::plan_w4a16_gemm(M, N, K, gate, g_tuning.gemm_tile - 1, g_tuning.gemm_splits);
-        GemmParams p;
+        // ---- the tile GEMM ------------------------------------------------------------------------------------
+        // forced tile of the experiments hook: 1 .. 4 = 256, 128, 64, 32 rows; forced K ranges = workgroups per tile
+        static const int forced_rows[5] = {0, 256, 128, 64, 32};
+        const int f_rows = forced_rows[g_tuning.gemm_tile >= 0 && g_tuning.gemm_tile <= 4 ? g_tuning.gemm_tile : 0];
+        const workspace::SkPlan plan = workspace::plan_w4a16_sk_with(M, N, K, gate, num_cu, f_rows, g_tuning.gemm_splits);
+        if (plan.slots > 0 && !partial_ws)
+            return hipErrorInvalidValue;
+        if ((size_t)M * K * 2 + 8192 >= ((size_t)1 << 32) || (size_t)n_rows * (K >> 1) >= ((size_t)1 << 32))
+            return hipErrorInvalidValue; // the kernel addresses its operands with 32-bit byte offsets
+        SkGemmParams p;
         p.A = (const half_t*)A;
         p.Wq = (const uint8_t*)Wq;
         p.S = (const half_t*)S;
@@ -333,21 +361,28 @@ namespace nnf
         p.up_row_offset = N; // gate rows [0,N), up rows [N,2N)
         p.bias = (const half_t*)bias;
         p.residual = (const half_t*)residual;
-        if (plan.reduce_pass && !partial_ws)
-            return hipErrorInvalidValue;
-        p.partial = plan.reduce_pass ? (float*)partial_ws : nullptr;
-        p.splits = plan.splits;
-        p.ld_partial = gate ? 2 * N : N;
-        hipError_t e;
-        switch (plan.tile)
+        p.gamma = rms ? (const half_t*)rms_gamma : nullptr;
+        p.rstd = rms ? (const float*)rms_ws : nullptr;
+        p.partial = plan.slots ? (float*)partial_ws : nullptr;
+        p.tiles_m = plan.tiles_m;
+        p.tiles_n = plan.tiles_n;
+        p.supersteps = plan.supersteps;
+        p.units = plan.units;
+        if (rms)
         {
-        case workspace::GEMM_TILE_BIG: e = launch_gemm_big(stream, p, gate, hb, hr); break;
-        case workspace::GEMM_TILE_MID: e = launch_gemm_mid(stream, p, gate, hb, hr); break;
-        case workspace::GEMM_TILE_SMALL: e = launch_gemm_small(stream, p, gate, hb, hr); break;
-        default: e = launch_gemm_tiny(stream, p, gate, hb, hr); break;
+            if (!rms_ws)
+                return hipErrorInvalidValue;
+            hipLaunchKernelGGL(rms_rstd_kernel, dim3(M), dim3(256), 0, stream, (const half_t*)A, (float*)rms_ws, M, K, rms_eps);
         }
-        if (e != hipSuccess || !plan.reduce_pass)
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess)
             return e;
-        return launch_reduce_any(stream, p, gate, hb, hr);
+        switch (plan.tile_rows)
+        {
+        case 256: return launch_gemm_sk_256(stream, p, plan.grid, gate);
+        case 128: return launch_gemm_sk_128(stream, p, plan.grid, gate);
+        case 64: return launch_gemm_sk_64(stream, p, plan.grid, gate);
+        default: return launch_gemm_sk_32(stream, p, plan.grid, gate);
+        }
     }
 } // namespace nnf

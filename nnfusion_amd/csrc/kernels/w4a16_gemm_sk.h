@@ -1,0 +1,836 @@
+// fp16 x int4 (g128) MFMA tile GEMM for gfx950: four wavefronts side by side along N, work split evenly
+// over the CUs.
+//
+//   Y[M,N] = epilogue( prologue(A)[M,K] . ((Wq - zp) * S)^T )
+//
+// Replaces the cublasSgemm/cublasHgemm call that the reference's cuda::Dot emits
+// (src/nnfusion/core/kernels/cuda_gpu/kernels/dot.cpp:128-205, 271-363) for a weight-quantized Dot
+// with transpose_B, plus the element-wise kernels around it (RMSNorm ahead of it, bias / residual /
+// SiLU(gate) * up behind it; fusion precedent: cuda_gpu/kernels/elementwise_fused.cpp:43-288,
+// matmuladd.cpp:29-93).
+//
+// Two things bound a quantized GEMM on this chip besides the matrix cores.  The chip is power managed:
+// every byte of fresh data moved next to an MFMA lowers the clock the MFMAs run at.  And with the
+// accumulators of a 256 x 256 tile in registers there is one wavefront per SIMD, whose vector, LDS and
+// memory instructions are issued between its own MFMAs and not under them.  The structure therefore
+// minimises traffic and instructions per MFMA:
+//   * One workgroup = four wavefronts (one per SIMD, up to 512 registers each) over a (TM*32) x (TN*128)
+//     tile, each wavefront owning all TM*32 rows of a strip of TN*32 columns (TM x TN MFMA tiles of
+//     32x32x16).  A weight belongs to exactly one wavefront: it is unpacked once per workgroup (16 VALU
+//     operations per 8 weights, feeding TM MFMAs each), not once per wavefront row.
+//   * The weights never touch LDS.  A lane owns one weight row of each of its column tiles and one half
+//     of every 64-wide K step; it fetches its bytes straight into registers, one "superstep" of 256 k
+//     (two quantization groups, four K steps) at a time: four 16-byte loads that together with the
+//     other half's cover whole 128-byte lines of the row (a load per K step would touch 32 bytes of
+//     each line and fetch the line four times: the 32 KiB first-level cache does not hold a line that
+//     long).  Two register sets: superstep s+1 is requested while s is multiplied.  The group scales
+//     travel the same way (two 2-byte loads per row and superstep).
+//   * The activations go global -> LDS asynchronously (global_load_lds_dwordx4, no register staging)
+//     into a ring of three stages of BK = 64; the loads for K step kt+3 are issued from the barrier of
+//     step kt on, a quarter of them per quarter step.
+//   * One barrier per K step, placed ahead of the step's LAST quarter: at that point every fragment of
+//     the step is in registers, so the stage can be refilled at once, and the first fragments of the
+//     next step are read while the last MFMAs of this one run.
+//   * The instruction stream is laid out in regions of a few MFMAs + their fragment reads + a share of
+//     the unpacking + at most a few loads, so that no queue (LDS, address unit) sees a burst.  Every load
+//     has a scalar base and a 32-bit lane offset that never changes, and the waits on the loads into LDS
+//     and on the fragment reads are counted by hand (the compiler's own would drain everything in flight).
+//   * The workgroups of a launch split the flat list of (tile, superstep) units evenly ("stream-K"): a
+//     launch has one workgroup per CU with the same amount of work, whatever the tile count.  A
+//     workgroup that covers only part of a tile's K range writes its fp32 sums to the workspace in
+//     register order (1 KiB per store instruction); a second, small launch adds the parts of such tiles
+//     in K order and runs their epilogue, on all CUs (one CU would need tens of microseconds to pull the
+//     parts of a tile through its own registers).  Tiles with a single owner are finished here.
+//   * Epilogues round the way the unfused graph would: the GEMM result to fp16 first, then the
+//     element-wise operation in fp32, then fp16 again.  RMSNorm is folded in without materialising the
+//     normalised activations: gamma[k] multiplies the weights as they are unpacked, rstd[m] (from a
+//     small pre-pass over A) multiplies the fp32 row sums.
+#pragma once
+
+#include "nnf_device.h"
+#include "nnf_launch.h"
+
+namespace nnf
+{
+    struct SkGemmParams
+    {
+        const half_t* A;
+        const uint8_t* Wq;
+        const half_t* S;
+        half_t* Y;
+        int M, N, K, zp;        // N = output columns
+        int ldy;                // row stride of Y
+        int up_row_offset;      // GATE: weight row of the up projection that pairs with gate row 0
+        const half_t* bias;     // BIAS: [N]
+        const half_t* residual; // RESID: [M, ldy]
+        const half_t* gamma;    // RMS: [K]
+        const float* rstd;      // RMS: [M]
+        float* partial;         // slots of BM x BN fp32: workgroup v's first segment at slot v, a later one at grid + v
+        int tiles_m, tiles_n;
+        int supersteps;         // per tile: ceil(K / 256)
+        long long units;        // tiles_m * tiles_n * supersteps
+    };
+
+    namespace gemm_sk
+    {
+        constexpr int BK = 64;
+        constexpr int WAVES = 4;
+        constexpr int THREADS = WAVES * 64;
+        constexpr int STAGES = 3;
+
+        template <int TM, int TN>
+        struct Tile
+        {
+            static constexpr int BM = TM * 32;
+            static constexpr int BN = WAVES * TN * 32; // weight rows per tile (GATE: half gate, half up rows)
+            static constexpr int A_TILE_BYTES = BM * BK * 2;
+            // per wavefront 256 bytes: (RMS) the step's 64 gamma values twice over
+            static constexpr int CONST_BYTES = WAVES * 256;
+            static constexpr int STAGE_BYTES = A_TILE_BYTES + CONST_BYTES;
+            // the epilogue turns the results through a private piece of the ring per wavefront
+            static constexpr int EPILOGUE_BYTES = WAVES * (TM >= 2 ? 2 : 1) * 32 * (TN * 64 + 16);
+            static constexpr int LDS_BYTES = STAGES * STAGE_BYTES > EPILOGUE_BYTES ? STAGES * STAGE_BYTES : EPILOGUE_BYTES;
+            static constexpr size_t SLOT_FLOATS = (size_t)BM * BN;
+        };
+
+        // s_waitcnt with only the vector-memory counter set (gfx9 encoding: vmcnt = bits 3:0 and 15:14)
+        constexpr int vmcnt_imm(int n) { return (n & 0xF) | ((n >> 4) << 14) | (0x7 << 4) | (0xF << 8); }
+
+        // `grid` workgroups split `units` units as [v * units / grid, (v + 1) * units / grid)
+        __host__ __device__ inline long long first_unit_of(int v, long long units, int grid)
+        {
+            return ((long long)v * units) / grid;
+        }
+        // the workgroup that owns unit x
+        __host__ __device__ inline int owner_of_unit(long long x, long long units, int grid)
+        {
+            return (int)(((x + 1) * grid - 1) / units);
+        }
+
+        // Which loads a wavefront issues where.  A K step has four quarters of TM x TN MFMAs; step kt is of type
+        // T = kt mod 4 (its place in the superstep).
+        //   * The TM activation loads (+ gamma with RMS) for step kt+3 go out in four positions: position 0 in
+        //     quarter 3 of step kt (right behind the barrier that frees the stage), positions 1 .. 3 in quarters
+        //     0 .. 2 of step kt+1.
+        //   * The six loads (four of weights, two scales) per column tile for the next superstep go out in quarters
+        //     0 .. 2 of step T = w_step(tile), ahead of that quarter's activation loads.
+        template <int TM, int TN, bool RMS>
+        struct Sched
+        {
+            static constexpr int a_pos(int i) { return (i * 4) / TM; }
+            static constexpr int a_loads_at(int pos)
+            {
+                int n = (RMS && pos == 0) ? 1 : 0;
+                for (int i = 0; i < TM; ++i)
+                    n += a_pos(i) == pos ? 1 : 0;
+                return n;
+            }
+            static constexpr int a_loads_total() { return TM + (RMS ? 1 : 0); }
+            // two tiles in the first step where there are four: everything has been asked for by the end of step 2
+            static constexpr int w_step(int j) { return TN <= 3 ? j : (j < 2 ? 0 : j - 1); }
+            static constexpr int w_loads_in_step(int T)
+            {
+                int n = 0;
+                for (int j = 0; j < TN; ++j)
+                    n += w_step(j) == T ? 6 : 0;
+                return n;
+            }
+            // the step's weight loads number [w_begin(T, Q), w_begin(T, Q + 1)) go out in quarter Q (0 .. 2)
+            static constexpr int w_begin(int T, int Q) { return Q * w_loads_in_step(T) / 3; }
+            // the x-th weight load of a step of type T: column tile and which of its six loads
+            static constexpr int w_tile(int T, int x)
+            {
+                int seen = 0;
+                for (int j = 0; j < TN; ++j)
+                    if (w_step(j) == T)
+                    {
+                        if (x < seen + 6)
+                            return j;
+                        seen += 6;
+                    }
+                return -1;
+            }
+            static constexpr int w_which(int x) { return x % 6; }
+            static constexpr int loads_at(int T, int Q)
+            {
+                return Q == 3 ? a_loads_at(0) : (w_begin(T, Q + 1) - w_begin(T, Q)) + a_loads_at(Q + 1);
+            }
+            // loads issued behind the last activation load for step kt+1 up to the wait that opens quarter 3 of step
+            // kt (vector-memory operations complete in order): what may still be outstanding there
+            static constexpr int later(int T)
+            {
+                const int Tp = (T + 3) & 3;
+                const int lp = a_pos(TM - 1); // 0: the last one went out in quarter 3 of step kt-2, p: in quarter p-1 of step kt-1
+                int n = 0;
+                for (int Q = lp; Q < 3; ++Q)
+                    n += loads_at(Tp, Q);
+                n += loads_at(Tp, 3);
+                for (int Q = 0; Q < 3; ++Q)
+                    n += loads_at(T, Q);
+                // the last step of a superstep also wants the next superstep's weights: everything but the
+                // activation loads issued since quarter 3 of step 2
+                if (T == 3 && n > a_loads_total())
+                    n = a_loads_total();
+                return n;
+            }
+        };
+
+
+        // Every load is one the compiler can see, so that its own wait insertion protects the registers they fill
+        // (also against copies its register allocator may place): global -> LDS through the builtin, weights and
+        // scales as ordinary loads.  Two things keep them cheap.  Scalar base addresses pass through an empty asm
+        // statement: the compiler then keeps them in scalar registers; lane offsets are redefined where they are
+        // used: the widening to 64 bits stays next to the load and is folded into it (scalar base + 32-bit lane
+        // offset), instead of being hoisted out of the loop as a register pair.  And the workgroup barrier is
+        // written as assembly: ahead of a barrier it knows, the compiler waits for every load in flight.
+        __device__ __forceinline__ const uint8_t* scalar_base(const uint8_t* ptr)
+        {
+            asm("" : "+s"(ptr));
+            return ptr;
+        }
+        __device__ __forceinline__ uint32_t here(uint32_t off)
+        {
+            asm volatile("" : "+v"(off));
+            return off;
+        }
+        typedef const void __attribute__((address_space(1))) * global_ptr;
+        typedef void __attribute__((address_space(3))) * lds_ptr;
+        __device__ __forceinline__ void workgroup_barrier()
+        {
+            asm volatile("s_barrier" ::: "memory");
+        }
+
+        // regions per quarter and fragments per region
+        constexpr int regions_of(int TM) { return TM < 4 ? TM : 4; }
+    } // namespace gemm_sk
+
+    // Epilogue of one round (ROUND_TM blocks of 32 rows) of a wavefront's strip of a tile.  Lane (m = l32, h) holds, in
+    // element e of MFMA tile (ii, j), column n = 8*(e/4) + 4*h + (e%4) of row ii*32 + m.  The sums are rounded (GATE:
+    // combined) in registers, turned through a private piece of LDS and finished as whole rows of the strip, 16 bytes
+    // (8 columns) per lane: bias, residual, store.  Rounding as the unfused graph would: the GEMM result to fp16 first,
+    // then the element-wise operation in fp32, then fp16 again.
+    template <int TM, int TN, bool GATE, bool BIAS, bool RESID, bool RMS>
+    __device__ __forceinline__ void sk_finish_round(const SkGemmParams& p, const floatx16 (&c)[TM >= 2 ? 2 : 1][TN], int r, int m0, int n0,
+                                                    uint8_t* staging, int wave, int lane)
+    {
+        constexpr int OUT_TN = GATE ? TN / 2 : TN;
+        constexpr int ROUND_TM = TM >= 2 ? 2 : 1;
+        constexpr int PITCH = OUT_TN * 64 + 16; // bytes per staged row (padding spreads the banks)
+        constexpr int REGION = ROUND_TM * 32 * PITCH;
+        constexpr int LANES_PER_ROW = OUT_TN * 4, ROWS_PER_READ = 64 / LANES_PER_ROW;
+        uint8_t* region = staging + wave * REGION;
+        const int l32 = lane & 31, h = lane >> 5;
+        const int n_wave = n0 + wave * (OUT_TN * 32);
+        const int piece = lane % LANES_PER_ROW;
+        const int n_lane = n_wave + piece * 8; // first of this lane's 8 columns in the row phase
+        bool vec = ((p.N & 7) == 0) && ((p.ldy & 7) == 0) && ((reinterpret_cast<uintptr_t>(p.Y) & 15) == 0);
+        if (RESID)
+            vec = vec && ((reinterpret_cast<uintptr_t>(p.residual) & 15) == 0);
+        float bias[8];
+        if (BIAS)
+        {
+#pragma unroll
+            for (int k = 0; k < 8; ++k)
+                bias[k] = (float)p.bias[min(n_lane + k, p.N - 1)];
+        }
+#pragma unroll
+        for (int ii = 0; ii < ROUND_TM; ++ii)
+        {
+            const int i = r * ROUND_TM + ii;
+            float rs = 1.0f;
+            if (RMS)
+                rs = p.rstd[min(m0 + i * 32 + l32, p.M - 1)];
+#pragma unroll
+            for (int j = 0; j < OUT_TN; ++j)
+#pragma unroll
+                for (int g = 0; g < 4; ++g)
+                {
+                    half4_t y;
+#pragma unroll
+                    for (int k = 0; k < 4; ++k)
+                    {
+                        if (GATE)
+                        {
+                            const float gt = (float)(half_t)(RMS ? c[ii][j][4 * g + k] * rs : c[ii][j][4 * g + k]);
+                            const float up =
+                                (float)(half_t)(RMS ? c[ii][j + TN / 2][4 * g + k] * rs : c[ii][j + TN / 2][4 * g + k]);
+                            y[k] = (half_t)(gt * (1.0f / (1.0f + __expf(-gt))) * up);
+                        }
+                        else
+                        {
+                            y[k] = (half_t)(RMS ? c[ii][j][4 * g + k] * rs : c[ii][j][4 * g + k]);
+                        }
+                    }
+                    *reinterpret_cast<half4_t*>(region + (ii * 32 + l32) * PITCH + (j * 32 + 8 * g + 4 * h) * 2) = y;
+                }
+        }
+        // LDS operations of one wavefront execute in order: no barrier around the private region
+#pragma unroll
+        for (int it = 0; it < ROUND_TM * 32 / ROWS_PER_READ; ++it)
+        {
+            const int row = it * ROWS_PER_READ + lane / LANES_PER_ROW;
+            half8_t o = *reinterpret_cast<const half8_t*>(region + row * PITCH + piece * 16);
+            const int m = m0 + r * (ROUND_TM * 32) + row;
+            if (m >= p.M || n_lane >= p.N)
+                continue;
+            const size_t at = (size_t)m * p.ldy + n_lane;
+            if (BIAS)
+            {
+#pragma unroll
+                for (int k = 0; k < 8; ++k)
+                    o[k] = (half_t)((float)o[k] + bias[k]);
+            }
+            if (RESID)
+            {
+                half8_t res;
+                if (vec)
+                    res = *reinterpret_cast<const half8_t*>(p.residual + at);
+                else
+                    for (int k = 0; k < 8; ++k)
+                        res[k] = p.residual[n_lane + k < p.N ? at + k : at];
+#pragma unroll
+                for (int k = 0; k < 8; ++k)
+                    o[k] = (half_t)((float)o[k] + (float)res[k]);
+            }
+            if (vec)
+                *reinterpret_cast<half8_t*>(p.Y + at) = o;
+            else
+                for (int k = 0; k < 8; ++k)
+                    if (n_lane + k < p.N)
+                        p.Y[at + k] = o[k];
+        }
+    }
+
+    template <int TM, int TN, bool GATE, bool BIAS, bool RESID, bool RMS>
+    __global__ __launch_bounds__(256, 1) void w4a16_gemm_sk_kernel(SkGemmParams p)
+    {
+        using namespace gemm_sk;
+        using T = Tile<TM, TN>;
+        using SCH = Sched<TM, TN, RMS>;
+        static_assert(!(GATE && (BIAS || RESID)), "SiLU-gate is not combined with bias or residual");
+        static_assert(TN == 2 || TN == 4, "column tiles per wavefront");
+        constexpr int BM = T::BM, BN = T::BN;
+        constexpr int A_TILE_BYTES = T::A_TILE_BYTES, STAGE_BYTES = T::STAGE_BYTES;
+        constexpr int BN_OUT = GATE ? BN / 2 : BN;
+        constexpr int NREG = regions_of(TM); // regions per quarter
+        constexpr int FPR = TM / NREG;       // activation fragments per region
+        extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+        // volatile: the vector move has to stay here, where every lane is active
+        uint32_t MASK, MAGIC, SEL[4];
+        asm volatile("v_mov_b32 %0, 0x54006400" : "=v"(MAGIC));
+        asm volatile("s_mov_b32 %0, 0x00F0000F" : "=s"(MASK));
+        asm volatile("s_mov_b32 %0, 0x0c000c00" : "=s"(SEL[0]));
+        asm volatile("s_mov_b32 %0, 0x0c010c01" : "=s"(SEL[1]));
+        asm volatile("s_mov_b32 %0, 0x0c020c02" : "=s"(SEL[2]));
+        asm volatile("s_mov_b32 %0, 0x0c030c03" : "=s"(SEL[3]));
+        const int tid = threadIdx.x;
+        const int lane = tid & 63;
+        const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+        const int l32 = lane & 31, h = lane >> 5;
+        const int K = p.K;
+        const int G = K >> 7;
+        const int SS = p.supersteps;
+        const int grid = (int)gridDim.x;
+        const uint32_t lds0 = lds_address(smem);
+
+        // workgroup ids are dealt round-robin to the 8 XCDs: number the workgroups so that an XCD (own L2) holds a
+        // contiguous run of them, i.e. of units, i.e. of tiles
+        int v;
+        {
+            const int pid = (int)blockIdx.x;
+            const int per_xcd = (grid + 7) >> 3;
+            const int full = grid - (per_xcd - 1) * 8;
+            const int xcd = pid & 7, idx = pid >> 3;
+            v = (xcd < full) ? xcd * per_xcd + idx : full * per_xcd + (xcd - full) * (per_xcd - 1) + idx;
+        }
+        const long long u_begin = first_unit_of(v, p.units, grid), u_end = first_unit_of(v + 1, p.units, grid);
+
+        // (q - zp) from (1024 + q_even, 64 + q_odd): exact
+        const half2_t dq_add = half2_t{(half_t)(-(1024.0f + (float)p.zp)), (half_t)(-(64.0f + (float)p.zp))};
+
+        // per-lane fragment addresses within a stage: row l32 of every 32-row block shares its swizzle
+        uint32_t a_rd[4]; // quarter s: piece (4h + s) ^ swizzle of row l32
+#pragma unroll
+        for (int s = 0; s < 4; ++s)
+            a_rd[s] = lds0 + (uint32_t)(l32 * 128 + ((((h << 2) + s) ^ ((l32 >> 1) & 7)) << 4));
+        // gamma of quarter s: the 8 values at k = 32h + 8s of the wavefront's private copy
+        const uint32_t g_rd = lds0 + (uint32_t)(A_TILE_BYTES + wave * 256 + h * 64);
+        // LDS destinations of this wavefront's loads within a stage
+        const uint32_t lds_a = (uint32_t)(wave * TM * 1024);
+        const uint32_t lds_g = (uint32_t)(A_TILE_BYTES + wave * 256);
+
+        for (long long u = u_begin; u < u_end;)
+        {
+            // ---- this segment: tile and range of supersteps ----------------------------------------------------
+            const int tile = (int)(u / SS);
+            const int ss_begin = (int)(u - (long long)tile * SS);
+            const int ss_end = (int)min((long long)SS, ss_begin + (u_end - u));
+            const int NSS = ss_end - ss_begin;
+            const bool whole = NSS == SS;
+            const bool first_of_mine = u == u_begin;
+            u += NSS;
+            int tm, tn;
+            {
+                // four tile rows advance together along N
+                constexpr int GM = 4;
+                const int per_group = GM * p.tiles_n;
+                const int g = tile / per_group;
+                const int first_m = g * GM;
+                const int gm = min(GM, p.tiles_m - first_m);
+                const int r = tile - g * per_group;
+                tm = first_m + r % gm;
+                tn = r / gm;
+            }
+            const int m0 = tm * BM, n0 = tn * BN_OUT;
+            const int k_begin = ss_begin * 256;
+            const int KT = 4 * NSS;                             // K steps of this segment (the last two may lie past K)
+            const int kt_max = min(KT, (K - k_begin) >> 6) - 1; // last K step inside K
+
+            // ---- activations: direct-load map ------------------------------------------------------------------
+            // chunk c fills LDS rows c*8 .. +7; lane l lands at (row = c*8 + l/8, slot = l%8) and therefore
+            // fetches piece  slot ^ ((row >> 1) & 7)  of that row.  Wavefront w fetches chunks w*TM .. +TM-1.
+            // (byte offsets from the operand's base: the matrices are below 4 GiB, checked by the launcher)
+            uint32_t a_off[TM];
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+            {
+                const int row = (wave * TM + i) * 8 + (lane >> 3);
+                const int piece = (lane & 7) ^ ((row >> 1) & 7);
+                a_off[i] = (uint32_t)(((size_t)min(m0 + row, p.M - 1) * K + k_begin + piece * 8) * 2);
+            }
+            const uint8_t* a_bytes = reinterpret_cast<const uint8_t*>(p.A);
+            const uint8_t* g_bytes = reinterpret_cast<const uint8_t*>(p.gamma) + (size_t)k_begin * 2;
+            const uint32_t g_off = (uint32_t)(lane & 31) * 4u;
+            // scalar base of K step kt (clamped to the last inside K: past it a valid tile goes to a free stage, or is
+            // multiplied by weights of zero)
+            auto a_base_of = [&](int kt) { return scalar_base(a_bytes + (size_t)min(kt, kt_max) * (BK * 2)); };
+            auto g_base_of = [&](int kt) { return scalar_base(g_bytes + (size_t)min(kt, kt_max) * (BK * 2)); };
+            // activation load i of a K step -> stage
+            auto load_a = [&](auto i_c, const uint8_t* a_base, uint32_t stage_off) {
+                constexpr int i = decltype(i_c)::value;
+                __builtin_amdgcn_global_load_lds((global_ptr)(a_base + here(a_off[i])), (lds_ptr)(smem + stage_off + lds_a + i * 1024), 16, 0, 0);
+            };
+            auto load_gamma = [&](const uint8_t* g_base, uint32_t stage_off) {
+                __builtin_amdgcn_global_load_lds((global_ptr)(g_base + here(g_off)), (lds_ptr)(smem + stage_off + lds_g), 4, 0, 0);
+            };
+
+            // ---- weights and scales: straight into registers -----------------------------------------------------
+            // lane (l32, h) owns weight row l32 of each of the wavefront's column tiles; of K step t of a
+            // superstep it owns k = 64 t + 32 h .. + 31: the 16 bytes at 32 t + 16 h of the superstep's 128
+            uint32_t w_off[TN], s_off[TN];
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+            {
+                int gn;
+                if (GATE) // column tiles 0 .. TN/2-1: gate rows, the others: the up rows that pair with them
+                    gn = min((j >= TN / 2 ? p.up_row_offset + n0 + (j - TN / 2) * 32 : n0 + j * 32) + wave * (TN / 2) * 32 + l32,
+                             p.up_row_offset + p.N - 1);
+                else
+                    gn = min(n0 + wave * (TN * 32) + j * 32 + l32, p.N - 1);
+                w_off[j] = (uint32_t)((size_t)gn * (K >> 1) + (k_begin >> 1) + h * 16);
+                s_off[j] = (uint32_t)(((size_t)gn * G + 2 * ss_begin) * 2);
+            }
+            const uint8_t* s_bytes = reinterpret_cast<const uint8_t*>(p.S);
+            uintx4 wbuf[2][TN][4];   // [register set][column tile][K step of the superstep]
+            uint32_t sraw[2][TN][2]; // the two group scales of the superstep, as loaded
+            half2_t sc[2][TN][2];    // ... as (s, s); zero for a group past K
+            // Scalar bases of superstep s of the segment (clamped to the last): weights of K steps 0 .. 1 and 2 .. 3,
+            // first and second scale.  K not a multiple of 256: the last superstep has one group; its second half
+            // repeats the first (and is multiplied by a scale of zero).
+            struct WBase
+            {
+                const uint8_t *w_lo, *w_hi, *s_lo, *s_hi;
+            };
+            auto w_base_of = [&](int s) {
+                s = min(s, NSS - 1);
+                const bool second_valid = 2 * (ss_begin + s) + 1 < G;
+                WBase b;
+                b.w_lo = scalar_base(p.Wq + (size_t)s * 128);
+                b.w_hi = scalar_base(p.Wq + (size_t)s * 128 + (second_valid ? 64 : 0));
+                b.s_lo = scalar_base(s_bytes + (size_t)s * 4);
+                b.s_hi = scalar_base(s_bytes + (size_t)s * 4 + (second_valid ? 2 : 0));
+                return b;
+            };
+            // load x (0 .. 3: weights of K step x, 4 .. 5: scales) of column tile j -> register set
+            auto load_w = [&](auto set_c, auto j_c, auto x_c, const WBase& b) {
+                constexpr int set = decltype(set_c)::value, j = decltype(j_c)::value, x = decltype(x_c)::value;
+                if constexpr (x < 4)
+                    wbuf[set][j][x] = *(const uintx4 __attribute__((address_space(1)))*)((x < 2 ? b.w_lo : b.w_hi) + (x & 1) * 32 + here(w_off[j]));
+                else
+                    sraw[set][j][x - 4] = *(const uint16_t __attribute__((address_space(1)))*)((x == 4 ? b.s_lo : b.s_hi) + here(s_off[j]));
+            };
+            // (s, s) of both groups of superstep s (as clamped by w_base_of)
+            auto prepare_scales = [&](auto set_c, int s) {
+                constexpr int set = decltype(set_c)::value;
+                s = min(s, NSS - 1);
+                const bool second_valid = 2 * (ss_begin + s) + 1 < G;
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                {
+                    sc[set][j][0] = as_half2(__builtin_amdgcn_perm(sraw[set][j][0], sraw[set][j][0], 0x01000100u));
+                    sc[set][j][1] = as_half2(second_valid ? __builtin_amdgcn_perm(sraw[set][j][1], sraw[set][j][1], 0x01000100u) : 0u);
+                }
+            };
+
+            floatx16 acc[TM][TN];
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e)
+                        acc[i][j][e] = 0.f;
+
+            half8_t af[2][TM];     // activation fragments: two sets, used by alternating quarters
+            uint32_t bw[2][TN][4]; // unpacked weight fragments, likewise
+            uintx4 gm[4];          // RMS: gamma of the four quarters of a K step
+            // Fragment reads the compiler does not track (it would wait for every LDS read in flight ahead of the first
+            // use of any): valid after the wait of the region that uses them.  LDS operations complete in order.
+            auto read_frag = [&](auto set_c, auto f_c, uint32_t addr) {
+                lds_read_b128_nowait<decltype(f_c)::value * 4096>(af[decltype(set_c)::value][decltype(f_c)::value], addr);
+            };
+            // one half2 of the unpacked operand: weights 2e, 2e+1 of word `w` -> (q - zp) * scale (* gamma)
+            auto unpack_piece = [&](auto set_c, auto j_c, auto e_c, uint32_t w, half2_t scale, const uintx4& gam) {
+                constexpr int set = decltype(set_c)::value, j = decltype(j_c)::value, e = decltype(e_c)::value;
+                const uint32_t x = __builtin_amdgcn_perm(w, w, SEL[e]); // bytes (b_e, 0, b_e, 0)
+                const half2_t y = as_half2((x & MASK) | MAGIC);         // (1024 + q_2e, 64 + q_2e+1)
+                half2_t z = (y + dq_add) * scale;                       // (q - zp) * scale: one rounding
+                if (RMS)
+                    z = z * as_half2(e == 0 ? gam.x : e == 1 ? gam.y : e == 2 ? gam.z : gam.w);
+                bw[set][j][e] = as_u32(z);
+            };
+
+            // ---- one K step --------------------------------------------------------------------------------------
+            // Quarter q multiplies the fragments of k16 block q (operand set q & 1) while the other set is filled for
+            // the next quarter.  Region r of a quarter: wait for its FPR fragments, ask for those of the next quarter,
+            // FPR x TN MFMAs, a share of the next quarter's unpacking; wavefront r's loads of the quarter.
+            //   t: K step within the superstep; s: superstep within the segment;
+            //   prev_off / stage_off / next_off: LDS offsets of the stages of steps kt-1, kt, kt+1
+            auto k_step = [&](auto t_c, int s, uint32_t prev_off, uint32_t stage_off, uint32_t next_off) {
+                constexpr int T_ = decltype(t_c)::value;
+                const int kt = 4 * s + T_;
+                // loads of this step: positions 1 .. 3 of the activations of step kt+2 (-> the stage of step kt-1),
+                // position 0 of step kt+3 (-> this step's stage), weights of superstep s+1
+                const uint8_t* a_late = a_base_of(kt + 2);
+                const uint8_t* a_next = a_base_of(kt + 3);
+                const uint8_t* g_next = RMS ? g_base_of(kt + 3) : nullptr;
+                const WBase w_next = w_base_of(s + 1);
+                unroll_for<0, 4>([&](auto q_c) {
+                    constexpr int Q = decltype(q_c)::value;
+                    constexpr int SET = Q & 1, OTHER = SET ^ 1;
+                    using OTHER_C = std::integral_constant<int, OTHER>;
+                    if constexpr (Q == 3)
+                    {
+                        // every fragment of this step is in registers; step kt+1 has landed for this wavefront once only
+                        // what it issued behind its loads is outstanding
+                        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                        __builtin_amdgcn_s_waitcnt(vmcnt_imm(SCH::later(T_)));
+                        workgroup_barrier();
+                        __builtin_amdgcn_sched_barrier(0);
+                        if constexpr (T_ == 3)
+                            prepare_scales(std::integral_constant<int, 1>{}, s + 1);
+                    }
+                    unroll_for<0, NREG>([&](auto r_c) {
+                        constexpr int R = decltype(r_c)::value;
+                        // the fragments of this region's MFMAs: behind the last of them, the reads of the regions after
+                        // this one a quarter ago and of the regions before this one in this quarter
+                        if constexpr (Q == 3)
+                        {
+                            unroll_for<0, FPR>([&](auto f_c) { lds_wait_also(af[SET][R * FPR + decltype(f_c)::value]); });
+                        }
+                        else
+                        {
+                            constexpr int DENSE = 2 * R < NREG ? 2 * R : NREG;
+                            constexpr int BEHIND = (NREG - 1 - R) * FPR + (Q == 2 ? DENSE : R) * FPR;
+                            lds_wait<BEHIND>(af[SET][R * FPR + FPR - 1]);
+                            unroll_for<0, FPR - 1>([&](auto f_c) { lds_wait_also(af[SET][R * FPR + decltype(f_c)::value]); });
+                        }
+                        // RMS: gamma of the next K step (landed with its stage), all four quarters: quarters 1 .. 3 of
+                        // this step's have been used up by the unpacking in quarters 0 .. 2, quarter 0's in the step before
+                        if constexpr (RMS && Q == 3 && R == 0)
+                            unroll_for<0, 4>([&](auto g_c) { lds_read_b128_nowait<decltype(g_c)::value * 16>(gm[decltype(g_c)::value], g_rd + next_off); });
+                        // fragments of the next quarter (quarter 3's: two regions' worth per region, so that they have
+                        // arrived at the barrier)
+                        if constexpr (Q == 0 || Q == 1)
+                            unroll_for<0, FPR>([&](auto f_c) {
+                                read_frag(OTHER_C{}, std::integral_constant<int, R * FPR + decltype(f_c)::value>{}, a_rd[Q + 1] + stage_off);
+                            });
+                        else if constexpr (Q == 2)
+                            unroll_for<0, 2 * FPR>([&](auto f_c) {
+                                constexpr int F = 2 * R * FPR + decltype(f_c)::value;
+                                if constexpr (F < TM)
+                                    read_frag(OTHER_C{}, std::integral_constant<int, F>{}, a_rd[3] + stage_off);
+                            });
+                        else
+                            unroll_for<0, FPR>([&](auto f_c) {
+                                read_frag(OTHER_C{}, std::integral_constant<int, R * FPR + decltype(f_c)::value>{}, a_rd[0] + next_off);
+                            });
+                        // the MFMAs: the weight fragment is the first operand: D[n][m], lane (m = l32, h) holds four
+                        // consecutive output columns per group of four elements, which is what the row-wise epilogue wants
+#pragma unroll
+                        for (int f = 0; f < FPR; ++f)
+#pragma unroll
+                            for (int j = 0; j < TN; ++j)
+                                acc[R * FPR + f][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+                                    __builtin_bit_cast(half8_t, uintx4{bw[SET][j][0], bw[SET][j][1], bw[SET][j][2], bw[SET][j][3]}),
+                                    af[SET][R * FPR + f], acc[R * FPR + f][j], 0, 0, 0);
+                        // this region's share of the unpacking for the next quarter: pieces (j, e).  (RMS, quarter 3: the
+                        // gamma values have just been asked for: the unpacking starts one region later.)
+                        constexpr int PIECES = 4 * TN;
+                        constexpr bool SHIFTED = RMS && Q == 3 && NREG > 1;
+                        constexpr int NR1 = NREG > 1 ? NREG - 1 : 1;
+                        constexpr int P0 = SHIFTED ? (R == 0 ? 0 : (R - 1) * PIECES / NR1) : R * PIECES / NREG;
+                        constexpr int P1 = SHIFTED ? (R == 0 ? 0 : R * PIECES / NR1) : (R + 1) * PIECES / NREG;
+                        if constexpr (RMS && Q == 3 && (NREG > 1 ? R == 1 : R == 0))
+                        {
+                            // behind the gamma reads: the fragment reads of the regions so far
+                            lds_wait<(NREG > 1 ? 2 * FPR : FPR)>(gm[0]);
+                            lds_wait_also(gm[1]);
+                            lds_wait_also(gm[2]);
+                            lds_wait_also(gm[3]);
+                        }
+                        unroll_for<P0, P1>([&](auto pc_c) {
+                            constexpr int pc = decltype(pc_c)::value;
+                            constexpr int j = pc / 4, e = pc % 4;
+                            // word Q+1 of this step, or word 0 of the next step
+                            constexpr int NT = Q == 3 ? (T_ + 1) & 3 : T_;
+                            constexpr int NSET = (Q == 3 && T_ == 3) ? 1 : 0;
+                            constexpr int NQ = (Q + 1) & 3;
+                            const uintx4& wq = wbuf[NSET][j][NT];
+                            const uint32_t w = NQ == 0 ? wq.x : NQ == 1 ? wq.y : NQ == 2 ? wq.z : wq.w;
+                            unpack_piece(OTHER_C{}, std::integral_constant<int, j>{}, std::integral_constant<int, e>{}, w,
+                                         sc[NSET][j][NT >> 1], gm[NQ]);
+                        });
+                        // this quarter's loads, spread over its regions
+                        constexpr int N_W = Q < 3 ? SCH::w_begin(T_, Q + 1) - SCH::w_begin(T_, Q) : 0;
+                        constexpr int N_A = SCH::a_loads_at(Q == 3 ? 0 : Q + 1) - ((RMS && Q == 3) ? 1 : 0);
+                        constexpr int N_L = N_W + N_A + ((RMS && Q == 3) ? 1 : 0);
+                        unroll_for<R * N_L / NREG, (R + 1) * N_L / NREG>([&](auto l_c) {
+                            constexpr int L = decltype(l_c)::value;
+                            if constexpr (L < N_W)
+                            {
+                                constexpr int X = SCH::w_begin(T_, Q) + L;
+                                load_w(std::integral_constant<int, 1>{}, std::integral_constant<int, SCH::w_tile(T_, X)>{},
+                                       std::integral_constant<int, SCH::w_which(X)>{}, w_next);
+                            }
+                            else if constexpr (L < N_W + N_A)
+                            {
+                                // the (L - N_W)-th activation load of this position
+                                constexpr int POS = Q == 3 ? 0 : Q + 1;
+                                constexpr int FIRST = (POS * TM + 3) / 4; // smallest i with a_pos(i) == POS
+                                static_assert(SCH::a_pos(FIRST + L - N_W) == POS, "activation loads of a position are consecutive");
+                                load_a(std::integral_constant<int, FIRST + L - N_W>{}, Q == 3 ? a_next : a_late, Q == 3 ? stage_off : prev_off);
+                            }
+                            else
+                                load_gamma(g_next, stage_off);
+                        });
+                        asm volatile("" ::: "memory");
+                        __builtin_amdgcn_sched_barrier(0);
+                    });
+                });
+                // the accumulators stay in the accumulation registers
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int j = 0; j < TN; ++j)
+                        asm volatile("" : "+a"(acc[i][j]));
+            };
+
+            // ---- K loop ---------------------------------------------------------------------------------------
+            using I0 = std::integral_constant<int, 0>;
+            using I1 = std::integral_constant<int, 1>;
+            using I2 = std::integral_constant<int, 2>;
+            using I3 = std::integral_constant<int, 3>;
+            {
+                // steps 0 and 1 and superstep 0 in full, of step 2 what quarter 3 of a step before the first would
+                // have asked for
+                const WBase w0 = w_base_of(0);
+                unroll_for<0, TM>([&](auto i_c) { load_a(i_c, a_base_of(0), 0u); });
+                unroll_for<0, TN>([&](auto j_c) { unroll_for<0, 6>([&](auto x_c) { load_w(I0{}, j_c, x_c, w0); }); });
+                if constexpr (RMS)
+                    load_gamma(g_base_of(0), 0u);
+                unroll_for<0, TM>([&](auto i_c) { load_a(i_c, a_base_of(1), (uint32_t)STAGE_BYTES); });
+                if constexpr (RMS)
+                    load_gamma(g_base_of(1), (uint32_t)STAGE_BYTES);
+                unroll_for<0, TM>([&](auto i_c) {
+                    if constexpr (SCH::a_pos(decltype(i_c)::value) == 0)
+                        load_a(i_c, a_base_of(2), (uint32_t)(2 * STAGE_BYTES));
+                });
+                if constexpr (RMS)
+                    load_gamma(g_base_of(2), (uint32_t)(2 * STAGE_BYTES));
+            }
+            __builtin_amdgcn_s_waitcnt(vmcnt_imm(SCH::a_loads_total() + SCH::a_loads_at(0))); // step 0 and superstep 0 have landed
+            workgroup_barrier();
+            __builtin_amdgcn_sched_barrier(0);
+            prepare_scales(I0{}, 0);
+            if constexpr (RMS)
+                unroll_for<0, 4>([&](auto g_c) { lds_read_b128_nowait<decltype(g_c)::value * 16>(gm[decltype(g_c)::value], g_rd); });
+            unroll_for<0, TM>([&](auto f_c) { read_frag(I0{}, f_c, a_rd[0]); });
+            if constexpr (RMS)
+            {
+                lds_wait<(TM < 15 ? TM : 15)>(gm[0]);
+                lds_wait_also(gm[1]);
+                lds_wait_also(gm[2]);
+                lds_wait_also(gm[3]);
+            }
+            unroll_for<0, 4 * TN>([&](auto pc_c) {
+                constexpr int pc = decltype(pc_c)::value;
+                unpack_piece(I0{}, std::integral_constant<int, pc / 4>{}, std::integral_constant<int, pc % 4>{}, wbuf[0][pc / 4][0].x,
+                             sc[0][pc / 4][0], gm[0]);
+            });
+            __builtin_amdgcn_sched_barrier(0);
+            // No LDS read other than the fragments of quarter 0 is in flight at the top of a K step.
+            {
+                constexpr uint32_t RING = (uint32_t)(STAGES * STAGE_BYTES);
+                auto next_of = [](uint32_t o) { return o + STAGE_BYTES == RING ? 0u : o + (uint32_t)STAGE_BYTES; };
+                uint32_t pv = RING - (uint32_t)STAGE_BYTES, st = 0;
+                // one loop body: the superstep works on register set 0 and fills set 1, which moves to set 0 at its end
+                // (a few dozen register moves per 256 MFMAs)
+                for (int s = 0; s < NSS; ++s)
+                {
+                    k_step(I0{}, s, pv, st, next_of(st));
+                    pv = st, st = next_of(st);
+                    k_step(I1{}, s, pv, st, next_of(st));
+                    pv = st, st = next_of(st);
+                    k_step(I2{}, s, pv, st, next_of(st));
+                    pv = st, st = next_of(st);
+                    k_step(I3{}, s, pv, st, next_of(st));
+                    pv = st, st = next_of(st);
+#pragma unroll
+                    for (int j = 0; j < TN; ++j)
+                    {
+#pragma unroll
+                        for (int x = 0; x < 4; ++x)
+                            wbuf[0][j][x] = wbuf[1][j][x];
+                        sc[0][j][0] = sc[1][j][0];
+                        sc[0][j][1] = sc[1][j][1];
+                    }
+                }
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); // the fragments read ahead for a step that does not exist
+            __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));          // nothing may land in LDS or in registers any more ...
+            __syncthreads();                                   // ... from any wavefront: the ring is free
+
+            // ---- a tile shared with other workgroups: park the sums in register order (element block q of MFMA tile
+            // (i, j) of all 256 threads is one contiguous 4 KiB); w4a16_gemm_sk_fixup_kernel adds the parts and finishes
+            if (!whole)
+            {
+                float* mine = p.partial + ((size_t)v + (first_of_mine ? 0 : (size_t)grid)) * T::SLOT_FLOATS + (size_t)tid * 4;
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int j = 0; j < TN; ++j)
+#pragma unroll
+                        for (int q = 0; q < 4; ++q)
+                        {
+                            *reinterpret_cast<floatx4*>(mine + (size_t)(((i * TN + j) * 4 + q) * THREADS * 4)) =
+                                floatx4{acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+                            __builtin_amdgcn_sched_barrier(0); // (one quarter of a tile at a time: few registers)
+                        }
+            }
+            else
+            {
+                // ---- epilogue: two blocks of 32 rows at a time ------------------------------------------------------
+                constexpr int ROUND_TM = TM >= 2 ? 2 : 1;
+#pragma unroll
+                for (int r = 0; r < TM / ROUND_TM; ++r)
+                {
+                    floatx16 c[ROUND_TM][TN];
+#pragma unroll
+                    for (int ii = 0; ii < ROUND_TM; ++ii)
+#pragma unroll
+                        for (int j = 0; j < TN; ++j)
+                            c[ii][j] = acc[r * ROUND_TM + ii][j];
+                    sk_finish_round<TM, TN, GATE, BIAS, RESID, RMS>(p, c, r, m0, n0, smem, wave, lane);
+                    __builtin_amdgcn_sched_barrier(0); // (one round at a time: few registers)
+                }
+            }
+            if (u < u_end)
+                __syncthreads(); // the staging regions are read before the next segment's tiles land in them
+        }
+    }
+
+    // Adds the parts of the tiles that several workgroups of w4a16_gemm_sk_kernel worked on, in K order (so the result
+    // does not depend on timing), and runs the epilogue.  One workgroup per tile and round of two 32-row blocks; a
+    // workgroup whose tile had a single owner has nothing to do.  `gemm_grid`: workgroups of the GEMM launch.
+    template <int TM, int TN, bool GATE, bool BIAS, bool RESID, bool RMS>
+    __global__ __launch_bounds__(256) void w4a16_gemm_sk_fixup_kernel(SkGemmParams p, int gemm_grid)
+    {
+        using namespace gemm_sk;
+        using T = Tile<TM, TN>;
+        constexpr int ROUND_TM = TM >= 2 ? 2 : 1;
+        constexpr int ROUNDS = TM / ROUND_TM;
+        constexpr int BN_OUT = GATE ? T::BN / 2 : T::BN;
+        __shared__ __attribute__((aligned(16))) uint8_t stage[WAVES * ROUND_TM * 32 * (TN * 64 + 16)];
+        const int tid = threadIdx.x, lane = tid & 63;
+        const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+        const int tile = (int)blockIdx.x / ROUNDS, r = (int)blockIdx.x % ROUNDS;
+        const int SS = p.supersteps;
+        const long long t0 = (long long)tile * SS;
+        const int v_first = owner_of_unit(t0, p.units, gemm_grid);
+        const int n_seg = owner_of_unit(t0 + SS - 1, p.units, gemm_grid) - v_first + 1;
+        if (n_seg == 1)
+            return;
+        // the first owner parked this tile in its second slot when its range began in an earlier tile
+        const bool first_is_second_slot = first_unit_of(v_first, p.units, gemm_grid) < t0;
+        int tm, tn;
+        {
+            constexpr int GM = 4;
+            const int per_group = GM * p.tiles_n;
+            const int g = tile / per_group;
+            const int first_m = g * GM;
+            const int gm = min(GM, p.tiles_m - first_m);
+            const int rr = tile - g * per_group;
+            tm = first_m + rr % gm;
+            tn = rr / gm;
+        }
+        const int m0 = tm * T::BM, n0 = tn * BN_OUT;
+        floatx16 c[ROUND_TM][TN];
+#pragma unroll
+        for (int ii = 0; ii < ROUND_TM; ++ii)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int e = 0; e < 16; ++e)
+                    c[ii][j][e] = 0.f;
+        // parts in K order, four at a time in flight
+        for (int sg0 = 0; sg0 < n_seg; sg0 += 4)
+        {
+            floatx4 x[4][ROUND_TM][TN][4];
+#pragma unroll
+            for (int d = 0; d < 4; ++d)
+            {
+                const int sg = min(sg0 + d, n_seg - 1);
+                const float* theirs = p.partial +
+                                      ((size_t)(v_first + sg) + ((sg == 0 && first_is_second_slot) ? (size_t)gemm_grid : 0)) * T::SLOT_FLOATS +
+                                      (size_t)tid * 4;
+#pragma unroll
+                for (int ii = 0; ii < ROUND_TM; ++ii)
+#pragma unroll
+                    for (int j = 0; j < TN; ++j)
+#pragma unroll
+                        for (int q = 0; q < 4; ++q)
+                            x[d][ii][j][q] =
+                                *reinterpret_cast<const floatx4*>(theirs + (size_t)((((r * ROUND_TM + ii) * TN + j) * 4 + q) * THREADS * 4));
+            }
+#pragma unroll
+            for (int d = 0; d < 4; ++d)
+                if (sg0 + d < n_seg)
+                {
+#pragma unroll
+                    for (int ii = 0; ii < ROUND_TM; ++ii)
+#pragma unroll
+                        for (int j = 0; j < TN; ++j)
+#pragma unroll
+                            for (int q = 0; q < 4; ++q)
+                            {
+                                c[ii][j][4 * q] += x[d][ii][j][q].x;
+                                c[ii][j][4 * q + 1] += x[d][ii][j][q].y;
+                                c[ii][j][4 * q + 2] += x[d][ii][j][q].z;
+                                c[ii][j][4 * q + 3] += x[d][ii][j][q].w;
+                            }
+                }
+        }
+        sk_finish_round<TM, TN, GATE, BIAS, RESID, RMS>(p, c, r, m0, n0, stage, wave, lane);
+    }
+} // namespace nnf

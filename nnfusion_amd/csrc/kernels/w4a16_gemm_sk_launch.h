@@ -1,0 +1,72 @@
+// Host side of one tile height of the fp16 x int4 tile GEMM (w4a16_gemm_sk.h): picks the instantiation for the
+// epilogue asked for and launches it.  Included by one translation unit per tile height, so that they compile in
+// parallel.
+#pragma once
+
+#include "w4a16_gemm_sk.h"
+
+namespace nnf
+{
+    namespace gemm_sk
+    {
+        // per (kernel, device): has the kernel been allowed its dynamic LDS yet
+        template <int TM, int TN, bool GATE, bool BIAS, bool RESID, bool RMS>
+        hipError_t launch_instance(hipStream_t stream, const SkGemmParams& p, int grid)
+        {
+            using T = Tile<TM, TN>;
+            auto kernel = &w4a16_gemm_sk_kernel<TM, TN, GATE, BIAS, RESID, RMS>;
+            if (T::LDS_BYTES > 48 * 1024)
+            {
+                static bool attr_set[64] = {};
+                int dev = 0;
+                hipError_t e = hipGetDevice(&dev);
+                if (e != hipSuccess)
+                    return e;
+                if (dev < 0 || dev >= 64 || !attr_set[dev])
+                {
+                    e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                            T::LDS_BYTES);
+                    if (e != hipSuccess)
+                        return e;
+                    if (dev >= 0 && dev < 64)
+                        attr_set[dev] = true;
+                }
+            }
+            hipLaunchKernelGGL(kernel, dim3(grid), dim3(THREADS), T::LDS_BYTES, stream, p);
+            hipError_t e = hipGetLastError();
+            if (e != hipSuccess || !p.partial)
+                return e;
+            // tiles shared by several workgroups: their parts are added and finished by a second launch
+            constexpr int ROUNDS = TM >= 2 ? TM / 2 : 1;
+            hipLaunchKernelGGL((w4a16_gemm_sk_fixup_kernel<TM, TN, GATE, BIAS, RESID, RMS>), dim3(p.tiles_m * p.tiles_n * ROUNDS),
+                               dim3(THREADS), 0, stream, p, grid);
+            return hipGetLastError();
+        }
+
+        template <int TM, int TN>
+        hipError_t launch_tile_height(hipStream_t stream, const SkGemmParams& p, int grid, bool gate)
+        {
+            const bool hb = p.bias != nullptr, hr = p.residual != nullptr, rms = p.gamma != nullptr;
+            if (gate)
+                return rms ? launch_instance<TM, TN, true, false, false, true>(stream, p, grid)
+                           : launch_instance<TM, TN, true, false, false, false>(stream, p, grid);
+            if (hb && hr)
+                return rms ? launch_instance<TM, TN, false, true, true, true>(stream, p, grid)
+                           : launch_instance<TM, TN, false, true, true, false>(stream, p, grid);
+            if (hb)
+                return rms ? launch_instance<TM, TN, false, true, false, true>(stream, p, grid)
+                           : launch_instance<TM, TN, false, true, false, false>(stream, p, grid);
+            if (hr)
+                return rms ? launch_instance<TM, TN, false, false, true, true>(stream, p, grid)
+                           : launch_instance<TM, TN, false, false, true, false>(stream, p, grid);
+            return rms ? launch_instance<TM, TN, false, false, false, true>(stream, p, grid)
+                       : launch_instance<TM, TN, false, false, false, false>(stream, p, grid);
+        }
+    } // namespace gemm_sk
+
+    // one per tile height (w4a16_gemm_sk_32.hip ... _256.hip)
+    hipError_t launch_gemm_sk_32(hipStream_t stream, const SkGemmParams& p, int grid, bool gate);
+    hipError_t launch_gemm_sk_64(hipStream_t stream, const SkGemmParams& p, int grid, bool gate);
+    hipError_t launch_gemm_sk_128(hipStream_t stream, const SkGemmParams& p, int grid, bool gate);
+    hipError_t launch_gemm_sk_256(hipStream_t stream, const SkGemmParams& p, int grid, bool gate);
+} // namespace nnf

@@ -122,9 +122,10 @@ namespace
     // fused: a call that may run the GEMV kernel into scratch (fp16 [M, N or 2N]) ahead of an element-wise epilogue
     size_t tuned_partial_bytes(int M, int N, int K, bool gate, bool fused = false)
     {
-        const size_t a = nnf::workspace::gemm_partial_bytes(
-            M, N, gate,
-            nnf::workspace::plan_w4a16_gemm(M, N, K, gate, nnf::g_tuning.gemm_tile - 1, nnf::g_tuning.gemm_splits));
+        static const int forced_rows[5] = {0, 256, 128, 64, 32};
+        const int f_rows = forced_rows[nnf::g_tuning.gemm_tile >= 0 && nnf::g_tuning.gemm_tile <= 4 ? nnf::g_tuning.gemm_tile : 0];
+        const size_t a =
+            nnf::workspace::plan_w4a16_sk_with(M, N, K, gate, nnf::workspace::PLAN_CUS, f_rows, nnf::g_tuning.gemm_splits).bytes();
         // the M <= 16 kernels over ranges of K write partial sums too
         const size_t b = nnf::workspace::skinny_split_bytes(M, gate ? 2 * N : N, K);
         const size_t c = nnf::workspace::mrows_split_bytes(M, gate ? 2 * N : N, K);
@@ -197,7 +198,7 @@ size_t nnf_w4a16_gemm_variant_workspace_bytes(int M, int N, int K, int group, in
     if (M <= 0 || N <= 0 || K < 128)
         return 0;
     if (variant == NNF_W4A16_GEMM_MFMA)
-        return nnf::workspace::gemm_partial_bytes(M, N, false, nnf::workspace::plan_w4a16_gemm(M, N, K, false));
+        return nnf::workspace::plan_w4a16_sk(M, N, K, false, nnf::workspace::PLAN_CUS).bytes();
     if (variant == NNF_W4A16_AUTO)
         return nnf::workspace::w4a16_gemm(M, N, K, group);
     return 0;

@@ -106,6 +106,72 @@ namespace nnf
             return p.reduce_pass ? align256((size_t)p.splits * M * (gate ? 2 : 1) * N * sizeof(float)) : 0;
         }
 
+        // ---- plan of the fp16 x int4 tile GEMM (w4a16_gemm_sk.h) ----------------------------------------------
+        // Tiles of tile_rows x 256 weight rows (SiLU-gate: 128 gate + 128 up rows, i.e. 128 output columns); the
+        // (tile, superstep of 256 k) units of the whole product are split evenly over `grid` workgroups, one per CU.
+        // A tile whose units belong to more than one workgroup is summed through the workspace: slots of
+        // tile_rows x 256 fp32; workgroup v parks the first segment of its range in slot v and a later one in slot
+        // grid + v; a second launch adds them up.
+        struct SkPlan
+        {
+            int tile_rows = 0; // 32, 64, 128 or 256
+            int tiles_m = 0, tiles_n = 0;
+            int supersteps = 0; // per tile: ceil(K / 256)
+            long long units = 0;
+            int grid = 0;
+            int slots = 0;     // 0: every tile belongs to one workgroup (no workspace, no second launch)
+            size_t bytes() const { return (size_t)slots * tile_rows * 256 * sizeof(float); }
+        };
+        // forced_tile_rows / forced_grid: 0 = the plan's own choice
+        inline SkPlan plan_w4a16_sk(int M, int N, int K, bool gate, int num_cu, int forced_tile_rows = 0, int forced_grid = 0)
+        {
+            SkPlan p;
+            if (M <= 0 || N <= 0 || K < 128 || num_cu < 1)
+                return p;
+            // 256-row tiles unpack every weight once per 256 rows and are the fastest from about 1500 rows on; below,
+            // 128-row tiles (twice the tiles, half as large parked sums per workgroup) measured 5-20 % faster
+            int rows = M <= 32 ? 32 : M <= 64 ? 64 : M <= 1536 ? 128 : 256;
+            if (forced_tile_rows == 32 || forced_tile_rows == 64 || forced_tile_rows == 128 || forced_tile_rows == 256)
+                rows = forced_tile_rows;
+            p.tile_rows = rows;
+            p.tiles_m = ceil_div(M, rows);
+            p.tiles_n = ceil_div(N, gate ? 128 : 256);
+            const int G = (K / 128 + 1) / 2; // supersteps per tile
+            p.supersteps = G;
+            p.units = (long long)p.tiles_m * p.tiles_n * G;
+            // a workgroup keeps at least two supersteps (eight K steps) unless forced
+            long long grid = p.units / 2 < 1 ? 1 : p.units / 2;
+            if (grid > num_cu)
+                grid = num_cu;
+            if (forced_grid > 0)
+                grid = forced_grid < p.units ? forced_grid : p.units;
+            p.grid = (int)grid;
+            bool first_used = false, later_used = false;
+            for (int v = 0; v < p.grid; ++v)
+            {
+                const long long u0 = ((long long)v * p.units) / p.grid, u1 = ((long long)(v + 1) * p.units) / p.grid;
+                if (u1 <= u0)
+                    continue;
+                if (u0 % G != 0 || u1 - u0 < G - u0 % G) // the first segment is not a whole tile
+                    first_used = true;
+                const long long last_tile_begin = ((u1 - 1) / G) * G;
+                if (last_tile_begin > u0 && u1 % G != 0) // a later segment that stops short of its tile's end
+                    later_used = true;
+            }
+            p.slots = later_used ? 2 * p.grid : first_used ? p.grid : 0;
+            return p;
+        }
+
+        // the plan with a forced tile height (0 = the plan's own) and a forced number of workgroups per tile (0 = the
+        // plan's own grid)
+        inline SkPlan plan_w4a16_sk_with(int M, int N, int K, bool gate, int num_cu, int tile_rows, int workgroups_per_tile)
+        {
+            if (workgroups_per_tile <= 0)
+                return plan_w4a16_sk(M, N, K, gate, num_cu, tile_rows, 0);
+            const SkPlan t = plan_w4a16_sk(M, N, K, gate, num_cu, tile_rows, 0);
+            return plan_w4a16_sk(M, N, K, gate, num_cu, tile_rows, t.tiles_m * t.tiles_n * workgroups_per_tile);
+        }
+
         // ---- plan of the skinny (M <= 16) MFMA GEMV kernel ---------------------------------------------
         constexpr size_t LDS_BYTES_PER_CU = 160 * 1024; // gfx950
         struct SkinnyPlan
@@ -279,7 +345,14 @@ namespace nnf
         }
 
         // normalised activations of the RMSNorm prologue (fp16 [M, K])
-        inline size_t rms_rows(int M, int K) { return (M > 0 && K > 0) ? align256((size_t)M * K * 2) : 0; }
+        // RMSNorm prologue.  The tile GEMM folds the normalisation in and needs one fp32 per row (rstd); the kernels
+        // that serve up to 40 rows read normalised activations: fp16 [M, K].
+        inline size_t rms_rows(int M, int K)
+        {
+            if (M <= 0 || K <= 0)
+                return 0;
+            return M <= 40 ? align256((size_t)M * K * 2) : align256((size_t)M * sizeof(float));
+        }
 
         inline size_t mrows_split_bytes(int M, int N_total, int K); // the row-streaming MFMA kernel over ranges of K
         // Fused calls with at most 32 rows may run the GEMV kernel into scratch and an element-wise epilogue from
@@ -293,7 +366,7 @@ namespace nnf
                 return 0;
             if (w4a16_skinny_fits(M, N, K))
                 return 0; // served by the skinny kernel
-            const size_t a = gemm_partial_bytes(M, N, false, plan_w4a16_gemm(M, N, K, false));
+            const size_t a = plan_w4a16_sk(M, N, K, false, PLAN_CUS).bytes();
             const size_t b = skinny_split_bytes(M, N, K), c = mrows_split_bytes(M, N, K);
             return a > b ? (a > c ? a : c) : (b > c ? b : c);
         }
@@ -303,7 +376,7 @@ namespace nnf
             if (M <= 0 || N <= 0 || K < 128)
                 return 0;
             const bool gate = act == 1;
-            const size_t a = gemm_partial_bytes(M, N, gate, plan_w4a16_gemm(M, N, K, gate));
+            const size_t a = plan_w4a16_sk(M, N, K, gate, PLAN_CUS).bytes();
             const size_t b = skinny_split_bytes(M, gate ? 2 * N : N, K), c = mrows_split_bytes(M, gate ? 2 * N : N, K);
             const size_t d = gemv_scratch_bytes(M, gate ? 2 * N : N);
             const size_t bc = b > c ? b : c, ad = a > d ? a : d;
@@ -556,8 +629,8 @@ namespace nnf
         {
             if (M <= 0 || I <= 0 || H < 128 || I < 128)
                 return 0;
-            size_t a = gemm_partial_bytes(M, I, true, plan_w4a16_gemm(M, I, H, true));
-            size_t b = gemm_partial_bytes(M, H, false, plan_w4a16_gemm(M, H, I, false));
+            size_t a = plan_w4a16_sk(M, I, H, true, PLAN_CUS).bytes();
+            size_t b = plan_w4a16_sk(M, H, I, false, PLAN_CUS).bytes();
             size_t c = skinny_split_bytes(M, 2 * I, H), d = skinny_split_bytes(M, H, I);
             const size_t e = mrows_split_bytes(M, 2 * I, H), f = mrows_split_bytes(M, H, I);
             const size_t g = gemv_scratch_bytes(M, 2 * I); // gate | up of the first GEMM at M <= 32

@@ -352,16 +352,15 @@ int main(int argc, char** argv)
         CONTAINS(deps, "typedef _Float16 half;");
         EXPECT(deps.find("cuda") == std::string::npos && deps.find("cublas") == std::string::npos);
 
-        // fused variant: gamma, bias; the scratch tensor appears in signature and call.  Its size: the normalised
-        // activations (256 x 4096 fp16) + the partial sums of the plan for this shape (128 x 128 tiles: 2 x 32 of
-        // them, K split 4 ways: 4 x 256 x 4096 fp32)
+        // fused variant: gamma, bias; the scratch tensor appears in signature and call.  Its size: one fp32 per row
+        // (rstd) + the parked sums of the plan for this shape (32 tiles of 128 x 256 x 16 supersteps over 256 workgroups: one slot each)
         graph::Graph g2;
         auto n2 = quant_dot_graph(g2, 256, 4096, 4096, "{\"rms_norm\": true, \"has_bias\": true, \"rms_eps\": 1e-5}", true, true);
         auto k2 = sel.pick_first(n2, ROCM_GPU).second;
         auto fu2 = k2->get_or_emit_source();
         CONTAINS(fu2->body_unit->get_code(), "nnf_w4a16_gemm_fused(stream, input0, input1, input2, output0, 256, 4096, 4096, 128, 8, input3, 1.000000000e-05f, input4, nullptr, NNF_ACT_NONE, ");
         EXPECT(k2->m_context->tensors.size() == 1 &&
-               k2->m_context->tensors[0]->size() == (size_t)256 * 4096 * 2 + (size_t)4 * 256 * 4096 * 4);
+               k2->m_context->tensors[0]->size() == (size_t)256 * 4 + (size_t)256 * 128 * 256 * 4);
         CONTAINS(fu2->signature_unit->get_code(), "char* " + k2->m_context->tensors[0]->get_name());
         CONTAINS(fu2->call_unit->get_code(), k2->m_context->tensors[0]->get_name() + ");");
         // SiLU gate: N is half the weight rows
@@ -437,12 +436,12 @@ int main(int argc, char** argv)
         auto k = sel.pick_first(mlp, ROCM_GPU).second;
         auto fm = k->get_or_emit_source();
         CONTAINS(fm->body_unit->get_code(), "nnf_fused_mlp_w4a16(stream, input0, input1, 1.000000000e-06f, input2, input3, input4, input5, output0, 256, 4096, 11008, 128, 8, ");
-        // RMSNorm(x) [256, 4096] fp16 + h [256, 11008] fp16 + the larger of the two partial-sum areas: gate/up
-        // (86 tiles of 256 x (128 + 128), K split in 2: 2 x 256 x 22016 fp32) vs down (2 x 32 tiles of 128 x 128,
-        // K split 4 ways: 4 x 256 x 4096 fp32)
+        // rstd [256] fp32 + h [256, 11008] fp16 + the larger of the two areas of parked sums: both GEMMs run 256
+        // workgroups over tiles of 128 x 256 weight rows; gate/up (2 x 86 tiles x 16 supersteps) needs two slots per
+        // workgroup
         EXPECT(k->m_context->tensors.size() == 1 &&
                k->m_context->tensors[0]->size() ==
-                   (size_t)256 * 4096 * 2 + (size_t)256 * 11008 * 2 + (size_t)2 * 256 * 22016 * 4);
+                   (size_t)256 * 4 + (size_t)256 * 11008 * 2 + (size_t)2 * 256 * 128 * 256 * 4);
     });
 
     run_case("codegen_project", [&] {
