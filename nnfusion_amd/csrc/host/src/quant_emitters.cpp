@@ -146,8 +146,7 @@ namespace nnfusion
                         return nullptr;
                     size_t ws_bytes = 0;
                     if (VARIANT == 3)
-                        ws_bytes = nnf::workspace::gemm_partial_bytes(
-                            (int)M, (int)N, false, nnf::workspace::plan_w4a16_gemm((int)M, (int)N, (int)K, false));
+                        ws_bytes = nnf::workspace::plan_w4a16_sk((int)M, (int)N, (int)K, false, nnf::workspace::PLAN_CUS).bytes();
                     std::string ws = "nullptr";
                     if (ws_bytes > 0)
                         ws = allocate_tensor(Shape{ws_bytes}, element::character)->get_name();

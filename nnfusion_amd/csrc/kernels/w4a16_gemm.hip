@@ -1,16 +1,16 @@
-// fp16 x int4 (g128) GEMM for M > 16 on the gfx950 matrix cores: dispatcher, the big-tile
-// instantiations of the kernel template in w4a16_gemm_dl.h, the RMSNorm pre-pass and the split-K
-// reduction pass.
+// fp16 x int4 (g128) products beyond one activation row: the dispatcher between the row-streaming /
+// split-K GEMV kernels (up to 40 rows) and the tile GEMM (w4a16_gemm_sk.h), the RMSNorm pre-passes, the
+// reduction pass behind the GEMV kernels that run over ranges of K, and their element-wise epilogues.
 //
 //   Y[M,N] = epilogue( prologue(A)[M,K] . ((Wq - zp) * S)^T )
 //
-//   * prologue: RMSNorm.  x * rsqrt(mean(x^2) + eps) * gamma is computed in fp32 and rounded to fp16 into
-//     scratch memory (the normalised activation tensor of the unfused graph); the GEMM then reads that.
+//   * prologue: RMSNorm.  The tile GEMM folds it in (a pre-pass computes rstd[m] only); the GEMV
+//     kernels read normalised activations, fp16(x * rsqrt(mean(x^2) + eps) * gamma) written to scratch
+//     memory by a pre-pass (the tensor of the unfused graph, at most 40 rows of it).
 //   * epilogues: bias, residual add, SiLU(gate) * up with the gate and up projections as two halves of
-//     the N tile -- in the GEMM kernel, or in the reduction pass when K is split.
-//   * the tile shape and the number of K ranges follow nnf::workspace::plan_w4a16_gemm: 256 x 256 tiles
-//     when they fill the GPU, otherwise 128 x 128 or 64 x 256 tiles with K split across workgroups so
-//     that about two workgroups per CU are in flight.
+//     the N tile -- in the tile GEMM's epilogue, in the reduction pass, or in an element-wise kernel
+//     behind a GEMV kernel.
+//   * tile height and split of the work over the CUs follow nnf::workspace::plan_w4a16_sk.
 #include "w4a16_gemm_sk_launch.h"
 
 #include "../nnf_workspace.h"

@@ -905,18 +905,30 @@ int main(int argc, char** argv)
             EXPECT(ws::w8a8_skinny_fits(1, k) && ws::w8a8_gemm(1, 4096, k) == 0);
         }
         EXPECT(!ws::w8a8_skinny_fits(16, 8192) && ws::w8a8_gemm(16, 8192, 8192) > 0);
-        // GEMM tile plans: a split count the K loop can be cut into, partial sums sized for it
+        // fp16 x int4 tile GEMM: the (tile, superstep) units are split evenly over at most one workgroup per CU; a
+        // workgroup parks at most two partial tiles; whole tiles need no workspace
         {
             const int ms[] = {17, 64, 128, 256, 1024, 4096};
             for (int m : ms)
                 for (int gate = 0; gate < 2; ++gate)
                 {
-                    const auto p = ws::plan_w4a16_gemm(m, 8192, 8192, gate != 0);
-                    EXPECT(p.splits >= 1 && p.splits <= 16 && (8192 / 128) / p.splits >= 4);
-                    EXPECT((p.splits > 1 || p.reduce_pass) == (ws::gemm_partial_bytes(m, 8192, gate != 0, p) > 0));
+                    const auto p = ws::plan_w4a16_sk(m, 8192, 8192, gate != 0, 256);
+                    EXPECT(p.supersteps == 32 && p.units == (long long)p.tiles_m * p.tiles_n * 32);
+                    EXPECT(p.grid >= 1 && p.grid <= 256 && p.units / p.grid >= 2);
+                    EXPECT(p.tiles_m * p.tile_rows >= m && (p.tiles_m - 1) * p.tile_rows < m);
+                    EXPECT(p.slots == 0 || p.slots == p.grid || p.slots == 2 * p.grid);
+                    EXPECT(p.bytes() == (size_t)p.slots * p.tile_rows * 256 * 4);
+                    // every unit has exactly one owner, and owners follow each other
+                    long long covered = 0;
+                    for (int v = 0; v < p.grid; ++v)
+                        covered += ((long long)(v + 1) * p.units) / p.grid - ((long long)v * p.units) / p.grid;
+                    EXPECT(covered == p.units);
                 }
-            EXPECT(ws::plan_w4a16_gemm(4096, 8192, 8192, false).tile == ws::GEMM_TILE_BIG);
-            EXPECT(ws::plan_w4a16_gemm(32, 8192, 8192, false).reduce_pass);
+            const auto big = ws::plan_w4a16_sk(4096, 8192, 8192, false, 256);
+            EXPECT(big.tile_rows == 256 && big.grid == 256 && big.slots == 0 && big.bytes() == 0);
+            EXPECT(ws::plan_w4a16_sk(128, 8192, 8192, false, 256).slots > 0);
+            // K = 128 * odd: the last superstep of a tile holds one group
+            EXPECT(ws::plan_w4a16_sk(64, 512, 384, false, 256).supersteps == 2);
         }
     });
 

@@ -38,7 +38,9 @@ def test_mlp_matches_unfused_oracle(gpu, m, h, i):
 
 def test_mlp_full_size_rows(gpu):
     """configs[4]: M = 256, 4096 -> 11008 -> 4096.  The oracle runs the first 8 token rows (rows are
-    independent); the other rows are covered by the identity out(x_row) for duplicated rows."""
+    independent); the other rows are covered by duplicated rows, which must give the same outputs up to the
+    rounding of a different summation order (the rows sit in different tiles, whose K ranges are cut at different
+    places by the even split of the work over the CUs; run to run the result is bit-identical: see below)."""
     import torch
 
     from nnfusion_amd import ops
@@ -51,7 +53,10 @@ def test_mlp_full_size_rows(gpu):
     ref = oracle.fused_mlp_w4a16(x[:8].copy(), gamma, wgu, sgu, wd, sd)
     err = float(np.abs(out[:8].astype(np.float32) - ref.astype(np.float32)).max())
     assert err <= 1e-2 * _rms(ref), (err, _rms(ref))
-    assert np.array_equal(out[128:136], out[0:8])
+    dup = float(np.abs(out[128:136].astype(np.float32) - out[0:8].astype(np.float32)).max())
+    assert dup <= 2e-3 * _rms(ref), (dup, _rms(ref))
+    again = ops.fused_mlp_w4a16(*_t(gpu, x, gamma, wgu, sgu, wd, sd)).cpu().numpy()
+    assert np.array_equal(again, out)
 
 
 def test_mlp_workspace_contract(gpu):
