@@ -122,25 +122,23 @@ namespace nnf
             int slots = 0;     // 0: every tile belongs to one workgroup (no workspace, no second launch)
             size_t bytes() const { return (size_t)slots * tile_rows * 256 * sizeof(float); }
         };
+        // tiles_n column tiles, `per_tile` units of K per tile, at least `min_units` units per workgroup (unless forced);
         // forced_tile_rows / forced_grid: 0 = the plan's own choice
-        inline SkPlan plan_w4a16_sk(int M, int N, int K, bool gate, int num_cu, int forced_tile_rows = 0, int forced_grid = 0)
+        inline SkPlan plan_sk(int M, int tiles_n, int per_tile, int min_units, int num_cu, int forced_tile_rows, int forced_grid)
         {
             SkPlan p;
-            if (M <= 0 || N <= 0 || K < 128 || num_cu < 1)
-                return p;
-            // 256-row tiles unpack every weight once per 256 rows and are the fastest from about 1500 rows on; below,
+            // 256-row tiles touch every weight once per 256 rows and are the fastest from about 1500 rows on; below,
             // 128-row tiles (twice the tiles, half as large parked sums per workgroup) measured 5-20 % faster
             int rows = M <= 32 ? 32 : M <= 64 ? 64 : M <= 1536 ? 128 : 256;
             if (forced_tile_rows == 32 || forced_tile_rows == 64 || forced_tile_rows == 128 || forced_tile_rows == 256)
                 rows = forced_tile_rows;
             p.tile_rows = rows;
             p.tiles_m = ceil_div(M, rows);
-            p.tiles_n = ceil_div(N, gate ? 128 : 256);
-            const int G = (K / 128 + 1) / 2; // supersteps per tile
+            p.tiles_n = tiles_n;
+            const int G = per_tile;
             p.supersteps = G;
             p.units = (long long)p.tiles_m * p.tiles_n * G;
-            // a workgroup keeps at least two supersteps (eight K steps) unless forced
-            long long grid = p.units / 2 < 1 ? 1 : p.units / 2;
+            long long grid = p.units / min_units < 1 ? 1 : p.units / min_units;
             if (grid > num_cu)
                 grid = num_cu;
             if (forced_grid > 0)
@@ -161,6 +159,20 @@ namespace nnf
             p.slots = later_used ? 2 * p.grid : first_used ? p.grid : 0;
             return p;
         }
+        // fp16 x int4: units of 256 k (supersteps), a workgroup keeps at least two (eight K steps of 64)
+        inline SkPlan plan_w4a16_sk(int M, int N, int K, bool gate, int num_cu, int forced_tile_rows = 0, int forced_grid = 0)
+        {
+            if (M <= 0 || N <= 0 || K < 128 || num_cu < 1)
+                return SkPlan();
+            return plan_sk(M, ceil_div(N, gate ? 128 : 256), (K / 128 + 1) / 2, 2, num_cu, forced_tile_rows, forced_grid);
+        }
+        // W8A8 (w8a8_gemm_sk.h): units of 128 k (its K steps), a workgroup keeps at least four; slots of int32
+        inline SkPlan plan_w8a8_sk(int M, int N, int K, int num_cu, int forced_tile_rows = 0, int forced_grid = 0)
+        {
+            if (M <= 0 || N <= 0 || K < 128 || num_cu < 1)
+                return SkPlan();
+            return plan_sk(M, ceil_div(N, 256), K / 128, 4, num_cu, forced_tile_rows, forced_grid);
+        }
 
         // the plan with a forced tile height (0 = the plan's own) and a forced number of workgroups per tile (0 = the
         // plan's own grid)
@@ -170,6 +182,13 @@ namespace nnf
                 return plan_w4a16_sk(M, N, K, gate, num_cu, tile_rows, 0);
             const SkPlan t = plan_w4a16_sk(M, N, K, gate, num_cu, tile_rows, 0);
             return plan_w4a16_sk(M, N, K, gate, num_cu, tile_rows, t.tiles_m * t.tiles_n * workgroups_per_tile);
+        }
+        inline SkPlan plan_w8a8_sk_with(int M, int N, int K, int num_cu, int tile_rows, int workgroups_per_tile)
+        {
+            if (workgroups_per_tile <= 0)
+                return plan_w8a8_sk(M, N, K, num_cu, tile_rows, 0);
+            const SkPlan t = plan_w8a8_sk(M, N, K, num_cu, tile_rows, 0);
+            return plan_w8a8_sk(M, N, K, num_cu, tile_rows, t.tiles_m * t.tiles_n * workgroups_per_tile);
         }
 
         // ---- plan of the skinny (M <= 16) MFMA GEMV kernel ---------------------------------------------
@@ -617,7 +636,7 @@ namespace nnf
                 return 0;
             if (w8a8_skinny_fits(M, K))
                 return 0;
-            return gemm_partial_bytes(M, N, false, plan_w8a8_gemm(M, N, K));
+            return plan_w8a8_sk(M, N, K, PLAN_CUS).bytes();
         }
         // nnf_fused_mlp_w4a16: [ normalised x: M x H fp16 ][ h: M x I fp16 ][ partial sums of either GEMM ]
         inline size_t fused_mlp_h_offset(int M, int H) { return rms_rows(M, H); }
