@@ -12,13 +12,22 @@ decoder walks its layers.  Inputs are resident in HBM before the timed region; t
 steps captured in one HIP graph (launch-bound otherwise: each kernel runs for a few microseconds),
 bracketed by synchronisation.
 
+Before anything is timed, every configuration that will be timed is run once and compared with the CPU
+oracle (the sweep on whole outputs; the large configurations on sampled output columns / token rows);
+a mismatch aborts the run with a non-zero exit status and no JSON line.
+
 Prints ONE JSON line.  `value` = algorithmic bytes of a step (every operand read once, output written
-once) / time per step.  `roofline` covers the kernel that dominates the step; `cpu_baseline` times the
-same sweep on the host cores with the reference's CPU GEMM (MLAS built from the reference tree, or the
-oracle's own port when that library is absent) on fp32 weights dequantised beforehand.  `extra` holds
-the other configurations (prefill GEMM, W8A8, fused MLP), each measured for a few iterations.
+once) / time per step.  `roofline` covers the kernel that dominates the step; `roofline_extra` holds the
+same figures for every other configuration (prefill GEMM, batched decode, W8A8, fused MLP), each
+measured for a few iterations (`extra` has their plain timings); `traffic` fields are HBM bytes per launch
+from hardware-counter runs, read from the summaries under profiles/ (null where none is recorded).
+`cpu_baseline` times the sweep on the host cores with the reference's CPU GEMM (MLAS built from the
+reference tree, or the oracle's own port when that library is absent) on fp32 weights dequantised
+beforehand.
 """
 import argparse
+import ctypes
+import glob
 import json
 import os
 import sys
@@ -35,11 +44,29 @@ MFMA_I8_PEAK_TOPS = 5000.0     # dense int8 MFMA
 
 DECODE_SHAPES = [(12288, 4096), (4096, 4096), (22016, 4096), (4096, 11008)]  # (N, K), M = 1
 GROUP = 128
-PROBE_BYTES = 1 << 30  # size of the calibration copy of --pmc-probe
-# HBM bytes per launch of the K = 4096 row-streaming kernel (mean over its three launches of a step), from two
-# rocprofv3 --pmc runs of `bench.py --pmc-probe`: FETCH_SIZE 13268.7 KiB x 2.000 (the factor by which the
-# counter under-reports the 1 GiB calibration copy) + WRITE_SIZE 27.3 KiB x 1.000.  Algorithmic: 27 067 392.
-ROWS_K4096_TRAFFIC_BYTES = int((13268.7 * 2.0 + 27.3) * 1024)
+PROBE_BYTES = 1 << 30  # size of the calibration copy of --pmc-probe and of the large plain read
+W4A16_TOL = 1e-2       # max |y - y_ref| <= W4A16_TOL * RMS(y_ref): the tolerance of the fp16 x int4 path
+PROBES_SO = os.path.join(ROOT, "nnfusion_amd", "lib", "libnnf_bench_probes.so")
+PROFILES_DIR = os.path.join(ROOT, "profiles")
+
+GEMM_NK = 8192
+GEMM_MS = (16, 128, 1024, 4096)       # configs[2]
+W8A8_MS = (1, 32, 512, 4096)          # configs[3]
+SMALL_BATCHES = (2, 4, 8, 16)         # the sweep's shapes with a few rows
+MLP_SHAPE = (256, 4096, 11008)        # configs[4]
+
+# the kernel that dominates each configuration row (what a kernel trace of the row shows)
+DOMINANT_KERNEL = {
+    "w4a16_gemm_N8192_K8192.M16": "nnf::w4a16_mrows_kernel<2, 4, 1> (row-streaming MFMA kernel)",
+    "w4a16_gemm_N8192_K8192.M128": "nnf::gemm_sk::w4a16_gemm_sk_kernel<4, 2, ...> + w4a16_gemm_sk_fixup_kernel",
+    "w4a16_gemm_N8192_K8192.M1024": "nnf::gemm_sk::w4a16_gemm_sk_kernel<4, 2, ...> + w4a16_gemm_sk_fixup_kernel",
+    "w4a16_gemm_N8192_K8192.M4096": "nnf::gemm_sk::w4a16_gemm_sk_kernel<8, 2, ...>",
+    "w8a8_gemm_N8192_K8192.M1": "nnf::w8a8_gemv_rows_kernel",
+    "w8a8_gemm_N8192_K8192.M32": "nnf::w8a8_mrows_kernel",
+    "w8a8_gemm_N8192_K8192.M512": "nnf::w8a8_gemm_dl_kernel (128 x 128 tiles)",
+    "w8a8_gemm_N8192_K8192.M4096": "nnf::w8a8_gemm_dl_kernel (256 x 256 tiles)",
+    "fused_mlp_M256_4096_11008": "rms_rstd_kernel + 2 x (nnf::gemm_sk::w4a16_gemm_sk_kernel<4, 2, ...> + fixup)",
+}
 
 
 def w4a16_bytes(m, n, k):
@@ -51,6 +78,39 @@ def w8a8_bytes(m, n, k):
     return n * k + n * 4 + m * k + m * 4 + m * n * 2
 
 
+def mlp_bytes(m, h, i):
+    """x, gamma, both weight matrices with scales, h written and read once (it is a tensor of the block), out."""
+    return m * h * 2 + h * 2 + (2 * i * h // 2 + 2 * i * (h // GROUP) * 2) + (h * i // 2 + h * (i // GROUP) * 2) + \
+        2 * m * i * 2 + m * h * 2
+
+
+def load_traffic():
+    """`traffic_bytes_per_launch <row key> <bytes>` lines of the hardware-counter summaries under profiles/."""
+    out = {}
+    for path in sorted(glob.glob(os.path.join(PROFILES_DIR, "*.txt"))):
+        with open(path) as f:
+            for line in f:
+                parts = line.split()
+                if len(parts) == 3 and parts[0] == "traffic_bytes_per_launch":
+                    try:
+                        out[parts[1]] = int(parts[2])
+                    except ValueError:
+                        pass
+    return out
+
+
+def load_probes():
+    if not os.path.exists(PROBES_SO):
+        sys.exit(f"bench.py: {PROBES_SO} is not built (make -C nnfusion_amd/csrc)")
+    lib = ctypes.CDLL(PROBES_SO)
+    lib.nnf_probe_read.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_longlong, ctypes.c_int, ctypes.c_int]
+    lib.nnf_probe_read.restype = ctypes.c_int
+    lib.nnf_probe_mfma.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_double),
+                                   ctypes.POINTER(ctypes.c_double)]
+    lib.nnf_probe_mfma.restype = ctypes.c_int
+    return lib
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -60,8 +120,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true")
     ap.add_argument("--pmc-probe", action="store_true",
-                    help="for hardware-counter runs: a plain copy of known size, then the sweep launched eagerly; "
-                         "no timing, no JSON")
+                    help="for hardware-counter runs: a plain copy of known size, then every configuration launched "
+                         "eagerly, a marker launch ahead of each; prints the order of the rows, no timing")
     ap.add_argument("--mfma-probe", action="store_true",
                     help="print the MFMA-only rates (no memory traffic) for different operand values and exit")
     ap.add_argument("--gemm-probe", action="store_true",
@@ -80,12 +140,13 @@ def main():
         sys.exit("bench.py: no GPU visible")
     dev = torch.device("cuda:0")
     lib = _lib.kernels()
-
-    def dev_t(a):
-        return torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    env = Env(torch, np, dev, lib, datagen, ops)
 
     if args.gemm_probe:
-        print(json.dumps(run_gemm_probe(torch, dev, datagen, ops)))
+        print(json.dumps(run_gemm_probe(env)))
+        return
+    if args.mfma_probe:
+        print(json.dumps(run_mfma_probe(env, load_probes())))
         return
 
     # ---- resident inputs ------------------------------------------------------------------------
@@ -97,7 +158,7 @@ def main():
             a, wq, s = datagen.w4a16_case(layer, 1, n, k)  # seed = layer index; layer 0 is "seed 0"
             if layer == 0:
                 host_layer0.append((a, wq, s))
-            shapes.append((dev_t(a), dev_t(wq), dev_t(s), torch.empty((1, n), dtype=torch.float16, device=dev)))
+            shapes.append((env.dev_t(a), env.dev_t(wq), env.dev_t(s), torch.empty((1, n), dtype=torch.float16, device=dev)))
         layers.append(shapes)
     ws = torch.empty(1 << 20, dtype=torch.uint8, device=dev)
 
@@ -114,50 +175,21 @@ def main():
         for sh in layers[i % args.layers]:
             launch(sh)
 
-    def timed_graph(fn_list, reps):
-        """Capture fn_list (callables that enqueue launches) into one graph; return mean microseconds of
-        one replay over `reps` replays, measured with events on the launch stream."""
-        g = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(g):
-            for fn in fn_list:
-                fn()
-        g.replay()
-        torch.cuda.synchronize()
-        e0 = torch.cuda.Event(enable_timing=True)
-        e1 = torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(reps):
-            g.replay()
-        e1.record()
-        torch.cuda.synchronize()
-        return e0.elapsed_time(e1) * 1000.0 / reps
-
-    if args.mfma_probe:
-        print(json.dumps(run_mfma_probe(torch, lib)))
-        return
-
     if args.pmc_probe:
-        # Calibration for FETCH_SIZE / WRITE_SIZE: a device-to-device copy that reads and writes exactly
-        # PROBE_BYTES, larger than the last-level cache, followed by the sweep over every resident layer.
-        src = torch.empty(PROBE_BYTES // 4, dtype=torch.float32, device=dev).normal_()
-        dst = torch.empty_like(src)
-        torch.cuda.synchronize()
-        for _ in range(4):
-            dst.copy_(src)
-        torch.cuda.synchronize()
-        for i in range(2 * args.layers):
-            step(i)
-        torch.cuda.synchronize()
-        # the same weights with 16 activation rows (the row-streaming MFMA kernel; K = 11008: three ranges of K
-        # and the reduction pass), over every resident layer
-        ws16 = torch.empty(16 << 20, dtype=torch.uint8, device=dev)
-        for shapes in layers:
-            for (_, wq, s, _) in shapes:
-                a16 = torch.empty((16, wq.shape[1] * 2), dtype=torch.float16, device=dev).normal_()
-                ops.w4a16_gemm(a16, wq, s, workspace=ws16)
-        torch.cuda.synchronize()
-        print(f"pmc probe: copy of {PROBE_BYTES} bytes x4, then {2 * args.layers} sweeps, then {args.layers} sweeps with 16 rows", flush=True)
+        run_pmc_probe(env, load_probes(), layers, step, args.layers)
         return
+
+    # ---- parity gate: nothing is timed unless the results are the oracle's ----------------------------
+    import oracle
+
+    parity = {}
+    step(0)
+    torch.cuda.synchronize()
+    for (a, wq, s), (_, _, _, y) in zip(host_layer0, layers[0]):
+        ref = oracle.w4a16_gemm(a, wq, s, f32_out=True)
+        check_w4a16(np, parity, f"decode_sweep.N{wq.shape[0]}_K{a.shape[1]}", y.cpu().numpy(), ref)
+    if not args.no_extra:
+        parity_extra(env, oracle, parity)
 
     # ---- warm-up (untimed), then exactly K steps in the timed region ------------------------------
     for i in range(args.warmup):
@@ -184,6 +216,7 @@ def main():
     # ---- per-shape launch durations -------------------------------------------------------------
     # Events around a graph of one shape walking enough copies of its weights (device-side clones of the
     # layers) that no launch finds them in the last-level cache, as in the timed region above.
+    traffic = load_traffic()
     per_shape = []
     for si, (n, k) in enumerate(DECODE_SHAPES):
         n_copies = max(args.layers, -(-COLD_FOOTPRINT_BYTES // w4a16_bytes(1, n, k)))
@@ -192,16 +225,21 @@ def main():
             a, wq, s, y = layers[c % args.layers][si]
             copies.append((a, wq, s, y) if c < args.layers else (a, wq.clone(), s.clone(), y))
         fns = [(lambda t=t: launch(t)) for t in copies]
-        us = timed_graph(fns, 4) / len(fns)
+        us = env.timed_graph(fns, 4) / len(fns)
         del copies
         per_shape.append({"N": n, "K": k, "us": round(us, 3), "GB/s": round(w4a16_bytes(1, n, k) / us / 1e3, 1),
-                          "frac_hbm": round(w4a16_bytes(1, n, k) / us / 1e3 / HBM_PEAK_GBS, 4)})
+                          "frac_hbm": round(w4a16_bytes(1, n, k) / us / 1e3 / HBM_PEAK_GBS, 4),
+                          "traffic": traffic.get(f"decode_sweep.N{n}_K{k}")})
+    plain_read = None
     if not args.no_extra:
-        run_read_probe(torch, dev, lib, args.layers, per_shape, timed_graph)
+        probes = load_probes()
+        run_read_probe(env, probes, args.layers, per_shape)
+        plain_read = run_large_read_probe(env, probes)
     # dominant kernel: the K = 4096 instantiations of the row-streaming kernel serve three of the four launches
     k4096 = [p for p in per_shape if p["K"] == 4096]
     dom_us = sum(p["us"] for p in k4096) / len(k4096)
     dom_bytes = sum(w4a16_bytes(1, p["N"], p["K"]) for p in k4096) / len(k4096)
+    dom_traffic = [p["traffic"] for p in k4096]
     roofline = {
         "bound": "hbm",
         "kernel": "nnf::w4a16_gemv_rows_kernel<2, D, 8> (K=4096: two KiB per row; mean over its three launches per step)",
@@ -209,14 +247,16 @@ def main():
         "peak": HBM_PEAK_GBS,
         "unit": "GB/s",
         "frac": round(dom_bytes / dom_us / 1e3 / HBM_PEAK_GBS, 4),
-        "traffic": ROWS_K4096_TRAFFIC_BYTES,
+        "traffic": None if any(t is None for t in dom_traffic) else int(sum(dom_traffic) / len(dom_traffic)),
         "bytes_per_launch": int(dom_bytes),
         "us_per_launch": round(dom_us, 3),
     }
+    if plain_read is not None:
+        roofline["frac_of_plain_read_1GiB"] = round(dom_bytes / dom_us / 1e3 / plain_read, 4)
 
-    extra = {}
+    extra, roofline_extra = {}, []
     if not args.no_extra:
-        extra = run_extra(torch, np, dev, lib, datagen, ops)
+        extra, roofline_extra = run_extra(env, traffic)
 
     cpu_baseline = None
     if not args.no_cpu_baseline:
@@ -243,29 +283,169 @@ def main():
             "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
             "timed_region_wall_ms": round(wall_ms, 3),
         },
+        "parity": parity,
+        "plain_read_1GiB_GB/s": plain_read,
         "per_shape": per_shape,
         "roofline": roofline,
+        "roofline_extra": roofline_extra,
         "cpu_baseline": cpu_baseline,
         "extra": extra,
     }
     print(json.dumps(out))
 
 
-def run_read_probe(torch, dev, lib, n_layers, per_shape, timed_graph):
+class Env:
+    """What the measuring functions share: modules, the device, the library and the timers."""
+
+    def __init__(self, torch, np, dev, lib, datagen, ops):
+        self.torch, self.np, self.dev, self.lib, self.datagen, self.ops = torch, np, dev, lib, datagen, ops
+
+    def dev_t(self, a):
+        return self.torch.from_numpy(self.np.ascontiguousarray(a)).to(self.dev)
+
+    def timed_graph(self, fn_list, reps):
+        """Capture fn_list (callables that enqueue launches) into one graph; return mean microseconds of
+        one replay over `reps` replays, measured with events on the launch stream."""
+        torch = self.torch
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for fn in fn_list:
+                fn()
+        g.replay()
+        torch.cuda.synchronize()
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            g.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1000.0 / reps
+
+    def time_us(self, fn, iters):
+        torch = self.torch
+        for _ in range(10):
+            fn()
+        torch.cuda.synchronize()
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(iters):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1000.0 / iters
+
+    def time_cold_us(self, make_fn, weight_sets):
+        """Launches walking device-side copies of the weights (more than the last-level cache holds), captured in
+        one graph: for the rows whose time is a memory time."""
+        torch = self.torch
+        fns = [make_fn(*w) for w in weight_sets]
+        fns[0]()
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for f in fns:
+                f()
+        # untimed replays first: after the host-side preparation of a row the first replays run 5-13 % slow
+        for _ in range(6):
+            g.replay()
+        torch.cuda.synchronize()
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(6):
+            g.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1000.0 / (6 * len(fns))
+
+    def copies_of(self, *tensors):
+        nbytes = sum(t.numel() * t.element_size() for t in tensors)
+        return [tensors] + [tuple(t.clone() for t in tensors) for _ in range(-(-COLD_FOOTPRINT_BYTES // nbytes))]
+
+    def workspace(self, nbytes):
+        return self.torch.empty(max(int(nbytes), 256), dtype=self.torch.uint8, device=self.dev)
+
+
+# ---- parity gate ----------------------------------------------------------------------------------------
+def parity_fail(name, detail):
+    sys.stderr.write(f"bench.py: PARITY FAILURE in {name}: {detail}; nothing was timed\n")
+    sys.exit(1)
+
+
+def check_w4a16(np, parity, name, y, ref, tol=W4A16_TOL):
+    rms = float(np.sqrt(np.mean(ref.astype(np.float64) ** 2)))
+    err = float(np.abs(y.astype(np.float32) - ref.astype(np.float32)).max())
+    if not (err <= tol * max(rms, 1e-6)):
+        parity_fail(name, f"max |y - oracle| = {err:.4g} > {tol} x RMS(oracle) = {tol * rms:.4g}")
+    parity[name] = {"max_err_over_rms": round(err / max(rms, 1e-30), 6), "tol": tol}
+
+
+def parity_extra(env, oracle, parity):
+    """The configurations of run_extra, each run once and compared with the oracle: the GEMMs on sampled output
+    columns (the oracle computes those columns from the same weight rows), W8A8 bit for bit, the MLP block on its
+    first token rows (rows are independent)."""
+    np, torch, ops, datagen = env.np, env.torch, env.ops, env.datagen
+    n = k = GEMM_NK
+    rng = np.random.default_rng(0)
+    cols = np.sort(rng.choice(n, 96, replace=False))
+    _, wq, s = datagen.w4a16_case(0, 1, n, k)
+    twq, ts = env.dev_t(wq), env.dev_t(s)
+    for m in GEMM_MS:
+        a = datagen.normal_f16(0, datagen.S_ACT, (m, k))
+        y = ops.w4a16_gemm(env.dev_t(a), twq, ts)
+        torch.cuda.synchronize()
+        ref = oracle.w4a16_gemm(a, wq[cols], s[cols], f32_out=True)
+        check_w4a16(np, parity, f"w4a16_gemm_N{n}_K{k}.M{m}", y.cpu().numpy()[:, cols], ref)
+    del twq, ts
+    for (sn, sk) in DECODE_SHAPES:
+        _, wq, s = datagen.w4a16_case(0, 1, sn, sk)
+        twq, ts = env.dev_t(wq), env.dev_t(s)
+        scols = np.sort(rng.choice(sn, 96, replace=False))
+        for m in SMALL_BATCHES:
+            a = datagen.normal_f16(0, datagen.S_ACT, (m, sk))
+            y = ops.w4a16_gemm(env.dev_t(a), twq, ts)
+            torch.cuda.synchronize()
+            ref = oracle.w4a16_gemm(a, wq[scols], s[scols], f32_out=True)
+            check_w4a16(np, parity, f"decode_sweep_M{m}.N{sn}_K{sk}", y.cpu().numpy()[:, scols], ref)
+        del twq, ts
+    _, _, w8, s_ch = datagen.w8a8_case(0, 1, n, k)
+    tw8, tsch = env.dev_t(w8), env.dev_t(s_ch)
+    cols8 = np.sort(rng.choice(n, 64, replace=False))
+    for m in W8A8_MS:
+        a8 = datagen.uniform_i8(0, datagen.S_A8, (m, k))
+        st = datagen.uniform_f32(0, datagen.S_STOK, (m,), 0.001, 0.01)
+        y = ops.w8a8_gemm(env.dev_t(a8), env.dev_t(st), tw8, tsch)
+        torch.cuda.synchronize()
+        acc = oracle.w8a8_acc(a8, w8[cols8])
+        ref = oracle.w8a8_epilogue(acc, st, s_ch[cols8])
+        name = f"w8a8_gemm_N{n}_K{k}.M{m}"
+        if not np.array_equal(y.cpu().numpy()[:, cols8].view(np.uint16), ref.view(np.uint16)):
+            parity_fail(name, "fp16 outputs differ from the oracle's (the bar is bit-exact)")
+        parity[name] = {"bit_exact_columns": int(len(cols8))}
+    del tw8, tsch
+    m, h, i = MLP_SHAPE
+    x, gamma, wgu, sgu, wd, sd = datagen.mlp_case(0, m, h, i)
+    out = ops.fused_mlp_w4a16(*[env.dev_t(t) for t in (x, gamma, wgu, sgu, wd, sd)])
+    torch.cuda.synchronize()
+    ref = oracle.fused_mlp_w4a16(x[:8].copy(), gamma, wgu, sgu, wd, sd)
+    check_w4a16(np, parity, f"fused_mlp_M{m}_{h}_{i}.rows0-7", out.cpu().numpy()[:8], ref)
+
+
+# ---- probes ---------------------------------------------------------------------------------------------
+def run_read_probe(env, probes, n_layers, per_shape):
     """What a launch costs that does nothing but read the same number of bytes once: plain 128-bit loads, one
     workgroup per CU, three depths of loads in flight (the best is kept as plain_read_us); the same bytes in the
     M <= 16 kernel's tile order; and in plain order but through LDS.  Timed exactly like the GEMV launches, over
     as many distinct buffers (nothing is found in the last-level cache)."""
-    import ctypes
-
-    fn = lib.nnf_internal_read_probe
-    fn.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_longlong, ctypes.c_int, ctypes.c_int]
-    fn.restype = ctypes.c_int
+    torch = env.torch
+    fn = probes.nnf_probe_read
     num_cu = torch.cuda.get_device_properties(0).multi_processor_count
     for entry in per_shape:
         nbytes = (w4a16_bytes(1, entry["N"], entry["K"]) + 15) // 16 * 16
         n_bufs = max(n_layers, -(-COLD_FOOTPRINT_BYTES // nbytes))
-        bufs = [torch.randint(0, 255, (nbytes,), dtype=torch.uint8, device=dev) for _ in range(n_bufs)]
+        bufs = [torch.randint(0, 255, (nbytes,), dtype=torch.uint8, device=env.dev) for _ in range(n_bufs)]
         best = None
         by_variant = []
         for variant in range(5):
@@ -273,12 +453,12 @@ def run_read_probe(torch, dev, lib, n_layers, per_shape, timed_graph):
                 def call():
                     st = fn(torch.cuda.current_stream().cuda_stream, buf.data_ptr(), nbytes, variant, num_cu)
                     if st != 0:
-                        raise RuntimeError(f"nnf_internal_read_probe failed: {st}")
+                        raise RuntimeError(f"nnf_probe_read failed: {st}")
                 return call
             fns = [make(b) for b in bufs]
             fns[0]()
             torch.cuda.synchronize()
-            us = timed_graph(fns, 4) / len(fns)
+            us = env.timed_graph(fns, 4) / len(fns)
             if variant < 3:
                 best = us if best is None else min(best, us)
             by_variant.append(round(us, 3))
@@ -290,8 +470,28 @@ def run_read_probe(torch, dev, lib, n_layers, per_shape, timed_graph):
         del bufs
 
 
-def run_gemm_probe(torch, dev, datagen, ops, m=4096, n=8192, k=8192, launches=12):
+def run_large_read_probe(env, probes):
+    """GB/s of one launch that reads 1 GiB once with plain 128-bit loads (the best of the three depths of loads in
+    flight): the rate this box's HBM gives a kernel that does nothing else, next to the published 8 TB/s."""
+    torch = env.torch
+    fn = probes.nnf_probe_read
+    num_cu = torch.cuda.get_device_properties(0).multi_processor_count
+    buf = torch.randint(0, 255, (PROBE_BYTES,), dtype=torch.uint8, device=env.dev)
+    best = None
+    for variant in range(3):
+        def call(variant=variant):
+            st = fn(torch.cuda.current_stream().cuda_stream, buf.data_ptr(), PROBE_BYTES, variant, num_cu)
+            if st != 0:
+                raise RuntimeError(f"nnf_probe_read failed: {st}")
+        us = env.time_us(call, 10)
+        best = us if best is None else min(best, us)
+    del buf
+    return round(PROBE_BYTES / best / 1e3, 1)
+
+
+def run_gemm_probe(env, m=4096, n=8192, k=8192, launches=12):
     """The two compute-bound GEMMs of the extra configurations on their own (what a counter run looks at)."""
+    torch, datagen, ops, dev = env.torch, env.datagen, env.ops, env.dev
     ws = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
 
     def timed(fn):
@@ -321,165 +521,197 @@ def run_gemm_probe(torch, dev, datagen, ops, m=4096, n=8192, k=8192, launches=12
             "w8a8_us": round(us8, 1), "w8a8_tops": round(ops_total / us8 / 1e6, 1)}
 
 
-def run_mfma_probe(torch, lib):
+def run_mfma_probe(env, probes):
     """MFMA-only loops (operands in registers, two wavefronts per SIMD, eight accumulators each): the rate the
     matrix cores sustain depends on the operand values, because the chip is power managed."""
-    import ctypes
-
-    fn = lib.nnf_internal_mfma_probe
-    fn.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_double),
-                   ctypes.POINTER(ctypes.c_double)]
-    fn.restype = ctypes.c_int
-    num_cu = torch.cuda.get_device_properties(0).multi_processor_count
+    fn = probes.nnf_probe_mfma
+    num_cu = env.torch.cuda.get_device_properties(0).multi_processor_count
     out = {"num_cu": num_cu, "unit": "Tera-op/s", "note": "published dense peaks: fp16 2500, int8 5000"}
     for kind, kname in ((0, "f16_32x32x16"), (1, "i8_32x32x32")):
         for mode, mname in ((0, "all_ones"), (1, "normal_or_uniform_random"), (2, "small_integers")):
             tops, mhz = ctypes.c_double(0.0), ctypes.c_double(0.0)
             st = fn(kind, mode, 60000, num_cu, ctypes.byref(tops), ctypes.byref(mhz))
             if st != 0:
-                raise RuntimeError(f"nnf_internal_mfma_probe failed: {st}")
+                raise RuntimeError(f"nnf_probe_mfma failed: {st}")
             out[f"{kname}.{mname}"] = {"tops": round(tops.value, 1), "shader_mhz": round(mhz.value)}
     return out
 
 
-def run_extra(torch, np, dev, lib, datagen, ops):
-    """The other benchmark configurations, a few iterations each (not part of `value`).  Rows with M <= 128 are
-    memory-bound: they are timed over copies of the weights that miss the last-level cache."""
-
-    def dev_t(a):
-        return torch.from_numpy(np.ascontiguousarray(a)).to(dev)
-
-    def time_us(fn, iters):
-        for _ in range(10):
-            fn()
-        torch.cuda.synchronize()
-        e0 = torch.cuda.Event(enable_timing=True)
-        e1 = torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(iters):
-            fn()
-        e1.record()
-        torch.cuda.synchronize()
-        return e0.elapsed_time(e1) * 1000.0 / iters
-
-    def time_cold_us(make_fn, weight_sets):
-        """Launches walking device-side copies of the weights (more than the last-level cache holds), captured in
-        one graph: for the rows whose time is a memory time."""
-        fns = [make_fn(*w) for w in weight_sets]
-        fns[0]()
-        torch.cuda.synchronize()
-        g = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(g):
-            for f in fns:
-                f()
-        # untimed replays first: after the host-side preparation of a row the first replays run 5-13 % slow
-        for _ in range(6):
-            g.replay()
-        torch.cuda.synchronize()
-        e0 = torch.cuda.Event(enable_timing=True)
-        e1 = torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(6):
-            g.replay()
-        e1.record()
-        torch.cuda.synchronize()
-        return e0.elapsed_time(e1) * 1000.0 / (6 * len(fns))
-
-    def copies_of(*tensors):
-        nbytes = sum(t.numel() * t.element_size() for t in tensors)
-        return [tensors] + [tuple(t.clone() for t in tensors) for _ in range(-(-COLD_FOOTPRINT_BYTES // nbytes))]
-
-    res = {}
-    # configs[2]: fp16 x int4 GEMM, N = K = 8192
-    n = k = 8192
+def extra_rows(env):
+    """The configurations beside the sweep as (row key, algorithmic bytes, operations, callable factory, weight
+    tensors): the factory takes (copies of) the weights and returns the callable that enqueues the row once."""
+    torch, datagen, ops, lib, dev = env.torch, env.datagen, env.ops, env.lib, env.dev
+    n = k = GEMM_NK
+    rows = []
     _, wq, s = datagen.w4a16_case(0, 1, n, k)
-    twq, ts = dev_t(wq), dev_t(s)
-    rows = []
-    for m in (16, 128, 1024, 4096):
-        a = dev_t(datagen.normal_f16(0, datagen.S_ACT, (m, k)))
+    twq, ts = env.dev_t(wq), env.dev_t(s)
+    for m in GEMM_MS:
+        a = env.dev_t(datagen.normal_f16(0, datagen.S_ACT, (m, k)))
         y = torch.empty((m, n), dtype=torch.float16, device=dev)
-        ws = torch.empty(max(lib.nnf_w4a16_gemm_workspace_bytes(m, n, k, GROUP), 256), dtype=torch.uint8, device=dev)
-        if m <= 128:
-            sets = copies_of(twq, ts)
-            us = time_cold_us(lambda w, sc: (lambda: ops.w4a16_gemm(a, w, sc, out=y, workspace=ws)), sets)
-            del sets
-        else:
-            us = time_us(lambda: ops.w4a16_gemm(a, twq, ts, out=y, workspace=ws), 20)
-        fl = 2.0 * m * n * k
-        rows.append({"M": m, "us": round(us, 2), "TFLOP/s": round(fl / us / 1e6, 1),
-                     "frac_mfma_f16": round(fl / us / 1e6 / MFMA_F16_PEAK_TFLOPS, 4),
-                     "GB/s": round(w4a16_bytes(m, n, k) / us / 1e3, 1)})
-    res["w4a16_gemm_N8192_K8192"] = rows
-    del twq, ts
-    # the decode sweep's shapes with a handful of rows (batched decode; not one of the benchmark's configurations):
-    # cold weights, the time of the whole sweep per batch size
-    rows = []
-    shapes = [(12288, 4096), (4096, 4096), (22016, 4096), (4096, 11008)]
-    weights = []
-    for (sn, sk) in shapes:
-        _, wq, s = datagen.w4a16_case(0, 1, sn, sk)
-        weights.append((dev_t(wq), dev_t(s)))
-    for m in (2, 4, 8, 16):
-        total_us, total_bytes = 0.0, 0
-        for (sn, sk), (twq, ts) in zip(shapes, weights):
-            a = dev_t(datagen.normal_f16(0, datagen.S_ACT, (m, sk)))
-            y = torch.empty((m, sn), dtype=torch.float16, device=dev)
-            ws = torch.empty(max(lib.nnf_w4a16_gemm_workspace_bytes(m, sn, sk, GROUP), 256), dtype=torch.uint8, device=dev)
-            sets = copies_of(twq, ts)
-            total_us += time_cold_us(lambda w, sc: (lambda: ops.w4a16_gemm(a, w, sc, out=y, workspace=ws)), sets)
-            total_bytes += w4a16_bytes(m, sn, sk)
-            del sets
-        rows.append({"M": m, "us_per_sweep": round(total_us, 2), "GB/s": round(total_bytes / total_us / 1e3, 1)})
-    res["w4a16_decode_sweep_small_batches"] = rows
-    del weights
-    # configs[3]: W8A8, N = K = 8192
+        ws = env.workspace(lib.nnf_w4a16_gemm_workspace_bytes(m, n, k, GROUP))
+        rows.append({"key": f"w4a16_gemm_N{n}_K{k}.M{m}", "group": f"w4a16_gemm_N{n}_K{k}", "M": m,
+                     "bytes": w4a16_bytes(m, n, k), "ops": 2.0 * m * n * k, "int8": False, "weights": (twq, ts),
+                     "make": (lambda w, sc, a=a, y=y, ws=ws: (lambda: ops.w4a16_gemm(a, w, sc, out=y, workspace=ws)))})
     _, _, w8, s_ch = datagen.w8a8_case(0, 1, n, k)
-    tw8, tsch = dev_t(w8), dev_t(s_ch)
-    rows = []
-    for m in (1, 32, 512, 4096):
-        a8 = dev_t(datagen.uniform_i8(0, datagen.S_A8, (m, k)))
-        st = dev_t(datagen.uniform_f32(0, datagen.S_STOK, (m,), 0.001, 0.01))
+    tw8, tsch = env.dev_t(w8), env.dev_t(s_ch)
+    for m in W8A8_MS:
+        a8 = env.dev_t(datagen.uniform_i8(0, datagen.S_A8, (m, k)))
+        st = env.dev_t(datagen.uniform_f32(0, datagen.S_STOK, (m,), 0.001, 0.01))
         y = torch.empty((m, n), dtype=torch.float16, device=dev)
-        ws = torch.empty(max(lib.nnf_w8a8_gemm_workspace_bytes(m, n, k), 256), dtype=torch.uint8, device=dev)
-        if m <= 128:
-            sets = copies_of(tw8)
-            us = time_cold_us(lambda w: (lambda: ops.w8a8_gemm(a8, st, w, tsch, out=y, workspace=ws)), sets)
+        ws = env.workspace(lib.nnf_w8a8_gemm_workspace_bytes(m, n, k))
+        rows.append({"key": f"w8a8_gemm_N{n}_K{k}.M{m}", "group": f"w8a8_gemm_N{n}_K{k}", "M": m,
+                     "bytes": w8a8_bytes(m, n, k), "ops": 2.0 * m * n * k, "int8": True, "weights": (tw8,),
+                     "make": (lambda w, a8=a8, st=st, y=y, ws=ws: (lambda: ops.w8a8_gemm(a8, st, w, tsch, out=y, workspace=ws)))})
+    m, h, i = MLP_SHAPE
+    tens = [env.dev_t(t) for t in datagen.mlp_case(0, m, h, i)]
+    out = torch.empty((m, h), dtype=torch.float16, device=dev)
+    wsm = env.workspace(lib.nnf_fused_mlp_w4a16_workspace_bytes(m, h, i, GROUP))
+    x, gamma, wgu, sgu, wd, sd = tens
+    rows.append({"key": f"fused_mlp_M{m}_{h}_{i}", "group": None, "M": m, "bytes": mlp_bytes(m, h, i),
+                 "ops": 2.0 * m * (2 * i) * h + 2.0 * m * h * i, "int8": False, "weights": (wgu, sgu, wd, sd),
+                 "make": (lambda a, b, c, d: (lambda: ops.fused_mlp_w4a16(x, gamma, a, b, c, d, out=out, workspace=wsm)))})
+    return rows
+
+
+def small_batch_rows(env):
+    """The decode sweep's shapes with a handful of rows (batched decode), per batch size: a list of
+    (bytes, factory, weights) per shape."""
+    torch, datagen, ops, lib, dev = env.torch, env.datagen, env.ops, env.lib, env.dev
+    weights = []
+    for (sn, sk) in DECODE_SHAPES:
+        _, wq, s = datagen.w4a16_case(0, 1, sn, sk)
+        weights.append((env.dev_t(wq), env.dev_t(s)))
+    out = []
+    for m in SMALL_BATCHES:
+        shapes = []
+        for (sn, sk), (twq, ts) in zip(DECODE_SHAPES, weights):
+            a = env.dev_t(datagen.normal_f16(0, datagen.S_ACT, (m, sk)))
+            y = torch.empty((m, sn), dtype=torch.float16, device=dev)
+            ws = env.workspace(lib.nnf_w4a16_gemm_workspace_bytes(m, sn, sk, GROUP))
+            shapes.append({"key": f"decode_sweep_M{m}.N{sn}_K{sk}", "bytes": w4a16_bytes(m, sn, sk), "weights": (twq, ts),
+                           "make": (lambda w, sc, a=a, y=y, ws=ws: (lambda: ops.w4a16_gemm(a, w, sc, out=y, workspace=ws)))})
+        out.append((m, shapes))
+    return out
+
+
+def run_extra(env, traffic):
+    """The other benchmark configurations, a few iterations each (not part of `value`).  Rows with M <= 128 are
+    memory-bound: they are timed over copies of the weights that miss the last-level cache.  Returns the plain
+    timings and, per row, the roofline figures: the ceiling is the matrix cores' when the row's operations per
+    algorithmic byte exceed peak operations / peak bandwidth, else HBM's."""
+    torch = env.torch
+    res, roofs = {}, []
+    for row in extra_rows(env):
+        if row["M"] <= 128:
+            sets = env.copies_of(*row["weights"])
+            us = env.time_cold_us(row["make"], sets)
             del sets
         else:
-            us = time_us(lambda: ops.w8a8_gemm(a8, st, tw8, tsch, out=y, workspace=ws), 20)
-        op = 2.0 * m * n * k
-        rows.append({"M": m, "us": round(us, 2), "TOP/s": round(op / us / 1e6, 1),
-                     "frac_mfma_i8": round(op / us / 1e6 / MFMA_I8_PEAK_TOPS, 4),
-                     "GB/s": round(w8a8_bytes(m, n, k) / us / 1e3, 1)})
-    res["w8a8_gemm_N8192_K8192"] = rows
-    del tw8, tsch
-    # configs[4]: fused MLP block, M = 256
-    m, h, i = 256, 4096, 11008
-    tens = [dev_t(t) for t in datagen.mlp_case(0, m, h, i)]
-    out = torch.empty((m, h), dtype=torch.float16, device=dev)
-    wsz = lib.nnf_fused_mlp_w4a16_workspace_bytes(m, h, i, GROUP)
-    wsm = torch.empty(wsz, dtype=torch.uint8, device=dev)
-    us = time_us(lambda: ops.fused_mlp_w4a16(*tens, out=out, workspace=wsm), 20)
-    fl = 2.0 * m * (2 * i) * h + 2.0 * m * h * i
-    res["fused_mlp_M256_4096_11008"] = {"us": round(us, 2), "TFLOP/s": round(fl / us / 1e6, 1),
-                                        "frac_mfma_f16": round(fl / us / 1e6 / MFMA_F16_PEAK_TFLOPS, 4)}
-    del tens, out, wsm
+            us = env.time_us(row["make"](*row["weights"]), 20)
+        peak_ops = MFMA_I8_PEAK_TOPS if row["int8"] else MFMA_F16_PEAK_TFLOPS
+        rate = row["ops"] / us / 1e6  # Tera-op/s
+        gbs = row["bytes"] / us / 1e3
+        unit_ops = "TOP/s" if row["int8"] else "TFLOP/s"
+        entry = {"M": row["M"], "us": round(us, 2), unit_ops: round(rate, 1),
+                 ("frac_mfma_i8" if row["int8"] else "frac_mfma_f16"): round(rate / peak_ops, 4), "GB/s": round(gbs, 1)}
+        if row["group"]:
+            res.setdefault(row["group"], []).append(entry)
+        else:
+            entry.pop("M")
+            res[row["key"]] = entry
+        mfma_bound = row["ops"] / row["bytes"] > peak_ops * 1e12 / (HBM_PEAK_GBS * 1e9)
+        roofs.append({"row": row["key"], "kernel": DOMINANT_KERNEL.get(row["key"]),
+                      "bound": "mfma" if mfma_bound else "hbm",
+                      "achieved": round(rate if mfma_bound else gbs, 1),
+                      "peak": peak_ops if mfma_bound else HBM_PEAK_GBS,
+                      "unit": unit_ops if mfma_bound else "GB/s",
+                      "frac": round(rate / peak_ops if mfma_bound else gbs / HBM_PEAK_GBS, 4),
+                      "traffic": traffic.get(row["key"]), "algorithmic_bytes": int(row["bytes"]),
+                      "us_per_launch": round(us, 2)})
+    sweep = []
+    for m, shapes in small_batch_rows(env):
+        total_us, total_bytes, total_traffic = 0.0, 0, 0
+        for sh in shapes:
+            sets = env.copies_of(*sh["weights"])
+            total_us += env.time_cold_us(sh["make"], sets)
+            total_bytes += sh["bytes"]
+            t = traffic.get(sh["key"])
+            total_traffic = None if (t is None or total_traffic is None) else total_traffic + t
+            del sets
+        sweep.append({"M": m, "us_per_sweep": round(total_us, 2), "GB/s": round(total_bytes / total_us / 1e3, 1)})
+        roofs.append({"row": f"decode_sweep_M{m}", "kernel": "nnf::w4a16_mrows_kernel / w4a16_mrows_any_kernel (+ splitk_reduce_kernel at K=11008)",
+                      "bound": "hbm", "achieved": round(total_bytes / total_us / 1e3, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                      "frac": round(total_bytes / total_us / 1e3 / HBM_PEAK_GBS, 4), "traffic": total_traffic,
+                      "algorithmic_bytes": int(total_bytes), "us_per_launch": round(total_us, 2)})
+    res["w4a16_decode_sweep_small_batches"] = sweep
     # For scale only: the vendor library's unquantized GEMMs on the same box and value distributions (fp16 weights,
     # four times the bytes, no unpacking; int8 x int8 -> int32 without the scaling epilogue), M = 4096, N = K = 8192.
     try:
         m, n, k = 4096, 8192, 8192
+        dev = env.dev
         a = torch.randn(m, k, device=dev, dtype=torch.float16)
         w = torch.randn(n, k, device=dev, dtype=torch.float16)
         y = torch.empty(m, n, device=dev, dtype=torch.float16)
-        us16 = time_us(lambda: torch.matmul(a, w.t(), out=y), 20)
+        us16 = env.time_us(lambda: torch.matmul(a, w.t(), out=y), 20)
         a8 = torch.randint(-127, 128, (m, k), device=dev, dtype=torch.int8)
         w8 = torch.randint(-127, 128, (n, k), device=dev, dtype=torch.int8)
-        us8 = time_us(lambda: torch._int_mm(a8, w8.t()), 20)
+        us8 = env.time_us(lambda: torch._int_mm(a8, w8.t()), 20)
         res["vendor_library_for_scale_M4096"] = {"fp16_matmul_us": round(us16, 1), "fp16_TFLOP/s": round(2.0 * m * n * k / us16 / 1e6, 1),
                                                  "int8_mm_us": round(us8, 1), "int8_TOP/s": round(2.0 * m * n * k / us8 / 1e6, 1)}
     except Exception as e:  # a yardstick, not part of the benchmark
         res["vendor_library_for_scale_M4096"] = {"error": str(e)[:200]}
-    return res
+    return res, roofs
+
+
+def run_pmc_probe(env, probes, layers, step, n_layers):
+    """For FETCH_SIZE / WRITE_SIZE runs.  Calibration: a device-to-device copy that reads and writes exactly
+    PROBE_BYTES, larger than the last-level cache.  Then every configuration row, launched eagerly a few times, each
+    behind one marker launch (the read probe on 16 x (row index + 1) bytes) by which a reader of the counter file
+    tells the rows apart.  Prints the rows in launch order with their algorithmic bytes."""
+    torch = env.torch
+    num_cu = torch.cuda.get_device_properties(0).multi_processor_count
+    src = torch.empty(PROBE_BYTES // 4, dtype=torch.float32, device=env.dev).normal_()
+    dst = torch.empty_like(src)
+    marker_buf = torch.zeros(4096, dtype=torch.uint8, device=env.dev)
+    torch.cuda.synchronize()
+    for _ in range(4):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+    del src, dst
+    order = []
+
+    def marker():
+        st = probes.nnf_probe_read(torch.cuda.current_stream().cuda_stream, marker_buf.data_ptr(), 16 * (len(order) + 1), 0, num_cu)
+        if st != 0:
+            raise RuntimeError(f"nnf_probe_read failed: {st}")
+
+    # the sweep, shape by shape over every resident layer
+    for si, (n, k) in enumerate(DECODE_SHAPES):
+        marker()
+        for layer in layers:
+            a, wq, s, y = layer[si]
+            st = env.lib.nnf_w4a16_gemm(torch.cuda.current_stream().cuda_stream, a.data_ptr(), wq.data_ptr(), s.data_ptr(),
+                                        y.data_ptr(), 1, n, k, GROUP, 8, None, 0)
+            if st != 0:
+                raise RuntimeError(f"nnf_w4a16_gemm failed: {st}")
+        order.append({"row": f"decode_sweep.N{n}_K{k}", "launches": n_layers, "algorithmic_bytes": w4a16_bytes(1, n, k)})
+    torch.cuda.synchronize()
+    for m, shapes in small_batch_rows(env):
+        for sh in shapes:
+            marker()
+            fn = sh["make"](*sh["weights"])
+            for _ in range(3):
+                fn()
+            order.append({"row": sh["key"], "launches": 3, "algorithmic_bytes": sh["bytes"]})
+        torch.cuda.synchronize()
+    for row in extra_rows(env):
+        marker()
+        fn = row["make"](*row["weights"])
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        order.append({"row": row["key"], "launches": 3, "algorithmic_bytes": int(row["bytes"])})
+    print(json.dumps({"pmc_probe": {"calibration_copy_bytes": PROBE_BYTES, "calibration_copies": 4, "rows": order}}), flush=True)
 
 
 def run_cpu_baseline(np, host_layer0, step_bytes):

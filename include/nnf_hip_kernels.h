@@ -62,8 +62,11 @@ const char* nnf_status_string(int status);
 /* ---------------------------------------------------------------------------------------------
  * fp16 x int4 (group-scaled) GEMM / GEMV:  Y[M,N] = A[M,K] . ((Wq - zp) * scales)^T
  * Replaces the cublasHgemm / cublasSgemm call of cuda::Dot (cuda_gpu/kernels/dot.cpp:128-205,
- * :271-363) for a weight-quantized Dot node with transpose_B = true.  M <= 16 takes the
- * bandwidth-bound split-K GEMV path, larger M the MFMA path.
+ * :271-363) for a weight-quantized Dot node with transpose_B = true.  By shape: M = 1 the row-streaming
+ * GEMV kernel; 2 <= M <= 32 (40 for long K) the row-streaming MFMA kernel, over ranges of K (partial sums in
+ * `workspace`, then a reduction pass) where the activations exceed one workgroup's registers; other M <= 16
+ * shapes the MFMA GEMV kernel over K ranges; everything else the MFMA tile GEMM, whose work is split evenly
+ * over the CUs (tiles shared by several workgroups are summed through `workspace` by a second launch).
  * ------------------------------------------------------------------------------------------- */
 size_t nnf_w4a16_gemm_workspace_bytes(int M, int N, int K, int group);
 
@@ -94,18 +97,34 @@ enum nnf_w4a16_variant
 {
     NNF_W4A16_AUTO = 0,
     NNF_W4A16_GEMV_VALU = 1, /* M <= 16: v_dot2 GEMV, exact (q - zp) unpacking; cross-check implementation */
-    NNF_W4A16_GEMV_MFMA = 2, /* M <= 16: MFMA 16x16x32 weight-streaming kernel (activations held per workgroup) */
+    NNF_W4A16_GEMV_MFMA = 2, /* M <= 16: MFMA 16x16x32 weight-streaming kernel (activations held per workgroup; over ranges
+                                of K with partial sums in the workspace when they exceed its LDS) */
     NNF_W4A16_GEMM_MFMA = 3, /* any M: MFMA 32x32x16 tile GEMM (may split K: workspace) */
     NNF_W4A16_GEMV_ROWS = 4  /* row-streaming kernels, one workgroup per CU: M = 1 (K a multiple of 256, 1024 .. 16384),
-                                M = 2 .. 16 on MFMA (K a multiple of 256, 1024 .. 8192, N >= 16), M = 17 .. 32 up to K = 4096 */
+                                M = 2 .. 16 on MFMA (K a multiple of 256, 1024 .. 8192, N >= 16), M = 17 .. 32 up to K = 4096;
+                                longer K (to 65536; M = 33 .. 40: 2048 < K <= 4096) over ranges of K with partial sums
+                                in the workspace */
 };
+/* What else a candidate may fix about the tile GEMM (variant NNF_*_GEMM_MFMA; ignored by the other variants).
+ * Passed per call: the library keeps no dispatch state, calls with different plans may run concurrently.
+ * NULL, or a field that is 0: the library's own choice for the shape. */
+typedef struct nnf_plan
+{
+    int tile_rows; /* rows of an output tile: 256, 128, 64 (fp16 x int4 also 32); tiles are 256 columns wide
+                      (W8A8 128-row tiles: 128 columns) */
+    int k_parts;   /* fp16 x int4: workgroups that share one output tile, each a contiguous part of K, summed by a
+                      second launch (the grid is tiles x k_parts, work split evenly); W8A8: ranges of K, int32
+                      partial sums added exactly by a reduction pass */
+} nnf_plan;
 /* 1 when the variant can serve the shape (decided on the host, for a 256-CU device), else 0. */
 int nnf_w4a16_variant_supported(int M, int N, int K, int group, int variant);
-size_t nnf_w4a16_gemm_variant_workspace_bytes(int M, int N, int K, int group, int variant);
-/* As nnf_w4a16_gemm through the given variant; NNF_ERR_UNSUPPORTED_SHAPE when it cannot serve the shape. */
+/* Upper bound for a 256-CU device; the call itself checks what its launch writes on the device at hand. */
+size_t nnf_w4a16_gemm_variant_workspace_bytes(int M, int N, int K, int group, int variant, const nnf_plan* plan);
+/* As nnf_w4a16_gemm through the given variant; NNF_ERR_UNSUPPORTED_SHAPE when it cannot serve the shape,
+ * NNF_ERR_INVALID_ARGUMENT for a variant or plan value outside the ones listed. */
 int nnf_w4a16_gemm_variant(nnf_stream_t stream,
                            const void* A, const void* Wq, const void* scales, void* Y,
-                           int M, int N, int K, int group, int zp, int variant,
+                           int M, int N, int K, int group, int zp, int variant, const nnf_plan* plan,
                            void* workspace, size_t workspace_bytes);
 
 /* Epilogue / prologue selectors for nnf_w4a16_gemm_fused. */
@@ -138,6 +157,18 @@ int nnf_w4a16_gemm_fused(nnf_stream_t stream,
                          const void* bias, const void* residual, int act,
                          void* workspace, size_t workspace_bytes);
 
+/* nnf_w4a16_gemm_fused as a selectable candidate: any variant but NNF_W4A16_GEMV_VALU (which has no fused form:
+ * NNF_ERR_UNSUPPORTED_SHAPE, as for a variant that cannot serve the shape); `plan` for the tile GEMM.
+ * A workspace of nnf_w4a16_gemm_fused_workspace_bytes + nnf_w4a16_gemm_variant_workspace_bytes(.., plan) of the
+ * weight rows (2N with NNF_ACT_SILU_GATE) always suffices. */
+int nnf_w4a16_gemm_fused_variant(nnf_stream_t stream,
+                                 const void* A, const void* Wq, const void* scales, void* Y,
+                                 int M, int N, int K, int group, int zp,
+                                 const void* rms_gamma, float rms_eps,
+                                 const void* bias, const void* residual, int act,
+                                 int variant, const nnf_plan* plan,
+                                 void* workspace, size_t workspace_bytes);
+
 /* ---------------------------------------------------------------------------------------------
  * W8A8: int8 x int8 -> int32 on the int8 MFMA, then the per-token / per-channel dequantisation.
  * The reference has no emitter for this; the nearest routine in its tree is MLAS's u8 x s8
@@ -156,6 +187,22 @@ int nnf_w8a8_gemm_acc(nnf_stream_t stream,
                       const void* A, const void* W, void* acc,
                       int M, int N, int K,
                       void* workspace, size_t workspace_bytes);
+
+/* The kernels behind nnf_w8a8_gemm as selectable variants (see nnf_w4a16_variant); `plan` as above. */
+enum nnf_w8a8_variant
+{
+    NNF_W8A8_AUTO = 0,
+    NNF_W8A8_GEMV_MFMA = 1, /* M <= 16: int8 MFMA kernel over ranges of K inside one workgroup */
+    NNF_W8A8_GEMM_MFMA = 2, /* any M: int8 MFMA 32x32x32 tile GEMM (may split K: workspace) */
+    NNF_W8A8_GEMV_ROWS = 3  /* row-streaming kernels: M = 1; M = 2 .. 32 on MFMA (K a multiple of 256, 1024 .. 16384) */
+};
+int nnf_w8a8_variant_supported(int M, int N, int K, int variant);
+size_t nnf_w8a8_gemm_variant_workspace_bytes(int M, int N, int K, int variant, const nnf_plan* plan);
+/* Exactly one of Y (with s_tok, s_ch) and acc is non-NULL: the fp16 result or the raw int32 accumulators. */
+int nnf_w8a8_gemm_variant(nnf_stream_t stream,
+                          const void* A, const void* s_tok, const void* W, const void* s_ch, void* Y, void* acc,
+                          int M, int N, int K, int variant, const nnf_plan* plan,
+                          void* workspace, size_t workspace_bytes);
 
 /* ---------------------------------------------------------------------------------------------
  * Fused Llama-style MLP block (one emitted function for the sub-graph

@@ -36,10 +36,15 @@ KERNEL_ABI = {
     "nnf_w4a16_gemm": (_c_int, [_c_vp] * 5 + [_c_int] * 5 + [_c_vp, _c_sz]),
     "nnf_w4a16_gemm_static_scratch": (_c_int, [_c_vp] * 5 + [_c_int] * 5),
     "nnf_w4a16_variant_supported": (_c_int, [_c_int] * 5),
-    "nnf_w4a16_gemm_variant_workspace_bytes": (_c_sz, [_c_int] * 5),
-    "nnf_w4a16_gemm_variant": (_c_int, [_c_vp] * 5 + [_c_int] * 6 + [_c_vp, _c_sz]),
+    "nnf_w4a16_gemm_variant_workspace_bytes": (_c_sz, [_c_int] * 5 + [_c_vp]),
+    "nnf_w4a16_gemm_variant": (_c_int, [_c_vp] * 5 + [_c_int] * 6 + [_c_vp, _c_vp, _c_sz]),
     "nnf_w4a16_gemm_fused_workspace_bytes": (_c_sz, [_c_int] * 5),
     "nnf_w4a16_gemm_fused": (_c_int, [_c_vp] * 5 + [_c_int] * 5 + [_c_vp, _c_f, _c_vp, _c_vp, _c_int, _c_vp, _c_sz]),
+    "nnf_w4a16_gemm_fused_variant": (_c_int, [_c_vp] * 5 + [_c_int] * 5 + [_c_vp, _c_f, _c_vp, _c_vp, _c_int, _c_int, _c_vp,
+                                              _c_vp, _c_sz]),
+    "nnf_w8a8_variant_supported": (_c_int, [_c_int] * 4),
+    "nnf_w8a8_gemm_variant_workspace_bytes": (_c_sz, [_c_int] * 4 + [_c_vp]),
+    "nnf_w8a8_gemm_variant": (_c_int, [_c_vp] * 7 + [_c_int] * 4 + [_c_vp, _c_vp, _c_sz]),
     "nnf_w8a8_gemm_workspace_bytes": (_c_sz, [_c_int] * 3),
     "nnf_w8a8_gemm": (_c_int, [_c_vp] * 6 + [_c_int] * 3 + [_c_vp, _c_sz]),
     "nnf_w8a8_gemm_acc": (_c_int, [_c_vp] * 4 + [_c_int] * 3 + [_c_vp, _c_sz]),

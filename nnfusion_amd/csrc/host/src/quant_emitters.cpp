@@ -147,12 +147,17 @@ namespace nnfusion
                     size_t ws_bytes = 0;
                     if (VARIANT == 3)
                         ws_bytes = nnf::workspace::plan_w4a16_sk((int)M, (int)N, (int)K, false, nnf::workspace::PLAN_CUS).bytes();
+                    // the GEMV kernels over ranges of K (activations beyond one workgroup's LDS / registers): fp32 partial sums
+                    if (VARIANT == 2 && !nnf::workspace::w4a16_skinny_fits((int)M, (int)N, (int)K))
+                        ws_bytes = nnf::workspace::skinny_split_bytes((int)M, (int)N, (int)K);
+                    if (VARIANT == 4 && M > 1 && !nnf::workspace::w4a16_mrows_fits((int)M, (int)N, (int)K, nnf::workspace::PLAN_CUS))
+                        ws_bytes = nnf::workspace::mrows_split_bytes((int)M, (int)N, (int)K);
                     std::string ws = "nullptr";
                     if (ws_bytes > 0)
                         ws = allocate_tensor(Shape{ws_bytes}, element::character)->get_name();
                     LanguageUnit_p lu(new LanguageUnit(get_function_name()));
                     *lu << "NNF_HIP_CHECK(nnf_w4a16_gemm_variant(stream, input0, input1, input2, output0, " << M << ", " << N
-                        << ", " << K << ", " << group << ", " << zp << ", " << variant_enum() << ", " << ws << ", "
+                        << ", " << K << ", " << group << ", " << zp << ", " << variant_enum() << ", nullptr, " << ws << ", "
                         << ws_bytes << "));\n";
                     return lu;
                 }

@@ -3,6 +3,7 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+#include <atomic>
 #include <stddef.h>
 #include <stdint.h>
 
@@ -10,6 +11,37 @@ namespace nnf
 {
     // largest dynamic LDS a workgroup may ask for on gfx950 (160 KiB per CU)
     constexpr size_t MAX_LDS_BYTES = 160 * 1024;
+
+    // Lifts a kernel's dynamic-LDS limit to `bytes`, once per (kernel, device): `granted` is a static of the calling
+    // template instantiation (one per kernel).  Racing first calls at worst set the attribute twice.
+    struct LdsGrant
+    {
+        std::atomic<int> bytes[64] = {};
+    };
+    inline hipError_t allow_dynamic_lds(const void* kernel, LdsGrant& granted, int bytes)
+    {
+        int dev = 0;
+        hipError_t e = hipGetDevice(&dev);
+        if (e != hipSuccess)
+            return e;
+        const bool cached = dev >= 0 && dev < 64;
+        if (cached && granted.bytes[dev].load(std::memory_order_relaxed) >= bytes)
+            return hipSuccess;
+        e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+        if (e == hipSuccess && cached)
+            granted.bytes[dev].store(bytes, std::memory_order_relaxed);
+        return e;
+    }
+
+    // What a call fixes about its launch (all zero: the library's own choice by shape).  Filled from the variant and
+    // plan arguments of the C ABI and passed down by value: the library keeps no dispatch state between calls.
+    struct LaunchChoice
+    {
+        int path = 0;      // the nnf_w4a16_variant / nnf_w8a8_variant values: 1 VALU GEMV, 2 MFMA GEMV over K ranges,
+                           // 3 tile GEMM, 4 row-streaming kernels
+        int tile_rows = 0; // tile GEMM: rows of an output tile (256, 128, 64; fp16 x int4 also 32)
+        int k_parts = 0;   // tile GEMM: workgroups that share an output tile (fp16 x int4) / ranges of K (W8A8)
+    };
 
     hipError_t launch_w4a16_gemv(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y,
                                  int M, int N, int K, int zp, int num_cu);
@@ -35,7 +67,6 @@ namespace nnf
                                    int N, int K, int zp, int num_cu);
     // true when one workgroup can hold the activations (M <= 16 rows of K) in LDS
     bool w4a16_skinny_supported(int M, int N, int K);
-    int& skinny_direct_min_rows(); // experiments: see w4a16_skinny.hip
 
     // M <= 16 with activations too large for LDS: the same kernel over `ksplits` ranges of K, fp32 partial sums
     // [ksplits][M][N] (to be added by the GEMM's reduction pass); w4a16_skinny_ksplits returns 0 when not applicable
@@ -47,19 +78,32 @@ namespace nnf
     // rms_ws: nnf::workspace::rms_rows(M, K) bytes, needed when rms_gamma != nullptr;
     // partial_ws: nnf::workspace::gemm_partial_bytes(...) for the plan of the shape (may be 0 bytes).
     // M <= 16 shapes that the GEMV kernel can serve go through it (plus an element-wise epilogue kernel),
-    // unless gemm_only asks for the MFMA GEMM tiles whatever M is.
+    // unless choice.path asks for the MFMA GEMM tiles whatever M is.
     hipError_t launch_w4a16_gemm(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M,
                                  int N, int K, int zp, const void* rms_gamma, float rms_eps, const void* bias,
                                  const void* residual, int act, void* rms_ws, void* partial_ws, int num_cu,
-                                 bool gemm_only = false);
+                                 const LaunchChoice& choice = LaunchChoice());
+    // bytes launch_w4a16_gemm writes at partial_ws for this call (0: it needs none)
+    // whether the kernel family `choice.path` names (0, 2, 3, 4) serves the product of M rows with N outputs (act 1: 2N
+    // weight rows)
+    bool w4a16_path_supported(int M, int N, int K, int act, int num_cu, int path);
+    // (in_place_residual: the residual is the output buffer itself)
+    size_t w4a16_gemm_partial_bytes(int M, int N, int K, int act, bool in_place_residual, int num_cu,
+                                    const LaunchChoice& choice = LaunchChoice());
 
     // W8A8: acc != nullptr writes the raw int32 accumulators, otherwise Y = fp16(acc * s_tok * s_ch).
     // partial_ws: nnf::workspace::w8a8_gemm(M, N, K) bytes (0 for the M <= 16 kernel)
     hipError_t launch_w8a8(hipStream_t stream, const void* A, const void* s_tok, const void* W, const void* s_ch,
-                           void* Y, void* acc, int M, int N, int K, int num_cu, void* partial_ws);
+                           void* Y, void* acc, int M, int N, int K, int num_cu, void* partial_ws,
+                           const LaunchChoice& choice = LaunchChoice());
+    // bytes launch_w8a8 writes at partial_ws for this call (0: the kernel it picks needs none)
+    size_t w8a8_partial_bytes(int M, int N, int K, int num_cu, const LaunchChoice& choice = LaunchChoice());
+    // whether the kernel family `path` names can serve the shape
+    bool w8a8_path_supported(int M, int N, int K, int num_cu, int path);
     // the MFMA GEMM behind launch_w8a8 (any M)
     hipError_t launch_w8a8_gemm(hipStream_t stream, const void* A, const void* s_tok, const void* W, const void* s_ch,
-                                void* Y, void* acc, int M, int N, int K, void* partial_ws);
+                                void* Y, void* acc, int M, int N, int K, void* partial_ws,
+                                const LaunchChoice& choice = LaunchChoice());
     bool w8a8_skinny_supported(int M, int K);
     // one activation row (M = 1): the row-streaming kernel; acc != nullptr writes the raw int32 sums
     hipError_t launch_w8a8_gemv_rows(hipStream_t stream, const void* A, const void* s_tok, const void* W, const void* s_ch,
@@ -71,15 +115,4 @@ namespace nnf
     bool w8a8_mrows_supported(int M, int N, int K, int num_cu);
     bool w8a8_mrows_preferred(int M, int N, int K, int num_cu); // where the library picks it without being told
 
-    // Tuning knobs for experiments (not part of the public ABI): 0 = automatic.
-    struct Tuning
-    {
-        int force_path = 0;  // 1 = VALU GEMV, 2 = MFMA skinny, 3 = MFMA GEMM, 4 = row-streaming GEMV (M = 1),
-                             // 5 = row-streaming MFMA kernel (2 <= M <= 16) where it applies
-        int skinny_cps = 0;  // chunks (groups of 128) per wavefront
-        int skinny_wg_per_cu = 0;
-        int gemm_tile = 0;   // 1 + nnf::workspace::GemmTile
-        int gemm_splits = 0; // K ranges of the mid / small tile kernels
-    };
-    extern Tuning g_tuning;
 } // namespace nnf

@@ -1,4 +1,4 @@
-// Measurement probes (not part of the public ABI): how fast the matrix cores run on their own --
+// Measurement probes of bench.py, built into libnnf_bench_probes.so (not part of the product library): how fast the matrix cores run on their own --
 // no memory traffic at all -- as a function of the operand VALUES.  The chip is power managed: the
 // same MFMA loop is clocked lower when the operand bits toggle more, so the attainable MFMA rate of a
 // GEMM depends on its data.  bench.py --mfma-probe prints the figures.
@@ -244,7 +244,7 @@ namespace nnf
 // 32, 64 or 128 KiB in flight per CU; variant 3 reads the whole 32 KiB tiles of it in the skinny
 // kernel's order, variant 4 in plain order but through LDS (global_load_lds).  Returns a hipError_t.  May be captured into a graph after one
 // eager call.
-extern "C" int nnf_internal_read_probe(void* stream, const void* src, long long bytes, int variant, int num_cu)
+extern "C" int nnf_probe_read(void* stream, const void* src, long long bytes, int variant, int num_cu)
 {
     using namespace nnf;
     static uint32_t* sink = nullptr;
@@ -277,7 +277,7 @@ extern "C" int nnf_internal_read_probe(void* stream, const void* src, long long 
 // Runs `iters` rounds of 8 MFMAs per wavefront on one workgroup of 8 wavefronts per CU and returns the
 // rate in tera-operations per second through *tops (fp16: 32x32x16, int8: 32x32x32) and the shader clock
 // during the run through *shader_mhz.  Returns a hipError_t.
-extern "C" int nnf_internal_mfma_probe(int kind, int mode, int iters, int num_cu, double* tops, double* shader_mhz)
+extern "C" int nnf_probe_mfma(int kind, int mode, int iters, int num_cu, double* tops, double* shader_mhz)
 {
     using namespace nnf;
     uint32_t* tab = nullptr;

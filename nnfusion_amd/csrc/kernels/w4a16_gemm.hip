@@ -260,32 +260,87 @@ namespace nnf
         }
     } // namespace
 
+    namespace
+    {
+        // Which kernel serves a call and what it parks in scratch memory: decided once, from the shape and the
+        // device's CU count alone, for the launcher and for the entry points' workspace checks alike.
+        struct Route
+        {
+            enum Kind { NONE, ROWS, MROWS, SKINNY, MROWS_SPLIT, SKINNY_SPLIT, TILE } kind = NONE; // NONE: the family asked for
+                                                                                                  // cannot serve the shape
+            int ksplits = 0;          // *_SPLIT: ranges of K
+            bool via_scratch = false; // GEMV kernels: products to scratch first, the element-wise epilogue reads them
+            workspace::SkPlan plan;   // TILE
+            size_t bytes = 0;         // written at partial_ws
+        };
+
+        Route route_w4a16(int M, int N, int K, bool gate, bool in_place_residual, int num_cu, const LaunchChoice& choice)
+        {
+            Route r;
+            const int n_rows = gate ? 2 * N : N; // weight rows
+            // choice.path: 0 the library's order of preference, 2 / 4 one family of GEMV kernels only, 3 the tile GEMM
+            const bool any = choice.path == 0, rows_family = any || choice.path == 4, skinny_family = any || choice.path == 2;
+            if (choice.path != 3)
+            {
+                // the products go to scratch first when the epilogue cannot work in place: the [M, 2N] gate | up pair,
+                // or a residual that is the output buffer itself
+                r.via_scratch = gate || in_place_residual;
+                const size_t scratch = r.via_scratch ? workspace::align256((size_t)M * n_rows * 2) : 0;
+                if (rows_family && w4a16_gemv_rows_supported(M, n_rows, K, num_cu))
+                    return r.kind = Route::ROWS, r.bytes = scratch, r;
+                if (rows_family && M > 1 && (any ? w4a16_mrows_preferred(M, n_rows, K, num_cu) : w4a16_mrows_supported(M, n_rows, K, num_cu)))
+                    return r.kind = Route::MROWS, r.bytes = scratch, r;
+                if (skinny_family && M <= 16 && w4a16_skinny_supported(M, n_rows, K))
+                    return r.kind = Route::SKINNY, r.bytes = scratch, r;
+                // more activations than one workgroup holds: ranges of K, fp32 sums per range, and the reduction pass
+                // (K above 8192 in multiples of 256: the row-streaming MFMA kernel, otherwise the split-K one)
+                r.via_scratch = false;
+                if (rows_family && (r.ksplits = w4a16_mrows_ksplits(M, n_rows, K, num_cu)) > 0)
+                    return r.kind = Route::MROWS_SPLIT, r.bytes = workspace::align256((size_t)r.ksplits * M * n_rows * 4), r;
+                if (skinny_family && (r.ksplits = w4a16_skinny_ksplits(M, n_rows, K)) > 0)
+                    return r.kind = Route::SKINNY_SPLIT, r.bytes = workspace::align256((size_t)r.ksplits * M * n_rows * 4), r;
+                if (!any)
+                    return r;
+            }
+            r.kind = Route::TILE;
+            r.plan = workspace::plan_w4a16_sk_with(M, N, K, gate, num_cu, choice.tile_rows, choice.k_parts);
+            r.bytes = r.plan.bytes();
+            return r;
+        }
+    } // namespace
+
+    size_t w4a16_gemm_partial_bytes(int M, int N, int K, int act, bool in_place_residual, int num_cu,
+                                    const LaunchChoice& choice)
+    {
+        return route_w4a16(M, N, K, act == 1, in_place_residual, num_cu, choice).bytes;
+    }
+
+    bool w4a16_path_supported(int M, int N, int K, int act, int num_cu, int path)
+    {
+        LaunchChoice choice;
+        choice.path = path;
+        return route_w4a16(M, N, K, act == 1, false, num_cu, choice).kind != Route::NONE;
+    }
+
     hipError_t launch_w4a16_gemm(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M,
                                  int N, int K, int zp, const void* rms_gamma, float rms_eps, const void* bias,
                                  const void* residual, int act, void* rms_ws, void* partial_ws, int num_cu,
-                                 bool gemm_only)
+                                 const LaunchChoice& choice)
     {
-        gemm_only = gemm_only || g_tuning.force_path == 3;
         const bool rms = rms_gamma != nullptr, hb = bias != nullptr, hr = residual != nullptr, gate = act == 1;
         // the combinations the fused entry points use; anything else is composed by the caller
         if (gate && (hb || hr))
             return hipErrorInvalidValue;
-        // which kernel serves the (gate: 2N) weight rows
-        const int n_rows = gate ? 2 * N : N;
-        const bool rows = !gemm_only && (g_tuning.force_path == 0 || g_tuning.force_path == 4) &&
-                          w4a16_gemv_rows_supported(M, n_rows, K, num_cu);
-        const bool mrows = !gemm_only && ((g_tuning.force_path == 5 && w4a16_mrows_supported(M, n_rows, K, num_cu)) ||
-                                          (g_tuning.force_path == 0 && w4a16_mrows_preferred(M, n_rows, K, num_cu)));
-        const bool one_launch_gemv = !gemm_only && (rows || mrows || (M <= 16 && w4a16_skinny_supported(M, n_rows, K)));
-        const int mr_splits = (!gemm_only && partial_ws && (g_tuning.force_path == 0 || g_tuning.force_path == 5))
-                                  ? w4a16_mrows_ksplits(M, n_rows, K, num_cu)
-                                  : 0;
-        const int ksplits = mr_splits ? mr_splits : (!gemm_only && partial_ws) ? w4a16_skinny_ksplits(M, n_rows, K) : 0;
-        // the products go to scratch first when the epilogue cannot work in place: the [M, 2N] gate | up pair, or a
-        // residual that is the output buffer itself
-        const bool via_scratch = gate || (hr && residual == Y);
-        const bool gemv_path = (one_launch_gemv && (!via_scratch || partial_ws)) || ksplits > 0;
-        if (rms && gemv_path)
+        const int n_rows = gate ? 2 * N : N; // weight rows
+        const Route route = route_w4a16(M, N, K, gate, hr && residual == Y, num_cu, choice);
+        if (route.kind == Route::NONE || (route.bytes > 0 && !partial_ws))
+            return hipErrorInvalidValue;
+        const bool rows = route.kind == Route::ROWS, mrows = route.kind == Route::MROWS;
+        const bool one_launch_gemv = rows || mrows || route.kind == Route::SKINNY;
+        const bool via_scratch = route.via_scratch;
+        const int ksplits = route.ksplits;
+        const bool mr_splits = route.kind == Route::MROWS_SPLIT;
+        if (rms && route.kind != Route::TILE)
         {
             // the GEMV kernels read normalised activations (the tile GEMM folds the normalisation in: below)
             if (!rms_ws)
@@ -300,7 +355,7 @@ namespace nnf
         // M <= 16 (<= 32 where the row-streaming MFMA kernel applies): the bandwidth-bound GEMV kernel on the
         // (normalised) activations, then a small element-wise
         // kernel for whatever epilogue is asked for
-        if (one_launch_gemv && (!via_scratch || partial_ws))
+        if (one_launch_gemv)
         {
             void* y_gemv = via_scratch ? partial_ws : Y;
             hipError_t e = rows ? launch_w4a16_gemv_rows(stream, A, Wq, S, y_gemv, n_rows, K, zp, num_cu)
@@ -340,12 +395,7 @@ namespace nnf
             return launch_reduce_any(stream, p, gate, hb, hr);
         }
         // ---- the tile GEMM ------------------------------------------------------------------------------------
-        // forced tile of the experiments hook: 1 .. 4 = 256, 128, 64, 32 rows; forced K ranges = workgroups per tile
-        static const int forced_rows[5] = {0, 256, 128, 64, 32};
-        const int f_rows = forced_rows[g_tuning.gemm_tile >= 0 && g_tuning.gemm_tile <= 4 ? g_tuning.gemm_tile : 0];
-        const workspace::SkPlan plan = workspace::plan_w4a16_sk_with(M, N, K, gate, num_cu, f_rows, g_tuning.gemm_splits);
-        if (plan.slots > 0 && !partial_ws)
-            return hipErrorInvalidValue;
+        const workspace::SkPlan& plan = route.plan;
         if ((size_t)M * K * 2 + 8192 >= ((size_t)1 << 32) || (size_t)n_rows * (K >> 1) >= ((size_t)1 << 32))
             return hipErrorInvalidValue; // the kernel addresses its operands with 32-bit byte offsets
         SkGemmParams p;

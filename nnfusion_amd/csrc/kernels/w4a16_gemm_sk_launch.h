@@ -9,7 +9,6 @@ namespace nnf
 {
     namespace gemm_sk
     {
-        // per (kernel, device): has the kernel been allowed its dynamic LDS yet
         template <int TM, int TN, bool GATE, bool BIAS, bool RESID, bool RMS>
         hipError_t launch_instance(hipStream_t stream, const SkGemmParams& p, int grid)
         {
@@ -17,20 +16,10 @@ namespace nnf
             auto kernel = &w4a16_gemm_sk_kernel<TM, TN, GATE, BIAS, RESID, RMS>;
             if (T::LDS_BYTES > 48 * 1024)
             {
-                static bool attr_set[64] = {};
-                int dev = 0;
-                hipError_t e = hipGetDevice(&dev);
+                static LdsGrant granted;
+                const hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), granted, T::LDS_BYTES);
                 if (e != hipSuccess)
                     return e;
-                if (dev < 0 || dev >= 64 || !attr_set[dev])
-                {
-                    e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                            T::LDS_BYTES);
-                    if (e != hipSuccess)
-                        return e;
-                    if (dev >= 0 && dev < 64)
-                        attr_set[dev] = true;
-                }
             }
             hipLaunchKernelGGL(kernel, dim3(grid), dim3(THREADS), T::LDS_BYTES, stream, p);
             hipError_t e = hipGetLastError();

@@ -111,8 +111,9 @@ namespace nnf
         size_t lds = (size_t)MB * C * 4 * 64 * 16;
         if (lds > 64 * 1024)
         {
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&w4a16_gemv_kernel<MB>),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            static LdsGrant granted;
+            const hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(&w4a16_gemv_kernel<MB>),
+                                                   granted, (int)MAX_LDS_BYTES);
             if (e != hipSuccess)
                 return e;
         }

@@ -333,8 +333,9 @@ namespace nnf
                 return hipErrorInvalidValue;
             if (lds_total > 64 * 1024)
             {
-                hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&w4a16_gemv_rows_kernel<SEG, D, WAVES>),
-                                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_total);
+                static LdsGrant granted;
+                const hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(&w4a16_gemv_rows_kernel<SEG, D, WAVES>),
+                                                       granted, (int)MAX_LDS_BYTES);
                 if (e != hipSuccess)
                     return e;
             }
@@ -353,7 +354,7 @@ namespace nnf
     hipError_t launch_w4a16_gemv_rows(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int N,
                                       int K, int zp, int num_cu)
     {
-        const RowsPlan p = workspace::plan_w4a16_rows(1, N, K, num_cu, g_tuning.skinny_cps);
+        const RowsPlan p = workspace::plan_w4a16_rows(1, N, K, num_cu, 0);
         const int grid = workspace::rows_grid(N, num_cu);
         switch (p.seg * 10 + p.depth)
         {

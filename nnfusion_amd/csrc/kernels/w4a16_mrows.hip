@@ -472,8 +472,8 @@ namespace nnf
             auto kernel = &w4a16_mrows_kernel<GW, STEPS, MB>;
             if (lds > 64 * 1024)
             {
-                hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                                   (int)lds);
+                static LdsGrant granted;
+                const hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), granted, (int)MAX_LDS_BYTES);
                 if (e != hipSuccess)
                     return e;
             }
@@ -511,8 +511,8 @@ namespace nnf
             auto kernel = &w4a16_mrows_any_kernel<GW, STEPS, MB>;
             if (lds > 64 * 1024)
             {
-                hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                                   (int)lds);
+                static LdsGrant granted;
+                const hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), granted, (int)MAX_LDS_BYTES);
                 if (e != hipSuccess)
                     return e;
             }

@@ -65,11 +65,7 @@ namespace nnf
 
     // rows of activations from which a wavefront loads its own operand instead of staging all rows in LDS
     // (below it the sixteen-fold repetition of the few rows costs more than the staging)
-    int& skinny_direct_min_rows()
-    {
-        static int v = 6; // measured: equal at 4 rows, 3-10 % faster from 6 rows on
-        return v;
-    }
+    constexpr int SKINNY_DIRECT_MIN_ROWS = 6; // measured: equal at 4 rows, 3-10 % faster from 6 rows on
 
     // pack = M | zp << 8 | wavefronts per workgroup << 16 | direct << 24 (A_REGS: every wavefront loads its own
     // share of the activations straight into registers, no staging in LDS);  n_wg: workgroups per K range;  a workgroup's tiles:
@@ -580,7 +576,7 @@ namespace nnf
     namespace
     {
         using workspace::SkinnyPlan;
-        SkinnyPlan plan_skinny(int M, int K) { return workspace::plan_w4a16_skinny(M, K, g_tuning.skinny_cps); }
+        SkinnyPlan plan_skinny(int M, int K) { return workspace::plan_w4a16_skinny(M, K, 0); }
 
         // K: the length of a K range (all of K without KSPLIT)
         template <int CPS, bool A_REGS, int H, bool KSPLIT = false>
@@ -590,9 +586,7 @@ namespace nnf
             const int n_tiles = (N + 15) / 16;
             const int ksplits = KSPLIT ? sp.ksplits : 1;
             // persistent workgroups: one per CU when it has >= 8 wavefronts, else two
-            int per_cu = p.ks >= 8 ? 1 : 2;
-            if (g_tuning.skinny_wg_per_cu > 0)
-                per_cu = g_tuning.skinny_wg_per_cu;
+            const int per_cu = p.ks >= 8 ? 1 : 2;
             // workgroups per K range
             int grid = std::min(n_tiles, std::max(1, num_cu * per_cu / ksplits));
             int tiles_per_wg = (n_tiles + grid - 1) / grid;
@@ -608,22 +602,23 @@ namespace nnf
                 return hipErrorInvalidValue;
             if (lds_total > 64 * 1024)
             {
-                hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&w4a16_skinny_kernel<CPS, A_REGS, H, KSPLIT>),
-                                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_total);
+                static LdsGrant granted;
+                const hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(&w4a16_skinny_kernel<CPS, A_REGS, H, KSPLIT>),
+                                                       granted, (int)MAX_LDS_BYTES);
                 if (e != hipSuccess)
                     return e;
             }
             hipLaunchKernelGGL((w4a16_skinny_kernel<CPS, A_REGS, H, KSPLIT>), dim3(grid * ksplits), dim3(p.ks * 64), lds_total,
                                stream, (const half_t*)A, (const uint8_t*)Wq, (const half_t*)S, (half_t*)Y, N, K,
                                n_tiles / grid, n_tiles % grid, grid,
-                               M | (zp << 8) | (p.ks << 16) | ((A_REGS && M >= skinny_direct_min_rows()) ? (1 << 24) : 0), sp);
+                               M | (zp << 8) | (p.ks << 16) | ((A_REGS && M >= SKINNY_DIRECT_MIN_ROWS) ? (1 << 24) : 0), sp);
             return hipGetLastError();
         }
     } // namespace
 
     bool w4a16_skinny_supported(int M, int N, int K)
     {
-        return workspace::w4a16_skinny_fits(M, N, K, g_tuning.skinny_cps);
+        return workspace::w4a16_skinny_fits(M, N, K, 0);
     }
 
     hipError_t launch_w4a16_skinny(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M,
@@ -644,7 +639,7 @@ namespace nnf
 
     int w4a16_skinny_ksplits(int M, int N, int K)
     {
-        return g_tuning.skinny_cps == 0 ? workspace::w4a16_skinny_ksplits(M, N, K) : 0;
+        return workspace::w4a16_skinny_ksplits(M, N, K);
     }
 
     hipError_t launch_w4a16_skinny_split(hipStream_t stream, const void* A, const void* Wq, const void* S, float* partial,

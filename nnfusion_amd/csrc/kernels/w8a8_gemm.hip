@@ -201,7 +201,7 @@ namespace nnf
     namespace
     {
         using Q8SkinnyPlan = workspace::Q8SkinnyPlan;
-        Q8SkinnyPlan plan_q8_skinny(int M, int K) { return workspace::plan_w8a8_skinny(M, K, g_tuning.skinny_cps); }
+        Q8SkinnyPlan plan_q8_skinny(int M, int K) { return workspace::plan_w8a8_skinny(M, K, 0); }
 
         template <int CPS, int KH, bool RAW_ACC>
         hipError_t launch_q8_skinny_cps(hipStream_t stream, const W8A8Params& p, const Q8SkinnyPlan& pl, int num_cu)
@@ -220,8 +220,9 @@ namespace nnf
                 return hipErrorInvalidValue;
             if (lds_total > 64 * 1024)
             {
-                hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&w8a8_skinny_kernel<CPS, KH, RAW_ACC>),
-                                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_total);
+                static LdsGrant granted;
+                const hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(&w8a8_skinny_kernel<CPS, KH, RAW_ACC>),
+                                                       granted, (int)MAX_LDS_BYTES);
                 if (e != hipSuccess)
                     return e;
             }
@@ -259,8 +260,48 @@ namespace nnf
 
     bool w8a8_skinny_supported(int M, int K) { return workspace::w8a8_skinny_fits(M, K); }
 
+    namespace
+    {
+        enum Q8Kind { Q8_NONE = -1, Q8_ROWS, Q8_MROWS, Q8_SKINNY, Q8_TILE };
+        // the kernel family that serves a call: the caller's choice where it made one (Q8_NONE: that family cannot
+        // serve the shape), otherwise by shape
+        Q8Kind pick_w8a8(int M, int N, int K, int num_cu, int path)
+        {
+            switch (path)
+            {
+            case 0:
+                if (w8a8_gemv_rows_supported(M, N, K, num_cu))
+                    return Q8_ROWS;
+                if (w8a8_mrows_preferred(M, N, K, num_cu))
+                    return Q8_MROWS;
+                return w8a8_skinny_supported(M, K) ? Q8_SKINNY : Q8_TILE;
+            case 2: return w8a8_skinny_supported(M, K) ? Q8_SKINNY : Q8_NONE;
+            case 3: return Q8_TILE;
+            case 4:
+                if (M == 1)
+                    return w8a8_gemv_rows_supported(M, N, K, num_cu) ? Q8_ROWS : Q8_NONE;
+                return w8a8_mrows_supported(M, N, K, num_cu) ? Q8_MROWS : Q8_NONE;
+            default: return Q8_NONE;
+            }
+        }
+    } // namespace
+
+    bool w8a8_path_supported(int M, int N, int K, int num_cu, int path)
+    {
+        return pick_w8a8(M, N, K, num_cu, path) != Q8_NONE;
+    }
+
+    size_t w8a8_partial_bytes(int M, int N, int K, int num_cu, const LaunchChoice& choice)
+    {
+        if (pick_w8a8(M, N, K, num_cu, choice.path) != Q8_TILE)
+            return 0;
+        const int tile = choice.tile_rows == 256 ? 0 : choice.tile_rows == 128 ? 1 : choice.tile_rows == 64 ? 2 : -1;
+        return workspace::gemm_partial_bytes(M, N, false, workspace::plan_w8a8_gemm(M, N, K, tile, choice.k_parts));
+    }
+
     hipError_t launch_w8a8(hipStream_t stream, const void* A, const void* s_tok, const void* W, const void* s_ch,
-                           void* Y, void* acc, int M, int N, int K, int num_cu, void* partial_ws)
+                           void* Y, void* acc, int M, int N, int K, int num_cu, void* partial_ws,
+                           const LaunchChoice& choice)
     {
         W8A8Params p;
         p.A = (const int8_t*)A;
@@ -273,14 +314,13 @@ namespace nnf
         p.N = N;
         p.K = K;
         const bool raw = acc != nullptr;
-        if ((g_tuning.force_path == 0 || g_tuning.force_path == 4) && w8a8_gemv_rows_supported(M, N, K, num_cu))
-            return launch_w8a8_gemv_rows(stream, A, s_tok, W, s_ch, Y, acc, N, K, num_cu);
-        if ((g_tuning.force_path == 5 && w8a8_mrows_supported(M, N, K, num_cu)) ||
-            (g_tuning.force_path == 0 && w8a8_mrows_preferred(M, N, K, num_cu)))
-            return launch_w8a8_mrows(stream, A, s_tok, W, s_ch, Y, acc, M, N, K, num_cu);
-        const bool skinny = g_tuning.force_path != 3 && w8a8_skinny_supported(M, K);
-        if (skinny)
-            return raw ? launch_q8_skinny<true>(stream, p, num_cu) : launch_q8_skinny<false>(stream, p, num_cu);
-        return launch_w8a8_gemm(stream, A, s_tok, W, s_ch, Y, acc, M, N, K, partial_ws);
+        switch (pick_w8a8(M, N, K, num_cu, choice.path))
+        {
+        case Q8_ROWS: return launch_w8a8_gemv_rows(stream, A, s_tok, W, s_ch, Y, acc, N, K, num_cu);
+        case Q8_MROWS: return launch_w8a8_mrows(stream, A, s_tok, W, s_ch, Y, acc, M, N, K, num_cu);
+        case Q8_SKINNY: return raw ? launch_q8_skinny<true>(stream, p, num_cu) : launch_q8_skinny<false>(stream, p, num_cu);
+        case Q8_TILE: return launch_w8a8_gemm(stream, A, s_tok, W, s_ch, Y, acc, M, N, K, partial_ws, choice);
+        default: return hipErrorInvalidValue;
+        }
     }
 } // namespace nnf

@@ -429,15 +429,10 @@ namespace nnf
             auto kernel = &w8a8_gemm_dl_kernel<WM, WN, TM, TN, STAGES, RAW, SPLITK, MINW>;
             if (T::LDS_BYTES > 64 * 1024)
             {
-                static bool attr_set = false;
-                if (!attr_set)
-                {
-                    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                                       hipFuncAttributeMaxDynamicSharedMemorySize, T::LDS_BYTES);
-                    if (e != hipSuccess)
-                        return e;
-                    attr_set = true;
-                }
+                static LdsGrant granted;
+                const hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), granted, T::LDS_BYTES);
+                if (e != hipSuccess)
+                    return e;
             }
             const int splits = SPLITK ? p.splits : 1;
             hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n * splits), dim3(q8dl::THREADS), T::LDS_BYTES, stream, p);
@@ -474,10 +469,10 @@ namespace nnf
     } // namespace
 
     hipError_t launch_w8a8_gemm(hipStream_t stream, const void* A, const void* s_tok, const void* W, const void* s_ch,
-                                void* Y, void* acc, int M, int N, int K, void* partial_ws)
+                                void* Y, void* acc, int M, int N, int K, void* partial_ws, const LaunchChoice& choice)
     {
-        const workspace::GemmPlan plan =
-            workspace::plan_w8a8_gemm(M, N, K, g_tuning.gemm_tile - 1, g_tuning.gemm_splits);
+        const int tile = choice.tile_rows == 256 ? 0 : choice.tile_rows == 128 ? 1 : choice.tile_rows == 64 ? 2 : -1;
+        const workspace::GemmPlan plan = workspace::plan_w8a8_gemm(M, N, K, tile, choice.k_parts);
         if (plan.reduce_pass && !partial_ws)
             return hipErrorInvalidValue;
         Q8GemmParams p;

@@ -237,8 +237,9 @@ namespace nnf
                 return hipErrorInvalidValue;
             if (lds_total > 64 * 1024)
             {
-                hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&w8a8_gemv_rows_kernel<SEG, D, WAVES, RAW>),
-                                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_total);
+                static LdsGrant granted;
+                const hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(&w8a8_gemv_rows_kernel<SEG, D, WAVES, RAW>),
+                                                       granted, (int)MAX_LDS_BYTES);
                 if (e != hipSuccess)
                     return e;
             }
@@ -252,7 +253,7 @@ namespace nnf
         hipError_t launch_q8_rows_any(hipStream_t stream, const void* A, const void* s_tok, const void* W, const void* s_ch,
                                       void* Y, void* acc, int N, int K, int num_cu)
         {
-            const Q8RowsPlan p = workspace::plan_w8a8_rows(1, N, K, num_cu, g_tuning.skinny_cps);
+            const Q8RowsPlan p = workspace::plan_w8a8_rows(1, N, K, num_cu, 0);
             const int grid = workspace::rows_grid(N, num_cu);
             switch (p.seg * 10 + p.depth)
             {

@@ -224,8 +224,8 @@ namespace nnf
             auto kernel = &w8a8_mrows_kernel<STEPS, MB, NS, RAW>;
             if (lds > 64 * 1024)
             {
-                hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                                   (int)lds);
+                static LdsGrant granted;
+                const hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), granted, (int)MAX_LDS_BYTES);
                 if (e != hipSuccess)
                     return e;
             }

@@ -67,33 +67,11 @@ namespace
     }
 } // namespace
 
-namespace nnf
-{
-    Tuning g_tuning;
-}
-
 extern "C" {
-
-// experiment hook, deliberately absent from the public header
-int nnf_internal_tune(int key, int value)
-{
-    switch (key)
-    {
-    case 0: nnf::g_tuning.force_path = value; return 0;
-    case 1: nnf::g_tuning.skinny_cps = value; return 0;
-    case 2: nnf::g_tuning.skinny_wg_per_cu = value; return 0;
-    case 3: nnf::g_tuning.gemm_tile = value; return 0;
-    case 4: nnf::g_tuning.gemm_splits = value; return 0;
-    case 5: nnf::workspace::skinny_min_splits() = value; return 0;
-    case 6: nnf::skinny_direct_min_rows() = value > 0 ? value : 6; return 0;
-    case 7: nnf::workspace::mrows_forced_ranges() = value; return 0;
-    default: return -1;
-    }
-}
 
 int nnf_abi_version(void)
 {
-    return 1;
+    return 2;
 }
 
 const char* nnf_status_string(int status)
@@ -118,20 +96,58 @@ const char* nnf_status_string(int status)
 
 namespace
 {
-    // partial-sum bytes of the GEMM plan in force (the automatic one unless an experiment overrides it)
-    // fused: a call that may run the GEMV kernel into scratch (fp16 [M, N or 2N]) ahead of an element-wise epilogue
-    size_t tuned_partial_bytes(int M, int N, int K, bool gate, bool fused = false)
+    // the caller's variant and plan arguments as the launchers take them; false: not a valid request
+    bool make_choice(int variant, const nnf_plan* plan, int max_variant, nnf::LaunchChoice& out)
     {
-        static const int forced_rows[5] = {0, 256, 128, 64, 32};
-        const int f_rows = forced_rows[nnf::g_tuning.gemm_tile >= 0 && nnf::g_tuning.gemm_tile <= 4 ? nnf::g_tuning.gemm_tile : 0];
-        const size_t a =
-            nnf::workspace::plan_w4a16_sk_with(M, N, K, gate, nnf::workspace::PLAN_CUS, f_rows, nnf::g_tuning.gemm_splits).bytes();
-        // the M <= 16 kernels over ranges of K write partial sums too
-        const size_t b = nnf::workspace::skinny_split_bytes(M, gate ? 2 * N : N, K);
-        const size_t c = nnf::workspace::mrows_split_bytes(M, gate ? 2 * N : N, K);
-        const size_t d = fused ? nnf::workspace::gemv_scratch_bytes(M, gate ? 2 * N : N) : 0;
-        const size_t bc = b > c ? b : c, ad = a > d ? a : d;
-        return ad > bc ? ad : bc;
+        if (variant < 0 || variant > max_variant)
+            return false;
+        out.path = variant;
+        if (plan)
+        {
+            const int r = plan->tile_rows;
+            if ((r != 0 && r != 32 && r != 64 && r != 128 && r != 256) || plan->k_parts < 0)
+                return false;
+            out.tile_rows = r;
+            out.k_parts = plan->k_parts;
+        }
+        return true;
+    }
+
+    // nnf_w8a8_variant -> the launchers' numbering of kernel families (that of nnf_w4a16_variant)
+    int w8a8_path(int variant) { return variant == NNF_W8A8_AUTO ? 0 : variant + 1; }
+
+    bool workspace_ok(size_t need, const void* workspace, size_t workspace_bytes)
+    {
+        return need == 0 || (workspace && aligned16(workspace) && workspace_bytes >= need);
+    }
+
+    int w4a16_gemm_checked(nnf_stream_t stream, const void* A, const void* Wq, const void* scales, void* Y, int M, int N,
+                           int K, int group, int zp, const nnf::LaunchChoice& choice, void* workspace,
+                           size_t workspace_bytes)
+    {
+        int st = check_w4a16(A, Wq, scales, Y, M, N, K, group, zp);
+        if (st != NNF_OK)
+            return st;
+        DeviceInfo dev;
+        st = current_device_info(dev);
+        if (st != NNF_OK)
+            return st;
+        const hipStream_t s = (hipStream_t)stream;
+        if (choice.path == NNF_W4A16_GEMV_VALU)
+        {
+            if (M > 16 || !nnf::w4a16_gemv_supported(M, K))
+                return NNF_ERR_UNSUPPORTED_SHAPE;
+            return (int)nnf::launch_w4a16_gemv(s, A, Wq, scales, Y, M, N, K, zp, dev.num_cu);
+        }
+        if (!nnf::w4a16_path_supported(M, N, K, NNF_ACT_NONE, dev.num_cu, choice.path))
+            return NNF_ERR_UNSUPPORTED_SHAPE;
+        // the GEMV kernels over ranges of K and the tile GEMM park partial sums in scratch memory; the check is for
+        // what this launch writes on this device
+        if (!workspace_ok(nnf::w4a16_gemm_partial_bytes(M, N, K, NNF_ACT_NONE, false, dev.num_cu, choice), workspace,
+                          workspace_bytes))
+            return NNF_ERR_WORKSPACE_TOO_SMALL;
+        return (int)nnf::launch_w4a16_gemm(s, A, Wq, scales, Y, M, N, K, zp, nullptr, 0.f, nullptr, nullptr, NNF_ACT_NONE,
+                                           nullptr, workspace, dev.num_cu, choice);
     }
 } // namespace
 
@@ -145,29 +161,8 @@ size_t nnf_w4a16_gemm_workspace_bytes(int M, int N, int K, int group)
 int nnf_w4a16_gemm(nnf_stream_t stream, const void* A, const void* Wq, const void* scales, void* Y, int M, int N,
                    int K, int group, int zp, void* workspace, size_t workspace_bytes)
 {
-    int st = check_w4a16(A, Wq, scales, Y, M, N, K, group, zp);
-    if (st != NNF_OK)
-        return st;
-    DeviceInfo dev;
-    st = current_device_info(dev);
-    if (st != NNF_OK)
-        return st;
-    const int force = nnf::g_tuning.force_path;
-    if ((force == 0 || force == 4) && nnf::w4a16_gemv_rows_supported(M, N, K, dev.num_cu))
-        return (int)nnf::launch_w4a16_gemv_rows((hipStream_t)stream, A, Wq, scales, Y, N, K, zp, dev.num_cu);
-    if ((force == 5 && nnf::w4a16_mrows_supported(M, N, K, dev.num_cu)) ||
-        (force == 0 && nnf::w4a16_mrows_preferred(M, N, K, dev.num_cu)))
-        return (int)nnf::launch_w4a16_mrows((hipStream_t)stream, A, Wq, scales, Y, M, N, K, zp, dev.num_cu);
-    if ((force == 0 || force == 2 || force == 4 || force == 5) && M <= 16 && nnf::w4a16_skinny_supported(M, N, K))
-        return (int)nnf::launch_w4a16_skinny((hipStream_t)stream, A, Wq, scales, Y, M, N, K, zp, dev.num_cu);
-    if (force == 1 && M <= 16 && nnf::w4a16_gemv_supported(M, K))
-        return (int)nnf::launch_w4a16_gemv((hipStream_t)stream, A, Wq, scales, Y, M, N, K, zp, dev.num_cu);
-    // the MFMA GEMM may split K and then needs room for its partial sums (the GEMV kernels need none)
-    const size_t need = tuned_partial_bytes(M, N, K, false);
-    if (need > 0 && (!workspace || !aligned16(workspace) || workspace_bytes < need))
-        return NNF_ERR_WORKSPACE_TOO_SMALL;
-    return (int)nnf::launch_w4a16_gemm((hipStream_t)stream, A, Wq, scales, Y, M, N, K, zp, nullptr, 0.f, nullptr,
-                                       nullptr, NNF_ACT_NONE, nullptr, workspace, dev.num_cu);
+    return w4a16_gemm_checked(stream, A, Wq, scales, Y, M, N, K, group, zp, nnf::LaunchChoice(), workspace,
+                              workspace_bytes);
 }
 
 int nnf_w4a16_gemm_static_scratch(nnf_stream_t stream, const void* A, const void* Wq, const void* scales, void* Y,
@@ -193,54 +188,32 @@ int nnf_w4a16_variant_supported(int M, int N, int K, int group, int variant)
     return (group == 128 && nnf::workspace::w4a16_variant_fits(M, N, K, variant)) ? 1 : 0;
 }
 
-size_t nnf_w4a16_gemm_variant_workspace_bytes(int M, int N, int K, int group, int variant)
+size_t nnf_w4a16_gemm_variant_workspace_bytes(int M, int N, int K, int group, int variant, const nnf_plan* plan)
 {
-    if (M <= 0 || N <= 0 || K < 128)
+    nnf::LaunchChoice choice;
+    if (M <= 0 || N <= 0 || K < 128 || !make_choice(variant, plan, NNF_W4A16_GEMV_ROWS, choice))
         return 0;
     if (variant == NNF_W4A16_GEMM_MFMA)
-        return nnf::workspace::plan_w4a16_sk(M, N, K, false, nnf::workspace::PLAN_CUS).bytes();
+        return nnf::workspace::plan_w4a16_sk_with(M, N, K, false, nnf::workspace::PLAN_CUS, choice.tile_rows, choice.k_parts)
+            .bytes();
     if (variant == NNF_W4A16_AUTO)
         return nnf::workspace::w4a16_gemm(M, N, K, group);
+    // the GEMV kernels over ranges of K (shapes whose activations exceed one workgroup's LDS / registers)
+    if (variant == NNF_W4A16_GEMV_MFMA && !nnf::workspace::w4a16_skinny_fits(M, N, K))
+        return nnf::workspace::skinny_split_bytes(M, N, K);
+    if (variant == NNF_W4A16_GEMV_ROWS && M > 1 && !nnf::workspace::w4a16_mrows_fits(M, N, K, nnf::workspace::PLAN_CUS))
+        return nnf::workspace::mrows_split_bytes(M, N, K);
     return 0;
 }
 
 int nnf_w4a16_gemm_variant(nnf_stream_t stream, const void* A, const void* Wq, const void* scales, void* Y, int M,
-                           int N, int K, int group, int zp, int variant, void* workspace, size_t workspace_bytes)
+                           int N, int K, int group, int zp, int variant, const nnf_plan* plan, void* workspace,
+                           size_t workspace_bytes)
 {
-    if (variant == NNF_W4A16_AUTO)
-        return nnf_w4a16_gemm(stream, A, Wq, scales, Y, M, N, K, group, zp, workspace, workspace_bytes);
-    int st = check_w4a16(A, Wq, scales, Y, M, N, K, group, zp);
-    if (st != NNF_OK)
-        return st;
-    if (variant < NNF_W4A16_AUTO || variant > NNF_W4A16_GEMV_ROWS)
+    nnf::LaunchChoice choice;
+    if (!make_choice(variant, plan, NNF_W4A16_GEMV_ROWS, choice))
         return NNF_ERR_INVALID_ARGUMENT;
-    DeviceInfo dev;
-    st = current_device_info(dev);
-    if (st != NNF_OK)
-        return st;
-    switch (variant)
-    {
-    case NNF_W4A16_GEMV_ROWS:
-        if (M > 1 && nnf::w4a16_mrows_supported(M, N, K, dev.num_cu))
-            return (int)nnf::launch_w4a16_mrows((hipStream_t)stream, A, Wq, scales, Y, M, N, K, zp, dev.num_cu);
-        if (!nnf::w4a16_gemv_rows_supported(M, N, K, dev.num_cu))
-            return NNF_ERR_UNSUPPORTED_SHAPE;
-        return (int)nnf::launch_w4a16_gemv_rows((hipStream_t)stream, A, Wq, scales, Y, N, K, zp, dev.num_cu);
-    case NNF_W4A16_GEMV_MFMA:
-        if (!nnf::workspace::w4a16_skinny_fits(M, N, K))
-            return NNF_ERR_UNSUPPORTED_SHAPE;
-        return (int)nnf::launch_w4a16_skinny((hipStream_t)stream, A, Wq, scales, Y, M, N, K, zp, dev.num_cu);
-    case NNF_W4A16_GEMV_VALU:
-        if (M > 16 || !nnf::w4a16_gemv_supported(M, K))
-            return NNF_ERR_UNSUPPORTED_SHAPE;
-        return (int)nnf::launch_w4a16_gemv((hipStream_t)stream, A, Wq, scales, Y, M, N, K, zp, dev.num_cu);
-    default: break;
-    }
-    const size_t need = nnf_w4a16_gemm_variant_workspace_bytes(M, N, K, group, NNF_W4A16_GEMM_MFMA);
-    if (need > 0 && (!workspace || !aligned16(workspace) || workspace_bytes < need))
-        return NNF_ERR_WORKSPACE_TOO_SMALL;
-    return (int)nnf::launch_w4a16_gemm((hipStream_t)stream, A, Wq, scales, Y, M, N, K, zp, nullptr, 0.f, nullptr,
-                                       nullptr, NNF_ACT_NONE, nullptr, workspace, dev.num_cu, true);
+    return w4a16_gemm_checked(stream, A, Wq, scales, Y, M, N, K, group, zp, choice, workspace, workspace_bytes);
 }
 
 size_t nnf_w4a16_gemm_fused_workspace_bytes(int M, int N, int K, int group, int act)
@@ -249,54 +222,50 @@ size_t nnf_w4a16_gemm_fused_workspace_bytes(int M, int N, int K, int group, int 
     return nnf::workspace::w4a16_gemm_fused(M, N, K, group, act);
 }
 
-int nnf_w4a16_gemm_fused(nnf_stream_t stream, const void* A, const void* Wq, const void* scales, void* Y, int M, int N,
-                         int K, int group, int zp, const void* rms_gamma, float rms_eps, const void* bias,
-                         const void* residual, int act, void* workspace, size_t workspace_bytes)
+int nnf_w4a16_gemm_fused_variant(nnf_stream_t stream, const void* A, const void* Wq, const void* scales, void* Y, int M,
+                                 int N, int K, int group, int zp, const void* rms_gamma, float rms_eps, const void* bias,
+                                 const void* residual, int act, int variant, const nnf_plan* plan, void* workspace,
+                                 size_t workspace_bytes)
 {
     int st = check_w4a16(A, Wq, scales, Y, M, N, K, group, zp);
     if (st != NNF_OK)
         return st;
-    if (act != NNF_ACT_NONE && act != NNF_ACT_SILU_GATE)
+    nnf::LaunchChoice choice;
+    if ((act != NNF_ACT_NONE && act != NNF_ACT_SILU_GATE) || !make_choice(variant, plan, NNF_W4A16_GEMV_ROWS, choice))
         return NNF_ERR_INVALID_ARGUMENT;
     if ((rms_gamma && !aligned16(rms_gamma)) || (bias && !aligned16(bias)) || (residual && !aligned16(residual)))
         return NNF_ERR_INVALID_ARGUMENT;
-    // combinations without a fused kernel (see launch_w4a16_gemm)
-    if (act == NNF_ACT_SILU_GATE && (bias || residual))
+    // combinations without a fused kernel: the gate product with a bias or residual; the VALU GEMV
+    if ((act == NNF_ACT_SILU_GATE && (bias || residual)) || variant == NNF_W4A16_GEMV_VALU)
         return NNF_ERR_UNSUPPORTED_SHAPE;
-    const size_t need = (rms_gamma ? nnf::workspace::rms_rows(M, K) : 0) + tuned_partial_bytes(M, N, K, act == NNF_ACT_SILU_GATE, true);
-    if (need > 0 && (!workspace || !aligned16(workspace) || workspace_bytes < need))
-        return NNF_ERR_WORKSPACE_TOO_SMALL;
     DeviceInfo dev;
     st = current_device_info(dev);
     if (st != NNF_OK)
         return st;
+    if (!nnf::w4a16_path_supported(M, N, K, act, dev.num_cu, choice.path))
+        return NNF_ERR_UNSUPPORTED_SHAPE;
+    // [ RMSNorm scratch ][ what this launch parks, on this device ]
+    const size_t rms_bytes = rms_gamma ? nnf::workspace::rms_rows(M, K) : 0;
+    const size_t need = rms_bytes + nnf::w4a16_gemm_partial_bytes(M, N, K, act, residual == Y, dev.num_cu, choice);
+    if (!workspace_ok(need, workspace, workspace_bytes))
+        return NNF_ERR_WORKSPACE_TOO_SMALL;
     uint8_t* ws = (uint8_t*)workspace;
     return (int)nnf::launch_w4a16_gemm((hipStream_t)stream, A, Wq, scales, Y, M, N, K, zp, rms_gamma, rms_eps, bias,
-                                       residual, act, ws, ws ? ws + (rms_gamma ? nnf::workspace::rms_rows(M, K) : 0) : nullptr,
-                                       dev.num_cu);
+                                       residual, act, ws, ws ? ws + rms_bytes : nullptr, dev.num_cu, choice);
+}
+
+int nnf_w4a16_gemm_fused(nnf_stream_t stream, const void* A, const void* Wq, const void* scales, void* Y, int M, int N,
+                         int K, int group, int zp, const void* rms_gamma, float rms_eps, const void* bias,
+                         const void* residual, int act, void* workspace, size_t workspace_bytes)
+{
+    return nnf_w4a16_gemm_fused_variant(stream, A, Wq, scales, Y, M, N, K, group, zp, rms_gamma, rms_eps, bias, residual,
+                                        act, NNF_W4A16_AUTO, nullptr, workspace, workspace_bytes);
 }
 
 // ---- W8A8 ---------------------------------------------------------------------------------------
 size_t nnf_w8a8_gemm_workspace_bytes(int M, int N, int K)
 {
     return nnf::workspace::w8a8_gemm(M, N, K);
-}
-
-// room for the int32 partial sums when the MFMA GEMM serves the shape (the M <= 16 kernel needs none)
-static int check_w8a8_workspace(int M, int N, int K, int num_cu, const void* workspace, size_t workspace_bytes)
-{
-    if ((nnf::g_tuning.force_path == 0 || nnf::g_tuning.force_path == 4) && nnf::w8a8_gemv_rows_supported(M, N, K, num_cu))
-        return NNF_OK;
-    if ((nnf::g_tuning.force_path == 5 && nnf::w8a8_mrows_supported(M, N, K, num_cu)) ||
-        (nnf::g_tuning.force_path == 0 && nnf::w8a8_mrows_preferred(M, N, K, num_cu)))
-        return NNF_OK;
-    if (nnf::g_tuning.force_path != 3 && nnf::w8a8_skinny_supported(M, K))
-        return NNF_OK;
-    const size_t need = nnf::workspace::gemm_partial_bytes(
-        M, N, false, nnf::workspace::plan_w8a8_gemm(M, N, K, nnf::g_tuning.gemm_tile - 1, nnf::g_tuning.gemm_splits));
-    if (need > 0 && (!workspace || !aligned16(workspace) || workspace_bytes < need))
-        return NNF_ERR_WORKSPACE_TOO_SMALL;
-    return NNF_OK;
 }
 
 static int check_w8a8(const void* A, const void* W, const void* out, int M, int N, int K)
@@ -311,39 +280,64 @@ static int check_w8a8(const void* A, const void* W, const void* out, int M, int 
     return NNF_OK;
 }
 
-int nnf_w8a8_gemm(nnf_stream_t stream, const void* A, const void* s_tok, const void* W, const void* s_ch, void* Y,
-                  int M, int N, int K, void* workspace, size_t workspace_bytes)
+int nnf_w8a8_variant_supported(int M, int N, int K, int variant)
 {
-    int st = check_w8a8(A, W, Y, M, N, K);
+    if (M <= 0 || N <= 0 || K <= 0 || K % 128 != 0 || K > 133000 || variant < NNF_W8A8_AUTO || variant > NNF_W8A8_GEMV_ROWS)
+        return 0;
+    return nnf::w8a8_path_supported(M, N, K, nnf::workspace::PLAN_CUS, w8a8_path(variant)) ? 1 : 0;
+}
+
+size_t nnf_w8a8_gemm_variant_workspace_bytes(int M, int N, int K, int variant, const nnf_plan* plan)
+{
+    nnf::LaunchChoice choice;
+    if (!make_choice(variant, plan, NNF_W8A8_GEMV_ROWS, choice) || !nnf_w8a8_variant_supported(M, N, K, variant))
+        return 0;
+    choice.path = w8a8_path(variant);
+    return nnf::w8a8_partial_bytes(M, N, K, nnf::workspace::PLAN_CUS, choice);
+}
+
+int nnf_w8a8_gemm_variant(nnf_stream_t stream, const void* A, const void* s_tok, const void* W, const void* s_ch, void* Y,
+                          void* acc, int M, int N, int K, int variant, const nnf_plan* plan, void* workspace,
+                          size_t workspace_bytes)
+{
+    // exactly one of the two outputs
+    if ((Y != nullptr) == (acc != nullptr))
+        return NNF_ERR_INVALID_ARGUMENT;
+    int st = check_w8a8(A, W, Y ? Y : acc, M, N, K);
     if (st != NNF_OK)
         return st;
-    if (!s_tok || !s_ch)
+    nnf::LaunchChoice choice;
+    if ((Y && (!s_tok || !s_ch)) || !make_choice(variant, plan, NNF_W8A8_GEMV_ROWS, choice))
         return NNF_ERR_INVALID_ARGUMENT;
+    choice.path = w8a8_path(variant);
     DeviceInfo dev;
     st = current_device_info(dev);
     if (st != NNF_OK)
         return st;
-    st = check_w8a8_workspace(M, N, K, dev.num_cu, workspace, workspace_bytes);
-    if (st != NNF_OK)
-        return st;
-    return (int)nnf::launch_w8a8((hipStream_t)stream, A, s_tok, W, s_ch, Y, nullptr, M, N, K, dev.num_cu, workspace);
+    if (!nnf::w8a8_path_supported(M, N, K, dev.num_cu, choice.path))
+        return NNF_ERR_UNSUPPORTED_SHAPE;
+    if (!workspace_ok(nnf::w8a8_partial_bytes(M, N, K, dev.num_cu, choice), workspace, workspace_bytes))
+        return NNF_ERR_WORKSPACE_TOO_SMALL;
+    return (int)nnf::launch_w8a8((hipStream_t)stream, A, Y ? s_tok : nullptr, W, Y ? s_ch : nullptr, Y, acc, M, N, K,
+                                 dev.num_cu, workspace, choice);
+}
+
+int nnf_w8a8_gemm(nnf_stream_t stream, const void* A, const void* s_tok, const void* W, const void* s_ch, void* Y,
+                  int M, int N, int K, void* workspace, size_t workspace_bytes)
+{
+    if (!Y)
+        return NNF_ERR_INVALID_ARGUMENT;
+    return nnf_w8a8_gemm_variant(stream, A, s_tok, W, s_ch, Y, nullptr, M, N, K, NNF_W8A8_AUTO, nullptr, workspace,
+                                 workspace_bytes);
 }
 
 int nnf_w8a8_gemm_acc(nnf_stream_t stream, const void* A, const void* W, void* acc, int M, int N, int K,
                       void* workspace, size_t workspace_bytes)
 {
-    int st = check_w8a8(A, W, acc, M, N, K);
-    if (st != NNF_OK)
-        return st;
-    DeviceInfo dev;
-    st = current_device_info(dev);
-    if (st != NNF_OK)
-        return st;
-    st = check_w8a8_workspace(M, N, K, dev.num_cu, workspace, workspace_bytes);
-    if (st != NNF_OK)
-        return st;
-    return (int)nnf::launch_w8a8((hipStream_t)stream, A, nullptr, W, nullptr, nullptr, acc, M, N, K, dev.num_cu,
-                                 workspace);
+    if (!acc)
+        return NNF_ERR_INVALID_ARGUMENT;
+    return nnf_w8a8_gemm_variant(stream, A, nullptr, W, nullptr, nullptr, acc, M, N, K, NNF_W8A8_AUTO, nullptr, workspace,
+                                 workspace_bytes);
 }
 
 // ---- fused MLP block ------------------------------------------------------------------------------
@@ -364,15 +358,18 @@ int nnf_fused_mlp_w4a16(nnf_stream_t stream, const void* x, const void* gamma, f
         return NNF_ERR_INVALID_ARGUMENT;
     if (group != 128 || H % group != 0 || I % group != 0 || zp < 0 || zp > 15)
         return NNF_ERR_UNSUPPORTED_SHAPE;
-    {
-        const size_t a = tuned_partial_bytes(M, I, H, true, true), b = tuned_partial_bytes(M, H, I, false);
-        if (!workspace || workspace_bytes < nnf::workspace::fused_mlp_partial_offset(M, H, I) + (a > b ? a : b))
-            return NNF_ERR_WORKSPACE_TOO_SMALL;
-    }
     DeviceInfo dev;
     int st = current_device_info(dev);
     if (st != NNF_OK)
         return st;
+    {
+        // what the two launches park behind h, on this device (the down projection's residual is x: in place when
+        // the caller passes out == x)
+        const size_t a = nnf::w4a16_gemm_partial_bytes(M, I, H, NNF_ACT_SILU_GATE, false, dev.num_cu);
+        const size_t b = nnf::w4a16_gemm_partial_bytes(M, H, I, NNF_ACT_NONE, out == x, dev.num_cu);
+        if (!workspace || workspace_bytes < nnf::workspace::fused_mlp_partial_offset(M, H, I) + (a > b ? a : b))
+            return NNF_ERR_WORKSPACE_TOO_SMALL;
+    }
     uint8_t* ws = (uint8_t*)workspace;
     void* h = ws + nnf::workspace::fused_mlp_h_offset(M, H);
     void* partial = ws + nnf::workspace::fused_mlp_partial_offset(M, H, I);

@@ -12,13 +12,13 @@ namespace nnf
     {
         inline size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
 
-        // ---- tile plan of the fp16 x int4 MFMA GEMM -------------------------------------------------
+        // ---- tile plan of the W8A8 MFMA GEMM (w8a8_gemm_dl.hip) ----------------------------------------
         enum GemmTile
         {
-            GEMM_TILE_BIG = 0,   // 256 x 256 outputs (SiLU-gate: 256 x 128)
+            GEMM_TILE_BIG = 0,   // 256 x 256 outputs
             GEMM_TILE_MID = 1,   // 128 x 128
             GEMM_TILE_SMALL = 2, //  64 x 256
-            GEMM_TILE_TINY = 3,  //  32 x 256
+            GEMM_TILE_TINY = 3,  //  32 x 256 (not built for W8A8)
         };
         struct GemmPlan
         {
@@ -57,12 +57,7 @@ namespace nnf
             return t;
         }
 
-        inline double estimate_w4a16_gemm(int M, int N, int K, bool gate, int tile, int splits)
-        {
-            return estimate_gemm(M, N, K, gate, tile, splits, false);
-        }
-
-        // N: output columns.  forced_tile >= 0 / forced_splits > 0 override the choice (experiments).
+        // N: output columns.  forced_tile >= 0 / forced_splits > 0 override the choice (a caller's plan argument).
         inline GemmPlan plan_gemm(int M, int N, int K, bool gate, bool w8a8, int forced_tile, int forced_splits)
         {
             static const int split_options[] = {1, 2, 3, 4, 6, 8, 12, 16};
@@ -92,10 +87,6 @@ namespace nnf
             }
             best.reduce_pass = best.splits > 1 || best.tile >= GEMM_TILE_SMALL;
             return best;
-        }
-        inline GemmPlan plan_w4a16_gemm(int M, int N, int K, bool gate, int forced_tile = -1, int forced_splits = 0)
-        {
-            return plan_gemm(M, N, K, gate, false, forced_tile, forced_splits);
         }
         inline GemmPlan plan_w8a8_gemm(int M, int N, int K, int forced_tile = -1, int forced_splits = 0)
         {
@@ -166,13 +157,6 @@ namespace nnf
                 return SkPlan();
             return plan_sk(M, ceil_div(N, gate ? 128 : 256), (K / 128 + 1) / 2, 2, num_cu, forced_tile_rows, forced_grid);
         }
-        // W8A8 (w8a8_gemm_sk.h): units of 128 k (its K steps), a workgroup keeps at least four; slots of int32
-        inline SkPlan plan_w8a8_sk(int M, int N, int K, int num_cu, int forced_tile_rows = 0, int forced_grid = 0)
-        {
-            if (M <= 0 || N <= 0 || K < 128 || num_cu < 1)
-                return SkPlan();
-            return plan_sk(M, ceil_div(N, 256), K / 128, 4, num_cu, forced_tile_rows, forced_grid);
-        }
 
         // the plan with a forced tile height (0 = the plan's own) and a forced number of workgroups per tile (0 = the
         // plan's own grid)
@@ -182,13 +166,6 @@ namespace nnf
                 return plan_w4a16_sk(M, N, K, gate, num_cu, tile_rows, 0);
             const SkPlan t = plan_w4a16_sk(M, N, K, gate, num_cu, tile_rows, 0);
             return plan_w4a16_sk(M, N, K, gate, num_cu, tile_rows, t.tiles_m * t.tiles_n * workgroups_per_tile);
-        }
-        inline SkPlan plan_w8a8_sk_with(int M, int N, int K, int num_cu, int tile_rows, int workgroups_per_tile)
-        {
-            if (workgroups_per_tile <= 0)
-                return plan_w8a8_sk(M, N, K, num_cu, tile_rows, 0);
-            const SkPlan t = plan_w8a8_sk(M, N, K, num_cu, tile_rows, 0);
-            return plan_w8a8_sk(M, N, K, num_cu, tile_rows, t.tiles_m * t.tiles_n * workgroups_per_tile);
         }
 
         // ---- plan of the skinny (M <= 16) MFMA GEMV kernel ---------------------------------------------
@@ -257,12 +234,6 @@ namespace nnf
         // equal ranges (multiples of 1024 columns, at most 4096) when K divides that way, otherwise ranges of a
         // multiple of 1024 and a shorter last one of at least 1024.  Returns the length of the ranges (of all but
         // the last), or 0 when this does not apply.
-        // experiments only: the smallest number of equal ranges to consider (0: no preference)
-        inline int& skinny_min_splits()
-        {
-            static int v = 0;
-            return v;
-        }
         inline int w4a16_skinny_split_range(int M, int N, int K)
         {
             if (M < 1 || M > 16 || N < 16 || K < 2048 || (K & 127) || w4a16_skinny_fits(M, N, K))
@@ -273,8 +244,6 @@ namespace nnf
             for (int s : equal)
             {
                 const int r = K / s;
-                if (s < skinny_min_splits())
-                    continue;
                 if (K % s == 0 && (r & 1023) == 0 && r <= 4096 && w4a16_skinny_fits(M, N, r))
                     return r;
             }
@@ -374,9 +343,9 @@ namespace nnf
         }
 
         inline size_t mrows_split_bytes(int M, int N_total, int K); // the row-streaming MFMA kernel over ranges of K
-        // Fused calls with at most 32 rows may run the GEMV kernel into scratch and an element-wise epilogue from
+        // Fused calls with at most 40 rows may run the GEMV kernel into scratch and an element-wise epilogue from
         // there (the [M, 2N] gate | up pair; a residual that is the output buffer): fp16 [M, N_total].
-        inline size_t gemv_scratch_bytes(int M, int N_total) { return (M > 0 && M <= 32) ? align256((size_t)M * N_total * 2) : 0; }
+        inline size_t gemv_scratch_bytes(int M, int N_total) { return (M > 0 && M <= 40) ? align256((size_t)M * N_total * 2) : 0; }
 
         // nnf_w4a16_gemm: [ partial sums ]
         inline size_t w4a16_gemm(int M, int N, int K, int)
@@ -512,12 +481,6 @@ namespace nnf
         // reduction pass.  Every workgroup fetches the activations of its range, so shorter ranges mean less of that
         // traffic (CUs x M x K / ranges x 2 bytes): ranges of at most 32 groups (GW = 2) measured fastest (K = 11008:
         // 3 ranges, 14336: 4, 28672: 7-8; 10-25 % faster than the fewest ranges that fit the registers).
-        // experiments only: a number of ranges to use instead of the plan's (0: no preference)
-        inline int& mrows_forced_ranges()
-        {
-            static int v = 0;
-            return v;
-        }
         struct MrowsSplit
         {
             int ranges = 0, range_groups = 0, gw = 0;
@@ -534,8 +497,6 @@ namespace nnf
             const int G = K >> 7;
             // 33 .. 64 rows: four blocks of rows leave registers for two groups per wavefront: ranges of 16 groups
             int ranges = M <= 32 ? (G + 31) / 32 : (G + 15) / 16;
-            if (mrows_forced_ranges() >= 2)
-                ranges = mrows_forced_ranges();
             const int rg = (((G + ranges - 1) / ranges) + 1) & ~1;
             const int gw = rg <= 16 ? (M <= 32 ? 2 : 1) : rg <= 32 ? 2 : rg <= 48 ? 3 : 4;
             if ((M > 32 && gw > 1) || (M > 16 && gw > 2)) // (only with a forced number of ranges)
@@ -582,8 +543,10 @@ namespace nnf
             case 3: // MFMA tile GEMM
                 return true;
             case 1: return w4a16_gemv_valu_fits(M, K);
-            case 2: return w4a16_skinny_fits(M, N, K);
-            case 4: return plan_w4a16_rows(M, N, K, num_cu, 0).seg != 0 || w4a16_mrows_fits(M, N, K, num_cu);
+            case 2: return w4a16_skinny_fits(M, N, K) || w4a16_skinny_ksplits(M, N, K) > 0;
+            case 4:
+                return plan_w4a16_rows(M, N, K, num_cu, 0).seg != 0 || w4a16_mrows_fits(M, N, K, num_cu) ||
+                       w4a16_mrows_split(M, N, K, num_cu).ranges > 0;
             default: return false;
             }
         }
@@ -636,7 +599,7 @@ namespace nnf
                 return 0;
             if (w8a8_skinny_fits(M, K))
                 return 0;
-            return plan_w8a8_sk(M, N, K, PLAN_CUS).bytes();
+            return gemm_partial_bytes(M, N, false, plan_w8a8_gemm(M, N, K));
         }
         // nnf_fused_mlp_w4a16: [ normalised x: M x H fp16 ][ h: M x I fp16 ][ partial sums of either GEMM ]
         inline size_t fused_mlp_h_offset(int M, int H) { return rms_rows(M, H); }
@@ -652,7 +615,11 @@ namespace nnf
             size_t b = plan_w4a16_sk(M, H, I, false, PLAN_CUS).bytes();
             size_t c = skinny_split_bytes(M, 2 * I, H), d = skinny_split_bytes(M, H, I);
             const size_t e = mrows_split_bytes(M, 2 * I, H), f = mrows_split_bytes(M, H, I);
-            const size_t g = gemv_scratch_bytes(M, 2 * I); // gate | up of the first GEMM at M <= 32
+            // the GEMV kernels' products ahead of an element-wise epilogue: gate | up of the first GEMM, and the
+            // second GEMM's when its residual x is the output buffer itself
+            size_t g = gemv_scratch_bytes(M, 2 * I);
+            const size_t g2 = gemv_scratch_bytes(M, H);
+            g = g > g2 ? g : g2;
             c = c > e ? c : e;
             c = c > g ? c : g;
             d = d > f ? d : f;

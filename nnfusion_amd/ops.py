@@ -4,9 +4,25 @@ torch is used for device memory and streams only; every computation happens in
 libnnf_hip_kernels.so.  A non-zero status from the library raises NnfError (the emitted host
 wrappers of the codegen path throw std::runtime_error in the same situation).
 """
+import ctypes
+
 import torch
 
 from . import _lib
+
+
+class NnfPlan(ctypes.Structure):
+    """struct nnf_plan of the C header: what a kernel-selection candidate fixes about the tile GEMM."""
+    _fields_ = [("tile_rows", ctypes.c_int), ("k_parts", ctypes.c_int)]
+
+
+def _plan_arg(plan):
+    """None, an NnfPlan or a (tile_rows, k_parts) pair -> (object to keep alive, pointer argument)."""
+    if plan is None:
+        return None, None
+    if not isinstance(plan, NnfPlan):
+        plan = NnfPlan(int(plan[0]), int(plan[1]))
+    return plan, ctypes.cast(ctypes.pointer(plan), ctypes.c_void_p)
 
 
 class NnfError(RuntimeError):
@@ -55,9 +71,13 @@ def w4a16_gemm(a, wq, scales, group=128, zp=8, out=None, workspace=None):
 VARIANTS = {"auto": 0, "gemv_valu": 1, "gemv_mfma": 2, "gemm_mfma": 3, "gemv_rows": 4}
 
 
-def w4a16_gemm_variant(a, wq, scales, variant, group=128, zp=8, out=None, workspace=None):
-    """As w4a16_gemm through one kernel variant (a key of VARIANTS); raises NnfError with status -2 when the
-    variant cannot serve the shape."""
+def w4a16_variant_supported(m, n, k, variant, group=128):
+    return bool(_lib.kernels().nnf_w4a16_variant_supported(m, n, k, group, VARIANTS[variant]))
+
+
+def w4a16_gemm_variant(a, wq, scales, variant, plan=None, group=128, zp=8, out=None, workspace=None):
+    """As w4a16_gemm through one kernel variant (a key of VARIANTS) and, for the tile GEMM, a plan (tile_rows,
+    k_parts); raises NnfError with status -2 when the variant cannot serve the shape."""
     lib = _lib.kernels()
     m, k = a.shape
     n = wq.shape[0]
@@ -66,23 +86,36 @@ def w4a16_gemm_variant(a, wq, scales, variant, group=128, zp=8, out=None, worksp
     assert a.is_contiguous() and wq.is_contiguous() and scales.is_contiguous()
     if out is None:
         out = torch.empty((m, n), dtype=torch.float16, device=a.device)
+    keep, plan_ptr = _plan_arg(plan)
     if workspace is None:
-        workspace = _ws(lib.nnf_w4a16_gemm_variant_workspace_bytes(m, n, k, group, v), a.device)
+        workspace = _ws(lib.nnf_w4a16_gemm_variant_workspace_bytes(m, n, k, group, v, plan_ptr), a.device)
     _check(lib.nnf_w4a16_gemm_variant(_stream(), a.data_ptr(), wq.data_ptr(), scales.data_ptr(), out.data_ptr(),
-                                      m, n, k, group, zp, v, workspace.data_ptr(), workspace.numel()),
+                                      m, n, k, group, zp, v, plan_ptr, workspace.data_ptr(), workspace.numel()),
            "nnf_w4a16_gemm_variant")
     return out
 
 
 def w4a16_gemm_fused(a, wq, scales, group=128, zp=8, rms_gamma=None, rms_eps=1e-6, bias=None, residual=None,
-                     act=0, out=None, workspace=None):
-    """GEMM with the fused RMSNorm prologue / bias, residual, SiLU-gate epilogues (see the C header)."""
+                     act=0, out=None, workspace=None, variant="auto", plan=None):
+    """GEMM with the fused RMSNorm prologue / bias, residual, SiLU-gate epilogues (see the C header); variant
+    "gemm_mfma" and a plan (tile_rows, k_parts) go through nnf_w4a16_gemm_fused_variant."""
     lib = _lib.kernels()
     m, k = a.shape
     n = wq.shape[0] // (2 if act == 1 else 1)
     if out is None:
         out = torch.empty((m, n), dtype=torch.float16, device=a.device)
     need = lib.nnf_w4a16_gemm_fused_workspace_bytes(m, n, k, group, act)
+    if variant != "auto" or plan is not None:
+        keep, plan_ptr = _plan_arg(plan)
+        v = VARIANTS[variant]
+        if workspace is None:
+            workspace = _ws(need + lib.nnf_w4a16_gemm_variant_workspace_bytes(m, wq.shape[0], k, group, v, plan_ptr),
+                            a.device)
+        _check(lib.nnf_w4a16_gemm_fused_variant(_stream(), a.data_ptr(), wq.data_ptr(), scales.data_ptr(),
+                                                out.data_ptr(), m, n, k, group, zp, _p(rms_gamma), float(rms_eps),
+                                                _p(bias), _p(residual), int(act), v, plan_ptr, workspace.data_ptr(),
+                                                workspace.numel()), "nnf_w4a16_gemm_fused_variant")
+        return out
     if workspace is None:
         workspace = _ws(need, a.device)
     _check(lib.nnf_w4a16_gemm_fused(_stream(), a.data_ptr(), wq.data_ptr(), scales.data_ptr(), out.data_ptr(),
@@ -91,8 +124,28 @@ def w4a16_gemm_fused(a, wq, scales, group=128, zp=8, rms_gamma=None, rms_eps=1e-
     return out
 
 
-def w8a8_gemm(a, s_tok, w, s_ch, out=None, workspace=None):
-    """Y fp16 [M,N] = fp16((float)(A . W^T) * s_tok[m] * s_ch[n]) ; a i8 [M,K], w i8 [N,K]."""
+W8A8_VARIANTS = {"auto": 0, "gemv_mfma": 1, "gemm_mfma": 2, "gemv_rows": 3}
+
+
+def w8a8_variant_supported(m, n, k, variant):
+    return bool(_lib.kernels().nnf_w8a8_variant_supported(m, n, k, W8A8_VARIANTS[variant]))
+
+
+def _w8a8_variant(a, s_tok, w, s_ch, y, acc, variant, plan, workspace):
+    lib = _lib.kernels()
+    m, k = a.shape
+    n = w.shape[0]
+    v = W8A8_VARIANTS[variant]
+    keep, plan_ptr = _plan_arg(plan)
+    if workspace is None:
+        workspace = _ws(lib.nnf_w8a8_gemm_variant_workspace_bytes(m, n, k, v, plan_ptr), a.device)
+    _check(lib.nnf_w8a8_gemm_variant(_stream(), a.data_ptr(), _p(s_tok), w.data_ptr(), _p(s_ch), _p(y), _p(acc), m, n, k,
+                                     v, plan_ptr, workspace.data_ptr(), workspace.numel()), "nnf_w8a8_gemm_variant")
+
+
+def w8a8_gemm(a, s_tok, w, s_ch, out=None, workspace=None, variant="auto", plan=None):
+    """Y fp16 [M,N] = fp16((float)(A . W^T) * s_tok[m] * s_ch[n]) ; a i8 [M,K], w i8 [N,K].  A variant (a key of
+    W8A8_VARIANTS) or plan (tile_rows, k_parts) goes through nnf_w8a8_gemm_variant."""
     lib = _lib.kernels()
     m, k = a.shape
     n = w.shape[0]
@@ -100,6 +153,9 @@ def w8a8_gemm(a, s_tok, w, s_ch, out=None, workspace=None):
     assert s_tok.dtype == torch.float32 and s_ch.dtype == torch.float32
     if out is None:
         out = torch.empty((m, n), dtype=torch.float16, device=a.device)
+    if variant != "auto" or plan is not None:
+        _w8a8_variant(a, s_tok, w, s_ch, out, None, variant, plan, workspace)
+        return out
     need = lib.nnf_w8a8_gemm_workspace_bytes(m, n, k)
     if workspace is None:
         workspace = _ws(need, a.device)
@@ -108,7 +164,7 @@ def w8a8_gemm(a, s_tok, w, s_ch, out=None, workspace=None):
     return out
 
 
-def w8a8_gemm_acc(a, w, out=None, workspace=None):
+def w8a8_gemm_acc(a, w, out=None, workspace=None, variant="auto", plan=None):
     """acc i32 [M,N] = A . W^T, exact."""
     lib = _lib.kernels()
     m, k = a.shape
@@ -116,6 +172,9 @@ def w8a8_gemm_acc(a, w, out=None, workspace=None):
     assert a.dtype == torch.int8 and w.dtype == torch.int8
     if out is None:
         out = torch.empty((m, n), dtype=torch.int32, device=a.device)
+    if variant != "auto" or plan is not None:
+        _w8a8_variant(a, None, w, None, None, out, variant, plan, workspace)
+        return out
     need = lib.nnf_w8a8_gemm_workspace_bytes(m, n, k)
     if workspace is None:
         workspace = _ws(need, a.device)

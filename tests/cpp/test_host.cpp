@@ -565,8 +565,10 @@ int main(int argc, char** argv)
         EXPECT(k8.size() == 5 && has(k8, "rocm_gemv_rows")); // 2 .. 16 rows: the row-streaming MFMA kernel
         auto k8odd = kinds(8, 4096, 4224);                   // ... which takes multiples of 256 (1024 .. 8192) only
         EXPECT(k8odd.size() == 4 && !has(k8odd, "rocm_gemv_rows"));
-        auto k16 = kinds(16, 8192, 8192); // too many activations for one workgroup's LDS: no single-pass MFMA GEMV
-        EXPECT(!has(k16, "rocm_gemv_mfma") && has(k16, "rocm_gemm_mfma"));
+        auto k16 = kinds(16, 8192, 8192); // too many activations for one workgroup's LDS: the MFMA GEMV over ranges of K
+        EXPECT(has(k16, "rocm_gemv_mfma") && has(k16, "rocm_gemm_mfma"));
+        auto k40 = kinds(40, 8192, 8192); // more rows than any GEMV kernel takes
+        EXPECT(k40.size() == 2 && !has(k40, "rocm_gemv_mfma") && !has(k40, "rocm_gemv_rows"));
         auto kbig = kinds(4096, 8192, 8192);
         EXPECT(kbig.size() == 2 && kbig[1] == "rocm_gemm_mfma");
         auto kfused = kinds(4, 256, 256, "{\"rms_norm\": true}", true);
@@ -586,7 +588,7 @@ int main(int argc, char** argv)
             if (pc->kernel->get_kernel_type() == "rocm_gemv_rows")
             {
                 ++rows;
-                CONTAINS(pc->source_code, "nnf_w4a16_gemm_variant(stream, input0, input1, input2, output0, 1, 4096, 4096, 128, 8, NNF_W4A16_GEMV_ROWS, nullptr, 0)");
+                CONTAINS(pc->source_code, "nnf_w4a16_gemm_variant(stream, input0, input1, input2, output0, 1, 4096, 4096, 128, 8, NNF_W4A16_GEMV_ROWS, nullptr, nullptr, 0)");
                 CONTAINS(pc->entry_name, "_rocm_gemv_rows_");
             }
         }

@@ -68,7 +68,9 @@ def test_mlp_workspace_contract(gpu):
     tens = _t(gpu, *datagen.mlp_case(1, m, h, i))
     need = _lib.kernels().nnf_fused_mlp_w4a16_workspace_bytes(m, h, i, 128)
     assert need >= m * i * 2
-    small = torch.empty(need - 256, dtype=torch.uint8, device=gpu)
+    # the query is an upper bound over the kernels the library may pick; a call checks what its own launches write:
+    # always the block's h tensor, which alone is M x I fp16
+    small = torch.empty(m * i * 2 - 256, dtype=torch.uint8, device=gpu)
     with pytest.raises(ops.NnfError) as e:
         ops.fused_mlp_w4a16(*tens, workspace=small)
     assert e.value.status == -3

@@ -16,23 +16,31 @@ TOL = 1e-2
 
 @pytest.fixture(params=["auto", "valu_gemv", "mfma_skinny", "rows_gemv", "mfma_rows"])
 def path(request):
-    """Runs a test once per kernel family that can serve M <= 16 (auto = the library's own choice;
-    rows_gemv = the M = 1 row-streaming kernel where it applies, otherwise the library's choice;
-    mfma_rows = the row-streaming MFMA kernel for 2 <= M <= 16 and K = 1024, 1280 .. 8192 where it applies)."""
-    from nnfusion_amd import _lib
-
-    tune = _lib.kernels().nnf_internal_tune
-    tune(0, {"auto": 0, "valu_gemv": 1, "mfma_skinny": 2, "rows_gemv": 4, "mfma_rows": 5}[request.param])
-    yield request.param
-    tune(0, 0)
+    """Runs a test once per kernel family that can serve a few rows, through nnf_w4a16_gemm_variant where the family
+    takes the shape and the library's own choice where it does not (auto = the library's own choice;
+    rows_gemv = the M = 1 row-streaming kernel; mfma_rows = the row-streaming MFMA kernel for M >= 2, in one launch
+    or over ranges of K; mfma_skinny = the MFMA GEMV kernel, likewise)."""
+    return request.param
 
 
-def _run(gpu, a, wq, s, zp=8):
+_PATH_VARIANT = {"valu_gemv": "gemv_valu", "mfma_skinny": "gemv_mfma", "rows_gemv": "gemv_rows", "mfma_rows": "gemv_rows"}
+
+
+def _run(gpu, a, wq, s, zp=8, path="auto"):
     import torch
 
     from nnfusion_amd import ops
 
-    y = ops.w4a16_gemm(torch.from_numpy(a).to(gpu), torch.from_numpy(wq).to(gpu), torch.from_numpy(s).to(gpu), zp=zp)
+    m, k = a.shape
+    n = wq.shape[0]
+    ta, tw, ts = torch.from_numpy(a).to(gpu), torch.from_numpy(wq).to(gpu), torch.from_numpy(s).to(gpu)
+    variant = _PATH_VARIANT.get(path)
+    if path == "rows_gemv" and m != 1 or path == "mfma_rows" and m == 1:
+        variant = None
+    if variant is not None and ops.w4a16_variant_supported(m, n, k, variant):
+        y = ops.w4a16_gemm_variant(ta, tw, ts, variant, zp=zp)
+    else:
+        y = ops.w4a16_gemm(ta, tw, ts, zp=zp)
     torch.cuda.synchronize()
     return y.cpu().numpy()
 
@@ -75,7 +83,7 @@ def _check(y, ref):
 def test_gemv_matches_oracle(gpu, path, m, n, k):
     print(f"case M={m} N={n} K={k}", flush=True)
     a, wq, s = datagen.w4a16_case(0, m, n, k)
-    y = _run(gpu, a, wq, s)
+    y = _run(gpu, a, wq, s, path=path)
     ref = oracle.w4a16_gemm(a, wq, s, f32_out=True)
     _check(y, ref)
 
@@ -106,7 +114,7 @@ def test_gemv_all_zero_point_is_zero(gpu, path):
     k = 512
     a, wq, s = datagen.w4a16_case(1, 2, 96, k)
     wq[:] = 0x88
-    y = _run(gpu, a, wq, s)
+    y = _run(gpu, a, wq, s, path=path)
     if path == "valu_gemv":
         assert np.all(y == 0)
     else:
@@ -122,14 +130,14 @@ def test_gemv_one_hot_reads_single_weight(gpu, path):
     for kk in (0, 1, 2, 7, 8, 31, 32, 127, 128, 129, 255, 511):
         a = np.zeros((1, k), np.float16)
         a[0, kk] = 1.0
-        y = _run(gpu, a, wq, s)
+        y = _run(gpu, a, wq, s, path=path)
         np.testing.assert_array_equal(y[0], wd[:, kk].astype(np.float16))
 
 
 @pytest.mark.parametrize("zp", [0, 7, 15])
 def test_gemv_other_zero_points(gpu, path, zp):
     a, wq, s = datagen.w4a16_case(3, 2, 128, 1024)
-    y = _run(gpu, a, wq, s, zp=zp)
+    y = _run(gpu, a, wq, s, zp=zp, path=path)
     ref = oracle.w4a16_gemm(a, wq, s, zp=zp, f32_out=True)
     _check(y, ref)
 
@@ -158,5 +166,5 @@ def test_every_kernel_variant_that_accepts_a_shape_matches_the_oracle(gpu, m, n,
                 ops.w4a16_gemm_variant(ta, tw, ts, name)
             assert e.value.status == -2
     assert "auto" in served and "gemm_mfma" in served
-    assert ("gemv_rows" in served) == (m == 1 or (m <= 32 and k % 256 == 0 and 1024 <= k <= (8192 if m <= 16 else 4096)))
+    assert ("gemv_rows" in served) == (m == 1 or (m <= 32 and k % 256 == 0 and k >= 1024))
     assert ("gemv_valu" in served) == (m <= 16)

@@ -31,33 +31,25 @@ def _check(y, ref, tol=TOL):
     assert err <= tol * max(rms, 1e-6), (err, rms)
 
 
-@pytest.fixture
-def force_gemm():
-    """Route every M through the MFMA GEMM kernel (the library would pick the skinny kernel for M <= 16)."""
-    from nnfusion_amd import _lib
-
-    tune = _lib.kernels().nnf_internal_tune
-    tune(0, 3)
-    yield
-    tune(0, 0)
+# Plans of the MFMA tile GEMM, passed per call through nnf_w4a16_gemm_variant / nnf_w4a16_gemm_fused_variant (struct
+# nnf_plan): None = the library's own choice of kernel and plan; otherwise (tile_rows, k_parts): tiles of 256, 128, 64 or
+# 32 rows by 256 columns, and the number of workgroups that share a tile (each a part of K; parts parked in the workspace
+# and added by the second launch)
+PLANS = [None, (256, 1), (256, 2), (128, 1), (128, 3), (64, 1), (64, 2), (32, 1), (32, 3)]
 
 
-# (tile, splits) of the MFMA GEMM: None = the library's own plan; tiles 1 big 256x256, 2 mid 128x128,
-# 3 small 64x256, 4 tiny 32x256; splits = K ranges (> 1, and always for the small tile: fp32 partial sums + reduction pass)
-PLANS = [None, (1, 1), (1, 2), (2, 1), (2, 3), (3, 1), (3, 2), (4, 1), (4, 3)]
-
-
-@pytest.fixture(params=PLANS, ids=lambda p: "auto" if p is None else f"tile{p[0]}-splits{p[1]}")
+@pytest.fixture(params=PLANS, ids=lambda p: "auto" if p is None else f"rows{p[0]}-parts{p[1]}")
 def plan(request):
-    from nnfusion_amd import _lib
+    """Keyword arguments for ops.w4a16_gemm_fused / _gemm below."""
+    return {} if request.param is None else {"variant": "gemm_mfma", "plan": request.param}
 
-    tune = _lib.kernels().nnf_internal_tune
-    if request.param is not None:
-        tune(3, request.param[0])
-        tune(4, request.param[1])
-    yield request.param
-    tune(3, 0)
-    tune(4, 0)
+
+def _gemm(ta, tw, ts, plan_kw, workspace=None):
+    from nnfusion_amd import ops
+
+    if plan_kw:
+        return ops.w4a16_gemm_variant(ta, tw, ts, plan_kw["variant"], plan=plan_kw["plan"], workspace=workspace)
+    return ops.w4a16_gemm(ta, tw, ts, workspace=workspace)
 
 
 def _big_ws(gpu):
@@ -75,7 +67,7 @@ def test_gemm_every_tile_plan_matches_oracle(gpu, plan, m, n, k):
     print(f"case plan={plan} M={m} N={n} K={k}", flush=True)
     a, wq, s = datagen.w4a16_case(2, m, n, k)
     ta, tw, ts = _t(gpu, a, wq, s)
-    y = ops.w4a16_gemm(ta, tw, ts, workspace=_big_ws(gpu))
+    y = _gemm(ta, tw, ts, plan, workspace=_big_ws(gpu))
     torch.cuda.synchronize()
     _check(y.cpu().numpy(), oracle.w4a16_gemm(a, wq, s, f32_out=True))
 
@@ -99,14 +91,15 @@ def test_gemm_matches_oracle(gpu, m, n, k):
 
 
 @pytest.mark.parametrize("m", [1, 5, 16])
-def test_gemm_kernel_serves_small_m(gpu, force_gemm, m):
+def test_gemm_kernel_serves_small_m(gpu, m):
+    """The tile GEMM asked for by variant (the library's own choice for these shapes is a GEMV kernel)."""
     import torch
 
     from nnfusion_amd import ops
 
     a, wq, s = datagen.w4a16_case(4, m, 320, 512)
     ta, tw, ts = _t(gpu, a, wq, s)
-    y = ops.w4a16_gemm(ta, tw, ts, workspace=_big_ws(gpu))
+    y = ops.w4a16_gemm_variant(ta, tw, ts, "gemm_mfma", workspace=_big_ws(gpu))
     torch.cuda.synchronize()
     _check(y.cpu().numpy(), oracle.w4a16_gemm(a, wq, s, f32_out=True))
 
@@ -168,9 +161,9 @@ def test_fused_bias_residual(gpu, plan):
     res = datagen.normal_f16(6, datagen.S_RES, (m, n))
     ta, tw, ts, tb, tr = _t(gpu, a, wq, s, bias, res)
     ws = _big_ws(gpu)
-    y_b = ops.w4a16_gemm_fused(ta, tw, ts, bias=tb, workspace=ws).cpu().numpy()
-    y_r = ops.w4a16_gemm_fused(ta, tw, ts, residual=tr, workspace=ws).cpu().numpy()
-    y_br = ops.w4a16_gemm_fused(ta, tw, ts, bias=tb, residual=tr, workspace=ws).cpu().numpy()
+    y_b = ops.w4a16_gemm_fused(ta, tw, ts, bias=tb, workspace=ws, **plan).cpu().numpy()
+    y_r = ops.w4a16_gemm_fused(ta, tw, ts, residual=tr, workspace=ws, **plan).cpu().numpy()
+    y_br = ops.w4a16_gemm_fused(ta, tw, ts, bias=tb, residual=tr, workspace=ws, **plan).cpu().numpy()
     torch.cuda.synchronize()
     d = oracle.w4a16_gemm(a, wq, s)  # fp16 tensor of the unfused Dot
     ref_b = oracle.add_f16(d, np.broadcast_to(bias, (m, n)).copy())
@@ -194,8 +187,8 @@ def test_fused_bias_residual_ragged_columns(gpu, plan, m, n, k):
     res = datagen.normal_f16(13, datagen.S_RES, (m, n))
     ta, tw, ts, tb, tr = _t(gpu, a, wq, s, bias, res)
     ws = _big_ws(gpu)
-    y = ops.w4a16_gemm(ta, tw, ts, workspace=ws).cpu().numpy()
-    y_br = ops.w4a16_gemm_fused(ta, tw, ts, bias=tb, residual=tr, workspace=ws).cpu().numpy()
+    y = _gemm(ta, tw, ts, plan, workspace=ws).cpu().numpy()
+    y_br = ops.w4a16_gemm_fused(ta, tw, ts, bias=tb, residual=tr, workspace=ws, **plan).cpu().numpy()
     torch.cuda.synchronize()
     d = oracle.w4a16_gemm(a, wq, s)
     _check(y, oracle.w4a16_gemm(a, wq, s, f32_out=True))
@@ -210,7 +203,7 @@ def test_fused_silu_gate_ragged_columns(gpu, plan):
     m, n, k = 70, 100, 256
     a, wq, s = datagen.w4a16_case(14, m, 2 * n, k)
     ta, tw, ts = _t(gpu, a, wq, s)
-    y = ops.w4a16_gemm_fused(ta, tw, ts, act=1, workspace=_big_ws(gpu)).cpu().numpy()
+    y = ops.w4a16_gemm_fused(ta, tw, ts, act=1, workspace=_big_ws(gpu), **plan).cpu().numpy()
     torch.cuda.synchronize()
     gu = oracle.w4a16_gemm(a, wq, s)
     ref = oracle.silu_mul_f16(np.ascontiguousarray(gu[:, :n]), np.ascontiguousarray(gu[:, n:]))
@@ -228,7 +221,7 @@ def test_fused_rmsnorm_prologue(gpu, plan):
     a, wq, s = datagen.w4a16_case(7, m, n, k)
     gamma = datagen.normal_f16(7, datagen.S_GAMMA, (k,), 1.0, 0.1)
     ta, tw, ts, tg = _t(gpu, a, wq, s, gamma)
-    y = ops.w4a16_gemm_fused(ta, tw, ts, rms_gamma=tg, rms_eps=1e-6, workspace=_big_ws(gpu)).cpu().numpy()
+    y = ops.w4a16_gemm_fused(ta, tw, ts, rms_gamma=tg, rms_eps=1e-6, workspace=_big_ws(gpu), **plan).cpu().numpy()
     torch.cuda.synchronize()
     xn = oracle.rmsnorm_f16(a, gamma, 1e-6)
     _check(y, oracle.w4a16_gemm(xn, wq, s, f32_out=True))
@@ -242,7 +235,7 @@ def test_fused_silu_gate(gpu, plan):
     m, n, k = 150, 192, 512  # n = intermediate size; weights hold 2n rows (gate then up)
     a, wq, s = datagen.w4a16_case(8, m, 2 * n, k)
     ta, tw, ts = _t(gpu, a, wq, s)
-    y = ops.w4a16_gemm_fused(ta, tw, ts, act=1, workspace=_big_ws(gpu)).cpu().numpy()
+    y = ops.w4a16_gemm_fused(ta, tw, ts, act=1, workspace=_big_ws(gpu), **plan).cpu().numpy()
     torch.cuda.synchronize()
     gu = oracle.w4a16_gemm(a, wq, s)
     g = np.ascontiguousarray(gu[:, :n])

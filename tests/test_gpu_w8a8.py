@@ -15,28 +15,28 @@ def _t(gpu, *arrays):
     return [torch.from_numpy(np.ascontiguousarray(a)).to(gpu) for a in arrays]
 
 
-# "auto": the library's own choice (the M = 1 / M <= 16 / M <= 32 kernels where they apply); "skinny": the split-K
-# M <= 16 kernel; "mfma_rows": the row-streaming MFMA kernel (2 <= M <= 32, K = 1024 .. 16384 in multiples of 256); otherwise the MFMA GEMM with a
-# forced tile (1 big 256x256, 2 mid 128x128, 3 small 64x256) and number of K ranges (int32 partial sums,
-# added exactly by the reduction pass)
-@pytest.fixture(params=["auto", "skinny", "mfma_rows", (0, 0), (1, 1), (1, 2), (2, 1), (2, 3), (3, 1), (3, 2)],
-                ids=lambda p: p if isinstance(p, str) else f"gemm-tile{p[0]}-splits{p[1]}")
+# Kernel families, asked for per call through nnf_w8a8_gemm_variant where the family takes the shape (the library's own
+# choice where it does not): "auto"; "skinny": the split-K M <= 16 kernel; "mfma_rows": the row-streaming MFMA kernel
+# (2 <= M <= 32, K = 1024 .. 16384 in multiples of 256); otherwise the MFMA tile GEMM with a plan (tile_rows, k_parts):
+# tiles of 256 x 256, 128 x 128 or 64 x 256 outputs (0: the library's choice) and the number of K ranges (int32 partial
+# sums, added exactly by the reduction pass)
+@pytest.fixture(params=["auto", "skinny", "mfma_rows", (0, 0), (256, 1), (256, 2), (128, 1), (128, 3), (64, 1), (64, 2)],
+                ids=lambda p: p if isinstance(p, str) else f"gemm-rows{p[0]}-parts{p[1]}")
 def path(request):
-    from nnfusion_amd import _lib
+    return request.param
 
-    tune = _lib.kernels().nnf_internal_tune
-    if request.param == "skinny":
-        tune(0, 2)  # the M <= 16 kernel where it applies (never the M = 1 row-streaming one)
-    elif request.param == "mfma_rows":
-        tune(0, 5)
-    elif request.param != "auto":
-        tune(0, 3)
-        tune(3, request.param[0])
-        tune(4, request.param[1])
-    yield request.param
-    tune(0, 0)
-    tune(3, 0)
-    tune(4, 0)
+
+def _kw(path, m, n, k):
+    """Keyword arguments of ops.w8a8_gemm / w8a8_gemm_acc for a fixture value."""
+    from nnfusion_amd import ops
+
+    if path == "skinny":
+        return {"variant": "gemv_mfma"} if ops.w8a8_variant_supported(m, n, k, "gemv_mfma") else {}
+    if path == "mfma_rows":
+        return {"variant": "gemv_rows"} if m > 1 and ops.w8a8_variant_supported(m, n, k, "gemv_rows") else {}
+    if path == "auto":
+        return {}
+    return {"variant": "gemm_mfma", "plan": path}
 
 
 def _big_ws(gpu):
@@ -69,8 +69,9 @@ def test_accumulators_bit_exact(gpu, path, m, n, k):
     a, s_tok, w, s_ch = datagen.w8a8_case(0, m, n, k)
     ta, tw, tst, tsc = _t(gpu, a, w, s_tok, s_ch)
     ws = _big_ws(gpu)
-    acc = ops.w8a8_gemm_acc(ta, tw, workspace=ws).cpu().numpy()
-    y = ops.w8a8_gemm(ta, tst, tw, tsc, workspace=ws).cpu().numpy()
+    kw = _kw(path, m, n, k)
+    acc = ops.w8a8_gemm_acc(ta, tw, workspace=ws, **kw).cpu().numpy()
+    y = ops.w8a8_gemm(ta, tst, tw, tsc, workspace=ws, **kw).cpu().numpy()
     torch.cuda.synchronize()
     ref = oracle.w8a8_acc(a, w)
     assert np.array_equal(acc, ref)
@@ -90,7 +91,7 @@ def test_extreme_values_do_not_overflow(gpu, path):
     w = np.full((n, k), 127, np.int8)
     w[::2] = -127
     ta, tw = _t(gpu, a, w)
-    acc = ops.w8a8_gemm_acc(ta, tw, workspace=_big_ws(gpu)).cpu().numpy()
+    acc = ops.w8a8_gemm_acc(ta, tw, workspace=_big_ws(gpu), **_kw(path, m, n, k)).cpu().numpy()
     torch.cuda.synchronize()
     assert np.array_equal(acc, oracle.w8a8_acc(a, w))
     assert abs(int(acc[0, 1])) == 8192 * 127 * 127
