@@ -27,6 +27,11 @@
  *   scales  fp16  [N, K/group]      one scale per output channel and K-group (group = 128)
  *   zp      int   scalar            zero point (8): W[n,k] = (q[n,k] - zp) * scales[n, k/group]
  *   Y       fp16  [M, N]            Y = A . W^T, accumulated in fp32, rounded to nearest even
+ * Input range: any finite fp16 activations, subnormals included.  No kernel rescales the activations; the
+ * 4-bit weights are decoded to exact fp16 integers (q - zp, or q plus a constant that is removed from the fp32
+ * sum), so a product a * (q - zp) is exact in fp32 whatever the magnitude of a.  The scales are applied in fp32
+ * (GEMV kernels: to the fp32 sum of a group) or as fp16((q - zp) * scale) weights (tile GEMM); a result beyond
+ * the fp16 range becomes +-inf as in any fp16 tensor.
  *   W8A8:   A i8 [M,K], s_tok f32 [M], W i8 [N,K], s_ch f32 [N], acc i32 [M,N] (exact),
  *           Y = fp16( (float)acc * s_tok[m] * s_ch[n] ) evaluated left to right in fp32
  */

@@ -15,12 +15,13 @@
 //   * the group scales of all the workgroup's rows (a contiguous block of S) are fetched into LDS in the
 //     prologue, so that a row can go to any wavefront;
 //   * a lane always meets the same 32 (x SEG) activations, whatever the row: they live in registers for
-//     the whole kernel, already paired and pre-scaled for the nibble trick below, and nothing but the
+//     the whole kernel, already paired for the nibble trick below, and nothing but the
 //     weights is read per row (plus two bytes of scale per lane and load, from LDS);
-//   * nibbles become fp16 with one v_and_or_b32 per pair: (q | 0x6400) = 1024 + q and, four bits up,
-//     1024 + 16 q; the dot products run on v_dot2_f32_f16 (fp32 accumulate) against (a_even, a_odd / 16),
-//     and the constant part  (1024 + zp) sum a_even + (64 + zp) sum a_odd  of a lane's sum is the same
-//     for every row: it is computed once and used as the negative initial accumulator;
+//   * nibbles become fp16 with one v_and_or_b32 per pair: (q | 0x6400) = 1024 + q (0x6400 is 1024 with an ulp
+//     of 1) and, for a nibble four bits up, (16 q | 0x5400) = 64 + q (0x5400 is 64 with an ulp of 1/16): both
+//     exact, whatever the activations are; the dot products run on v_dot2_f32_f16 (fp32 accumulate) against
+//     (a_even, a_odd), and the constant part  (1024 + zp) sum a_even + (64 + zp) sum a_odd  of a lane's sum is
+//     the same for every row: it is computed once and used as the negative initial accumulator;
 //   * the 32 weights of a lane and load share one group scale (a group of 128 is 4 lanes); the lane's
 //     partial sum is multiplied by it in fp32, the 64 lanes are added with DPP row rotations, and the
 //     row's result is parked in LDS; outputs are written once, after the last row.
@@ -57,7 +58,7 @@ namespace nnf
 
     // LDS (bytes):  ring   [WAVES wavefronts][D rows][SEG] x 1 KiB
     //               act    K/8 16-byte units a[8u .. 8u+8), rounded up to whole KiB: first as in memory, then
-    //                      as (a0,a4) (a1,a5)/16 (a2,a6) (a3,a7)/16; followed by four units of zeros (what a
+    //                      as (a0,a4) (a1,a5) (a2,a6) (a3,a7); followed by four units of zeros (what a
     //                      lane past the end of K multiplies with)
     //               corr   one fp32 per unit: its part of the constant that the nibble trick adds to a row
     //               scales [rows of the workgroup][K/128] fp16 as in memory, rounded up to whole KiB
@@ -75,8 +76,9 @@ namespace nnf
                                                                          int rows_q, int rows_r, int pack)
     {
         extern __shared__ uintx4 lds[];
-        uint32_t MAGIC, MASK_LO, MASK_HI;
+        uint32_t MAGIC, MAGIC_HI, MASK_LO, MASK_HI;
         asm volatile("v_mov_b32 %0, 0x64006400" : "=v"(MAGIC));
+        asm volatile("v_mov_b32 %0, 0x54005400" : "=v"(MAGIC_HI));
         asm volatile("s_mov_b32 %0, 0x000F000F" : "=s"(MASK_LO));
         asm volatile("s_mov_b32 %0, 0x00F000F0" : "=s"(MASK_HI));
         const int tid = threadIdx.x;
@@ -171,21 +173,18 @@ namespace nnf
 
         // ---- activations: prepared once per workgroup, then LDS -> registers ------------------------------
         // A lane of a fetching wavefront gets back exactly the unit it asked for (no barrier needed for that):
-        // it stores the unit as (a0,a4) (a1,a5)/16 (a2,a6) (a3,a7)/16 and, next to it, the unit's part of the
+        // it stores the unit as (a0,a4) (a1,a5) (a2,a6) (a3,a7) and, next to it, the unit's part of the
         // constant  (1024 + zp) sum a_even + (64 + zp) sum a_odd  that the nibble trick adds to every row.
         // Only the weights asked for above may still be in flight afterwards: the scales have landed too.
         __builtin_amdgcn_s_waitcnt(rows_vmcnt(D0 * SEG));
         if (a_loader)
         {
-            const half2_t sixteenth = half2_t{(half_t)0.0625f, (half_t)0.0625f};
             const float ce = -(1024.0f + (float)zp);
-            const float co = -16.0f * (64.0f + (float)zp);
+            const float co = -(64.0f + (float)zp);
             for (int u0 = wave * 64; u0 < a_units; u0 += WAVES * 64)
             {
                 const int u = u0 + lane;
-                uintx4 a = permute_a8(act[u]);
-                a.y = as_u32(as_half2(a.y) * sixteenth);
-                a.w = as_u32(as_half2(a.w) * sixteenth);
+                const uintx4 a = permute_a8(act[u]);
                 const half2_t x = as_half2(a.x), y = as_half2(a.y), z = as_half2(a.z), w = as_half2(a.w);
                 const float se = ((float)x.x + (float)x.y) + ((float)z.x + (float)z.y);
                 const float so = ((float)y.x + (float)y.y) + ((float)w.x + (float)w.y);
@@ -235,9 +234,9 @@ namespace nnf
                     const uint32_t w8 = w >> 8;
                     const uintx4 a = areg[j][d];
                     t = dot2(as_half2((w & MASK_LO) | MAGIC), as_half2(a.x), t);  // 1024 + (q0, q4)
-                    t = dot2(as_half2((w & MASK_HI) | MAGIC), as_half2(a.y), t);  // 1024 + 16 (q1, q5)
+                    t = dot2(as_half2((w & MASK_HI) | MAGIC_HI), as_half2(a.y), t); // 64 + (q1, q5)
                     t = dot2(as_half2((w8 & MASK_LO) | MAGIC), as_half2(a.z), t); // 1024 + (q2, q6)
-                    t = dot2(as_half2((w8 & MASK_HI) | MAGIC), as_half2(a.w), t); // 1024 + 16 (q3, q7)
+                    t = dot2(as_half2((w8 & MASK_HI) | MAGIC_HI), as_half2(a.w), t); // 64 + (q3, q7)
                 }
                 v = __builtin_fmaf(t, sv[j], v);
             }

@@ -20,7 +20,7 @@
 //     piece it fetches), so the 128-bit operand reads are conflict free.
 //   * The activations never touch LDS: lane (m, kq) loads the 64 bytes of row m that its MFMA operand holds of
 //     each of the wavefront's groups, once, and keeps them (16 VGPRs per group; hence K <= 8192), in the pair
-//     order and with the 1/16 of the nibble trick; the constant part of a group sum is an MFMA against a
+//     order of the nibble trick; the constant part of a group sum is an MFMA against a
 //     constant operand and becomes the (negative) initial accumulator of the group (see w4a16_skinny.hip).
 //   * Per step: GW x 4 MFMAs (v_mfma_f32_16x16x32_f16, weights as the B operand) per wavefront, the group sum
 //     times the group scale in fp32; per tile the eight partial 16 x 16 tiles meet in LDS (one LDS-only barrier,
@@ -47,13 +47,12 @@ namespace nnf
 
     // ---- pieces shared by the two forms of the kernel ----------------------------------------------------------------
     // The activations of a wavefront as loaded -> the MFMA operand order of the nibble trick (pairs (a0,a4) (a1,a5)
-    // (a2,a6) (a3,a7), the odd words times 1/16), and per group the constant part of its sum (an MFMA against a
+    // (a2,a6) (a3,a7)), and per group the constant part of its sum (an MFMA against a
     // constant operand), negative, as the initial accumulator of the group.
     template <int MB, int GA>
     __device__ __forceinline__ void mrows_prepare_a(uintx4 (&areg)[MB][GA][4], floatx4 (&ncorr)[MB][GA], int zp)
     {
-        const half2_t sixteenth = half2_t{(half_t)0.0625f, (half_t)0.0625f};
-        const half_t ceh = (half_t)(-(1024.0f + (float)zp)), coh = (half_t)(-16.0f * (64.0f + (float)zp)); // exact
+        const half_t ceh = (half_t)(-(1024.0f + (float)zp)), coh = (half_t)(-(64.0f + (float)zp)); // exact
         const uint32_t ce2 = as_u32(half2_t{ceh, ceh}), co2 = as_u32(half2_t{coh, coh});
         const uintx4 cvec = {ce2, co2, ce2, co2};
 #pragma unroll
@@ -65,9 +64,7 @@ namespace nnf
 #pragma unroll
                 for (int j = 0; j < 4; ++j)
                 {
-                    uintx4 a = permute_a8(areg[mb][g][j]);
-                    a.y = as_u32(as_half2(a.y) * sixteenth);
-                    a.w = as_u32(as_half2(a.w) * sixteenth);
+                    const uintx4 a = permute_a8(areg[mb][g][j]);
                     areg[mb][g][j] = a;
                     t = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, a), __builtin_bit_cast(half8_t, cvec), t,
                                                                0, 0, 0);
@@ -77,11 +74,12 @@ namespace nnf
     }
 
     // One group of 128 along K: the lane's 16 bytes of weights (32 nibbles) against group ga of the activations,
-    // the fp32 group sum times the group's scale onto acc.  consts = {0x64006400, 0x000F000F, 0x00F000F0}.
+    // the fp32 group sum times the group's scale onto acc.  MAGIC = 0x64006400 (1024 + q for a nibble in bits 0..3),
+    // MAGIC_HI = 0x54005400 (64 + q for a nibble in bits 4..7), MASK_LO = 0x000F000F, MASK_HI = 0x00F000F0.
     template <int MB, int GA>
     __device__ __forceinline__ void mrows_group(floatx4 (&acc)[MB], const uintx4 (&areg)[MB][GA][4],
                                                 const floatx4 (&ncorr)[MB][GA], int ga, uintx4 wv, float scale, uint32_t MAGIC,
-                                                uint32_t MASK_LO, uint32_t MASK_HI)
+                                                uint32_t MAGIC_HI, uint32_t MASK_LO, uint32_t MASK_HI)
     {
         floatx4 t[MB];
 #pragma unroll
@@ -95,9 +93,9 @@ namespace nnf
             const uint32_t w8 = w >> 8;
             uintx4 bq;
             bq.x = (w & MASK_LO) | MAGIC;  // 1024 + (q0, q4)
-            bq.y = (w & MASK_HI) | MAGIC;  // 1024 + 16 (q1, q5)
+            bq.y = (w & MASK_HI) | MAGIC_HI; // 64 + (q1, q5)
             bq.z = (w8 & MASK_LO) | MAGIC; // 1024 + (q2, q6)
-            bq.w = (w8 & MASK_HI) | MAGIC; // 1024 + 16 (q3, q7)
+            bq.w = (w8 & MASK_HI) | MAGIC_HI; // 64 + (q3, q7)
 #pragma unroll
             for (int mb = 0; mb < MB; ++mb)
                 t[mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, areg[mb][ga][j]),
@@ -165,8 +163,9 @@ namespace nnf
         constexpr int LT = GW + 1;             // loads per step and wavefront (weights + scales)
         constexpr int SC_LANES = (GW + 1) / 2; // 4-byte scale loads per row (odd GW: one half-word of a neighbour comes along)
         extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-        uint32_t MAGIC, MASK_LO, MASK_HI;
+        uint32_t MAGIC, MAGIC_HI, MASK_LO, MASK_HI;
         asm volatile("v_mov_b32 %0, 0x64006400" : "=v"(MAGIC));
+        asm volatile("v_mov_b32 %0, 0x54005400" : "=v"(MAGIC_HI));
         asm volatile("s_mov_b32 %0, 0x000F000F" : "=s"(MASK_LO));
         asm volatile("s_mov_b32 %0, 0x00F000F0" : "=s"(MASK_HI));
 
@@ -281,7 +280,7 @@ namespace nnf
                 slot ^= 1;
 #pragma unroll
                 for (int g = 0; g < GW; ++g)
-                    mrows_group<MB, GA>(acc, areg, ncorr, st * GW + g, wv[g], sv[g], MAGIC, MASK_LO, MASK_HI);
+                    mrows_group<MB, GA>(acc, areg, ncorr, st * GW + g, wv[g], sv[g], MAGIC, MAGIC_HI, MASK_LO, MASK_HI);
             }
             mrows_reduce_park<MB>(acc, red, red_addr, parked_addr, it & 1, it, M, tid);
         }
@@ -321,8 +320,9 @@ namespace nnf
         constexpr int LT = GW + 1;             // loads per step and wavefront (weights + scales)
         constexpr int SC_LANES = GW / 2 + 1;   // 4-byte scale loads per row: GW groups from any 2-byte offset
         extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-        uint32_t MAGIC, MASK_LO, MASK_HI;
+        uint32_t MAGIC, MAGIC_HI, MASK_LO, MASK_HI;
         asm volatile("v_mov_b32 %0, 0x64006400" : "=v"(MAGIC));
+        asm volatile("v_mov_b32 %0, 0x54005400" : "=v"(MAGIC_HI));
         asm volatile("s_mov_b32 %0, 0x000F000F" : "=s"(MASK_LO));
         asm volatile("s_mov_b32 %0, 0x00F000F0" : "=s"(MASK_HI));
 
@@ -437,7 +437,7 @@ namespace nnf
                     slot ^= 1;
 #pragma unroll
                     for (int g = 0; g < GW; ++g)
-                        mrows_group<MB, GA>(acc, areg, ncorr, st * GW + g, wv[g], sv[g], MAGIC, MASK_LO, MASK_HI);
+                        mrows_group<MB, GA>(acc, areg, ncorr, st * GW + g, wv[g], sv[g], MAGIC, MAGIC_HI, MASK_LO, MASK_HI);
                 }
                 mrows_reduce_park<MB>(acc, red, red_addr, parked_addr, it & 1, it, M, tid);
             }

@@ -14,13 +14,14 @@
 //   * the dot products run on v_mfma_f32_16x16x32_f16 with the weight tile as the B operand
 //     (columns = n) and the M <= 16 activation rows as the A operand (rows = m), so the cost per
 //     weight byte does not depend on M.  The A operand is staged once per workgroup in LDS (already
-//     permuted and pre-scaled); with up to two groups per wavefront it is then kept in registers --
+//     permuted); with up to two groups per wavefront it is then kept in registers --
 //     and from six rows on each wavefront loads its share straight from global memory into those
 //     registers, in the MFMA operand layout (16 rows x 64 bytes per load), instead of the staging;
-//   * nibbles are turned into fp16 with one v_and_or_b32 per pair: (q | 0x6400) = 1024 + q, and a
-//     nibble four bits up gives 1024 + 16 q.  Instead of subtracting the 1024 / zero point from
-//     every weight, the activations of the "16 q" slots are pre-divided by 16 and the constant part
-//         corr[m, group] = (1024 + zp) * sum_even a + (64 + zp) * 16 * sum_odd (a / 16)
+//   * nibbles are turned into fp16 with one v_and_or_b32 per pair: (q | 0x6400) = 1024 + q (0x6400 is
+//     1024 with an ulp of 1), and a nibble four bits up gives (16 q | 0x5400) = 64 + q (0x5400 is 64
+//     with an ulp of 1/16): both exact, and the activations are used as they are.  Instead of
+//     subtracting the 1024 / 64 and the zero point from every weight, the constant part
+//         corr[m, group] = (1024 + zp) * sum_even a + (64 + zp) * sum_odd a
 //     is computed once per wavefront (one MFMA chain against a constant operand) and used as the
 //     negative initial accumulator of each group.  Products are exact in fp32, the sum of a group
 //     is of order 1e4 at fp32 precision, i.e. an absolute error of ~1e-3 on a group sum of order 50;
@@ -41,7 +42,7 @@ namespace nnf
     // LDS, in this order (A_REGS: the partial sums and the parked outputs reuse the space of the staged
     // activations, which are only needed until every wavefront has copied its share into registers):
     //   activations as 16-byte units  unit(m, c, kq, j) = m*(16 G + 1) + (c*4 + kq)*4 + j  holding
-    //       the eight fp16  a[m][c*128 + kq*32 + j*8 + {0,4,1,5,2,6,3,7}]  with slots 2,3,6,7 (odd k) times 1/16
+    //       the eight fp16  a[m][c*128 + kq*32 + j*8 + {0,4,1,5,2,6,3,7}]
     //       (a row of A is staged in memory order; the odd row stride keeps rows on different banks)
     //   ncorr    [G][16 m] fp32: constant part of every group sum, negated
     //   scales   sc[2][16 rows][G] fp16 (as in memory), each copy padded to 16 bytes
@@ -83,8 +84,9 @@ namespace nnf
         static_assert(!A_REGS || H == 1, "register-resident activations only with one pass");
         extern __shared__ uintx4 lds[];
         // volatile: the vector move must stay here, where every lane is active
-        uint32_t MAGIC, MASK_LO, MASK_HI;
+        uint32_t MAGIC, MAGIC_HI, MASK_LO, MASK_HI;
         asm volatile("v_mov_b32 %0, 0x64006400" : "=v"(MAGIC));
+        asm volatile("v_mov_b32 %0, 0x54005400" : "=v"(MAGIC_HI));
         asm volatile("s_mov_b32 %0, 0x000F000F" : "=s"(MASK_LO));
         asm volatile("s_mov_b32 %0, 0x00F000F0" : "=s"(MASK_HI));
         // ---- up to the first loads: as few instructions as possible ----------------------------------------
@@ -261,15 +263,12 @@ namespace nnf
         // loading its own operand straight from global memory would cost 8 load instructions per
         // wavefront, almost all of whose lanes are redundant.
         // The constant part of a group sum,
-        //     corr[m, group] = (1024 + zp) * sum_even a + 16 (64 + zp) * sum_odd (a / 16),
+        //     corr[m, group] = (1024 + zp) * sum_even a + (64 + zp) * sum_odd a,
         // is accumulated on the way: the 16 units of a group sit in 16 consecutive lanes.
-        const half2_t sixteenth = half2_t{(half_t)0.0625f, (half_t)0.0625f};
         const float ce = -(1024.0f + (float)zp);
-        const float co = -16.0f * (64.0f + (float)zp);
+        const float co = -(64.0f + (float)zp);
         auto stage_unit = [&](uintx4 a, int m, int u) {
             a = permute_a8(a);
-            a.y = as_u32(as_half2(a.y) * sixteenth);
-            a.w = as_u32(as_half2(a.w) * sixteenth);
             lds[m * row_units + u] = a;
             const half2_t x = as_half2(a.x), y = as_half2(a.y), z = as_half2(a.z), w = as_half2(a.w);
             float se = ((float)x.x + (float)x.y) + ((float)z.x + (float)z.y);
@@ -331,9 +330,9 @@ namespace nnf
         // A_REGS without direct loads: the operand and its constants are read from LDS once
         if (A_REGS && direct)
         {
-            // the pair order and the 1/16 of the nibble trick in registers; the constant part of a group sum is
+            // the pair order of the nibble trick in registers; the constant part of a group sum is
             // a product with a constant vector: four MFMAs whose B operand is (ce, co, ce, co) for every column
-            const half_t ceh = (half_t)ce, coh = (half_t)co; // -(1024 + zp) and -16 (64 + zp): exact in fp16
+            const half_t ceh = (half_t)ce, coh = (half_t)co; // -(1024 + zp) and -(64 + zp): exact in fp16
             const uint32_t ce2 = as_u32(half2_t{ceh, ceh}), co2 = as_u32(half2_t{coh, coh});
             const uintx4 cvec = {ce2, co2, ce2, co2};
 #pragma unroll
@@ -343,9 +342,7 @@ namespace nnf
 #pragma unroll
                 for (int j = 0; j < 4; ++j)
                 {
-                    uintx4 a = permute_a8(areg[A_REGS ? c : 0][j]);
-                    a.y = as_u32(as_half2(a.y) * sixteenth);
-                    a.w = as_u32(as_half2(a.w) * sixteenth);
+                    const uintx4 a = permute_a8(areg[A_REGS ? c : 0][j]);
                     areg[A_REGS ? c : 0][j] = a;
                     t = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, a),
                                                                __builtin_bit_cast(half8_t, cvec), t, 0, 0, 0);
@@ -408,9 +405,9 @@ namespace nnf
                     uint32_t w8 = w >> 8;
                     uintx4 b;
                     b.x = (w & MASK_LO) | MAGIC;  // 1024 + (q0, q4)
-                    b.y = (w & MASK_HI) | MAGIC;  // 1024 + 16 (q1, q5)
+                    b.y = (w & MASK_HI) | MAGIC_HI; // 64 + (q1, q5)
                     b.z = (w8 & MASK_LO) | MAGIC; // 1024 + (q2, q6)
-                    b.w = (w8 & MASK_HI) | MAGIC; // 1024 + 16 (q3, q7)
+                    b.w = (w8 & MASK_HI) | MAGIC_HI; // 64 + (q3, q7)
                     t = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, a_op(h, c, j)),
                                                                __builtin_bit_cast(half8_t, b), t, 0, 0, 0);
                 }

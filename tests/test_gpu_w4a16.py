@@ -88,6 +88,21 @@ def test_gemv_matches_oracle(gpu, path, m, n, k):
     _check(y, ref)
 
 
+@pytest.mark.parametrize("log2_scale", [-12, -16])
+@pytest.mark.parametrize("m,n,k", [(1, 4096, 4096), (1, 512, 11008), (4, 300, 2048), (16, 1040, 8192), (16, 520, 11008),
+                                   (24, 300, 4096), (24, 300, 8192), (36, 300, 3584)])
+def test_gemv_small_activations_lose_nothing(gpu, path, m, n, k, log2_scale):
+    """Activations scaled down by 2^12 and 2^16 (into and below the fp16 subnormal range), on every kernel family
+    and on the forms over ranges of K: no kernel may rescale them on the way (a 1/16 on the activations of the high
+    nibbles would drop their low bits below 2^-10).  Same tolerance as everywhere, against the oracle on the same
+    fp16 inputs."""
+    a, wq, s = datagen.w4a16_case(9, m, n, k)
+    a = (a.astype(np.float32) * np.float32(2.0 ** log2_scale)).astype(np.float16)
+    y = _run(gpu, a, wq, s, path=path)
+    ref = oracle.w4a16_gemm(a, wq, s, f32_out=True)
+    _check(y, ref)
+
+
 def test_gemv_very_large_n_parks_outputs_in_more_workgroups(gpu):
     """N so large that one workgroup per CU could not park its tiles' outputs in LDS: the launcher uses more,
     shorter workgroups.  Checked on sampled columns."""
