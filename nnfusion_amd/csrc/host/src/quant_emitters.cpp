@@ -144,14 +144,11 @@ namespace nnfusion
                     const size_t N = w[0];
                     if (!nnf::workspace::w4a16_variant_fits((int)M, (int)N, (int)K, VARIANT))
                         return nullptr;
-                    size_t ws_bytes = 0;
-                    if (VARIANT == 3)
-                        ws_bytes = nnf::workspace::plan_w4a16_sk((int)M, (int)N, (int)K, false, nnf::workspace::PLAN_CUS).bytes();
-                    // the GEMV kernels over ranges of K (activations beyond one workgroup's LDS / registers): fp32 partial sums
-                    if (VARIANT == 2 && !nnf::workspace::w4a16_skinny_fits((int)M, (int)N, (int)K))
-                        ws_bytes = nnf::workspace::skinny_split_bytes((int)M, (int)N, (int)K);
-                    if (VARIANT == 4 && M > 1 && !nnf::workspace::w4a16_mrows_fits((int)M, (int)N, (int)K, nnf::workspace::PLAN_CUS))
-                        ws_bytes = nnf::workspace::mrows_split_bytes((int)M, (int)N, (int)K);
+                    // partial sums of the tile GEMM (tiles shared by several workgroups) or of a GEMV kernel over ranges of K
+                    const size_t ws_bytes = VARIANT == 1 ? 0
+                                                         : nnf::workspace::route_w4a16((int)M, (int)N, (int)K, false, false, false,
+                                                                                       nnf::workspace::PLAN_CUS, VARIANT)
+                                                               .partial_bytes;
                     std::string ws = "nullptr";
                     if (ws_bytes > 0)
                         ws = allocate_tensor(Shape{ws_bytes}, element::character)->get_name();

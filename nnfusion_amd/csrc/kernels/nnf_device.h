@@ -150,6 +150,32 @@ namespace nnf
     }
 
     // sum over a row of 16 lanes (lanes 16i .. 16i+15), in every lane; four DPP row rotations
+    // ---- element-wise tail of a fused product, on fp16 tensors as the unfused graph holds them -------------------
+    // the kernels' view of nnf::GemvFusion (nnf_launch.h)
+    struct GemvFusionArgs
+    {
+        const half_t* gamma;
+        const float* rstd;
+        const half_t* bias;
+        const half_t* residual;
+    };
+    // y = fp16(sum) (+ bias[n]) (+ residual[at]), each step rounded to fp16
+    __device__ __forceinline__ half_t finish_bias_residual(float sum, const half_t* bias, int n, const half_t* residual, size_t at)
+    {
+        half_t y = (half_t)sum;
+        if (bias)
+            y = (half_t)((float)y + (float)bias[n]);
+        if (residual)
+            y = (half_t)((float)y + (float)residual[at]);
+        return y;
+    }
+    // fp16(SiLU(g) * u) of the fp16-rounded gate and up products
+    __device__ __forceinline__ half_t finish_silu_gate(float gate_sum, float up_sum)
+    {
+        const float g = (float)(half_t)gate_sum, u = (float)(half_t)up_sum;
+        return (half_t)(g * (1.0f / (1.0f + __expf(-g))) * u);
+    }
+
     __device__ __forceinline__ float row16_sum(float v)
     {
         v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x128, 0xF, 0xF, false)); // row_ror:8

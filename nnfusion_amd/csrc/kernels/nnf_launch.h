@@ -33,6 +33,19 @@ namespace nnf
         return e;
     }
 
+    // Optional prologue and epilogue of the row-streaming GEMV kernels (every pointer may be null), applied as the unfused
+    // graph would on fp16 tensors: y = fp16(rstd[m] * sum); gate: y = fp16(silu(y_gate) * y_up); y = fp16(y + bias[n]);
+    // y = fp16(y + residual[m, n]).
+    struct GemvFusion
+    {
+        const void* gamma = nullptr;    // fp16 [K]: RMSNorm weight, multiplied onto the activations on the way in ...
+        const float* rstd = nullptr;    // fp32 [M]: ... with the sums of row m scaled by rstd[m] on the way out
+        const void* bias = nullptr;     // fp16 [N]
+        const void* residual = nullptr; // fp16 [M, N]; may be the output buffer itself
+        bool gate = false;              // N outputs from 2 N weight rows (gate rows, then up rows): SiLU(gate) * up
+        bool any() const { return gamma || rstd || bias || residual || gate; }
+    };
+
     // What a call fixes about its launch (all zero: the library's own choice by shape).  Filled from the variant and
     // plan arguments of the C ABI and passed down by value: the library keeps no dispatch state between calls.
     struct LaunchChoice
@@ -49,19 +62,22 @@ namespace nnf
     bool w4a16_gemv_supported(int M, int K);
 
     // one activation row (M = 1): the row-streaming kernel
+    // (N: outputs; with fusion.gate from 2 N weight rows)
     hipError_t launch_w4a16_gemv_rows(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int N,
-                                      int K, int zp, int num_cu);
-    bool w4a16_gemv_rows_supported(int M, int N, int K, int num_cu);
+                                      int K, int zp, int num_cu, const GemvFusion& fusion = GemvFusion());
+    bool w4a16_gemv_rows_supported(int M, int N, int K, int num_cu, bool gate = false);
 
     // 2 <= M <= 16, K = 1024 / 2048 / 4096 / 8192: weights streamed through LDS rings, activations in registers
+    // (N: outputs; gate / fusion.gate: from 2 N weight rows)
     hipError_t launch_w4a16_mrows(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M, int N,
-                                  int K, int zp, int num_cu);
-    bool w4a16_mrows_supported(int M, int N, int K, int num_cu);
-    bool w4a16_mrows_preferred(int M, int N, int K, int num_cu); // where the library picks it without being told
+                                  int K, int zp, int num_cu, const GemvFusion& fusion = GemvFusion());
+    bool w4a16_mrows_supported(int M, int N, int K, int num_cu, bool gate = false);
+    bool w4a16_mrows_preferred(int M, int N, int K, int num_cu, bool gate = false); // where the library picks it without being told
     // K above 8192: the same kernel over ranges of K, fp32 sums to partial[ranges][M][N] for the reduction pass
     int w4a16_mrows_ksplits(int M, int N, int K, int num_cu); // 0: does not apply
+    // (gamma: fp16 [K] or null, the RMSNorm weight multiplied onto the activations)
     hipError_t launch_w4a16_mrows_split(hipStream_t stream, const void* A, const void* Wq, const void* S, float* partial,
-                                        int M, int N, int K, int zp, int num_cu);
+                                        int M, int N, int K, int zp, int num_cu, const void* gamma = nullptr);
 
     hipError_t launch_w4a16_skinny(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M,
                                    int N, int K, int zp, int num_cu);
@@ -74,22 +90,16 @@ namespace nnf
     hipError_t launch_w4a16_skinny_split(hipStream_t stream, const void* A, const void* Wq, const void* S, float* partial,
                                          int M, int N, int K, int zp, int ksplits, int num_cu);
 
-    // MFMA GEMM (any M) with the RMSNorm prologue and bias / residual / SiLU-gate epilogues.
-    // rms_ws: nnf::workspace::rms_rows(M, K) bytes, needed when rms_gamma != nullptr;
-    // partial_ws: nnf::workspace::gemm_partial_bytes(...) for the plan of the shape (may be 0 bytes).
-    // M <= 16 shapes that the GEMV kernel can serve go through it (plus an element-wise epilogue kernel),
-    // unless choice.path asks for the MFMA GEMM tiles whatever M is.
+    // Y = epilogue(prologue(A) . W^T) through the kernel that nnf::workspace::route_w4a16 names for the shape, the fused
+    // parts and choice: the RMSNorm prologue and the bias / residual / SiLU-gate epilogues inside the row-streaming
+    // kernels and the tile GEMM, in the reduction pass behind a GEMV kernel over ranges of K, or (MFMA GEMV kernel) as a
+    // pre-pass and an element-wise kernel.  rms_ws / partial_ws: the route's rms_bytes / partial_bytes (null when 0).
     hipError_t launch_w4a16_gemm(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M,
                                  int N, int K, int zp, const void* rms_gamma, float rms_eps, const void* bias,
                                  const void* residual, int act, void* rms_ws, void* partial_ws, int num_cu,
                                  const LaunchChoice& choice = LaunchChoice());
     // bytes launch_w4a16_gemm writes at partial_ws for this call (0: it needs none)
-    // whether the kernel family `choice.path` names (0, 2, 3, 4) serves the product of M rows with N outputs (act 1: 2N
-    // weight rows)
-    bool w4a16_path_supported(int M, int N, int K, int act, int num_cu, int path);
-    // (in_place_residual: the residual is the output buffer itself)
-    size_t w4a16_gemm_partial_bytes(int M, int N, int K, int act, bool in_place_residual, int num_cu,
-                                    const LaunchChoice& choice = LaunchChoice());
+
 
     // W8A8: acc != nullptr writes the raw int32 accumulators, otherwise Y = fp16(acc * s_tok * s_ch).
     // partial_ws: nnf::workspace::w8a8_gemm(M, N, K) bytes (0 for the M <= 16 kernel)

@@ -27,6 +27,7 @@ namespace nnf
         int ldy;                // row stride of Y
         const half_t* bias;     // BIAS: [N]
         const half_t* residual; // RESID: [M, ldy]
+        const float* rstd;      // [M] or null: the sums of row m are scaled by rstd[m] (RMSNorm prologue)
         float* partial;         // [splits][M][ld_partial] fp32
         int splits;             // number of K ranges
         int ld_partial;         // N, or 2 N with GATE (gate columns, then up columns)
@@ -131,12 +132,13 @@ namespace nnf
     }
 
     // Y[m, n] = epilogue( sum_s partial[s][m][n] ); four consecutive columns per thread.
-    // GATE: partial columns [0, N) are the gate, [N, 2N) the up projection.
+    // GATE: partial columns [0, N) are the gate, [N, 2N) the up projection.  rstd (or null): the sums of row m times
+    // rstd[m] first (the kernel that wrote them multiplied the RMSNorm weight onto the activations).
     template <bool GATE, bool BIAS, bool RESID>
     __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ partial, int splits, int M,
                                                                 int N, int ld_partial, const half_t* __restrict__ bias,
                                                                 const half_t* __restrict__ residual, half_t* __restrict__ Y,
-                                                                int ldy)
+                                                                int ldy, const float* __restrict__ rstd)
     {
         // grid: x over groups of four columns, y = row
         const int quads = (N + 3) >> 2;
@@ -176,16 +178,17 @@ namespace nnf
                     }
             }
         }
+        const float rs = rstd ? rstd[m] : 1.0f;
         half_t out[4];
         for (int j = 0; j < 4; ++j)
         {
             if (n + j >= N)
                 break;
-            float v = a[j];
+            float v = a[j] * rs;
             if (GATE)
             {
-                float g = (float)(half_t)a[j];
-                float up = (float)(half_t)u[j];
+                float g = (float)(half_t)v;
+                float up = (float)(half_t)(u[j] * rs);
                 v = g * (1.0f / (1.0f + __expf(-g))) * up;
             }
             if (BIAS)
@@ -242,7 +245,7 @@ namespace nnf
             const int quads = (p.N + 3) >> 2;
             hipLaunchKernelGGL((splitk_reduce_kernel<GATE, BIAS, RESID>), dim3((unsigned)((quads + 255) / 256), (unsigned)p.M), dim3(256), 0,
                                stream, (const float*)p.partial, p.splits, p.M, p.N, p.ld_partial, p.bias, p.residual, p.Y,
-                               p.ldy);
+                               p.ldy, p.rstd);
             return hipGetLastError();
         }
 
@@ -260,107 +263,57 @@ namespace nnf
         }
     } // namespace
 
-    namespace
-    {
-        // Which kernel serves a call and what it parks in scratch memory: decided once, from the shape and the
-        // device's CU count alone, for the launcher and for the entry points' workspace checks alike.
-        struct Route
-        {
-            enum Kind { NONE, ROWS, MROWS, SKINNY, MROWS_SPLIT, SKINNY_SPLIT, TILE } kind = NONE; // NONE: the family asked for
-                                                                                                  // cannot serve the shape
-            int ksplits = 0;          // *_SPLIT: ranges of K
-            bool via_scratch = false; // GEMV kernels: products to scratch first, the element-wise epilogue reads them
-            workspace::SkPlan plan;   // TILE
-            size_t bytes = 0;         // written at partial_ws
-        };
-
-        Route route_w4a16(int M, int N, int K, bool gate, bool in_place_residual, int num_cu, const LaunchChoice& choice)
-        {
-            Route r;
-            const int n_rows = gate ? 2 * N : N; // weight rows
-            // choice.path: 0 the library's order of preference, 2 / 4 one family of GEMV kernels only, 3 the tile GEMM
-            const bool any = choice.path == 0, rows_family = any || choice.path == 4, skinny_family = any || choice.path == 2;
-            if (choice.path != 3)
-            {
-                // the products go to scratch first when the epilogue cannot work in place: the [M, 2N] gate | up pair,
-                // or a residual that is the output buffer itself
-                r.via_scratch = gate || in_place_residual;
-                const size_t scratch = r.via_scratch ? workspace::align256((size_t)M * n_rows * 2) : 0;
-                if (rows_family && w4a16_gemv_rows_supported(M, n_rows, K, num_cu))
-                    return r.kind = Route::ROWS, r.bytes = scratch, r;
-                if (rows_family && M > 1 && (any ? w4a16_mrows_preferred(M, n_rows, K, num_cu) : w4a16_mrows_supported(M, n_rows, K, num_cu)))
-                    return r.kind = Route::MROWS, r.bytes = scratch, r;
-                if (skinny_family && M <= 16 && w4a16_skinny_supported(M, n_rows, K))
-                    return r.kind = Route::SKINNY, r.bytes = scratch, r;
-                // more activations than one workgroup holds: ranges of K, fp32 sums per range, and the reduction pass
-                // (K above 8192 in multiples of 256: the row-streaming MFMA kernel, otherwise the split-K one)
-                r.via_scratch = false;
-                if (rows_family && (r.ksplits = w4a16_mrows_ksplits(M, n_rows, K, num_cu)) > 0)
-                    return r.kind = Route::MROWS_SPLIT, r.bytes = workspace::align256((size_t)r.ksplits * M * n_rows * 4), r;
-                if (skinny_family && (r.ksplits = w4a16_skinny_ksplits(M, n_rows, K)) > 0)
-                    return r.kind = Route::SKINNY_SPLIT, r.bytes = workspace::align256((size_t)r.ksplits * M * n_rows * 4), r;
-                if (!any)
-                    return r;
-            }
-            r.kind = Route::TILE;
-            r.plan = workspace::plan_w4a16_sk_with(M, N, K, gate, num_cu, choice.tile_rows, choice.k_parts);
-            r.bytes = r.plan.bytes();
-            return r;
-        }
-    } // namespace
-
-    size_t w4a16_gemm_partial_bytes(int M, int N, int K, int act, bool in_place_residual, int num_cu,
-                                    const LaunchChoice& choice)
-    {
-        return route_w4a16(M, N, K, act == 1, in_place_residual, num_cu, choice).bytes;
-    }
-
-    bool w4a16_path_supported(int M, int N, int K, int act, int num_cu, int path)
-    {
-        LaunchChoice choice;
-        choice.path = path;
-        return route_w4a16(M, N, K, act == 1, false, num_cu, choice).kind != Route::NONE;
-    }
-
     hipError_t launch_w4a16_gemm(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M,
                                  int N, int K, int zp, const void* rms_gamma, float rms_eps, const void* bias,
                                  const void* residual, int act, void* rms_ws, void* partial_ws, int num_cu,
                                  const LaunchChoice& choice)
     {
+        using workspace::W4A16Route;
         const bool rms = rms_gamma != nullptr, hb = bias != nullptr, hr = residual != nullptr, gate = act == 1;
         // the combinations the fused entry points use; anything else is composed by the caller
         if (gate && (hb || hr))
             return hipErrorInvalidValue;
         const int n_rows = gate ? 2 * N : N; // weight rows
-        const Route route = route_w4a16(M, N, K, gate, hr && residual == Y, num_cu, choice);
-        if (route.kind == Route::NONE || (route.bytes > 0 && !partial_ws))
+        const W4A16Route route =
+            workspace::route_w4a16(M, N, K, gate, rms, hr && residual == Y, num_cu, choice.path, choice.tile_rows, choice.k_parts);
+        if (route.kind == W4A16Route::NONE || (route.partial_bytes > 0 && !partial_ws) || (route.rms_bytes > 0 && !rms_ws))
             return hipErrorInvalidValue;
-        const bool rows = route.kind == Route::ROWS, mrows = route.kind == Route::MROWS;
-        const bool one_launch_gemv = rows || mrows || route.kind == Route::SKINNY;
-        const bool via_scratch = route.via_scratch;
-        const int ksplits = route.ksplits;
-        const bool mr_splits = route.kind == Route::MROWS_SPLIT;
-        if (rms && route.kind != Route::TILE)
+        // ---- RMSNorm pre-pass: rstd[m] for the kernels that multiply the weight in themselves, the normalised
+        // activations for the MFMA GEMV kernel -------------------------------------------------------------------
+        const bool normalised_copy = route.kind == W4A16Route::SKINNY || route.kind == W4A16Route::SKINNY_SPLIT;
+        if (rms)
         {
-            // the GEMV kernels read normalised activations (the tile GEMM folds the normalisation in: below)
-            if (!rms_ws)
-                return hipErrorInvalidValue;
-            hipLaunchKernelGGL(rms_norm_kernel, dim3(M), dim3(256), 0, stream, (const half_t*)A,
-                               (const half_t*)rms_gamma, (half_t*)rms_ws, M, K, rms_eps);
-            hipError_t e = hipGetLastError();
+            if (normalised_copy)
+            {
+                hipLaunchKernelGGL(rms_norm_kernel, dim3(M), dim3(256), 0, stream, (const half_t*)A, (const half_t*)rms_gamma,
+                                   (half_t*)rms_ws, M, K, rms_eps);
+                A = rms_ws;
+            }
+            else
+                hipLaunchKernelGGL(rms_rstd_kernel, dim3(M), dim3(256), 0, stream, (const half_t*)A, (float*)rms_ws, M, K, rms_eps);
+            const hipError_t e = hipGetLastError();
             if (e != hipSuccess)
                 return e;
-            A = rms_ws;
         }
-        // M <= 16 (<= 32 where the row-streaming MFMA kernel applies): the bandwidth-bound GEMV kernel on the
-        // (normalised) activations, then a small element-wise
-        // kernel for whatever epilogue is asked for
-        if (one_launch_gemv)
+        const float* rstd = (rms && !normalised_copy) ? (const float*)rms_ws : nullptr;
+        // ---- the row-streaming kernels (one row; up to 32 rows): prologue and epilogue inside the one launch ------
+        if (route.kind == W4A16Route::ROWS || route.kind == W4A16Route::MROWS)
         {
-            void* y_gemv = via_scratch ? partial_ws : Y;
-            hipError_t e = rows ? launch_w4a16_gemv_rows(stream, A, Wq, S, y_gemv, n_rows, K, zp, num_cu)
-                                : mrows ? launch_w4a16_mrows(stream, A, Wq, S, y_gemv, M, n_rows, K, zp, num_cu)
-                                        : launch_w4a16_skinny(stream, A, Wq, S, y_gemv, M, n_rows, K, zp, num_cu);
+            GemvFusion fusion;
+            fusion.gamma = rms_gamma;
+            fusion.rstd = rstd;
+            fusion.bias = bias;
+            fusion.residual = residual;
+            fusion.gate = gate;
+            return route.kind == W4A16Route::ROWS ? launch_w4a16_gemv_rows(stream, A, Wq, S, Y, N, K, zp, num_cu, fusion)
+                                                  : launch_w4a16_mrows(stream, A, Wq, S, Y, M, N, K, zp, num_cu, fusion);
+        }
+        // ---- the MFMA GEMV kernel on the (normalised) activations, then a small element-wise kernel for whatever
+        // epilogue is asked for ----------------------------------------------------------------------------------
+        if (route.kind == W4A16Route::SKINNY)
+        {
+            void* y_gemv = route.via_scratch ? partial_ws : Y;
+            hipError_t e = launch_w4a16_skinny(stream, A, Wq, S, y_gemv, M, n_rows, K, zp, num_cu);
             if (e != hipSuccess || (!gate && !hb && !hr))
                 return e;
             const int blocks = (M * N + 255) / 256;
@@ -372,14 +325,14 @@ namespace nnf
                                    (half_t*)Y, (const half_t*)bias, (const half_t*)residual, M, N);
             return hipGetLastError();
         }
-        // M <= 16 with too many activations for one workgroup's LDS: the GEMV kernel over ranges of K, then the
-        // reduction pass (which applies the epilogue)
-        // (K above 8192 in multiples of 256: the row-streaming MFMA kernel, otherwise the split-K one)
-        if (ksplits > 0)
+        // ---- more activations than one workgroup holds: a GEMV kernel over ranges of K, then the reduction pass
+        // (which applies rstd and the epilogue) ------------------------------------------------------------------
+        if (route.kind == W4A16Route::MROWS_SPLIT || route.kind == W4A16Route::SKINNY_SPLIT)
         {
-            hipError_t e = mr_splits
-                               ? launch_w4a16_mrows_split(stream, A, Wq, S, (float*)partial_ws, M, n_rows, K, zp, num_cu)
-                               : launch_w4a16_skinny_split(stream, A, Wq, S, (float*)partial_ws, M, n_rows, K, zp, ksplits, num_cu);
+            hipError_t e = route.kind == W4A16Route::MROWS_SPLIT
+                               ? launch_w4a16_mrows_split(stream, A, Wq, S, (float*)partial_ws, M, n_rows, K, zp, num_cu, rms_gamma)
+                               : launch_w4a16_skinny_split(stream, A, Wq, S, (float*)partial_ws, M, n_rows, K, zp, route.ksplits,
+                                                           num_cu);
             if (e != hipSuccess)
                 return e;
             GemmParams p;
@@ -389,8 +342,9 @@ namespace nnf
             p.ldy = N;
             p.bias = (const half_t*)bias;
             p.residual = (const half_t*)residual;
+            p.rstd = rstd;
             p.partial = (float*)partial_ws;
-            p.splits = ksplits;
+            p.splits = route.ksplits;
             p.ld_partial = n_rows;
             return launch_reduce_any(stream, p, gate, hb, hr);
         }
@@ -418,15 +372,6 @@ namespace nnf
         p.tiles_n = plan.tiles_n;
         p.supersteps = plan.supersteps;
         p.units = plan.units;
-        if (rms)
-        {
-            if (!rms_ws)
-                return hipErrorInvalidValue;
-            hipLaunchKernelGGL(rms_rstd_kernel, dim3(M), dim3(256), 0, stream, (const half_t*)A, (float*)rms_ws, M, K, rms_eps);
-        }
-        hipError_t e = hipGetLastError();
-        if (e != hipSuccess)
-            return e;
         switch (plan.tile_rows)
         {
         case 256: return launch_gemm_sk_256(stream, p, plan.grid, gate);

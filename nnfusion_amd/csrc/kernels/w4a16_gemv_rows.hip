@@ -67,14 +67,18 @@ namespace nnf
     // SEG: wavefront-wide loads (1 KiB of a row each) per row and wavefront; D: rows in flight per wavefront;
     // WAVES: wavefronts per workgroup (one workgroup per CU).
     // pack = zp | log2(KSW) << 8, KSW = wavefronts sharing a row (each a segment of SEG KiB).
-    // Workgroup b owns rows_q rows (one more for b < rows_r), contiguous.
-    template <int SEG, int D, int WAVES>
+    // Workgroup b owns rows_q outputs (one more for b < rows_r), contiguous.
+    // EPI: 0 plain; 1 the optional parts of `f` (RMSNorm: gamma onto the activations, rstd onto the sums; bias;
+    // residual); 2 SiLU-gate (N outputs from 2 N weight rows: the workgroup walks the gate rows of its outputs, then
+    // their up rows N further down; scales: two blocks in LDS) with the optional RMSNorm.
+    template <int SEG, int D, int WAVES, int EPI>
     __global__ __launch_bounds__(WAVES * 64) void w4a16_gemv_rows_kernel(const half_t* __restrict__ A,
                                                                          const uint8_t* __restrict__ Wq,
                                                                          const half_t* __restrict__ S,
                                                                          half_t* __restrict__ Y, int N, int K,
-                                                                         int rows_q, int rows_r, int pack)
+                                                                         int rows_q, int rows_r, int pack, GemvFusionArgs f)
     {
+        constexpr bool GATE = EPI == 2;
         extern __shared__ uintx4 lds[];
         uint32_t MAGIC, MAGIC_HI, MASK_LO, MASK_HI;
         asm volatile("v_mov_b32 %0, 0x64006400" : "=v"(MAGIC));
@@ -90,20 +94,25 @@ namespace nnf
         const int gpw = WAVES >> kshift; // wavefronts per K segment
         const int widx = wave >> kshift; // this one among them
         const int out0 = (int)blockIdx.x * rows_q + min((int)blockIdx.x, rows_r);
-        const int n_rows = rows_q + ((int)blockIdx.x < rows_r ? 1 : 0); // >= 1: the grid never exceeds N
+        const int n_out = rows_q + ((int)blockIdx.x < rows_r ? 1 : 0); // >= 1: the grid never exceeds N
+        const int n_rows = GATE ? 2 * n_out : n_out;                   // weight rows this workgroup walks
         const uint32_t row_bytes = (uint32_t)K >> 1;
         const int G = K >> 7;
         const int a_units = K >> 3;
         const int a_pad = (a_units + 63) & ~63; // whole wavefront-wide loads of activations
-        const int sc_bytes = n_rows * G * 2;    // this workgroup's block of S
+        const int sc_bytes = n_out * G * 2;     // this workgroup's block of S (GATE: one such block for the gate rows,
+                                                // one for the up rows)
+        const int sc_block = (((rows_q + 1) * G * 2) + 1023) & ~1023; // LDS bytes of a block
+        // weight row r of the workgroup (relative) -> row of Wq / S
+        auto phys_row = [&](int r) { return (GATE && r >= n_out) ? N + out0 + (r - n_out) : out0 + r; };
 
         uint8_t* lds_bytes = reinterpret_cast<uint8_t*>(lds);
         uint8_t* ring = lds_bytes + wave * (D * SEG * 1024);
         uintx4* act = lds + (WAVES * D * SEG * 1024) / 16;
         float* corr = reinterpret_cast<float*>(act + a_pad + 4);
         uint8_t* scales = reinterpret_cast<uint8_t*>(corr + a_pad + 4);
-        float* outb = reinterpret_cast<float*>(scales + ((((rows_q + 1) * G * 2) + 1023) & ~1023));
-        int* next_row = reinterpret_cast<int*>(outb + ((rows_q + 1) << kshift));
+        float* outb = reinterpret_cast<float*>(scales + (GATE ? 2 : 1) * sc_block);
+        int* next_row = reinterpret_cast<int*>(outb + (((GATE ? 2 : 1) * (rows_q + 1)) << kshift));
 
         // ---- activations and scales: requested first (few loads, cache hits), once per workgroup ------------
         // (global -> LDS like the weights: a load into registers followed by an LDS write would be made to wait
@@ -115,20 +124,36 @@ namespace nnf
             __builtin_amdgcn_global_load_lds((global_ptr_t)(reinterpret_cast<const uint8_t*>(A) + (size_t)(u * 16u)),
                                              (lds_ptr_t)(reinterpret_cast<uint8_t*>(act) + u0 * 16), 16, 0, 0);
         }
+#pragma unroll
+        for (int half = 0; half < (GATE ? 2 : 1); ++half)
         {
             // whole KiB of the block with 16 bytes per lane, the rest (a multiple of 4 bytes) with 4 bytes per
             // lane, lanes past the end re-reading its last word: nothing is read beyond the block
-            const uint8_t* blk = reinterpret_cast<const uint8_t*>(S) + (size_t)out0 * G * 2;
+            const uint8_t* blk = reinterpret_cast<const uint8_t*>(S) + (size_t)(out0 + half * N) * G * 2;
+            uint8_t* dst = scales + half * sc_block;
             const int full = sc_bytes >> 10;
             for (int i = wave; i < full; i += WAVES)
-                __builtin_amdgcn_global_load_lds((global_ptr_t)(blk + i * 1024 + lane * 16), (lds_ptr_t)(scales + i * 1024),
-                                                 16, 0, 0);
+                __builtin_amdgcn_global_load_lds((global_ptr_t)(blk + i * 1024 + lane * 16), (lds_ptr_t)(dst + i * 1024), 16, 0,
+                                                 0);
             const int tail_loads = ((sc_bytes & 1023) + 255) >> 8;
             for (int t = wave; t < tail_loads; t += WAVES)
             {
                 const int off = full * 1024 + t * 256;
                 __builtin_amdgcn_global_load_lds((global_ptr_t)(blk + min(off + lane * 4, sc_bytes - 4)),
-                                                 (lds_ptr_t)(scales + off), 4, 0, 0);
+                                                 (lds_ptr_t)(dst + off), 4, 0, 0);
+            }
+        }
+        // RMSNorm weight of the units this lane prepares below: into registers, ahead of the weights (vector-memory
+        // operations complete in order: the wait for the activations covers them)
+        constexpr int GQ = EPI != 0 ? 2048 / (WAVES * 64) : 1; // units per lane at the largest K
+        uintx4 gq[GQ];
+        if (EPI != 0 && f.gamma)
+        {
+#pragma unroll
+            for (int e = 0; e < GQ; ++e)
+            {
+                const int u = min(wave * 64 + e * (WAVES * 64) + lane, a_units - 1);
+                gq[e] = reinterpret_cast<const uintx4*>(f.gamma)[u];
             }
         }
 
@@ -145,7 +170,7 @@ namespace nnf
         }
         // weights of row r (relative to the workgroup's first; rows past the end re-read the last row) -> ring slot
         auto issue = [&](int r, int slot) {
-            const uint8_t* src = Wq + (size_t)(out0 + min(r, n_rows - 1)) * row_bytes;
+            const uint8_t* src = Wq + (size_t)phys_row(min(r, n_rows - 1)) * row_bytes;
 #pragma unroll
             for (int j = 0; j < SEG; ++j)
                 __builtin_amdgcn_global_load_lds((global_ptr_t)(src + w_off[j]),
@@ -181,10 +206,24 @@ namespace nnf
         {
             const float ce = -(1024.0f + (float)zp);
             const float co = -(64.0f + (float)zp);
-            for (int u0 = wave * 64; u0 < a_units; u0 += WAVES * 64)
+            int e = 0;
+            for (int u0 = wave * 64; u0 < a_units; u0 += WAVES * 64, ++e)
             {
                 const int u = u0 + lane;
-                const uintx4 a = permute_a8(act[u]);
+                uintx4 raw = act[u];
+                if (EPI != 0 && f.gamma)
+                {
+                    // fp16(a * gamma): the product of two fp16 values, rounded once
+                    uintx4 g = gq[0];
+#pragma unroll
+                    for (int i = 1; i < GQ; ++i)
+                        g = e == i ? gq[i] : g;
+                    raw.x = as_u32(as_half2(raw.x) * as_half2(g.x));
+                    raw.y = as_u32(as_half2(raw.y) * as_half2(g.y));
+                    raw.z = as_u32(as_half2(raw.z) * as_half2(g.z));
+                    raw.w = as_u32(as_half2(raw.w) * as_half2(g.w));
+                }
+                const uintx4 a = permute_a8(raw);
                 const half2_t x = as_half2(a.x), y = as_half2(a.y), z = as_half2(a.z), w = as_half2(a.w);
                 const float se = ((float)x.x + (float)x.y) + ((float)z.x + (float)z.y);
                 const float so = ((float)y.x + (float)y.y) + ((float)w.x + (float)w.y);
@@ -212,7 +251,7 @@ namespace nnf
         uintx4 wv[SEG];
         float sv[SEG];
         auto read_slot = [&](int r, int slot) {
-            const uint8_t* sc_row = scales + r * (G * 2);
+            const uint8_t* sc_row = scales + ((GATE && r >= n_out) ? sc_block + (r - n_out) * (G * 2) : r * (G * 2));
 #pragma unroll
             for (int j = 0; j < SEG; ++j)
             {
@@ -310,12 +349,23 @@ namespace nnf
 
         // ---- outputs ------------------------------------------------------------------------------------
         lds_barrier();
-        for (int r = tid; r < n_rows; r += WAVES * 64)
+        const float rs = (EPI != 0 && f.rstd) ? f.rstd[0] : 1.0f;
+        for (int r = tid; r < n_out; r += WAVES * 64)
         {
             float y = 0.f;
             for (int kp = 0; kp < ksw; ++kp)
                 y += outb[(r << kshift) + kp];
-            Y[out0 + r] = (half_t)y;
+            if (EPI == 0)
+                Y[out0 + r] = (half_t)y;
+            else if (EPI == 1)
+                Y[out0 + r] = finish_bias_residual(y * rs, f.bias, out0 + r, f.residual, (size_t)(out0 + r));
+            else
+            {
+                float up = 0.f;
+                for (int kp = 0; kp < ksw; ++kp)
+                    up += outb[((r + n_out) << kshift) + kp];
+                Y[out0 + r] = finish_silu_gate(y * rs, up * rs);
+            }
         }
     }
 
@@ -323,42 +373,50 @@ namespace nnf
     {
         using workspace::RowsPlan;
 
-        template <int SEG, int D, int WAVES>
+        template <int SEG, int D, int WAVES, int EPI>
         hipError_t launch_rows(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int N, int K,
-                               int zp, const RowsPlan& p, int grid)
+                               int zp, const RowsPlan& p, int grid, const GemvFusion& fusion)
         {
-            const size_t lds_total = p.lds_bytes(N, K, grid);
+            const size_t lds_total = p.lds_bytes(N, K, grid, EPI == 2);
+            const GemvFusionArgs f = {(const half_t*)fusion.gamma, fusion.rstd, (const half_t*)fusion.bias,
+                                      (const half_t*)fusion.residual};
             if (lds_total > MAX_LDS_BYTES)
                 return hipErrorInvalidValue;
             if (lds_total > 64 * 1024)
             {
                 static LdsGrant granted;
-                const hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(&w4a16_gemv_rows_kernel<SEG, D, WAVES>),
+                const hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(&w4a16_gemv_rows_kernel<SEG, D, WAVES, EPI>),
                                                        granted, (int)MAX_LDS_BYTES);
                 if (e != hipSuccess)
                     return e;
             }
-            hipLaunchKernelGGL((w4a16_gemv_rows_kernel<SEG, D, WAVES>), dim3(grid), dim3(WAVES * 64), lds_total, stream,
+            hipLaunchKernelGGL((w4a16_gemv_rows_kernel<SEG, D, WAVES, EPI>), dim3(grid), dim3(WAVES * 64), lds_total, stream,
                                (const half_t*)A, (const uint8_t*)Wq, (const half_t*)S, (half_t*)Y, N, K, N / grid, N % grid,
-                               zp | (p.kshift << 8));
+                               zp | (p.kshift << 8), f);
             return hipGetLastError();
         }
     } // namespace
 
-    bool w4a16_gemv_rows_supported(int M, int N, int K, int num_cu)
+    bool w4a16_gemv_rows_supported(int M, int N, int K, int num_cu, bool gate)
     {
-        return workspace::plan_w4a16_rows(M, N, K, num_cu).seg != 0;
+        return workspace::plan_w4a16_rows(M, N, K, num_cu, 0, gate).seg != 0;
     }
 
     hipError_t launch_w4a16_gemv_rows(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int N,
-                                      int K, int zp, int num_cu)
+                                      int K, int zp, int num_cu, const GemvFusion& fusion)
     {
-        const RowsPlan p = workspace::plan_w4a16_rows(1, N, K, num_cu, 0);
+        const RowsPlan p = workspace::plan_w4a16_rows(1, N, K, num_cu, 0, fusion.gate);
         const int grid = workspace::rows_grid(N, num_cu);
+        if (fusion.gate && (fusion.bias || fusion.residual))
+            return hipErrorInvalidValue;
+        const int epi = fusion.gate ? 2 : fusion.any() ? 1 : 0;
         switch (p.seg * 10 + p.depth)
         {
 #define NNF_ROWS_CASE(SEG, D)                                                                                          \
-    case SEG * 10 + D: return launch_rows<SEG, D, workspace::ROWS_WAVES>(stream, A, Wq, S, Y, N, K, zp, p, grid);
+    case SEG * 10 + D:                                                                                                 \
+        return epi == 0   ? launch_rows<SEG, D, workspace::ROWS_WAVES, 0>(stream, A, Wq, S, Y, N, K, zp, p, grid, fusion)  \
+               : epi == 1 ? launch_rows<SEG, D, workspace::ROWS_WAVES, 1>(stream, A, Wq, S, Y, N, K, zp, p, grid, fusion)  \
+                          : launch_rows<SEG, D, workspace::ROWS_WAVES, 2>(stream, A, Wq, S, Y, N, K, zp, p, grid, fusion);
             NNF_ROWS_CASE(1, 1)
             NNF_ROWS_CASE(1, 2)
             NNF_ROWS_CASE(1, 3)

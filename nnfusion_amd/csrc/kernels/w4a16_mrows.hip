@@ -49,6 +49,60 @@ namespace nnf
     // The activations of a wavefront as loaded -> the MFMA operand order of the nibble trick (pairs (a0,a4) (a1,a5)
     // (a2,a6) (a3,a7)), and per group the constant part of its sum (an MFMA against a
     // constant operand), negative, as the initial accumulator of the group.
+    // areg[.][g][.] *= the RMSNorm weight of the same k (fp16 products, rounded once); gsrc: the lane's 64 bytes of
+    // gamma for group g start at gsrc(g)
+    template <int MB, int GA, class F>
+    __device__ __forceinline__ void mrows_scale_a(uintx4 (&areg)[MB][GA][4], F&& gsrc)
+    {
+#pragma unroll
+        for (int g = 0; g < GA; ++g)
+        {
+            const uintx4* gp = reinterpret_cast<const uintx4*>(gsrc(g));
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+            {
+                const uintx4 gm = gp[j];
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb)
+                {
+                    uintx4 a = areg[mb][g][j];
+                    a.x = as_u32(as_half2(a.x) * as_half2(gm.x));
+                    a.y = as_u32(as_half2(a.y) * as_half2(gm.y));
+                    a.z = as_u32(as_half2(a.z) * as_half2(gm.z));
+                    a.w = as_u32(as_half2(a.w) * as_half2(gm.w));
+                    areg[mb][g][j] = a;
+                }
+            }
+        }
+    }
+
+    // The workgroup's parked sums -> Y.  Plain: fp16 of the sum.  Fused (see GemvFusion in nnf_launch.h): the sums of
+    // row m times rstd[m]; gate: tiles 2 i and 2 i + 1 of the workgroup are the gate and the up rows of its output tile
+    // i; bias and residual.  t0: the workgroup's first output tile, T_out of them; N: output columns.
+    template <bool FUSED>
+    __device__ __forceinline__ void mrows_flush(const float* parked, half_t* __restrict__ Y, int t0, int T_out, int M, int N,
+                                                int tid, const GemvFusionArgs& f, int gate)
+    {
+        for (int idx = tid; idx < T_out * M * 16; idx += 512)
+        {
+            const int n = idx & 15;
+            const int im = idx >> 4;
+            const int it = im / M, m = im - it * M;
+            const int nn = min((t0 + it) * 16, N - 16) + n;
+            const size_t at = (size_t)m * N + nn;
+            if (!FUSED)
+                Y[at] = (half_t)parked[idx];
+            else
+            {
+                const float rs = f.rstd ? f.rstd[m] : 1.0f;
+                if (gate)
+                    Y[at] = finish_silu_gate(parked[((2 * it) * M + m) * 16 + n] * rs, parked[((2 * it + 1) * M + m) * 16 + n] * rs);
+                else
+                    Y[at] = finish_bias_residual(parked[idx] * rs, f.bias, nn, f.residual, at);
+            }
+        }
+    }
+
     template <int MB, int GA>
     __device__ __forceinline__ void mrows_prepare_a(uintx4 (&areg)[MB][GA][4], floatx4 (&ncorr)[MB][GA], int zp)
     {
@@ -146,11 +200,13 @@ namespace nnf
     // K = GW * STEPS * 1024; MB = blocks of 16 activation rows (1 or 2).
     // LDS (bytes): weights [8 wavefronts][2 slots][GW KiB] | scales [8][2][256] | partial tiles [2][8][MB KiB] |
     //              parked sums [tiles of the workgroup][M][16] fp32
-    // pack = M | zp << 8;  a workgroup's tiles: tiles_q, one more for the first tiles_r workgroups.
-    template <int GW, int STEPS, int MB>
+    // pack = M | zp << 8;  a workgroup's output tiles: tiles_q, one more for the first tiles_r workgroups.
+    // FUSED: the prologue / epilogue of `f`; gate != 0: N outputs from 2 N weight rows, the workgroup walks the gate and
+    // the up tile of each of its output tiles in turn (twice the tiles).
+    template <int GW, int STEPS, int MB, bool FUSED>
     __global__ __launch_bounds__(512) void w4a16_mrows_kernel(const half_t* __restrict__ A, const uint8_t* __restrict__ Wq,
                                                               const half_t* __restrict__ S, half_t* __restrict__ Y, int N,
-                                                              int tiles_q, int tiles_r, int pack)
+                                                              int tiles_q, int tiles_r, int pack, GemvFusionArgs f, int gate)
     {
         static_assert(GW >= 1 && GW <= 8 && STEPS >= 1 && GW * STEPS <= 8, "K = GW * STEPS * 1024");
         static_assert(MB == 1 || (MB == 2 && GW * STEPS <= 4), "two blocks of rows: 32 VGPRs per group");
@@ -177,9 +233,15 @@ namespace nnf
         const int M = pack & 0xff, zp = (pack >> 8) & 0xff;
         const int b = blockIdx.x;
         const int t0 = b * tiles_q + min(b, tiles_r);
-        const int T = tiles_q + (b < tiles_r ? 1 : 0);
-        // the last tile of an N that is not a multiple of 16 is moved back to rows N-16 .. N-1
-        auto row0_of = [&](int tile) { return __builtin_amdgcn_readfirstlane(min(tile * 16, N - 16)); };
+        const int T_out = tiles_q + (b < tiles_r ? 1 : 0);
+        const int T = (FUSED && gate) ? 2 * T_out : T_out; // weight tiles this workgroup walks
+        // weight rows of the workgroup's tile i (the last tile of an N that is not a multiple of 16 is moved back to
+        // rows N-16 .. N-1)
+        auto row0_of = [&](int i) {
+            if (FUSED && gate)
+                return __builtin_amdgcn_readfirstlane(((i & 1) ? N : 0) + min((t0 + (i >> 1)) * 16, N - 16));
+            return __builtin_amdgcn_readfirstlane(min((t0 + i) * 16, N - 16));
+        };
 
         uint8_t* ring = smem + wave * (2 * TILE_BYTES);
         uint8_t* sc_ring = smem + MR_WAVES * 2 * TILE_BYTES + wave * 512;
@@ -224,8 +286,8 @@ namespace nnf
         // (the activations are requested last: vector-memory operations complete in order and the compiler waits
         // for them where they are used, which then also covers the two tiles -- requested first, those tiles'
         // loads are not held back by anything)
-        issue(t0, 0, 0);
-        issue(t0 + min(1 / STEPS, T - 1), 1 % STEPS, 1);
+        issue(0, 0, 0);
+        issue(min(1 / STEPS, T - 1), 1 % STEPS, 1);
         uintx4 areg[MB][GA][4];
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb)
@@ -240,6 +302,10 @@ namespace nnf
                     areg[mb][g][j] = *reinterpret_cast<const uintx4*>(
                         a_bytes + (size_t)(a_off + (g / GW) * (SPAN * 4) + (g % GW) * 256 + j * 16));
         }
+        if (FUSED && f.gamma)
+            mrows_scale_a<MB, GA>(areg, [&](int g) {
+                return reinterpret_cast<const uint8_t*>(f.gamma) + wave * (GW * 256) + kq * 64 + (g / GW) * (SPAN * 4) + (g % GW) * 256;
+            });
         floatx4 ncorr[MB][GA];
         mrows_prepare_a<MB, GA>(areg, ncorr, zp);
 
@@ -276,7 +342,7 @@ namespace nnf
                 // the slot has been read before it is refilled with the step after next (past the end: a valid
                 // tile again, so that the wait count above holds for every step)
                 asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-                issue(t0 + min(it + (st + 2) / STEPS, T - 1), (st + 2) % STEPS, slot);
+                issue(min(it + (st + 2) / STEPS, T - 1), (st + 2) % STEPS, slot);
                 slot ^= 1;
 #pragma unroll
                 for (int g = 0; g < GW; ++g)
@@ -287,13 +353,7 @@ namespace nnf
         __builtin_amdgcn_s_waitcnt(mr_vmcnt(0)); // the reloads past the end, before the LDS goes away
         asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
         // ---- flush: parked sums -> Y -----------------------------------------------------------------------------
-        for (int idx = tid; idx < T * M * 16; idx += 512)
-        {
-            const int n = idx & 15;
-            const int im = idx >> 4;
-            const int it = im / M, m = im - it * M;
-            Y[(size_t)m * N + min((t0 + it) * 16, N - 16) + n] = (half_t)parked[idx];
-        }
+        mrows_flush<FUSED>(parked, Y, t0, T_out, M, N, tid, f, gate);
     }
 
     // The same kernel with K as a run-time value: any multiple of 256 up to 8 * GW * STEPS groups (2 <= M <= 16).
@@ -306,11 +366,13 @@ namespace nnf
     // groups); the workgroups of a range write its fp32 sums to partial[range][M][N] for the reduction pass.
     // MB = 2 (17 .. 32 rows): at most four groups per wavefront; MB = 4 (33 .. 64 rows): at most two.  LDS as above.
     // pack = M | zp << 8.
-    template <int GW, int STEPS, int MB>
+    // FUSED: as in w4a16_mrows_kernel; over ranges of K only the RMSNorm weight applies here (the sums of a range go to
+    // `partial` as they are: rstd and the rest of the epilogue belong to the reduction pass).
+    template <int GW, int STEPS, int MB, bool FUSED>
     __global__ __launch_bounds__(512) void w4a16_mrows_any_kernel(const half_t* __restrict__ A, const uint8_t* __restrict__ Wq,
                                                                   const half_t* __restrict__ S, half_t* __restrict__ Y,
                                                                   float* __restrict__ partial, int N, int K, int range_groups,
-                                                                  int tiles_q, int tiles_r, int pack)
+                                                                  int tiles_q, int tiles_r, int pack, GemvFusionArgs f, int gate)
     {
         static_assert(GW >= 1 && GW <= 7 && STEPS >= 1 && GW * STEPS <= 8, "groups per wavefront");
         static_assert(MB == 1 || (MB == 2 && GW * STEPS <= 4) || (MB == 4 && GW * STEPS <= 2), "16 VGPRs per group and block of rows");
@@ -335,8 +397,15 @@ namespace nnf
         const int G = K >> 7, ROW_BYTES = K >> 1;
         const int b = blockIdx.x;
         const int t0 = b * tiles_q + min(b, tiles_r);
-        const int T = tiles_q + (b < tiles_r ? 1 : 0);
-        auto row0_of = [&](int tile) { return __builtin_amdgcn_readfirstlane(min(tile * 16, N - 16)); };
+        const int T_out = tiles_q + (b < tiles_r ? 1 : 0);
+        const int T = (FUSED && gate) ? 2 * T_out : T_out; // weight tiles this workgroup walks
+        // weight rows of the workgroup's tile i (the last tile of an N that is not a multiple of 16 is moved back to
+        // rows N-16 .. N-1)
+        auto row0_of = [&](int i) {
+            if (FUSED && gate)
+                return __builtin_amdgcn_readfirstlane(((i & 1) ? N : 0) + min((t0 + (i >> 1)) * 16, N - 16));
+            return __builtin_amdgcn_readfirstlane(min((t0 + i) * 16, N - 16));
+        };
         const int g_lo = (int)blockIdx.y * range_groups, g_hi = min(G, g_lo + range_groups); // this workgroup's part of K
         // first group that wavefront `wave` owns in step st, and the first group it fetches
         auto own_group = [&](int st) { return g_lo + st * (8 * GW) + wave * GW; };
@@ -375,8 +444,8 @@ namespace nnf
             __builtin_amdgcn_global_load_lds((mr_global_ptr_t)(reinterpret_cast<const uint8_t*>(S) + (size_t)row0 * (G * 2) + s_off),
                                              (mr_lds_ptr_t)(sc_ring + slot * 256), 4, 0, 0);
         };
-        issue(t0, 0, 0);
-        issue(t0 + min(1 / STEPS, T - 1), 1 % STEPS, 1);
+        issue(0, 0, 0);
+        issue(min(1 / STEPS, T - 1), 1 % STEPS, 1);
 
         const uint32_t rd_base = (uint32_t)col * SLICE;
         const int rd_swz = swz(col);
@@ -403,6 +472,10 @@ namespace nnf
                         for (int j = 0; j < 4; ++j)
                             areg[mb][st * GW + g][j] = *reinterpret_cast<const uintx4*>(a_src + g * 256 + j * 16);
                 }
+            if (FUSED && f.gamma)
+                mrows_scale_a<MB, GA>(areg, [&](int g) {
+                    return reinterpret_cast<const uint8_t*>(f.gamma) + kq * 64 + (size_t)fetch_group(g / GW) * 256 + (g % GW) * 256;
+                });
             mrows_prepare_a<MB, GA>(areg, ncorr, zp);
             for (int it = 0; it < T; ++it)
             {
@@ -433,7 +506,7 @@ namespace nnf
                         }
                     }
                     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-                    issue(t0 + min(it + (st + 2) / STEPS, T - 1), (st + 2) % STEPS, slot);
+                    issue(min(it + (st + 2) / STEPS, T - 1), (st + 2) % STEPS, slot);
                     slot ^= 1;
 #pragma unroll
                     for (int g = 0; g < GW; ++g)
@@ -444,32 +517,40 @@ namespace nnf
         }
         __builtin_amdgcn_s_waitcnt(mr_vmcnt(0)); // the reloads past the end, before the LDS goes away
         asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-        for (int idx = tid; idx < T * M * 16; idx += 512)
+        if (partial)
         {
-            const int n = idx & 15;
-            const int im = idx >> 4;
-            const int it = im / M, m = im - it * M;
-            const size_t at = (size_t)m * N + min((t0 + it) * 16, N - 16) + n;
-            if (partial)
-                partial[(size_t)blockIdx.y * M * N + at] = parked[idx];
-            else
-                Y[at] = (half_t)parked[idx];
+            for (int idx = tid; idx < T * M * 16; idx += 512)
+            {
+                const int n = idx & 15;
+                const int im = idx >> 4;
+                const int it = im / M, m = im - it * M;
+                partial[(size_t)blockIdx.y * M * N + (size_t)m * N + min((t0 + it) * 16, N - 16) + n] = parked[idx];
+            }
         }
+        else
+            mrows_flush<FUSED>(parked, Y, t0, T_out, M, N, tid, f, gate);
     }
 
     namespace
     {
-        template <int GW, int STEPS, int MB>
+        GemvFusionArgs fusion_args(const GemvFusion& fusion)
+        {
+            return GemvFusionArgs{(const half_t*)fusion.gamma, fusion.rstd, (const half_t*)fusion.bias, (const half_t*)fusion.residual};
+        }
+
+        // N: output columns (fusion.gate: from 2 N weight rows)
+        template <int GW, int STEPS, int MB, bool FUSED>
         hipError_t launch_mrows_mb(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M, int N, int zp,
-                                int num_cu)
+                                   int num_cu, const GemvFusion& fusion)
         {
             const int n_tiles = (N + 15) / 16;
             const int grid = n_tiles < num_cu ? n_tiles : num_cu;
             const int tiles_q = n_tiles / grid, tiles_r = n_tiles % grid;
-            const size_t lds = workspace::w4a16_mrows_lds_bytes(GW * STEPS * 1024, M, tiles_q + (tiles_r ? 1 : 0));
+            const size_t lds =
+                workspace::w4a16_mrows_lds_bytes(GW * STEPS * 1024, M, (fusion.gate ? 2 : 1) * (tiles_q + (tiles_r ? 1 : 0)));
             if (lds > MAX_LDS_BYTES)
                 return hipErrorInvalidValue;
-            auto kernel = &w4a16_mrows_kernel<GW, STEPS, MB>;
+            auto kernel = &w4a16_mrows_kernel<GW, STEPS, MB, FUSED>;
             if (lds > 64 * 1024)
             {
                 static LdsGrant granted;
@@ -478,18 +559,22 @@ namespace nnf
                     return e;
             }
             hipLaunchKernelGGL(kernel, dim3(grid), dim3(MR_WAVES * 64), lds, stream, (const half_t*)A, (const uint8_t*)Wq,
-                               (const half_t*)S, (half_t*)Y, N, tiles_q, tiles_r, M | (zp << 8));
+                               (const half_t*)S, (half_t*)Y, N, tiles_q, tiles_r, M | (zp << 8), fusion_args(fusion),
+                               fusion.gate ? 1 : 0);
             return hipGetLastError();
         }
 
         template <int GW, int STEPS>
         hipError_t launch_mrows(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M, int N, int zp,
-                                int num_cu)
+                                int num_cu, const GemvFusion& fusion)
         {
+            const bool fused = fusion.any();
             if (M <= 16)
-                return launch_mrows_mb<GW, STEPS, 1>(stream, A, Wq, S, Y, M, N, zp, num_cu);
+                return fused ? launch_mrows_mb<GW, STEPS, 1, true>(stream, A, Wq, S, Y, M, N, zp, num_cu, fusion)
+                             : launch_mrows_mb<GW, STEPS, 1, false>(stream, A, Wq, S, Y, M, N, zp, num_cu, fusion);
             if constexpr (GW * STEPS <= 4)
-                return launch_mrows_mb<GW, STEPS, 2>(stream, A, Wq, S, Y, M, N, zp, num_cu);
+                return fused ? launch_mrows_mb<GW, STEPS, 2, true>(stream, A, Wq, S, Y, M, N, zp, num_cu, fusion)
+                             : launch_mrows_mb<GW, STEPS, 2, false>(stream, A, Wq, S, Y, M, N, zp, num_cu, fusion);
             return hipErrorInvalidValue;
         }
     } // namespace
@@ -497,18 +582,18 @@ namespace nnf
     namespace
     {
         // ranges == 1: the whole of K, fp16 results to Y; otherwise ranges of range_groups groups, fp32 sums to partial
-        template <int GW, int STEPS, int MB>
+        template <int GW, int STEPS, int MB, bool FUSED>
         hipError_t launch_mrows_any_mb(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M, int N, int K,
-                                    int zp, int num_cu, float* partial, int ranges, int range_groups)
+                                       int zp, int num_cu, float* partial, int ranges, int range_groups, const GemvFusion& fusion)
         {
             const int n_tiles = (N + 15) / 16;
             const int per_range = num_cu / ranges > 0 ? num_cu / ranges : 1;
             const int grid = n_tiles < per_range ? n_tiles : per_range;
             const int tiles_q = n_tiles / grid, tiles_r = n_tiles % grid;
-            const size_t lds = workspace::w4a16_mrows_lds_bytes_gw(GW, M, tiles_q + (tiles_r ? 1 : 0));
-            if (lds > MAX_LDS_BYTES)
+            const size_t lds = workspace::w4a16_mrows_lds_bytes_gw(GW, M, (fusion.gate ? 2 : 1) * (tiles_q + (tiles_r ? 1 : 0)));
+            if (lds > MAX_LDS_BYTES || (ranges > 1 && (fusion.gate || fusion.bias || fusion.residual || fusion.rstd)))
                 return hipErrorInvalidValue;
-            auto kernel = &w4a16_mrows_any_kernel<GW, STEPS, MB>;
+            auto kernel = &w4a16_mrows_any_kernel<GW, STEPS, MB, FUSED>;
             if (lds > 64 * 1024)
             {
                 static LdsGrant granted;
@@ -518,41 +603,61 @@ namespace nnf
             }
             hipLaunchKernelGGL(kernel, dim3(grid, ranges), dim3(MR_WAVES * 64), lds, stream, (const half_t*)A, (const uint8_t*)Wq,
                                (const half_t*)S, (half_t*)Y, ranges > 1 ? partial : nullptr, N, K, range_groups, tiles_q, tiles_r,
-                               M | (zp << 8));
+                               M | (zp << 8), fusion_args(fusion), fusion.gate ? 1 : 0);
             return hipGetLastError();
+        }
+
+        template <int GW, int STEPS, bool FUSED>
+        hipError_t launch_mrows_any_f(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M, int N, int K,
+                                      int zp, int num_cu, float* partial, int ranges, int range_groups, const GemvFusion& fusion)
+        {
+            if (M <= 16)
+                return launch_mrows_any_mb<GW, STEPS, 1, FUSED>(stream, A, Wq, S, Y, M, N, K, zp, num_cu, partial, ranges, range_groups,
+                                                                fusion);
+            if constexpr (GW * STEPS <= 4)
+                if (M <= 32)
+                    return launch_mrows_any_mb<GW, STEPS, 2, FUSED>(stream, A, Wq, S, Y, M, N, K, zp, num_cu, partial, ranges,
+                                                                    range_groups, fusion);
+            if constexpr (GW * STEPS <= 2)
+                if (M <= 64)
+                    return launch_mrows_any_mb<GW, STEPS, 4, FUSED>(stream, A, Wq, S, Y, M, N, K, zp, num_cu, partial, ranges,
+                                                                    range_groups, fusion);
+            return hipErrorInvalidValue;
         }
 
         template <int GW, int STEPS>
         hipError_t launch_mrows_any(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M, int N, int K,
-                                    int zp, int num_cu, float* partial = nullptr, int ranges = 1, int range_groups = 64)
+                                    int zp, int num_cu, const GemvFusion& fusion, float* partial = nullptr, int ranges = 1,
+                                    int range_groups = 64)
         {
-            if (M <= 16)
-                return launch_mrows_any_mb<GW, STEPS, 1>(stream, A, Wq, S, Y, M, N, K, zp, num_cu, partial, ranges, range_groups);
-            if constexpr (GW * STEPS <= 4)
-                if (M <= 32)
-                    return launch_mrows_any_mb<GW, STEPS, 2>(stream, A, Wq, S, Y, M, N, K, zp, num_cu, partial, ranges, range_groups);
-            if constexpr (GW * STEPS <= 2)
-                if (M <= 64)
-                    return launch_mrows_any_mb<GW, STEPS, 4>(stream, A, Wq, S, Y, M, N, K, zp, num_cu, partial, ranges, range_groups);
-            return hipErrorInvalidValue;
+            return fusion.any() ? launch_mrows_any_f<GW, STEPS, true>(stream, A, Wq, S, Y, M, N, K, zp, num_cu, partial, ranges,
+                                                                      range_groups, fusion)
+                                : launch_mrows_any_f<GW, STEPS, false>(stream, A, Wq, S, Y, M, N, K, zp, num_cu, partial, ranges,
+                                                                       range_groups, fusion);
         }
     } // namespace
 
-    bool w4a16_mrows_supported(int M, int N, int K, int num_cu) { return workspace::w4a16_mrows_fits(M, N, K, num_cu); }
-    bool w4a16_mrows_preferred(int M, int N, int K, int num_cu) { return workspace::w4a16_mrows_preferred(M, N, K, num_cu); }
+    bool w4a16_mrows_supported(int M, int N, int K, int num_cu, bool gate)
+    {
+        return workspace::w4a16_mrows_fits(M, N, K, num_cu, gate);
+    }
+    bool w4a16_mrows_preferred(int M, int N, int K, int num_cu, bool gate)
+    {
+        return workspace::w4a16_mrows_preferred(M, N, K, num_cu, gate);
+    }
 
     hipError_t launch_w4a16_mrows(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M, int N,
-                                  int K, int zp, int num_cu)
+                                  int K, int zp, int num_cu, const GemvFusion& fusion)
     {
-        if (!w4a16_mrows_supported(M, N, K, num_cu))
+        if (!w4a16_mrows_supported(M, N, K, num_cu, fusion.gate) || (fusion.gate && (fusion.bias || fusion.residual)))
             return hipErrorInvalidValue;
         if (!workspace::w4a16_mrows_fixed_k(M, K))
         {
             switch (workspace::w4a16_mrows_step_groups(M, K))
             {
-            case 2: return launch_mrows_any<2, 2>(stream, A, Wq, S, Y, M, N, K, zp, num_cu);
-            case 3: return launch_mrows_any<3, 2>(stream, A, Wq, S, Y, M, N, K, zp, num_cu);
-            default: return launch_mrows_any<4, 2>(stream, A, Wq, S, Y, M, N, K, zp, num_cu);
+            case 2: return launch_mrows_any<2, 2>(stream, A, Wq, S, Y, M, N, K, zp, num_cu, fusion);
+            case 3: return launch_mrows_any<3, 2>(stream, A, Wq, S, Y, M, N, K, zp, num_cu, fusion);
+            default: return launch_mrows_any<4, 2>(stream, A, Wq, S, Y, M, N, K, zp, num_cu, fusion);
             }
         }
         // K / 1024 = groups per wavefront and tile, walked in STEPS steps of GW groups.  Two steps per tile where
@@ -561,12 +666,12 @@ namespace nnf
         // 5-25 % faster than either at K = 4096, 6144 and 8192.
         switch (K >> 10)
         {
-        case 1: return launch_mrows<1, 1>(stream, A, Wq, S, Y, M, N, zp, num_cu);
-        case 2: return launch_mrows<1, 2>(stream, A, Wq, S, Y, M, N, zp, num_cu);
-        case 3: return launch_mrows<3, 1>(stream, A, Wq, S, Y, M, N, zp, num_cu);
-        case 4: return launch_mrows<2, 2>(stream, A, Wq, S, Y, M, N, zp, num_cu);
-        case 6: return launch_mrows<3, 2>(stream, A, Wq, S, Y, M, N, zp, num_cu);
-        default: return launch_mrows<4, 2>(stream, A, Wq, S, Y, M, N, zp, num_cu);
+        case 1: return launch_mrows<1, 1>(stream, A, Wq, S, Y, M, N, zp, num_cu, fusion);
+        case 2: return launch_mrows<1, 2>(stream, A, Wq, S, Y, M, N, zp, num_cu, fusion);
+        case 3: return launch_mrows<3, 1>(stream, A, Wq, S, Y, M, N, zp, num_cu, fusion);
+        case 4: return launch_mrows<2, 2>(stream, A, Wq, S, Y, M, N, zp, num_cu, fusion);
+        case 6: return launch_mrows<3, 2>(stream, A, Wq, S, Y, M, N, zp, num_cu, fusion);
+        default: return launch_mrows<4, 2>(stream, A, Wq, S, Y, M, N, zp, num_cu, fusion);
         }
     }
 
@@ -575,17 +680,19 @@ namespace nnf
     int w4a16_mrows_ksplits(int M, int N, int K, int num_cu) { return workspace::w4a16_mrows_split(M, N, K, num_cu).ranges; }
 
     hipError_t launch_w4a16_mrows_split(hipStream_t stream, const void* A, const void* Wq, const void* S, float* partial, int M,
-                                        int N, int K, int zp, int num_cu)
+                                        int N, int K, int zp, int num_cu, const void* gamma)
     {
+        GemvFusion fusion; // of the fused parts only the RMSNorm weight belongs to this launch
+        fusion.gamma = gamma;
         const workspace::MrowsSplit sp = workspace::w4a16_mrows_split(M, N, K, num_cu);
         if (sp.ranges < 2 || !partial)
             return hipErrorInvalidValue;
         switch (sp.gw)
         {
-        case 1: return launch_mrows_any<1, 2>(stream, A, Wq, S, nullptr, M, N, K, zp, num_cu, partial, sp.ranges, sp.range_groups);
-        case 2: return launch_mrows_any<2, 2>(stream, A, Wq, S, nullptr, M, N, K, zp, num_cu, partial, sp.ranges, sp.range_groups);
-        case 3: return launch_mrows_any<3, 2>(stream, A, Wq, S, nullptr, M, N, K, zp, num_cu, partial, sp.ranges, sp.range_groups);
-        default: return launch_mrows_any<4, 2>(stream, A, Wq, S, nullptr, M, N, K, zp, num_cu, partial, sp.ranges, sp.range_groups);
+        case 1: return launch_mrows_any<1, 2>(stream, A, Wq, S, nullptr, M, N, K, zp, num_cu, fusion, partial, sp.ranges, sp.range_groups);
+        case 2: return launch_mrows_any<2, 2>(stream, A, Wq, S, nullptr, M, N, K, zp, num_cu, fusion, partial, sp.ranges, sp.range_groups);
+        case 3: return launch_mrows_any<3, 2>(stream, A, Wq, S, nullptr, M, N, K, zp, num_cu, fusion, partial, sp.ranges, sp.range_groups);
+        default: return launch_mrows_any<4, 2>(stream, A, Wq, S, nullptr, M, N, K, zp, num_cu, fusion, partial, sp.ranges, sp.range_groups);
         }
     }
 } // namespace nnf

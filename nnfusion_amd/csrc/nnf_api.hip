@@ -139,12 +139,13 @@ namespace
                 return NNF_ERR_UNSUPPORTED_SHAPE;
             return (int)nnf::launch_w4a16_gemv(s, A, Wq, scales, Y, M, N, K, zp, dev.num_cu);
         }
-        if (!nnf::w4a16_path_supported(M, N, K, NNF_ACT_NONE, dev.num_cu, choice.path))
+        const nnf::workspace::W4A16Route route =
+            nnf::workspace::route_w4a16(M, N, K, false, false, false, dev.num_cu, choice.path, choice.tile_rows, choice.k_parts);
+        if (route.kind == nnf::workspace::W4A16Route::NONE)
             return NNF_ERR_UNSUPPORTED_SHAPE;
         // the GEMV kernels over ranges of K and the tile GEMM park partial sums in scratch memory; the check is for
         // what this launch writes on this device
-        if (!workspace_ok(nnf::w4a16_gemm_partial_bytes(M, N, K, NNF_ACT_NONE, false, dev.num_cu, choice), workspace,
-                          workspace_bytes))
+        if (!workspace_ok(route.partial_bytes, workspace, workspace_bytes))
             return NNF_ERR_WORKSPACE_TOO_SMALL;
         return (int)nnf::launch_w4a16_gemm(s, A, Wq, scales, Y, M, N, K, zp, nullptr, 0.f, nullptr, nullptr, NNF_ACT_NONE,
                                            nullptr, workspace, dev.num_cu, choice);
@@ -193,17 +194,11 @@ size_t nnf_w4a16_gemm_variant_workspace_bytes(int M, int N, int K, int group, in
     nnf::LaunchChoice choice;
     if (M <= 0 || N <= 0 || K < 128 || !make_choice(variant, plan, NNF_W4A16_GEMV_ROWS, choice))
         return 0;
-    if (variant == NNF_W4A16_GEMM_MFMA)
-        return nnf::workspace::plan_w4a16_sk_with(M, N, K, false, nnf::workspace::PLAN_CUS, choice.tile_rows, choice.k_parts)
-            .bytes();
-    if (variant == NNF_W4A16_AUTO)
-        return nnf::workspace::w4a16_gemm(M, N, K, group);
-    // the GEMV kernels over ranges of K (shapes whose activations exceed one workgroup's LDS / registers)
-    if (variant == NNF_W4A16_GEMV_MFMA && !nnf::workspace::w4a16_skinny_fits(M, N, K))
-        return nnf::workspace::skinny_split_bytes(M, N, K);
-    if (variant == NNF_W4A16_GEMV_ROWS && M > 1 && !nnf::workspace::w4a16_mrows_fits(M, N, K, nnf::workspace::PLAN_CUS))
-        return nnf::workspace::mrows_split_bytes(M, N, K);
-    return 0;
+    if (variant == NNF_W4A16_GEMV_VALU || group != 128)
+        return 0;
+    return nnf::workspace::route_w4a16(M, N, K, false, false, false, nnf::workspace::PLAN_CUS, variant, choice.tile_rows,
+                                       choice.k_parts)
+        .partial_bytes;
 }
 
 int nnf_w4a16_gemm_variant(nnf_stream_t stream, const void* A, const void* Wq, const void* scales, void* Y, int M,
@@ -242,16 +237,18 @@ int nnf_w4a16_gemm_fused_variant(nnf_stream_t stream, const void* A, const void*
     st = current_device_info(dev);
     if (st != NNF_OK)
         return st;
-    if (!nnf::w4a16_path_supported(M, N, K, act, dev.num_cu, choice.path))
+    const nnf::workspace::W4A16Route route =
+        nnf::workspace::route_w4a16(M, N, K, act == NNF_ACT_SILU_GATE, rms_gamma != nullptr, residual == Y, dev.num_cu,
+                                    choice.path, choice.tile_rows, choice.k_parts);
+    if (route.kind == nnf::workspace::W4A16Route::NONE)
         return NNF_ERR_UNSUPPORTED_SHAPE;
     // [ RMSNorm scratch ][ what this launch parks, on this device ]
-    const size_t rms_bytes = rms_gamma ? nnf::workspace::rms_rows(M, K) : 0;
-    const size_t need = rms_bytes + nnf::w4a16_gemm_partial_bytes(M, N, K, act, residual == Y, dev.num_cu, choice);
-    if (!workspace_ok(need, workspace, workspace_bytes))
+    if (!workspace_ok(route.rms_bytes + route.partial_bytes, workspace, workspace_bytes))
         return NNF_ERR_WORKSPACE_TOO_SMALL;
     uint8_t* ws = (uint8_t*)workspace;
     return (int)nnf::launch_w4a16_gemm((hipStream_t)stream, A, Wq, scales, Y, M, N, K, zp, rms_gamma, rms_eps, bias,
-                                       residual, act, ws, ws ? ws + rms_bytes : nullptr, dev.num_cu, choice);
+                                       residual, act, route.rms_bytes ? ws : nullptr,
+                                       route.partial_bytes ? ws + route.rms_bytes : nullptr, dev.num_cu, choice);
 }
 
 int nnf_w4a16_gemm_fused(nnf_stream_t stream, const void* A, const void* Wq, const void* scales, void* Y, int M, int N,
@@ -365,14 +362,14 @@ int nnf_fused_mlp_w4a16(nnf_stream_t stream, const void* x, const void* gamma, f
     {
         // what the two launches park behind h, on this device (the down projection's residual is x: in place when
         // the caller passes out == x)
-        const size_t a = nnf::w4a16_gemm_partial_bytes(M, I, H, NNF_ACT_SILU_GATE, false, dev.num_cu);
-        const size_t b = nnf::w4a16_gemm_partial_bytes(M, H, I, NNF_ACT_NONE, out == x, dev.num_cu);
-        if (!workspace || workspace_bytes < nnf::workspace::fused_mlp_partial_offset(M, H, I) + (a > b ? a : b))
+        const size_t a = nnf::workspace::route_w4a16(M, I, H, true, true, false, dev.num_cu).partial_bytes;
+        const size_t b = nnf::workspace::route_w4a16(M, H, I, false, false, out == x, dev.num_cu).partial_bytes;
+        if (!workspace || workspace_bytes < nnf::workspace::fused_mlp_partial_offset(M, H, I, dev.num_cu) + (a > b ? a : b))
             return NNF_ERR_WORKSPACE_TOO_SMALL;
     }
     uint8_t* ws = (uint8_t*)workspace;
-    void* h = ws + nnf::workspace::fused_mlp_h_offset(M, H);
-    void* partial = ws + nnf::workspace::fused_mlp_partial_offset(M, H, I);
+    void* h = ws + nnf::workspace::fused_mlp_h_offset(M, H, I, dev.num_cu);
+    void* partial = ws + nnf::workspace::fused_mlp_partial_offset(M, H, I, dev.num_cu);
     // h = SiLU(gate) * up, gate|up = RMSNorm(x) . Wgu^T : the normalisation pre-pass, then one GEMM with the
     // gate and up projections as the two halves of every N tile
     hipError_t e = nnf::launch_w4a16_gemm((hipStream_t)stream, x, Wgu, Sgu, h, M, I, H, zp, gamma, eps, nullptr,

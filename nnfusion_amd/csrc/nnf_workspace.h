@@ -290,16 +290,20 @@ namespace nnf
             int kshift = 0; // log2 of the wavefronts that share a row
             int depth = 0;  // rows in flight per wavefront
             // ring + activations (+ zeros) + their constants + the workgroup's scales + parked outputs + row counters
-            size_t lds_bytes(int N, int K, int grid) const
+            // (gate: N outputs from 2 N weight rows; a workgroup holds the scales of its gate rows and of its up rows as
+            // two blocks, each rounded up to whole KiB)
+            size_t lds_bytes(int N, int K, int grid, bool gate = false) const
             {
-                const size_t rows = (size_t)(N / grid + 1);                       // of a workgroup, at most
+                const size_t rows = (size_t)(N / grid + 1);                       // outputs of a workgroup, at most
                 const size_t a_pad = (((size_t)(K >> 3) + 63) & ~(size_t)63) + 4; // 16-byte units of activations
+                const size_t halves = gate ? 2 : 1;
                 return (size_t)ROWS_WAVES * depth * seg * 1024 + a_pad * 16 + a_pad * 4 +
-                       ((rows * (size_t)(K >> 7) * 2 + 1023) & ~(size_t)1023) + (rows << kshift) * sizeof(float) + 64;
+                       halves * ((rows * (size_t)(K >> 7) * 2 + 1023) & ~(size_t)1023) +
+                       ((halves * rows) << kshift) * sizeof(float) + 64;
             }
         };
-        // forced_depth: for experiments (0: the plan's own choice)
-        inline RowsPlan plan_w4a16_rows(int M, int N, int K, int num_cu, int forced_depth = 0)
+        // N: outputs (gate: from 2 N weight rows).  forced_depth: 0 = the plan's own choice
+        inline RowsPlan plan_w4a16_rows(int M, int N, int K, int num_cu, int forced_depth = 0, bool gate = false)
         {
             RowsPlan p;
             // whole 16-byte pieces of scales per segment, 4-byte aligned: K a multiple of 256
@@ -316,7 +320,7 @@ namespace nnf
             p.seg = (loads_per_row + (1 << kshift) - 1) >> kshift;
             const int grid = rows_grid(N, num_cu);
             // rows per wavefront of a K segment: the first `depth` of them are fixed
-            const int rows_q = (N / grid) / (ROWS_WAVES >> kshift);
+            const int rows_q = ((gate ? 2 : 1) * (N / grid)) / (ROWS_WAVES >> kshift);
             // Two rows in flight per wavefront (a CU takes about 64 wavefront-wide loads in flight; more and the
             // wavefronts stall at issue), a little deeper when a wavefront has many rows to walk (measured).
             const int depth_max = p.seg == 3 ? 2 : 4;
@@ -325,51 +329,13 @@ namespace nnf
                 p.depth = depth_max;
             if (p.depth > rows_q)
                 p.depth = rows_q < 1 ? 1 : rows_q;
-            while (p.depth > 1 && p.lds_bytes(N, K, grid) > LDS_BYTES_PER_CU)
+            while (p.depth > 1 && p.lds_bytes(N, K, grid, gate) > LDS_BYTES_PER_CU)
                 --p.depth;
-            if (p.lds_bytes(N, K, grid) > LDS_BYTES_PER_CU)
+            if (p.lds_bytes(N, K, grid, gate) > LDS_BYTES_PER_CU)
                 p.seg = 0;
             return p;
         }
 
-        // normalised activations of the RMSNorm prologue (fp16 [M, K])
-        // RMSNorm prologue.  The tile GEMM folds the normalisation in and needs one fp32 per row (rstd); the kernels
-        // that serve up to 40 rows read normalised activations: fp16 [M, K].
-        inline size_t rms_rows(int M, int K)
-        {
-            if (M <= 0 || K <= 0)
-                return 0;
-            return M <= 40 ? align256((size_t)M * K * 2) : align256((size_t)M * sizeof(float));
-        }
-
-        inline size_t mrows_split_bytes(int M, int N_total, int K); // the row-streaming MFMA kernel over ranges of K
-        // Fused calls with at most 40 rows may run the GEMV kernel into scratch and an element-wise epilogue from
-        // there (the [M, 2N] gate | up pair; a residual that is the output buffer): fp16 [M, N_total].
-        inline size_t gemv_scratch_bytes(int M, int N_total) { return (M > 0 && M <= 40) ? align256((size_t)M * N_total * 2) : 0; }
-
-        // nnf_w4a16_gemm: [ partial sums ]
-        inline size_t w4a16_gemm(int M, int N, int K, int)
-        {
-            if (M <= 0 || N <= 0 || K < 128)
-                return 0;
-            if (w4a16_skinny_fits(M, N, K))
-                return 0; // served by the skinny kernel
-            const size_t a = plan_w4a16_sk(M, N, K, false, PLAN_CUS).bytes();
-            const size_t b = skinny_split_bytes(M, N, K), c = mrows_split_bytes(M, N, K);
-            return a > b ? (a > c ? a : c) : (b > c ? b : c);
-        }
-        // nnf_w4a16_gemm_fused: [ normalised activations ][ partial sums ]
-        inline size_t w4a16_gemm_fused(int M, int N, int K, int, int act)
-        {
-            if (M <= 0 || N <= 0 || K < 128)
-                return 0;
-            const bool gate = act == 1;
-            const size_t a = plan_w4a16_sk(M, N, K, gate, PLAN_CUS).bytes();
-            const size_t b = skinny_split_bytes(M, gate ? 2 * N : N, K), c = mrows_split_bytes(M, gate ? 2 * N : N, K);
-            const size_t d = gemv_scratch_bytes(M, gate ? 2 * N : N);
-            const size_t bc = b > c ? b : c, ad = a > d ? a : d;
-            return rms_rows(M, K) + (ad > bc ? ad : bc);
-        }
         // ---- W8A8 ---------------------------------------------------------------------------------------
         constexpr int Q8_SKINNY_CPS = 2; // preferred chunks per wavefront and pass (more in flight measured slower)
         struct Q8SkinnyPlan
@@ -466,7 +432,8 @@ namespace nnf
         {
             return w4a16_mrows_lds_bytes_gw(w4a16_mrows_step_groups(M, K), M, tiles);
         }
-        inline bool w4a16_mrows_fits(int M, int N, int K, int num_cu)
+        // N: output columns; gate: from 2 N weight rows (a workgroup walks the gate and the up tile of each output tile)
+        inline bool w4a16_mrows_fits(int M, int N, int K, int num_cu, bool gate = false)
         {
             if (M < 2 || M > 32 || N < 16 || num_cu < 1 || K < 1024 || K > 8192 || (K & 255))
                 return false;
@@ -474,7 +441,7 @@ namespace nnf
                 return false;
             const int n_tiles = (N + 15) / 16;
             const int grid = n_tiles < num_cu ? n_tiles : num_cu;
-            return w4a16_mrows_lds_bytes(K, M, (n_tiles + grid - 1) / grid) <= LDS_BYTES_PER_CU;
+            return w4a16_mrows_lds_bytes(K, M, (gate ? 2 : 1) * ((n_tiles + grid - 1) / grid)) <= LDS_BYTES_PER_CU;
         }
         // K above 8192 (above 4096 for 17 .. 32 rows, above 2048 for 33 .. 64; a multiple of 256): the run-time-K form over equal ranges of K (in whole pairs of
         // groups; the last range may be shorter), each on its share of the CUs; fp32 sums per range, added by the
@@ -522,9 +489,9 @@ namespace nnf
         // run-time K: 0-5 % / 15-35 % faster at K = 3584, 5120, 7168 (but up to 19 % slower below eight rows at K = 7168), level
         // at K = 2560, slower at K = 1536 and 2304, where most of what the wavefronts fetch is discarded: taken when at
         // least three quarters of the fetched groups count.
-        inline bool w4a16_mrows_preferred(int M, int N, int K, int num_cu)
+        inline bool w4a16_mrows_preferred(int M, int N, int K, int num_cu, bool gate = false)
         {
-            if (!w4a16_mrows_fits(M, N, K, num_cu))
+            if (!w4a16_mrows_fits(M, N, K, num_cu, gate))
                 return false;
             if (w4a16_mrows_fixed_k(M, K))
                 return true;
@@ -532,23 +499,6 @@ namespace nnf
             if (gw == 4 && M < 8) // K = 6400 .. 7936: N = K = 7168 takes 10.7 us at M = 2 against 9.0 (level from M = 6 on)
                 return false;
             return 4 * (K >> 7) >= 3 * 16 * gw;
-        }
-        inline bool w4a16_variant_fits(int M, int N, int K, int variant, int num_cu)
-        {
-            if (M <= 0 || N <= 0 || K < 128 || (K & 127))
-                return false;
-            switch (variant)
-            {
-            case 0: // automatic
-            case 3: // MFMA tile GEMM
-                return true;
-            case 1: return w4a16_gemv_valu_fits(M, K);
-            case 2: return w4a16_skinny_fits(M, N, K) || w4a16_skinny_ksplits(M, N, K) > 0;
-            case 4:
-                return plan_w4a16_rows(M, N, K, num_cu, 0).seg != 0 || w4a16_mrows_fits(M, N, K, num_cu) ||
-                       w4a16_mrows_split(M, N, K, num_cu).ranges > 0;
-            default: return false;
-            }
         }
         // ---- W8A8, one activation row: the row-streaming GEMV (w8a8_gemv_rows.hip) ----
         struct Q8RowsPlan
@@ -601,31 +551,117 @@ namespace nnf
                 return 0;
             return gemm_partial_bytes(M, N, false, plan_w8a8_gemm(M, N, K));
         }
-        // nnf_fused_mlp_w4a16: [ normalised x: M x H fp16 ][ h: M x I fp16 ][ partial sums of either GEMM ]
-        inline size_t fused_mlp_h_offset(int M, int H) { return rms_rows(M, H); }
-        inline size_t fused_mlp_partial_offset(int M, int H, int I)
+        // ---- which kernel serves an fp16 x int4 product, and the scratch memory that launch uses --------------------
+        // Decided from the shape, the fused parts asked for and the device's CU count alone: the launcher, the entry
+        // points' workspace checks and the *_workspace_bytes queries (for PLAN_CUS) all ask this one function.
+        struct W4A16Route
         {
-            return rms_rows(M, H) + align256((size_t)M * I * 2);
+            // NONE: the kernel family asked for cannot serve the shape
+            enum Kind { NONE, ROWS, MROWS, SKINNY, MROWS_SPLIT, SKINNY_SPLIT, TILE } kind = NONE;
+            int ksplits = 0;          // *_SPLIT: ranges of K (fp32 partial sums, then the reduction pass)
+            bool via_scratch = false; // SKINNY: products to scratch first, an element-wise epilogue kernel reads them
+            SkPlan plan;              // TILE
+            size_t partial_bytes = 0; // partial sums / parked tiles / the products ahead of an element-wise epilogue
+            size_t rms_bytes = 0;     // RMSNorm prologue: rstd, fp32 [M] (the kernels multiply the RMSNorm weight in
+                                      // themselves), or for the MFMA GEMV kernel the normalised activations, fp16 [M, K]
+        };
+        // N: output columns (gate: from 2 N weight rows); rms: with the RMSNorm prologue; in_place_residual: the residual
+        // is the output buffer itself.  path: 0 the library's order of preference, 2 / 4 one family of GEMV kernels only
+        // (values of nnf_w4a16_variant), 3 the tile GEMM with tile_rows / k_parts (0: its own plan).
+        inline W4A16Route route_w4a16(int M, int N, int K, bool gate, bool rms, bool in_place_residual, int num_cu, int path = 0,
+                                      int tile_rows = 0, int k_parts = 0)
+        {
+            W4A16Route r;
+            if (M <= 0 || N <= 0 || K < 128 || (K & 127) || num_cu < 1)
+                return r;
+            const int n_rows = gate ? 2 * N : N; // weight rows
+            const bool any = path == 0, rows_family = any || path == 4, skinny_family = any || path == 2;
+            const size_t rstd_bytes = rms ? align256((size_t)M * sizeof(float)) : 0;
+            const size_t xn_bytes = rms ? align256((size_t)M * K * 2) : 0;
+            if (path != 3)
+            {
+                // the row-streaming kernels apply prologue and epilogue themselves: one launch, no scratch memory
+                if (rows_family && plan_w4a16_rows(M, N, K, num_cu, 0, gate).seg != 0)
+                    return r.kind = W4A16Route::ROWS, r.rms_bytes = rstd_bytes, r;
+                if (rows_family && M > 1 && (any ? w4a16_mrows_preferred(M, N, K, num_cu, gate) : w4a16_mrows_fits(M, N, K, num_cu, gate)))
+                    return r.kind = W4A16Route::MROWS, r.rms_bytes = rstd_bytes, r;
+                // the MFMA GEMV kernel writes plain products: an epilogue that cannot work in place (the [M, 2N] gate | up
+                // pair, a residual that is the output buffer) reads them from scratch memory
+                if (skinny_family && M <= 16 && w4a16_skinny_fits(M, n_rows, K))
+                {
+                    r.kind = W4A16Route::SKINNY;
+                    r.via_scratch = gate || in_place_residual;
+                    r.partial_bytes = r.via_scratch ? align256((size_t)M * n_rows * 2) : 0;
+                    r.rms_bytes = xn_bytes;
+                    return r;
+                }
+                // more activations than one workgroup holds: ranges of K, fp32 sums per range, and the reduction pass
+                // (K above 8192 in multiples of 256: the row-streaming MFMA kernel, otherwise the split-K one)
+                if (rows_family && (r.ksplits = w4a16_mrows_split(M, n_rows, K, num_cu).ranges) > 0)
+                {
+                    r.kind = W4A16Route::MROWS_SPLIT;
+                    r.partial_bytes = align256((size_t)r.ksplits * M * n_rows * sizeof(float));
+                    r.rms_bytes = rstd_bytes;
+                    return r;
+                }
+                if (skinny_family && (r.ksplits = w4a16_skinny_ksplits(M, n_rows, K)) > 0)
+                {
+                    r.kind = W4A16Route::SKINNY_SPLIT;
+                    r.partial_bytes = align256((size_t)r.ksplits * M * n_rows * sizeof(float));
+                    r.rms_bytes = xn_bytes;
+                    return r;
+                }
+                r.ksplits = 0;
+                if (!any)
+                    return r;
+            }
+            r.kind = W4A16Route::TILE;
+            r.plan = plan_w4a16_sk_with(M, N, K, gate, num_cu, tile_rows, k_parts);
+            r.partial_bytes = r.plan.bytes();
+            r.rms_bytes = rstd_bytes;
+            return r;
         }
-        inline size_t fused_mlp_w4a16(int M, int H, int I, int)
+
+        inline bool w4a16_variant_fits(int M, int N, int K, int variant, int num_cu)
+        {
+            if (M <= 0 || N <= 0 || K < 128 || (K & 127))
+                return false;
+            if (variant == 1)
+                return w4a16_gemv_valu_fits(M, K);
+            return variant >= 0 && variant <= 4 && route_w4a16(M, N, K, false, false, false, num_cu, variant).kind != W4A16Route::NONE;
+        }
+        // nnf_w4a16_gemm: [ partial sums ]
+        inline size_t w4a16_gemm(int M, int N, int K, int, int num_cu = PLAN_CUS)
+        {
+            return route_w4a16(M, N, K, false, false, false, num_cu).partial_bytes;
+        }
+        // nnf_w4a16_gemm_fused: [ RMSNorm scratch ][ partial sums ], whichever of the optional parts the call uses
+        inline size_t w4a16_gemm_fused(int M, int N, int K, int, int act, int num_cu = PLAN_CUS)
+        {
+            const bool gate = act == 1;
+            const W4A16Route a = route_w4a16(M, N, K, gate, true, false, num_cu);
+            const W4A16Route b = route_w4a16(M, N, K, gate, true, !gate, num_cu);
+            return a.rms_bytes + (a.partial_bytes > b.partial_bytes ? a.partial_bytes : b.partial_bytes);
+        }
+        // nnf_fused_mlp_w4a16: [ RMSNorm scratch of the first product ][ h: M x I fp16 ][ partial sums of either product ]
+        inline size_t fused_mlp_h_offset(int M, int H, int I, int num_cu = PLAN_CUS)
+        {
+            return route_w4a16(M, I, H, true, true, false, num_cu).rms_bytes;
+        }
+        inline size_t fused_mlp_partial_offset(int M, int H, int I, int num_cu = PLAN_CUS)
+        {
+            return fused_mlp_h_offset(M, H, I, num_cu) + align256((size_t)M * I * 2);
+        }
+        inline size_t fused_mlp_w4a16(int M, int H, int I, int, int num_cu = PLAN_CUS)
         {
             if (M <= 0 || I <= 0 || H < 128 || I < 128)
                 return 0;
-            size_t a = plan_w4a16_sk(M, I, H, true, PLAN_CUS).bytes();
-            size_t b = plan_w4a16_sk(M, H, I, false, PLAN_CUS).bytes();
-            size_t c = skinny_split_bytes(M, 2 * I, H), d = skinny_split_bytes(M, H, I);
-            const size_t e = mrows_split_bytes(M, 2 * I, H), f = mrows_split_bytes(M, H, I);
-            // the GEMV kernels' products ahead of an element-wise epilogue: gate | up of the first GEMM, and the
-            // second GEMM's when its residual x is the output buffer itself
-            size_t g = gemv_scratch_bytes(M, 2 * I);
-            const size_t g2 = gemv_scratch_bytes(M, H);
-            g = g > g2 ? g : g2;
-            c = c > e ? c : e;
-            c = c > g ? c : g;
-            d = d > f ? d : f;
-            a = a > b ? a : b;
-            b = c > d ? c : d;
-            return fused_mlp_partial_offset(M, H, I) + (a > b ? a : b);
+            const size_t a = route_w4a16(M, I, H, true, true, false, num_cu).partial_bytes;
+            // (the second product's residual x may be the output buffer itself)
+            const size_t b = route_w4a16(M, H, I, false, false, false, num_cu).partial_bytes;
+            const size_t c = route_w4a16(M, H, I, false, false, true, num_cu).partial_bytes;
+            const size_t bc = b > c ? b : c;
+            return fused_mlp_partial_offset(M, H, I, num_cu) + (a > bc ? a : bc);
         }
     } // namespace workspace
 } // namespace nnf

@@ -891,7 +891,35 @@ int main(int argc, char** argv)
                    !ws::w4a16_skinny_fits(4, 8, 4096));
             // weights addressed with 32-bit offsets
             EXPECT(!ws::w4a16_skinny_fits(1, 1 << 20, 8192) && ws::w4a16_skinny_fits(1, 1 << 19, 8192));
-            EXPECT(ws::w4a16_gemm(1, 4096, 4096, 128) == 0 && ws::w4a16_gemm(16, 8192, 8192, 128) > 0);
+            // one launch, no scratch memory, where a row-streaming kernel serves the shape; ranges of K and shared tiles park sums
+            EXPECT(ws::w4a16_gemm(1, 4096, 4096, 128) == 0 && ws::w4a16_gemm(16, 8192, 8192, 128) == 0);
+            EXPECT(ws::w4a16_gemm(16, 4096, 11008, 128) == (size_t)3 * 16 * 4096 * 4 && ws::w4a16_gemm(128, 8192, 8192, 128) > 0);
+            // the decode route of a fused MLP block: the row-streaming kernels take the RMSNorm weight, the gate product and
+            // the residual themselves: rstd is the only scratch of the first product, the second needs none
+            for (int m : {1, 16, 32})
+            {
+                const auto up = ws::route_w4a16(m, 11008, 4096, true, true, false, 256);
+                EXPECT(up.kind == (m == 1 ? ws::W4A16Route::ROWS : ws::W4A16Route::MROWS) && up.partial_bytes == 0 &&
+                       up.rms_bytes == 256);
+                const auto down = ws::route_w4a16(m, 4096, 11008, false, false, true, 256);
+                EXPECT(down.kind == (m == 1 ? ws::W4A16Route::ROWS : ws::W4A16Route::MROWS_SPLIT));
+                EXPECT(down.partial_bytes == (m == 1 ? 0 : (size_t)3 * m * 4096 * 4) && down.rms_bytes == 0);
+                EXPECT(ws::fused_mlp_w4a16(m, 4096, 11008, 128) == 256 + ws::align256((size_t)m * 11008 * 2) + down.partial_bytes);
+            }
+            // (four rows of K = 11008 still fit one workgroup's LDS: the MFMA GEMV kernel in one launch, its products in
+            // scratch when the residual is the output buffer)
+            EXPECT(ws::route_w4a16(4, 4096, 11008, false, false, true, 256).kind == ws::W4A16Route::SKINNY &&
+                   ws::route_w4a16(4, 4096, 11008, false, false, true, 256).partial_bytes == (size_t)4 * 4096 * 2 &&
+                   ws::route_w4a16(4, 4096, 11008, false, false, false, 256).partial_bytes == 0);
+            // one family of kernels only: the MFMA GEMV kernel reads normalised activations and leaves gate | up in scratch
+            {
+                const auto r = ws::route_w4a16(8, 11008, 4096, true, true, false, 256, 2);
+                EXPECT(r.kind == ws::W4A16Route::SKINNY && r.via_scratch && r.partial_bytes == (size_t)8 * 22016 * 2 &&
+                       r.rms_bytes == (size_t)8 * 4096 * 2);
+                EXPECT(ws::route_w4a16(64, 4096, 4096, false, false, false, 256, 2).kind == ws::W4A16Route::NONE);
+                EXPECT(ws::route_w4a16(64, 4096, 4096, false, false, false, 256, 4).kind == ws::W4A16Route::NONE);
+                EXPECT(ws::route_w4a16(64, 4096, 4096, false, false, false, 256, 0).kind == ws::W4A16Route::TILE);
+            }
             for (int k = 128; k <= 16384; k += 128)
             {
                 const auto p = ws::plan_w4a16_skinny(4, k);

@@ -319,3 +319,67 @@ def test_rejects_bad_arguments(gpu):
     assert lib.nnf_w4a16_gemm(None, None, *args[1:], 4, 64, 256, 128, 8, None, 0) == -1  # null pointer
     assert lib.nnf_w4a16_gemm(None, args[0] + 2, *args[1:], 4, 64, 256, 128, 8, None, 0) == -1  # misaligned
     assert b"unsupported" in lib.nnf_status_string(-2)
+
+
+# ---- the fused parts on the kernels that serve a few rows ------------------------------------------------------------
+# auto: the library's choice (one row: the row-streaming GEMV; up to 32 rows: the row-streaming MFMA kernel, over ranges
+# of K with the reduction pass where K is long; otherwise the MFMA GEMV kernel with a pre-pass and an element-wise
+# kernel); gemv_rows / gemv_mfma: that family only, where it takes the shape.
+@pytest.mark.parametrize("variant", ["auto", "gemv_rows", "gemv_mfma"])
+@pytest.mark.parametrize("m,n,k", [(1, 4096, 4096), (1, 300, 1024), (1, 1000, 11008), (3, 304, 2048), (16, 4096, 4096),
+                                   (16, 520, 3584), (8, 1000, 11008), (24, 304, 4096), (24, 1000, 8192), (7, 100, 2176)])
+def test_fused_parts_with_few_rows(gpu, variant, m, n, k):
+    import torch
+
+    from nnfusion_amd import ops
+
+    print(f"case variant={variant} M={m} N={n} K={k}", flush=True)
+    a, wq, s = datagen.w4a16_case(21, m, 2 * n, k)  # 2n weight rows: the gate product uses all, the others the first n
+    bias = datagen.normal_f16(21, datagen.S_BIAS, (n,))
+    res = datagen.normal_f16(21, datagen.S_RES, (m, n))
+    gamma = datagen.normal_f16(21, datagen.S_GAMMA, (k,), 1.0, 0.1)
+    ta, tw, ts, tb, tr, tg = _t(gpu, a, wq, s, bias, res, gamma)
+    tw1, ts1 = tw[:n].contiguous(), ts[:n].contiguous()
+    kw = {} if variant == "auto" else {"variant": variant}
+    ws = _big_ws(gpu)
+
+    def run(w, sc, **fused):
+        try:
+            return ops.w4a16_gemm_fused(ta, w, sc, workspace=ws, **fused, **kw)
+        except ops.NnfError as e:
+            assert e.status == -2 and variant != "auto"  # this family does not take the shape
+            return None
+
+    d = oracle.w4a16_gemm(a, wq[:n], s[:n])  # fp16 tensor of the unfused Dot
+    ref_b = oracle.add_f16(d, np.broadcast_to(bias, (m, n)).copy())
+    y = run(tw1, ts1, bias=tb)
+    if y is None:
+        pytest.skip("variant does not serve this shape")
+    _check(y.cpu().numpy(), ref_b)
+    _check(run(tw1, ts1, residual=tr).cpu().numpy(), oracle.add_f16(d, res))
+    _check(run(tw1, ts1, bias=tb, residual=tr).cpu().numpy(), oracle.add_f16(ref_b, res))
+    # the residual in place: the output buffer holds it
+    out = tr.clone()
+    y_in_place = ops.w4a16_gemm_fused(ta, tw1, ts1, bias=tb, residual=out, out=out, workspace=ws, **kw)
+    _check(y_in_place.cpu().numpy(), oracle.add_f16(ref_b, res))
+    # RMSNorm prologue alone and with everything behind it
+    xn = oracle.rmsnorm_f16(a, gamma, 1e-6)
+    dn32 = oracle.w4a16_gemm(xn, wq[:n], s[:n], f32_out=True)
+    _check(run(tw1, ts1, rms_gamma=tg, rms_eps=1e-6).cpu().numpy(), dn32)
+    dn = oracle.w4a16_gemm(xn, wq[:n], s[:n])
+    ref_nbr = oracle.add_f16(oracle.add_f16(dn, np.broadcast_to(bias, (m, n)).copy()), res)
+    _check(run(tw1, ts1, rms_gamma=tg, rms_eps=1e-6, bias=tb, residual=tr).cpu().numpy(), ref_nbr)
+    # SiLU-gate, without and with the prologue
+    for x, fused in ((a, {}), (xn, {"rms_gamma": tg, "rms_eps": 1e-6})):
+        gu = oracle.w4a16_gemm(x, wq, s)
+        g, u = np.ascontiguousarray(gu[:, :n]), np.ascontiguousarray(gu[:, n:])
+        ref = oracle.silu_mul_f16(g, u)
+        yg = run(tw, ts, act=1, **fused).cpu().numpy()
+        assert yg.shape == (m, n)
+        delta = TOL * _rms(gu)
+        g32, u32 = g.astype(np.float32), u.astype(np.float32)
+        silu = g32 / (1.0 + np.exp(-g32))
+        bound = delta * (1.1 * np.abs(u32) + np.abs(silu)) + np.abs(ref.astype(np.float32)) * 2.0 ** -10 + 1e-6
+        err = np.abs(yg.astype(np.float32) - ref.astype(np.float32))
+        assert np.all(err <= bound), float((err - bound).max())
+    torch.cuda.synchronize()
