@@ -26,7 +26,6 @@ def lib():
             "oracle_f16_to_f32": (None, [_vp, _vp, _sz]),
             "oracle_f32_to_f16": (None, [_vp, _vp, _sz]),
             "oracle_dequantize_w4": (None, [_vp, _vp, _i, _i, _i, _i, _vp]),
-            "oracle_dequantize_i8": (None, [_vp, _vp, _i, _i, _vp]),
             "oracle_dot_f32": (None, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i]),
             "oracle_dot_general": (None, [_vp, _vp, _i, _vp, _vp, _i, _i, _vp]),
             "oracle_gemm_nt_f64": (None, [_vp, _vp, _vp, _i, _i, _i]),
@@ -97,14 +96,6 @@ def dequantize_w4(wq, scales, group=128, zp=8):
     n, k = wq.shape[0], wq.shape[1] * 2
     out = np.empty((n, k), np.float32)
     lib().oracle_dequantize_w4(_p(wq), _p(s), n, k, group, zp, _p(out))
-    return out
-
-
-def dequantize_i8(w, scale):
-    w = _c(w, np.int8)
-    scale = _c(scale, np.float32)
-    out = np.empty(w.shape, np.float32)
-    lib().oracle_dequantize_i8(_p(w), _p(scale), w.shape[0], w.shape[1], _p(out))
     return out
 
 

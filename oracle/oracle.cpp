@@ -225,14 +225,6 @@ void oracle_dequantize_w4(const uint8_t* wq, const uint16_t* scales, int N, int 
         }
 }
 
-// Per-output-channel int8 weights (offset 0): out[n,k] = REAL(w[n,k] - 0) * scale[n].
-void oracle_dequantize_i8(const int8_t* w, const float* scale, int N, int K, float* out)
-{
-    for (int n = 0; n < N; ++n)
-        for (int k = 0; k < K; ++k)
-            out[(size_t)n * K + k] = static_cast<float>((int)w[(size_t)n * K + k] - 0) * scale[n];
-}
-
 // The 2-D Dot as cpu::DotMlas hands it to MlasGemm: C[M,N] = op(A) . op(B), row-major,
 // op(A) is [M,K] (stored [K,M] with lda = M when transA), op(B) is [K,N] (stored [N,K] with
 // ldb = K when transB), alpha 1, beta 0.
