@@ -142,9 +142,12 @@ enum nnf_activation
     NNF_ACT_SILU_GATE = 1
 };
 
-/* Same GEMM with prologue / epilogue in one call (the epilogues run inside the GEMM kernel or its
- * reduction pass; RMSNorm writes the normalised activations to `workspace` first, rounded to fp16 as
- * the unfused graph would hold them; M <= 16 runs the GEMV kernel plus one element-wise kernel):
+/* Same GEMM with prologue / epilogue in one call.  They run inside the kernel that serves the shape: the
+ * row-streaming kernels (M = 1; M <= 32) and the tile GEMM multiply gamma in on the way in, rstd[m] (from a
+ * small pre-pass over A, fp32 [M] in `workspace`) and the epilogue at their end; a GEMV kernel over ranges
+ * of K leaves rstd and the epilogue to its reduction pass.  Only the MFMA GEMV kernel (M <= 16 with K not a
+ * multiple of 256) reads normalised activations written to `workspace` by a pre-pass and leaves its
+ * products to one element-wise kernel.
  *   rms_gamma != NULL : A is replaced by RMSNorm(A) = A * rsqrt(mean_k(A^2) + rms_eps) * gamma[k]
  *                       (rsqrt(x + eps) as in LayerNorm, cuda_gpu/cuda_langunit.cpp:618)
  *   bias      != NULL : fp16 [N], added to every row (MatMulAdd precedent,
@@ -214,9 +217,13 @@ int nnf_w8a8_gemm_variant(nnf_stream_t stream,
  *   RMSNorm -> QuantDot(gate|up) -> SiLU*mul -> QuantDot(down) -> Add(residual) ):
  *   out[M,H] = x + W_down . ( SiLU(W_gate . n) * (W_up . n) ),  n = RMSNorm(x, gamma, eps)
  * Wgu u8 [2I, H/2] (gate rows then up rows), Sgu fp16 [2I, H/group], Wd u8 [H, I/2],
- * Sd fp16 [H, I/group].  Intermediates in `workspace`: RMSNorm(x) fp16 [M, H], h fp16 [M, I], and
- * the partial sums of a split GEMM; SiLU, the gate product and the residual add touch no memory of
- * their own.
+ * Sd fp16 [H, I/group].  Intermediates in `workspace`: rstd fp32 [M] (RMSNorm(x) itself is never
+ * written: gamma is multiplied in inside the first product's kernel, rstd at its end), h fp16 [M, I],
+ * and the partial sums of a product that several workgroups share; SiLU, the gate product and the
+ * residual add touch no memory of their own.  (Shapes that only the MFMA GEMV kernel serves -- up to
+ * 16 rows with K not a multiple of 256 -- still go through RMSNorm(x) fp16 [M, H] and gate | up
+ * fp16 [M, 2I] in the workspace.)
+ * `out` may be `x` itself (the residual is then added in place); no other buffers may overlap.
  * The element-wise semantics follow the reference's ops (Sigmoid, Multiply, Add, Rsqrt:
  * cuda_gpu/cuda_kernelops.hpp:206-210,408,416,447-451); the reference has no RMSNorm op.
  * ------------------------------------------------------------------------------------------- */

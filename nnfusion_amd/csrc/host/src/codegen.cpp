@@ -581,6 +581,24 @@ namespace nnfusion
         }
         pass::graph::DefaultKernelSelector selector;
         NNFUSION_CHECK(selector.run_on_graph(graph));
+        // Only the quantized products (and Slice) have emitters for this device.  Element-wise operators of an imported
+        // model must have been absorbed by the fusion passes above; one that was not (a gate product with a second
+        // consumer, a bias added after the residual, a normalisation that feeds another operator ...) is named here,
+        // before any code is written.
+        {
+            std::string unserved;
+            for (auto& node : graph->get_ordered_ops())
+            {
+                if (node->is_parameter() || node->is_constant() || node->is_output())
+                    continue;
+                if (!(*node)["Kernel_Selection_Result"].is_valid())
+                    unserved += (unserved.empty() ? "" : ", ") + node->get_name() + " (" + node->get_op_type() + ")";
+            }
+            NNFUSION_CHECK(unserved.empty())
+                << "no " << get_device_str(ROCM_GPU) << " kernel for: " << unserved
+                << "; the quantized fusion passes did not absorb these operators, and only QuantDot, QuantDotW8A8, "
+                   "FusedQuantMLP and Slice have emitters";
+        }
         auto tu = visit_graph(graph);
         auto ctx = std::make_shared<InterpreterContext>();
         ctx->m_graph = graph;

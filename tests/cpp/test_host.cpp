@@ -680,6 +680,26 @@ int main(int argc, char** argv)
             results += n->is_output();
         }
         EXPECT(adds == 2 && consts == 2 && params == 1 && results == 1);
+        // ... but an Add that no quantized product absorbs has no kernel on this device: code generation stops before
+        // writing anything, naming every such node
+        threw = false;
+        try
+        {
+            ROCmEngine engine(tmp + "/unfused_project/");
+            engine.run_on_graph(g);
+        }
+        catch (const CheckError& e)
+        {
+            const std::string what = e.what();
+            threw = what.find("no ROCM_GPU kernel for: ") != std::string::npos && what.find("(Add)") != std::string::npos &&
+                    what.find("fusion passes did not absorb") != std::string::npos;
+            size_t named = 0;
+            for (size_t at = what.find("(Add)"); at != std::string::npos; at = what.find("(Add)", at + 1))
+                ++named;
+            EXPECT(named == 2);
+        }
+        EXPECT(threw);
+        EXPECT(!std::ifstream(tmp + "/unfused_project/nnfusion_rt.hip").good());
     });
 
     run_case("quant_fusion_passes", [] {

@@ -59,6 +59,25 @@ def test_mlp_full_size_rows(gpu):
     assert np.array_equal(again, out)
 
 
+@pytest.mark.parametrize("m,h,i", [(1, 1024, 2816), (4, 1024, 11008), (16, 2048, 5632), (24, 1024, 2816),
+                                   (16, 1024, 8704), (64, 512, 1408)])
+def test_mlp_output_may_be_the_input_buffer(gpu, m, h, i):
+    """out == x: the residual of the down projection is then the output buffer itself (the decode kernels add it in
+    place at their flush; the MFMA GEMV kernel goes through scratch memory; the tile GEMM reads each element before it
+    writes it).  Same results as with a separate output."""
+    import torch
+
+    from nnfusion_amd import ops
+
+    tens = _t(gpu, *datagen.mlp_case(2, m, h, i))
+    want = ops.fused_mlp_w4a16(*tens)
+    x = tens[0].clone()
+    got = ops.fused_mlp_w4a16(x, *tens[1:], out=x)
+    torch.cuda.synchronize()
+    assert got.data_ptr() == x.data_ptr()
+    assert torch.equal(got, want)
+
+
 def test_mlp_workspace_contract(gpu):
     import torch
 
