@@ -53,7 +53,8 @@ GEMM_NK = 8192
 GEMM_MS = (16, 128, 1024, 4096)       # configs[2]
 W8A8_MS = (1, 32, 512, 4096)          # configs[3]
 SMALL_BATCHES = (2, 4, 8, 16)         # the sweep's shapes with a few rows
-MLP_SHAPE = (256, 4096, 11008)        # configs[4]
+MLP_HI = (4096, 11008)                # configs[4]: hidden and intermediate size
+MLP_MS = (1, 16, 256)                 # ... at M = 256; the same block at decode sizes beside it
 
 # the kernel that dominates each configuration row (what a kernel trace of the row shows)
 DOMINANT_KERNEL = {
@@ -65,6 +66,9 @@ DOMINANT_KERNEL = {
     "w8a8_gemm_N8192_K8192.M32": "nnf::w8a8_mrows_kernel",
     "w8a8_gemm_N8192_K8192.M512": "nnf::w8a8_gemm_dl_kernel (128 x 128 tiles)",
     "w8a8_gemm_N8192_K8192.M4096": "nnf::w8a8_gemm_dl_kernel (256 x 256 tiles)",
+    "fused_mlp_M1_4096_11008": "rms_rstd_kernel + 2 x nnf::w4a16_gemv_rows_kernel (gate|up with SiLU, down with the residual)",
+    "fused_mlp_M16_4096_11008": "rms_rstd_kernel + nnf::w4a16_mrows_kernel (gate|up) + w4a16_mrows_any_kernel over 3 ranges of K + "
+                                "splitk_reduce_kernel (down)",
     "fused_mlp_M256_4096_11008": "rms_rstd_kernel + 2 x (nnf::gemm_sk::w4a16_gemm_sk_kernel<4, 2, ...> + fixup)",
 }
 
@@ -425,12 +429,14 @@ def parity_extra(env, oracle, parity):
             parity_fail(name, "fp16 outputs differ from the oracle's (the bar is bit-exact)")
         parity[name] = {"bit_exact_columns": int(len(cols8))}
     del tw8, tsch
-    m, h, i = MLP_SHAPE
-    x, gamma, wgu, sgu, wd, sd = datagen.mlp_case(0, m, h, i)
-    out = ops.fused_mlp_w4a16(*[env.dev_t(t) for t in (x, gamma, wgu, sgu, wd, sd)])
-    torch.cuda.synchronize()
-    ref = oracle.fused_mlp_w4a16(x[:8].copy(), gamma, wgu, sgu, wd, sd)
-    check_w4a16(np, parity, f"fused_mlp_M{m}_{h}_{i}.rows0-7", out.cpu().numpy()[:8], ref)
+    h, i = MLP_HI
+    for m in MLP_MS:
+        x, gamma, wgu, sgu, wd, sd = datagen.mlp_case(0, m, h, i)
+        out = ops.fused_mlp_w4a16(*[env.dev_t(t) for t in (x, gamma, wgu, sgu, wd, sd)])
+        torch.cuda.synchronize()
+        rows = min(m, 8)
+        ref = oracle.fused_mlp_w4a16(x[:rows].copy(), gamma, wgu, sgu, wd, sd)
+        check_w4a16(np, parity, f"fused_mlp_M{m}_{h}_{i}.rows0-{rows - 1}", out.cpu().numpy()[:rows], ref)
 
 
 # ---- probes ---------------------------------------------------------------------------------------------
@@ -562,14 +568,16 @@ def extra_rows(env):
         rows.append({"key": f"w8a8_gemm_N{n}_K{k}.M{m}", "group": f"w8a8_gemm_N{n}_K{k}", "M": m,
                      "bytes": w8a8_bytes(m, n, k), "ops": 2.0 * m * n * k, "int8": True, "weights": (tw8,),
                      "make": (lambda w, a8=a8, st=st, y=y, ws=ws: (lambda: ops.w8a8_gemm(a8, st, w, tsch, out=y, workspace=ws)))})
-    m, h, i = MLP_SHAPE
-    tens = [env.dev_t(t) for t in datagen.mlp_case(0, m, h, i)]
-    out = torch.empty((m, h), dtype=torch.float16, device=dev)
-    wsm = env.workspace(lib.nnf_fused_mlp_w4a16_workspace_bytes(m, h, i, GROUP))
-    x, gamma, wgu, sgu, wd, sd = tens
-    rows.append({"key": f"fused_mlp_M{m}_{h}_{i}", "group": None, "M": m, "bytes": mlp_bytes(m, h, i),
-                 "ops": 2.0 * m * (2 * i) * h + 2.0 * m * h * i, "int8": False, "weights": (wgu, sgu, wd, sd),
-                 "make": (lambda a, b, c, d: (lambda: ops.fused_mlp_w4a16(x, gamma, a, b, c, d, out=out, workspace=wsm)))})
+    h, i = MLP_HI
+    _, gamma, wgu, sgu, wd, sd = [env.dev_t(t) for t in datagen.mlp_case(0, 1, h, i)]  # the weights do not depend on M
+    for m in MLP_MS:
+        x = env.dev_t(datagen.mlp_case(0, m, h, i)[0])
+        out = torch.empty((m, h), dtype=torch.float16, device=dev)
+        wsm = env.workspace(lib.nnf_fused_mlp_w4a16_workspace_bytes(m, h, i, GROUP))
+        rows.append({"key": f"fused_mlp_M{m}_{h}_{i}", "group": None, "M": m, "bytes": mlp_bytes(m, h, i),
+                     "ops": 2.0 * m * (2 * i) * h + 2.0 * m * h * i, "int8": False, "weights": (wgu, sgu, wd, sd),
+                     "make": (lambda a, b, c, d, x=x, out=out, wsm=wsm:
+                              (lambda: ops.fused_mlp_w4a16(x, gamma, a, b, c, d, out=out, workspace=wsm)))})
     return rows
 
 

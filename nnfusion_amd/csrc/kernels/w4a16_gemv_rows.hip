@@ -72,11 +72,9 @@ namespace nnf
     // residual); 2 SiLU-gate (N outputs from 2 N weight rows: the workgroup walks the gate rows of its outputs, then
     // their up rows N further down; scales: two blocks in LDS) with the optional RMSNorm.
     template <int SEG, int D, int WAVES, int EPI>
-    __global__ __launch_bounds__(WAVES * 64) void w4a16_gemv_rows_kernel(const half_t* __restrict__ A,
-                                                                         const uint8_t* __restrict__ Wq,
-                                                                         const half_t* __restrict__ S,
-                                                                         half_t* __restrict__ Y, int N, int K,
-                                                                         int rows_q, int rows_r, int pack, GemvFusionArgs f)
+    __device__ __forceinline__ void gemv_rows_body(const half_t* __restrict__ A, const uint8_t* __restrict__ Wq,
+                                                   const half_t* __restrict__ S, half_t* __restrict__ Y, int N, int K,
+                                                   int rows_q, int rows_r, int pack, const GemvFusionArgs& f)
     {
         constexpr bool GATE = EPI == 2;
         extern __shared__ uintx4 lds[];
@@ -331,15 +329,18 @@ namespace nnf
                     }
                 });
             }
-            // the D - 1 rows still in flight, oldest first: the slots after the one the loop was left in
+            // the D - 1 rows still in flight, oldest first: the slots after the one the loop was left in.  Their row
+            // numbers are picked by a run-time slot: from the lanes of one register (indexed as an array they would
+            // be kept in scratch memory for the whole kernel)
+            int rows_by_slot = 0;
+#pragma unroll
+            for (int d = 0; d < D; ++d)
+                rows_by_slot = lane == d ? in_slot[d] : rows_by_slot;
             static_for<0, D - 1>([&](auto tc) {
                 constexpr int t = decltype(tc)::value;
                 int slot = exit_slot + 1 + t;
                 slot = slot >= D ? slot - D : slot;
-                int row = in_slot[0];
-#pragma unroll
-                for (int d = 1; d < D; ++d)
-                    row = slot == d ? in_slot[d] : row;
+                const int row = __builtin_amdgcn_readlane(rows_by_slot, slot);
                 __builtin_amdgcn_s_waitcnt(rows_vmcnt((D - 2 - t) * SEG));
                 read_slot(row, slot);
                 compute(row);
@@ -369,6 +370,29 @@ namespace nnf
         }
     }
 
+    // The plain kernel keeps its arguments within the sixteen dwords that are preloaded into scalar registers at launch
+    // (measured with FETCH_SIZE / WRITE_SIZE: with the fused kernel's longer argument list the same code wrote its
+    // outputs as 16-byte pieces, 8 x the bytes, and fetched 3 % more).
+    template <int SEG, int D, int WAVES>
+    __global__ __launch_bounds__(WAVES * 64) void w4a16_gemv_rows_kernel(const half_t* __restrict__ A,
+                                                                         const uint8_t* __restrict__ Wq,
+                                                                         const half_t* __restrict__ S,
+                                                                         half_t* __restrict__ Y, int N, int K,
+                                                                         int rows_q, int rows_r, int pack)
+    {
+        gemv_rows_body<SEG, D, WAVES, 0>(A, Wq, S, Y, N, K, rows_q, rows_r, pack, GemvFusionArgs{nullptr, nullptr, nullptr, nullptr});
+    }
+    template <int SEG, int D, int WAVES, int EPI>
+    __global__ __launch_bounds__(WAVES * 64) void w4a16_gemv_rows_fused_kernel(const half_t* __restrict__ A,
+                                                                               const uint8_t* __restrict__ Wq,
+                                                                               const half_t* __restrict__ S,
+                                                                               half_t* __restrict__ Y, int N, int K,
+                                                                               int rows_q, int rows_r, int pack, GemvFusionArgs f)
+    {
+        static_assert(EPI == 1 || EPI == 2, "the plain kernel is w4a16_gemv_rows_kernel");
+        gemv_rows_body<SEG, D, WAVES, EPI>(A, Wq, S, Y, N, K, rows_q, rows_r, pack, f);
+    }
+
     namespace
     {
         using workspace::RowsPlan;
@@ -382,17 +406,26 @@ namespace nnf
                                       (const half_t*)fusion.residual};
             if (lds_total > MAX_LDS_BYTES)
                 return hipErrorInvalidValue;
+            const void* kernel;
+            if constexpr (EPI == 0)
+                kernel = reinterpret_cast<const void*>(&w4a16_gemv_rows_kernel<SEG, D, WAVES>);
+            else
+                kernel = reinterpret_cast<const void*>(&w4a16_gemv_rows_fused_kernel<SEG, D, WAVES, EPI>);
             if (lds_total > 64 * 1024)
             {
                 static LdsGrant granted;
-                const hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(&w4a16_gemv_rows_kernel<SEG, D, WAVES, EPI>),
-                                                       granted, (int)MAX_LDS_BYTES);
+                const hipError_t e = allow_dynamic_lds(kernel, granted, (int)MAX_LDS_BYTES);
                 if (e != hipSuccess)
                     return e;
             }
-            hipLaunchKernelGGL((w4a16_gemv_rows_kernel<SEG, D, WAVES, EPI>), dim3(grid), dim3(WAVES * 64), lds_total, stream,
-                               (const half_t*)A, (const uint8_t*)Wq, (const half_t*)S, (half_t*)Y, N, K, N / grid, N % grid,
-                               zp | (p.kshift << 8), f);
+            if constexpr (EPI == 0)
+                hipLaunchKernelGGL((w4a16_gemv_rows_kernel<SEG, D, WAVES>), dim3(grid), dim3(WAVES * 64), lds_total, stream,
+                                   (const half_t*)A, (const uint8_t*)Wq, (const half_t*)S, (half_t*)Y, N, K, N / grid, N % grid,
+                                   zp | (p.kshift << 8));
+            else
+                hipLaunchKernelGGL((w4a16_gemv_rows_fused_kernel<SEG, D, WAVES, EPI>), dim3(grid), dim3(WAVES * 64), lds_total,
+                                   stream, (const half_t*)A, (const uint8_t*)Wq, (const half_t*)S, (half_t*)Y, N, K, N / grid,
+                                   N % grid, zp | (p.kshift << 8), f);
             return hipGetLastError();
         }
     } // namespace

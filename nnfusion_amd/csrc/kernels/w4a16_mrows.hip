@@ -89,6 +89,10 @@ namespace nnf
             const int im = idx >> 4;
             const int it = im / M, m = im - it * M;
             const int nn = min((t0 + it) * 16, N - 16) + n;
+            // (the last tile of an N that is not a multiple of 16 was moved back over columns that the tile before it
+            // owns: written once, so that a residual that is the output buffer itself is added once)
+            if (nn < (t0 + it) * 16)
+                continue;
             const size_t at = (size_t)m * N + nn;
             if (!FUSED)
                 Y[at] = (half_t)parked[idx];

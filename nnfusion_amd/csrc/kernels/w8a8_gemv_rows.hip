@@ -188,15 +188,18 @@ namespace nnf
                     }
                 });
             }
-            // the D - 1 rows still in flight, oldest first: the slots after the one the loop was left in
+            // the D - 1 rows still in flight, oldest first: the slots after the one the loop was left in.  Their row
+            // numbers are picked by a run-time slot: from the lanes of one register (indexed as an array they would
+            // be kept in scratch memory for the whole kernel)
+            int rows_by_slot = 0;
+#pragma unroll
+            for (int d = 0; d < D; ++d)
+                rows_by_slot = lane == d ? in_slot[d] : rows_by_slot;
             q8_static_for<0, D - 1>([&](auto tc) {
                 constexpr int t = decltype(tc)::value;
                 int slot = exit_slot + 1 + t;
                 slot = slot >= D ? slot - D : slot;
-                int row = in_slot[0];
-#pragma unroll
-                for (int d = 1; d < D; ++d)
-                    row = slot == d ? in_slot[d] : row;
+                const int row = __builtin_amdgcn_readlane(rows_by_slot, slot);
                 __builtin_amdgcn_s_waitcnt(q8_vmcnt((D - 2 - t) * SEG));
                 read_slot(slot);
                 compute(row);
