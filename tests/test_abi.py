@@ -45,6 +45,17 @@ def test_pure_host_queries_work_without_a_gpu():
     assert lib.nnf_w4a16_gemm_workspace_bytes(1, 4096, 4096, 128) == 0
     m, h, i = 256, 4096, 11008
     assert lib.nnf_fused_mlp_w4a16_workspace_bytes(m, h, i, 128) >= m * i * 2 + m * 4
+    # decode-size fused calls: rstd (fp32 [M]) is the only scratch of the RMSNorm prologue, the gate | up pair needs none;
+    # the MLP block adds its h tensor
+    assert lib.nnf_w4a16_gemm_fused_workspace_bytes(1, 11008, 4096, 128, 1) == 256
+    assert lib.nnf_w4a16_gemm_fused_workspace_bytes(16, 11008, 4096, 128, 1) == 256
+    assert lib.nnf_w4a16_gemm_fused_workspace_bytes(1, 4096, 4096, 128, 0) == 256
+    assert lib.nnf_fused_mlp_w4a16_workspace_bytes(1, 4096, 11008, 128) == 256 + 11008 * 2
+    assert lib.nnf_fused_mlp_w4a16_workspace_bytes(256, 4096, 11008, 128) < 256 * 4096 * 2 + 256 * 11008 * 2 + (128 << 20)
+    # variant / plan queries are host arithmetic too
+    assert lib.nnf_w4a16_variant_supported(1, 4096, 4096, 128, 4) == 1 and lib.nnf_w4a16_variant_supported(64, 4096, 4096, 128, 4) == 0
+    assert lib.nnf_w8a8_variant_supported(1, 4096, 4096, 3) == 1 and lib.nnf_w8a8_variant_supported(64, 4096, 4096, 1) == 0
+    assert lib.nnf_w4a16_gemm_variant_workspace_bytes(4096, 8192, 8192, 128, 3, None) == 0
     # argument checks come before any device access
     assert lib.nnf_w4a16_gemm(None, None, None, None, None, 1, 1, 128, 128, 8, None, 0) == -1
     assert lib.nnf_w8a8_gemm_acc(None, None, None, None, 1, 1, 128, None, 0) == -1

@@ -256,8 +256,10 @@ def test_fused_silu_gate(gpu, plan):
 @pytest.mark.parametrize("m,n,k", [(1, 320, 1024), (5, 320, 1024), (16, 320, 1024), (2, 520, 4096), (24, 320, 2048), (32, 1000, 4096),
                                    (16, 136, 11008), (24, 264, 8192), (7, 320, 3584)])
 def test_fused_small_m_goes_through_the_gemv_kernel(gpu, m, n, k):
-    """Decode shapes with a prologue / epilogue: RMSNorm pre-pass, a GEMV kernel (M = 1; 2 .. 32 rows in one launch or
-    over ranges of K), an element-wise epilogue or the reduction pass's."""
+    """Decode shapes with a prologue / epilogue: the GEMV kernels (M = 1; 2 .. 32 rows in one launch or over ranges of
+    K) multiply the RMSNorm weight in themselves and apply rstd, bias, residual and the gate at their flush (over ranges
+    of K: in the reduction pass).  The workspace is the one the query asks for: rstd and partial sums, no M x K
+    activations and no M x 2N products."""
     import torch
 
     from nnfusion_amd import ops
