@@ -29,6 +29,8 @@ def lib():
             "oracle_dot_f32": (None, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i]),
             "oracle_dot_general": (None, [_vp, _vp, _i, _vp, _vp, _i, _i, _vp]),
             "oracle_gemm_nt_f64": (None, [_vp, _vp, _vp, _i, _i, _i]),
+            "oracle_dequantize_wn": (None, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
+            "oracle_wna16_gemm": (None, [_vp, _vp, _vp, _vp, _vp] + [_i] * 8),
             "oracle_w4a16_gemm_f32": (None, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i]),
             "oracle_w4a16_gemm": (None, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i]),
             "oracle_w8a8_acc": (None, [_vp, _vp, _vp, _i, _i, _i, _i]),
@@ -146,6 +148,36 @@ def w4a16_gemm(a, wq, scales, group=128, zp=8, threads=0, f32_out=False):
     out = np.empty((m, n), np.uint16)
     lib().oracle_w4a16_gemm(_p(a16), _p(wq), _p(s), _p(out), m, n, k, group, zp, threads)
     return out.view(np.float16)
+
+
+def dequantize_wn(wq, scales, bits, group, zp=8, zero_points=None):
+    """fp32 [N, K] = (q - zero point) * scale for 4- or 8-bit weights, any group size that divides K, a scalar zero point
+    or one per (row, group) (u8; bits = 4: packed two per byte along the groups, low nibble = even group)."""
+    wq = _c(wq, np.uint8)
+    s = _c(scales.view(np.uint16), np.uint16)
+    n = wq.shape[0]
+    k = wq.shape[1] * 8 // bits
+    assert bits in (4, 8) and k % group == 0 and s.shape == (n, k // group)
+    z = None if zero_points is None else _c(zero_points, np.uint8)
+    assert z is None or z.shape == (n, (k // group * bits + 7) // 8)
+    out = np.empty((n, k), np.float32)
+    lib().oracle_dequantize_wn(_p(wq), _p(s), None if z is None else _p(z), n, k, bits, group, zp, _p(out))
+    return out
+
+
+def wna16_gemm(a, wq, scales, bits, group, zp=8, zero_points=None, threads=0, f32_out=False):
+    """Y = A . dequantize_wn(W)^T, accumulated in fp32; fp32, or rounded to fp16 as the output tensor type asks."""
+    a16 = _c(a.view(np.uint16), np.uint16)
+    wq = _c(wq, np.uint8)
+    s = _c(scales.view(np.uint16), np.uint16)
+    m, k = a16.shape
+    n = wq.shape[0]
+    assert wq.shape[1] * 8 // bits == k and k % group == 0
+    z = None if zero_points is None else _c(zero_points, np.uint8)
+    out = np.empty((m, n), np.float32 if f32_out else np.uint16)
+    lib().oracle_wna16_gemm(_p(a16), _p(wq), _p(s), None if z is None else _p(z), _p(out), m, n, k, bits, group, zp,
+                            0 if f32_out else 1, threads)
+    return out if f32_out else out.view(np.float16)
 
 
 def w8a8_acc(a, w, threads=0):

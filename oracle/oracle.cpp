@@ -7,7 +7,7 @@
 // library (libnnf_hip_kernels.so) never links or calls it.
 //
 // Reference sources each function follows (paths relative to the nnfusion tree):
-//   oracle_dequantize_w4 / _i8   src/nnfusion/core/kernels/cpu/reference/kernels.cpp:601-623
+//   oracle_dequantize_w4 / _wn   src/nnfusion/core/kernels/cpu/reference/kernels.cpp:601-623
 //                                (integer subtract of the offset, cast to REAL, multiply by scale)
 //   oracle_dot_f32               src/nnfusion/core/kernels/cpu/mlas/dot.cpp:25-102
 //                                (M/N/K, lda = transA ? M : K, ldb = transB ? K : N, ldc = N,
@@ -225,6 +225,46 @@ void oracle_dequantize_w4(const uint8_t* wq, const uint16_t* scales, int N, int 
         }
 }
 
+// The same dequantisation with the block parameters of the reference's signature left open
+// (cpu_reference_dequantize, kernels.cpp:601-623: per-block offset and scale, the integer subtract done before
+// the cast): `bits` 4 (two weights per byte as above) or 8 (one byte per weight, wq [N, K]); `group` any divisor
+// of K; zero points either the scalar `zp` (zps == nullptr) or one per (row, group): u8, row stride
+// ceil(G * bits / 8) bytes, bits = 4 packed two per byte along the groups, low nibble = even group -- the packing of
+// ONNX com.microsoft::MatMulNBits' zero_points input.
+void oracle_dequantize_wn(const uint8_t* wq, const uint16_t* scales, const uint8_t* zps, int N, int K, int bits,
+                          int group, int zp, float* out)
+{
+    const int G = K / group;
+    const size_t w_stride = (size_t)K * bits / 8;
+    const size_t z_stride = ((size_t)G * bits + 7) / 8;
+#pragma omp parallel for schedule(static)
+    for (int n = 0; n < N; ++n)
+        for (int k = 0; k < K; ++k)
+        {
+            int q;
+            if (bits == 4)
+            {
+                const uint8_t byte = wq[(size_t)n * w_stride + k / 2];
+                q = (k & 1) ? (byte >> 4) : (byte & 0xF);
+            }
+            else
+                q = wq[(size_t)n * w_stride + k];
+            const int g = k / group;
+            int z = zp;
+            if (zps)
+            {
+                if (bits == 4)
+                {
+                    const uint8_t byte = zps[(size_t)n * z_stride + g / 2];
+                    z = (g & 1) ? (byte >> 4) : (byte & 0xF);
+                }
+                else
+                    z = zps[(size_t)n * z_stride + g];
+            }
+            out[(size_t)n * K + k] = static_cast<float>(q - z) * h2f(scales[(size_t)n * G + g]);
+        }
+}
+
 // The 2-D Dot as cpu::DotMlas hands it to MlasGemm: C[M,N] = op(A) . op(B), row-major,
 // op(A) is [M,K] (stored [K,M] with lda = M when transA), op(B) is [K,N] (stored [N,K] with
 // ldb = K when transB), alpha 1, beta 0.
@@ -323,6 +363,23 @@ void oracle_w4a16_gemm(const uint16_t* A, const uint8_t* wq, const uint16_t* sca
     std::vector<float> y((size_t)M * N);
     oracle_w4a16_gemm_f32(A, wq, scales, y.data(), M, N, K, group, zp, nthreads);
     oracle_f32_to_f16(y.data(), Y, (size_t)M * N);
+}
+
+// Y = A . dequantize_wn(W)^T, fp32-accumulated, fp32 result (f16_out == 0) or rounded to fp16 (Y then holds uint16).
+void oracle_wna16_gemm(const uint16_t* A, const uint8_t* wq, const uint16_t* scales, const uint8_t* zps, void* Y, int M,
+                       int N, int K, int bits, int group, int zp, int f16_out, int nthreads)
+{
+    std::vector<float> a((size_t)M * K), w((size_t)N * K), y;
+    oracle_f16_to_f32(A, a.data(), (size_t)M * K);
+    oracle_dequantize_wn(wq, scales, zps, N, K, bits, group, zp, w.data());
+    if (!f16_out)
+    {
+        gemm_nt(a.data(), w.data(), static_cast<float*>(Y), M, N, K, nthreads);
+        return;
+    }
+    y.resize((size_t)M * N);
+    gemm_nt(a.data(), w.data(), y.data(), M, N, K, nthreads);
+    oracle_f32_to_f16(y.data(), static_cast<uint16_t*>(Y), (size_t)M * N);
 }
 
 // Raw int32 accumulators of the W8A8 product: acc[m,n] = sum_k A[m,k] * W[n,k].

@@ -157,3 +157,106 @@ def test_fused_mlp_is_the_composition_of_its_nodes():
     np.testing.assert_array_equal(hbuf.view(np.uint16), hh.view(np.uint16))
     d = oracle.w4a16_gemm(hh, wd, sd)
     np.testing.assert_array_equal(out.view(np.uint16), oracle.add_f16(d, x).view(np.uint16))
+
+
+# ---- the general form: 4 / 8 bits, groups of 32 / 64 / 128, scalar or per-(row, group) zero points ---------------------
+def _rand_quant_case(seed, n, k, bits, group, zp_tensor):
+    rng = np.random.default_rng(seed)
+    wq = rng.integers(0, 256, (n, k * bits // 8), dtype=np.uint8)
+    s = (rng.uniform(0.005, 0.02, (n, k // group))).astype(np.float16)
+    g = k // group
+    zps = rng.integers(0, 256, (n, (g * bits + 7) // 8), dtype=np.uint8) if zp_tensor else None
+    return wq, s, zps
+
+
+def _python_dequant_wn(wq, s, zps, bits, group, zp):
+    """Element by element, from the definition: q and the zero point are unpacked with shifts, subtracted as integers,
+    cast, multiplied by the scale of the block (cpu_reference_dequantize)."""
+    n = wq.shape[0]
+    k = wq.shape[1] * 8 // bits
+    out = np.zeros((n, k), np.float32)
+    for i in range(n):
+        for kk in range(k):
+            if bits == 4:
+                q = (int(wq[i, kk // 2]) >> (4 * (kk % 2))) & 0xF
+            else:
+                q = int(wq[i, kk])
+            g = kk // group
+            if zps is None:
+                z = zp
+            elif bits == 4:
+                z = (int(zps[i, g // 2]) >> (4 * (g % 2))) & 0xF
+            else:
+                z = int(zps[i, g])
+            out[i, kk] = np.float32(q - z) * np.float32(s[i, g])
+    return out
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("group", [32, 64, 128])
+@pytest.mark.parametrize("zp_tensor", [False, True])
+def test_dequantize_wn_brute_force(bits, group, zp_tensor):
+    wq, s, zps = _rand_quant_case(bits * 1000 + group + zp_tensor, 5, 384, bits, group, zp_tensor)
+    zp = 8 if bits == 4 else 128
+    out = oracle.dequantize_wn(wq, s, bits, group, zp=zp, zero_points=zps)
+    np.testing.assert_array_equal(out, _python_dequant_wn(wq, s, zps, bits, group, zp))
+
+
+def test_dequantize_wn_reduces_to_the_w4_g128_form():
+    _, wq, s = datagen.w4a16_case(12, 1, 9, 512)
+    np.testing.assert_array_equal(oracle.dequantize_wn(wq, s, 4, 128, zp=8), oracle.dequantize_w4(wq, s))
+    # ... and a zero-point tensor that holds the scalar everywhere changes nothing
+    zps = np.full((9, 2), 0x88, np.uint8)
+    np.testing.assert_array_equal(oracle.dequantize_wn(wq, s, 4, 128, zero_points=zps), oracle.dequantize_w4(wq, s))
+
+
+def test_dequantize_wn_element_and_zero_point_order():
+    """One weight / one zero point set at a time: pins byte and nibble order of both tensors and the block a scale and
+    a zero point belong to."""
+    n, k = 3, 256
+    for bits, group in ((4, 32), (4, 64), (8, 32), (8, 128)):
+        g = k // group
+        s = (np.arange(n * g, dtype=np.float32).reshape(n, g) + 1).astype(np.float16)  # every block its own scale
+        zero = np.zeros((n, k * bits // 8), np.uint8)
+        zps0 = np.zeros((n, (g * bits + 7) // 8), np.uint8)
+        for (row, kk) in ((0, 0), (1, 1), (2, 33), (1, 255), (0, 130)):
+            wq = zero.copy()
+            if bits == 4:
+                wq[row, kk // 2] = 5 << (4 * (kk % 2))
+            else:
+                wq[row, kk] = 5
+            out = oracle.dequantize_wn(wq, s, bits, group, zp=0, zero_points=zps0)
+            want = np.zeros((n, k), np.float32)
+            want[row, kk] = 5.0 * float(s[row, kk // group])
+            np.testing.assert_array_equal(out, want)
+        for (row, gg) in ((0, 0), (1, 1), (2, g - 1)):
+            zps = zps0.copy()
+            if bits == 4:
+                zps[row, gg // 2] = 3 << (4 * (gg % 2))
+            else:
+                zps[row, gg] = 3
+            out = oracle.dequantize_wn(zero, s, bits, group, zp=0, zero_points=zps)
+            want = np.zeros((n, k), np.float32)
+            want[row, gg * group:(gg + 1) * group] = -3.0 * float(s[row, gg])
+            np.testing.assert_array_equal(out, want)
+
+
+@pytest.mark.parametrize("bits,group,zp_tensor", [(4, 32, True), (4, 64, False), (8, 128, True), (8, 32, False), (4, 128, True)])
+def test_wna16_gemm_against_fp64_and_one_hot(bits, group, zp_tensor):
+    m, n, k = 7, 33, 512
+    wq, s, zps = _rand_quant_case(77 + bits + group, n, k, bits, group, zp_tensor)
+    zp = 8 if bits == 4 else 128
+    a = datagen.normal_f16(5, datagen.S_ACT, (m, k))
+    wd = _python_dequant_wn(wq, s, zps, bits, group, zp) if n * k <= 20000 else oracle.dequantize_wn(wq, s, bits, group, zp, zps)
+    ref64 = a.astype(np.float64) @ wd.astype(np.float64).T
+    y32 = oracle.wna16_gemm(a, wq, s, bits, group, zp=zp, zero_points=zps, f32_out=True)
+    bound = 4 * k * 2.0 ** -24 * (np.abs(a.astype(np.float64)) @ np.abs(wd.astype(np.float64)).T) + 1e-30
+    assert np.all(np.abs(y32 - ref64) <= bound)
+    y16 = oracle.wna16_gemm(a, wq, s, bits, group, zp=zp, zero_points=zps)
+    np.testing.assert_array_equal(y16.view(np.uint16), oracle.f32_to_f16(y32).view(np.uint16))
+    # A = e_k picks column k of the dequantised weights, rounded to fp16
+    for kk in (0, 1, 31, 32, 63, 64, 127, 128, 511):
+        e = np.zeros((1, k), np.float16)
+        e[0, kk] = 1.0
+        y = oracle.wna16_gemm(e, wq, s, bits, group, zp=zp, zero_points=zps)
+        np.testing.assert_array_equal(y[0], wd[:, kk].astype(np.float16))
