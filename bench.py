@@ -53,6 +53,10 @@ GEMM_NK = 8192
 GEMM_MS = (16, 128, 1024, 4096)       # configs[2]
 W8A8_MS = (1, 32, 512, 4096)          # configs[3]
 SMALL_BATCHES = (2, 4, 8, 16)         # the sweep's shapes with a few rows
+# the fp16 x int-N product with other block parameters (bits, group, zero point per (row, group)?) than the benchmark's,
+# on the two plain kernels that serve them, at N = K = GEMM_NK
+WNA16_CASES = ((8, 128, False), (4, 64, True))
+WNA16_MS = (1, 4096)
 MLP_HI = (4096, 11008)                # configs[4]: hidden and intermediate size
 MLP_MS = (1, 16, 256)                 # ... at M = 256; the same block at decode sizes beside it
 
@@ -66,6 +70,10 @@ DOMINANT_KERNEL = {
     "w8a8_gemm_N8192_K8192.M32": "nnf::w8a8_mrows_kernel",
     "w8a8_gemm_N8192_K8192.M512": "nnf::w8a8_gemm_dl_kernel (128 x 128 tiles)",
     "w8a8_gemm_N8192_K8192.M4096": "nnf::w8a8_gemm_dl_kernel (256 x 256 tiles)",
+    "wna16_b8_g128_zp_scalar_N8192_K8192.M1": "nnf::wna16_gemv_kernel<8>",
+    "wna16_b8_g128_zp_scalar_N8192_K8192.M4096": "nnf::wna16_tile_kernel<8>",
+    "wna16_b4_g64_zp_tensor_N8192_K8192.M1": "nnf::wna16_gemv_kernel<4>",
+    "wna16_b4_g64_zp_tensor_N8192_K8192.M4096": "nnf::wna16_tile_kernel<4>",
     "fused_mlp_M1_4096_11008": "rms_rstd_kernel + 2 x nnf::w4a16_gemv_rows_kernel (gate|up with SiLU, down with the residual)",
     "fused_mlp_M16_4096_11008": "rms_rstd_kernel + nnf::w4a16_mrows_kernel (gate|up) + w4a16_mrows_any_kernel over 3 ranges of K + "
                                 "splitk_reduce_kernel (down)",
@@ -73,9 +81,19 @@ DOMINANT_KERNEL = {
 }
 
 
+def wna16_key(bits, group, zp_tensor, n, k, m):
+    return f"wna16_b{bits}_g{group}_{'zp_tensor' if zp_tensor else 'zp_scalar'}_N{n}_K{k}.M{m}"
+
+
 def w4a16_bytes(m, n, k):
     """Algorithmic bytes: int4 weights + fp16 group scales + fp16 activations + fp16 output."""
     return n * k // 2 + n * (k // GROUP) * 2 + m * k * 2 + m * n * 2
+
+
+def wna16_bytes(m, n, k, bits, group, zp_tensor):
+    """Weights of `bits` bits + fp16 scales (+ one zero point of `bits` bits) per group + fp16 activations and output."""
+    g = k // group
+    return n * k * bits // 8 + n * g * 2 + (n * ((g * bits + 7) // 8) if zp_tensor else 0) + m * k * 2 + m * n * 2
 
 
 def w8a8_bytes(m, n, k):
@@ -429,6 +447,17 @@ def parity_extra(env, oracle, parity):
             parity_fail(name, "fp16 outputs differ from the oracle's (the bar is bit-exact)")
         parity[name] = {"bit_exact_columns": int(len(cols8))}
     del tw8, tsch
+    for bits, group, zpt in WNA16_CASES:
+        _, wq, s, z = datagen.wna16_case(0, 1, n, k, bits, group, zpt)
+        tw, tsc, tz = env.dev_t(wq), env.dev_t(s), (env.dev_t(z) if zpt else None)
+        for m in WNA16_MS:
+            a = datagen.normal_f16(0, datagen.S_ACT, (m, k))
+            y = ops.wna16_gemm(env.dev_t(a), tw, tsc, bits=bits, group=group, zp=1 << (bits - 1), zero_points=tz)
+            torch.cuda.synchronize()
+            ref = oracle.wna16_gemm(a, wq[cols], s[cols], bits, group, zp=1 << (bits - 1),
+                                    zero_points=None if z is None else z[cols], f32_out=True)
+            check_w4a16(np, parity, wna16_key(bits, group, zpt, n, k, m), y.cpu().numpy()[:, cols], ref)
+        del tw, tsc, tz
     h, i = MLP_HI
     for m in MLP_MS:
         x, gamma, wgu, sgu, wd, sd = datagen.mlp_case(0, m, h, i)
@@ -568,6 +597,18 @@ def extra_rows(env):
         rows.append({"key": f"w8a8_gemm_N{n}_K{k}.M{m}", "group": f"w8a8_gemm_N{n}_K{k}", "M": m,
                      "bytes": w8a8_bytes(m, n, k), "ops": 2.0 * m * n * k, "int8": True, "weights": (tw8,),
                      "make": (lambda w, a8=a8, st=st, y=y, ws=ws: (lambda: ops.w8a8_gemm(a8, st, w, tsch, out=y, workspace=ws)))})
+    for bits, group, zpt in WNA16_CASES:
+        _, wq, s, z = datagen.wna16_case(0, 1, n, k, bits, group, zpt)
+        tw, tsc, tz = env.dev_t(wq), env.dev_t(s), (env.dev_t(z) if zpt else None)
+        for m in WNA16_MS:
+            a = env.dev_t(datagen.normal_f16(0, datagen.S_ACT, (m, k)))
+            y = torch.empty((m, n), dtype=torch.float16, device=dev)
+            rows.append({"key": wna16_key(bits, group, zpt, n, k, m), "group": None, "M": m,
+                         "bytes": wna16_bytes(m, n, k, bits, group, zpt), "ops": 2.0 * m * n * k, "int8": False,
+                         "weights": (tw, tsc) + ((tz,) if zpt else ()),
+                         "make": (lambda w, sc, zz=None, a=a, y=y, bits=bits, group=group:
+                                  (lambda: ops.wna16_gemm(a, w, sc, bits=bits, group=group, zp=1 << (bits - 1), zero_points=zz,
+                                                          out=y)))})
     h, i = MLP_HI
     _, gamma, wgu, sgu, wd, sd = [env.dev_t(t) for t in datagen.mlp_case(0, 1, h, i)]  # the weights do not depend on M
     for m in MLP_MS:

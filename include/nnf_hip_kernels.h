@@ -132,6 +132,34 @@ int nnf_w4a16_gemm_variant(nnf_stream_t stream,
                            int M, int N, int K, int group, int zp, int variant, const nnf_plan* plan,
                            void* workspace, size_t workspace_bytes);
 
+/* The same product with every block parameter the reference's dequantisation takes: its Dequantize scales and
+ * offsets are tensors over blocks of any shape (core/kernels/cpu/reference/kernels.cpp:601-623: integer subtract of
+ * the offset, cast, multiply by the scale), and the ONNX operator that carries such weights (MatMulNBits) stores
+ * `bits`, `block_size` and an optional zero-point tensor.
+ *   w[n,k] = (q[n,k] - z[n, k / group]) * scales[n, k / group]
+ *   bits = 4 : Wq u8 [N, K/2], weight k in the low (k even) or high (k odd) nibble of byte k/2
+ *   bits = 8 : Wq u8 [N, K]
+ *   zero_points == NULL : z = zero_point everywhere (0 .. 2^bits - 1)
+ *   zero_points != NULL : u8 [N, ceil(K/group * bits / 8)], one per (row, group); 4-bit ones packed two to a byte along
+ *                         the groups of a row, even group in the low nibble
+ * bits 4, group 128 and no zero-point tensor is nnf_w4a16_gemm itself (same kernels, same workspace); every other
+ * combination (group 32 / 64 / 128, K a multiple of group) runs on two plain kernels: a wavefront per weight row for
+ * M <= 16, 64 x 64 MFMA tiles above. */
+typedef struct nnf_quant
+{
+    int bits;                /* 4 or 8 */
+    int group;               /* 32, 64 or 128 */
+    int zero_point;          /* used when zero_points is NULL */
+    const void* zero_points; /* device pointer or NULL */
+} nnf_quant;
+/* 1 when nnf_wna16_gemm serves the shape with these parameters (zero_points is not read), else 0. */
+int nnf_wna16_supported(int M, int N, int K, const nnf_quant* q);
+size_t nnf_wna16_gemm_workspace_bytes(int M, int N, int K, const nnf_quant* q);
+int nnf_wna16_gemm(nnf_stream_t stream,
+                   const void* A, const void* Wq, const void* scales, void* Y,
+                   int M, int N, int K, const nnf_quant* q,
+                   void* workspace, size_t workspace_bytes);
+
 /* Epilogue / prologue selectors for nnf_w4a16_gemm_fused. */
 enum nnf_activation
 {

@@ -487,38 +487,57 @@ namespace nnfusion
                 }
                 else if (n.op_type == "MatMulNBits")
                 {
-                    // A [.., K]; B u8 [N, K/block, block/2] (two 4-bit values per byte, low nibble first);
-                    // scales [N * K/block]; optional zero_points (packed 4-bit, one per block)
+                    // A [.., K]; B u8 [N, K/block, block*bits/8] (4 bits: two values per byte, low nibble first);
+                    // scales [N * K/block]; optional zero_points u8 [N, ceil(K/block * bits / 8)], one per block
+                    // (4-bit ones two per byte along the blocks of a row, even block in the low nibble); without them the
+                    // zero point is 2^(bits-1)
                     const int64_t K = n.get_int("K", 0), N = n.get_int("N", 0);
                     const int64_t bits = n.get_int("bits", 4), block = n.get_int("block_size", 0);
-                    NNFUSION_CHECK(bits == 4 && block == 128 && K > 0 && N > 0 && K % block == 0)
-                        << "onnx: MatMulNBits " << n.name << ": only bits = 4, block_size = 128 (K a multiple of it) is supported";
+                    NNFUSION_CHECK((bits == 4 || bits == 8) && (block == 32 || block == 64 || block == 128) && K > 0 && N > 0 &&
+                                   K % block == 0)
+                        << "onnx: MatMulNBits " << n.name
+                        << ": bits = 4 or 8 and block_size = 32, 64 or 128 (K a multiple of it) are supported";
                     NNFUSION_CHECK(!has_input(n, 4) && !has_input(n, 5)) << "onnx: MatMulNBits with g_idx or bias is not supported";
                     auto wi = init.find(n.inputs.at(1));
                     auto si = init.find(n.inputs.at(2));
                     NNFUSION_CHECK(wi != init.end() && si != init.end()) << "onnx: MatMulNBits weights and scales must be initializers";
                     const Tensor& wt = *wi->second;
-                    NNFUSION_CHECK(wt.data_type == UINT8 && wt.bytes.size() == (size_t)(N * K / 2))
-                        << "onnx: MatMulNBits B must be uint8 with N*K/2 bytes";
-                    int zp = 8;
+                    NNFUSION_CHECK(wt.data_type == UINT8 && wt.bytes.size() == (size_t)(N * K * bits / 8))
+                        << "onnx: MatMulNBits B must be uint8 with N*K*bits/8 bytes";
+                    int zp = 1 << (bits - 1);
+                    std::shared_ptr<graph::GNode> zps; // set when the zero points differ between blocks
                     if (has_input(n, 3))
                     {
+                        const int64_t blocks = K / block, z_stride = (blocks * bits + 7) / 8;
                         auto zi = init.find(n.inputs[3]);
-                        NNFUSION_CHECK(zi != init.end() && zi->second->data_type == UINT8 && !zi->second->bytes.empty())
-                            << "onnx: MatMulNBits zero points must be a packed uint8 initializer";
+                        NNFUSION_CHECK(zi != init.end() && zi->second->data_type == UINT8 &&
+                                       zi->second->bytes.size() == (size_t)(N * z_stride))
+                            << "onnx: MatMulNBits zero points must be a packed uint8 initializer of N * ceil(K/block_size*bits/8) bytes";
                         const std::vector<uint8_t>& z = zi->second->bytes;
-                        zp = z[0] & 0xF;
-                        const int64_t blocks = K / block;
-                        for (int64_t r = 0; r < N; ++r)
+                        auto at = [&](int64_t r, int64_t b) -> int {
+                            if (bits == 8)
+                                return z[(size_t)(r * z_stride + b)];
+                            const uint8_t byte = z[(size_t)(r * z_stride + b / 2)];
+                            return (b & 1) ? (byte >> 4) : (byte & 0xF);
+                        };
+                        zp = at(0, 0);
+                        bool uniform = true;
+                        for (int64_t r = 0; r < N && uniform; ++r)
                             for (int64_t b = 0; b < blocks; ++b)
-                            {
-                                const uint8_t byte = z[(size_t)(r * ((blocks + 1) / 2) + b / 2)];
-                                NNFUSION_CHECK(((b & 1) ? (byte >> 4) : (byte & 0xF)) == zp)
-                                    << "onnx: MatMulNBits with per-block zero points is not supported (a uniform one is)";
-                            }
+                                if (at(r, b) != zp)
+                                {
+                                    uniform = false;
+                                    break;
+                                }
+                        // one value everywhere is the scalar attribute (the specialised kernels take it); otherwise the
+                        // tensor travels with the node
+                        if (!uniform)
+                            zps = g->add_node_and_edge(
+                                std::make_shared<op::Constant>(element::u8, Shape{(size_t)N, (size_t)z_stride}, z.data()),
+                                graph::GNodeVector{});
                     }
                     auto wq = g->add_node_and_edge(
-                        std::make_shared<op::Constant>(element::u8, Shape{(size_t)N, (size_t)(K / 2)}, wt.bytes.data()), graph::GNodeVector{});
+                        std::make_shared<op::Constant>(element::u8, Shape{(size_t)N, (size_t)(K * bits / 8)}, wt.bytes.data()), graph::GNodeVector{});
                     const Tensor& st = *si->second;
                     const size_t n_scales = (size_t)(N * (K / block));
                     std::vector<uint16_t> sc(n_scales);
@@ -539,7 +558,13 @@ namespace nnfusion
                     }
                     auto s = g->add_node_and_edge(
                         std::make_shared<op::Constant>(element::f16, Shape{(size_t)N, (size_t)(K / block)}, sc.data()), graph::GNodeVector{});
-                    out = generic(n, "QuantDot", {input_of(n, 0), wq, s}, "{\"zero_point\": " + std::to_string(zp) + "}");
+                    std::string attrs = "{\"bits\": " + std::to_string(bits) + ", \"group_size\": " + std::to_string(block) +
+                                        ", \"zero_point\": " + std::to_string(zps ? 0 : zp) +
+                                        ", \"has_zero_points\": " + (zps ? "true" : "false") + "}";
+                    graph::GNodeVector ins = {input_of(n, 0), wq, s};
+                    if (zps)
+                        ins.push_back(zps);
+                    out = generic(n, "QuantDot", ins, attrs);
                 }
                 else if (n.op_type == "SimplifiedLayerNormalization" || n.op_type == "RMSNormalization")
                 {

@@ -49,8 +49,10 @@ namespace nnfusion
                     const bool has_bias = cfg["has_bias"].get<bool>();
                     const bool has_res = cfg["has_residual"].get<bool>();
                     const bool gate = cfg["act"].get<std::string>() == "silu_gate";
+                    const int bits = cfg["bits"].get<int>();
+                    const bool has_z = cfg["has_zero_points"].get<bool>();
                     // what the launcher supports; anything else is left to other emitters
-                    if (cfg["bits"].get<int>() != 4 || group != 128 || !cfg["transpose_B"].get<bool>())
+                    if (!cfg["transpose_B"].get<bool>())
                         return nullptr;
                     if (m_context->inputs[0]->get_element_type() != element::f16 ||
                         m_context->inputs[2]->get_element_type() != element::f16)
@@ -62,7 +64,22 @@ namespace nnfusion
                     const size_t K = a.back();
                     const size_t M = shape_size(a) / K;
                     const size_t N = gate ? w[0] / 2 : w[0];
-                    if (K % 128 != 0 || M == 0 || N == 0)
+                    if (M == 0 || N == 0)
+                        return nullptr;
+                    if (bits != 4 || group != 128 || has_z)
+                    {
+                        // other block parameters: the plain product only (nnf_wna16_gemm), no scratch memory
+                        if (rms || has_bias || has_res || gate || (bits != 4 && bits != 8) ||
+                            (group != 32 && group != 64 && group != 128) || K % group != 0)
+                            return nullptr;
+                        LanguageUnit_p lu(new LanguageUnit(get_function_name()));
+                        *lu << "const nnf_quant quant = {" << bits << ", " << group << ", " << zp << ", "
+                            << (has_z ? "input3" : "nullptr") << "};\n";
+                        *lu << "NNF_HIP_CHECK(nnf_wna16_gemm(stream, input0, input1, input2, output0, " << M << ", " << N << ", "
+                            << K << ", &quant, nullptr, 0));\n";
+                        return lu;
+                    }
+                    if (K % 128 != 0)
                         return nullptr;
 
                     size_t idx = 3;
@@ -132,7 +149,8 @@ namespace nnfusion
                     if (cfg["rms_norm"].get<bool>() || cfg["has_bias"].get<bool>() || cfg["has_residual"].get<bool>() ||
                         cfg["act"].get<std::string>() == "silu_gate")
                         return nullptr;
-                    if (cfg["bits"].get<int>() != 4 || group != 128 || !cfg["transpose_B"].get<bool>())
+                    if (cfg["bits"].get<int>() != 4 || group != 128 || cfg["has_zero_points"].get<bool>() ||
+                        !cfg["transpose_B"].get<bool>())
                         return nullptr;
                     if (m_context->inputs[0]->get_element_type() != element::f16 ||
                         m_context->inputs[2]->get_element_type() != element::f16)

@@ -3,9 +3,11 @@
 // They are GenericOps, not op::Dot: Dot's validation merges the element types of its two inputs and
 // rejects fp16 x u8 (src/nnfusion/core/operators/op_define/dot.cpp:47-53).
 //
-//   QuantDot       inputs: A f16 [M,K], Wq u8 [N,K/2] (int4 x2) , S f16 [N,K/group]
-//                          [, gamma f16 [K]] [, bias f16 [N]] [, residual f16 [M,N]]   (in this order, by attribute)
-//                  attrs : bits 4, group_size 128, zero_point 8, transpose_B true,
+//   QuantDot       inputs: A f16 [M,K], Wq u8 [N,K*bits/8] (bits 4: two per byte, low nibble first), S f16 [N,K/group]
+//                          [, Z u8 [N, ceil(K/group*bits/8)]] [, gamma f16 [K]] [, bias f16 [N]] [, residual f16 [M,N]]
+//                          (in this order, by attribute; Z: one zero point per (row, group), 4-bit ones two per byte)
+//                  attrs : bits 4|8, group_size 128, zero_point 8 (scalar, when has_zero_points is false), transpose_B true,
+//                          has_zero_points false,
 //                          rms_norm false, rms_eps 1e-6, has_bias false, has_residual false, act "none"|"silu_gate"
 //                  output: Y f16 [M, N]   (N = rows of Wq; half of them when act == "silu_gate")
 //   QuantDotW8A8   inputs: A i8 [M,K], s_tok f32 [M], W i8 [N,K], s_ch f32 [N];  attr out_type "f16"|"i32"
@@ -34,16 +36,18 @@ REGISTER_OP(QuantDot)
     .attr<int>("group_size", 128)
     .attr<int>("zero_point", 8)
     .attr<bool>("transpose_B", true)
+    .attr<bool>("has_zero_points", false)
     .attr<bool>("rms_norm", false)
     .attr<double>("rms_eps", 1e-6)
     .attr<bool>("has_bias", false)
     .attr<bool>("has_residual", false)
     .attr<std::string>("act", "none")
     .constrait([](const op::OpConfig::any& config) -> bool {
-        if (config.at("bits").get<int>() != 4)
+        const int bits = config.at("bits").get<int>();
+        if (bits != 4 && bits != 8)
             return false;
         int zp = config.at("zero_point").get<int>();
-        if (zp < 0 || zp > 15 || config.at("group_size").get<int>() <= 0)
+        if (zp < 0 || zp >= (1 << bits) || config.at("group_size").get<int>() <= 0)
             return false;
         auto act = config.at("act").get<std::string>();
         return act == "none" || act == "silu_gate";
@@ -51,18 +55,27 @@ REGISTER_OP(QuantDot)
     .infershape([](std::shared_ptr<graph::GNode> gnode) -> void {
         auto gop = std::dynamic_pointer_cast<op::GenericOp>(gnode->get_op_ptr());
         NNFUSION_CHECK_NOT_NULLPTR(gop);
-        size_t expect = 3 + (bool_attr(gop, "rms_norm") ? 1 : 0) + (bool_attr(gop, "has_bias") ? 1 : 0) +
+        const bool has_z = bool_attr(gop, "has_zero_points");
+        size_t expect = 3 + (has_z ? 1 : 0) + (bool_attr(gop, "rms_norm") ? 1 : 0) + (bool_attr(gop, "has_bias") ? 1 : 0) +
                         (bool_attr(gop, "has_residual") ? 1 : 0);
         OP_VALIDATION(gop, gnode->get_input_size() == expect) << "expected " << expect << " inputs";
         const Shape& a = gnode->get_input_shape(0);
         const Shape& w = gnode->get_input_shape(1);
         const Shape& s = gnode->get_input_shape(2);
         OP_VALIDATION(gop, a.size() >= 1 && w.size() == 2 && s.size() == 2) << "bad ranks";
-        OP_VALIDATION(gop, gnode->get_input_element_type(1) == element::u8) << "packed int4 weights travel as u8";
+        OP_VALIDATION(gop, gnode->get_input_element_type(1) == element::u8) << "quantized weights travel as u8";
         const size_t K = a.back();
         const size_t group = (size_t)int_attr(gop, "group_size");
-        OP_VALIDATION(gop, w[1] * 2 == K) << "Wq must be [N, K/2]";
+        const size_t bits = (size_t)int_attr(gop, "bits");
+        OP_VALIDATION(gop, w[1] * 8 == K * bits) << "Wq must be [N, K*bits/8]";
         OP_VALIDATION(gop, K % group == 0 && s[0] == w[0] && s[1] == K / group) << "scales must be [N, K/group]";
+        if (has_z)
+        {
+            const Shape& z = gnode->get_input_shape(3);
+            OP_VALIDATION(gop, gnode->get_input_element_type(3) == element::u8 && z.size() == 2 && z[0] == w[0] &&
+                                   z[1] == (K / group * bits + 7) / 8)
+                << "zero points must be u8 [N, ceil(K/group*bits/8)]";
+        }
         size_t N = w[0];
         if (gop->localOpConfig.getRoot()["act"].get<std::string>() == "silu_gate")
         {

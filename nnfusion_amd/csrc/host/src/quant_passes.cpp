@@ -96,6 +96,9 @@ namespace
         q.zp = cfg["zero_point"].get<int>();
         q.bits = cfg["bits"].get<int>();
         q.eps = cfg["rms_eps"].get<double>();
+        // only the specialised kernels have fused forms: a product with other block parameters stays as it is
+        if (q.bits != 4 || q.group != 128 || cfg["has_zero_points"].get<bool>())
+            return false;
         size_t i = 0;
         q.a = input_of(n, i++);
         q.wq = input_of(n, i++);

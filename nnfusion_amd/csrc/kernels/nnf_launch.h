@@ -98,8 +98,12 @@ namespace nnf
                                  int N, int K, int zp, const void* rms_gamma, float rms_eps, const void* bias,
                                  const void* residual, int act, void* rms_ws, void* partial_ws, int num_cu,
                                  const LaunchChoice& choice = LaunchChoice());
-    // bytes launch_w4a16_gemm writes at partial_ws for this call (0: it needs none)
 
+    // fp16 activations x 4- or 8-bit weights, groups of 32 / 64 / 128, a scalar zero point or one per (row, group)
+    // (zero_points: u8 [N, ceil(K/group * bits / 8)], 4-bit ones two to a byte, even group low): wna16_generic.hip
+    bool wna16_supported(int M, int N, int K, int bits, int group);
+    hipError_t launch_wna16_generic(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M, int N,
+                                    int K, int bits, int group, int zp, const void* zero_points, int num_cu);
 
     // W8A8: acc != nullptr writes the raw int32 accumulators, otherwise Y = fp16(acc * s_tok * s_ch).
     // partial_ws: nnf::workspace::w8a8_gemm(M, N, K) bytes (0 for the M <= 16 kernel)

@@ -1,0 +1,233 @@
+// fp16 activations x 4- or 8-bit weights with the block parameters the specialised kernels do not take: groups of
+// 32 / 64 / 128, one zero point per (row, group), 8-bit weights.
+//
+//   Y[M,N] = A[M,K] . ((Wq - zero point) * S)^T
+//
+// The reference's dequantize takes a scale and an offset per block of any shape
+// (src/nnfusion/core/kernels/cpu/reference/kernels.cpp:601-623: integer subtract of the offset, cast, multiply by
+// the scale); the kernels in w4a16_*.hip serve the one combination the benchmark uses (4 bits, groups of 128, a
+// scalar zero point) as fast as the hardware allows, these two serve every other one correctly and simply:
+//   * wna16_gemv_kernel (M <= 16): a wavefront per weight row, a lane dequantises eight weights at a time to fp32
+//     ((q - z) * s, as the oracle's weights) and multiplies them with the eight activations of every row;
+//   * wna16_tile_kernel (any M): 64 x 64 output tiles, four wavefronts of 32 x 32 (v_mfma_f32_32x32x16_f16), K steps of
+//     32: the weights of a step are dequantised to fp16((q - z) * s) on their way into LDS (what the tile GEMM's
+//     unpacking produces as well), the next step's operands are fetched into registers while this step's MFMAs run.
+#include "nnf_device.h"
+#include "nnf_launch.h"
+
+namespace nnf
+{
+    namespace
+    {
+        struct QuantArgs
+        {
+            const uint8_t* zps; // per-(row, group) zero points or null
+            int group_shift;    // log2 of the group size (32, 64 or 128)
+            int zp;             // scalar zero point (zps == null)
+            int zp_stride;      // bytes per row of zps
+        };
+
+        // eight consecutive weights of a row starting at k (a multiple of 8), as integers
+        template <int BITS>
+        __device__ __forceinline__ void load_q8(const uint8_t* __restrict__ row, int k, int (&q)[8])
+        {
+            if constexpr (BITS == 4)
+            {
+                const uint32_t w = *reinterpret_cast<const uint32_t*>(row + (k >> 1)); // nibble i = k + i
+#pragma unroll
+                for (int i = 0; i < 8; ++i)
+                    q[i] = (int)((w >> (4 * i)) & 0xFu);
+            }
+            else
+            {
+                const uintx2 w = *reinterpret_cast<const uintx2*>(row + k);
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                {
+                    q[i] = (int)((w.x >> (8 * i)) & 0xFFu);
+                    q[4 + i] = (int)((w.y >> (8 * i)) & 0xFFu);
+                }
+            }
+        }
+
+        template <int BITS>
+        __device__ __forceinline__ int zero_point_of(const QuantArgs& qa, int n, int g)
+        {
+            if (!qa.zps)
+                return qa.zp;
+            if constexpr (BITS == 4)
+            {
+                const uint8_t b = qa.zps[(size_t)n * qa.zp_stride + (g >> 1)];
+                return (g & 1) ? (b >> 4) : (b & 0xF);
+            }
+            else
+                return qa.zps[(size_t)n * qa.zp_stride + g];
+        }
+    } // namespace
+
+    // grid: any; each wavefront walks the rows n = its number, + the number of wavefronts, ...
+    template <int BITS>
+    __global__ __launch_bounds__(256) void wna16_gemv_kernel(const half_t* __restrict__ A, const uint8_t* __restrict__ Wq,
+                                                             const half_t* __restrict__ S, half_t* __restrict__ Y, int M, int N,
+                                                             int K, QuantArgs qa)
+    {
+        const int lane = threadIdx.x & 63;
+        const int wave = (int)blockIdx.x * 4 + (threadIdx.x >> 6), n_waves = (int)gridDim.x * 4;
+        const int G = K >> qa.group_shift;
+        const size_t row_bytes = (size_t)K * BITS / 8;
+        for (int n = wave; n < N; n += n_waves)
+        {
+            float acc[16];
+#pragma unroll
+            for (int m = 0; m < 16; ++m)
+                acc[m] = 0.f;
+            const uint8_t* row = Wq + (size_t)n * row_bytes;
+            for (int k = lane * 8; k < K; k += 64 * 8)
+            {
+                int q[8];
+                load_q8<BITS>(row, k, q);
+                const int g = k >> qa.group_shift; // eight consecutive weights never straddle a group (a multiple of 32)
+                const int z = zero_point_of<BITS>(qa, n, g);
+                const float s = (float)S[(size_t)n * G + g];
+                float w[8];
+#pragma unroll
+                for (int i = 0; i < 8; ++i)
+                    w[i] = (float)(q[i] - z) * s;
+#pragma unroll
+                for (int m = 0; m < 16; ++m)
+                    if (m < M)
+                    {
+                        const half8_t a = *reinterpret_cast<const half8_t*>(A + (size_t)m * K + k);
+                        float t = acc[m];
+#pragma unroll
+                        for (int i = 0; i < 8; ++i)
+                            t = __builtin_fmaf((float)a[i], w[i], t);
+                        acc[m] = t;
+                    }
+            }
+#pragma unroll
+            for (int m = 0; m < 16; ++m)
+                if (m < M)
+                {
+                    const float t = wave_sum(acc[m]);
+                    if (lane == 0)
+                        Y[(size_t)m * N + n] = (half_t)t;
+                }
+        }
+    }
+
+    // one workgroup of four wavefronts per 64 x 64 output tile (blockIdx.x: column tile, blockIdx.y: row tile)
+    template <int BITS>
+    __global__ __launch_bounds__(256) void wna16_tile_kernel(const half_t* __restrict__ A, const uint8_t* __restrict__ Wq,
+                                                             const half_t* __restrict__ S, half_t* __restrict__ Y, int M, int N,
+                                                             int K, QuantArgs qa)
+    {
+        constexpr int PITCH = 40; // halves per staged row: 32 of K + 8 of padding (80 bytes: 16-byte pieces stay aligned)
+        __shared__ __attribute__((aligned(16))) half_t a_s[64 * PITCH];
+        __shared__ __attribute__((aligned(16))) half_t w_s[64 * PITCH];
+        const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+        const int m0 = (int)blockIdx.y * 64, n0 = (int)blockIdx.x * 64;
+        const int G = K >> qa.group_shift;
+        const size_t row_bytes = (size_t)K * BITS / 8;
+        // staging: thread t moves eight elements of K (piece t % 4) of row t / 4 of either operand
+        const int s_row = tid >> 2, s_k = (tid & 3) * 8;
+        const bool a_ok = m0 + s_row < M, w_ok = n0 + s_row < N;
+        const half_t* a_src = A + (size_t)min(m0 + s_row, M - 1) * K + s_k;
+        const uint8_t* w_row = Wq + (size_t)min(n0 + s_row, N - 1) * row_bytes;
+        const int w_n = min(n0 + s_row, N - 1);
+        // fragments: wavefront (wm, wn) owns rows [32 wm, +32) x columns [32 wn, +32); lane l holds eight elements of K
+        // (block l / 32 of the 16) of row / column l % 32
+        const int wm = wave >> 1, wn = wave & 1;
+        const int f_row = lane & 31, f_k = (lane >> 5) * 8;
+
+        uintx4 a_next = {0u, 0u, 0u, 0u};
+        int q_next[8];
+        float s_next = 0.f;
+        int z_next = 0;
+        auto fetch = [&](int k0) {
+            if (a_ok)
+                a_next = *reinterpret_cast<const uintx4*>(a_src + k0);
+            load_q8<BITS>(w_row, k0 + s_k, q_next);
+            const int g = (k0 + s_k) >> qa.group_shift;
+            z_next = zero_point_of<BITS>(qa, w_n, g);
+            s_next = (float)S[(size_t)w_n * G + g];
+        };
+        auto stage = [&]() {
+            *reinterpret_cast<uintx4*>(a_s + s_row * PITCH + s_k) = a_next; // rows past M stay zero
+            half8_t w;
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                w[i] = w_ok ? (half_t)((float)(q_next[i] - z_next) * s_next) : (half_t)0.f;
+            *reinterpret_cast<half8_t*>(w_s + s_row * PITCH + s_k) = w;
+        };
+        floatx16 acc;
+#pragma unroll
+        for (int i = 0; i < 16; ++i)
+            acc[i] = 0.f;
+        fetch(0);
+        for (int k0 = 0; k0 < K; k0 += 32)
+        {
+            stage();
+            __syncthreads();
+            if (k0 + 32 < K)
+                fetch(k0 + 32);
+#pragma unroll
+            for (int kk = 0; kk < 2; ++kk)
+            {
+                const half8_t fa = *reinterpret_cast<const half8_t*>(a_s + (wm * 32 + f_row) * PITCH + kk * 16 + f_k);
+                const half8_t fw = *reinterpret_cast<const half8_t*>(w_s + (wn * 32 + f_row) * PITCH + kk * 16 + f_k);
+                acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa, fw, acc, 0, 0, 0);
+            }
+            __syncthreads();
+        }
+        // D[m][n]: lane l holds column l % 32; element i is row 8 (i / 4) + 4 (l / 32) + i % 4
+        const int n = n0 + wn * 32 + (lane & 31);
+#pragma unroll
+        for (int i = 0; i < 16; ++i)
+        {
+            const int m = m0 + wm * 32 + 8 * (i >> 2) + 4 * (lane >> 5) + (i & 3);
+            if (m < M && n < N)
+                Y[(size_t)m * N + n] = (half_t)acc[i];
+        }
+    }
+
+    bool wna16_supported(int M, int N, int K, int bits, int group)
+    {
+        return M > 0 && N > 0 && K > 0 && (bits == 4 || bits == 8) && (group == 32 || group == 64 || group == 128) && K % group == 0;
+    }
+
+    hipError_t launch_wna16_generic(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M, int N, int K,
+                                    int bits, int group, int zp, const void* zero_points, int num_cu)
+    {
+        if (!wna16_supported(M, N, K, bits, group))
+            return hipErrorInvalidValue;
+        QuantArgs qa;
+        qa.zps = (const uint8_t*)zero_points;
+        qa.group_shift = group == 32 ? 5 : group == 64 ? 6 : 7;
+        qa.zp = zp;
+        qa.zp_stride = (K / group * bits + 7) / 8;
+        if (M <= 16)
+        {
+            // enough wavefronts to cover the rows once, at most eight workgroups of four per CU
+            const int want = (N + 3) / 4, cap = num_cu * 8;
+            const dim3 grid((unsigned)(want < cap ? want : cap));
+            if (bits == 4)
+                hipLaunchKernelGGL(wna16_gemv_kernel<4>, grid, dim3(256), 0, stream, (const half_t*)A, (const uint8_t*)Wq,
+                                   (const half_t*)S, (half_t*)Y, M, N, K, qa);
+            else
+                hipLaunchKernelGGL(wna16_gemv_kernel<8>, grid, dim3(256), 0, stream, (const half_t*)A, (const uint8_t*)Wq,
+                                   (const half_t*)S, (half_t*)Y, M, N, K, qa);
+            return hipGetLastError();
+        }
+        const dim3 grid((unsigned)((N + 63) / 64), (unsigned)((M + 63) / 64));
+        if (grid.y > 65535u)
+            return hipErrorInvalidValue;
+        if (bits == 4)
+            hipLaunchKernelGGL(wna16_tile_kernel<4>, grid, dim3(256), 0, stream, (const half_t*)A, (const uint8_t*)Wq,
+                               (const half_t*)S, (half_t*)Y, M, N, K, qa);
+        else
+            hipLaunchKernelGGL(wna16_tile_kernel<8>, grid, dim3(256), 0, stream, (const half_t*)A, (const uint8_t*)Wq,
+                               (const half_t*)S, (half_t*)Y, M, N, K, qa);
+        return hipGetLastError();
+    }
+} // namespace nnf

@@ -184,6 +184,45 @@ int nnf_w4a16_gemm_static_scratch(nnf_stream_t stream, const void* A, const void
     return nnf_w4a16_gemm(stream, A, Wq, scales, Y, M, N, K, group, zp, dev.static_scratch, STATIC_SCRATCH_BYTES);
 }
 
+int nnf_wna16_supported(int M, int N, int K, const nnf_quant* q)
+{
+    if (!q || q->zero_point < 0 || q->zero_point >= (1 << (q->bits == 8 ? 8 : 4)))
+        return 0;
+    return nnf::wna16_supported(M, N, K, q->bits, q->group) ? 1 : 0;
+}
+
+namespace
+{
+    // the parameters of the specialised fp16 x int4 kernels
+    bool is_plain_w4a16(const nnf_quant* q) { return q->bits == 4 && q->group == 128 && !q->zero_points; }
+} // namespace
+
+size_t nnf_wna16_gemm_workspace_bytes(int M, int N, int K, const nnf_quant* q)
+{
+    return (q && is_plain_w4a16(q)) ? nnf::workspace::w4a16_gemm(M, N, K, q->group) : 0;
+}
+
+int nnf_wna16_gemm(nnf_stream_t stream, const void* A, const void* Wq, const void* scales, void* Y, int M, int N, int K,
+                   const nnf_quant* q, void* workspace, size_t workspace_bytes)
+{
+    if (!q)
+        return NNF_ERR_INVALID_ARGUMENT;
+    if (is_plain_w4a16(q))
+        return nnf_w4a16_gemm(stream, A, Wq, scales, Y, M, N, K, q->group, q->zero_point, workspace, workspace_bytes);
+    if (!A || !Wq || !scales || !Y || M <= 0 || N <= 0 || K <= 0)
+        return NNF_ERR_INVALID_ARGUMENT;
+    if (!aligned16(A) || !aligned16(Wq) || !aligned16(scales) || !aligned16(Y))
+        return NNF_ERR_INVALID_ARGUMENT;
+    if (!nnf_wna16_supported(M, N, K, q))
+        return NNF_ERR_UNSUPPORTED_SHAPE;
+    DeviceInfo dev;
+    const int st = current_device_info(dev);
+    if (st != NNF_OK)
+        return st;
+    return (int)nnf::launch_wna16_generic((hipStream_t)stream, A, Wq, scales, Y, M, N, K, q->bits, q->group, q->zero_point,
+                                          q->zero_points, dev.num_cu);
+}
+
 int nnf_w4a16_variant_supported(int M, int N, int K, int group, int variant)
 {
     return (group == 128 && nnf::workspace::w4a16_variant_fits(M, N, K, variant)) ? 1 : 0;

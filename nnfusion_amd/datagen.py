@@ -10,7 +10,7 @@ import numpy as np
 from . import _lib
 
 # stream ids
-S_ACT, S_WQ, S_SCALE, S_GAMMA, S_A8, S_W8, S_STOK, S_SCH, S_WQ2, S_SCALE2, S_BIAS, S_RES = range(1, 13)
+S_ACT, S_WQ, S_SCALE, S_GAMMA, S_A8, S_W8, S_STOK, S_SCH, S_WQ2, S_SCALE2, S_BIAS, S_RES, S_ZP = range(1, 14)
 
 
 def _ptr(a):
@@ -55,6 +55,23 @@ def w4a16_case(seed, m, n, k, group=128):
     wq = uniform_u4_packed(seed, S_WQ, n, k)
     s = uniform_f16(seed, S_SCALE, (n, k // group), 0.005, 0.02)
     return a, wq, s
+
+
+def wna16_case(seed, m, n, k, bits, group, zero_points=False):
+    """(A fp16 [m,k], Wq u8 [n,k*bits/8], scales fp16 [n,k/group], zero points u8 [n, ceil(k/group*bits/8)] or None) with
+    4- or 8-bit weights: weights and zero points uniform over their whole range, scales uniform [0.005, 0.02) / 2^(bits-4)
+    (the same spread of dequantised values for either width)."""
+    assert bits in (4, 8) and k % group == 0
+    a = normal_f16(seed, S_ACT, (m, k))
+    g = k // group
+    if bits == 4:
+        wq = uniform_u4_packed(seed, S_WQ, n, k)
+        z = uniform_u4_packed(seed, S_ZP, n, g + (g & 1)) if zero_points else None
+    else:
+        wq = uniform_i8(seed, S_WQ, (n, k), -128, 127).view(np.uint8)
+        z = uniform_i8(seed, S_ZP, (n, g), -128, 127).view(np.uint8) if zero_points else None
+    s = uniform_f16(seed, S_SCALE, (n, g), 0.005 / (1 << (bits - 4)), 0.02 / (1 << (bits - 4)))
+    return a, wq, s, z
 
 
 def w8a8_case(seed, m, n, k):

@@ -1,4 +1,4 @@
-"""Writes small ONNX models of the quantized path (com.microsoft::MatMulNBits, 4 bits, block 128) without the
+"""Writes small ONNX models of the quantized path (com.microsoft::MatMulNBits) without the
 `onnx` package: a minimal encoder of the protobuf wire format for the messages of onnx.proto3 that such a model
 needs.  The layouts are those of the operator: B = uint8 [N, K/128, 64] with the even k in the low nibble, scales
 [N * K/128], which is byte for byte the `Wq [N, K/2]` / `scales [N, K/128]` layout of include/nnf_hip_kernels.h.
@@ -70,9 +70,9 @@ def _node(op_type, inputs, outputs, name, attrs=(), domain=""):
     return msg
 
 
-def _matmul_nbits(name, a, w_name, s_name, out, n, k):
-    return _node("MatMulNBits", [a, w_name, s_name], [out], name,
-                 [_attr_int("K", k), _attr_int("N", n), _attr_int("bits", 4), _attr_int("block_size", 128)],
+def _matmul_nbits(name, a, w_name, s_name, out, n, k, bits=4, block=128, z_name=None):
+    return _node("MatMulNBits", [a, w_name, s_name] + ([z_name] if z_name else []), [out], name,
+                 [_attr_int("K", k), _attr_int("N", n), _attr_int("bits", bits), _attr_int("block_size", block)],
                  domain="com.microsoft")
 
 
@@ -94,10 +94,21 @@ def _weights(prefix, wq, scales):
             _tensor(prefix + "_scales", scales.reshape(-1), FLOAT16)], n, k
 
 
-def write_quant_linear(path, m, wq, scales):
-    """y [m, N] = MatMulNBits(x [m, K], B, scales)"""
-    inits, n, k = _weights("linear", wq, scales)
-    nodes = [_matmul_nbits("linear", "x", "linear_B", "linear_scales", "y", n, k)]
+def write_quant_linear(path, m, wq, scales, bits=4, block=128, zero_points=None):
+    """y [m, N] = MatMulNBits(x [m, K], B, scales[, zero_points]); scales fp16 or fp32 [N, K/block], zero_points u8
+    [N, ceil(K/block*bits/8)] (4-bit ones two per byte, even block in the low nibble)."""
+    if (bits, block) == (4, 128) and zero_points is None and scales.dtype == np.float16:
+        inits, n, k = _weights("linear", wq, scales)
+    else:
+        n, k = wq.shape[0], wq.shape[1] * 8 // bits
+        assert wq.dtype == np.uint8 and scales.shape == (n, k // block) and scales.dtype in (np.float16, np.float32)
+        inits = [_tensor("linear_B", wq, UINT8, dims=(n, k // block, block * bits // 8)),
+                 _tensor("linear_scales", scales.reshape(-1), FLOAT16 if scales.dtype == np.float16 else FLOAT)]
+        if zero_points is not None:
+            assert zero_points.dtype == np.uint8 and zero_points.shape == (n, (k // block * bits + 7) // 8)
+            inits.append(_tensor("linear_zp", zero_points.reshape(-1), UINT8))
+    nodes = [_matmul_nbits("linear", "x", "linear_B", "linear_scales", "y", n, k, bits, block,
+                           "linear_zp" if zero_points is not None else None)]
     data = _model("quant_linear", nodes, inits, [_value_info("x", FLOAT16, (m, k))], [_value_info("y", FLOAT16, (m, n))])
     with open(path, "wb") as f:
         f.write(data)

@@ -68,6 +68,44 @@ def w4a16_gemm(a, wq, scales, group=128, zp=8, out=None, workspace=None):
     return out
 
 
+class NnfQuant(ctypes.Structure):
+    """struct nnf_quant of the C header: the block parameters of the weights."""
+    _fields_ = [("bits", ctypes.c_int), ("group", ctypes.c_int), ("zero_point", ctypes.c_int),
+                ("zero_points", ctypes.c_void_p)]
+
+
+def _quant_arg(bits, group, zp, zero_points):
+    q = NnfQuant(int(bits), int(group), int(zp), _p(zero_points))
+    return q, ctypes.cast(ctypes.pointer(q), ctypes.c_void_p)
+
+
+def wna16_supported(m, n, k, bits, group, zp=8):
+    _, qp = _quant_arg(bits, group, zp, None)
+    return bool(_lib.kernels().nnf_wna16_supported(m, n, k, qp))
+
+
+def wna16_gemm(a, wq, scales, bits=4, group=128, zp=8, zero_points=None, out=None, workspace=None):
+    """Y[M,N] = A[M,K] . ((Wq - z) * scales)^T with 4- or 8-bit weights (wq u8 [N, K*bits/8]), groups of 32 / 64 / 128
+    and either a scalar zero point or zero_points u8 [N, ceil(K/group*bits/8)] (4-bit: two per byte, even group low)."""
+    lib = _lib.kernels()
+    m, k = a.shape
+    n = wq.shape[0]
+    assert a.dtype == torch.float16 and wq.dtype == torch.uint8 and scales.dtype == torch.float16
+    assert a.is_contiguous() and wq.is_contiguous() and scales.is_contiguous()
+    assert wq.shape[1] * 8 == k * bits and tuple(scales.shape) == (n, k // group)
+    if zero_points is not None:
+        assert zero_points.dtype == torch.uint8 and zero_points.is_contiguous()
+        assert tuple(zero_points.shape) == (n, (k // group * bits + 7) // 8)
+    if out is None:
+        out = torch.empty((m, n), dtype=torch.float16, device=a.device)
+    keep, qp = _quant_arg(bits, group, zp, zero_points)
+    if workspace is None:
+        workspace = _ws(lib.nnf_wna16_gemm_workspace_bytes(m, n, k, qp), a.device)
+    _check(lib.nnf_wna16_gemm(_stream(), a.data_ptr(), wq.data_ptr(), scales.data_ptr(), out.data_ptr(), m, n, k, qp,
+                              workspace.data_ptr(), workspace.numel()), "nnf_wna16_gemm")
+    return out
+
+
 VARIANTS = {"auto": 0, "gemv_valu": 1, "gemv_mfma": 2, "gemm_mfma": 3, "gemv_rows": 4}
 
 

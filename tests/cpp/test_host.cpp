@@ -373,11 +373,11 @@ int main(int argc, char** argv)
     run_case("quant_dot_emitter_declines", [] {
         pass::graph::DefaultKernelSelector sel;
         {
-            graph::Graph g; // group 64 is a legal op, but this emitter does not serve it
+            graph::Graph g; // groups of 16 are a legal op, but no kernel serves them
             auto a = param(g, element::f16, Shape{1, 256});
             auto w = param(g, element::u8, Shape{8, 128});
-            auto s = param(g, element::f16, Shape{8, 4});
-            auto n = g.add_node_and_edge(std::make_shared<op::GenericOp>("x", "QuantDot", op::OpConfig::any::parse("{\"group_size\": 64}")),
+            auto s = param(g, element::f16, Shape{8, 16});
+            auto n = g.add_node_and_edge(std::make_shared<op::GenericOp>("x", "QuantDot", op::OpConfig::any::parse("{\"group_size\": 16}")),
                                          {a, w, s});
             EXPECT(sel.pick_first(n, ROCM_GPU).second == nullptr);
         }
@@ -852,6 +852,86 @@ int main(int argc, char** argv)
             auto sl = find(g, "Slice");
             CONTAINS(sel.pick_first(sl, ROCM_GPU).second->get_or_emit_source()->body_unit->get_code(),
                      "hipMemcpy2DAsync(output0, 256, (const char*)input0 + 0, 512, 256, 8, hipMemcpyDeviceToDevice, stream)");
+        }
+    });
+
+    // QuantDot with other block parameters than the specialised kernels': shapes, emitter, and that the fusion passes
+    // leave such a node alone (only the 4-bit / 128 / scalar-zero-point product has fused forms)
+    run_case("quant_dot_block_parameters", [] {
+        auto cst = [](graph::Graph& g, const element::Type& t, const Shape& s) {
+            std::vector<uint8_t> d(shape_size(s) * t.size(), 1);
+            return g.add_node_and_edge(std::make_shared<op::Constant>(t, s, d.data()), graph::GNodeVector{});
+        };
+        auto quant_dot = [](graph::Graph& g, const graph::GNodeVector& in, const std::string& cfg) {
+            return g.add_node_and_edge(std::make_shared<op::GenericOp>("qd", "QuantDot", op::OpConfig::any::parse(cfg)), in);
+        };
+        const size_t M = 4, N = 48, K = 320;
+        pass::graph::DefaultKernelSelector sel;
+        {
+            // 8 bits, groups of 64, a zero point per (row, group): five groups of a row in five bytes
+            auto g = std::make_shared<graph::Graph>();
+            auto x = param(*g, element::f16, Shape{M, K});
+            auto q = quant_dot(*g, {x, cst(*g, element::u8, Shape{N, K}), cst(*g, element::f16, Shape{N, K / 64}),
+                                    cst(*g, element::u8, Shape{N, K / 64})},
+                               "{\"bits\": 8, \"group_size\": 64, \"zero_point\": 0, \"has_zero_points\": true}");
+            EXPECT(q->get_output_shape(0) == (Shape{M, N}) && q->get_output_element_type(0) == element::f16);
+            const std::string body = sel.pick_first(q, ROCM_GPU).second->get_or_emit_source()->body_unit->get_code();
+            CONTAINS(body, "const nnf_quant quant = {8, 64, 0, input3};");
+            CONTAINS(body, "nnf_wna16_gemm(stream, input0, input1, input2, output0, 4, 48, 320, &quant, nullptr, 0)");
+        }
+        {
+            // 4 bits, groups of 32, scalar zero point; ten groups, and with a tensor five bytes of two zero points each
+            auto g = std::make_shared<graph::Graph>();
+            auto x = param(*g, element::f16, Shape{M, K});
+            auto q = quant_dot(*g, {x, cst(*g, element::u8, Shape{N, K / 2}), cst(*g, element::f16, Shape{N, K / 32})},
+                               "{\"group_size\": 32, \"zero_point\": 3}");
+            CONTAINS(sel.pick_first(q, ROCM_GPU).second->get_or_emit_source()->body_unit->get_code(),
+                     "const nnf_quant quant = {4, 32, 3, nullptr};");
+            bool threw = false;
+            try
+            {
+                quant_dot(*g, {x, cst(*g, element::u8, Shape{N, K / 2}), cst(*g, element::f16, Shape{N, K / 32}),
+                               cst(*g, element::u8, Shape{N, K / 32})},
+                          "{\"group_size\": 32, \"has_zero_points\": true}");
+            }
+            catch (const CheckError&)
+            {
+                threw = true; // zero points of 4 bits come two to a byte: [N, 5]
+            }
+            EXPECT(threw);
+            threw = false;
+            try
+            {
+                quant_dot(*g, {x, cst(*g, element::u8, Shape{N, K / 2}), cst(*g, element::f16, Shape{N, K / 32})},
+                          "{\"bits\": 8, \"group_size\": 32}"); // 8-bit weights are [N, K]
+            }
+            catch (const CheckError&)
+            {
+                threw = true;
+            }
+            EXPECT(threw);
+        }
+        {
+            // RMSNorm -> QuantDot(groups of 64) -> Add: nothing folds into a product the fused kernels do not serve
+            auto g = std::make_shared<graph::Graph>();
+            auto x = param(*g, element::f16, Shape{M, K});
+            auto r = param(*g, element::f16, Shape{M, N});
+            auto n = g->add_node_and_edge(std::make_shared<op::GenericOp>("norm", "RMSNorm", op::OpConfig::any()),
+                                          {x, cst(*g, element::f16, Shape{K})});
+            auto q = quant_dot(*g, {n, cst(*g, element::u8, Shape{N, K / 2}), cst(*g, element::f16, Shape{N, K / 64})},
+                               "{\"group_size\": 64}");
+            auto y = g->add_node_and_edge(std::make_shared<op::GenericOp>("y", "Add", op::OpConfig::any()), {q, r});
+            g->add_node_and_edge(std::make_shared<op::Result>(), {y});
+            pass::graph::QuantEpilogueFusionPass fusion;
+            pass::graph::QuantGemmFusionPass merge;
+            EXPECT(fusion.run_on_graph(g) && fusion.fused == 0 && merge.run_on_graph(g) && merge.merged_groups == 0);
+            size_t norms = 0, adds = 0;
+            for (auto& node : g->get_ordered_ops())
+            {
+                norms += node->get_op_type() == "RMSNorm";
+                adds += node->get_op_type() == "Add";
+            }
+            EXPECT(norms == 1 && adds == 1);
         }
     });
 

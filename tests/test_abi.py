@@ -56,6 +56,23 @@ def test_pure_host_queries_work_without_a_gpu():
     assert lib.nnf_w4a16_variant_supported(1, 4096, 4096, 128, 4) == 1 and lib.nnf_w4a16_variant_supported(64, 4096, 4096, 128, 4) == 0
     assert lib.nnf_w8a8_variant_supported(1, 4096, 4096, 3) == 1 and lib.nnf_w8a8_variant_supported(64, 4096, 4096, 1) == 0
     assert lib.nnf_w4a16_gemm_variant_workspace_bytes(4096, 8192, 8192, 128, 3, None) == 0
+    # the general quantisation parameters: which combinations are served, and that only the specialised kernels use scratch
+    from nnfusion_amd.ops import NnfQuant
+
+    def qp(*f):
+        q = NnfQuant(*f)
+        return q, ctypes.cast(ctypes.pointer(q), ctypes.c_void_p)
+
+    for fields, ok in (((4, 32, 8, None), 1), ((8, 128, 255, None), 1), ((8, 64, 256, None), 0), ((4, 16, 8, None), 0),
+                       ((2, 32, 0, None), 0), ((4, 64, 16, None), 0)):
+        keep, p = qp(*fields)
+        assert lib.nnf_wna16_supported(8, 64, 256, p) == ok, fields
+    keep, p = qp(4, 64, 8, None)
+    assert lib.nnf_wna16_supported(8, 64, 96, p) == 0  # K % group
+    assert lib.nnf_wna16_gemm_workspace_bytes(128, 4096, 4096, p) == 0
+    keep, p = qp(4, 128, 8, None)
+    assert lib.nnf_wna16_gemm_workspace_bytes(128, 4096, 4096, p) == lib.nnf_w4a16_gemm_workspace_bytes(128, 4096, 4096, 128) > 0
+    assert lib.nnf_wna16_gemm(None, None, None, None, None, 1, 64, 128, p, None, 0) == -1
     # argument checks come before any device access
     assert lib.nnf_w4a16_gemm(None, None, None, None, None, 1, 1, 128, 128, 8, None, 0) == -1
     assert lib.nnf_w8a8_gemm_acc(None, None, None, None, 1, 1, 128, None, 0) == -1

@@ -69,6 +69,26 @@ def test_onnx_front_door_imports_fuses_and_generates(tmp_path):
     out2 = str(tmp_path / "rt2") + "/"
     subprocess.run([TOOL, "onnx", out2, lin], check=True, timeout=60)
     assert "nnf_w4a16_gemm(stream, input0, input1, input2, output0, 2, 64, 256, 128, 8, nullptr, 0)" in open(out2 + "nnfusion_rt.cpp").read()
+    # other block parameters: 8 bits, blocks of 64, a zero point per block and fp32 scales go to nnf_wna16_gemm with the
+    # zero points as a fourth input; a zero-point tensor that holds one value becomes the scalar of the plain call
+    _, wq8, s8, z8 = datagen.wna16_case(0, 2, 64, 256, 8, 64, True)
+    onnx_writer.write_quant_linear(lin, 2, wq8, s8.astype(np.float32), bits=8, block=64, zero_points=z8)
+    out4 = str(tmp_path / "rt4") + "/"
+    subprocess.run([TOOL, "onnx", out4, lin], check=True, timeout=60)
+    text = open(out4 + "nnfusion_rt.cpp").read()
+    assert "const nnf_quant quant = {8, 64, 0, input3};" in text
+    assert "nnf_wna16_gemm(stream, input0, input1, input2, output0, 2, 64, 256, &quant, nullptr, 0)" in text
+    blobs = {os.path.getsize(out4 + "Constant/" + c): open(out4 + "Constant/" + c, "rb").read() for c in os.listdir(out4 + "Constant")}
+    assert blobs[wq8.nbytes] == wq8.tobytes() and blobs[z8.nbytes] == z8.tobytes() and blobs[s8.nbytes] == s8.tobytes()
+    onnx_writer.write_quant_linear(lin, 2, wq, s, zero_points=np.full((64, 1), 0x55, np.uint8))
+    out5 = str(tmp_path / "rt5") + "/"
+    subprocess.run([TOOL, "onnx", out5, lin], check=True, timeout=60)
+    assert "nnf_w4a16_gemm(stream, input0, input1, input2, output0, 2, 64, 256, 128, 5, nullptr, 0)" in open(out5 + "nnfusion_rt.cpp").read()
+    _, wq4, s4, z4 = datagen.wna16_case(0, 2, 64, 256, 4, 32, True)
+    onnx_writer.write_quant_linear(lin, 2, wq4, s4, bits=4, block=32, zero_points=z4)
+    out6 = str(tmp_path / "rt6") + "/"
+    subprocess.run([TOOL, "onnx", out6, lin], check=True, timeout=60)
+    assert "const nnf_quant quant = {4, 32, 0, input3};" in open(out6 + "nnfusion_rt.cpp").read()
     bad = subprocess.run([TOOL, "onnx", str(tmp_path / "rt3") + "/", os.path.join(ROOT, "tests", "golden", "onnx", "gemm_op.onnx")],
                          stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=60)
     assert bad.returncode == 1 and "unsupported operator Gemm" in bad.stderr
@@ -152,6 +172,12 @@ def test_generated_runtime_of_an_onnx_model(gpu):
     a, wq, s = datagen.w4a16_case(0, m, n, k)
     y = _run_generated("onnx_linear", [a], (m, n), torch.float16, gpu)
     ref = oracle.w4a16_gemm(a, wq, s, f32_out=True)
+    assert np.abs(y.astype(np.float32) - ref).max() <= 1e-2 * _rms(ref)
+    # 8-bit weights in blocks of 64 with a zero point each (fp32 scales in the file, fp16 on the device)
+    _, m, n, k = entry.ONNX_EXAMPLES["onnx_linear_w8"]
+    a, wq, s, z = datagen.wna16_case(0, m, n, k, 8, 64, True)
+    y = _run_generated("onnx_linear_w8", [a], (m, n), torch.float16, gpu)
+    ref = oracle.wna16_gemm(a, wq, s, 8, 64, zero_points=z, f32_out=True)
     assert np.abs(y.astype(np.float32) - ref).max() <= 1e-2 * _rms(ref)
 
 

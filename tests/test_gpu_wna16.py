@@ -1,0 +1,129 @@
+"""Parity of nnf_wna16_gemm (4- or 8-bit weights, groups of 32 / 64 / 128, scalar or per-(row, group) zero points; HIP,
+through the C ABI) against the CPU oracle.
+
+Tolerance (stated by the task): max|y - y_ref| <= 1e-2 * RMS(y_ref), y_ref = the oracle's fp32-accumulated product with
+the weights dequantised as (q - z) * s; a one-hot activation row must return the dequantised weights exactly.
+"""
+import ctypes
+
+import numpy as np
+import pytest
+
+import oracle
+from nnfusion_amd import datagen
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-2
+
+
+def _case(seed, m, n, k, bits, group, zp_tensor):
+    return datagen.wna16_case(seed, m, n, k, bits, group, zp_tensor)
+
+
+def _run(gpu, a, wq, s, bits, group, zp, zps):
+    import torch
+
+    from nnfusion_amd import ops
+
+    t = [torch.from_numpy(x).to(gpu) for x in (a, wq, s)]
+    tz = None if zps is None else torch.from_numpy(zps).to(gpu)
+    y = ops.wna16_gemm(*t, bits=bits, group=group, zp=zp, zero_points=tz)
+    torch.cuda.synchronize()
+    return y.cpu().numpy()
+
+
+def _check(y, ref):
+    rms = float(np.sqrt(np.mean(ref.astype(np.float64) ** 2)))
+    err = float(np.abs(y.astype(np.float32) - ref).max())
+    assert np.isfinite(y).all()
+    assert err <= TOL * max(rms, 1e-6), (err, rms)
+
+
+SHAPES = [
+    # the wavefront-per-row kernel (M <= 16): one row, ragged N, K shorter than one pass of a wavefront, an odd number
+    # of groups, the benchmark's shapes
+    (1, 4096, 4096), (1, 33, 128), (3, 1000, 512), (16, 257, 2048), (5, 64, 160), (1, 12288, 4096), (8, 300, 11008),
+    (16, 4111, 4096), (2, 7, 384),
+    # the tile kernel: one partial tile, ragged M and N, many tiles, a long K
+    (17, 33, 128), (64, 64, 512), (100, 1000, 160), (300, 257, 2048), (128, 4096, 4096), (33, 520, 11008), (1024, 130, 384),
+]
+
+
+@pytest.mark.parametrize("m,n,k", SHAPES)
+@pytest.mark.parametrize("bits,group,zp_tensor", [
+    (4, 32, False), (4, 32, True), (4, 64, False), (4, 64, True), (4, 128, True),
+    (8, 32, False), (8, 32, True), (8, 64, True), (8, 128, False), (8, 128, True),
+])
+def test_wna16_matches_oracle(gpu, m, n, k, bits, group, zp_tensor):
+    if k % group:
+        pytest.skip("K is not a multiple of the group")
+    a, wq, s, zps = _case(m * 131 + n + k + bits + group, m, n, k, bits, group, zp_tensor)
+    zp = 7 if bits == 4 else 131
+    ref = oracle.wna16_gemm(a, wq, s, bits, group, zp=zp, zero_points=zps, f32_out=True)
+    _check(_run(gpu, a, wq, s, bits, group, zp, zps), ref)
+
+
+@pytest.mark.parametrize("m", [4, 40])
+@pytest.mark.parametrize("bits,group,zp_tensor", [(4, 32, True), (4, 64, False), (8, 64, True), (8, 128, False), (8, 32, True)])
+def test_one_hot_rows_return_the_dequantised_weights(gpu, m, bits, group, zp_tensor):
+    """A = e_k: 1 * w is exact in either kernel, so the output is fp16((q - z) * s) bit for bit; pins nibble and byte
+    order of weights and zero points and the block each scale belongs to, on the device."""
+    n, k = 70, 640
+    _, wq, s, zps = _case(5, m, n, k, bits, group, zp_tensor)
+    zp = 3 if bits == 4 else 200
+    wd = oracle.dequantize_wn(wq, s, bits, group, zp=zp, zero_points=zps)
+    ks = [0, 1, 7, 8, 31, 32, 63, 64, 127, 128, 255, 256, 511, 512, 639][:m] if m <= 16 else list(range(0, 640, 16))
+    a = np.zeros((m, k), np.float16)
+    for r, kk in enumerate(ks):
+        a[r, kk] = 1.0
+    y = _run(gpu, a, wq, s, bits, group, zp, zps)
+    for r, kk in enumerate(ks):
+        np.testing.assert_array_equal(y[r], wd[:, kk].astype(np.float16))
+    assert not y[len(ks):].any()
+
+
+def test_default_parameters_are_the_specialised_kernels(gpu):
+    import torch
+
+    from nnfusion_amd import ops
+
+    for m, n, k in ((1, 4096, 4096), (16, 1000, 2048), (128, 512, 4096)):
+        a, wq, s = datagen.w4a16_case(3, m, n, k)
+        t = [torch.from_numpy(x).to(gpu) for x in (a, wq, s)]
+        y0 = ops.w4a16_gemm(*t, zp=8)
+        y1 = ops.wna16_gemm(*t, bits=4, group=128, zp=8)
+        assert torch.equal(y0, y1)
+        # ... and a zero-point tensor holding the scalar everywhere takes the plain kernels to the same product
+        zps = torch.full((n, (k // 128 + 1) // 2), 0x88, dtype=torch.uint8, device=gpu)
+        y2 = ops.wna16_gemm(*t, bits=4, group=128, zero_points=zps)
+        torch.cuda.synchronize()
+        ref = oracle.wna16_gemm(a, wq, s, 4, 128, zp=8, f32_out=True)
+        _check(y2.cpu().numpy(), ref)
+
+
+def test_wna16_argument_errors(gpu):
+    import torch
+
+    from nnfusion_amd import _lib
+    from nnfusion_amd.ops import NnfQuant
+
+    lib = _lib.kernels()
+    buf = torch.zeros(1 << 16, dtype=torch.uint8, device=gpu)
+    p = buf.data_ptr()
+
+    def call(q, m=4, n=64, k=256, a=p):
+        qp = None if q is None else ctypes.cast(ctypes.pointer(q), ctypes.c_void_p)
+        return lib.nnf_wna16_gemm(None, a, p, p, p, m, n, k, qp, None, 0)
+
+    assert call(None) == -1
+    assert call(NnfQuant(4, 64, 8, None), a=None) == -1
+    assert call(NnfQuant(4, 64, 8, None), a=p + 2) == -1
+    assert call(NnfQuant(4, 64, 8, None), m=0) == -1
+    assert call(NnfQuant(3, 64, 8, None)) == -2      # bits
+    assert call(NnfQuant(4, 16, 8, None)) == -2      # group
+    assert call(NnfQuant(4, 64, 16, None)) == -2     # zero point outside 4 bits
+    assert call(NnfQuant(8, 64, 256, None)) == -2    # ... outside 8 bits
+    assert call(NnfQuant(8, 128, 0, None), k=192) == -2  # K % group
+    assert call(NnfQuant(8, 64, 255, None)) == 0
+    torch.cuda.synchronize()
