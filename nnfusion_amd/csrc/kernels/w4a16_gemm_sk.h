@@ -206,19 +206,24 @@ namespace nnf
 
     // Epilogue of one round (ROUND_TM blocks of 32 rows) of a wavefront's strip of a tile.  Lane (m = l32, h) holds, in
     // element e of MFMA tile (ii, j), column n = 8*(e/4) + 4*h + (e%4) of row ii*32 + m.  The sums are rounded (GATE:
-    // combined) in registers, turned through a private piece of LDS and finished as whole rows of the strip, 16 bytes
+    // combined) in registers, turned through a private piece of LDS (`region`: sk_region_bytes) and finished as whole rows of the strip, 16 bytes
     // (8 columns) per lane: bias, residual, store.  Rounding as the unfused graph would: the GEMM result to fp16 first,
     // then the element-wise operation in fp32, then fp16 again.
+    // bytes of LDS sk_finish_round uses per wavefront
+    template <int TM, int TN, bool GATE>
+    constexpr int sk_region_bytes()
+    {
+        return (TM >= 2 ? 2 : 1) * 32 * ((GATE ? TN / 2 : TN) * 64 + 16);
+    }
+
     template <int TM, int TN, bool GATE, bool BIAS, bool RESID, bool RMS>
     __device__ __forceinline__ void sk_finish_round(const SkGemmParams& p, const floatx16 (&c)[TM >= 2 ? 2 : 1][TN], int r, int m0, int n0,
-                                                    uint8_t* staging, int wave, int lane)
+                                                    uint8_t* region, int wave, int lane)
     {
         constexpr int OUT_TN = GATE ? TN / 2 : TN;
         constexpr int ROUND_TM = TM >= 2 ? 2 : 1;
         constexpr int PITCH = OUT_TN * 64 + 16; // bytes per staged row (padding spreads the banks)
-        constexpr int REGION = ROUND_TM * 32 * PITCH;
         constexpr int LANES_PER_ROW = OUT_TN * 4, ROWS_PER_READ = 64 / LANES_PER_ROW;
-        uint8_t* region = staging + wave * REGION;
         const int l32 = lane & 31, h = lane >> 5;
         const int n_wave = n0 + wave * (OUT_TN * 32);
         const int piece = lane % LANES_PER_ROW;
@@ -741,7 +746,7 @@ namespace nnf
 #pragma unroll
                         for (int j = 0; j < TN; ++j)
                             c[ii][j] = acc[r * ROUND_TM + ii][j];
-                    sk_finish_round<TM, TN, GATE, BIAS, RESID, RMS>(p, c, r, m0, n0, smem, wave, lane);
+                    sk_finish_round<TM, TN, GATE, BIAS, RESID, RMS>(p, c, r, m0, n0, smem + wave * sk_region_bytes<TM, TN, GATE>(), wave, lane);
                     __builtin_amdgcn_sched_barrier(0); // (one round at a time: few registers)
                 }
             }
@@ -751,20 +756,22 @@ namespace nnf
     }
 
     // Adds the parts of the tiles that several workgroups of w4a16_gemm_sk_kernel worked on, in K order (so the result
-    // does not depend on timing), and runs the epilogue.  One workgroup per tile and round of two 32-row blocks; a
-    // workgroup whose tile had a single owner has nothing to do.  `gemm_grid`: workgroups of the GEMM launch.
+    // does not depend on timing), and runs the epilogue.  The strips of the GEMM's four wavefronts are independent of one
+    // another here: one workgroup of a single wavefront per tile, block of 32 rows and strip (a few dozen tiles
+    // then still spread over all CUs); one whose tile had a single owner has nothing to do.  `gemm_grid`: workgroups of
+    // the GEMM launch.
     template <int TM, int TN, bool GATE, bool BIAS, bool RESID, bool RMS>
-    __global__ __launch_bounds__(256) void w4a16_gemm_sk_fixup_kernel(SkGemmParams p, int gemm_grid)
+    __global__ __launch_bounds__(64) void w4a16_gemm_sk_fixup_kernel(SkGemmParams p, int gemm_grid)
     {
         using namespace gemm_sk;
         using T = Tile<TM, TN>;
-        constexpr int ROUND_TM = TM >= 2 ? 2 : 1;
-        constexpr int ROUNDS = TM / ROUND_TM;
+        constexpr int ROUND_TM = 1, ROUNDS = TM; // (the epilogue routine of a tile one block high)
         constexpr int BN_OUT = GATE ? T::BN / 2 : T::BN;
-        __shared__ __attribute__((aligned(16))) uint8_t stage[WAVES * ROUND_TM * 32 * (TN * 64 + 16)];
-        const int tid = threadIdx.x, lane = tid & 63;
-        const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-        const int tile = (int)blockIdx.x / ROUNDS, r = (int)blockIdx.x % ROUNDS;
+        __shared__ __attribute__((aligned(16))) uint8_t stage[ROUND_TM * 32 * (TN * 64 + 16)];
+        const int lane = threadIdx.x;
+        const int wave = (int)blockIdx.x % WAVES; // the strip: what wavefront `wave` of the GEMM's workgroup parked
+        const int tid = wave * 64 + lane;
+        const int tile = (int)blockIdx.x / (WAVES * ROUNDS), r = ((int)blockIdx.x / WAVES) % ROUNDS;
         const int SS = p.supersteps;
         const long long t0 = (long long)tile * SS;
         const int v_first = owner_of_unit(t0, p.units, gemm_grid);
@@ -793,12 +800,13 @@ namespace nnf
 #pragma unroll
                 for (int e = 0; e < 16; ++e)
                     c[ii][j][e] = 0.f;
-        // parts in K order, four at a time in flight
-        for (int sg0 = 0; sg0 < n_seg; sg0 += 4)
+        // parts in K order, eight at a time in flight
+        constexpr int D = 8;
+        for (int sg0 = 0; sg0 < n_seg; sg0 += D)
         {
-            floatx4 x[4][ROUND_TM][TN][4];
+            floatx4 x[D][ROUND_TM][TN][4];
 #pragma unroll
-            for (int d = 0; d < 4; ++d)
+            for (int d = 0; d < D; ++d)
             {
                 const int sg = min(sg0 + d, n_seg - 1);
                 const float* theirs = p.partial +
@@ -814,7 +822,7 @@ namespace nnf
                                 *reinterpret_cast<const floatx4*>(theirs + (size_t)((((r * ROUND_TM + ii) * TN + j) * 4 + q) * THREADS * 4));
             }
 #pragma unroll
-            for (int d = 0; d < 4; ++d)
+            for (int d = 0; d < D; ++d)
                 if (sg0 + d < n_seg)
                 {
 #pragma unroll
@@ -831,6 +839,6 @@ namespace nnf
                             }
                 }
         }
-        sk_finish_round<TM, TN, GATE, BIAS, RESID, RMS>(p, c, r, m0, n0, stage, wave, lane);
+        sk_finish_round<1, TN, GATE, BIAS, RESID, RMS>(p, c, r, m0, n0, stage, wave, lane);
     }
 } // namespace nnf

@@ -26,9 +26,9 @@ namespace nnf
             if (e != hipSuccess || !p.partial)
                 return e;
             // tiles shared by several workgroups: their parts are added and finished by a second launch
-            constexpr int ROUNDS = TM >= 2 ? TM / 2 : 1;
-            hipLaunchKernelGGL((w4a16_gemm_sk_fixup_kernel<TM, TN, GATE, BIAS, RESID, RMS>), dim3(p.tiles_m * p.tiles_n * ROUNDS),
-                               dim3(THREADS), 0, stream, p, grid);
+            constexpr int ROUNDS = TM; // blocks of 32 rows
+            hipLaunchKernelGGL((w4a16_gemm_sk_fixup_kernel<TM, TN, GATE, BIAS, RESID, RMS>), dim3(p.tiles_m * p.tiles_n * ROUNDS * WAVES),
+                               dim3(64), 0, stream, p, grid);
             return hipGetLastError();
         }
 

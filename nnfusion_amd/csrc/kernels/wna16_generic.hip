@@ -7,8 +7,9 @@
 // (src/nnfusion/core/kernels/cpu/reference/kernels.cpp:601-623: integer subtract of the offset, cast, multiply by
 // the scale); the kernels in w4a16_*.hip serve the one combination the benchmark uses (4 bits, groups of 128, a
 // scalar zero point) as fast as the hardware allows, these two serve every other one correctly and simply:
-//   * wna16_gemv_kernel (M <= 16): a wavefront per weight row, a lane dequantises eight weights at a time to fp32
-//     ((q - z) * s, as the oracle's weights) and multiplies them with the eight activations of every row;
+//   * wna16_gemv_kernel (M <= 16): a wavefront per block of four weight rows; a lane turns 16 bytes of weights into the exact
+//     integers q - z in fp16, multiplies them with the activations of every row (v_dot2_f32_f16, fp32 sums) and applies
+//     the group's scale to the sum over its piece of the group;
 //   * wna16_tile_kernel (any M): 64 x 64 output tiles, four wavefronts of 32 x 32 (v_mfma_f32_32x32x16_f16), K steps of
 //     32: the weights of a step are dequantised to fp16((q - z) * s) on their way into LDS (what the tile GEMM's
 //     unpacking produces as well), the next step's operands are fetched into registers while this step's MFMAs run.
@@ -65,55 +66,140 @@ namespace nnf
         }
     } // namespace
 
-    // grid: any; each wavefront walks the rows n = its number, + the number of wavefronts, ...
+    // The exact integers (q - z) of eight weights as four fp16 pairs (|q - z| <= 255), by the offset trick of dequant8
+    // (nnf_device.h): a byte or nibble placed in the mantissa of 1024.0 is 1024 + q, and subtracting 1024 + z is exact.
+    // 4 bits: `w` holds the eight, pairs come out as (0,4) (1,5) (2,6) (3,7); 8 bits: `w` then `w_hi`, pairs in order.
     template <int BITS>
+    struct ExactWeights
+    {
+        DequantConst c4;
+        half2_t c8;
+        __device__ __forceinline__ explicit ExactWeights(int z)
+        {
+            if constexpr (BITS == 4)
+                c4 = make_dequant_const(z);
+            else
+            {
+                const half_t c = (half_t)(-(1024.0f + (float)z));
+                c8 = half2_t{c, c};
+            }
+        }
+        __device__ __forceinline__ void operator()(uint32_t w, uint32_t w_hi, half2_t (&out)[4]) const
+        {
+            if constexpr (BITS == 4)
+                dequant8(w, c4, out);
+            else
+            {
+                // v_perm_b32(S0, S1, sel): selectors 0-3 pick bytes of S1, 4-7 of S0
+                out[0] = as_half2(__builtin_amdgcn_perm(0x64646464u, w, 0x04010400u)) + c8;
+                out[1] = as_half2(__builtin_amdgcn_perm(0x64646464u, w, 0x04030402u)) + c8;
+                out[2] = as_half2(__builtin_amdgcn_perm(0x64646464u, w_hi, 0x04010400u)) + c8;
+                out[3] = as_half2(__builtin_amdgcn_perm(0x64646464u, w_hi, 0x04030402u)) + c8;
+            }
+        }
+    };
+
+    // grid: any; each wavefront walks blocks of R consecutive rows (R x its number, + R x the number of wavefronts, ...);
+    // a lane takes 16 bytes of each of the R rows per pass over K (32 or 16 weights, inside one group): the sum of
+    // a x (q - z) over them (v_dot2_f32_f16 on exact operands) times the group's scale is added to the lane's fp32 sums.
+    // The activations a lane meets are fetched once per pass for all R rows.  MB: upper bound of M.
+    template <int BITS, int R, int MB>
     __global__ __launch_bounds__(256) void wna16_gemv_kernel(const half_t* __restrict__ A, const uint8_t* __restrict__ Wq,
                                                              const half_t* __restrict__ S, half_t* __restrict__ Y, int M, int N,
                                                              int K, QuantArgs qa)
     {
+        constexpr int WPL = 128 / BITS; // weights per lane and pass
         const int lane = threadIdx.x & 63;
         const int wave = (int)blockIdx.x * 4 + (threadIdx.x >> 6), n_waves = (int)gridDim.x * 4;
         const int G = K >> qa.group_shift;
         const size_t row_bytes = (size_t)K * BITS / 8;
-        for (int n = wave; n < N; n += n_waves)
+        for (int n = wave * R; n < N; n += n_waves * R)
         {
-            float acc[16];
+            int row[R]; // (rows past the end of a ragged N are computed on the last row and dropped)
+            float acc[MB][R];
 #pragma unroll
-            for (int m = 0; m < 16; ++m)
-                acc[m] = 0.f;
-            const uint8_t* row = Wq + (size_t)n * row_bytes;
-            for (int k = lane * 8; k < K; k += 64 * 8)
+            for (int r = 0; r < R; ++r)
             {
-                int q[8];
-                load_q8<BITS>(row, k, q);
-                const int g = k >> qa.group_shift; // eight consecutive weights never straddle a group (a multiple of 32)
-                const int z = zero_point_of<BITS>(qa, n, g);
-                const float s = (float)S[(size_t)n * G + g];
-                float w[8];
+                row[r] = min(n + r, N - 1);
 #pragma unroll
-                for (int i = 0; i < 8; ++i)
-                    w[i] = (float)(q[i] - z) * s;
+                for (int m = 0; m < MB; ++m)
+                    acc[m][r] = 0.f;
+            }
+            for (int k = lane * WPL; k < K; k += 64 * WPL)
+            {
+                const int g = k >> qa.group_shift;
+                uintx4 w[R];
+                float sc[R];
+                int z[R];
 #pragma unroll
-                for (int m = 0; m < 16; ++m)
-                    if (m < M)
+                for (int r = 0; r < R; ++r)
+                {
+                    w[r] = *reinterpret_cast<const uintx4*>(Wq + (size_t)row[r] * row_bytes + (size_t)k * BITS / 8);
+                    z[r] = zero_point_of<BITS>(qa, row[r], g);
+                    sc[r] = (float)S[(size_t)row[r] * G + g];
+                }
+                float part[MB][R];
+#pragma unroll
+                for (int m = 0; m < MB; ++m)
+#pragma unroll
+                    for (int r = 0; r < R; ++r)
+                        part[m][r] = 0.f;
+#pragma unroll
+                for (int p = 0; p < WPL / 8; ++p)
+                {
+                    half2_t v[R][4];
+#pragma unroll
+                    for (int r = 0; r < R; ++r)
                     {
-                        const half8_t a = *reinterpret_cast<const half8_t*>(A + (size_t)m * K + k);
-                        float t = acc[m];
-#pragma unroll
-                        for (int i = 0; i < 8; ++i)
-                            t = __builtin_fmaf((float)a[i], w[i], t);
-                        acc[m] = t;
+                        const ExactWeights<BITS> exact(z[r]);
+                        if constexpr (BITS == 4)
+                            exact(w[r][p], 0u, v[r]);
+                        else
+                            exact(w[r][2 * p], w[r][2 * p + 1], v[r]);
                     }
+#pragma unroll
+                    for (int m = 0; m < MB; ++m)
+                        if (m < M)
+                        {
+                            uintx4 a = *reinterpret_cast<const uintx4*>(A + (size_t)m * K + k + 8 * p);
+                            if constexpr (BITS == 4)
+                                a = permute_a8(a);
+#pragma unroll
+                            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                                for (int r = 0; r < R; ++r)
+                                    part[m][r] = dot2(as_half2(a[i]), v[r][i], part[m][r]);
+                        }
+                }
+#pragma unroll
+                for (int m = 0; m < MB; ++m)
+#pragma unroll
+                    for (int r = 0; r < R; ++r)
+                        acc[m][r] = __builtin_fmaf(part[m][r], sc[r], acc[m][r]);
             }
 #pragma unroll
-            for (int m = 0; m < 16; ++m)
+            for (int m = 0; m < MB; ++m)
                 if (m < M)
                 {
-                    const float t = wave_sum(acc[m]);
-                    if (lane == 0)
-                        Y[(size_t)m * N + n] = (half_t)t;
+#pragma unroll
+                    for (int r = 0; r < R; ++r)
+                    {
+                        const float t = wave_sum(acc[m][r]);
+                        if (lane == 0 && n + r < N)
+                            Y[(size_t)m * N + n + r] = (half_t)t;
+                    }
                 }
         }
+    }
+
+    template <int BITS, int R, int MB>
+    void launch_wna16_gemv(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M, int N, int K,
+                           const QuantArgs& qa, int num_cu)
+    {
+        // enough wavefronts to cover the blocks of rows once, at most eight workgroups of four per CU
+        const int want = (N + 4 * R - 1) / (4 * R), cap = num_cu * 8;
+        hipLaunchKernelGGL((wna16_gemv_kernel<BITS, R, MB>), dim3((unsigned)(want < cap ? want : cap)), dim3(256), 0, stream,
+                           (const half_t*)A, (const uint8_t*)Wq, (const half_t*)S, (half_t*)Y, M, N, K, qa);
     }
 
     // one workgroup of four wavefronts per 64 x 64 output tile (blockIdx.x: column tile, blockIdx.y: row tile)
@@ -208,15 +294,24 @@ namespace nnf
         qa.zp_stride = (K / group * bits + 7) / 8;
         if (M <= 16)
         {
-            // enough wavefronts to cover the rows once, at most eight workgroups of four per CU
-            const int want = (N + 3) / 4, cap = num_cu * 8;
-            const dim3 grid((unsigned)(want < cap ? want : cap));
             if (bits == 4)
-                hipLaunchKernelGGL(wna16_gemv_kernel<4>, grid, dim3(256), 0, stream, (const half_t*)A, (const uint8_t*)Wq,
-                                   (const half_t*)S, (half_t*)Y, M, N, K, qa);
+            {
+                if (M == 1)
+                    launch_wna16_gemv<4, 4, 1>(stream, A, Wq, S, Y, M, N, K, qa, num_cu);
+                else if (M <= 4)
+                    launch_wna16_gemv<4, 4, 4>(stream, A, Wq, S, Y, M, N, K, qa, num_cu);
+                else
+                    launch_wna16_gemv<4, 4, 16>(stream, A, Wq, S, Y, M, N, K, qa, num_cu);
+            }
             else
-                hipLaunchKernelGGL(wna16_gemv_kernel<8>, grid, dim3(256), 0, stream, (const half_t*)A, (const uint8_t*)Wq,
-                                   (const half_t*)S, (half_t*)Y, M, N, K, qa);
+            {
+                if (M == 1)
+                    launch_wna16_gemv<8, 4, 1>(stream, A, Wq, S, Y, M, N, K, qa, num_cu);
+                else if (M <= 4)
+                    launch_wna16_gemv<8, 4, 4>(stream, A, Wq, S, Y, M, N, K, qa, num_cu);
+                else
+                    launch_wna16_gemv<8, 4, 16>(stream, A, Wq, S, Y, M, N, K, qa, num_cu);
+            }
             return hipGetLastError();
         }
         const dim3 grid((unsigned)((N + 63) / 64), (unsigned)((M + 63) / 64));
