@@ -56,7 +56,7 @@ SMALL_BATCHES = (2, 4, 8, 16)         # the sweep's shapes with a few rows
 # the fp16 x int-N product with other block parameters (bits, group, zero point per (row, group)?) than the benchmark's,
 # on the two plain kernels that serve them, at N = K = GEMM_NK
 WNA16_CASES = ((8, 128, False), (4, 64, True))
-WNA16_MS = (1, 4096)
+WNA16_MS = (1, 16, 4096)
 MLP_HI = (4096, 11008)                # configs[4]: hidden and intermediate size
 MLP_MS = (1, 16, 256)                 # ... at M = 256; the same block at decode sizes beside it
 
@@ -70,10 +70,12 @@ DOMINANT_KERNEL = {
     "w8a8_gemm_N8192_K8192.M32": "nnf::w8a8_mrows_kernel",
     "w8a8_gemm_N8192_K8192.M512": "nnf::w8a8_gemm_dl_kernel (128 x 128 tiles)",
     "w8a8_gemm_N8192_K8192.M4096": "nnf::w8a8_gemm_dl_kernel (256 x 256 tiles)",
-    "wna16_b8_g128_zp_scalar_N8192_K8192.M1": "nnf::wna16_gemv_kernel<8>",
-    "wna16_b8_g128_zp_scalar_N8192_K8192.M4096": "nnf::wna16_tile_kernel<8>",
-    "wna16_b4_g64_zp_tensor_N8192_K8192.M1": "nnf::wna16_gemv_kernel<4>",
-    "wna16_b4_g64_zp_tensor_N8192_K8192.M4096": "nnf::wna16_tile_kernel<4>",
+    "wna16_b8_g128_zp_scalar_N8192_K8192.M1": "nnf::wna16_gemv_kernel<8, 4, 1>",
+    "wna16_b8_g128_zp_scalar_N8192_K8192.M16": "nnf::wna16_skinny_kernel<8, 2>",
+    "wna16_b8_g128_zp_scalar_N8192_K8192.M4096": "nnf::wna16_tile128_kernel<8>",
+    "wna16_b4_g64_zp_tensor_N8192_K8192.M1": "nnf::wna16_gemv_kernel<4, 4, 1>",
+    "wna16_b4_g64_zp_tensor_N8192_K8192.M16": "nnf::wna16_skinny_kernel<4, 2>",
+    "wna16_b4_g64_zp_tensor_N8192_K8192.M4096": "nnf::wna16_tile128_kernel<4>",
     "fused_mlp_M1_4096_11008": "rms_rstd_kernel + 2 x nnf::w4a16_gemv_rows_kernel (gate|up with SiLU, down with the residual)",
     "fused_mlp_M16_4096_11008": "rms_rstd_kernel + nnf::w4a16_mrows_kernel (gate|up) + w4a16_mrows_any_kernel over 3 ranges of K + "
                                 "splitk_reduce_kernel (down)",

@@ -143,8 +143,9 @@ int nnf_w4a16_gemm_variant(nnf_stream_t stream,
  *   zero_points != NULL : u8 [N, ceil(K/group * bits / 8)], one per (row, group); 4-bit ones packed two to a byte along
  *                         the groups of a row, even group in the low nibble
  * bits 4, group 128 and no zero-point tensor is nnf_w4a16_gemm itself (same kernels, same workspace); every other
- * combination (group 32 / 64 / 128, K a multiple of group) runs on two plain kernels: a wavefront per weight row for
- * M <= 16, 64 x 64 MFMA tiles above. */
+ * combination (group 32 / 64 / 128, K a multiple of group) runs on plain kernels of its own: a row-per-wavefront GEMV
+ * for M = 1, an MFMA kernel with the operands fetched straight into registers for 2 <= M <= 16, MFMA tiles through
+ * LDS above.  They need no workspace. */
 typedef struct nnf_quant
 {
     int bits;                /* 4 or 8 */

@@ -6,13 +6,16 @@
 // The reference's dequantize takes a scale and an offset per block of any shape
 // (src/nnfusion/core/kernels/cpu/reference/kernels.cpp:601-623: integer subtract of the offset, cast, multiply by
 // the scale); the kernels in w4a16_*.hip serve the one combination the benchmark uses (4 bits, groups of 128, a
-// scalar zero point) as fast as the hardware allows, these two serve every other one correctly and simply:
-//   * wna16_gemv_kernel (M <= 16): a wavefront per block of four weight rows; a lane turns 16 bytes of weights into the exact
-//     integers q - z in fp16, multiplies them with the activations of every row (v_dot2_f32_f16, fp32 sums) and applies
-//     the group's scale to the sum over its piece of the group;
-//   * wna16_tile_kernel (any M): 64 x 64 output tiles, four wavefronts of 32 x 32 (v_mfma_f32_32x32x16_f16), K steps of
-//     32: the weights of a step are dequantised to fp16((q - z) * s) on their way into LDS (what the tile GEMM's
-//     unpacking produces as well), the next step's operands are fetched into registers while this step's MFMAs run.
+// scalar zero point) as fast as the hardware allows, these serve every other one correctly and simply:
+//   * wna16_gemv_kernel (M = 1): a wavefront per block of four weight rows; a lane turns 16 bytes of weights of each
+//     into the exact integers q - z in fp16, multiplies them with the activations (v_dot2_f32_f16, fp32 sums) and
+//     applies the group's scale to the sum over its piece of the group;
+//   * wna16_skinny_kernel (2 <= M <= 16): v_mfma_f32_16x16x32_f16, activations and weights fetched straight into the
+//     operand registers, eight wavefronts share the K range of two tiles of 16 weight rows;
+//   * wna16_tile_kernel / wna16_tile128_kernel (M > 16): 64 x 64 or, once they fill the chip, 128 x 128 output tiles on
+//     v_mfma_f32_32x32x16_f16, K steps of 32 through LDS, the next step's operands fetched into registers while this
+//     step's MFMAs run.
+// The MFMA kernels dequantise to fp16((q - z) * s) (what the specialised tile GEMM's unpacking produces as well).
 #include "nnf_device.h"
 #include "nnf_launch.h"
 
@@ -202,6 +205,114 @@ namespace nnf
                            (const half_t*)A, (const uint8_t*)Wq, (const half_t*)S, (half_t*)Y, M, N, K, qa);
     }
 
+    // 2 <= M <= 16 on the matrix cores (v_mfma_f32_16x16x32_f16: activations as the 16-row operand, 16 weight rows as
+    // the other).  A workgroup of eight wavefronts walks blocks of NT tiles of 16 weight rows; the wavefronts take the
+    // chunks of K in turn (a chunk: 4 x 16 bytes of each weight row, 128 or 64 values of K): lane (row l % 16, quarter
+    // l / 16) fetches 16 bytes of its row of every tile and the activations of the same K positions of row l % 16 (once
+    // for the NT tiles) straight into the MFMA operand registers (the next chunk's while this one is computed),
+    // dequantises to fp16((q - z) * s) (the exact integers by the offset trick, one rounding in the multiply) and issues
+    // one MFMA per tile and eight values of K.  The eight partial 16 x 16 tiles of every tile meet in LDS.
+    constexpr int SKINNY_WAVES = 8;
+    template <int BITS, int NT>
+    __global__ __launch_bounds__(SKINNY_WAVES * 64) void wna16_skinny_kernel(const half_t* __restrict__ A,
+                                                                             const uint8_t* __restrict__ Wq,
+                                                                             const half_t* __restrict__ S, half_t* __restrict__ Y,
+                                                                             int M, int N, int K, QuantArgs qa)
+    {
+        constexpr int WPL = 128 / BITS;  // weights per lane, tile and chunk
+        constexpr int PIECES = WPL / 8;  // MFMAs per tile and chunk
+        constexpr int CHUNK = 4 * WPL;   // values of K per chunk
+        __shared__ __attribute__((aligned(16))) floatx4 red[SKINNY_WAVES][NT][64];
+        const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+        const int col = lane & 15, kq = lane >> 4;
+        const int G = K >> qa.group_shift;
+        const size_t row_bytes = (size_t)K * BITS / 8;
+        const int n_chunks = (K + CHUNK - 1) / CHUNK;
+        const half_t* a_row = A + (size_t)min(col, M - 1) * K; // (rows past M repeat the last one and are dropped)
+        struct Operands
+        {
+            uintx4 w[NT], a[PIECES];
+            float s[NT];
+            int z[NT];
+        };
+        for (int block = (int)blockIdx.x; block * (16 * NT) < N; block += (int)gridDim.x)
+        {
+            int n[NT]; // (rows past N repeat the last one and are dropped)
+#pragma unroll
+            for (int t = 0; t < NT; ++t)
+                n[t] = min((block * NT + t) * 16 + col, N - 1);
+            auto fetch = [&](int c, Operands& o) {
+                // a lane past the end of K (the last chunk of a K that is not a multiple of it) repeats the row's last
+                // piece with a scale of zero
+                const int k_raw = c * CHUNK + kq * WPL;
+                const int k = min(k_raw, K - WPL);
+                const int g = k >> qa.group_shift;
+#pragma unroll
+                for (int t = 0; t < NT; ++t)
+                {
+                    o.w[t] = *reinterpret_cast<const uintx4*>(Wq + (size_t)n[t] * row_bytes + (size_t)k * BITS / 8);
+                    o.z[t] = zero_point_of<BITS>(qa, n[t], g);
+                    o.s[t] = k_raw < K ? (float)S[(size_t)n[t] * G + g] : 0.f;
+                }
+#pragma unroll
+                for (int p = 0; p < PIECES; ++p)
+                    o.a[p] = *reinterpret_cast<const uintx4*>(a_row + k + 8 * p);
+            };
+            floatx4 acc[NT];
+#pragma unroll
+            for (int t = 0; t < NT; ++t)
+                acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+            Operands cur, nxt;
+            if (wave < n_chunks)
+                fetch(wave, cur);
+            for (int c = wave; c < n_chunks; c += SKINNY_WAVES)
+            {
+                if (c + SKINNY_WAVES < n_chunks)
+                    fetch(c + SKINNY_WAVES, nxt);
+#pragma unroll
+                for (int p = 0; p < PIECES; ++p)
+                {
+                    uintx4 a = cur.a[p];
+                    if constexpr (BITS == 4)
+                        a = permute_a8(a); // the pair order of the unpacked nibbles
+#pragma unroll
+                    for (int t = 0; t < NT; ++t)
+                    {
+                        const ExactWeights<BITS> exact(cur.z[t]);
+                        const half_t sh = (half_t)cur.s[t];
+                        const half2_t s2 = half2_t{sh, sh};
+                        half2_t v[4];
+                        if constexpr (BITS == 4)
+                            exact(cur.w[t][p], 0u, v);
+                        else
+                            exact(cur.w[t][2 * p], cur.w[t][2 * p + 1], v);
+                        const uintx4 b = {as_u32(v[0] * s2), as_u32(v[1] * s2), as_u32(v[2] * s2), as_u32(v[3] * s2)};
+                        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, a), __builtin_bit_cast(half8_t, b),
+                                                                        acc[t], 0, 0, 0);
+                    }
+                }
+                cur = nxt;
+            }
+            // D: lane (n = col, kq), element e: row m = 4 kq + e
+#pragma unroll
+            for (int t = 0; t < NT; ++t)
+                red[wave][t][lane] = acc[t];
+            __syncthreads();
+            for (int o = tid; o < NT * 256; o += SKINNY_WAVES * 64)
+            {
+                const int l = o & 63, e = (o >> 6) & 3, t = o >> 8;
+                float sum = 0.f;
+#pragma unroll
+                for (int w = 0; w < SKINNY_WAVES; ++w)
+                    sum += red[w][t][l][e];
+                const int m = 4 * (l >> 4) + e, nn = (block * NT + t) * 16 + (l & 15);
+                if (m < M && nn < N)
+                    Y[(size_t)m * N + nn] = (half_t)sum;
+            }
+            __syncthreads(); // the partial tiles are read before the next block's are written
+        }
+    }
+
     // one workgroup of four wavefronts per 64 x 64 output tile (blockIdx.x: column tile, blockIdx.y: row tile)
     template <int BITS>
     __global__ __launch_bounds__(256) void wna16_tile_kernel(const half_t* __restrict__ A, const uint8_t* __restrict__ Wq,
@@ -277,6 +388,157 @@ namespace nnf
         }
     }
 
+    // 128 x 128 output tiles for products large enough to fill the chip with them: four wavefronts of 64 x 64 (2 x 2 MFMA
+    // tiles each), K steps of 32 through two LDS buffers (the next step's operands are fetched into registers ahead of
+    // this step's MFMAs and stored behind them: one barrier per step).  A thread stages 16 activations of two rows and
+    // dequantises 16 weights of one row per step: the exact integers q - z in fp16 (offset trick) times the scale, one
+    // rounding, which is fp16((q - z) * s).  Tiles are numbered in groups of eight tile rows, tile row fastest, so that
+    // the workgroups in flight together share activations and weights in the caches.
+    template <int BITS>
+    __global__ __launch_bounds__(256) void wna16_tile128_kernel(const half_t* __restrict__ A, const uint8_t* __restrict__ Wq,
+                                                                const half_t* __restrict__ S, half_t* __restrict__ Y, int M, int N,
+                                                                int K, int tiles_m, int tiles_n, QuantArgs qa)
+    {
+        constexpr int PITCH = 40;              // halves per staged row: 32 of K + 8 of padding
+        constexpr int OPERAND = 128 * PITCH;   // halves of one staged operand
+        __shared__ __attribute__((aligned(16))) half_t lds[2][2][OPERAND]; // [buffer][A, W]
+        const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+        int tm, tn;
+        {
+            constexpr int GM = 8;
+            const int tile = (int)blockIdx.x, per_group = GM * tiles_n;
+            const int g = tile / per_group, first_m = g * GM, gm = min(GM, tiles_m - first_m), rr = tile - g * per_group;
+            tm = first_m + rr % gm;
+            tn = rr / gm;
+        }
+        const int m0 = tm * 128, n0 = tn * 128;
+        const int G = K >> qa.group_shift;
+        const size_t row_bytes = (size_t)K * BITS / 8;
+        // staging: activations: piece tid % 4 (8 halves) of rows tid / 4 and 64 + tid / 4; weights: half tid % 2 (16 of the
+        // step's 32) of row tid / 2
+        const int a_row = tid >> 2, a_k = (tid & 3) * 8;
+        const bool a_ok0 = m0 + a_row < M, a_ok1 = m0 + 64 + a_row < M;
+        const half_t* a_src0 = A + (size_t)min(m0 + a_row, M - 1) * K + a_k;
+        const half_t* a_src1 = A + (size_t)min(m0 + 64 + a_row, M - 1) * K + a_k;
+        const int w_row = tid >> 1, w_k = (tid & 1) * 16;
+        const int w_n = min(n0 + w_row, N - 1);
+        const bool w_ok = n0 + w_row < N;
+        const uint8_t* w_src = Wq + (size_t)w_n * row_bytes;
+        // fragments: wavefront (wm, wn) owns rows [64 wm, +64) x columns [64 wn, +64)
+        const int wm = wave >> 1, wn = wave & 1;
+        const int f_row = lane & 31, f_k = (lane >> 5) * 8;
+
+        uintx4 a_next0 = {0u, 0u, 0u, 0u}, a_next1 = {0u, 0u, 0u, 0u}, w_next = {0u, 0u, 0u, 0u};
+        float s_next = 0.f;
+        int z_next = 0;
+        auto fetch = [&](int k0) {
+            if (a_ok0)
+                a_next0 = *reinterpret_cast<const uintx4*>(a_src0 + k0);
+            if (a_ok1)
+                a_next1 = *reinterpret_cast<const uintx4*>(a_src1 + k0);
+            const int k = k0 + w_k;
+            if constexpr (BITS == 4)
+            {
+                const uintx2 w = *reinterpret_cast<const uintx2*>(w_src + (k >> 1));
+                w_next.x = w.x, w_next.y = w.y;
+            }
+            else
+                w_next = *reinterpret_cast<const uintx4*>(w_src + k);
+            const int g = k >> qa.group_shift;
+            z_next = zero_point_of<BITS>(qa, w_n, g);
+            s_next = w_ok ? (float)S[(size_t)w_n * G + g] : 0.f; // (columns past N: weights of zero)
+        };
+        auto stage = [&](int buf) {
+            *reinterpret_cast<uintx4*>(&lds[buf][0][a_row * PITCH + a_k]) = a_next0; // rows past M stay zero
+            *reinterpret_cast<uintx4*>(&lds[buf][0][(64 + a_row) * PITCH + a_k]) = a_next1;
+            const ExactWeights<BITS> exact(z_next);
+            const half_t sh = (half_t)s_next;
+            const half2_t s2 = half2_t{sh, sh};
+            uintx4 lo, hi; // the 16 weights in order of k, as fp16
+            if constexpr (BITS == 4)
+            {
+                half2_t v[4];
+                exact(w_next.x, 0u, v); // pairs (0,4) (1,5) (2,6) (3,7) -> order of k
+                for (int i = 0; i < 4; ++i)
+                    v[i] = v[i] * s2;
+                lo.x = __builtin_amdgcn_perm(as_u32(v[1]), as_u32(v[0]), 0x05040100u);
+                lo.y = __builtin_amdgcn_perm(as_u32(v[3]), as_u32(v[2]), 0x05040100u);
+                lo.z = __builtin_amdgcn_perm(as_u32(v[1]), as_u32(v[0]), 0x07060302u);
+                lo.w = __builtin_amdgcn_perm(as_u32(v[3]), as_u32(v[2]), 0x07060302u);
+                exact(w_next.y, 0u, v);
+                for (int i = 0; i < 4; ++i)
+                    v[i] = v[i] * s2;
+                hi.x = __builtin_amdgcn_perm(as_u32(v[1]), as_u32(v[0]), 0x05040100u);
+                hi.y = __builtin_amdgcn_perm(as_u32(v[3]), as_u32(v[2]), 0x05040100u);
+                hi.z = __builtin_amdgcn_perm(as_u32(v[1]), as_u32(v[0]), 0x07060302u);
+                hi.w = __builtin_amdgcn_perm(as_u32(v[3]), as_u32(v[2]), 0x07060302u);
+            }
+            else
+            {
+                half2_t v[4];
+                exact(w_next.x, w_next.y, v);
+                lo = uintx4{as_u32(v[0] * s2), as_u32(v[1] * s2), as_u32(v[2] * s2), as_u32(v[3] * s2)};
+                exact(w_next.z, w_next.w, v);
+                hi = uintx4{as_u32(v[0] * s2), as_u32(v[1] * s2), as_u32(v[2] * s2), as_u32(v[3] * s2)};
+            }
+            *reinterpret_cast<uintx4*>(&lds[buf][1][w_row * PITCH + w_k]) = lo;
+            *reinterpret_cast<uintx4*>(&lds[buf][1][w_row * PITCH + w_k + 8]) = hi;
+        };
+        floatx16 acc[2][2];
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int e = 0; e < 16; ++e)
+                    acc[i][j][e] = 0.f;
+        fetch(0);
+        stage(0);
+        __syncthreads();
+        int buf = 0;
+        for (int k0 = 0; k0 < K; k0 += 32)
+        {
+            const bool more = k0 + 32 < K;
+            if (more)
+                fetch(k0 + 32);
+#pragma unroll
+            for (int kk = 0; kk < 2; ++kk)
+            {
+                half8_t fa[2], fw[2];
+#pragma unroll
+                for (int i = 0; i < 2; ++i)
+                {
+                    fa[i] = *reinterpret_cast<const half8_t*>(&lds[buf][0][(wm * 64 + i * 32 + f_row) * PITCH + kk * 16 + f_k]);
+                    fw[i] = *reinterpret_cast<const half8_t*>(&lds[buf][1][(wn * 64 + i * 32 + f_row) * PITCH + kk * 16 + f_k]);
+                }
+#pragma unroll
+                for (int i = 0; i < 2; ++i)
+#pragma unroll
+                    for (int j = 0; j < 2; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[i], fw[j], acc[i][j], 0, 0, 0);
+            }
+            if (more)
+                stage(buf ^ 1); // last read a step ago, before the barrier at its end
+            __syncthreads();
+            buf ^= 1;
+        }
+        // D[m][n]: lane l holds column l % 32; element e is row 8 (e / 4) + 4 (l / 32) + e % 4
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+            {
+                const int n = n0 + wn * 64 + j * 32 + (lane & 31);
+#pragma unroll
+                for (int e = 0; e < 16; ++e)
+                {
+                    const int m = m0 + wm * 64 + i * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
+                    if (m < M && n < N)
+                        Y[(size_t)m * N + n] = (half_t)acc[i][j][e];
+                }
+            }
+    }
+
     bool wna16_supported(int M, int N, int K, int bits, int group)
     {
         return M > 0 && N > 0 && K > 0 && (bits == 4 || bits == 8) && (group == 32 || group == 64 || group == 128) && K % group == 0;
@@ -294,24 +556,35 @@ namespace nnf
         qa.zp_stride = (K / group * bits + 7) / 8;
         if (M <= 16)
         {
-            if (bits == 4)
+            if (M == 1)
             {
-                if (M == 1)
+                if (bits == 4)
                     launch_wna16_gemv<4, 4, 1>(stream, A, Wq, S, Y, M, N, K, qa, num_cu);
-                else if (M <= 4)
-                    launch_wna16_gemv<4, 4, 4>(stream, A, Wq, S, Y, M, N, K, qa, num_cu);
                 else
-                    launch_wna16_gemv<4, 4, 16>(stream, A, Wq, S, Y, M, N, K, qa, num_cu);
-            }
-            else
-            {
-                if (M == 1)
                     launch_wna16_gemv<8, 4, 1>(stream, A, Wq, S, Y, M, N, K, qa, num_cu);
-                else if (M <= 4)
-                    launch_wna16_gemv<8, 4, 4>(stream, A, Wq, S, Y, M, N, K, qa, num_cu);
-                else
-                    launch_wna16_gemv<8, 4, 16>(stream, A, Wq, S, Y, M, N, K, qa, num_cu);
+                return hipGetLastError();
             }
+            // blocks of two tiles of 16 rows, at most four workgroups per CU
+            const int blocks = (N + 31) / 32, cap = num_cu * 4;
+            const dim3 grid((unsigned)(blocks < cap ? blocks : cap));
+            if (bits == 4)
+                hipLaunchKernelGGL((wna16_skinny_kernel<4, 2>), grid, dim3(SKINNY_WAVES * 64), 0, stream, (const half_t*)A,
+                                   (const uint8_t*)Wq, (const half_t*)S, (half_t*)Y, M, N, K, qa);
+            else
+                hipLaunchKernelGGL((wna16_skinny_kernel<8, 2>), grid, dim3(SKINNY_WAVES * 64), 0, stream, (const half_t*)A,
+                                   (const uint8_t*)Wq, (const half_t*)S, (half_t*)Y, M, N, K, qa);
+            return hipGetLastError();
+        }
+        const int tiles_m = (M + 127) / 128, tiles_n = (N + 127) / 128;
+        if ((long long)tiles_m * tiles_n >= num_cu)
+        {
+            const dim3 grid128((unsigned)(tiles_m * tiles_n));
+            if (bits == 4)
+                hipLaunchKernelGGL(wna16_tile128_kernel<4>, grid128, dim3(256), 0, stream, (const half_t*)A, (const uint8_t*)Wq,
+                                   (const half_t*)S, (half_t*)Y, M, N, K, tiles_m, tiles_n, qa);
+            else
+                hipLaunchKernelGGL(wna16_tile128_kernel<8>, grid128, dim3(256), 0, stream, (const half_t*)A, (const uint8_t*)Wq,
+                                   (const half_t*)S, (half_t*)Y, M, N, K, tiles_m, tiles_n, qa);
             return hipGetLastError();
         }
         const dim3 grid((unsigned)((N + 63) / 64), (unsigned)((M + 63) / 64));

@@ -47,6 +47,8 @@ SHAPES = [
     (16, 4111, 4096), (2, 7, 384),
     # the tile kernel: one partial tile, ragged M and N, many tiles, a long K
     (17, 33, 128), (64, 64, 512), (100, 1000, 160), (300, 257, 2048), (128, 4096, 4096), (33, 520, 11008), (1024, 130, 384),
+    # enough 128 x 128 tiles to fill the chip: the larger tile kernel; ragged M and N, an odd number of groups
+    (2048, 2048, 512), (1100, 4100, 160), (4096, 1030, 384),
 ]
 
 
@@ -64,16 +66,16 @@ def test_wna16_matches_oracle(gpu, m, n, k, bits, group, zp_tensor):
     _check(_run(gpu, a, wq, s, bits, group, zp, zps), ref)
 
 
-@pytest.mark.parametrize("m", [4, 40])
+@pytest.mark.parametrize("m,n", [(4, 70), (40, 70), (2000, 2100)])
 @pytest.mark.parametrize("bits,group,zp_tensor", [(4, 32, True), (4, 64, False), (8, 64, True), (8, 128, False), (8, 32, True)])
-def test_one_hot_rows_return_the_dequantised_weights(gpu, m, bits, group, zp_tensor):
-    """A = e_k: 1 * w is exact in either kernel, so the output is fp16((q - z) * s) bit for bit; pins nibble and byte
-    order of weights and zero points and the block each scale belongs to, on the device."""
-    n, k = 70, 640
+def test_one_hot_rows_return_the_dequantised_weights(gpu, m, n, bits, group, zp_tensor):
+    """A = e_k: 1 * w is exact in every kernel (m = 2000: the 128 x 128 tiles), so the output is fp16((q - z) * s) bit for
+    bit; pins nibble and byte order of weights and zero points and the block each scale belongs to, on the device."""
+    k = 640
     _, wq, s, zps = _case(5, m, n, k, bits, group, zp_tensor)
     zp = 3 if bits == 4 else 200
     wd = oracle.dequantize_wn(wq, s, bits, group, zp=zp, zero_points=zps)
-    ks = [0, 1, 7, 8, 31, 32, 63, 64, 127, 128, 255, 256, 511, 512, 639][:m] if m <= 16 else list(range(0, 640, 16))
+    ks = [0, 1, 7, 8, 31, 32, 63, 64, 127, 128, 255, 256, 511, 512, 639][:m] if m <= 16 else [(7 * r) % k for r in range(min(m, 640))]
     a = np.zeros((m, k), np.float16)
     for r, kk in enumerate(ks):
         a[r, kk] = 1.0
