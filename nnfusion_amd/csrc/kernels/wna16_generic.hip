@@ -392,7 +392,7 @@ namespace nnf
     // tiles each), K steps of 32 through two LDS buffers (the next step's operands are fetched into registers ahead of
     // this step's MFMAs and stored behind them: one barrier per step).  A thread stages 16 activations of two rows and
     // dequantises 16 weights of one row per step: the exact integers q - z in fp16 (offset trick) times the scale, one
-    // rounding, which is fp16((q - z) * s).  Tiles are numbered in groups of eight tile rows, tile row fastest, so that
+    // rounding, which is fp16((q - z) * s).  Tiles are numbered in groups of four tile rows, tile row fastest, so that
     // the workgroups in flight together share activations and weights in the caches.
     template <int BITS>
     __global__ __launch_bounds__(256) void wna16_tile128_kernel(const half_t* __restrict__ A, const uint8_t* __restrict__ Wq,
@@ -405,8 +405,13 @@ namespace nnf
         const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
         int tm, tn;
         {
-            constexpr int GM = 8;
-            const int tile = (int)blockIdx.x, per_group = GM * tiles_n;
+            // workgroups go to the eight XCDs in turn: XCD x takes a contiguous run of tile numbers, so that what its
+            // workgroups in flight share stays in its own L2
+            constexpr int GM = 4;
+            const int total = tiles_m * tiles_n, per = total / 8, rem = total % 8;
+            const int xcd = (int)blockIdx.x % 8, i = (int)blockIdx.x / 8;
+            const int tile = (xcd < rem ? xcd * (per + 1) : rem * (per + 1) + (xcd - rem) * per) + i;
+            const int per_group = GM * tiles_n;
             const int g = tile / per_group, first_m = g * GM, gm = min(GM, tiles_m - first_m), rr = tile - g * per_group;
             tm = first_m + rr % gm;
             tn = rr / gm;
