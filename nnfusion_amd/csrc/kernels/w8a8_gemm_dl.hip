@@ -34,12 +34,13 @@ namespace nnf
     namespace q8dl
     {
         constexpr int BK = 64; // bytes (= int8 elements) of K per step
-        constexpr int THREADS = 512;
 
         template <int WM, int WN, int TM, int TN, int STAGES_>
         struct Tile
         {
-            static_assert(WM * WN == 8, "eight wavefronts per workgroup");
+            static constexpr int WAVES = WM * WN;
+            static_assert(WAVES == 8 || WAVES == 4, "eight wavefronts per workgroup, or four with one SIMD each");
+            static constexpr int THREADS = WAVES * 64;
             static constexpr int STAGES = STAGES_;
             static constexpr int BM = WM * TM * 32;
             static constexpr int BN = WN * TN * 32;
@@ -48,11 +49,11 @@ namespace nnf
             static constexpr int STAGE_BYTES = A_TILE_BYTES + W_TILE_BYTES;
             static constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
             // a wavefront-wide load covers 16 rows of 64 bytes; every wavefront issues the same number of loads
-            // (with fewer than 8 chunks two wavefronts fetch the same chunk into the same place)
+            // (with fewer chunks than wavefronts two wavefronts fetch the same chunk into the same place)
             static constexpr int A_CHUNKS = BM / 16;
             static constexpr int W_CHUNKS = BN / 16;
-            static constexpr int A_LOADS = A_CHUNKS >= 8 ? A_CHUNKS / 8 : 1;
-            static constexpr int W_LOADS = W_CHUNKS >= 8 ? W_CHUNKS / 8 : 1;
+            static constexpr int A_LOADS = A_CHUNKS >= WAVES ? A_CHUNKS / WAVES : 1;
+            static constexpr int W_LOADS = W_CHUNKS >= WAVES ? W_CHUNKS / WAVES : 1;
             static constexpr int TILE_LOADS = A_LOADS + W_LOADS;
         };
 
@@ -60,7 +61,7 @@ namespace nnf
     } // namespace q8dl
 
     template <int WM, int WN, int TM, int TN, int STAGES, bool RAW, bool SPLITK, int MINW>
-    __global__ __launch_bounds__(512, MINW) void w8a8_gemm_dl_kernel(Q8GemmParams p)
+    __global__ __launch_bounds__(WM * WN * 64, MINW) void w8a8_gemm_dl_kernel(Q8GemmParams p)
     {
         using namespace q8dl;
         using T = Tile<WM, WN, TM, TN, STAGES>;
@@ -193,12 +194,45 @@ namespace nnf
             unroll_for<0, TN>(
                 [&](auto j) { lds_read_b128_nowait<A_TILE_BYTES + decltype(j)::value * 2048>(bf[set][j], ww); });
         };
+        // read x of a set: the TM activation fragments, then the TN weight fragments
+        auto read_one_frag = [&](int stage, auto s_c, auto set_c, auto x_c) {
+            constexpr int s = decltype(s_c)::value, set = decltype(set_c)::value, x = decltype(x_c)::value;
+            const uint32_t off = (uint32_t)(stage * STAGE_BYTES);
+            if constexpr (x < TM)
+                lds_read_b128_nowait<x * 2048>(af[set][x], a_addr[s] + off);
+            else
+                lds_read_b128_nowait<A_TILE_BYTES + (x - TM) * 2048>(bf[set][x - TM], w_addr[s] + off);
+        };
+        // load x of a K step: the A_LOADS activation loads, then the W_LOADS weight loads
+        auto issue_one_load = [&](int kt, int stage, auto x_c) {
+            constexpr int x = decltype(x_c)::value;
+            uint8_t* base = smem + stage * STAGE_BYTES;
+            const int k0 = kt * BK;
+            if constexpr (x < A_LOADS)
+                __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1)))*)(a_src[x] + k0),
+                                                 (void __attribute__((address_space(3)))*)(base + a_chunk[x] * 1024), 16, 0, 0);
+            else
+                __builtin_amdgcn_global_load_lds(
+                    (const void __attribute__((address_space(1)))*)(w_src[x - A_LOADS] + k0),
+                    (void __attribute__((address_space(3)))*)(base + A_TILE_BYTES + w_chunk[x - A_LOADS] * 1024), 16, 0, 0);
+        };
         // the set is usable once at most `later` LDS reads issued after it are in flight
         auto wait_frags = [&](auto set_c, auto later_c) {
             constexpr int set = decltype(set_c)::value;
             lds_wait<decltype(later_c)::value>(af[set][0]);
             unroll_for<1, TM>([&](auto i) { lds_wait_also(af[set][i]); });
             unroll_for<0, TN>([&](auto j) { lds_wait_also(bf[set][j]); });
+        };
+        // MFMAs [FIRST, LAST) of a sub-step, numbered j * TM + i
+        auto mfma_range = [&](auto set_c, auto first_c, auto last_c) {
+            constexpr int set = decltype(set_c)::value;
+            unroll_for<decltype(first_c)::value, decltype(last_c)::value>([&](auto x_c) {
+                constexpr int j = decltype(x_c)::value / TM, i = decltype(x_c)::value % TM;
+                if (RAW || SPLITK)
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[set][i], bf[set][j], acc[i][j], 0, 0, 0);
+                else
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[set][j], af[set][i], acc[i][j], 0, 0, 0);
+            });
         };
         auto mfmas = [&](auto set_c) {
             constexpr int set = decltype(set_c)::value;
@@ -238,37 +272,70 @@ namespace nnf
             __builtin_amdgcn_s_barrier();
             read_frags(0, I0{}, I0{});
         }
+        constexpr int NM = TM * TN; // MFMAs per sub-step
         for (int kt = 0; kt < KT; ++kt)
         {
             __builtin_amdgcn_s_waitcnt(vmcnt_imm(WAIT_LOADS));
             __builtin_amdgcn_s_barrier();
+            if constexpr (AHEAD)
             {
-                // past the end: reload a valid tile into the free stage
+                // The fragments of sub-step 0 were read during the step before: the first MFMA goes out right behind the
+                // barrier, and everything else this step issues goes out one piece at a time between two MFMAs (it
+                // executes while the matrix core works): the LDS reads of sub-step 1 behind the first MFMAs of sub-step
+                // 0, this step's loads behind its later ones, the reads of the next step's sub-step 0 behind the first
+                // MFMAs of sub-step 1.
+                constexpr int HALF = NM / 2;
+                constexpr int RPM = (FRAG_READS + HALF - 1) / HALF, LPM = (TILE_LOADS + HALF - 1) / HALF;
                 int st = stage + STAGES - 1;
                 st = st >= STAGES ? st - STAGES : st;
-                issue_tile_loads(min(kt + STAGES - 1, KT - 1), st);
-            }
-            const int next_stage = stage + 1 == STAGES ? 0 : stage + 1;
-            if (!AHEAD)
-                read_frags(stage, I0{}, I0{});
-            read_frags(stage, I1{}, I1{});
-            wait_frags(I0{}, ONE_SET{});
-            __builtin_amdgcn_sched_barrier(0);
-            mfmas(I0{});
-            __builtin_amdgcn_sched_barrier(0);
-            if (AHEAD)
-            {
-                read_frags(next_stage, I0{}, I0{}); // after the last step: a stage nobody uses any more
-                wait_frags(I1{}, ONE_SET{});
+                const int kt_load = min(kt + STAGES - 1, KT - 1);
+                const int next_stage = stage + 1 == STAGES ? 0 : stage + 1;
+                wait_frags(I0{}, NONE{});
+                unroll_for<0, NM>([&](auto x_c) {
+                    constexpr int x = decltype(x_c)::value;
+                    __builtin_amdgcn_sched_barrier(0);
+                    mfma_range(I0{}, x_c, std::integral_constant<int, x + 1>{});
+                    __builtin_amdgcn_sched_barrier(0);
+                    if constexpr (x < HALF)
+                        unroll_for<x * RPM, (x + 1) * RPM < FRAG_READS ? (x + 1) * RPM : FRAG_READS>(
+                            [&](auto r_c) { read_one_frag(stage, I1{}, I1{}, r_c); });
+                    else
+                        unroll_for<(x - HALF) * LPM, (x - HALF + 1) * LPM < TILE_LOADS ? (x - HALF + 1) * LPM : TILE_LOADS>(
+                            [&](auto l_c) { issue_one_load(kt_load, st, l_c); });
+                });
+                __builtin_amdgcn_sched_barrier(0);
+                wait_frags(I1{}, NONE{});
+                unroll_for<0, NM>([&](auto x_c) {
+                    constexpr int x = decltype(x_c)::value;
+                    __builtin_amdgcn_sched_barrier(0);
+                    mfma_range(I1{}, x_c, std::integral_constant<int, x + 1>{});
+                    __builtin_amdgcn_sched_barrier(0);
+                    if constexpr (x < HALF) // (after the last step: a stage nobody uses any more)
+                        unroll_for<x * RPM, (x + 1) * RPM < FRAG_READS ? (x + 1) * RPM : FRAG_READS>(
+                            [&](auto r_c) { read_one_frag(next_stage, I0{}, I0{}, r_c); });
+                });
+                __builtin_amdgcn_sched_barrier(0);
+                stage = next_stage;
             }
             else
             {
+                // three stages: the fragments of a step are read behind its barrier (past the end: a valid tile is
+                // reloaded into the free stage)
+                int st = stage + STAGES - 1;
+                st = st >= STAGES ? st - STAGES : st;
+                issue_tile_loads(min(kt + STAGES - 1, KT - 1), st);
+                read_frags(stage, I0{}, I0{});
+                read_frags(stage, I1{}, I1{});
+                wait_frags(I0{}, ONE_SET{});
+                __builtin_amdgcn_sched_barrier(0);
+                mfmas(I0{});
+                __builtin_amdgcn_sched_barrier(0);
                 wait_frags(I1{}, NONE{});
+                __builtin_amdgcn_sched_barrier(0);
+                mfmas(I1{});
+                __builtin_amdgcn_sched_barrier(0);
+                stage = stage + 1 == STAGES ? 0 : stage + 1;
             }
-            __builtin_amdgcn_sched_barrier(0);
-            mfmas(I1{});
-            __builtin_amdgcn_sched_barrier(0);
-            stage = next_stage;
         }
         if (AHEAD)
             wait_frags(I0{}, NONE{}); // the registers of the last, unused set are free only now
@@ -308,7 +375,7 @@ namespace nnf
         constexpr int ROUND_TM = TM >= 2 ? 2 : 1;  // 32-row blocks per pass through LDS
         constexpr int PITCH = TN * 64 + 16;        // bytes per staged row (padding spreads the banks)
         constexpr int REGION = ROUND_TM * 32 * PITCH;
-        static_assert(8 * REGION <= T::LDS_BYTES, "the staging regions reuse the ring");
+        static_assert(T::WAVES * REGION <= T::LDS_BYTES, "the staging regions reuse the ring");
         constexpr int LANES_PER_ROW = TN * 4, ROWS_PER_READ = 64 / LANES_PER_ROW;
         __builtin_amdgcn_s_barrier(); // every wavefront has read its last fragments
         uint8_t* region = smem + wave * REGION;
@@ -435,7 +502,7 @@ namespace nnf
                     return e;
             }
             const int splits = SPLITK ? p.splits : 1;
-            hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n * splits), dim3(q8dl::THREADS), T::LDS_BYTES, stream, p);
+            hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n * splits), dim3(T::THREADS), T::LDS_BYTES, stream, p);
             return hipGetLastError();
         }
 
