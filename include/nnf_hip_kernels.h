@@ -116,10 +116,12 @@ enum nnf_w4a16_variant
 typedef struct nnf_plan
 {
     int tile_rows; /* rows of an output tile: 256, 128, 64 (fp16 x int4 also 32); tiles are 256 columns wide
-                      (W8A8 128-row tiles: 128 columns) */
+                      (W8A8 128-row tiles: 128 columns; W8A8 256-row tiles: see tile_cols) */
     int k_parts;   /* fp16 x int4: workgroups that share one output tile, each a contiguous part of K, summed by a
                       second launch (the grid is tiles x k_parts, work split evenly); W8A8: ranges of K, int32
                       partial sums added exactly by a reduction pass */
+    int tile_cols; /* W8A8 with 256-row tiles: 256 or 128 columns (0: whichever fills the CUs better for the shape);
+                      0 everywhere else */
 } nnf_plan;
 /* 1 when the variant can serve the shape (decided on the host, for a 256-CU device), else 0. */
 int nnf_w4a16_variant_supported(int M, int N, int K, int group, int variant);

@@ -54,6 +54,7 @@ namespace nnf
                            // 3 tile GEMM, 4 row-streaming kernels
         int tile_rows = 0; // tile GEMM: rows of an output tile (256, 128, 64; fp16 x int4 also 32)
         int k_parts = 0;   // tile GEMM: workgroups that share an output tile (fp16 x int4) / ranges of K (W8A8)
+        int tile_cols = 0; // W8A8 tile GEMM with 256-row tiles: 256 or 128 columns
     };
 
     hipError_t launch_w4a16_gemv(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y,

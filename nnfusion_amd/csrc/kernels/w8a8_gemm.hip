@@ -295,7 +295,7 @@ namespace nnf
     {
         if (pick_w8a8(M, N, K, num_cu, choice.path) != Q8_TILE)
             return 0;
-        const int tile = choice.tile_rows == 256 ? 0 : choice.tile_rows == 128 ? 1 : choice.tile_rows == 64 ? 2 : -1;
+        const int tile = workspace::w8a8_forced_tile(choice.tile_rows, choice.tile_cols);
         return workspace::gemm_partial_bytes(M, N, false, workspace::plan_w8a8_gemm(M, N, K, tile, choice.k_parts));
     }
 

@@ -517,6 +517,11 @@ namespace nnf
                     return launch_tile<2, 4, 4, 2, 4, RAW, false, 2>(stream, p);
                 e = launch_tile<2, 4, 4, 2, 4, RAW, true, 2>(stream, p);
                 break;
+            case workspace::GEMM_TILE_TALL: // 256 x 128, four stages, one workgroup per CU
+                if (!plan.reduce_pass)
+                    return launch_tile<2, 4, 4, 1, 4, RAW, false, 2>(stream, p);
+                e = launch_tile<2, 4, 4, 1, 4, RAW, true, 2>(stream, p);
+                break;
             case workspace::GEMM_TILE_MID: // 128 x 128
                 if (!plan.reduce_pass)
                     return launch_tile<2, 4, 2, 1, 3, RAW, false, 4>(stream, p);
@@ -538,7 +543,7 @@ namespace nnf
     hipError_t launch_w8a8_gemm(hipStream_t stream, const void* A, const void* s_tok, const void* W, const void* s_ch,
                                 void* Y, void* acc, int M, int N, int K, void* partial_ws, const LaunchChoice& choice)
     {
-        const int tile = choice.tile_rows == 256 ? 0 : choice.tile_rows == 128 ? 1 : choice.tile_rows == 64 ? 2 : -1;
+        const int tile = workspace::w8a8_forced_tile(choice.tile_rows, choice.tile_cols);
         const workspace::GemmPlan plan = workspace::plan_w8a8_gemm(M, N, K, tile, choice.k_parts);
         if (plan.reduce_pass && !partial_ws)
             return hipErrorInvalidValue;

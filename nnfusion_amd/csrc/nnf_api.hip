@@ -71,7 +71,7 @@ extern "C" {
 
 int nnf_abi_version(void)
 {
-    return 2;
+    return 3;
 }
 
 const char* nnf_status_string(int status)
@@ -105,10 +105,12 @@ namespace
         if (plan)
         {
             const int r = plan->tile_rows;
-            if ((r != 0 && r != 32 && r != 64 && r != 128 && r != 256) || plan->k_parts < 0)
+            const int c = plan->tile_cols;
+            if ((r != 0 && r != 32 && r != 64 && r != 128 && r != 256) || plan->k_parts < 0 || (c != 0 && c != 128 && c != 256))
                 return false;
             out.tile_rows = r;
             out.k_parts = plan->k_parts;
+            out.tile_cols = c;
         }
         return true;
     }

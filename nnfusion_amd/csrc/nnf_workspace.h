@@ -19,6 +19,7 @@ namespace nnf
             GEMM_TILE_MID = 1,   // 128 x 128
             GEMM_TILE_SMALL = 2, //  64 x 256
             GEMM_TILE_TINY = 3,  //  32 x 256 (not built for W8A8)
+            GEMM_TILE_TALL = 4,  // 256 x 128 (W8A8 only: fills the chip where 256 x 256 tiles leave CUs idle)
         };
         struct GemmPlan
         {
@@ -34,13 +35,13 @@ namespace nnf
         // N(0,1) activations (the GEMMs are power bound: ~950 / 700 / 450 TFLOP/s for the three tile shapes when
         // every CU has a workgroup, and a CU runs faster when fewer are busy: hence the square root), ~6 TB/s for
         // the partial sums (written, then read by the reduction pass) and ~3 us for the second launch.
-        // w8a8: the same tiles on the int8 matrix cores (~1870 / 1450 / 900 TOP/s; its weight bytes differ too, but
-        // a memory-bound W8A8 shape is decided by the partial-sum term either way)
+        // w8a8: the same tiles on the int8 matrix cores (~1870 / 1450 / 900 TOP/s, 1700 for 256 x 128; its weight bytes
+        // differ too, but a memory-bound W8A8 shape is decided by the partial-sum term either way)
         inline double estimate_gemm(int M, int N, int K, bool gate, int tile, int splits, bool w8a8)
         {
-            const int bm = tile == GEMM_TILE_BIG ? 256 : tile == GEMM_TILE_MID ? 128 : tile == GEMM_TILE_SMALL ? 64 : 32;
-            const int bn = tile == GEMM_TILE_BIG ? (gate ? 128 : 256) : tile == GEMM_TILE_MID ? 128 : 256;
-            static const double rates[2][4] = {{950e12, 700e12, 450e12, 300e12}, {1870e12, 1450e12, 900e12, 600e12}};
+            const int bm = tile == GEMM_TILE_BIG || tile == GEMM_TILE_TALL ? 256 : tile == GEMM_TILE_MID ? 128 : tile == GEMM_TILE_SMALL ? 64 : 32;
+            const int bn = tile == GEMM_TILE_BIG ? (gate ? 128 : 256) : tile == GEMM_TILE_MID || tile == GEMM_TILE_TALL ? 128 : 256;
+            static const double rates[2][5] = {{950e12, 700e12, 450e12, 300e12, 800e12}, {1870e12, 1450e12, 900e12, 600e12, 1700e12}};
             const double rate = rates[w8a8 ? 1 : 0][tile];
             const int tiles_m = ceil_div(M, bm), tiles_n = ceil_div(N, bn);
             const double blocks = (double)tiles_m * tiles_n * splits;
@@ -52,7 +53,7 @@ namespace nnf
             const double weight_time = n_total * K / 2.0 / 4e12;
             if (t < weight_time)
                 t = weight_time;
-            if (splits > 1 || tile >= GEMM_TILE_SMALL)
+            if (splits > 1 || tile == GEMM_TILE_SMALL || tile == GEMM_TILE_TINY)
                 t += 2.0 * splits * M * n_total * 4.0 / 6e12 + 3e-6;
             return t;
         }
@@ -64,11 +65,16 @@ namespace nnf
             const int G = K / 128;
             GemmPlan best;
             double best_t = -1.0;
-            for (int tile = GEMM_TILE_BIG; tile <= GEMM_TILE_TINY; ++tile)
+            for (int tile = GEMM_TILE_BIG; tile <= GEMM_TILE_TALL; ++tile)
             {
+                // (forced_tile -2: 256-row tiles, their width left to the plan)
+                if (tile == GEMM_TILE_TALL && !w8a8)
+                    continue;
                 if (forced_tile >= 0 ? tile != forced_tile
-                                     : ((tile == GEMM_TILE_BIG && M <= 128) || (tile == GEMM_TILE_SMALL && M > 64) ||
-                                        (tile == GEMM_TILE_MID && M <= 64) || (tile == GEMM_TILE_TINY && (M > 32 || w8a8))))
+                    : forced_tile == -2 ? (tile != GEMM_TILE_BIG && tile != GEMM_TILE_TALL)
+                                     : (((tile == GEMM_TILE_BIG || tile == GEMM_TILE_TALL) && M <= 128) ||
+                                        (tile == GEMM_TILE_SMALL && M > 64) || (tile == GEMM_TILE_MID && M <= 64) ||
+                                        (tile == GEMM_TILE_TINY && (M > 32 || w8a8))))
                     continue;
                 for (int s : split_options)
                 {
@@ -85,12 +91,20 @@ namespace nnf
                     }
                 }
             }
-            best.reduce_pass = best.splits > 1 || best.tile >= GEMM_TILE_SMALL;
+            best.reduce_pass = best.splits > 1 || best.tile == GEMM_TILE_SMALL || best.tile == GEMM_TILE_TINY;
             return best;
         }
         inline GemmPlan plan_w8a8_gemm(int M, int N, int K, int forced_tile = -1, int forced_splits = 0)
         {
             return plan_gemm(M, N, K, false, true, forced_tile, forced_splits);
+        }
+        // a caller's tile_rows / tile_cols as a forced tile of plan_w8a8_gemm (-1: none; -2: 256-row tiles of the
+        // plan's own width)
+        inline int w8a8_forced_tile(int tile_rows, int tile_cols)
+        {
+            if (tile_rows == 256)
+                return tile_cols == 256 ? GEMM_TILE_BIG : tile_cols == 128 ? GEMM_TILE_TALL : -2;
+            return tile_rows == 128 ? GEMM_TILE_MID : tile_rows == 64 ? GEMM_TILE_SMALL : -1;
         }
         inline size_t gemm_partial_bytes(int M, int N, bool gate, const GemmPlan& p)
         {

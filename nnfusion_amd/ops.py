@@ -13,15 +13,15 @@ from . import _lib
 
 class NnfPlan(ctypes.Structure):
     """struct nnf_plan of the C header: what a kernel-selection candidate fixes about the tile GEMM."""
-    _fields_ = [("tile_rows", ctypes.c_int), ("k_parts", ctypes.c_int)]
+    _fields_ = [("tile_rows", ctypes.c_int), ("k_parts", ctypes.c_int), ("tile_cols", ctypes.c_int)]
 
 
 def _plan_arg(plan):
-    """None, an NnfPlan or a (tile_rows, k_parts) pair -> (object to keep alive, pointer argument)."""
+    """None, an NnfPlan or a (tile_rows, k_parts[, tile_cols]) tuple -> (object to keep alive, pointer argument)."""
     if plan is None:
         return None, None
     if not isinstance(plan, NnfPlan):
-        plan = NnfPlan(int(plan[0]), int(plan[1]))
+        plan = NnfPlan(int(plan[0]), int(plan[1]), int(plan[2]) if len(plan) > 2 else 0)
     return plan, ctypes.cast(ctypes.pointer(plan), ctypes.c_void_p)
 
 

@@ -18,10 +18,11 @@ def _t(gpu, *arrays):
 # Kernel families, asked for per call through nnf_w8a8_gemm_variant where the family takes the shape (the library's own
 # choice where it does not): "auto"; "skinny": the split-K M <= 16 kernel; "mfma_rows": the row-streaming MFMA kernel
 # (2 <= M <= 32, K = 1024 .. 16384 in multiples of 256); otherwise the MFMA tile GEMM with a plan (tile_rows, k_parts):
-# tiles of 256 x 256, 128 x 128 or 64 x 256 outputs (0: the library's choice) and the number of K ranges (int32 partial
-# sums, added exactly by the reduction pass)
-@pytest.fixture(params=["auto", "skinny", "mfma_rows", (0, 0), (256, 1), (256, 2), (128, 1), (128, 3), (64, 1), (64, 2)],
-                ids=lambda p: p if isinstance(p, str) else f"gemm-rows{p[0]}-parts{p[1]}")
+# tiles of 256 x 256, 256 x 128 (third value: the columns), 128 x 128 or 64 x 256 outputs (0: the library's choice) and the
+# number of K ranges (int32 partial sums, added exactly by the reduction pass)
+@pytest.fixture(params=["auto", "skinny", "mfma_rows", (0, 0), (256, 1, 256), (256, 2, 256), (256, 1, 128), (256, 3, 128), (256, 0),
+                        (128, 1), (128, 3), (64, 1), (64, 2)],
+                ids=lambda p: p if isinstance(p, str) else "gemm-rows%d-parts%d" % p[:2] + ("-cols%d" % p[2] if len(p) > 2 else ""))
 def path(request):
     return request.param
 
