@@ -347,18 +347,24 @@ class Env:
         return e0.elapsed_time(e1) * 1000.0 / reps
 
     def time_us(self, fn, iters):
+        """Mean microseconds per call in a sustained run: the compute-bound rows run 10-15 % slower for the first tens of
+        milliseconds after the chip has been idle (vendor library included), so about 40 ms of untimed calls go ahead
+        of at least `iters` timed ones (at least 20 ms of them)."""
         torch = self.torch
-        for _ in range(10):
-            fn()
-        torch.cuda.synchronize()
-        e0 = torch.cuda.Event(enable_timing=True)
-        e1 = torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(iters):
-            fn()
-        e1.record()
-        torch.cuda.synchronize()
-        return e0.elapsed_time(e1) * 1000.0 / iters
+
+        def run(n):
+            e0 = torch.cuda.Event(enable_timing=True)
+            e1 = torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(n):
+                fn()
+            e1.record()
+            torch.cuda.synchronize()
+            return e0.elapsed_time(e1) * 1000.0 / n
+
+        first = run(5)
+        run(max(5, min(2000, int(40e3 / max(first, 1.0)))))
+        return run(max(iters, min(2000, int(20e3 / max(first, 1.0)))))
 
     def time_cold_us(self, make_fn, weight_sets):
         """Launches walking device-side copies of the weights (more than the last-level cache holds), captured in
