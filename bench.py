@@ -76,8 +76,8 @@ DOMINANT_KERNEL = {
     "wna16_b4_g64_zp_tensor_N8192_K8192.M1": "nnf::wna16_gemv_kernel<4, 4, 1>",
     "wna16_b4_g64_zp_tensor_N8192_K8192.M16": "nnf::wna16_skinny_kernel<4, 2>",
     "wna16_b4_g64_zp_tensor_N8192_K8192.M4096": "nnf::wna16_tile128_kernel<4>",
-    "fused_mlp_M1_4096_11008": "rms_rstd_kernel + 2 x nnf::w4a16_gemv_rows_kernel (gate|up with SiLU, down with the residual)",
-    "fused_mlp_M16_4096_11008": "rms_rstd_kernel + nnf::w4a16_mrows_kernel (gate|up) + w4a16_mrows_any_kernel over 3 ranges of K + "
+    "fused_mlp_M1_4096_11008": "2 x nnf::w4a16_gemv_rows_fused_kernel (gate|up with RMSNorm and SiLU, down with the residual)",
+    "fused_mlp_M16_4096_11008": "nnf::w4a16_mrows_kernel (gate|up with RMSNorm and SiLU) + w4a16_mrows_any_kernel over 3 ranges of K + "
                                 "splitk_reduce_kernel (down)",
     "fused_mlp_M256_4096_11008": "rms_rstd_kernel + 2 x (nnf::gemm_sk::w4a16_gemm_sk_kernel<4, 2, ...> + fixup)",
 }

@@ -174,9 +174,11 @@ enum nnf_activation
 };
 
 /* Same GEMM with prologue / epilogue in one call.  They run inside the kernel that serves the shape: the
- * row-streaming kernels (M = 1; M <= 32) and the tile GEMM multiply gamma in on the way in, rstd[m] (from a
- * small pre-pass over A, fp32 [M] in `workspace`) and the epilogue at their end; a GEMV kernel over ranges
- * of K leaves rstd and the epilogue to its reduction pass.  Only the MFMA GEMV kernel (M <= 16 with K not a
+ * row-streaming kernels (M = 1; M <= 32) and the tile GEMM multiply gamma in on the way in, rstd[m] and the
+ * epilogue at their end.  The row-streaming kernels add up the squares of the activations they hold themselves
+ * (K a multiple of 1024 up to 8192; M = 1: any K they take): one launch in all; the tile GEMM and the other
+ * forms take rstd from a small pre-pass over A (fp32 [M] in `workspace`); a GEMV kernel over ranges of K
+ * leaves rstd and the epilogue to its reduction pass.  Only the MFMA GEMV kernel (M <= 16 with K not a
  * multiple of 256) reads normalised activations written to `workspace` by a pre-pass and leaves its
  * products to one element-wise kernel.
  *   rms_gamma != NULL : A is replaced by RMSNorm(A) = A * rsqrt(mean_k(A^2) + rms_eps) * gamma[k]

@@ -158,6 +158,7 @@ namespace nnf
         const float* rstd;
         const half_t* bias;
         const half_t* residual;
+        float rms_eps; // gamma without rstd: the kernel computes rsqrt(mean(a^2) + rms_eps) of its activation row itself
     };
     // y = fp16(sum) (+ bias[n]) (+ residual[at]), each step rounded to fp16
     __device__ __forceinline__ half_t finish_bias_residual(float sum, const half_t* bias, int n, const half_t* residual, size_t at)

@@ -40,6 +40,7 @@ namespace nnf
     {
         const void* gamma = nullptr;    // fp16 [K]: RMSNorm weight, multiplied onto the activations on the way in ...
         const float* rstd = nullptr;    // fp32 [M]: ... with the sums of row m scaled by rstd[m] on the way out
+        float rms_eps = 0.f;            // gamma without rstd (the row-streaming kernels with a fixed K): rstd computed inside the kernel with this eps
         const void* bias = nullptr;     // fp16 [N]
         const void* residual = nullptr; // fp16 [M, N]; may be the output buffer itself
         bool gate = false;              // N outputs from 2 N weight rows (gate rows, then up rows): SiLU(gate) * up

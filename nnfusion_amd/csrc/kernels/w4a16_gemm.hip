@@ -280,8 +280,12 @@ namespace nnf
             return hipErrorInvalidValue;
         // ---- RMSNorm pre-pass: rstd[m] for the kernels that multiply the weight in themselves, the normalised
         // activations for the MFMA GEMV kernel -------------------------------------------------------------------
+        // (the row-streaming kernels add up the squares of the activations they hold themselves: no pre-pass; the form
+        // with a run-time K keeps it)
         const bool normalised_copy = route.kind == W4A16Route::SKINNY || route.kind == W4A16Route::SKINNY_SPLIT;
-        if (rms)
+        const bool rstd_in_kernel =
+            route.kind == W4A16Route::ROWS || (route.kind == W4A16Route::MROWS && workspace::w4a16_mrows_fixed_k(M, K));
+        if (rms && !rstd_in_kernel)
         {
             if (normalised_copy)
             {
@@ -295,13 +299,14 @@ namespace nnf
             if (e != hipSuccess)
                 return e;
         }
-        const float* rstd = (rms && !normalised_copy) ? (const float*)rms_ws : nullptr;
+        const float* rstd = (rms && !normalised_copy && !rstd_in_kernel) ? (const float*)rms_ws : nullptr;
         // ---- the row-streaming kernels (one row; up to 32 rows): prologue and epilogue inside the one launch ------
         if (route.kind == W4A16Route::ROWS || route.kind == W4A16Route::MROWS)
         {
             GemvFusion fusion;
             fusion.gamma = rms_gamma;
             fusion.rstd = rstd;
+            fusion.rms_eps = rms_eps;
             fusion.bias = bias;
             fusion.residual = residual;
             fusion.gate = gate;

@@ -111,6 +111,8 @@ namespace nnf
         uint8_t* scales = reinterpret_cast<uint8_t*>(corr + a_pad + 4);
         float* outb = reinterpret_cast<float*>(scales + (GATE ? 2 : 1) * sc_block);
         int* next_row = reinterpret_cast<int*>(outb + (((GATE ? 2 : 1) * (rows_q + 1)) << kshift));
+        float* sum_sq = reinterpret_cast<float*>(next_row + 8); // per wavefront: its share of sum a^2 (RMSNorm inside the kernel)
+        const bool own_rstd = EPI != 0 && f.gamma && !f.rstd;
 
         // ---- activations and scales: requested first (few loads, cache hits), once per workgroup ------------
         // (global -> LDS like the weights: a load into registers followed by an LDS write would be made to wait
@@ -204,11 +206,23 @@ namespace nnf
         {
             const float ce = -(1024.0f + (float)zp);
             const float co = -(64.0f + (float)zp);
+            float ss = 0.f;
             int e = 0;
             for (int u0 = wave * 64; u0 < a_units; u0 += WAVES * 64, ++e)
             {
                 const int u = u0 + lane;
                 uintx4 raw = act[u];
+                if (own_rstd && u < a_units)
+                {
+                    // RMSNorm without a pass of its own: every unit of the row goes through exactly one lane here
+                    const uint32_t rr[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                    {
+                        const half2_t hh = as_half2(rr[i]);
+                        ss += (float)hh.x * (float)hh.x + (float)hh.y * (float)hh.y;
+                    }
+                }
                 if (EPI != 0 && f.gamma)
                 {
                     // fp16(a * gamma): the product of two fp16 values, rounded once
@@ -227,6 +241,14 @@ namespace nnf
                 const float so = ((float)y.x + (float)y.y) + ((float)w.x + (float)w.y);
                 act[u] = a;
                 corr[u] = ce * se + co * so;
+            }
+            if (own_rstd)
+            {
+                ss = row16_sum(ss);
+                ss += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, ss), 0x142, 0xA, 0xF, false));
+                ss += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, ss), 0x143, 0xC, 0xF, false));
+                if (lane == 63)
+                    sum_sq[wave] = ss;
             }
         }
         lds_barrier();
@@ -350,7 +372,14 @@ namespace nnf
 
         // ---- outputs ------------------------------------------------------------------------------------
         lds_barrier();
-        const float rs = (EPI != 0 && f.rstd) ? f.rstd[0] : 1.0f;
+        float rs = (EPI != 0 && f.rstd) ? f.rstd[0] : 1.0f;
+        if (own_rstd)
+        {
+            float total = 0.f;
+            for (int w = 0; w * 64 < a_units && w < WAVES; ++w) // the wavefronts that fetched a share of the row
+                total += sum_sq[w];
+            rs = 1.0f / __builtin_sqrtf(total / (float)K + f.rms_eps);
+        }
         for (int r = tid; r < n_out; r += WAVES * 64)
         {
             float y = 0.f;
@@ -380,7 +409,7 @@ namespace nnf
                                                                          half_t* __restrict__ Y, int N, int K,
                                                                          int rows_q, int rows_r, int pack)
     {
-        gemv_rows_body<SEG, D, WAVES, 0>(A, Wq, S, Y, N, K, rows_q, rows_r, pack, GemvFusionArgs{nullptr, nullptr, nullptr, nullptr});
+        gemv_rows_body<SEG, D, WAVES, 0>(A, Wq, S, Y, N, K, rows_q, rows_r, pack, GemvFusionArgs{nullptr, nullptr, nullptr, nullptr, 0.f});
     }
     template <int SEG, int D, int WAVES, int EPI>
     __global__ __launch_bounds__(WAVES * 64) void w4a16_gemv_rows_fused_kernel(const half_t* __restrict__ A,
@@ -403,7 +432,7 @@ namespace nnf
         {
             const size_t lds_total = p.lds_bytes(N, K, grid, EPI == 2);
             const GemvFusionArgs f = {(const half_t*)fusion.gamma, fusion.rstd, (const half_t*)fusion.bias,
-                                      (const half_t*)fusion.residual};
+                                      (const half_t*)fusion.residual, fusion.rms_eps};
             if (lds_total > MAX_LDS_BYTES)
                 return hipErrorInvalidValue;
             const void* kernel;

@@ -79,9 +79,10 @@ namespace nnf
     // The workgroup's parked sums -> Y.  Plain: fp16 of the sum.  Fused (see GemvFusion in nnf_launch.h): the sums of
     // row m times rstd[m]; gate: tiles 2 i and 2 i + 1 of the workgroup are the gate and the up rows of its output tile
     // i; bias and residual.  t0: the workgroup's first output tile, T_out of them; N: output columns.
-    template <bool FUSED>
+    // sum_sq ([8 wavefronts][MB x 16 rows], or null) and K: RMSNorm without a pass of its own (gamma, no rstd).
+    template <bool FUSED, int MB>
     __device__ __forceinline__ void mrows_flush(const float* parked, half_t* __restrict__ Y, int t0, int T_out, int M, int N,
-                                                int tid, const GemvFusionArgs& f, int gate)
+                                                int tid, const GemvFusionArgs& f, int gate, const float* sum_sq = nullptr, int K = 0)
     {
         for (int idx = tid; idx < T_out * M * 16; idx += 512)
         {
@@ -98,7 +99,15 @@ namespace nnf
                 Y[at] = (half_t)parked[idx];
             else
             {
-                const float rs = f.rstd ? f.rstd[m] : 1.0f;
+                float rs = f.rstd ? f.rstd[m] : 1.0f;
+                if (sum_sq)
+                {
+                    float total = 0.f;
+#pragma unroll
+                    for (int w = 0; w < MR_WAVES; ++w)
+                        total += sum_sq[w * (MB * 16) + m];
+                    rs = 1.0f / __builtin_sqrtf(total / (float)K + f.rms_eps);
+                }
                 if (gate)
                     Y[at] = finish_silu_gate(parked[((2 * it) * M + m) * 16 + n] * rs, parked[((2 * it + 1) * M + m) * 16 + n] * rs);
                 else
@@ -250,7 +259,8 @@ namespace nnf
         uint8_t* ring = smem + wave * (2 * TILE_BYTES);
         uint8_t* sc_ring = smem + MR_WAVES * 2 * TILE_BYTES + wave * 512;
         uint8_t* red = smem + MR_WAVES * 2 * TILE_BYTES + MR_WAVES * 512; // [2][8][1024]
-        float* parked = reinterpret_cast<float*>(red + 2 * MR_WAVES * MB * 1024);
+        float* sum_sq = reinterpret_cast<float*>(red + 2 * MR_WAVES * MB * 1024); // [8][MB x 16]
+        float* parked = sum_sq + MR_WAVES * MB * 16;
 
         // ---- what each lane fetches -------------------------------------------------------------------------
         // Load c of a tile fills bytes [c KiB, (c+1) KiB) of the slot; lane i lands at byte c*1024 + 16 i =
@@ -306,6 +316,33 @@ namespace nnf
                     areg[mb][g][j] = *reinterpret_cast<const uintx4*>(
                         a_bytes + (size_t)(a_off + (g / GW) * (SPAN * 4) + (g % GW) * 256 + j * 16));
         }
+        // RMSNorm without a pass of its own: the wavefront's share of sum a^2 of every row, from the registers
+        const bool own_rstd = FUSED && f.gamma && !f.rstd;
+        if (own_rstd)
+        {
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb)
+            {
+                float ss = 0.f;
+#pragma unroll
+                for (int g = 0; g < GA; ++g)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                    {
+                        const uint32_t rr[4] = {areg[mb][g][j].x, areg[mb][g][j].y, areg[mb][g][j].z, areg[mb][g][j].w};
+#pragma unroll
+                        for (int i = 0; i < 4; ++i)
+                        {
+                            const half2_t hh = as_half2(rr[i]);
+                            ss += (float)hh.x * (float)hh.x + (float)hh.y * (float)hh.y;
+                        }
+                    }
+                ss += __shfl_xor(ss, 16, 64);
+                ss += __shfl_xor(ss, 32, 64);
+                if (kq == 0)
+                    sum_sq[wave * (MB * 16) + mb * 16 + col] = ss;
+            }
+        }
         if (FUSED && f.gamma)
             mrows_scale_a<MB, GA>(areg, [&](int g) {
                 return reinterpret_cast<const uint8_t*>(f.gamma) + wave * (GW * 256) + kq * 64 + (g / GW) * (SPAN * 4) + (g % GW) * 256;
@@ -357,7 +394,7 @@ namespace nnf
         __builtin_amdgcn_s_waitcnt(mr_vmcnt(0)); // the reloads past the end, before the LDS goes away
         asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
         // ---- flush: parked sums -> Y -----------------------------------------------------------------------------
-        mrows_flush<FUSED>(parked, Y, t0, T_out, M, N, tid, f, gate);
+        mrows_flush<FUSED, MB>(parked, Y, t0, T_out, M, N, tid, f, gate, own_rstd ? sum_sq : nullptr, K);
     }
 
     // The same kernel with K as a run-time value: any multiple of 256 up to 8 * GW * STEPS groups (2 <= M <= 16).
@@ -418,7 +455,8 @@ namespace nnf
         uint8_t* ring = smem + wave * (2 * TILE_BYTES);
         uint8_t* sc_ring = smem + MR_WAVES * 2 * TILE_BYTES + wave * 512;
         uint8_t* red = smem + MR_WAVES * 2 * TILE_BYTES + MR_WAVES * 512; // [2][8][1024]
-        float* parked = reinterpret_cast<float*>(red + 2 * MR_WAVES * MB * 1024);
+        float* sum_sq = reinterpret_cast<float*>(red + 2 * MR_WAVES * MB * 1024); // [8][MB x 16]
+        float* parked = sum_sq + MR_WAVES * MB * 16;
 
         auto swz = [](int r) { return GW % 4 == 0 ? (r & 15) : GW % 2 == 0 ? (r >> 1) & 7 : (r >> 2) & 3; };
         uint32_t w_off[GW];
@@ -532,14 +570,15 @@ namespace nnf
             }
         }
         else
-            mrows_flush<FUSED>(parked, Y, t0, T_out, M, N, tid, f, gate);
+            mrows_flush<FUSED, MB>(parked, Y, t0, T_out, M, N, tid, f, gate);
     }
 
     namespace
     {
         GemvFusionArgs fusion_args(const GemvFusion& fusion)
         {
-            return GemvFusionArgs{(const half_t*)fusion.gamma, fusion.rstd, (const half_t*)fusion.bias, (const half_t*)fusion.residual};
+            return GemvFusionArgs{(const half_t*)fusion.gamma, fusion.rstd, (const half_t*)fusion.bias, (const half_t*)fusion.residual,
+                                  fusion.rms_eps};
         }
 
         // N: output columns (fusion.gate: from 2 N weight rows)

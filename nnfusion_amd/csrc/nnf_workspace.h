@@ -303,7 +303,7 @@ namespace nnf
             int seg = 0;    // wavefront-wide loads (1 KiB of a weight row) per row and wavefront; 0: not applicable
             int kshift = 0; // log2 of the wavefronts that share a row
             int depth = 0;  // rows in flight per wavefront
-            // ring + activations (+ zeros) + their constants + the workgroup's scales + parked outputs + row counters
+            // ring + activations (+ zeros) + their constants + the workgroup's scales + parked outputs + row counters (32 bytes) + the wavefronts' sums of squares for RMSNorm (32 bytes)
             // (gate: N outputs from 2 N weight rows; a workgroup holds the scales of its gate rows and of its up rows as
             // two blocks, each rounded up to whole KiB)
             size_t lds_bytes(int N, int K, int grid, bool gate = false) const
@@ -440,7 +440,9 @@ namespace nnf
         }
         inline size_t w4a16_mrows_lds_bytes_gw(int gw, int M, int tiles)
         {
-            return (size_t)8 * 2 * gw * 1024 + 8 * 512 + (size_t)2 * 8 * (M <= 16 ? 1 : M <= 32 ? 2 : 4) * 1024 + (size_t)tiles * M * 64;
+            const size_t mb = M <= 16 ? 1 : M <= 32 ? 2 : 4; // blocks of 16 rows
+            // ring, scales, partial tiles, the wavefronts' sums of squares per row (RMSNorm inside the kernel), parked sums
+            return (size_t)8 * 2 * gw * 1024 + 8 * 512 + (size_t)2 * 8 * mb * 1024 + 8 * mb * 64 + (size_t)tiles * M * 64;
         }
         inline size_t w4a16_mrows_lds_bytes(int K, int M, int tiles)
         {
