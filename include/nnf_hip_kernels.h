@@ -115,13 +115,14 @@ enum nnf_w4a16_variant
  * NULL, or a field that is 0: the library's own choice for the shape. */
 typedef struct nnf_plan
 {
-    int tile_rows; /* rows of an output tile: 256, 128, 64 (fp16 x int4 also 32); tiles are 256 columns wide
-                      (W8A8 128-row tiles: 128 columns; W8A8 256-row tiles: see tile_cols) */
+    int tile_rows; /* rows of an output tile: 256, 128, 64 (fp16 x int4 also 32); see tile_cols for their width
+                      (W8A8 128-row tiles: 128 columns, 64-row tiles: 256) */
     int k_parts;   /* fp16 x int4: workgroups that share one output tile, each a contiguous part of K, summed by a
                       second launch (the grid is tiles x k_parts, work split evenly); W8A8: ranges of K, int32
                       partial sums added exactly by a reduction pass */
-    int tile_cols; /* W8A8 with 256-row tiles: 256 or 128 columns (0: whichever fills the CUs better for the shape);
-                      0 everywhere else */
+    int tile_cols; /* columns of an output tile, 256 or 128 (0: the library's choice): W8A8 with 256-row tiles;
+                      fp16 x int4 with 64-, 128- or 256-row tiles and no SiLU-gate (the gate | up halves need the
+                      256 weight rows of a full tile); ignored elsewhere */
 } nnf_plan;
 /* 1 when the variant can serve the shape (decided on the host, for a 256-CU device), else 0. */
 int nnf_w4a16_variant_supported(int M, int N, int K, int group, int variant);

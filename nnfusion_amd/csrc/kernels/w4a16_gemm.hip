@@ -275,7 +275,7 @@ namespace nnf
             return hipErrorInvalidValue;
         const int n_rows = gate ? 2 * N : N; // weight rows
         const W4A16Route route =
-            workspace::route_w4a16(M, N, K, gate, rms, hr && residual == Y, num_cu, choice.path, choice.tile_rows, choice.k_parts);
+            workspace::route_w4a16(M, N, K, gate, rms, hr && residual == Y, num_cu, choice.path, choice.tile_rows, choice.k_parts, choice.tile_cols);
         if (route.kind == W4A16Route::NONE || (route.partial_bytes > 0 && !partial_ws) || (route.rms_bytes > 0 && !rms_ws))
             return hipErrorInvalidValue;
         // ---- RMSNorm pre-pass: rstd[m] for the kernels that multiply the weight in themselves, the normalised
@@ -377,6 +377,10 @@ namespace nnf
         p.tiles_n = plan.tiles_n;
         p.supersteps = plan.supersteps;
         p.units = plan.units;
+        if (plan.tile_weight_rows == 128)
+            return plan.tile_rows == 256 ? launch_gemm_sk_256_narrow(stream, p, plan.grid)
+                   : plan.tile_rows == 128 ? launch_gemm_sk_128_narrow(stream, p, plan.grid)
+                                           : launch_gemm_sk_64_narrow(stream, p, plan.grid);
         switch (plan.tile_rows)
         {
         case 256: return launch_gemm_sk_256(stream, p, plan.grid, gate);

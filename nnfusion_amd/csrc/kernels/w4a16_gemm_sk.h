@@ -313,7 +313,8 @@ namespace nnf
         using T = Tile<TM, TN>;
         using SCH = Sched<TM, TN, RMS>;
         static_assert(!(GATE && (BIAS || RESID)), "SiLU-gate is not combined with bias or residual");
-        static_assert(TN == 2 || TN == 4, "column tiles per wavefront");
+        static_assert(TN == 1 || TN == 2 || TN == 4, "column tiles per wavefront");
+        static_assert(!GATE || TN >= 2, "gate and up rows are the two halves of a wavefront's column tiles");
         constexpr int BM = T::BM, BN = T::BN;
         constexpr int A_TILE_BYTES = T::A_TILE_BYTES, STAGE_BYTES = T::STAGE_BYTES;
         constexpr int BN_OUT = GATE ? BN / 2 : BN;

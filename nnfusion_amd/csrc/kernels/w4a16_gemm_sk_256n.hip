@@ -1,0 +1,10 @@
+// fp16 x int4 tile GEMM, tiles of 256 x 128 (one column tile per wavefront): the instantiations of w4a16_gemm_sk.h.
+#include "w4a16_gemm_sk_launch.h"
+
+namespace nnf
+{
+    hipError_t launch_gemm_sk_256_narrow(hipStream_t stream, const SkGemmParams& p, int grid)
+    {
+        return gemm_sk::launch_tile_height_plain<8, 1>(stream, p, grid);
+    }
+} // namespace nnf

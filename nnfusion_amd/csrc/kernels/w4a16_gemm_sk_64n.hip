@@ -1,0 +1,10 @@
+// fp16 x int4 tile GEMM, tiles of 64 x 128 (one column tile per wavefront): the instantiations of w4a16_gemm_sk.h.
+#include "w4a16_gemm_sk_launch.h"
+
+namespace nnf
+{
+    hipError_t launch_gemm_sk_64_narrow(hipStream_t stream, const SkGemmParams& p, int grid)
+    {
+        return gemm_sk::launch_tile_height_plain<2, 1>(stream, p, grid);
+    }
+} // namespace nnf

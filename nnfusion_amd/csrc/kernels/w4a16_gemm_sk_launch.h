@@ -51,9 +51,29 @@ namespace nnf
             return rms ? launch_instance<TM, TN, false, false, false, true>(stream, p, grid)
                        : launch_instance<TM, TN, false, false, false, false>(stream, p, grid);
         }
+        // the forms without SiLU-gate (tiles one column tile per wavefront wide have no gate | up pairs)
+        template <int TM, int TN>
+        hipError_t launch_tile_height_plain(hipStream_t stream, const SkGemmParams& p, int grid)
+        {
+            const bool hb = p.bias != nullptr, hr = p.residual != nullptr, rms = p.gamma != nullptr;
+            if (hb && hr)
+                return rms ? launch_instance<TM, TN, false, true, true, true>(stream, p, grid)
+                           : launch_instance<TM, TN, false, true, true, false>(stream, p, grid);
+            if (hb)
+                return rms ? launch_instance<TM, TN, false, true, false, true>(stream, p, grid)
+                           : launch_instance<TM, TN, false, true, false, false>(stream, p, grid);
+            if (hr)
+                return rms ? launch_instance<TM, TN, false, false, true, true>(stream, p, grid)
+                           : launch_instance<TM, TN, false, false, true, false>(stream, p, grid);
+            return rms ? launch_instance<TM, TN, false, false, false, true>(stream, p, grid)
+                       : launch_instance<TM, TN, false, false, false, false>(stream, p, grid);
+        }
     } // namespace gemm_sk
 
-    // one per tile height (w4a16_gemm_sk_32.hip ... _256.hip)
+    // one per tile height (w4a16_gemm_sk_32.hip ... _256.hip); narrow: 128 x 128 tiles, plain product, bias, residual, RMSNorm
+    hipError_t launch_gemm_sk_64_narrow(hipStream_t stream, const SkGemmParams& p, int grid);
+    hipError_t launch_gemm_sk_128_narrow(hipStream_t stream, const SkGemmParams& p, int grid);
+    hipError_t launch_gemm_sk_256_narrow(hipStream_t stream, const SkGemmParams& p, int grid);
     hipError_t launch_gemm_sk_32(hipStream_t stream, const SkGemmParams& p, int grid, bool gate);
     hipError_t launch_gemm_sk_64(hipStream_t stream, const SkGemmParams& p, int grid, bool gate);
     hipError_t launch_gemm_sk_128(hipStream_t stream, const SkGemmParams& p, int grid, bool gate);

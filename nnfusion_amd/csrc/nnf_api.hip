@@ -142,7 +142,8 @@ namespace
             return (int)nnf::launch_w4a16_gemv(s, A, Wq, scales, Y, M, N, K, zp, dev.num_cu);
         }
         const nnf::workspace::W4A16Route route =
-            nnf::workspace::route_w4a16(M, N, K, false, false, false, dev.num_cu, choice.path, choice.tile_rows, choice.k_parts);
+            nnf::workspace::route_w4a16(M, N, K, false, false, false, dev.num_cu, choice.path, choice.tile_rows, choice.k_parts,
+                                        choice.tile_cols);
         if (route.kind == nnf::workspace::W4A16Route::NONE)
             return NNF_ERR_UNSUPPORTED_SHAPE;
         // the GEMV kernels over ranges of K and the tile GEMM park partial sums in scratch memory; the check is for
@@ -238,7 +239,7 @@ size_t nnf_w4a16_gemm_variant_workspace_bytes(int M, int N, int K, int group, in
     if (variant == NNF_W4A16_GEMV_VALU || group != 128)
         return 0;
     return nnf::workspace::route_w4a16(M, N, K, false, false, false, nnf::workspace::PLAN_CUS, variant, choice.tile_rows,
-                                       choice.k_parts)
+                                       choice.k_parts, choice.tile_cols)
         .partial_bytes;
 }
 
@@ -280,7 +281,7 @@ int nnf_w4a16_gemm_fused_variant(nnf_stream_t stream, const void* A, const void*
         return st;
     const nnf::workspace::W4A16Route route =
         nnf::workspace::route_w4a16(M, N, K, act == NNF_ACT_SILU_GATE, rms_gamma != nullptr, residual == Y, dev.num_cu,
-                                    choice.path, choice.tile_rows, choice.k_parts);
+                                    choice.path, choice.tile_rows, choice.k_parts, choice.tile_cols);
     if (route.kind == nnf::workspace::W4A16Route::NONE)
         return NNF_ERR_UNSUPPORTED_SHAPE;
     // [ RMSNorm scratch ][ what this launch parks, on this device ]

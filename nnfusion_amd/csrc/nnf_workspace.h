@@ -112,7 +112,8 @@ namespace nnf
         }
 
         // ---- plan of the fp16 x int4 tile GEMM (w4a16_gemm_sk.h) ----------------------------------------------
-        // Tiles of tile_rows x 256 weight rows (SiLU-gate: 128 gate + 128 up rows, i.e. 128 output columns); the
+        // Tiles of tile_rows x 256 weight rows (SiLU-gate: 128 gate + 128 up rows, i.e. 128 output columns) or, for
+        // the products without SiLU-gate, tile_rows x 128; the
         // (tile, superstep of 256 k) units of the whole product are split evenly over `grid` workgroups, one per CU.
         // A tile whose units belong to more than one workgroup is summed through the workspace: slots of
         // tile_rows x 256 fp32; workgroup v parks the first segment of its range in slot v and a later one in slot
@@ -120,23 +121,46 @@ namespace nnf
         struct SkPlan
         {
             int tile_rows = 0; // 32, 64, 128 or 256
+            int tile_weight_rows = 256; // weight rows of a tile: 256, or 128 (narrow tiles: plain product only)
             int tiles_m = 0, tiles_n = 0;
             int supersteps = 0; // per tile: ceil(K / 256)
             long long units = 0;
             int grid = 0;
             int slots = 0;     // 0: every tile belongs to one workgroup (no workspace, no second launch)
-            size_t bytes() const { return (size_t)slots * tile_rows * 256 * sizeof(float); }
+            size_t bytes() const { return (size_t)slots * tile_rows * tile_weight_rows * sizeof(float); }
         };
+        // Tile shape.  What the caller fixes (forced_rows 32 / 64 / 128 / 256, forced_cols 128 / 256) is kept, the rest
+        // is chosen by M (measured at N = K = 8192 and on the Llama shapes, alternating the candidates in one process):
+        // 256-row tiles touch every weight once per 256 rows and are the fastest from about 1500 rows on; below, with
+        // every output tile shared by several workgroups, tiles of 128 columns halve what each of them parks and are
+        // 6-14 % faster (M = 64: 26.5 -> 22.8 us, 128: 35.7 -> 30.8, 512: 83 -> 76, 1024: 134 -> 123) although an
+        // activation fragment then feeds one MFMA instead of two; 256 rows where M fills them to within an eighth,
+        // else 128.  SiLU-gate needs the gate | up halves of a 256-row weight tile; 32-row tiles exist 256 wide only.
+        inline void sk_tile_shape(int M, bool gate, int forced_rows, int forced_cols, int& rows, int& cols)
+        {
+            const bool rows_forced = forced_rows == 32 || forced_rows == 64 || forced_rows == 128 || forced_rows == 256;
+            if (rows_forced)
+            {
+                rows = forced_rows;
+                cols = (forced_cols == 128 && !gate && rows != 32) ? 128 : 256;
+                return;
+            }
+            cols = 256;
+            if (gate || M <= 32 || M > 1536)
+                rows = M <= 32 ? 32 : M <= 64 ? 64 : M <= 1536 ? 128 : 256;
+            else
+            {
+                const int padded = ceil_div(M, 256) * 256;
+                rows = M <= 64 ? 64 : M <= 128 ? 128 : ((padded - M) * 8 <= M ? 256 : 128);
+                cols = forced_cols == 256 ? 256 : 128;
+            }
+        }
         // tiles_n column tiles, `per_tile` units of K per tile, at least `min_units` units per workgroup (unless forced);
-        // forced_tile_rows / forced_grid: 0 = the plan's own choice
+        // forced_grid: 0 = the plan's own choice
         inline SkPlan plan_sk(int M, int tiles_n, int per_tile, int min_units, int num_cu, int forced_tile_rows, int forced_grid)
         {
             SkPlan p;
-            // 256-row tiles touch every weight once per 256 rows and are the fastest from about 1500 rows on; below,
-            // 128-row tiles (twice the tiles, half as large parked sums per workgroup) measured 5-20 % faster
-            int rows = M <= 32 ? 32 : M <= 64 ? 64 : M <= 1536 ? 128 : 256;
-            if (forced_tile_rows == 32 || forced_tile_rows == 64 || forced_tile_rows == 128 || forced_tile_rows == 256)
-                rows = forced_tile_rows;
+            const int rows = forced_tile_rows;
             p.tile_rows = rows;
             p.tiles_m = ceil_div(M, rows);
             p.tiles_n = tiles_n;
@@ -165,21 +189,28 @@ namespace nnf
             return p;
         }
         // fp16 x int4: units of 256 k (supersteps), a workgroup keeps at least two (eight K steps of 64)
-        inline SkPlan plan_w4a16_sk(int M, int N, int K, bool gate, int num_cu, int forced_tile_rows = 0, int forced_grid = 0)
+        // forced_tile_rows / forced_cols: 0 = the plan's own choice (sk_tile_shape)
+        inline SkPlan plan_w4a16_sk(int M, int N, int K, bool gate, int num_cu, int forced_tile_rows = 0, int forced_grid = 0,
+                                    int forced_cols = 0)
         {
             if (M <= 0 || N <= 0 || K < 128 || num_cu < 1)
                 return SkPlan();
-            return plan_sk(M, ceil_div(N, gate ? 128 : 256), (K / 128 + 1) / 2, 2, num_cu, forced_tile_rows, forced_grid);
+            int rows, cols;
+            sk_tile_shape(M, gate, forced_tile_rows, forced_cols, rows, cols);
+            SkPlan p = plan_sk(M, ceil_div(N, (gate || cols == 128) ? 128 : 256), (K / 128 + 1) / 2, 2, num_cu, rows, forced_grid);
+            p.tile_weight_rows = cols;
+            return p;
         }
 
         // the plan with a forced tile height (0 = the plan's own) and a forced number of workgroups per tile (0 = the
         // plan's own grid)
-        inline SkPlan plan_w4a16_sk_with(int M, int N, int K, bool gate, int num_cu, int tile_rows, int workgroups_per_tile)
+        inline SkPlan plan_w4a16_sk_with(int M, int N, int K, bool gate, int num_cu, int tile_rows, int workgroups_per_tile,
+                                         int tile_cols = 0)
         {
             if (workgroups_per_tile <= 0)
-                return plan_w4a16_sk(M, N, K, gate, num_cu, tile_rows, 0);
-            const SkPlan t = plan_w4a16_sk(M, N, K, gate, num_cu, tile_rows, 0);
-            return plan_w4a16_sk(M, N, K, gate, num_cu, tile_rows, t.tiles_m * t.tiles_n * workgroups_per_tile);
+                return plan_w4a16_sk(M, N, K, gate, num_cu, tile_rows, 0, tile_cols);
+            const SkPlan t = plan_w4a16_sk(M, N, K, gate, num_cu, tile_rows, 0, tile_cols);
+            return plan_w4a16_sk(M, N, K, gate, num_cu, tile_rows, t.tiles_m * t.tiles_n * workgroups_per_tile, tile_cols);
         }
 
         // ---- plan of the skinny (M <= 16) MFMA GEMV kernel ---------------------------------------------
@@ -585,7 +616,7 @@ namespace nnf
         // is the output buffer itself.  path: 0 the library's order of preference, 2 / 4 one family of GEMV kernels only
         // (values of nnf_w4a16_variant), 3 the tile GEMM with tile_rows / k_parts (0: its own plan).
         inline W4A16Route route_w4a16(int M, int N, int K, bool gate, bool rms, bool in_place_residual, int num_cu, int path = 0,
-                                      int tile_rows = 0, int k_parts = 0)
+                                      int tile_rows = 0, int k_parts = 0, int tile_cols = 0)
         {
             W4A16Route r;
             if (M <= 0 || N <= 0 || K < 128 || (K & 127) || num_cu < 1)
@@ -632,7 +663,7 @@ namespace nnf
                     return r;
             }
             r.kind = W4A16Route::TILE;
-            r.plan = plan_w4a16_sk_with(M, N, K, gate, num_cu, tile_rows, k_parts);
+            r.plan = plan_w4a16_sk_with(M, N, K, gate, num_cu, tile_rows, k_parts, tile_cols);
             r.partial_bytes = r.plan.bytes();
             r.rms_bytes = rstd_bytes;
             return r;

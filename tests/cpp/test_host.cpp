@@ -1047,7 +1047,10 @@ int main(int argc, char** argv)
                     EXPECT(p.grid >= 1 && p.grid <= 256 && p.units / p.grid >= 2);
                     EXPECT(p.tiles_m * p.tile_rows >= m && (p.tiles_m - 1) * p.tile_rows < m);
                     EXPECT(p.slots == 0 || p.slots == p.grid || p.slots == 2 * p.grid);
-                    EXPECT(p.bytes() == (size_t)p.slots * p.tile_rows * 256 * 4);
+                    // tiles of 128 columns for the plain product up to 1536 rows (not for 32-row tiles), else 256 weight rows
+                    EXPECT(p.tile_weight_rows == ((gate || m <= 32 || m > 1536) ? 256 : 128));
+                    EXPECT(p.tiles_n == 8192 / ((gate || p.tile_weight_rows == 128) ? 128 : 256));
+                    EXPECT(p.bytes() == (size_t)p.slots * p.tile_rows * p.tile_weight_rows * 4);
                     // every unit has exactly one owner, and owners follow each other
                     long long covered = 0;
                     for (int v = 0; v < p.grid; ++v)
@@ -1057,6 +1060,13 @@ int main(int argc, char** argv)
             const auto big = ws::plan_w4a16_sk(4096, 8192, 8192, false, 256);
             EXPECT(big.tile_rows == 256 && big.grid == 256 && big.slots == 0 && big.bytes() == 0);
             EXPECT(ws::plan_w4a16_sk(128, 8192, 8192, false, 256).slots > 0);
+            // 256 rows where M fills them to within an eighth, else 128; what a caller fixes is kept
+            EXPECT(ws::plan_w4a16_sk(1024, 8192, 8192, false, 256).tile_rows == 256 && ws::plan_w4a16_sk(300, 8192, 8192, false, 256).tile_rows == 128);
+            EXPECT(ws::plan_w4a16_sk(480, 8192, 8192, false, 256).tile_rows == 256 && ws::plan_w4a16_sk(100, 8192, 8192, false, 256).tile_rows == 128);
+            const auto forced = ws::plan_w4a16_sk(1024, 8192, 8192, false, 256, 128, 0, 256);
+            EXPECT(forced.tile_rows == 128 && forced.tile_weight_rows == 256 && forced.tiles_n == 32);
+            EXPECT(ws::plan_w4a16_sk(1024, 8192, 8192, true, 256, 128, 0, 128).tile_weight_rows == 256); // SiLU-gate: full tiles
+            EXPECT(ws::plan_w4a16_sk(4096, 8192, 8192, false, 256, 0, 0, 128).tile_weight_rows == 256);  // width alone: the plan's
             // K = 128 * odd: the last superstep of a tile holds one group
             EXPECT(ws::plan_w4a16_sk(64, 512, 384, false, 256).supersteps == 2);
         }

@@ -32,13 +32,14 @@ def _check(y, ref, tol=TOL):
 
 
 # Plans of the MFMA tile GEMM, passed per call through nnf_w4a16_gemm_variant / nnf_w4a16_gemm_fused_variant (struct
-# nnf_plan): None = the library's own choice of kernel and plan; otherwise (tile_rows, k_parts): tiles of 256, 128, 64 or
-# 32 rows by 256 columns, and the number of workgroups that share a tile (each a part of K; parts parked in the workspace
-# and added by the second launch)
-PLANS = [None, (256, 1), (256, 2), (128, 1), (128, 3), (64, 1), (64, 2), (32, 1), (32, 3)]
+# nnf_plan): None = the library's own choice of kernel and plan; otherwise (tile_rows, k_parts[, tile_cols]): tiles of
+# 256, 128, 64 or 32 rows by 256 columns (128 where given: products without SiLU-gate), and the number of workgroups that
+# share a tile (each a part of K; parts parked in the workspace and added by the second launch)
+PLANS = [None, (256, 1, 256), (256, 2, 256), (128, 1, 256), (128, 3, 256), (64, 1, 256), (64, 2, 256), (32, 1), (32, 3),
+         (256, 1, 128), (256, 3, 128), (128, 1, 128), (128, 2, 128), (64, 1, 128), (64, 3, 128)]
 
 
-@pytest.fixture(params=PLANS, ids=lambda p: "auto" if p is None else f"rows{p[0]}-parts{p[1]}")
+@pytest.fixture(params=PLANS, ids=lambda p: "auto" if p is None else "rows%d-parts%d" % p[:2] + ("-cols%d" % p[2] if len(p) > 2 else ""))
 def plan(request):
     """Keyword arguments for ops.w4a16_gemm_fused / _gemm below."""
     return {} if request.param is None else {"variant": "gemm_mfma", "plan": request.param}
