@@ -70,13 +70,27 @@ namespace nnf
     // Workgroup b owns rows_q outputs (one more for b < rows_r), contiguous.
     // EPI: 0 plain; 1 the optional parts of `f` (RMSNorm: gamma onto the activations, rstd onto the sums; bias;
     // residual); 2 SiLU-gate (N outputs from 2 N weight rows: the workgroup walks the gate rows of its outputs, then
-    // their up rows N further down; scales: two blocks in LDS) with the optional RMSNorm.
+    // their up rows N further down; scales: two blocks in LDS) with the optional RMSNorm; 4 and 3: other block
+    // parameters, pack = zp | log2(KSW) << 8 | log2(group) << 16 with groups of 32 / 64 / 128 (a lane's 32 weights of a
+    // load lie in one group whatever its size: only the place of its scale changes) and, for 3, a zero point per
+    // (row, group) in `zps`, u8 [N, (K / group + 1) / 2], even group in the low nibble.  With the weights of a row a
+    // wavefront then fetches the bytes that hold the zero points of its K segment (one byte per lane, global -> LDS like
+    // the weights: 256 bytes more per ring slot and 64 groups, waited for with the weights), and the constant part of a
+    // lane's sum becomes  base - z (sum of the lane's activations),  base the constant for z = 0; both stay in registers.
     template <int SEG, int D, int WAVES, int EPI>
     __device__ __forceinline__ void gemv_rows_body(const half_t* __restrict__ A, const uint8_t* __restrict__ Wq,
                                                    const half_t* __restrict__ S, half_t* __restrict__ Y, int N, int K,
-                                                   int rows_q, int rows_r, int pack, const GemvFusionArgs& f)
+                                                   int rows_q, int rows_r, int pack, const GemvFusionArgs& f,
+                                                   const uint8_t* __restrict__ zps = nullptr)
     {
         constexpr bool GATE = EPI == 2;
+        constexpr bool QZT = EPI == 3;            // zero points from `zps`
+        constexpr bool QG = EPI == 3 || EPI == 4; // group size from `pack`
+        constexpr int ZL = QZT ? (SEG + 1) / 2 : 0; // loads of zero points per row and wavefront (64 bytes = 128 groups each;
+                                                    // a segment of SEG KiB of weights has at most 64 SEG groups)
+        constexpr int LPR = SEG + ZL;               // vector-memory loads per row and wavefront
+        constexpr int SLOT_BYTES = SEG * 1024 + ZL * 256;
+        const int gshift = QG ? (pack >> 16) : 7;
         extern __shared__ uintx4 lds[];
         uint32_t MAGIC, MAGIC_HI, MASK_LO, MASK_HI;
         asm volatile("v_mov_b32 %0, 0x64006400" : "=v"(MAGIC));
@@ -86,7 +100,7 @@ namespace nnf
         const int tid = threadIdx.x;
         const int lane = tid & 63;
         const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-        const int zp = pack & 0xff, kshift = pack >> 8;
+        const int zp = pack & 0xff, kshift = QG ? (pack >> 8) & 0xff : pack >> 8;
         const int ksw = 1 << kshift;
         const int kpart = wave & (ksw - 1);
         const int gpw = WAVES >> kshift; // wavefronts per K segment
@@ -95,7 +109,7 @@ namespace nnf
         const int n_out = rows_q + ((int)blockIdx.x < rows_r ? 1 : 0); // >= 1: the grid never exceeds N
         const int n_rows = GATE ? 2 * n_out : n_out;                   // weight rows this workgroup walks
         const uint32_t row_bytes = (uint32_t)K >> 1;
-        const int G = K >> 7;
+        const int G = K >> gshift;
         const int a_units = K >> 3;
         const int a_pad = (a_units + 63) & ~63; // whole wavefront-wide loads of activations
         const int sc_bytes = n_out * G * 2;     // this workgroup's block of S (GATE: one such block for the gate rows,
@@ -105,10 +119,11 @@ namespace nnf
         auto phys_row = [&](int r) { return (GATE && r >= n_out) ? N + out0 + (r - n_out) : out0 + r; };
 
         uint8_t* lds_bytes = reinterpret_cast<uint8_t*>(lds);
-        uint8_t* ring = lds_bytes + wave * (D * SEG * 1024);
-        uintx4* act = lds + (WAVES * D * SEG * 1024) / 16;
+        uint8_t* ring = lds_bytes + wave * (D * SLOT_BYTES);
+        uintx4* act = lds + (WAVES * D * SLOT_BYTES) / 16;
         float* corr = reinterpret_cast<float*>(act + a_pad + 4);
-        uint8_t* scales = reinterpret_cast<uint8_t*>(corr + a_pad + 4);
+        float* asum_u = corr + a_pad + 4; // QZT: one fp32 per unit, the sum of its eight activations
+        uint8_t* scales = reinterpret_cast<uint8_t*>(corr + (QZT ? 2 : 1) * (a_pad + 4));
         float* outb = reinterpret_cast<float*>(scales + (GATE ? 2 : 1) * sc_block);
         int* next_row = reinterpret_cast<int*>(outb + (((GATE ? 2 : 1) * (rows_q + 1)) << kshift));
         float* sum_sq = reinterpret_cast<float*>(next_row + 8); // per wavefront: its share of sum a^2 (RMSNorm inside the kernel)
@@ -168,13 +183,41 @@ namespace nnf
             valid[j] = b < row_bytes;
             w_off[j] = min(b, row_bytes - 16u);
         }
+        // zero points: the first byte of this wavefront's K segment in a row of `zps` (a segment starts at an even
+        // group), the byte each lane fetches (past the end of the row: its last byte), and where a lane finds the zero
+        // point of its load j afterwards: byte (one per lane and four bytes of LDS) and nibble
+        const int zp_stride = (G + 1) >> 1;
+        const int g_seg0 = (kpart * SEG * 2048) >> gshift;
+        uint32_t z_off[ZL > 0 ? ZL : 1], z_rd[SEG], z_sh[SEG];
+        if constexpr (QZT)
+        {
+#pragma unroll
+            for (int i = 0; i < ZL; ++i)
+                z_off[i] = (uint32_t)min((g_seg0 >> 1) + i * 64 + lane, zp_stride - 1);
+#pragma unroll
+            for (int j = 0; j < SEG; ++j)
+            {
+                const int g = min(g_seg0 + ((j * 2048 + lane * 32) >> gshift), G - 1);
+                z_rd[j] = (uint32_t)((g >> 1) - (g_seg0 >> 1)) * 4u;
+                z_sh[j] = (uint32_t)(g & 1) * 4u;
+            }
+        }
         // weights of row r (relative to the workgroup's first; rows past the end re-read the last row) -> ring slot
         auto issue = [&](int r, int slot) {
-            const uint8_t* src = Wq + (size_t)phys_row(min(r, n_rows - 1)) * row_bytes;
+            const int row = phys_row(min(r, n_rows - 1));
+            const uint8_t* src = Wq + (size_t)row * row_bytes;
 #pragma unroll
             for (int j = 0; j < SEG; ++j)
                 __builtin_amdgcn_global_load_lds((global_ptr_t)(src + w_off[j]),
-                                                 (lds_ptr_t)(ring + (slot * SEG + j) * 1024), 16, 0, 0);
+                                                 (lds_ptr_t)(ring + slot * SLOT_BYTES + j * 1024), 16, 0, 0);
+            if constexpr (QZT)
+            {
+                const uint8_t* zsrc = zps + (size_t)row * zp_stride;
+#pragma unroll
+                for (int i = 0; i < ZL; ++i)
+                    __builtin_amdgcn_global_load_lds((global_ptr_t)(zsrc + z_off[i]),
+                                                     (lds_ptr_t)(ring + slot * SLOT_BYTES + SEG * 1024 + i * 256), 1, 0, 0);
+            }
         };
         // (two rows now; the rest of the ring after the activations are in registers: with everything asked for at
         // once the last wavefronts stall at issue -- a CU takes about 64 wavefront-wide loads -- and hold up the barrier)
@@ -189,23 +232,26 @@ namespace nnf
         {
             act[a_pad + tid] = uintx4{0u, 0u, 0u, 0u};
             corr[a_pad + tid] = 0.f;
+            if (QZT)
+                asum_u[a_pad + tid] = 0.f;
         }
         // where the lane finds the scale of its load j in a row of scales (a lane past the end of K: the last one)
         uint32_t s_rd[SEG];
 #pragma unroll
         for (int j = 0; j < SEG; ++j)
-            s_rd[j] = (uint32_t)min(kpart * SEG * 16 + j * 16 + (lane >> 2), G - 1) * 2u;
+            s_rd[j] = QG ? (uint32_t)min((kpart * SEG * 2048 + j * 2048 + lane * 32) >> gshift, G - 1) * 2u
+                         : (uint32_t)min(kpart * SEG * 16 + j * 16 + (lane >> 2), G - 1) * 2u;
 
         // ---- activations: prepared once per workgroup, then LDS -> registers ------------------------------
         // A lane of a fetching wavefront gets back exactly the unit it asked for (no barrier needed for that):
         // it stores the unit as (a0,a4) (a1,a5) (a2,a6) (a3,a7) and, next to it, the unit's part of the
         // constant  (1024 + zp) sum a_even + (64 + zp) sum a_odd  that the nibble trick adds to every row.
         // Only the weights asked for above may still be in flight afterwards: the scales have landed too.
-        __builtin_amdgcn_s_waitcnt(rows_vmcnt(D0 * SEG));
+        __builtin_amdgcn_s_waitcnt(rows_vmcnt(D0 * LPR));
         if (a_loader)
         {
-            const float ce = -(1024.0f + (float)zp);
-            const float co = -(64.0f + (float)zp);
+            const float ce = -(1024.0f + (QZT ? 0.f : (float)zp));
+            const float co = -(64.0f + (QZT ? 0.f : (float)zp));
             float ss = 0.f;
             int e = 0;
             for (int u0 = wave * 64; u0 < a_units; u0 += WAVES * 64, ++e)
@@ -241,6 +287,8 @@ namespace nnf
                 const float so = ((float)y.x + (float)y.y) + ((float)w.x + (float)w.y);
                 act[u] = a;
                 corr[u] = ce * se + co * so;
+                if (QZT)
+                    asum_u[u] = se + so;
             }
             if (own_rstd)
             {
@@ -253,7 +301,7 @@ namespace nnf
         }
         lds_barrier();
         uintx4 areg[SEG][4];
-        float ncorr[SEG];
+        float ncorr[SEG], asum[SEG];
 #pragma unroll
         for (int j = 0; j < SEG; ++j)
         {
@@ -261,6 +309,11 @@ namespace nnf
             const int u0 = valid[j] ? (int)((seg_byte0 + j * 1024 + lane * 16) >> 2) : a_pad;
             const floatx4 c4 = *reinterpret_cast<const floatx4*>(corr + u0);
             ncorr[j] = (c4.x + c4.y) + (c4.z + c4.w);
+            if constexpr (QZT)
+            {
+                const floatx4 s4 = *reinterpret_cast<const floatx4*>(asum_u + u0);
+                asum[j] = (s4.x + s4.y) + (s4.z + s4.w);
+            }
 #pragma unroll
             for (int d = 0; d < 4; ++d)
                 areg[j][d] = act[u0 + d];
@@ -269,14 +322,16 @@ namespace nnf
         // ---- rows -------------------------------------------------------------------------------------
         const uint32_t lane16 = (uint32_t)lane * 16u;
         uintx4 wv[SEG];
-        float sv[SEG];
+        float sv[SEG], zv[SEG];
         auto read_slot = [&](int r, int slot) {
             const uint8_t* sc_row = scales + ((GATE && r >= n_out) ? sc_block + (r - n_out) * (G * 2) : r * (G * 2));
 #pragma unroll
             for (int j = 0; j < SEG; ++j)
             {
-                wv[j] = *reinterpret_cast<const uintx4*>(ring + (slot * SEG + j) * 1024 + lane16);
+                wv[j] = *reinterpret_cast<const uintx4*>(ring + slot * SLOT_BYTES + j * 1024 + lane16);
                 sv[j] = (float)*reinterpret_cast<const half_t*>(sc_row + s_rd[j]);
+                if constexpr (QZT)
+                    zv[j] = (float)(((uint32_t)ring[slot * SLOT_BYTES + SEG * 1024 + z_rd[j]] >> z_sh[j]) & 15u);
             }
         };
         auto compute = [&](int r) {
@@ -286,6 +341,8 @@ namespace nnf
             {
                 const uint32_t ww[4] = {wv[j].x, wv[j].y, wv[j].z, wv[j].w};
                 float t = ncorr[j];
+                if constexpr (QZT)
+                    t = __builtin_fmaf(-zv[j], asum[j], t);
 #pragma unroll
                 for (int d = 0; d < 4; ++d)
                 {
@@ -335,7 +392,7 @@ namespace nnf
                         int nx = 0;
                         if (lane == 0)
                             asm volatile("ds_add_rtn_u32 %0, %1, %2" : "=v"(nx) : "v"(next_addr), "v"(1) : "memory");
-                        __builtin_amdgcn_s_waitcnt(rows_vmcnt((D - 1) * SEG));
+                        __builtin_amdgcn_s_waitcnt(rows_vmcnt((D - 1) * LPR));
                         read_slot(in_slot[slot], slot);
                         // the slot has been read before it is refilled
                         asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(nx)::"memory");
@@ -363,7 +420,7 @@ namespace nnf
                 int slot = exit_slot + 1 + t;
                 slot = slot >= D ? slot - D : slot;
                 const int row = __builtin_amdgcn_readlane(rows_by_slot, slot);
-                __builtin_amdgcn_s_waitcnt(rows_vmcnt((D - 2 - t) * SEG));
+                __builtin_amdgcn_s_waitcnt(rows_vmcnt((D - 2 - t) * LPR));
                 read_slot(row, slot);
                 compute(row);
             });
@@ -385,7 +442,7 @@ namespace nnf
             float y = 0.f;
             for (int kp = 0; kp < ksw; ++kp)
                 y += outb[(r << kshift) + kp];
-            if (EPI == 0)
+            if (EPI == 0 || QG)
                 Y[out0 + r] = (half_t)y;
             else if (EPI == 1)
                 Y[out0 + r] = finish_bias_residual(y * rs, f.bias, out0 + r, f.residual, (size_t)(out0 + r));
@@ -422,9 +479,44 @@ namespace nnf
         gemv_rows_body<SEG, D, WAVES, EPI>(A, Wq, S, Y, N, K, rows_q, rows_r, pack, f);
     }
 
+    // Other block parameters (EPI 4: group size; 3: a zero point per (row, group) as well).  Sixteen dwords of arguments,
+    // like the plain kernel.
+    template <int SEG, int D, int WAVES, int EPI>
+    __global__ __launch_bounds__(WAVES * 64) void w4a16_gemv_rows_q_kernel(const half_t* __restrict__ A,
+                                                                           const uint8_t* __restrict__ Wq,
+                                                                           const half_t* __restrict__ S,
+                                                                           half_t* __restrict__ Y, int N, int K,
+                                                                           int rows_q, int rows_r, int pack,
+                                                                           const uint8_t* __restrict__ zps)
+    {
+        static_assert(EPI == 3 || EPI == 4, "the plain kernel is w4a16_gemv_rows_kernel");
+        gemv_rows_body<SEG, D, WAVES, EPI>(A, Wq, S, Y, N, K, rows_q, rows_r, pack, GemvFusionArgs{nullptr, nullptr, nullptr, nullptr, 0.f}, zps);
+    }
+
     namespace
     {
         using workspace::RowsPlan;
+
+        template <int SEG, int D, int WAVES, int EPI>
+        hipError_t launch_rows_q(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int N, int K,
+                                 int zp, int group_shift, const void* zps, const RowsPlan& p, int grid)
+        {
+            const size_t lds_total = p.lds_bytes(N, K, grid, false, group_shift, EPI == 3);
+            if (lds_total > MAX_LDS_BYTES)
+                return hipErrorInvalidValue;
+            if (lds_total > 64 * 1024)
+            {
+                static LdsGrant granted;
+                const hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(&w4a16_gemv_rows_q_kernel<SEG, D, WAVES, EPI>),
+                                                       granted, (int)MAX_LDS_BYTES);
+                if (e != hipSuccess)
+                    return e;
+            }
+            hipLaunchKernelGGL((w4a16_gemv_rows_q_kernel<SEG, D, WAVES, EPI>), dim3(grid), dim3(WAVES * 64), lds_total, stream,
+                               (const half_t*)A, (const uint8_t*)Wq, (const half_t*)S, (half_t*)Y, N, K, N / grid, N % grid,
+                               zp | (p.kshift << 8) | (group_shift << 16), (const uint8_t*)zps);
+            return hipGetLastError();
+        }
 
         template <int SEG, int D, int WAVES, int EPI>
         hipError_t launch_rows(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int N, int K,
@@ -479,6 +571,39 @@ namespace nnf
         return epi == 0   ? launch_rows<SEG, D, workspace::ROWS_WAVES, 0>(stream, A, Wq, S, Y, N, K, zp, p, grid, fusion)  \
                : epi == 1 ? launch_rows<SEG, D, workspace::ROWS_WAVES, 1>(stream, A, Wq, S, Y, N, K, zp, p, grid, fusion)  \
                           : launch_rows<SEG, D, workspace::ROWS_WAVES, 2>(stream, A, Wq, S, Y, N, K, zp, p, grid, fusion);
+            NNF_ROWS_CASE(1, 1)
+            NNF_ROWS_CASE(1, 2)
+            NNF_ROWS_CASE(1, 3)
+            NNF_ROWS_CASE(1, 4)
+            NNF_ROWS_CASE(2, 1)
+            NNF_ROWS_CASE(2, 2)
+            NNF_ROWS_CASE(2, 3)
+            NNF_ROWS_CASE(2, 4)
+            NNF_ROWS_CASE(3, 1)
+            NNF_ROWS_CASE(3, 2)
+#undef NNF_ROWS_CASE
+        default: return hipErrorInvalidValue;
+        }
+    }
+
+    bool w4a16_gemv_rows_q_supported(int M, int N, int K, int group_shift, bool zero_points, int num_cu)
+    {
+        return workspace::plan_w4a16_rows(M, N, K, num_cu, 0, false, group_shift, zero_points).seg != 0;
+    }
+
+    hipError_t launch_w4a16_gemv_rows_q(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int N,
+                                        int K, int group_shift, int zp, const void* zero_points, int num_cu)
+    {
+        const RowsPlan p = workspace::plan_w4a16_rows(1, N, K, num_cu, 0, false, group_shift, zero_points != nullptr);
+        const int grid = workspace::rows_grid(N, num_cu);
+        switch (p.seg * 10 + p.depth)
+        {
+#define NNF_ROWS_CASE(SEG, D)                                                                                          \
+    case SEG * 10 + D:                                                                                                 \
+        return zero_points ? launch_rows_q<SEG, D, workspace::ROWS_WAVES, 3>(stream, A, Wq, S, Y, N, K, zp, group_shift,  \
+                                                                            zero_points, p, grid)                       \
+                           : launch_rows_q<SEG, D, workspace::ROWS_WAVES, 4>(stream, A, Wq, S, Y, N, K, zp, group_shift,  \
+                                                                            nullptr, p, grid);
             NNF_ROWS_CASE(1, 1)
             NNF_ROWS_CASE(1, 2)
             NNF_ROWS_CASE(1, 3)

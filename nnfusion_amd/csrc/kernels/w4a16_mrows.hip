@@ -397,6 +397,212 @@ namespace nnf
         mrows_flush<FUSED, MB>(parked, Y, t0, T_out, M, N, tid, f, gate, own_rstd ? sum_sq : nullptr, K);
     }
 
+    // ---- other block parameters ------------------------------------------------------------------------------------
+    // The same kernel for groups of 2^GSHIFT = 32 / 64 / 128 weights and (ZPT) a zero point per (row, group) from
+    // `zps`, u8 [N, K / group / 2], even group in the low nibble; 2 <= M <= 16, K = GW * 2048 (two steps per tile).
+    // A lane's 16-byte piece of a weight row (32 weights) lies in one group whatever its size, but the four lanes that meet
+    // in one MFMA column hold pieces of up to four groups: a scale cannot be applied to the MFMA's sum.  The weights
+    // are therefore dequantised before the MFMA, as the tile GEMM does:  fp16((q - z) * s),  q - z exact (nibble trick
+    // plus -(1024 + z) or -(64 + z), which is the same trick applied to z with the sign bit set), one rounding in the
+    // product; the accumulators take the MFMA results as they are.
+    // Per step a wavefront fetches, next to its weights, the SPR = GW * 128 / group scales of each of the 16 rows (4-byte
+    // loads, NSL of them) and, ZPT, their zero points (one byte per lane, NZL loads; a byte load lands in a lane's four
+    // bytes of LDS).
+    // LDS (bytes): weights [8 wavefronts][2 slots][GW KiB] | scales and zero points [8][2][(NSL + NZL) x 256] |
+    //              partial tiles [2][8][1 KiB] | parked sums [tiles of the workgroup][M][16] fp32
+    // pack = M | zp << 8.
+    template <int GW, int GSHIFT, bool ZPT>
+    __global__ __launch_bounds__(512) void w4a16_mrows_q_kernel(const half_t* __restrict__ A, const uint8_t* __restrict__ Wq,
+                                                                const half_t* __restrict__ S, half_t* __restrict__ Y,
+                                                                const uint8_t* __restrict__ zps, int N, int tiles_q,
+                                                                int tiles_r, int pack)
+    {
+        static_assert(GW == 1 || GW == 2 || GW == 4, "K = 2048, 4096, 8192");
+        static_assert(GSHIFT >= 5 && GSHIFT <= 7 && ((GW << (7 - GSHIFT)) & 1) == 0, "whole words of scales, whole bytes of zero points");
+        constexpr int STEPS = 2, MB = 1;
+        constexpr int K = GW * STEPS * 1024, G = K >> GSHIFT;
+        constexpr int GA = GW * STEPS;         // groups of 128 of a wavefront
+        constexpr int ROW_BYTES = K / 2;       // a weight row
+        constexpr int SLICE = GW * 64;         // a wavefront's bytes of a weight row per step
+        constexpr int SPAN = 8 * SLICE;        // bytes of a weight row that the workgroup covers per step
+        constexpr int TILE_BYTES = 16 * SLICE; // = GW KiB: GW wavefront-wide loads
+        constexpr int SPR = GW << (7 - GSHIFT); // scales per row, step and wavefront
+        constexpr int WPR = SPR / 2;            // ... as 4-byte words = bytes of zero points
+        constexpr int NSL = (16 * WPR + 63) / 64;
+        constexpr int NZL = ZPT ? NSL : 0;
+        constexpr int AUX = (NSL + NZL) * 256;
+        constexpr int LT = GW + NSL + NZL;      // loads per step and wavefront
+        extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+        uint32_t MAGIC, MAGIC_HI, MASK_LO, MASK_HI;
+        asm volatile("v_mov_b32 %0, 0x64006400" : "=v"(MAGIC));
+        asm volatile("v_mov_b32 %0, 0x54005400" : "=v"(MAGIC_HI));
+        asm volatile("s_mov_b32 %0, 0x000F000F" : "=s"(MASK_LO));
+        asm volatile("s_mov_b32 %0, 0x00F000F0" : "=s"(MASK_HI));
+
+        const int tid = threadIdx.x;
+        const int lane = tid & 63;
+        const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+        const int col = lane & 15; // n within the tile (B operand / D column), m for the A operand
+        const int kq = lane >> 4;  // K quarter of the MFMA operands, row quad of D
+        const int M = pack & 0xff, zp = (pack >> 8) & 0xff;
+        const int b = blockIdx.x;
+        const int t0 = b * tiles_q + min(b, tiles_r);
+        const int T = tiles_q + (b < tiles_r ? 1 : 0);
+        auto row0_of = [&](int i) { return __builtin_amdgcn_readfirstlane(min((t0 + i) * 16, N - 16)); };
+
+        uint8_t* ring = smem + wave * (2 * TILE_BYTES);
+        uint8_t* aux = smem + MR_WAVES * 2 * TILE_BYTES + wave * (2 * AUX);
+        uint8_t* red = smem + MR_WAVES * 2 * TILE_BYTES + MR_WAVES * 2 * AUX; // [2][8][1024]
+        float* parked = reinterpret_cast<float*>(red + 2 * MR_WAVES * MB * 1024);
+
+        // weights: as in w4a16_mrows_kernel
+        auto swz = [](int r) { return GW % 4 == 0 ? (r & 15) : GW % 2 == 0 ? (r >> 1) & 7 : (r >> 2) & 3; };
+        uint32_t w_off[GW];
+#pragma unroll
+        for (int c = 0; c < GW; ++c)
+        {
+            const int pos = c * 1024 + 16 * lane;
+            const int r = pos / SLICE, q = (pos % SLICE) >> 4;
+            w_off[c] = (uint32_t)r * ROW_BYTES + (uint32_t)wave * SLICE + (uint32_t)((q ^ swz(r)) << 4);
+        }
+        // scales: lane l of load i fetches word (64 i + l) % WPR of row (64 i + l) / WPR (lanes past the 16 rows: the
+        // last row again); zero points: the same with bytes
+        uint32_t s_off[NSL], z_off[NSL];
+#pragma unroll
+        for (int i = 0; i < NSL; ++i)
+        {
+            const int at = i * 64 + lane;
+            const int r = min(at / WPR, 15), wd = at % WPR;
+            s_off[i] = (uint32_t)r * (G * 2) + (uint32_t)wave * (SPR * 2) + (uint32_t)wd * 4u;
+            z_off[i] = (uint32_t)r * (G / 2) + (uint32_t)wave * WPR + (uint32_t)wd;
+        }
+
+        // step st (0 .. 1) of tile `tile` into slot `slot`
+        auto issue = [&](int tile, int st, int slot) {
+            const uint32_t row0 = (uint32_t)row0_of(tile);
+            const uint8_t* wsrc = Wq + (size_t)row0 * ROW_BYTES + st * SPAN;
+#pragma unroll
+            for (int c = 0; c < GW; ++c)
+                __builtin_amdgcn_global_load_lds((mr_global_ptr_t)(wsrc + w_off[c]),
+                                                 (mr_lds_ptr_t)(ring + slot * TILE_BYTES + c * 1024), 16, 0, 0);
+            const uint8_t* ssrc = reinterpret_cast<const uint8_t*>(S) + (size_t)row0 * (G * 2) + st * (8 * SPR * 2);
+#pragma unroll
+            for (int i = 0; i < NSL; ++i)
+                __builtin_amdgcn_global_load_lds((mr_global_ptr_t)(ssrc + s_off[i]), (mr_lds_ptr_t)(aux + slot * AUX + i * 256), 4, 0, 0);
+            if constexpr (ZPT)
+            {
+                const uint8_t* zsrc = zps + (size_t)row0 * (G / 2) + st * (8 * WPR);
+#pragma unroll
+                for (int i = 0; i < NSL; ++i)
+                    __builtin_amdgcn_global_load_lds((mr_global_ptr_t)(zsrc + z_off[i]),
+                                                     (mr_lds_ptr_t)(aux + slot * AUX + (NSL + i) * 256), 1, 0, 0);
+            }
+        };
+
+        issue(0, 0, 0);
+        issue(0, 1, 1);
+        // activations: straight into the MFMA operand registers, in the pair order of the nibble trick
+        uintx4 areg[MB][GA][4];
+        {
+            const uint8_t* a_bytes = reinterpret_cast<const uint8_t*>(A);
+            const uint32_t a_off = (uint32_t)min(col, M - 1) * (uint32_t)(K * 2) + (uint32_t)wave * (GW * 256) + (uint32_t)kq * 64u;
+#pragma unroll
+            for (int g = 0; g < GA; ++g)
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    areg[0][g][j] = *reinterpret_cast<const uintx4*>(
+                        a_bytes + (size_t)(a_off + (g / GW) * (SPAN * 4) + (g % GW) * 256 + j * 16));
+#pragma unroll
+            for (int g = 0; g < GA; ++g)
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    areg[0][g][j] = permute_a8(areg[0][g][j]);
+        }
+
+        // ---- tile loop ---------------------------------------------------------------------------------------
+        const uint32_t rd_base = (uint32_t)col * SLICE;
+        const int rd_swz = swz(col);
+        const uint32_t red_addr = lds_address(red) + (uint32_t)(wave * (MB * 1024) + lane * 16);
+        const uint32_t parked_addr = lds_address(parked);
+        // the lane's piece of group g of a step lies in scale (g * 128 + kq * 32) >> GSHIFT of the row's SPR
+        uint32_t sc_rd[GW], z_rd[GW], z_sh[GW];
+#pragma unroll
+        for (int g = 0; g < GW; ++g)
+        {
+            const int i = (g * 128 + kq * 32) >> GSHIFT;
+            sc_rd[g] = (uint32_t)(col * SPR + i) * 2u;
+            z_rd[g] = (uint32_t)(NSL * 256 + (col * WPR + (i >> 1)) * 4);
+            z_sh[g] = (uint32_t)(i & 1) * 4u;
+        }
+        const uint32_t zp16 = (uint32_t)zp | ((uint32_t)zp << 16);
+        float one; // a 1.0 the compiler cannot fold
+        asm volatile("v_mov_b32 %0, 1.0" : "=v"(one));
+        int slot = 0;
+        for (int it = 0; it < T; ++it)
+        {
+            floatx4 acc[MB] = {floatx4{0.f, 0.f, 0.f, 0.f}};
+#pragma unroll
+            for (int st = 0; st < STEPS; ++st)
+            {
+                __builtin_amdgcn_s_waitcnt(mr_vmcnt(LT));
+                uintx4 wv[GW];
+                uint32_t s2[GW], z16[GW];
+                {
+                    const uint8_t* sl = ring + slot * TILE_BYTES + rd_base;
+                    const uint8_t* ax = aux + slot * AUX;
+#pragma unroll
+                    for (int g = 0; g < GW; ++g)
+                    {
+                        wv[g] = *reinterpret_cast<const uintx4*>(sl + (((g * 4 + kq) ^ rd_swz) << 4));
+                        const uint32_t sh = *reinterpret_cast<const uint16_t*>(ax + sc_rd[g]);
+                        s2[g] = sh | (sh << 16);
+                        if constexpr (ZPT)
+                        {
+                            const uint32_t z = ((uint32_t)ax[z_rd[g]] >> z_sh[g]) & 15u;
+                            z16[g] = z | (z << 16);
+                        }
+                        else
+                            z16[g] = zp16;
+                    }
+                }
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                issue(min(it + (st + 2) / STEPS, T - 1), (st + 2) % STEPS, slot);
+                slot ^= 1;
+#pragma unroll
+                for (int g = 0; g < GW; ++g)
+                {
+                    const half2_t sc = as_half2(s2[g]);
+                    const half2_t lo_add = as_half2(z16[g] | 0xE400E400u);        // -(1024 + z)
+                    const half2_t hi_add = as_half2((z16[g] << 4) | 0xD400D400u); // -(64 + z)
+                    const uint32_t ww[4] = {wv[g].x, wv[g].y, wv[g].z, wv[g].w};
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                    {
+                        const uint32_t w = ww[j];
+                        const uint32_t w8 = w >> 8;
+                        uintx4 bq;
+                        bq.x = as_u32((as_half2((w & MASK_LO) | MAGIC) + lo_add) * sc);     // (q0, q4)
+                        bq.y = as_u32((as_half2((w & MASK_HI) | MAGIC_HI) + hi_add) * sc);  // (q1, q5)
+                        bq.z = as_u32((as_half2((w8 & MASK_LO) | MAGIC) + lo_add) * sc);    // (q2, q6)
+                        bq.w = as_u32((as_half2((w8 & MASK_HI) | MAGIC_HI) + hi_add) * sc); // (q3, q7)
+                        acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, areg[0][st * GW + g][j]),
+                                                                        __builtin_bit_cast(half8_t, bq), acc[0], 0, 0, 0);
+                    }
+                }
+            }
+            // (mrows_reduce_park stores the sums with inline assembly, and the wait between an MFMA and a read of its
+            // result is only inserted ahead of instructions the compiler emits itself: one such instruction)
+            acc[0].x *= one;
+            acc[0].y *= one;
+            acc[0].z *= one;
+            acc[0].w *= one;
+            mrows_reduce_park<MB>(acc, red, red_addr, parked_addr, it & 1, it, M, tid);
+        }
+        __builtin_amdgcn_s_waitcnt(mr_vmcnt(0)); // the reloads past the end, before the LDS goes away
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        mrows_flush<false, MB>(parked, Y, t0, T, M, N, tid, GemvFusionArgs{nullptr, nullptr, nullptr, nullptr, 0.f}, 0);
+    }
+
     // The same kernel with K as a run-time value: any multiple of 256 up to 8 * GW * STEPS groups (2 <= M <= 16).
     // A wavefront whose GW groups of a step would reach past the end of K fetches the last GW groups of the row
     // instead (the loads of every wavefront and step stay the same in number, which the hand-written wait counts
@@ -715,6 +921,69 @@ namespace nnf
         case 4: return launch_mrows<2, 2>(stream, A, Wq, S, Y, M, N, zp, num_cu, fusion);
         case 6: return launch_mrows<3, 2>(stream, A, Wq, S, Y, M, N, zp, num_cu, fusion);
         default: return launch_mrows<4, 2>(stream, A, Wq, S, Y, M, N, zp, num_cu, fusion);
+        }
+    }
+
+    namespace
+    {
+        template <int GW, int GSHIFT, bool ZPT>
+        hipError_t launch_mrows_q(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M, int N, int zp,
+                                  const void* zps, int num_cu)
+        {
+            if constexpr (((GW << (7 - GSHIFT)) & 1) != 0)
+                return hipErrorInvalidValue;
+            else
+            {
+                const int n_tiles = (N + 15) / 16;
+                const int grid = n_tiles < num_cu ? n_tiles : num_cu;
+                const int tiles_q = n_tiles / grid, tiles_r = n_tiles % grid;
+                const size_t lds = workspace::w4a16_mrows_q_lds_bytes(GW * 2048, M, tiles_q + (tiles_r ? 1 : 0), GSHIFT, ZPT);
+                if (lds > MAX_LDS_BYTES)
+                    return hipErrorInvalidValue;
+                auto kernel = &w4a16_mrows_q_kernel<GW, GSHIFT, ZPT>;
+                if (lds > 64 * 1024)
+                {
+                    static LdsGrant granted;
+                    const hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), granted, (int)MAX_LDS_BYTES);
+                    if (e != hipSuccess)
+                        return e;
+                }
+                hipLaunchKernelGGL(kernel, dim3(grid), dim3(MR_WAVES * 64), lds, stream, (const half_t*)A, (const uint8_t*)Wq,
+                                   (const half_t*)S, (half_t*)Y, (const uint8_t*)zps, N, tiles_q, tiles_r, M | (zp << 8));
+                return hipGetLastError();
+            }
+        }
+        template <int GW>
+        hipError_t launch_mrows_q_gw(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M, int N,
+                                     int group_shift, int zp, const void* zps, int num_cu)
+        {
+            switch (group_shift * 2 + (zps ? 1 : 0))
+            {
+            case 10: return launch_mrows_q<GW, 5, false>(stream, A, Wq, S, Y, M, N, zp, zps, num_cu);
+            case 11: return launch_mrows_q<GW, 5, true>(stream, A, Wq, S, Y, M, N, zp, zps, num_cu);
+            case 12: return launch_mrows_q<GW, 6, false>(stream, A, Wq, S, Y, M, N, zp, zps, num_cu);
+            case 13: return launch_mrows_q<GW, 6, true>(stream, A, Wq, S, Y, M, N, zp, zps, num_cu);
+            case 15: return launch_mrows_q<GW, 7, true>(stream, A, Wq, S, Y, M, N, zp, zps, num_cu);
+            default: return hipErrorInvalidValue; // groups of 128 with a scalar zero point: w4a16_mrows_kernel
+            }
+        }
+    } // namespace
+
+    bool w4a16_mrows_q_supported(int M, int N, int K, int group_shift, bool zero_points, int num_cu)
+    {
+        return !(group_shift == 7 && !zero_points) && workspace::w4a16_mrows_q_fits(M, N, K, group_shift, zero_points, num_cu);
+    }
+
+    hipError_t launch_w4a16_mrows_q(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M, int N,
+                                    int K, int group_shift, int zp, const void* zero_points, int num_cu)
+    {
+        if (!w4a16_mrows_q_supported(M, N, K, group_shift, zero_points != nullptr, num_cu))
+            return hipErrorInvalidValue;
+        switch (K >> 11)
+        {
+        case 1: return launch_mrows_q_gw<1>(stream, A, Wq, S, Y, M, N, group_shift, zp, zero_points, num_cu);
+        case 2: return launch_mrows_q_gw<2>(stream, A, Wq, S, Y, M, N, group_shift, zp, zero_points, num_cu);
+        default: return launch_mrows_q_gw<4>(stream, A, Wq, S, Y, M, N, group_shift, zp, zero_points, num_cu);
         }
     }
 

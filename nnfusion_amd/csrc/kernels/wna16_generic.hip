@@ -563,12 +563,18 @@ namespace nnf
         {
             if (M == 1)
             {
+                // 4-bit weights in rows the row-streaming kernel can walk: that kernel
+                if (bits == 4 && w4a16_gemv_rows_q_supported(1, N, K, qa.group_shift, zero_points != nullptr, num_cu))
+                    return launch_w4a16_gemv_rows_q(stream, A, Wq, S, Y, N, K, qa.group_shift, zp, zero_points, num_cu);
                 if (bits == 4)
                     launch_wna16_gemv<4, 4, 1>(stream, A, Wq, S, Y, M, N, K, qa, num_cu);
                 else
                     launch_wna16_gemv<8, 4, 1>(stream, A, Wq, S, Y, M, N, K, qa, num_cu);
                 return hipGetLastError();
             }
+            // 4-bit weights with K = 2048 / 4096 / 8192: the row-streaming MFMA kernel
+            if (bits == 4 && w4a16_mrows_q_supported(M, N, K, qa.group_shift, zero_points != nullptr, num_cu))
+                return launch_w4a16_mrows_q(stream, A, Wq, S, Y, M, N, K, qa.group_shift, zp, zero_points, num_cu);
             // blocks of two tiles of 16 rows, at most four workgroups per CU
             const int blocks = (N + 31) / 32, cap = num_cu * 4;
             const dim3 grid((unsigned)(blocks < cap ? blocks : cap));

@@ -337,23 +337,28 @@ namespace nnf
             // ring + activations (+ zeros) + their constants + the workgroup's scales + parked outputs + row counters (32 bytes) + the wavefronts' sums of squares for RMSNorm (32 bytes)
             // (gate: N outputs from 2 N weight rows; a workgroup holds the scales of its gate rows and of its up rows as
             // two blocks, each rounded up to whole KiB)
-            size_t lds_bytes(int N, int K, int grid, bool gate = false) const
+            // group_shift: log2 of the group size; zero_points: a zero point per (row, group): 256 bytes more per ring slot
+            // and 64 groups, and a second constant per unit of activations
+            size_t lds_bytes(int N, int K, int grid, bool gate = false, int group_shift = 7, bool zero_points = false) const
             {
                 const size_t rows = (size_t)(N / grid + 1);                       // outputs of a workgroup, at most
                 const size_t a_pad = (((size_t)(K >> 3) + 63) & ~(size_t)63) + 4; // 16-byte units of activations
                 const size_t halves = gate ? 2 : 1;
-                return (size_t)ROWS_WAVES * depth * seg * 1024 + a_pad * 16 + a_pad * 4 +
-                       halves * ((rows * (size_t)(K >> 7) * 2 + 1023) & ~(size_t)1023) +
+                const size_t slot = (size_t)seg * 1024 + (zero_points ? (size_t)((seg + 1) / 2) * 256 : 0);
+                return (size_t)ROWS_WAVES * depth * slot + a_pad * 16 + a_pad * 4 * (zero_points ? 2 : 1) +
+                       halves * ((rows * (size_t)(K >> group_shift) * 2 + 1023) & ~(size_t)1023) +
                        ((halves * rows) << kshift) * sizeof(float) + 64;
             }
         };
         // N: outputs (gate: from 2 N weight rows).  forced_depth: 0 = the plan's own choice
-        inline RowsPlan plan_w4a16_rows(int M, int N, int K, int num_cu, int forced_depth = 0, bool gate = false)
+        inline RowsPlan plan_w4a16_rows(int M, int N, int K, int num_cu, int forced_depth = 0, bool gate = false,
+                                        int group_shift = 7, bool zero_points = false)
         {
             RowsPlan p;
             // whole 16-byte pieces of scales per segment, 4-byte aligned: K a multiple of 256
             // (the activations are fetched as at most 2048 16-byte units: K <= 16384)
-            if (M != 1 || N < 1 || K < 1024 || K > 16384 || (K & 255) || num_cu < 1)
+            if (M != 1 || N < 1 || K < 1024 || K > 16384 || (K & 255) || num_cu < 1 || group_shift < 5 || group_shift > 7 ||
+                (gate && (group_shift != 7 || zero_points)))
                 return p;
             const int loads_per_row = ((K >> 1) + 1023) >> 10;
             int kshift = 0;
@@ -374,9 +379,9 @@ namespace nnf
                 p.depth = depth_max;
             if (p.depth > rows_q)
                 p.depth = rows_q < 1 ? 1 : rows_q;
-            while (p.depth > 1 && p.lds_bytes(N, K, grid, gate) > LDS_BYTES_PER_CU)
+            while (p.depth > 1 && p.lds_bytes(N, K, grid, gate, group_shift, zero_points) > LDS_BYTES_PER_CU)
                 --p.depth;
-            if (p.lds_bytes(N, K, grid, gate) > LDS_BYTES_PER_CU)
+            if (p.lds_bytes(N, K, grid, gate, group_shift, zero_points) > LDS_BYTES_PER_CU)
                 p.seg = 0;
             return p;
         }
@@ -489,6 +494,28 @@ namespace nnf
             const int n_tiles = (N + 15) / 16;
             const int grid = n_tiles < num_cu ? n_tiles : num_cu;
             return w4a16_mrows_lds_bytes(K, M, (gate ? 2 : 1) * ((n_tiles + grid - 1) / grid)) <= LDS_BYTES_PER_CU;
+        }
+        // The same kernel for groups of 32 / 64 / 128 and zero points per (row, group) (w4a16_mrows_q_kernel): 2 .. 16 rows,
+        // K = 2048, 4096, 8192 (GW = K / 2048 groups of 128 per wavefront and step); per wavefront and ring slot 256 bytes
+        // per 64 4-byte words of scales (GW x 128 / group scales for each of 16 rows) and as much again for zero points.
+        inline size_t w4a16_mrows_q_lds_bytes(int K, int M, int tiles, int group_shift, bool zero_points)
+        {
+            const int gw = K >> 11;
+            const int words = (gw << (7 - group_shift)) / 2; // of scales per row, step and wavefront
+            const int loads = (16 * words + 63) / 64;
+            const size_t aux = (size_t)(zero_points ? 2 : 1) * loads * 256;
+            return (size_t)8 * 2 * gw * 1024 + 8 * 2 * aux + (size_t)2 * 8 * 1024 + (size_t)tiles * M * 64;
+        }
+        inline bool w4a16_mrows_q_fits(int M, int N, int K, int group_shift, bool zero_points, int num_cu)
+        {
+            if (M < 2 || M > 16 || N < 16 || num_cu < 1 || (K != 2048 && K != 4096 && K != 8192) || group_shift < 5 ||
+                group_shift > 7)
+                return false;
+            if (((K >> 11) << (7 - group_shift)) & 1) // K = 2048 with groups of 128: half a word of scales per step
+                return false;
+            const int n_tiles = (N + 15) / 16;
+            const int grid = n_tiles < num_cu ? n_tiles : num_cu;
+            return w4a16_mrows_q_lds_bytes(K, M, (n_tiles + grid - 1) / grid, group_shift, zero_points) <= LDS_BYTES_PER_CU;
         }
         // K above 8192 (above 4096 for 17 .. 32 rows, above 2048 for 33 .. 64; a multiple of 256): the run-time-K form over equal ranges of K (in whole pairs of
         // groups; the last range may be shorter), each on its share of the CUs; fp32 sums per range, added by the

@@ -975,6 +975,43 @@ int main(int argc, char** argv)
                     EXPECT(p.depth == 1 || p.depth * (ws::ROWS_WAVES >> p.kshift) <= n / grid);
                 }
             EXPECT(ws::plan_w4a16_rows(1, 1000000, 16384, 256).seg == 0);
+            // other block parameters: groups of 32 / 64 (more scales per row) and zero-point tensors (256 bytes more per
+            // ring slot and 64 groups, a second constant per unit of activations); not with the SiLU-gate
+            p = ws::plan_w4a16_rows(1, 4096, 4096, 256, 0, false, 5, true);
+            EXPECT(p.seg == 2 && p.kshift == 0 && p.depth == 2);
+            EXPECT(p.lds_bytes(4096, 4096, 256, false, 5, true) ==
+                   (size_t)8 * 2 * (2 * 1024 + 256) + 516 * 16 + 2 * 516 * 4 + 5120 + 17 * 4 + 64);
+            EXPECT(ws::plan_w4a16_rows(1, 4096, 11008, 256, 0, false, 5, true).seg == 3);
+            EXPECT(ws::plan_w4a16_rows(1, 4096, 4096, 256, 0, false, 4, false).seg == 0);
+            EXPECT(ws::plan_w4a16_rows(1, 4096, 4096, 256, 0, false, 8, false).seg == 0);
+            EXPECT(ws::plan_w4a16_rows(1, 4096, 4096, 256, 0, true, 6, false).seg == 0);
+            EXPECT(ws::plan_w4a16_rows(1, 4096, 4096, 256, 0, true, 7, true).seg == 0);
+            for (int n : ns)
+                for (int k = 1024; k <= 16384; k += 1280)
+                    for (int gs = 5; gs <= 7; ++gs)
+                    {
+                        p = ws::plan_w4a16_rows(1, n, k, 256, 0, false, gs, true);
+                        if (p.seg == 0)
+                            continue;
+                        const int grid = ws::rows_grid(n, 256);
+                        EXPECT(p.lds_bytes(n, k, grid, false, gs, true) <= ws::LDS_BYTES_PER_CU);
+                        EXPECT(p.lds_bytes(n, k, grid, false, gs, true) > p.lds_bytes(n, k, grid, false, gs, false));
+                        EXPECT(p.depth == 1 || p.depth * (ws::ROWS_WAVES >> p.kshift) <= n / grid);
+                    }
+        }
+        // a few rows with other block parameters: K = 2048 / 4096 / 8192, whole words of scales per step and wavefront
+        {
+            EXPECT(ws::w4a16_mrows_q_fits(16, 8192, 8192, 6, true, 256));
+            EXPECT(ws::w4a16_mrows_q_fits(2, 4096, 4096, 5, false, 256));
+            EXPECT(ws::w4a16_mrows_q_fits(8, 300, 2048, 6, true, 256));
+            EXPECT(!ws::w4a16_mrows_q_fits(8, 300, 2048, 7, true, 256)); // half a word of scales
+            EXPECT(!ws::w4a16_mrows_q_fits(1, 4096, 4096, 5, false, 256) && !ws::w4a16_mrows_q_fits(17, 4096, 4096, 5, false, 256));
+            EXPECT(!ws::w4a16_mrows_q_fits(8, 4096, 6144, 5, false, 256) && !ws::w4a16_mrows_q_fits(8, 4096, 11008, 5, false, 256));
+            EXPECT(!ws::w4a16_mrows_q_fits(8, 4096, 4096, 4, false, 256) && !ws::w4a16_mrows_q_fits(8, 8, 4096, 5, false, 256));
+            // ring 8 x 2 x 4 KiB, scales and zero points 8 x 2 x (2 + 2) x 256, partial tiles 16 KiB, two parked tiles
+            EXPECT(ws::w4a16_mrows_q_lds_bytes(8192, 16, 2, 5, true) == 65536 + 16384 + 16384 + 2 * 16 * 64);
+            EXPECT(ws::w4a16_mrows_q_lds_bytes(4096, 16, 1, 6, false) == 32768 + 4096 + 16384 + 1024);
+            EXPECT(!ws::w4a16_mrows_q_fits(16, 1000000, 8192, 5, true, 256)); // the parked sums do not fit
         }
         // M <= 16: one workgroup holds the activations, or K is cut into ranges
         {

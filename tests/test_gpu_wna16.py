@@ -45,6 +45,12 @@ SHAPES = [
     # of groups, the benchmark's shapes
     (1, 4096, 4096), (1, 33, 128), (3, 1000, 512), (16, 257, 2048), (5, 64, 160), (1, 12288, 4096), (8, 300, 11008),
     (16, 4111, 4096), (2, 7, 384),
+    # one row of 4-bit weights, K a multiple of 256: the row-streaming kernel (one, two and three loads per row and
+    # wavefront; one, two and four wavefronts per row; fewer rows than wavefronts)
+    (1, 300, 1024), (1, 22016, 4096), (1, 4096, 11008), (1, 1000, 8192), (1, 5000, 16384), (1, 257, 2560), (1, 5, 4096),
+    # a few rows of 4-bit weights with K = 2048 / 4096 / 8192: the row-streaming MFMA kernel (one, two and four loads per
+    # step and wavefront; fewer tiles than CUs, a ragged last tile, several tiles per workgroup)
+    (2, 4096, 4096), (5, 300, 2048), (8, 1000, 8192), (16, 48, 8192), (13, 12288, 4096), (16, 9000, 2048),
     # the tile kernel: one partial tile, ragged M and N, many tiles, a long K
     (17, 33, 128), (64, 64, 512), (100, 1000, 160), (300, 257, 2048), (128, 4096, 4096), (33, 520, 11008), (1024, 130, 384),
     # enough 128 x 128 tiles to fill the chip: the larger tile kernel; ragged M and N, an odd number of groups
@@ -83,6 +89,28 @@ def test_one_hot_rows_return_the_dequantised_weights(gpu, m, n, bits, group, zp_
     for r, kk in enumerate(ks):
         np.testing.assert_array_equal(y[r], wd[:, kk].astype(np.float16))
     assert not y[len(ks):].any()
+
+
+@pytest.mark.parametrize("m,k", [(1, 1024), (1, 4096), (1, 11008), (1, 16384), (7, 2048), (16, 4096), (3, 8192)])
+@pytest.mark.parametrize("group,zp_tensor", [(32, True), (64, True), (128, True), (32, False), (64, False)])
+def test_one_hot_rows_through_the_row_streaming_kernels(gpu, m, k, group, zp_tensor):
+    """4-bit weights with one row and K a multiple of 256, or a few rows and K = 2048 / 4096 / 8192, run on the
+    row-streaming kernels: the same pin for their scales and zero points (first and last weight of a group, of a
+    wavefront's load, of a wavefront's K segment, of a step, of the row)."""
+    n = 700
+    _, wq, s, zps = _case(11, 1, n, k, 4, group, zp_tensor)
+    wd = oracle.dequantize_wn(wq, s, 4, group, zp=5, zero_points=zps)
+    kks = [kk for kk in sorted({0, 1, 31, 32, 63, 64, 127, 128, 255, 256, 511, 512, 1023, 1024, 2047, 2048, 4095, 4096, 6143,
+                                6144, 8191, 8192, k // 2 - 1, k // 2, k - 129, k - 33, k - 1}) if kk < k]
+    for c in range(0, len(kks), m):
+        chunk = kks[c:c + m]
+        a = np.zeros((m, k), np.float16)
+        for r, kk in enumerate(chunk):
+            a[r, kk] = 1.0
+        y = _run(gpu, a, wq, s, 4, group, 5, zps)
+        for r, kk in enumerate(chunk):
+            np.testing.assert_array_equal(y[r], wd[:, kk].astype(np.float16), err_msg="k = %d" % kk)
+        assert not y[len(chunk):].any()
 
 
 def test_default_parameters_are_the_specialised_kernels(gpu):
