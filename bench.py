@@ -611,12 +611,13 @@ def extra_rows(env):
         for m in WNA16_MS:
             a = env.dev_t(datagen.normal_f16(0, datagen.S_ACT, (m, k)))
             y = torch.empty((m, n), dtype=torch.float16, device=dev)
+            wsq = env.workspace(ops.wna16_workspace_bytes(m, n, k, bits, group, tz))
             rows.append({"key": wna16_key(bits, group, zpt, n, k, m), "group": None, "M": m,
                          "bytes": wna16_bytes(m, n, k, bits, group, zpt), "ops": 2.0 * m * n * k, "int8": False,
                          "weights": (tw, tsc) + ((tz,) if zpt else ()),
-                         "make": (lambda w, sc, zz=None, a=a, y=y, bits=bits, group=group:
+                         "make": (lambda w, sc, zz=None, a=a, y=y, bits=bits, group=group, wsq=wsq:
                                   (lambda: ops.wna16_gemm(a, w, sc, bits=bits, group=group, zp=1 << (bits - 1), zero_points=zz,
-                                                          out=y)))})
+                                                          out=y, workspace=wsq)))})
     h, i = MLP_HI
     _, gamma, wgu, sgu, wd, sd = [env.dev_t(t) for t in datagen.mlp_case(0, 1, h, i)]  # the weights do not depend on M
     for m in MLP_MS:

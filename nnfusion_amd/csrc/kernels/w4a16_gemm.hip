@@ -377,6 +377,7 @@ namespace nnf
         p.tiles_n = plan.tiles_n;
         p.supersteps = plan.supersteps;
         p.units = plan.units;
+        p.zps = nullptr;
         if (plan.tile_weight_rows == 128)
             return plan.tile_rows == 256 ? launch_gemm_sk_256_narrow(stream, p, plan.grid)
                    : plan.tile_rows == 128 ? launch_gemm_sk_128_narrow(stream, p, plan.grid)
@@ -387,6 +388,53 @@ namespace nnf
         case 128: return launch_gemm_sk_128(stream, p, plan.grid, gate);
         case 64: return launch_gemm_sk_64(stream, p, plan.grid, gate);
         default: return launch_gemm_sk_32(stream, p, plan.grid, gate);
+        }
+    }
+
+    // ---- the tile GEMM with other block parameters ----------------------------------------------------------------------
+    bool w4a16_gemm_q_supported(int M, int N, int K, int group_shift)
+    {
+        return M > 16 && N >= 1 && K >= 256 && !(K & 255) && group_shift >= 5 && group_shift <= 7 &&
+               (size_t)M * K * 2 + 8192 < ((size_t)1 << 32) && (size_t)N * (K >> 1) < ((size_t)1 << 32);
+    }
+    size_t w4a16_gemm_q_workspace_bytes(int M, int N, int K, int num_cu)
+    {
+        return workspace::plan_w4a16_sk(M, N, K, false, num_cu).bytes();
+    }
+    hipError_t launch_w4a16_gemm_q(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M, int N,
+                                   int K, int group_shift, int zp, const void* zero_points, void* partial_ws, int num_cu)
+    {
+        if (!w4a16_gemm_q_supported(M, N, K, group_shift))
+            return hipErrorInvalidValue;
+        const workspace::SkPlan plan = workspace::plan_w4a16_sk(M, N, K, false, num_cu);
+        if (plan.slots && !partial_ws)
+            return hipErrorInvalidValue;
+        SkGemmParams p;
+        p.A = (const half_t*)A;
+        p.Wq = (const uint8_t*)Wq;
+        p.S = (const half_t*)S;
+        p.Y = (half_t*)Y;
+        p.M = M;
+        p.N = N;
+        p.K = K;
+        p.zp = zp;
+        p.ldy = N;
+        p.up_row_offset = N;
+        p.bias = nullptr;
+        p.residual = nullptr;
+        p.gamma = nullptr;
+        p.rstd = nullptr;
+        p.partial = plan.slots ? (float*)partial_ws : nullptr;
+        p.tiles_m = plan.tiles_m;
+        p.tiles_n = plan.tiles_n;
+        p.supersteps = plan.supersteps;
+        p.units = plan.units;
+        p.zps = (const uint8_t*)zero_points;
+        switch (group_shift)
+        {
+        case 5: return launch_gemm_sk_q5(stream, p, plan.grid, plan.tile_rows, plan.tile_weight_rows);
+        case 6: return launch_gemm_sk_q6(stream, p, plan.grid, plan.tile_rows, plan.tile_weight_rows);
+        default: return launch_gemm_sk_q7(stream, p, plan.grid, plan.tile_rows, plan.tile_weight_rows);
         }
     }
 } // namespace nnf

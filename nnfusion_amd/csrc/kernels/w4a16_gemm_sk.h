@@ -69,6 +69,7 @@ namespace nnf
         int tiles_m, tiles_n;
         int supersteps;         // per tile: ceil(K / 256)
         long long units;        // tiles_m * tiles_n * supersteps
+        const uint8_t* zps;     // QG != 0: zero points, u8 [N, K / group / 2] (even group in the low nibble), or null: zp
     };
 
     namespace gemm_sk
@@ -306,7 +307,12 @@ namespace nnf
         }
     }
 
-    template <int TM, int TN, bool GATE, bool BIAS, bool RESID, bool RMS>
+    // QG = 0: groups of 128, the zero point p.zp.  QG = 5, 6, 7: groups of 2^QG and, with p.zps, a zero point per
+    // (row, group); K a multiple of 256.  A lane's 32 weights of a K step lie in one group whatever its size: per column
+    // tile and superstep it fetches the 256 / group scales of its row in one load (4, 8 or 16 bytes) and the byte(s) that
+    // hold their zero points in another (1, 2 or 4 bytes; without p.zps: the scales again, unused) -- six loads per
+    // column tile as for QG = 0, on the same schedule -- and keeps a scale and the pair -(1024 + z), -(64 + z) per K step.
+    template <int TM, int TN, bool GATE, bool BIAS, bool RESID, bool RMS, int QG = 0>
     __global__ __launch_bounds__(256, 1) void w4a16_gemm_sk_kernel(SkGemmParams p)
     {
         using namespace gemm_sk;
@@ -315,6 +321,11 @@ namespace nnf
         static_assert(!(GATE && (BIAS || RESID)), "SiLU-gate is not combined with bias or residual");
         static_assert(TN == 1 || TN == 2 || TN == 4, "column tiles per wavefront");
         static_assert(!GATE || TN >= 2, "gate and up rows are the two halves of a wavefront's column tiles");
+        static_assert(QG == 0 || (QG >= 5 && QG <= 7), "groups of 32, 64 or 128");
+        constexpr bool QZ = QG != 0;
+        constexpr int GSH = QZ ? QG : 7;                    // log2 of the group size
+        constexpr int NSC = QZ ? (QG == 7 ? 2 : 4) : 2;     // scales a lane keeps per column tile and superstep
+        constexpr int SW = QZ ? (QG == 5 ? 4 : QG == 6 ? 2 : 1) : 2; // registers of scales as loaded
         constexpr int BM = T::BM, BN = T::BN;
         constexpr int A_TILE_BYTES = T::A_TILE_BYTES, STAGE_BYTES = T::STAGE_BYTES;
         constexpr int BN_OUT = GATE ? BN / 2 : BN;
@@ -334,7 +345,7 @@ namespace nnf
         const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
         const int l32 = lane & 31, h = lane >> 5;
         const int K = p.K;
-        const int G = K >> 7;
+        const int G = K >> GSH;
         const int SS = p.supersteps;
         const int grid = (int)gridDim.x;
         const uint32_t lds0 = lds_address(smem);
@@ -423,7 +434,7 @@ namespace nnf
             // ---- weights and scales: straight into registers -----------------------------------------------------
             // lane (l32, h) owns weight row l32 of each of the wavefront's column tiles; of K step t of a
             // superstep it owns k = 64 t + 32 h .. + 31: the 16 bytes at 32 t + 16 h of the superstep's 128
-            uint32_t w_off[TN], s_off[TN];
+            uint32_t w_off[TN], s_off[TN], z_off[TN];
 #pragma unroll
             for (int j = 0; j < TN; ++j)
             {
@@ -434,12 +445,21 @@ namespace nnf
                 else
                     gn = min(n0 + wave * (TN * 32) + j * 32 + l32, p.N - 1);
                 w_off[j] = (uint32_t)((size_t)gn * (K >> 1) + (k_begin >> 1) + h * 16);
-                s_off[j] = (uint32_t)(((size_t)gn * G + 2 * ss_begin) * 2);
+                if constexpr (QZ)
+                {
+                    // the scales of the row's groups of this superstep; their zero points, or (no tensor) the scales again
+                    s_off[j] = (uint32_t)(((size_t)gn * G + (size_t)(256 >> GSH) * ss_begin) * 2);
+                    z_off[j] = p.zps ? (uint32_t)((size_t)gn * (G >> 1) + (size_t)(128 >> GSH) * ss_begin) : s_off[j];
+                }
+                else
+                    s_off[j] = (uint32_t)(((size_t)gn * G + 2 * ss_begin) * 2);
             }
             const uint8_t* s_bytes = reinterpret_cast<const uint8_t*>(p.S);
-            uintx4 wbuf[2][TN][4];   // [register set][column tile][K step of the superstep]
-            uint32_t sraw[2][TN][2]; // the two group scales of the superstep, as loaded
-            half2_t sc[2][TN][2];    // ... as (s, s); zero for a group past K
+            uintx4 wbuf[2][TN][4];    // [register set][column tile][K step of the superstep]
+            uint32_t sraw[2][TN][SW]; // the group scales of the superstep, as loaded
+            half2_t sc[2][TN][NSC];   // ... as (s, s); zero for a group past K
+            uint32_t zraw[2][TN];     // QZ: the zero points of the superstep, as loaded
+            half2_t dq[2][TN][NSC];   // QZ: (-(1024 + z), -(64 + z)) of the same groups
             // Scalar bases of superstep s of the segment (clamped to the last): weights of K steps 0 .. 1 and 2 .. 3,
             // first and second scale.  K not a multiple of 256: the last superstep has one group; its second half
             // repeats the first (and is multiplied by a scale of zero).
@@ -449,8 +469,17 @@ namespace nnf
             };
             auto w_base_of = [&](int s) {
                 s = min(s, NSS - 1);
-                const bool second_valid = 2 * (ss_begin + s) + 1 < G;
                 WBase b;
+                if constexpr (QZ)
+                {
+                    // (K is a multiple of 256)  s_lo: the scales; s_hi: the zero points, or the scales again
+                    b.w_lo = scalar_base(p.Wq + (size_t)s * 128);
+                    b.w_hi = scalar_base(p.Wq + (size_t)s * 128 + 64);
+                    b.s_lo = scalar_base(s_bytes + (size_t)s * (512 >> GSH));
+                    b.s_hi = p.zps ? scalar_base(p.zps + (size_t)s * (128 >> GSH)) : b.s_lo;
+                    return b;
+                }
+                const bool second_valid = 2 * (ss_begin + s) + 1 < G;
                 b.w_lo = scalar_base(p.Wq + (size_t)s * 128);
                 b.w_hi = scalar_base(p.Wq + (size_t)s * 128 + (second_valid ? 64 : 0));
                 b.s_lo = scalar_base(s_bytes + (size_t)s * 4);
@@ -462,12 +491,63 @@ namespace nnf
                 constexpr int set = decltype(set_c)::value, j = decltype(j_c)::value, x = decltype(x_c)::value;
                 if constexpr (x < 4)
                     wbuf[set][j][x] = *(const uintx4 __attribute__((address_space(1)))*)((x < 2 ? b.w_lo : b.w_hi) + (x & 1) * 32 + here(w_off[j]));
-                else
+                else if constexpr (!QZ)
                     sraw[set][j][x - 4] = *(const uint16_t __attribute__((address_space(1)))*)((x == 4 ? b.s_lo : b.s_hi) + here(s_off[j]));
+                else if constexpr (x == 4)
+                {
+                    if constexpr (QG == 5)
+                    {
+                        const uintx4 v = *(const uintx4 __attribute__((address_space(1)))*)(b.s_lo + here(s_off[j]));
+                        sraw[set][j][0] = v.x, sraw[set][j][1] = v.y, sraw[set][j][2] = v.z, sraw[set][j][3] = v.w;
+                    }
+                    else if constexpr (QG == 6)
+                    {
+                        const uintx2 v = *(const uintx2 __attribute__((address_space(1)))*)(b.s_lo + here(s_off[j]));
+                        sraw[set][j][0] = v.x, sraw[set][j][1] = v.y;
+                    }
+                    else
+                        sraw[set][j][0] = *(const uint32_t __attribute__((address_space(1)))*)(b.s_lo + here(s_off[j]));
+                }
+                else
+                {
+                    if constexpr (QG == 5)
+                        zraw[set][j] = *(const uint32_t __attribute__((address_space(1)))*)(b.s_hi + here(z_off[j]));
+                    else if constexpr (QG == 6)
+                        zraw[set][j] = *(const uint16_t __attribute__((address_space(1)))*)(b.s_hi + here(z_off[j]));
+                    else
+                        zraw[set][j] = *(const uint8_t __attribute__((address_space(1)))*)(b.s_hi + here(z_off[j]));
+                }
             };
+            // QZ: a lane's group in K step t of a superstep is 2 t + h (groups of 32), t (64), t / 2 (128)
+            const uint32_t h_sel = h ? 0x03020302u : 0x01000100u; // the half-word of a pair of scales that belongs to h
+            const uint32_t z_and = p.zps ? 15u : 0u, z_or = p.zps ? 0u : (uint32_t)p.zp;
             // (s, s) of both groups of superstep s (as clamped by w_base_of)
             auto prepare_scales = [&](auto set_c, int s) {
                 constexpr int set = decltype(set_c)::value;
+                if constexpr (QZ)
+                {
+#pragma unroll
+                    for (int j = 0; j < TN; ++j)
+#pragma unroll
+                        for (int i = 0; i < NSC; ++i)
+                        {
+                            uint32_t sv, z;
+                            if constexpr (QG == 5)
+                            {
+                                sv = __builtin_amdgcn_perm(sraw[set][j][i], sraw[set][j][i], h_sel);
+                                z = zraw[set][j] >> (uint32_t)(8 * i + 4 * h);
+                            }
+                            else
+                            {
+                                sv = __builtin_amdgcn_perm(sraw[set][j][i >> 1], sraw[set][j][i >> 1], (i & 1) ? 0x03020302u : 0x01000100u);
+                                z = zraw[set][j] >> (uint32_t)(4 * i);
+                            }
+                            z = (z & z_and) | z_or;
+                            sc[set][j][i] = as_half2(sv);
+                            dq[set][j][i] = as_half2((z | (z << 20)) | 0xD400E400u);
+                        }
+                    return;
+                }
                 s = min(s, NSS - 1);
                 const bool second_valid = 2 * (ss_begin + s) + 1 < G;
 #pragma unroll
@@ -496,6 +576,13 @@ namespace nnf
                 lds_read_b128_nowait<decltype(f_c)::value * 4096>(af[decltype(set_c)::value][decltype(f_c)::value], addr);
             };
             // one half2 of the unpacked operand: weights 2e, 2e+1 of word `w` -> (q - zp) * scale (* gamma)
+            // (QZ: `add` is the group's pair -(1024 + z), -(64 + z))
+            auto unpack_piece_q = [&](auto set_c, auto j_c, auto e_c, uint32_t w, half2_t scale, half2_t add) {
+                constexpr int set = decltype(set_c)::value, j = decltype(j_c)::value, e = decltype(e_c)::value;
+                const uint32_t x = __builtin_amdgcn_perm(w, w, SEL[e]);
+                const half2_t y = as_half2((x & MASK) | MAGIC);
+                bw[set][j][e] = as_u32((y + add) * scale);
+            };
             auto unpack_piece = [&](auto set_c, auto j_c, auto e_c, uint32_t w, half2_t scale, const uintx4& gam) {
                 constexpr int set = decltype(set_c)::value, j = decltype(j_c)::value, e = decltype(e_c)::value;
                 const uint32_t x = __builtin_amdgcn_perm(w, w, SEL[e]); // bytes (b_e, 0, b_e, 0)
@@ -604,8 +691,15 @@ namespace nnf
                             constexpr int NQ = (Q + 1) & 3;
                             const uintx4& wq = wbuf[NSET][j][NT];
                             const uint32_t w = NQ == 0 ? wq.x : NQ == 1 ? wq.y : NQ == 2 ? wq.z : wq.w;
-                            unpack_piece(OTHER_C{}, std::integral_constant<int, j>{}, std::integral_constant<int, e>{}, w,
-                                         sc[NSET][j][NT >> 1], gm[NQ]);
+                            if constexpr (QZ)
+                            {
+                                constexpr int SI = QG != 7 ? NT : NT >> 1; // the group of K step NT
+                                unpack_piece_q(OTHER_C{}, std::integral_constant<int, j>{}, std::integral_constant<int, e>{}, w,
+                                               sc[NSET][j][SI], dq[NSET][j][SI]);
+                            }
+                            else
+                                unpack_piece(OTHER_C{}, std::integral_constant<int, j>{}, std::integral_constant<int, e>{}, w,
+                                             sc[NSET][j][NT >> 1], gm[NQ]);
                         });
                         // this quarter's loads, spread over its regions
                         constexpr int N_W = Q < 3 ? SCH::w_begin(T_, Q + 1) - SCH::w_begin(T_, Q) : 0;
@@ -681,8 +775,12 @@ namespace nnf
             }
             unroll_for<0, 4 * TN>([&](auto pc_c) {
                 constexpr int pc = decltype(pc_c)::value;
-                unpack_piece(I0{}, std::integral_constant<int, pc / 4>{}, std::integral_constant<int, pc % 4>{}, wbuf[0][pc / 4][0].x,
-                             sc[0][pc / 4][0], gm[0]);
+                if constexpr (QZ)
+                    unpack_piece_q(I0{}, std::integral_constant<int, pc / 4>{}, std::integral_constant<int, pc % 4>{}, wbuf[0][pc / 4][0].x,
+                                   sc[0][pc / 4][0], dq[0][pc / 4][0]);
+                else
+                    unpack_piece(I0{}, std::integral_constant<int, pc / 4>{}, std::integral_constant<int, pc % 4>{}, wbuf[0][pc / 4][0].x,
+                                 sc[0][pc / 4][0], gm[0]);
             });
             __builtin_amdgcn_sched_barrier(0);
             // No LDS read other than the fragments of quarter 0 is in flight at the top of a K step.
@@ -708,8 +806,17 @@ namespace nnf
 #pragma unroll
                         for (int x = 0; x < 4; ++x)
                             wbuf[0][j][x] = wbuf[1][j][x];
-                        sc[0][j][0] = sc[1][j][0];
-                        sc[0][j][1] = sc[1][j][1];
+                        if constexpr (QZ)
+                        {
+#pragma unroll
+                            for (int i = 0; i < NSC; ++i)
+                                sc[0][j][i] = sc[1][j][i], dq[0][j][i] = dq[1][j][i];
+                        }
+                        else
+                        {
+                            sc[0][j][0] = sc[1][j][0];
+                            sc[0][j][1] = sc[1][j][1];
+                        }
                     }
                 }
             }

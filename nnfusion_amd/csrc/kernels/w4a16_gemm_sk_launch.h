@@ -68,8 +68,47 @@ namespace nnf
             return rms ? launch_instance<TM, TN, false, false, false, true>(stream, p, grid)
                        : launch_instance<TM, TN, false, false, false, false>(stream, p, grid);
         }
+        // other block parameters (QG = log2 of the group size; zero points per (row, group) when p.zps is set): the
+        // plain product; the second launch does not depend on them
+        template <int TM, int TN, int QG>
+        hipError_t launch_instance_q(hipStream_t stream, const SkGemmParams& p, int grid)
+        {
+            using T = Tile<TM, TN>;
+            auto kernel = &w4a16_gemm_sk_kernel<TM, TN, false, false, false, false, QG>;
+            if (T::LDS_BYTES > 48 * 1024)
+            {
+                static LdsGrant granted;
+                const hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), granted, T::LDS_BYTES);
+                if (e != hipSuccess)
+                    return e;
+            }
+            hipLaunchKernelGGL(kernel, dim3(grid), dim3(THREADS), T::LDS_BYTES, stream, p);
+            hipError_t e = hipGetLastError();
+            if (e != hipSuccess || !p.partial)
+                return e;
+            hipLaunchKernelGGL((w4a16_gemm_sk_fixup_kernel<TM, TN, false, false, false, false>), dim3(p.tiles_m * p.tiles_n * TM * WAVES),
+                               dim3(64), 0, stream, p, grid);
+            return hipGetLastError();
+        }
+        // tile_rows x tile_cols as sk_tile_shape chooses them for a plain product
+        template <int QG>
+        hipError_t launch_tiles_q(hipStream_t stream, const SkGemmParams& p, int grid, int tile_rows, int tile_cols)
+        {
+            if (tile_cols == 128)
+                return tile_rows == 256   ? launch_instance_q<8, 1, QG>(stream, p, grid)
+                       : tile_rows == 128 ? launch_instance_q<4, 1, QG>(stream, p, grid)
+                       : tile_rows == 64  ? launch_instance_q<2, 1, QG>(stream, p, grid)
+                                          : hipErrorInvalidValue;
+            return tile_rows == 256 ? launch_instance_q<8, 2, QG>(stream, p, grid)
+                   : tile_rows == 32 ? launch_instance_q<1, 2, QG>(stream, p, grid)
+                                     : hipErrorInvalidValue;
+        }
     } // namespace gemm_sk
 
+    // groups of 32 / 64 / 128 with p.zps or p.zp (w4a16_gemm_sk_q5.hip ... _q7.hip)
+    hipError_t launch_gemm_sk_q5(hipStream_t stream, const SkGemmParams& p, int grid, int tile_rows, int tile_cols);
+    hipError_t launch_gemm_sk_q6(hipStream_t stream, const SkGemmParams& p, int grid, int tile_rows, int tile_cols);
+    hipError_t launch_gemm_sk_q7(hipStream_t stream, const SkGemmParams& p, int grid, int tile_rows, int tile_cols);
     // one per tile height (w4a16_gemm_sk_32.hip ... _256.hip); narrow: 128 x 128 tiles, plain product, bias, residual, RMSNorm
     hipError_t launch_gemm_sk_64_narrow(hipStream_t stream, const SkGemmParams& p, int grid);
     hipError_t launch_gemm_sk_128_narrow(hipStream_t stream, const SkGemmParams& p, int grid);

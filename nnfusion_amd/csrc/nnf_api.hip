@@ -200,9 +200,21 @@ namespace
     bool is_plain_w4a16(const nnf_quant* q) { return q->bits == 4 && q->group == 128 && !q->zero_points; }
 } // namespace
 
+namespace
+{
+    int group_shift_of(int group) { return group == 32 ? 5 : group == 64 ? 6 : 7; }
+} // namespace
+
 size_t nnf_wna16_gemm_workspace_bytes(int M, int N, int K, const nnf_quant* q)
 {
-    return (q && is_plain_w4a16(q)) ? nnf::workspace::w4a16_gemm(M, N, K, q->group) : 0;
+    if (!q)
+        return 0;
+    if (is_plain_w4a16(q))
+        return nnf::workspace::w4a16_gemm(M, N, K, q->group);
+    // 4-bit weights above 16 rows: the tile GEMM where tiles are shared between workgroups (without it: the plain tile kernel)
+    if (q->bits == 4 && nnf_wna16_supported(M, N, K, q) && nnf::w4a16_gemm_q_supported(M, N, K, group_shift_of(q->group)))
+        return nnf::w4a16_gemm_q_workspace_bytes(M, N, K, nnf::workspace::PLAN_CUS);
+    return 0;
 }
 
 int nnf_wna16_gemm(nnf_stream_t stream, const void* A, const void* Wq, const void* scales, void* Y, int M, int N, int K,
@@ -222,6 +234,16 @@ int nnf_wna16_gemm(nnf_stream_t stream, const void* A, const void* Wq, const voi
     const int st = current_device_info(dev);
     if (st != NNF_OK)
         return st;
+    // 4-bit weights above 16 rows: the stream-K tile GEMM, given the workspace its plan on this device needs (and
+    // zero points it can fetch four bytes at a time)
+    if (q->bits == 4 && nnf::w4a16_gemm_q_supported(M, N, K, group_shift_of(q->group)) &&
+        (reinterpret_cast<uintptr_t>(q->zero_points) & 3) == 0)
+    {
+        const size_t need = nnf::w4a16_gemm_q_workspace_bytes(M, N, K, dev.num_cu);
+        if (need == 0 || (workspace && aligned16(workspace) && workspace_bytes >= need))
+            return (int)nnf::launch_w4a16_gemm_q((hipStream_t)stream, A, Wq, scales, Y, M, N, K, group_shift_of(q->group),
+                                                 q->zero_point, q->zero_points, workspace, dev.num_cu);
+    }
     return (int)nnf::launch_wna16_generic((hipStream_t)stream, A, Wq, scales, Y, M, N, K, q->bits, q->group, q->zero_point,
                                           q->zero_points, dev.num_cu);
 }

@@ -84,6 +84,12 @@ def wna16_supported(m, n, k, bits, group, zp=8):
     return bool(_lib.kernels().nnf_wna16_supported(m, n, k, qp))
 
 
+def wna16_workspace_bytes(m, n, k, bits, group, zero_points=None):
+    """Bytes of workspace nnf_wna16_gemm wants for this product (0: none)."""
+    _, qp = _quant_arg(bits, group, 0, zero_points)
+    return int(_lib.kernels().nnf_wna16_gemm_workspace_bytes(m, n, k, qp))
+
+
 def wna16_gemm(a, wq, scales, bits=4, group=128, zp=8, zero_points=None, out=None, workspace=None):
     """Y[M,N] = A[M,K] . ((Wq - z) * scales)^T with 4- or 8-bit weights (wq u8 [N, K*bits/8]), groups of 32 / 64 / 128
     and either a scalar zero point or zero_points u8 [N, ceil(K/group*bits/8)] (4-bit: two per byte, even group low)."""

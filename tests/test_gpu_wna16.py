@@ -53,6 +53,10 @@ SHAPES = [
     (2, 4096, 4096), (5, 300, 2048), (8, 1000, 8192), (16, 48, 8192), (13, 12288, 4096), (16, 9000, 2048),
     # the tile kernel: one partial tile, ragged M and N, many tiles, a long K
     (17, 33, 128), (64, 64, 512), (100, 1000, 160), (300, 257, 2048), (128, 4096, 4096), (33, 520, 11008), (1024, 130, 384),
+    # 4-bit weights above 16 rows with K a multiple of 256: the stream-K tile GEMM (tiles of 32 x 256, 64 x 128, 128 x 128,
+    # 256 x 128, 256 x 256; tiles shared between workgroups and not; ragged M and N)
+    (17, 300, 256), (40, 1000, 1024), (100, 257, 2048), (130, 4096, 4096), (700, 3000, 1280), (1100, 2050, 768),
+    (1600, 520, 2560), (2000, 8192, 512), (30, 22016, 4096),
     # enough 128 x 128 tiles to fill the chip: the larger tile kernel; ragged M and N, an odd number of groups
     (2048, 2048, 512), (1100, 4100, 160), (4096, 1030, 384),
 ]
@@ -72,16 +76,18 @@ def test_wna16_matches_oracle(gpu, m, n, k, bits, group, zp_tensor):
     _check(_run(gpu, a, wq, s, bits, group, zp, zps), ref)
 
 
-@pytest.mark.parametrize("m,n", [(4, 70), (40, 70), (2000, 2100)])
-@pytest.mark.parametrize("bits,group,zp_tensor", [(4, 32, True), (4, 64, False), (8, 64, True), (8, 128, False), (8, 32, True)])
-def test_one_hot_rows_return_the_dequantised_weights(gpu, m, n, bits, group, zp_tensor):
-    """A = e_k: 1 * w is exact in every kernel (m = 2000: the 128 x 128 tiles), so the output is fp16((q - z) * s) bit for
-    bit; pins nibble and byte order of weights and zero points and the block each scale belongs to, on the device."""
-    k = 640
+@pytest.mark.parametrize("m,n,k", [(4, 70, 640), (40, 70, 640), (2000, 2100, 640), (40, 300, 1024), (300, 520, 768),
+                                   (2000, 2100, 512)])
+@pytest.mark.parametrize("bits,group,zp_tensor", [(4, 32, True), (4, 64, False), (8, 64, True), (8, 128, False), (8, 32, True),
+                                                   (4, 64, True), (4, 128, True), (4, 32, False)])
+def test_one_hot_rows_return_the_dequantised_weights(gpu, m, n, k, bits, group, zp_tensor):
+    """A = e_k: 1 * w is exact in every kernel (m = 2000: the 128 x 128 tiles; K a multiple of 256 with 4-bit weights: the
+    stream-K tile GEMM), so the output is fp16((q - z) * s) bit for bit; pins nibble and byte order of weights and zero
+    points and the block each scale belongs to, on the device."""
     _, wq, s, zps = _case(5, m, n, k, bits, group, zp_tensor)
     zp = 3 if bits == 4 else 200
     wd = oracle.dequantize_wn(wq, s, bits, group, zp=zp, zero_points=zps)
-    ks = [0, 1, 7, 8, 31, 32, 63, 64, 127, 128, 255, 256, 511, 512, 639][:m] if m <= 16 else [(7 * r) % k for r in range(min(m, 640))]
+    ks = [0, 1, 7, 8, 31, 32, 63, 64, 127, 128, 255, 256, 511, 512, 639][:m] if m <= 16 else [(7 * r) % k for r in range(min(m, k))]
     a = np.zeros((m, k), np.float16)
     for r, kk in enumerate(ks):
         a[r, kk] = 1.0
