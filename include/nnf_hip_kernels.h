@@ -145,12 +145,14 @@ int nnf_w4a16_gemm_variant(nnf_stream_t stream,
  *   zero_points == NULL : z = zero_point everywhere (0 .. 2^bits - 1)
  *   zero_points != NULL : u8 [N, ceil(K/group * bits / 8)], one per (row, group); 4-bit ones packed two to a byte along
  *                         the groups of a row, even group in the low nibble
- * bits 4, group 128 and no zero-point tensor is nnf_w4a16_gemm itself (same kernels, same workspace).  Every other
- * combination (group 32 / 64 / 128, K a multiple of group) needs no workspace.  4-bit weights run on the row-streaming
- * kernels of nnf_w4a16_gemm where those apply: M = 1 with K a multiple of 256 from 1024 to 16384, and 2 <= M <= 16 with
- * K = 2048 / 4096 / 8192 (groups of 128 with a zero-point tensor: 4096 / 8192).  Everything else runs on plain kernels:
- * a row-per-wavefront GEMV for M = 1, an MFMA kernel with the operands fetched straight into registers for
- * 2 <= M <= 16, MFMA tiles through LDS above. */
+ * bits 4, group 128 and no zero-point tensor is nnf_w4a16_gemm itself (same kernels, same workspace).  For every other
+ * combination (group 32 / 64 / 128, K a multiple of group) 4-bit weights run on the kernels of nnf_w4a16_gemm where
+ * those apply: the row-streaming kernels for M = 1 with K a multiple of 256 from 1024 to 16384 and for 2 <= M <= 16
+ * with K = 2048 / 4096 / 8192 (groups of 128 with a zero-point tensor: 4096 / 8192), and the tile GEMM above 16 rows
+ * with K a multiple of 256 and zero_points 4-byte aligned.  The tile GEMM wants nnf_wna16_gemm_workspace_bytes of
+ * workspace; called with less (or NULL) the product runs on a plain tile kernel instead, at less than half the rate.
+ * Everything else runs on plain kernels that need no workspace: a row-per-wavefront GEMV for M = 1, an MFMA kernel
+ * with the operands fetched straight into registers for 2 <= M <= 16, MFMA tiles through LDS above. */
 typedef struct nnf_quant
 {
     int bits;                /* 4 or 8 */

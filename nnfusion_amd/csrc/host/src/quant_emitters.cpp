@@ -68,15 +68,20 @@ namespace nnfusion
                         return nullptr;
                     if (bits != 4 || group != 128 || has_z)
                     {
-                        // other block parameters: the plain product only (nnf_wna16_gemm), no scratch memory
+                        // other block parameters: the plain product only (nnf_wna16_gemm); scratch memory for the tile
+                        // GEMM of 4-bit weights
                         if (rms || has_bias || has_res || gate || (bits != 4 && bits != 8) ||
                             (group != 32 && group != 64 && group != 128) || K % group != 0)
                             return nullptr;
+                        const size_t q_ws_bytes = nnf::workspace::wna16_gemm((int)M, (int)N, (int)K, bits, group);
+                        std::string q_ws = "nullptr";
+                        if (q_ws_bytes > 0)
+                            q_ws = allocate_tensor(Shape{q_ws_bytes}, element::character)->get_name();
                         LanguageUnit_p lu(new LanguageUnit(get_function_name()));
                         *lu << "const nnf_quant quant = {" << bits << ", " << group << ", " << zp << ", "
                             << (has_z ? "input3" : "nullptr") << "};\n";
                         *lu << "NNF_HIP_CHECK(nnf_wna16_gemm(stream, input0, input1, input2, output0, " << M << ", " << N << ", "
-                            << K << ", &quant, nullptr, 0));\n";
+                            << K << ", &quant, " << q_ws << ", " << q_ws_bytes << "));\n";
                         return lu;
                     }
                     if (K % 128 != 0)

@@ -107,9 +107,8 @@ namespace nnf
     // kernels and the tile GEMM, in the reduction pass behind a GEMV kernel over ranges of K, or (MFMA GEMV kernel) as a
     // pre-pass and an element-wise kernel.  rms_ws / partial_ws: the route's rms_bytes / partial_bytes (null when 0).
     // the tile GEMM for groups of 2^group_shift = 32 / 64 / 128 and a scalar zero point or (zero_points != null) one per
-    // (row, group): M > 16, K a multiple of 256; partial_ws: w4a16_gemm_q_workspace_bytes (0: not needed)
+    // (row, group): M > 16, K a multiple of 256; partial_ws: workspace::wna16_gemm bytes (0: not needed)
     bool w4a16_gemm_q_supported(int M, int N, int K, int group_shift);
-    size_t w4a16_gemm_q_workspace_bytes(int M, int N, int K, int num_cu);
     hipError_t launch_w4a16_gemm_q(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M, int N,
                                    int K, int group_shift, int zp, const void* zero_points, void* partial_ws, int num_cu);
     hipError_t launch_w4a16_gemm(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M,

@@ -392,15 +392,7 @@ namespace nnf
     }
 
     // ---- the tile GEMM with other block parameters ----------------------------------------------------------------------
-    bool w4a16_gemm_q_supported(int M, int N, int K, int group_shift)
-    {
-        return M > 16 && N >= 1 && K >= 256 && !(K & 255) && group_shift >= 5 && group_shift <= 7 &&
-               (size_t)M * K * 2 + 8192 < ((size_t)1 << 32) && (size_t)N * (K >> 1) < ((size_t)1 << 32);
-    }
-    size_t w4a16_gemm_q_workspace_bytes(int M, int N, int K, int num_cu)
-    {
-        return workspace::plan_w4a16_sk(M, N, K, false, num_cu).bytes();
-    }
+    bool w4a16_gemm_q_supported(int M, int N, int K, int group_shift) { return workspace::w4a16_gemm_q_fits(M, N, K, group_shift); }
     hipError_t launch_w4a16_gemm_q(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M, int N,
                                    int K, int group_shift, int zp, const void* zero_points, void* partial_ws, int num_cu)
     {

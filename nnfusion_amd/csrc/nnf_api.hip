@@ -212,9 +212,7 @@ size_t nnf_wna16_gemm_workspace_bytes(int M, int N, int K, const nnf_quant* q)
     if (is_plain_w4a16(q))
         return nnf::workspace::w4a16_gemm(M, N, K, q->group);
     // 4-bit weights above 16 rows: the tile GEMM where tiles are shared between workgroups (without it: the plain tile kernel)
-    if (q->bits == 4 && nnf_wna16_supported(M, N, K, q) && nnf::w4a16_gemm_q_supported(M, N, K, group_shift_of(q->group)))
-        return nnf::w4a16_gemm_q_workspace_bytes(M, N, K, nnf::workspace::PLAN_CUS);
-    return 0;
+    return nnf_wna16_supported(M, N, K, q) ? nnf::workspace::wna16_gemm(M, N, K, q->bits, q->group) : 0;
 }
 
 int nnf_wna16_gemm(nnf_stream_t stream, const void* A, const void* Wq, const void* scales, void* Y, int M, int N, int K,
@@ -239,7 +237,7 @@ int nnf_wna16_gemm(nnf_stream_t stream, const void* A, const void* Wq, const voi
     if (q->bits == 4 && nnf::w4a16_gemm_q_supported(M, N, K, group_shift_of(q->group)) &&
         (reinterpret_cast<uintptr_t>(q->zero_points) & 3) == 0)
     {
-        const size_t need = nnf::w4a16_gemm_q_workspace_bytes(M, N, K, dev.num_cu);
+        const size_t need = nnf::workspace::wna16_gemm(M, N, K, q->bits, q->group, dev.num_cu);
         if (need == 0 || (workspace && aligned16(workspace) && workspace_bytes >= need))
             return (int)nnf::launch_w4a16_gemm_q((hipStream_t)stream, A, Wq, scales, Y, M, N, K, group_shift_of(q->group),
                                                  q->zero_point, q->zero_points, workspace, dev.num_cu);

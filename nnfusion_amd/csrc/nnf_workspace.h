@@ -213,6 +213,23 @@ namespace nnf
             return plan_w4a16_sk(M, N, K, gate, num_cu, tile_rows, t.tiles_m * t.tiles_n * workgroups_per_tile, tile_cols);
         }
 
+        // The tile GEMM with other block parameters (groups of 32 / 64 / 128, zero points per (row, group)): above 16 rows,
+        // K a multiple of 256 (the kernel addresses its operands with 32-bit byte offsets); the plain product, same plan
+        inline bool w4a16_gemm_q_fits(int M, int N, int K, int group_shift)
+        {
+            return M > 16 && N >= 1 && K >= 256 && !(K & 255) && group_shift >= 5 && group_shift <= 7 &&
+                   (size_t)M * K * 2 + 8192 < ((size_t)1 << 32) && (size_t)N * (K >> 1) < ((size_t)1 << 32);
+        }
+        // nnf_wna16_gemm with parameters other than 4 bits / groups of 128 / scalar zero point: [ parked tiles ] for 4-bit
+        // weights on the tile GEMM, nothing otherwise
+        inline size_t wna16_gemm(int M, int N, int K, int bits, int group, int num_cu = PLAN_CUS)
+        {
+            const int gs = group == 32 ? 5 : group == 64 ? 6 : group == 128 ? 7 : 0;
+            if (bits != 4 || !w4a16_gemm_q_fits(M, N, K, gs))
+                return 0;
+            return plan_w4a16_sk(M, N, K, false, num_cu).bytes();
+        }
+
         // ---- plan of the skinny (M <= 16) MFMA GEMV kernel ---------------------------------------------
         constexpr size_t LDS_BYTES_PER_CU = 160 * 1024; // gfx950
         struct SkinnyPlan

@@ -912,6 +912,25 @@ int main(int argc, char** argv)
             EXPECT(threw);
         }
         {
+            // 4-bit weights above 16 rows with K a multiple of 256: the tile GEMM's scratch memory comes with the call
+            auto g = std::make_shared<graph::Graph>();
+            auto x = param(*g, element::f16, Shape{128, 4096});
+            auto q = quant_dot(*g, {x, cst(*g, element::u8, Shape{4096, 2048}), cst(*g, element::f16, Shape{4096, 64}),
+                                    cst(*g, element::u8, Shape{4096, 32})},
+                               "{\"group_size\": 64, \"has_zero_points\": true}");
+            auto k = sel.pick_first(q, ROCM_GPU).second;
+            const std::string body = k->get_or_emit_source()->body_unit->get_code();
+            const size_t ws = nnf::workspace::wna16_gemm(128, 4096, 4096, 4, 64);
+            EXPECT(ws > 0 && ws == nnf::workspace::plan_w4a16_sk(128, 4096, 4096, false, nnf::workspace::PLAN_CUS).bytes());
+            CONTAINS(body, "const nnf_quant quant = {4, 64, 8, input3};");
+            CONTAINS(body, "nnf_wna16_gemm(stream, input0, input1, input2, output0, 128, 4096, 4096, &quant, ");
+            CONTAINS(body, ", " + std::to_string(ws) + "));");
+            EXPECT(body.find("&quant, nullptr") == std::string::npos);
+            // 8-bit weights, K not a multiple of 256, 16 rows: the kernels that need none
+            EXPECT(nnf::workspace::wna16_gemm(128, 4096, 4096, 8, 64) == 0 && nnf::workspace::wna16_gemm(128, 4096, 4096 + 128, 4, 64) == 0 &&
+                   nnf::workspace::wna16_gemm(16, 4096, 4096, 4, 64) == 0 && nnf::workspace::wna16_gemm(128, 4096, 4096, 4, 16) == 0);
+        }
+        {
             // RMSNorm -> QuantDot(groups of 64) -> Add: nothing folds into a product the fused kernels do not serve
             auto g = std::make_shared<graph::Graph>();
             auto x = param(*g, element::f16, Shape{M, K});

@@ -69,6 +69,11 @@ def test_pure_host_queries_work_without_a_gpu():
         assert lib.nnf_wna16_supported(8, 64, 256, p) == ok, fields
     keep, p = qp(4, 64, 8, None)
     assert lib.nnf_wna16_supported(8, 64, 96, p) == 0  # K % group
+    # 4-bit weights above 16 rows: the tile GEMM's parked tiles; none for 8-bit weights, up to 16 rows, other K
+    assert lib.nnf_wna16_gemm_workspace_bytes(128, 4096, 4096, p) == lib.nnf_w4a16_gemm_workspace_bytes(128, 4096, 4096, 128) > 0
+    assert lib.nnf_wna16_gemm_workspace_bytes(16, 4096, 4096, p) == 0
+    assert lib.nnf_wna16_gemm_workspace_bytes(128, 4096, 4096 + 64, p) == 0
+    keep, p = qp(8, 64, 8, None)
     assert lib.nnf_wna16_gemm_workspace_bytes(128, 4096, 4096, p) == 0
     keep, p = qp(4, 128, 8, None)
     assert lib.nnf_wna16_gemm_workspace_bytes(128, 4096, 4096, p) == lib.nnf_w4a16_gemm_workspace_bytes(128, 4096, 4096, 128) > 0

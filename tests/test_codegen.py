@@ -179,6 +179,12 @@ def test_generated_runtime_of_an_onnx_model(gpu):
     y = _run_generated("onnx_linear_w8", [a], (m, n), torch.float16, gpu)
     ref = oracle.wna16_gemm(a, wq, s, 8, 64, zero_points=z, f32_out=True)
     assert np.abs(y.astype(np.float32) - ref).max() <= 1e-2 * _rms(ref)
+    # 4-bit weights in blocks of 32 with a zero point each, 200 rows: the tile GEMM with the generated code's scratch memory
+    _, m, n, k = entry.ONNX_EXAMPLES["onnx_linear_w4z"]
+    a, wq, s, z = datagen.wna16_case(0, m, n, k, 4, 32, True)
+    y = _run_generated("onnx_linear_w4z", [a], (m, n), torch.float16, gpu)
+    ref = oracle.wna16_gemm(a, wq, s, 4, 32, zero_points=z, f32_out=True)
+    assert np.abs(y.astype(np.float32) - ref).max() <= 1e-2 * _rms(ref)
 
 
 @pytest.mark.gpu
