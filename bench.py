@@ -73,9 +73,9 @@ DOMINANT_KERNEL = {
     "wna16_b8_g128_zp_scalar_N8192_K8192.M1": "nnf::wna16_gemv_kernel<8, 4, 1>",
     "wna16_b8_g128_zp_scalar_N8192_K8192.M16": "nnf::wna16_skinny_kernel<8, 2>",
     "wna16_b8_g128_zp_scalar_N8192_K8192.M4096": "nnf::wna16_tile128_kernel<8>",
-    "wna16_b4_g64_zp_tensor_N8192_K8192.M1": "nnf::wna16_gemv_kernel<4, 4, 1>",
-    "wna16_b4_g64_zp_tensor_N8192_K8192.M16": "nnf::wna16_skinny_kernel<4, 2>",
-    "wna16_b4_g64_zp_tensor_N8192_K8192.M4096": "nnf::wna16_tile128_kernel<4>",
+    "wna16_b4_g64_zp_tensor_N8192_K8192.M1": "nnf::w4a16_gemv_rows_q_kernel<2, D, 8, 3> (row-streaming GEMV, zero points per group)",
+    "wna16_b4_g64_zp_tensor_N8192_K8192.M16": "nnf::w4a16_mrows_q_kernel<4, 6, true> (row-streaming MFMA kernel)",
+    "wna16_b4_g64_zp_tensor_N8192_K8192.M4096": "nnf::gemm_sk::w4a16_gemm_sk_kernel<8, 2, ..., 6> (stream-K tile GEMM, groups of 64)",
     "fused_mlp_M1_4096_11008": "2 x nnf::w4a16_gemv_rows_fused_kernel (gate|up with RMSNorm and SiLU, down with the residual)",
     "fused_mlp_M16_4096_11008": "nnf::w4a16_mrows_kernel (gate|up with RMSNorm and SiLU) + w4a16_mrows_any_kernel over 3 ranges of K + "
                                 "splitk_reduce_kernel (down)",
