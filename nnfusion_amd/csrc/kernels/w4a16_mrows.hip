@@ -399,7 +399,7 @@ namespace nnf
 
     // ---- other block parameters ------------------------------------------------------------------------------------
     // The same kernel for groups of 2^GSHIFT = 32 / 64 / 128 weights and (ZPT) a zero point per (row, group) from
-    // `zps`, u8 [N, K / group / 2], even group in the low nibble; 2 <= M <= 16, K = GW * 2048 (two steps per tile).
+    // `zps`, u8 [N, K / group / 2], even group in the low nibble; 2 <= M <= 16 MB, K = GW * 2048 (two steps per tile).
     // A lane's 16-byte piece of a weight row (32 weights) lies in one group whatever its size, but the four lanes that meet
     // in one MFMA column hold pieces of up to four groups: a scale cannot be applied to the MFMA's sum.  The weights
     // are therefore dequantised before the MFMA, as the tile GEMM does:  fp16((q - z) * s),  q - z exact (nibble trick
@@ -409,9 +409,9 @@ namespace nnf
     // loads, NSL of them) and, ZPT, their zero points (one byte per lane, NZL loads; a byte load lands in a lane's four
     // bytes of LDS).
     // LDS (bytes): weights [8 wavefronts][2 slots][GW KiB] | scales and zero points [8][2][(NSL + NZL) x 256] |
-    //              partial tiles [2][8][1 KiB] | parked sums [tiles of the workgroup][M][16] fp32
+    //              partial tiles [2][8][MB KiB] | parked sums [tiles of the workgroup][M][16] fp32
     // pack = M | zp << 8.
-    template <int GW, int GSHIFT, bool ZPT>
+    template <int GW, int GSHIFT, bool ZPT, int MB>
     __global__ __launch_bounds__(512) void w4a16_mrows_q_kernel(const half_t* __restrict__ A, const uint8_t* __restrict__ Wq,
                                                                 const half_t* __restrict__ S, half_t* __restrict__ Y,
                                                                 const uint8_t* __restrict__ zps, int N, int tiles_q,
@@ -419,7 +419,8 @@ namespace nnf
     {
         static_assert(GW == 1 || GW == 2 || GW == 4, "K = 2048, 4096, 8192");
         static_assert(GSHIFT >= 5 && GSHIFT <= 7 && ((GW << (7 - GSHIFT)) & 1) == 0, "whole words of scales, whole bytes of zero points");
-        constexpr int STEPS = 2, MB = 1;
+        static_assert(MB == 1 || (MB == 2 && GW <= 2), "two blocks of rows: 32 VGPRs per group");
+        constexpr int STEPS = 2;
         constexpr int K = GW * STEPS * 1024, G = K >> GSHIFT;
         constexpr int GA = GW * STEPS;         // groups of 128 of a wavefront
         constexpr int ROW_BYTES = K / 2;       // a weight row
@@ -503,21 +504,26 @@ namespace nnf
         issue(0, 1, 1);
         // activations: straight into the MFMA operand registers, in the pair order of the nibble trick
         uintx4 areg[MB][GA][4];
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
         {
             const uint8_t* a_bytes = reinterpret_cast<const uint8_t*>(A);
-            const uint32_t a_off = (uint32_t)min(col, M - 1) * (uint32_t)(K * 2) + (uint32_t)wave * (GW * 256) + (uint32_t)kq * 64u;
+            const uint32_t a_off =
+                (uint32_t)min(mb * 16 + col, M - 1) * (uint32_t)(K * 2) + (uint32_t)wave * (GW * 256) + (uint32_t)kq * 64u;
 #pragma unroll
             for (int g = 0; g < GA; ++g)
 #pragma unroll
                 for (int j = 0; j < 4; ++j)
-                    areg[0][g][j] = *reinterpret_cast<const uintx4*>(
+                    areg[mb][g][j] = *reinterpret_cast<const uintx4*>(
                         a_bytes + (size_t)(a_off + (g / GW) * (SPAN * 4) + (g % GW) * 256 + j * 16));
+        }
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
             for (int g = 0; g < GA; ++g)
 #pragma unroll
                 for (int j = 0; j < 4; ++j)
-                    areg[0][g][j] = permute_a8(areg[0][g][j]);
-        }
+                    areg[mb][g][j] = permute_a8(areg[mb][g][j]);
 
         // ---- tile loop ---------------------------------------------------------------------------------------
         const uint32_t rd_base = (uint32_t)col * SLICE;
@@ -540,7 +546,10 @@ namespace nnf
         int slot = 0;
         for (int it = 0; it < T; ++it)
         {
-            floatx4 acc[MB] = {floatx4{0.f, 0.f, 0.f, 0.f}};
+            floatx4 acc[MB];
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb)
+                acc[mb] = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int st = 0; st < STEPS; ++st)
             {
@@ -585,17 +594,23 @@ namespace nnf
                         bq.y = as_u32((as_half2((w & MASK_HI) | MAGIC_HI) + hi_add) * sc);  // (q1, q5)
                         bq.z = as_u32((as_half2((w8 & MASK_LO) | MAGIC) + lo_add) * sc);    // (q2, q6)
                         bq.w = as_u32((as_half2((w8 & MASK_HI) | MAGIC_HI) + hi_add) * sc); // (q3, q7)
-                        acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, areg[0][st * GW + g][j]),
-                                                                        __builtin_bit_cast(half8_t, bq), acc[0], 0, 0, 0);
+#pragma unroll
+                        for (int mb = 0; mb < MB; ++mb)
+                            acc[mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, areg[mb][st * GW + g][j]),
+                                                                             __builtin_bit_cast(half8_t, bq), acc[mb], 0, 0, 0);
                     }
                 }
             }
             // (mrows_reduce_park stores the sums with inline assembly, and the wait between an MFMA and a read of its
             // result is only inserted ahead of instructions the compiler emits itself: one such instruction)
-            acc[0].x *= one;
-            acc[0].y *= one;
-            acc[0].z *= one;
-            acc[0].w *= one;
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb)
+            {
+                acc[mb].x *= one;
+                acc[mb].y *= one;
+                acc[mb].z *= one;
+                acc[mb].w *= one;
+            }
             mrows_reduce_park<MB>(acc, red, red_addr, parked_addr, it & 1, it, M, tid);
         }
         __builtin_amdgcn_s_waitcnt(mr_vmcnt(0)); // the reloads past the end, before the LDS goes away
@@ -926,11 +941,11 @@ namespace nnf
 
     namespace
     {
-        template <int GW, int GSHIFT, bool ZPT>
-        hipError_t launch_mrows_q(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M, int N, int zp,
-                                  const void* zps, int num_cu)
+        template <int GW, int GSHIFT, bool ZPT, int MB>
+        hipError_t launch_mrows_q_mb(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M, int N, int zp,
+                                     const void* zps, int num_cu)
         {
-            if constexpr (((GW << (7 - GSHIFT)) & 1) != 0)
+            if constexpr (((GW << (7 - GSHIFT)) & 1) != 0 || (MB == 2 && GW > 2))
                 return hipErrorInvalidValue;
             else
             {
@@ -940,7 +955,7 @@ namespace nnf
                 const size_t lds = workspace::w4a16_mrows_q_lds_bytes(GW * 2048, M, tiles_q + (tiles_r ? 1 : 0), GSHIFT, ZPT);
                 if (lds > MAX_LDS_BYTES)
                     return hipErrorInvalidValue;
-                auto kernel = &w4a16_mrows_q_kernel<GW, GSHIFT, ZPT>;
+                auto kernel = &w4a16_mrows_q_kernel<GW, GSHIFT, ZPT, MB>;
                 if (lds > 64 * 1024)
                 {
                     static LdsGrant granted;
@@ -952,6 +967,13 @@ namespace nnf
                                    (const half_t*)S, (half_t*)Y, (const uint8_t*)zps, N, tiles_q, tiles_r, M | (zp << 8));
                 return hipGetLastError();
             }
+        }
+        template <int GW, int GSHIFT, bool ZPT>
+        hipError_t launch_mrows_q(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M, int N, int zp,
+                                  const void* zps, int num_cu)
+        {
+            return M <= 16 ? launch_mrows_q_mb<GW, GSHIFT, ZPT, 1>(stream, A, Wq, S, Y, M, N, zp, zps, num_cu)
+                           : launch_mrows_q_mb<GW, GSHIFT, ZPT, 2>(stream, A, Wq, S, Y, M, N, zp, zps, num_cu);
         }
         template <int GW>
         hipError_t launch_mrows_q_gw(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M, int N,

@@ -559,6 +559,9 @@ namespace nnf
         qa.group_shift = group == 32 ? 5 : group == 64 ? 6 : 7;
         qa.zp = zp;
         qa.zp_stride = (K / group * bits + 7) / 8;
+        // 4-bit weights, a few rows (up to 32 at K = 2048 / 4096, 16 at 8192): the row-streaming MFMA kernel
+        if (bits == 4 && M >= 2 && w4a16_mrows_q_supported(M, N, K, qa.group_shift, zero_points != nullptr, num_cu))
+            return launch_w4a16_mrows_q(stream, A, Wq, S, Y, M, N, K, qa.group_shift, zp, zero_points, num_cu);
         if (M <= 16)
         {
             if (M == 1)
@@ -572,9 +575,6 @@ namespace nnf
                     launch_wna16_gemv<8, 4, 1>(stream, A, Wq, S, Y, M, N, K, qa, num_cu);
                 return hipGetLastError();
             }
-            // 4-bit weights with K = 2048 / 4096 / 8192: the row-streaming MFMA kernel
-            if (bits == 4 && w4a16_mrows_q_supported(M, N, K, qa.group_shift, zero_points != nullptr, num_cu))
-                return launch_w4a16_mrows_q(stream, A, Wq, S, Y, M, N, K, qa.group_shift, zp, zero_points, num_cu);
             // blocks of two tiles of 16 rows, at most four workgroups per CU
             const int blocks = (N + 31) / 32, cap = num_cu * 4;
             const dim3 grid((unsigned)(blocks < cap ? blocks : cap));

@@ -235,6 +235,7 @@ int nnf_wna16_gemm(nnf_stream_t stream, const void* A, const void* Wq, const voi
     // 4-bit weights above 16 rows: the stream-K tile GEMM, given the workspace its plan on this device needs (and
     // zero points it can fetch four bytes at a time)
     if (q->bits == 4 && nnf::w4a16_gemm_q_supported(M, N, K, group_shift_of(q->group)) &&
+        !nnf::w4a16_mrows_q_supported(M, N, K, group_shift_of(q->group), q->zero_points != nullptr, dev.num_cu) &&
         (reinterpret_cast<uintptr_t>(q->zero_points) & 3) == 0)
     {
         const size_t need = nnf::workspace::wna16_gemm(M, N, K, q->bits, q->group, dev.num_cu);

@@ -213,23 +213,6 @@ namespace nnf
             return plan_w4a16_sk(M, N, K, gate, num_cu, tile_rows, t.tiles_m * t.tiles_n * workgroups_per_tile, tile_cols);
         }
 
-        // The tile GEMM with other block parameters (groups of 32 / 64 / 128, zero points per (row, group)): above 16 rows,
-        // K a multiple of 256 (the kernel addresses its operands with 32-bit byte offsets); the plain product, same plan
-        inline bool w4a16_gemm_q_fits(int M, int N, int K, int group_shift)
-        {
-            return M > 16 && N >= 1 && K >= 256 && !(K & 255) && group_shift >= 5 && group_shift <= 7 &&
-                   (size_t)M * K * 2 + 8192 < ((size_t)1 << 32) && (size_t)N * (K >> 1) < ((size_t)1 << 32);
-        }
-        // nnf_wna16_gemm with parameters other than 4 bits / groups of 128 / scalar zero point: [ parked tiles ] for 4-bit
-        // weights on the tile GEMM, nothing otherwise
-        inline size_t wna16_gemm(int M, int N, int K, int bits, int group, int num_cu = PLAN_CUS)
-        {
-            const int gs = group == 32 ? 5 : group == 64 ? 6 : group == 128 ? 7 : 0;
-            if (bits != 4 || !w4a16_gemm_q_fits(M, N, K, gs))
-                return 0;
-            return plan_w4a16_sk(M, N, K, false, num_cu).bytes();
-        }
-
         // ---- plan of the skinny (M <= 16) MFMA GEMV kernel ---------------------------------------------
         constexpr size_t LDS_BYTES_PER_CU = 160 * 1024; // gfx950
         struct SkinnyPlan
@@ -512,8 +495,8 @@ namespace nnf
             const int grid = n_tiles < num_cu ? n_tiles : num_cu;
             return w4a16_mrows_lds_bytes(K, M, (gate ? 2 : 1) * ((n_tiles + grid - 1) / grid)) <= LDS_BYTES_PER_CU;
         }
-        // The same kernel for groups of 32 / 64 / 128 and zero points per (row, group) (w4a16_mrows_q_kernel): 2 .. 16 rows,
-        // K = 2048, 4096, 8192 (GW = K / 2048 groups of 128 per wavefront and step); per wavefront and ring slot 256 bytes
+        // The same kernel for groups of 32 / 64 / 128 and zero points per (row, group) (w4a16_mrows_q_kernel): 2 .. 16 rows
+        // (.. 32 up to K = 4096), K = 2048, 4096, 8192 (GW = K / 2048 groups of 128 per wavefront and step); per wavefront and ring slot 256 bytes
         // per 64 4-byte words of scales (GW x 128 / group scales for each of 16 rows) and as much again for zero points.
         inline size_t w4a16_mrows_q_lds_bytes(int K, int M, int tiles, int group_shift, bool zero_points)
         {
@@ -521,18 +504,38 @@ namespace nnf
             const int words = (gw << (7 - group_shift)) / 2; // of scales per row, step and wavefront
             const int loads = (16 * words + 63) / 64;
             const size_t aux = (size_t)(zero_points ? 2 : 1) * loads * 256;
-            return (size_t)8 * 2 * gw * 1024 + 8 * 2 * aux + (size_t)2 * 8 * 1024 + (size_t)tiles * M * 64;
+            const size_t mb = M <= 16 ? 1 : 2; // blocks of 16 rows
+            return (size_t)8 * 2 * gw * 1024 + 8 * 2 * aux + (size_t)2 * 8 * mb * 1024 + (size_t)tiles * M * 64;
         }
+        // (17 .. 32 rows: two blocks of rows in registers, up to K = 4096)
         inline bool w4a16_mrows_q_fits(int M, int N, int K, int group_shift, bool zero_points, int num_cu)
         {
-            if (M < 2 || M > 16 || N < 16 || num_cu < 1 || (K != 2048 && K != 4096 && K != 8192) || group_shift < 5 ||
-                group_shift > 7)
+            if (M < 2 || M > 32 || (M > 16 && K > 4096) || N < 16 || num_cu < 1 || (K != 2048 && K != 4096 && K != 8192) ||
+                group_shift < 5 || group_shift > 7)
                 return false;
             if (((K >> 11) << (7 - group_shift)) & 1) // K = 2048 with groups of 128: half a word of scales per step
                 return false;
             const int n_tiles = (N + 15) / 16;
             const int grid = n_tiles < num_cu ? n_tiles : num_cu;
             return w4a16_mrows_q_lds_bytes(K, M, (n_tiles + grid - 1) / grid, group_shift, zero_points) <= LDS_BYTES_PER_CU;
+        }
+        // The tile GEMM with other block parameters (groups of 32 / 64 / 128, zero points per (row, group)): above 16 rows,
+        // K a multiple of 256 (the kernel addresses its operands with 32-bit byte offsets); the plain product, same plan
+        inline bool w4a16_gemm_q_fits(int M, int N, int K, int group_shift)
+        {
+            return M > 16 && N >= 1 && K >= 256 && !(K & 255) && group_shift >= 5 && group_shift <= 7 &&
+                   (size_t)M * K * 2 + 8192 < ((size_t)1 << 32) && (size_t)N * (K >> 1) < ((size_t)1 << 32);
+        }
+        // nnf_wna16_gemm with parameters other than 4 bits / groups of 128 / scalar zero point: [ parked tiles ] for 4-bit
+        // weights on the tile GEMM, nothing otherwise
+        inline size_t wna16_gemm(int M, int N, int K, int bits, int group, int num_cu = PLAN_CUS)
+        {
+            const int gs = group == 32 ? 5 : group == 64 ? 6 : group == 128 ? 7 : 0;
+            if (bits != 4 || !w4a16_gemm_q_fits(M, N, K, gs))
+                return 0;
+            if (w4a16_mrows_q_fits(M, N, K, gs, true, num_cu)) // up to 32 rows: the row-streaming kernel
+                return 0;
+            return plan_w4a16_sk(M, N, K, false, num_cu).bytes();
         }
         // K above 8192 (above 4096 for 17 .. 32 rows, above 2048 for 33 .. 64; a multiple of 256): the run-time-K form over equal ranges of K (in whole pairs of
         // groups; the last range may be shorter), each on its share of the CUs; fp32 sums per range, added by the

@@ -1024,7 +1024,13 @@ int main(int argc, char** argv)
             EXPECT(ws::w4a16_mrows_q_fits(2, 4096, 4096, 5, false, 256));
             EXPECT(ws::w4a16_mrows_q_fits(8, 300, 2048, 6, true, 256));
             EXPECT(!ws::w4a16_mrows_q_fits(8, 300, 2048, 7, true, 256)); // half a word of scales
-            EXPECT(!ws::w4a16_mrows_q_fits(1, 4096, 4096, 5, false, 256) && !ws::w4a16_mrows_q_fits(17, 4096, 4096, 5, false, 256));
+            EXPECT(!ws::w4a16_mrows_q_fits(1, 4096, 4096, 5, false, 256) && !ws::w4a16_mrows_q_fits(33, 4096, 4096, 5, false, 256));
+            // 17 .. 32 rows: two blocks of rows in registers, up to K = 4096 (no workspace: not the tile GEMM)
+            EXPECT(ws::w4a16_mrows_q_fits(17, 4096, 4096, 5, false, 256) && ws::w4a16_mrows_q_fits(32, 12288, 2048, 6, true, 256));
+            EXPECT(!ws::w4a16_mrows_q_fits(17, 8192, 8192, 5, false, 256));
+            EXPECT(ws::w4a16_mrows_q_lds_bytes(4096, 32, 1, 6, false) == 32768 + 4096 + 32768 + 2048);
+            EXPECT(ws::wna16_gemm(32, 4096, 4096, 4, 64) == 0 && ws::wna16_gemm(32, 8192, 8192, 4, 64) > 0 &&
+                   ws::wna16_gemm(33, 4096, 4096, 4, 64) > 0);
             EXPECT(!ws::w4a16_mrows_q_fits(8, 4096, 6144, 5, false, 256) && !ws::w4a16_mrows_q_fits(8, 4096, 11008, 5, false, 256));
             EXPECT(!ws::w4a16_mrows_q_fits(8, 4096, 4096, 4, false, 256) && !ws::w4a16_mrows_q_fits(8, 8, 4096, 5, false, 256));
             // ring 8 x 2 x 4 KiB, scales and zero points 8 x 2 x (2 + 2) x 256, partial tiles 16 KiB, two parked tiles

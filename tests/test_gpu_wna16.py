@@ -51,6 +51,7 @@ SHAPES = [
     # a few rows of 4-bit weights with K = 2048 / 4096 / 8192: the row-streaming MFMA kernel (one, two and four loads per
     # step and wavefront; fewer tiles than CUs, a ragged last tile, several tiles per workgroup)
     (2, 4096, 4096), (5, 300, 2048), (8, 1000, 8192), (16, 48, 8192), (13, 12288, 4096), (16, 9000, 2048),
+    (17, 4096, 4096), (32, 1000, 2048), (25, 12288, 4096), (31, 40, 4096),
     # the tile kernel: one partial tile, ragged M and N, many tiles, a long K
     (17, 33, 128), (64, 64, 512), (100, 1000, 160), (300, 257, 2048), (128, 4096, 4096), (33, 520, 11008), (1024, 130, 384),
     # 4-bit weights above 16 rows with K a multiple of 256: the stream-K tile GEMM (tiles of 32 x 256, 64 x 128, 128 x 128,
@@ -97,7 +98,8 @@ def test_one_hot_rows_return_the_dequantised_weights(gpu, m, n, k, bits, group, 
     assert not y[len(ks):].any()
 
 
-@pytest.mark.parametrize("m,k", [(1, 1024), (1, 4096), (1, 11008), (1, 16384), (7, 2048), (16, 4096), (3, 8192)])
+@pytest.mark.parametrize("m,k", [(1, 1024), (1, 4096), (1, 11008), (1, 16384), (7, 2048), (16, 4096), (3, 8192), (32, 4096),
+                                 (20, 2048)])
 @pytest.mark.parametrize("group,zp_tensor", [(32, True), (64, True), (128, True), (32, False), (64, False)])
 def test_one_hot_rows_through_the_row_streaming_kernels(gpu, m, k, group, zp_tensor):
     """4-bit weights with one row and K a multiple of 256, or a few rows and K = 2048 / 4096 / 8192, run on the
@@ -117,6 +119,26 @@ def test_one_hot_rows_through_the_row_streaming_kernels(gpu, m, k, group, zp_ten
         for r, kk in enumerate(chunk):
             np.testing.assert_array_equal(y[r], wd[:, kk].astype(np.float16), err_msg="k = %d" % kk)
         assert not y[len(chunk):].any()
+
+
+def test_tile_gemm_without_its_workspace_runs_on_the_plain_kernel(gpu):
+    """Above 16 rows 4-bit weights want the stream-K tile GEMM's workspace; a caller that brings none (or too little)
+    gets the same product from the plain tile kernel."""
+    import torch
+
+    from nnfusion_amd import ops
+
+    m, n, k, group = 130, 1024, 4096, 64
+    a, wq, s, zps = _case(21, m, n, k, 4, group, True)
+    need = ops.wna16_workspace_bytes(m, n, k, 4, group)
+    assert need > 0
+    t = [torch.from_numpy(x).to(gpu) for x in (a, wq, s, zps)]
+    ref = oracle.wna16_gemm(a, wq, s, 4, group, zero_points=zps, f32_out=True)
+    for ws_bytes in (need, need - 16, 16):
+        y = ops.wna16_gemm(t[0], t[1], t[2], bits=4, group=group, zero_points=t[3],
+                           workspace=torch.empty(ws_bytes, dtype=torch.uint8, device=gpu))
+        torch.cuda.synchronize()
+        _check(y.cpu().numpy(), ref)
 
 
 def test_default_parameters_are_the_specialised_kernels(gpu):
