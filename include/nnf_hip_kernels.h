@@ -148,9 +148,10 @@ int nnf_w4a16_gemm_variant(nnf_stream_t stream,
  * bits 4, group 128 and no zero-point tensor is nnf_w4a16_gemm itself (same kernels, same workspace).  For every other
  * combination (group 32 / 64 / 128, K a multiple of group) 4-bit weights run on the kernels of nnf_w4a16_gemm where
  * those apply: the row-streaming kernels for M = 1 with K a multiple of 256 from 1024 to 16384 and for 2 <= M <= 16
- * with K = 2048 / 4096 / 8192 (up to 32 rows at 2048 / 4096; groups of 128 with a zero-point tensor: not 2048), and the
- * tile GEMM for the other shapes above 16 rows with K a multiple of 256 and zero_points 4-byte aligned.  The tile GEMM wants nnf_wna16_gemm_workspace_bytes of
- * workspace; called with less (or NULL) the product runs on a plain tile kernel instead, at less than half the rate.
+ * with K a multiple of 256 from about 2560 on (2048 / 4096 also up to 32 rows; above K = 8192 over ranges of K with a
+ * reduction pass), and the tile GEMM for the other shapes above 16 rows with K a multiple of 256 and zero_points
+ * 4-byte aligned.  The ranges of K and the tile GEMM want nnf_wna16_gemm_workspace_bytes of workspace; called with
+ * less (or NULL) the product runs on a plain kernel instead, at about half the rate.
  * Everything else runs on plain kernels that need no workspace: a row-per-wavefront GEMV for M = 1, an MFMA kernel
  * with the operands fetched straight into registers for 2 <= M <= 16, MFMA tiles through LDS above. */
 typedef struct nnf_quant

@@ -81,6 +81,13 @@ namespace nnf
     hipError_t launch_w4a16_mrows_q(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M, int N,
                                     int K, int group_shift, int zp, const void* zero_points, int num_cu);
     bool w4a16_mrows_q_supported(int M, int N, int K, int group_shift, bool zero_points, int num_cu);
+    // ... with K any other multiple of 256 (2 <= M <= 16).  w4a16_mrows_q_any_ranges: 0 does not apply; 1: results to Y;
+    // more: fp32 sums of each range of K to partial[ranges][M][N], Y is not written (launch_wna16_reduce adds them up)
+    int w4a16_mrows_q_any_ranges(int M, int N, int K, int group_shift, bool zero_points, int num_cu);
+    hipError_t launch_w4a16_mrows_q_any(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, float* partial,
+                                        int M, int N, int K, int group_shift, int zp, const void* zero_points, int num_cu);
+    // Y [M, N] = fp16(sum over the ranges of partial[ranges][M][N])
+    hipError_t launch_wna16_reduce(hipStream_t stream, const float* partial, int ranges, void* Y, int M, int N);
     hipError_t launch_w4a16_mrows(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M, int N,
                                   int K, int zp, int num_cu, const GemvFusion& fusion = GemvFusion());
     bool w4a16_mrows_supported(int M, int N, int K, int num_cu, bool gate = false);

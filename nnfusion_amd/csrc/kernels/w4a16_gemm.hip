@@ -391,6 +391,22 @@ namespace nnf
         }
     }
 
+    hipError_t launch_wna16_reduce(hipStream_t stream, const float* partial, int ranges, void* Y, int M, int N)
+    {
+        GemmParams p;
+        p.Y = (half_t*)Y;
+        p.M = M;
+        p.N = N;
+        p.ldy = N;
+        p.bias = nullptr;
+        p.residual = nullptr;
+        p.rstd = nullptr;
+        p.partial = const_cast<float*>(partial);
+        p.splits = ranges;
+        p.ld_partial = N;
+        return launch_reduce_any(stream, p, false, false, false);
+    }
+
     // ---- the tile GEMM with other block parameters ----------------------------------------------------------------------
     bool w4a16_gemm_q_supported(int M, int N, int K, int group_shift) { return workspace::w4a16_gemm_q_fits(M, N, K, group_shift); }
     hipError_t launch_w4a16_gemm_q(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M, int N,

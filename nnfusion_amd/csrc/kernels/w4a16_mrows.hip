@@ -618,6 +618,220 @@ namespace nnf
         mrows_flush<false, MB>(parked, Y, t0, T, M, N, tid, GemvFusionArgs{nullptr, nullptr, nullptr, nullptr, 0.f}, 0);
     }
 
+    // w4a16_mrows_q_kernel with K as a run-time value (any multiple of 256; 2 <= M <= 16), as w4a16_mrows_any_kernel below
+    // does it for groups of 128 with a scalar zero point: two steps of 8 * GW blocks of 128 weights; a wavefront whose
+    // blocks of a step would reach past the end of its range of K fetches the last GW blocks of the range instead and
+    // multiplies what another wavefront already covers by scales of zero.  blockIdx.y numbers ranges of range_blocks
+    // blocks of K (the last one may be shorter, at least GW blocks); with `partial` the workgroups of a range write its
+    // fp32 sums to partial[range][M][N] for the reduction pass.
+    // A block of 128 weights has SPC = 128 / group scales; with groups of 128 a wavefront's first block may be an odd one:
+    // its scales are fetched from the 4-byte word, its zero points from the byte, at or below it (`skip` = 1), and
+    // one word / byte more per row comes along.
+    template <int GW, int GSHIFT, bool ZPT>
+    __global__ __launch_bounds__(512) void w4a16_mrows_q_any_kernel(const half_t* __restrict__ A, const uint8_t* __restrict__ Wq,
+                                                                    const half_t* __restrict__ S, half_t* __restrict__ Y,
+                                                                    const uint8_t* __restrict__ zps, float* __restrict__ partial,
+                                                                    int N, int K, int range_blocks, int tiles_q, int tiles_r,
+                                                                    int pack)
+    {
+        static_assert(GW >= 2 && GW <= 4 && GSHIFT >= 5 && GSHIFT <= 7, "blocks per wavefront and step; groups of 32 / 64 / 128");
+        constexpr int STEPS = 2, MB = 1;
+        constexpr int GA = GW * STEPS;
+        constexpr int SLICE = GW * 64;
+        constexpr int TILE_BYTES = 16 * SLICE;
+        constexpr int SPC = 1 << (7 - GSHIFT);                     // scales per block of 128 weights
+        constexpr int WPR = SPC == 1 ? GW / 2 + 1 : GW * SPC / 2;  // 4-byte words of scales (= bytes of zero points) per row
+        constexpr int NSL = (16 * WPR + 63) / 64;
+        constexpr int NZL = ZPT ? NSL : 0;
+        constexpr int AUX = (NSL + NZL) * 256;
+        constexpr int LT = GW + NSL + NZL;
+        extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+        uint32_t MAGIC, MAGIC_HI, MASK_LO, MASK_HI;
+        asm volatile("v_mov_b32 %0, 0x64006400" : "=v"(MAGIC));
+        asm volatile("v_mov_b32 %0, 0x54005400" : "=v"(MAGIC_HI));
+        asm volatile("s_mov_b32 %0, 0x000F000F" : "=s"(MASK_LO));
+        asm volatile("s_mov_b32 %0, 0x00F000F0" : "=s"(MASK_HI));
+
+        const int tid = threadIdx.x;
+        const int lane = tid & 63;
+        const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+        const int col = lane & 15;
+        const int kq = lane >> 4;
+        const int M = pack & 0xff, zp = (pack >> 8) & 0xff;
+        const int B = K >> 7, ROW_BYTES = K >> 1; // blocks of 128 weights in a row
+        const int SROW = (K >> GSHIFT) * 2;       // bytes of a row of scales
+        const int ZROW = K >> (GSHIFT + 1);       // bytes of a row of zero points
+        const int b = blockIdx.x;
+        const int t0 = b * tiles_q + min(b, tiles_r);
+        const int T = tiles_q + (b < tiles_r ? 1 : 0);
+        auto row0_of = [&](int i) { return __builtin_amdgcn_readfirstlane(min((t0 + i) * 16, N - 16)); };
+        const int b_lo = (int)blockIdx.y * range_blocks, b_hi = min(B, b_lo + range_blocks); // this workgroup's part of K
+        auto own_block = [&](int st) { return b_lo + st * (8 * GW) + wave * GW; };
+        auto fetch_block = [&](int st) { return min(own_block(st), b_hi - GW); };
+
+        uint8_t* ring = smem + wave * (2 * TILE_BYTES);
+        uint8_t* aux = smem + MR_WAVES * 2 * TILE_BYTES + wave * (2 * AUX);
+        uint8_t* red = smem + MR_WAVES * 2 * TILE_BYTES + MR_WAVES * 2 * AUX; // [2][8][1024]
+        float* parked = reinterpret_cast<float*>(red + 2 * MR_WAVES * MB * 1024);
+
+        auto swz = [](int r) { return GW % 4 == 0 ? (r & 15) : GW % 2 == 0 ? (r >> 1) & 7 : (r >> 2) & 3; };
+        uint32_t w_off[GW];
+#pragma unroll
+        for (int c = 0; c < GW; ++c)
+        {
+            const int pos = c * 1024 + 16 * lane;
+            const int r = pos / SLICE, q = (pos % SLICE) >> 4;
+            w_off[c] = (uint32_t)r * (uint32_t)ROW_BYTES + (uint32_t)((q ^ swz(r)) << 4);
+        }
+        // scales / zero points: lane l of load i fetches word / byte (64 i + l) % WPR of row (64 i + l) / WPR, counted from
+        // the word / byte that holds the first fetched block's (never past the end of the row: the last one again instead)
+        int aux_row[NSL], aux_word[NSL];
+#pragma unroll
+        for (int i = 0; i < NSL; ++i)
+        {
+            const int at = i * 64 + lane;
+            aux_row[i] = min(at / WPR, 15);
+            aux_word[i] = at % WPR;
+        }
+
+        auto issue = [&](int tile, int st, int slot) {
+            const uint32_t row0 = (uint32_t)row0_of(tile);
+            const int bs = fetch_block(st);
+            const uint8_t* wsrc = Wq + (size_t)row0 * ROW_BYTES + bs * 64;
+#pragma unroll
+            for (int c = 0; c < GW; ++c)
+                __builtin_amdgcn_global_load_lds((mr_global_ptr_t)(wsrc + w_off[c]),
+                                                 (mr_lds_ptr_t)(ring + slot * TILE_BYTES + c * 1024), 16, 0, 0);
+            const int s_first = (bs * SPC * 2) & ~3;            // byte of the first word within the row's scales
+            const int s_last = ((SROW - s_first) >> 2) - 1;     // last word of this window that is still inside the row
+            const uint8_t* ssrc = reinterpret_cast<const uint8_t*>(S) + (size_t)row0 * SROW + s_first;
+#pragma unroll
+            for (int i = 0; i < NSL; ++i)
+                __builtin_amdgcn_global_load_lds((mr_global_ptr_t)(ssrc + (uint32_t)(aux_row[i] * SROW + 4 * min(aux_word[i], s_last))),
+                                                 (mr_lds_ptr_t)(aux + slot * AUX + i * 256), 4, 0, 0);
+            if constexpr (ZPT)
+            {
+                const int z_first = (bs * SPC) >> 1;
+                const int z_last = ZROW - z_first - 1;
+                const uint8_t* zsrc = zps + (size_t)row0 * ZROW + z_first;
+#pragma unroll
+                for (int i = 0; i < NSL; ++i)
+                    __builtin_amdgcn_global_load_lds((mr_global_ptr_t)(zsrc + (uint32_t)(aux_row[i] * ZROW + min(aux_word[i], z_last))),
+                                                     (mr_lds_ptr_t)(aux + slot * AUX + (NSL + i) * 256), 1, 0, 0);
+            }
+        };
+        issue(0, 0, 0);
+        issue(0, 1, 1);
+
+        const uint32_t rd_base = (uint32_t)col * SLICE;
+        const int rd_swz = swz(col);
+        const uint32_t red_addr = lds_address(red) + (uint32_t)(wave * (MB * 1024) + lane * 16);
+        const uint32_t parked_addr = lds_address(parked);
+        // activations: straight into the MFMA operand registers, in the pair order of the nibble trick
+        uintx4 areg[GA][4];
+        {
+            const uint8_t* a_row = reinterpret_cast<const uint8_t*>(A) + (size_t)min(col, M - 1) * (size_t)(K * 2) + kq * 64;
+#pragma unroll
+            for (int st = 0; st < STEPS; ++st)
+            {
+                const uint8_t* a_src = a_row + (size_t)fetch_block(st) * 256;
+#pragma unroll
+                for (int g = 0; g < GW; ++g)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        areg[st * GW + g][j] = *reinterpret_cast<const uintx4*>(a_src + g * 256 + j * 16);
+            }
+#pragma unroll
+            for (int g = 0; g < GA; ++g)
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    areg[g][j] = permute_a8(areg[g][j]);
+        }
+        const uint32_t zp16 = (uint32_t)zp | ((uint32_t)zp << 16);
+        const int sub = (kq * 32) >> GSHIFT; // the lane's scale within a block
+        float one; // a 1.0 the compiler cannot fold
+        asm volatile("v_mov_b32 %0, 1.0" : "=v"(one));
+        int slot = 0;
+        for (int it = 0; it < T; ++it)
+        {
+            floatx4 acc[MB] = {floatx4{0.f, 0.f, 0.f, 0.f}};
+#pragma unroll
+            for (int st = 0; st < STEPS; ++st)
+            {
+                // the blocks of this step that no other wavefront covers: from `fresh` on
+                const int bs = fetch_block(st);
+                const int fresh = own_block(st) - bs;
+                const int skip = SPC == 1 ? (bs & 1) : 0;
+                __builtin_amdgcn_s_waitcnt(mr_vmcnt(LT));
+                uintx4 wv[GW];
+                uint32_t s2[GW], z16[GW];
+                {
+                    const uint8_t* sl = ring + slot * TILE_BYTES + rd_base;
+                    const uint8_t* ax = aux + slot * AUX;
+#pragma unroll
+                    for (int g = 0; g < GW; ++g)
+                    {
+                        wv[g] = *reinterpret_cast<const uintx4*>(sl + (((g * 4 + kq) ^ rd_swz) << 4));
+                        const int idx = skip + g * SPC + sub; // among the scales this row fetched
+                        const uint32_t sh = *reinterpret_cast<const uint16_t*>(ax + (col * (WPR * 2) + idx) * 2);
+                        s2[g] = g >= fresh ? (sh | (sh << 16)) : 0u;
+                        if constexpr (ZPT)
+                        {
+                            const uint32_t z = ((uint32_t)ax[NSL * 256 + (col * WPR + (idx >> 1)) * 4] >> ((idx & 1) * 4)) & 15u;
+                            z16[g] = z | (z << 16);
+                        }
+                        else
+                            z16[g] = zp16;
+                    }
+                }
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                issue(min(it + (st + 2) / STEPS, T - 1), (st + 2) % STEPS, slot);
+                slot ^= 1;
+#pragma unroll
+                for (int g = 0; g < GW; ++g)
+                {
+                    const half2_t sc = as_half2(s2[g]);
+                    const half2_t lo_add = as_half2(z16[g] | 0xE400E400u);        // -(1024 + z)
+                    const half2_t hi_add = as_half2((z16[g] << 4) | 0xD400D400u); // -(64 + z)
+                    const uint32_t ww[4] = {wv[g].x, wv[g].y, wv[g].z, wv[g].w};
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                    {
+                        const uint32_t w = ww[j];
+                        const uint32_t w8 = w >> 8;
+                        uintx4 bq;
+                        bq.x = as_u32((as_half2((w & MASK_LO) | MAGIC) + lo_add) * sc);
+                        bq.y = as_u32((as_half2((w & MASK_HI) | MAGIC_HI) + hi_add) * sc);
+                        bq.z = as_u32((as_half2((w8 & MASK_LO) | MAGIC) + lo_add) * sc);
+                        bq.w = as_u32((as_half2((w8 & MASK_HI) | MAGIC_HI) + hi_add) * sc);
+                        acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, areg[st * GW + g][j]),
+                                                                        __builtin_bit_cast(half8_t, bq), acc[0], 0, 0, 0);
+                    }
+                }
+            }
+            // (one compiler-emitted instruction between the MFMAs and the inline-assembly stores of mrows_reduce_park)
+            acc[0].x *= one;
+            acc[0].y *= one;
+            acc[0].z *= one;
+            acc[0].w *= one;
+            mrows_reduce_park<MB>(acc, red, red_addr, parked_addr, it & 1, it, M, tid);
+        }
+        __builtin_amdgcn_s_waitcnt(mr_vmcnt(0)); // the reloads past the end, before the LDS goes away
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        if (partial)
+        {
+            for (int idx = tid; idx < T * M * 16; idx += 512)
+            {
+                const int n = idx & 15;
+                const int im = idx >> 4;
+                const int it = im / M, m = im - it * M;
+                partial[(size_t)blockIdx.y * M * N + (size_t)m * N + min((t0 + it) * 16, N - 16) + n] = parked[idx];
+            }
+        }
+        else
+            mrows_flush<false, MB>(parked, Y, t0, T, M, N, tid, GemvFusionArgs{nullptr, nullptr, nullptr, nullptr, 0.f}, 0);
+    }
+
     // The same kernel with K as a run-time value: any multiple of 256 up to 8 * GW * STEPS groups (2 <= M <= 16).
     // A wavefront whose GW groups of a step would reach past the end of K fetches the last GW groups of the row
     // instead (the loads of every wavefront and step stay the same in number, which the hand-written wait counts
@@ -1006,6 +1220,75 @@ namespace nnf
         case 1: return launch_mrows_q_gw<1>(stream, A, Wq, S, Y, M, N, group_shift, zp, zero_points, num_cu);
         case 2: return launch_mrows_q_gw<2>(stream, A, Wq, S, Y, M, N, group_shift, zp, zero_points, num_cu);
         default: return launch_mrows_q_gw<4>(stream, A, Wq, S, Y, M, N, group_shift, zp, zero_points, num_cu);
+        }
+    }
+
+    namespace
+    {
+        template <int GW, int GSHIFT, bool ZPT>
+        hipError_t launch_mrows_q_any(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M, int N, int K,
+                                      int zp, const void* zps, float* partial, int ranges, int range_blocks, int num_cu)
+        {
+            const int n_tiles = (N + 15) / 16;
+            const int per_range = num_cu / ranges > 0 ? num_cu / ranges : 1;
+            const int grid = n_tiles < per_range ? n_tiles : per_range;
+            const int tiles_q = n_tiles / grid, tiles_r = n_tiles % grid;
+            const size_t lds = workspace::w4a16_mrows_q_any_lds_bytes(GW, M, tiles_q + (tiles_r ? 1 : 0), GSHIFT, ZPT);
+            if (lds > MAX_LDS_BYTES)
+                return hipErrorInvalidValue;
+            auto kernel = &w4a16_mrows_q_any_kernel<GW, GSHIFT, ZPT>;
+            if (lds > 64 * 1024)
+            {
+                static LdsGrant granted;
+                const hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), granted, (int)MAX_LDS_BYTES);
+                if (e != hipSuccess)
+                    return e;
+            }
+            hipLaunchKernelGGL(kernel, dim3(grid, ranges), dim3(MR_WAVES * 64), lds, stream, (const half_t*)A, (const uint8_t*)Wq,
+                               (const half_t*)S, (half_t*)Y, (const uint8_t*)zps, ranges > 1 ? partial : nullptr, N, K, range_blocks,
+                               tiles_q, tiles_r, M | (zp << 8));
+            return hipGetLastError();
+        }
+        template <int GW>
+        hipError_t launch_mrows_q_any_gw(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M, int N,
+                                         int K, int group_shift, int zp, const void* zps, float* partial, int ranges,
+                                         int range_blocks, int num_cu)
+        {
+            switch (group_shift * 2 + (zps ? 1 : 0))
+            {
+#define NNF_Q_ANY(GS, Z)                                                                                                          \
+    return launch_mrows_q_any<GW, GS, Z>(stream, A, Wq, S, Y, M, N, K, zp, zps, partial, ranges, range_blocks, num_cu)
+            case 10: NNF_Q_ANY(5, false);
+            case 11: NNF_Q_ANY(5, true);
+            case 12: NNF_Q_ANY(6, false);
+            case 13: NNF_Q_ANY(6, true);
+            case 15: NNF_Q_ANY(7, true);
+#undef NNF_Q_ANY
+            default: return hipErrorInvalidValue; // groups of 128 with a scalar zero point: w4a16_mrows_any_kernel
+            }
+        }
+    } // namespace
+
+    // ranges of K of the run-time-K form: 0 does not apply, 1 straight to Y, more: fp32 sums to partial[ranges][M][N] (the
+    // caller runs the reduction pass)
+    int w4a16_mrows_q_any_ranges(int M, int N, int K, int group_shift, bool zero_points, int num_cu)
+    {
+        if (group_shift == 7 && !zero_points)
+            return 0;
+        return workspace::w4a16_mrows_q_any_plan(M, N, K, group_shift, zero_points, num_cu).ranges;
+    }
+
+    hipError_t launch_w4a16_mrows_q_any(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, float* partial,
+                                        int M, int N, int K, int group_shift, int zp, const void* zero_points, int num_cu)
+    {
+        const workspace::MrowsQAny pl = workspace::w4a16_mrows_q_any_plan(M, N, K, group_shift, zero_points != nullptr, num_cu);
+        if (pl.ranges < 1 || (pl.ranges > 1 && !partial) || (group_shift == 7 && !zero_points))
+            return hipErrorInvalidValue;
+        switch (pl.gw)
+        {
+        case 2: return launch_mrows_q_any_gw<2>(stream, A, Wq, S, Y, M, N, K, group_shift, zp, zero_points, partial, pl.ranges, pl.range_blocks, num_cu);
+        case 3: return launch_mrows_q_any_gw<3>(stream, A, Wq, S, Y, M, N, K, group_shift, zp, zero_points, partial, pl.ranges, pl.range_blocks, num_cu);
+        default: return launch_mrows_q_any_gw<4>(stream, A, Wq, S, Y, M, N, K, group_shift, zp, zero_points, partial, pl.ranges, pl.range_blocks, num_cu);
         }
     }
 

@@ -232,6 +232,24 @@ int nnf_wna16_gemm(nnf_stream_t stream, const void* A, const void* Wq, const voi
     const int st = current_device_info(dev);
     if (st != NNF_OK)
         return st;
+    // 4-bit weights, 2 .. 16 rows, a K the fixed-K row-streaming kernel does not take: its run-time-K form, above K = 8192
+    // over ranges of K with the reduction pass (given the workspace for the sums of the ranges)
+    const int gs = group_shift_of(q->group);
+    if (q->bits == 4 && M >= 2 && M <= 16 && !nnf::w4a16_mrows_q_supported(M, N, K, gs, q->zero_points != nullptr, dev.num_cu))
+    {
+        const int ranges = nnf::w4a16_mrows_q_any_ranges(M, N, K, gs, q->zero_points != nullptr, dev.num_cu);
+        if (ranges == 1)
+            return (int)nnf::launch_w4a16_mrows_q_any((hipStream_t)stream, A, Wq, scales, Y, nullptr, M, N, K, gs, q->zero_point,
+                                                      q->zero_points, dev.num_cu);
+        if (ranges > 1 && workspace && aligned16(workspace) && workspace_bytes >= (size_t)ranges * M * N * sizeof(float))
+        {
+            const hipError_t e = nnf::launch_w4a16_mrows_q_any((hipStream_t)stream, A, Wq, scales, nullptr, (float*)workspace, M, N, K,
+                                                               gs, q->zero_point, q->zero_points, dev.num_cu);
+            if (e != hipSuccess)
+                return (int)e;
+            return (int)nnf::launch_wna16_reduce((hipStream_t)stream, (const float*)workspace, ranges, Y, M, N);
+        }
+    }
     // 4-bit weights above 16 rows: the stream-K tile GEMM, given the workspace its plan on this device needs (and
     // zero points it can fetch four bytes at a time)
     if (q->bits == 4 && nnf::w4a16_gemm_q_supported(M, N, K, group_shift_of(q->group)) &&

@@ -519,6 +519,52 @@ namespace nnf
             const int grid = n_tiles < num_cu ? n_tiles : num_cu;
             return w4a16_mrows_q_lds_bytes(K, M, (n_tiles + grid - 1) / grid, group_shift, zero_points) <= LDS_BYTES_PER_CU;
         }
+        // ... and with K as a run-time value (w4a16_mrows_q_any_kernel): 2 .. 16 rows, any other multiple of 256.  Up to
+        // K = 8192 in one piece (two steps of 8 x gw blocks of 128 weights, when at least three quarters of what the
+        // wavefronts fetch counts), above over ranges of at most 32 blocks with fp32 sums per range and the reduction pass
+        // (as w4a16_mrows_split does it for groups of 128 with a scalar zero point).
+        struct MrowsQAny
+        {
+            int ranges = 0, range_blocks = 0, gw = 0; // ranges 0: not applicable; 1: no workspace
+        };
+        inline size_t w4a16_mrows_q_any_lds_bytes(int gw, int M, int tiles, int group_shift, bool zero_points)
+        {
+            const int spc = 1 << (7 - group_shift);
+            const int words = spc == 1 ? gw / 2 + 1 : gw * spc / 2;
+            const int loads = (16 * words + 63) / 64;
+            const size_t aux = (size_t)(zero_points ? 2 : 1) * loads * 256;
+            return (size_t)8 * 2 * gw * 1024 + 8 * 2 * aux + (size_t)2 * 8 * 1024 + (size_t)tiles * M * 64;
+        }
+        inline MrowsQAny w4a16_mrows_q_any_plan(int M, int N, int K, int group_shift, bool zero_points, int num_cu)
+        {
+            MrowsQAny p;
+            if (M < 2 || M > 16 || N < 16 || K < 1024 || K > 65536 || (K & 255) || num_cu < 16 || group_shift < 5 || group_shift > 7)
+                return p;
+            const int B = K >> 7;
+            int ranges = 1, rb = B, gw;
+            if (K <= 8192)
+            {
+                gw = B <= 32 ? 2 : B <= 48 ? 3 : 4;
+                if (4 * B < 3 * 16 * gw)
+                    return p;
+            }
+            else
+            {
+                ranges = (B + 31) / 32;
+                rb = (((B + ranges - 1) / ranges) + 1) & ~1;
+                gw = 2;
+                if (B - (ranges - 1) * rb < gw)
+                    return p;
+            }
+            const int n_tiles = (N + 15) / 16, per_range = num_cu / ranges;
+            const int grid = n_tiles < per_range ? n_tiles : per_range;
+            if (w4a16_mrows_q_any_lds_bytes(gw, M, (n_tiles + grid - 1) / grid, group_shift, zero_points) > LDS_BYTES_PER_CU)
+                return p;
+            p.ranges = ranges;
+            p.range_blocks = rb;
+            p.gw = gw;
+            return p;
+        }
         // The tile GEMM with other block parameters (groups of 32 / 64 / 128, zero points per (row, group)): above 16 rows,
         // K a multiple of 256 (the kernel addresses its operands with 32-bit byte offsets); the plain product, same plan
         inline bool w4a16_gemm_q_fits(int M, int N, int K, int group_shift)
@@ -526,14 +572,19 @@ namespace nnf
             return M > 16 && N >= 1 && K >= 256 && !(K & 255) && group_shift >= 5 && group_shift <= 7 &&
                    (size_t)M * K * 2 + 8192 < ((size_t)1 << 32) && (size_t)N * (K >> 1) < ((size_t)1 << 32);
         }
-        // nnf_wna16_gemm with parameters other than 4 bits / groups of 128 / scalar zero point: [ parked tiles ] for 4-bit
-        // weights on the tile GEMM, nothing otherwise
+        // nnf_wna16_gemm with parameters other than 4 bits / groups of 128 / scalar zero point, 4-bit weights: [ parked tiles ]
+        // on the tile GEMM, [ fp32 sums per range of K ] for 2 .. 16 rows with K above 8192; nothing otherwise
         inline size_t wna16_gemm(int M, int N, int K, int bits, int group, int num_cu = PLAN_CUS)
         {
             const int gs = group == 32 ? 5 : group == 64 ? 6 : group == 128 ? 7 : 0;
-            if (bits != 4 || !w4a16_gemm_q_fits(M, N, K, gs))
+            if (bits != 4 || gs == 0)
                 return 0;
             if (w4a16_mrows_q_fits(M, N, K, gs, true, num_cu)) // up to 32 rows: the row-streaming kernel
+                return 0;
+            const MrowsQAny any = w4a16_mrows_q_any_plan(M, N, K, gs, true, num_cu); // ... over ranges of K: their fp32 sums
+            if (any.ranges > 0)
+                return any.ranges > 1 ? align256((size_t)any.ranges * M * N * sizeof(float)) : 0;
+            if (!w4a16_gemm_q_fits(M, N, K, gs))
                 return 0;
             return plan_w4a16_sk(M, N, K, false, num_cu).bytes();
         }

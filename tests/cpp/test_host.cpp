@@ -1038,6 +1038,24 @@ int main(int argc, char** argv)
             EXPECT(ws::w4a16_mrows_q_lds_bytes(4096, 16, 1, 6, false) == 32768 + 4096 + 16384 + 1024);
             EXPECT(!ws::w4a16_mrows_q_fits(16, 1000000, 8192, 5, true, 256)); // the parked sums do not fit
         }
+        // ... with a run-time K: one piece up to 8192 where most of what is fetched counts, ranges of at most 32 blocks above
+        {
+            auto p = ws::w4a16_mrows_q_any_plan(16, 4096, 11008, 7, true, 256);
+            EXPECT(p.ranges == 3 && p.range_blocks == 30 && p.gw == 2);
+            EXPECT(ws::wna16_gemm(16, 4096, 11008, 4, 128) == (size_t)3 * 16 * 4096 * 4);
+            p = ws::w4a16_mrows_q_any_plan(8, 4096, 5120, 5, false, 256);
+            EXPECT(p.ranges == 1 && p.gw == 3 && p.range_blocks == 40);
+            EXPECT(ws::wna16_gemm(8, 4096, 5120, 4, 32) == 0);
+            EXPECT(ws::w4a16_mrows_q_any_plan(8, 4096, 7168, 6, true, 256).gw == 4);
+            EXPECT(ws::w4a16_mrows_q_any_plan(8, 4096, 2304, 6, true, 256).ranges == 0); // 18 of 32 fetched blocks count
+            EXPECT(ws::w4a16_mrows_q_any_plan(17, 4096, 11008, 6, true, 256).ranges == 0);
+            EXPECT(ws::w4a16_mrows_q_any_plan(8, 4096, 11008 + 128, 6, true, 256).ranges == 0);
+            p = ws::w4a16_mrows_q_any_plan(4, 8192, 28672, 7, true, 256);
+            EXPECT(p.ranges == 7 && p.range_blocks == 32 && p.gw == 2);
+            // scales of a step: groups of 128: gw / 2 + 1 words a row; 32: gw * 2 words (two loads from gw = 3 on)
+            EXPECT(ws::w4a16_mrows_q_any_lds_bytes(2, 16, 1, 7, true) == 32768 + 8 * 2 * 512 + 16384 + 1024);
+            EXPECT(ws::w4a16_mrows_q_any_lds_bytes(4, 16, 1, 5, false) == 65536 + 8 * 2 * 512 + 16384 + 1024);
+        }
         // M <= 16: one workgroup holds the activations, or K is cut into ranges
         {
             for (int m = 1; m <= 16; ++m)

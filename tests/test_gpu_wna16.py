@@ -52,6 +52,10 @@ SHAPES = [
     # step and wavefront; fewer tiles than CUs, a ragged last tile, several tiles per workgroup)
     (2, 4096, 4096), (5, 300, 2048), (8, 1000, 8192), (16, 48, 8192), (13, 12288, 4096), (16, 9000, 2048),
     (17, 4096, 4096), (32, 1000, 2048), (25, 12288, 4096), (31, 40, 4096),
+    # ... with any other K that is a multiple of 256: one piece up to 8192 (two, three, four blocks of 128 per wavefront and
+    # step; wavefronts past the end of K), ranges of K above (11008: three; 14336: four; 28672: seven)
+    (4, 4096, 3584), (16, 1000, 5120), (9, 300, 7168), (2, 4096, 11008), (16, 4096, 11008), (8, 520, 14336), (5, 64, 28672),
+    (16, 33, 2560),
     # the tile kernel: one partial tile, ragged M and N, many tiles, a long K
     (17, 33, 128), (64, 64, 512), (100, 1000, 160), (300, 257, 2048), (128, 4096, 4096), (33, 520, 11008), (1024, 130, 384),
     # 4-bit weights above 16 rows with K a multiple of 256: the stream-K tile GEMM (tiles of 32 x 256, 64 x 128, 128 x 128,
@@ -99,7 +103,7 @@ def test_one_hot_rows_return_the_dequantised_weights(gpu, m, n, k, bits, group, 
 
 
 @pytest.mark.parametrize("m,k", [(1, 1024), (1, 4096), (1, 11008), (1, 16384), (7, 2048), (16, 4096), (3, 8192), (32, 4096),
-                                 (20, 2048)])
+                                 (20, 2048), (16, 11008), (6, 5120), (11, 7168), (16, 3584)])
 @pytest.mark.parametrize("group,zp_tensor", [(32, True), (64, True), (128, True), (32, False), (64, False)])
 def test_one_hot_rows_through_the_row_streaming_kernels(gpu, m, k, group, zp_tensor):
     """4-bit weights with one row and K a multiple of 256, or a few rows and K = 2048 / 4096 / 8192, run on the
