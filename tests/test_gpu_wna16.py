@@ -125,6 +125,30 @@ def test_one_hot_rows_through_the_row_streaming_kernels(gpu, m, k, group, zp_ten
         assert not y[len(chunk):].any()
 
 
+def _random_shapes(count):
+    rng = np.random.default_rng(20240607)
+    ks = [128, 256, 384, 512, 768, 1024, 1280, 2048, 2560, 3584, 4096, 5120, 7168, 8192, 11008, 14336]
+    out = []
+    for i in range(count):
+        m = int(rng.choice([1, 1, 2, 3, 7, 8, 15, 16, 17, 24, 32, 33, 63, 64, 100, 129, 257, 300]))
+        n = int(rng.choice([16, 17, 31, 33, 64, 100, 255, 256, 257, 500, 1000, 1024, 2000, 4096]))
+        k = int(rng.choice(ks))
+        if m * n * k > 300 * 2000 * 4096:
+            n = 256
+        out.append((m, n, k, int(rng.choice([4, 4, 4, 8])), int(rng.choice([32, 64, 128])), bool(rng.integers(0, 2)), int(rng.integers(0, 16))))
+    return out
+
+
+@pytest.mark.parametrize("m,n,k,bits,group,zp_tensor,zp", _random_shapes(120))
+def test_wna16_random_shapes(gpu, m, n, k, bits, group, zp_tensor, zp):
+    """Shapes drawn across the routes of nnf_wna16_gemm (row-streaming kernels with a fixed and a run-time K, ranges of K,
+    stream-K tiles, plain kernels), every block parameter and zero point."""
+    a, wq, s, zps = _case(m + 3 * n + 7 * k + bits + group, m, n, k, bits, group, zp_tensor)
+    zp = zp if bits == 4 else 16 * zp + 3
+    ref = oracle.wna16_gemm(a, wq, s, bits, group, zp=zp, zero_points=zps, f32_out=True)
+    _check(_run(gpu, a, wq, s, bits, group, zp, zps), ref)
+
+
 def test_tile_gemm_without_its_workspace_runs_on_the_plain_kernel(gpu):
     """Above 16 rows 4-bit weights want the stream-K tile GEMM's workspace; a caller that brings none (or too little)
     gets the same product from the plain tile kernel."""
