@@ -91,6 +91,35 @@ def test_gemm_matches_oracle(gpu, m, n, k):
     _check(y.cpu().numpy(), ref)
 
 
+def _random_shapes(count):
+    rng = np.random.default_rng(777)
+    out = []
+    for _ in range(count):
+        m = int(rng.choice([1, 2, 3, 8, 15, 16, 17, 31, 32, 33, 40, 41, 64, 65, 127, 128, 129, 200, 256, 300, 513]))
+        n = int(rng.choice([1, 15, 16, 17, 64, 100, 255, 256, 257, 500, 1000, 1024, 2000, 4096, 5000]))
+        k = int(rng.choice([128, 256, 384, 512, 640, 1024, 1152, 2048, 2560, 3072, 4096, 5120, 6144, 7168, 8192, 11008, 14336]))
+        if m * n * k > 300 * 2000 * 4096:
+            n = 256
+        out.append((m, n, k, int(rng.integers(0, 16))))
+    return out
+
+
+@pytest.mark.parametrize("m,n,k,zp", _random_shapes(150))
+def test_gemm_random_shapes(gpu, m, n, k, zp):
+    """Shapes drawn across the routes of nnf_w4a16_gemm (the row-streaming kernels with a fixed and a run-time K, ranges of
+    K, the MFMA GEMV, stream-K tiles of every height), every zero point."""
+    import torch
+
+    from nnfusion_amd import ops
+
+    a, wq, s = datagen.w4a16_case(m + 5 * n + 11 * k + zp, m, n, k)
+    ta, tw, ts = _t(gpu, a, wq, s)
+    y = ops.w4a16_gemm(ta, tw, ts, zp=zp)
+    torch.cuda.synchronize()
+    ref = oracle.w4a16_gemm(a, wq, s, zp=zp, f32_out=True)
+    _check(y.cpu().numpy(), ref)
+
+
 @pytest.mark.parametrize("m", [1, 5, 16])
 def test_gemm_kernel_serves_small_m(gpu, m):
     """The tile GEMM asked for by variant (the library's own choice for these shapes is a GEMV kernel)."""
