@@ -41,6 +41,11 @@
 #include <stddef.h>
 #include <stdint.h>
 
+/* The library is built with hidden visibility; these declarations are its whole exported surface. */
+#ifndef NNF_API
+#define NNF_API __attribute__((visibility("default")))
+#endif
+
 #ifdef __cplusplus
 extern "C" {
 #endif
@@ -59,10 +64,10 @@ enum nnf_status
 };
 
 /* ABI version of this header (bumped on any signature change). */
-int nnf_abi_version(void);
+NNF_API int nnf_abi_version(void);
 
 /* Human-readable text for a status returned by any function below (static storage). */
-const char* nnf_status_string(int status);
+NNF_API const char* nnf_status_string(int status);
 
 /* ---------------------------------------------------------------------------------------------
  * fp16 x int4 (group-scaled) GEMM / GEMV:  Y[M,N] = A[M,K] . ((Wq - zp) * scales)^T
@@ -73,24 +78,25 @@ const char* nnf_status_string(int status);
  * shapes the MFMA GEMV kernel over K ranges; everything else the MFMA tile GEMM, whose work is split evenly
  * over the CUs (tiles shared by several workgroups are summed through `workspace` by a second launch).
  * ------------------------------------------------------------------------------------------- */
-size_t nnf_w4a16_gemm_workspace_bytes(int M, int N, int K, int group);
+NNF_API size_t nnf_w4a16_gemm_workspace_bytes(int M, int N, int K, int group);
 
-int nnf_w4a16_gemm(nnf_stream_t stream,
+NNF_API int nnf_w4a16_gemm(nnf_stream_t stream,
                    const void* A, const void* Wq, const void* scales, void* Y,
                    int M, int N, int K, int group, int zp,
                    void* workspace, size_t workspace_bytes);
 
 /* nnf_w4a16_gemm for callers that can neither allocate nor pass a workspace (code under HIP graph capture,
  * tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same kernels and
- * results as nnf_w4a16_gemm; the partial sums of a GEMM whose K range is split go to a buffer of
+ * results as nnf_w4a16_gemm (the tile GEMM in its one-launch form, see nnf_plan::sync_flags, with synchronisation
+ * words of the library's own); the partial sums of a GEMM whose K range is split go to a buffer of
  * NNF_STATIC_SCRATCH_BYTES that the library holds in device memory (a static __device__ array: each GPU the
  * library is used on keeps its own copy until the process ends).  Calls no hipMalloc / hipFree.  A shape whose
  * nnf_w4a16_gemm_workspace_bytes exceeds the buffer is rejected with NNF_ERR_STATIC_SCRATCH_LIMIT.  All calls
  * on one GPU share the buffer: calls that overlap on one GPU (different streams) race; calls on one stream
- * are ordered and safe.  The first call of any entry point on a device looks the buffer's address up
+ * are ordered and safe.  The first call of this entry point on a device looks the buffer's address up
  * (hipGetSymbolAddress): make that call outside stream capture. */
 #define NNF_STATIC_SCRATCH_BYTES ((size_t)32 << 20)
-int nnf_w4a16_gemm_static_scratch(nnf_stream_t stream,
+NNF_API int nnf_w4a16_gemm_static_scratch(nnf_stream_t stream,
                                   const void* A, const void* Wq, const void* scales, void* Y,
                                   int M, int N, int K, int group, int zp);
 
@@ -113,24 +119,50 @@ enum nnf_w4a16_variant
 /* What else a candidate may fix about the tile GEMM (variant NNF_*_GEMM_MFMA; ignored by the other variants).
  * Passed per call: the library keeps no dispatch state, calls with different plans may run concurrently.
  * NULL, or a field that is 0: the library's own choice for the shape. */
+#define NNF_MAX_K_PARTS 64
+/* Synchronisation words for the one-launch form of the fp16 x int4 tile GEMM: two 32-bit words per output tile; a
+ * buffer of NNF_SYNC_FLAGS_BYTES serves every shape up to 8192 tiles (a launch with more tiles than the buffer
+ * given takes the two-launch form). */
+#define NNF_SYNC_FLAGS_BYTES ((size_t)64 << 10)
 typedef struct nnf_plan
 {
     int tile_rows; /* rows of an output tile: 256, 128, 64 (fp16 x int4 also 32); see tile_cols for their width
                       (W8A8 128-row tiles: 128 columns, 64-row tiles: 256) */
     int k_parts;   /* fp16 x int4: workgroups that share one output tile, each a contiguous part of K, summed by a
                       second launch (the grid is tiles x k_parts, work split evenly); W8A8: ranges of K, int32
-                      partial sums added exactly by a reduction pass */
+                      partial sums added exactly by a reduction pass.  At most NNF_MAX_K_PARTS (and never more
+                      workgroups than the product has units of 256 k). */
     int tile_cols; /* columns of an output tile, 256 or 128 (0: the library's choice): W8A8 with 256-row tiles;
                       fp16 x int4 with 64-, 128- or 256-row tiles and no SiLU-gate (the gate | up halves need the
                       256 weight rows of a full tile); ignored elsewhere */
+    /* fp16 x int4 tile GEMM in one launch (any variant that ends up on it; ignored by every other kernel and by W8A8).
+     * The work of the GEMM is split evenly over the CUs, so most output tiles of a mid-sized product are shared by
+     * several workgroups.  Without sync_flags their parts are added up by a second launch.  With sync_flags the
+     * workgroups count themselves in at their tiles there, and each adds up and finishes its share of a tile's rows
+     * once all that hold a part have arrived -- same summation order, bit-identical results, one launch less.
+     *   sync_flags: device memory, 16-byte aligned, ALL ZERO before the first call that uses it; every call leaves it
+     *     all zero again, so it needs clearing once (when it is allocated), not per call.  It must not be scratch
+     *     memory that other kernels write between calls, and calls that may overlap on the device (different
+     *     streams) need buffers of their own.  The reference's counterpart is the persistent, zero-initialised
+     *     `be_state_buffer` tensor of its BlockFusion kernels
+     *     (src/nnfusion/engine/pass/graph/blockfusion/blockfusion_codegen.cpp:295-304): an emitter reserves it
+     *     with KernelEmitter::allocate_tensor + set_memset(true, 0) + set_persistent(true).
+     *   sync_flags_bytes: its size; NNF_SYNC_FLAGS_BYTES always suffices.
+     *   spin_limit: how many times (about a microsecond each) a workgroup polls for the other arrivals before it hands
+     *     its share of the rows to the last workgroup to arrive, which never waits (so a launch whose workgroups are
+     *     not all resident at once still ends).  0: the library's default (some ten milliseconds); negative: do not
+     *     wait at all (every tile is then finished by its last arriver; for tests of that path). */
+    void* sync_flags;
+    size_t sync_flags_bytes;
+    int spin_limit;
 } nnf_plan;
 /* 1 when the variant can serve the shape (decided on the host, for a 256-CU device), else 0. */
-int nnf_w4a16_variant_supported(int M, int N, int K, int group, int variant);
+NNF_API int nnf_w4a16_variant_supported(int M, int N, int K, int group, int variant);
 /* Upper bound for a 256-CU device; the call itself checks what its launch writes on the device at hand. */
-size_t nnf_w4a16_gemm_variant_workspace_bytes(int M, int N, int K, int group, int variant, const nnf_plan* plan);
+NNF_API size_t nnf_w4a16_gemm_variant_workspace_bytes(int M, int N, int K, int group, int variant, const nnf_plan* plan);
 /* As nnf_w4a16_gemm through the given variant; NNF_ERR_UNSUPPORTED_SHAPE when it cannot serve the shape,
  * NNF_ERR_INVALID_ARGUMENT for a variant or plan value outside the ones listed. */
-int nnf_w4a16_gemm_variant(nnf_stream_t stream,
+NNF_API int nnf_w4a16_gemm_variant(nnf_stream_t stream,
                            const void* A, const void* Wq, const void* scales, void* Y,
                            int M, int N, int K, int group, int zp, int variant, const nnf_plan* plan,
                            void* workspace, size_t workspace_bytes);
@@ -162,9 +194,9 @@ typedef struct nnf_quant
     const void* zero_points; /* device pointer or NULL */
 } nnf_quant;
 /* 1 when nnf_wna16_gemm serves the shape with these parameters (zero_points is not read), else 0. */
-int nnf_wna16_supported(int M, int N, int K, const nnf_quant* q);
-size_t nnf_wna16_gemm_workspace_bytes(int M, int N, int K, const nnf_quant* q);
-int nnf_wna16_gemm(nnf_stream_t stream,
+NNF_API int nnf_wna16_supported(int M, int N, int K, const nnf_quant* q);
+NNF_API size_t nnf_wna16_gemm_workspace_bytes(int M, int N, int K, const nnf_quant* q);
+NNF_API int nnf_wna16_gemm(nnf_stream_t stream,
                    const void* A, const void* Wq, const void* scales, void* Y,
                    int M, int N, int K, const nnf_quant* q,
                    void* workspace, size_t workspace_bytes);
@@ -195,9 +227,9 @@ enum nnf_activation
  *                       may alias Y
  *   act               : nnf_activation
  */
-size_t nnf_w4a16_gemm_fused_workspace_bytes(int M, int N, int K, int group, int act);
+NNF_API size_t nnf_w4a16_gemm_fused_workspace_bytes(int M, int N, int K, int group, int act);
 
-int nnf_w4a16_gemm_fused(nnf_stream_t stream,
+NNF_API int nnf_w4a16_gemm_fused(nnf_stream_t stream,
                          const void* A, const void* Wq, const void* scales, void* Y,
                          int M, int N, int K, int group, int zp,
                          const void* rms_gamma, float rms_eps,
@@ -208,7 +240,7 @@ int nnf_w4a16_gemm_fused(nnf_stream_t stream,
  * NNF_ERR_UNSUPPORTED_SHAPE, as for a variant that cannot serve the shape); `plan` for the tile GEMM.
  * A workspace of nnf_w4a16_gemm_fused_workspace_bytes + nnf_w4a16_gemm_variant_workspace_bytes(.., plan) of the
  * weight rows (2N with NNF_ACT_SILU_GATE) always suffices. */
-int nnf_w4a16_gemm_fused_variant(nnf_stream_t stream,
+NNF_API int nnf_w4a16_gemm_fused_variant(nnf_stream_t stream,
                                  const void* A, const void* Wq, const void* scales, void* Y,
                                  int M, int N, int K, int group, int zp,
                                  const void* rms_gamma, float rms_eps,
@@ -221,16 +253,16 @@ int nnf_w4a16_gemm_fused_variant(nnf_stream_t stream,
  * The reference has no emitter for this; the nearest routine in its tree is MLAS's u8 x s8
  * MlasGemm (thirdparty/mlas/inc/mlas.h:147-163).
  * ------------------------------------------------------------------------------------------- */
-size_t nnf_w8a8_gemm_workspace_bytes(int M, int N, int K);
+NNF_API size_t nnf_w8a8_gemm_workspace_bytes(int M, int N, int K);
 
 /* Y fp16 [M,N] = fp16((float)acc * s_tok[m] * s_ch[n]) */
-int nnf_w8a8_gemm(nnf_stream_t stream,
+NNF_API int nnf_w8a8_gemm(nnf_stream_t stream,
                   const void* A, const void* s_tok, const void* W, const void* s_ch, void* Y,
                   int M, int N, int K,
                   void* workspace, size_t workspace_bytes);
 
 /* Raw accumulators: acc i32 [M,N] = A . W^T (exact). */
-int nnf_w8a8_gemm_acc(nnf_stream_t stream,
+NNF_API int nnf_w8a8_gemm_acc(nnf_stream_t stream,
                       const void* A, const void* W, void* acc,
                       int M, int N, int K,
                       void* workspace, size_t workspace_bytes);
@@ -243,10 +275,10 @@ enum nnf_w8a8_variant
     NNF_W8A8_GEMM_MFMA = 2, /* any M: int8 MFMA 32x32x32 tile GEMM (may split K: workspace) */
     NNF_W8A8_GEMV_ROWS = 3  /* row-streaming kernels: M = 1; M = 2 .. 32 on MFMA (K a multiple of 256, 1024 .. 16384) */
 };
-int nnf_w8a8_variant_supported(int M, int N, int K, int variant);
-size_t nnf_w8a8_gemm_variant_workspace_bytes(int M, int N, int K, int variant, const nnf_plan* plan);
+NNF_API int nnf_w8a8_variant_supported(int M, int N, int K, int variant);
+NNF_API size_t nnf_w8a8_gemm_variant_workspace_bytes(int M, int N, int K, int variant, const nnf_plan* plan);
 /* Exactly one of Y (with s_tok, s_ch) and acc is non-NULL: the fp16 result or the raw int32 accumulators. */
-int nnf_w8a8_gemm_variant(nnf_stream_t stream,
+NNF_API int nnf_w8a8_gemm_variant(nnf_stream_t stream,
                           const void* A, const void* s_tok, const void* W, const void* s_ch, void* Y, void* acc,
                           int M, int N, int K, int variant, const nnf_plan* plan,
                           void* workspace, size_t workspace_bytes);
@@ -266,14 +298,28 @@ int nnf_w8a8_gemm_variant(nnf_stream_t stream,
  * The element-wise semantics follow the reference's ops (Sigmoid, Multiply, Add, Rsqrt:
  * cuda_gpu/cuda_kernelops.hpp:206-210,408,416,447-451); the reference has no RMSNorm op.
  * ------------------------------------------------------------------------------------------- */
-size_t nnf_fused_mlp_w4a16_workspace_bytes(int M, int H, int I, int group);
+NNF_API size_t nnf_fused_mlp_w4a16_workspace_bytes(int M, int H, int I, int group);
 
-int nnf_fused_mlp_w4a16(nnf_stream_t stream,
+NNF_API int nnf_fused_mlp_w4a16(nnf_stream_t stream,
                         const void* x, const void* gamma, float eps,
                         const void* Wgu, const void* Sgu, const void* Wd, const void* Sd,
                         void* out,
                         int M, int H, int I, int group, int zp,
                         void* workspace, size_t workspace_bytes);
+
+/* The same block with an nnf_plan for each of its two products (NULL: the library's own choice): the tile shapes a
+ * profiling selector wants to try, and the sync_flags that make each tile GEMM a single launch (both plans may name
+ * the same buffer: the two products run one after the other on `stream`).  A plan that fixes a tile shape or k_parts
+ * puts that product on the tile GEMM.  Workspace: nnf_fused_mlp_w4a16_workspace_bytes for NULL plans or plans that
+ * only carry sync_flags; with a fixed tile shape add nnf_w4a16_gemm_variant_workspace_bytes of that product
+ * (gate | up: M x 2I x H; down: M x H x I). */
+NNF_API int nnf_fused_mlp_w4a16_planned(nnf_stream_t stream,
+                                const void* x, const void* gamma, float eps,
+                                const void* Wgu, const void* Sgu, const void* Wd, const void* Sd,
+                                void* out,
+                                int M, int H, int I, int group, int zp,
+                                const nnf_plan* gate_up_plan, const nnf_plan* down_plan,
+                                void* workspace, size_t workspace_bytes);
 
 #ifdef __cplusplus
 }

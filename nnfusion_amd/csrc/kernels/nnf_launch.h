@@ -56,7 +56,15 @@ namespace nnf
         int tile_rows = 0; // tile GEMM: rows of an output tile (256, 128, 64; fp16 x int4 also 32)
         int k_parts = 0;   // tile GEMM: workgroups that share an output tile (fp16 x int4) / ranges of K (W8A8)
         int tile_cols = 0; // W8A8 tile GEMM with 256-row tiles: 256 or 128 columns
+        // fp16 x int4 tile GEMM in one launch: zeroed words the workgroups that share a tile synchronise through (left
+        // zero again), their size, and how many polls a workgroup waits for the others (0: DEFAULT_SPIN_LIMIT)
+        void* sync_flags = nullptr;
+        size_t sync_bytes = 0;
+        int spin_limit = 0;
     };
+    // a poll is an atomic load from device memory and a short sleep, about a microsecond: a workgroup that has waited some
+    // ten milliseconds hands its share to the last arriver
+    constexpr int DEFAULT_SPIN_LIMIT = 1 << 13;
 
     hipError_t launch_w4a16_gemv(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y,
                                  int M, int N, int K, int zp, int num_cu);
@@ -117,7 +125,8 @@ namespace nnf
     // (row, group): M > 16, K a multiple of 256; partial_ws: workspace::wna16_gemm bytes (0: not needed)
     bool w4a16_gemm_q_supported(int M, int N, int K, int group_shift);
     hipError_t launch_w4a16_gemm_q(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M, int N,
-                                   int K, int group_shift, int zp, const void* zero_points, void* partial_ws, int num_cu);
+                                   int K, int group_shift, int zp, const void* zero_points, void* partial_ws, int num_cu,
+                                   const LaunchChoice& choice = LaunchChoice());
     hipError_t launch_w4a16_gemm(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M,
                                  int N, int K, int zp, const void* rms_gamma, float rms_eps, const void* bias,
                                  const void* residual, int act, void* rms_ws, void* partial_ws, int num_cu,

@@ -263,6 +263,19 @@ namespace nnf
         }
     } // namespace
 
+    namespace
+    {
+        // one launch where the caller gave enough zeroed synchronisation words for the plan's tiles, else two
+        void set_sync(SkGemmParams& p, const workspace::SkPlan& plan, const LaunchChoice& choice)
+        {
+            p.partial_bytes = plan.bytes();
+            // (the one-launch form addresses the parked tiles with 32-bit byte offsets)
+            const bool one_launch = plan.slots && choice.sync_flags && choice.sync_bytes >= plan.sync_bytes() && plan.bytes() < ((size_t)1 << 32);
+            p.sync = one_launch ? (uint32_t*)choice.sync_flags : nullptr;
+            p.spin_limit = choice.spin_limit > 0 ? choice.spin_limit : choice.spin_limit < 0 ? 0 : DEFAULT_SPIN_LIMIT;
+        }
+    } // namespace
+
     hipError_t launch_w4a16_gemm(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M,
                                  int N, int K, int zp, const void* rms_gamma, float rms_eps, const void* bias,
                                  const void* residual, int act, void* rms_ws, void* partial_ws, int num_cu,
@@ -378,6 +391,7 @@ namespace nnf
         p.supersteps = plan.supersteps;
         p.units = plan.units;
         p.zps = nullptr;
+        set_sync(p, plan, choice);
         if (plan.tile_weight_rows == 128)
             return plan.tile_rows == 256 ? launch_gemm_sk_256_narrow(stream, p, plan.grid)
                    : plan.tile_rows == 128 ? launch_gemm_sk_128_narrow(stream, p, plan.grid)
@@ -410,7 +424,8 @@ namespace nnf
     // ---- the tile GEMM with other block parameters ----------------------------------------------------------------------
     bool w4a16_gemm_q_supported(int M, int N, int K, int group_shift) { return workspace::w4a16_gemm_q_fits(M, N, K, group_shift); }
     hipError_t launch_w4a16_gemm_q(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M, int N,
-                                   int K, int group_shift, int zp, const void* zero_points, void* partial_ws, int num_cu)
+                                   int K, int group_shift, int zp, const void* zero_points, void* partial_ws, int num_cu,
+                                   const LaunchChoice& choice)
     {
         if (!w4a16_gemm_q_supported(M, N, K, group_shift))
             return hipErrorInvalidValue;
@@ -438,6 +453,7 @@ namespace nnf
         p.supersteps = plan.supersteps;
         p.units = plan.units;
         p.zps = (const uint8_t*)zero_points;
+        set_sync(p, plan, choice);
         switch (group_shift)
         {
         case 5: return launch_gemm_sk_q5(stream, p, plan.grid, plan.tile_rows, plan.tile_weight_rows);

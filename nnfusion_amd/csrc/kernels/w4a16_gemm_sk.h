@@ -41,6 +41,9 @@
 //     register order (1 KiB per store instruction); a second, small launch adds the parts of such tiles
 //     in K order and runs their epilogue, on all CUs (one CU would need tens of microseconds to pull the
 //     parts of a tile through its own registers).  Tiles with a single owner are finished here.
+//     Given two zeroed words per tile (SkGemmParams::sync) the second launch is not needed: the workgroups that
+//     share a tile count their arrivals there and each adds up and finishes its share of the tile's 32-row blocks
+//     once all have arrived, in the same K order (same bits as the second launch gives).
 //   * Epilogues round the way the unfused graph would: the GEMM result to fp16 first, then the
 //     element-wise operation in fp32, then fp16 again.  RMSNorm is folded in without materialising the
 //     normalised activations: gamma[k] multiplies the weights as they are unpacked, rstd[m] (from a
@@ -66,10 +69,16 @@ namespace nnf
         const half_t* gamma;    // RMS: [K]
         const float* rstd;      // RMS: [M]
         float* partial;         // slots of BM x BN fp32: workgroup v's first segment at slot v, a later one at grid + v
+        size_t partial_bytes;   // all slots
         int tiles_m, tiles_n;
         int supersteps;         // per tile: ceil(K / 256)
         long long units;        // tiles_m * tiles_n * supersteps
         const uint8_t* zps;     // QG != 0: zero points, u8 [N, K / group / 2] (even group in the low nibble), or null: zp
+        // One launch instead of two: two words per tile, all zero when the launch starts and zero again when it ends.
+        // Non-null: the workgroups that share a tile add its parts up themselves (sk_reduce_shared_tile below) and no
+        // second launch follows.
+        uint32_t* sync;
+        int spin_limit;         // polls of a tile's arrival count before a workgroup leaves its share to the last arriver
     };
 
     namespace gemm_sk
@@ -203,6 +212,34 @@ namespace nnf
 
         // regions per quarter and fragments per region
         constexpr int regions_of(int TM) { return TM < 4 ? TM : 4; }
+
+        // Parked sums that other workgroups of the SAME launch read (SkGemmParams::sync): stores and loads at device
+        // scope (the sc1 bit), i.e. written through to, and read from, the level of the memory system that all eight
+        // L2s of the chip agree on.  A release / acquire fence pair would do the same for ordinary accesses, but on
+        // this chip such a fence writes back / invalidates a whole L2 under the 32 CUs that share it: with fences
+        // the one-launch form measured twice as slow as the two-launch form.  Buffer instructions, because their
+        // intrinsics take the cache policy as an argument and the compiler tracks them like any other load (a load
+        // written as inline assembly would land in registers the compiler may have given away again).
+        typedef __amdgpu_buffer_rsrc_t buffer_t;
+        constexpr int DEVICE_SCOPE = 16; // sc1
+        __device__ __forceinline__ buffer_t parked_buffer(float* base, size_t bytes)
+        {
+            // raw buffer over [base, base + bytes): accesses beyond it read zero / are dropped
+            return __builtin_amdgcn_make_buffer_rsrc(base, 0, (int)(bytes > 0xFFFFFFFFull ? 0xFFFFFFFFull : bytes), 0x00020000);
+        }
+        __device__ __forceinline__ void store_device_scope(buffer_t buf, uint32_t byte_offset, const floatx4& v)
+        {
+            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uintx4, v), buf, (int)byte_offset, 0, DEVICE_SCOPE);
+        }
+        __device__ __forceinline__ floatx4 load_device_scope(buffer_t buf, uint32_t byte_offset)
+        {
+            return __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(buf, (int)byte_offset, 0, DEVICE_SCOPE));
+        }
+        // every vector-memory operation of this wavefront is complete (stores: acknowledged at their scope)
+        __device__ __forceinline__ void wait_vector_memory()
+        {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        }
     } // namespace gemm_sk
 
     // Epilogue of one round (ROUND_TM blocks of 32 rows) of a wavefront's strip of a tile.  Lane (m = l32, h) holds, in
@@ -307,6 +344,110 @@ namespace nnf
         }
     }
 
+    // Block `r` (32 rows) of strip `wave` of a tile that `n_seg` workgroups (v_first, v_first + 1, ...) of a launch of
+    // `gemm_grid` worked on: adds their parked parts in K order, eight in flight, and finishes the block (epilogue,
+    // stores).  Used by the second launch and, with SkGemmParams::sync, by the GEMM's own workgroups: same order, same bits.
+    // SAME_LAUNCH: the parts were parked by other workgroups of the launch that is still running (device-scope loads).
+    template <int TM, int TN, bool GATE, bool BIAS, bool RESID, bool RMS, bool SAME_LAUNCH>
+    __device__ __forceinline__ void sk_sum_block(const SkGemmParams& p, int gemm_grid, int tile, int r, int v_first, int n_seg,
+                                                 bool first_is_second_slot, uint8_t* stage, int wave, int lane)
+    {
+        using namespace gemm_sk;
+        using T = Tile<TM, TN>;
+        constexpr int BN_OUT = GATE ? T::BN / 2 : T::BN;
+        const int tid = wave * 64 + lane;
+        int tm, tn;
+        {
+            constexpr int GM = 4;
+            const int per_group = GM * p.tiles_n;
+            const int g = tile / per_group;
+            const int first_m = g * GM;
+            const int gm = min(GM, p.tiles_m - first_m);
+            const int rr = tile - g * per_group;
+            tm = first_m + rr % gm;
+            tn = rr / gm;
+        }
+        const int m0 = tm * T::BM, n0 = tn * BN_OUT;
+        floatx16 c[1][TN];
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e)
+                c[0][j][e] = 0.f;
+        // SAME_LAUNCH: inside the GEMM kernel, with its accumulation registers still set aside: four parts in flight
+        constexpr int D = SAME_LAUNCH ? 4 : 8;
+        buffer_t parked;
+        if constexpr (SAME_LAUNCH)
+            parked = parked_buffer(p.partial, p.partial_bytes);
+        for (int sg0 = 0; sg0 < n_seg; sg0 += D)
+        {
+            floatx4 x[D][TN][4];
+#pragma unroll
+            for (int d = 0; d < D; ++d)
+            {
+                const int sg = min(sg0 + d, n_seg - 1);
+                const size_t first_float =
+                    ((size_t)(v_first + sg) + ((sg == 0 && first_is_second_slot) ? (size_t)gemm_grid : 0)) * T::SLOT_FLOATS + (size_t)tid * 4;
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int q = 0; q < 4; ++q)
+                    {
+                        const size_t at = first_float + (size_t)(((r * TN + j) * 4 + q) * THREADS * 4);
+                        if constexpr (SAME_LAUNCH)
+                            x[d][j][q] = load_device_scope(parked, (uint32_t)(at * sizeof(float)));
+                        else
+                            x[d][j][q] = *reinterpret_cast<const floatx4*>(p.partial + at);
+                    }
+            }
+#pragma unroll
+            for (int d = 0; d < D; ++d)
+                if (sg0 + d < n_seg)
+                {
+#pragma unroll
+                    for (int j = 0; j < TN; ++j)
+#pragma unroll
+                        for (int q = 0; q < 4; ++q)
+                        {
+                            c[0][j][4 * q] += x[d][j][q].x;
+                            c[0][j][4 * q + 1] += x[d][j][q].y;
+                            c[0][j][4 * q + 2] += x[d][j][q].z;
+                            c[0][j][4 * q + 3] += x[d][j][q].w;
+                        }
+                }
+        }
+        sk_finish_round<1, TN, GATE, BIAS, RESID, RMS>(p, c, r, m0, n0, stage, wave, lane);
+    }
+
+    // SkGemmParams::sync, word 0 of a tile: bits 0 .. 15 count the workgroups that have parked their part of it, bits
+    // 16 .. 23 mark the 32-row blocks whose owner stopped waiting (the last arriver takes them over); word 1 counts the
+    // blocks that are finished: whoever finishes the last one sets both words to zero again.
+    // Thread 0 of a workgroup that has arrived (`old`: the word as its own arrival found it) and owns the blocks
+    // `own_mask`: the blocks to add up and finish now.  Waits at most `spin_limit` polls for the other arrivals.
+    __device__ __forceinline__ uint32_t sk_blocks_to_finish(uint32_t* state, uint32_t old, int n_seg, uint32_t own_mask, int spin_limit)
+    {
+        if ((old & 0xFFFFu) == (uint32_t)(n_seg - 1))
+            return own_mask | ((old >> 16) & 0xFFu);
+        if (own_mask == 0)
+            return 0;
+        for (int polls = 0;; ++polls)
+        {
+            const uint32_t s = __hip_atomic_load(state, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if ((s & 0xFFFFu) == (uint32_t)n_seg)
+                return own_mask;
+            if (polls >= spin_limit)
+            {
+                // hand the blocks over -- unless an arrival gets in first (the exchange fails: look again)
+                uint32_t expected = s;
+                if (__hip_atomic_compare_exchange_strong(state, &expected, s | (own_mask << 16), __ATOMIC_RELAXED, __ATOMIC_RELAXED,
+                                                         __HIP_MEMORY_SCOPE_AGENT))
+                    return 0;
+                continue;
+            }
+            __builtin_amdgcn_s_sleep(2);
+        }
+    }
+
     // QG = 0: groups of 128, the zero point p.zp.  QG = 5, 6, 7: groups of 2^QG and, with p.zps, a zero point per
     // (row, group); K a multiple of 256.  A lane's 32 weights of a K step lie in one group whatever its size: per column
     // tile and superstep it fetches the 256 / group scales of its row in one load (4, 8 or 16 bytes) and the byte(s) that
@@ -375,6 +516,12 @@ namespace nnf
         // LDS destinations of this wavefront's loads within a stage
         const uint32_t lds_a = (uint32_t)(wave * TM * 1024);
         const uint32_t lds_g = (uint32_t)(A_TILE_BYTES + wave * 256);
+
+        // (sync) the shared tiles this workgroup has parked a part of -- its first and its last segment -- and, in
+        // thread 0, the tile's first sync word as the arrival found it
+        __shared__ uint32_t sync_note;
+        int pend_tile[2] = {-1, -1};
+        uint32_t pend_old[2] = {0u, 0u};
 
         for (long long u = u_begin; u < u_end;)
         {
@@ -828,7 +975,10 @@ namespace nnf
             // (i, j) of all 256 threads is one contiguous 4 KiB); w4a16_gemm_sk_fixup_kernel adds the parts and finishes
             if (!whole)
             {
-                float* mine = p.partial + ((size_t)v + (first_of_mine ? 0 : (size_t)grid)) * T::SLOT_FLOATS + (size_t)tid * 4;
+                const size_t first_float = ((size_t)v + (first_of_mine ? 0 : (size_t)grid)) * T::SLOT_FLOATS + (size_t)tid * 4;
+                float* mine = p.partial + first_float;
+                const bool same_launch = p.sync != nullptr;
+                const buffer_t parked = parked_buffer(p.partial, p.partial_bytes);
 #pragma unroll
                 for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -836,10 +986,27 @@ namespace nnf
 #pragma unroll
                         for (int q = 0; q < 4; ++q)
                         {
-                            *reinterpret_cast<floatx4*>(mine + (size_t)(((i * TN + j) * 4 + q) * THREADS * 4)) =
-                                floatx4{acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+                            const size_t at = (size_t)(((i * TN + j) * 4 + q) * THREADS * 4);
+                            const floatx4 part = floatx4{acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+                            if (same_launch)
+                                store_device_scope(parked, (uint32_t)((first_float + at) * sizeof(float)), part);
+                            else
+                                *reinterpret_cast<floatx4*>(mine + at) = part;
                             __builtin_amdgcn_sched_barrier(0); // (one quarter of a tile at a time: few registers)
                         }
+                if (same_launch)
+                {
+                    // every wavefront's part has arrived where every CU sees it before thread 0 counts the workgroup in
+                    wait_vector_memory();
+                    __syncthreads();
+                    uint32_t old = 0u;
+                    if (tid == 0)
+                        old = atomicAdd(p.sync + 2 * (size_t)tile, 1u);
+                    if (first_of_mine)
+                        pend_tile[0] = tile, pend_old[0] = old;
+                    else
+                        pend_tile[1] = tile, pend_old[1] = old;
+                }
             }
             else
             {
@@ -861,6 +1028,58 @@ namespace nnf
             if (u < u_end)
                 __syncthreads(); // the staging regions are read before the next segment's tiles land in them
         }
+
+        // ---- (sync) shared tiles: once every workgroup that holds a part has arrived, each of them adds up and
+        // finishes its share of the tile's 32-row blocks (block i belongs to the (i mod n)-th of the n workgroups).
+        // Every workgroup has counted itself in at all its tiles before it waits here, so the waits cannot form a
+        // cycle; they are bounded all the same (workgroups of a grid that is not resident as a whole): a workgroup
+        // whose wait runs out marks its blocks for the last arriver, who never waits.
+        if (p.sync && (pend_tile[0] >= 0 || pend_tile[1] >= 0))
+        {
+            __syncthreads(); // the epilogue's staging regions are free
+            uint8_t* stage = smem + wave * sk_region_bytes<1, TN, GATE>();
+#pragma unroll
+            for (int slot = 0; slot < 2; ++slot)
+            {
+                const int tile = pend_tile[slot];
+                if (tile < 0)
+                    continue;
+                const long long t0 = (long long)tile * SS;
+                const int v_first = owner_of_unit(t0, p.units, grid);
+                const int n_seg = owner_of_unit(t0 + SS - 1, p.units, grid) - v_first + 1;
+                const bool first_is_second_slot = first_unit_of(v_first, p.units, grid) < t0;
+                uint32_t* state = p.sync + 2 * (size_t)tile;
+                if (tid == 0)
+                {
+                    uint32_t own = 0u;
+                    for (int i = v - v_first; i < TM; i += n_seg)
+                        own |= 1u << i;
+                    sync_note = sk_blocks_to_finish(state, pend_old[slot], n_seg, own, p.spin_limit);
+                }
+                __syncthreads();
+                const uint32_t blocks = sync_note;
+                if (blocks)
+                {
+                    // (every part was complete at device scope before its workgroup counted itself in, the count was read
+                    // at device scope, and so are the parts)
+                    for (int i = 0; i < TM; ++i)
+                        if ((blocks >> i) & 1u)
+                            sk_sum_block<TM, TN, GATE, BIAS, RESID, RMS, true>(p, grid, tile, i, v_first, n_seg, first_is_second_slot, stage,
+                                                                               wave, lane);
+                }
+                __syncthreads(); // sync_note is read; (blocks) every wavefront's strips are finished
+                if (blocks && tid == 0)
+                {
+                    const uint32_t n = (uint32_t)__builtin_popcount(blocks);
+                    if (atomicAdd(state + 1, n) + n == (uint32_t)TM)
+                    {
+                        // nobody looks at this tile's words any more: leave them as the next launch wants them
+                        atomicExch(state, 0u);
+                        atomicExch(state + 1, 0u);
+                    }
+                }
+            }
+        }
     }
 
     // Adds the parts of the tiles that several workgroups of w4a16_gemm_sk_kernel worked on, in K order (so the result
@@ -874,11 +1093,9 @@ namespace nnf
         using namespace gemm_sk;
         using T = Tile<TM, TN>;
         constexpr int ROUND_TM = 1, ROUNDS = TM; // (the epilogue routine of a tile one block high)
-        constexpr int BN_OUT = GATE ? T::BN / 2 : T::BN;
         __shared__ __attribute__((aligned(16))) uint8_t stage[ROUND_TM * 32 * (TN * 64 + 16)];
         const int lane = threadIdx.x;
         const int wave = (int)blockIdx.x % WAVES; // the strip: what wavefront `wave` of the GEMM's workgroup parked
-        const int tid = wave * 64 + lane;
         const int tile = (int)blockIdx.x / (WAVES * ROUNDS), r = ((int)blockIdx.x / WAVES) % ROUNDS;
         const int SS = p.supersteps;
         const long long t0 = (long long)tile * SS;
@@ -888,65 +1105,6 @@ namespace nnf
             return;
         // the first owner parked this tile in its second slot when its range began in an earlier tile
         const bool first_is_second_slot = first_unit_of(v_first, p.units, gemm_grid) < t0;
-        int tm, tn;
-        {
-            constexpr int GM = 4;
-            const int per_group = GM * p.tiles_n;
-            const int g = tile / per_group;
-            const int first_m = g * GM;
-            const int gm = min(GM, p.tiles_m - first_m);
-            const int rr = tile - g * per_group;
-            tm = first_m + rr % gm;
-            tn = rr / gm;
-        }
-        const int m0 = tm * T::BM, n0 = tn * BN_OUT;
-        floatx16 c[ROUND_TM][TN];
-#pragma unroll
-        for (int ii = 0; ii < ROUND_TM; ++ii)
-#pragma unroll
-            for (int j = 0; j < TN; ++j)
-#pragma unroll
-                for (int e = 0; e < 16; ++e)
-                    c[ii][j][e] = 0.f;
-        // parts in K order, eight at a time in flight
-        constexpr int D = 8;
-        for (int sg0 = 0; sg0 < n_seg; sg0 += D)
-        {
-            floatx4 x[D][ROUND_TM][TN][4];
-#pragma unroll
-            for (int d = 0; d < D; ++d)
-            {
-                const int sg = min(sg0 + d, n_seg - 1);
-                const float* theirs = p.partial +
-                                      ((size_t)(v_first + sg) + ((sg == 0 && first_is_second_slot) ? (size_t)gemm_grid : 0)) * T::SLOT_FLOATS +
-                                      (size_t)tid * 4;
-#pragma unroll
-                for (int ii = 0; ii < ROUND_TM; ++ii)
-#pragma unroll
-                    for (int j = 0; j < TN; ++j)
-#pragma unroll
-                        for (int q = 0; q < 4; ++q)
-                            x[d][ii][j][q] =
-                                *reinterpret_cast<const floatx4*>(theirs + (size_t)((((r * ROUND_TM + ii) * TN + j) * 4 + q) * THREADS * 4));
-            }
-#pragma unroll
-            for (int d = 0; d < D; ++d)
-                if (sg0 + d < n_seg)
-                {
-#pragma unroll
-                    for (int ii = 0; ii < ROUND_TM; ++ii)
-#pragma unroll
-                        for (int j = 0; j < TN; ++j)
-#pragma unroll
-                            for (int q = 0; q < 4; ++q)
-                            {
-                                c[ii][j][4 * q] += x[d][ii][j][q].x;
-                                c[ii][j][4 * q + 1] += x[d][ii][j][q].y;
-                                c[ii][j][4 * q + 2] += x[d][ii][j][q].z;
-                                c[ii][j][4 * q + 3] += x[d][ii][j][q].w;
-                            }
-                }
-        }
-        sk_finish_round<1, TN, GATE, BIAS, RESID, RMS>(p, c, r, m0, n0, stage, wave, lane);
+        sk_sum_block<TM, TN, GATE, BIAS, RESID, RMS, false>(p, gemm_grid, tile, r, v_first, n_seg, first_is_second_slot, stage, wave, lane);
     }
 } // namespace nnf

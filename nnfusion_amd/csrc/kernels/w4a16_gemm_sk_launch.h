@@ -23,9 +23,10 @@ namespace nnf
             }
             hipLaunchKernelGGL(kernel, dim3(grid), dim3(THREADS), T::LDS_BYTES, stream, p);
             hipError_t e = hipGetLastError();
-            if (e != hipSuccess || !p.partial)
+            if (e != hipSuccess || !p.partial || p.sync)
                 return e;
-            // tiles shared by several workgroups: their parts are added and finished by a second launch
+            // tiles shared by several workgroups: their parts are added and finished by a second launch (unless the
+            // workgroups did it themselves: p.sync)
             constexpr int ROUNDS = TM; // blocks of 32 rows
             hipLaunchKernelGGL((w4a16_gemm_sk_fixup_kernel<TM, TN, GATE, BIAS, RESID, RMS>), dim3(p.tiles_m * p.tiles_n * ROUNDS * WAVES),
                                dim3(64), 0, stream, p, grid);
@@ -84,7 +85,7 @@ namespace nnf
             }
             hipLaunchKernelGGL(kernel, dim3(grid), dim3(THREADS), T::LDS_BYTES, stream, p);
             hipError_t e = hipGetLastError();
-            if (e != hipSuccess || !p.partial)
+            if (e != hipSuccess || !p.partial || p.sync)
                 return e;
             hipLaunchKernelGGL((w4a16_gemm_sk_fixup_kernel<TM, TN, false, false, false, false>), dim3(p.tiles_m * p.tiles_n * TM * WAVES),
                                dim3(64), 0, stream, p, grid);

@@ -6,47 +6,84 @@
 
 #include <hip/hip_runtime.h>
 
+#include <atomic>
+#include <mutex>
+
 namespace
 {
     struct DeviceInfo
     {
-        int valid = 0;
         int num_cu = 0;
-        void* static_scratch = nullptr; // this device's copy of `scratch` below
     };
 
-    // Scratch memory owned by the library, for nnf_w4a16_gemm_static_scratch (callers that cannot allocate).
-    // Every device the library runs on holds its own copy, at its own address, until the process ends.  In host
-    // code the array's name is only a handle: the device address comes from hipGetSymbolAddress, once per device.
+    // Scratch memory owned by the library, for nnf_w4a16_gemm_static_scratch (callers that cannot allocate): parked
+    // tiles / partial sums, and the synchronisation words of the one-launch tile GEMM (zero when the module is
+    // loaded, and every launch leaves them zero).  Every device the library runs on holds its own copy, at its own
+    // address, until the process ends.  In host code the arrays' names are only handles: the device addresses come
+    // from hipGetSymbolAddress, once per device, at that entry point's first call there.
     constexpr size_t STATIC_SCRATCH_BYTES = NNF_STATIC_SCRATCH_BYTES;
     static __device__ __align__(256) unsigned char scratch[STATIC_SCRATCH_BYTES];
+    static __device__ __align__(256) unsigned int scratch_sync[NNF_SYNC_FLAGS_BYTES / sizeof(unsigned int)];
 
-    // Lazily cached properties of each device (with `scratch`, the only global state of the library).
-    DeviceInfo g_dev[64];
+    constexpr int MAX_DEVICES = 64;
+    // Lazily cached properties of each device (with the arrays above, the only global state of the library).  A slot is
+    // written once, under its once_flag, and only read afterwards.
+    struct DeviceSlot
+    {
+        std::once_flag once;
+        int status = NNF_ERR_NO_DEVICE;
+        DeviceInfo info;
+    };
+    DeviceSlot g_dev[MAX_DEVICES];
+    struct ScratchSlot
+    {
+        std::once_flag once;
+        int status = NNF_ERR_NO_DEVICE;
+        void* scratch = nullptr;
+        void* sync = nullptr;
+    };
+    ScratchSlot g_scratch[MAX_DEVICES];
+
+    int current_device(int& dev)
+    {
+        dev = -1;
+        const hipError_t e = hipGetDevice(&dev);
+        return (e != hipSuccess || dev < 0 || dev >= MAX_DEVICES) ? NNF_ERR_NO_DEVICE : NNF_OK;
+    }
 
     int current_device_info(DeviceInfo& out)
     {
-        int dev = -1;
-        hipError_t e = hipGetDevice(&dev);
-        if (e != hipSuccess || dev < 0 || dev >= 64)
+        int dev;
+        if (current_device(dev) != NNF_OK)
             return NNF_ERR_NO_DEVICE;
-        if (!g_dev[dev].valid)
-        {
+        DeviceSlot& slot = g_dev[dev];
+        std::call_once(slot.once, [&] {
             hipDeviceProp_t prop;
-            e = hipGetDeviceProperties(&prop, dev);
-            if (e != hipSuccess)
-                return (int)e;
-            g_dev[dev].num_cu = prop.multiProcessorCount;
-            // device `dev` is current here: the address is that of its own copy
-            void* ptr = nullptr;
-            e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
-            if (e != hipSuccess)
-                return (int)e;
-            g_dev[dev].static_scratch = ptr;
-            g_dev[dev].valid = 1;
-        }
-        out = g_dev[dev];
-        return NNF_OK;
+            const hipError_t e = hipGetDeviceProperties(&prop, dev);
+            slot.info.num_cu = prop.multiProcessorCount;
+            slot.status = e == hipSuccess ? NNF_OK : (int)e;
+        });
+        out = slot.info;
+        return slot.status;
+    }
+
+    // the current device's copies of `scratch` and `scratch_sync` (that device is current here: the addresses are
+    // those of its own copies)
+    int current_static_scratch(void*& scratch_ptr, void*& sync_ptr)
+    {
+        int dev;
+        if (current_device(dev) != NNF_OK)
+            return NNF_ERR_NO_DEVICE;
+        ScratchSlot& slot = g_scratch[dev];
+        std::call_once(slot.once, [&] {
+            hipError_t e = hipGetSymbolAddress(&slot.scratch, HIP_SYMBOL(scratch));
+            if (e == hipSuccess)
+                e = hipGetSymbolAddress(&slot.sync, HIP_SYMBOL(scratch_sync));
+            slot.status = e == hipSuccess ? NNF_OK : (int)e;
+        });
+        scratch_ptr = slot.scratch;
+        sync_ptr = slot.sync;
+        return slot.status;
     }
 
     inline bool aligned16(const void* p)
@@ -71,7 +108,7 @@ extern "C" {
 
 int nnf_abi_version(void)
 {
-    return 3;
+    return 4;
 }
 
 const char* nnf_status_string(int status)
@@ -106,14 +143,24 @@ namespace
         {
             const int r = plan->tile_rows;
             const int c = plan->tile_cols;
-            if ((r != 0 && r != 32 && r != 64 && r != 128 && r != 256) || plan->k_parts < 0 || (c != 0 && c != 128 && c != 256))
+            if ((r != 0 && r != 32 && r != 64 && r != 128 && r != 256) || plan->k_parts < 0 || plan->k_parts > NNF_MAX_K_PARTS ||
+                (c != 0 && c != 128 && c != 256))
+                return false;
+            if (plan->sync_flags && (!aligned16(plan->sync_flags) || plan->sync_flags_bytes < 8))
                 return false;
             out.tile_rows = r;
             out.k_parts = plan->k_parts;
             out.tile_cols = c;
+            out.sync_flags = plan->sync_flags;
+            out.sync_bytes = plan->sync_flags ? plan->sync_flags_bytes : 0;
+            out.spin_limit = plan->spin_limit;
         }
         return true;
     }
+
+    // the parameters of the specialised fp16 x int4 kernels
+    bool is_plain_w4a16(const nnf_quant* q) { return q->bits == 4 && q->group == 128 && !q->zero_points; }
+    int group_shift_of(int group) { return group == 32 ? 5 : group == 64 ? 6 : 7; }
 
     // nnf_w8a8_variant -> the launchers' numbering of kernel families (that of nnf_w4a16_variant)
     int w8a8_path(int variant) { return variant == NNF_W8A8_AUTO ? 0 : variant + 1; }
@@ -175,16 +222,28 @@ int nnf_w4a16_gemm_static_scratch(nnf_stream_t stream, const void* A, const void
     int st = check_w4a16(A, Wq, scales, Y, M, N, K, group, zp);
     if (st != NNF_OK)
         return st;
-    // the partial sums of every path nnf_w4a16_gemm may take for this shape
-    if (nnf::workspace::w4a16_gemm(M, N, K, group) > STATIC_SCRATCH_BYTES)
-        return NNF_ERR_STATIC_SCRATCH_LIMIT;
     DeviceInfo dev;
     st = current_device_info(dev);
     if (st != NNF_OK)
         return st;
+    // what the launch parks on this device
+    const nnf::workspace::W4A16Route route = nnf::workspace::route_w4a16(M, N, K, false, false, false, dev.num_cu);
+    if (route.kind == nnf::workspace::W4A16Route::NONE)
+        return NNF_ERR_UNSUPPORTED_SHAPE;
+    if (route.partial_bytes > STATIC_SCRATCH_BYTES)
+        return NNF_ERR_STATIC_SCRATCH_LIMIT;
+    void *buffer = nullptr, *sync = nullptr;
+    st = current_static_scratch(buffer, sync);
+    if (st != NNF_OK)
+        return st;
     // Same kernels, with the device's static buffer in the place of the caller's workspace.  Nothing in it has to
-    // start at zero: every partial sum is written by the GEMM kernel before the reduction pass reads it.
-    return nnf_w4a16_gemm(stream, A, Wq, scales, Y, M, N, K, group, zp, dev.static_scratch, STATIC_SCRATCH_BYTES);
+    // start at zero: every partial sum is written before it is read.  The synchronisation words are the library's
+    // own as well (zero at load, left zero by every launch): tiles shared between workgroups need no second launch.
+    nnf::LaunchChoice choice;
+    choice.sync_flags = sync;
+    choice.sync_bytes = NNF_SYNC_FLAGS_BYTES;
+    st = w4a16_gemm_checked(stream, A, Wq, scales, Y, M, N, K, group, zp, choice, buffer, STATIC_SCRATCH_BYTES);
+    return st == NNF_ERR_WORKSPACE_TOO_SMALL ? NNF_ERR_STATIC_SCRATCH_LIMIT : st;
 }
 
 int nnf_wna16_supported(int M, int N, int K, const nnf_quant* q)
@@ -193,17 +252,6 @@ int nnf_wna16_supported(int M, int N, int K, const nnf_quant* q)
         return 0;
     return nnf::wna16_supported(M, N, K, q->bits, q->group) ? 1 : 0;
 }
-
-namespace
-{
-    // the parameters of the specialised fp16 x int4 kernels
-    bool is_plain_w4a16(const nnf_quant* q) { return q->bits == 4 && q->group == 128 && !q->zero_points; }
-} // namespace
-
-namespace
-{
-    int group_shift_of(int group) { return group == 32 ? 5 : group == 64 ? 6 : 7; }
-} // namespace
 
 size_t nnf_wna16_gemm_workspace_bytes(int M, int N, int K, const nnf_quant* q)
 {
@@ -429,6 +477,24 @@ int nnf_fused_mlp_w4a16(nnf_stream_t stream, const void* x, const void* gamma, f
                         const void* Sgu, const void* Wd, const void* Sd, void* out, int M, int H, int I, int group,
                         int zp, void* workspace, size_t workspace_bytes)
 {
+    return nnf_fused_mlp_w4a16_planned(stream, x, gamma, eps, Wgu, Sgu, Wd, Sd, out, M, H, I, group, zp, nullptr, nullptr,
+                                       workspace, workspace_bytes);
+}
+
+int nnf_fused_mlp_w4a16_planned(nnf_stream_t stream, const void* x, const void* gamma, float eps, const void* Wgu,
+                                const void* Sgu, const void* Wd, const void* Sd, void* out, int M, int H, int I, int group,
+                                int zp, const nnf_plan* gate_up_plan, const nnf_plan* down_plan, void* workspace,
+                                size_t workspace_bytes)
+{
+    nnf::LaunchChoice choice_gu, choice_d;
+    if (!make_choice(NNF_W4A16_AUTO, gate_up_plan, NNF_W4A16_GEMV_ROWS, choice_gu) ||
+        !make_choice(NNF_W4A16_AUTO, down_plan, NNF_W4A16_GEMV_ROWS, choice_d))
+        return NNF_ERR_INVALID_ARGUMENT;
+    // a plan that fixes the tile shape or the split means the tile GEMM
+    if (choice_gu.tile_rows || choice_gu.k_parts || choice_gu.tile_cols)
+        choice_gu.path = NNF_W4A16_GEMM_MFMA;
+    if (choice_d.tile_rows || choice_d.k_parts || choice_d.tile_cols)
+        choice_d.path = NNF_W4A16_GEMM_MFMA;
     if (!x || !gamma || !Wgu || !Sgu || !Wd || !Sd || !out || M <= 0 || H <= 0 || I <= 0)
         return NNF_ERR_INVALID_ARGUMENT;
     if (!aligned16(x) || !aligned16(gamma) || !aligned16(Wgu) || !aligned16(Sgu) || !aligned16(Wd) ||
@@ -440,26 +506,31 @@ int nnf_fused_mlp_w4a16(nnf_stream_t stream, const void* x, const void* gamma, f
     int st = current_device_info(dev);
     if (st != NNF_OK)
         return st;
-    {
-        // what the two launches park behind h, on this device (the down projection's residual is x: in place when
-        // the caller passes out == x)
-        const size_t a = nnf::workspace::route_w4a16(M, I, H, true, true, false, dev.num_cu).partial_bytes;
-        const size_t b = nnf::workspace::route_w4a16(M, H, I, false, false, out == x, dev.num_cu).partial_bytes;
-        if (!workspace || workspace_bytes < nnf::workspace::fused_mlp_partial_offset(M, H, I, dev.num_cu) + (a > b ? a : b))
-            return NNF_ERR_WORKSPACE_TOO_SMALL;
-    }
+    // workspace = [ rstd of the first product ][ h: M x I fp16 ][ what either launch parks, on this device ] (the down
+    // projection's residual is x: in place when the caller passes out == x)
+    const nnf::workspace::W4A16Route route_gu = nnf::workspace::route_w4a16(
+        M, I, H, true, true, false, dev.num_cu, choice_gu.path, choice_gu.tile_rows, choice_gu.k_parts, choice_gu.tile_cols);
+    const nnf::workspace::W4A16Route route_d = nnf::workspace::route_w4a16(
+        M, H, I, false, false, out == x, dev.num_cu, choice_d.path, choice_d.tile_rows, choice_d.k_parts, choice_d.tile_cols);
+    if (route_gu.kind == nnf::workspace::W4A16Route::NONE || route_d.kind == nnf::workspace::W4A16Route::NONE)
+        return NNF_ERR_UNSUPPORTED_SHAPE;
+    const size_t h_offset = route_gu.rms_bytes;
+    const size_t partial_offset = h_offset + nnf::workspace::align256((size_t)M * I * 2);
+    const size_t parked = route_gu.partial_bytes > route_d.partial_bytes ? route_gu.partial_bytes : route_d.partial_bytes;
+    if (!workspace || workspace_bytes < partial_offset + parked)
+        return NNF_ERR_WORKSPACE_TOO_SMALL;
     uint8_t* ws = (uint8_t*)workspace;
-    void* h = ws + nnf::workspace::fused_mlp_h_offset(M, H, I, dev.num_cu);
-    void* partial = ws + nnf::workspace::fused_mlp_partial_offset(M, H, I, dev.num_cu);
-    // h = SiLU(gate) * up, gate|up = RMSNorm(x) . Wgu^T : the normalisation pre-pass, then one GEMM with the
-    // gate and up projections as the two halves of every N tile
+    void* h = ws + h_offset;
+    void* partial = ws + partial_offset;
+    // h = SiLU(gate) * up, gate|up = RMSNorm(x) . Wgu^T : one GEMM with the gate and up projections as the two halves
+    // of every N tile, the RMSNorm weight and rstd inside it
     hipError_t e = nnf::launch_w4a16_gemm((hipStream_t)stream, x, Wgu, Sgu, h, M, I, H, zp, gamma, eps, nullptr,
-                                          nullptr, NNF_ACT_SILU_GATE, ws, partial, dev.num_cu);
+                                          nullptr, NNF_ACT_SILU_GATE, ws, partial, dev.num_cu, choice_gu);
     if (e != hipSuccess)
         return (int)e;
     // out = h . Wd^T + x
     e = nnf::launch_w4a16_gemm((hipStream_t)stream, h, Wd, Sd, out, M, H, I, zp, nullptr, 0.f, nullptr, x, NNF_ACT_NONE,
-                               nullptr, partial, dev.num_cu);
+                               nullptr, partial, dev.num_cu, choice_d);
     return (int)e;
 }
 

@@ -128,6 +128,9 @@ namespace nnf
             int grid = 0;
             int slots = 0;     // 0: every tile belongs to one workgroup (no workspace, no second launch)
             size_t bytes() const { return (size_t)slots * tile_rows * tile_weight_rows * sizeof(float); }
+            // two synchronisation words per tile for the one-launch form (workgroups that share a tile add its parts
+            // up themselves); 0: no tile is shared
+            size_t sync_bytes() const { return slots ? (size_t)tiles_m * tiles_n * 2 * sizeof(unsigned) : 0; }
         };
         // Tile shape.  What the caller fixes (forced_rows 32 / 64 / 128 / 256, forced_cols 128 / 256) is kept, the rest
         // is chosen by M (measured at N = K = 8192 and on the Llama shapes, alternating the candidates in one process):
@@ -157,7 +160,7 @@ namespace nnf
         }
         // tiles_n column tiles, `per_tile` units of K per tile, at least `min_units` units per workgroup (unless forced);
         // forced_grid: 0 = the plan's own choice
-        inline SkPlan plan_sk(int M, int tiles_n, int per_tile, int min_units, int num_cu, int forced_tile_rows, int forced_grid)
+        inline SkPlan plan_sk(int M, int tiles_n, int per_tile, int min_units, int num_cu, int forced_tile_rows, long long forced_grid)
         {
             SkPlan p;
             const int rows = forced_tile_rows;
@@ -190,7 +193,7 @@ namespace nnf
         }
         // fp16 x int4: units of 256 k (supersteps), a workgroup keeps at least two (eight K steps of 64)
         // forced_tile_rows / forced_cols: 0 = the plan's own choice (sk_tile_shape)
-        inline SkPlan plan_w4a16_sk(int M, int N, int K, bool gate, int num_cu, int forced_tile_rows = 0, int forced_grid = 0,
+        inline SkPlan plan_w4a16_sk(int M, int N, int K, bool gate, int num_cu, int forced_tile_rows = 0, long long forced_grid = 0,
                                     int forced_cols = 0)
         {
             if (M <= 0 || N <= 0 || K < 128 || num_cu < 1)
@@ -209,8 +212,9 @@ namespace nnf
         {
             if (workgroups_per_tile <= 0)
                 return plan_w4a16_sk(M, N, K, gate, num_cu, tile_rows, 0, tile_cols);
+            // (at most one workgroup per unit of 256 k: plan_sk limits the grid to the number of units)
             const SkPlan t = plan_w4a16_sk(M, N, K, gate, num_cu, tile_rows, 0, tile_cols);
-            return plan_w4a16_sk(M, N, K, gate, num_cu, tile_rows, t.tiles_m * t.tiles_n * workgroups_per_tile, tile_cols);
+            return plan_w4a16_sk(M, N, K, gate, num_cu, tile_rows, (long long)t.tiles_m * t.tiles_n * workgroups_per_tile, tile_cols);
         }
 
         // ---- plan of the skinny (M <= 16) MFMA GEMV kernel ---------------------------------------------

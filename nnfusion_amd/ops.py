@@ -12,16 +12,32 @@ from . import _lib
 
 
 class NnfPlan(ctypes.Structure):
-    """struct nnf_plan of the C header: what a kernel-selection candidate fixes about the tile GEMM."""
-    _fields_ = [("tile_rows", ctypes.c_int), ("k_parts", ctypes.c_int), ("tile_cols", ctypes.c_int)]
+    """struct nnf_plan of the C header: what a kernel-selection candidate fixes about the tile GEMM, and the
+    synchronisation words that make the fp16 x int4 tile GEMM a single launch."""
+    _fields_ = [("tile_rows", ctypes.c_int), ("k_parts", ctypes.c_int), ("tile_cols", ctypes.c_int),
+                ("sync_flags", ctypes.c_void_p), ("sync_flags_bytes", ctypes.c_size_t), ("spin_limit", ctypes.c_int)]
 
 
-def _plan_arg(plan):
-    """None, an NnfPlan or a (tile_rows, k_parts[, tile_cols]) tuple -> (object to keep alive, pointer argument)."""
-    if plan is None:
+SYNC_FLAGS_BYTES = 64 << 10  # NNF_SYNC_FLAGS_BYTES
+
+
+def sync_flags(device):
+    """A zeroed buffer for nnf_plan::sync_flags (cleared once here; every call leaves it zero again)."""
+    return torch.zeros(SYNC_FLAGS_BYTES, dtype=torch.uint8, device=device)
+
+
+def _plan_arg(plan, sync=None, spin_limit=0):
+    """None, an NnfPlan or a (tile_rows, k_parts[, tile_cols]) tuple, plus an optional sync_flags tensor
+    -> (object to keep alive, pointer argument)."""
+    if plan is None and sync is None:
         return None, None
     if not isinstance(plan, NnfPlan):
-        plan = NnfPlan(int(plan[0]), int(plan[1]), int(plan[2]) if len(plan) > 2 else 0)
+        t = tuple(plan) if plan is not None else (0, 0, 0)
+        plan = NnfPlan(int(t[0]), int(t[1]), int(t[2]) if len(t) > 2 else 0, None, 0, 0)
+    if sync is not None:
+        plan.sync_flags = sync.data_ptr()
+        plan.sync_flags_bytes = sync.numel() * sync.element_size()
+        plan.spin_limit = int(spin_limit)
     return plan, ctypes.cast(ctypes.pointer(plan), ctypes.c_void_p)
 
 
@@ -119,7 +135,8 @@ def w4a16_variant_supported(m, n, k, variant, group=128):
     return bool(_lib.kernels().nnf_w4a16_variant_supported(m, n, k, group, VARIANTS[variant]))
 
 
-def w4a16_gemm_variant(a, wq, scales, variant, plan=None, group=128, zp=8, out=None, workspace=None):
+def w4a16_gemm_variant(a, wq, scales, variant, plan=None, group=128, zp=8, out=None, workspace=None, sync=None,
+                       spin_limit=0):
     """As w4a16_gemm through one kernel variant (a key of VARIANTS) and, for the tile GEMM, a plan (tile_rows,
     k_parts); raises NnfError with status -2 when the variant cannot serve the shape."""
     lib = _lib.kernels()
@@ -130,7 +147,7 @@ def w4a16_gemm_variant(a, wq, scales, variant, plan=None, group=128, zp=8, out=N
     assert a.is_contiguous() and wq.is_contiguous() and scales.is_contiguous()
     if out is None:
         out = torch.empty((m, n), dtype=torch.float16, device=a.device)
-    keep, plan_ptr = _plan_arg(plan)
+    keep, plan_ptr = _plan_arg(plan, sync, spin_limit)
     if workspace is None:
         workspace = _ws(lib.nnf_w4a16_gemm_variant_workspace_bytes(m, n, k, group, v, plan_ptr), a.device)
     _check(lib.nnf_w4a16_gemm_variant(_stream(), a.data_ptr(), wq.data_ptr(), scales.data_ptr(), out.data_ptr(),
@@ -140,7 +157,7 @@ def w4a16_gemm_variant(a, wq, scales, variant, plan=None, group=128, zp=8, out=N
 
 
 def w4a16_gemm_fused(a, wq, scales, group=128, zp=8, rms_gamma=None, rms_eps=1e-6, bias=None, residual=None,
-                     act=0, out=None, workspace=None, variant="auto", plan=None):
+                     act=0, out=None, workspace=None, variant="auto", plan=None, sync=None, spin_limit=0):
     """GEMM with the fused RMSNorm prologue / bias, residual, SiLU-gate epilogues (see the C header); variant
     "gemm_mfma" and a plan (tile_rows, k_parts) go through nnf_w4a16_gemm_fused_variant."""
     lib = _lib.kernels()
@@ -149,8 +166,8 @@ def w4a16_gemm_fused(a, wq, scales, group=128, zp=8, rms_gamma=None, rms_eps=1e-
     if out is None:
         out = torch.empty((m, n), dtype=torch.float16, device=a.device)
     need = lib.nnf_w4a16_gemm_fused_workspace_bytes(m, n, k, group, act)
-    if variant != "auto" or plan is not None:
-        keep, plan_ptr = _plan_arg(plan)
+    if variant != "auto" or plan is not None or sync is not None:
+        keep, plan_ptr = _plan_arg(plan, sync, spin_limit)
         v = VARIANTS[variant]
         if workspace is None:
             workspace = _ws(need + lib.nnf_w4a16_gemm_variant_workspace_bytes(m, wq.shape[0], k, group, v, plan_ptr),
@@ -227,14 +244,29 @@ def w8a8_gemm_acc(a, w, out=None, workspace=None, variant="auto", plan=None):
     return out
 
 
-def fused_mlp_w4a16(x, gamma, wgu, sgu, wd, sd, eps=1e-6, group=128, zp=8, out=None, workspace=None):
-    """out = x + Wd . (SiLU(Wg . n) * (Wu . n)), n = RMSNorm(x, gamma, eps)."""
+def fused_mlp_w4a16(x, gamma, wgu, sgu, wd, sd, eps=1e-6, group=128, zp=8, out=None, workspace=None, sync=None,
+                    spin_limit=0, gate_up_plan=None, down_plan=None):
+    """out = x + Wd . (SiLU(Wg . n) * (Wu . n)), n = RMSNorm(x, gamma, eps).  `sync` (see sync_flags) or a plan for
+    either product goes through nnf_fused_mlp_w4a16_planned."""
     lib = _lib.kernels()
     m, h = x.shape
     i = wgu.shape[0] // 2
     if out is None:
         out = torch.empty((m, h), dtype=torch.float16, device=x.device)
     need = lib.nnf_fused_mlp_w4a16_workspace_bytes(m, h, i, group)
+    if sync is not None or gate_up_plan is not None or down_plan is not None:
+        keep_a, plan_a = _plan_arg(gate_up_plan, sync, spin_limit)
+        keep_b, plan_b = _plan_arg(down_plan, sync, spin_limit)
+        if workspace is None:
+            v = VARIANTS["gemm_mfma"]
+            extra = (lib.nnf_w4a16_gemm_variant_workspace_bytes(m, 2 * i, h, group, v, plan_a) if gate_up_plan is not None else 0) + \
+                    (lib.nnf_w4a16_gemm_variant_workspace_bytes(m, h, i, group, v, plan_b) if down_plan is not None else 0)
+            workspace = _ws(need + extra, x.device)
+        _check(lib.nnf_fused_mlp_w4a16_planned(_stream(), x.data_ptr(), gamma.data_ptr(), float(eps), wgu.data_ptr(),
+                                               sgu.data_ptr(), wd.data_ptr(), sd.data_ptr(), out.data_ptr(), m, h, i, group,
+                                               zp, plan_a, plan_b, workspace.data_ptr(), workspace.numel()),
+               "nnf_fused_mlp_w4a16_planned")
+        return out
     if workspace is None:
         workspace = _ws(need, x.device)
     _check(lib.nnf_fused_mlp_w4a16(_stream(), x.data_ptr(), gamma.data_ptr(), float(eps), wgu.data_ptr(),

@@ -39,7 +39,7 @@ def test_ctypes_table_covers_the_header():
 
 def test_pure_host_queries_work_without_a_gpu():
     lib = _lib.kernels()
-    assert lib.nnf_abi_version() == 3
+    assert lib.nnf_abi_version() == 4
     assert lib.nnf_status_string(0) == b"ok"
     assert b"workspace" in lib.nnf_status_string(-3)
     assert lib.nnf_w4a16_gemm_workspace_bytes(1, 4096, 4096, 128) == 0

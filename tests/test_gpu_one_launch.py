@@ -1,0 +1,141 @@
+"""The one-launch form of the fp16 x int4 tile GEMM (nnf_plan::sync_flags): the workgroups that share an output tile add
+its parts up themselves instead of leaving them to a second launch.
+
+Both forms add the parts in the same order, so the test is bit-for-bit equality with the two-launch form (which the
+oracle tests cover), plus the oracle itself, plus the contract of the synchronisation words: all zero again after every
+call.  The path taken when a workgroup's wait runs out (its rows handed to the last arriver) is forced from the host
+with a negative spin limit; every kernel still ends normally.
+"""
+import numpy as np
+import pytest
+
+import oracle
+from nnfusion_amd import datagen
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-2
+
+
+def _t(gpu, *arrays):
+    import torch
+
+    return [None if a is None else torch.from_numpy(np.ascontiguousarray(a)).to(gpu) for a in arrays]
+
+
+def _check(y, ref, tol=TOL):
+    err = float(np.abs(y.astype(np.float32) - ref.astype(np.float32)).max())
+    rms = float(np.sqrt(np.mean(np.asarray(ref, np.float64) ** 2)))
+    assert err <= tol * max(rms, 1e-6), (err, rms)
+
+
+def _ws(gpu, nbytes=96 << 20):
+    import torch
+
+    return torch.empty(nbytes, dtype=torch.uint8, device=gpu)
+
+
+# (tile_rows, k_parts, tile_cols): every tile height and width, tiles shared by 2 .. 5 workgroups, and the library's own
+# even split (None), which cuts tiles at arbitrary places
+PLANS = [None, (256, 2, 256), (256, 3, 128), (128, 2, 256), (128, 3, 128), (128, 5, 128), (64, 2, 256), (64, 4, 128), (32, 3)]
+SHAPES = [(200, 300, 1024), (64, 520, 2048), (130, 128, 1536), (17, 40, 1280), (256, 1024, 4096)]
+
+
+@pytest.mark.parametrize("spin_limit", [0, -1], ids=["wait", "hand-over"])
+@pytest.mark.parametrize("plan", PLANS, ids=lambda p: "auto" if p is None else "rows%d-parts%d" % p[:2] + ("-cols%d" % p[2] if len(p) > 2 else ""))
+@pytest.mark.parametrize("m,n,k", SHAPES)
+def test_one_launch_equals_two_launches(gpu, m, n, k, plan, spin_limit):
+    import torch
+
+    from nnfusion_amd import ops
+
+    print(f"case one-launch M={m} N={n} K={k} plan={plan} spin_limit={spin_limit}", flush=True)
+    a, wq, s = datagen.w4a16_case(3, m, n, k)
+    ta, tw, ts = _t(gpu, a, wq, s)
+    ws = _ws(gpu)
+    two = ops.w4a16_gemm_variant(ta, tw, ts, "gemm_mfma", plan=plan, workspace=ws)
+    sync = ops.sync_flags(gpu)
+    one = ops.w4a16_gemm_variant(ta, tw, ts, "gemm_mfma", plan=plan, workspace=ws, sync=sync, spin_limit=spin_limit)
+    torch.cuda.synchronize()
+    assert int(sync.count_nonzero()) == 0, "the synchronisation words are zero again after the call"
+    assert torch.equal(one, two)
+    _check(one.cpu().numpy(), oracle.w4a16_gemm(a, wq, s, f32_out=True))
+    # the same buffer again, without clearing it, on a smaller product
+    m2 = max(17, m // 2)
+    one2 = ops.w4a16_gemm_variant(ta[:m2].contiguous(), tw, ts, "gemm_mfma", plan=plan, workspace=ws, sync=sync, spin_limit=spin_limit)
+    two2 = ops.w4a16_gemm_variant(ta[:m2].contiguous(), tw, ts, "gemm_mfma", plan=plan, workspace=ws)
+    torch.cuda.synchronize()
+    assert int(sync.count_nonzero()) == 0
+    assert torch.equal(one2, two2)
+
+
+@pytest.mark.parametrize("spin_limit", [0, -1], ids=["wait", "hand-over"])
+@pytest.mark.parametrize("fused", ["bias+residual", "rms+gate", "rms+bias", "residual-in-place"])
+def test_one_launch_fused_forms(gpu, fused, spin_limit):
+    import torch
+
+    from nnfusion_amd import ops
+
+    m, n, k = 150, 384, 2048
+    gate = "gate" in fused
+    a, wq, s = datagen.w4a16_case(7, m, 2 * n if gate else n, k)
+    rng = np.random.default_rng(11)
+    gamma = (1.0 + 0.1 * rng.standard_normal(k)).astype(np.float16) if "rms" in fused else None
+    bias = rng.standard_normal(n).astype(np.float16) if "bias" in fused else None
+    resid = rng.standard_normal((m, n)).astype(np.float16) if "residual" in fused else None
+    ta, tw, ts, tg, tb, tr = _t(gpu, a, wq, s, gamma, bias, resid)
+    kw = dict(rms_gamma=tg, bias=tb, act=1 if gate else 0, variant="gemm_mfma", plan=(128, 3, 256 if gate else 128))
+    ws = _ws(gpu)
+    if fused == "residual-in-place":
+        out_two, out_one = tr.clone(), tr.clone()
+        two = ops.w4a16_gemm_fused(ta, tw, ts, residual=out_two, out=out_two, workspace=ws, **kw)
+        sync = ops.sync_flags(gpu)
+        one = ops.w4a16_gemm_fused(ta, tw, ts, residual=out_one, out=out_one, workspace=ws, sync=sync, spin_limit=spin_limit, **kw)
+    else:
+        two = ops.w4a16_gemm_fused(ta, tw, ts, residual=tr, workspace=ws, **kw)
+        sync = ops.sync_flags(gpu)
+        one = ops.w4a16_gemm_fused(ta, tw, ts, residual=tr, workspace=ws, sync=sync, spin_limit=spin_limit, **kw)
+    torch.cuda.synchronize()
+    assert int(sync.count_nonzero()) == 0
+    assert torch.equal(one, two)
+
+
+@pytest.mark.parametrize("spin_limit", [0, -1], ids=["wait", "hand-over"])
+@pytest.mark.parametrize("m", [40, 256])
+def test_one_launch_mlp_block(gpu, m, spin_limit):
+    """The fused MLP with the same synchronisation words for both of its products."""
+    import torch
+
+    from nnfusion_amd import ops
+
+    h, i = 1024, 2816
+    x, gamma, wgu, sgu, wd, sd = datagen.mlp_case(5, m, h, i)
+    tx, tg, twgu, tsgu, twd, tsd = _t(gpu, x, gamma, wgu, sgu, wd, sd)
+    two = ops.fused_mlp_w4a16(tx, tg, twgu, tsgu, twd, tsd)
+    sync = ops.sync_flags(gpu)
+    one = ops.fused_mlp_w4a16(tx, tg, twgu, tsgu, twd, tsd, sync=sync, spin_limit=spin_limit)
+    again = ops.fused_mlp_w4a16(tx, tg, twgu, tsgu, twd, tsd, sync=sync, spin_limit=spin_limit)
+    torch.cuda.synchronize()
+    assert int(sync.count_nonzero()) == 0
+    assert torch.equal(one, two) and torch.equal(again, two)
+
+
+def test_one_launch_full_size_rows(gpu):
+    """configs[2] at M = 128 and the MLP block's first product at M = 256, the library's own plans: both forms agree bit for
+    bit, twice in a row on the same words."""
+    import torch
+
+    from nnfusion_amd import ops
+
+    for (m, n, k) in [(128, 8192, 8192), (256, 4096, 11008)]:
+        print(f"case one-launch full size M={m} N={n} K={k}", flush=True)
+        a, wq, s = datagen.w4a16_case(1, m, n, k)
+        ta, tw, ts = _t(gpu, a, wq, s)
+        ws = _ws(gpu)
+        two = ops.w4a16_gemm(ta, tw, ts, workspace=ws)
+        sync = ops.sync_flags(gpu)
+        for _ in range(2):
+            one = ops.w4a16_gemm_variant(ta, tw, ts, "auto", workspace=ws, sync=sync)
+            torch.cuda.synchronize()
+            assert int(sync.count_nonzero()) == 0
+            assert torch.equal(one, two)
