@@ -201,6 +201,32 @@ NNF_API int nnf_wna16_gemm(nnf_stream_t stream,
                    int M, int N, int K, const nnf_quant* q,
                    void* workspace, size_t workspace_bytes);
 
+/* ---------------------------------------------------------------------------------------------
+ * The nodes around a quantized product, for graphs in which no fusion pattern absorbed them (a gate
+ * product with a second consumer, a normalisation that feeds something else as well, ...): fp16
+ * tensors, fp32 arithmetic, one rounding to fp16 per node.  The reference emits such nodes through its
+ * element-wise emitter (cuda_gpu/kernels/elementwise.cpp; the operators' bodies are the CudaOpMap entries
+ * of cuda_gpu/cuda_kernelops.hpp:408 Add, :416 Multiply, :447-451 Sigmoid) and layer_norm.cpp.
+ * ------------------------------------------------------------------------------------------- */
+enum nnf_elementwise_op
+{
+    NNF_EW_ADD = 0,      /* a + b */
+    NNF_EW_MULTIPLY = 1, /* a * b */
+    NNF_EW_SIGMOID = 2,  /* 1 / (1 + exp(-a)) */
+    NNF_EW_SWISH = 3     /* a * sigmoid(a) */
+};
+/* y[r, c] = op(a[r, c], b[r, c]) over fp16 [rows, cols]; b_is_row != 0: b is [cols], the same for every row
+ * (a bias).  Unary operators ignore b.  y may be a or b. */
+NNF_API int nnf_elementwise_f16(nnf_stream_t stream, int op, const void* a, const void* b, void* y,
+                        size_t rows, int cols, int b_is_row);
+/* y[m, :] = x[m, :] * rsqrt(mean_k(x[m, k]^2) + eps) * gamma  (rsqrt(x + eps) as in the reference's LayerNorm,
+ * cuda_gpu/cuda_langunit.cpp:618; the reference has no RMSNorm operator).  K a multiple of 8. */
+NNF_API int nnf_rms_norm_f16(nnf_stream_t stream, const void* x, const void* gamma, void* y, int M, int K, float eps);
+/* W fp16 [N, K] = (q - zero point) * scale per block of `group` weights along K: the reference's Dequantize
+ * (core/kernels/cpu/reference/kernels.cpp:601-623: integer subtract, cast, multiply) for the weight layouts of
+ * nnf_wna16_gemm.  For a Dequantize node that does not feed a product (one that does is folded into it). */
+NNF_API int nnf_dequantize_f16(nnf_stream_t stream, const void* Wq, const void* scales, void* W, int N, int K, const nnf_quant* q);
+
 /* Epilogue / prologue selectors for nnf_w4a16_gemm_fused. */
 enum nnf_activation
 {
@@ -247,6 +273,18 @@ NNF_API int nnf_w4a16_gemm_fused_variant(nnf_stream_t stream,
                                  const void* bias, const void* residual, int act,
                                  int variant, const nnf_plan* plan,
                                  void* workspace, size_t workspace_bytes);
+
+/* nnf_w4a16_gemm_fused for every block parameter of nnf_wna16_gemm (act == NNF_ACT_SILU_GATE: Wq, scales and the zero
+ * points hold 2N rows).  4 bits / groups of 128 / a scalar zero point is nnf_w4a16_gemm_fused itself; the other
+ * combinations run the nodes one after the other -- RMSNorm (into `workspace`), the product on nnf_wna16_gemm's
+ * kernels, one element-wise kernel for the epilogue -- with the fp16 tensors of the unfused graph between them. */
+NNF_API size_t nnf_wna16_gemm_fused_workspace_bytes(int M, int N, int K, const nnf_quant* q, int act);
+NNF_API int nnf_wna16_gemm_fused(nnf_stream_t stream,
+                         const void* A, const void* Wq, const void* scales, void* Y,
+                         int M, int N, int K, const nnf_quant* q,
+                         const void* rms_gamma, float rms_eps,
+                         const void* bias, const void* residual, int act,
+                         void* workspace, size_t workspace_bytes);
 
 /* ---------------------------------------------------------------------------------------------
  * W8A8: int8 x int8 -> int32 on the int8 MFMA, then the per-token / per-channel dequantisation.
@@ -320,6 +358,17 @@ NNF_API int nnf_fused_mlp_w4a16_planned(nnf_stream_t stream,
                                 int M, int H, int I, int group, int zp,
                                 const nnf_plan* gate_up_plan, const nnf_plan* down_plan,
                                 void* workspace, size_t workspace_bytes);
+
+/* The same block for every block parameter of nnf_wna16_gemm, one nnf_quant per weight matrix (their zero-point
+ * tensors differ).  Both plain (4 bits, groups of 128, the same scalar zero point): nnf_fused_mlp_w4a16 itself;
+ * otherwise the nodes one after the other, as nnf_wna16_gemm_fused does. */
+NNF_API size_t nnf_fused_mlp_wna16_workspace_bytes(int M, int H, int I, const nnf_quant* q_gate_up, const nnf_quant* q_down);
+NNF_API int nnf_fused_mlp_wna16(nnf_stream_t stream,
+                        const void* x, const void* gamma, float eps,
+                        const void* Wgu, const void* Sgu, const void* Wd, const void* Sd,
+                        void* out,
+                        int M, int H, int I, const nnf_quant* q_gate_up, const nnf_quant* q_down,
+                        void* workspace, size_t workspace_bytes);
 
 #ifdef __cplusplus
 }

@@ -53,6 +53,13 @@ KERNEL_ABI = {
     "nnf_w8a8_gemm_acc": (_c_int, [_c_vp] * 4 + [_c_int] * 3 + [_c_vp, _c_sz]),
     "nnf_fused_mlp_w4a16_workspace_bytes": (_c_sz, [_c_int] * 4),
     "nnf_fused_mlp_w4a16": (_c_int, [_c_vp, _c_vp, _c_vp, _c_f] + [_c_vp] * 5 + [_c_int] * 5 + [_c_vp, _c_sz]),
+    "nnf_elementwise_f16": (_c_int, [_c_vp, _c_int, _c_vp, _c_vp, _c_vp, _c_sz, _c_int, _c_int]),
+    "nnf_rms_norm_f16": (_c_int, [_c_vp] * 4 + [_c_int, _c_int, _c_f]),
+    "nnf_dequantize_f16": (_c_int, [_c_vp] * 4 + [_c_int, _c_int, _c_vp]),
+    "nnf_wna16_gemm_fused_workspace_bytes": (_c_sz, [_c_int] * 3 + [_c_vp, _c_int]),
+    "nnf_wna16_gemm_fused": (_c_int, [_c_vp] * 5 + [_c_int] * 3 + [_c_vp, _c_vp, _c_f, _c_vp, _c_vp, _c_int, _c_vp, _c_sz]),
+    "nnf_fused_mlp_wna16_workspace_bytes": (_c_sz, [_c_int] * 3 + [_c_vp, _c_vp]),
+    "nnf_fused_mlp_wna16": (_c_int, [_c_vp, _c_vp, _c_vp, _c_f] + [_c_vp] * 5 + [_c_int] * 3 + [_c_vp, _c_vp, _c_vp, _c_sz]),
     "nnf_fused_mlp_w4a16_planned": (_c_int, [_c_vp, _c_vp, _c_vp, _c_f] + [_c_vp] * 5 + [_c_int] * 5 + [_c_vp, _c_vp, _c_vp, _c_sz]),
 }
 

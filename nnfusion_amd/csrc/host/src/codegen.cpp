@@ -317,6 +317,12 @@ namespace nnfusion
                 *m_globals << "static " << ctype(pt.first) << "* " << pt.first->get_name() << " = nullptr;\n";
                 *m_init << pt.first->get_name() << " = (" << ctype(pt.first) << "*)(group_0_ROCM_GPU_0_memory_pool + "
                         << pt.second << ");\n";
+                // a tensor its kernel wants cleared (descriptor::Tensor::set_memset): nothing else lives at its place in
+                // the pool, and the kernels that ask for this leave it cleared, so once, here, is enough (the reference
+                // clears its memset pool at the top of every kernel_entry: cuda_codegen_pass.cpp:154-161)
+                if (pt.first->is_memset())
+                    *m_init << "HIP_SAFE_CALL(hipMemset(" << pt.first->get_name() << ", " << pt.first->get_memset_value() << ", "
+                            << pt.first->size() << "));\n";
             }
             for (auto& kv : alias)
             {

@@ -55,13 +55,13 @@ namespace nnfusion
                 bufs.push_back({ctx->outputs[i]->get_element_type().c_type_string(),
                                 "output" + std::to_string(i) + "_host", "output" + std::to_string(i),
                                 ctx->outputs[i]->size(), 1});
-            for (auto& t : ctx->tensors)
-                bufs.push_back({t->get_element_type().c_type_string(), "", t->get_name(), t->size(), 2});
+            for (auto& t : ctx->tensors) // dir 3: scratch that its kernel wants cleared
+                bufs.push_back({t->get_element_type().c_type_string(), "", t->get_name(), t->size(), t->is_memset() ? 3 : 2});
 
             std::vector<std::string> host_params, call_args{"stream"};
             for (auto& b : bufs)
             {
-                if (b.dir != 2)
+                if (b.dir < 2)
                     host_params.push_back(b.type + "* " + b.host);
                 call_args.push_back(b.dev);
             }
@@ -74,6 +74,8 @@ namespace nnfusion
                 src << "PROF_CHECK(hipMalloc((void**)&" << b.dev << ", " << std::max<size_t>(b.bytes, 16) << "));\n";
                 if (b.dir == 0 && b.bytes)
                     src << "PROF_CHECK(hipMemcpy(" << b.dev << ", " << b.host << ", " << b.bytes << ", hipMemcpyHostToDevice));\n";
+                if (b.dir == 3)
+                    src << "PROF_CHECK(hipMemset(" << b.dev << ", 0, " << std::max<size_t>(b.bytes, 16) << "));\n";
             }
             const std::string call = name + "(" + join(call_args, ", ") + ");\n";
             src << "try\n";

@@ -7,6 +7,7 @@
 // (src/nnfusion/engine/pass/graph/kernel_selection.cpp:185-187) and with a priority above every Dot
 // emitter of the reference (2); an unsupported node is declined by returning nullptr.
 #include "../../nnf_workspace.h"
+#include "nnf_hip_kernels.h"
 #include "nnfusion/core/kernels/hip_gpu/hip_emitter.hpp"
 #include "nnfusion/core/kernels/kernel_registration.hpp"
 #include "nnfusion/core/operators/generic_op/generic_op.hpp"
@@ -29,11 +30,41 @@ namespace nnfusion
                 }
             } // namespace
 
-            class QuantDot : public HipLibEmitter
+            // What the emitters of the fp16 x int4 products share.
+            class QuantLibEmitter : public HipLibEmitter
+            {
+            public:
+                using HipLibEmitter::HipLibEmitter;
+
+            protected:
+                // Synchronisation words for the one-launch form of the tile GEMM (nnf_plan::sync_flags), when the product
+                // of these sizes runs on it: a persistent tensor that is zero when the runtime is initialised -- what
+                // be_state_buffer is to the reference's BlockFusion kernels
+                // (src/nnfusion/engine/pass/graph/blockfusion/blockfusion_codegen.cpp:295-304).  Every launch leaves the
+                // words zero again, so one tensor serves all launches of the emitted function.  Returns the statement
+                // that declares `name` as the call's nnf_plan, or "" when the product needs none (then pass nullptr).
+                std::string declare_sync_plan(const std::string& name, int M, int N, int K, bool gate, bool rms)
+                {
+                    const nnf::workspace::W4A16Route route =
+                        nnf::workspace::route_w4a16(M, N, K, gate, rms, false, nnf::workspace::PLAN_CUS);
+                    if (route.kind != nnf::workspace::W4A16Route::TILE)
+                        return "";
+                    const size_t bytes = ((size_t)route.plan.tiles_m * route.plan.tiles_n * 2 * sizeof(uint32_t) + 63) & ~(size_t)63;
+                    if (bytes > NNF_SYNC_FLAGS_BYTES)
+                        return "";
+                    auto flags = allocate_tensor(Shape{bytes}, element::character, "", ROCM_GPU, true);
+                    flags->set_memset(true, 0);
+                    std::ostringstream ss;
+                    ss << "const nnf_plan " << name << " = {0, 0, 0, " << flags->get_name() << ", " << bytes << ", 0};\n";
+                    return ss.str();
+                }
+            };
+
+            class QuantDot : public QuantLibEmitter
             {
             public:
                 explicit QuantDot(std::shared_ptr<KernelContext> ctx)
-                    : HipLibEmitter(ctx)
+                    : QuantLibEmitter(ctx)
                 {
                 }
 
@@ -103,19 +134,28 @@ namespace nnfusion
                     if (ws_bytes > 0)
                         ws = allocate_tensor(Shape{ws_bytes}, element::character)->get_name();
 
+                    // the tile GEMM in one launch (ahead of the body's text: the tensor is part of the kernel's context)
+                    const std::string plan = declare_sync_plan("plan", (int)M, (int)N, (int)K, gate, rms);
                     LanguageUnit_p lu(new LanguageUnit(get_function_name()));
-                    if (!fused)
+                    *lu << plan;
+                    if (!fused && plan.empty())
                     {
                         *lu << "NNF_HIP_CHECK(nnf_w4a16_gemm(stream, input0, input1, input2, output0, " << M << ", " << N
                             << ", " << K << ", " << group << ", " << zp << ", " << ws << ", " << ws_bytes << "));\n";
                     }
+                    else if (!fused)
+                    {
+                        *lu << "NNF_HIP_CHECK(nnf_w4a16_gemm_variant(stream, input0, input1, input2, output0, " << M << ", " << N
+                            << ", " << K << ", " << group << ", " << zp << ", NNF_W4A16_AUTO, &plan, " << ws << ", " << ws_bytes
+                            << "));\n";
+                    }
                     else
                     {
-                        *lu << "NNF_HIP_CHECK(nnf_w4a16_gemm_fused(stream, input0, input1, input2, output0, " << M << ", "
+                        *lu << "NNF_HIP_CHECK(nnf_w4a16_gemm_fused_variant(stream, input0, input1, input2, output0, " << M << ", "
                             << N << ", " << K << ", " << group << ", " << zp << ", " << gamma << ", "
                             << float_literal(cfg["rms_eps"].get<double>()) << ", " << bias << ", " << residual << ", "
-                            << (gate ? "NNF_ACT_SILU_GATE" : "NNF_ACT_NONE") << ", " << ws << ", " << ws_bytes
-                            << "));\n";
+                            << (gate ? "NNF_ACT_SILU_GATE" : "NNF_ACT_NONE") << ", NNF_W4A16_AUTO, "
+                            << (plan.empty() ? "nullptr" : "&plan") << ", " << ws << ", " << ws_bytes << "));\n";
                     }
                     return lu;
                 }
@@ -218,11 +258,11 @@ namespace nnfusion
                 }
             };
 
-            class FusedQuantMLP : public HipLibEmitter
+            class FusedQuantMLP : public QuantLibEmitter
             {
             public:
                 explicit FusedQuantMLP(std::shared_ptr<KernelContext> ctx)
-                    : HipLibEmitter(ctx)
+                    : QuantLibEmitter(ctx)
                 {
                 }
 
@@ -241,11 +281,16 @@ namespace nnfusion
                     const size_t ws_bytes = nnf::workspace::fused_mlp_w4a16((int)M, (int)H, (int)I, group);
                     // the only intermediate that reaches HBM: h [M, I] fp16 (plus M row statistics)
                     auto ws = allocate_tensor(Shape{ws_bytes}, element::character);
+                    // either product on the tile GEMM: in one launch each
+                    const std::string plan_gu = declare_sync_plan("gate_up_plan", (int)M, (int)I, (int)H, true, true);
+                    const std::string plan_d = declare_sync_plan("down_plan", (int)M, (int)H, (int)I, false, false);
                     LanguageUnit_p lu(new LanguageUnit(get_function_name()));
-                    *lu << "NNF_HIP_CHECK(nnf_fused_mlp_w4a16(stream, input0, input1, "
+                    *lu << plan_gu << plan_d;
+                    *lu << "NNF_HIP_CHECK(nnf_fused_mlp_w4a16_planned(stream, input0, input1, "
                         << float_literal(cfg["rms_eps"].get<double>()) << ", input2, input3, input4, input5, output0, " << M
-                        << ", " << H << ", " << I << ", " << group << ", " << zp << ", " << ws->get_name() << ", "
-                        << ws_bytes << "));\n";
+                        << ", " << H << ", " << I << ", " << group << ", " << zp << ", "
+                        << (plan_gu.empty() ? "nullptr" : "&gate_up_plan") << ", " << (plan_d.empty() ? "nullptr" : "&down_plan")
+                        << ", " << ws->get_name() << ", " << ws_bytes << "));\n";
                     return lu;
                 }
             };

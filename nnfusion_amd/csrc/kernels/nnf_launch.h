@@ -132,6 +132,21 @@ namespace nnf
                                  const void* residual, int act, void* rms_ws, void* partial_ws, int num_cu,
                                  const LaunchChoice& choice = LaunchChoice());
 
+    // ---- the nodes around a product as kernels of their own (elementwise.hip, w4a16_gemm.hip) --------------------------
+    enum ElementwiseOp { EW_ADD = 0, EW_MULTIPLY = 1, EW_SIGMOID = 2, EW_SWISH = 3 }; // values of nnf_elementwise_op
+    // y[r, c] = fp16(op(a[r, c], b[r, c] or (b_is_row) b[c])), fp32 arithmetic; unary operators ignore b
+    hipError_t launch_elementwise(hipStream_t stream, int op, const void* a, const void* b, void* y, long long rows, int cols,
+                                  bool b_is_row);
+    // W fp16 [N, K] = fp16((q - z) * s): bits 4 / 8, groups of 2^group_shift, zero_points (or null: zp) as nnf_wna16_gemm takes them
+    hipError_t launch_dequantize(hipStream_t stream, const void* Wq, const void* S, const void* zero_points, void* W, int N, int K,
+                                 int bits, int group_shift, int zp);
+    // Xn fp16 [M, K] = fp16(x * rsqrt(mean_k(x^2) + eps) * gamma[k]); K a multiple of 8
+    hipError_t launch_rms_norm(hipStream_t stream, const void* X, const void* gamma, void* Xn, int M, int K, float eps);
+    // Y [M, N] = fp16(SiLU(T[m, n]) * T[m, N + n]) from T fp16 [M, 2N]
+    hipError_t launch_silu_gate(hipStream_t stream, const void* T, void* Y, int M, int N);
+    // Y [M, N] = fp16(fp16(T + bias[n]) + residual[m, n]) (either may be null); T and residual may be Y
+    hipError_t launch_bias_residual(hipStream_t stream, const void* T, void* Y, const void* bias, const void* residual, int M, int N);
+
     // fp16 activations x 4- or 8-bit weights, groups of 32 / 64 / 128, a scalar zero point or one per (row, group)
     // (zero_points: u8 [N, ceil(K/group * bits / 8)], 4-bit ones two to a byte, even group low): wna16_generic.hip
     bool wna16_supported(int M, int N, int K, int bits, int group);

@@ -314,3 +314,51 @@ extern "C" int nnf_probe_mfma(int kind, int mode, int iters, int num_cu, double*
     *shader_mhz = clocks[1] ? (double)clocks[0] / (double)clocks[1] * 100.0 : 0.0;
     return (int)hipGetLastError();
 }
+
+// ---- where a launch of the tile GEMM spends its time ------------------------------------------------------------------
+// The product's own kernel (w4a16_gemm_sk.h), compiled here once more with time stamps (NNF_SK_TRACE): the plain product
+// on 128-row tiles of 128 or 256 columns, in its one-launch form.  trace: 16 x grid 64-bit stamps of the 100 MHz clock
+// (0 start, 1 first operands arrived, 2 K loop of the last segment over, 3 parked, 4 counted in, 5 / 7 wait for the
+// first / last tile's other workgroups over, 6 / 8 share of that tile finished, 9 end).  Returns the grid, or -1.
+#define NNF_SK_TRACE 1
+#include "../nnf_workspace.h"
+#include "w4a16_gemm_sk.h"
+
+extern "C" int nnf_probe_gemm_timeline(void* stream, const void* A, const void* Wq, const void* S, void* Y, int M, int N, int K,
+                                       int tile_cols, void* workspace, size_t workspace_bytes, void* sync, size_t sync_bytes,
+                                       unsigned long long* trace, int num_cu)
+{
+    using namespace nnf;
+    const workspace::SkPlan plan = workspace::plan_w4a16_sk(M, N, K, false, num_cu, 128, 0, tile_cols);
+    if (plan.tile_rows != 128 || plan.bytes() > workspace_bytes || plan.sync_bytes() > sync_bytes || (K & 255))
+        return -1;
+    SkGemmParams p = {};
+    p.A = (const half_t*)A;
+    p.Wq = (const uint8_t*)Wq;
+    p.S = (const half_t*)S;
+    p.Y = (half_t*)Y;
+    p.M = M, p.N = N, p.K = K, p.zp = 8, p.ldy = N, p.up_row_offset = N;
+    p.partial = plan.slots ? (float*)workspace : nullptr;
+    p.partial_bytes = plan.bytes();
+    p.tiles_m = plan.tiles_m, p.tiles_n = plan.tiles_n, p.supersteps = plan.supersteps, p.units = plan.units;
+    p.sync = plan.slots ? (uint32_t*)sync : nullptr;
+    p.spin_limit = 1 << 13;
+    p.trace = trace;
+    if (plan.tile_weight_rows == 128)
+    {
+        using T = gemm_sk::Tile<4, 1>;
+        auto kernel = &w4a16_gemm_sk_kernel<4, 1, false, false, false, false>;
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, T::LDS_BYTES) != hipSuccess)
+            return -1;
+        hipLaunchKernelGGL(kernel, dim3(plan.grid), dim3(gemm_sk::THREADS), T::LDS_BYTES, (hipStream_t)stream, p);
+    }
+    else
+    {
+        using T = gemm_sk::Tile<4, 2>;
+        auto kernel = &w4a16_gemm_sk_kernel<4, 2, false, false, false, false>;
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, T::LDS_BYTES) != hipSuccess)
+            return -1;
+        hipLaunchKernelGGL(kernel, dim3(plan.grid), dim3(gemm_sk::THREADS), T::LDS_BYTES, (hipStream_t)stream, p);
+    }
+    return hipGetLastError() == hipSuccess ? plan.grid : -1;
+}

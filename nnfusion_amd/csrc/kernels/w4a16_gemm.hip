@@ -269,6 +269,7 @@ namespace nnf
         void set_sync(SkGemmParams& p, const workspace::SkPlan& plan, const LaunchChoice& choice)
         {
             p.partial_bytes = plan.bytes();
+            p.trace = nullptr;
             // (the one-launch form addresses the parked tiles with 32-bit byte offsets)
             const bool one_launch = plan.slots && choice.sync_flags && choice.sync_bytes >= plan.sync_bytes() && plan.bytes() < ((size_t)1 << 32);
             p.sync = one_launch ? (uint32_t*)choice.sync_flags : nullptr;
@@ -403,6 +404,23 @@ namespace nnf
         case 64: return launch_gemm_sk_64(stream, p, plan.grid, gate);
         default: return launch_gemm_sk_32(stream, p, plan.grid, gate);
         }
+    }
+
+    hipError_t launch_rms_norm(hipStream_t stream, const void* X, const void* gamma, void* Xn, int M, int K, float eps)
+    {
+        hipLaunchKernelGGL(rms_norm_kernel, dim3(M), dim3(256), 0, stream, (const half_t*)X, (const half_t*)gamma, (half_t*)Xn, M, K, eps);
+        return hipGetLastError();
+    }
+    hipError_t launch_silu_gate(hipStream_t stream, const void* T, void* Y, int M, int N)
+    {
+        hipLaunchKernelGGL(skinny_silu_gate_kernel, dim3((M * N + 255) / 256), dim3(256), 0, stream, (const half_t*)T, (half_t*)Y, M, N);
+        return hipGetLastError();
+    }
+    hipError_t launch_bias_residual(hipStream_t stream, const void* T, void* Y, const void* bias, const void* residual, int M, int N)
+    {
+        hipLaunchKernelGGL(skinny_bias_residual_kernel, dim3((M * N + 255) / 256), dim3(256), 0, stream, (const half_t*)T, (half_t*)Y,
+                           (const half_t*)bias, (const half_t*)residual, M, N);
+        return hipGetLastError();
     }
 
     hipError_t launch_wna16_reduce(hipStream_t stream, const float* partial, int ranges, void* Y, int M, int N)

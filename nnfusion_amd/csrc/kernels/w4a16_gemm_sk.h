@@ -79,7 +79,25 @@ namespace nnf
         // second launch follows.
         uint32_t* sync;
         int spin_limit;         // polls of a tile's arrival count before a workgroup leaves its share to the last arriver
+        // NNF_SK_TRACE builds only (the measurement probes): 16 time stamps of the 100 MHz clock per workgroup, or null
+        unsigned long long* trace;
     };
+
+    // Time stamps inside the GEMM kernel for the measurement probes: compiled in only with NNF_SK_TRACE (the product
+    // library is built without it).  Stamp i of workgroup v: thread 0, SkGemmParams::trace[16 v + i].
+#ifdef NNF_SK_TRACE
+#define NNF_SK_STAMP(i)                                                                                                 \
+    do                                                                                                                  \
+    {                                                                                                                   \
+        if (p.trace && threadIdx.x == 0)                                                                                \
+            p.trace[(size_t)v * 16 + (i)] = __builtin_amdgcn_s_memrealtime();                                          \
+    } while (0)
+#else
+#define NNF_SK_STAMP(i)                                                                                                 \
+    do                                                                                                                  \
+    {                                                                                                                   \
+    } while (0)
+#endif
 
     namespace gemm_sk
     {
@@ -502,6 +520,7 @@ namespace nnf
             v = (xcd < full) ? xcd * per_xcd + idx : full * per_xcd + (xcd - full) * (per_xcd - 1) + idx;
         }
         const long long u_begin = first_unit_of(v, p.units, grid), u_end = first_unit_of(v + 1, p.units, grid);
+        NNF_SK_STAMP(0); // the workgroup runs
 
         // (q - zp) from (1024 + q_even, 64 + q_odd): exact
         const half2_t dq_add = half2_t{(half_t)(-(1024.0f + (float)p.zp)), (half_t)(-(64.0f + (float)p.zp))};
@@ -909,6 +928,8 @@ namespace nnf
             __builtin_amdgcn_s_waitcnt(vmcnt_imm(SCH::a_loads_total() + SCH::a_loads_at(0))); // step 0 and superstep 0 have landed
             workgroup_barrier();
             __builtin_amdgcn_sched_barrier(0);
+            if (first_of_mine)
+                NNF_SK_STAMP(1); // the first operands have arrived
             prepare_scales(I0{}, 0);
             if constexpr (RMS)
                 unroll_for<0, 4>([&](auto g_c) { lds_read_b128_nowait<decltype(g_c)::value * 16>(gm[decltype(g_c)::value], g_rd); });
@@ -970,6 +991,8 @@ namespace nnf
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); // the fragments read ahead for a step that does not exist
             __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));          // nothing may land in LDS or in registers any more ...
             __syncthreads();                                   // ... from any wavefront: the ring is free
+            if (u >= u_end)
+                NNF_SK_STAMP(2); // the K loop of the last segment is over
 
             // ---- a tile shared with other workgroups: park the sums in register order (element block q of MFMA tile
             // (i, j) of all 256 threads is one contiguous 4 KiB); w4a16_gemm_sk_fixup_kernel adds the parts and finishes
@@ -999,9 +1022,13 @@ namespace nnf
                     // every wavefront's part has arrived where every CU sees it before thread 0 counts the workgroup in
                     wait_vector_memory();
                     __syncthreads();
+                    if (u >= u_end)
+                        NNF_SK_STAMP(3); // its part is parked
                     uint32_t old = 0u;
                     if (tid == 0)
                         old = atomicAdd(p.sync + 2 * (size_t)tile, 1u);
+                    if (u >= u_end)
+                        NNF_SK_STAMP(4 + (old & 0u)); // ... and counted in
                     if (first_of_mine)
                         pend_tile[0] = tile, pend_old[0] = old;
                     else
@@ -1058,6 +1085,7 @@ namespace nnf
                 }
                 __syncthreads();
                 const uint32_t blocks = sync_note;
+                NNF_SK_STAMP(5 + 2 * slot); // the wait for the tile's other workgroups is over
                 if (blocks)
                 {
                     // (every part was complete at device scope before its workgroup counted itself in, the count was read
@@ -1068,6 +1096,7 @@ namespace nnf
                                                                                wave, lane);
                 }
                 __syncthreads(); // sync_note is read; (blocks) every wavefront's strips are finished
+                NNF_SK_STAMP(6 + 2 * slot); // its share of the tile is finished
                 if (blocks && tid == 0)
                 {
                     const uint32_t n = (uint32_t)__builtin_popcount(blocks);
@@ -1080,6 +1109,7 @@ namespace nnf
                 }
             }
         }
+        NNF_SK_STAMP(9); // done
     }
 
     // Adds the parts of the tiles that several workgroups of w4a16_gemm_sk_kernel worked on, in K order (so the result

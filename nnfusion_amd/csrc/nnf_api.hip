@@ -313,6 +313,111 @@ int nnf_wna16_gemm(nnf_stream_t stream, const void* A, const void* Wq, const voi
                                           q->zero_points, dev.num_cu);
 }
 
+// ---- the nodes around a product as calls of their own ------------------------------------------------------------------
+int nnf_elementwise_f16(nnf_stream_t stream, int op, const void* a, const void* b, void* y, size_t rows, int cols, int b_is_row)
+{
+    if (op < NNF_EW_ADD || op > NNF_EW_SWISH || !a || !y || rows == 0 || cols <= 0)
+        return NNF_ERR_INVALID_ARGUMENT;
+    const bool binary = op == NNF_EW_ADD || op == NNF_EW_MULTIPLY;
+    if (binary && !b)
+        return NNF_ERR_INVALID_ARGUMENT;
+    if (rows > ((size_t)1 << 40) / (size_t)cols)
+        return NNF_ERR_UNSUPPORTED_SHAPE;
+    return (int)nnf::launch_elementwise((hipStream_t)stream, op, a, binary ? b : a, y, (long long)rows, cols, binary && b_is_row != 0);
+}
+
+int nnf_rms_norm_f16(nnf_stream_t stream, const void* x, const void* gamma, void* y, int M, int K, float eps)
+{
+    if (!x || !gamma || !y || M <= 0 || K <= 0 || !aligned16(x) || !aligned16(gamma) || !aligned16(y))
+        return NNF_ERR_INVALID_ARGUMENT;
+    if (K % 8 != 0)
+        return NNF_ERR_UNSUPPORTED_SHAPE;
+    return (int)nnf::launch_rms_norm((hipStream_t)stream, x, gamma, y, M, K, eps);
+}
+
+int nnf_dequantize_f16(nnf_stream_t stream, const void* Wq, const void* scales, void* W, int N, int K, const nnf_quant* q)
+{
+    if (!Wq || !scales || !W || !q || N <= 0 || K <= 0 || !aligned16(Wq) || !aligned16(W))
+        return NNF_ERR_INVALID_ARGUMENT;
+    if ((q->bits != 4 && q->bits != 8) || (q->group != 32 && q->group != 64 && q->group != 128) || K % q->group != 0 ||
+        q->zero_point < 0 || q->zero_point >= (1 << q->bits))
+        return NNF_ERR_UNSUPPORTED_SHAPE;
+    return (int)nnf::launch_dequantize((hipStream_t)stream, Wq, scales, q->zero_points, W, N, K, q->bits, group_shift_of(q->group),
+                                       q->zero_point);
+}
+
+// The fused product with other block parameters: the plain product between the kernels of the nodes around it, as the
+// unfused graph would run them.  workspace = [ RMSNorm(A): M x K fp16 ][ product: M x rows fp16 ][ the product's own ]
+namespace
+{
+    struct QFusedLayout
+    {
+        size_t xn = 0, product = 0, gemm = 0;
+        size_t total() const { return xn + product + gemm; }
+    };
+    QFusedLayout q_fused_layout(int M, int N, int K, const nnf_quant* q, bool rms, bool gate, bool through_scratch)
+    {
+        QFusedLayout l;
+        const int rows = gate ? 2 * N : N;
+        l.xn = rms ? nnf::workspace::align256((size_t)M * K * 2) : 0;
+        l.product = (gate || through_scratch) ? nnf::workspace::align256((size_t)M * rows * 2) : 0;
+        l.gemm = nnf::workspace::align256(nnf_wna16_gemm_workspace_bytes(M, rows, K, q));
+        return l;
+    }
+} // namespace
+
+size_t nnf_wna16_gemm_fused_workspace_bytes(int M, int N, int K, const nnf_quant* q, int act)
+{
+    if (!q || M <= 0 || N <= 0 || K <= 0)
+        return 0;
+    if (is_plain_w4a16(q))
+        return nnf::workspace::w4a16_gemm_fused(M, N, K, q->group, act);
+    return q_fused_layout(M, N, K, q, true, act == NNF_ACT_SILU_GATE, true).total();
+}
+
+int nnf_wna16_gemm_fused(nnf_stream_t stream, const void* A, const void* Wq, const void* scales, void* Y, int M, int N, int K,
+                         const nnf_quant* q, const void* rms_gamma, float rms_eps, const void* bias, const void* residual, int act,
+                         void* workspace, size_t workspace_bytes)
+{
+    if (!q)
+        return NNF_ERR_INVALID_ARGUMENT;
+    if (is_plain_w4a16(q))
+        return nnf_w4a16_gemm_fused(stream, A, Wq, scales, Y, M, N, K, q->group, q->zero_point, rms_gamma, rms_eps, bias, residual, act,
+                                    workspace, workspace_bytes);
+    if (!A || !Wq || !scales || !Y || M <= 0 || N <= 0 || K <= 0 || (act != NNF_ACT_NONE && act != NNF_ACT_SILU_GATE))
+        return NNF_ERR_INVALID_ARGUMENT;
+    if ((rms_gamma && !aligned16(rms_gamma)) || (bias && !aligned16(bias)) || (residual && !aligned16(residual)))
+        return NNF_ERR_INVALID_ARGUMENT;
+    const bool gate = act == NNF_ACT_SILU_GATE, rms = rms_gamma != nullptr;
+    if ((gate && (bias || residual)) || (rms && K % 8 != 0))
+        return NNF_ERR_UNSUPPORTED_SHAPE;
+    const int rows = gate ? 2 * N : N;
+    if (!nnf_wna16_supported(M, rows, K, q))
+        return NNF_ERR_UNSUPPORTED_SHAPE;
+    // a residual that is the output buffer itself must not be overwritten by the product
+    const QFusedLayout l = q_fused_layout(M, N, K, q, rms, gate, residual == Y);
+    if (l.total() > 0 && (!workspace || !aligned16(workspace) || workspace_bytes < l.total()))
+        return NNF_ERR_WORKSPACE_TOO_SMALL;
+    uint8_t* ws = (uint8_t*)workspace;
+    const hipStream_t s = (hipStream_t)stream;
+    if (rms)
+    {
+        const hipError_t e = nnf::launch_rms_norm(s, A, rms_gamma, ws, M, K, rms_eps);
+        if (e != hipSuccess)
+            return (int)e;
+        A = ws;
+    }
+    void* product = l.product ? (void*)(ws + l.xn) : Y;
+    const int st = nnf_wna16_gemm(stream, A, Wq, scales, product, M, rows, K, q, l.gemm ? ws + l.xn + l.product : nullptr, l.gemm);
+    if (st != NNF_OK)
+        return st;
+    if (gate)
+        return (int)nnf::launch_silu_gate(s, product, Y, M, N);
+    if (bias || residual)
+        return (int)nnf::launch_bias_residual(s, product, Y, bias, residual, M, N);
+    return NNF_OK;
+}
+
 int nnf_w4a16_variant_supported(int M, int N, int K, int group, int variant)
 {
     return (group == 128 && nnf::workspace::w4a16_variant_fits(M, N, K, variant)) ? 1 : 0;
@@ -532,6 +637,60 @@ int nnf_fused_mlp_w4a16_planned(nnf_stream_t stream, const void* x, const void* 
     e = nnf::launch_w4a16_gemm((hipStream_t)stream, h, Wd, Sd, out, M, H, I, zp, nullptr, 0.f, nullptr, x, NNF_ACT_NONE,
                                nullptr, partial, dev.num_cu, choice_d);
     return (int)e;
+}
+
+// workspace = [ RMSNorm(x): M x H fp16 ][ gate | up products: M x 2I fp16, then the down product: M x H fp16 ][ h: M x I fp16 ]
+//             [ the products' own ]
+size_t nnf_fused_mlp_wna16_workspace_bytes(int M, int H, int I, const nnf_quant* q_gate_up, const nnf_quant* q_down)
+{
+    if (!q_gate_up || !q_down || M <= 0 || H <= 0 || I <= 0)
+        return 0;
+    if (is_plain_w4a16(q_gate_up) && is_plain_w4a16(q_down) && q_gate_up->zero_point == q_down->zero_point)
+        return nnf::workspace::fused_mlp_w4a16(M, H, I, 128);
+    const size_t a = nnf_wna16_gemm_workspace_bytes(M, 2 * I, H, q_gate_up), b = nnf_wna16_gemm_workspace_bytes(M, H, I, q_down);
+    const size_t wide = (size_t)(2 * I > H ? 2 * I : H);
+    return nnf::workspace::align256((size_t)M * H * 2) + nnf::workspace::align256((size_t)M * wide * 2) +
+           nnf::workspace::align256((size_t)M * I * 2) + nnf::workspace::align256(a > b ? a : b);
+}
+
+int nnf_fused_mlp_wna16(nnf_stream_t stream, const void* x, const void* gamma, float eps, const void* Wgu, const void* Sgu,
+                        const void* Wd, const void* Sd, void* out, int M, int H, int I, const nnf_quant* q_gate_up,
+                        const nnf_quant* q_down, void* workspace, size_t workspace_bytes)
+{
+    if (!q_gate_up || !q_down)
+        return NNF_ERR_INVALID_ARGUMENT;
+    if (is_plain_w4a16(q_gate_up) && is_plain_w4a16(q_down) && q_gate_up->zero_point == q_down->zero_point)
+        return nnf_fused_mlp_w4a16(stream, x, gamma, eps, Wgu, Sgu, Wd, Sd, out, M, H, I, 128, q_gate_up->zero_point, workspace,
+                                   workspace_bytes);
+    if (!x || !gamma || !Wgu || !Sgu || !Wd || !Sd || !out || M <= 0 || H <= 0 || I <= 0)
+        return NNF_ERR_INVALID_ARGUMENT;
+    if (!aligned16(x) || !aligned16(gamma) || !aligned16(out) || !aligned16(workspace))
+        return NNF_ERR_INVALID_ARGUMENT;
+    if (H % 8 != 0 || !nnf_wna16_supported(M, 2 * I, H, q_gate_up) || !nnf_wna16_supported(M, H, I, q_down))
+        return NNF_ERR_UNSUPPORTED_SHAPE;
+    if (!workspace || workspace_bytes < nnf_fused_mlp_wna16_workspace_bytes(M, H, I, q_gate_up, q_down))
+        return NNF_ERR_WORKSPACE_TOO_SMALL;
+    const size_t wide = (size_t)(2 * I > H ? 2 * I : H);
+    uint8_t* xn = (uint8_t*)workspace;
+    uint8_t* product = xn + nnf::workspace::align256((size_t)M * H * 2);
+    uint8_t* h = product + nnf::workspace::align256((size_t)M * wide * 2);
+    uint8_t* own = h + nnf::workspace::align256((size_t)M * I * 2);
+    const size_t own_bytes = workspace_bytes - (size_t)(own - xn);
+    const hipStream_t s = (hipStream_t)stream;
+    // the nodes of the block, one after the other, fp16 tensors between them
+    hipError_t e = nnf::launch_rms_norm(s, x, gamma, xn, M, H, eps);
+    if (e != hipSuccess)
+        return (int)e;
+    int st = nnf_wna16_gemm(stream, xn, Wgu, Sgu, product, M, 2 * I, H, q_gate_up, own, own_bytes);
+    if (st != NNF_OK)
+        return st;
+    e = nnf::launch_silu_gate(s, product, h, M, I);
+    if (e != hipSuccess)
+        return (int)e;
+    st = nnf_wna16_gemm(stream, h, Wd, Sd, product, M, H, I, q_down, own, own_bytes);
+    if (st != NNF_OK)
+        return st;
+    return (int)nnf::launch_bias_residual(s, product, out, nullptr, x, M, H); // out may be x
 }
 
 } // extern "C"

@@ -273,3 +273,79 @@ def fused_mlp_w4a16(x, gamma, wgu, sgu, wd, sd, eps=1e-6, group=128, zp=8, out=N
                                    sgu.data_ptr(), wd.data_ptr(), sd.data_ptr(), out.data_ptr(), m, h, i, group, zp,
                                    workspace.data_ptr(), workspace.numel()), "nnf_fused_mlp_w4a16")
     return out
+
+
+EW_OPS = {"add": 0, "multiply": 1, "sigmoid": 2, "swish": 3}
+
+
+def elementwise(op, a, b=None, out=None):
+    """y = op(a, b) over fp16 tensors (b of a's shape, or a row [cols] broadcast over a's leading axes)."""
+    lib = _lib.kernels()
+    assert a.dtype == torch.float16 and a.is_contiguous()
+    cols = a.shape[-1]
+    rows = a.numel() // cols
+    b_is_row = 0
+    if b is not None:
+        assert b.dtype == torch.float16 and b.is_contiguous()
+        b_is_row = 1 if (b.dim() == 1 and a.dim() > 1) else 0
+        assert b_is_row or b.shape == a.shape
+    if out is None:
+        out = torch.empty_like(a)
+    _check(lib.nnf_elementwise_f16(_stream(), EW_OPS[op], a.data_ptr(), _p(b), out.data_ptr(), rows, cols, b_is_row),
+           "nnf_elementwise_f16")
+    return out
+
+
+def rms_norm(x, gamma, eps=1e-6, out=None):
+    lib = _lib.kernels()
+    m, k = x.shape
+    if out is None:
+        out = torch.empty_like(x)
+    _check(lib.nnf_rms_norm_f16(_stream(), x.data_ptr(), gamma.data_ptr(), out.data_ptr(), m, k, float(eps)), "nnf_rms_norm_f16")
+    return out
+
+
+def dequantize(wq, scales, bits=4, group=128, zp=8, zero_points=None, out=None):
+    """W fp16 [N, K] = (q - z) * s per block of `group` weights."""
+    lib = _lib.kernels()
+    n = wq.shape[0]
+    k = wq.shape[1] * 8 // bits
+    if out is None:
+        out = torch.empty((n, k), dtype=torch.float16, device=wq.device)
+    keep, qp = _quant_arg(bits, group, zp, zero_points)
+    _check(lib.nnf_dequantize_f16(_stream(), wq.data_ptr(), scales.data_ptr(), out.data_ptr(), n, k, qp), "nnf_dequantize_f16")
+    return out
+
+
+def wna16_gemm_fused(a, wq, scales, bits=4, group=128, zp=8, zero_points=None, rms_gamma=None, rms_eps=1e-6, bias=None,
+                     residual=None, act=0, out=None, workspace=None):
+    """nnf_wna16_gemm_fused: the fused product for every block parameter."""
+    lib = _lib.kernels()
+    m, k = a.shape
+    n = wq.shape[0] // (2 if act == 1 else 1)
+    if out is None:
+        out = torch.empty((m, n), dtype=torch.float16, device=a.device)
+    keep, qp = _quant_arg(bits, group, zp, zero_points)
+    if workspace is None:
+        workspace = _ws(lib.nnf_wna16_gemm_fused_workspace_bytes(m, n, k, qp, int(act)), a.device)
+    _check(lib.nnf_wna16_gemm_fused(_stream(), a.data_ptr(), wq.data_ptr(), scales.data_ptr(), out.data_ptr(), m, n, k, qp,
+                                    _p(rms_gamma), float(rms_eps), _p(bias), _p(residual), int(act), workspace.data_ptr(),
+                                    workspace.numel()), "nnf_wna16_gemm_fused")
+    return out
+
+
+def fused_mlp_wna16(x, gamma, wgu, sgu, wd, sd, bits=4, group=128, zp=8, zgu=None, zd=None, eps=1e-6, out=None, workspace=None):
+    """The MLP block for every block parameter (zgu / zd: zero-point tensors of the two weight matrices, or None)."""
+    lib = _lib.kernels()
+    m, h = x.shape
+    i = wgu.shape[0] // 2
+    if out is None:
+        out = torch.empty((m, h), dtype=torch.float16, device=x.device)
+    keep_a, qa = _quant_arg(bits, group, zp, zgu)
+    keep_b, qb = _quant_arg(bits, group, zp, zd)
+    if workspace is None:
+        workspace = _ws(lib.nnf_fused_mlp_wna16_workspace_bytes(m, h, i, qa, qb), x.device)
+    _check(lib.nnf_fused_mlp_wna16(_stream(), x.data_ptr(), gamma.data_ptr(), float(eps), wgu.data_ptr(), sgu.data_ptr(),
+                                   wd.data_ptr(), sd.data_ptr(), out.data_ptr(), m, h, i, qa, qb, workspace.data_ptr(),
+                                   workspace.numel()), "nnf_fused_mlp_wna16")
+    return out

@@ -358,11 +358,16 @@ int main(int argc, char** argv)
         auto n2 = quant_dot_graph(g2, 256, 4096, 4096, "{\"rms_norm\": true, \"has_bias\": true, \"rms_eps\": 1e-5}", true, true);
         auto k2 = sel.pick_first(n2, ROCM_GPU).second;
         auto fu2 = k2->get_or_emit_source();
-        CONTAINS(fu2->body_unit->get_code(), "nnf_w4a16_gemm_fused(stream, input0, input1, input2, output0, 256, 4096, 4096, 128, 8, input3, 1.000000000e-05f, input4, nullptr, NNF_ACT_NONE, ");
-        EXPECT(k2->m_context->tensors.size() == 1 &&
+        CONTAINS(fu2->body_unit->get_code(), "nnf_w4a16_gemm_fused_variant(stream, input0, input1, input2, output0, 256, 4096, 4096, 128, 8, input3, 1.000000000e-05f, input4, nullptr, NNF_ACT_NONE, NNF_W4A16_AUTO, &plan, ");
+        // ... and, because the product runs on the tile GEMM, a second tensor: its synchronisation words (two per tile:
+        // 2 x 16 tiles), persistent and cleared at initialisation, named by the nnf_plan the body declares
+        EXPECT(k2->m_context->tensors.size() == 2 &&
                k2->m_context->tensors[0]->size() == (size_t)256 * 4 + (size_t)256 * 128 * 256 * 4);
+        EXPECT(k2->m_context->tensors[1]->size() == 256 && k2->m_context->tensors[1]->is_persistent() &&
+               k2->m_context->tensors[1]->is_memset() && k2->m_context->tensors[1]->get_memset_value() == 0);
+        CONTAINS(fu2->body_unit->get_code(), "const nnf_plan plan = {0, 0, 0, " + k2->m_context->tensors[1]->get_name() + ", 256, 0};");
         CONTAINS(fu2->signature_unit->get_code(), "char* " + k2->m_context->tensors[0]->get_name());
-        CONTAINS(fu2->call_unit->get_code(), k2->m_context->tensors[0]->get_name() + ");");
+        CONTAINS(fu2->call_unit->get_code(), k2->m_context->tensors[1]->get_name() + ");");
         // SiLU gate: N is half the weight rows
         graph::Graph g3;
         auto n3 = quant_dot_graph(g3, 256, 11008, 4096, "{\"act\": \"silu_gate\"}", false, false, false, 2);
@@ -435,13 +440,16 @@ int main(int argc, char** argv)
         EXPECT(mlp->get_output_shape(0) == (Shape{256, 4096}));
         auto k = sel.pick_first(mlp, ROCM_GPU).second;
         auto fm = k->get_or_emit_source();
-        CONTAINS(fm->body_unit->get_code(), "nnf_fused_mlp_w4a16(stream, input0, input1, 1.000000000e-06f, input2, input3, input4, input5, output0, 256, 4096, 11008, 128, 8, ");
+        CONTAINS(fm->body_unit->get_code(), "nnf_fused_mlp_w4a16_planned(stream, input0, input1, 1.000000000e-06f, input2, input3, input4, input5, output0, 256, 4096, 11008, 128, 8, &gate_up_plan, &down_plan, ");
         // rstd [256] fp32 + h [256, 11008] fp16 + the larger of the two areas of parked sums: both GEMMs run 256
         // workgroups over tiles of 128 x 256 weight rows; gate/up (2 x 86 tiles x 16 supersteps) needs two slots per
         // workgroup
-        EXPECT(k->m_context->tensors.size() == 1 &&
+        // ... and the synchronisation words of either product (2 x 86 and 1 x 32 tiles, two words each)
+        EXPECT(k->m_context->tensors.size() == 3 &&
                k->m_context->tensors[0]->size() ==
                    (size_t)256 * 4 + (size_t)256 * 11008 * 2 + (size_t)2 * 256 * 128 * 256 * 4);
+        EXPECT(k->m_context->tensors[1]->size() == 1408 && k->m_context->tensors[2]->size() == 256 &&
+               k->m_context->tensors[1]->is_memset() && k->m_context->tensors[2]->is_memset());
     });
 
     run_case("codegen_project", [&] {

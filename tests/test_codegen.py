@@ -58,7 +58,7 @@ def test_onnx_front_door_imports_fuses_and_generates(tmp_path):
     subprocess.run([TOOL, "onnx", out, model], check=True, timeout=60)
     text = open(out + "nnfusion_rt.cpp").read()
     assert text.count("NNF_HIP_CHECK(nnf_") == 1
-    assert "nnf_fused_mlp_w4a16(stream, input0, input1," in text and ", 8, 256, 384, 128, 8, " in text
+    assert "nnf_fused_mlp_w4a16_planned(stream, input0, input1," in text and ", 8, 256, 384, 128, 8, " in text
     blobs = {os.path.getsize(out + "Constant/" + c): open(out + "Constant/" + c, "rb").read() for c in os.listdir(out + "Constant")}
     assert blobs[wgu.nbytes] == wgu.tobytes() and blobs[wd.nbytes] == wd.tobytes() and blobs[gamma.nbytes] == gamma.tobytes()
     assert blobs[sgu.nbytes] == sgu.tobytes()
