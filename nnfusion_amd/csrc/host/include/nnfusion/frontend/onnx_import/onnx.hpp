@@ -31,7 +31,8 @@ namespace nnfusion
             enum DataType
             {
                 UNDEFINED = 0, FLOAT = 1, UINT8 = 2, INT8 = 3, UINT16 = 4, INT16 = 5, INT32 = 6, INT64 = 7,
-                STRING = 8, BOOL = 9, FLOAT16 = 10, DOUBLE = 11, UINT32 = 12, UINT64 = 13
+                STRING = 8, BOOL = 9, FLOAT16 = 10, DOUBLE = 11, UINT32 = 12, UINT64 = 13,
+                UINT4 = 21, INT4 = 22 // two per byte in raw_data, the first element in the low nibble
             };
             struct Tensor
             {

@@ -10,6 +10,7 @@
 #include <cstring>
 #include <fstream>
 #include <iterator>
+#include <set>
 
 namespace nnfusion
 {
@@ -409,6 +410,8 @@ namespace nnfusion
                 }
             }
 
+            size_t type_bytes(int dt) { return dt == FLOAT16 ? 2 : dt == FLOAT ? 4 : 1; }
+
             // fp32 -> fp16 bits, round to nearest even (scales stored as fp32 in a model)
             uint16_t float_to_half_bits(float f)
             {
@@ -474,6 +477,45 @@ namespace nnfusion
                 return g->add_node_and_edge(std::make_shared<op::GenericOp>(name, type, config), in);
             };
 
+            // input i of node n as an fp16 row of `len` values: a value of the graph, or an initializer (fp16, or fp32 rounded)
+            auto half_row = [&](const Node& n, size_t i, size_t len) -> std::shared_ptr<graph::GNode> {
+                auto ti = init.find(n.inputs[i]);
+                if (ti == init.end() || ti->second->data_type == FLOAT16)
+                {
+                    auto v = input_of(n, i);
+                    NNFUSION_CHECK(shape_size(v->get_output_shape(0)) == len && v->get_output_element_type(0) == element::f16)
+                        << "onnx: " << n.op_type << " " << n.name << ": input " << i << " must be fp16 [" << len << "]";
+                    return v;
+                }
+                const Tensor& t = *ti->second;
+                NNFUSION_CHECK(t.data_type == FLOAT && t.bytes.size() == len * 4)
+                    << "onnx: " << n.op_type << " " << n.name << ": input " << i << " must be fp16 or fp32 [" << len << "]";
+                std::vector<uint16_t> h(len);
+                for (size_t j = 0; j < len; ++j)
+                {
+                    float f;
+                    memcpy(&f, t.bytes.data() + 4 * j, 4);
+                    h[j] = float_to_half_bits(f);
+                }
+                return g->add_node_and_edge(std::make_shared<op::Constant>(element::f16, Shape{len}, h.data()), graph::GNodeVector{});
+            };
+            // values produced by a DequantizeLinear of weights [K, N]: held as the Dequantize of the weights in the
+            // layout of the kernels, [N, K] -- a MatMul that reads one becomes a Dot with transpose_B
+            std::set<std::string> transposed_weights;
+            // element (r, c) of a 2-D initializer of 4- or 8-bit integers, as an unsigned value (signed types: + 2^(bits-1))
+            auto small_int_at = [](const Tensor& t, int bits, bool is_signed, size_t cols, size_t r, size_t c) -> int {
+                const size_t i = r * cols + c;
+                int v;
+                if (bits == 8)
+                    v = is_signed ? (int)(int8_t)t.bytes[i] + 128 : (int)t.bytes[i];
+                else
+                {
+                    const int nib = (t.bytes[i >> 1] >> (4 * (i & 1))) & 0xF;
+                    v = is_signed ? ((nib ^ 8) - 8) + 8 : nib; // sign-extend, then shift the range to 0 .. 15
+                }
+                return v;
+            };
+
             for (auto& n : model.nodes) // ONNX keeps nodes in topological order
             {
                 NNFUSION_CHECK(!n.outputs.empty()) << "onnx: node without outputs";
@@ -497,7 +539,7 @@ namespace nnfusion
                                    K % block == 0)
                         << "onnx: MatMulNBits " << n.name
                         << ": bits = 4 or 8 and block_size = 32, 64 or 128 (K a multiple of it) are supported";
-                    NNFUSION_CHECK(!has_input(n, 4) && !has_input(n, 5)) << "onnx: MatMulNBits with g_idx or bias is not supported";
+                    NNFUSION_CHECK(!has_input(n, 4)) << "onnx: MatMulNBits with g_idx is not supported";
                     auto wi = init.find(n.inputs.at(1));
                     auto si = init.find(n.inputs.at(2));
                     NNFUSION_CHECK(wi != init.end() && si != init.end()) << "onnx: MatMulNBits weights and scales must be initializers";
@@ -558,13 +600,117 @@ namespace nnfusion
                     }
                     auto s = g->add_node_and_edge(
                         std::make_shared<op::Constant>(element::f16, Shape{(size_t)N, (size_t)(K / block)}, sc.data()), graph::GNodeVector{});
+                    // input 5: a bias [N], added to every row: the product's own epilogue
+                    std::shared_ptr<graph::GNode> bias;
+                    if (has_input(n, 5))
+                        bias = half_row(n, 5, (size_t)N);
                     std::string attrs = "{\"bits\": " + std::to_string(bits) + ", \"group_size\": " + std::to_string(block) +
                                         ", \"zero_point\": " + std::to_string(zps ? 0 : zp) +
-                                        ", \"has_zero_points\": " + (zps ? "true" : "false") + "}";
+                                        ", \"has_zero_points\": " + (zps ? "true" : "false") +
+                                        ", \"has_bias\": " + (bias ? "true" : "false") + "}";
                     graph::GNodeVector ins = {input_of(n, 0), wq, s};
                     if (zps)
                         ins.push_back(zps);
+                    if (bias)
+                        ins.push_back(bias);
                     out = generic(n, "QuantDot", ins, attrs);
+                }
+                else if (n.op_type == "DequantizeLinear")
+                {
+                    // Blocked dequantisation of a weight matrix W [K, N] (the B operand of a MatMul): axis = 0,
+                    // block_size = 32 / 64 / 128 along K, x_scale [K / block, N], optional x_zero_point of x's type and
+                    // x_scale's shape; y = (x - zero point) * scale.  4-bit types two per byte, first element low.  Signed
+                    // types are shifted to unsigned ones with the zero point (q + 2^(bits-1), z + 2^(bits-1)).
+                    auto xi = init.find(n.inputs.at(0));
+                    auto si = init.find(n.inputs.at(1));
+                    NNFUSION_CHECK(xi != init.end() && si != init.end())
+                        << "onnx: DequantizeLinear " << n.name << ": only quantized weights (initializers) are supported";
+                    const Tensor& xt = *xi->second;
+                    const Tensor& st = *si->second;
+                    const int dt = xt.data_type;
+                    NNFUSION_CHECK(dt == UINT8 || dt == INT8 || dt == UINT4 || dt == INT4)
+                        << "onnx: DequantizeLinear " << n.name << ": weights must be (u)int8 or (u)int4";
+                    const int bits = (dt == UINT8 || dt == INT8) ? 8 : 4;
+                    const bool is_signed = dt == INT8 || dt == INT4;
+                    const int64_t block = n.get_int("block_size", 0), axis = n.get_int("axis", 1);
+                    NNFUSION_CHECK(xt.dims.size() == 2 && (axis == 0 || axis == -2) && (block == 32 || block == 64 || block == 128) &&
+                                   xt.dims[0] % block == 0)
+                        << "onnx: DequantizeLinear " << n.name
+                        << ": a weight matrix [K, N] with axis = 0 and block_size = 32, 64 or 128 (K a multiple of it) is supported";
+                    const size_t K = (size_t)xt.dims[0], N = (size_t)xt.dims[1], G = K / (size_t)block;
+                    NNFUSION_CHECK(xt.bytes.size() == (K * N * bits + 7) / 8) << "onnx: DequantizeLinear " << n.name << ": wrong data size";
+                    NNFUSION_CHECK(st.dims.size() == 2 && (size_t)st.dims[0] == G && (size_t)st.dims[1] == N &&
+                                   (st.data_type == FLOAT16 || st.data_type == FLOAT) && st.bytes.size() == G * N * type_bytes(st.data_type))
+                        << "onnx: DequantizeLinear " << n.name << ": scales must be fp16 or fp32 [K / block_size, N]";
+                    // weights -> [N, K * bits / 8], packed along K (4 bits: even k in the low nibble)
+                    std::vector<uint8_t> wq(N * K * bits / 8, 0);
+                    for (size_t k = 0; k < K; ++k)
+                        for (size_t c = 0; c < N; ++c)
+                        {
+                            const int v = small_int_at(xt, bits, is_signed, N, k, c);
+                            if (bits == 8)
+                                wq[c * K + k] = (uint8_t)v;
+                            else
+                                wq[c * (K / 2) + k / 2] |= (uint8_t)(v << (4 * (k & 1)));
+                        }
+                    // scales -> fp16 [N, K / block]
+                    std::vector<uint16_t> sc(N * G);
+                    for (size_t b = 0; b < G; ++b)
+                        for (size_t c = 0; c < N; ++c)
+                        {
+                            if (st.data_type == FLOAT16)
+                                memcpy(&sc[c * G + b], st.bytes.data() + 2 * (b * N + c), 2);
+                            else
+                            {
+                                float f;
+                                memcpy(&f, st.bytes.data() + 4 * (b * N + c), 4);
+                                sc[c * G + b] = float_to_half_bits(f);
+                            }
+                        }
+                    // zero points: one value everywhere is the scalar attribute, otherwise u8 [N, ceil(G * bits / 8)]
+                    int zp = is_signed ? (1 << (bits - 1)) : 0;
+                    std::vector<uint8_t> zq;
+                    bool uniform = true;
+                    if (has_input(n, 2))
+                    {
+                        auto zi = init.find(n.inputs[2]);
+                        NNFUSION_CHECK(zi != init.end() && zi->second->data_type == dt && zi->second->dims.size() == 2 &&
+                                       (size_t)zi->second->dims[0] == G && (size_t)zi->second->dims[1] == N &&
+                                       zi->second->bytes.size() == (G * N * bits + 7) / 8)
+                            << "onnx: DequantizeLinear " << n.name << ": zero points must have the weights' type and the scales' shape";
+                        const Tensor& zt = *zi->second;
+                        const size_t z_stride = (G * bits + 7) / 8;
+                        zq.assign(N * z_stride, 0);
+                        zp = small_int_at(zt, bits, is_signed, N, 0, 0);
+                        for (size_t b = 0; b < G; ++b)
+                            for (size_t c = 0; c < N; ++c)
+                            {
+                                const int v = small_int_at(zt, bits, is_signed, N, b, c);
+                                uniform = uniform && v == zp;
+                                if (bits == 8)
+                                    zq[c * z_stride + b] = (uint8_t)v;
+                                else
+                                    zq[c * z_stride + b / 2] |= (uint8_t)(v << (4 * (b & 1)));
+                            }
+                    }
+                    graph::GNodeVector ins = {
+                        g->add_node_and_edge(std::make_shared<op::Constant>(element::u8, Shape{N, K * bits / 8}, wq.data()), graph::GNodeVector{}),
+                        g->add_node_and_edge(std::make_shared<op::Constant>(element::f16, Shape{N, G}, sc.data()), graph::GNodeVector{})};
+                    const bool has_z = !zq.empty() && !uniform;
+                    if (has_z)
+                        ins.push_back(g->add_node_and_edge(
+                            std::make_shared<op::Constant>(element::u8, Shape{N, (G * bits + 7) / 8}, zq.data()), graph::GNodeVector{}));
+                    const std::string attrs = "{\"bits\": " + std::to_string(bits) + ", \"group_size\": " + std::to_string(block) +
+                                              ", \"zero_point\": " + std::to_string(has_z ? 0 : zp) +
+                                              ", \"has_zero_points\": " + (has_z ? "true" : "false") + "}";
+                    out = generic(n, "Dequantize", ins, attrs);
+                    transposed_weights.insert(n.outputs[0]);
+                }
+                else if (n.op_type == "MatMul")
+                {
+                    // (a Dot of two fp16 values has no kernel in this library: the fold into QuantDot is what makes it run)
+                    const bool tb = transposed_weights.count(n.inputs.at(1)) != 0;
+                    out = generic(n, "Dot", {input_of(n, 0), input_of(n, 1)}, std::string("{\"transpose_B\": ") + (tb ? "true" : "false") + "}");
                 }
                 else if (n.op_type == "SimplifiedLayerNormalization" || n.op_type == "RMSNormalization")
                 {

@@ -99,20 +99,39 @@ namespace nnfusion
                         return nullptr;
                     if (bits != 4 || group != 128 || has_z)
                     {
-                        // other block parameters: the plain product only (nnf_wna16_gemm); scratch memory for the tile
-                        // GEMM of 4-bit weights
-                        if (rms || has_bias || has_res || gate || (bits != 4 && bits != 8) ||
-                            (group != 32 && group != 64 && group != 128) || K % group != 0)
+                        // other block parameters: nnf_wna16_gemm, and for the fused forms nnf_wna16_gemm_fused, which
+                        // runs the nodes around the product one after the other (RMSNorm and the product's fp16 output
+                        // through scratch memory)
+                        if ((bits != 4 && bits != 8) || (group != 32 && group != 64 && group != 128) || K % group != 0 ||
+                            (rms && K % 8 != 0))
                             return nullptr;
-                        const size_t q_ws_bytes = nnf::workspace::wna16_gemm((int)M, (int)N, (int)K, bits, group);
+                        const bool q_fused = rms || has_bias || has_res || gate;
+                        // (a residual may turn out to be the output buffer itself: room for the product either way)
+                        const size_t q_ws_bytes =
+                            q_fused ? nnf::workspace::wna16_fused_layout((int)M, (int)N, (int)K, bits, group, rms, gate, has_res).total()
+                                    : nnf::workspace::wna16_gemm((int)M, (int)N, (int)K, bits, group);
                         std::string q_ws = "nullptr";
                         if (q_ws_bytes > 0)
                             q_ws = allocate_tensor(Shape{q_ws_bytes}, element::character)->get_name();
+                        size_t qi = 3 + (has_z ? 1 : 0);
+                        std::string q_gamma = "nullptr", q_bias = "nullptr", q_res = "nullptr";
+                        if (rms)
+                            q_gamma = "input" + std::to_string(qi++);
+                        if (has_bias)
+                            q_bias = "input" + std::to_string(qi++);
+                        if (has_res)
+                            q_res = "input" + std::to_string(qi++);
                         LanguageUnit_p lu(new LanguageUnit(get_function_name()));
                         *lu << "const nnf_quant quant = {" << bits << ", " << group << ", " << zp << ", "
                             << (has_z ? "input3" : "nullptr") << "};\n";
-                        *lu << "NNF_HIP_CHECK(nnf_wna16_gemm(stream, input0, input1, input2, output0, " << M << ", " << N << ", "
-                            << K << ", &quant, " << q_ws << ", " << q_ws_bytes << "));\n";
+                        if (!q_fused)
+                            *lu << "NNF_HIP_CHECK(nnf_wna16_gemm(stream, input0, input1, input2, output0, " << M << ", " << N << ", "
+                                << K << ", &quant, " << q_ws << ", " << q_ws_bytes << "));\n";
+                        else
+                            *lu << "NNF_HIP_CHECK(nnf_wna16_gemm_fused(stream, input0, input1, input2, output0, " << M << ", " << N
+                                << ", " << K << ", &quant, " << q_gamma << ", " << float_literal(cfg["rms_eps"].get<double>()) << ", "
+                                << q_bias << ", " << q_res << ", " << (gate ? "NNF_ACT_SILU_GATE" : "NNF_ACT_NONE") << ", " << q_ws
+                                << ", " << q_ws_bytes << "));\n";
                         return lu;
                     }
                     if (K % 128 != 0)
@@ -276,7 +295,29 @@ namespace nnfusion
                     const int zp = cfg["zero_point"].get<int>();
                     const Shape& x = m_context->inputs[0]->get_shape();
                     const size_t M = x[0], H = x[1], I = m_context->inputs[2]->get_shape()[0] / 2;
-                    if (group != 128 || H % 128 != 0 || I % 128 != 0 || M == 0)
+                    const int bits = cfg["bits"].get<int>();
+                    const int zp_down = cfg["zero_point_down"].get<int>() < 0 ? zp : cfg["zero_point_down"].get<int>();
+                    const bool z_gu = cfg["has_zero_points_gate_up"].get<bool>(), z_d = cfg["has_zero_points_down"].get<bool>();
+                    if (bits != 4 || group != 128 || z_gu || z_d || zp_down != zp)
+                    {
+                        // other block parameters: the nodes of the block one after the other inside one call
+                        if ((bits != 4 && bits != 8) || (group != 32 && group != 64 && group != 128) || H % group != 0 || I % group != 0 ||
+                            H % 8 != 0 || M == 0)
+                            return nullptr;
+                        const size_t q_bytes = nnf::workspace::fused_mlp_wna16((int)M, (int)H, (int)I, bits, group);
+                        auto q_ws = allocate_tensor(Shape{q_bytes}, element::character);
+                        size_t zi = 6;
+                        const std::string zgu = z_gu ? "input" + std::to_string(zi++) : "nullptr";
+                        const std::string zd = z_d ? "input" + std::to_string(zi++) : "nullptr";
+                        LanguageUnit_p lu(new LanguageUnit(get_function_name()));
+                        *lu << "const nnf_quant quant_gate_up = {" << bits << ", " << group << ", " << zp << ", " << zgu << "};\n";
+                        *lu << "const nnf_quant quant_down = {" << bits << ", " << group << ", " << zp_down << ", " << zd << "};\n";
+                        *lu << "NNF_HIP_CHECK(nnf_fused_mlp_wna16(stream, input0, input1, " << float_literal(cfg["rms_eps"].get<double>())
+                            << ", input2, input3, input4, input5, output0, " << M << ", " << H << ", " << I
+                            << ", &quant_gate_up, &quant_down, " << q_ws->get_name() << ", " << q_bytes << "));\n";
+                        return lu;
+                    }
+                    if (H % 128 != 0 || I % 128 != 0 || M == 0)
                         return nullptr;
                     const size_t ws_bytes = nnf::workspace::fused_mlp_w4a16((int)M, (int)H, (int)I, group);
                     // the only intermediate that reaches HBM: h [M, I] fp16 (plus M row statistics)

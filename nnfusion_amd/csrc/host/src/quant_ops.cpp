@@ -12,8 +12,10 @@
 //                  output: Y f16 [M, N]   (N = rows of Wq; half of them when act == "silu_gate")
 //   QuantDotW8A8   inputs: A i8 [M,K], s_tok f32 [M], W i8 [N,K], s_ch f32 [N];  attr out_type "f16"|"i32"
 //                  output: Y f16 [M,N] = fp16((float)acc * s_tok * s_ch), or the raw i32 accumulators
-//   FusedQuantMLP  inputs: x f16 [M,H], gamma f16 [H], Wgu u8 [2I,H/2], Sgu f16 [2I,H/g], Wd u8 [H,I/2], Sd f16 [H,I/g]
-//                  attrs : group_size 128, zero_point 8, rms_eps 1e-6
+//   FusedQuantMLP  inputs: x f16 [M,H], gamma f16 [H], Wgu u8 [2I,H*bits/8], Sgu f16 [2I,H/g], Wd u8 [H,I*bits/8], Sd f16 [H,I/g]
+//                          [, Zgu u8] [, Zd u8] (zero points per (row, group) of either matrix, by attribute)
+//                  attrs : bits 4, group_size 128, zero_point 8, zero_point_down -1 (= zero_point), has_zero_points_gate_up false,
+//                          has_zero_points_down false, rms_eps 1e-6
 //                  output: out f16 [M,H] = x + Wd . (SiLU(Wg . n) * (Wu . n)), n = RMSNorm(x)
 #include "nnfusion/core/operators/generic_op/generic_op.hpp"
 
@@ -110,18 +112,68 @@ REGISTER_OP(QuantDotW8A8)
     });
 
 REGISTER_OP(FusedQuantMLP)
+    .attr<int>("bits", 4)
     .attr<int>("group_size", 128)
     .attr<int>("zero_point", 8)
+    .attr<int>("zero_point_down", -1) // -1: the same as zero_point
+    .attr<bool>("has_zero_points_gate_up", false)
+    .attr<bool>("has_zero_points_down", false)
     .attr<double>("rms_eps", 1e-6)
     .infershape([](std::shared_ptr<graph::GNode> gnode) -> void {
         auto gop = std::dynamic_pointer_cast<op::GenericOp>(gnode->get_op_ptr());
         NNFUSION_CHECK_NOT_NULLPTR(gop);
-        OP_VALIDATION(gop, gnode->get_input_size() == 6) << "inputs: x, gamma, Wgu, Sgu, Wd, Sd";
+        const size_t expect = 6 + (bool_attr(gop, "has_zero_points_gate_up") ? 1 : 0) + (bool_attr(gop, "has_zero_points_down") ? 1 : 0);
+        OP_VALIDATION(gop, gnode->get_input_size() == expect) << "inputs: x, gamma, Wgu, Sgu, Wd, Sd [, Zgu] [, Zd]";
         const Shape& x = gnode->get_input_shape(0);
         const Shape& wgu = gnode->get_input_shape(2);
         const Shape& wd = gnode->get_input_shape(4);
         OP_VALIDATION(gop, x.size() == 2 && wgu.size() == 2 && wd.size() == 2) << "bad ranks";
+        const size_t bits = (size_t)int_attr(gop, "bits");
+        OP_VALIDATION(gop, bits == 4 || bits == 8) << "4- or 8-bit weights";
         const size_t H = x[1], I = wgu[0] / 2;
-        OP_VALIDATION(gop, wgu[1] * 2 == H && wd[0] == H && wd[1] * 2 == I && wgu[0] % 2 == 0) << "shape mismatch";
+        OP_VALIDATION(gop, wgu[1] * 8 == H * bits && wd[0] == H && wd[1] * 8 == I * bits && wgu[0] % 2 == 0) << "shape mismatch";
         gnode->set_output_type_and_shape(0, gnode->get_input_element_type(0), x);
+    });
+
+// Dequantize of block-quantized weights: the reference's Dequantize (core/operators/op_define/dequantize.hpp; arithmetic
+// core/kernels/cpu/reference/kernels.cpp:601-623) with scales and offsets per block of `group_size` weights along K.
+//   inputs: Wq u8 [N, K*bits/8], S f16 [N, K/group] [, Z u8 [N, ceil(K/group*bits/8)]]   output: W f16 [N, K]
+REGISTER_OP(Dequantize)
+    .attr<int>("bits", 4)
+    .attr<int>("group_size", 128)
+    .attr<int>("zero_point", 8)
+    .attr<bool>("has_zero_points", false)
+    .infershape([](std::shared_ptr<graph::GNode> gnode) -> void {
+        auto gop = std::dynamic_pointer_cast<op::GenericOp>(gnode->get_op_ptr());
+        NNFUSION_CHECK_NOT_NULLPTR(gop);
+        const bool has_z = bool_attr(gop, "has_zero_points");
+        OP_VALIDATION(gop, gnode->get_input_size() == (has_z ? 3u : 2u)) << "inputs: Wq, S [, Z]";
+        const Shape& w = gnode->get_input_shape(0);
+        const Shape& s = gnode->get_input_shape(1);
+        const size_t bits = (size_t)int_attr(gop, "bits"), group = (size_t)int_attr(gop, "group_size");
+        OP_VALIDATION(gop, w.size() == 2 && s.size() == 2 && (bits == 4 || bits == 8) && group > 0) << "bad ranks or attributes";
+        const size_t K = w[1] * 8 / bits;
+        OP_VALIDATION(gop, K % group == 0 && s[0] == w[0] && s[1] == K / group) << "scales must be [N, K/group]";
+        gnode->set_output_type_and_shape(0, gnode->get_input_element_type(1), Shape{w[0], K});
+    });
+
+// The unquantized product, as far as the fold into QuantDot needs it: one reduction axis, A [.., K] . B [K, N] or (transpose_B)
+// B [N, K]; operands of one element type (src/nnfusion/core/operators/op_define/dot.cpp:47-53, 116-125).
+REGISTER_OP(Dot)
+    .attr<bool>("transpose_A", false)
+    .attr<bool>("transpose_B", false)
+    .infershape([](std::shared_ptr<graph::GNode> gnode) -> void {
+        auto gop = std::dynamic_pointer_cast<op::GenericOp>(gnode->get_op_ptr());
+        NNFUSION_CHECK_NOT_NULLPTR(gop);
+        OP_VALIDATION(gop, gnode->get_input_size() == 2) << "two inputs";
+        OP_VALIDATION(gop, gnode->get_input_element_type(0) == gnode->get_input_element_type(1)) << "arguments do not have the same element type";
+        OP_VALIDATION(gop, !bool_attr(gop, "transpose_A")) << "transpose_A is not supported";
+        const Shape& a = gnode->get_input_shape(0);
+        const Shape& b = gnode->get_input_shape(1);
+        OP_VALIDATION(gop, a.size() >= 1 && b.size() == 2) << "bad ranks";
+        const bool tb = bool_attr(gop, "transpose_B");
+        OP_VALIDATION(gop, a.back() == (tb ? b[1] : b[0])) << "reduction axes do not match";
+        Shape out(a.begin(), a.end() - 1);
+        out.push_back(tb ? b[0] : b[1]);
+        gnode->set_output_type_and_shape(0, gnode->get_input_element_type(0), out);
     });

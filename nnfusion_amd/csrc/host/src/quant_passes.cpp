@@ -78,10 +78,14 @@ namespace
 
     struct QuantDotInfo
     {
-        bool rms = false, has_bias = false, has_res = false, gate = false;
+        bool rms = false, has_bias = false, has_res = false, gate = false, has_z = false;
         int group = 128, zp = 8, bits = 4;
         double eps = 1e-6;
-        NodeOut a, wq, s, gamma, bias, res;
+        NodeOut a, wq, s, z, gamma, bias, res;
+        bool same_block_parameters(const QuantDotInfo& o) const
+        {
+            return group == o.group && bits == o.bits && has_z == o.has_z && (has_z || zp == o.zp);
+        }
     };
     bool quant_dot_info(const std::shared_ptr<GNode>& n, QuantDotInfo& q)
     {
@@ -96,13 +100,15 @@ namespace
         q.zp = cfg["zero_point"].get<int>();
         q.bits = cfg["bits"].get<int>();
         q.eps = cfg["rms_eps"].get<double>();
-        // only the specialised kernels have fused forms: a product with other block parameters stays as it is
-        if (q.bits != 4 || q.group != 128 || cfg["has_zero_points"].get<bool>())
-            return false;
+        q.has_z = cfg["has_zero_points"].get<bool>();
+        // (every block parameter has fused forms: the specialised kernels' own, or the nodes run one after the other
+        // inside one call of the launcher library)
         size_t i = 0;
         q.a = input_of(n, i++);
         q.wq = input_of(n, i++);
         q.s = input_of(n, i++);
+        if (q.has_z)
+            q.z = input_of(n, i++);
         if (q.rms)
             q.gamma = input_of(n, i++);
         if (q.has_bias)
@@ -117,6 +123,7 @@ namespace
         cfg["bits"] = op::OpConfig::any(q.bits);
         cfg["group_size"] = op::OpConfig::any(q.group);
         cfg["zero_point"] = op::OpConfig::any(q.zp);
+        cfg["has_zero_points"] = op::OpConfig::any(q.has_z);
         cfg["rms_norm"] = op::OpConfig::any(q.rms);
         cfg["rms_eps"] = op::OpConfig::any(q.eps);
         cfg["has_bias"] = op::OpConfig::any(q.has_bias);
@@ -271,9 +278,12 @@ namespace
         return true;
     }
 
-    std::vector<NodeOut> quant_dot_inputs(Rebuilder& rb, const QuantDotInfo& q, const NodeOut& wq, const NodeOut& s)
+    // (z: the zero-point tensor as placed in the new graph; unused without one)
+    std::vector<NodeOut> quant_dot_inputs(Rebuilder& rb, const QuantDotInfo& q, const NodeOut& wq, const NodeOut& s, const NodeOut& z)
     {
         std::vector<NodeOut> ins = {rb.map(q.a), wq, s};
+        if (q.has_z)
+            ins.push_back(z);
         if (q.rms)
             ins.push_back(rb.map(q.gamma));
         if (q.has_bias)
@@ -290,6 +300,29 @@ namespace
         Rebuilder rb(graph);
         auto replace = [&](const std::shared_ptr<GNode>& n, Rebuilder& r, std::vector<NodeOut>& outs) -> bool {
             QuantDotInfo q;
+            // (0) Dot{transpose_B}(A, Dequantize(Wq, S [, Z]))  ->  QuantDot(A, Wq, S [, Z]): the dequantised weights are
+            // never written (precedent: the reference folds MatMul + Add into one node,
+            // engine/pass/graph/subgraph_fusion_optimizer/matmuladd_fusion_optimizer.cpp)
+            if (is_op(n, "Dot"))
+            {
+                auto& dcfg = generic(n)->localOpConfig.getRoot();
+                NodeOut w = input_of(n, 1);
+                if (!dcfg["transpose_B"].get<bool>() || dcfg["transpose_A"].get<bool>() || !is_op(w.first, "Dequantize"))
+                    return false;
+                auto& qcfg = generic(w.first)->localOpConfig.getRoot();
+                QuantDotInfo f;
+                f.bits = qcfg["bits"].get<int>();
+                f.group = qcfg["group_size"].get<int>();
+                f.zp = qcfg["zero_point"].get<int>();
+                f.has_z = qcfg["has_zero_points"].get<bool>();
+                f.a = input_of(n, 0);
+                auto node = r.add(std::make_shared<op::GenericOp>(n->get_name(), "QuantDot", quant_dot_config(f)),
+                                  quant_dot_inputs(r, f, r.map(input_of(w.first, 0)), r.map(input_of(w.first, 1)),
+                                                   f.has_z ? r.map(input_of(w.first, 2)) : NodeOut()));
+                outs = {{node, 0}};
+                ++count;
+                return true;
+            }
             // (1) SiLU(QuantDot_gate(x)) * QuantDot_up(x)  ->  QuantDot{act = silu_gate} over [gate; up]
             if (is_op(n, "Multiply"))
             {
@@ -305,9 +338,10 @@ namespace
                         continue;
                     if (!same(qg.a, qu.a) || qg.rms != qu.rms || (qg.rms && (!same(qg.gamma, qu.gamma) || qg.eps != qu.eps)))
                         continue;
-                    if (qg.group != qu.group || qg.zp != qu.zp || qg.bits != qu.bits)
+                    if (!qg.same_block_parameters(qu))
                         continue;
-                    if (!constant_of(qg.wq) || !constant_of(qg.s) || !constant_of(qu.wq) || !constant_of(qu.s))
+                    if (!constant_of(qg.wq) || !constant_of(qg.s) || !constant_of(qu.wq) || !constant_of(qu.s) ||
+                        (qg.has_z && (!constant_of(qg.z) || !constant_of(qu.z))))
                         continue;
                     if (gate.first->get_output_shape(0) != up.first->get_output_shape(0))
                         continue;
@@ -320,10 +354,13 @@ namespace
                         continue;
                     auto wq = stack_rows(r, {qg.wq, qu.wq});
                     auto s = stack_rows(r, {qg.s, qu.s});
+                    NodeOut z;
+                    if (qg.has_z)
+                        z = {stack_rows(r, {qg.z, qu.z}), 0};
                     QuantDotInfo f = qg;
                     f.gate = true;
                     auto node = r.add(std::make_shared<op::GenericOp>(n->get_name() + "_gate_up", "QuantDot", quant_dot_config(f)),
-                                      quant_dot_inputs(r, f, {wq, 0}, {s, 0}));
+                                      quant_dot_inputs(r, f, {wq, 0}, {s, 0}, z));
                     outs = {{node, 0}};
                     ++count;
                     return true;
@@ -356,7 +393,7 @@ namespace
                     // the other operand must not depend on the QuantDot being rewritten: it is an earlier node or
                     // a constant, which the rebuild has already placed
                     auto node = r.add(std::make_shared<op::GenericOp>(d.first->get_name(), "QuantDot", quant_dot_config(f)),
-                                      quant_dot_inputs(r, f, r.map(q.wq), r.map(q.s)));
+                                      quant_dot_inputs(r, f, r.map(q.wq), r.map(q.s), q.has_z ? r.map(q.z) : NodeOut()));
                     outs = {{node, 0}};
                     ++count;
                     return true;
@@ -374,7 +411,7 @@ namespace
                 f.gamma = input_of(q.a.first, 1);
                 f.eps = generic(q.a.first)->localOpConfig.getRoot()["eps"].get<double>();
                 auto node = r.add(std::make_shared<op::GenericOp>(n->get_name(), "QuantDot", quant_dot_config(f)),
-                                  quant_dot_inputs(r, f, r.map(q.wq), r.map(q.s)));
+                                  quant_dot_inputs(r, f, r.map(q.wq), r.map(q.s), q.has_z ? r.map(q.z) : NodeOut()));
                 outs = {{node, 0}};
                 ++count;
                 return true;
@@ -383,14 +420,22 @@ namespace
             QuantDotInfo gu;
             if (q.has_res && !q.has_bias && !q.rms && !q.gate && quant_dot_info(q.a.first, gu) && gu.rms && gu.gate &&
                 !gu.has_bias && !gu.has_res && same(gu.a, q.res) && r.single_user(q.a.first) && gu.group == q.group &&
-                gu.zp == q.zp && gu.bits == q.bits && n->get_output_shape(0).size() == 2)
+                gu.bits == q.bits && n->get_output_shape(0).size() == 2)
             {
                 op::OpConfig::any cfg = op::OpConfig::any::object();
+                cfg["bits"] = op::OpConfig::any(q.bits);
                 cfg["group_size"] = op::OpConfig::any(q.group);
-                cfg["zero_point"] = op::OpConfig::any(q.zp);
+                cfg["zero_point"] = op::OpConfig::any(gu.zp);
+                cfg["zero_point_down"] = op::OpConfig::any(q.zp);
+                cfg["has_zero_points_gate_up"] = op::OpConfig::any(gu.has_z);
+                cfg["has_zero_points_down"] = op::OpConfig::any(q.has_z);
                 cfg["rms_eps"] = op::OpConfig::any(gu.eps);
-                auto node = r.add(std::make_shared<op::GenericOp>(n->get_name() + "_mlp", "FusedQuantMLP", cfg),
-                                  {r.map(gu.a), r.map(gu.gamma), r.map(gu.wq), r.map(gu.s), r.map(q.wq), r.map(q.s)});
+                std::vector<NodeOut> ins = {r.map(gu.a), r.map(gu.gamma), r.map(gu.wq), r.map(gu.s), r.map(q.wq), r.map(q.s)};
+                if (gu.has_z)
+                    ins.push_back(r.map(gu.z));
+                if (q.has_z)
+                    ins.push_back(r.map(q.z));
+                auto node = r.add(std::make_shared<op::GenericOp>(n->get_name() + "_mlp", "FusedQuantMLP", cfg), ins);
                 outs = {{node, 0}};
                 ++count;
                 return true;
@@ -432,11 +477,12 @@ bool pass::graph::QuantGemmFusionPass::run_on_graph(std::shared_ptr<Graph>& grap
         for (auto& n : graph->get_ordered_ops())
         {
             QuantDotInfo q;
-            if (!quant_dot_info(n, q) || q.has_bias || q.has_res || q.gate || !constant_of(q.wq) || !constant_of(q.s))
+            if (!quant_dot_info(n, q) || q.has_bias || q.has_res || q.gate || !constant_of(q.wq) || !constant_of(q.s) ||
+                (q.has_z && !constant_of(q.z)))
                 continue;
             std::ostringstream key;
             key << (void*)q.a.first.get() << ':' << q.a.second << '|' << q.rms << '|' << (void*)q.gamma.first.get() << '|' << q.eps
-                << '|' << q.group << '|' << q.zp << '|' << q.bits << '|' << q.wq.first->get_output_shape(0)[1];
+                << '|' << q.group << '|' << (q.has_z ? -1 : q.zp) << '|' << q.bits << '|' << q.wq.first->get_output_shape(0)[1];
             auto it = by_key.find(key.str());
             if (it == by_key.end())
             {
@@ -462,7 +508,7 @@ bool pass::graph::QuantGemmFusionPass::run_on_graph(std::shared_ptr<Graph>& grap
         const Group& grp = groups[it->second];
         if (!slices.count(it->second))
         {
-            std::vector<NodeOut> wqs, ss;
+            std::vector<NodeOut> wqs, ss, zs;
             QuantDotInfo q0;
             quant_dot_info(grp.members[0], q0);
             for (auto& m : grp.members)
@@ -471,11 +517,16 @@ bool pass::graph::QuantGemmFusionPass::run_on_graph(std::shared_ptr<Graph>& grap
                 quant_dot_info(m, q);
                 wqs.push_back(q.wq);
                 ss.push_back(q.s);
+                if (q.has_z)
+                    zs.push_back(q.z);
             }
             auto wq = stack_rows(r, wqs);
             auto s = stack_rows(r, ss);
+            NodeOut z;
+            if (q0.has_z)
+                z = {stack_rows(r, zs), 0};
             auto wide = r.add(std::make_shared<op::GenericOp>(grp.members[0]->get_name() + "_merged", "QuantDot", quant_dot_config(q0)),
-                              quant_dot_inputs(r, q0, {wq, 0}, {s, 0}));
+                              quant_dot_inputs(r, q0, {wq, 0}, {s, 0}, z));
             int begin = 0;
             for (auto& m : grp.members)
             {

@@ -348,31 +348,13 @@ int nnf_dequantize_f16(nnf_stream_t stream, const void* Wq, const void* scales, 
 
 // The fused product with other block parameters: the plain product between the kernels of the nodes around it, as the
 // unfused graph would run them.  workspace = [ RMSNorm(A): M x K fp16 ][ product: M x rows fp16 ][ the product's own ]
-namespace
-{
-    struct QFusedLayout
-    {
-        size_t xn = 0, product = 0, gemm = 0;
-        size_t total() const { return xn + product + gemm; }
-    };
-    QFusedLayout q_fused_layout(int M, int N, int K, const nnf_quant* q, bool rms, bool gate, bool through_scratch)
-    {
-        QFusedLayout l;
-        const int rows = gate ? 2 * N : N;
-        l.xn = rms ? nnf::workspace::align256((size_t)M * K * 2) : 0;
-        l.product = (gate || through_scratch) ? nnf::workspace::align256((size_t)M * rows * 2) : 0;
-        l.gemm = nnf::workspace::align256(nnf_wna16_gemm_workspace_bytes(M, rows, K, q));
-        return l;
-    }
-} // namespace
-
 size_t nnf_wna16_gemm_fused_workspace_bytes(int M, int N, int K, const nnf_quant* q, int act)
 {
     if (!q || M <= 0 || N <= 0 || K <= 0)
         return 0;
     if (is_plain_w4a16(q))
         return nnf::workspace::w4a16_gemm_fused(M, N, K, q->group, act);
-    return q_fused_layout(M, N, K, q, true, act == NNF_ACT_SILU_GATE, true).total();
+    return nnf::workspace::wna16_fused_layout(M, N, K, q->bits, q->group, true, act == NNF_ACT_SILU_GATE, true).total();
 }
 
 int nnf_wna16_gemm_fused(nnf_stream_t stream, const void* A, const void* Wq, const void* scales, void* Y, int M, int N, int K,
@@ -395,7 +377,7 @@ int nnf_wna16_gemm_fused(nnf_stream_t stream, const void* A, const void* Wq, con
     if (!nnf_wna16_supported(M, rows, K, q))
         return NNF_ERR_UNSUPPORTED_SHAPE;
     // a residual that is the output buffer itself must not be overwritten by the product
-    const QFusedLayout l = q_fused_layout(M, N, K, q, rms, gate, residual == Y);
+    const nnf::workspace::QFusedLayout l = nnf::workspace::wna16_fused_layout(M, N, K, q->bits, q->group, rms, gate, residual == Y);
     if (l.total() > 0 && (!workspace || !aligned16(workspace) || workspace_bytes < l.total()))
         return NNF_ERR_WORKSPACE_TOO_SMALL;
     uint8_t* ws = (uint8_t*)workspace;
@@ -647,10 +629,8 @@ size_t nnf_fused_mlp_wna16_workspace_bytes(int M, int H, int I, const nnf_quant*
         return 0;
     if (is_plain_w4a16(q_gate_up) && is_plain_w4a16(q_down) && q_gate_up->zero_point == q_down->zero_point)
         return nnf::workspace::fused_mlp_w4a16(M, H, I, 128);
-    const size_t a = nnf_wna16_gemm_workspace_bytes(M, 2 * I, H, q_gate_up), b = nnf_wna16_gemm_workspace_bytes(M, H, I, q_down);
-    const size_t wide = (size_t)(2 * I > H ? 2 * I : H);
-    return nnf::workspace::align256((size_t)M * H * 2) + nnf::workspace::align256((size_t)M * wide * 2) +
-           nnf::workspace::align256((size_t)M * I * 2) + nnf::workspace::align256(a > b ? a : b);
+    const int bits = q_gate_up->bits, group = q_gate_up->group;
+    return nnf::workspace::fused_mlp_wna16(M, H, I, bits, group);
 }
 
 int nnf_fused_mlp_wna16(nnf_stream_t stream, const void* x, const void* gamma, float eps, const void* Wgu, const void* Sgu,
@@ -666,7 +646,8 @@ int nnf_fused_mlp_wna16(nnf_stream_t stream, const void* x, const void* gamma, f
         return NNF_ERR_INVALID_ARGUMENT;
     if (!aligned16(x) || !aligned16(gamma) || !aligned16(out) || !aligned16(workspace))
         return NNF_ERR_INVALID_ARGUMENT;
-    if (H % 8 != 0 || !nnf_wna16_supported(M, 2 * I, H, q_gate_up) || !nnf_wna16_supported(M, H, I, q_down))
+    if (H % 8 != 0 || q_gate_up->bits != q_down->bits || q_gate_up->group != q_down->group ||
+        !nnf_wna16_supported(M, 2 * I, H, q_gate_up) || !nnf_wna16_supported(M, H, I, q_down))
         return NNF_ERR_UNSUPPORTED_SHAPE;
     if (!workspace || workspace_bytes < nnf_fused_mlp_wna16_workspace_bytes(M, H, I, q_gate_up, q_down))
         return NNF_ERR_WORKSPACE_TOO_SMALL;

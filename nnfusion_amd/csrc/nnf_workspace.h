@@ -592,6 +592,44 @@ namespace nnf
                 return 0;
             return plan_w4a16_sk(M, N, K, false, num_cu).bytes();
         }
+        // ---- the fused product / MLP block for block parameters that run the nodes one after the other ----------------------
+        inline size_t w4a16_gemm(int M, int N, int K, int, int num_cu = PLAN_CUS);
+        // nnf_wna16_gemm's own scratch memory, whichever form the zero point takes
+        inline size_t wna16_gemm_any(int M, int N, int K, int bits, int group, int num_cu = PLAN_CUS)
+        {
+            size_t a = wna16_gemm(M, N, K, bits, group, num_cu);
+            if (bits == 4 && group == 128)
+            {
+                const size_t b = w4a16_gemm(M, N, K, group, num_cu);
+                a = b > a ? b : a;
+            }
+            return align256(a);
+        }
+        // nnf_wna16_gemm_fused: [ RMSNorm(A): M x K fp16 ][ the product, where the epilogue cannot read it from Y: M x rows fp16 ]
+        //                       [ the product's own ]
+        struct QFusedLayout
+        {
+            size_t xn = 0, product = 0, gemm = 0;
+            size_t total() const { return xn + product + gemm; }
+        };
+        inline QFusedLayout wna16_fused_layout(int M, int N, int K, int bits, int group, bool rms, bool gate, bool through_scratch)
+        {
+            QFusedLayout l;
+            const int rows = gate ? 2 * N : N;
+            l.xn = rms ? align256((size_t)M * K * 2) : 0;
+            l.product = (gate || through_scratch) ? align256((size_t)M * rows * 2) : 0;
+            l.gemm = wna16_gemm_any(M, rows, K, bits, group);
+            return l;
+        }
+        // nnf_fused_mlp_wna16: [ RMSNorm(x): M x H fp16 ][ gate | up products M x 2I fp16, then the down product M x H fp16 ]
+        //                      [ h: M x I fp16 ][ the products' own ]
+        inline size_t fused_mlp_wna16(int M, int H, int I, int bits, int group)
+        {
+            const size_t a = wna16_gemm_any(M, 2 * I, H, bits, group), b = wna16_gemm_any(M, H, I, bits, group);
+            const size_t wide = (size_t)(2 * I > H ? 2 * I : H);
+            return align256((size_t)M * H * 2) + align256((size_t)M * wide * 2) + align256((size_t)M * I * 2) + (a > b ? a : b);
+        }
+
         // K above 8192 (above 4096 for 17 .. 32 rows, above 2048 for 33 .. 64; a multiple of 256): the run-time-K form over equal ranges of K (in whole pairs of
         // groups; the last range may be shorter), each on its share of the CUs; fp32 sums per range, added by the
         // reduction pass.  Every workgroup fetches the activations of its range, so shorter ranges mean less of that
@@ -780,7 +818,7 @@ namespace nnf
             return variant >= 0 && variant <= 4 && route_w4a16(M, N, K, false, false, false, num_cu, variant).kind != W4A16Route::NONE;
         }
         // nnf_w4a16_gemm: [ partial sums ]
-        inline size_t w4a16_gemm(int M, int N, int K, int, int num_cu = PLAN_CUS)
+        inline size_t w4a16_gemm(int M, int N, int K, int, int num_cu)
         {
             return route_w4a16(M, N, K, false, false, false, num_cu).partial_bytes;
         }

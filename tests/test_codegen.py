@@ -95,7 +95,8 @@ def test_onnx_front_door_imports_fuses_and_generates(tmp_path):
 
 
 def _run_generated(name, inputs, out_shape, out_dtype, gpu, n_outputs=1):
-    """dlopen nnfusion_amd/generated/<name>, init, kernel_entry(inputs..., outputs...), free."""
+    """dlopen nnfusion_amd/generated/<name>, init, kernel_entry(inputs..., outputs...), free.  out_shape: one shape for
+    all outputs, or a list of one shape per output."""
     import torch
 
     d = os.path.join(GEN, name)
@@ -108,7 +109,9 @@ def _run_generated(name, inputs, out_shape, out_dtype, gpu, n_outputs=1):
         assert rt.get_device_type() == 1
         rt.rocm_init()
         dev_in = [torch.from_numpy(np.ascontiguousarray(a)).to(gpu) for a in inputs]
-        outs = [torch.empty(out_shape, dtype=out_dtype, device=gpu) for _ in range(n_outputs)]
+        shapes = out_shape if isinstance(out_shape, list) else [out_shape] * n_outputs
+        n_outputs = len(shapes)
+        outs = [torch.empty(sh, dtype=out_dtype, device=gpu) for sh in shapes]
         rt.kernel_entry.argtypes = [ctypes.c_void_p] * (len(dev_in) + n_outputs)
         rt.kernel_entry.restype = ctypes.c_int
         assert rt.kernel_entry(*[t.data_ptr() for t in dev_in], *[o.data_ptr() for o in outs]) == 0
@@ -202,3 +205,66 @@ def test_generated_qkv_graph_runtime(gpu):
     assert src.count("NNF_HIP_CHECK(nnf_w4a16_gemm") == 1 and src.count("hipMemcpy2DAsync(") == 3
     for i, y in enumerate(ys):
         assert np.abs(y.astype(np.float32) - ref[:, i * n:(i + 1) * n]).max() <= 1e-2 * _rms(ref)
+
+
+def _gen_src(name):
+    return open(os.path.join(GEN, name, "nnfusion_rt.cpp")).read()
+
+
+@pytest.mark.gpu
+def test_generated_runtimes_of_the_other_onnx_forms(gpu):
+    """MatMulNBits with a bias; DequantizeLinear + MatMul (the Dequantize -> Dot fold); the MLP block with blocks of 32 and
+    zero points (one FusedQuantMLP); and the same block with its gate product as a second result of the graph, which keeps
+    RMSNorm-folded products, Sigmoid, two Multiplies and the fused down projection as separate nodes."""
+    import torch
+
+    import __graft_entry__ as entry
+
+    tol = 1e-2
+    _, m, n, k = entry.ONNX_EXAMPLES["onnx_linear_bias"]
+    a, wq, s = datagen.w4a16_case(0, m, n, k)
+    bias = datagen.normal_f16(0, datagen.S_BIAS, (n,))
+    y = _run_generated("onnx_linear_bias", [a], (m, n), torch.float16, gpu)
+    ref = oracle.add_f16(oracle.w4a16_gemm(a, wq, s), np.broadcast_to(bias, (m, n)).copy())
+    assert np.abs(y.astype(np.float32) - ref.astype(np.float32)).max() <= tol * _rms(ref)
+    assert _gen_src("onnx_linear_bias").count("NNF_HIP_CHECK(nnf_") == 1
+
+    _, m, n, k = entry.ONNX_EXAMPLES["onnx_qdq_u4"]
+    a, wq, s, z = datagen.wna16_case(0, m, n, k, 4, 64, True)
+    y = _run_generated("onnx_qdq_u4", [a], (m, n), torch.float16, gpu)
+    ref = oracle.wna16_gemm(a, wq, s, 4, 64, zero_points=z, f32_out=True)
+    assert np.abs(y.astype(np.float32) - ref).max() <= tol * _rms(ref)
+    src = _gen_src("onnx_qdq_u4")
+    assert src.count("NNF_HIP_CHECK(nnf_") == 1 and "nnf_wna16_gemm(" in src and "nnf_dequantize_f16" not in src
+
+    _, m, n, k = entry.ONNX_EXAMPLES["onnx_qdq_i8"]
+    a, wq, s, _ = datagen.wna16_case(0, m, n, k, 8, 128, False)
+    y = _run_generated("onnx_qdq_i8", [a], (m, n), torch.float16, gpu)
+    ref = oracle.wna16_gemm(a, wq, s, 8, 128, zp=128, f32_out=True)
+    assert np.abs(y.astype(np.float32) - ref).max() <= tol * _rms(ref)
+
+    def mlp_reference(m, h, i):
+        x, gamma, gate, up, down = entry.mlp_q_case(m, h, i)
+        xn = oracle.rmsnorm_f16(x, gamma, 1e-6)
+        g = oracle.wna16_gemm(xn, gate[0], gate[1], 4, 32, zero_points=gate[2])
+        u = oracle.wna16_gemm(xn, up[0], up[1], 4, 32, zero_points=up[2])
+        hh = oracle.silu_mul_f16(g, u)
+        return x, g, oracle.add_f16(oracle.wna16_gemm(hh, down[0], down[1], 4, 32, zero_points=down[2]), x)
+
+    _, m, h, i = entry.ONNX_EXAMPLES["onnx_mlp_w4z32"]
+    x, _, ref = mlp_reference(m, h, i)
+    y = _run_generated("onnx_mlp_w4z32", [x], (m, h), torch.float16, gpu)
+    assert np.abs(y.astype(np.float32) - ref.astype(np.float32)).max() <= tol * _rms(ref)
+    src = _gen_src("onnx_mlp_w4z32")
+    assert src.count("NNF_HIP_CHECK(nnf_") == 1 and "nnf_fused_mlp_wna16(" in src
+
+    _, m, h, i = entry.ONNX_EXAMPLES["onnx_mlp_unfused"]
+    x, g_ref, ref = mlp_reference(m, h, i)
+    y, g = _run_generated("onnx_mlp_unfused", [x], [(m, h), (m, i)], torch.float16, gpu)
+    assert np.abs(g.astype(np.float32) - g_ref.astype(np.float32)).max() <= tol * _rms(g_ref)
+    assert np.abs(y.astype(np.float32) - ref.astype(np.float32)).max() <= tol * _rms(ref)
+    src = _gen_src("onnx_mlp_unfused")
+    # gate and up products with the norm folded in, Sigmoid, Multiply x 2 (one definition: the code generator shares functions
+    # with the same signature and body), the down projection with the residual folded in
+    assert src.count("NNF_HIP_CHECK(nnf_wna16_gemm_fused(") == 3 and src.count("NNF_HIP_CHECK(nnf_elementwise_f16(") == 2
+    assert "NNF_EW_SIGMOID" in src and "NNF_EW_MULTIPLY" in src and "nnf_rms_norm_f16" not in src
