@@ -125,6 +125,9 @@ namespace nnf
         constexpr int vmcnt_imm(int n) { return (n & 0xF) | ((n >> 4) << 14) | (0x7 << 4) | (0xF << 8); }
 
         // `grid` workgroups split `units` units as [v * units / grid, (v + 1) * units / grid)
+        // (Shares weighted by what a second K loop in a workgroup costs -- its first loads, parking the part it leaves
+        // behind: about one and a half units -- were tried: with whole units to deal out the longest share stays the same
+        // for the MLP block's products, and a table of bounds in the kernel arguments made every launch slower.)
         __host__ __device__ inline long long first_unit_of(int v, long long units, int grid)
         {
             return ((long long)v * units) / grid;
@@ -365,23 +368,76 @@ namespace nnf
     // Block `r` (32 rows) of strip `wave` of a tile that `n_seg` workgroups (v_first, v_first + 1, ...) of a launch of
     // `gemm_grid` worked on: adds their parked parts in K order, eight in flight, and finishes the block (epilogue,
     // stores).  Used by the second launch and, with SkGemmParams::sync, by the GEMM's own workgroups: same order, same bits.
+    // Where a shared tile's parts lie and what its rows and columns are: what sk_request_parts / sk_finish_block need
+    struct SkSharedTile
+    {
+        int tile, v_first, n_seg;
+        bool first_is_second_slot; // the first owner parked this tile in its second slot (its range began in an earlier tile)
+    };
+    // Parts of a block kept in flight at once (16 TN registers each).  SAME_LAUNCH: inside the GEMM kernel, with its
+    // accumulation registers still set aside, and (sk_loads_ahead) two blocks' worth of them in flight.
+    template <int TM, int TN>
+    constexpr bool sk_loads_ahead()
+    {
+        return TM * TN <= 8;
+    }
+    template <int TM, int TN, bool SAME_LAUNCH>
+    struct SkPartsInFlight
+    {
+        static constexpr int D = !SAME_LAUNCH ? 8 : (sk_loads_ahead<TM, TN>() && TN >= 2) ? 3 : 4;
+        floatx4 v[D][TN][4]; // [part][column tile][quarter of its 16 elements]
+    };
+    // Asks for parts sg0 .. sg0 + D - 1 (clamped to the last) of block `r` (32 rows) of strip `wave` of a shared tile.
     // SAME_LAUNCH: the parts were parked by other workgroups of the launch that is still running (device-scope loads).
+    template <int TM, int TN, bool SAME_LAUNCH>
+    __device__ __forceinline__ void sk_request_parts(SkPartsInFlight<TM, TN, SAME_LAUNCH>& x, const SkGemmParams& p,
+                                                     int gemm_grid, const SkSharedTile& t, int r, int sg0, int tid)
+    {
+        using namespace gemm_sk;
+        using T = Tile<TM, TN>;
+        constexpr int D = SkPartsInFlight<TM, TN, SAME_LAUNCH>::D;
+        buffer_t parked;
+        if constexpr (SAME_LAUNCH)
+            parked = parked_buffer(p.partial, p.partial_bytes);
+#pragma unroll
+        for (int d = 0; d < D; ++d)
+        {
+            const int sg = min(sg0 + d, t.n_seg - 1);
+            const size_t first_float =
+                ((size_t)(t.v_first + sg) + ((sg == 0 && t.first_is_second_slot) ? (size_t)gemm_grid : 0)) * T::SLOT_FLOATS + (size_t)tid * 4;
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+                {
+                    const size_t at = first_float + (size_t)(((r * TN + j) * 4 + q) * THREADS * 4);
+                    if constexpr (SAME_LAUNCH)
+                        x.v[d][j][q] = load_device_scope(parked, (uint32_t)(at * sizeof(float)));
+                    else
+                        x.v[d][j][q] = *reinterpret_cast<const floatx4*>(p.partial + at);
+                }
+        }
+    }
+    // Block `r` (32 rows) of strip `wave` of a tile that t.n_seg workgroups (t.v_first, t.v_first + 1, ...) of a launch of
+    // `gemm_grid` worked on: adds their parked parts in K order -- the first ones have been asked for into `x` -- and
+    // finishes the block (epilogue, stores).  Used by the second launch and, with SkGemmParams::sync, by the GEMM's own
+    // workgroups: same order, same bits.
     template <int TM, int TN, bool GATE, bool BIAS, bool RESID, bool RMS, bool SAME_LAUNCH>
-    __device__ __forceinline__ void sk_sum_block(const SkGemmParams& p, int gemm_grid, int tile, int r, int v_first, int n_seg,
-                                                 bool first_is_second_slot, uint8_t* stage, int wave, int lane)
+    __device__ __forceinline__ void sk_finish_block(SkPartsInFlight<TM, TN, SAME_LAUNCH>& x, const SkGemmParams& p,
+                                                    int gemm_grid, const SkSharedTile& t, int r, uint8_t* stage, int wave, int lane)
     {
         using namespace gemm_sk;
         using T = Tile<TM, TN>;
         constexpr int BN_OUT = GATE ? T::BN / 2 : T::BN;
-        const int tid = wave * 64 + lane;
+        constexpr int D = SkPartsInFlight<TM, TN, SAME_LAUNCH>::D;
         int tm, tn;
         {
             constexpr int GM = 4;
             const int per_group = GM * p.tiles_n;
-            const int g = tile / per_group;
+            const int g = t.tile / per_group;
             const int first_m = g * GM;
             const int gm = min(GM, p.tiles_m - first_m);
-            const int rr = tile - g * per_group;
+            const int rr = t.tile - g * per_group;
             tm = first_m + rr % gm;
             tn = rr / gm;
         }
@@ -392,45 +448,23 @@ namespace nnf
 #pragma unroll
             for (int e = 0; e < 16; ++e)
                 c[0][j][e] = 0.f;
-        // SAME_LAUNCH: inside the GEMM kernel, with its accumulation registers still set aside: four parts in flight
-        constexpr int D = SAME_LAUNCH ? 4 : 8;
-        buffer_t parked;
-        if constexpr (SAME_LAUNCH)
-            parked = parked_buffer(p.partial, p.partial_bytes);
-        for (int sg0 = 0; sg0 < n_seg; sg0 += D)
+        for (int sg0 = 0; sg0 < t.n_seg; sg0 += D)
         {
-            floatx4 x[D][TN][4];
+            if (sg0 > 0)
+                sk_request_parts<TM, TN, SAME_LAUNCH>(x, p, gemm_grid, t, r, sg0, wave * 64 + lane);
 #pragma unroll
             for (int d = 0; d < D; ++d)
-            {
-                const int sg = min(sg0 + d, n_seg - 1);
-                const size_t first_float =
-                    ((size_t)(v_first + sg) + ((sg == 0 && first_is_second_slot) ? (size_t)gemm_grid : 0)) * T::SLOT_FLOATS + (size_t)tid * 4;
-#pragma unroll
-                for (int j = 0; j < TN; ++j)
-#pragma unroll
-                    for (int q = 0; q < 4; ++q)
-                    {
-                        const size_t at = first_float + (size_t)(((r * TN + j) * 4 + q) * THREADS * 4);
-                        if constexpr (SAME_LAUNCH)
-                            x[d][j][q] = load_device_scope(parked, (uint32_t)(at * sizeof(float)));
-                        else
-                            x[d][j][q] = *reinterpret_cast<const floatx4*>(p.partial + at);
-                    }
-            }
-#pragma unroll
-            for (int d = 0; d < D; ++d)
-                if (sg0 + d < n_seg)
+                if (sg0 + d < t.n_seg)
                 {
 #pragma unroll
                     for (int j = 0; j < TN; ++j)
 #pragma unroll
                         for (int q = 0; q < 4; ++q)
                         {
-                            c[0][j][4 * q] += x[d][j][q].x;
-                            c[0][j][4 * q + 1] += x[d][j][q].y;
-                            c[0][j][4 * q + 2] += x[d][j][q].z;
-                            c[0][j][4 * q + 3] += x[d][j][q].w;
+                            c[0][j][4 * q] += x.v[d][j][q].x;
+                            c[0][j][4 * q + 1] += x.v[d][j][q].y;
+                            c[0][j][4 * q + 2] += x.v[d][j][q].z;
+                            c[0][j][4 * q + 3] += x.v[d][j][q].w;
                         }
                 }
         }
@@ -538,7 +572,7 @@ namespace nnf
 
         // (sync) the shared tiles this workgroup has parked a part of -- its first and its last segment -- and, in
         // thread 0, the tile's first sync word as the arrival found it
-        __shared__ uint32_t sync_note;
+        __shared__ uint32_t sync_note[2];
         int pend_tile[2] = {-1, -1};
         uint32_t pend_old[2] = {0u, 0u};
 
@@ -1065,48 +1099,95 @@ namespace nnf
         {
             __syncthreads(); // the epilogue's staging regions are free
             uint8_t* stage = smem + wave * sk_region_bytes<1, TN, GATE>();
+            SkSharedTile shared[2];
+            uint32_t blocks[2] = {0u, 0u};
 #pragma unroll
             for (int slot = 0; slot < 2; ++slot)
             {
                 const int tile = pend_tile[slot];
-                if (tile < 0)
-                    continue;
-                const long long t0 = (long long)tile * SS;
-                const int v_first = owner_of_unit(t0, p.units, grid);
-                const int n_seg = owner_of_unit(t0 + SS - 1, p.units, grid) - v_first + 1;
-                const bool first_is_second_slot = first_unit_of(v_first, p.units, grid) < t0;
-                uint32_t* state = p.sync + 2 * (size_t)tile;
-                if (tid == 0)
+                const long long t0 = (long long)max(tile, 0) * SS;
+                shared[slot].tile = tile;
+                shared[slot].v_first = owner_of_unit(t0, p.units, grid);
+                shared[slot].n_seg = owner_of_unit(t0 + SS - 1, p.units, grid) - shared[slot].v_first + 1;
+                shared[slot].first_is_second_slot = first_unit_of(shared[slot].v_first, p.units, grid) < t0;
+                if (tile >= 0 && tid == 0)
                 {
                     uint32_t own = 0u;
-                    for (int i = v - v_first; i < TM; i += n_seg)
+                    for (int i = v - shared[slot].v_first; i < TM; i += shared[slot].n_seg)
                         own |= 1u << i;
-                    sync_note = sk_blocks_to_finish(state, pend_old[slot], n_seg, own, p.spin_limit);
+                    sync_note[slot] = sk_blocks_to_finish(p.sync + 2 * (size_t)tile, pend_old[slot], shared[slot].n_seg, own, p.spin_limit);
                 }
-                __syncthreads();
-                const uint32_t blocks = sync_note;
-                NNF_SK_STAMP(5 + 2 * slot); // the wait for the tile's other workgroups is over
-                if (blocks)
+            }
+            __syncthreads();
+            blocks[0] = pend_tile[0] >= 0 ? sync_note[0] : 0u;
+            blocks[1] = pend_tile[1] >= 0 ? sync_note[1] : 0u;
+            NNF_SK_STAMP(5); // the waits for the tiles' other workgroups are over
+            // (every part was complete at device scope before its workgroup counted itself in, the counts were read at
+            // device scope, and so are the parts)
+            // The blocks to finish, those of the first tile in bits 0 .. 7, of the second in bits 8 .. 15, one after the
+            // other; where the registers allow it the parts of the next block are asked for ahead of this block's sums.
+            constexpr bool AHEAD = sk_loads_ahead<TM, TN>();
+            uint32_t todo = blocks[0] | (blocks[1] << 8);
+            // (selected field by field: an array indexed at run time would live in private memory)
+            auto tile_of = [&](int task) {
+                const bool second = task >= 8;
+                SkSharedTile t;
+                t.tile = second ? shared[1].tile : shared[0].tile;
+                t.v_first = second ? shared[1].v_first : shared[0].v_first;
+                t.n_seg = second ? shared[1].n_seg : shared[0].n_seg;
+                t.first_is_second_slot = second ? shared[1].first_is_second_slot : shared[0].first_is_second_slot;
+                return t;
+            };
+            if constexpr (AHEAD)
+            {
+                SkPartsInFlight<TM, TN, true> x0, x1;
+                int cur = todo ? __builtin_ctz(todo) : -1;
+                if (cur >= 0)
+                    sk_request_parts<TM, TN, true>(x0, p, grid, tile_of(cur), cur & 7, 0, tid);
+                while (cur >= 0)
                 {
-                    // (every part was complete at device scope before its workgroup counted itself in, the count was read
-                    // at device scope, and so are the parts)
-                    for (int i = 0; i < TM; ++i)
-                        if ((blocks >> i) & 1u)
-                            sk_sum_block<TM, TN, GATE, BIAS, RESID, RMS, true>(p, grid, tile, i, v_first, n_seg, first_is_second_slot, stage,
-                                                                               wave, lane);
+                    todo &= todo - 1;
+                    int nxt = todo ? __builtin_ctz(todo) : -1;
+                    if (nxt >= 0)
+                        sk_request_parts<TM, TN, true>(x1, p, grid, tile_of(nxt), nxt & 7, 0, tid);
+                    sk_finish_block<TM, TN, GATE, BIAS, RESID, RMS, true>(x0, p, grid, tile_of(cur), cur & 7, stage, wave, lane);
+                    if (nxt < 0)
+                        break;
+                    todo &= todo - 1;
+                    cur = todo ? __builtin_ctz(todo) : -1;
+                    if (cur >= 0)
+                        sk_request_parts<TM, TN, true>(x0, p, grid, tile_of(cur), cur & 7, 0, tid);
+                    sk_finish_block<TM, TN, GATE, BIAS, RESID, RMS, true>(x1, p, grid, tile_of(nxt), nxt & 7, stage, wave, lane);
                 }
-                __syncthreads(); // sync_note is read; (blocks) every wavefront's strips are finished
-                NNF_SK_STAMP(6 + 2 * slot); // its share of the tile is finished
-                if (blocks && tid == 0)
+            }
+            else
+            {
+                SkPartsInFlight<TM, TN, true> x;
+                while (todo)
                 {
-                    const uint32_t n = (uint32_t)__builtin_popcount(blocks);
-                    if (atomicAdd(state + 1, n) + n == (uint32_t)TM)
+                    const int cur = __builtin_ctz(todo);
+                    todo &= todo - 1;
+                    sk_request_parts<TM, TN, true>(x, p, grid, tile_of(cur), cur & 7, 0, tid);
+                    sk_finish_block<TM, TN, GATE, BIAS, RESID, RMS, true>(x, p, grid, tile_of(cur), cur & 7, stage, wave, lane);
+                }
+            }
+            __syncthreads(); // every wavefront's strips are finished
+            NNF_SK_STAMP(6); // this workgroup's share of its tiles is finished
+            if (tid == 0)
+            {
+#pragma unroll
+                for (int slot = 0; slot < 2; ++slot)
+                    if (blocks[slot])
                     {
-                        // nobody looks at this tile's words any more: leave them as the next launch wants them
-                        atomicExch(state, 0u);
-                        atomicExch(state + 1, 0u);
+                        uint32_t* state = p.sync + 2 * (size_t)pend_tile[slot];
+                        const uint32_t n = (uint32_t)__builtin_popcount(blocks[slot]);
+                        if (atomicAdd(state + 1, n) + n == (uint32_t)TM)
+                        {
+                            // nobody looks at this tile's words any more: leave them as the next launch wants them
+                            atomicExch(state, 0u);
+                            atomicExch(state + 1, 0u);
+                        }
                     }
-                }
             }
         }
         NNF_SK_STAMP(9); // done
@@ -1135,6 +1216,10 @@ namespace nnf
             return;
         // the first owner parked this tile in its second slot when its range began in an earlier tile
         const bool first_is_second_slot = first_unit_of(v_first, p.units, gemm_grid) < t0;
-        sk_sum_block<TM, TN, GATE, BIAS, RESID, RMS, false>(p, gemm_grid, tile, r, v_first, n_seg, first_is_second_slot, stage, wave, lane);
+        SkSharedTile t;
+        t.tile = tile, t.v_first = v_first, t.n_seg = n_seg, t.first_is_second_slot = first_is_second_slot;
+        SkPartsInFlight<TM, TN, false> x;
+        sk_request_parts<TM, TN, false>(x, p, gemm_grid, t, r, 0, wave * 64 + lane);
+        sk_finish_block<TM, TN, GATE, BIAS, RESID, RMS, false>(x, p, gemm_grid, t, r, stage, wave, lane);
     }
 } // namespace nnf
