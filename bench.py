@@ -60,27 +60,23 @@ WNA16_MS = (1, 16, 4096)
 MLP_HI = (4096, 11008)                # configs[4]: hidden and intermediate size
 MLP_MS = (1, 16, 256)                 # ... at M = 256; the same block at decode sizes beside it
 
-# the kernel that dominates each configuration row (what a kernel trace of the row shows)
-DOMINANT_KERNEL = {
-    "w4a16_gemm_N8192_K8192.M16": "nnf::w4a16_mrows_kernel<2, 4, 1> (row-streaming MFMA kernel)",
-    "w4a16_gemm_N8192_K8192.M128": "nnf::gemm_sk::w4a16_gemm_sk_kernel<4, 2, ...> + w4a16_gemm_sk_fixup_kernel",
-    "w4a16_gemm_N8192_K8192.M1024": "nnf::gemm_sk::w4a16_gemm_sk_kernel<4, 2, ...> + w4a16_gemm_sk_fixup_kernel",
-    "w4a16_gemm_N8192_K8192.M4096": "nnf::gemm_sk::w4a16_gemm_sk_kernel<8, 2, ...>",
-    "w8a8_gemm_N8192_K8192.M1": "nnf::w8a8_gemv_rows_kernel",
-    "w8a8_gemm_N8192_K8192.M32": "nnf::w8a8_mrows_kernel",
-    "w8a8_gemm_N8192_K8192.M512": "nnf::w8a8_gemm_dl_kernel (128 x 128 tiles)",
-    "w8a8_gemm_N8192_K8192.M4096": "nnf::w8a8_gemm_dl_kernel (256 x 256 tiles)",
-    "wna16_b8_g128_zp_scalar_N8192_K8192.M1": "nnf::wna16_gemv_kernel<8, 4, 1>",
-    "wna16_b8_g128_zp_scalar_N8192_K8192.M16": "nnf::wna16_skinny_kernel<8, 2>",
-    "wna16_b8_g128_zp_scalar_N8192_K8192.M4096": "nnf::wna16_tile128_kernel<8>",
-    "wna16_b4_g64_zp_tensor_N8192_K8192.M1": "nnf::w4a16_gemv_rows_q_kernel<2, D, 8, 3> (row-streaming GEMV, zero points per group)",
-    "wna16_b4_g64_zp_tensor_N8192_K8192.M16": "nnf::w4a16_mrows_q_kernel<4, 6, true> (row-streaming MFMA kernel)",
-    "wna16_b4_g64_zp_tensor_N8192_K8192.M4096": "nnf::gemm_sk::w4a16_gemm_sk_kernel<8, 2, ..., 6> (stream-K tile GEMM, groups of 64)",
-    "fused_mlp_M1_4096_11008": "2 x nnf::w4a16_gemv_rows_fused_kernel (gate|up with RMSNorm and SiLU, down with the residual)",
-    "fused_mlp_M16_4096_11008": "nnf::w4a16_mrows_kernel (gate|up with RMSNorm and SiLU) + w4a16_mrows_any_kernel over 3 ranges of K + "
-                                "splitk_reduce_kernel (down)",
-    "fused_mlp_M256_4096_11008": "rms_rstd_kernel + 2 x (nnf::gemm_sk::w4a16_gemm_sk_kernel<4, 2, ...> + fixup)",
-}
+def load_row_kernels():
+    """The kernels each configuration row launches, as a kernel trace of `bench.py --pmc-probe` shows them: the last
+    column of the rows of profiles/bench_configurations_hbm_traffic.txt (`<row key> <five numbers>  <kernels>`)."""
+    out = {}
+    path = os.path.join(PROFILES_DIR, "bench_configurations_hbm_traffic.txt")
+    if not os.path.exists(path):
+        return out
+    with open(path) as f:
+        for line in f:
+            parts = line.split(None, 6)
+            if len(parts) == 7 and parts[0] != "row":
+                try:
+                    [float(x) for x in parts[1:6]]
+                except ValueError:
+                    continue
+                out[parts[0]] = parts[6].strip()
+    return out
 
 
 def wna16_key(bits, group, zp_tensor, n, k, m):
@@ -132,6 +128,11 @@ def load_probes():
     lib.nnf_probe_mfma.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_double),
                                    ctypes.POINTER(ctypes.c_double)]
     lib.nnf_probe_mfma.restype = ctypes.c_int
+    vp, ci = ctypes.c_void_p, ctypes.c_int
+    lib.nnf_probe_gemv_timeline.argtypes = [vp] * 5 + [ci, ci, vp, ci]
+    lib.nnf_probe_gemv_timeline.restype = ci
+    lib.nnf_probe_gemm_timeline.argtypes = [vp] * 5 + [ci] * 4 + [vp, ctypes.c_size_t, vp, ctypes.c_size_t, vp, ci]
+    lib.nnf_probe_gemm_timeline.restype = ci
     return lib
 
 
@@ -151,6 +152,9 @@ def main():
     ap.add_argument("--gemm-probe", action="store_true",
                     help="for hardware-counter runs: the fp16 x int4 and the W8A8 GEMM at M=4096, N=K=8192, twelve "
                          "launches each; prints their event-timed means, no JSON line of the benchmark")
+    ap.add_argument("--timeline", action="store_true",
+                    help="time stamps from inside the kernels (the probe library's builds of the single-row GEMV and of "
+                         "the tile GEMM in its one-launch form): prints a table per shape, no JSON line of the benchmark")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU (no sharding, no collectives); use --gpus 1")
@@ -171,6 +175,9 @@ def main():
         return
     if args.mfma_probe:
         print(json.dumps(run_mfma_probe(env, load_probes())))
+        return
+    if args.timeline:
+        run_timeline(env, load_probes())
         return
 
     # ---- resident inputs ------------------------------------------------------------------------
@@ -323,6 +330,9 @@ class Env:
 
     def __init__(self, torch, np, dev, lib, datagen, ops):
         self.torch, self.np, self.dev, self.lib, self.datagen, self.ops = torch, np, dev, lib, datagen, ops
+        # nnf_plan::sync_flags: cleared once here, left clear by every call; what an emitted function's persistent,
+        # zero-initialised tensor is.  With it the tile GEMM adds up the tiles its workgroups share inside its one launch.
+        self.sync = ops.sync_flags(dev)
 
     def dev_t(self, a):
         return self.torch.from_numpy(self.np.ascontiguousarray(a)).to(self.dev)
@@ -424,7 +434,7 @@ def parity_extra(env, oracle, parity):
     twq, ts = env.dev_t(wq), env.dev_t(s)
     for m in GEMM_MS:
         a = datagen.normal_f16(0, datagen.S_ACT, (m, k))
-        y = ops.w4a16_gemm(env.dev_t(a), twq, ts)
+        y = ops.w4a16_gemm_variant(env.dev_t(a), twq, ts, "auto", sync=env.sync)
         torch.cuda.synchronize()
         ref = oracle.w4a16_gemm(a, wq[cols], s[cols], f32_out=True)
         check_w4a16(np, parity, f"w4a16_gemm_N{n}_K{k}.M{m}", y.cpu().numpy()[:, cols], ref)
@@ -469,7 +479,7 @@ def parity_extra(env, oracle, parity):
     h, i = MLP_HI
     for m in MLP_MS:
         x, gamma, wgu, sgu, wd, sd = datagen.mlp_case(0, m, h, i)
-        out = ops.fused_mlp_w4a16(*[env.dev_t(t) for t in (x, gamma, wgu, sgu, wd, sd)])
+        out = ops.fused_mlp_w4a16(*[env.dev_t(t) for t in (x, gamma, wgu, sgu, wd, sd)], sync=env.sync)
         torch.cuda.synchronize()
         rows = min(m, 8)
         ref = oracle.fused_mlp_w4a16(x[:rows].copy(), gamma, wgu, sgu, wd, sd)
@@ -564,6 +574,82 @@ def run_gemm_probe(env, m=4096, n=8192, k=8192, launches=12):
             "w8a8_us": round(us8, 1), "w8a8_tops": round(ops_total / us8 / 1e6, 1)}
 
 
+def run_timeline(env, probes):
+    """Where a launch spends its time, from stamps of the 100 MHz clock taken inside the kernels (the probe library compiles
+    the product's kernel bodies once more with the stamps).  Every launch reads weights that no cache holds (copies walked
+    in turn), alone on the device; per stamp: the earliest, the mean and the latest workgroup, in us since the first
+    workgroup of the launch started, means over ten launches."""
+    torch, np, datagen, dev = env.torch, env.np, env.datagen, env.dev
+    stream = torch.cuda.current_stream().cuda_stream
+    num_cu = torch.cuda.get_device_properties(dev).multi_processor_count
+
+    def table(title, names, launch, per_wg, n_copies):
+        trace = torch.zeros(1024 * per_wg, dtype=torch.int64, device=dev)
+        rows, spans = [], []
+        for it in range(12):
+            trace.zero_()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            grid = launch(it % n_copies, trace)
+            e1.record()
+            torch.cuda.synchronize()
+            if grid <= 0:
+                sys.exit(f"bench.py: the timeline probe does not cover {title}")
+            if it < 2:
+                continue
+            tr = trace.cpu().numpy().reshape(-1, per_wg)[:grid].astype(np.float64)
+            rel = (tr - tr[:, 0].min()) / 100.0
+            rel[tr == 0] = np.nan
+            rows.append(rel)
+            spans.append(e0.elapsed_time(e1) * 1e3)
+        rel = np.nanmean(np.stack(rows), axis=0)
+        print(f"{title}: grid {grid}; events around the launch (eager, launch overhead included): {sum(spans) / len(spans):.1f} us")
+        print(f"    {'stamp':<58} {'first':>8} {'mean':>8} {'last':>8}")
+        for i, name in names:
+            col = rel[:, i]
+            if not np.all(np.isnan(col)):
+                print(f"    {name:<58} {np.nanmin(col):>8.2f} {np.nanmean(col):>8.2f} {np.nanmax(col):>8.2f}")
+        print()
+
+    gemv_names = [(0, "workgroup starts"), (1, "activations and scales arrived (first wavefront)"),
+                  (2, "activations prepared by every wavefront"), (3, "first row's weights arrived"),
+                  (4, "first wavefront's last row added up"), (5, "every wavefront's last row added up"), (7, "outputs written, end")]
+    for (n, k) in DECODE_SHAPES:
+        a, wq, s = datagen.w4a16_case(0, 1, n, k)
+        ta = env.dev_t(a)
+        copies = [(env.dev_t(wq), env.dev_t(s)) for _ in range(max(2, -(-COLD_FOOTPRINT_BYTES // wq.nbytes)))]
+        y = torch.empty((1, n), dtype=torch.float16, device=dev)
+        us = w4a16_bytes(1, n, k) / 8e3 / 1e3
+
+        def launch(c, trace, ta=ta, copies=copies, y=y, n=n, k=k):
+            return probes.nnf_probe_gemv_timeline(stream, ta.data_ptr(), copies[c][0].data_ptr(), copies[c][1].data_ptr(), y.data_ptr(),
+                                                  n, k, trace.data_ptr(), num_cu)
+
+        table(f"single-row GEMV N={n} K={k} ({w4a16_bytes(1, n, k)} bytes: {us:.2f} us at 8 TB/s)", gemv_names, launch, 8, len(copies))
+        del copies
+
+    gemm_names = [(0, "workgroup starts"), (1, "first operands arrived"), (2, "K loop of its last segment over"), (3, "its part parked"),
+                  (4, "... and counted in"), (5, "waits for the other workgroups of its shared tiles over"),
+                  (6, "its share of those tiles finished"), (9, "end")]
+    ws = env.workspace(256 << 20)
+    for (m, n, k, cols) in ((128, 8192, 8192, 128), (256, 2 * MLP_HI[1], MLP_HI[0], 256), (256, MLP_HI[0], MLP_HI[1], 128)):
+        if k % 256:
+            continue
+        _, wq, s = datagen.w4a16_case(0, 1, n, k)
+        ta = env.dev_t(datagen.normal_f16(0, datagen.S_ACT, (m, k)))
+        copies = [(env.dev_t(wq), env.dev_t(s)) for _ in range(max(2, -(-COLD_FOOTPRINT_BYTES // wq.nbytes)))]
+        y = torch.empty((m, n), dtype=torch.float16, device=dev)
+
+        def launch(c, trace, ta=ta, copies=copies, y=y, m=m, n=n, k=k, cols=cols):
+            return probes.nnf_probe_gemm_timeline(stream, ta.data_ptr(), copies[c][0].data_ptr(), copies[c][1].data_ptr(), y.data_ptr(),
+                                                  m, n, k, cols, ws.data_ptr(), ws.numel(), env.sync.data_ptr(), env.sync.numel(),
+                                                  trace.data_ptr(), num_cu)
+
+        table(f"tile GEMM (one launch, 128 x {cols} tiles) M={m} N={n} K={k}", gemm_names, launch, 16, len(copies))
+        del copies
+
+
 def run_mfma_probe(env, probes):
     """MFMA-only loops (operands in registers, two wavefronts per SIMD, eight accumulators each): the rate the
     matrix cores sustain depends on the operand values, because the chip is power managed."""
@@ -594,7 +680,8 @@ def extra_rows(env):
         ws = env.workspace(lib.nnf_w4a16_gemm_workspace_bytes(m, n, k, GROUP))
         rows.append({"key": f"w4a16_gemm_N{n}_K{k}.M{m}", "group": f"w4a16_gemm_N{n}_K{k}", "M": m,
                      "bytes": w4a16_bytes(m, n, k), "ops": 2.0 * m * n * k, "int8": False, "weights": (twq, ts),
-                     "make": (lambda w, sc, a=a, y=y, ws=ws: (lambda: ops.w4a16_gemm(a, w, sc, out=y, workspace=ws)))})
+                     "make": (lambda w, sc, a=a, y=y, ws=ws: (lambda: ops.w4a16_gemm_variant(a, w, sc, "auto", out=y, workspace=ws,
+                                                                                            sync=env.sync)))})
     _, _, w8, s_ch = datagen.w8a8_case(0, 1, n, k)
     tw8, tsch = env.dev_t(w8), env.dev_t(s_ch)
     for m in W8A8_MS:
@@ -627,7 +714,7 @@ def extra_rows(env):
         rows.append({"key": f"fused_mlp_M{m}_{h}_{i}", "group": None, "M": m, "bytes": mlp_bytes(m, h, i),
                      "ops": 2.0 * m * (2 * i) * h + 2.0 * m * h * i, "int8": False, "weights": (wgu, sgu, wd, sd),
                      "make": (lambda a, b, c, d, x=x, out=out, wsm=wsm:
-                              (lambda: ops.fused_mlp_w4a16(x, gamma, a, b, c, d, out=out, workspace=wsm)))})
+                              (lambda: ops.fused_mlp_w4a16(x, gamma, a, b, c, d, out=out, workspace=wsm, sync=env.sync)))})
     return rows
 
 
@@ -659,6 +746,7 @@ def run_extra(env, traffic):
     algorithmic byte exceed peak operations / peak bandwidth, else HBM's."""
     torch = env.torch
     res, roofs = {}, []
+    row_kernels = load_row_kernels()
     for row in extra_rows(env):
         if row["M"] <= 128:
             sets = env.copies_of(*row["weights"])
@@ -678,7 +766,7 @@ def run_extra(env, traffic):
             entry.pop("M")
             res[row["key"]] = entry
         mfma_bound = row["ops"] / row["bytes"] > peak_ops * 1e12 / (HBM_PEAK_GBS * 1e9)
-        roofs.append({"row": row["key"], "kernel": DOMINANT_KERNEL.get(row["key"]),
+        roofs.append({"row": row["key"], "kernel": row_kernels.get(row["key"]),
                       "bound": "mfma" if mfma_bound else "hbm",
                       "achieved": round(rate if mfma_bound else gbs, 1),
                       "peak": peak_ops if mfma_bound else HBM_PEAK_GBS,
@@ -697,27 +785,35 @@ def run_extra(env, traffic):
             total_traffic = None if (t is None or total_traffic is None) else total_traffic + t
             del sets
         sweep.append({"M": m, "us_per_sweep": round(total_us, 2), "GB/s": round(total_bytes / total_us / 1e3, 1)})
-        roofs.append({"row": f"decode_sweep_M{m}", "kernel": "nnf::w4a16_mrows_kernel / w4a16_mrows_any_kernel (+ splitk_reduce_kernel at K=11008)",
+        roofs.append({"row": f"decode_sweep_M{m}", "kernel": " | ".join(sorted({row_kernels.get(sh["key"], "?") for sh in shapes})),
                       "bound": "hbm", "achieved": round(total_bytes / total_us / 1e3, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                       "frac": round(total_bytes / total_us / 1e3 / HBM_PEAK_GBS, 4), "traffic": total_traffic,
                       "algorithmic_bytes": int(total_bytes), "us_per_launch": round(total_us, 2)})
     res["w4a16_decode_sweep_small_batches"] = sweep
-    # For scale only: the vendor library's unquantized GEMMs on the same box and value distributions (fp16 weights,
-    # four times the bytes, no unpacking; int8 x int8 -> int32 without the scaling epilogue), M = 4096, N = K = 8192.
+    # For scale only: the vendor library's unquantized GEMMs on the same box and value distributions (fp16 weights, four
+    # times the bytes, no unpacking; int8 x int8 -> int32 without the scaling epilogue) at the shapes of the compute-bound
+    # rows: N = K = 8192 at M = 128 .. 4096, and the two products of the MLP block at M = 256.
+    vendor = {}
     try:
-        m, n, k = 4096, 8192, 8192
         dev = env.dev
-        a = torch.randn(m, k, device=dev, dtype=torch.float16)
-        w = torch.randn(n, k, device=dev, dtype=torch.float16)
-        y = torch.empty(m, n, device=dev, dtype=torch.float16)
-        us16 = env.time_us(lambda: torch.matmul(a, w.t(), out=y), 20)
-        a8 = torch.randint(-127, 128, (m, k), device=dev, dtype=torch.int8)
-        w8 = torch.randint(-127, 128, (n, k), device=dev, dtype=torch.int8)
-        us8 = env.time_us(lambda: torch._int_mm(a8, w8.t()), 20)
-        res["vendor_library_for_scale_M4096"] = {"fp16_matmul_us": round(us16, 1), "fp16_TFLOP/s": round(2.0 * m * n * k / us16 / 1e6, 1),
-                                                 "int8_mm_us": round(us8, 1), "int8_TOP/s": round(2.0 * m * n * k / us8 / 1e6, 1)}
+        for (m, n, k, int8_too) in ((128, 8192, 8192, False), (512, 8192, 8192, True), (1024, 8192, 8192, False),
+                                    (4096, 8192, 8192, True), (256, 2 * MLP_HI[1], MLP_HI[0], False), (256, MLP_HI[0], MLP_HI[1], False)):
+            a = torch.randn(m, k, device=dev, dtype=torch.float16)
+            w = torch.randn(n, k, device=dev, dtype=torch.float16)
+            y = torch.empty(m, n, device=dev, dtype=torch.float16)
+            us16 = env.time_us(lambda: torch.matmul(a, w.t(), out=y), 20)
+            entry = {"fp16_matmul_us": round(us16, 1), "fp16_TFLOP/s": round(2.0 * m * n * k / us16 / 1e6, 1)}
+            del a, w, y
+            if int8_too:
+                a8 = torch.randint(-127, 128, (m, k), device=dev, dtype=torch.int8)
+                w8 = torch.randint(-127, 128, (n, k), device=dev, dtype=torch.int8)
+                us8 = env.time_us(lambda: torch._int_mm(a8, w8.t()), 20)
+                entry.update({"int8_mm_us": round(us8, 1), "int8_TOP/s": round(2.0 * m * n * k / us8 / 1e6, 1)})
+                del a8, w8
+            vendor[f"M{m}_N{n}_K{k}"] = entry
     except Exception as e:  # a yardstick, not part of the benchmark
-        res["vendor_library_for_scale_M4096"] = {"error": str(e)[:200]}
+        vendor["error"] = str(e)[:200]
+    res["vendor_library_for_scale"] = vendor
     return res, roofs
 
 

@@ -49,8 +49,8 @@ namespace nnfusion
                         nnf::workspace::route_w4a16(M, N, K, gate, rms, false, nnf::workspace::PLAN_CUS);
                     if (route.kind != nnf::workspace::W4A16Route::TILE)
                         return "";
-                    const size_t bytes = ((size_t)route.plan.tiles_m * route.plan.tiles_n * 2 * sizeof(uint32_t) + 63) & ~(size_t)63;
-                    if (bytes > NNF_SYNC_FLAGS_BYTES)
+                    const size_t bytes = (route.plan.sync_bytes(rms) + 63) & ~(size_t)63;
+                    if (bytes == 0 || bytes > NNF_SYNC_FLAGS_BYTES)
                         return "";
                     auto flags = allocate_tensor(Shape{bytes}, element::character, "", ROCM_GPU, true);
                     flags->set_memset(true, 0);

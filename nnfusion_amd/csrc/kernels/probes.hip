@@ -362,3 +362,56 @@ extern "C" int nnf_probe_gemm_timeline(void* stream, const void* A, const void* 
     }
     return hipGetLastError() == hipSuccess ? plan.grid : -1;
 }
+
+// ---- where a launch of the single-row GEMV spends its time -------------------------------------------------------------
+// The product's own kernel body (w4a16_gemv_rows.h), compiled here once more with time stamps: per workgroup and for its
+// first wavefront, eight stamps of the 100 MHz clock (0 start, 1 activations and scales arrived, 2 activations prepared by
+// every wavefront, 3 the first row's weights arrived, 4 its last row added up, 5 every wavefront's, 7 outputs written).
+// For the plans of the decode shapes (K = 4096: two loads per row, K = 11008: three loads per half row; two rows in
+// flight).  Returns the grid, or -1.
+__device__ unsigned long long* g_rows_trace;
+#define NNF_ROWS_TRACE g_rows_trace
+#include "w4a16_gemv_rows.h"
+
+namespace
+{
+    template <int SEG, int D>
+    __global__ __launch_bounds__(nnf::workspace::ROWS_WAVES * 64) void gemv_rows_traced_kernel(const nnf::half_t* __restrict__ A,
+                                                                                               const uint8_t* __restrict__ Wq,
+                                                                                               const nnf::half_t* __restrict__ S,
+                                                                                               nnf::half_t* __restrict__ Y, int N, int K,
+                                                                                               int rows_q, int rows_r, int pack)
+    {
+        nnf::gemv_rows_body<SEG, D, nnf::workspace::ROWS_WAVES, 0>(A, Wq, S, Y, N, K, rows_q, rows_r, pack,
+                                                                   nnf::GemvFusionArgs{nullptr, nullptr, nullptr, nullptr, 0.f});
+    }
+
+    template <int SEG, int D>
+    int launch_traced(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int N, int K, int grid,
+                      const nnf::workspace::RowsPlan& p)
+    {
+        const size_t lds_total = p.lds_bytes(N, K, grid, false);
+        auto kernel = &gemv_rows_traced_kernel<SEG, D>;
+        if (lds_total > nnf::MAX_LDS_BYTES ||
+            hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)nnf::MAX_LDS_BYTES) != hipSuccess)
+            return -1;
+        hipLaunchKernelGGL(kernel, dim3(grid), dim3(nnf::workspace::ROWS_WAVES * 64), lds_total, stream, (const nnf::half_t*)A,
+                           (const uint8_t*)Wq, (const nnf::half_t*)S, (nnf::half_t*)Y, N, K, N / grid, N % grid, 8 | (p.kshift << 8));
+        return hipGetLastError() == hipSuccess ? grid : -1;
+    }
+} // namespace
+
+extern "C" int nnf_probe_gemv_timeline(void* stream, const void* A, const void* Wq, const void* S, void* Y, int N, int K,
+                                       unsigned long long* trace, int num_cu)
+{
+    using namespace nnf;
+    const workspace::RowsPlan p = workspace::plan_w4a16_rows(1, N, K, num_cu);
+    const int grid = workspace::rows_grid(N, num_cu);
+    if (p.seg == 0 || !trace || hipMemcpyToSymbol(HIP_SYMBOL(g_rows_trace), &trace, sizeof(trace)) != hipSuccess)
+        return -1;
+    if (p.seg == 2 && p.depth == 2)
+        return launch_traced<2, 2>((hipStream_t)stream, A, Wq, S, Y, N, K, grid, p);
+    if (p.seg == 3 && p.depth == 2)
+        return launch_traced<3, 2>((hipStream_t)stream, A, Wq, S, Y, N, K, grid, p);
+    return -1;
+}

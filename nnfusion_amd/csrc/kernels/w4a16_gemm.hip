@@ -272,8 +272,16 @@ namespace nnf
             p.trace = nullptr;
             // (the one-launch form addresses the parked tiles with 32-bit byte offsets)
             const bool one_launch = plan.slots && choice.sync_flags && choice.sync_bytes >= plan.sync_bytes() && plan.bytes() < ((size_t)1 << 32);
-            p.sync = one_launch ? (uint32_t*)choice.sync_flags : nullptr;
+            p.sync = one_launch ? (uint32_t*)choice.sync_flags + 2 : nullptr; // (the first two words: rstd_sync)
             p.spin_limit = choice.spin_limit > 0 ? choice.spin_limit : choice.spin_limit < 0 ? 0 : DEFAULT_SPIN_LIMIT;
+            p.rstd_out = nullptr;
+            p.rstd_sync = nullptr;
+            p.rms_eps = 0.f;
+        }
+        // RMSNorm's rstd[] can be left to the GEMM launch itself: the caller gave (zeroed) synchronisation words
+        bool rstd_inside_tile_gemm(const workspace::SkPlan& plan, const LaunchChoice& choice)
+        {
+            return choice.sync_flags && choice.sync_bytes >= plan.sync_bytes(true);
         }
     } // namespace
 
@@ -297,8 +305,9 @@ namespace nnf
         // (the row-streaming kernels add up the squares of the activations they hold themselves: no pre-pass; the form
         // with a run-time K keeps it)
         const bool normalised_copy = route.kind == W4A16Route::SKINNY || route.kind == W4A16Route::SKINNY_SPLIT;
-        const bool rstd_in_kernel =
-            route.kind == W4A16Route::ROWS || (route.kind == W4A16Route::MROWS && workspace::w4a16_mrows_fixed_k(M, K));
+        const bool rstd_in_tile_gemm = rms && route.kind == W4A16Route::TILE && rstd_inside_tile_gemm(route.plan, choice);
+        const bool rstd_in_kernel = route.kind == W4A16Route::ROWS ||
+                                    (route.kind == W4A16Route::MROWS && workspace::w4a16_mrows_fixed_k(M, K)) || rstd_in_tile_gemm;
         if (rms && !rstd_in_kernel)
         {
             if (normalised_copy)
@@ -393,6 +402,12 @@ namespace nnf
         p.units = plan.units;
         p.zps = nullptr;
         set_sync(p, plan, choice);
+        if (rstd_in_tile_gemm)
+        {
+            p.rstd_out = (float*)rms_ws;
+            p.rstd_sync = (uint32_t*)choice.sync_flags;
+            p.rms_eps = rms_eps;
+        }
         if (plan.tile_weight_rows == 128)
             return plan.tile_rows == 256 ? launch_gemm_sk_256_narrow(stream, p, plan.grid)
                    : plan.tile_rows == 128 ? launch_gemm_sk_128_narrow(stream, p, plan.grid)

@@ -46,8 +46,10 @@
 //     once all have arrived, in the same K order (same bits as the second launch gives).
 //   * Epilogues round the way the unfused graph would: the GEMM result to fp16 first, then the
 //     element-wise operation in fp32, then fp16 again.  RMSNorm is folded in without materialising the
-//     normalised activations: gamma[k] multiplies the weights as they are unpacked, rstd[m] (from a
-//     small pre-pass over A) multiplies the fp32 row sums.
+//     normalised activations: gamma[k] multiplies the weights as they are unpacked, rstd[m] multiplies the
+//     fp32 row sums.  rstd[] comes from a small pre-pass over A, or (SkGemmParams::rstd_out, one-launch form) from
+//     the launch itself: every workgroup adds up the squares of a few rows before its first tile, and an
+//     epilogue waits (bounded) until all have.
 #pragma once
 
 #include "nnf_device.h"
@@ -79,6 +81,12 @@ namespace nnf
         // second launch follows.
         uint32_t* sync;
         int spin_limit;         // polls of a tile's arrival count before a workgroup leaves its share to the last arriver
+        // RMS without a pass of its own: non-null, the launch computes rstd[] itself -- workgroup v the rows v, v + grid,
+        // ... before its first tile, into `rstd_out` (= rstd) -- and counts in rstd_sync[0] the workgroups that have done
+        // so, in rstd_sync[1] those that have ended (two more words, zero at the start, zero again at the end).
+        float* rstd_out;
+        uint32_t* rstd_sync;
+        float rms_eps;
         // NNF_SK_TRACE builds only (the measurement probes): 16 time stamps of the 100 MHz clock per workgroup, or null
         unsigned long long* trace;
     };
@@ -302,8 +310,8 @@ namespace nnf
         {
             const int i = r * ROUND_TM + ii;
             float rs = 1.0f;
-            if (RMS)
-                rs = p.rstd[min(m0 + i * 32 + l32, p.M - 1)];
+            if (RMS) // (device scope: other workgroups of this launch may have written it)
+                rs = __hip_atomic_load(p.rstd + min(m0 + i * 32 + l32, p.M - 1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 #pragma unroll
             for (int j = 0; j < OUT_TN; ++j)
 #pragma unroll
@@ -471,6 +479,40 @@ namespace nnf
         sk_finish_round<1, TN, GATE, BIAS, RESID, RMS>(p, c, r, m0, n0, stage, wave, lane);
     }
 
+    // rstd[m] = rsqrt(mean_k(A[m, k]^2) + eps) for rows first, first + step, ... < end by the 256 threads of a workgroup
+    // (the summation order of the pre-pass kernel, rms_rstd_kernel: same bits), stored at device scope; complete for
+    // every thread of the workgroup on return.  part: four floats of LDS.
+    __device__ __forceinline__ void sk_rstd_rows(const SkGemmParams& p, int first, int end, int step, float* part, int tid)
+    {
+        const int units = p.K >> 3;
+        for (int m = first; m < end; m += step)
+        {
+            const uintx4* row = reinterpret_cast<const uintx4*>(p.A + (size_t)m * p.K);
+            float ss = 0.f;
+            for (int i = tid; i < units; i += gemm_sk::THREADS)
+            {
+                const uintx4 v = row[i];
+                const uint32_t vv[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                {
+                    const half2_t hh = as_half2(vv[j]);
+                    ss += (float)hh.x * (float)hh.x + (float)hh.y * (float)hh.y;
+                }
+            }
+            ss = wave_sum(ss);
+            if ((tid & 63) == 0)
+                part[tid >> 6] = ss;
+            __syncthreads();
+            if (tid == 0)
+                __hip_atomic_store(p.rstd_out + m, 1.0f / __builtin_sqrtf(((part[0] + part[1]) + (part[2] + part[3])) / (float)p.K + p.rms_eps),
+                                   __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __syncthreads();
+        }
+        gemm_sk::wait_vector_memory();
+        __syncthreads();
+    }
+
     // SkGemmParams::sync, word 0 of a tile: bits 0 .. 15 count the workgroups that have parked their part of it, bits
     // 16 .. 23 mark the 32-row blocks whose owner stopped waiting (the last arriver takes them over); word 1 counts the
     // blocks that are finished: whoever finishes the last one sets both words to zero again.
@@ -555,6 +597,48 @@ namespace nnf
         }
         const long long u_begin = first_unit_of(v, p.units, grid), u_end = first_unit_of(v + 1, p.units, grid);
         NNF_SK_STAMP(0); // the workgroup runs
+
+        // ---- (rstd_out) RMSNorm's rstd[] inside this launch: this workgroup's rows now, counted in once they are
+        // visible to every CU; an epilogue looks at the count before it reads rstd[] (ensure_rstd) ------------------
+        __shared__ float rstd_part[4];
+        __shared__ uint32_t rstd_note;
+        bool rstd_ok = true; // (uniform) rstd[] is known to be complete
+        if constexpr (RMS)
+        {
+            if (p.rstd_out)
+            {
+                rstd_ok = false;
+                sk_rstd_rows(p, v, p.M, grid, rstd_part, tid);
+                if (tid == 0)
+                    atomicAdd(p.rstd_sync, 1u);
+            }
+        }
+        // before an epilogue of rows [m_first, m_end): every workgroup has counted itself in -- or, when the (bounded)
+        // wait for that runs out, the rows are computed here (the same values, whoever stores them)
+        auto ensure_rstd = [&](int m_first, int m_end) {
+            if constexpr (RMS)
+            {
+                if (rstd_ok)
+                    return;
+                if (tid == 0)
+                {
+                    uint32_t seen = 0u;
+                    for (int polls = 0; polls < p.spin_limit; ++polls)
+                    {
+                        seen = __hip_atomic_load(p.rstd_sync, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        if (seen == (uint32_t)grid)
+                            break;
+                        __builtin_amdgcn_s_sleep(2);
+                    }
+                    rstd_note = seen == (uint32_t)grid ? 1u : 0u;
+                }
+                __syncthreads();
+                rstd_ok = rstd_note != 0u;
+                __syncthreads();
+                if (!rstd_ok)
+                    sk_rstd_rows(p, m_first, min(m_end, p.M), 1, rstd_part, tid);
+            }
+        };
 
         // (q - zp) from (1024 + q_even, 64 + q_odd): exact
         const half2_t dq_add = half2_t{(half_t)(-(1024.0f + (float)p.zp)), (half_t)(-(64.0f + (float)p.zp))};
@@ -1073,6 +1157,7 @@ namespace nnf
             {
                 // ---- epilogue: two blocks of 32 rows at a time ------------------------------------------------------
                 constexpr int ROUND_TM = TM >= 2 ? 2 : 1;
+                ensure_rstd(m0, m0 + BM);
 #pragma unroll
                 for (int r = 0; r < TM / ROUND_TM; ++r)
                 {
@@ -1122,6 +1207,20 @@ namespace nnf
             blocks[0] = pend_tile[0] >= 0 ? sync_note[0] : 0u;
             blocks[1] = pend_tile[1] >= 0 ? sync_note[1] : 0u;
             NNF_SK_STAMP(5); // the waits for the tiles' other workgroups are over
+            if constexpr (RMS)
+            {
+#pragma unroll
+                for (int slot = 0; slot < 2; ++slot)
+                    if (blocks[slot]) // (uniform)
+                    {
+                        // the tile's rows (tiles are numbered as in the K loop: four tile rows advance together along N)
+                        const int per_group = 4 * p.tiles_n;
+                        const int g = shared[slot].tile / per_group;
+                        const int gm = min(4, p.tiles_m - g * 4);
+                        const int tm = g * 4 + (shared[slot].tile - g * per_group) % gm;
+                        ensure_rstd(tm * BM, tm * BM + BM);
+                    }
+            }
             // (every part was complete at device scope before its workgroup counted itself in, the counts were read at
             // device scope, and so are the parts)
             // The blocks to finish, those of the first tile in bits 0 .. 7, of the second in bits 8 .. 15, one after the
@@ -1190,6 +1289,15 @@ namespace nnf
                     }
             }
         }
+        if constexpr (RMS)
+        {
+            // (rstd_out) the last workgroup to end leaves the two words as the next launch wants them
+            if (p.rstd_out && tid == 0 && atomicAdd(p.rstd_sync + 1, 1u) == (uint32_t)(grid - 1))
+            {
+                atomicExch(p.rstd_sync, 0u);
+                atomicExch(p.rstd_sync + 1, 0u);
+            }
+        }
         NNF_SK_STAMP(9); // done
     }
 
@@ -1202,7 +1310,6 @@ namespace nnf
     __global__ __launch_bounds__(64) void w4a16_gemm_sk_fixup_kernel(SkGemmParams p, int gemm_grid)
     {
         using namespace gemm_sk;
-        using T = Tile<TM, TN>;
         constexpr int ROUND_TM = 1, ROUNDS = TM; // (the epilogue routine of a tile one block high)
         __shared__ __attribute__((aligned(16))) uint8_t stage[ROUND_TM * 32 * (TN * 64 + 16)];
         const int lane = threadIdx.x;

@@ -186,12 +186,28 @@ namespace nnf
                                                       uint32_t parked_addr, int rbuf, int it, int M, int tid)
     {
         const int lane = tid & 63, col = lane & 15, kq = lane >> 4;
-#pragma unroll
-        for (int mb = 0; mb < MB; ++mb)
-        {
-            const uint32_t at = red_addr + (uint32_t)(rbuf * MR_WAVES * MB * 1024 + mb * 1024);
-            asm volatile("ds_write_b128 %0, %1" ::"v"(at), "v"(acc[mb]) : "memory");
-        }
+        // Hazard: the accumulators may come straight out of an MFMA, and a read of an MFMA's result needs wait states
+        // after it (up to 19 for a 16-pass MFMA) that the compiler inserts only ahead of instructions it emits itself,
+        // not ahead of inline assembly.  They are therefore part of the block that holds the stores: one block, which
+        // reads every accumulator, so that no MFMA can be scheduled behind the wait states.
+        static_assert(MB >= 1 && MB <= 4, "up to four blocks of 16 rows");
+        const uint32_t at = red_addr + (uint32_t)(rbuf * MR_WAVES * MB * 1024);
+#define NNF_PARK_WAIT "s_nop 15\n\ts_nop 3\n\t"
+        if constexpr (MB == 1)
+            asm volatile(NNF_PARK_WAIT "ds_write_b128 %0, %1" ::"v"(at), "v"(acc[0]) : "memory");
+        else if constexpr (MB == 2)
+            asm volatile(NNF_PARK_WAIT "ds_write_b128 %0, %1\n\tds_write_b128 %0, %2 offset:1024" ::"v"(at), "v"(acc[0]), "v"(acc[MB - 1])
+                         : "memory");
+        else if constexpr (MB == 3)
+            asm volatile(NNF_PARK_WAIT "ds_write_b128 %0, %1\n\tds_write_b128 %0, %2 offset:1024\n\tds_write_b128 %0, %3 offset:2048" ::"v"(at),
+                         "v"(acc[0]), "v"(acc[1]), "v"(acc[MB - 1])
+                         : "memory");
+        else
+            asm volatile(NNF_PARK_WAIT "ds_write_b128 %0, %1\n\tds_write_b128 %0, %2 offset:1024\n\tds_write_b128 %0, %3 offset:2048\n\t"
+                                       "ds_write_b128 %0, %4 offset:3072" ::"v"(at),
+                         "v"(acc[0]), "v"(acc[1]), "v"(acc[2]), "v"(acc[MB - 1])
+                         : "memory");
+#undef NNF_PARK_WAIT
         asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
         for (int o = tid; o < MB * 256; o += MR_WAVES * 64) // (o & 63 == lane)
         {
@@ -541,8 +557,6 @@ namespace nnf
             z_sh[g] = (uint32_t)(i & 1) * 4u;
         }
         const uint32_t zp16 = (uint32_t)zp | ((uint32_t)zp << 16);
-        float one; // a 1.0 the compiler cannot fold
-        asm volatile("v_mov_b32 %0, 1.0" : "=v"(one));
         int slot = 0;
         for (int it = 0; it < T; ++it)
         {
@@ -600,16 +614,6 @@ namespace nnf
                                                                              __builtin_bit_cast(half8_t, bq), acc[mb], 0, 0, 0);
                     }
                 }
-            }
-            // (mrows_reduce_park stores the sums with inline assembly, and the wait between an MFMA and a read of its
-            // result is only inserted ahead of instructions the compiler emits itself: one such instruction)
-#pragma unroll
-            for (int mb = 0; mb < MB; ++mb)
-            {
-                acc[mb].x *= one;
-                acc[mb].y *= one;
-                acc[mb].z *= one;
-                acc[mb].w *= one;
             }
             mrows_reduce_park<MB>(acc, red, red_addr, parked_addr, it & 1, it, M, tid);
         }
@@ -749,8 +753,6 @@ namespace nnf
         }
         const uint32_t zp16 = (uint32_t)zp | ((uint32_t)zp << 16);
         const int sub = (kq * 32) >> GSHIFT; // the lane's scale within a block
-        float one; // a 1.0 the compiler cannot fold
-        asm volatile("v_mov_b32 %0, 1.0" : "=v"(one));
         int slot = 0;
         for (int it = 0; it < T; ++it)
         {
@@ -809,11 +811,6 @@ namespace nnf
                     }
                 }
             }
-            // (one compiler-emitted instruction between the MFMAs and the inline-assembly stores of mrows_reduce_park)
-            acc[0].x *= one;
-            acc[0].y *= one;
-            acc[0].z *= one;
-            acc[0].w *= one;
             mrows_reduce_park<MB>(acc, red, red_addr, parked_addr, it & 1, it, M, tid);
         }
         __builtin_amdgcn_s_waitcnt(mr_vmcnt(0)); // the reloads past the end, before the LDS goes away

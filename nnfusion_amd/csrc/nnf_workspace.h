@@ -128,9 +128,10 @@ namespace nnf
             int grid = 0;
             int slots = 0;     // 0: every tile belongs to one workgroup (no workspace, no second launch)
             size_t bytes() const { return (size_t)slots * tile_rows * tile_weight_rows * sizeof(float); }
-            // two synchronisation words per tile for the one-launch form (workgroups that share a tile add its parts
-            // up themselves); 0: no tile is shared
-            size_t sync_bytes() const { return slots ? (size_t)tiles_m * tiles_n * 2 * sizeof(unsigned) : 0; }
+            // Synchronisation words for the one-launch form: two for RMSNorm's rstd[] computed inside the launch, then
+            // two per tile (workgroups that share a tile add its parts up themselves).  0: no tile is shared and (rms)
+            // there is no RMSNorm
+            size_t sync_bytes(bool rms = false) const { return (slots || rms) ? ((size_t)tiles_m * tiles_n + 1) * 2 * sizeof(unsigned) : 0; }
         };
         // Tile shape.  What the caller fixes (forced_rows 32 / 64 / 128 / 256, forced_cols 128 / 256) is kept, the rest
         // is chosen by M (measured at N = K = 8192 and on the Llama shapes, alternating the candidates in one process):

@@ -359,13 +359,14 @@ int main(int argc, char** argv)
         auto k2 = sel.pick_first(n2, ROCM_GPU).second;
         auto fu2 = k2->get_or_emit_source();
         CONTAINS(fu2->body_unit->get_code(), "nnf_w4a16_gemm_fused_variant(stream, input0, input1, input2, output0, 256, 4096, 4096, 128, 8, input3, 1.000000000e-05f, input4, nullptr, NNF_ACT_NONE, NNF_W4A16_AUTO, &plan, ");
-        // ... and, because the product runs on the tile GEMM, a second tensor: its synchronisation words (two per tile:
-        // 2 x 16 tiles), persistent and cleared at initialisation, named by the nnf_plan the body declares
+        // ... and, because the product runs on the tile GEMM, a second tensor: its synchronisation words (two for rstd[],
+        // two per tile: 2 x 16 tiles; in whole 64 bytes), persistent and cleared at initialisation, named by the nnf_plan
+        // the body declares
         EXPECT(k2->m_context->tensors.size() == 2 &&
                k2->m_context->tensors[0]->size() == (size_t)256 * 4 + (size_t)256 * 128 * 256 * 4);
-        EXPECT(k2->m_context->tensors[1]->size() == 256 && k2->m_context->tensors[1]->is_persistent() &&
+        EXPECT(k2->m_context->tensors[1]->size() == 320 && k2->m_context->tensors[1]->is_persistent() &&
                k2->m_context->tensors[1]->is_memset() && k2->m_context->tensors[1]->get_memset_value() == 0);
-        CONTAINS(fu2->body_unit->get_code(), "const nnf_plan plan = {0, 0, 0, " + k2->m_context->tensors[1]->get_name() + ", 256, 0};");
+        CONTAINS(fu2->body_unit->get_code(), "const nnf_plan plan = {0, 0, 0, " + k2->m_context->tensors[1]->get_name() + ", 320, 0};");
         CONTAINS(fu2->signature_unit->get_code(), "char* " + k2->m_context->tensors[0]->get_name());
         CONTAINS(fu2->call_unit->get_code(), k2->m_context->tensors[1]->get_name() + ");");
         // SiLU gate: N is half the weight rows
@@ -444,11 +445,11 @@ int main(int argc, char** argv)
         // rstd [256] fp32 + h [256, 11008] fp16 + the larger of the two areas of parked sums: both GEMMs run 256
         // workgroups over tiles of 128 x 256 weight rows; gate/up (2 x 86 tiles x 16 supersteps) needs two slots per
         // workgroup
-        // ... and the synchronisation words of either product (2 x 86 and 1 x 32 tiles, two words each)
+        // ... and the synchronisation words of either product (2 x 86 and 1 x 32 tiles, two words each, and two more)
         EXPECT(k->m_context->tensors.size() == 3 &&
                k->m_context->tensors[0]->size() ==
                    (size_t)256 * 4 + (size_t)256 * 11008 * 2 + (size_t)2 * 256 * 128 * 256 * 4);
-        EXPECT(k->m_context->tensors[1]->size() == 1408 && k->m_context->tensors[2]->size() == 256 &&
+        EXPECT(k->m_context->tensors[1]->size() == 1408 && k->m_context->tensors[2]->size() == 320 &&
                k->m_context->tensors[1]->is_memset() && k->m_context->tensors[2]->is_memset());
     });
 

@@ -33,6 +33,15 @@ def test_library_exports_every_declared_symbol():
     assert not missing, missing
 
 
+def test_library_exports_nothing_but_the_header():
+    """Built with hidden visibility and a version script: the dynamic symbol table holds the header's functions only."""
+    import subprocess
+
+    out = subprocess.run(["nm", "-D", "--defined-only", _lib.KERNELS_SO], capture_output=True, text=True, check=True).stdout
+    exported = sorted(line.split()[-1] for line in out.splitlines() if line.split()[1:2] and line.split()[1] in "TW")
+    assert exported == _declared_functions(), sorted(set(exported) ^ set(_declared_functions()))
+
+
 def test_ctypes_table_covers_the_header():
     assert sorted(_lib.KERNEL_ABI) == _declared_functions()
 

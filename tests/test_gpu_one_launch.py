@@ -70,8 +70,12 @@ def test_one_launch_equals_two_launches(gpu, m, n, k, plan, spin_limit):
 
 
 @pytest.mark.parametrize("spin_limit", [0, -1], ids=["wait", "hand-over"])
-@pytest.mark.parametrize("fused", ["bias+residual", "rms+gate", "rms+bias", "residual-in-place"])
+@pytest.mark.parametrize("fused", ["bias+residual", "rms+gate", "rms+bias", "residual-in-place", "rms-whole-tiles"])
 def test_one_launch_fused_forms(gpu, fused, spin_limit):
+    """With RMSNorm the one-launch form also computes rstd[] inside the GEMM launch (every workgroup a few rows, counted in
+    two more synchronisation words; an epilogue whose wait for the count runs out -- forced here with the negative spin
+    limit -- adds up the rows it needs itself): the same bits as the pass of its own that the two-launch form runs.
+    rms-whole-tiles: no tile is shared (nothing is parked), only rstd[] goes through the synchronisation words."""
     import torch
 
     from nnfusion_amd import ops
@@ -84,7 +88,8 @@ def test_one_launch_fused_forms(gpu, fused, spin_limit):
     bias = rng.standard_normal(n).astype(np.float16) if "bias" in fused else None
     resid = rng.standard_normal((m, n)).astype(np.float16) if "residual" in fused else None
     ta, tw, ts, tg, tb, tr = _t(gpu, a, wq, s, gamma, bias, resid)
-    kw = dict(rms_gamma=tg, bias=tb, act=1 if gate else 0, variant="gemm_mfma", plan=(128, 3, 256 if gate else 128))
+    kw = dict(rms_gamma=tg, bias=tb, act=1 if gate else 0, variant="gemm_mfma",
+              plan=(128, 1 if fused == "rms-whole-tiles" else 3, 256 if gate else 128))
     ws = _ws(gpu)
     if fused == "residual-in-place":
         out_two, out_one = tr.clone(), tr.clone()
@@ -98,6 +103,34 @@ def test_one_launch_fused_forms(gpu, fused, spin_limit):
     torch.cuda.synchronize()
     assert int(sync.count_nonzero()) == 0
     assert torch.equal(one, two)
+    if "rms" in fused and not gate:
+        xn = oracle.rmsnorm_f16(a, gamma)
+        ref = oracle.w4a16_gemm(xn, wq, s, f32_out=True)
+        if bias is not None:
+            ref = ref + bias.astype(np.float32)[None, :]
+        # the product of the normalised activations; rstd applied to the fp32 sums instead of to fp16 activations
+        _check(one.cpu().numpy(), ref, 2e-2)
+
+
+@pytest.mark.parametrize("m,k", [(300, 1024), (1000, 4096)])
+def test_rstd_inside_the_launch_with_more_rows_than_workgroups(gpu, m, k):
+    """More activation rows than the launch has workgroups: each adds up the squares of several rows."""
+    import torch
+
+    from nnfusion_amd import ops
+
+    n = 512
+    a, wq, s = datagen.w4a16_case(4, m, n, k)
+    gamma = (1.0 + 0.1 * np.random.default_rng(2).standard_normal(k)).astype(np.float16)
+    ta, tw, ts, tg = _t(gpu, a, wq, s, gamma)
+    ws = _ws(gpu)
+    two = ops.w4a16_gemm_fused(ta, tw, ts, rms_gamma=tg, variant="gemm_mfma", workspace=ws)
+    sync = ops.sync_flags(gpu)
+    for spin_limit in (0, -1):
+        one = ops.w4a16_gemm_fused(ta, tw, ts, rms_gamma=tg, variant="gemm_mfma", workspace=ws, sync=sync, spin_limit=spin_limit)
+        torch.cuda.synchronize()
+        assert int(sync.count_nonzero()) == 0
+        assert torch.equal(one, two)
 
 
 @pytest.mark.parametrize("spin_limit", [0, -1], ids=["wait", "hand-over"])
