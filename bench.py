@@ -734,7 +734,8 @@ def small_batch_rows(env):
             y = torch.empty((m, sn), dtype=torch.float16, device=dev)
             ws = env.workspace(lib.nnf_w4a16_gemm_workspace_bytes(m, sn, sk, GROUP))
             shapes.append({"key": f"decode_sweep_M{m}.N{sn}_K{sk}", "bytes": w4a16_bytes(m, sn, sk), "weights": (twq, ts),
-                           "make": (lambda w, sc, a=a, y=y, ws=ws: (lambda: ops.w4a16_gemm(a, w, sc, out=y, workspace=ws)))})
+                           "make": (lambda w, sc, a=a, y=y, ws=ws: (lambda: ops.w4a16_gemm_variant(a, w, sc, "auto", out=y, workspace=ws,
+                                                                                                  sync=env.sync)))})
         out.append((m, shapes))
     return out
 

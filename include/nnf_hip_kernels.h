@@ -120,9 +120,9 @@ enum nnf_w4a16_variant
  * Passed per call: the library keeps no dispatch state, calls with different plans may run concurrently.
  * NULL, or a field that is 0: the library's own choice for the shape. */
 #define NNF_MAX_K_PARTS 64
-/* Synchronisation words for the one-launch form of the fp16 x int4 tile GEMM: two 32-bit words per output tile; a
- * buffer of NNF_SYNC_FLAGS_BYTES serves every shape up to 8192 tiles (a launch with more tiles than the buffer
- * given takes the two-launch form). */
+/* Synchronisation words for the one-launch forms of the fp16 x int4 kernels: two 32-bit words per output tile of the
+ * tile GEMM and two more; a buffer of NNF_SYNC_FLAGS_BYTES serves every shape up to 8191 tiles (a launch with more
+ * tiles than the buffer given takes the two-launch form). */
 #define NNF_SYNC_FLAGS_BYTES ((size_t)64 << 10)
 typedef struct nnf_plan
 {
@@ -135,11 +135,16 @@ typedef struct nnf_plan
     int tile_cols; /* columns of an output tile, 256 or 128 (0: the library's choice): W8A8 with 256-row tiles;
                       fp16 x int4 with 64-, 128- or 256-row tiles and no SiLU-gate (the gate | up halves need the
                       256 weight rows of a full tile); ignored elsewhere */
-    /* fp16 x int4 tile GEMM in one launch (any variant that ends up on it; ignored by every other kernel and by W8A8).
+    /* fp16 x int4 products in one launch (any variant that ends up on one of the kernels below; ignored by every other
+     * kernel and by W8A8).
      * The work of the GEMM is split evenly over the CUs, so most output tiles of a mid-sized product are shared by
      * several workgroups.  Without sync_flags their parts are added up by a second launch.  With sync_flags the
      * workgroups count themselves in at their tiles there, and each adds up and finishes its share of a tile's rows
      * once all that hold a part have arrived -- same summation order, bit-identical results, one launch less.
+     * Two more launches go the same way: a fused RMSNorm's rstd[] is computed by the GEMM launch itself (every
+     * workgroup a few rows before its first tile; no pass of its own), and the row-streaming kernel for a few
+     * activation rows and K above 8192, which works on ranges of K, adds the ranges up itself (the last workgroup to
+     * arrive at a group of columns, in the order of the ranges; no reduction pass).
      *   sync_flags: device memory, 16-byte aligned, ALL ZERO before the first call that uses it; every call leaves it
      *     all zero again, so it needs clearing once (when it is allocated), not per call.  It must not be scratch
      *     memory that other kernels write between calls, and calls that may overlap on the device (different

@@ -37,8 +37,8 @@ namespace nnfusion
                 using HipLibEmitter::HipLibEmitter;
 
             protected:
-                // Synchronisation words for the one-launch form of the tile GEMM (nnf_plan::sync_flags), when the product
-                // of these sizes runs on it: a persistent tensor that is zero when the runtime is initialised -- what
+                // Synchronisation words for the one-launch forms (nnf_plan::sync_flags), when the product of these sizes
+                // runs on the tile GEMM or on the row-streaming kernel over ranges of K: a persistent tensor that is zero when the runtime is initialised -- what
                 // be_state_buffer is to the reference's BlockFusion kernels
                 // (src/nnfusion/engine/pass/graph/blockfusion/blockfusion_codegen.cpp:295-304).  Every launch leaves the
                 // words zero again, so one tensor serves all launches of the emitted function.  Returns the statement
@@ -47,9 +47,13 @@ namespace nnfusion
                 {
                     const nnf::workspace::W4A16Route route =
                         nnf::workspace::route_w4a16(M, N, K, gate, rms, false, nnf::workspace::PLAN_CUS);
-                    if (route.kind != nnf::workspace::W4A16Route::TILE)
+                    // (the row-streaming kernel over ranges of K -- a few rows, K above 8192 -- adds its ranges up inside
+                    // its launch with one word per workgroup of a range)
+                    const bool split = route.kind == nnf::workspace::W4A16Route::MROWS_SPLIT && !gate;
+                    if (route.kind != nnf::workspace::W4A16Route::TILE && !split)
                         return "";
-                    const size_t bytes = (route.plan.sync_bytes(rms) + 63) & ~(size_t)63;
+                    const size_t bytes =
+                        ((split ? nnf::workspace::mrows_split_sync_bytes(nnf::workspace::PLAN_CUS) : route.plan.sync_bytes(rms)) + 63) & ~(size_t)63;
                     if (bytes == 0 || bytes > NNF_SYNC_FLAGS_BYTES)
                         return "";
                     auto flags = allocate_tensor(Shape{bytes}, element::character, "", ROCM_GPU, true);

@@ -103,8 +103,12 @@ namespace nnf
     // K above 8192: the same kernel over ranges of K, fp32 sums to partial[ranges][M][N] for the reduction pass
     int w4a16_mrows_ksplits(int M, int N, int K, int num_cu); // 0: does not apply
     // (gamma: fp16 [K] or null, the RMSNorm weight multiplied onto the activations)
+    // sync: w4a16_mrows_split_sync_bytes() of zeroed words (zero again afterwards): the launch adds the ranges up itself, in
+    // order, and writes epilogue(sums) to Y (rstd, bias, residual of `epilogue`; no gate): no reduction pass follows
+    size_t w4a16_mrows_split_sync_bytes(int num_cu);
     hipError_t launch_w4a16_mrows_split(hipStream_t stream, const void* A, const void* Wq, const void* S, float* partial,
-                                        int M, int N, int K, int zp, int num_cu, const void* gamma = nullptr);
+                                        int M, int N, int K, int zp, int num_cu, const void* gamma = nullptr, void* Y = nullptr,
+                                        const GemvFusion* epilogue = nullptr, uint32_t* sync = nullptr);
 
     hipError_t launch_w4a16_skinny(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M,
                                    int N, int K, int zp, int num_cu);

@@ -357,6 +357,17 @@ namespace nnf
         // (which applies rstd and the epilogue) ------------------------------------------------------------------
         if (route.kind == W4A16Route::MROWS_SPLIT || route.kind == W4A16Route::SKINNY_SPLIT)
         {
+            // (the row-streaming kernel adds its ranges up itself where the caller gave synchronisation words for it)
+            if (route.kind == W4A16Route::MROWS_SPLIT && !gate && choice.sync_flags &&
+                choice.sync_bytes >= w4a16_mrows_split_sync_bytes(num_cu))
+            {
+                GemvFusion epilogue;
+                epilogue.rstd = rstd;
+                epilogue.bias = bias;
+                epilogue.residual = residual;
+                return launch_w4a16_mrows_split(stream, A, Wq, S, (float*)partial_ws, M, n_rows, K, zp, num_cu, rms_gamma, Y, &epilogue,
+                                                (uint32_t*)choice.sync_flags);
+            }
             hipError_t e = route.kind == W4A16Route::MROWS_SPLIT
                                ? launch_w4a16_mrows_split(stream, A, Wq, S, (float*)partial_ws, M, n_rows, K, zp, num_cu, rms_gamma)
                                : launch_w4a16_skinny_split(stream, A, Wq, S, (float*)partial_ws, M, n_rows, K, zp, route.ksplits,

@@ -845,7 +845,8 @@ namespace nnf
     __global__ __launch_bounds__(512) void w4a16_mrows_any_kernel(const half_t* __restrict__ A, const uint8_t* __restrict__ Wq,
                                                                   const half_t* __restrict__ S, half_t* __restrict__ Y,
                                                                   float* __restrict__ partial, int N, int K, int range_groups,
-                                                                  int tiles_q, int tiles_r, int pack, GemvFusionArgs f, int gate)
+                                                                  int tiles_q, int tiles_r, int pack, GemvFusionArgs f, int gate,
+                                                                  uint32_t* sync)
     {
         static_assert(GW >= 1 && GW <= 7 && STEPS >= 1 && GW * STEPS <= 8, "groups per wavefront");
         static_assert(MB == 1 || (MB == 2 && GW * STEPS <= 4) || (MB == 4 && GW * STEPS <= 2), "16 VGPRs per group and block of rows");
@@ -991,7 +992,7 @@ namespace nnf
         }
         __builtin_amdgcn_s_waitcnt(mr_vmcnt(0)); // the reloads past the end, before the LDS goes away
         asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-        if (partial)
+        if (partial && !sync)
         {
             for (int idx = tid; idx < T * M * 16; idx += 512)
             {
@@ -999,6 +1000,63 @@ namespace nnf
                 const int im = idx >> 4;
                 const int it = im / M, m = im - it * M;
                 partial[(size_t)blockIdx.y * M * N + (size_t)m * N + min((t0 + it) * 16, N - 16) + n] = parked[idx];
+            }
+        }
+        else if (partial)
+        {
+            // ---- ranges of K added up inside the launch: the workgroups that walked these tiles (one per range: same
+            // blockIdx.x) count themselves in at sync[blockIdx.x] once their sums are visible to every CU (stores at device
+            // scope, completed); the last to arrive adds the ranges in order -- so the result does not depend on who that
+            // is -- runs the epilogue of the reduction pass (rstd, bias, residual: same roundings) and leaves the word zero
+            // for the next launch.  Nobody waits.
+            for (int idx = tid; idx < T * M * 16; idx += 512)
+            {
+                const int n = idx & 15;
+                const int im = idx >> 4;
+                const int it = im / M, m = im - it * M;
+                __hip_atomic_store(partial + (size_t)blockIdx.y * M * N + (size_t)m * N + min((t0 + it) * 16, N - 16) + n, parked[idx],
+                                   __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+            __builtin_amdgcn_s_waitcnt(mr_vmcnt(0));
+            // (a word of the partial tiles' LDS, free since the barrier above: the kernel's dynamic LDS may be all there is)
+            volatile uint32_t* arrived_before = reinterpret_cast<volatile uint32_t*>(red);
+            __syncthreads();
+            if (tid == 0)
+                *arrived_before = atomicAdd(sync + blockIdx.x, 1u);
+            __syncthreads();
+            if (*arrived_before == gridDim.y - 1)
+            {
+                const int ranges = (int)gridDim.y;
+                for (int idx = tid; idx < T * M * 16; idx += 512)
+                {
+                    const int n = idx & 15;
+                    const int im = idx >> 4;
+                    const int it = im / M, m = im - it * M;
+                    const int nn = min((t0 + it) * 16, N - 16) + n;
+                    if (nn < (t0 + it) * 16) // (a last tile moved back: these columns belong to the tile before it)
+                        continue;
+                    const size_t at = (size_t)m * N + nn;
+                    // (four ranges in flight, added in order)
+                    float sum = 0.f;
+                    for (int r0 = 0; r0 < ranges; r0 += 4)
+                    {
+                        float part[4];
+#pragma unroll
+                        for (int d = 0; d < 4; ++d)
+                            part[d] = __hip_atomic_load(partial + (size_t)min(r0 + d, ranges - 1) * M * N + at, __ATOMIC_RELAXED,
+                                                        __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+                        for (int d = 0; d < 4; ++d)
+                            if (r0 + d < ranges)
+                                sum += part[d];
+                    }
+                    if (FUSED)
+                        Y[at] = finish_bias_residual(sum * (f.rstd ? f.rstd[m] : 1.0f), f.bias, nn, f.residual, at);
+                    else
+                        Y[at] = (half_t)sum;
+                }
+                if (tid == 0)
+                    atomicExch(sync + blockIdx.x, 0u);
             }
         }
         else
@@ -1059,14 +1117,16 @@ namespace nnf
         // ranges == 1: the whole of K, fp16 results to Y; otherwise ranges of range_groups groups, fp32 sums to partial
         template <int GW, int STEPS, int MB, bool FUSED>
         hipError_t launch_mrows_any_mb(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M, int N, int K,
-                                       int zp, int num_cu, float* partial, int ranges, int range_groups, const GemvFusion& fusion)
+                                       int zp, int num_cu, float* partial, int ranges, int range_groups, const GemvFusion& fusion,
+                                       uint32_t* sync)
         {
             const int n_tiles = (N + 15) / 16;
             const int per_range = num_cu / ranges > 0 ? num_cu / ranges : 1;
             const int grid = n_tiles < per_range ? n_tiles : per_range;
             const int tiles_q = n_tiles / grid, tiles_r = n_tiles % grid;
             const size_t lds = workspace::w4a16_mrows_lds_bytes_gw(GW, M, (fusion.gate ? 2 : 1) * (tiles_q + (tiles_r ? 1 : 0)));
-            if (lds > MAX_LDS_BYTES || (ranges > 1 && (fusion.gate || fusion.bias || fusion.residual || fusion.rstd)))
+            // over ranges of K the epilogue belongs to whoever adds the ranges up: the reduction pass, or (sync) the launch itself
+            if (lds > MAX_LDS_BYTES || (ranges > 1 && (fusion.gate || (!sync && (fusion.bias || fusion.residual || fusion.rstd)))))
                 return hipErrorInvalidValue;
             auto kernel = &w4a16_mrows_any_kernel<GW, STEPS, MB, FUSED>;
             if (lds > 64 * 1024)
@@ -1078,37 +1138,38 @@ namespace nnf
             }
             hipLaunchKernelGGL(kernel, dim3(grid, ranges), dim3(MR_WAVES * 64), lds, stream, (const half_t*)A, (const uint8_t*)Wq,
                                (const half_t*)S, (half_t*)Y, ranges > 1 ? partial : nullptr, N, K, range_groups, tiles_q, tiles_r,
-                               M | (zp << 8), fusion_args(fusion), fusion.gate ? 1 : 0);
+                               M | (zp << 8), fusion_args(fusion), fusion.gate ? 1 : 0, ranges > 1 ? sync : nullptr);
             return hipGetLastError();
         }
 
         template <int GW, int STEPS, bool FUSED>
         hipError_t launch_mrows_any_f(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M, int N, int K,
-                                      int zp, int num_cu, float* partial, int ranges, int range_groups, const GemvFusion& fusion)
+                                      int zp, int num_cu, float* partial, int ranges, int range_groups, const GemvFusion& fusion,
+                                      uint32_t* sync)
         {
             if (M <= 16)
                 return launch_mrows_any_mb<GW, STEPS, 1, FUSED>(stream, A, Wq, S, Y, M, N, K, zp, num_cu, partial, ranges, range_groups,
-                                                                fusion);
+                                                                fusion, sync);
             if constexpr (GW * STEPS <= 4)
                 if (M <= 32)
                     return launch_mrows_any_mb<GW, STEPS, 2, FUSED>(stream, A, Wq, S, Y, M, N, K, zp, num_cu, partial, ranges,
-                                                                    range_groups, fusion);
+                                                                    range_groups, fusion, sync);
             if constexpr (GW * STEPS <= 2)
                 if (M <= 64)
                     return launch_mrows_any_mb<GW, STEPS, 4, FUSED>(stream, A, Wq, S, Y, M, N, K, zp, num_cu, partial, ranges,
-                                                                    range_groups, fusion);
+                                                                    range_groups, fusion, sync);
             return hipErrorInvalidValue;
         }
 
         template <int GW, int STEPS>
         hipError_t launch_mrows_any(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M, int N, int K,
                                     int zp, int num_cu, const GemvFusion& fusion, float* partial = nullptr, int ranges = 1,
-                                    int range_groups = 64)
+                                    int range_groups = 64, uint32_t* sync = nullptr)
         {
             return fusion.any() ? launch_mrows_any_f<GW, STEPS, true>(stream, A, Wq, S, Y, M, N, K, zp, num_cu, partial, ranges,
-                                                                      range_groups, fusion)
+                                                                      range_groups, fusion, sync)
                                 : launch_mrows_any_f<GW, STEPS, false>(stream, A, Wq, S, Y, M, N, K, zp, num_cu, partial, ranges,
-                                                                       range_groups, fusion);
+                                                                       range_groups, fusion, sync);
         }
     } // namespace
 
@@ -1293,20 +1354,32 @@ namespace nnf
     // partial[ranges][M][N] (the caller runs the reduction pass).  Returns the number of ranges; 0: does not apply.
     int w4a16_mrows_ksplits(int M, int N, int K, int num_cu) { return workspace::w4a16_mrows_split(M, N, K, num_cu).ranges; }
 
+    size_t w4a16_mrows_split_sync_bytes(int num_cu) { return workspace::mrows_split_sync_bytes(num_cu); }
+
     hipError_t launch_w4a16_mrows_split(hipStream_t stream, const void* A, const void* Wq, const void* S, float* partial, int M,
-                                        int N, int K, int zp, int num_cu, const void* gamma)
+                                        int N, int K, int zp, int num_cu, const void* gamma, void* Y, const GemvFusion* epilogue,
+                                        uint32_t* sync)
     {
-        GemvFusion fusion; // of the fused parts only the RMSNorm weight belongs to this launch
+        // Of the fused parts only the RMSNorm weight belongs to the sums of a range.  With synchronisation words (one per
+        // workgroup of a range, zero before and after) the launch adds the ranges up itself and runs `epilogue` (rstd,
+        // bias, residual) on the way to Y; without them the sums stay in `partial` for the reduction pass.
+        GemvFusion fusion;
+        if (sync)
+        {
+            if (!Y || !epilogue || epilogue->gate)
+                return hipErrorInvalidValue;
+            fusion = *epilogue;
+        }
         fusion.gamma = gamma;
         const workspace::MrowsSplit sp = workspace::w4a16_mrows_split(M, N, K, num_cu);
         if (sp.ranges < 2 || !partial)
             return hipErrorInvalidValue;
         switch (sp.gw)
         {
-        case 1: return launch_mrows_any<1, 2>(stream, A, Wq, S, nullptr, M, N, K, zp, num_cu, fusion, partial, sp.ranges, sp.range_groups);
-        case 2: return launch_mrows_any<2, 2>(stream, A, Wq, S, nullptr, M, N, K, zp, num_cu, fusion, partial, sp.ranges, sp.range_groups);
-        case 3: return launch_mrows_any<3, 2>(stream, A, Wq, S, nullptr, M, N, K, zp, num_cu, fusion, partial, sp.ranges, sp.range_groups);
-        default: return launch_mrows_any<4, 2>(stream, A, Wq, S, nullptr, M, N, K, zp, num_cu, fusion, partial, sp.ranges, sp.range_groups);
+        case 1: return launch_mrows_any<1, 2>(stream, A, Wq, S, Y, M, N, K, zp, num_cu, fusion, partial, sp.ranges, sp.range_groups, sync);
+        case 2: return launch_mrows_any<2, 2>(stream, A, Wq, S, Y, M, N, K, zp, num_cu, fusion, partial, sp.ranges, sp.range_groups, sync);
+        case 3: return launch_mrows_any<3, 2>(stream, A, Wq, S, Y, M, N, K, zp, num_cu, fusion, partial, sp.ranges, sp.range_groups, sync);
+        default: return launch_mrows_any<4, 2>(stream, A, Wq, S, Y, M, N, K, zp, num_cu, fusion, partial, sp.ranges, sp.range_groups, sync);
         }
     }
 } // namespace nnf

@@ -667,6 +667,8 @@ namespace nnf
             sp.gw = gw;
             return sp;
         }
+        // synchronisation words for adding the ranges up inside the launch: one per workgroup of a range
+        inline size_t mrows_split_sync_bytes(int num_cu) { return (size_t)num_cu * sizeof(unsigned); }
         inline size_t mrows_split_bytes(int M, int N_total, int K)
         {
             const int r = w4a16_mrows_split(M, N_total, K, PLAN_CUS).ranges;

@@ -172,3 +172,47 @@ def test_one_launch_full_size_rows(gpu):
             torch.cuda.synchronize()
             assert int(sync.count_nonzero()) == 0
             assert torch.equal(one, two)
+
+
+@pytest.mark.parametrize("fused", ["plain", "bias+residual", "residual-in-place", "rms+bias"])
+@pytest.mark.parametrize("m,n,k", [(16, 4096, 11008), (8, 100, 11008), (3, 520, 16384), (24, 260, 8448), (40, 64, 4352), (12, 33, 13824)])
+def test_ranges_of_k_added_up_inside_the_launch(gpu, m, n, k, fused):
+    """A few activation rows and K above what one workgroup holds: the row-streaming kernel works on ranges of K; with
+    synchronisation words the last workgroup to arrive at a group of columns adds the ranges up, in their order, and runs
+    the epilogue -- the same bits as the reduction pass gives, no second launch, the words zero again afterwards.  N not
+    a multiple of 16 (a last tile moved back over its neighbour's columns) with the residual in the output buffer: every
+    output is written once."""
+    import torch
+
+    from nnfusion_amd import ops
+
+    if not ops.w4a16_variant_supported(m, n, k, "gemv_rows"):
+        pytest.skip("the row-streaming kernel does not take this shape")
+    print(f"case ranges-of-K M={m} N={n} K={k} {fused}", flush=True)
+    a, wq, s = datagen.w4a16_case(m + n, m, n, k)
+    rng = np.random.default_rng(k)
+    gamma = (1.0 + 0.1 * rng.standard_normal(k)).astype(np.float16) if "rms" in fused else None
+    bias = rng.standard_normal(n).astype(np.float16) if "bias" in fused else None
+    resid = rng.standard_normal((m, n)).astype(np.float16) if "residual" in fused else None
+    ta, tw, ts, tg, tb, tr = _t(gpu, a, wq, s, gamma, bias, resid)
+    ws = _ws(gpu)
+    sync = ops.sync_flags(gpu)
+    if fused == "plain":
+        two = ops.w4a16_gemm_variant(ta, tw, ts, "gemv_rows", workspace=ws)
+        one = ops.w4a16_gemm_variant(ta, tw, ts, "gemv_rows", workspace=ws, sync=sync)
+        again = ops.w4a16_gemm_variant(ta, tw, ts, "gemv_rows", workspace=ws, sync=sync)
+        torch.cuda.synchronize()
+        _check(one.cpu().numpy(), oracle.w4a16_gemm(a, wq, s, f32_out=True))
+    elif fused == "residual-in-place":
+        out_two, out_one, out_again = tr.clone(), tr.clone(), tr.clone()
+        two = ops.w4a16_gemm_fused(ta, tw, ts, residual=out_two, out=out_two, variant="gemv_rows", workspace=ws)
+        one = ops.w4a16_gemm_fused(ta, tw, ts, residual=out_one, out=out_one, variant="gemv_rows", workspace=ws, sync=sync)
+        again = ops.w4a16_gemm_fused(ta, tw, ts, residual=out_again, out=out_again, variant="gemv_rows", workspace=ws, sync=sync)
+    else:
+        kw = dict(rms_gamma=tg, bias=tb, residual=tr, variant="gemv_rows", workspace=ws)
+        two = ops.w4a16_gemm_fused(ta, tw, ts, **kw)
+        one = ops.w4a16_gemm_fused(ta, tw, ts, sync=sync, **kw)
+        again = ops.w4a16_gemm_fused(ta, tw, ts, sync=sync, **kw)
+    torch.cuda.synchronize()
+    assert int(sync.count_nonzero()) == 0
+    assert torch.equal(one, two) and torch.equal(again, two)
