@@ -32,6 +32,7 @@ import json
 import os
 import sys
 import time
+import warnings
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
@@ -273,7 +274,9 @@ def main():
     dom_traffic = [p["traffic"] for p in k4096]
     roofline = {
         "bound": "hbm",
-        "kernel": "nnf::w4a16_gemv_rows_kernel<2, D, 8> (K=4096: two KiB per row; mean over its three launches per step)",
+        # (as the kernel trace behind profiles/bench_configurations_hbm_traffic.txt names it)
+        "kernel": " | ".join(sorted({load_row_kernels().get(f"decode_sweep.N{p['N']}_K{p['K']}", "?") for p in k4096})) +
+                  " (the K=4096 launches: two KiB per weight row; mean over the three of them in a step)",
         "achieved": round(dom_bytes / dom_us / 1e3, 1),
         "peak": HBM_PEAK_GBS,
         "unit": "GB/s",
@@ -619,7 +622,9 @@ def run_timeline(env, probes):
             rel[tr == 0] = np.nan
             rows.append(rel)
             spans.append(e0.elapsed_time(e1) * 1e3)
-        rel = np.nanmean(np.stack(rows), axis=0)
+        with np.errstate(all="ignore"), warnings.catch_warnings():
+            warnings.simplefilter("ignore", RuntimeWarning)  # (stamps that a kernel does not take: columns of NaN)
+            rel = np.nanmean(np.stack(rows), axis=0)
         print(f"{title}: grid {grid}; events around the launch (eager, launch overhead included): {sum(spans) / len(spans):.1f} us")
         print(f"    {'stamp':<58} {'first':>8} {'mean':>8} {'last':>8}")
         for i, name in names:

@@ -4,6 +4,8 @@
     python3 -m nnfusion_amd.profile_summary traffic  <FETCH_SIZE dir> <WRITE_SIZE dir> <probe log>  > HBM bytes per row
     python3 -m nnfusion_amd.profile_summary counters <dir of a --pmc run> <probe log> [row prefix ...]
                                                                                       > counters per row and kernel
+    python3 -m nnfusion_amd.profile_summary kernels  <dir of a --pmc run> <last n> [name part ...]
+                                                       > counters per kernel: means over its last n dispatches
 
 `bench.py --pmc-probe` launches every configuration row eagerly with a marker launch (probe_read_kernel) ahead of each
 and prints the order of the rows as one JSON line ({"pmc_probe": ...}): the probe log is the file that line went to.  The
@@ -34,8 +36,12 @@ def short(name, width=64):
     """nnf::gemm_sk::kernel<4, 2, ...>(args) -> kernel<4, 2, ...>, cut to `width`."""
     name = demangle(name)
     name = re.sub(r"\b(nnf|gemm_sk)::", "", name)
-    m = re.match(r"_ZN3nnf\d+([a-z0-9_]+?_kernel)", name)
-    return (m.group(1) if m else name)[:width]
+    # (a name the demangler at hand does not know -- the _Float16 mangling -- : the kernel's name and its literal arguments)
+    m = re.match(r"_ZN3nnf\d+([a-z0-9_]+?_kernel)(?:I((?:L[ib]\d+E)+)E)?", name)
+    if m:
+        args = [("true" if v == "1" else "false") if t == "b" else v for t, v in re.findall(r"L([ib])(\d+)E", m.group(2) or "")]
+        name = m.group(1) + (f"<{', '.join(args)}>" if args else "")
+    return name[:width]
 
 
 def csv_rows(directory, suffix):
@@ -170,6 +176,36 @@ def counters(directory, log, prefixes):
     return out + ["", "derived:"] + derived
 
 
+def kernels(directory, last, parts):
+    """Per kernel (no marker launches needed: for `bench.py --gemm-probe`, which launches two kernels some times each): the
+    means of duration and counters over the kernel's last `last` dispatches."""
+    by_dispatch = collections.OrderedDict()
+    for r in sorted(csv_rows(directory, "counter_collection.csv"), key=lambda r: int(r["Dispatch_Id"])):
+        d = by_dispatch.setdefault(int(r["Dispatch_Id"]), {"kernel": r["Kernel_Name"]})
+        d[r["Counter_Name"]] = d.get(r["Counter_Name"], 0.0) + float(r["Counter_Value"])
+        if r.get("Start_Timestamp") and r.get("End_Timestamp"):
+            d["us"] = (int(r["End_Timestamp"]) - int(r["Start_Timestamp"])) / 1e3
+    groups = collections.OrderedDict()
+    for d in by_dispatch.values():
+        name = short(d["kernel"], 60)
+        if not parts or any(p in name for p in parts):
+            groups.setdefault(name, []).append(d)
+    names = sorted({k for g in groups.values() for d in g for k in d if k not in ("kernel", "us")})
+    out = [f"means over the last {last} dispatches of each kernel; counters summed over the chip", ""]
+    for name, g in groups.items():
+        g = g[-last:]
+        out.append(f"{name}: {len(g)} dispatches, {sum(d.get('us', 0.0) for d in g) / len(g):.1f} us")
+        mean = {n: sum(d.get(n, 0.0) for d in g) / len(g) for n in names}
+        for n in names:
+            out.append(f"    {n:<34} {mean[n]:>16.0f}")
+        if mean.get("SQ_BUSY_CYCLES") and mean.get("SQ_VALU_MFMA_BUSY_CYCLES"):
+            cyc = mean["SQ_BUSY_CYCLES"] / 32  # per shader engine, 32 of them: the launch in cycles
+            us = sum(d.get("us", 0.0) for d in g) / len(g)
+            out.append(f"    launch {cyc:.0f} cycles ({cyc / us / 1e3:.2f} GHz); matrix cores busy "
+                       f"{100 * mean['SQ_VALU_MFMA_BUSY_CYCLES'] / 1024 / cyc:.1f} % of them (SQ_VALU_MFMA_BUSY_CYCLES is per SIMD, 1024 of them)")
+    return out
+
+
 def main(argv):
     if len(argv) >= 2 and argv[0] == "stats":
         lines = stats(argv[1])
@@ -177,6 +213,8 @@ def main(argv):
         lines = traffic(argv[1], argv[2], argv[3])
     elif len(argv) >= 3 and argv[0] == "counters":
         lines = counters(argv[1], argv[2], argv[3:])
+    elif len(argv) >= 3 and argv[0] == "kernels":
+        lines = kernels(argv[1], int(argv[2]), argv[3:])
     else:
         raise SystemExit(__doc__)
     print("\n".join(lines))
