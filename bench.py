@@ -650,7 +650,9 @@ def run_timeline(env, probes):
         table(f"single-row GEMV N={n} K={k} ({w4a16_bytes(1, n, k)} bytes: {us:.2f} us at 8 TB/s)", gemv_names, launch, 8, len(copies))
         del copies
 
-    gemm_names = [(0, "workgroup starts"), (1, "first operands arrived"), (2, "K loop of its last segment over"), (3, "its part parked"),
+    gemm_names = [(0, "workgroup starts"), (1, "first operands arrived"), (10, "(two segments) K loop of the first over"),
+                  (11, "(two segments) its part parked and counted in"), (12, "(two segments) first operands of the last arrived"),
+                  (2, "K loop of its last segment over"), (3, "its part parked"),
                   (4, "... and counted in"), (5, "waits for the other workgroups of its shared tiles over"),
                   (6, "its share of those tiles finished"), (9, "end")]
     ws = env.workspace(256 << 20)

@@ -319,7 +319,9 @@ extern "C" int nnf_probe_mfma(int kind, int mode, int iters, int num_cu, double*
 // The product's own kernel (w4a16_gemm_sk.h), compiled here once more with time stamps (NNF_SK_TRACE): the plain product
 // on 128-row tiles of 128 or 256 columns, in its one-launch form.  trace: 16 x grid 64-bit stamps of the 100 MHz clock
 // (0 start, 1 first operands arrived, 2 K loop of the last segment over, 3 its part parked, 4 counted in, 5 waits for the
-// other workgroups of its shared tiles over, 6 its share of those tiles finished, 9 end).  Returns the grid, or -1.
+// other workgroups of its shared tiles over, 6 its share of those tiles finished, 9 end; for a workgroup with two segments
+// also 10 K loop of the first over, 11 its part parked and counted in, 12 first operands of the last arrived).
+// Returns the grid, or -1.
 #define NNF_SK_TRACE 1
 #include "../nnf_workspace.h"
 #include "w4a16_gemm_sk.h"

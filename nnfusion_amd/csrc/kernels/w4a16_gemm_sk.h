@@ -133,6 +133,12 @@ namespace nnf
         constexpr int vmcnt_imm(int n) { return (n & 0xF) | ((n >> 4) << 14) | (0x7 << 4) | (0xF << 8); }
 
         // `grid` workgroups split `units` units as [v * units / grid, (v + 1) * units / grid)
+        // (A workgroup whose share spans two tiles parks the first tile's part in the middle of the launch, where the
+        // acknowledgement of its device-scope stores takes about 5 us against 2-3 us at the end of the launch.  Issuing the
+        // next segment's first loads ahead of those stores was tried: the acknowledgement, not the loads, is what the
+        // workgroup waits for, and nothing was gained.  Stores and loads at the scope of one XCD's L2 instead of the device
+        // -- valid only among workgroups known to sit on one XCD -- were timed in the measurement probe: acknowledged in 2 us
+        // there, but the last workgroup of the launch ended less than a microsecond earlier.)
         // (Shares weighted by what a second K loop in a workgroup costs -- its first loads, parking the part it leaves
         // behind: about one and a half units -- were tried: with whole units to deal out the longest share stays the same
         // for the MLP block's products, and a table of bounds in the kernel arguments made every launch slower.)
@@ -1048,6 +1054,8 @@ namespace nnf
             __builtin_amdgcn_sched_barrier(0);
             if (first_of_mine)
                 NNF_SK_STAMP(1); // the first operands have arrived
+            else if (u >= u_end)
+                NNF_SK_STAMP(12); // ... and those of the last segment, when it is not the first
             prepare_scales(I0{}, 0);
             if constexpr (RMS)
                 unroll_for<0, 4>([&](auto g_c) { lds_read_b128_nowait<decltype(g_c)::value * 16>(gm[decltype(g_c)::value], g_rd); });
@@ -1111,6 +1119,8 @@ namespace nnf
             __syncthreads();                                   // ... from any wavefront: the ring is free
             if (u >= u_end)
                 NNF_SK_STAMP(2); // the K loop of the last segment is over
+            else if (first_of_mine)
+                NNF_SK_STAMP(10); // ... of the first segment, when it is not the last
 
             // ---- a tile shared with other workgroups: park the sums in register order (element block q of MFMA tile
             // (i, j) of all 256 threads is one contiguous 4 KiB); w4a16_gemm_sk_fixup_kernel adds the parts and finishes
@@ -1147,6 +1157,8 @@ namespace nnf
                         old = atomicAdd(p.sync + 2 * (size_t)tile, 1u);
                     if (u >= u_end)
                         NNF_SK_STAMP(4 + (old & 0u)); // ... and counted in
+                    else if (first_of_mine)
+                        NNF_SK_STAMP(11 + (old & 0u)); // (the first segment's part, when it is not the last)
                     if (first_of_mine)
                         pend_tile[0] = tile, pend_old[0] = old;
                     else
