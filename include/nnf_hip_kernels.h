@@ -205,6 +205,14 @@ NNF_API int nnf_wna16_gemm(nnf_stream_t stream,
                    const void* A, const void* Wq, const void* scales, void* Y,
                    int M, int N, int K, const nnf_quant* q,
                    void* workspace, size_t workspace_bytes);
+/* The same with an nnf_plan (NULL: nnf_wna16_gemm): its sync_flags make the tile GEMM of these parameters a single
+ * launch, as they do for nnf_w4a16_gemm_variant (same contract: all zero before the first call, left all zero by every
+ * call); the tile fields apply to 4 bits / 128 / no zero-point tensor only (the other parameters keep the library's tile
+ * shapes).  Same results bit for bit. */
+NNF_API int nnf_wna16_gemm_planned(nnf_stream_t stream,
+                   const void* A, const void* Wq, const void* scales, void* Y,
+                   int M, int N, int K, const nnf_quant* q, const nnf_plan* plan,
+                   void* workspace, size_t workspace_bytes);
 
 /* ---------------------------------------------------------------------------------------------
  * The nodes around a quantized product, for graphs in which no fusion pattern absorbed them (a gate

@@ -41,6 +41,7 @@ KERNEL_ABI = {
     "nnf_wna16_supported": (_c_int, [_c_int] * 3 + [_c_vp]),
     "nnf_wna16_gemm_workspace_bytes": (_c_sz, [_c_int] * 3 + [_c_vp]),
     "nnf_wna16_gemm": (_c_int, [_c_vp] * 5 + [_c_int] * 3 + [_c_vp, _c_vp, _c_sz]),
+    "nnf_wna16_gemm_planned": (_c_int, [_c_vp] * 5 + [_c_int] * 3 + [_c_vp, _c_vp, _c_vp, _c_sz]),
     "nnf_w4a16_gemm_fused_workspace_bytes": (_c_sz, [_c_int] * 5),
     "nnf_w4a16_gemm_fused": (_c_int, [_c_vp] * 5 + [_c_int] * 5 + [_c_vp, _c_f, _c_vp, _c_vp, _c_int, _c_vp, _c_sz]),
     "nnf_w4a16_gemm_fused_variant": (_c_int, [_c_vp] * 5 + [_c_int] * 5 + [_c_vp, _c_f, _c_vp, _c_vp, _c_int, _c_int, _c_vp,

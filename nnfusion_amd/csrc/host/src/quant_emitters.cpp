@@ -52,8 +52,13 @@ namespace nnfusion
                     const bool split = route.kind == nnf::workspace::W4A16Route::MROWS_SPLIT && !gate;
                     if (route.kind != nnf::workspace::W4A16Route::TILE && !split)
                         return "";
-                    const size_t bytes =
-                        ((split ? nnf::workspace::mrows_split_sync_bytes(nnf::workspace::PLAN_CUS) : route.plan.sync_bytes(rms)) + 63) & ~(size_t)63;
+                    return declare_sync_words(name, split ? nnf::workspace::mrows_split_sync_bytes(nnf::workspace::PLAN_CUS)
+                                                          : route.plan.sync_bytes(rms));
+                }
+                // `name` as an nnf_plan over a persistent, zero-initialised tensor of (at least) `need` bytes; "": none needed
+                std::string declare_sync_words(const std::string& name, size_t need)
+                {
+                    const size_t bytes = (need + 63) & ~(size_t)63;
                     if (bytes == 0 || bytes > NNF_SYNC_FLAGS_BYTES)
                         return "";
                     auto flags = allocate_tensor(Shape{bytes}, element::character, "", ROCM_GPU, true);
@@ -128,7 +133,15 @@ namespace nnfusion
                         LanguageUnit_p lu(new LanguageUnit(get_function_name()));
                         *lu << "const nnf_quant quant = {" << bits << ", " << group << ", " << zp << ", "
                             << (has_z ? "input3" : "nullptr") << "};\n";
-                        if (!q_fused)
+                        // 4-bit weights on the stream-K tile GEMM (above 16 rows, K a multiple of 256): its synchronisation words
+                        std::string q_plan;
+                        if (!q_fused && bits == 4 && M > 16 && nnf::workspace::w4a16_gemm_q_fits((int)M, (int)N, (int)K, group == 32 ? 5 : group == 64 ? 6 : 7))
+                            q_plan = declare_sync_words("plan", nnf::workspace::plan_w4a16_sk((int)M, (int)N, (int)K, false, nnf::workspace::PLAN_CUS).sync_bytes());
+                        *lu << q_plan;
+                        if (!q_fused && !q_plan.empty())
+                            *lu << "NNF_HIP_CHECK(nnf_wna16_gemm_planned(stream, input0, input1, input2, output0, " << M << ", " << N << ", "
+                                << K << ", &quant, &plan, " << q_ws << ", " << q_ws_bytes << "));\n";
+                        else if (!q_fused)
                             *lu << "NNF_HIP_CHECK(nnf_wna16_gemm(stream, input0, input1, input2, output0, " << M << ", " << N << ", "
                                 << K << ", &quant, " << q_ws << ", " << q_ws_bytes << "));\n";
                         else

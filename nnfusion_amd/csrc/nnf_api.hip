@@ -266,10 +266,23 @@ size_t nnf_wna16_gemm_workspace_bytes(int M, int N, int K, const nnf_quant* q)
 int nnf_wna16_gemm(nnf_stream_t stream, const void* A, const void* Wq, const void* scales, void* Y, int M, int N, int K,
                    const nnf_quant* q, void* workspace, size_t workspace_bytes)
 {
+    return nnf_wna16_gemm_planned(stream, A, Wq, scales, Y, M, N, K, q, nullptr, workspace, workspace_bytes);
+}
+
+int nnf_wna16_gemm_planned(nnf_stream_t stream, const void* A, const void* Wq, const void* scales, void* Y, int M, int N, int K,
+                           const nnf_quant* q, const nnf_plan* plan, void* workspace, size_t workspace_bytes)
+{
     if (!q)
         return NNF_ERR_INVALID_ARGUMENT;
     if (is_plain_w4a16(q))
-        return nnf_w4a16_gemm(stream, A, Wq, scales, Y, M, N, K, q->group, q->zero_point, workspace, workspace_bytes);
+        return plan ? nnf_w4a16_gemm_variant(stream, A, Wq, scales, Y, M, N, K, q->group, q->zero_point, NNF_W4A16_AUTO, plan, workspace,
+                                             workspace_bytes)
+                    : nnf_w4a16_gemm(stream, A, Wq, scales, Y, M, N, K, q->group, q->zero_point, workspace, workspace_bytes);
+    // (of a plan only the synchronisation words apply to these parameters)
+    nnf::LaunchChoice choice;
+    if (!make_choice(NNF_W4A16_AUTO, plan, NNF_W4A16_GEMV_ROWS, choice))
+        return NNF_ERR_INVALID_ARGUMENT;
+    choice.tile_rows = choice.k_parts = choice.tile_cols = 0;
     if (!A || !Wq || !scales || !Y || M <= 0 || N <= 0 || K <= 0)
         return NNF_ERR_INVALID_ARGUMENT;
     if (!aligned16(A) || !aligned16(Wq) || !aligned16(scales) || !aligned16(Y))
@@ -307,7 +320,7 @@ int nnf_wna16_gemm(nnf_stream_t stream, const void* A, const void* Wq, const voi
         const size_t need = nnf::workspace::wna16_gemm(M, N, K, q->bits, q->group, dev.num_cu);
         if (need == 0 || (workspace && aligned16(workspace) && workspace_bytes >= need))
             return (int)nnf::launch_w4a16_gemm_q((hipStream_t)stream, A, Wq, scales, Y, M, N, K, group_shift_of(q->group),
-                                                 q->zero_point, q->zero_points, workspace, dev.num_cu);
+                                                 q->zero_point, q->zero_points, workspace, dev.num_cu, choice);
     }
     return (int)nnf::launch_wna16_generic((hipStream_t)stream, A, Wq, scales, Y, M, N, K, q->bits, q->group, q->zero_point,
                                           q->zero_points, dev.num_cu);

@@ -106,9 +106,10 @@ def wna16_workspace_bytes(m, n, k, bits, group, zero_points=None):
     return int(_lib.kernels().nnf_wna16_gemm_workspace_bytes(m, n, k, qp))
 
 
-def wna16_gemm(a, wq, scales, bits=4, group=128, zp=8, zero_points=None, out=None, workspace=None):
+def wna16_gemm(a, wq, scales, bits=4, group=128, zp=8, zero_points=None, out=None, workspace=None, sync=None, spin_limit=0):
     """Y[M,N] = A[M,K] . ((Wq - z) * scales)^T with 4- or 8-bit weights (wq u8 [N, K*bits/8]), groups of 32 / 64 / 128
-    and either a scalar zero point or zero_points u8 [N, ceil(K/group*bits/8)] (4-bit: two per byte, even group low)."""
+    and either a scalar zero point or zero_points u8 [N, ceil(K/group*bits/8)] (4-bit: two per byte, even group low).
+    sync: synchronisation words (sync_flags()) for the one-launch form of the tile GEMM: nnf_wna16_gemm_planned."""
     lib = _lib.kernels()
     m, k = a.shape
     n = wq.shape[0]
@@ -123,6 +124,11 @@ def wna16_gemm(a, wq, scales, bits=4, group=128, zp=8, zero_points=None, out=Non
     keep, qp = _quant_arg(bits, group, zp, zero_points)
     if workspace is None:
         workspace = _ws(lib.nnf_wna16_gemm_workspace_bytes(m, n, k, qp), a.device)
+    if sync is not None:
+        keep_plan, plan_ptr = _plan_arg(None, sync, spin_limit)
+        _check(lib.nnf_wna16_gemm_planned(_stream(), a.data_ptr(), wq.data_ptr(), scales.data_ptr(), out.data_ptr(), m, n, k, qp,
+                                          plan_ptr, workspace.data_ptr(), workspace.numel()), "nnf_wna16_gemm_planned")
+        return out
     _check(lib.nnf_wna16_gemm(_stream(), a.data_ptr(), wq.data_ptr(), scales.data_ptr(), out.data_ptr(), m, n, k, qp,
                               workspace.data_ptr(), workspace.numel()), "nnf_wna16_gemm")
     return out

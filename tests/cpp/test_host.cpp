@@ -1033,7 +1033,12 @@ int main(int argc, char** argv)
             const size_t ws = nnf::workspace::wna16_gemm(128, 4096, 4096, 4, 64);
             EXPECT(ws > 0 && ws == nnf::workspace::plan_w4a16_sk(128, 4096, 4096, false, nnf::workspace::PLAN_CUS).bytes());
             CONTAINS(body, "const nnf_quant quant = {4, 64, 8, input3};");
-            CONTAINS(body, "nnf_wna16_gemm(stream, input0, input1, input2, output0, 128, 4096, 4096, &quant, ");
+            // ... through the entry point that takes the synchronisation words of the one-launch form (two per tile, 32 tiles
+            // of 128 x 128, and two more: a second, persistent and zero-initialised tensor)
+            EXPECT(k->m_context->tensors.size() == 2 && k->m_context->tensors[1]->size() == 320 &&
+                   k->m_context->tensors[1]->is_persistent() && k->m_context->tensors[1]->is_memset());
+            CONTAINS(body, "const nnf_plan plan = {0, 0, 0, " + k->m_context->tensors[1]->get_name() + ", 320, 0};");
+            CONTAINS(body, "nnf_wna16_gemm_planned(stream, input0, input1, input2, output0, 128, 4096, 4096, &quant, &plan, ");
             CONTAINS(body, ", " + std::to_string(ws) + "));");
             EXPECT(body.find("&quant, nullptr") == std::string::npos);
             // 8-bit weights, K not a multiple of 256, 16 rows: the kernels that need none

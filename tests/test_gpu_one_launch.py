@@ -216,3 +216,23 @@ def test_ranges_of_k_added_up_inside_the_launch(gpu, m, n, k, fused):
     torch.cuda.synchronize()
     assert int(sync.count_nonzero()) == 0
     assert torch.equal(one, two) and torch.equal(again, two)
+
+
+@pytest.mark.parametrize("bits,group,zpt", [(4, 32, True), (4, 64, False), (4, 128, True)])
+@pytest.mark.parametrize("m,n,k", [(200, 300, 1024), (64, 520, 2048), (130, 128, 1536), (256, 1024, 4096)])
+def test_one_launch_with_other_block_parameters(gpu, m, n, k, bits, group, zpt):
+    """nnf_wna16_gemm_planned: the tile GEMM for groups of 32 / 64 / 128 and zero-point tensors in one launch."""
+    import torch
+
+    from nnfusion_amd import ops
+
+    a, wq, s, z = datagen.wna16_case(m + k, m, n, k, bits, group, zpt)
+    ta, tw, ts, tz = _t(gpu, a, wq, s, z if zpt else None)
+    two = ops.wna16_gemm(ta, tw, ts, bits=bits, group=group, zp=8, zero_points=tz)
+    sync = ops.sync_flags(gpu)
+    for spin_limit in (0, -1):
+        one = ops.wna16_gemm(ta, tw, ts, bits=bits, group=group, zp=8, zero_points=tz, sync=sync, spin_limit=spin_limit)
+        torch.cuda.synchronize()
+        assert int(sync.count_nonzero()) == 0
+        assert torch.equal(one, two)
+    _check(one.cpu().numpy(), oracle.wna16_gemm(a, wq, s, bits, group, zp=8, zero_points=z if zpt else None).astype(np.float32))
