@@ -160,6 +160,16 @@ namespace nnf
         const half_t* residual;
         float rms_eps; // gamma without rstd: the kernel computes rsqrt(mean(a^2) + rms_eps) of its activation row itself
     };
+    // a * b rounded to fp32, as a value of its own: a conversion to fp16 that follows then rounds a second time wherever it
+    // is compiled.  (Left to the compiler, product and conversion may or may not become one mixed-precision instruction
+    // that rounds once: two kernels that must agree bit for bit -- the reduction pass and the kernels that add their ranges
+    // up themselves -- would differ in the last fp16 bit now and then.)
+    __device__ __forceinline__ float f32_product(float a, float b)
+    {
+        float v = a * b;
+        asm volatile("" : "+v"(v));
+        return v;
+    }
     // y = fp16(sum) (+ bias[n]) (+ residual[at]), each step rounded to fp16
     __device__ __forceinline__ half_t finish_bias_residual(float sum, const half_t* bias, int n, const half_t* residual, size_t at)
     {

@@ -184,11 +184,11 @@ namespace nnf
         {
             if (n + j >= N)
                 break;
-            float v = a[j] * rs;
+            float v = f32_product(a[j], rs);
             if (GATE)
             {
                 float g = (float)(half_t)v;
-                float up = (float)(half_t)(u[j] * rs);
+                float up = (float)(half_t)f32_product(u[j], rs);
                 v = g * (1.0f / (1.0f + __expf(-g))) * up;
             }
             if (BIAS)

@@ -1051,7 +1051,7 @@ namespace nnf
                                 sum += part[d];
                     }
                     if (FUSED)
-                        Y[at] = finish_bias_residual(sum * (f.rstd ? f.rstd[m] : 1.0f), f.bias, nn, f.residual, at);
+                        Y[at] = finish_bias_residual(f32_product(sum, f.rstd ? f.rstd[m] : 1.0f), f.bias, nn, f.residual, at);
                     else
                         Y[at] = (half_t)sum;
                 }

@@ -174,12 +174,13 @@ def test_one_launch_full_size_rows(gpu):
             assert torch.equal(one, two)
 
 
-@pytest.mark.parametrize("fused", ["plain", "bias+residual", "residual-in-place", "rms+bias"])
+@pytest.mark.parametrize("fused", ["plain", "bias+residual", "residual-in-place", "rms+bias", "rms"])
 @pytest.mark.parametrize("m,n,k", [(16, 4096, 11008), (8, 100, 11008), (3, 520, 16384), (24, 260, 8448), (40, 64, 4352), (12, 33, 13824)])
 def test_ranges_of_k_added_up_inside_the_launch(gpu, m, n, k, fused):
     """A few activation rows and K above what one workgroup holds: the row-streaming kernel works on ranges of K; with
     synchronisation words the last workgroup to arrive at a group of columns adds the ranges up, in their order, and runs
-    the epilogue -- the same bits as the reduction pass gives, no second launch, the words zero again afterwards.  N not
+    the epilogue -- the same bits as the reduction pass gives (rstd alone included: both round the fp32 product of sum and
+    rstd to fp32 before the conversion to fp16), no second launch, the words zero again afterwards.  N not
     a multiple of 16 (a last tile moved back over its neighbour's columns) with the residual in the output buffer: every
     output is written once."""
     import torch
@@ -236,3 +237,50 @@ def test_one_launch_with_other_block_parameters(gpu, m, n, k, bits, group, zpt):
         assert int(sync.count_nonzero()) == 0
         assert torch.equal(one, two)
     _check(one.cpu().numpy(), oracle.wna16_gemm(a, wq, s, bits, group, zp=8, zero_points=z if zpt else None).astype(np.float32))
+
+
+def test_one_launch_random_shapes_and_plans(gpu):
+    """Sixty seeded random products -- tile GEMM with any tile shape and split, the row-streaming kernel over ranges of K,
+    plain and fused -- four calls each on one set of synchronisation words (the last with the wait forced to run out):
+    bit for bit the two-launch result, the words zero after every call."""
+    import torch
+
+    from nnfusion_amd import ops
+
+    rng = np.random.default_rng(2024)
+    ws = _ws(gpu, 256 << 20)
+    sync = ops.sync_flags(gpu)
+    done = 0
+    for c in range(60):
+        if c % 4 == 3:  # a few rows, K above 8192: ranges of K
+            m, n, k = int(rng.integers(2, 33)), int(rng.integers(16, 3000)), int(rng.integers(33, 80)) * 256
+            plan, variant = None, "gemv_rows"
+            if not ops.w4a16_variant_supported(m, n, k, variant):
+                continue
+        else:
+            m, k = int(rng.integers(17, 600)), int(rng.integers(2, 40)) * 128
+            n = int(rng.integers(8, 1000)) * 8 if rng.random() < 0.7 else int(rng.integers(17, 3000))
+            rows = int(rng.choice([0, 32, 64, 128, 256]))
+            cols = int(rng.choice([0, 128, 256])) if rows in (64, 128, 256) else 0
+            parts = int(rng.integers(0, 7))
+            plan, variant = ((rows, parts, cols) if (rows or parts or cols) else None), "gemm_mfma"
+        fused = int(rng.integers(0, 4))  # 0 plain, 1 rms, 2 bias + residual, 3 rms + gate (tile GEMM) / rms (ranges of K)
+        gate = fused == 3 and variant == "gemm_mfma"
+        print(f"case random {c}: M={m} N={n} K={k} plan={plan} {variant} fused={fused}", flush=True)
+        a, wq, s = datagen.w4a16_case(c, m, 2 * n if gate else n, k)
+        gamma = (1.0 + 0.1 * rng.standard_normal(k)).astype(np.float16) if fused in (1, 3) else None
+        bias = rng.standard_normal(n).astype(np.float16) if fused == 2 else None
+        resid = rng.standard_normal((m, n)).astype(np.float16) if fused == 2 else None
+        ta, tw, ts, tg, tb, tr = _t(gpu, a, wq, s, gamma, bias, resid)
+        kw = dict(rms_gamma=tg, bias=tb, residual=tr, act=1 if gate else 0, variant=variant, plan=plan, workspace=ws)
+        try:
+            two = ops.w4a16_gemm_fused(ta, tw, ts, **kw)
+        except ops.NnfError:  # (a plan the shape does not take)
+            continue
+        for rep in range(4):
+            one = ops.w4a16_gemm_fused(ta, tw, ts, sync=sync, spin_limit=-1 if rep == 3 else 0, **kw)
+            torch.cuda.synchronize()
+            assert int(sync.count_nonzero()) == 0, (c, rep)
+            assert torch.equal(one, two), (c, rep, m, n, k, plan, fused)
+        done += 1
+    assert done >= 40
