@@ -1083,7 +1083,8 @@ namespace nnf
                 auto next_of = [](uint32_t o) { return o + STAGE_BYTES == RING ? 0u : o + (uint32_t)STAGE_BYTES; };
                 uint32_t pv = RING - (uint32_t)STAGE_BYTES, st = 0;
                 // one loop body: the superstep works on register set 0 and fills set 1, which moves to set 0 at its end
-                // (a few dozen register moves per 256 MFMAs)
+                // (a few dozen register moves per 256 MFMAs; two bodies that swap the roles of the sets instead measured the
+                // same at every M, and spilled registers under the 256 x 256 tile)
                 for (int s = 0; s < NSS; ++s)
                 {
                     k_step(I0{}, s, pv, st, next_of(st));
