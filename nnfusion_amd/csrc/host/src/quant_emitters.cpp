@@ -49,7 +49,8 @@ namespace nnfusion
                         nnf::workspace::route_w4a16(M, N, K, gate, rms, false, nnf::workspace::PLAN_CUS);
                     // (the row-streaming kernel over ranges of K -- a few rows, K above 8192 -- adds its ranges up inside
                     // its launch with one word per workgroup of a range)
-                    const bool split = route.kind == nnf::workspace::W4A16Route::MROWS_SPLIT && !gate;
+                    const bool split = route.kind == nnf::workspace::W4A16Route::MROWS_SPLIT && !gate &&
+                                       nnf::workspace::mrows_split_adds_in_launch(N, route.ksplits, nnf::workspace::PLAN_CUS);
                     if (route.kind != nnf::workspace::W4A16Route::TILE && !split)
                         return "";
                     return declare_sync_words(name, split ? nnf::workspace::mrows_split_sync_bytes(nnf::workspace::PLAN_CUS)

@@ -359,7 +359,8 @@ namespace nnf
         {
             // (the row-streaming kernel adds its ranges up itself where the caller gave synchronisation words for it)
             if (route.kind == W4A16Route::MROWS_SPLIT && !gate && choice.sync_flags &&
-                choice.sync_bytes >= w4a16_mrows_split_sync_bytes(num_cu))
+                choice.sync_bytes >= w4a16_mrows_split_sync_bytes(num_cu) &&
+                workspace::mrows_split_adds_in_launch(n_rows, route.ksplits, num_cu))
             {
                 GemvFusion epilogue;
                 epilogue.rstd = rstd;

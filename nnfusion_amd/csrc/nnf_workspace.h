@@ -646,8 +646,11 @@ namespace nnf
             // (33 .. 64 rows run on the kernel, but against the tile GEMM, measured alternately: 33 / 40 rows take 25.9 / 27.4 us
             // against 29.1 / 29.3 at N = 22016, K = 4096 and 12.2 / 12.9 against 14.8 / 15.3 at N = K = 4096, are level at K = 8192 and
             // 11008, 8-10 % slower at K = 5120, and slower everywhere from about 48 rows on: taken up to 40 rows and K = 4096)
-            if (M < 2 || M > 40 || N < 16 || K <= (M <= 16 ? 8192 : M <= 32 ? 4096 : 2048) || K > (M <= 32 ? 65536 : 4096) || (K & 255) ||
-                num_cu < 16)
+            // (8 .. 16 rows at K = 8192, up to 16384 weight rows: in one launch every workgroup fetches all M x 8192 activations
+            // ahead of its first MFMA; over two ranges it fetches half of them: 10-18 % faster at 12 .. 16 rows, 0-10 % at 8,
+            // with the reduction pass or without it; slower at K = 5120 / 6144, level from about 28000 weight rows on)
+            const int longest_single = M <= 16 ? ((M >= 8 && K == 8192 && N <= 16384) ? 8191 : 8192) : M <= 32 ? 4096 : 2048;
+            if (M < 2 || M > 40 || N < 16 || K <= longest_single || K > (M <= 32 ? 65536 : 4096) || (K & 255) || num_cu < 16)
                 return sp;
             const int G = K >> 7;
             // 33 .. 64 rows: four blocks of rows leave registers for two groups per wavefront: ranges of 16 groups
@@ -669,6 +672,14 @@ namespace nnf
         }
         // synchronisation words for adding the ranges up inside the launch: one per workgroup of a range
         inline size_t mrows_split_sync_bytes(int num_cu) { return (size_t)num_cu * sizeof(unsigned); }
+        // Adding the ranges up inside the launch pays while a workgroup has few output tiles: the last arriver adds its
+        // tiles up one after the other, the reduction pass works on all of them at once (N = 28672 at 16 rows: 32 us
+        // against 30.7 with the pass; N <= 14336: level or up to 8 % faster in the launch).
+        inline bool mrows_split_adds_in_launch(int N, int ranges, int num_cu)
+        {
+            const int per_range = num_cu / ranges > 0 ? num_cu / ranges : 1;
+            return ((N + 15) / 16 + per_range - 1) / per_range <= 8;
+        }
         inline size_t mrows_split_bytes(int M, int N_total, int K)
         {
             const int r = w4a16_mrows_split(M, N_total, K, PLAN_CUS).ranges;
@@ -773,7 +784,11 @@ namespace nnf
                 // the row-streaming kernels apply prologue and epilogue themselves: one launch, no scratch memory
                 if (rows_family && plan_w4a16_rows(M, N, K, num_cu, 0, gate).seg != 0)
                     return r.kind = W4A16Route::ROWS, r.rms_bytes = rstd_bytes, r;
-                if (rows_family && M > 1 && (any ? w4a16_mrows_preferred(M, N, K, num_cu, gate) : w4a16_mrows_fits(M, N, K, num_cu, gate)))
+                // (K = 8192 at 8 .. 16 rows: over two ranges of K, see w4a16_mrows_split -- not with SiLU-gate, whose two halves
+                // the reduction would have to pair, nor with RMSNorm, which the single launch folds in without a pre-pass)
+                const bool two_ranges = !gate && !rms && K == 8192 && M >= 8 && M <= 16 && w4a16_mrows_split(M, n_rows, K, num_cu).ranges > 1;
+                if (rows_family && M > 1 && !two_ranges &&
+                    (any ? w4a16_mrows_preferred(M, N, K, num_cu, gate) : w4a16_mrows_fits(M, N, K, num_cu, gate)))
                     return r.kind = W4A16Route::MROWS, r.rms_bytes = rstd_bytes, r;
                 // the MFMA GEMV kernel writes plain products: an epilogue that cannot work in place (the [M, 2N] gate | up
                 // pair, a residual that is the output buffer) reads them from scratch memory
