@@ -714,7 +714,7 @@ def extra_rows(env):
         ws = env.workspace(lib.nnf_w8a8_gemm_workspace_bytes(m, n, k))
         rows.append({"key": f"w8a8_gemm_N{n}_K{k}.M{m}", "group": f"w8a8_gemm_N{n}_K{k}", "M": m,
                      "bytes": w8a8_bytes(m, n, k), "ops": 2.0 * m * n * k, "int8": True, "weights": (tw8,),
-                     "make": (lambda w, a8=a8, st=st, y=y, ws=ws: (lambda: ops.w8a8_gemm(a8, st, w, tsch, out=y, workspace=ws)))})
+                     "make": (lambda w, a8=a8, st=st, y=y, ws=ws: (lambda: ops.w8a8_gemm(a8, st, w, tsch, out=y, workspace=ws, sync=env.sync)))})
     for bits, group, zpt in WNA16_CASES:
         _, wq, s, z = datagen.wna16_case(0, 1, n, k, bits, group, zpt)
         tw, tsc, tz = env.dev_t(wq), env.dev_t(s), (env.dev_t(z) if zpt else None)

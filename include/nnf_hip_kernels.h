@@ -136,7 +136,7 @@ typedef struct nnf_plan
                       fp16 x int4 with 64-, 128- or 256-row tiles and no SiLU-gate (the gate | up halves need the
                       256 weight rows of a full tile); ignored elsewhere */
     /* fp16 x int4 products in one launch (any variant that ends up on one of the kernels below; ignored by every other
-     * kernel and by W8A8).
+     * kernel; W8A8: see the last sentence).
      * The work of the GEMM is split evenly over the CUs, so most output tiles of a mid-sized product are shared by
      * several workgroups.  Without sync_flags their parts are added up by a second launch.  With sync_flags the
      * workgroups count themselves in at their tiles there, and each adds up and finishes its share of a tile's rows
@@ -144,7 +144,9 @@ typedef struct nnf_plan
      * Two more launches go the same way: a fused RMSNorm's rstd[] is computed by the GEMM launch itself (every
      * workgroup a few rows before its first tile; no pass of its own), and the row-streaming kernel for a few
      * activation rows and K above 8192, which works on ranges of K, adds the ranges up itself (the last workgroup to
-     * arrive at a group of columns, in the order of the ranges; no reduction pass).
+     * arrive at a group of columns, in the order of the ranges; no reduction pass).  W8A8 with 8 .. 32 rows and K from
+     * 8192 runs its row-streaming kernel over two ranges of K the same way (int32 sums: exact), given sync_flags and
+     * nnf_w8a8_gemm_variant_workspace_bytes of workspace; without either, in one pass over K (same bits, ~1 us more).
      *   sync_flags: device memory, 16-byte aligned, ALL ZERO before the first call that uses it; every call leaves it
      *     all zero again, so it needs clearing once (when it is allocated), not per call.  It must not be scratch
      *     memory that other kernels write between calls, and calls that may overlap on the device (different
@@ -318,7 +320,8 @@ NNF_API int nnf_w8a8_gemm_acc(nnf_stream_t stream,
                       int M, int N, int K,
                       void* workspace, size_t workspace_bytes);
 
-/* The kernels behind nnf_w8a8_gemm as selectable variants (see nnf_w4a16_variant); `plan` as above. */
+/* The kernels behind nnf_w8a8_gemm as selectable variants (see nnf_w4a16_variant); `plan` as above (tile_rows, tile_cols and
+ * k_parts for the tile GEMM; sync_flags for the row-streaming kernel over two ranges of K). */
 enum nnf_w8a8_variant
 {
     NNF_W8A8_AUTO = 0,

@@ -30,7 +30,7 @@ namespace nnfusion
                 }
             } // namespace
 
-            // What the emitters of the fp16 x int4 products share.
+            // What the emitters of the quantised products share.
             class QuantLibEmitter : public HipLibEmitter
             {
             public:
@@ -260,11 +260,11 @@ namespace nnfusion
                 }
             };
 
-            class QuantDotW8A8 : public HipLibEmitter
+            class QuantDotW8A8 : public QuantLibEmitter
             {
             public:
                 explicit QuantDotW8A8(std::shared_ptr<KernelContext> ctx)
-                    : HipLibEmitter(ctx)
+                    : QuantLibEmitter(ctx)
                 {
                 }
 
@@ -284,8 +284,19 @@ namespace nnfusion
                     std::string ws = "nullptr";
                     if (ws_bytes > 0)
                         ws = allocate_tensor(Shape{ws_bytes}, element::character)->get_name();
+                    // a few rows with a long K: the row-streaming kernel over two ranges of K, which meet at one word per
+                    // workgroup of a range
+                    std::string plan;
+                    if (nnf::workspace::w8a8_mrows_preferred((int)M, (int)N, (int)K, nnf::workspace::PLAN_CUS) &&
+                        nnf::workspace::w8a8_mrows_ranges((int)M, (int)N, (int)K, nnf::workspace::PLAN_CUS) > 1)
+                        plan = declare_sync_words("plan", nnf::workspace::mrows_split_sync_bytes(nnf::workspace::PLAN_CUS));
                     LanguageUnit_p lu(new LanguageUnit(get_function_name()));
-                    if (raw)
+                    *lu << plan;
+                    if (!plan.empty())
+                        *lu << "NNF_HIP_CHECK(nnf_w8a8_gemm_variant(stream, input0, " << (raw ? "nullptr" : "input1") << ", input2, "
+                            << (raw ? "nullptr" : "input3") << ", " << (raw ? "nullptr, output0" : "output0, nullptr") << ", " << M
+                            << ", " << N << ", " << K << ", NNF_W8A8_AUTO, &plan, " << ws << ", " << ws_bytes << "));\n";
+                    else if (raw)
                         *lu << "NNF_HIP_CHECK(nnf_w8a8_gemm_acc(stream, input0, input2, output0, " << M << ", " << N << ", "
                             << K << ", " << ws << ", " << ws_bytes << "));\n";
                     else

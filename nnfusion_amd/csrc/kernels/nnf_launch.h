@@ -158,12 +158,14 @@ namespace nnf
                                     int K, int bits, int group, int zp, const void* zero_points, int num_cu);
 
     // W8A8: acc != nullptr writes the raw int32 accumulators, otherwise Y = fp16(acc * s_tok * s_ch).
-    // partial_ws: nnf::workspace::w8a8_gemm(M, N, K) bytes (0 for the M <= 16 kernel)
+    // partial_ws: w8a8_partial_bytes(...) bytes
     hipError_t launch_w8a8(hipStream_t stream, const void* A, const void* s_tok, const void* W, const void* s_ch,
-                           void* Y, void* acc, int M, int N, int K, int num_cu, void* partial_ws,
+                           void* Y, void* acc, int M, int N, int K, int num_cu, void* partial_ws, size_t partial_bytes,
                            const LaunchChoice& choice = LaunchChoice());
     // bytes launch_w8a8 writes at partial_ws for this call (0: the kernel it picks needs none)
     size_t w8a8_partial_bytes(int M, int N, int K, int num_cu, const LaunchChoice& choice = LaunchChoice());
+    // true: the kernel it picks runs without those bytes as well (another way round, a little slower)
+    bool w8a8_partial_optional(int M, int N, int K, int num_cu, const LaunchChoice& choice = LaunchChoice());
     // whether the kernel family `path` names can serve the shape
     bool w8a8_path_supported(int M, int N, int K, int num_cu, int path);
     // the MFMA GEMM behind launch_w8a8 (any M)
@@ -176,8 +178,11 @@ namespace nnf
                                      void* Y, void* acc, int N, int K, int num_cu);
     bool w8a8_gemv_rows_supported(int M, int N, int K, int num_cu);
     // 2 <= M <= 32, K = 2048, 4096, 6144 or 8192: the row-streaming MFMA kernel (w8a8_mrows.hip)
+    // partial_ws (workspace::w8a8_mrows_ranges_bytes(...)) and sync (workspace::mrows_split_sync_bytes(num_cu), zeroed, left
+    // zero): what the form over two ranges of K needs; without either, one pass over K
     hipError_t launch_w8a8_mrows(hipStream_t stream, const void* A, const void* s_tok, const void* W, const void* s_ch,
-                                 void* Y, void* acc, int M, int N, int K, int num_cu);
+                                 void* Y, void* acc, int M, int N, int K, int num_cu, void* partial_ws = nullptr,
+                                 size_t partial_bytes = 0, uint32_t* sync = nullptr, size_t sync_bytes = 0);
     bool w8a8_mrows_supported(int M, int N, int K, int num_cu);
     bool w8a8_mrows_preferred(int M, int N, int K, int num_cu); // where the library picks it without being told
 

@@ -293,14 +293,24 @@ namespace nnf
 
     size_t w8a8_partial_bytes(int M, int N, int K, int num_cu, const LaunchChoice& choice)
     {
-        if (pick_w8a8(M, N, K, num_cu, choice.path) != Q8_TILE)
+        const Q8Kind kind = pick_w8a8(M, N, K, num_cu, choice.path);
+        if (kind == Q8_MROWS) // (two ranges of K, their sums added up in the launch: with synchronisation words only)
+            return choice.sync_flags && choice.sync_bytes >= workspace::mrows_split_sync_bytes(num_cu)
+                       ? workspace::w8a8_mrows_ranges_bytes(M, N, K, num_cu)
+                       : 0;
+        if (kind != Q8_TILE)
             return 0;
         const int tile = workspace::w8a8_forced_tile(choice.tile_rows, choice.tile_cols);
         return workspace::gemm_partial_bytes(M, N, false, workspace::plan_w8a8_gemm(M, N, K, tile, choice.k_parts));
     }
 
+    bool w8a8_partial_optional(int M, int N, int K, int num_cu, const LaunchChoice& choice)
+    {
+        return pick_w8a8(M, N, K, num_cu, choice.path) == Q8_MROWS;
+    }
+
     hipError_t launch_w8a8(hipStream_t stream, const void* A, const void* s_tok, const void* W, const void* s_ch,
-                           void* Y, void* acc, int M, int N, int K, int num_cu, void* partial_ws,
+                           void* Y, void* acc, int M, int N, int K, int num_cu, void* partial_ws, size_t partial_bytes,
                            const LaunchChoice& choice)
     {
         W8A8Params p;
@@ -317,7 +327,9 @@ namespace nnf
         switch (pick_w8a8(M, N, K, num_cu, choice.path))
         {
         case Q8_ROWS: return launch_w8a8_gemv_rows(stream, A, s_tok, W, s_ch, Y, acc, N, K, num_cu);
-        case Q8_MROWS: return launch_w8a8_mrows(stream, A, s_tok, W, s_ch, Y, acc, M, N, K, num_cu);
+        case Q8_MROWS:
+            return launch_w8a8_mrows(stream, A, s_tok, W, s_ch, Y, acc, M, N, K, num_cu, partial_ws, partial_bytes,
+                                     (uint32_t*)choice.sync_flags, choice.sync_bytes);
         case Q8_SKINNY: return raw ? launch_q8_skinny<true>(stream, p, num_cu) : launch_q8_skinny<false>(stream, p, num_cu);
         case Q8_TILE: return launch_w8a8_gemm(stream, A, s_tok, W, s_ch, Y, acc, M, N, K, partial_ws, choice);
         default: return hipErrorInvalidValue;

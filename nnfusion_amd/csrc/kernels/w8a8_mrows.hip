@@ -51,8 +51,13 @@ namespace nnf
     __global__ __launch_bounds__(512) void w8a8_mrows_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ W,
                                                              const float* __restrict__ s_tok, const float* __restrict__ s_ch,
                                                              half_t* __restrict__ Y, int32_t* __restrict__ ACC, int M, int N,
-                                                             int K, int tiles_q, int tiles_r)
+                                                             int K, int tiles_q, int tiles_r, int ld, int32_t* __restrict__ part,
+                                                             uint32_t* __restrict__ sync)
     {
+        // K: the length of this workgroup's range of K, which starts at byte blockIdx.y * K of a row of ld bytes (one range:
+        // ld = K, part = null).  Ranges: the sums of range r go to part + r * M * N, and the last workgroup of a
+        // blockIdx.x to get there (sync: a zeroed word per blockIdx.x) adds them up and writes Y or ACC
+        const int k0 = (int)blockIdx.y * K;
         static_assert(STEPS >= 1 && STEPS * MB <= 12 && STEPS <= 8 && (MB == 1 || MB == 2) && NS >= 2 && NS <= 4, "shape of the kernel");
         constexpr int CH = STEPS * 4;    // a wavefront's 64-byte chunks of a row (one MFMA each)
         constexpr int LPS = 4;           // loads per step and wavefront
@@ -81,14 +86,14 @@ namespace nnf
         for (int c = 0; c < LPS; ++c)
         {
             const int r = c * 4 + kq, q = col;
-            w_off[c] = (uint32_t)r * (uint32_t)K + (uint32_t)((q ^ r) << 4);
+            w_off[c] = (uint32_t)r * (uint32_t)ld + (uint32_t)((q ^ r) << 4);
         }
         // where this wavefront's 256 bytes of step st start within a row; past the end of K: the row's last 256 bytes
         auto own_byte = [&](int st) { return st * (Q8MR_WAVES * Q8MR_STEP_BYTES) + wave * Q8MR_STEP_BYTES; };
         auto fetch_byte = [&](int st) { return min(own_byte(st), K - Q8MR_STEP_BYTES); };
         // step st (0 .. STEPS-1) of tile `tile` into slot `slot`
         auto issue = [&](int tile, int st, int slot) {
-            const int8_t* wsrc = W + (size_t)row0_of(tile) * K + fetch_byte(st);
+            const int8_t* wsrc = W + (size_t)row0_of(tile) * ld + k0 + fetch_byte(st);
 #pragma unroll
             for (int c = 0; c < LPS; ++c)
                 __builtin_amdgcn_global_load_lds((q8mr_global_ptr_t)(wsrc + w_off[c]),
@@ -107,7 +112,7 @@ namespace nnf
 #pragma unroll
             for (int mb = 0; mb < MB; ++mb)
             {
-                const uint8_t* a_row = reinterpret_cast<const uint8_t*>(A) + (size_t)min(mb * 16 + col, M - 1) * (size_t)K + kq * 16;
+                const uint8_t* a_row = reinterpret_cast<const uint8_t*>(A) + (size_t)min(mb * 16 + col, M - 1) * (size_t)ld + k0 + kq * 16;
 #pragma unroll
                 for (int c = 0; c < CH; ++c)
                 {
@@ -191,6 +196,58 @@ namespace nnf
         __builtin_amdgcn_s_waitcnt(q8mr_vmcnt(0)); // the reloads past the end, before the LDS goes away
         asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
         // ---- flush: parked sums -> Y (scaled) or ACC ---------------------------------------------------------------
+        if (part)
+        {
+            int32_t* mine = part + (size_t)blockIdx.y * M * N;
+            for (int idx = tid; idx < T * M * 16; idx += 512)
+            {
+                const int n = idx & 15;
+                const int im = idx >> 4;
+                const int it = im / M, m = im - it * M;
+                const size_t at = (size_t)m * N + min((t0 + it) * 16, N - 16) + n;
+                __hip_atomic_store(mine + at, parked[idx], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+            // The sums are visible to every CU (device scope, completed) before this workgroup counts itself in; the last
+            // of the ranges' workgroups to arrive adds the ranges (int32: exact in any order), finishes and leaves the word
+            // zero for the next launch.  Nobody waits.
+            __builtin_amdgcn_s_waitcnt(q8mr_vmcnt(0));
+            volatile uint32_t* arrived_before = reinterpret_cast<volatile uint32_t*>(red);
+            __syncthreads();
+            if (tid == 0)
+                *arrived_before = atomicAdd(sync + blockIdx.x, 1u);
+            __syncthreads();
+            if (*arrived_before != gridDim.y - 1)
+                return;
+            const int ranges = (int)gridDim.y;
+            for (int idx = tid; idx < T * M * 16; idx += 512)
+            {
+                const int n = idx & 15;
+                const int im = idx >> 4;
+                const int it = im / M, m = im - it * M;
+                const int gn = min((t0 + it) * 16, N - 16) + n;
+                if (gn < (t0 + it) * 16) // (a last tile moved back: these columns belong to the tile before it)
+                    continue;
+                const size_t at = (size_t)m * N + gn;
+                int32_t sum = 0;
+                for (int r0 = 0; r0 < ranges; r0 += 4)
+                {
+                    int32_t v[4];
+#pragma unroll
+                    for (int d = 0; d < 4; ++d)
+                        v[d] = __hip_atomic_load(part + (size_t)min(r0 + d, ranges - 1) * M * N + at, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+                    for (int d = 0; d < 4; ++d)
+                        sum += r0 + d < ranges ? v[d] : 0;
+                }
+                if (RAW_ACC)
+                    ACC[at] = sum;
+                else
+                    Y[at] = f32_to_f16_two_step((float)sum * s_tok[m] * s_ch[gn]);
+            }
+            if (tid == 0)
+                atomicExch(sync + blockIdx.x, 0u);
+            return;
+        }
         for (int idx = tid; idx < T * M * 16; idx += 512)
         {
             const int n = idx & 15;
@@ -213,10 +270,13 @@ namespace nnf
     {
         template <int STEPS, int MB, int NS, bool RAW>
         hipError_t launch_q8_mrows(hipStream_t stream, const void* A, const void* s_tok, const void* W, const void* s_ch, void* Y,
-                                   void* acc, int M, int N, int K, int num_cu)
+                                   void* acc, int M, int N, int K, int num_cu, int ranges = 1, int ld = 0, void* part = nullptr,
+                                   uint32_t* sync = nullptr)
         {
+            // (ranges > 1: K is the length of a range, ld the whole row, part the room for the [ranges][M][N] sums)
             const int n_tiles = (N + 15) / 16;
-            const int grid = n_tiles < num_cu ? n_tiles : num_cu;
+            const int per_range = num_cu / ranges > 0 ? num_cu / ranges : 1;
+            const int grid = n_tiles < per_range ? n_tiles : per_range;
             const int tiles_q = n_tiles / grid, tiles_r = n_tiles % grid;
             const size_t lds = workspace::w8a8_mrows_lds_bytes(M, NS, tiles_q + (tiles_r ? 1 : 0));
             if (lds > MAX_LDS_BYTES)
@@ -229,37 +289,40 @@ namespace nnf
                 if (e != hipSuccess)
                     return e;
             }
-            hipLaunchKernelGGL(kernel, dim3(grid), dim3(Q8MR_WAVES * 64), lds, stream, (const int8_t*)A, (const int8_t*)W,
-                               (const float*)s_tok, (const float*)s_ch, (half_t*)Y, (int32_t*)acc, M, N, K, tiles_q, tiles_r);
+            hipLaunchKernelGGL(kernel, dim3(grid, ranges), dim3(Q8MR_WAVES * 64), lds, stream, (const int8_t*)A, (const int8_t*)W,
+                               (const float*)s_tok, (const float*)s_ch, (half_t*)Y, (int32_t*)acc, M, N, K, tiles_q, tiles_r,
+                               ld ? ld : K, (int32_t*)part, sync);
             return hipGetLastError();
         }
 
         template <int STEPS, bool RAW>
         hipError_t launch_q8_mrows_m(hipStream_t stream, const void* A, const void* s_tok, const void* W, const void* s_ch,
-                                     void* Y, void* acc, int M, int N, int K, int num_cu)
+                                     void* Y, void* acc, int M, int N, int K, int num_cu, int ranges = 1, int ld = 0,
+                                     void* part = nullptr, uint32_t* sync = nullptr)
         {
             constexpr int NS = workspace::W8A8_MROWS_SLOTS;
             if (M <= 16)
-                return launch_q8_mrows<STEPS, 1, NS, RAW>(stream, A, s_tok, W, s_ch, Y, acc, M, N, K, num_cu);
+                return launch_q8_mrows<STEPS, 1, NS, RAW>(stream, A, s_tok, W, s_ch, Y, acc, M, N, K, num_cu, ranges, ld, part, sync);
             if constexpr (STEPS <= 6) // 16 VGPRs of activations per step and block of rows
-                return launch_q8_mrows<STEPS, 2, NS, RAW>(stream, A, s_tok, W, s_ch, Y, acc, M, N, K, num_cu);
+                return launch_q8_mrows<STEPS, 2, NS, RAW>(stream, A, s_tok, W, s_ch, Y, acc, M, N, K, num_cu, ranges, ld, part, sync);
             return hipErrorInvalidValue;
         }
 
         template <bool RAW>
         hipError_t launch_q8_mrows_any(hipStream_t stream, const void* A, const void* s_tok, const void* W, const void* s_ch,
-                                       void* Y, void* acc, int M, int N, int K, int num_cu)
+                                       void* Y, void* acc, int M, int N, int K, int num_cu, int ranges = 1, int ld = 0,
+                                       void* part = nullptr, uint32_t* sync = nullptr)
         {
             switch ((K + 2047) >> 11) // steps of 2 KiB of K
             {
-            case 1: return launch_q8_mrows_m<1, RAW>(stream, A, s_tok, W, s_ch, Y, acc, M, N, K, num_cu);
-            case 2: return launch_q8_mrows_m<2, RAW>(stream, A, s_tok, W, s_ch, Y, acc, M, N, K, num_cu);
-            case 3: return launch_q8_mrows_m<3, RAW>(stream, A, s_tok, W, s_ch, Y, acc, M, N, K, num_cu);
-            case 4: return launch_q8_mrows_m<4, RAW>(stream, A, s_tok, W, s_ch, Y, acc, M, N, K, num_cu);
-            case 5: return launch_q8_mrows_m<5, RAW>(stream, A, s_tok, W, s_ch, Y, acc, M, N, K, num_cu);
-            case 6: return launch_q8_mrows_m<6, RAW>(stream, A, s_tok, W, s_ch, Y, acc, M, N, K, num_cu);
-            case 7: return launch_q8_mrows_m<7, RAW>(stream, A, s_tok, W, s_ch, Y, acc, M, N, K, num_cu);
-            default: return launch_q8_mrows_m<8, RAW>(stream, A, s_tok, W, s_ch, Y, acc, M, N, K, num_cu);
+            case 1: return launch_q8_mrows_m<1, RAW>(stream, A, s_tok, W, s_ch, Y, acc, M, N, K, num_cu, ranges, ld, part, sync);
+            case 2: return launch_q8_mrows_m<2, RAW>(stream, A, s_tok, W, s_ch, Y, acc, M, N, K, num_cu, ranges, ld, part, sync);
+            case 3: return launch_q8_mrows_m<3, RAW>(stream, A, s_tok, W, s_ch, Y, acc, M, N, K, num_cu, ranges, ld, part, sync);
+            case 4: return launch_q8_mrows_m<4, RAW>(stream, A, s_tok, W, s_ch, Y, acc, M, N, K, num_cu, ranges, ld, part, sync);
+            case 5: return launch_q8_mrows_m<5, RAW>(stream, A, s_tok, W, s_ch, Y, acc, M, N, K, num_cu, ranges, ld, part, sync);
+            case 6: return launch_q8_mrows_m<6, RAW>(stream, A, s_tok, W, s_ch, Y, acc, M, N, K, num_cu, ranges, ld, part, sync);
+            case 7: return launch_q8_mrows_m<7, RAW>(stream, A, s_tok, W, s_ch, Y, acc, M, N, K, num_cu, ranges, ld, part, sync);
+            default: return launch_q8_mrows_m<8, RAW>(stream, A, s_tok, W, s_ch, Y, acc, M, N, K, num_cu, ranges, ld, part, sync);
             }
         }
     } // namespace
@@ -269,10 +332,17 @@ namespace nnf
 
     // acc != nullptr: the raw int32 sums, otherwise Y = fp16(acc * s_tok[m] * s_ch[n])
     hipError_t launch_w8a8_mrows(hipStream_t stream, const void* A, const void* s_tok, const void* W, const void* s_ch, void* Y,
-                                 void* acc, int M, int N, int K, int num_cu)
+                                 void* acc, int M, int N, int K, int num_cu, void* partial_ws, size_t partial_bytes, uint32_t* sync,
+                                 size_t sync_bytes)
     {
         if (!w8a8_mrows_supported(M, N, K, num_cu))
             return hipErrorInvalidValue;
+        // over two ranges of K where that pays, given the room for their sums and the words to meet at
+        const int ranges = workspace::w8a8_mrows_ranges(M, N, K, num_cu);
+        if (ranges > 1 && partial_ws && partial_bytes >= workspace::w8a8_mrows_ranges_bytes(M, N, K, num_cu) && sync &&
+            sync_bytes >= workspace::mrows_split_sync_bytes(num_cu))
+            return acc ? launch_q8_mrows_any<true>(stream, A, s_tok, W, s_ch, Y, acc, M, N, K / ranges, num_cu, ranges, K, partial_ws, sync)
+                       : launch_q8_mrows_any<false>(stream, A, s_tok, W, s_ch, Y, acc, M, N, K / ranges, num_cu, ranges, K, partial_ws, sync);
         return acc ? launch_q8_mrows_any<true>(stream, A, s_tok, W, s_ch, Y, acc, M, N, K, num_cu)
                    : launch_q8_mrows_any<false>(stream, A, s_tok, W, s_ch, Y, acc, M, N, K, num_cu);
     }

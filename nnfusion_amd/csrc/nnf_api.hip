@@ -543,9 +543,13 @@ int nnf_w8a8_gemm_variant(nnf_stream_t stream, const void* A, const void* s_tok,
     if (!nnf::w8a8_path_supported(M, N, K, dev.num_cu, choice.path))
         return NNF_ERR_UNSUPPORTED_SHAPE;
     if (!workspace_ok(nnf::w8a8_partial_bytes(M, N, K, dev.num_cu, choice), workspace, workspace_bytes))
-        return NNF_ERR_WORKSPACE_TOO_SMALL;
+    {
+        if (!nnf::w8a8_partial_optional(M, N, K, dev.num_cu, choice))
+            return NNF_ERR_WORKSPACE_TOO_SMALL;
+        workspace = nullptr, workspace_bytes = 0;
+    }
     return (int)nnf::launch_w8a8((hipStream_t)stream, A, Y ? s_tok : nullptr, W, Y ? s_ch : nullptr, Y, acc, M, N, K,
-                                 dev.num_cu, workspace, choice);
+                                 dev.num_cu, workspace, workspace_bytes, choice);
 }
 
 int nnf_w8a8_gemm(nnf_stream_t stream, const void* A, const void* s_tok, const void* W, const void* s_ch, void* Y,

@@ -198,21 +198,22 @@ def w8a8_variant_supported(m, n, k, variant):
     return bool(_lib.kernels().nnf_w8a8_variant_supported(m, n, k, W8A8_VARIANTS[variant]))
 
 
-def _w8a8_variant(a, s_tok, w, s_ch, y, acc, variant, plan, workspace):
+def _w8a8_variant(a, s_tok, w, s_ch, y, acc, variant, plan, workspace, sync=None):
     lib = _lib.kernels()
     m, k = a.shape
     n = w.shape[0]
     v = W8A8_VARIANTS[variant]
-    keep, plan_ptr = _plan_arg(plan)
+    keep, plan_ptr = _plan_arg(plan, sync)
     if workspace is None:
         workspace = _ws(lib.nnf_w8a8_gemm_variant_workspace_bytes(m, n, k, v, plan_ptr), a.device)
     _check(lib.nnf_w8a8_gemm_variant(_stream(), a.data_ptr(), _p(s_tok), w.data_ptr(), _p(s_ch), _p(y), _p(acc), m, n, k,
                                      v, plan_ptr, workspace.data_ptr(), workspace.numel()), "nnf_w8a8_gemm_variant")
 
 
-def w8a8_gemm(a, s_tok, w, s_ch, out=None, workspace=None, variant="auto", plan=None):
+def w8a8_gemm(a, s_tok, w, s_ch, out=None, workspace=None, variant="auto", plan=None, sync=None):
     """Y fp16 [M,N] = fp16((float)(A . W^T) * s_tok[m] * s_ch[n]) ; a i8 [M,K], w i8 [N,K].  A variant (a key of
-    W8A8_VARIANTS) or plan (tile_rows, k_parts) goes through nnf_w8a8_gemm_variant."""
+    W8A8_VARIANTS), a plan (tile_rows, k_parts) or `sync` (see sync_flags: a few rows with a long K then run over
+    two ranges of K in one launch) goes through nnf_w8a8_gemm_variant."""
     lib = _lib.kernels()
     m, k = a.shape
     n = w.shape[0]
@@ -220,8 +221,8 @@ def w8a8_gemm(a, s_tok, w, s_ch, out=None, workspace=None, variant="auto", plan=
     assert s_tok.dtype == torch.float32 and s_ch.dtype == torch.float32
     if out is None:
         out = torch.empty((m, n), dtype=torch.float16, device=a.device)
-    if variant != "auto" or plan is not None:
-        _w8a8_variant(a, s_tok, w, s_ch, out, None, variant, plan, workspace)
+    if variant != "auto" or plan is not None or sync is not None:
+        _w8a8_variant(a, s_tok, w, s_ch, out, None, variant, plan, workspace, sync)
         return out
     need = lib.nnf_w8a8_gemm_workspace_bytes(m, n, k)
     if workspace is None:
@@ -231,7 +232,7 @@ def w8a8_gemm(a, s_tok, w, s_ch, out=None, workspace=None, variant="auto", plan=
     return out
 
 
-def w8a8_gemm_acc(a, w, out=None, workspace=None, variant="auto", plan=None):
+def w8a8_gemm_acc(a, w, out=None, workspace=None, variant="auto", plan=None, sync=None):
     """acc i32 [M,N] = A . W^T, exact."""
     lib = _lib.kernels()
     m, k = a.shape
@@ -239,8 +240,8 @@ def w8a8_gemm_acc(a, w, out=None, workspace=None, variant="auto", plan=None):
     assert a.dtype == torch.int8 and w.dtype == torch.int8
     if out is None:
         out = torch.empty((m, n), dtype=torch.int32, device=a.device)
-    if variant != "auto" or plan is not None:
-        _w8a8_variant(a, None, w, None, None, out, variant, plan, workspace)
+    if variant != "auto" or plan is not None or sync is not None:
+        _w8a8_variant(a, None, w, None, None, out, variant, plan, workspace, sync)
         return out
     need = lib.nnf_w8a8_gemm_workspace_bytes(m, n, k)
     if workspace is None:

@@ -418,16 +418,34 @@ int main(int argc, char** argv)
         EXPECT(n->get_output_element_type(0) == element::f16 && n->get_output_shape(0) == (Shape{32, 8192}));
         auto kq = sel.pick_first(n, ROCM_GPU).second;
         auto fu = kq->get_or_emit_source();
-        // M = 32: 64 x 256 tiles (32 of them), K split 8 ways: 8 x 32 x 8192 int32 partial sums in a scratch tensor
-        EXPECT(kq->m_context->tensors.size() == 1 && kq->m_context->tensors[0]->size() == (size_t)8 * 32 * 8192 * 4);
+        // M = 32: 64 x 256 tiles (32 of them), K split 8 ways: 8 x 32 x 8192 int32 partial sums in a scratch tensor; the
+        // row-streaming kernel, which the library prefers here, runs over two ranges of K that meet at a word per workgroup
+        EXPECT(kq->m_context->tensors.size() == 2 && kq->m_context->tensors[0]->size() == (size_t)8 * 32 * 8192 * 4 &&
+               kq->m_context->tensors[1]->size() == 1024 && kq->m_context->tensors[1]->is_persistent());
         EXPECT(fu->body_unit->get_code() ==
-               "NNF_HIP_CHECK(nnf_w8a8_gemm(stream, input0, input1, input2, input3, output0, 32, 8192, 8192, " +
+               "const nnf_plan plan = {0, 0, 0, " + kq->m_context->tensors[1]->get_name() + ", 1024, 0};\n" +
+                   "NNF_HIP_CHECK(nnf_w8a8_gemm_variant(stream, input0, input1, input2, input3, output0, nullptr, 32, 8192, 8192, "
+                   "NNF_W8A8_AUTO, &plan, " +
                    kq->m_context->tensors[0]->get_name() + ", 8388608));\n");
         auto n2 = g.add_node_and_edge(std::make_shared<op::GenericOp>("q", "QuantDotW8A8", op::OpConfig::any::parse("{\"out_type\": \"i32\"}")),
                                       {a, st, w, sc});
         EXPECT(n2->get_output_element_type(0) == element::i32);
         CONTAINS(sel.pick_first(n2, ROCM_GPU).second->get_or_emit_source()->body_unit->get_code(),
-                 "nnf_w8a8_gemm_acc(stream, input0, input2, output0, 32, 8192, 8192");
+                 "nnf_w8a8_gemm_variant(stream, input0, nullptr, input2, nullptr, nullptr, output0, 32, 8192, 8192, NNF_W8A8_AUTO, &plan, ");
+        {
+            // a product the tile GEMM takes: the plain calls
+            graph::Graph g3;
+            auto a3 = param(g3, element::i8, Shape{512, 8192});
+            auto st3 = param(g3, element::f32, Shape{512});
+            auto n3 = g3.add_node_and_edge(std::make_shared<op::GenericOp>("q", "QuantDotW8A8", op::OpConfig::any()),
+                                           {a3, st3, param(g3, element::i8, Shape{8192, 8192}), param(g3, element::f32, Shape{8192})});
+            CONTAINS(sel.pick_first(n3, ROCM_GPU).second->get_or_emit_source()->body_unit->get_code(),
+                     "nnf_w8a8_gemm(stream, input0, input1, input2, input3, output0, 512, 8192, 8192");
+            auto n4 = g3.add_node_and_edge(std::make_shared<op::GenericOp>("q", "QuantDotW8A8", op::OpConfig::any::parse("{\"out_type\": \"i32\"}")),
+                                           {a3, st3, param(g3, element::i8, Shape{8192, 8192}), param(g3, element::f32, Shape{8192})});
+            CONTAINS(sel.pick_first(n4, ROCM_GPU).second->get_or_emit_source()->body_unit->get_code(),
+                     "nnf_w8a8_gemm_acc(stream, input0, input2, output0, 512, 8192, 8192");
+        }
 
         graph::Graph g2;
         auto x = param(g2, element::f16, Shape{256, 4096});
@@ -1248,6 +1266,13 @@ int main(int argc, char** argv)
             EXPECT(ws::w8a8_skinny_fits(1, k) && ws::w8a8_gemm(1, 4096, k) == 0);
         }
         EXPECT(!ws::w8a8_skinny_fits(16, 8192) && ws::w8a8_gemm(16, 8192, 8192) > 0);
+        // the row-streaming kernel over two ranges of K: 8 .. 32 rows, K from 8192 in multiples of 512, at most four tiles
+        // per workgroup of a range; the workspace query covers the ranges' int32 sums
+        EXPECT(ws::w8a8_mrows_ranges(8, 4096, 8192, 256) == 2 && ws::w8a8_mrows_ranges(32, 8192, 8192, 256) == 2 &&
+               ws::w8a8_mrows_ranges(16, 4096, 14336, 256) == 2);
+        EXPECT(ws::w8a8_mrows_ranges(7, 4096, 8192, 256) == 1 && ws::w8a8_mrows_ranges(32, 8192, 4096, 256) == 1 &&
+               ws::w8a8_mrows_ranges(32, 8208, 8192, 256) == 1 && ws::w8a8_mrows_ranges(16, 4096, 11008, 256) == 1);
+        EXPECT(ws::w8a8_mrows_ranges_bytes(8, 4096, 8192, 256) == (size_t)2 * 8 * 4096 * 4 && ws::w8a8_gemm(8, 4096, 8192) >= (size_t)2 * 8 * 4096 * 4);
         // fp16 x int4 tile GEMM: the (tile, superstep) units are split evenly over at most one workgroup per CU; a
         // workgroup parks at most two partial tiles; whole tiles need no workspace
         {

@@ -19,8 +19,9 @@ def _t(gpu, *arrays):
 # choice where it does not): "auto"; "skinny": the split-K M <= 16 kernel; "mfma_rows": the row-streaming MFMA kernel
 # (2 <= M <= 32, K = 1024 .. 16384 in multiples of 256); otherwise the MFMA tile GEMM with a plan (tile_rows, k_parts):
 # tiles of 256 x 256, 256 x 128 (third value: the columns), 128 x 128 or 64 x 256 outputs (0: the library's choice) and the
-# number of K ranges (int32 partial sums, added exactly by the reduction pass)
-@pytest.fixture(params=["auto", "skinny", "mfma_rows", (0, 0), (256, 1, 256), (256, 2, 256), (256, 1, 128), (256, 3, 128), (256, 0),
+# number of K ranges (int32 partial sums, added exactly by the reduction pass); "auto-sync": the library's choice given
+# synchronisation words (8 .. 32 rows with K from 8192: the row-streaming kernel over two ranges of K in one launch)
+@pytest.fixture(params=["auto", "auto-sync", "skinny", "mfma_rows", (0, 0), (256, 1, 256), (256, 2, 256), (256, 1, 128), (256, 3, 128), (256, 0),
                         (128, 1), (128, 3), (64, 1), (64, 2)],
                 ids=lambda p: p if isinstance(p, str) else "gemm-rows%d-parts%d" % p[:2] + ("-cols%d" % p[2] if len(p) > 2 else ""))
 def path(request):
@@ -37,7 +38,15 @@ def _kw(path, m, n, k):
         return {"variant": "gemv_rows"} if m > 1 and ops.w8a8_variant_supported(m, n, k, "gemv_rows") else {}
     if path == "auto":
         return {}
+    if path == "auto-sync":
+        import torch
+
+        return {"sync": ops.sync_flags(torch.device("cuda:0"))}
     return {"variant": "gemm_mfma", "plan": path}
+
+
+def _words_left_zero(kw):
+    return "sync" not in kw or int(kw["sync"].count_nonzero()) == 0
 
 
 def _big_ws(gpu):
@@ -60,6 +69,8 @@ def _big_ws(gpu):
     # K that does not fill the last 2-KiB step, K above 8192
     (16, 4111, 11008), (5, 100, 1024), (9, 520, 2560), (32, 300, 7168), (24, 1000, 3584), (12, 2000, 14336), (16, 64, 16384),
     (17, 250, 5376), (32, 4111, 11008), (20, 300, 12288), (24, 100, 9216),
+    # two ranges of K given synchronisation words: one to four tiles per workgroup, a last tile moved back, K = 16384
+    (8, 4096, 8192), (32, 4111, 8192), (13, 6000, 16384), (24, 8192, 9216),
 ])
 def test_accumulators_bit_exact(gpu, path, m, n, k):
     import torch
@@ -78,6 +89,7 @@ def test_accumulators_bit_exact(gpu, path, m, n, k):
     assert np.array_equal(acc, ref)
     # the epilogue is a closed form of exact inputs: bit-identical fp16
     assert np.array_equal(y.view(np.uint16), oracle.w8a8_epilogue(ref, s_tok, s_ch).view(np.uint16))
+    assert _words_left_zero(kw)
 
 
 def test_extreme_values_do_not_overflow(gpu, path):
@@ -92,9 +104,11 @@ def test_extreme_values_do_not_overflow(gpu, path):
     w = np.full((n, k), 127, np.int8)
     w[::2] = -127
     ta, tw = _t(gpu, a, w)
-    acc = ops.w8a8_gemm_acc(ta, tw, workspace=_big_ws(gpu), **_kw(path, m, n, k)).cpu().numpy()
+    kw = _kw(path, m, n, k)
+    acc = ops.w8a8_gemm_acc(ta, tw, workspace=_big_ws(gpu), **kw).cpu().numpy()
     torch.cuda.synchronize()
     assert np.array_equal(acc, oracle.w8a8_acc(a, w))
+    assert _words_left_zero(kw)
     assert abs(int(acc[0, 1])) == 8192 * 127 * 127
 
 
