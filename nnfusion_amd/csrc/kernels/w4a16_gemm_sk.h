@@ -18,13 +18,17 @@
 //     tile, each wavefront owning all TM*32 rows of a strip of TN*32 columns (TM x TN MFMA tiles of
 //     32x32x16).  A weight belongs to exactly one wavefront: it is unpacked once per workgroup (16 VALU
 //     operations per 8 weights, feeding TM MFMAs each), not once per wavefront row.
-//   * The weights never touch LDS.  A lane owns one weight row of each of its column tiles and one half
-//     of every 64-wide K step; it fetches its bytes straight into registers, one "superstep" of 256 k
-//     (two quantization groups, four K steps) at a time: four 16-byte loads that together with the
-//     other half's cover whole 128-byte lines of the row (a load per K step would touch 32 bytes of
-//     each line and fetch the line four times: the 32 KiB first-level cache does not hold a line that
-//     long).  Two register sets: superstep s+1 is requested while s is multiplied.  The group scales
-//     travel the same way (two 2-byte loads per row and superstep).
+//   * A lane owns one weight row of each of its column tiles and one half of every 64-wide K step, and holds the
+//     weights of one "superstep" of 256 k (two quantization groups, four K steps) in registers at a time: 4 x 16
+//     bytes per column tile.  The largest tile (256 x 256) fetches them straight into registers, two register sets,
+//     superstep s+1 requested while s is multiplied.  Such a load touches 32 bytes of each of 32 rows; measured
+//     with the same bytes fetched as whole lines, loads of that shape cost the memory pipeline about four times
+//     what loads of whole 128-byte lines cost it, and with smaller tiles -- fewer MFMAs per load -- the K loop
+//     waits for them.  Every other tile therefore moves a superstep's 32 x 128 bytes per column tile global -> LDS
+//     (four loads of 8 whole rows, global_load_lds_dwordx4, into an area of the wavefront's own: no barrier) one
+//     superstep ahead, and from there into the registers (four ds_read_b128 per column tile) at the last barrier
+//     of the superstep before, under that quarter's MFMAs.  The group scales are two 2-byte loads per row and
+//     superstep into registers in both forms.
 //   * The activations go global -> LDS asynchronously (global_load_lds_dwordx4, no register staging)
 //     into a ring of three stages of BK = 64; the loads for K step kt+3 are issued from the barrier of
 //     step kt on, a quarter of them per quarter step.
@@ -125,7 +129,14 @@ namespace nnf
             static constexpr int STAGE_BYTES = A_TILE_BYTES + CONST_BYTES;
             // the epilogue turns the results through a private piece of the ring per wavefront
             static constexpr int EPILOGUE_BYTES = WAVES * (TM >= 2 ? 2 : 1) * 32 * (TN * 64 + 16);
-            static constexpr int LDS_BYTES = STAGES * STAGE_BYTES > EPILOGUE_BYTES ? STAGES * STAGE_BYTES : EPILOGUE_BYTES;
+            // Weights through LDS (see the kernel): every tile but the largest, whose K step is long enough for the loads
+            // it has and which has the least LDS bandwidth to spare (M = 4096, N = K = 8192: 2 % slower that way;
+            // M = 1024 on 256 x 128 tiles: 3 % faster; 128-row tiles: 3 - 7 % faster).  Behind the ring: per wavefront
+            // and column tile the 32 x 128 bytes of the next superstep
+            static constexpr bool W_VIA_LDS = !(TM == 8 && TN >= 2);
+            static constexpr int W_LDS_OFFSET = STAGES * STAGE_BYTES > EPILOGUE_BYTES ? STAGES * STAGE_BYTES : EPILOGUE_BYTES;
+            static constexpr int W_LDS_BYTES = W_VIA_LDS ? WAVES * TN * 4096 : 0;
+            static constexpr int LDS_BYTES = W_LDS_OFFSET + W_LDS_BYTES;
             static constexpr size_t SLOT_FLOATS = (size_t)BM * BN;
         };
 
@@ -659,6 +670,12 @@ namespace nnf
         // LDS destinations of this wavefront's loads within a stage
         const uint32_t lds_a = (uint32_t)(wave * TM * 1024);
         const uint32_t lds_g = (uint32_t)(A_TILE_BYTES + wave * 256);
+        // the wavefront's weights of the next superstep; a lane's piece for K step x: piece 2 x + h of row l32
+        const uint32_t lds_w = (uint32_t)(T::W_LDS_OFFSET + wave * TN * 4096);
+        uint32_t w_rd[4];
+#pragma unroll
+        for (int x = 0; x < 4; ++x)
+            w_rd[x] = lds0 + lds_w + (uint32_t)(l32 * 128 + (((2 * x + h) ^ ((l32 >> 1) & 7)) << 4));
 
         // (sync) the shared tiles this workgroup has parked a part of -- its first and its last segment -- and, in
         // thread 0, the tile's first sync word as the arrival found it
@@ -721,20 +738,41 @@ namespace nnf
                 __builtin_amdgcn_global_load_lds((global_ptr)(g_base + here(g_off)), (lds_ptr)(smem + stage_off + lds_g), 4, 0, 0);
             };
 
-            // ---- weights and scales: straight into registers -----------------------------------------------------
+            // ---- weights and scales ----------------------------------------------------------------------------------
             // lane (l32, h) owns weight row l32 of each of the wavefront's column tiles; of K step t of a
-            // superstep it owns k = 64 t + 32 h .. + 31: the 16 bytes at 32 t + 16 h of the superstep's 128
-            uint32_t w_off[TN], s_off[TN], z_off[TN];
+            // superstep it owns k = 64 t + 32 h .. + 31: the 16 bytes at 32 t + 16 h of the superstep's 128.
+            // Fetched that way -- 32 bytes of each of 32 rows per load -- the loads cost the memory pipeline four times
+            // what whole 128-byte lines cost it (timed with the same bytes fetched as whole lines: M = 128, N = K = 8192
+            // 32.0 -> 27.6 us).  So a superstep's 32 x 128 bytes per column tile go global -> LDS as whole lines, four
+            // loads of 8 rows (lane i: row 8 c + i / 8, 16-byte piece (i % 8) ^ swizzle(row), as for the activations), into a
+            // private area of the wavefront, one superstep ahead, and move into the registers with four ds_read_b128
+            // when the superstep begins.
+            // the row of the wavefront's column tile j that sits at place r (0 .. 31)
+            auto weight_row = [&](int j, int r) {
+                if (GATE) // column tiles 0 .. TN/2-1: gate rows, the others: the up rows that pair with them
+                    return min((j >= TN / 2 ? p.up_row_offset + n0 + (j - TN / 2) * 32 : n0 + j * 32) + wave * (TN / 2) * 32 + r,
+                               p.up_row_offset + p.N - 1);
+                return min(n0 + wave * (TN * 32) + j * 32 + r, p.N - 1);
+            };
+            constexpr bool W_LDS = T::W_VIA_LDS;
+            constexpr int WSETS = W_LDS ? 1 : 2; // register sets of weights: without the detour the next superstep's as well
+            uint32_t w_off[TN][4], s_off[TN], z_off[TN]; // (straight into registers: w_off[j][0] only)
+            // 64 in the lanes that fetch a piece of the second 64 bytes (K not a multiple of 256: they repeat the first
+            // 64 in the last superstep), for loads 0 and 2 (the swizzle of rows 8 c + i / 8 flips it for loads 1 and 3)
+            const uint32_t w_second_half = (lane & 4) ? 64u : 0u;
 #pragma unroll
             for (int j = 0; j < TN; ++j)
             {
-                int gn;
-                if (GATE) // column tiles 0 .. TN/2-1: gate rows, the others: the up rows that pair with them
-                    gn = min((j >= TN / 2 ? p.up_row_offset + n0 + (j - TN / 2) * 32 : n0 + j * 32) + wave * (TN / 2) * 32 + l32,
-                             p.up_row_offset + p.N - 1);
-                else
-                    gn = min(n0 + wave * (TN * 32) + j * 32 + l32, p.N - 1);
-                w_off[j] = (uint32_t)((size_t)gn * (K >> 1) + (k_begin >> 1) + h * 16);
+#pragma unroll
+                for (int c = 0; c < 4; ++c)
+                {
+                    const int r = c * 8 + (lane >> 3);
+                    const int piece = (lane & 7) ^ ((r >> 1) & 7);
+                    w_off[j][c] = (uint32_t)((size_t)weight_row(j, r) * (K >> 1) + (k_begin >> 1) + piece * 16);
+                }
+                const int gn = weight_row(j, l32);
+                if constexpr (!W_LDS)
+                    w_off[j][0] = (uint32_t)((size_t)gn * (K >> 1) + (k_begin >> 1) + h * 16);
                 if constexpr (QZ)
                 {
                     // the scales of the row's groups of this superstep; their zero points, or (no tensor) the scales again
@@ -745,7 +783,9 @@ namespace nnf
                     s_off[j] = (uint32_t)(((size_t)gn * G + 2 * ss_begin) * 2);
             }
             const uint8_t* s_bytes = reinterpret_cast<const uint8_t*>(p.S);
-            uintx4 wbuf[2][TN][4];    // [register set][column tile][K step of the superstep]
+            // the weights of the superstep at work (set 0; straight into registers: and of the next one, set 1):
+            // [set][column tile][K step of the superstep]
+            uintx4 wbuf[WSETS][TN][4];
             uint32_t sraw[2][TN][SW]; // the group scales of the superstep, as loaded
             half2_t sc[2][TN][NSC];   // ... as (s, s); zero for a group past K
             uint32_t zraw[2][TN];     // QZ: the zero points of the superstep, as loaded
@@ -755,7 +795,8 @@ namespace nnf
             // repeats the first (and is multiplied by a scale of zero).
             struct WBase
             {
-                const uint8_t *w_lo, *w_hi, *s_lo, *s_hi;
+                const uint8_t *w, *s_lo, *s_hi;
+                uint32_t repeat; // 64: the second 64 bytes of the superstep do not exist
             };
             auto w_base_of = [&](int s) {
                 s = min(s, NSS - 1);
@@ -763,24 +804,31 @@ namespace nnf
                 if constexpr (QZ)
                 {
                     // (K is a multiple of 256)  s_lo: the scales; s_hi: the zero points, or the scales again
-                    b.w_lo = scalar_base(p.Wq + (size_t)s * 128);
-                    b.w_hi = scalar_base(p.Wq + (size_t)s * 128 + 64);
+                    b.w = scalar_base(p.Wq + (size_t)s * 128);
+                    b.repeat = 0u;
                     b.s_lo = scalar_base(s_bytes + (size_t)s * (512 >> GSH));
                     b.s_hi = p.zps ? scalar_base(p.zps + (size_t)s * (128 >> GSH)) : b.s_lo;
                     return b;
                 }
                 const bool second_valid = 2 * (ss_begin + s) + 1 < G;
-                b.w_lo = scalar_base(p.Wq + (size_t)s * 128);
-                b.w_hi = scalar_base(p.Wq + (size_t)s * 128 + (second_valid ? 64 : 0));
+                b.w = scalar_base(p.Wq + (size_t)s * 128);
+                b.repeat = second_valid ? 0u : 64u;
                 b.s_lo = scalar_base(s_bytes + (size_t)s * 4);
                 b.s_hi = scalar_base(s_bytes + (size_t)s * 4 + (second_valid ? 2 : 0));
                 return b;
             };
-            // load x (0 .. 3: weights of K step x, 4 .. 5: scales) of column tile j -> register set
+            // load x of column tile j.  0 .. 3: rows 8 x .. 8 x + 7 of its weights -> the wavefront's area in LDS;
+            // 4 .. 5: scales -> register set
             auto load_w = [&](auto set_c, auto j_c, auto x_c, const WBase& b) {
                 constexpr int set = decltype(set_c)::value, j = decltype(j_c)::value, x = decltype(x_c)::value;
-                if constexpr (x < 4)
-                    wbuf[set][j][x] = *(const uintx4 __attribute__((address_space(1)))*)((x < 2 ? b.w_lo : b.w_hi) + (x & 1) * 32 + here(w_off[j]));
+                if constexpr (x < 4 && W_LDS)
+                {
+                    const uint32_t second = (x & 1) ? 64u - w_second_half : w_second_half;
+                    __builtin_amdgcn_global_load_lds((global_ptr)(b.w + (here(w_off[j][x]) - (second & b.repeat))),
+                                                     (lds_ptr)(smem + lds_w + j * 4096 + x * 1024), 16, 0, 0);
+                }
+                else if constexpr (x < 4) // the 16 bytes at 32 x + 16 h of the lane's own row
+                    wbuf[set][j][x] = *(const uintx4 __attribute__((address_space(1)))*)(b.w + (x * 32 - (x >= 2 ? b.repeat : 0u)) + here(w_off[j][0]));
                 else if constexpr (!QZ)
                     sraw[set][j][x - 4] = *(const uint16_t __attribute__((address_space(1)))*)((x == 4 ? b.s_lo : b.s_hi) + here(s_off[j]));
                 else if constexpr (x == 4)
@@ -911,7 +959,18 @@ namespace nnf
                         workgroup_barrier();
                         __builtin_amdgcn_sched_barrier(0);
                         if constexpr (T_ == 3)
+                        {
                             prepare_scales(std::integral_constant<int, 1>{}, s + 1);
+                            // the next superstep's weights have landed in the wavefront's area (the wait above), this
+                            // superstep's are used up: LDS -> registers, waited for ahead of the first unpacking below
+                            if constexpr (W_LDS)
+                                unroll_for<0, TN>([&](auto j_c) {
+                                    unroll_for<0, 4>([&](auto x_c) {
+                                        lds_read_b128_nowait<decltype(j_c)::value * 4096>(wbuf[0][decltype(j_c)::value][decltype(x_c)::value],
+                                                                                          w_rd[decltype(x_c)::value]);
+                                    });
+                                });
+                        }
                     }
                     unroll_for<0, NREG>([&](auto r_c) {
                         constexpr int R = decltype(r_c)::value;
@@ -972,14 +1031,22 @@ namespace nnf
                             lds_wait_also(gm[2]);
                             lds_wait_also(gm[3]);
                         }
+                        if constexpr (W_LDS && Q == 3 && T_ == 3 && (SHIFTED ? R == 1 : R == 0))
+                        {
+                            // the weights read back at the top of this quarter: behind them this region's fragment reads
+                            // (RMS: the wait above was stricter)
+                            if constexpr (!RMS)
+                                lds_wait<FPR>(wbuf[0][0][0]);
+                            unroll_for<0, 4 * TN>([&](auto i_c) { lds_wait_also(wbuf[0][decltype(i_c)::value / 4][decltype(i_c)::value % 4]); });
+                        }
                         unroll_for<P0, P1>([&](auto pc_c) {
                             constexpr int pc = decltype(pc_c)::value;
                             constexpr int j = pc / 4, e = pc % 4;
                             // word Q+1 of this step, or word 0 of the next step
                             constexpr int NT = Q == 3 ? (T_ + 1) & 3 : T_;
-                            constexpr int NSET = (Q == 3 && T_ == 3) ? 1 : 0;
+                            constexpr int NSET = (Q == 3 && T_ == 3) ? 1 : 0; // (the scales; the weights are in place by then)
                             constexpr int NQ = (Q + 1) & 3;
-                            const uintx4& wq = wbuf[NSET][j][NT];
+                            const uintx4& wq = wbuf[W_LDS ? 0 : NSET][j][NT];
                             const uint32_t w = NQ == 0 ? wq.x : NQ == 1 ? wq.y : NQ == 2 ? wq.z : wq.w;
                             if constexpr (QZ)
                             {
@@ -1057,6 +1124,13 @@ namespace nnf
             else if (u >= u_end)
                 NNF_SK_STAMP(12); // ... and those of the last segment, when it is not the first
             prepare_scales(I0{}, 0);
+            // superstep 0's weights: LDS -> registers
+            if constexpr (W_LDS)
+                unroll_for<0, TN>([&](auto j_c) {
+                    unroll_for<0, 4>([&](auto x_c) {
+                        lds_read_b128_nowait<decltype(j_c)::value * 4096>(wbuf[0][decltype(j_c)::value][decltype(x_c)::value], w_rd[decltype(x_c)::value]);
+                    });
+                });
             if constexpr (RMS)
                 unroll_for<0, 4>([&](auto g_c) { lds_read_b128_nowait<decltype(g_c)::value * 16>(gm[decltype(g_c)::value], g_rd); });
             unroll_for<0, TM>([&](auto f_c) { read_frag(I0{}, f_c, a_rd[0]); });
@@ -1067,6 +1141,10 @@ namespace nnf
                 lds_wait_also(gm[2]);
                 lds_wait_also(gm[3]);
             }
+            else if constexpr (W_LDS)
+                lds_wait<(TM < 15 ? TM : 15)>(wbuf[0][0][0]);
+            if constexpr (W_LDS)
+                unroll_for<0, 4 * TN>([&](auto i_c) { lds_wait_also(wbuf[0][decltype(i_c)::value / 4][decltype(i_c)::value % 4]); });
             unroll_for<0, 4 * TN>([&](auto pc_c) {
                 constexpr int pc = decltype(pc_c)::value;
                 if constexpr (QZ)
@@ -1098,9 +1176,12 @@ namespace nnf
 #pragma unroll
                     for (int j = 0; j < TN; ++j)
                     {
+                        if constexpr (!W_LDS)
+                        {
 #pragma unroll
-                        for (int x = 0; x < 4; ++x)
-                            wbuf[0][j][x] = wbuf[1][j][x];
+                            for (int x = 0; x < 4; ++x)
+                                wbuf[0][j][x] = wbuf[WSETS - 1][j][x];
+                        }
                         if constexpr (QZ)
                         {
 #pragma unroll
