@@ -168,9 +168,10 @@ namespace nnf
         //   * The TM activation loads (+ gamma with RMS) for step kt+3 go out in four positions: position 0 in
         //     quarter 3 of step kt (right behind the barrier that frees the stage), positions 1 .. 3 in quarters
         //     0 .. 2 of step kt+1.
-        //   * The six loads (four of weights, two scales) per column tile for the next superstep go out in quarters
-        //     0 .. 2 of step T = w_step(tile), ahead of that quarter's activation loads.
-        template <int TM, int TN, bool RMS>
+        //   * The NW loads (four of weights, the others scales and zero points) per column tile for the next superstep
+        //     go out in quarters 0 .. 2 of step T = w_step(tile), ahead of that quarter's activation loads.
+        //     (NW: loads per column tile and superstep, weights and scales)
+        template <int TM, int TN, bool RMS, int NW>
         struct Sched
         {
             static constexpr int a_pos(int i) { return (i * 4) / TM; }
@@ -188,7 +189,7 @@ namespace nnf
             {
                 int n = 0;
                 for (int j = 0; j < TN; ++j)
-                    n += w_step(j) == T ? 6 : 0;
+                    n += w_step(j) == T ? NW : 0;
                 return n;
             }
             // the step's weight loads number [w_begin(T, Q), w_begin(T, Q + 1)) go out in quarter Q (0 .. 2)
@@ -200,13 +201,13 @@ namespace nnf
                 for (int j = 0; j < TN; ++j)
                     if (w_step(j) == T)
                     {
-                        if (x < seen + 6)
+                        if (x < seen + NW)
                             return j;
-                        seen += 6;
+                        seen += NW;
                     }
                 return -1;
             }
-            static constexpr int w_which(int x) { return x % 6; }
+            static constexpr int w_which(int x) { return x % NW; }
             static constexpr int loads_at(int T, int Q)
             {
                 return Q == 3 ? a_loads_at(0) : (w_begin(T, Q + 1) - w_begin(T, Q)) + a_loads_at(Q + 1);
@@ -569,7 +570,10 @@ namespace nnf
     {
         using namespace gemm_sk;
         using T = Tile<TM, TN>;
-        using SCH = Sched<TM, TN, RMS>;
+        // loads per column tile and superstep: four of weights; two of scales and zero points, or (the specialised kernel)
+        // three of scales, see load_w
+        constexpr int NW = QG != 0 ? 6 : 7;
+        using SCH = Sched<TM, TN, RMS, NW>;
         static_assert(!(GATE && (BIAS || RESID)), "SiLU-gate is not combined with bias or residual");
         static_assert(TN == 1 || TN == 2 || TN == 4, "column tiles per wavefront");
         static_assert(!GATE || TN >= 2, "gate and up rows are the two halves of a wavefront's column tiles");
@@ -577,7 +581,7 @@ namespace nnf
         constexpr bool QZ = QG != 0;
         constexpr int GSH = QZ ? QG : 7;                    // log2 of the group size
         constexpr int NSC = QZ ? (QG == 7 ? 2 : 4) : 2;     // scales a lane keeps per column tile and superstep
-        constexpr int SW = QZ ? (QG == 5 ? 4 : QG == 6 ? 2 : 1) : 2; // registers of scales as loaded
+        constexpr int SW = QZ ? (QG == 5 ? 4 : QG == 6 ? 2 : 1) : 3; // registers of scales as loaded
         constexpr int BM = T::BM, BN = T::BN;
         constexpr int A_TILE_BYTES = T::A_TILE_BYTES, STAGE_BYTES = T::STAGE_BYTES;
         constexpr int BN_OUT = GATE ? BN / 2 : BN;
@@ -598,6 +602,7 @@ namespace nnf
         const int l32 = lane & 31, h = lane >> 5;
         const int K = p.K;
         const int G = K >> GSH;
+        const bool g_even = !(G & 1);
         const int SS = p.supersteps;
         const int grid = (int)gridDim.x;
         const uint32_t lds0 = lds_address(smem);
@@ -830,7 +835,21 @@ namespace nnf
                 else if constexpr (x < 4) // the 16 bytes at 32 x + 16 h of the lane's own row
                     wbuf[set][j][x] = *(const uintx4 __attribute__((address_space(1)))*)(b.w + (x * 32 - (x >= 2 ? b.repeat : 0u)) + here(w_off[j][0]));
                 else if constexpr (!QZ)
-                    sraw[set][j][x - 4] = *(const uint16_t __attribute__((address_space(1)))*)((x == 4 ? b.s_lo : b.s_hi) + here(s_off[j]));
+                {
+                    // Loads 4 .. 6, the superstep's two scales of the lane's row.  A load costs by the lines it touches
+                    // (32 rows here).  An even number of groups per row (K a multiple of 256): the two are one aligned
+                    // word, load 4 brings it and loads 5 and 6 ask for the same two bytes in every lane (one line).
+                    // An odd number: load 4 is the one that asks for one line, loads 5 and 6 bring a scale each.
+                    // (One sequence of instructions for both: a branch around a load made the compiler drain every
+                    // load in flight.)
+                    const uint32_t mine = here(s_off[j]);
+                    if constexpr (x == 4)
+                        sraw[set][j][2] = *(const uint32_t __attribute__((address_space(1)))*)(b.s_lo + (g_even ? mine : 0u));
+                    else if constexpr (x == 5)
+                        sraw[set][j][0] = *(const uint16_t __attribute__((address_space(1)))*)(b.s_lo + (g_even ? 0u : mine));
+                    else
+                        sraw[set][j][1] = *(const uint16_t __attribute__((address_space(1)))*)((g_even ? b.s_lo : b.s_hi) + (g_even ? 0u : mine));
+                }
                 else if constexpr (x == 4)
                 {
                     if constexpr (QG == 5)
@@ -891,8 +910,10 @@ namespace nnf
 #pragma unroll
                 for (int j = 0; j < TN; ++j)
                 {
-                    sc[set][j][0] = as_half2(__builtin_amdgcn_perm(sraw[set][j][0], sraw[set][j][0], 0x01000100u));
-                    sc[set][j][1] = as_half2(second_valid ? __builtin_amdgcn_perm(sraw[set][j][1], sraw[set][j][1], 0x01000100u) : 0u);
+                    const uint32_t first = g_even ? sraw[set][j][2] : sraw[set][j][0];
+                    const uint32_t second = g_even ? sraw[set][j][2] : sraw[set][j][1];
+                    sc[set][j][0] = as_half2(__builtin_amdgcn_perm(first, first, 0x01000100u));
+                    sc[set][j][1] = as_half2(second_valid ? __builtin_amdgcn_perm(second, second, g_even ? 0x03020302u : 0x01000100u) : 0u);
                 }
             };
 
@@ -1103,7 +1124,7 @@ namespace nnf
                 // have asked for
                 const WBase w0 = w_base_of(0);
                 unroll_for<0, TM>([&](auto i_c) { load_a(i_c, a_base_of(0), 0u); });
-                unroll_for<0, TN>([&](auto j_c) { unroll_for<0, 6>([&](auto x_c) { load_w(I0{}, j_c, x_c, w0); }); });
+                unroll_for<0, TN>([&](auto j_c) { unroll_for<0, NW>([&](auto x_c) { load_w(I0{}, j_c, x_c, w0); }); });
                 if constexpr (RMS)
                     load_gamma(g_base_of(0), 0u);
                 unroll_for<0, TM>([&](auto i_c) { load_a(i_c, a_base_of(1), (uint32_t)STAGE_BYTES); });

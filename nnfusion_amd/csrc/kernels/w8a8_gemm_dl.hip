@@ -33,11 +33,16 @@ namespace nnf
 
     namespace q8dl
     {
-        constexpr int BK = 64; // bytes (= int8 elements) of K per step
-
-        template <int WM, int WN, int TM, int TN, int STAGES_>
+        // BK: bytes (= int8 elements) of K per step, 64 or 128.  With 128 a wavefront-wide load fetches whole 128-byte
+        // lines (8 rows); with 64 it fetches half of each of 16 lines, and the memory pipeline takes about as long over a
+        // line it fetches half of as over a whole one.
+        template <int WM, int WN, int TM, int TN, int STAGES_, int BK_ = 64>
         struct Tile
         {
+            static constexpr int BK = BK_;
+            static_assert(BK == 64 || BK == 128, "a K step is half a line or a line of every row");
+            static constexpr int NSUB = BK / 32;          // sub-steps (one MFMA deep) per K step
+            static constexpr int ROWS_PER_LOAD = 1024 / BK; // rows a wavefront-wide load covers
             static constexpr int WAVES = WM * WN;
             static_assert(WAVES == 8 || WAVES == 4, "eight wavefronts per workgroup, or four with one SIMD each");
             static constexpr int THREADS = WAVES * 64;
@@ -48,10 +53,10 @@ namespace nnf
             static constexpr int W_TILE_BYTES = BN * BK;
             static constexpr int STAGE_BYTES = A_TILE_BYTES + W_TILE_BYTES;
             static constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
-            // a wavefront-wide load covers 16 rows of 64 bytes; every wavefront issues the same number of loads
+            // a wavefront-wide load covers 16 rows of 64 bytes or 8 of 128; every wavefront issues the same number of loads
             // (with fewer chunks than wavefronts two wavefronts fetch the same chunk into the same place)
-            static constexpr int A_CHUNKS = BM / 16;
-            static constexpr int W_CHUNKS = BN / 16;
+            static constexpr int A_CHUNKS = BM / ROWS_PER_LOAD;
+            static constexpr int W_CHUNKS = BN / ROWS_PER_LOAD;
             static constexpr int A_LOADS = A_CHUNKS >= WAVES ? A_CHUNKS / WAVES : 1;
             static constexpr int W_LOADS = W_CHUNKS >= WAVES ? W_CHUNKS / WAVES : 1;
             static constexpr int TILE_LOADS = A_LOADS + W_LOADS;
@@ -60,12 +65,15 @@ namespace nnf
         constexpr int vmcnt_imm(int n) { return (n & 0xF) | ((n >> 4) << 14) | (0x7 << 4) | (0xF << 8); }
     } // namespace q8dl
 
-    template <int WM, int WN, int TM, int TN, int STAGES, bool RAW, bool SPLITK, int MINW>
+    template <int WM, int WN, int TM, int TN, int STAGES, bool RAW, bool SPLITK, int MINW, int BK = 64>
     __global__ __launch_bounds__(WM * WN * 64, MINW) void w8a8_gemm_dl_kernel(Q8GemmParams p)
     {
         using namespace q8dl;
-        using T = Tile<WM, WN, TM, TN, STAGES>;
-        constexpr int BM = T::BM, BN = T::BN;
+        using T = Tile<WM, WN, TM, TN, STAGES, BK>;
+        constexpr int BM = T::BM, BN = T::BN, NSUB = T::NSUB, RPL = T::ROWS_PER_LOAD;
+        constexpr int PIECES = BK / 16; // 16-byte pieces of a row of a stage
+        // the piece a row's data sits at is XORed with bits of the row so that the 128-bit fragment reads are conflict free
+        auto swizzle = [](int row) { return BK == 64 ? (row >> 2) & 3 : (row >> 1) & 7; };
         constexpr int A_LOADS = T::A_LOADS, W_LOADS = T::W_LOADS, TILE_LOADS = T::TILE_LOADS;
         constexpr int A_TILE_BYTES = T::A_TILE_BYTES, STAGE_BYTES = T::STAGE_BYTES;
         extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -106,19 +114,19 @@ namespace nnf
         // this workgroup's K range, in units of 128 (all of K without SPLITK)
         const int g_begin = SPLITK ? (int)(((long long)split * G) / p.splits) : 0;
         const int g_end = SPLITK ? (int)(((long long)(split + 1) * G) / p.splits) : G;
-        const int KT = 2 * (g_end - g_begin);
+        const int KT = (128 / BK) * (g_end - g_begin);
         const int k_begin = g_begin * 128;
 
-        // ---- direct-load maps: chunk c fills LDS rows c*16 .. +15 (64 B each); lane l lands at
-        // (row = c*16 + l/4, slot = l%4) and therefore fetches piece  slot ^ ((row >> 2) & 3)  of that row
+        // ---- direct-load maps: chunk c fills LDS rows c*16 .. +15 (64 B each; 128 B: c*8 .. +7); lane l lands at
+        // (row = c*16 + l/4, slot = l%4) and therefore fetches piece  slot ^ swizzle(row)  of that row
         const int8_t* a_src[A_LOADS];
         int a_chunk[A_LOADS];
 #pragma unroll
         for (int i = 0; i < A_LOADS; ++i)
         {
             a_chunk[i] = (wave * A_LOADS + i) % T::A_CHUNKS;
-            int row = a_chunk[i] * 16 + (lane >> 2);
-            int piece = (lane & 3) ^ ((row >> 2) & 3);
+            int row = a_chunk[i] * RPL + lane / PIECES;
+            int piece = (lane % PIECES) ^ swizzle(row);
             a_src[i] = p.A + (size_t)min(m0 + row, p.M - 1) * K + k_begin + piece * 16;
         }
         const int8_t* w_src[W_LOADS];
@@ -127,8 +135,8 @@ namespace nnf
         for (int i = 0; i < W_LOADS; ++i)
         {
             w_chunk[i] = (wave * W_LOADS + i) % T::W_CHUNKS;
-            int row = w_chunk[i] * 16 + (lane >> 2);
-            int piece = (lane & 3) ^ ((row >> 2) & 3);
+            int row = w_chunk[i] * RPL + lane / PIECES;
+            int piece = (lane % PIECES) ^ swizzle(row);
             w_src[i] = p.W + (size_t)min(n0 + row, p.N - 1) * K + k_begin + piece * 16;
         }
         auto issue_tile_loads = [&](int kt, int stage) {
@@ -152,15 +160,15 @@ namespace nnf
         for (int i = 0; i < TM; ++i)
         {
             int r = wm * (TM * 32) + i * 32 + l32;
-            a_frag[i] = r * 64;
-            a_swz[i] = (r >> 2) & 3;
+            a_frag[i] = r * BK;
+            a_swz[i] = swizzle(r);
         }
 #pragma unroll
         for (int j = 0; j < TN; ++j)
         {
             int r = wn * (TN * 32) + j * 32 + l32;
-            w_frag[j] = A_TILE_BYTES + r * 64;
-            w_swz[j] = (r >> 2) & 3;
+            w_frag[j] = A_TILE_BYTES + r * BK;
+            w_swz[j] = swizzle(r);
         }
 
         intx16 acc[TM][TN];
@@ -172,36 +180,36 @@ namespace nnf
                 for (int e = 0; e < 16; ++e)
                     acc[i][j][e] = 0;
 
-        // A K step is two sub-steps of 32 bytes; the fragments of a sub-step (TM + TN 128-bit reads) are
+        // A K step is NSUB sub-steps of 32 bytes; the fragments of a sub-step (TM + TN 128-bit reads) are
         // fetched from LDS while the MFMAs of the sub-step before it run, into the other of two register sets.
         // Row r of a fragment and row r + 32 share their swizzle: the reads of a set are one address per
         // operand plus constant offsets.
         intx4 af[2][TM], bf[2][TN];
-        uint32_t a_addr[2], w_addr[2];
+        uint32_t a_addr[NSUB], w_addr[NSUB];
 #pragma unroll
-        for (int s = 0; s < 2; ++s)
+        for (int s = 0; s < NSUB; ++s)
         {
-            const uint32_t piece = (uint32_t)(((2 * s + h) ^ ((l32 >> 2) & 3)) << 4);
-            a_addr[s] = lds_address(smem) + (uint32_t)((wm * (TM * 32) + l32) * 64) + piece;
-            w_addr[s] = lds_address(smem) + (uint32_t)((wn * (TN * 32) + l32) * 64) + piece;
+            const uint32_t piece = (uint32_t)(((2 * s + h) ^ swizzle(l32)) << 4);
+            a_addr[s] = lds_address(smem) + (uint32_t)((wm * (TM * 32) + l32) * BK) + piece;
+            w_addr[s] = lds_address(smem) + (uint32_t)((wn * (TN * 32) + l32) * BK) + piece;
         }
         constexpr int FRAG_READS = TM + TN;
         auto read_frags = [&](int stage, auto s_c, auto set_c) {
             constexpr int s = decltype(s_c)::value, set = decltype(set_c)::value;
             const uint32_t off = (uint32_t)(stage * STAGE_BYTES);
             const uint32_t aa = a_addr[s] + off, ww = w_addr[s] + off;
-            unroll_for<0, TM>([&](auto i) { lds_read_b128_nowait<decltype(i)::value * 2048>(af[set][i], aa); });
+            unroll_for<0, TM>([&](auto i) { lds_read_b128_nowait<decltype(i)::value * 32 * BK>(af[set][i], aa); });
             unroll_for<0, TN>(
-                [&](auto j) { lds_read_b128_nowait<A_TILE_BYTES + decltype(j)::value * 2048>(bf[set][j], ww); });
+                [&](auto j) { lds_read_b128_nowait<A_TILE_BYTES + decltype(j)::value * 32 * BK>(bf[set][j], ww); });
         };
         // read x of a set: the TM activation fragments, then the TN weight fragments
         auto read_one_frag = [&](int stage, auto s_c, auto set_c, auto x_c) {
             constexpr int s = decltype(s_c)::value, set = decltype(set_c)::value, x = decltype(x_c)::value;
             const uint32_t off = (uint32_t)(stage * STAGE_BYTES);
             if constexpr (x < TM)
-                lds_read_b128_nowait<x * 2048>(af[set][x], a_addr[s] + off);
+                lds_read_b128_nowait<x * 32 * BK>(af[set][x], a_addr[s] + off);
             else
-                lds_read_b128_nowait<A_TILE_BYTES + (x - TM) * 2048>(bf[set][x - TM], w_addr[s] + off);
+                lds_read_b128_nowait<A_TILE_BYTES + (x - TM) * 32 * BK>(bf[set][x - TM], w_addr[s] + off);
         };
         // load x of a K step: the A_LOADS activation loads, then the W_LOADS weight loads
         auto issue_one_load = [&](int kt, int stage, auto x_c) {
@@ -281,59 +289,64 @@ namespace nnf
             {
                 // The fragments of sub-step 0 were read during the step before: the first MFMA goes out right behind the
                 // barrier, and everything else this step issues goes out one piece at a time between two MFMAs (it
-                // executes while the matrix core works): the LDS reads of sub-step 1 behind the first MFMAs of sub-step
-                // 0, this step's loads behind its later ones, the reads of the next step's sub-step 0 behind the first
-                // MFMAs of sub-step 1.
+                // executes while the matrix core works): the LDS reads of the next sub-step behind the first MFMAs of a
+                // sub-step (behind those of the last one: the next step's sub-step 0), this step's loads behind the later
+                // MFMAs of every sub-step but the last.
                 constexpr int HALF = NM / 2;
-                constexpr int RPM = (FRAG_READS + HALF - 1) / HALF, LPM = (TILE_LOADS + HALF - 1) / HALF;
+                constexpr int LOAD_SLOTS = (NSUB - 1) * HALF; // MFMAs with loads behind them
+                constexpr int RPM = (FRAG_READS + HALF - 1) / HALF, LPM = (TILE_LOADS + LOAD_SLOTS - 1) / LOAD_SLOTS;
                 int st = stage + STAGES - 1;
                 st = st >= STAGES ? st - STAGES : st;
                 const int kt_load = min(kt + STAGES - 1, KT - 1);
                 const int next_stage = stage + 1 == STAGES ? 0 : stage + 1;
-                wait_frags(I0{}, NONE{});
-                unroll_for<0, NM>([&](auto x_c) {
-                    constexpr int x = decltype(x_c)::value;
+                unroll_for<0, NSUB>([&](auto u_c) {
+                    constexpr int U = decltype(u_c)::value;
+                    using SET = std::integral_constant<int, U & 1>;
+                    using OTHER = std::integral_constant<int, (U & 1) ^ 1>;
+                    using NEXT_SUB = std::integral_constant<int, U + 1 < NSUB ? U + 1 : 0>;
+                    wait_frags(SET{}, NONE{});
+                    unroll_for<0, NM>([&](auto x_c) {
+                        constexpr int x = decltype(x_c)::value;
+                        __builtin_amdgcn_sched_barrier(0);
+                        mfma_range(SET{}, x_c, std::integral_constant<int, x + 1>{});
+                        __builtin_amdgcn_sched_barrier(0);
+                        if constexpr (x < HALF) // (after the last step: a stage nobody uses any more)
+                            unroll_for<x * RPM, (x + 1) * RPM < FRAG_READS ? (x + 1) * RPM : FRAG_READS>(
+                                [&](auto r_c) { read_one_frag(U + 1 < NSUB ? stage : next_stage, NEXT_SUB{}, OTHER{}, r_c); });
+                        else if constexpr (U + 1 < NSUB)
+                        {
+                            constexpr int SLOT = U * HALF + (x - HALF);
+                            unroll_for<(SLOT * LPM < TILE_LOADS ? SLOT * LPM : TILE_LOADS), ((SLOT + 1) * LPM < TILE_LOADS ? (SLOT + 1) * LPM : TILE_LOADS)>(
+                                [&](auto l_c) { issue_one_load(kt_load, st, l_c); });
+                        }
+                    });
                     __builtin_amdgcn_sched_barrier(0);
-                    mfma_range(I0{}, x_c, std::integral_constant<int, x + 1>{});
-                    __builtin_amdgcn_sched_barrier(0);
-                    if constexpr (x < HALF)
-                        unroll_for<x * RPM, (x + 1) * RPM < FRAG_READS ? (x + 1) * RPM : FRAG_READS>(
-                            [&](auto r_c) { read_one_frag(stage, I1{}, I1{}, r_c); });
-                    else
-                        unroll_for<(x - HALF) * LPM, (x - HALF + 1) * LPM < TILE_LOADS ? (x - HALF + 1) * LPM : TILE_LOADS>(
-                            [&](auto l_c) { issue_one_load(kt_load, st, l_c); });
                 });
-                __builtin_amdgcn_sched_barrier(0);
-                wait_frags(I1{}, NONE{});
-                unroll_for<0, NM>([&](auto x_c) {
-                    constexpr int x = decltype(x_c)::value;
-                    __builtin_amdgcn_sched_barrier(0);
-                    mfma_range(I1{}, x_c, std::integral_constant<int, x + 1>{});
-                    __builtin_amdgcn_sched_barrier(0);
-                    if constexpr (x < HALF) // (after the last step: a stage nobody uses any more)
-                        unroll_for<x * RPM, (x + 1) * RPM < FRAG_READS ? (x + 1) * RPM : FRAG_READS>(
-                            [&](auto r_c) { read_one_frag(next_stage, I0{}, I0{}, r_c); });
-                });
-                __builtin_amdgcn_sched_barrier(0);
                 stage = next_stage;
             }
             else
             {
-                // three stages: the fragments of a step are read behind its barrier (past the end: a valid tile is
+                // two or three stages: the fragments of a step are read behind its barrier (past the end: a valid tile is
                 // reloaded into the free stage)
                 int st = stage + STAGES - 1;
                 st = st >= STAGES ? st - STAGES : st;
                 issue_tile_loads(min(kt + STAGES - 1, KT - 1), st);
                 read_frags(stage, I0{}, I0{});
                 read_frags(stage, I1{}, I1{});
-                wait_frags(I0{}, ONE_SET{});
-                __builtin_amdgcn_sched_barrier(0);
-                mfmas(I0{});
-                __builtin_amdgcn_sched_barrier(0);
-                wait_frags(I1{}, NONE{});
-                __builtin_amdgcn_sched_barrier(0);
-                mfmas(I1{});
-                __builtin_amdgcn_sched_barrier(0);
+                unroll_for<0, NSUB>([&](auto u_c) {
+                    constexpr int U = decltype(u_c)::value;
+                    using SET = std::integral_constant<int, U & 1>;
+                    // behind this sub-step's fragments: those of the next one
+                    if constexpr (U + 1 < NSUB)
+                        wait_frags(SET{}, ONE_SET{});
+                    else
+                        wait_frags(SET{}, NONE{});
+                    __builtin_amdgcn_sched_barrier(0);
+                    mfmas(SET{});
+                    __builtin_amdgcn_sched_barrier(0);
+                    if constexpr (U + 2 < NSUB)
+                        read_frags(stage, std::integral_constant<int, U + 2>{}, SET{});
+                });
                 stage = stage + 1 == STAGES ? 0 : stage + 1;
             }
         }
@@ -487,13 +500,13 @@ namespace nnf
 
     namespace
     {
-        template <int WM, int WN, int TM, int TN, int STAGES, bool RAW, bool SPLITK, int MINW>
+        template <int WM, int WN, int TM, int TN, int STAGES, bool RAW, bool SPLITK, int MINW, int BK = 64>
         hipError_t launch_tile(hipStream_t stream, const Q8GemmParams& p)
         {
-            using T = q8dl::Tile<WM, WN, TM, TN, STAGES>;
+            using T = q8dl::Tile<WM, WN, TM, TN, STAGES, BK>;
             const int tiles_m = (p.M + T::BM - 1) / T::BM;
             const int tiles_n = (p.N + T::BN - 1) / T::BN;
-            auto kernel = &w8a8_gemm_dl_kernel<WM, WN, TM, TN, STAGES, RAW, SPLITK, MINW>;
+            auto kernel = &w8a8_gemm_dl_kernel<WM, WN, TM, TN, STAGES, RAW, SPLITK, MINW, BK>;
             if (T::LDS_BYTES > 64 * 1024)
             {
                 static LdsGrant granted;
@@ -510,25 +523,39 @@ namespace nnf
         hipError_t launch_plan(hipStream_t stream, const Q8GemmParams& p, const workspace::GemmPlan& plan)
         {
             hipError_t e;
+            // K steps of 128 bytes (whole lines per load) wherever LDS holds three of them.  Measured against steps of
+            // 64 with the same tiles, weights no cache holds: 64 x 256 tiles 5 - 18 % faster (M = 40 .. 64), 128 x 128
+            // 10 - 17 % (M = 160 .. 512; one workgroup per CU with four stages against two with three), 256 x 128
+            // 4 - 13 % (M = 640 .. 2048).  Not for the 256 x 256 tile, where only two such stages fit (M = 4096: 1.5 %
+            // slower), nor for 128 x 128 tiles whose workgroups get less than 2560 of K (M = 128, N = K = 8192, four
+            // ranges of 2048: 25.1 -> 27.4 us; two resident workgroups with short loops cover for each other).
+            const bool long_k = p.K / (p.splits > 0 ? p.splits : 1) >= 2560;
             switch (plan.tile)
             {
-            case workspace::GEMM_TILE_BIG: // 256 x 256, four stages, one workgroup per CU
+            case workspace::GEMM_TILE_BIG: // 256 x 256, four stages of 64, one workgroup per CU
                 if (!plan.reduce_pass)
                     return launch_tile<2, 4, 4, 2, 4, RAW, false, 2>(stream, p);
                 e = launch_tile<2, 4, 4, 2, 4, RAW, true, 2>(stream, p);
                 break;
-            case workspace::GEMM_TILE_TALL: // 256 x 128, four stages, one workgroup per CU
+            case workspace::GEMM_TILE_TALL: // 256 x 128, three stages of 128, one workgroup per CU
                 if (!plan.reduce_pass)
-                    return launch_tile<2, 4, 4, 1, 4, RAW, false, 2>(stream, p);
-                e = launch_tile<2, 4, 4, 1, 4, RAW, true, 2>(stream, p);
+                    return launch_tile<2, 4, 4, 1, 3, RAW, false, 2, 128>(stream, p);
+                e = launch_tile<2, 4, 4, 1, 3, RAW, true, 2, 128>(stream, p);
                 break;
-            case workspace::GEMM_TILE_MID: // 128 x 128
+            case workspace::GEMM_TILE_MID: // 128 x 128: four stages of 128, one workgroup per CU; or three of 64, two per CU
+                if (long_k)
+                {
+                    if (!plan.reduce_pass)
+                        return launch_tile<2, 4, 2, 1, 4, RAW, false, 2, 128>(stream, p);
+                    e = launch_tile<2, 4, 2, 1, 4, RAW, true, 2, 128>(stream, p);
+                    break;
+                }
                 if (!plan.reduce_pass)
                     return launch_tile<2, 4, 2, 1, 3, RAW, false, 4>(stream, p);
                 e = launch_tile<2, 4, 2, 1, 3, RAW, true, 4>(stream, p);
                 break;
-            default: // 64 x 256, always through the partial sums
-                e = launch_tile<1, 8, 2, 1, 3, RAW, true, 4>(stream, p);
+            default: // 64 x 256, always through the partial sums: three stages of 128, one workgroup per CU
+                e = launch_tile<1, 8, 2, 1, 3, RAW, true, 2, 128>(stream, p);
                 break;
             }
             if (e != hipSuccess)
