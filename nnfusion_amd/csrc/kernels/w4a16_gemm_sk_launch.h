@@ -100,9 +100,10 @@ namespace nnf
                        : tile_rows == 128 ? launch_instance_q<4, 1, QG>(stream, p, grid)
                        : tile_rows == 64  ? launch_instance_q<2, 1, QG>(stream, p, grid)
                                           : hipErrorInvalidValue;
-            return tile_rows == 256 ? launch_instance_q<8, 2, QG>(stream, p, grid)
-                   : tile_rows == 32 ? launch_instance_q<1, 2, QG>(stream, p, grid)
-                                     : hipErrorInvalidValue;
+            return tile_rows == 256   ? launch_instance_q<8, 2, QG>(stream, p, grid)
+                   : tile_rows == 128 ? launch_instance_q<4, 2, QG>(stream, p, grid)
+                   : tile_rows == 32  ? launch_instance_q<1, 2, QG>(stream, p, grid)
+                                      : hipErrorInvalidValue;
         }
     } // namespace gemm_sk
 

@@ -134,13 +134,16 @@ namespace nnf
             size_t sync_bytes(bool rms = false) const { return (slots || rms) ? ((size_t)tiles_m * tiles_n + 1) * 2 * sizeof(unsigned) : 0; }
         };
         // Tile shape.  What the caller fixes (forced_rows 32 / 64 / 128 / 256, forced_cols 128 / 256) is kept, the rest
-        // is chosen by M (measured at N = K = 8192 and on the Llama shapes, alternating the candidates in one process):
-        // 256-row tiles touch every weight once per 256 rows and are the fastest from about 1500 rows on; below, with
-        // every output tile shared by several workgroups, tiles of 128 columns halve what each of them parks and are
-        // 6-14 % faster (M = 64: 26.5 -> 22.8 us, 128: 35.7 -> 30.8, 512: 83 -> 76, 1024: 134 -> 123) although an
-        // activation fragment then feeds one MFMA instead of two; 256 rows where M fills them to within an eighth,
-        // else 128.  SiLU-gate needs the gate | up halves of a 256-row weight tile; 32-row tiles exist 256 wide only.
-        inline void sk_tile_shape(int M, bool gate, int forced_rows, int forced_cols, int& rows, int& cols)
+        // is chosen by M and N (measured at N = K = 8192 and on the Llama shapes, the candidates in turns in one process):
+        // 256 x 256 tiles touch every weight once per 256 rows and are the fastest from about 1500 rows on.  Below, every
+        // output tile is shared by several workgroups and what a workgroup parks counts: up to 128 rows 128 x 128 tiles
+        // (64 x 128 up to 64); above, 256 x 128 where M fills the 256-row tiles (an even number of 128-row blocks, or
+        // less than a seventh of the rows wasted: M = 144 .. 256 40.8 - 42.2 us against 42.8 - 44.3 on 128 x 128 tiles,
+        // M = 896 116 against 144) and 128 x 256 where it does not (an odd number of blocks: M = 288 .. 384 61.3 - 62.7
+        // against 63.9 - 66.1, M = 576 .. 640 96 against 104); 128 x 128 again where 256-row tiles would leave fewer
+        // than 64 tiles (N = 4096 at M = 192 .. 256).  SiLU-gate needs the gate | up halves of a 256-row weight tile;
+        // 32-row tiles exist 256 wide only.
+        inline void sk_tile_shape(int M, int N, bool gate, int forced_rows, int forced_cols, int& rows, int& cols)
         {
             const bool rows_forced = forced_rows == 32 || forced_rows == 64 || forced_rows == 128 || forced_rows == 256;
             if (rows_forced)
@@ -151,13 +154,28 @@ namespace nnf
             }
             cols = 256;
             if (gate || M <= 32 || M > 1536)
+            {
                 rows = M <= 32 ? 32 : M <= 64 ? 64 : M <= 1536 ? 128 : 256;
-            else
+                return;
+            }
+            if (forced_cols == 256)
             {
                 const int padded = ceil_div(M, 256) * 256;
                 rows = M <= 64 ? 64 : M <= 128 ? 128 : ((padded - M) * 8 <= M ? 256 : 128);
-                cols = forced_cols == 256 ? 256 : 128;
+                return;
             }
+            cols = 128;
+            rows = M <= 64 ? 64 : 128;
+            if (M <= 128)
+                return;
+            const int blocks = ceil_div(M, 128), padded = ceil_div(M, 256) * 256;
+            if ((blocks & 1) == 0 || (padded - M) * 7 <= padded)
+            {
+                if ((padded / 256) * ceil_div(N, 128) >= 64)
+                    rows = 256;
+            }
+            else if (forced_cols != 128)
+                cols = 256;
         }
         // tiles_n column tiles, `per_tile` units of K per tile, at least `min_units` units per workgroup (unless forced);
         // forced_grid: 0 = the plan's own choice
@@ -200,7 +218,7 @@ namespace nnf
             if (M <= 0 || N <= 0 || K < 128 || num_cu < 1)
                 return SkPlan();
             int rows, cols;
-            sk_tile_shape(M, gate, forced_tile_rows, forced_cols, rows, cols);
+            sk_tile_shape(M, N, gate, forced_tile_rows, forced_cols, rows, cols);
             SkPlan p = plan_sk(M, ceil_div(N, (gate || cols == 128) ? 128 : 256), (K / 128 + 1) / 2, 2, num_cu, rows, forced_grid);
             p.tile_weight_rows = cols;
             return p;

@@ -353,20 +353,21 @@ int main(int argc, char** argv)
         EXPECT(deps.find("cuda") == std::string::npos && deps.find("cublas") == std::string::npos);
 
         // fused variant: gamma, bias; the scratch tensor appears in signature and call.  Its size: one fp32 per row
-        // (rstd) + the parked sums of the plan for this shape (32 tiles of 128 x 256 x 16 supersteps over 256 workgroups: one slot each)
+        // (rstd) + the parked sums of the plan for this shape (64 tiles of 128 x 128 -- 256-row tiles would leave 32 -- x 16 supersteps
+        // over 256 workgroups: one slot each)
         graph::Graph g2;
         auto n2 = quant_dot_graph(g2, 256, 4096, 4096, "{\"rms_norm\": true, \"has_bias\": true, \"rms_eps\": 1e-5}", true, true);
         auto k2 = sel.pick_first(n2, ROCM_GPU).second;
         auto fu2 = k2->get_or_emit_source();
         CONTAINS(fu2->body_unit->get_code(), "nnf_w4a16_gemm_fused_variant(stream, input0, input1, input2, output0, 256, 4096, 4096, 128, 8, input3, 1.000000000e-05f, input4, nullptr, NNF_ACT_NONE, NNF_W4A16_AUTO, &plan, ");
         // ... and, because the product runs on the tile GEMM, a second tensor: its synchronisation words (two for rstd[],
-        // two per tile: 2 x 16 tiles; in whole 64 bytes), persistent and cleared at initialisation, named by the nnf_plan
+        // two per tile: 2 x 32 tiles; in whole 64 bytes), persistent and cleared at initialisation, named by the nnf_plan
         // the body declares
         EXPECT(k2->m_context->tensors.size() == 2 &&
-               k2->m_context->tensors[0]->size() == (size_t)256 * 4 + (size_t)256 * 128 * 256 * 4);
-        EXPECT(k2->m_context->tensors[1]->size() == 320 && k2->m_context->tensors[1]->is_persistent() &&
+               k2->m_context->tensors[0]->size() == (size_t)256 * 4 + (size_t)256 * 128 * 128 * 4);
+        EXPECT(k2->m_context->tensors[1]->size() == 576 && k2->m_context->tensors[1]->is_persistent() &&
                k2->m_context->tensors[1]->is_memset() && k2->m_context->tensors[1]->get_memset_value() == 0);
-        CONTAINS(fu2->body_unit->get_code(), "const nnf_plan plan = {0, 0, 0, " + k2->m_context->tensors[1]->get_name() + ", 320, 0};");
+        CONTAINS(fu2->body_unit->get_code(), "const nnf_plan plan = {0, 0, 0, " + k2->m_context->tensors[1]->get_name() + ", 576, 0};");
         CONTAINS(fu2->signature_unit->get_code(), "char* " + k2->m_context->tensors[0]->get_name());
         CONTAINS(fu2->call_unit->get_code(), k2->m_context->tensors[1]->get_name() + ");");
         // SiLU gate: N is half the weight rows
@@ -461,13 +462,12 @@ int main(int argc, char** argv)
         auto fm = k->get_or_emit_source();
         CONTAINS(fm->body_unit->get_code(), "nnf_fused_mlp_w4a16_planned(stream, input0, input1, 1.000000000e-06f, input2, input3, input4, input5, output0, 256, 4096, 11008, 128, 8, &gate_up_plan, &down_plan, ");
         // rstd [256] fp32 + h [256, 11008] fp16 + the larger of the two areas of parked sums: both GEMMs run 256
-        // workgroups over tiles of 128 x 256 weight rows; gate/up (2 x 86 tiles x 16 supersteps) needs two slots per
-        // workgroup
-        // ... and the synchronisation words of either product (2 x 86 and 1 x 32 tiles, two words each, and two more)
+        // workgroups; gate/up (2 x 86 tiles of 128 x 256 weight rows x 16 supersteps) needs two slots per workgroup
+        // ... and the synchronisation words of either product (2 x 86 and 2 x 32 tiles, two words each, and two more)
         EXPECT(k->m_context->tensors.size() == 3 &&
                k->m_context->tensors[0]->size() ==
                    (size_t)256 * 4 + (size_t)256 * 11008 * 2 + (size_t)2 * 256 * 128 * 256 * 4);
-        EXPECT(k->m_context->tensors[1]->size() == 1408 && k->m_context->tensors[2]->size() == 320 &&
+        EXPECT(k->m_context->tensors[1]->size() == 1408 && k->m_context->tensors[2]->size() == 576 &&
                k->m_context->tensors[1]->is_memset() && k->m_context->tensors[2]->is_memset());
     });
 
