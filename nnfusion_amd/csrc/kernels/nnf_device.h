@@ -127,6 +127,36 @@ namespace nnf
     {
         asm volatile("" : "+v"(v));
     }
+    // Activation rows into MFMA operand registers by way of LDS.  A lane of a 16-row MFMA operand wants 16-byte pieces
+    // that lie 64 bytes apart in its row, so a load straight into the registers touches two lines of every row for
+    // 32 bytes each, four times over; the memory pipeline's time goes by the lines a load touches.  Instead a block of
+    // 16 rows x 256 bytes is fetched as whole lines (four wavefront-wide loads of 4 rows x 256 bytes, global -> LDS) and
+    // read from LDS in operand order.  Layout of a block: row r at 256 r, its 16 pieces XORed with r (conflict-free
+    // 128-bit reads: the 16 lanes of a row quad hit 16 different pieces).
+    constexpr int ROW_BLOCK_BYTES = 4096;
+    // issue the four loads: row `first_row + r` (clamped to last_row) of a row-major matrix (row_bytes per row), bytes
+    // [byte0, byte0 + 256)
+    __device__ __forceinline__ void row_block_fetch(const uint8_t* base, size_t row_bytes, int first_row, int last_row, size_t byte0,
+                                                    uint8_t* block, int lane)
+    {
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+        {
+            const int r = c * 4 + (lane >> 4);
+            const int piece = (lane & 15) ^ r;
+            const uint8_t* src = base + (size_t)min(first_row + r, last_row) * row_bytes + byte0 + piece * 16;
+            __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1)))*)src,
+                                             (void __attribute__((address_space(3)))*)(block + c * 1024), 16, 0, 0);
+        }
+    }
+    // piece p (0 .. 15) of row `row` of a landed block
+    __device__ __forceinline__ uintx4 row_block_piece(const uint8_t* block, int row, int p)
+    {
+        return *reinterpret_cast<const uintx4*>(block + row * 256 + ((p ^ row) << 4));
+    }
+    // vmcnt-only wait (gfx9 encoding)
+    __device__ __forceinline__ constexpr int vmcnt_only(int n) { return (n & 0xF) | ((n >> 4) << 14) | (0x7 << 4) | (0xF << 8); }
+
     __device__ __forceinline__ uint32_t lds_address(const void* p)
     {
         return (uint32_t)(uintptr_t)(const void __attribute__((address_space(3)))*)p;

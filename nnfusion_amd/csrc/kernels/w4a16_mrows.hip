@@ -318,19 +318,35 @@ namespace nnf
         // loads are not held back by anything)
         issue(0, 0, 0);
         issue(min(1 / STEPS, T - 1), 1 % STEPS, 1);
+        // (through LDS as whole lines, see row_block_fetch: two blocks per wavefront, over what holds the partial tiles
+        // and the parked sums later -- hence the barrier behind the last block)
         uintx4 areg[MB][GA][4];
-#pragma unroll
-        for (int mb = 0; mb < MB; ++mb)
         {
-            const uint8_t* a_bytes = reinterpret_cast<const uint8_t*>(A);
-            const uint32_t a_off =
-                (uint32_t)min(mb * 16 + col, M - 1) * (uint32_t)(K * 2) + (uint32_t)wave * (GW * 256) + (uint32_t)kq * 64u;
+            uint8_t* stage = red + wave * (2 * ROW_BLOCK_BYTES);
+            constexpr int NP = MB * GA;
+            auto fetch = [&](int p) {
+                const int mb = p / GA, g = p % GA;
+                row_block_fetch(reinterpret_cast<const uint8_t*>(A), (size_t)K * 2, mb * 16, M - 1,
+                                (size_t)((g / GW) * (SPAN * 4) + wave * (GW * 256) + (g % GW) * 256), stage + (p & 1) * ROW_BLOCK_BYTES, lane);
+            };
+            fetch(0);
 #pragma unroll
-            for (int g = 0; g < GA; ++g)
+            for (int p = 0; p < NP; ++p)
+            {
+                if (p + 1 < NP)
+                {
+                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); // block p-1 has been read out of the half that is filled next
+                    fetch(p + 1);
+                    __builtin_amdgcn_s_waitcnt(vmcnt_only(4));
+                }
+                else
+                    __builtin_amdgcn_s_waitcnt(vmcnt_only(0));
 #pragma unroll
                 for (int j = 0; j < 4; ++j)
-                    areg[mb][g][j] = *reinterpret_cast<const uintx4*>(
-                        a_bytes + (size_t)(a_off + (g / GW) * (SPAN * 4) + (g % GW) * 256 + j * 16));
+                    areg[p / GA][p % GA][j] = row_block_piece(stage + (p & 1) * ROW_BLOCK_BYTES, col, kq * 4 + j);
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            __syncthreads();
         }
         // RMSNorm without a pass of its own: the wavefront's share of sum a^2 of every row, from the registers
         const bool own_rstd = FUSED && f.gamma && !f.rstd;
@@ -926,27 +942,39 @@ namespace nnf
         const int rd_swz = swz(col);
         const uint32_t red_addr = lds_address(red) + (uint32_t)(wave * (MB * 1024) + lane * 16);
         const uint32_t parked_addr = lds_address(parked);
-        const uint8_t* a_row[MB];
-#pragma unroll
-        for (int mb = 0; mb < MB; ++mb)
-            a_row[mb] = reinterpret_cast<const uint8_t*>(A) + (size_t)min(mb * 16 + col, M - 1) * (size_t)(K * 2) + kq * 64;
         int slot = 0;
         {
-            // ---- the activations: straight into the MFMA operand registers ------------------------------------------
+            // ---- the activations: into the MFMA operand registers, through LDS as whole lines (see row_block_fetch: two
+            // blocks per wavefront, over what holds the partial tiles and the parked sums later -- hence the barrier)
             uintx4 areg[MB][GA][4];
             floatx4 ncorr[MB][GA];
+            {
+                uint8_t* stage = red + wave * (2 * ROW_BLOCK_BYTES);
+                constexpr int NP = MB * GA;
+                auto fetch = [&](int p) {
+                    const int mb = p / GA, ga = p % GA;
+                    row_block_fetch(reinterpret_cast<const uint8_t*>(A), (size_t)K * 2, mb * 16, M - 1,
+                                    (size_t)(fetch_group(ga / GW) + ga % GW) * 256, stage + (p & 1) * ROW_BLOCK_BYTES, lane);
+                };
+                fetch(0);
 #pragma unroll
-            for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-                for (int st = 0; st < STEPS; ++st)
+                for (int p = 0; p < NP; ++p)
                 {
-                    const uint8_t* a_src = a_row[mb] + (size_t)fetch_group(st) * 256;
+                    if (p + 1 < NP)
+                    {
+                        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); // block p-1 has been read out of the half that is filled next
+                        fetch(p + 1);
+                        __builtin_amdgcn_s_waitcnt(vmcnt_only(4));
+                    }
+                    else
+                        __builtin_amdgcn_s_waitcnt(vmcnt_only(0));
 #pragma unroll
-                    for (int g = 0; g < GW; ++g)
-#pragma unroll
-                        for (int j = 0; j < 4; ++j)
-                            areg[mb][st * GW + g][j] = *reinterpret_cast<const uintx4*>(a_src + g * 256 + j * 16);
+                    for (int j = 0; j < 4; ++j)
+                        areg[p / GA][p % GA][j] = row_block_piece(stage + (p & 1) * ROW_BLOCK_BYTES, col, kq * 4 + j);
                 }
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                __syncthreads();
+            }
             if (FUSED && f.gamma)
                 mrows_scale_a<MB, GA>(areg, [&](int g) {
                     return reinterpret_cast<const uint8_t*>(f.gamma) + kq * 64 + (size_t)fetch_group(g / GW) * 256 + (g % GW) * 256;

@@ -516,8 +516,11 @@ namespace nnf
         inline size_t w4a16_mrows_lds_bytes_gw(int gw, int M, int tiles)
         {
             const size_t mb = M <= 16 ? 1 : M <= 32 ? 2 : 4; // blocks of 16 rows
-            // ring, scales, partial tiles, the wavefronts' sums of squares per row (RMSNorm inside the kernel), parked sums
-            return (size_t)8 * 2 * gw * 1024 + 8 * 512 + (size_t)2 * 8 * mb * 1024 + 8 * mb * 64 + (size_t)tiles * M * 64;
+            // ring, scales; partial tiles, the wavefronts' sums of squares per row (RMSNorm inside the kernel), parked sums --
+            // or, while the kernel starts, two blocks of 16 rows x 256 bytes of activations per wavefront
+            const size_t tail = (size_t)2 * 8 * mb * 1024 + 8 * mb * 64 + (size_t)tiles * M * 64;
+            const size_t staging = (size_t)8 * 2 * 4096;
+            return (size_t)8 * 2 * gw * 1024 + 8 * 512 + (tail > staging ? tail : staging);
         }
         inline size_t w4a16_mrows_lds_bytes(int K, int M, int tiles)
         {

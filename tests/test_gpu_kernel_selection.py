@@ -37,7 +37,8 @@ def test_profiling_selector_times_every_candidate_and_keeps_the_fastest(gpu, nam
     assert all(c["ms"] > 0 for c in res["candidates"]), res
     assert res["ran"] == len(expected)
     times = {c["kernel"]: c["ms"] for c in res["candidates"]}
-    assert res["best"] == min(times, key=times.get)
+    # (two candidates may run the same kernel and tie at the printed precision)
+    assert times[res["best"]] == min(times.values())
     # same inputs, same product: fp16 results within a few ulps of each other (different summation orders)
     assert res["max_abs_diff"] <= 2e-2 * max(res["max_abs_ref"], 1e-3), res
     if m == 1:
