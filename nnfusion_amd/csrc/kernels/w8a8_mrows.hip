@@ -107,20 +107,54 @@ namespace nnf
 #pragma unroll
         for (int s = 0; s < NS; ++s)
             issue(t0 + min(s / STEPS, T - 1), s % STEPS, s);
+        // Two blocks of rows: through LDS as whole lines (see row_block_fetch: a block is a step's 256 bytes of 16 rows; two
+        // blocks per wavefront, over what holds the partial tiles and the parked sums later -- hence the barrier behind
+        // the last): N = 4096, K = 8192 at 32 rows 14.5 -> 12.3 us.  One block of rows: straight into the registers, 64
+        // bytes of each row per load (half the lines of a load of 16-bit activations: the detour costs more than it saves,
+        // N = K = 8192 at 8 rows 16.7 -> 18.7 us).
         uintx4 areg[MB][CH];
+        if constexpr (MB == 1)
         {
+            const uint8_t* a_row = reinterpret_cast<const uint8_t*>(A) + (size_t)min(col, M - 1) * (size_t)ld + k0 + kq * 16;
 #pragma unroll
-            for (int mb = 0; mb < MB; ++mb)
+            for (int c = 0; c < CH; ++c)
             {
-                const uint8_t* a_row = reinterpret_cast<const uint8_t*>(A) + (size_t)min(mb * 16 + col, M - 1) * (size_t)ld + k0 + kq * 16;
+                const uintx4 v = *reinterpret_cast<const uintx4*>(a_row + fetch_byte(c >> 2) + (c & 3) * 64);
+                const bool inside = own_byte(c >> 2) < K; // otherwise another wavefront covers these bytes
+                areg[0][c] = inside ? v : uintx4{0u, 0u, 0u, 0u};
+            }
+        }
+        else
+        {
+            uint8_t* stage = red + wave * (2 * ROW_BLOCK_BYTES);
+            constexpr int NP = MB * STEPS;
+            auto fetch = [&](int p) {
+                const int mb = p / STEPS, st = p % STEPS;
+                row_block_fetch(reinterpret_cast<const uint8_t*>(A), (size_t)ld, mb * 16, M - 1, (size_t)(k0 + fetch_byte(st)),
+                                stage + (p & 1) * ROW_BLOCK_BYTES, lane);
+            };
+            fetch(0);
 #pragma unroll
-                for (int c = 0; c < CH; ++c)
+            for (int p = 0; p < NP; ++p)
+            {
+                if (p + 1 < NP)
                 {
-                    const uintx4 v = *reinterpret_cast<const uintx4*>(a_row + fetch_byte(c >> 2) + (c & 3) * 64);
-                    const bool inside = own_byte(c >> 2) < K; // otherwise another wavefront covers these bytes
-                    areg[mb][c] = inside ? v : uintx4{0u, 0u, 0u, 0u};
+                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); // block p-1 has been read out of the half that is filled next
+                    fetch(p + 1);
+                    __builtin_amdgcn_s_waitcnt(vmcnt_only(4));
+                }
+                else
+                    __builtin_amdgcn_s_waitcnt(vmcnt_only(0));
+                const bool inside = own_byte(p % STEPS) < K; // otherwise another wavefront covers these bytes
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                {
+                    const uintx4 v = row_block_piece(stage + (p & 1) * ROW_BLOCK_BYTES, col, j * 4 + kq);
+                    areg[p / STEPS][(p % STEPS) * 4 + j] = inside ? v : uintx4{0u, 0u, 0u, 0u};
                 }
             }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            __syncthreads();
         }
 
         // ---- tile loop ---------------------------------------------------------------------------------------

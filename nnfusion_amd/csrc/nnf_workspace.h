@@ -453,7 +453,11 @@ namespace nnf
         constexpr int W8A8_MROWS_SLOTS = 2;
         inline size_t w8a8_mrows_lds_bytes(int M, int slots, int tiles)
         {
-            return (size_t)8 * slots * 4096 + (size_t)2 * 8 * (M <= 16 ? 1 : 2) * 1024 + (size_t)tiles * M * 64;
+            // ring; partial tiles and parked sums -- or, while the kernel starts, two blocks of 16 rows x 256 bytes of
+            // activations per wavefront
+            const size_t tail = (size_t)2 * 8 * (M <= 16 ? 1 : 2) * 1024 + (size_t)tiles * M * 64;
+            const size_t staging = M > 16 ? (size_t)8 * 2 * 4096 : 0;
+            return (size_t)8 * slots * 4096 + (tail > staging ? tail : staging);
         }
         inline bool w8a8_mrows_fits(int M, int N, int K, int num_cu)
         {
@@ -485,6 +489,10 @@ namespace nnf
         {
             const int per_range = num_cu / 2;
             if (M < 8 || K < 8192 || (K & 511) || per_range < 1 || (N + 15) / 16 > 4 * per_range)
+                return 1;
+            // (17 .. 32 rows, whose activations arrive as whole lines: only where a workgroup has more than one tile
+            // anyway -- N = 4096 at 32 rows: 12.3 us in one pass, 13.0 over two ranges; N = 8192: 20.9 / 19.6)
+            if (M > 16 && (N + 15) / 16 <= num_cu)
                 return 1;
             return w8a8_mrows_fits(M, N, K / 2, per_range) ? 2 : 1;
         }
@@ -683,10 +691,11 @@ namespace nnf
             // (33 .. 64 rows run on the kernel, but against the tile GEMM, measured alternately: 33 / 40 rows take 25.9 / 27.4 us
             // against 29.1 / 29.3 at N = 22016, K = 4096 and 12.2 / 12.9 against 14.8 / 15.3 at N = K = 4096, are level at K = 8192 and
             // 11008, 8-10 % slower at K = 5120, and slower everywhere from about 48 rows on: taken up to 40 rows and K = 4096)
-            // (8 .. 16 rows at K = 8192, up to 16384 weight rows: in one launch every workgroup fetches all M x 8192 activations
-            // ahead of its first MFMA; over two ranges it fetches half of them: 10-18 % faster at 12 .. 16 rows, 0-10 % at 8,
-            // with the reduction pass or without it; slower at K = 5120 / 6144, level from about 28000 weight rows on)
-            const int longest_single = M <= 16 ? ((M >= 8 && K == 8192 && N <= 16384) ? 8191 : 8192) : M <= 32 ? 4096 : 2048;
+            // (8 .. 16 rows at K = 8192, up to 8192 weight rows: in one launch every workgroup fetches all M x 8192 activations
+            // ahead of its first MFMA; over two ranges it fetches half of them.  With the activations fetched as whole lines
+            // that is worth 5 % at 8 rows and nothing at 12 .. 16 (it was 10-18 % before); at 16384 weight rows one range is
+            // 6 % faster, and it was slower at K = 5120 / 6144)
+            const int longest_single = M <= 16 ? ((M >= 8 && K == 8192 && N <= 8192) ? 8191 : 8192) : M <= 32 ? 4096 : 2048;
             if (M < 2 || M > 40 || N < 16 || K <= longest_single || K > (M <= 32 ? 65536 : 4096) || (K & 255) || num_cu < 16)
                 return sp;
             const int G = K >> 7;

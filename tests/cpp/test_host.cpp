@@ -1217,9 +1217,9 @@ int main(int argc, char** argv)
             // one launch, no scratch memory, where a row-streaming kernel serves the shape; ranges of K and shared tiles park sums
             EXPECT(ws::w4a16_gemm(1, 4096, 4096, 128) == 0 && ws::w4a16_gemm(16, 12288, 4096, 128) == 0 &&
                    ws::w4a16_gemm(7, 8192, 8192, 128) == 0);
-            // 8 .. 16 rows at K = 8192 (up to 16384 weight rows): two ranges of K (half the activations per workgroup)
+            // 8 .. 16 rows at K = 8192 (up to 8192 weight rows): two ranges of K (half the activations per workgroup)
             EXPECT(ws::w4a16_gemm(16, 8192, 8192, 128) == (size_t)2 * 16 * 8192 * 4 && ws::w4a16_gemm(8, 4096, 8192, 128) == (size_t)2 * 8 * 4096 * 4 &&
-                   ws::w4a16_gemm(16, 28672, 8192, 128) == 0);
+                   ws::w4a16_gemm(16, 16384, 8192, 128) == 0 && ws::w4a16_gemm(16, 28672, 8192, 128) == 0);
             EXPECT(ws::route_w4a16(16, 8192, 8192, false, true, false, 256).kind == ws::W4A16Route::MROWS &&
                    ws::route_w4a16(16, 4096, 8192, true, false, false, 256).kind == ws::W4A16Route::MROWS);
             EXPECT(ws::mrows_split_adds_in_launch(8192, 2, 256) && ws::mrows_split_adds_in_launch(4096, 3, 256) &&
