@@ -232,7 +232,8 @@ namespace nnf
     // pack = M | zp << 8;  a workgroup's output tiles: tiles_q, one more for the first tiles_r workgroups.
     // FUSED: the prologue / epilogue of `f`; gate != 0: N outputs from 2 N weight rows, the workgroup walks the gate and
     // the up tile of each of its output tiles in turn (twice the tiles).
-    template <int GW, int STEPS, int MB, bool FUSED>
+    // STAGE: the activations through LDS as whole lines (row_block_fetch); otherwise straight into the registers
+    template <int GW, int STEPS, int MB, bool FUSED, bool STAGE>
     __global__ __launch_bounds__(512) void w4a16_mrows_kernel(const half_t* __restrict__ A, const uint8_t* __restrict__ Wq,
                                                               const half_t* __restrict__ S, half_t* __restrict__ Y, int N,
                                                               int tiles_q, int tiles_r, int pack, GemvFusionArgs f, int gate)
@@ -320,7 +321,20 @@ namespace nnf
         issue(min(1 / STEPS, T - 1), 1 % STEPS, 1);
         // (through LDS as whole lines, see row_block_fetch: two blocks per wavefront, over what holds the partial tiles
         // and the parked sums later -- hence the barrier behind the last block)
+        // (a few rows: a load touches few lines as it is -- the lanes of the rows that do not exist ask for the last row
+        // again -- and the detour costs 0.3 - 0.5 us: straight into the registers)
         uintx4 areg[MB][GA][4];
+        if constexpr (!STAGE)
+        {
+            const uint8_t* a_bytes = reinterpret_cast<const uint8_t*>(A);
+            const uint32_t a_off = (uint32_t)min(col, M - 1) * (uint32_t)(K * 2) + (uint32_t)wave * (GW * 256) + (uint32_t)kq * 64u;
+#pragma unroll
+            for (int g = 0; g < GA; ++g)
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    areg[0][g][j] = *reinterpret_cast<const uintx4*>(a_bytes + (size_t)(a_off + (g / GW) * (SPAN * 4) + (g % GW) * 256 + j * 16));
+        }
+        else
         {
             uint8_t* stage = red + wave * (2 * ROW_BLOCK_BYTES);
             constexpr int NP = MB * GA;
@@ -857,7 +871,7 @@ namespace nnf
     // pack = M | zp << 8.
     // FUSED: as in w4a16_mrows_kernel; over ranges of K only the RMSNorm weight applies here (the sums of a range go to
     // `partial` as they are: rstd and the rest of the epilogue belong to the reduction pass).
-    template <int GW, int STEPS, int MB, bool FUSED>
+    template <int GW, int STEPS, int MB, bool FUSED, bool STAGE>
     __global__ __launch_bounds__(512) void w4a16_mrows_any_kernel(const half_t* __restrict__ A, const uint8_t* __restrict__ Wq,
                                                                   const half_t* __restrict__ S, half_t* __restrict__ Y,
                                                                   float* __restrict__ partial, int N, int K, int range_groups,
@@ -946,8 +960,19 @@ namespace nnf
         {
             // ---- the activations: into the MFMA operand registers, through LDS as whole lines (see row_block_fetch: two
             // blocks per wavefront, over what holds the partial tiles and the parked sums later -- hence the barrier)
+            // (a few rows: straight into the registers, as in the kernel above)
             uintx4 areg[MB][GA][4];
             floatx4 ncorr[MB][GA];
+            if constexpr (!STAGE)
+            {
+                const uint8_t* a_row = reinterpret_cast<const uint8_t*>(A) + (size_t)min(col, M - 1) * (size_t)(K * 2) + kq * 64;
+#pragma unroll
+                for (int ga = 0; ga < GA; ++ga)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        areg[0][ga][j] = *reinterpret_cast<const uintx4*>(a_row + (size_t)(fetch_group(ga / GW) + ga % GW) * 256 + j * 16);
+            }
+            else
             {
                 uint8_t* stage = red + wave * (2 * ROW_BLOCK_BYTES);
                 constexpr int NP = MB * GA;
@@ -1100,7 +1125,7 @@ namespace nnf
         }
 
         // N: output columns (fusion.gate: from 2 N weight rows)
-        template <int GW, int STEPS, int MB, bool FUSED>
+        template <int GW, int STEPS, int MB, bool FUSED, bool STAGE = true>
         hipError_t launch_mrows_mb(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M, int N, int zp,
                                    int num_cu, const GemvFusion& fusion)
         {
@@ -1111,7 +1136,7 @@ namespace nnf
                 workspace::w4a16_mrows_lds_bytes(GW * STEPS * 1024, M, (fusion.gate ? 2 : 1) * (tiles_q + (tiles_r ? 1 : 0)));
             if (lds > MAX_LDS_BYTES)
                 return hipErrorInvalidValue;
-            auto kernel = &w4a16_mrows_kernel<GW, STEPS, MB, FUSED>;
+            auto kernel = &w4a16_mrows_kernel<GW, STEPS, MB, FUSED, STAGE>;
             if (lds > 64 * 1024)
             {
                 static LdsGrant granted;
@@ -1130,6 +1155,9 @@ namespace nnf
                                 int num_cu, const GemvFusion& fusion)
         {
             const bool fused = fusion.any();
+            if (M <= 16 && !workspace::mrows_stages_activations(M, GW * STEPS * 1024))
+                return fused ? launch_mrows_mb<GW, STEPS, 1, true, false>(stream, A, Wq, S, Y, M, N, zp, num_cu, fusion)
+                             : launch_mrows_mb<GW, STEPS, 1, false, false>(stream, A, Wq, S, Y, M, N, zp, num_cu, fusion);
             if (M <= 16)
                 return fused ? launch_mrows_mb<GW, STEPS, 1, true>(stream, A, Wq, S, Y, M, N, zp, num_cu, fusion)
                              : launch_mrows_mb<GW, STEPS, 1, false>(stream, A, Wq, S, Y, M, N, zp, num_cu, fusion);
@@ -1143,7 +1171,7 @@ namespace nnf
     namespace
     {
         // ranges == 1: the whole of K, fp16 results to Y; otherwise ranges of range_groups groups, fp32 sums to partial
-        template <int GW, int STEPS, int MB, bool FUSED>
+        template <int GW, int STEPS, int MB, bool FUSED, bool STAGE = true>
         hipError_t launch_mrows_any_mb(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M, int N, int K,
                                        int zp, int num_cu, float* partial, int ranges, int range_groups, const GemvFusion& fusion,
                                        uint32_t* sync)
@@ -1156,7 +1184,7 @@ namespace nnf
             // over ranges of K the epilogue belongs to whoever adds the ranges up: the reduction pass, or (sync) the launch itself
             if (lds > MAX_LDS_BYTES || (ranges > 1 && (fusion.gate || (!sync && (fusion.bias || fusion.residual || fusion.rstd)))))
                 return hipErrorInvalidValue;
-            auto kernel = &w4a16_mrows_any_kernel<GW, STEPS, MB, FUSED>;
+            auto kernel = &w4a16_mrows_any_kernel<GW, STEPS, MB, FUSED, STAGE>;
             if (lds > 64 * 1024)
             {
                 static LdsGrant granted;
@@ -1175,6 +1203,9 @@ namespace nnf
                                       int zp, int num_cu, float* partial, int ranges, int range_groups, const GemvFusion& fusion,
                                       uint32_t* sync)
         {
+            if (M <= 16 && !workspace::mrows_stages_activations(M, K))
+                return launch_mrows_any_mb<GW, STEPS, 1, FUSED, false>(stream, A, Wq, S, Y, M, N, K, zp, num_cu, partial, ranges,
+                                                                       range_groups, fusion, sync);
             if (M <= 16)
                 return launch_mrows_any_mb<GW, STEPS, 1, FUSED>(stream, A, Wq, S, Y, M, N, K, zp, num_cu, partial, ranges, range_groups,
                                                                 fusion, sync);

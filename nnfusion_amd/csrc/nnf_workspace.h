@@ -521,6 +521,12 @@ namespace nnf
                 return (kw & 1) ? kw : kw / 2; // even K / 1024: two steps per tile
             return G <= 32 ? 2 : G <= 48 ? 3 : 4;
         }
+        // Whether the kernel brings its activations in through LDS as whole lines or straight into the registers.  Straight
+        // in, a load touches two lines of every row for 32 bytes each, four times over; through LDS every line is touched
+        // once, but the blocks come one behind the other (0.3 - 0.5 us).  Measured, K = 4096: 2 / 4 / 6 rows 4.84 / 5.07 /
+        // 5.20 us straight against 5.19 / 5.27 / 5.29, 8 / 12 / 16 rows 5.63 / 6.52 / 7.3 against 5.30 / 5.40 / 5.55;
+        // K = 8192: 4 / 6 rows 12.05 / 12.45 against 11.58 / 11.70; 32 rows at N = K = 4096: 10.8 against 7.1.
+        inline bool mrows_stages_activations(int M, int K) { return (long long)M * K >= 32768; }
         inline size_t w4a16_mrows_lds_bytes_gw(int gw, int M, int tiles)
         {
             const size_t mb = M <= 16 ? 1 : M <= 32 ? 2 : 4; // blocks of 16 rows
