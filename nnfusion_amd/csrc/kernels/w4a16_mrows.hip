@@ -548,20 +548,46 @@ namespace nnf
 
         issue(0, 0, 0);
         issue(0, 1, 1);
-        // activations: straight into the MFMA operand registers, in the pair order of the nibble trick
+        // activations: into the MFMA operand registers (through LDS as whole lines from a few rows on, see
+        // workspace::mrows_stages_activations), then in the pair order of the nibble trick
         uintx4 areg[MB][GA][4];
-#pragma unroll
-        for (int mb = 0; mb < MB; ++mb)
+        if (MB == 1 && !workspace::mrows_stages_activations(M, K))
         {
             const uint8_t* a_bytes = reinterpret_cast<const uint8_t*>(A);
-            const uint32_t a_off =
-                (uint32_t)min(mb * 16 + col, M - 1) * (uint32_t)(K * 2) + (uint32_t)wave * (GW * 256) + (uint32_t)kq * 64u;
+            const uint32_t a_off = (uint32_t)min(col, M - 1) * (uint32_t)(K * 2) + (uint32_t)wave * (GW * 256) + (uint32_t)kq * 64u;
 #pragma unroll
             for (int g = 0; g < GA; ++g)
 #pragma unroll
                 for (int j = 0; j < 4; ++j)
-                    areg[mb][g][j] = *reinterpret_cast<const uintx4*>(
-                        a_bytes + (size_t)(a_off + (g / GW) * (SPAN * 4) + (g % GW) * 256 + j * 16));
+                    areg[0][g][j] = *reinterpret_cast<const uintx4*>(a_bytes + (size_t)(a_off + (g / GW) * (SPAN * 4) + (g % GW) * 256 + j * 16));
+        }
+        else
+        {
+            uint8_t* stage = red + wave * (2 * ROW_BLOCK_BYTES);
+            constexpr int NP = MB * GA;
+            auto fetch = [&](int p) {
+                const int mb = p / GA, g = p % GA;
+                row_block_fetch(reinterpret_cast<const uint8_t*>(A), (size_t)K * 2, mb * 16, M - 1,
+                                (size_t)((g / GW) * (SPAN * 4) + wave * (GW * 256) + (g % GW) * 256), stage + (p & 1) * ROW_BLOCK_BYTES, lane);
+            };
+            fetch(0);
+#pragma unroll
+            for (int p = 0; p < NP; ++p)
+            {
+                if (p + 1 < NP)
+                {
+                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); // block p-1 has been read out of the half that is filled next
+                    fetch(p + 1);
+                    __builtin_amdgcn_s_waitcnt(vmcnt_only(4));
+                }
+                else
+                    __builtin_amdgcn_s_waitcnt(vmcnt_only(0));
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    areg[p / GA][p % GA][j] = row_block_piece(stage + (p & 1) * ROW_BLOCK_BYTES, col, kq * 4 + j);
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            __syncthreads();
         }
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb)
@@ -761,19 +787,49 @@ namespace nnf
         const int rd_swz = swz(col);
         const uint32_t red_addr = lds_address(red) + (uint32_t)(wave * (MB * 1024) + lane * 16);
         const uint32_t parked_addr = lds_address(parked);
-        // activations: straight into the MFMA operand registers, in the pair order of the nibble trick
+        // activations: into the MFMA operand registers (through LDS as whole lines from a few rows on, see
+        // workspace::mrows_stages_activations), then in the pair order of the nibble trick
         uintx4 areg[GA][4];
         {
-            const uint8_t* a_row = reinterpret_cast<const uint8_t*>(A) + (size_t)min(col, M - 1) * (size_t)(K * 2) + kq * 64;
-#pragma unroll
-            for (int st = 0; st < STEPS; ++st)
+            if (!workspace::mrows_stages_activations(M, K))
             {
-                const uint8_t* a_src = a_row + (size_t)fetch_block(st) * 256;
+                const uint8_t* a_row = reinterpret_cast<const uint8_t*>(A) + (size_t)min(col, M - 1) * (size_t)(K * 2) + kq * 64;
 #pragma unroll
-                for (int g = 0; g < GW; ++g)
+                for (int st = 0; st < STEPS; ++st)
+                {
+                    const uint8_t* a_src = a_row + (size_t)fetch_block(st) * 256;
+#pragma unroll
+                    for (int g = 0; g < GW; ++g)
+#pragma unroll
+                        for (int j = 0; j < 4; ++j)
+                            areg[st * GW + g][j] = *reinterpret_cast<const uintx4*>(a_src + g * 256 + j * 16);
+                }
+            }
+            else
+            {
+                uint8_t* stage = red + wave * (2 * ROW_BLOCK_BYTES);
+                auto fetch = [&](int p) {
+                    row_block_fetch(reinterpret_cast<const uint8_t*>(A), (size_t)K * 2, 0, M - 1, (size_t)(fetch_block(p / GW) + p % GW) * 256,
+                                    stage + (p & 1) * ROW_BLOCK_BYTES, lane);
+                };
+                fetch(0);
+#pragma unroll
+                for (int p = 0; p < GA; ++p)
+                {
+                    if (p + 1 < GA)
+                    {
+                        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); // block p-1 has been read out of the half that is filled next
+                        fetch(p + 1);
+                        __builtin_amdgcn_s_waitcnt(vmcnt_only(4));
+                    }
+                    else
+                        __builtin_amdgcn_s_waitcnt(vmcnt_only(0));
 #pragma unroll
                     for (int j = 0; j < 4; ++j)
-                        areg[st * GW + g][j] = *reinterpret_cast<const uintx4*>(a_src + g * 256 + j * 16);
+                        areg[p][j] = row_block_piece(stage + (p & 1) * ROW_BLOCK_BYTES, col, kq * 4 + j);
+                }
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                __syncthreads();
             }
 #pragma unroll
             for (int g = 0; g < GA; ++g)

@@ -526,7 +526,9 @@ namespace nnf
         // once, but the blocks come one behind the other (0.3 - 0.5 us).  Measured, K = 4096: 2 / 4 / 6 rows 4.84 / 5.07 /
         // 5.20 us straight against 5.19 / 5.27 / 5.29, 8 / 12 / 16 rows 5.63 / 6.52 / 7.3 against 5.30 / 5.40 / 5.55;
         // K = 8192: 4 / 6 rows 12.05 / 12.45 against 11.58 / 11.70; 32 rows at N = K = 4096: 10.8 against 7.1.
-        inline bool mrows_stages_activations(int M, int K) { return (long long)M * K >= 32768; }
+        constexpr bool mrows_stages_activations(int M, int K) { return (long long)M * K >= 32768; }
+        // the room for that: two blocks of 16 rows x 256 bytes per wavefront, where the partial tiles and parked sums go later
+        constexpr size_t mrows_tail_bytes(size_t tail) { return tail > (size_t)8 * 2 * 4096 ? tail : (size_t)8 * 2 * 4096; }
         inline size_t w4a16_mrows_lds_bytes_gw(int gw, int M, int tiles)
         {
             const size_t mb = M <= 16 ? 1 : M <= 32 ? 2 : 4; // blocks of 16 rows
@@ -561,7 +563,7 @@ namespace nnf
             const int loads = (16 * words + 63) / 64;
             const size_t aux = (size_t)(zero_points ? 2 : 1) * loads * 256;
             const size_t mb = M <= 16 ? 1 : 2; // blocks of 16 rows
-            return (size_t)8 * 2 * gw * 1024 + 8 * 2 * aux + (size_t)2 * 8 * mb * 1024 + (size_t)tiles * M * 64;
+            return (size_t)8 * 2 * gw * 1024 + 8 * 2 * aux + mrows_tail_bytes((size_t)2 * 8 * mb * 1024 + (size_t)tiles * M * 64);
         }
         // (17 .. 32 rows: two blocks of rows in registers, up to K = 4096)
         inline bool w4a16_mrows_q_fits(int M, int N, int K, int group_shift, bool zero_points, int num_cu)
@@ -589,7 +591,7 @@ namespace nnf
             const int words = spc == 1 ? gw / 2 + 1 : gw * spc / 2;
             const int loads = (16 * words + 63) / 64;
             const size_t aux = (size_t)(zero_points ? 2 : 1) * loads * 256;
-            return (size_t)8 * 2 * gw * 1024 + 8 * 2 * aux + (size_t)2 * 8 * 1024 + (size_t)tiles * M * 64;
+            return (size_t)8 * 2 * gw * 1024 + 8 * 2 * aux + mrows_tail_bytes((size_t)2 * 8 * 1024 + (size_t)tiles * M * 64);
         }
         inline MrowsQAny w4a16_mrows_q_any_plan(int M, int N, int K, int group_shift, bool zero_points, int num_cu)
         {

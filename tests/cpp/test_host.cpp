@@ -1171,14 +1171,15 @@ int main(int argc, char** argv)
             // 17 .. 32 rows: two blocks of rows in registers, up to K = 4096 (no workspace: not the tile GEMM)
             EXPECT(ws::w4a16_mrows_q_fits(17, 4096, 4096, 5, false, 256) && ws::w4a16_mrows_q_fits(32, 12288, 2048, 6, true, 256));
             EXPECT(!ws::w4a16_mrows_q_fits(17, 8192, 8192, 5, false, 256));
-            EXPECT(ws::w4a16_mrows_q_lds_bytes(4096, 32, 1, 6, false) == 32768 + 4096 + 32768 + 2048);
+            EXPECT(ws::w4a16_mrows_q_lds_bytes(4096, 32, 1, 6, false) == 32768 + 4096 + 65536);
             EXPECT(ws::wna16_gemm(32, 4096, 4096, 4, 64) == 0 && ws::wna16_gemm(32, 8192, 8192, 4, 64) > 0 &&
                    ws::wna16_gemm(33, 4096, 4096, 4, 64) > 0);
             EXPECT(!ws::w4a16_mrows_q_fits(8, 4096, 6144, 5, false, 256) && !ws::w4a16_mrows_q_fits(8, 4096, 11008, 5, false, 256));
             EXPECT(!ws::w4a16_mrows_q_fits(8, 4096, 4096, 4, false, 256) && !ws::w4a16_mrows_q_fits(8, 8, 4096, 5, false, 256));
-            // ring 8 x 2 x 4 KiB, scales and zero points 8 x 2 x (2 + 2) x 256, partial tiles 16 KiB, two parked tiles
-            EXPECT(ws::w4a16_mrows_q_lds_bytes(8192, 16, 2, 5, true) == 65536 + 16384 + 16384 + 2 * 16 * 64);
-            EXPECT(ws::w4a16_mrows_q_lds_bytes(4096, 16, 1, 6, false) == 32768 + 4096 + 16384 + 1024);
+            // ring 8 x 2 x 4 KiB, scales and zero points 8 x 2 x (2 + 2) x 256, then the larger of partial tiles 16 KiB + parked tiles
+            // and the 64 KiB through which the activations arrive
+            EXPECT(ws::w4a16_mrows_q_lds_bytes(8192, 16, 2, 5, true) == 65536 + 16384 + 65536);
+            EXPECT(ws::w4a16_mrows_q_lds_bytes(4096, 16, 1, 6, false) == 32768 + 4096 + 65536);
             EXPECT(!ws::w4a16_mrows_q_fits(16, 1000000, 8192, 5, true, 256)); // the parked sums do not fit
         }
         // ... with a run-time K: one piece up to 8192 where most of what is fetched counts, ranges of at most 32 blocks above
@@ -1196,8 +1197,8 @@ int main(int argc, char** argv)
             p = ws::w4a16_mrows_q_any_plan(4, 8192, 28672, 7, true, 256);
             EXPECT(p.ranges == 7 && p.range_blocks == 32 && p.gw == 2);
             // scales of a step: groups of 128: gw / 2 + 1 words a row; 32: gw * 2 words (two loads from gw = 3 on)
-            EXPECT(ws::w4a16_mrows_q_any_lds_bytes(2, 16, 1, 7, true) == 32768 + 8 * 2 * 512 + 16384 + 1024);
-            EXPECT(ws::w4a16_mrows_q_any_lds_bytes(4, 16, 1, 5, false) == 65536 + 8 * 2 * 512 + 16384 + 1024);
+            EXPECT(ws::w4a16_mrows_q_any_lds_bytes(2, 16, 1, 7, true) == 32768 + 8 * 2 * 512 + 65536);
+            EXPECT(ws::w4a16_mrows_q_any_lds_bytes(4, 16, 1, 5, false) == 65536 + 8 * 2 * 512 + 65536);
         }
         // M <= 16: one workgroup holds the activations, or K is cut into ranges
         {
