@@ -12,6 +12,7 @@ namespace nnf
     typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
     typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
     typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+    typedef float floatx2 __attribute__((ext_vector_type(2)));
     typedef float floatx4 __attribute__((ext_vector_type(4)));
     typedef float floatx16 __attribute__((ext_vector_type(16)));
     typedef int intx4 __attribute__((ext_vector_type(4)));

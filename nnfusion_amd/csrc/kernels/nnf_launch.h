@@ -76,11 +76,12 @@ namespace nnf
     hipError_t launch_w4a16_gemv_rows(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int N,
                                       int K, int zp, int num_cu, const GemvFusion& fusion = GemvFusion());
     bool w4a16_gemv_rows_supported(int M, int N, int K, int num_cu, bool gate = false);
-    // the same kernel for 4-bit weights with groups of 2^group_shift = 32 / 64 / 128 and a scalar zero point or
-    // (zero_points != null) one per (row, group): u8 [N, (K / group + 1) / 2], even group in the low nibble
+    // the same kernel for 4- or 8-bit weights with groups of 2^group_shift = 32 / 64 / 128 and a scalar zero point or
+    // (zero_points != null) one per (row, group): 4 bits: u8 [N, (K / group + 1) / 2], even group in the low nibble;
+    // 8 bits: u8 [N, K / group]
     hipError_t launch_w4a16_gemv_rows_q(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int N,
-                                        int K, int group_shift, int zp, const void* zero_points, int num_cu);
-    bool w4a16_gemv_rows_q_supported(int M, int N, int K, int group_shift, bool zero_points, int num_cu);
+                                        int K, int group_shift, int zp, const void* zero_points, int num_cu, int bits = 4);
+    bool w4a16_gemv_rows_q_supported(int M, int N, int K, int group_shift, bool zero_points, int num_cu, int bits = 4);
 
     // 2 <= M <= 16, K = 1024 / 2048 / 4096 / 8192: weights streamed through LDS rings, activations in registers
     // (N: outputs; gate / fusion.gate: from 2 N weight rows)

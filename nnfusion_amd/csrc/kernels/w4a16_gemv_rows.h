@@ -79,7 +79,10 @@ namespace nnf
     // wavefront then fetches the bytes that hold the zero points of its K segment (one byte per lane, global -> LDS like
     // the weights: 256 bytes more per ring slot and 64 groups, waited for with the weights), and the constant part of a
     // lane's sum becomes  base - z (sum of the lane's activations),  base the constant for z = 0; both stay in registers.
-    template <int SEG, int D, int WAVES, int EPI>
+    // BITS = 8 (with EPI 3 / 4 only): a row is K bytes, a lane's 16 bytes of a load are 16 weights (two units of
+    // activations, kept in memory order), a byte b becomes 1024 + b with one v_perm_b32 per pair (0x64 above it: the
+    // mantissa of 1024.0), and `zps` holds one byte per (row, group).
+    template <int SEG, int D, int WAVES, int EPI, int BITS = 4>
     __device__ __forceinline__ void gemv_rows_body(const half_t* __restrict__ A, const uint8_t* __restrict__ Wq,
                                                    const half_t* __restrict__ S, half_t* __restrict__ Y, int N, int K,
                                                    int rows_q, int rows_r, int pack, const GemvFusionArgs& f,
@@ -88,6 +91,11 @@ namespace nnf
         constexpr bool GATE = EPI == 2;
         constexpr bool QZT = EPI == 3;            // zero points from `zps`
         constexpr bool QG = EPI == 3 || EPI == 4; // group size from `pack`
+        constexpr bool W8 = BITS == 8;
+        static_assert(BITS == 4 || (W8 && QG), "8-bit weights: the kernels for other block parameters only");
+        constexpr int LOAD_K = W8 ? 1024 : 2048; // weights per wavefront-wide load
+        constexpr int LANE_K = LOAD_K / 64;      // ... and lane
+        constexpr int UPL = LANE_K / 8;          // units of activations a lane meets per load
         constexpr int ZL = QZT ? (SEG + 1) / 2 : 0; // loads of zero points per row and wavefront (64 bytes = 128 groups each;
                                                     // a segment of SEG KiB of weights has at most 64 SEG groups)
         constexpr int LPR = SEG + ZL;               // vector-memory loads per row and wavefront
@@ -112,7 +120,7 @@ namespace nnf
         const int out0 = (int)blockIdx.x * rows_q + min((int)blockIdx.x, rows_r);
         const int n_out = rows_q + ((int)blockIdx.x < rows_r ? 1 : 0); // >= 1: the grid never exceeds N
         const int n_rows = GATE ? 2 * n_out : n_out;                   // weight rows this workgroup walks
-        const uint32_t row_bytes = (uint32_t)K >> 1;
+        const uint32_t row_bytes = W8 ? (uint32_t)K : (uint32_t)K >> 1;
         const int G = K >> gshift;
         const int a_units = K >> 3;
         const int a_pad = (a_units + 63) & ~63; // whole wavefront-wide loads of activations
@@ -190,20 +198,20 @@ namespace nnf
         // zero points: the first byte of this wavefront's K segment in a row of `zps` (a segment starts at an even
         // group), the byte each lane fetches (past the end of the row: its last byte), and where a lane finds the zero
         // point of its load j afterwards: byte (one per lane and four bytes of LDS) and nibble
-        const int zp_stride = (G + 1) >> 1;
-        const int g_seg0 = (kpart * SEG * 2048) >> gshift;
+        const int zp_stride = W8 ? G : (G + 1) >> 1;
+        const int g_seg0 = (kpart * SEG * LOAD_K) >> gshift;
         uint32_t z_off[ZL > 0 ? ZL : 1], z_rd[SEG], z_sh[SEG];
         if constexpr (QZT)
         {
 #pragma unroll
             for (int i = 0; i < ZL; ++i)
-                z_off[i] = (uint32_t)min((g_seg0 >> 1) + i * 64 + lane, zp_stride - 1);
+                z_off[i] = (uint32_t)min((W8 ? g_seg0 : g_seg0 >> 1) + i * 64 + lane, zp_stride - 1);
 #pragma unroll
             for (int j = 0; j < SEG; ++j)
             {
-                const int g = min(g_seg0 + ((j * 2048 + lane * 32) >> gshift), G - 1);
-                z_rd[j] = (uint32_t)((g >> 1) - (g_seg0 >> 1)) * 4u;
-                z_sh[j] = (uint32_t)(g & 1) * 4u;
+                const int g = min(g_seg0 + ((j * LOAD_K + lane * LANE_K) >> gshift), G - 1);
+                z_rd[j] = W8 ? (uint32_t)(g - g_seg0) * 4u : (uint32_t)((g >> 1) - (g_seg0 >> 1)) * 4u;
+                z_sh[j] = W8 ? 0u : (uint32_t)(g & 1) * 4u;
             }
         }
         // weights of row r (relative to the workgroup's first; rows past the end re-read the last row) -> ring slot
@@ -243,7 +251,7 @@ namespace nnf
         uint32_t s_rd[SEG];
 #pragma unroll
         for (int j = 0; j < SEG; ++j)
-            s_rd[j] = QG ? (uint32_t)min((kpart * SEG * 2048 + j * 2048 + lane * 32) >> gshift, G - 1) * 2u
+            s_rd[j] = QG ? (uint32_t)min((kpart * SEG * LOAD_K + j * LOAD_K + lane * LANE_K) >> gshift, G - 1) * 2u
                          : (uint32_t)min(kpart * SEG * 16 + j * 16 + (lane >> 2), G - 1) * 2u;
 
         // ---- activations: prepared once per workgroup, then LDS -> registers ------------------------------
@@ -256,7 +264,7 @@ namespace nnf
         if (a_loader)
         {
             const float ce = -(1024.0f + (QZT ? 0.f : (float)zp));
-            const float co = -(64.0f + (QZT ? 0.f : (float)zp));
+            const float co = W8 ? ce : -(64.0f + (QZT ? 0.f : (float)zp));
             float ss = 0.f;
             int e = 0;
             for (int u0 = wave * 64; u0 < a_units; u0 += WAVES * 64, ++e)
@@ -286,7 +294,7 @@ namespace nnf
                     raw.z = as_u32(as_half2(raw.z) * as_half2(g.z));
                     raw.w = as_u32(as_half2(raw.w) * as_half2(g.w));
                 }
-                const uintx4 a = permute_a8(raw);
+                const uintx4 a = W8 ? raw : permute_a8(raw);
                 const half2_t x = as_half2(a.x), y = as_half2(a.y), z = as_half2(a.z), w = as_half2(a.w);
                 const float se = ((float)x.x + (float)x.y) + ((float)z.x + (float)z.y);
                 const float so = ((float)y.x + (float)y.y) + ((float)w.x + (float)w.y);
@@ -306,22 +314,35 @@ namespace nnf
         }
         lds_barrier();
         NNF_ROWS_STAMP(2); // every wavefront has prepared its share of the activations
-        uintx4 areg[SEG][4];
+        uintx4 areg[SEG][UPL];
         float ncorr[SEG], asum[SEG];
 #pragma unroll
         for (int j = 0; j < SEG; ++j)
         {
-            // 4 bytes of weights per unit; a lane past the end of K gets the zeros
-            const int u0 = valid[j] ? (int)((seg_byte0 + j * 1024 + lane * 16) >> 2) : a_pad;
-            const floatx4 c4 = *reinterpret_cast<const floatx4*>(corr + u0);
-            ncorr[j] = (c4.x + c4.y) + (c4.z + c4.w);
-            if constexpr (QZT)
+            // 4 (8) bytes of weights per unit; a lane past the end of K gets the zeros
+            const int u0 = valid[j] ? (int)((seg_byte0 + j * 1024 + lane * 16) >> (W8 ? 3 : 2)) : a_pad;
+            if constexpr (W8)
             {
-                const floatx4 s4 = *reinterpret_cast<const floatx4*>(asum_u + u0);
-                asum[j] = (s4.x + s4.y) + (s4.z + s4.w);
+                const floatx2 c2 = *reinterpret_cast<const floatx2*>(corr + u0);
+                ncorr[j] = c2.x + c2.y;
+                if constexpr (QZT)
+                {
+                    const floatx2 s2 = *reinterpret_cast<const floatx2*>(asum_u + u0);
+                    asum[j] = s2.x + s2.y;
+                }
+            }
+            else
+            {
+                const floatx4 c4 = *reinterpret_cast<const floatx4*>(corr + u0);
+                ncorr[j] = (c4.x + c4.y) + (c4.z + c4.w);
+                if constexpr (QZT)
+                {
+                    const floatx4 s4 = *reinterpret_cast<const floatx4*>(asum_u + u0);
+                    asum[j] = (s4.x + s4.y) + (s4.z + s4.w);
+                }
             }
 #pragma unroll
-            for (int d = 0; d < 4; ++d)
+            for (int d = 0; d < UPL; ++d)
                 areg[j][d] = act[u0 + d];
         }
 
@@ -337,7 +358,7 @@ namespace nnf
                 wv[j] = *reinterpret_cast<const uintx4*>(ring + slot * SLOT_BYTES + j * 1024 + lane16);
                 sv[j] = (float)*reinterpret_cast<const half_t*>(sc_row + s_rd[j]);
                 if constexpr (QZT)
-                    zv[j] = (float)(((uint32_t)ring[slot * SLOT_BYTES + SEG * 1024 + z_rd[j]] >> z_sh[j]) & 15u);
+                    zv[j] = (float)(((uint32_t)ring[slot * SLOT_BYTES + SEG * 1024 + z_rd[j]] >> z_sh[j]) & (W8 ? 255u : 15u));
             }
         };
         auto compute = [&](int r) {
@@ -349,6 +370,21 @@ namespace nnf
                 float t = ncorr[j];
                 if constexpr (QZT)
                     t = __builtin_fmaf(-zv[j], asum[j], t);
+                if constexpr (W8)
+                {
+                    // v_perm_b32(S0, S1, sel): selectors 0-3 pick bytes of S1, 4-7 of S0
+#pragma unroll
+                    for (int d = 0; d < UPL; ++d)
+                    {
+                        const uintx4 a = areg[j][d];
+                        const uint32_t w0 = ww[2 * d], w1 = ww[2 * d + 1];
+                        t = dot2(as_half2(__builtin_amdgcn_perm(0x64646464u, w0, 0x04010400u)), as_half2(a.x), t);
+                        t = dot2(as_half2(__builtin_amdgcn_perm(0x64646464u, w0, 0x04030402u)), as_half2(a.y), t);
+                        t = dot2(as_half2(__builtin_amdgcn_perm(0x64646464u, w1, 0x04010400u)), as_half2(a.z), t);
+                        t = dot2(as_half2(__builtin_amdgcn_perm(0x64646464u, w1, 0x04030402u)), as_half2(a.w), t);
+                    }
+                }
+                else
 #pragma unroll
                 for (int d = 0; d < 4; ++d)
                 {

@@ -55,9 +55,9 @@ namespace nnf
         gemv_rows_body<SEG, D, WAVES, EPI>(A, Wq, S, Y, N, K, rows_q, rows_r, pack, f);
     }
 
-    // Other block parameters (EPI 4: group size; 3: a zero point per (row, group) as well).  Sixteen dwords of arguments,
-    // like the plain kernel.
-    template <int SEG, int D, int WAVES, int EPI>
+    // Other block parameters (EPI 4: group size; 3: a zero point per (row, group) as well; BITS: 4 or 8).  Sixteen dwords
+    // of arguments, like the plain kernel.
+    template <int SEG, int D, int WAVES, int EPI, int BITS>
     __global__ __launch_bounds__(WAVES * 64) void w4a16_gemv_rows_q_kernel(const half_t* __restrict__ A,
                                                                            const uint8_t* __restrict__ Wq,
                                                                            const half_t* __restrict__ S,
@@ -66,14 +66,14 @@ namespace nnf
                                                                            const uint8_t* __restrict__ zps)
     {
         static_assert(EPI == 3 || EPI == 4, "the plain kernel is w4a16_gemv_rows_kernel");
-        gemv_rows_body<SEG, D, WAVES, EPI>(A, Wq, S, Y, N, K, rows_q, rows_r, pack, GemvFusionArgs{nullptr, nullptr, nullptr, nullptr, 0.f}, zps);
+        gemv_rows_body<SEG, D, WAVES, EPI, BITS>(A, Wq, S, Y, N, K, rows_q, rows_r, pack, GemvFusionArgs{nullptr, nullptr, nullptr, nullptr, 0.f}, zps);
     }
 
     namespace
     {
         using workspace::RowsPlan;
 
-        template <int SEG, int D, int WAVES, int EPI>
+        template <int SEG, int D, int WAVES, int EPI, int BITS>
         hipError_t launch_rows_q(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int N, int K,
                                  int zp, int group_shift, const void* zps, const RowsPlan& p, int grid)
         {
@@ -83,12 +83,12 @@ namespace nnf
             if (lds_total > 64 * 1024)
             {
                 static LdsGrant granted;
-                const hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(&w4a16_gemv_rows_q_kernel<SEG, D, WAVES, EPI>),
+                const hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(&w4a16_gemv_rows_q_kernel<SEG, D, WAVES, EPI, BITS>),
                                                        granted, (int)MAX_LDS_BYTES);
                 if (e != hipSuccess)
                     return e;
             }
-            hipLaunchKernelGGL((w4a16_gemv_rows_q_kernel<SEG, D, WAVES, EPI>), dim3(grid), dim3(WAVES * 64), lds_total, stream,
+            hipLaunchKernelGGL((w4a16_gemv_rows_q_kernel<SEG, D, WAVES, EPI, BITS>), dim3(grid), dim3(WAVES * 64), lds_total, stream,
                                (const half_t*)A, (const uint8_t*)Wq, (const half_t*)S, (half_t*)Y, N, K, N / grid, N % grid,
                                zp | (p.kshift << 8) | (group_shift << 16), (const uint8_t*)zps);
             return hipGetLastError();
@@ -162,24 +162,25 @@ namespace nnf
         }
     }
 
-    bool w4a16_gemv_rows_q_supported(int M, int N, int K, int group_shift, bool zero_points, int num_cu)
+    bool w4a16_gemv_rows_q_supported(int M, int N, int K, int group_shift, bool zero_points, int num_cu, int bits)
     {
-        return workspace::plan_w4a16_rows(M, N, K, num_cu, 0, false, group_shift, zero_points).seg != 0;
+        return workspace::plan_w4a16_rows(M, N, K, num_cu, 0, false, group_shift, zero_points, bits).seg != 0;
     }
 
     hipError_t launch_w4a16_gemv_rows_q(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int N,
-                                        int K, int group_shift, int zp, const void* zero_points, int num_cu)
+                                        int K, int group_shift, int zp, const void* zero_points, int num_cu, int bits)
     {
-        const RowsPlan p = workspace::plan_w4a16_rows(1, N, K, num_cu, 0, false, group_shift, zero_points != nullptr);
+        const RowsPlan p = workspace::plan_w4a16_rows(1, N, K, num_cu, 0, false, group_shift, zero_points != nullptr, bits);
         const int grid = workspace::rows_grid(N, num_cu);
         switch (p.seg * 10 + p.depth)
         {
+#define NNF_ROWS_Q(SEG, D, EPI, BITS, ZPS)                                                                             \
+    launch_rows_q<SEG, D, workspace::ROWS_WAVES, EPI, BITS>(stream, A, Wq, S, Y, N, K, zp, group_shift, ZPS, p, grid)
 #define NNF_ROWS_CASE(SEG, D)                                                                                          \
     case SEG * 10 + D:                                                                                                 \
-        return zero_points ? launch_rows_q<SEG, D, workspace::ROWS_WAVES, 3>(stream, A, Wq, S, Y, N, K, zp, group_shift,  \
-                                                                            zero_points, p, grid)                       \
-                           : launch_rows_q<SEG, D, workspace::ROWS_WAVES, 4>(stream, A, Wq, S, Y, N, K, zp, group_shift,  \
-                                                                            nullptr, p, grid);
+        if (bits == 8)                                                                                                 \
+            return zero_points ? NNF_ROWS_Q(SEG, D, 3, 8, zero_points) : NNF_ROWS_Q(SEG, D, 4, 8, nullptr);            \
+        return zero_points ? NNF_ROWS_Q(SEG, D, 3, 4, zero_points) : NNF_ROWS_Q(SEG, D, 4, 4, nullptr);
             NNF_ROWS_CASE(1, 1)
             NNF_ROWS_CASE(1, 2)
             NNF_ROWS_CASE(1, 3)
@@ -191,6 +192,7 @@ namespace nnf
             NNF_ROWS_CASE(3, 1)
             NNF_ROWS_CASE(3, 2)
 #undef NNF_ROWS_CASE
+#undef NNF_ROWS_Q
         default: return hipErrorInvalidValue;
         }
     }

@@ -7,9 +7,10 @@
 // (src/nnfusion/core/kernels/cpu/reference/kernels.cpp:601-623: integer subtract of the offset, cast, multiply by
 // the scale); the kernels in w4a16_*.hip serve the one combination the benchmark uses (4 bits, groups of 128, a
 // scalar zero point) as fast as the hardware allows, these serve every other one correctly and simply:
-//   * wna16_gemv_kernel (M = 1): a wavefront per block of four weight rows; a lane turns 16 bytes of weights of each
-//     into the exact integers q - z in fp16, multiplies them with the activations (v_dot2_f32_f16, fp32 sums) and
-//     applies the group's scale to the sum over its piece of the group;
+//   * wna16_gemv_kernel (M = 1 where K is not a multiple of 256; the others run on the row-streaming kernel of
+//     w4a16_gemv_rows.hip, 4- and 8-bit weights alike): a wavefront per block of four weight rows; a lane turns 16
+//     bytes of weights of each into the exact integers q - z in fp16, multiplies them with the activations
+//     (v_dot2_f32_f16, fp32 sums) and applies the group's scale to the sum over its piece of the group;
 //   * wna16_skinny_kernel (2 <= M <= 16): v_mfma_f32_16x16x32_f16, activations and weights fetched straight into the
 //     operand registers, eight wavefronts share the K range of two tiles of 16 weight rows;
 //   * wna16_tile_kernel / wna16_tile128_kernel (M > 16): 64 x 64 or, once they fill the chip, 128 x 128 output tiles on
@@ -566,9 +567,9 @@ namespace nnf
         {
             if (M == 1)
             {
-                // 4-bit weights in rows the row-streaming kernel can walk: that kernel
-                if (bits == 4 && w4a16_gemv_rows_q_supported(1, N, K, qa.group_shift, zero_points != nullptr, num_cu))
-                    return launch_w4a16_gemv_rows_q(stream, A, Wq, S, Y, N, K, qa.group_shift, zp, zero_points, num_cu);
+                // rows the row-streaming kernel can walk: that kernel
+                if (w4a16_gemv_rows_q_supported(1, N, K, qa.group_shift, zero_points != nullptr, num_cu, bits))
+                    return launch_w4a16_gemv_rows_q(stream, A, Wq, S, Y, N, K, qa.group_shift, zp, zero_points, num_cu, bits);
                 if (bits == 4)
                     launch_wna16_gemv<4, 4, 1>(stream, A, Wq, S, Y, M, N, K, qa, num_cu);
                 else

@@ -375,15 +375,15 @@ namespace nnf
         };
         // N: outputs (gate: from 2 N weight rows).  forced_depth: 0 = the plan's own choice
         inline RowsPlan plan_w4a16_rows(int M, int N, int K, int num_cu, int forced_depth = 0, bool gate = false,
-                                        int group_shift = 7, bool zero_points = false)
+                                        int group_shift = 7, bool zero_points = false, int bits = 4)
         {
             RowsPlan p;
             // whole 16-byte pieces of scales per segment, 4-byte aligned: K a multiple of 256
             // (the activations are fetched as at most 2048 16-byte units: K <= 16384)
             if (M != 1 || N < 1 || K < 1024 || K > 16384 || (K & 255) || num_cu < 1 || group_shift < 5 || group_shift > 7 ||
-                (gate && (group_shift != 7 || zero_points)))
+                (gate && (group_shift != 7 || zero_points)) || (bits != 4 && (bits != 8 || gate)))
                 return p;
-            const int loads_per_row = ((K >> 1) + 1023) >> 10;
+            const int loads_per_row = ((bits == 8 ? K : K >> 1) + 1023) >> 10;
             int kshift = 0;
             while ((1 << kshift) <= ROWS_WAVES && (loads_per_row + (1 << kshift) - 1) >> kshift > 3)
                 ++kshift;

@@ -45,7 +45,7 @@ SHAPES = [
     # of groups, the benchmark's shapes
     (1, 4096, 4096), (1, 33, 128), (3, 1000, 512), (16, 257, 2048), (5, 64, 160), (1, 12288, 4096), (8, 300, 11008),
     (16, 4111, 4096), (2, 7, 384),
-    # one row of 4-bit weights, K a multiple of 256: the row-streaming kernel (one, two and three loads per row and
+    # one row, K a multiple of 256: the row-streaming kernel (one, two and three loads per row and
     # wavefront; one, two and four wavefronts per row; fewer rows than wavefronts)
     (1, 300, 1024), (1, 22016, 4096), (1, 4096, 11008), (1, 1000, 8192), (1, 5000, 16384), (1, 257, 2560), (1, 5, 4096),
     # a few rows of 4-bit weights with K = 2048 / 4096 / 8192: the row-streaming MFMA kernel (one, two and four loads per
@@ -123,6 +123,24 @@ def test_one_hot_rows_through_the_row_streaming_kernels(gpu, m, k, group, zp_ten
         for r, kk in enumerate(chunk):
             np.testing.assert_array_equal(y[r], wd[:, kk].astype(np.float16), err_msg="k = %d" % kk)
         assert not y[len(chunk):].any()
+
+
+@pytest.mark.parametrize("k", [1024, 2048, 2560, 4096, 8192, 11008, 16384])
+@pytest.mark.parametrize("group,zp_tensor", [(32, True), (64, True), (128, True), (32, False), (128, False)])
+def test_one_hot_rows_through_the_row_streaming_kernel_with_8_bit_weights(gpu, k, group, zp_tensor):
+    """8-bit weights with one row and K a multiple of 256 run on the row-streaming kernel as well (a row is K bytes, a
+    lane meets 16 weights per load): the same pin (first and last weight of a group, of a lane, of a wavefront's load,
+    of a wavefront's K segment, of the row)."""
+    n = 700
+    _, wq, s, zps = _case(13, 1, n, k, 8, group, zp_tensor)
+    wd = oracle.dequantize_wn(wq, s, 8, group, zp=201, zero_points=zps)
+    kks = [kk for kk in sorted({0, 1, 15, 16, 31, 32, 63, 64, 127, 128, 255, 256, 1023, 1024, 2047, 2048, 3071, 3072, 4095, 4096,
+                                6143, 6144, 8191, 8192, k // 2 - 1, k // 2, k - 129, k - 33, k - 17, k - 1}) if kk < k]
+    for kk in kks:
+        a = np.zeros((1, k), np.float16)
+        a[0, kk] = 1.0
+        y = _run(gpu, a, wq, s, 8, group, 201, zps)
+        np.testing.assert_array_equal(y[0], wd[:, kk].astype(np.float16), err_msg="k = %d" % kk)
 
 
 def _random_shapes(count):
