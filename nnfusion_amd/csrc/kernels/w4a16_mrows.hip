@@ -678,6 +678,225 @@ namespace nnf
         mrows_flush<false, MB>(parked, Y, t0, T, M, N, tid, GemvFusionArgs{nullptr, nullptr, nullptr, nullptr, 0.f}, 0);
     }
 
+    // ---- 8-bit weights -------------------------------------------------------------------------------------------------
+    // w4a16_mrows_q_kernel for 8-bit weights (u8 [N, K]; zero points, ZPT, u8 [N, K / group]), 2 <= M <= 16.  The geometry
+    // in bytes is the same (a wavefront takes GW x 64 bytes of each of a tile's 16 weight rows per step, the eight
+    // wavefronts side by side along the row), so K = GW x 512 x STEPS; a lane's 16 bytes are 16 weights and meet 32 bytes
+    // of activations (two MFMAs per piece instead of four), kept in memory order: a byte b becomes 1024 + b with one
+    // v_perm_b32 per pair (0x64 above it), -(1024 + z) is the same pattern applied to z with the sign bit set, then the
+    // scale: fp16((q - z) * s) with one rounding.
+    // Per step a wavefront fetches the SPR = GW x 64 / group scales of each of the 16 rows (4-byte loads) and, ZPT, their
+    // zero points (one byte per lane).  LDS and `pack` as in w4a16_mrows_q_kernel.
+    template <int GW, int STEPS, int GSHIFT, bool ZPT>
+    __global__ __launch_bounds__(512) void w8a16_mrows_q_kernel(const half_t* __restrict__ A, const uint8_t* __restrict__ Wq,
+                                                                const half_t* __restrict__ S, half_t* __restrict__ Y,
+                                                                const uint8_t* __restrict__ zps, int N, int tiles_q,
+                                                                int tiles_r, int pack)
+    {
+        static_assert((GW == 2 || GW == 4) && (STEPS == 2 || STEPS == 4), "K = 2048, 4096, 8192");
+        static_assert(GSHIFT >= 5 && GSHIFT <= 7 && (((GW * 64) >> GSHIFT) & 1) == 0 && ((GW * 64) >> GSHIFT) >= 2, "whole words of scales");
+        constexpr int MB = 1;
+        constexpr int ROW_BYTES = GW * 512 * STEPS; // a weight row
+        constexpr int K = ROW_BYTES, G = K >> GSHIFT;
+        constexpr int GA = GW * STEPS;          // 64-byte pieces of a weight row per wavefront
+        constexpr int SLICE = GW * 64;          // a wavefront's bytes of a weight row per step
+        constexpr int SPAN = 8 * SLICE;         // bytes of a weight row that the workgroup covers per step
+        constexpr int TILE_BYTES = 16 * SLICE;  // = GW KiB: GW wavefront-wide loads
+        constexpr int SPR = (GW * 64) >> GSHIFT; // scales (and zero points) per row, step and wavefront
+        constexpr int WPR = SPR / 2;             // ... as 4-byte words
+        constexpr int NSL = (16 * WPR + 63) / 64;
+        constexpr int NZL = ZPT ? (16 * SPR + 63) / 64 : 0;
+        constexpr int AUX = (NSL + NZL) * 256;
+        constexpr int LT = GW + NSL + NZL; // loads per step and wavefront
+        extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+
+        const int tid = threadIdx.x;
+        const int lane = tid & 63;
+        const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+        const int col = lane & 15; // n within the tile (B operand / D column), m for the A operand
+        const int kq = lane >> 4;  // K quarter of the MFMA operands, row quad of D
+        const int M = pack & 0xff, zp = (pack >> 8) & 0xff;
+        const int b = blockIdx.x;
+        const int t0 = b * tiles_q + min(b, tiles_r);
+        const int T = tiles_q + (b < tiles_r ? 1 : 0);
+        auto row0_of = [&](int i) { return __builtin_amdgcn_readfirstlane(min((t0 + i) * 16, N - 16)); };
+
+        uint8_t* ring = smem + wave * (2 * TILE_BYTES);
+        uint8_t* aux = smem + MR_WAVES * 2 * TILE_BYTES + wave * (2 * AUX);
+        uint8_t* red = smem + MR_WAVES * 2 * TILE_BYTES + MR_WAVES * 2 * AUX; // [2][8][1024]
+        float* parked = reinterpret_cast<float*>(red + 2 * MR_WAVES * MB * 1024);
+
+        // weights: as in w4a16_mrows_kernel
+        auto swz = [](int r) { return GW % 4 == 0 ? (r & 15) : (r >> 1) & 7; };
+        uint32_t w_off[GW];
+#pragma unroll
+        for (int c = 0; c < GW; ++c)
+        {
+            const int pos = c * 1024 + 16 * lane;
+            const int r = pos / SLICE, q = (pos % SLICE) >> 4;
+            w_off[c] = (uint32_t)r * ROW_BYTES + (uint32_t)wave * SLICE + (uint32_t)((q ^ swz(r)) << 4);
+        }
+        // scales: lane l of load i fetches word (64 i + l) % WPR of row (64 i + l) / WPR (lanes past the 16 rows: the
+        // last row again); zero points: the same with the SPR bytes of a row
+        uint32_t s_off[NSL], z_off[NZL > 0 ? NZL : 1];
+#pragma unroll
+        for (int i = 0; i < NSL; ++i)
+        {
+            const int at = i * 64 + lane;
+            const int r = min(at / WPR, 15), wd = at % WPR;
+            s_off[i] = (uint32_t)r * (G * 2) + (uint32_t)wave * (SPR * 2) + (uint32_t)wd * 4u;
+        }
+#pragma unroll
+        for (int i = 0; i < NZL; ++i)
+        {
+            const int at = i * 64 + lane;
+            const int r = min(at / SPR, 15), bz = at % SPR;
+            z_off[i] = (uint32_t)r * G + (uint32_t)wave * SPR + (uint32_t)bz;
+        }
+
+        // step st of tile `tile` into slot `slot`
+        auto issue = [&](int tile, int st, int slot) {
+            const uint32_t row0 = (uint32_t)row0_of(tile);
+            const uint8_t* wsrc = Wq + (size_t)row0 * ROW_BYTES + st * SPAN;
+#pragma unroll
+            for (int c = 0; c < GW; ++c)
+                __builtin_amdgcn_global_load_lds((mr_global_ptr_t)(wsrc + w_off[c]),
+                                                 (mr_lds_ptr_t)(ring + slot * TILE_BYTES + c * 1024), 16, 0, 0);
+            const uint8_t* ssrc = reinterpret_cast<const uint8_t*>(S) + (size_t)row0 * (G * 2) + st * (8 * SPR * 2);
+#pragma unroll
+            for (int i = 0; i < NSL; ++i)
+                __builtin_amdgcn_global_load_lds((mr_global_ptr_t)(ssrc + s_off[i]), (mr_lds_ptr_t)(aux + slot * AUX + i * 256), 4, 0, 0);
+            if constexpr (ZPT)
+            {
+                const uint8_t* zsrc = zps + (size_t)row0 * G + st * (8 * SPR);
+#pragma unroll
+                for (int i = 0; i < NZL; ++i)
+                    __builtin_amdgcn_global_load_lds((mr_global_ptr_t)(zsrc + z_off[i]),
+                                                     (mr_lds_ptr_t)(aux + slot * AUX + (NSL + i) * 256), 1, 0, 0);
+            }
+        };
+
+        issue(0, 0, 0);
+        issue(0, 1, 1);
+        // activations: into the MFMA operand registers (through LDS as whole lines from a few rows on, see
+        // workspace::mrows_stages_activations); a block of 16 rows x 256 bytes holds two neighbouring pieces
+        uintx4 areg[GA][2];
+        if (!workspace::mrows_stages_activations(M, K))
+        {
+            const uint8_t* a_bytes = reinterpret_cast<const uint8_t*>(A);
+            const uint32_t a_off = (uint32_t)min(col, M - 1) * (uint32_t)(K * 2) + (uint32_t)wave * (GW * 128) + (uint32_t)kq * 32u;
+#pragma unroll
+            for (int g = 0; g < GA; ++g)
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    areg[g][j] = *reinterpret_cast<const uintx4*>(a_bytes + (size_t)(a_off + (g / GW) * (SPAN * 2) + (g % GW) * 128 + j * 16));
+        }
+        else
+        {
+            uint8_t* stage = red + wave * (2 * ROW_BLOCK_BYTES);
+            constexpr int NP = GA / 2;
+            auto fetch = [&](int p) {
+                const int g = 2 * p;
+                row_block_fetch(reinterpret_cast<const uint8_t*>(A), (size_t)K * 2, 0, M - 1,
+                                (size_t)((g / GW) * (SPAN * 2) + wave * (GW * 128) + (g % GW) * 128), stage + (p & 1) * ROW_BLOCK_BYTES, lane);
+            };
+            fetch(0);
+#pragma unroll
+            for (int p = 0; p < NP; ++p)
+            {
+                if (p + 1 < NP)
+                {
+                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); // block p-1 has been read out of the half that is filled next
+                    fetch(p + 1);
+                    __builtin_amdgcn_s_waitcnt(vmcnt_only(4));
+                }
+                else
+                    __builtin_amdgcn_s_waitcnt(vmcnt_only(0));
+#pragma unroll
+                for (int h = 0; h < 2; ++h)
+#pragma unroll
+                    for (int j = 0; j < 2; ++j)
+                        areg[2 * p + h][j] = row_block_piece(stage + (p & 1) * ROW_BLOCK_BYTES, col, h * 8 + kq * 2 + j);
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            __syncthreads();
+        }
+
+        // ---- tile loop ---------------------------------------------------------------------------------------
+        const uint32_t rd_base = (uint32_t)col * SLICE;
+        const int rd_swz = swz(col);
+        const uint32_t red_addr = lds_address(red) + (uint32_t)(wave * (MB * 1024) + lane * 16);
+        const uint32_t parked_addr = lds_address(parked);
+        // the lane's piece g of a step lies in scale (g * 64 + kq * 16) >> GSHIFT of the row's SPR
+        uint32_t sc_rd[GW], z_rd[GW];
+#pragma unroll
+        for (int g = 0; g < GW; ++g)
+        {
+            const int i = (g * 64 + kq * 16) >> GSHIFT;
+            sc_rd[g] = (uint32_t)(col * SPR + i) * 2u;
+            z_rd[g] = (uint32_t)(NSL * 256 + (col * SPR + i) * 4);
+        }
+        const uint32_t zp16 = (uint32_t)zp | ((uint32_t)zp << 16);
+        int slot = 0;
+        for (int it = 0; it < T; ++it)
+        {
+            floatx4 acc[MB];
+            acc[0] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int st = 0; st < STEPS; ++st)
+            {
+                __builtin_amdgcn_s_waitcnt(mr_vmcnt(LT));
+                uintx4 wv[GW];
+                uint32_t s2[GW], z16[GW];
+                {
+                    const uint8_t* sl = ring + slot * TILE_BYTES + rd_base;
+                    const uint8_t* ax = aux + slot * AUX;
+#pragma unroll
+                    for (int g = 0; g < GW; ++g)
+                    {
+                        wv[g] = *reinterpret_cast<const uintx4*>(sl + (((g * 4 + kq) ^ rd_swz) << 4));
+                        const uint32_t sh = *reinterpret_cast<const uint16_t*>(ax + sc_rd[g]);
+                        s2[g] = sh | (sh << 16);
+                        if constexpr (ZPT)
+                        {
+                            const uint32_t z = (uint32_t)ax[z_rd[g]];
+                            z16[g] = z | (z << 16);
+                        }
+                        else
+                            z16[g] = zp16;
+                    }
+                }
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                issue(min(it + (st + 2) / STEPS, T - 1), (st + 2) % STEPS, slot);
+                slot ^= 1;
+#pragma unroll
+                for (int g = 0; g < GW; ++g)
+                {
+                    const half2_t sc = as_half2(s2[g]);
+                    const half2_t add = as_half2(z16[g] | 0xE400E400u); // -(1024 + z)
+                    const uint32_t ww[4] = {wv[g].x, wv[g].y, wv[g].z, wv[g].w};
+#pragma unroll
+                    for (int j = 0; j < 2; ++j)
+                    {
+                        // v_perm_b32(S0, S1, sel): selectors 0-3 pick bytes of S1, 4-7 of S0
+                        const uint32_t w0 = ww[2 * j], w1 = ww[2 * j + 1];
+                        uintx4 bq;
+                        bq.x = as_u32((as_half2(__builtin_amdgcn_perm(0x64646464u, w0, 0x04010400u)) + add) * sc);
+                        bq.y = as_u32((as_half2(__builtin_amdgcn_perm(0x64646464u, w0, 0x04030402u)) + add) * sc);
+                        bq.z = as_u32((as_half2(__builtin_amdgcn_perm(0x64646464u, w1, 0x04010400u)) + add) * sc);
+                        bq.w = as_u32((as_half2(__builtin_amdgcn_perm(0x64646464u, w1, 0x04030402u)) + add) * sc);
+                        acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, areg[st * GW + g][j]),
+                                                                        __builtin_bit_cast(half8_t, bq), acc[0], 0, 0, 0);
+                    }
+                }
+            }
+            mrows_reduce_park<MB>(acc, red, red_addr, parked_addr, it & 1, it, M, tid);
+        }
+        __builtin_amdgcn_s_waitcnt(mr_vmcnt(0)); // the reloads past the end, before the LDS goes away
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        mrows_flush<false, MB>(parked, Y, t0, T, M, N, tid, GemvFusionArgs{nullptr, nullptr, nullptr, nullptr, 0.f}, 0);
+    }
+
     // w4a16_mrows_q_kernel with K as a run-time value (any multiple of 256; 2 <= M <= 16), as w4a16_mrows_any_kernel below
     // does it for groups of 128 with a scalar zero point: two steps of 8 * GW blocks of 128 weights; a wavefront whose
     // blocks of a step would reach past the end of its range of K fetches the last GW blocks of the range instead and
@@ -1393,6 +1612,70 @@ namespace nnf
         case 1: return launch_mrows_q_gw<1>(stream, A, Wq, S, Y, M, N, group_shift, zp, zero_points, num_cu);
         case 2: return launch_mrows_q_gw<2>(stream, A, Wq, S, Y, M, N, group_shift, zp, zero_points, num_cu);
         default: return launch_mrows_q_gw<4>(stream, A, Wq, S, Y, M, N, group_shift, zp, zero_points, num_cu);
+        }
+    }
+
+    namespace
+    {
+        template <int GW, int STEPS, int GSHIFT, bool ZPT>
+        hipError_t launch_mrows_q8(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M, int N, int zp,
+                                   const void* zps, int num_cu)
+        {
+            if constexpr (((GW * 64) >> GSHIFT) < 2)
+                return hipErrorInvalidValue;
+            else
+            {
+                const int n_tiles = (N + 15) / 16;
+                const int grid = n_tiles < num_cu ? n_tiles : num_cu;
+                const int tiles_q = n_tiles / grid, tiles_r = n_tiles % grid;
+                const size_t lds = workspace::w8a16_mrows_q_lds_bytes(GW * 512 * STEPS, M, tiles_q + (tiles_r ? 1 : 0), GSHIFT, ZPT);
+                if (lds > MAX_LDS_BYTES)
+                    return hipErrorInvalidValue;
+                auto kernel = &w8a16_mrows_q_kernel<GW, STEPS, GSHIFT, ZPT>;
+                if (lds > 64 * 1024)
+                {
+                    static LdsGrant granted;
+                    const hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), granted, (int)MAX_LDS_BYTES);
+                    if (e != hipSuccess)
+                        return e;
+                }
+                hipLaunchKernelGGL(kernel, dim3(grid), dim3(MR_WAVES * 64), lds, stream, (const half_t*)A, (const uint8_t*)Wq,
+                                   (const half_t*)S, (half_t*)Y, (const uint8_t*)zps, N, tiles_q, tiles_r, M | (zp << 8));
+                return hipGetLastError();
+            }
+        }
+        template <int GW, int STEPS>
+        hipError_t launch_mrows_q8_gw(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M, int N,
+                                      int group_shift, int zp, const void* zps, int num_cu)
+        {
+            switch (group_shift * 2 + (zps ? 1 : 0))
+            {
+            case 10: return launch_mrows_q8<GW, STEPS, 5, false>(stream, A, Wq, S, Y, M, N, zp, zps, num_cu);
+            case 11: return launch_mrows_q8<GW, STEPS, 5, true>(stream, A, Wq, S, Y, M, N, zp, zps, num_cu);
+            case 12: return launch_mrows_q8<GW, STEPS, 6, false>(stream, A, Wq, S, Y, M, N, zp, zps, num_cu);
+            case 13: return launch_mrows_q8<GW, STEPS, 6, true>(stream, A, Wq, S, Y, M, N, zp, zps, num_cu);
+            case 14: return launch_mrows_q8<GW, STEPS, 7, false>(stream, A, Wq, S, Y, M, N, zp, zps, num_cu);
+            case 15: return launch_mrows_q8<GW, STEPS, 7, true>(stream, A, Wq, S, Y, M, N, zp, zps, num_cu);
+            default: return hipErrorInvalidValue;
+            }
+        }
+    } // namespace
+
+    bool w8a16_mrows_q_supported(int M, int N, int K, int group_shift, bool zero_points, int num_cu)
+    {
+        return workspace::w8a16_mrows_q_fits(M, N, K, group_shift, zero_points, num_cu);
+    }
+
+    hipError_t launch_w8a16_mrows_q(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M, int N,
+                                    int K, int group_shift, int zp, const void* zero_points, int num_cu)
+    {
+        if (!w8a16_mrows_q_supported(M, N, K, group_shift, zero_points != nullptr, num_cu))
+            return hipErrorInvalidValue;
+        switch (K)
+        {
+        case 2048: return launch_mrows_q8_gw<2, 2>(stream, A, Wq, S, Y, M, N, group_shift, zp, zero_points, num_cu);
+        case 4096: return launch_mrows_q8_gw<4, 2>(stream, A, Wq, S, Y, M, N, group_shift, zp, zero_points, num_cu);
+        default: return launch_mrows_q8_gw<4, 4>(stream, A, Wq, S, Y, M, N, group_shift, zp, zero_points, num_cu);
         }
     }
 

@@ -577,6 +577,24 @@ namespace nnf
             const int grid = n_tiles < num_cu ? n_tiles : num_cu;
             return w4a16_mrows_q_lds_bytes(K, M, (n_tiles + grid - 1) / grid, group_shift, zero_points) <= LDS_BYTES_PER_CU;
         }
+        // 8-bit weights, 2 .. 16 rows (w8a16_mrows_q_kernel): K = 4096 / 8192 (four 64-byte pieces of a weight row per
+        // wavefront and step, two / four steps), K = 2048 with groups of 32 / 64 (two pieces, two steps)
+        inline size_t w8a16_mrows_q_lds_bytes(int K, int M, int tiles, int group_shift, bool zero_points)
+        {
+            const int gw = K == 2048 ? 2 : 4;
+            const int spr = (gw * 64) >> group_shift; // scales per row, step and wavefront
+            const int loads = (16 * (spr / 2) + 63) / 64 + (zero_points ? (16 * spr + 63) / 64 : 0);
+            return (size_t)8 * 2 * gw * 1024 + (size_t)8 * 2 * loads * 256 + mrows_tail_bytes((size_t)2 * 8 * 1024 + (size_t)tiles * M * 64);
+        }
+        inline bool w8a16_mrows_q_fits(int M, int N, int K, int group_shift, bool zero_points, int num_cu)
+        {
+            if (M < 2 || M > 16 || N < 16 || num_cu < 1 || (K != 2048 && K != 4096 && K != 8192) || group_shift < 5 ||
+                group_shift > 7 || (K == 2048 && group_shift == 7))
+                return false;
+            const int n_tiles = (N + 15) / 16;
+            const int grid = n_tiles < num_cu ? n_tiles : num_cu;
+            return w8a16_mrows_q_lds_bytes(K, M, (n_tiles + grid - 1) / grid, group_shift, zero_points) <= LDS_BYTES_PER_CU;
+        }
         // ... and with K as a run-time value (w4a16_mrows_q_any_kernel): 2 .. 16 rows, any other multiple of 256.  Up to
         // K = 8192 in one piece (two steps of 8 x gw blocks of 128 weights, when at least three quarters of what the
         // wavefronts fetch counts), above over ranges of at most 32 blocks with fp32 sums per range and the reduction pass

@@ -125,22 +125,27 @@ def test_one_hot_rows_through_the_row_streaming_kernels(gpu, m, k, group, zp_ten
         assert not y[len(chunk):].any()
 
 
-@pytest.mark.parametrize("k", [1024, 2048, 2560, 4096, 8192, 11008, 16384])
+@pytest.mark.parametrize("m,k", [(1, 1024), (1, 2048), (1, 2560), (1, 4096), (1, 8192), (1, 11008), (1, 16384), (16, 2048), (7, 4096),
+                                 (16, 4096), (3, 8192), (16, 8192)])
 @pytest.mark.parametrize("group,zp_tensor", [(32, True), (64, True), (128, True), (32, False), (128, False)])
-def test_one_hot_rows_through_the_row_streaming_kernel_with_8_bit_weights(gpu, k, group, zp_tensor):
-    """8-bit weights with one row and K a multiple of 256 run on the row-streaming kernel as well (a row is K bytes, a
-    lane meets 16 weights per load): the same pin (first and last weight of a group, of a lane, of a wavefront's load,
-    of a wavefront's K segment, of the row)."""
+def test_one_hot_rows_through_the_row_streaming_kernels_with_8_bit_weights(gpu, m, k, group, zp_tensor):
+    """8-bit weights with one row and K a multiple of 256, or 2 .. 16 rows and K = 2048 / 4096 / 8192, run on the
+    row-streaming kernels as well (a row is K bytes, a lane meets 16 weights per load): the same pin (first and last
+    weight of a group, of a lane, of a wavefront's load, of a wavefront's K segment, of a step, of the row)."""
     n = 700
     _, wq, s, zps = _case(13, 1, n, k, 8, group, zp_tensor)
     wd = oracle.dequantize_wn(wq, s, 8, group, zp=201, zero_points=zps)
-    kks = [kk for kk in sorted({0, 1, 15, 16, 31, 32, 63, 64, 127, 128, 255, 256, 1023, 1024, 2047, 2048, 3071, 3072, 4095, 4096,
-                                6143, 6144, 8191, 8192, k // 2 - 1, k // 2, k - 129, k - 33, k - 17, k - 1}) if kk < k]
-    for kk in kks:
-        a = np.zeros((1, k), np.float16)
-        a[0, kk] = 1.0
+    kks = [kk for kk in sorted({0, 1, 15, 16, 31, 32, 63, 64, 127, 128, 255, 256, 511, 512, 1023, 1024, 2047, 2048, 3071, 3072,
+                                4095, 4096, 6143, 6144, 8191, 8192, k // 2 - 1, k // 2, k - 129, k - 33, k - 17, k - 1}) if kk < k]
+    for c in range(0, len(kks), m):
+        chunk = kks[c:c + m]
+        a = np.zeros((m, k), np.float16)
+        for r, kk in enumerate(chunk):
+            a[r, kk] = 1.0
         y = _run(gpu, a, wq, s, 8, group, 201, zps)
-        np.testing.assert_array_equal(y[0], wd[:, kk].astype(np.float16), err_msg="k = %d" % kk)
+        for r, kk in enumerate(chunk):
+            np.testing.assert_array_equal(y[r], wd[:, kk].astype(np.float16), err_msg="k = %d" % kk)
+        assert not y[len(chunk):].any()
 
 
 def _random_shapes(count):
