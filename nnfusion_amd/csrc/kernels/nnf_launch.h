@@ -90,7 +90,7 @@ namespace nnf
     hipError_t launch_w4a16_mrows_q(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M, int N,
                                     int K, int group_shift, int zp, const void* zero_points, int num_cu);
     bool w4a16_mrows_q_supported(int M, int N, int K, int group_shift, bool zero_points, int num_cu);
-    // ... for 8-bit weights (u8 [N, K]; zero points u8 [N, K / group]): 2 <= M <= 16, K = 2048 (groups of 32 / 64) / 4096 /
+    // ... for 8-bit weights (u8 [N, K]; zero points u8 [N, K / group]): 2 <= M <= 16 (32 up to K = 4096), K = 2048 (groups of 32 / 64) / 4096 /
     // 8192
     hipError_t launch_w8a16_mrows_q(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M, int N,
                                     int K, int group_shift, int zp, const void* zero_points, int num_cu);

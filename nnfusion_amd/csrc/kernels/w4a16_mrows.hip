@@ -679,7 +679,8 @@ namespace nnf
     }
 
     // ---- 8-bit weights -------------------------------------------------------------------------------------------------
-    // w4a16_mrows_q_kernel for 8-bit weights (u8 [N, K]; zero points, ZPT, u8 [N, K / group]), 2 <= M <= 16.  The geometry
+    // w4a16_mrows_q_kernel for 8-bit weights (u8 [N, K]; zero points, ZPT, u8 [N, K / group]), 2 <= M <= 16 MB (two
+    // blocks of rows up to K = 4096).  The geometry
     // in bytes is the same (a wavefront takes GW x 64 bytes of each of a tile's 16 weight rows per step, the eight
     // wavefronts side by side along the row), so K = GW x 512 x STEPS; a lane's 16 bytes are 16 weights and meet 32 bytes
     // of activations (two MFMAs per piece instead of four), kept in memory order: a byte b becomes 1024 + b with one
@@ -687,7 +688,7 @@ namespace nnf
     // scale: fp16((q - z) * s) with one rounding.
     // Per step a wavefront fetches the SPR = GW x 64 / group scales of each of the 16 rows (4-byte loads) and, ZPT, their
     // zero points (one byte per lane).  LDS and `pack` as in w4a16_mrows_q_kernel.
-    template <int GW, int STEPS, int GSHIFT, bool ZPT>
+    template <int GW, int STEPS, int GSHIFT, bool ZPT, int MB>
     __global__ __launch_bounds__(512) void w8a16_mrows_q_kernel(const half_t* __restrict__ A, const uint8_t* __restrict__ Wq,
                                                                 const half_t* __restrict__ S, half_t* __restrict__ Y,
                                                                 const uint8_t* __restrict__ zps, int N, int tiles_q,
@@ -695,7 +696,7 @@ namespace nnf
     {
         static_assert((GW == 2 || GW == 4) && (STEPS == 2 || STEPS == 4), "K = 2048, 4096, 8192");
         static_assert(GSHIFT >= 5 && GSHIFT <= 7 && (((GW * 64) >> GSHIFT) & 1) == 0 && ((GW * 64) >> GSHIFT) >= 2, "whole words of scales");
-        constexpr int MB = 1;
+        static_assert(MB == 1 || (MB == 2 && GW * STEPS <= 8), "two blocks of rows: 16 VGPRs per piece");
         constexpr int ROW_BYTES = GW * 512 * STEPS; // a weight row
         constexpr int K = ROW_BYTES, G = K >> GSHIFT;
         constexpr int GA = GW * STEPS;          // 64-byte pieces of a weight row per wavefront
@@ -780,8 +781,8 @@ namespace nnf
         issue(0, 1, 1);
         // activations: into the MFMA operand registers (through LDS as whole lines from a few rows on, see
         // workspace::mrows_stages_activations); a block of 16 rows x 256 bytes holds two neighbouring pieces
-        uintx4 areg[GA][2];
-        if (!workspace::mrows_stages_activations(M, K))
+        uintx4 areg[MB][GA][2];
+        if (MB == 1 && !workspace::mrows_stages_activations(M, K))
         {
             const uint8_t* a_bytes = reinterpret_cast<const uint8_t*>(A);
             const uint32_t a_off = (uint32_t)min(col, M - 1) * (uint32_t)(K * 2) + (uint32_t)wave * (GW * 128) + (uint32_t)kq * 32u;
@@ -789,15 +790,15 @@ namespace nnf
             for (int g = 0; g < GA; ++g)
 #pragma unroll
                 for (int j = 0; j < 2; ++j)
-                    areg[g][j] = *reinterpret_cast<const uintx4*>(a_bytes + (size_t)(a_off + (g / GW) * (SPAN * 2) + (g % GW) * 128 + j * 16));
+                    areg[0][g][j] = *reinterpret_cast<const uintx4*>(a_bytes + (size_t)(a_off + (g / GW) * (SPAN * 2) + (g % GW) * 128 + j * 16));
         }
         else
         {
             uint8_t* stage = red + wave * (2 * ROW_BLOCK_BYTES);
-            constexpr int NP = GA / 2;
+            constexpr int NP = MB * (GA / 2);
             auto fetch = [&](int p) {
-                const int g = 2 * p;
-                row_block_fetch(reinterpret_cast<const uint8_t*>(A), (size_t)K * 2, 0, M - 1,
+                const int mb = p / (GA / 2), g = 2 * (p % (GA / 2));
+                row_block_fetch(reinterpret_cast<const uint8_t*>(A), (size_t)K * 2, mb * 16, M - 1,
                                 (size_t)((g / GW) * (SPAN * 2) + wave * (GW * 128) + (g % GW) * 128), stage + (p & 1) * ROW_BLOCK_BYTES, lane);
             };
             fetch(0);
@@ -816,7 +817,7 @@ namespace nnf
                 for (int h = 0; h < 2; ++h)
 #pragma unroll
                     for (int j = 0; j < 2; ++j)
-                        areg[2 * p + h][j] = row_block_piece(stage + (p & 1) * ROW_BLOCK_BYTES, col, h * 8 + kq * 2 + j);
+                        areg[p / (GA / 2)][2 * (p % (GA / 2)) + h][j] = row_block_piece(stage + (p & 1) * ROW_BLOCK_BYTES, col, h * 8 + kq * 2 + j);
             }
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
             __syncthreads();
@@ -841,7 +842,9 @@ namespace nnf
         for (int it = 0; it < T; ++it)
         {
             floatx4 acc[MB];
-            acc[0] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb)
+                acc[mb] = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int st = 0; st < STEPS; ++st)
             {
@@ -885,8 +888,10 @@ namespace nnf
                         bq.y = as_u32((as_half2(__builtin_amdgcn_perm(0x64646464u, w0, 0x04030402u)) + add) * sc);
                         bq.z = as_u32((as_half2(__builtin_amdgcn_perm(0x64646464u, w1, 0x04010400u)) + add) * sc);
                         bq.w = as_u32((as_half2(__builtin_amdgcn_perm(0x64646464u, w1, 0x04030402u)) + add) * sc);
-                        acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, areg[st * GW + g][j]),
-                                                                        __builtin_bit_cast(half8_t, bq), acc[0], 0, 0, 0);
+#pragma unroll
+                        for (int mb = 0; mb < MB; ++mb)
+                            acc[mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, areg[mb][st * GW + g][j]),
+                                                                             __builtin_bit_cast(half8_t, bq), acc[mb], 0, 0, 0);
                     }
                 }
             }
@@ -1617,11 +1622,11 @@ namespace nnf
 
     namespace
     {
-        template <int GW, int STEPS, int GSHIFT, bool ZPT>
-        hipError_t launch_mrows_q8(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M, int N, int zp,
-                                   const void* zps, int num_cu)
+        template <int GW, int STEPS, int GSHIFT, bool ZPT, int MB>
+        hipError_t launch_mrows_q8_mb(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M, int N, int zp,
+                                      const void* zps, int num_cu)
         {
-            if constexpr (((GW * 64) >> GSHIFT) < 2)
+            if constexpr (((GW * 64) >> GSHIFT) < 2 || (MB == 2 && GW * STEPS > 8))
                 return hipErrorInvalidValue;
             else
             {
@@ -1631,7 +1636,7 @@ namespace nnf
                 const size_t lds = workspace::w8a16_mrows_q_lds_bytes(GW * 512 * STEPS, M, tiles_q + (tiles_r ? 1 : 0), GSHIFT, ZPT);
                 if (lds > MAX_LDS_BYTES)
                     return hipErrorInvalidValue;
-                auto kernel = &w8a16_mrows_q_kernel<GW, STEPS, GSHIFT, ZPT>;
+                auto kernel = &w8a16_mrows_q_kernel<GW, STEPS, GSHIFT, ZPT, MB>;
                 if (lds > 64 * 1024)
                 {
                     static LdsGrant granted;
@@ -1643,6 +1648,13 @@ namespace nnf
                                    (const half_t*)S, (half_t*)Y, (const uint8_t*)zps, N, tiles_q, tiles_r, M | (zp << 8));
                 return hipGetLastError();
             }
+        }
+        template <int GW, int STEPS, int GSHIFT, bool ZPT>
+        hipError_t launch_mrows_q8(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M, int N, int zp,
+                                   const void* zps, int num_cu)
+        {
+            return M <= 16 ? launch_mrows_q8_mb<GW, STEPS, GSHIFT, ZPT, 1>(stream, A, Wq, S, Y, M, N, zp, zps, num_cu)
+                           : launch_mrows_q8_mb<GW, STEPS, GSHIFT, ZPT, 2>(stream, A, Wq, S, Y, M, N, zp, zps, num_cu);
         }
         template <int GW, int STEPS>
         hipError_t launch_mrows_q8_gw(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M, int N,

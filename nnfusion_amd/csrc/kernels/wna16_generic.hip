@@ -563,7 +563,7 @@ namespace nnf
         // 4-bit weights, a few rows (up to 32 at K = 2048 / 4096, 16 at 8192): the row-streaming MFMA kernel
         if (bits == 4 && M >= 2 && w4a16_mrows_q_supported(M, N, K, qa.group_shift, zero_points != nullptr, num_cu))
             return launch_w4a16_mrows_q(stream, A, Wq, S, Y, M, N, K, qa.group_shift, zp, zero_points, num_cu);
-        // 8-bit weights, 2 .. 16 rows at K = 2048 / 4096 / 8192: the same kernel on bytes
+        // 8-bit weights, 2 .. 16 rows at K = 2048 / 4096 / 8192 (up to 32 at 2048 / 4096): the same kernel on bytes
         if (bits == 8 && M >= 2 && w8a16_mrows_q_supported(M, N, K, qa.group_shift, zero_points != nullptr, num_cu))
             return launch_w8a16_mrows_q(stream, A, Wq, S, Y, M, N, K, qa.group_shift, zp, zero_points, num_cu);
         if (M <= 16)

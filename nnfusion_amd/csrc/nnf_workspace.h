@@ -577,18 +577,20 @@ namespace nnf
             const int grid = n_tiles < num_cu ? n_tiles : num_cu;
             return w4a16_mrows_q_lds_bytes(K, M, (n_tiles + grid - 1) / grid, group_shift, zero_points) <= LDS_BYTES_PER_CU;
         }
-        // 8-bit weights, 2 .. 16 rows (w8a16_mrows_q_kernel): K = 4096 / 8192 (four 64-byte pieces of a weight row per
+        // 8-bit weights, 2 .. 16 rows, up to 32 at K <= 4096 (w8a16_mrows_q_kernel): K = 4096 / 8192 (four 64-byte pieces of a weight row per
         // wavefront and step, two / four steps), K = 2048 with groups of 32 / 64 (two pieces, two steps)
         inline size_t w8a16_mrows_q_lds_bytes(int K, int M, int tiles, int group_shift, bool zero_points)
         {
             const int gw = K == 2048 ? 2 : 4;
             const int spr = (gw * 64) >> group_shift; // scales per row, step and wavefront
             const int loads = (16 * (spr / 2) + 63) / 64 + (zero_points ? (16 * spr + 63) / 64 : 0);
-            return (size_t)8 * 2 * gw * 1024 + (size_t)8 * 2 * loads * 256 + mrows_tail_bytes((size_t)2 * 8 * 1024 + (size_t)tiles * M * 64);
+            const size_t mb = M <= 16 ? 1 : 2; // blocks of 16 rows
+            return (size_t)8 * 2 * gw * 1024 + (size_t)8 * 2 * loads * 256 + mrows_tail_bytes((size_t)2 * 8 * mb * 1024 + (size_t)tiles * M * 64);
         }
+        // (17 .. 32 rows: two blocks of rows in registers, up to K = 4096)
         inline bool w8a16_mrows_q_fits(int M, int N, int K, int group_shift, bool zero_points, int num_cu)
         {
-            if (M < 2 || M > 16 || N < 16 || num_cu < 1 || (K != 2048 && K != 4096 && K != 8192) || group_shift < 5 ||
+            if (M < 2 || M > 32 || (M > 16 && K > 4096) || N < 16 || num_cu < 1 || (K != 2048 && K != 4096 && K != 8192) || group_shift < 5 ||
                 group_shift > 7 || (K == 2048 && group_shift == 7))
                 return false;
             const int n_tiles = (N + 15) / 16;

@@ -126,10 +126,11 @@ def test_one_hot_rows_through_the_row_streaming_kernels(gpu, m, k, group, zp_ten
 
 
 @pytest.mark.parametrize("m,k", [(1, 1024), (1, 2048), (1, 2560), (1, 4096), (1, 8192), (1, 11008), (1, 16384), (16, 2048), (7, 4096),
-                                 (16, 4096), (3, 8192), (16, 8192)])
+                                 (16, 4096), (3, 8192), (16, 8192), (20, 2048), (32, 4096)])
 @pytest.mark.parametrize("group,zp_tensor", [(32, True), (64, True), (128, True), (32, False), (128, False)])
 def test_one_hot_rows_through_the_row_streaming_kernels_with_8_bit_weights(gpu, m, k, group, zp_tensor):
-    """8-bit weights with one row and K a multiple of 256, or 2 .. 16 rows and K = 2048 / 4096 / 8192, run on the
+    """8-bit weights with one row and K a multiple of 256, or 2 .. 16 rows and K = 2048 / 4096 / 8192 (up to 32 rows at
+    2048 / 4096), run on the
     row-streaming kernels as well (a row is K bytes, a lane meets 16 weights per load): the same pin (first and last
     weight of a group, of a lane, of a wavefront's load, of a wavefront's K segment, of a step, of the row)."""
     n = 700
