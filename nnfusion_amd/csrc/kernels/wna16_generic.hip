@@ -566,6 +566,29 @@ namespace nnf
         // 8-bit weights, 2 .. 16 rows at K = 2048 / 4096 / 8192 (up to 32 at 2048 / 4096): the same kernel on bytes
         if (bits == 8 && M >= 2 && w8a16_mrows_q_supported(M, N, K, qa.group_shift, zero_points != nullptr, num_cu))
             return launch_w8a16_mrows_q(stream, A, Wq, S, Y, M, N, K, qa.group_shift, zp, zero_points, num_cu);
+        // ... and up to six blocks of 32 rows (of 16 at K = 8192) one block after the other: the plain tile kernels below
+        // spend half a microsecond per 32 values of K whatever M is (N = K = 4096: 68 - 71 us from 33 to 256 rows; a block
+        // of 32 rows takes 9.6 us here), so re-reading the weights per block is the faster way up to there
+        if (bits == 8 && M > 16)
+        {
+            const int block = K == 8192 ? 16 : 32;
+            const int blocks = (M + block - 1) / block;
+            if (blocks <= 6 && w8a16_mrows_q_supported(block, N, K, qa.group_shift, zero_points != nullptr, num_cu))
+            {
+                for (int m0 = 0; m0 < M; m0 += block)
+                {
+                    // (a last block of one row runs as two: the row before it is computed twice, to the same value)
+                    const int rows = M - m0 < block ? M - m0 : block;
+                    const int first = rows == 1 ? m0 - 1 : m0;
+                    const hipError_t e = launch_w8a16_mrows_q(stream, (const half_t*)A + (size_t)first * K, Wq, S,
+                                                              (half_t*)Y + (size_t)first * N, m0 + rows - first, N, K,
+                                                              qa.group_shift, zp, zero_points, num_cu);
+                    if (e != hipSuccess)
+                        return e;
+                }
+                return hipSuccess;
+            }
+        }
         if (M <= 16)
         {
             if (M == 1)

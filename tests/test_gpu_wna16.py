@@ -62,6 +62,9 @@ SHAPES = [
     # 256 x 128, 256 x 256; tiles shared between workgroups and not; ragged M and N)
     (17, 300, 256), (40, 1000, 1024), (100, 257, 2048), (130, 4096, 4096), (700, 3000, 1280), (1100, 2050, 768),
     (1600, 520, 2560), (2000, 8192, 512), (30, 22016, 4096),
+    # 8-bit weights above 32 rows (16 at K = 8192): up to six blocks of rows through the row-streaming kernel, the last
+    # block of one, two and all rows; seven blocks: the tile kernel
+    (33, 4096, 4096), (65, 1000, 2048), (192, 520, 4096), (96, 300, 8192), (97, 300, 8192), (50, 4111, 4096),
     # enough 128 x 128 tiles to fill the chip: the larger tile kernel; ragged M and N, an odd number of groups
     (2048, 2048, 512), (1100, 4100, 160), (4096, 1030, 384),
 ]
@@ -126,11 +129,11 @@ def test_one_hot_rows_through_the_row_streaming_kernels(gpu, m, k, group, zp_ten
 
 
 @pytest.mark.parametrize("m,k", [(1, 1024), (1, 2048), (1, 2560), (1, 4096), (1, 8192), (1, 11008), (1, 16384), (16, 2048), (7, 4096),
-                                 (16, 4096), (3, 8192), (16, 8192), (20, 2048), (32, 4096)])
+                                 (16, 4096), (3, 8192), (16, 8192), (20, 2048), (32, 4096), (33, 2048), (40, 4096), (24, 8192)])
 @pytest.mark.parametrize("group,zp_tensor", [(32, True), (64, True), (128, True), (32, False), (128, False)])
 def test_one_hot_rows_through_the_row_streaming_kernels_with_8_bit_weights(gpu, m, k, group, zp_tensor):
     """8-bit weights with one row and K a multiple of 256, or 2 .. 16 rows and K = 2048 / 4096 / 8192 (up to 32 rows at
-    2048 / 4096), run on the
+    2048 / 4096, and a few blocks of that many rows one after the other), run on the
     row-streaming kernels as well (a row is K bytes, a lane meets 16 weights per load): the same pin (first and last
     weight of a group, of a lane, of a wavefront's load, of a wavefront's K segment, of a step, of the row)."""
     n = 700
