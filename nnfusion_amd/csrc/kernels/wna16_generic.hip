@@ -13,9 +13,9 @@
 //     (v_dot2_f32_f16, fp32 sums) and applies the group's scale to the sum over its piece of the group;
 //   * wna16_skinny_kernel (2 <= M <= 16): v_mfma_f32_16x16x32_f16, activations and weights fetched straight into the
 //     operand registers, eight wavefronts share the K range of two tiles of 16 weight rows;
-//   * wna16_tile_kernel / wna16_tile128_kernel (M > 16): 64 x 64 or, once they fill the chip, 128 x 128 output tiles on
-//     v_mfma_f32_32x32x16_f16, K steps of 32 through LDS, the next step's operands fetched into registers while this
-//     step's MFMAs run.
+//   * wna16_tile_kernel (M > 16): 64 x 64 or, once they fill the chip, 128 x 128 output tiles on
+//     v_mfma_f32_32x32x16_f16, K steps of 64 through two LDS buffers, the operands of the step after next on their
+//     way into registers while this step's MFMAs run.
 // The MFMA kernels dequantise to fp16((q - z) * s) (what the specialised tile GEMM's unpacking produces as well).
 #include "nnf_device.h"
 #include "nnf_launch.h"
@@ -31,29 +31,6 @@ namespace nnf
             int zp;             // scalar zero point (zps == null)
             int zp_stride;      // bytes per row of zps
         };
-
-        // eight consecutive weights of a row starting at k (a multiple of 8), as integers
-        template <int BITS>
-        __device__ __forceinline__ void load_q8(const uint8_t* __restrict__ row, int k, int (&q)[8])
-        {
-            if constexpr (BITS == 4)
-            {
-                const uint32_t w = *reinterpret_cast<const uint32_t*>(row + (k >> 1)); // nibble i = k + i
-#pragma unroll
-                for (int i = 0; i < 8; ++i)
-                    q[i] = (int)((w >> (4 * i)) & 0xFu);
-            }
-            else
-            {
-                const uintx2 w = *reinterpret_cast<const uintx2*>(row + k);
-#pragma unroll
-                for (int i = 0; i < 4; ++i)
-                {
-                    q[i] = (int)((w.x >> (8 * i)) & 0xFFu);
-                    q[4 + i] = (int)((w.y >> (8 * i)) & 0xFFu);
-                }
-            }
-        }
 
         template <int BITS>
         __device__ __forceinline__ int zero_point_of(const QuantArgs& qa, int n, int g)
@@ -314,236 +291,238 @@ namespace nnf
         }
     }
 
-    // one workgroup of four wavefronts per 64 x 64 output tile (blockIdx.x: column tile, blockIdx.y: row tile)
-    template <int BITS>
+    // Output tiles of 64 WT x 64 WT (WT = 1, or 2 for products large enough to fill the chip with 128 x 128 tiles): four
+    // wavefronts of WT x WT MFMA tiles (v_mfma_f32_32x32x16_f16), K steps of 64 through two LDS buffers, one barrier per
+    // step.  A step's operands travel global -> registers -> LDS: the activations as they are (16-byte pieces, a
+    // wavefront-wide load takes whole 128-byte lines of 8 rows), the weights dequantised on the way by the thread that
+    // fetched them -- the exact integers q - z in fp16 (offset trick) times the scale, one rounding, which is
+    // fp16((q - z) * s).  Two sets of staging registers: the loads of step s + 2 are issued ahead of the MFMAs of step s
+    // and stored behind the MFMAs of step s + 1, so a load has two steps to arrive (with one set a step lasted as long
+    // as a load from memory, half a microsecond, whatever M was).  The loads are issued and stored every step, past the
+    // end of K at clamped addresses and as zeros: a branch around them would make the compiler wait for every load in
+    // flight at the top of the loop.  Tiles are numbered in groups of four tile rows, tile row fastest, and dealt to the eight XCDs in
+    // contiguous runs, so that the workgroups in flight together share activations and weights in one L2.
+    template <int BITS, int WT>
     __global__ __launch_bounds__(256) void wna16_tile_kernel(const half_t* __restrict__ A, const uint8_t* __restrict__ Wq,
                                                              const half_t* __restrict__ S, half_t* __restrict__ Y, int M, int N,
-                                                             int K, QuantArgs qa)
+                                                             int K, int tiles_m, int tiles_n, QuantArgs qa)
     {
-        constexpr int PITCH = 40; // halves per staged row: 32 of K + 8 of padding (80 bytes: 16-byte pieces stay aligned)
-        __shared__ __attribute__((aligned(16))) half_t a_s[64 * PITCH];
-        __shared__ __attribute__((aligned(16))) half_t w_s[64 * PITCH];
-        const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-        const int m0 = (int)blockIdx.y * 64, n0 = (int)blockIdx.x * 64;
-        const int G = K >> qa.group_shift;
-        const size_t row_bytes = (size_t)K * BITS / 8;
-        // staging: thread t moves eight elements of K (piece t % 4) of row t / 4 of either operand
-        const int s_row = tid >> 2, s_k = (tid & 3) * 8;
-        const bool a_ok = m0 + s_row < M, w_ok = n0 + s_row < N;
-        const half_t* a_src = A + (size_t)min(m0 + s_row, M - 1) * K + s_k;
-        const uint8_t* w_row = Wq + (size_t)min(n0 + s_row, N - 1) * row_bytes;
-        const int w_n = min(n0 + s_row, N - 1);
-        // fragments: wavefront (wm, wn) owns rows [32 wm, +32) x columns [32 wn, +32); lane l holds eight elements of K
-        // (block l / 32 of the 16) of row / column l % 32
-        const int wm = wave >> 1, wn = wave & 1;
-        const int f_row = lane & 31, f_k = (lane >> 5) * 8;
-
-        uintx4 a_next = {0u, 0u, 0u, 0u};
-        int q_next[8];
-        float s_next = 0.f;
-        int z_next = 0;
-        auto fetch = [&](int k0) {
-            if (a_ok)
-                a_next = *reinterpret_cast<const uintx4*>(a_src + k0);
-            load_q8<BITS>(w_row, k0 + s_k, q_next);
-            const int g = (k0 + s_k) >> qa.group_shift;
-            z_next = zero_point_of<BITS>(qa, w_n, g);
-            s_next = (float)S[(size_t)w_n * G + g];
-        };
-        auto stage = [&]() {
-            *reinterpret_cast<uintx4*>(a_s + s_row * PITCH + s_k) = a_next; // rows past M stay zero
-            half8_t w;
-#pragma unroll
-            for (int i = 0; i < 8; ++i)
-                w[i] = w_ok ? (half_t)((float)(q_next[i] - z_next) * s_next) : (half_t)0.f;
-            *reinterpret_cast<half8_t*>(w_s + s_row * PITCH + s_k) = w;
-        };
-        floatx16 acc;
-#pragma unroll
-        for (int i = 0; i < 16; ++i)
-            acc[i] = 0.f;
-        fetch(0);
-        for (int k0 = 0; k0 < K; k0 += 32)
-        {
-            stage();
-            __syncthreads();
-            if (k0 + 32 < K)
-                fetch(k0 + 32);
-#pragma unroll
-            for (int kk = 0; kk < 2; ++kk)
-            {
-                const half8_t fa = *reinterpret_cast<const half8_t*>(a_s + (wm * 32 + f_row) * PITCH + kk * 16 + f_k);
-                const half8_t fw = *reinterpret_cast<const half8_t*>(w_s + (wn * 32 + f_row) * PITCH + kk * 16 + f_k);
-                acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa, fw, acc, 0, 0, 0);
-            }
-            __syncthreads();
-        }
-        // D[m][n]: lane l holds column l % 32; element i is row 8 (i / 4) + 4 (l / 32) + i % 4
-        const int n = n0 + wn * 32 + (lane & 31);
-#pragma unroll
-        for (int i = 0; i < 16; ++i)
-        {
-            const int m = m0 + wm * 32 + 8 * (i >> 2) + 4 * (lane >> 5) + (i & 3);
-            if (m < M && n < N)
-                Y[(size_t)m * N + n] = (half_t)acc[i];
-        }
-    }
-
-    // 128 x 128 output tiles for products large enough to fill the chip with them: four wavefronts of 64 x 64 (2 x 2 MFMA
-    // tiles each), K steps of 32 through two LDS buffers (the next step's operands are fetched into registers ahead of
-    // this step's MFMAs and stored behind them: one barrier per step).  A thread stages 16 activations of two rows and
-    // dequantises 16 weights of one row per step: the exact integers q - z in fp16 (offset trick) times the scale, one
-    // rounding, which is fp16((q - z) * s).  Tiles are numbered in groups of four tile rows, tile row fastest, so that
-    // the workgroups in flight together share activations and weights in the caches.
-    template <int BITS>
-    __global__ __launch_bounds__(256) void wna16_tile128_kernel(const half_t* __restrict__ A, const uint8_t* __restrict__ Wq,
-                                                                const half_t* __restrict__ S, half_t* __restrict__ Y, int M, int N,
-                                                                int K, int tiles_m, int tiles_n, QuantArgs qa)
-    {
-        constexpr int PITCH = 40;              // halves per staged row: 32 of K + 8 of padding
-        constexpr int OPERAND = 128 * PITCH;   // halves of one staged operand
-        __shared__ __attribute__((aligned(16))) half_t lds[2][2][OPERAND]; // [buffer][A, W]
+        constexpr int T = 64 * WT;        // rows and columns of the output tile
+        constexpr int KS = 64;            // values of K per step
+        constexpr int PITCH = KS + 8;     // halves per staged row (144 bytes: 16-byte pieces stay aligned)
+        constexpr int OPERAND = T * PITCH; // halves of one staged operand
+        constexpr int WPP = 128 / BITS;   // weights of a 16-byte piece (inside one group)
+        constexpr int PPR = KS / WPP;     // pieces per weight row and step
+        constexpr int A_PER = T / 32;     // pieces of activations per thread and step: piece tid % 8 of rows tid / 8 + 32 i
+        constexpr int W_PIECES = T * PPR;
+        constexpr int W_PER = (W_PIECES + 255) / 256; // pieces of weights per thread and step: piece p % PPR of row p / PPR, p = tid + 256 j
+        extern __shared__ __attribute__((aligned(16))) half_t lds[]; // [buffer][A, W][OPERAND]
         const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
         int tm, tn;
         {
-            // workgroups go to the eight XCDs in turn: XCD x takes a contiguous run of tile numbers, so that what its
-            // workgroups in flight share stays in its own L2
             constexpr int GM = 4;
             const int total = tiles_m * tiles_n, per = total / 8, rem = total % 8;
             const int xcd = (int)blockIdx.x % 8, i = (int)blockIdx.x / 8;
+            if (i >= per + (xcd < rem ? 1 : 0))
+                return; // (a grid rounded up to whole rounds of the XCDs)
             const int tile = (xcd < rem ? xcd * (per + 1) : rem * (per + 1) + (xcd - rem) * per) + i;
             const int per_group = GM * tiles_n;
             const int g = tile / per_group, first_m = g * GM, gm = min(GM, tiles_m - first_m), rr = tile - g * per_group;
             tm = first_m + rr % gm;
             tn = rr / gm;
         }
-        const int m0 = tm * 128, n0 = tn * 128;
+        const int m0 = tm * T, n0 = tn * T;
         const int G = K >> qa.group_shift;
         const size_t row_bytes = (size_t)K * BITS / 8;
-        // staging: activations: piece tid % 4 (8 halves) of rows tid / 4 and 64 + tid / 4; weights: half tid % 2 (16 of the
-        // step's 32) of row tid / 2
-        const int a_row = tid >> 2, a_k = (tid & 3) * 8;
-        const bool a_ok0 = m0 + a_row < M, a_ok1 = m0 + 64 + a_row < M;
-        const half_t* a_src0 = A + (size_t)min(m0 + a_row, M - 1) * K + a_k;
-        const half_t* a_src1 = A + (size_t)min(m0 + 64 + a_row, M - 1) * K + a_k;
-        const int w_row = tid >> 1, w_k = (tid & 1) * 16;
-        const int w_n = min(n0 + w_row, N - 1);
-        const bool w_ok = n0 + w_row < N;
-        const uint8_t* w_src = Wq + (size_t)w_n * row_bytes;
-        // fragments: wavefront (wm, wn) owns rows [64 wm, +64) x columns [64 wn, +64)
+        const int steps = (K + KS - 1) / KS;
+        const int a_row = tid >> 3, a_k = (tid & 7) * 8;
+        // fragments: wavefront (wm, wn) owns rows [32 WT wm, +32 WT) x columns [32 WT wn, +32 WT)
         const int wm = wave >> 1, wn = wave & 1;
         const int f_row = lane & 31, f_k = (lane >> 5) * 8;
 
-        uintx4 a_next0 = {0u, 0u, 0u, 0u}, a_next1 = {0u, 0u, 0u, 0u}, w_next = {0u, 0u, 0u, 0u};
-        float s_next = 0.f;
-        int z_next = 0;
-        auto fetch = [&](int k0) {
-            if (a_ok0)
-                a_next0 = *reinterpret_cast<const uintx4*>(a_src0 + k0);
-            if (a_ok1)
-                a_next1 = *reinterpret_cast<const uintx4*>(a_src1 + k0);
-            const int k = k0 + w_k;
-            if constexpr (BITS == 4)
-            {
-                const uintx2 w = *reinterpret_cast<const uintx2*>(w_src + (k >> 1));
-                w_next.x = w.x, w_next.y = w.y;
-            }
-            else
-                w_next = *reinterpret_cast<const uintx4*>(w_src + k);
-            const int g = k >> qa.group_shift;
-            z_next = zero_point_of<BITS>(qa, w_n, g);
-            s_next = w_ok ? (float)S[(size_t)w_n * G + g] : 0.f; // (columns past N: weights of zero)
+        // what a thread fetches per step, as it arrives: anything computed from it here would be waited for here
+        struct Staged
+        {
+            uintx4 a[A_PER], w[W_PER];
+            half_t s[W_PER];  // the piece's scale
+            uint8_t z[W_PER]; // the byte that holds its zero point (widened where it is used: widened here, it would be waited for here)
         };
-        auto stage = [&](int buf) {
-            *reinterpret_cast<uintx4*>(&lds[buf][0][a_row * PITCH + a_k]) = a_next0; // rows past M stay zero
-            *reinterpret_cast<uintx4*>(&lds[buf][0][(64 + a_row) * PITCH + a_k]) = a_next1;
-            const ExactWeights<BITS> exact(z_next);
-            const half_t sh = (half_t)s_next;
-            const half2_t s2 = half2_t{sh, sh};
-            uintx4 lo, hi; // the 16 weights in order of k, as fp16
-            if constexpr (BITS == 4)
-            {
-                half2_t v[4];
-                exact(w_next.x, 0u, v); // pairs (0,4) (1,5) (2,6) (3,7) -> order of k
-                for (int i = 0; i < 4; ++i)
-                    v[i] = v[i] * s2;
-                lo.x = __builtin_amdgcn_perm(as_u32(v[1]), as_u32(v[0]), 0x05040100u);
-                lo.y = __builtin_amdgcn_perm(as_u32(v[3]), as_u32(v[2]), 0x05040100u);
-                lo.z = __builtin_amdgcn_perm(as_u32(v[1]), as_u32(v[0]), 0x07060302u);
-                lo.w = __builtin_amdgcn_perm(as_u32(v[3]), as_u32(v[2]), 0x07060302u);
-                exact(w_next.y, 0u, v);
-                for (int i = 0; i < 4; ++i)
-                    v[i] = v[i] * s2;
-                hi.x = __builtin_amdgcn_perm(as_u32(v[1]), as_u32(v[0]), 0x05040100u);
-                hi.y = __builtin_amdgcn_perm(as_u32(v[3]), as_u32(v[2]), 0x05040100u);
-                hi.z = __builtin_amdgcn_perm(as_u32(v[1]), as_u32(v[0]), 0x07060302u);
-                hi.w = __builtin_amdgcn_perm(as_u32(v[3]), as_u32(v[2]), 0x07060302u);
-            }
-            else
-            {
-                half2_t v[4];
-                exact(w_next.x, w_next.y, v);
-                lo = uintx4{as_u32(v[0] * s2), as_u32(v[1] * s2), as_u32(v[2] * s2), as_u32(v[3] * s2)};
-                exact(w_next.z, w_next.w, v);
-                hi = uintx4{as_u32(v[0] * s2), as_u32(v[1] * s2), as_u32(v[2] * s2), as_u32(v[3] * s2)};
-            }
-            *reinterpret_cast<uintx4*>(&lds[buf][1][w_row * PITCH + w_k]) = lo;
-            *reinterpret_cast<uintx4*>(&lds[buf][1][w_row * PITCH + w_k + 8]) = hi;
+        // (no zero-point tensor: the byte is fetched all the same, from the scales, and not used -- a branch around the
+        // load would make the compiler wait for every load in flight behind it)
+        const uint8_t* z_base = qa.zps ? qa.zps : reinterpret_cast<const uint8_t*>(S);
+        // piece j of this thread: its weight row (clamped to N - 1), the first of its weights in step `step` (clamped to
+        // the last whole piece of the row), its group
+        auto w_piece = [&](int step, int j, int& row, int& k, int& n, int& kc, int& g) {
+            const int p = min(tid + 256 * j, W_PIECES - 1);
+            row = p / PPR;
+            k = step * KS + (p % PPR) * WPP;
+            kc = min(k, K - WPP);
+            n = min(n0 + row, N - 1);
+            g = kc >> qa.group_shift;
         };
-        floatx16 acc[2][2];
+        auto fetch = [&](int step_raw, Staged& r) {
+            const int step = min(step_raw, steps - 1);
 #pragma unroll
-        for (int i = 0; i < 2; ++i)
+            for (int i = 0; i < A_PER; ++i)
+            {
+                const int row = min(m0 + a_row + 32 * i, M - 1), k = min(step * KS + a_k, K - 8);
+                r.a[i] = *reinterpret_cast<const uintx4*>(A + (size_t)row * K + k);
+            }
 #pragma unroll
-            for (int j = 0; j < 2; ++j)
+            for (int j = 0; j < W_PER; ++j)
+            {
+                int row, k, n, kc, g;
+                w_piece(step, j, row, k, n, kc, g);
+                r.w[j] = *reinterpret_cast<const uintx4*>(Wq + (size_t)n * row_bytes + (size_t)kc * BITS / 8);
+                r.s[j] = S[(size_t)n * G + g];
+                r.z[j] = z_base[(size_t)n * qa.zp_stride + (BITS == 4 ? g >> 1 : g)];
+            }
+        };
+        auto stage = [&](int step, const Staged& r) {
+            half_t* a_s = lds + (size_t)(step & 1) * 2 * OPERAND;
+            half_t* w_s = a_s + OPERAND;
+#pragma unroll
+            for (int i = 0; i < A_PER; ++i)
+            {
+                // rows past M, a last step of 32: zeros
+                const bool real = m0 + a_row + 32 * i < M && step * KS + a_k < K;
+                *reinterpret_cast<uintx4*>(a_s + (a_row + 32 * i) * PITCH + a_k) = real ? r.a[i] : uintx4{0u, 0u, 0u, 0u};
+            }
+#pragma unroll
+            for (int j = 0; j < W_PER; ++j)
+            {
+                if (W_PIECES % 256 != 0 && tid + 256 * j >= W_PIECES)
+                    continue;
+                int row, k, n, kc, g;
+                w_piece(step, j, row, k, n, kc, g);
+                const int zt = BITS == 4 ? (int)(((uint32_t)r.z[j] >> ((g & 1) * 4)) & 15u) : (int)r.z[j];
+                const ExactWeights<BITS> exact(qa.zps ? zt : qa.zp);
+                // columns past N, a last step of 32: weights of zero
+                const half_t sh = (n0 + row < N && k < K) ? r.s[j] : (half_t)0.f;
+                const half2_t s2 = half2_t{sh, sh};
+                const uint32_t ww[4] = {r.w[j].x, r.w[j].y, r.w[j].z, r.w[j].w};
+                half_t* dst = w_s + row * PITCH + (k - step * KS);
+                if constexpr (BITS == 4)
+                {
+#pragma unroll
+                    for (int d = 0; d < 4; ++d)
+                    {
+                        half2_t v[4];
+                        exact(ww[d], 0u, v); // pairs (0,4) (1,5) (2,6) (3,7) -> order of k
+#pragma unroll
+                        for (int i = 0; i < 4; ++i)
+                            v[i] = v[i] * s2;
+                        uintx4 o;
+                        o.x = __builtin_amdgcn_perm(as_u32(v[1]), as_u32(v[0]), 0x05040100u);
+                        o.y = __builtin_amdgcn_perm(as_u32(v[3]), as_u32(v[2]), 0x05040100u);
+                        o.z = __builtin_amdgcn_perm(as_u32(v[1]), as_u32(v[0]), 0x07060302u);
+                        o.w = __builtin_amdgcn_perm(as_u32(v[3]), as_u32(v[2]), 0x07060302u);
+                        *reinterpret_cast<uintx4*>(dst + 8 * d) = o;
+                    }
+                }
+                else
+                {
+#pragma unroll
+                    for (int d = 0; d < 2; ++d)
+                    {
+                        half2_t v[4];
+                        exact(ww[2 * d], ww[2 * d + 1], v);
+                        *reinterpret_cast<uintx4*>(dst + 8 * d) =
+                            uintx4{as_u32(v[0] * s2), as_u32(v[1] * s2), as_u32(v[2] * s2), as_u32(v[3] * s2)};
+                    }
+                }
+            }
+        };
+        floatx16 acc[WT][WT];
+#pragma unroll
+        for (int i = 0; i < WT; ++i)
+#pragma unroll
+            for (int j = 0; j < WT; ++j)
 #pragma unroll
                 for (int e = 0; e < 16; ++e)
                     acc[i][j][e] = 0.f;
-        fetch(0);
-        stage(0);
-        __syncthreads();
-        int buf = 0;
-        for (int k0 = 0; k0 < K; k0 += 32)
-        {
-            const bool more = k0 + 32 < K;
-            if (more)
-                fetch(k0 + 32);
+        // step s: the loads of step s + 2 into the set step s was stored from, the MFMAs of step s, the other set (step
+        // s + 1) into the other buffer, barrier
+        auto step = [&](int s, Staged& refill, const Staged& ready) {
+            fetch(s + 2, refill);
+            // (the loads stay here, ahead of the MFMAs: moved down among them, their registers were shared with the
+            // fragments' and every load in flight was waited for at the top of the loop)
+            __builtin_amdgcn_sched_barrier(0);
+            const half_t* a_s = lds + (size_t)(s & 1) * 2 * OPERAND;
+            const half_t* w_s = a_s + OPERAND;
 #pragma unroll
-            for (int kk = 0; kk < 2; ++kk)
+            for (int kk = 0; kk < KS / 16; ++kk)
             {
-                half8_t fa[2], fw[2];
+                half8_t fa[WT], fw[WT];
 #pragma unroll
-                for (int i = 0; i < 2; ++i)
+                for (int i = 0; i < WT; ++i)
                 {
-                    fa[i] = *reinterpret_cast<const half8_t*>(&lds[buf][0][(wm * 64 + i * 32 + f_row) * PITCH + kk * 16 + f_k]);
-                    fw[i] = *reinterpret_cast<const half8_t*>(&lds[buf][1][(wn * 64 + i * 32 + f_row) * PITCH + kk * 16 + f_k]);
+                    fa[i] = *reinterpret_cast<const half8_t*>(a_s + ((wm * WT + i) * 32 + f_row) * PITCH + kk * 16 + f_k);
+                    fw[i] = *reinterpret_cast<const half8_t*>(w_s + ((wn * WT + i) * 32 + f_row) * PITCH + kk * 16 + f_k);
                 }
 #pragma unroll
-                for (int i = 0; i < 2; ++i)
+                for (int i = 0; i < WT; ++i)
 #pragma unroll
-                    for (int j = 0; j < 2; ++j)
+                    for (int j = 0; j < WT; ++j)
                         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[i], fw[j], acc[i][j], 0, 0, 0);
             }
-            if (more)
-                stage(buf ^ 1); // last read a step ago, before the barrier at its end
+            __builtin_amdgcn_sched_barrier(0);
+            stage(s + 1, ready); // its buffer was last read a step ago, before the barrier at its end
             __syncthreads();
-            buf ^= 1;
+        };
+        Staged r0, r1;
+        fetch(0, r0);
+        fetch(1, r1);
+        stage(0, r0);
+        __syncthreads();
+        // (no branch around a step or its stores either: past the end of K a step stores and multiplies zeros)
+        for (int s = 0; s < steps; s += 2)
+        {
+            step(s, r0, r1);
+            step(s + 1, r1, r0);
         }
         // D[m][n]: lane l holds column l % 32; element e is row 8 (e / 4) + 4 (l / 32) + e % 4
 #pragma unroll
-        for (int i = 0; i < 2; ++i)
+        for (int i = 0; i < WT; ++i)
 #pragma unroll
-            for (int j = 0; j < 2; ++j)
+            for (int j = 0; j < WT; ++j)
             {
-                const int n = n0 + wn * 64 + j * 32 + (lane & 31);
+                const int n = n0 + (wn * WT + j) * 32 + (lane & 31);
 #pragma unroll
                 for (int e = 0; e < 16; ++e)
                 {
-                    const int m = m0 + wm * 64 + i * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
+                    const int m = m0 + (wm * WT + i) * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
                     if (m < M && n < N)
                         Y[(size_t)m * N + n] = (half_t)acc[i][j][e];
                 }
             }
     }
+
+    namespace
+    {
+        template <int BITS, int WT>
+        hipError_t launch_wna16_tile(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M, int N, int K,
+                                     const QuantArgs& qa)
+        {
+            constexpr int T = 64 * WT;
+            constexpr int LDS = 2 * 2 * T * (64 + 8) * (int)sizeof(half_t);
+            const int tiles_m = (M + T - 1) / T, tiles_n = (N + T - 1) / T;
+            if ((long long)tiles_m * tiles_n > 0x7fffff00ll)
+                return hipErrorInvalidValue;
+            auto kernel = &wna16_tile_kernel<BITS, WT>;
+            if (LDS > 64 * 1024)
+            {
+                static LdsGrant granted;
+                const hipError_t e = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), granted, LDS);
+                if (e != hipSuccess)
+                    return e;
+            }
+            const int grid = (tiles_m * tiles_n + 7) / 8 * 8; // whole rounds of the XCDs
+            hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(256), LDS, stream, (const half_t*)A, (const uint8_t*)Wq,
+                               (const half_t*)S, (half_t*)Y, M, N, K, tiles_m, tiles_n, qa);
+            return hipGetLastError();
+        }
+    } // namespace
 
     bool wna16_supported(int M, int N, int K, int bits, int group)
     {
@@ -613,27 +592,12 @@ namespace nnf
                                    (const uint8_t*)Wq, (const half_t*)S, (half_t*)Y, M, N, K, qa);
             return hipGetLastError();
         }
+        // 128 x 128 tiles once they fill the chip, 64 x 64 below
         const int tiles_m = (M + 127) / 128, tiles_n = (N + 127) / 128;
         if ((long long)tiles_m * tiles_n >= num_cu)
-        {
-            const dim3 grid128((unsigned)(tiles_m * tiles_n));
-            if (bits == 4)
-                hipLaunchKernelGGL(wna16_tile128_kernel<4>, grid128, dim3(256), 0, stream, (const half_t*)A, (const uint8_t*)Wq,
-                                   (const half_t*)S, (half_t*)Y, M, N, K, tiles_m, tiles_n, qa);
-            else
-                hipLaunchKernelGGL(wna16_tile128_kernel<8>, grid128, dim3(256), 0, stream, (const half_t*)A, (const uint8_t*)Wq,
-                                   (const half_t*)S, (half_t*)Y, M, N, K, tiles_m, tiles_n, qa);
-            return hipGetLastError();
-        }
-        const dim3 grid((unsigned)((N + 63) / 64), (unsigned)((M + 63) / 64));
-        if (grid.y > 65535u)
-            return hipErrorInvalidValue;
-        if (bits == 4)
-            hipLaunchKernelGGL(wna16_tile_kernel<4>, grid, dim3(256), 0, stream, (const half_t*)A, (const uint8_t*)Wq,
-                               (const half_t*)S, (half_t*)Y, M, N, K, qa);
-        else
-            hipLaunchKernelGGL(wna16_tile_kernel<8>, grid, dim3(256), 0, stream, (const half_t*)A, (const uint8_t*)Wq,
-                               (const half_t*)S, (half_t*)Y, M, N, K, qa);
-        return hipGetLastError();
+            return bits == 4 ? launch_wna16_tile<4, 2>(stream, A, Wq, S, Y, M, N, K, qa)
+                             : launch_wna16_tile<8, 2>(stream, A, Wq, S, Y, M, N, K, qa);
+        return bits == 4 ? launch_wna16_tile<4, 1>(stream, A, Wq, S, Y, M, N, K, qa)
+                         : launch_wna16_tile<8, 1>(stream, A, Wq, S, Y, M, N, K, qa);
     }
 } // namespace nnf
