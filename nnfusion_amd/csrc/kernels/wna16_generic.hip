@@ -545,14 +545,15 @@ namespace nnf
         // 8-bit weights, 2 .. 16 rows at K = 2048 / 4096 / 8192 (up to 32 at 2048 / 4096): the same kernel on bytes
         if (bits == 8 && M >= 2 && w8a16_mrows_q_supported(M, N, K, qa.group_shift, zero_points != nullptr, num_cu))
             return launch_w8a16_mrows_q(stream, A, Wq, S, Y, M, N, K, qa.group_shift, zp, zero_points, num_cu);
-        // ... and up to six blocks of 32 rows (of 16 at K = 8192) one block after the other: the plain tile kernels below
-        // spend half a microsecond per 32 values of K whatever M is (N = K = 4096: 68 - 71 us from 33 to 256 rows; a block
-        // of 32 rows takes 9.6 us here), so re-reading the weights per block is the faster way up to there
+        // ... and two or three blocks of 32 rows (of 16 at K = 8192) one block after the other: re-reading the weights per
+        // block is faster than the tile kernel below up to there (N = K = 4096: 14 / 16.5 / 23.3 us at 33 / 64 / 96 rows
+        // against 31; N = K = 8192: 38 / 56 us at 32 / 48 rows against 62; level at 128 rows resp. N = 22016, behind
+        // beyond)
         if (bits == 8 && M > 16)
         {
             const int block = K == 8192 ? 16 : 32;
             const int blocks = (M + block - 1) / block;
-            if (blocks <= 6 && w8a16_mrows_q_supported(block, N, K, qa.group_shift, zero_points != nullptr, num_cu))
+            if (blocks <= (N <= 8192 ? 3 : 2) && w8a16_mrows_q_supported(block, N, K, qa.group_shift, zero_points != nullptr, num_cu))
             {
                 for (int m0 = 0; m0 < M; m0 += block)
                 {

@@ -62,9 +62,10 @@ SHAPES = [
     # 256 x 128, 256 x 256; tiles shared between workgroups and not; ragged M and N)
     (17, 300, 256), (40, 1000, 1024), (100, 257, 2048), (130, 4096, 4096), (700, 3000, 1280), (1100, 2050, 768),
     (1600, 520, 2560), (2000, 8192, 512), (30, 22016, 4096),
-    # 8-bit weights above 32 rows (16 at K = 8192): up to six blocks of rows through the row-streaming kernel, the last
-    # block of one, two and all rows; seven blocks: the tile kernel
-    (33, 4096, 4096), (65, 1000, 2048), (192, 520, 4096), (96, 300, 8192), (97, 300, 8192), (50, 4111, 4096),
+    # 8-bit weights above 32 rows (16 at K = 8192): two or three blocks of rows through the row-streaming kernel (two
+    # above N = 8192), the last block of one, two and all rows; one block more: the tile kernel
+    (33, 4096, 4096), (65, 1000, 2048), (96, 520, 4096), (97, 520, 4096), (48, 300, 8192), (49, 300, 8192), (50, 4111, 4096),
+    (64, 9000, 2048), (65, 9000, 2048),
     # enough 128 x 128 tiles to fill the chip: the larger tile kernel; ragged M and N, an odd number of groups
     (2048, 2048, 512), (1100, 4100, 160), (4096, 1030, 384),
 ]
