@@ -124,13 +124,14 @@ namespace nnf
             rp[32] = acc.z;
             rp[48] = acc.w;
             lds_barrier();
-            if (tid < M * 16)
+            // (K = 128: two wavefronts, fewer threads than the M x 16 outputs of a tile from 9 rows on)
+            for (int o = tid; o < M * 16; o += (int)blockDim.x)
             {
-                const int32_t* rr = red + buf * KS * 256 + tid;
+                const int32_t* rr = red + buf * KS * 256 + o;
                 int32_t v = 0;
                 for (int w = 0; w < KS; ++w)
                     v += rr[w * 256];
-                outb[local_tile * M * 16 + tid] = v;
+                outb[local_tile * M * 16 + o] = v;
             }
             buf ^= 1;
             ++local_tile;

@@ -920,10 +920,18 @@ namespace nnf
         // nnf_w4a16_gemm_fused: [ RMSNorm scratch ][ partial sums ], whichever of the optional parts the call uses
         inline size_t w4a16_gemm_fused(int M, int N, int K, int, int act, int num_cu = PLAN_CUS)
         {
+            // (with and without the RMSNorm prologue, with the residual in place or not: the routes differ -- 8 .. 16 rows
+            // at K = 8192 run over two ranges of K only without the prologue)
             const bool gate = act == 1;
-            const W4A16Route a = route_w4a16(M, N, K, gate, true, false, num_cu);
-            const W4A16Route b = route_w4a16(M, N, K, gate, true, !gate, num_cu);
-            return a.rms_bytes + (a.partial_bytes > b.partial_bytes ? a.partial_bytes : b.partial_bytes);
+            size_t most = 0;
+            for (int rms = 0; rms < 2; ++rms)
+                for (int in_place = 0; in_place < (gate ? 1 : 2); ++in_place)
+                {
+                    const W4A16Route r = route_w4a16(M, N, K, gate, rms != 0, in_place != 0, num_cu);
+                    const size_t bytes = r.rms_bytes + r.partial_bytes;
+                    most = bytes > most ? bytes : most;
+                }
+            return most;
         }
         // nnf_fused_mlp_w4a16: [ RMSNorm scratch of the first product ][ h: M x I fp16 ][ partial sums of either product ]
         inline size_t fused_mlp_h_offset(int M, int H, int I, int num_cu = PLAN_CUS)

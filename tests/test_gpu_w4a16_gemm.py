@@ -420,3 +420,35 @@ def test_fused_parts_with_few_rows(gpu, variant, m, n, k):
         err = np.abs(yg.astype(np.float32) - ref.astype(np.float32))
         assert np.all(err <= bound), float((err - bound).max())
     torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("m,n,k", [(11, 981, 8192), (16, 4096, 8192), (8, 300, 8192), (12, 9000, 8192), (24, 304, 8192),
+                                   (8, 1000, 11008), (3, 520, 4096), (200, 300, 1024), (1, 4096, 4096), (16, 48, 2304)])
+def test_fused_parts_in_the_workspace_the_query_asks_for(gpu, m, n, k):
+    """nnf_w4a16_gemm_fused_workspace_bytes does not know which of the optional parts a call will use, and the kernels
+    that serve them differ (8 .. 16 rows at K = 8192 run over two ranges of K without the RMSNorm prologue, in one launch
+    with it): a workspace of exactly that size serves every combination."""
+    import torch
+
+    from nnfusion_amd import ops
+
+    a, wq, s = datagen.w4a16_case(23, m, 2 * n, k)
+    bias = datagen.normal_f16(23, datagen.S_BIAS, (n,))
+    res = datagen.normal_f16(23, datagen.S_RES, (m, n))
+    gamma = datagen.normal_f16(23, datagen.S_GAMMA, (k,), 1.0, 0.1)
+    ta, tw, ts, tb, tr, tg = _t(gpu, a, wq, s, bias, res, gamma)
+    tw1, ts1 = tw[:n].contiguous(), ts[:n].contiguous()
+    d = oracle.w4a16_gemm(a, wq[:n], s[:n])
+    ref_b = oracle.add_f16(d, np.broadcast_to(bias, (m, n)).copy())
+    _check(ops.w4a16_gemm_fused(ta, tw1, ts1, bias=tb).cpu().numpy(), ref_b)
+    _check(ops.w4a16_gemm_fused(ta, tw1, ts1, residual=tr).cpu().numpy(), oracle.add_f16(d, res))
+    out = tr.clone()
+    _check(ops.w4a16_gemm_fused(ta, tw1, ts1, bias=tb, residual=out, out=out).cpu().numpy(), oracle.add_f16(ref_b, res))
+    xn = oracle.rmsnorm_f16(a, gamma, 1e-6)
+    _check(ops.w4a16_gemm_fused(ta, tw1, ts1, rms_gamma=tg, rms_eps=1e-6).cpu().numpy(),
+           oracle.w4a16_gemm(xn, wq[:n], s[:n], f32_out=True))
+    dn = oracle.w4a16_gemm(xn, wq[:n], s[:n])
+    _check(ops.w4a16_gemm_fused(ta, tw1, ts1, rms_gamma=tg, rms_eps=1e-6, residual=tr).cpu().numpy(), oracle.add_f16(dn, res))
+    assert ops.w4a16_gemm_fused(ta, tw, ts, act=1).shape == (m, n)
+    assert ops.w4a16_gemm_fused(ta, tw, ts, act=1, rms_gamma=tg, rms_eps=1e-6).shape == (m, n)
+    torch.cuda.synchronize()

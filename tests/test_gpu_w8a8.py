@@ -60,6 +60,8 @@ def _big_ws(gpu):
     (256, 256, 128), (512, 1024, 2048), (1, 8192, 8192), (32, 4096, 4096),
     # M <= 16 with chunk counts that leave wavefronts partly idle, two passes over K per tile, many tiles
     (5, 200, 2176), (2, 100, 11008), (7, 48, 16384), (9, 1000, 8320), (1, 33000, 1024), (13, 8200, 4096),
+    # ... and with K so short that the workgroup has fewer threads than a tile has outputs (two wavefronts, 9 .. 16 rows)
+    (14, 4128, 128), (9, 100, 128), (16, 300, 128), (13, 64, 128), (8, 520, 128), (12, 1000, 128),
     # one activation row: rows shared by 1..8 wavefronts, ragged last K segment, fewer rows than wavefronts
     (1, 300, 4096), (1, 4096, 11008), (1, 100, 16384), (1, 50, 2048), (1, 513, 5248), (1, 2000, 24576), (1, 40, 1152),
     # 2 .. 32 rows through the row-streaming MFMA kernel: every K it takes, one and two blocks of 16 rows, ragged N,
