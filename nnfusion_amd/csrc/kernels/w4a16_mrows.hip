@@ -375,13 +375,12 @@ namespace nnf
 #pragma unroll
                     for (int j = 0; j < 4; ++j)
                     {
+                        // (v_dot2_f32_f16: one instruction per pair; with conversions and multiplies of its own the sum took
+                        // more than a microsecond of a SIMD's vector unit at 16 rows x 4096)
                         const uint32_t rr[4] = {areg[mb][g][j].x, areg[mb][g][j].y, areg[mb][g][j].z, areg[mb][g][j].w};
 #pragma unroll
                         for (int i = 0; i < 4; ++i)
-                        {
-                            const half2_t hh = as_half2(rr[i]);
-                            ss += (float)hh.x * (float)hh.x + (float)hh.y * (float)hh.y;
-                        }
+                            ss = dot2(as_half2(rr[i]), as_half2(rr[i]), ss);
                     }
                 ss += __shfl_xor(ss, 16, 64);
                 ss += __shfl_xor(ss, 32, 64);
@@ -1369,6 +1368,13 @@ namespace nnf
                     if (nn < (t0 + it) * 16) // (a last tile moved back: these columns belong to the tile before it)
                         continue;
                     const size_t at = (size_t)m * N + nn;
+                    // (bias and residual requested ahead of the ranges' sums: behind them, they were one more round trip)
+                    half_t bias_n = (half_t)0.f, residual_at = (half_t)0.f;
+                    if constexpr (FUSED)
+                    {
+                        bias_n = f.bias ? f.bias[nn] : (half_t)0.f;
+                        residual_at = f.residual ? f.residual[at] : (half_t)0.f;
+                    }
                     // (four ranges in flight, added in order)
                     float sum = 0.f;
                     for (int r0 = 0; r0 < ranges; r0 += 4)
@@ -1384,7 +1390,15 @@ namespace nnf
                                 sum += part[d];
                     }
                     if (FUSED)
-                        Y[at] = finish_bias_residual(f32_product(sum, f.rstd ? f.rstd[m] : 1.0f), f.bias, nn, f.residual, at);
+                    {
+                        // y = fp16(sum) (+ bias) (+ residual), each step rounded to fp16 (finish_bias_residual)
+                        half_t y = (half_t)f32_product(sum, f.rstd ? f.rstd[m] : 1.0f);
+                        if (f.bias)
+                            y = (half_t)((float)y + (float)bias_n);
+                        if (f.residual)
+                            y = (half_t)((float)y + (float)residual_at);
+                        Y[at] = y;
+                    }
                     else
                         Y[at] = (half_t)sum;
                 }
