@@ -229,14 +229,14 @@ namespace nnf
     // K = GW * STEPS * 1024; MB = blocks of 16 activation rows (1 or 2).
     // LDS (bytes): weights [8 wavefronts][2 slots][GW KiB] | scales [8][2][256] | partial tiles [2][8][MB KiB] |
     //              parked sums [tiles of the workgroup][M][16] fp32
-    // pack = M | zp << 8;  a workgroup's output tiles: tiles_q, one more for the first tiles_r workgroups.
+    // pack = M | zp << 8 | gate << 16;  a workgroup's output tiles: tiles_q, one more for the first tiles_r workgroups.
     // FUSED: the prologue / epilogue of `f`; gate != 0: N outputs from 2 N weight rows, the workgroup walks the gate and
     // the up tile of each of its output tiles in turn (twice the tiles).
     // STAGE: the activations through LDS as whole lines (row_block_fetch); otherwise straight into the registers
     template <int GW, int STEPS, int MB, bool FUSED, bool STAGE>
     __global__ __launch_bounds__(512) void w4a16_mrows_kernel(const half_t* __restrict__ A, const uint8_t* __restrict__ Wq,
                                                               const half_t* __restrict__ S, half_t* __restrict__ Y, int N,
-                                                              int tiles_q, int tiles_r, int pack, GemvFusionArgs f, int gate)
+                                                              int tiles_q, int tiles_r, int pack, GemvFusionArgs f)
     {
         static_assert(GW >= 1 && GW <= 8 && STEPS >= 1 && GW * STEPS <= 8, "K = GW * STEPS * 1024");
         static_assert(MB == 1 || (MB == 2 && GW * STEPS <= 4), "two blocks of rows: 32 VGPRs per group");
@@ -260,7 +260,9 @@ namespace nnf
         const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
         const int col = lane & 15; // n within the tile (B operand / D column), m for the A operand
         const int kq = lane >> 4;  // K quarter of the MFMA operands, row quad of D
-        const int M = pack & 0xff, zp = (pack >> 8) & 0xff;
+        // (gate rides in `pack`, among the arguments that arrive in scalar registers with the wavefront: as an argument of
+        // its own behind `f` it was loaded from memory and waited for ahead of the first weight load)
+        const int M = pack & 0xff, zp = (pack >> 8) & 0xff, gate = (pack >> 16) & 1;
         const int b = blockIdx.x;
         const int t0 = b * tiles_q + min(b, tiles_r);
         const int T_out = tiles_q + (b < tiles_r ? 1 : 0);
@@ -1153,9 +1155,8 @@ namespace nnf
     template <int GW, int STEPS, int MB, bool FUSED, bool STAGE>
     __global__ __launch_bounds__(512) void w4a16_mrows_any_kernel(const half_t* __restrict__ A, const uint8_t* __restrict__ Wq,
                                                                   const half_t* __restrict__ S, half_t* __restrict__ Y,
-                                                                  float* __restrict__ partial, int N, int K, int range_groups,
-                                                                  int tiles_q, int tiles_r, int pack, GemvFusionArgs f, int gate,
-                                                                  uint32_t* sync)
+                                                                  float* __restrict__ partial, int N, int K, int tiles,
+                                                                  int pack, GemvFusionArgs f, uint32_t* sync)
     {
         static_assert(GW >= 1 && GW <= 7 && STEPS >= 1 && GW * STEPS <= 8, "groups per wavefront");
         static_assert(MB == 1 || (MB == 2 && GW * STEPS <= 4) || (MB == 4 && GW * STEPS <= 2), "16 VGPRs per group and block of rows");
@@ -1176,7 +1177,11 @@ namespace nnf
         const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
         const int col = lane & 15;
         const int kq = lane >> 4;
-        const int M = pack & 0xff, zp = (pack >> 8) & 0xff;
+        // (fourteen dwords of arguments arrive in scalar registers with the wavefront: everything the first weight load
+        // needs is among them -- tiles = tiles_q | tiles_r << 16, pack = M | zp << 8 | gate << 16 | range_groups << 17;
+        // with more, the kernel began by waiting for a load of its own arguments)
+        const int M = pack & 0xff, zp = (pack >> 8) & 0xff, gate = (pack >> 16) & 1, range_groups = (int)((unsigned)pack >> 17);
+        const int tiles_q = tiles & 0xffff, tiles_r = (int)((unsigned)tiles >> 16);
         const int G = K >> 7, ROW_BYTES = K >> 1;
         const int b = blockIdx.x;
         const int t0 = b * tiles_q + min(b, tiles_r);
@@ -1439,8 +1444,8 @@ namespace nnf
                     return e;
             }
             hipLaunchKernelGGL(kernel, dim3(grid), dim3(MR_WAVES * 64), lds, stream, (const half_t*)A, (const uint8_t*)Wq,
-                               (const half_t*)S, (half_t*)Y, N, tiles_q, tiles_r, M | (zp << 8), fusion_args(fusion),
-                               fusion.gate ? 1 : 0);
+                               (const half_t*)S, (half_t*)Y, N, tiles_q, tiles_r, M | (zp << 8) | (fusion.gate ? 1 << 16 : 0),
+                               fusion_args(fusion));
             return hipGetLastError();
         }
 
@@ -1486,9 +1491,12 @@ namespace nnf
                 if (e != hipSuccess)
                     return e;
             }
+            if (tiles_q > 0xffff || tiles_r > 0xffff || range_groups > 0x7fff)
+                return hipErrorInvalidValue;
             hipLaunchKernelGGL(kernel, dim3(grid, ranges), dim3(MR_WAVES * 64), lds, stream, (const half_t*)A, (const uint8_t*)Wq,
-                               (const half_t*)S, (half_t*)Y, ranges > 1 ? partial : nullptr, N, K, range_groups, tiles_q, tiles_r,
-                               M | (zp << 8), fusion_args(fusion), fusion.gate ? 1 : 0, ranges > 1 ? sync : nullptr);
+                               (const half_t*)S, (half_t*)Y, ranges > 1 ? partial : nullptr, N, K, tiles_q | (tiles_r << 16),
+                               M | (zp << 8) | (fusion.gate ? 1 << 16 : 0) | (range_groups << 17), fusion_args(fusion),
+                               ranges > 1 ? sync : nullptr);
             return hipGetLastError();
         }
 
