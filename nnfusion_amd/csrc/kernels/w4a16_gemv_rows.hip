@@ -44,15 +44,20 @@ namespace nnf
     {
         gemv_rows_body<SEG, D, WAVES, 0>(A, Wq, S, Y, N, K, rows_q, rows_r, pack, GemvFusionArgs{nullptr, nullptr, nullptr, nullptr, 0.f});
     }
+    // (the RMSNorm weight's pointer, which the kernel needs for its first loads, as an argument of its own ahead of `f`,
+    // and K in the top byte of `pack`, in units of 256: fourteen dwords of scalar arguments arrive in registers with the
+    // wavefront, a structure passed by value does not)
     template <int SEG, int D, int WAVES, int EPI>
     __global__ __launch_bounds__(WAVES * 64) void w4a16_gemv_rows_fused_kernel(const half_t* __restrict__ A,
                                                                                const uint8_t* __restrict__ Wq,
                                                                                const half_t* __restrict__ S,
-                                                                               half_t* __restrict__ Y, int N, int K,
-                                                                               int rows_q, int rows_r, int pack, GemvFusionArgs f)
+                                                                               half_t* __restrict__ Y, int N, int rows_q,
+                                                                               int rows_r, int pack, const half_t* gamma,
+                                                                               GemvFusionArgs f)
     {
         static_assert(EPI == 1 || EPI == 2, "the plain kernel is w4a16_gemv_rows_kernel");
-        gemv_rows_body<SEG, D, WAVES, EPI>(A, Wq, S, Y, N, K, rows_q, rows_r, pack, f);
+        const GemvFusionArgs g = {gamma, f.rstd, f.bias, f.residual, f.rms_eps};
+        gemv_rows_body<SEG, D, WAVES, EPI>(A, Wq, S, Y, N, (int)((unsigned)pack >> 24) << 8, rows_q, rows_r, pack & 0xffffff, g);
     }
 
     // Other block parameters (EPI 4: group size; 3: a zero point per (row, group) as well; BITS: 4 or 8).  Sixteen dwords
@@ -121,8 +126,8 @@ namespace nnf
                                    zp | (p.kshift << 8));
             else
                 hipLaunchKernelGGL((w4a16_gemv_rows_fused_kernel<SEG, D, WAVES, EPI>), dim3(grid), dim3(WAVES * 64), lds_total,
-                                   stream, (const half_t*)A, (const uint8_t*)Wq, (const half_t*)S, (half_t*)Y, N, K, N / grid,
-                                   N % grid, zp | (p.kshift << 8), f);
+                                   stream, (const half_t*)A, (const uint8_t*)Wq, (const half_t*)S, (half_t*)Y, N, N / grid,
+                                   N % grid, zp | (p.kshift << 8) | ((K >> 8) << 24), f.gamma, f); // (K: a multiple of 256 up to 16384)
             return hipGetLastError();
         }
     } // namespace
