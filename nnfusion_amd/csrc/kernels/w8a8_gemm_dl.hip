@@ -66,8 +66,20 @@ namespace nnf
     } // namespace q8dl
 
     template <int WM, int WN, int TM, int TN, int STAGES, bool RAW, bool SPLITK, int MINW, int BK = 64>
-    __global__ __launch_bounds__(WM * WN * 64, MINW) void w8a8_gemm_dl_kernel(Q8GemmParams p)
+    __global__ __launch_bounds__(WM * WN * 64, MINW) void w8a8_gemm_dl_kernel(const int8_t* __restrict__ A_first,
+                                                                              const int8_t* __restrict__ W_first, int M_first,
+                                                                              int N_first, int K_first, int splits_first,
+                                                                              Q8GemmParams p_rest)
     {
+        // (what the first loads need, once more as arguments of their own: scalar arguments arrive in registers with the
+        // wavefront, a structure passed by value is loaded from memory -- the kernel began by waiting for it)
+        Q8GemmParams p = p_rest;
+        p.A = A_first;
+        p.W = W_first;
+        p.M = M_first;
+        p.N = N_first;
+        p.K = K_first;
+        p.splits = splits_first;
         using namespace q8dl;
         using T = Tile<WM, WN, TM, TN, STAGES, BK>;
         constexpr int BM = T::BM, BN = T::BN, NSUB = T::NSUB, RPL = T::ROWS_PER_LOAD;
@@ -515,7 +527,8 @@ namespace nnf
                     return e;
             }
             const int splits = SPLITK ? p.splits : 1;
-            hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n * splits), dim3(T::THREADS), T::LDS_BYTES, stream, p);
+            hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n * splits), dim3(T::THREADS), T::LDS_BYTES, stream, p.A, p.W, p.M, p.N,
+                               p.K, p.splits, p);
             return hipGetLastError();
         }
 

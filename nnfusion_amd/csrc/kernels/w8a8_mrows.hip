@@ -48,11 +48,13 @@ namespace nnf
     // STEPS = ceil(K / 2048) (steps per tile and wavefront), MB = blocks of 16 activation rows (1 or 2), NS = ring slots.
     // A workgroup's tiles: tiles_q, one more for the first tiles_r workgroups.
     template <int STEPS, int MB, int NS, bool RAW_ACC>
-    __global__ __launch_bounds__(512) void w8a8_mrows_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ W,
+    // (the arguments the first loads need come first: fourteen dwords arrive in scalar registers with the wavefront, the
+    // rest -- what the epilogue needs -- is loaded from memory while the weights are on their way)
+    __global__ __launch_bounds__(512) void w8a8_mrows_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ W, int M,
+                                                             int N, int K, int tiles_q, int tiles_r, int ld,
                                                              const float* __restrict__ s_tok, const float* __restrict__ s_ch,
-                                                             half_t* __restrict__ Y, int32_t* __restrict__ ACC, int M, int N,
-                                                             int K, int tiles_q, int tiles_r, int ld, int32_t* __restrict__ part,
-                                                             uint32_t* __restrict__ sync)
+                                                             half_t* __restrict__ Y, int32_t* __restrict__ ACC,
+                                                             int32_t* __restrict__ part, uint32_t* __restrict__ sync)
     {
         // K: the length of this workgroup's range of K, which starts at byte blockIdx.y * K of a row of ld bytes (one range:
         // ld = K, part = null).  Ranges: the sums of range r go to part + r * M * N, and the last workgroup of a
@@ -324,8 +326,8 @@ namespace nnf
                     return e;
             }
             hipLaunchKernelGGL(kernel, dim3(grid, ranges), dim3(Q8MR_WAVES * 64), lds, stream, (const int8_t*)A, (const int8_t*)W,
-                               (const float*)s_tok, (const float*)s_ch, (half_t*)Y, (int32_t*)acc, M, N, K, tiles_q, tiles_r,
-                               ld ? ld : K, (int32_t*)part, sync);
+                               M, N, K, tiles_q, tiles_r, ld ? ld : K, (const float*)s_tok, (const float*)s_ch, (half_t*)Y,
+                               (int32_t*)acc, (int32_t*)part, sync);
             return hipGetLastError();
         }
 
