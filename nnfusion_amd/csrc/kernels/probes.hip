@@ -352,7 +352,7 @@ extern "C" int nnf_probe_gemm_timeline(void* stream, const void* A, const void* 
         auto kernel = &w4a16_gemm_sk_kernel<4, 1, false, false, false, false>;
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, T::LDS_BYTES) != hipSuccess)
             return -1;
-        hipLaunchKernelGGL(kernel, dim3(plan.grid), dim3(gemm_sk::THREADS), T::LDS_BYTES, (hipStream_t)stream, p);
+        launch_sk_kernel(kernel, plan.grid, T::LDS_BYTES, (hipStream_t)stream, p);
     }
     else
     {
@@ -360,7 +360,7 @@ extern "C" int nnf_probe_gemm_timeline(void* stream, const void* A, const void* 
         auto kernel = &w4a16_gemm_sk_kernel<4, 2, false, false, false, false>;
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, T::LDS_BYTES) != hipSuccess)
             return -1;
-        hipLaunchKernelGGL(kernel, dim3(plan.grid), dim3(gemm_sk::THREADS), T::LDS_BYTES, (hipStream_t)stream, p);
+        launch_sk_kernel(kernel, plan.grid, T::LDS_BYTES, (hipStream_t)stream, p);
     }
     return hipGetLastError() == hipSuccess ? plan.grid : -1;
 }

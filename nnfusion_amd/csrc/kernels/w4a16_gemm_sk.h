@@ -566,8 +566,25 @@ namespace nnf
     // hold their zero points in another (1, 2 or 4 bytes; without p.zps: the scales again, unused) -- six loads per
     // column tile as for QG = 0, on the same schedule -- and keeps a scale and the pair -(1024 + z), -(64 + z) per K step.
     template <int TM, int TN, bool GATE, bool BIAS, bool RESID, bool RMS, int QG = 0>
-    __global__ __launch_bounds__(256, 1) void w4a16_gemm_sk_kernel(SkGemmParams p)
+    __global__ __launch_bounds__(256, 1) void w4a16_gemm_sk_kernel(const half_t* __restrict__ A_first,
+                                                                   const uint8_t* __restrict__ Wq_first,
+                                                                   const half_t* __restrict__ S_first, long long units_first,
+                                                                   int M_first, int N_first, int K_first, int tiles_n_first,
+                                                                   int supersteps_first, int grid_first, SkGemmParams p_rest)
     {
+        // (what the first loads need, once more as arguments of their own -- launch_sk_kernel passes them: fourteen dwords
+        // of scalar arguments arrive in registers with the wavefront, a structure passed by value and the size of the
+        // grid are loaded from memory, and the kernel began by waiting for them)
+        SkGemmParams p = p_rest;
+        p.A = A_first;
+        p.Wq = Wq_first;
+        p.S = S_first;
+        p.units = units_first;
+        p.M = M_first;
+        p.N = N_first;
+        p.K = K_first;
+        p.tiles_n = tiles_n_first;
+        p.supersteps = supersteps_first;
         using namespace gemm_sk;
         using T = Tile<TM, TN>;
         // loads per column tile and superstep: four of weights; two of scales and zero points, or (the specialised kernel)
@@ -604,7 +621,7 @@ namespace nnf
         const int G = K >> GSH;
         const bool g_even = !(G & 1);
         const int SS = p.supersteps;
-        const int grid = (int)gridDim.x;
+        const int grid = grid_first; // = gridDim.x
         const uint32_t lds0 = lds_address(smem);
 
         // workgroup ids are dealt round-robin to the 8 XCDs: number the workgroups so that an XCD (own L2) holds a
@@ -1414,6 +1431,14 @@ namespace nnf
             }
         }
         NNF_SK_STAMP(9); // done
+    }
+
+    // launches w4a16_gemm_sk_kernel<...> on `grid` workgroups
+    template <class Kernel>
+    inline void launch_sk_kernel(Kernel kernel, int grid, size_t lds_bytes, hipStream_t stream, const SkGemmParams& p)
+    {
+        hipLaunchKernelGGL(kernel, dim3(grid), dim3(gemm_sk::THREADS), lds_bytes, stream, p.A, p.Wq, p.S, p.units, p.M, p.N, p.K,
+                           p.tiles_n, p.supersteps, grid, p);
     }
 
     // Adds the parts of the tiles that several workgroups of w4a16_gemm_sk_kernel worked on, in K order (so the result

@@ -21,7 +21,7 @@ namespace nnf
                 if (e != hipSuccess)
                     return e;
             }
-            hipLaunchKernelGGL(kernel, dim3(grid), dim3(THREADS), T::LDS_BYTES, stream, p);
+            launch_sk_kernel(kernel, grid, T::LDS_BYTES, stream, p);
             hipError_t e = hipGetLastError();
             if (e != hipSuccess || !p.partial || p.sync)
                 return e;
@@ -83,7 +83,7 @@ namespace nnf
                 if (e != hipSuccess)
                     return e;
             }
-            hipLaunchKernelGGL(kernel, dim3(grid), dim3(THREADS), T::LDS_BYTES, stream, p);
+            launch_sk_kernel(kernel, grid, T::LDS_BYTES, stream, p);
             hipError_t e = hipGetLastError();
             if (e != hipSuccess || !p.partial || p.sync)
                 return e;
