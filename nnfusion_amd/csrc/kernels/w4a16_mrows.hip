@@ -241,6 +241,7 @@ namespace nnf
         static_assert(GW >= 1 && GW <= 8 && STEPS >= 1 && GW * STEPS <= 8, "K = GW * STEPS * 1024");
         static_assert(MB == 1 || (MB == 2 && GW * STEPS <= 4), "two blocks of rows: 32 VGPRs per group");
         constexpr int K = GW * STEPS * 1024, G = K / 128;
+        constexpr int GAMMA_LOADS = (GW * STEPS + 3) / 4; // of the RMSNorm weight into LDS: 1 KiB, four groups, each
         constexpr int GA = GW * STEPS;         // groups of a wavefront
         constexpr int ROW_BYTES = K / 2;       // a weight row
         constexpr int SLICE = GW * 64;         // a wavefront's bytes of a weight row per step
@@ -355,23 +356,39 @@ namespace nnf
                     fetch(p + 1);
                     __builtin_amdgcn_s_waitcnt(vmcnt_only(4));
                 }
+                else if (FUSED && f.gamma)
+                {
+                    // The RMSNorm weight of the wavefront's k positions (GA x 256 bytes) follows the last block into the
+                    // free half, one load per four groups: as sixteen 16-byte loads per lane straight into registers --
+                    // the sixteen lanes of a column asking for the same bytes -- it took the load pipeline a microsecond
+                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+                    for (int i = 0; i < GAMMA_LOADS; ++i)
+                    {
+                        const int g = min(4 * i + (lane >> 4), GA - 1);
+                        const uint8_t* src = reinterpret_cast<const uint8_t*>(f.gamma) + wave * (GW * 256) + (g / GW) * (SPAN * 4) +
+                                             (g % GW) * 256 + (lane & 15) * 16;
+                        __builtin_amdgcn_global_load_lds((mr_global_ptr_t)src, (mr_lds_ptr_t)(stage + (NP & 1) * ROW_BLOCK_BYTES + i * 1024),
+                                                         16, 0, 0);
+                    }
+                    __builtin_amdgcn_s_waitcnt(vmcnt_only(GAMMA_LOADS));
+                }
                 else
                     __builtin_amdgcn_s_waitcnt(vmcnt_only(0));
 #pragma unroll
                 for (int j = 0; j < 4; ++j)
                     areg[p / GA][p % GA][j] = row_block_piece(stage + (p & 1) * ROW_BLOCK_BYTES, col, kq * 4 + j);
             }
-            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-            __syncthreads();
         }
         // RMSNorm without a pass of its own: the wavefront's share of sum a^2 of every row, from the registers
         const bool own_rstd = FUSED && f.gamma && !f.rstd;
+        float ss[MB];
         if (own_rstd)
         {
 #pragma unroll
             for (int mb = 0; mb < MB; ++mb)
             {
-                float ss = 0.f;
+                ss[mb] = 0.f;
 #pragma unroll
                 for (int g = 0; g < GA; ++g)
 #pragma unroll
@@ -382,18 +399,34 @@ namespace nnf
                         const uint32_t rr[4] = {areg[mb][g][j].x, areg[mb][g][j].y, areg[mb][g][j].z, areg[mb][g][j].w};
 #pragma unroll
                         for (int i = 0; i < 4; ++i)
-                            ss = dot2(as_half2(rr[i]), as_half2(rr[i]), ss);
+                            ss[mb] = dot2(as_half2(rr[i]), as_half2(rr[i]), ss[mb]);
                     }
-                ss += __shfl_xor(ss, 16, 64);
-                ss += __shfl_xor(ss, 32, 64);
-                if (kq == 0)
-                    sum_sq[wave * (MB * 16) + mb * 16 + col] = ss;
+                ss[mb] += __shfl_xor(ss[mb], 16, 64);
+                ss[mb] += __shfl_xor(ss[mb], 32, 64);
             }
         }
-        if (FUSED && f.gamma)
+        if constexpr (STAGE)
+        {
+            if (FUSED && f.gamma)
+            {
+                const uint8_t* gamma_block = red + wave * (2 * ROW_BLOCK_BYTES) + ((MB * GA) & 1) * ROW_BLOCK_BYTES;
+                __builtin_amdgcn_s_waitcnt(vmcnt_only(0));
+                mrows_scale_a<MB, GA>(areg, [&](int g) { return gamma_block + g * 256 + kq * 64; });
+            }
+            // (the blocks lay over what holds the partial tiles, the sums of squares and the parked sums from here on)
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            __syncthreads();
+        }
+        else if (FUSED && f.gamma)
             mrows_scale_a<MB, GA>(areg, [&](int g) {
                 return reinterpret_cast<const uint8_t*>(f.gamma) + wave * (GW * 256) + kq * 64 + (g / GW) * (SPAN * 4) + (g % GW) * 256;
             });
+        if (own_rstd && kq == 0)
+        {
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb)
+                sum_sq[wave * (MB * 16) + mb * 16 + col] = ss[mb];
+        }
         floatx4 ncorr[MB][GA];
         mrows_prepare_a<MB, GA>(areg, ncorr, zp);
 
