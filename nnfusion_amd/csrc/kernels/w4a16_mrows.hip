@@ -1406,12 +1406,17 @@ namespace nnf
                     if (nn < (t0 + it) * 16) // (a last tile moved back: these columns belong to the tile before it)
                         continue;
                     const size_t at = (size_t)m * N + nn;
-                    // (bias and residual requested ahead of the ranges' sums: behind them, they were one more round trip)
+                    // (rstd, bias and residual are requested ahead of the ranges' sums and without a branch around the loads --
+                    // an absent one reads a word of the sums instead, unused: asked for where they are added, or under a
+                    // branch, each was a round trip of its own at the very end of the kernel)
                     half_t bias_n = (half_t)0.f, residual_at = (half_t)0.f;
+                    float rstd_m = 1.0f;
                     if constexpr (FUSED)
                     {
-                        bias_n = f.bias ? f.bias[nn] : (half_t)0.f;
-                        residual_at = f.residual ? f.residual[at] : (half_t)0.f;
+                        const half_t* spare = reinterpret_cast<const half_t*>(partial);
+                        bias_n = *(f.bias ? f.bias + nn : spare);
+                        residual_at = *(f.residual ? f.residual + at : spare);
+                        rstd_m = *(f.rstd ? f.rstd + m : reinterpret_cast<const float*>(partial));
                     }
                     // (four ranges in flight, added in order)
                     float sum = 0.f;
@@ -1430,7 +1435,7 @@ namespace nnf
                     if (FUSED)
                     {
                         // y = fp16(sum) (+ bias) (+ residual), each step rounded to fp16 (finish_bias_residual)
-                        half_t y = (half_t)f32_product(sum, f.rstd ? f.rstd[m] : 1.0f);
+                        half_t y = (half_t)f32_product(sum, f.rstd ? rstd_m : 1.0f);
                         if (f.bias)
                             y = (half_t)((float)y + (float)bias_n);
                         if (f.residual)
