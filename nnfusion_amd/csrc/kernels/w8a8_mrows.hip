@@ -264,6 +264,13 @@ namespace nnf
                 if (gn < (t0 + it) * 16) // (a last tile moved back: these columns belong to the tile before it)
                     continue;
                 const size_t at = (size_t)m * N + gn;
+                // (the two scales requested ahead of the ranges' sums: behind them, they were one more round trip)
+                float st = 1.0f, sc = 1.0f;
+                if constexpr (!RAW_ACC)
+                {
+                    st = s_tok[m];
+                    sc = s_ch[gn];
+                }
                 int32_t sum = 0;
                 for (int r0 = 0; r0 < ranges; r0 += 4)
                 {
@@ -278,7 +285,7 @@ namespace nnf
                 if (RAW_ACC)
                     ACC[at] = sum;
                 else
-                    Y[at] = f32_to_f16_two_step((float)sum * s_tok[m] * s_ch[gn]);
+                    Y[at] = f32_to_f16_two_step((float)sum * st * sc);
             }
             if (tid == 0)
                 atomicExch(sync + blockIdx.x, 0u);
