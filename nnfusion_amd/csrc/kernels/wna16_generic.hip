@@ -13,9 +13,9 @@
 //     (v_dot2_f32_f16, fp32 sums) and applies the group's scale to the sum over its piece of the group;
 //   * wna16_skinny_kernel (2 <= M <= 16): v_mfma_f32_16x16x32_f16, activations and weights fetched straight into the
 //     operand registers, eight wavefronts share the K range of two tiles of 16 weight rows;
-//   * wna16_tile_kernel (M > 16): 64 x 64 or, once they fill the chip, 128 x 128 output tiles on
-//     v_mfma_f32_32x32x16_f16, K steps of 64 through two LDS buffers, the operands of the step after next on their
-//     way into registers while this step's MFMAs run.
+//   * wna16_tile_kernel (M > 16): 64 x 64, 128 x 128, 256 x 128 or 256 x 256 output tiles (the shape with the lowest
+//     estimated time) on v_mfma_f32_32x32x16_f16, K steps of 64 through two LDS buffers, the operands of the step after
+//     next on their way into registers and the next step's on their way into LDS while this step's MFMAs run.
 // The MFMA kernels dequantise to fp16((q - z) * s) (what the specialised tile GEMM's unpacking produces as well).
 #include "nnf_device.h"
 #include "nnf_launch.h"
@@ -291,32 +291,37 @@ namespace nnf
         }
     }
 
-    // Output tiles of 64 WT x 64 WT (WT = 1, or 2 for products large enough to fill the chip with 128 x 128 tiles): four
-    // wavefronts of WT x WT MFMA tiles (v_mfma_f32_32x32x16_f16), K steps of 64 through two LDS buffers, one barrier per
-    // step.  A step's operands travel global -> registers -> LDS: the activations as they are (16-byte pieces, a
-    // wavefront-wide load takes whole 128-byte lines of 8 rows), the weights dequantised on the way by the thread that
-    // fetched them -- the exact integers q - z in fp16 (offset trick) times the scale, one rounding, which is
-    // fp16((q - z) * s).  Two sets of staging registers: the loads of step s + 2 are issued ahead of the MFMAs of step s
-    // and stored behind the MFMAs of step s + 1, so a load has two steps to arrive (with one set a step lasted as long
-    // as a load from memory, half a microsecond, whatever M was).  The loads are issued and stored every step, past the
-    // end of K at clamped addresses and as zeros: a branch around them would make the compiler wait for every load in
-    // flight at the top of the loop.  Tiles are numbered in groups of four tile rows, tile row fastest, and dealt to the eight XCDs in
-    // contiguous runs, so that the workgroups in flight together share activations and weights in one L2.
-    template <int BITS, int WT>
+    // Output tiles of 64 WM x 64 WN: four wavefronts (2 x 2) of WM x WN MFMA tiles each (v_mfma_f32_32x32x16_f16), K
+    // steps of 64 through two LDS buffers, one barrier per step.  A step's operands travel global -> registers -> LDS:
+    // the activations as they are (16-byte pieces, a wavefront-wide load takes whole 128-byte lines of 8 rows), the
+    // weights dequantised on the way by the thread that fetched them -- the exact integers q - z in fp16 (offset trick)
+    // times the scale, one rounding, which is fp16((q - z) * s).  Two sets of staging registers: the loads of step s + 2
+    // are issued ahead of the MFMAs of step s and stored among the MFMAs of step s + 1, so a load has two steps to
+    // arrive (with one set a step lasted as long as a load from memory, half a microsecond, whatever M was).  A step
+    // runs in quarters (16 values of K): the next quarter's fragments are read from LDS, this quarter's MFMAs issued,
+    // and a quarter of the next step's pieces unpacked and stored into the other buffer between them -- with one
+    // wavefront per SIMD nothing else would fill the matrix cores while a wavefront unpacks (M = 4096, N = K = 8192,
+    // 8 bits: 256 x 256 tiles 660 -> 574 us; 128 x 128 tiles, two workgroups per CU, 706 -> 699).  The loads are issued
+    // and stored every step, past the end of K at clamped addresses and as zeros: a branch around them would make the
+    // compiler wait for every load in flight at the top of the loop.  Tiles are numbered in groups of four tile rows,
+    // tile row fastest, and dealt to the eight XCDs in contiguous runs, so that the workgroups in flight together share
+    // activations and weights in one L2.
+    template <int BITS, int WM, int WN>
     __global__ __launch_bounds__(256) void wna16_tile_kernel(const half_t* __restrict__ A, const uint8_t* __restrict__ Wq,
                                                              const half_t* __restrict__ S, half_t* __restrict__ Y, int M, int N,
                                                              int K, int tiles_m, int tiles_n, QuantArgs qa)
     {
-        constexpr int T = 64 * WT;        // rows and columns of the output tile
+        constexpr int TM = 64 * WM, TN = 64 * WN; // rows and columns of the output tile
         constexpr int KS = 64;            // values of K per step
         constexpr int PITCH = KS + 8;     // halves per staged row (144 bytes: 16-byte pieces stay aligned)
-        constexpr int OPERAND = T * PITCH; // halves of one staged operand
+        constexpr int A_OPERAND = TM * PITCH, W_OPERAND = TN * PITCH; // halves of the staged operands
+        constexpr int BUFFER = A_OPERAND + W_OPERAND;
         constexpr int WPP = 128 / BITS;   // weights of a 16-byte piece (inside one group)
         constexpr int PPR = KS / WPP;     // pieces per weight row and step
-        constexpr int A_PER = T / 32;     // pieces of activations per thread and step: piece tid % 8 of rows tid / 8 + 32 i
-        constexpr int W_PIECES = T * PPR;
+        constexpr int A_PER = TM / 32;    // pieces of activations per thread and step: piece tid % 8 of rows tid / 8 + 32 i
+        constexpr int W_PIECES = TN * PPR;
         constexpr int W_PER = (W_PIECES + 255) / 256; // pieces of weights per thread and step: piece p % PPR of row p / PPR, p = tid + 256 j
-        extern __shared__ __attribute__((aligned(16))) half_t lds[]; // [buffer][A, W][OPERAND]
+        extern __shared__ __attribute__((aligned(16))) half_t lds[]; // [buffer][A: TM rows, W: TN rows][PITCH]
         const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
         int tm, tn;
         {
@@ -331,12 +336,12 @@ namespace nnf
             tm = first_m + rr % gm;
             tn = rr / gm;
         }
-        const int m0 = tm * T, n0 = tn * T;
+        const int m0 = tm * TM, n0 = tn * TN;
         const int G = K >> qa.group_shift;
         const size_t row_bytes = (size_t)K * BITS / 8;
         const int steps = (K + KS - 1) / KS;
         const int a_row = tid >> 3, a_k = (tid & 7) * 8;
-        // fragments: wavefront (wm, wn) owns rows [32 WT wm, +32 WT) x columns [32 WT wn, +32 WT)
+        // fragments: wavefront (wm, wn) owns rows [32 WM wm, +32 WM) x columns [32 WN wn, +32 WN)
         const int wm = wave >> 1, wn = wave & 1;
         const int f_row = lane & 31, f_k = (lane >> 5) * 8;
 
@@ -378,21 +383,18 @@ namespace nnf
                 r.z[j] = z_base[(size_t)n * qa.zp_stride + (BITS == 4 ? g >> 1 : g)];
             }
         };
-        auto stage = [&](int step, const Staged& r) {
-            half_t* a_s = lds + (size_t)(step & 1) * 2 * OPERAND;
-            half_t* w_s = a_s + OPERAND;
-#pragma unroll
-            for (int i = 0; i < A_PER; ++i)
-            {
-                // rows past M, a last step of 32: zeros
-                const bool real = m0 + a_row + 32 * i < M && step * KS + a_k < K;
-                *reinterpret_cast<uintx4*>(a_s + (a_row + 32 * i) * PITCH + a_k) = real ? r.a[i] : uintx4{0u, 0u, 0u, 0u};
-            }
-#pragma unroll
-            for (int j = 0; j < W_PER; ++j)
+        // piece i of the activations / piece j of the weights of step `step` into its buffer
+        auto stage_a = [&](int step, const Staged& r, int i) {
+            half_t* a_s = lds + (size_t)(step & 1) * BUFFER;
+            // rows past M, a last step of 32: zeros
+            const bool real = m0 + a_row + 32 * i < M && step * KS + a_k < K;
+            *reinterpret_cast<uintx4*>(a_s + (a_row + 32 * i) * PITCH + a_k) = real ? r.a[i] : uintx4{0u, 0u, 0u, 0u};
+        };
+        auto stage_w = [&](int step, const Staged& r, int j) {
+            half_t* w_s = lds + (size_t)(step & 1) * BUFFER + A_OPERAND;
             {
                 if (W_PIECES % 256 != 0 && tid + 256 * j >= W_PIECES)
-                    continue;
+                    return;
                 int row, k, n, kc, g;
                 w_piece(step, j, row, k, n, kc, g);
                 const int zt = BITS == 4 ? (int)(((uint32_t)r.z[j] >> ((g & 1) * 4)) & 15u) : (int)r.z[j];
@@ -433,11 +435,22 @@ namespace nnf
                 }
             }
         };
-        floatx16 acc[WT][WT];
+        // the pieces of quarter q of a step (all of them: q < 0)
+        auto stage = [&](int step, const Staged& r, int q) {
 #pragma unroll
-        for (int i = 0; i < WT; ++i)
+            for (int i = 0; i < A_PER; ++i)
+                if (q < 0 || i * 4 / A_PER == q)
+                    stage_a(step, r, i);
 #pragma unroll
-            for (int j = 0; j < WT; ++j)
+            for (int j = 0; j < W_PER; ++j)
+                if (q < 0 || j * 4 / W_PER == q)
+                    stage_w(step, r, j);
+        };
+        floatx16 acc[WM][WN];
+#pragma unroll
+        for (int i = 0; i < WM; ++i)
+#pragma unroll
+            for (int j = 0; j < WN; ++j)
 #pragma unroll
                 for (int e = 0; e < 16; ++e)
                     acc[i][j][e] = 0.f;
@@ -445,35 +458,42 @@ namespace nnf
         // s + 1) into the other buffer, barrier
         auto step = [&](int s, Staged& refill, const Staged& ready) {
             fetch(s + 2, refill);
-            // (the loads stay here, ahead of the MFMAs: moved down among them, their registers were shared with the
-            // fragments' and every load in flight was waited for at the top of the loop)
+            // (the loads stay here, ahead of the MFMAs: among the first quarter's MFMAs they gain nothing at 4096 rows
+            // and cost 5 % at a hundred)
             __builtin_amdgcn_sched_barrier(0);
-            const half_t* a_s = lds + (size_t)(s & 1) * 2 * OPERAND;
-            const half_t* w_s = a_s + OPERAND;
+            const half_t* a_s = lds + (size_t)(s & 1) * BUFFER;
+            const half_t* w_s = a_s + A_OPERAND;
+            half8_t fa[2][WM], fw[2][WN];
+            auto read_frags = [&](int kk) {
+#pragma unroll
+                for (int i = 0; i < WM; ++i)
+                    fa[kk & 1][i] = *reinterpret_cast<const half8_t*>(a_s + ((wm * WM + i) * 32 + f_row) * PITCH + kk * 16 + f_k);
+#pragma unroll
+                for (int j = 0; j < WN; ++j)
+                    fw[kk & 1][j] = *reinterpret_cast<const half8_t*>(w_s + ((wn * WN + j) * 32 + f_row) * PITCH + kk * 16 + f_k);
+            };
+            read_frags(0);
+            // a quarter of the step: the next quarter's fragments, this quarter's MFMAs and, between them, a quarter of
+            // the next step's pieces on their way into the other buffer (last read a step ago, before the barrier)
 #pragma unroll
             for (int kk = 0; kk < KS / 16; ++kk)
             {
-                half8_t fa[WT], fw[WT];
+                if (kk + 1 < KS / 16)
+                    read_frags(kk + 1);
 #pragma unroll
-                for (int i = 0; i < WT; ++i)
-                {
-                    fa[i] = *reinterpret_cast<const half8_t*>(a_s + ((wm * WT + i) * 32 + f_row) * PITCH + kk * 16 + f_k);
-                    fw[i] = *reinterpret_cast<const half8_t*>(w_s + ((wn * WT + i) * 32 + f_row) * PITCH + kk * 16 + f_k);
-                }
+                for (int i = 0; i < WM; ++i)
 #pragma unroll
-                for (int i = 0; i < WT; ++i)
-#pragma unroll
-                    for (int j = 0; j < WT; ++j)
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[i], fw[j], acc[i][j], 0, 0, 0);
+                    for (int j = 0; j < WN; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[kk & 1][i], fw[kk & 1][j], acc[i][j], 0, 0, 0);
+                stage(s + 1, ready, kk);
+                __builtin_amdgcn_sched_barrier(0);
             }
-            __builtin_amdgcn_sched_barrier(0);
-            stage(s + 1, ready); // its buffer was last read a step ago, before the barrier at its end
             __syncthreads();
         };
         Staged r0, r1;
         fetch(0, r0);
         fetch(1, r1);
-        stage(0, r0);
+        stage(0, r0, -1);
         __syncthreads();
         // (no branch around a step or its stores either: past the end of K a step stores and multiplies zeros)
         for (int s = 0; s < steps; s += 2)
@@ -483,15 +503,15 @@ namespace nnf
         }
         // D[m][n]: lane l holds column l % 32; element e is row 8 (e / 4) + 4 (l / 32) + e % 4
 #pragma unroll
-        for (int i = 0; i < WT; ++i)
+        for (int i = 0; i < WM; ++i)
 #pragma unroll
-            for (int j = 0; j < WT; ++j)
+            for (int j = 0; j < WN; ++j)
             {
-                const int n = n0 + (wn * WT + j) * 32 + (lane & 31);
+                const int n = n0 + (wn * WN + j) * 32 + (lane & 31);
 #pragma unroll
                 for (int e = 0; e < 16; ++e)
                 {
-                    const int m = m0 + (wm * WT + i) * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
+                    const int m = m0 + (wm * WM + i) * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
                     if (m < M && n < N)
                         Y[(size_t)m * N + n] = (half_t)acc[i][j][e];
                 }
@@ -500,16 +520,16 @@ namespace nnf
 
     namespace
     {
-        template <int BITS, int WT>
+        template <int BITS, int WM, int WN>
         hipError_t launch_wna16_tile(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M, int N, int K,
                                      const QuantArgs& qa)
         {
-            constexpr int T = 64 * WT;
-            constexpr int LDS = 2 * 2 * T * (64 + 8) * (int)sizeof(half_t);
-            const int tiles_m = (M + T - 1) / T, tiles_n = (N + T - 1) / T;
+            constexpr int TM = 64 * WM, TN = 64 * WN;
+            constexpr int LDS = 2 * (TM + TN) * (64 + 8) * (int)sizeof(half_t);
+            const int tiles_m = (M + TM - 1) / TM, tiles_n = (N + TN - 1) / TN;
             if ((long long)tiles_m * tiles_n > 0x7fffff00ll)
                 return hipErrorInvalidValue;
-            auto kernel = &wna16_tile_kernel<BITS, WT>;
+            auto kernel = &wna16_tile_kernel<BITS, WM, WN>;
             if (LDS > 64 * 1024)
             {
                 static LdsGrant granted;
@@ -593,12 +613,31 @@ namespace nnf
                                    (const uint8_t*)Wq, (const half_t*)S, (half_t*)Y, M, N, K, qa);
             return hipGetLastError();
         }
-        // 128 x 128 tiles once they fill the chip, 64 x 64 below
-        const int tiles_m = (M + 127) / 128, tiles_n = (N + 127) / 128;
-        if ((long long)tiles_m * tiles_n >= num_cu)
-            return bits == 4 ? launch_wna16_tile<4, 2>(stream, A, Wq, S, Y, M, N, K, qa)
-                             : launch_wna16_tile<8, 2>(stream, A, Wq, S, Y, M, N, K, qa);
-        return bits == 4 ? launch_wna16_tile<4, 1>(stream, A, Wq, S, Y, M, N, K, qa)
-                         : launch_wna16_tile<8, 1>(stream, A, Wq, S, Y, M, N, K, qa);
+        // 256 x 256, 256 x 128, 128 x 128 or 64 x 64 tiles: the shape with the lowest estimate, in thousandths of the
+        // time of one round of 256 x 256 tiles (one tile per CU).  Measured at K = 8192 and 4096 on 256 CUs: a round of
+        // 256 x 128 tiles takes 0.585 of that, 128 x 128 tiles 0.42 while every tile has a CU to itself and 0.68 per
+        // round of two tiles per CU, 64 x 64 tiles 0.125 + 0.132 per tile and CU (twelve products between 200 and 4096
+        // rows: the estimate picks the fastest of the four measured shapes in each).
+        const auto rounds = [&](int wm, int wn, int per_cu) {
+            const long long t = (long long)((M + 64 * wm - 1) / (64 * wm)) * ((N + 64 * wn - 1) / (64 * wn));
+            return (t + (long long)num_cu * per_cu - 1) / ((long long)num_cu * per_cu);
+        };
+        const long long c44 = 1000 * rounds(4, 4, 1), c42 = 585 * rounds(4, 2, 1);
+        const long long c22 = rounds(2, 2, 1) == 1 ? 420 : 680 * rounds(2, 2, 2);
+        const long long c11 = 125 + 132 * rounds(1, 1, 1);
+#ifdef NNF_TILE_FORCE
+        return launch_wna16_tile<8, NNF_TILE_FORCE>(stream, A, Wq, S, Y, M, N, K, qa);
+#endif
+        if (c44 <= c42 && c44 <= c22 && c44 <= c11)
+            return bits == 4 ? launch_wna16_tile<4, 4, 4>(stream, A, Wq, S, Y, M, N, K, qa)
+                             : launch_wna16_tile<8, 4, 4>(stream, A, Wq, S, Y, M, N, K, qa);
+        if (c42 <= c22 && c42 <= c11)
+            return bits == 4 ? launch_wna16_tile<4, 4, 2>(stream, A, Wq, S, Y, M, N, K, qa)
+                             : launch_wna16_tile<8, 4, 2>(stream, A, Wq, S, Y, M, N, K, qa);
+        if (c22 <= c11)
+            return bits == 4 ? launch_wna16_tile<4, 2, 2>(stream, A, Wq, S, Y, M, N, K, qa)
+                             : launch_wna16_tile<8, 2, 2>(stream, A, Wq, S, Y, M, N, K, qa);
+        return bits == 4 ? launch_wna16_tile<4, 1, 1>(stream, A, Wq, S, Y, M, N, K, qa)
+                         : launch_wna16_tile<8, 1, 1>(stream, A, Wq, S, Y, M, N, K, qa);
     }
 } // namespace nnf

@@ -68,6 +68,8 @@ SHAPES = [
     (64, 9000, 2048), (65, 9000, 2048),
     # enough 128 x 128 tiles to fill the chip: the larger tile kernel; ragged M and N, an odd number of groups
     (2048, 2048, 512), (1100, 4100, 160), (4096, 1030, 384),
+    # ... 256 x 128 tiles (one round of them beats two of 128 x 128), 256 x 256 tiles (they fill the chip): ragged M and N
+    (1000, 8100, 384), (1990, 8100, 160), (300, 22016, 128),
 ]
 
 
@@ -86,12 +88,12 @@ def test_wna16_matches_oracle(gpu, m, n, k, bits, group, zp_tensor):
 
 
 @pytest.mark.parametrize("m,n,k", [(4, 70, 640), (40, 70, 640), (2000, 2100, 640), (40, 300, 1024), (300, 520, 768),
-                                   (2000, 2100, 512)])
+                                   (2000, 2100, 512), (1990, 8100, 640)])
 @pytest.mark.parametrize("bits,group,zp_tensor", [(4, 32, True), (4, 64, False), (8, 64, True), (8, 128, False), (8, 32, True),
                                                    (4, 64, True), (4, 128, True), (4, 32, False)])
 def test_one_hot_rows_return_the_dequantised_weights(gpu, m, n, k, bits, group, zp_tensor):
-    """A = e_k: 1 * w is exact in every kernel (m = 2000: the 128 x 128 tiles; K a multiple of 256 with 4-bit weights: the
-    stream-K tile GEMM), so the output is fp16((q - z) * s) bit for bit; pins nibble and byte order of weights and zero
+    """A = e_k: 1 * w is exact in every kernel (m = 2000: the 256 x 128 tiles, m = 1990: the 256 x 256 tiles; K a multiple
+    of 256 with 4-bit weights: the stream-K tile GEMM), so the output is fp16((q - z) * s) bit for bit; pins nibble and byte order of weights and zero
     points and the block each scale belongs to, on the device."""
     _, wq, s, zps = _case(5, m, n, k, bits, group, zp_tensor)
     zp = 3 if bits == 4 else 200
