@@ -291,36 +291,48 @@ namespace nnf
         }
     }
 
-    // Output tiles of 64 WM x 64 WN: four wavefronts (2 x 2) of WM x WN MFMA tiles each (v_mfma_f32_32x32x16_f16), K
-    // steps of 64 through two LDS buffers, one barrier per step.  A step's operands travel global -> registers -> LDS:
-    // the activations as they are (16-byte pieces, a wavefront-wide load takes whole 128-byte lines of 8 rows), the
-    // weights dequantised on the way by the thread that fetched them -- the exact integers q - z in fp16 (offset trick)
-    // times the scale, one rounding, which is fp16((q - z) * s).  Two sets of staging registers: the loads of step s + 2
-    // are issued ahead of the MFMAs of step s and stored among the MFMAs of step s + 1, so a load has two steps to
-    // arrive (with one set a step lasted as long as a load from memory, half a microsecond, whatever M was).  A step
-    // runs in quarters (16 values of K): the next quarter's fragments are read from LDS, this quarter's MFMAs issued,
-    // and a quarter of the next step's pieces unpacked and stored into the other buffer between them -- with one
-    // wavefront per SIMD nothing else would fill the matrix cores while a wavefront unpacks (M = 4096, N = K = 8192,
-    // 8 bits: 256 x 256 tiles 660 -> 574 us; 128 x 128 tiles, two workgroups per CU, 706 -> 699).  The loads are issued
-    // and stored every step, past the end of K at clamped addresses and as zeros: a branch around them would make the
-    // compiler wait for every load in flight at the top of the loop.  Tiles are numbered in groups of four tile rows,
-    // tile row fastest, and dealt to the eight XCDs in contiguous runs, so that the workgroups in flight together share
-    // activations and weights in one L2.
-    template <int BITS, int WM, int WN>
-    __global__ __launch_bounds__(256) void wna16_tile_kernel(const half_t* __restrict__ A, const uint8_t* __restrict__ Wq,
+    // Output tiles of 32 WAVES_M WM x 32 WAVES_N WN: WAVES_M x WAVES_N wavefronts of WM x WN MFMA tiles each
+    // (v_mfma_f32_32x32x16_f16), K steps of 64 through two LDS buffers, one barrier per step.  A step's operands travel
+    // global -> registers -> LDS: the activations as they are (16-byte pieces, a wavefront-wide load takes whole
+    // 128-byte lines of 8 rows), the weights dequantised on the way by the thread that fetched them -- the exact
+    // integers q - z in fp16 (offset trick) times the scale, one rounding, which is fp16((q - z) * s).  Two sets of
+    // staging registers: the loads of step s + 2 are issued ahead of the MFMAs of step s and stored among the MFMAs of
+    // step s + 1, so a load has two steps to arrive (with one set a step lasted as long as a load from memory, half a
+    // microsecond, whatever M was).  A step runs in quarters (16 values of K): the next quarter's fragments are read
+    // from LDS, this quarter's MFMAs issued, and a slice of the next step's pieces unpacked and stored into the other
+    // buffer between them.  What a wavefront issues besides MFMAs hardly overlaps its own MFMAs (timing-only builds at
+    // 2048 x 8192 x 8192, 8 bits, 256 x 256 tiles on four wavefronts: MFMAs and fragment reads alone 213 us, everything
+    // 287, every load served by the same four cache lines 277), so the 256-row tiles run on eight wavefronts, two per
+    // SIMD (256 x 256: 563 -> 517 us at 4096 rows; 256 x 128: 171 -> 160 at 1024).  The loads are issued and stored
+    // every step, past the end of K at clamped addresses and as zeros: a branch around them would make the compiler wait
+    // for every load in flight at the top of the loop.  Tiles are numbered in groups of four tile rows, tile row fastest,
+    // and dealt to the eight XCDs in contiguous runs, so that the workgroups in flight together share activations and
+    // weights in one L2 (groups of 2, 8 or 16 tile rows measure the same).
+    template <int BITS, int WM, int WN, bool TAIL, int WAVES_M, int WAVES_N>
+    __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void wna16_tile_kernel(const half_t* __restrict__ A, const uint8_t* __restrict__ Wq,
                                                              const half_t* __restrict__ S, half_t* __restrict__ Y, int M, int N,
                                                              int K, int tiles_m, int tiles_n, QuantArgs qa)
     {
-        constexpr int TM = 64 * WM, TN = 64 * WN; // rows and columns of the output tile
+        constexpr int NW = WAVES_M * WAVES_N, THREADS = 64 * NW; // wavefronts: WAVES_M x WAVES_N
+        constexpr int TM = 32 * WAVES_M * WM, TN = 32 * WAVES_N * WN; // rows and columns of the output tile
+        constexpr int A_ROWS = THREADS / 8;                   // rows of activations the workgroup fetches per pass
         constexpr int KS = 64;            // values of K per step
         constexpr int PITCH = KS + 8;     // halves per staged row (144 bytes: 16-byte pieces stay aligned)
         constexpr int A_OPERAND = TM * PITCH, W_OPERAND = TN * PITCH; // halves of the staged operands
         constexpr int BUFFER = A_OPERAND + W_OPERAND;
         constexpr int WPP = 128 / BITS;   // weights of a 16-byte piece (inside one group)
         constexpr int PPR = KS / WPP;     // pieces per weight row and step
-        constexpr int A_PER = TM / 32;    // pieces of activations per thread and step: piece tid % 8 of rows tid / 8 + 32 i
+        constexpr int A_PER = TM / A_ROWS; // pieces of activations per thread and step: piece tid % 8 of rows tid / 8 + 32 i
         constexpr int W_PIECES = TN * PPR;
-        constexpr int W_PER = (W_PIECES + 255) / 256; // pieces of weights per thread and step: piece p % PPR of row p / PPR, p = tid + 256 j
+        // the activations (L2 hits) are fetched one step ahead where a step is long (256-row tiles: a microsecond and
+        // more), two steps ahead like the weights otherwise
+        constexpr int A_AHEAD = WM >= 4 ? 1 : 2;
+        // The barrier of a step stands behind its third quarter where the registers allow it (CARRY: the first fragments
+        // of the next step are read during the fourth quarter and carried into the next step; the 256 x 256 tile, whose
+        // sums take all 256 accumulation registers, has no room for that and keeps its barrier at the end of the step)
+        constexpr bool CARRY = WM * WN < 16 && NW != 8;
+        constexpr int SLICES = CARRY ? 3 : 4; // quarters that store pieces of the next step
+        constexpr int W_PER = (W_PIECES + THREADS - 1) / THREADS; // pieces of weights per thread and step: piece p % PPR of row p / PPR, p = tid + THREADS j
         extern __shared__ __attribute__((aligned(16))) half_t lds[]; // [buffer][A: TM rows, W: TN rows][PITCH]
         const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
         int tm, tn;
@@ -342,14 +354,14 @@ namespace nnf
         const int steps = (K + KS - 1) / KS;
         const int a_row = tid >> 3, a_k = (tid & 7) * 8;
         // fragments: wavefront (wm, wn) owns rows [32 WM wm, +32 WM) x columns [32 WN wn, +32 WN)
-        const int wm = wave >> 1, wn = wave & 1;
+        const int wm = wave / WAVES_N, wn = wave % WAVES_N;
         const int f_row = lane & 31, f_k = (lane >> 5) * 8;
 
         // what a thread fetches per step, as it arrives: anything computed from it here would be waited for here
         struct Staged
         {
             uintx4 a[A_PER], w[W_PER];
-            half_t s[W_PER];  // the piece's scale
+            unsigned short s[W_PER]; // the piece's scale (fp16 bits)
             uint8_t z[W_PER]; // the byte that holds its zero point (widened where it is used: widened here, it would be waited for here)
         };
         // (no zero-point tensor: the byte is fetched all the same, from the scales, and not used -- a branch around the
@@ -358,50 +370,55 @@ namespace nnf
         // piece j of this thread: its weight row (clamped to N - 1), the first of its weights in step `step` (clamped to
         // the last whole piece of the row), its group
         auto w_piece = [&](int step, int j, int& row, int& k, int& n, int& kc, int& g) {
-            const int p = min(tid + 256 * j, W_PIECES - 1);
+            const int p = min(tid + THREADS * j, W_PIECES - 1);
             row = p / PPR;
             k = step * KS + (p % PPR) * WPP;
             kc = min(k, K - WPP);
             n = min(n0 + row, N - 1);
             g = kc >> qa.group_shift;
         };
-        auto fetch = [&](int step_raw, Staged& r) {
+        auto fetch_a = [&](int step_raw, Staged& r) {
             const int step = min(step_raw, steps - 1);
 #pragma unroll
             for (int i = 0; i < A_PER; ++i)
             {
-                const int row = min(m0 + a_row + 32 * i, M - 1), k = min(step * KS + a_k, K - 8);
+                const int row = min(m0 + a_row + A_ROWS * i, M - 1), k = min(step * KS + a_k, K - 8);
                 r.a[i] = *reinterpret_cast<const uintx4*>(A + (size_t)row * K + k);
             }
+        };
+        auto fetch_w = [&](int step_raw, Staged& r) {
+            const int step = min(step_raw, steps - 1);
 #pragma unroll
             for (int j = 0; j < W_PER; ++j)
             {
                 int row, k, n, kc, g;
                 w_piece(step, j, row, k, n, kc, g);
                 r.w[j] = *reinterpret_cast<const uintx4*>(Wq + (size_t)n * row_bytes + (size_t)kc * BITS / 8);
-                r.s[j] = S[(size_t)n * G + g];
+                r.s[j] = reinterpret_cast<const unsigned short*>(S)[(size_t)n * G + g];
                 r.z[j] = z_base[(size_t)n * qa.zp_stride + (BITS == 4 ? g >> 1 : g)];
             }
         };
         // piece i of the activations / piece j of the weights of step `step` into its buffer
         auto stage_a = [&](int step, const Staged& r, int i) {
             half_t* a_s = lds + (size_t)(step & 1) * BUFFER;
-            // rows past M, a last step of 32: zeros
-            const bool real = m0 + a_row + 32 * i < M && step * KS + a_k < K;
-            *reinterpret_cast<uintx4*>(a_s + (a_row + 32 * i) * PITCH + a_k) = real ? r.a[i] : uintx4{0u, 0u, 0u, 0u};
+            // TAIL (K no multiple of 128: a last step of 32, or an odd number of steps, the loop running over an even
+            // one): zeros behind the end of K.  (Rows past M repeat row M - 1 and columns past N column N - 1: what they
+            // add up is never stored.)
+            const bool real = !TAIL || step * KS + a_k < K;
+            *reinterpret_cast<uintx4*>(a_s + (a_row + A_ROWS * i) * PITCH + a_k) = real ? r.a[i] : uintx4{0u, 0u, 0u, 0u};
         };
         auto stage_w = [&](int step, const Staged& r, int j) {
             half_t* w_s = lds + (size_t)(step & 1) * BUFFER + A_OPERAND;
             {
-                if (W_PIECES % 256 != 0 && tid + 256 * j >= W_PIECES)
+                if (W_PIECES % THREADS != 0 && tid + THREADS * j >= W_PIECES)
                     return;
                 int row, k, n, kc, g;
                 w_piece(step, j, row, k, n, kc, g);
                 const int zt = BITS == 4 ? (int)(((uint32_t)r.z[j] >> ((g & 1) * 4)) & 15u) : (int)r.z[j];
                 const ExactWeights<BITS> exact(qa.zps ? zt : qa.zp);
-                // columns past N, a last step of 32: weights of zero
-                const half_t sh = (n0 + row < N && k < K) ? r.s[j] : (half_t)0.f;
-                const half2_t s2 = half2_t{sh, sh};
+                // TAIL: weights of zero behind the end of K
+                const uint32_t su = (uint32_t)r.s[j];
+                const half2_t s2 = as_half2((!TAIL || k < K) ? __builtin_amdgcn_perm(su, su, 0x05040504u) : 0u);
                 const uint32_t ww[4] = {r.w[j].x, r.w[j].y, r.w[j].z, r.w[j].w};
                 half_t* dst = w_s + row * PITCH + (k - step * KS);
                 if constexpr (BITS == 4)
@@ -435,16 +452,18 @@ namespace nnf
                 }
             }
         };
-        // the pieces of quarter q of a step (all of them: q < 0)
-        auto stage = [&](int step, const Staged& r, int q) {
-#pragma unroll
-            for (int i = 0; i < A_PER; ++i)
-                if (q < 0 || i * 4 / A_PER == q)
-                    stage_a(step, r, i);
+        // slice q of the pieces of a step (all of them: q < 0): the weights first (ra: the set that holds the step's
+        // activations, rw: its weights); a piece of weights counts as three of activations
+        constexpr int UNITS = 3 * W_PER + A_PER;
+        auto stage = [&](int step, const Staged& ra, const Staged& rw, int q) {
 #pragma unroll
             for (int j = 0; j < W_PER; ++j)
-                if (q < 0 || j * 4 / W_PER == q)
-                    stage_w(step, r, j);
+                if (q < 0 || 3 * j * SLICES / UNITS == q)
+                    stage_w(step, rw, j);
+#pragma unroll
+            for (int i = 0; i < A_PER; ++i)
+                if (q < 0 || (3 * W_PER + i) * SLICES / UNITS == q)
+                    stage_a(step, ra, i);
         };
         floatx16 acc[WM][WN];
 #pragma unroll
@@ -454,48 +473,69 @@ namespace nnf
 #pragma unroll
                 for (int e = 0; e < 16; ++e)
                     acc[i][j][e] = 0.f;
-        // step s: the loads of step s + 2 into the set step s was stored from, the MFMAs of step s, the other set (step
-        // s + 1) into the other buffer, barrier
+        // step s: the loads of step s + 2 into the set step s was stored from; then in quarters (16 values of K): the
+        // next quarter's fragments, this quarter's MFMAs and, between them, a slice of the next step's pieces on their way
+        // into the other buffer (last read before the previous barrier).  With the barrier behind the third quarter
+        // every wavefront holds its last fragments of this step and has stored its pieces of the next by then, so the
+        // fourth quarter's MFMAs run while the next step's first fragments are read -- nothing waits for LDS behind
+        // the barrier.
+        half8_t fa_carried[2][WM], fw_carried[2][WN];
+        auto read_frags = [&](int s, int kk, half8_t (&fa)[2][WM], half8_t (&fw)[2][WN]) {
+            const half_t* a_s = lds + (size_t)(s & 1) * BUFFER;
+            const half_t* w_s = a_s + A_OPERAND;
+#pragma unroll
+            for (int i = 0; i < WM; ++i)
+                fa[kk & 1][i] = *reinterpret_cast<const half8_t*>(a_s + ((wm * WM + i) * 32 + f_row) * PITCH + kk * 16 + f_k);
+#pragma unroll
+            for (int j = 0; j < WN; ++j)
+                fw[kk & 1][j] = *reinterpret_cast<const half8_t*>(w_s + ((wn * WN + j) * 32 + f_row) * PITCH + kk * 16 + f_k);
+        };
         auto step = [&](int s, Staged& refill, const Staged& ready) {
-            fetch(s + 2, refill);
+            if constexpr (A_AHEAD == 1)
+                fetch_a(s + 1, refill);
+            else
+                fetch_a(s + 2, refill);
+            fetch_w(s + 2, refill);
             // (the loads stay here, ahead of the MFMAs: among the first quarter's MFMAs they gain nothing at 4096 rows
             // and cost 5 % at a hundred)
             __builtin_amdgcn_sched_barrier(0);
-            const half_t* a_s = lds + (size_t)(s & 1) * BUFFER;
-            const half_t* w_s = a_s + A_OPERAND;
-            half8_t fa[2][WM], fw[2][WN];
-            auto read_frags = [&](int kk) {
-#pragma unroll
-                for (int i = 0; i < WM; ++i)
-                    fa[kk & 1][i] = *reinterpret_cast<const half8_t*>(a_s + ((wm * WM + i) * 32 + f_row) * PITCH + kk * 16 + f_k);
-#pragma unroll
-                for (int j = 0; j < WN; ++j)
-                    fw[kk & 1][j] = *reinterpret_cast<const half8_t*>(w_s + ((wn * WN + j) * 32 + f_row) * PITCH + kk * 16 + f_k);
-            };
-            read_frags(0);
-            // a quarter of the step: the next quarter's fragments, this quarter's MFMAs and, between them, a quarter of
-            // the next step's pieces on their way into the other buffer (last read a step ago, before the barrier)
+            half8_t fa_local[2][WM], fw_local[2][WN];
+            half8_t (&fa)[2][WM] = CARRY ? fa_carried : fa_local;
+            half8_t (&fw)[2][WN] = CARRY ? fw_carried : fw_local;
+            if constexpr (!CARRY)
+                read_frags(s, 0, fa, fw);
 #pragma unroll
             for (int kk = 0; kk < KS / 16; ++kk)
             {
                 if (kk + 1 < KS / 16)
-                    read_frags(kk + 1);
+                    read_frags(s, kk + 1, fa, fw);
+                else if constexpr (CARRY)
+                    read_frags(s + 1, 0, fa, fw);
 #pragma unroll
                 for (int i = 0; i < WM; ++i)
 #pragma unroll
                     for (int j = 0; j < WN; ++j)
                         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[kk & 1][i], fw[kk & 1][j], acc[i][j], 0, 0, 0);
-                stage(s + 1, ready, kk);
+                if (kk < SLICES)
+                    stage(s + 1, A_AHEAD == 1 ? refill : ready, ready, kk);
                 __builtin_amdgcn_sched_barrier(0);
+                if (kk == SLICES - 1)
+                    __syncthreads();
             }
-            __syncthreads();
         };
         Staged r0, r1;
-        fetch(0, r0);
-        fetch(1, r1);
-        stage(0, r0, -1);
+        fetch_a(0, r0);
+        fetch_w(0, r0);
+        if constexpr (A_AHEAD == 2)
+            fetch_a(1, r1);
+        fetch_w(1, r1);
+        stage(0, r0, r0, -1);
         __syncthreads();
-        // (no branch around a step or its stores either: past the end of K a step stores and multiplies zeros)
+        if constexpr (CARRY)
+            read_frags(0, 0, fa_carried, fw_carried);
+        // (no branch around a step or its stores: with an odd number of steps the last one runs past the end of K,
+        // where TAIL stores zeros; a step peeled off behind the loop instead had the compiler move all 256 sums of the
+        // largest tile through memory)
         for (int s = 0; s < steps; s += 2)
         {
             step(s, r0, r1);
@@ -520,16 +560,17 @@ namespace nnf
 
     namespace
     {
-        template <int BITS, int WM, int WN>
-        hipError_t launch_wna16_tile(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M, int N, int K,
+        template <int BITS, int WM, int WN, bool TAIL, int WAVES_M = 2, int WAVES_N = 2>
+        hipError_t launch_wna16_tile_k(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M, int N, int K,
                                      const QuantArgs& qa)
         {
-            constexpr int TM = 64 * WM, TN = 64 * WN;
+            constexpr int NW = WAVES_M * WAVES_N;
+            constexpr int TM = 32 * WAVES_M * WM, TN = 32 * WAVES_N * WN;
             constexpr int LDS = 2 * (TM + TN) * (64 + 8) * (int)sizeof(half_t);
             const int tiles_m = (M + TM - 1) / TM, tiles_n = (N + TN - 1) / TN;
             if ((long long)tiles_m * tiles_n > 0x7fffff00ll)
                 return hipErrorInvalidValue;
-            auto kernel = &wna16_tile_kernel<BITS, WM, WN>;
+            auto kernel = &wna16_tile_kernel<BITS, WM, WN, TAIL, WAVES_M, WAVES_N>;
             if (LDS > 64 * 1024)
             {
                 static LdsGrant granted;
@@ -538,9 +579,21 @@ namespace nnf
                     return e;
             }
             const int grid = (tiles_m * tiles_n + 7) / 8 * 8; // whole rounds of the XCDs
-            hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(256), LDS, stream, (const half_t*)A, (const uint8_t*)Wq,
+            hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(64 * NW), LDS, stream, (const half_t*)A, (const uint8_t*)Wq,
                                (const half_t*)S, (half_t*)Y, M, N, K, tiles_m, tiles_n, qa);
             return hipGetLastError();
+        }
+    } // namespace
+
+    namespace
+    {
+        // (K is a multiple of 32; the kernel walks K in pairs of steps of 64)
+        template <int BITS, int WM, int WN, int WAVES_M, int WAVES_N>
+        hipError_t launch_wna16_tile(hipStream_t stream, const void* A, const void* Wq, const void* S, void* Y, int M, int N, int K,
+                                     const QuantArgs& qa)
+        {
+            return K % 128 ? launch_wna16_tile_k<BITS, WM, WN, true, WAVES_M, WAVES_N>(stream, A, Wq, S, Y, M, N, K, qa)
+                           : launch_wna16_tile_k<BITS, WM, WN, false, WAVES_M, WAVES_N>(stream, A, Wq, S, Y, M, N, K, qa);
         }
     } // namespace
 
@@ -613,31 +666,29 @@ namespace nnf
                                    (const uint8_t*)Wq, (const half_t*)S, (half_t*)Y, M, N, K, qa);
             return hipGetLastError();
         }
-        // 256 x 256, 256 x 128, 128 x 128 or 64 x 64 tiles: the shape with the lowest estimate, in thousandths of the
-        // time of one round of 256 x 256 tiles (one tile per CU).  Measured at K = 8192 and 4096 on 256 CUs: a round of
-        // 256 x 128 tiles takes 0.585 of that, 128 x 128 tiles 0.42 while every tile has a CU to itself and 0.68 per
-        // round of two tiles per CU, 64 x 64 tiles 0.125 + 0.132 per tile and CU (twelve products between 200 and 4096
-        // rows: the estimate picks the fastest of the four measured shapes in each).
-        const auto rounds = [&](int wm, int wn, int per_cu) {
-            const long long t = (long long)((M + 64 * wm - 1) / (64 * wm)) * ((N + 64 * wn - 1) / (64 * wn));
+        // 256 x 256 (eight wavefronts, 2 x 4, of 128 x 64), 256 x 128 (eight, 4 x 2, of 64 x 64), 128 x 128 or 64 x 64
+        // tiles (four wavefronts): the shape with the lowest estimate, in thousandths of the time of one round of
+        // 256 x 256 tiles (one tile per CU).  Measured at K = 8192 and 4096 on 256 CUs: a round of 256 x 128 tiles takes
+        // 0.60 of that, 128 x 128 tiles 0.45 while every tile has a CU to itself and 0.73 per round of two tiles per CU,
+        // 64 x 64 tiles 0.135 + 0.143 per tile and CU (twelve products between 200 and 4096 rows: the estimate picks
+        // the fastest of the four measured shapes in each).
+        const auto rounds = [&](int tm, int tn, int per_cu) {
+            const long long t = (long long)((M + tm - 1) / tm) * ((N + tn - 1) / tn);
             return (t + (long long)num_cu * per_cu - 1) / ((long long)num_cu * per_cu);
         };
-        const long long c44 = 1000 * rounds(4, 4, 1), c42 = 585 * rounds(4, 2, 1);
-        const long long c22 = rounds(2, 2, 1) == 1 ? 420 : 680 * rounds(2, 2, 2);
-        const long long c11 = 125 + 132 * rounds(1, 1, 1);
-#ifdef NNF_TILE_FORCE
-        return launch_wna16_tile<8, NNF_TILE_FORCE>(stream, A, Wq, S, Y, M, N, K, qa);
-#endif
-        if (c44 <= c42 && c44 <= c22 && c44 <= c11)
-            return bits == 4 ? launch_wna16_tile<4, 4, 4>(stream, A, Wq, S, Y, M, N, K, qa)
-                             : launch_wna16_tile<8, 4, 4>(stream, A, Wq, S, Y, M, N, K, qa);
-        if (c42 <= c22 && c42 <= c11)
-            return bits == 4 ? launch_wna16_tile<4, 4, 2>(stream, A, Wq, S, Y, M, N, K, qa)
-                             : launch_wna16_tile<8, 4, 2>(stream, A, Wq, S, Y, M, N, K, qa);
-        if (c22 <= c11)
-            return bits == 4 ? launch_wna16_tile<4, 2, 2>(stream, A, Wq, S, Y, M, N, K, qa)
-                             : launch_wna16_tile<8, 2, 2>(stream, A, Wq, S, Y, M, N, K, qa);
-        return bits == 4 ? launch_wna16_tile<4, 1, 1>(stream, A, Wq, S, Y, M, N, K, qa)
-                         : launch_wna16_tile<8, 1, 1>(stream, A, Wq, S, Y, M, N, K, qa);
+        const long long c256 = 1000 * rounds(256, 256, 1), c256n = 600 * rounds(256, 128, 1);
+        const long long c128 = rounds(128, 128, 1) == 1 ? 450 : 730 * rounds(128, 128, 2);
+        const long long c64 = 135 + 143 * rounds(64, 64, 1);
+        if (c256 <= c256n && c256 <= c128 && c256 <= c64)
+            return bits == 4 ? launch_wna16_tile<4, 4, 2, 2, 4>(stream, A, Wq, S, Y, M, N, K, qa)
+                             : launch_wna16_tile<8, 4, 2, 2, 4>(stream, A, Wq, S, Y, M, N, K, qa);
+        if (c256n <= c128 && c256n <= c64)
+            return bits == 4 ? launch_wna16_tile<4, 2, 2, 4, 2>(stream, A, Wq, S, Y, M, N, K, qa)
+                             : launch_wna16_tile<8, 2, 2, 4, 2>(stream, A, Wq, S, Y, M, N, K, qa);
+        if (c128 <= c64)
+            return bits == 4 ? launch_wna16_tile<4, 2, 2, 2, 2>(stream, A, Wq, S, Y, M, N, K, qa)
+                             : launch_wna16_tile<8, 2, 2, 2, 2>(stream, A, Wq, S, Y, M, N, K, qa);
+        return bits == 4 ? launch_wna16_tile<4, 1, 1, 2, 2>(stream, A, Wq, S, Y, M, N, K, qa)
+                         : launch_wna16_tile<8, 1, 1, 2, 2>(stream, A, Wq, S, Y, M, N, K, qa);
     }
 } // namespace nnf
