@@ -461,12 +461,13 @@ int main(int argc, char** argv)
         auto k = sel.pick_first(mlp, ROCM_GPU).second;
         auto fm = k->get_or_emit_source();
         CONTAINS(fm->body_unit->get_code(), "nnf_fused_mlp_w4a16_planned(stream, input0, input1, 1.000000000e-06f, input2, input3, input4, input5, output0, 256, 4096, 11008, 128, 8, &gate_up_plan, &down_plan, ");
-        // rstd [256] fp32 + h [256, 11008] fp16 + the larger of the two areas of parked sums: both GEMMs run 256
-        // workgroups; gate/up (2 x 86 tiles of 128 x 256 weight rows x 16 supersteps) needs two slots per workgroup
+        // rstd [256] fp32 + h [256, 11008] fp16 + the larger of the two areas of parked sums: gate/up (2 x 86 tiles of
+        // 128 x 256 weight rows, two thirds of the CUs) runs whole tiles, one workgroup each, and parks nothing; down
+        // (2 x 32 tiles of 128 x 128, 43 supersteps each, split evenly over 256 workgroups) one slot per workgroup
         // ... and the synchronisation words of either product (2 x 86 and 2 x 32 tiles, two words each, and two more)
         EXPECT(k->m_context->tensors.size() == 3 &&
                k->m_context->tensors[0]->size() ==
-                   (size_t)256 * 4 + (size_t)256 * 11008 * 2 + (size_t)2 * 256 * 128 * 256 * 4);
+                   (size_t)256 * 4 + (size_t)256 * 11008 * 2 + (size_t)256 * 128 * 128 * 4);
         EXPECT(k->m_context->tensors[1]->size() == 1408 && k->m_context->tensors[2]->size() == 576 &&
                k->m_context->tensors[1]->is_memset() && k->m_context->tensors[2]->is_memset());
     });

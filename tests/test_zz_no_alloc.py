@@ -54,7 +54,7 @@ def test_static_scratch_rejects_shapes_beyond_its_buffer(gpu):
     from nnfusion_amd import _lib
 
     lib = _lib.kernels()
-    m, n, k = 256, 22016, 4096
+    m, n, k = 384, 22016, 4096
     assert lib.nnf_w4a16_gemm_workspace_bytes(m, n, k, 128) > STATIC_SCRATCH_BYTES
     t = torch.zeros(256, dtype=torch.uint8, device=gpu)  # never touched: the call is refused on its shape
     st = lib.nnf_w4a16_gemm_static_scratch(torch.cuda.current_stream().cuda_stream, t.data_ptr(), t.data_ptr(),
