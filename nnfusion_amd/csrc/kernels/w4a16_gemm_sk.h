@@ -40,7 +40,9 @@
 //     has a scalar base and a 32-bit lane offset that never changes, and the waits on the loads into LDS
 //     and on the fragment reads are counted by hand (the compiler's own would drain everything in flight).
 //   * The workgroups of a launch split the flat list of (tile, superstep) units evenly ("stream-K"): a
-//     launch has one workgroup per CU with the same amount of work, whatever the tile count.  A
+//     launch has one workgroup per CU with the same amount of work, whatever the tile count (the plan launches one
+//     workgroup per tile instead where the tiles fill at least half of the CUs and K is short: sharing tiles costs
+//     more than the idle CUs there).  A
 //     workgroup that covers only part of a tile's K range writes its fp32 sums to the workspace in
 //     register order (1 KiB per store instruction); a second, small launch adds the parts of such tiles
 //     in K order and runs their epilogue, on all CUs (one CU would need tens of microseconds to pull the
