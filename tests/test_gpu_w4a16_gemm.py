@@ -152,9 +152,12 @@ def test_gemm_one_hot_rows_select_weights(gpu):
 
 
 @pytest.mark.parametrize("m,n,k", [(16, 8192, 8192), (128, 8192, 8192), (1024, 8192, 8192), (4096, 8192, 8192),
-                                   (32, 8192, 8192), (16, 22016, 4096), (16, 4096, 11008)])
+                                   (32, 8192, 8192), (16, 22016, 4096), (16, 4096, 11008),
+                                   (250, 21000, 1024), (100, 20004, 768), (640, 8192, 4096), (256, 22016, 4096)])
 def test_gemm_full_size_sampled_columns(gpu, m, n, k):
-    """configs[2] shapes (and batched-decode shapes on the row-streaming kernels: one launch, over ranges of K): all M rows, 192 sampled output columns against the oracle; and linearity in A
+    """configs[2] shapes (and batched-decode shapes on the row-streaming kernels: one launch, over ranges of K; and
+    products whose tiles fill at least half of the CUs, which run whole tiles, one workgroup each, with ragged rows
+    and columns): all M rows, 192 sampled output columns against the oracle; and linearity in A
     on the whole output (Y(2A) == 2 Y(A) bit for bit, as scaling by 2 is exact outside the subnormal range)."""
     import torch
 
