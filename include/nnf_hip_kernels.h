@@ -141,6 +141,8 @@ typedef struct nnf_plan
      * several workgroups.  Without sync_flags their parts are added up by a second launch.  With sync_flags the
      * workgroups count themselves in at their tiles there, and each adds up and finishes its share of a tile's rows
      * once all that hold a part have arrived -- same summation order, bit-identical results, one launch less.
+     * (A plan whose grid has more workgroups than the device has CUs keeps the second launch: workgroups that wait
+     * for one another must all be running.)
      * Two more launches go the same way: a fused RMSNorm's rstd[] is computed by the GEMM launch itself (every
      * workgroup a few rows before its first tile; no pass of its own), and the row-streaming kernel for a few
      * activation rows and K above 8192, which works on ranges of K, adds the ranges up itself (the last workgroup to

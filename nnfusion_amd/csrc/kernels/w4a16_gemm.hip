@@ -266,12 +266,15 @@ namespace nnf
     namespace
     {
         // one launch where the caller gave enough zeroed synchronisation words for the plan's tiles, else two
-        void set_sync(SkGemmParams& p, const workspace::SkPlan& plan, const LaunchChoice& choice)
+        // (and only where every workgroup of the grid has a CU: workgroups that wait for one another inside the launch
+        // must all be running -- a forced plan with more workgroups than CUs would spin to its limit, some milliseconds)
+        void set_sync(SkGemmParams& p, const workspace::SkPlan& plan, const LaunchChoice& choice, int num_cu)
         {
             p.partial_bytes = plan.bytes();
             p.trace = nullptr;
             // (the one-launch form addresses the parked tiles with 32-bit byte offsets)
-            const bool one_launch = plan.slots && choice.sync_flags && choice.sync_bytes >= plan.sync_bytes() && plan.bytes() < ((size_t)1 << 32);
+            const bool one_launch = plan.slots && plan.grid <= num_cu && choice.sync_flags && choice.sync_bytes >= plan.sync_bytes() &&
+                                    plan.bytes() < ((size_t)1 << 32);
             p.sync = one_launch ? (uint32_t*)choice.sync_flags + 2 : nullptr; // (the first two words: rstd_sync)
             p.spin_limit = choice.spin_limit > 0 ? choice.spin_limit : choice.spin_limit < 0 ? 0 : DEFAULT_SPIN_LIMIT;
             p.rstd_out = nullptr;
@@ -279,9 +282,9 @@ namespace nnf
             p.rms_eps = 0.f;
         }
         // RMSNorm's rstd[] can be left to the GEMM launch itself: the caller gave (zeroed) synchronisation words
-        bool rstd_inside_tile_gemm(const workspace::SkPlan& plan, const LaunchChoice& choice)
+        bool rstd_inside_tile_gemm(const workspace::SkPlan& plan, const LaunchChoice& choice, int num_cu)
         {
-            return choice.sync_flags && choice.sync_bytes >= plan.sync_bytes(true);
+            return plan.grid <= num_cu && choice.sync_flags && choice.sync_bytes >= plan.sync_bytes(true);
         }
     } // namespace
 
@@ -305,7 +308,7 @@ namespace nnf
         // (the row-streaming kernels add up the squares of the activations they hold themselves: no pre-pass; the form
         // with a run-time K keeps it)
         const bool normalised_copy = route.kind == W4A16Route::SKINNY || route.kind == W4A16Route::SKINNY_SPLIT;
-        const bool rstd_in_tile_gemm = rms && route.kind == W4A16Route::TILE && rstd_inside_tile_gemm(route.plan, choice);
+        const bool rstd_in_tile_gemm = rms && route.kind == W4A16Route::TILE && rstd_inside_tile_gemm(route.plan, choice, num_cu);
         const bool rstd_in_kernel = route.kind == W4A16Route::ROWS ||
                                     (route.kind == W4A16Route::MROWS && workspace::w4a16_mrows_fixed_k(M, K)) || rstd_in_tile_gemm;
         if (rms && !rstd_in_kernel)
@@ -413,7 +416,7 @@ namespace nnf
         p.supersteps = plan.supersteps;
         p.units = plan.units;
         p.zps = nullptr;
-        set_sync(p, plan, choice);
+        set_sync(p, plan, choice, num_cu);
         if (rstd_in_tile_gemm)
         {
             p.rstd_out = (float*)rms_ws;
@@ -498,7 +501,7 @@ namespace nnf
         p.supersteps = plan.supersteps;
         p.units = plan.units;
         p.zps = (const uint8_t*)zero_points;
-        set_sync(p, plan, choice);
+        set_sync(p, plan, choice, num_cu);
         switch (group_shift)
         {
         case 5: return launch_gemm_sk_q5(stream, p, plan.grid, plan.tile_rows, plan.tile_weight_rows);
